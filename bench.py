@@ -1,0 +1,168 @@
+#!/usr/bin/env python3
+"""Headline benchmark: batch-1 bf16 greedy decode, Llama-3.2-1B shape, one MI355X.
+
+Workload (BASELINE.json configs[1], the reference's `benchmarks.llm_decode` case at
+output length 1024): seeded random-init weights, 8-token random prompt, KV prefilled
+through the decode kernel, then forced greedy continuation.  One "step" is one
+decode step = one megakernel launch = one new token.
+
+  python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu-baseline]
+
+W untimed steps run as a separate short request first; then a fresh request is
+prefilled and exactly K decode steps are timed the way the reference times them
+(`qimeng_megakernel/models/LLM/decode.py:719-792`): one HIP event pair per step
+around the kernel launch only -> kernel_tok_s (the metric), one pair around the
+loop -> tok_s_gpu, perf_counter -> tok_s.  Prints ONE JSON line.
+
+`roofline.achieved` = algorithmic bytes of the K timed launches (bf16 weights +
+KV rows read + KV row written, see DecodeShape.step_bytes) / summed launch time.
+`cpu_baseline` = the CPU oracle (a PyTorch restatement of the reference's fused
+route) timed on the host cores over a bounded sample of the same workload.
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+import time
+from pathlib import Path
+
+ROOT = Path(__file__).resolve().parent
+sys.path.insert(0, str(ROOT))
+
+HBM_PEAK_GBPS = 8000.0
+
+
+def cpu_baseline(shape, weights, prompt, n_steps: int, cores: int) -> dict:
+    """Time the CPU oracle on single-token steps of the same request (bounded sample)."""
+    import torch
+
+    sys.path.insert(0, str(ROOT / "oracle"))
+    from fused_oracle import FusedOracle  # the checker, timed as the reported CPU baseline
+    from qimeng_megakernel_amd import synthetic
+
+    torch.set_num_threads(cores)
+    g = synthetic.build_globals(weights, shape, prompt.numel() + n_steps + 1, "cpu")
+    oracle = FusedOracle(shape)
+    toks = prompt.tolist()
+    # one untimed step pages the weights in
+    oracle.embed(g, toks[0]); g.position_id = 0; oracle.decode_step(g)
+    t0 = time.perf_counter()
+    for pos in range(n_steps):
+        oracle.embed(g, toks[pos]); g.position_id = pos
+        oracle.decode_step(g)
+        if pos + 1 >= len(toks):
+            toks.append(int(g.logits.argmax()))
+    dt = time.perf_counter() - t0
+    return {
+        "value": n_steps / dt,
+        "unit": "tok/s",
+        "cores": cores,
+        "kind": "port",
+        "sample": f"{n_steps} single-token decode steps (positions 0..{n_steps - 1}: the 8-token prompt through the "
+                  f"single-token path, then greedy steps) of the same seeded Llama-3.2-1B-shaped request, "
+                  f"torch {torch.__version__} bf16 on {cores} threads, {dt:.1f} s",
+    }
+
+
+def main() -> None:
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=1023)
+    ap.add_argument("--warmup", type=int, default=16)
+    ap.add_argument("--seed", type=int, default=0)
+    ap.add_argument("--prompt-len", type=int, default=8)
+    ap.add_argument("--cpu-steps", type=int, default=10)
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    args = ap.parse_args()
+    if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
+        raise SystemExit("bench.py: this path runs on exactly one GPU (batch-1 decode does not shard; "
+                         "see DESIGN.md 'More than one GPU'); run with --gpus 1")
+
+    import torch
+
+    from __graft_entry__ import LIBRARY, build_library, load_package
+
+    if not torch.cuda.is_available():
+        raise SystemExit("bench.py needs a GPU")
+    if not LIBRARY.is_file():
+        build_library()
+    load_package()
+    from qimeng_megakernel_amd import decode, synthetic
+    from qimeng_megakernel_amd.decode_schedule import mk_kernel
+    from qimeng_megakernel_amd.decode_schedule.model_config import LLAMA_3_2_1B, LlamaConfig
+
+    shape = LLAMA_3_2_1B
+    LlamaConfig.set_shape(shape)
+    device = torch.device("cuda:0")
+    torch.cuda.set_device(device)
+    new_tokens = args.steps + 1
+    kv_capacity = args.prompt_len + new_tokens
+    weights = synthetic.random_weights(shape, args.seed, max_positions=kv_capacity)
+    prompt = synthetic.random_prompt(shape, args.seed, args.prompt_len)
+    globs = synthetic.build_globals(weights, shape, kv_capacity, device)
+    mk = mk_kernel.get_mk()
+
+    if args.warmup > 0:
+        decode.decode(globs, prompt, min(args.warmup + 1, new_tokens), mk=mk, decode_time=False)
+    globs.k_cache.zero_(); globs.v_cache.zero_()
+    torch.cuda.synchronize(device)
+    out = decode.decode(globs, prompt, new_tokens, mk=mk, decode_time=True)
+    torch.cuda.synchronize(device)
+    t = out["timing"]
+    tokens = out["new_tokens"][0].tolist()
+
+    golden = ROOT / "tests" / "golden" / "llama1b_seed0.json"
+    match = None
+    if args.seed == 0 and args.prompt_len == 8 and golden.is_file():
+        want = json.loads(golden.read_text())["tokens"]
+        n = min(len(want), len(tokens))
+        match = next((i for i in range(n) if tokens[i] != want[i]), n)
+
+    ctx_first, ctx_last = args.prompt_len + 1, args.prompt_len + args.steps
+    achieved = t["achieved_GBps"]
+    line = {
+        "metric": "kernel_tok_s",
+        "value": t["kernel_tok_s"],
+        "unit": "tok/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": t["kernel_ms_per_step"],
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "bf16",
+        "data": "synthetic",
+        "config": {
+            "workload": f"Llama-3.2-1B-shaped batch-1 greedy decode, {args.prompt_len}-token prompt, "
+                        f"{new_tokens} new tokens (context {ctx_first}..{ctx_last}), seeded random-init bf16 weights",
+            "layers": shape.num_hidden_layers, "hidden": shape.hidden_size, "ffn": shape.intermediate_size,
+            "q_heads": shape.num_attention_heads, "kv_heads": shape.num_key_value_heads, "head_dim": shape.head_dim,
+            "vocab": shape.vocab_size, "batch": 1, "seed": args.seed,
+            "queues": int(globs.instructions.shape[0]), "instructions_per_queue": int(globs.instructions.shape[1]),
+        },
+        "tok_s": t["effective_tok_s_wall"],
+        "tok_s_gpu": t["effective_tok_s_gpu"],
+        "kernel_tok_s": t["kernel_tok_s"],
+        "golden_token_prefix_match": match,
+        "roofline": {
+            "bound": "hbm",
+            "achieved": achieved,
+            "peak": HBM_PEAK_GBPS,
+            "unit": "GB/s",
+            "frac": achieved / HBM_PEAK_GBPS,
+            "traffic": None,
+            "bytes_per_launch_avg": t["algorithmic_bytes"] / max(args.steps, 1),
+            "kernel": "decode_megakernel<Llama1B>",
+        },
+    }
+    if not args.no_cpu_baseline:
+        cores = min(os.cpu_count() or 1, 16)
+        line["cpu_baseline"] = cpu_baseline(shape, weights, prompt, args.cpu_steps, cores)
+    print(json.dumps(line))
+
+
+if __name__ == "__main__":
+    main()

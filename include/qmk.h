@@ -1,0 +1,153 @@
+/*
+ * qmk.h — C ABI of the gfx950 decode megakernel library (libqmk_hip.so).
+ *
+ * The library is the drop-in for the reference's per-route pybind module: one
+ * launch executes a host-built instruction tensor (32 int32 words per
+ * instruction, one queue per workgroup) over the caller's weight, KV-cache and
+ * scratch tensors.  All pointers are raw DEVICE pointers owned by the caller;
+ * the library allocates nothing, keeps no reference after the call returns and
+ * launches asynchronously on the stream it is given.
+ *
+ * Reference interfaces each entry point stands in for (paths under
+ * qimeng_megakernel/models/LLM/llama/llama3_2__1b/A100/single_batch/):
+ *   qmk_decode_step   <- void mk(22 x const torch::Tensor&, int pos_id,
+ *                        float attn_scale, float rms_norm_eps)
+ *                        decode_kernel/mk.h:4-30, launcher decode_kernel/mk.cu:97-198,
+ *                        python binding decode_kernel/pybind.cpp:8-39,
+ *                        call site decode_schedule/mk_kernel.py:56-94
+ *   qmk_query         <- KernelConfig (NUM_SMS, NUM_THREADS, SHARED_MEMORY_SIZE,
+ *                        INSTRUCTION_WIDTH) decode_kernel/kernel_config.cuh:6-14
+ *   qmk_status_*      <- the reference only printf()s launch errors
+ *                        (decode_kernel/mk.cu:185-197) and traps on bad opcodes
+ *                        (mk.cu:82-90); here both become return codes.
+ */
+#ifndef QMK_H_
+#define QMK_H_
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define QMK_ABI_VERSION 1
+#define QMK_INSTRUCTION_WORDS 32
+
+/* Return / status codes. 0 is success; everything else is an error. */
+enum {
+  QMK_OK = 0,
+  QMK_ERR_NULL_ARG = 1,        /* args or a required pointer is NULL            */
+  QMK_ERR_ABI = 2,             /* args->struct_size does not match this library */
+  QMK_ERR_SHAPE = 3,           /* a dimension is out of the supported range     */
+  QMK_ERR_POSITION = 4,        /* pos_id outside the KV cache / RoPE table      */
+  QMK_ERR_TOO_MANY_QUEUES = 5, /* more queues than co-resident workgroups       */
+  QMK_ERR_NO_DEVICE = 6,       /* no gfx950 device / HIP runtime error          */
+  QMK_ERR_LAUNCH = 7,          /* hipLaunchKernel failed                        */
+  QMK_ERR_MODEL = 8,           /* unknown model id                              */
+  /* device-side (reported through qmk_status_fetch) */
+  QMK_DEV_BAD_OPCODE = 32,     /* opcode outside 0..7                           */
+  QMK_DEV_BAD_OPERAND = 33,    /* an operand would index out of bounds          */
+  QMK_DEV_WAIT_TIMEOUT = 34    /* a counter never reached its expected value    */
+};
+
+/* Model shapes compiled into the library. */
+enum {
+  QMK_MODEL_LLAMA_3_2_1B = 0   /* H 2048, F 8192, 32 q / 8 kv heads, d 64 */
+};
+
+/* qmk_query selectors. */
+enum {
+  QMK_QUERY_ABI_VERSION = 0,
+  QMK_QUERY_CU_COUNT = 1,          /* compute units of the current device        */
+  QMK_QUERY_THREADS = 2,           /* threads per workgroup                      */
+  QMK_QUERY_LDS_BYTES = 3,         /* static LDS per workgroup                   */
+  QMK_QUERY_MAX_QUEUES = 4,        /* largest co-resident grid on this device    */
+  QMK_QUERY_INSTRUCTION_WORDS = 5,
+  QMK_QUERY_MAX_PARTIALS = 6       /* largest split-KV fan-out the kernel merges */
+};
+
+/* Flags. */
+#define QMK_FLAG_KEEP_BARRIERS 1u  /* leave the final counter values in `barriers`
+                                      (the reference's behaviour); by default the
+                                      last workgroup to retire clears them so the
+                                      host needs no barriers.zero_() per step.   */
+
+/*
+ * One decode step.  Tensor order and meaning follow mk(...) of the reference
+ * (decode_kernel/mk.h:4-30).  "bf16" is the raw 16-bit pattern.
+ */
+typedef struct QmkArgs {
+  uint32_t struct_size;            /* = sizeof(QmkArgs)                           */
+  uint32_t model;                  /* QMK_MODEL_*                                 */
+  uint32_t flags;                  /* QMK_FLAG_*                                  */
+  uint32_t spin_limit;             /* counter polls before QMK_DEV_WAIT_TIMEOUT; 0 = default */
+
+  const int32_t* instructions;     /* int32 [num_queues, num_insts, 32]           */
+  void* hidden_states;             /* bf16 [H]            in/out residual stream  */
+  void* q_post_rope;               /* bf16 [Hq*D]                                 */
+  void* k_cache;                   /* bf16 [L, 1, max_seq_len, Hkv, D]            */
+  void* v_cache;                   /* bf16 [L, 1, max_seq_len, Hkv, D]            */
+  void* attn_out;                  /* bf16 [Hq*D]                                 */
+  float* attn_lse_intermediates;   /* f32  [Hq, max_splits]      log2 domain      */
+  float* attn_out_intermediates;   /* f32  [Hq, max_splits, D]                    */
+  void* silu_out;                  /* bf16 [F]                                    */
+  void* logits;                    /* bf16 [vocab_size]                           */
+  const void* attn_norm_weights;   /* bf16 [L, H]                                 */
+  const void* qkv_weights;         /* bf16 [L, (Hq+2Hkv)*D, H]                    */
+  const float* rope_cos;           /* f32  [rope_rows, D]  pair-interleaved       */
+  const float* rope_sin;           /* f32  [rope_rows, D]                         */
+  const void* o_proj_weights;      /* bf16 [L, H, H]                              */
+  const void* mlp_norm_weights;    /* bf16 [L, H]                                 */
+  const void* up_proj_weights;     /* bf16 [L, F, H]                              */
+  const void* gate_proj_weights;   /* bf16 [L, F, H]                              */
+  const void* down_proj_weights;   /* bf16 [L, H, F]                              */
+  const void* lm_head_norm_weights;/* bf16 [H]                                    */
+  const void* lm_head_weights;     /* bf16 [vocab_size, H]                        */
+  int32_t* barriers;               /* int32 [num_layers, num_layer_barriers, barrier_slots] */
+
+  int32_t num_queues;              /* instructions.size(0) = workgroups launched  */
+  int32_t num_insts;               /* instructions.size(1)                        */
+  int32_t num_layers;              /* barriers.size(0)                            */
+  int32_t num_layer_barriers;      /* barriers.size(1)  (>= 8)                    */
+  int32_t barrier_slots;           /* barriers.size(2)  (>= Hq + 2*Hkv)           */
+  int32_t max_seq_len;             /* k_cache.size(2)                             */
+  int32_t max_splits;              /* attn_lse_intermediates.size(1)              */
+  int32_t vocab_size;              /* logits.size(0)                              */
+  int32_t rope_rows;               /* rope_cos.size(0)                            */
+  int32_t pos_id;                  /* index of the token being decoded            */
+  float attn_scale;                /* 1/sqrt(D)                                   */
+  float rms_norm_eps;
+
+  /* Final counter values implied by the scheduler's tile geometry.  0 selects
+   * the reference's (16-row tiles, 2048-wide K slices): 4, 128, 128, 512.       */
+  int32_t qkv_blocks_per_head;     /* D / qkv_tile_n                              */
+  int32_t oproj_blocks;            /* H / oproj_tile_n                            */
+  int32_t upgate_blocks_per_bucket;/* split_k / upgate_tile_n                     */
+  int32_t down_arrivals;           /* (H / down_tile_n) * (F / split_k)           */
+
+  uint64_t* timeline;              /* optional u64 [num_queues, num_insts, 4] device
+                                      buffer: start / after-wait / end timestamps
+                                      (100 MHz ticks) + opcode per instruction; NULL = off */
+  void* stream;                    /* hipStream_t; NULL = the null stream         */
+} QmkArgs;
+
+/* Launch one decode step asynchronously on args->stream.  Returns QMK_OK or a
+ * host-side QMK_ERR_*.  Device-side errors surface through qmk_status_fetch. */
+int qmk_decode_step(const QmkArgs* args);
+
+/* Device/library properties (QMK_QUERY_*); negative on error. */
+int qmk_query(int what);
+
+/* Synchronise `stream`, then return and clear the first device-side error the
+ * kernels on the current device recorded since the last fetch (QMK_OK if none).
+ * detail[0..3], when non-NULL, receive {workgroup, instruction index, opcode,
+ * operand/slot}. */
+int qmk_status_fetch(void* stream, int32_t detail[4]);
+
+/* Static, human-readable name of a return/status code. */
+const char* qmk_error_string(int code);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* QMK_H_ */

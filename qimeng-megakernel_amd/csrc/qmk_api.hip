@@ -1,0 +1,238 @@
+// The persistent decode megakernel for gfx950 and its C ABI (include/qmk.h).
+//
+// One workgroup per instruction queue walks its queue in order; each
+// instruction is one fused transformer op on a slice of the output.  Ordering
+// across workgroups uses monotone global counters (release/acquire at agent
+// scope).  The grid must be co-resident — the launcher checks it — and every
+// wait has a poll budget, so the grid drains even if a producer is missing.
+//
+// Replaces mk_kernel / mk of the reference
+// (qimeng_megakernel/models/LLM/llama/llama3_2__1b/A100/single_batch/decode_kernel/mk.cu:29-198).
+#include <hip/hip_runtime.h>
+
+#include <mutex>
+
+#include "qmk.h"
+#include "qmk_ops.h"
+
+namespace qmk {
+
+constexpr int kStatusWords = 8;
+constexpr int kMaxDevices = 16;
+
+// {code, workgroup, instruction, opcode, operand}; written only on errors.
+__device__ int32_t g_status[kStatusWords];
+
+template <class M>
+__global__ __launch_bounds__(kThreads, 1) void decode_megakernel(const Params p) {
+  __shared__ Smem<M> s;
+  if (threadIdx.x < 8) s.ctl[threadIdx.x] = 0;
+  __syncthreads();
+
+  const int32_t* queue = p.instructions + static_cast<size_t>(blockIdx.x) * p.num_insts * kInstWords;
+  bool ok = true;
+  for (int i = 0; i < p.num_insts && ok; ++i) {
+    if (threadIdx.x < kInstWords) s.inst[threadIdx.x] = queue[i * kInstWords + threadIdx.x];
+    __syncthreads();
+    const int opcode = s.inst[0];
+    const Ctx c{i, opcode};
+    unsigned long long t_start = 0;
+    if (p.timeline != nullptr && threadIdx.x == 0) {
+      t_start = wall_clock64();
+    }
+    switch (opcode) {
+      case OP_NOOP: break;
+      case OP_RMS_QKV_ROPE: ok = op_rms_qkv_rope<M>(p, s, c); break;
+      case OP_ATTN_SPLITKV: ok = op_attn_splitkv<M>(p, s, c); break;
+      case OP_ATTN_REDUCE: ok = op_attn_reduce<M>(p, s, c); break;
+      case OP_OPROJ_RESIDUAL: ok = op_oproj_residual<M>(p, s, c); break;
+      case OP_RMS_UPGATE_SILU: ok = op_rms_upgate_silu<M>(p, s, c); break;
+      case OP_DOWN_RESIDUAL: ok = op_down_residual<M>(p, s, c); break;
+      case OP_RMS_LMHEAD: ok = op_rms_lmhead<M>(p, s, c); break;
+      default:
+        if (threadIdx.x == 0) report_error(p, QMK_DEV_BAD_OPCODE, i, opcode, 0);
+        ok = false;
+        break;
+    }
+    if (p.timeline != nullptr && threadIdx.x == 0) {
+      uint64_t* rec = p.timeline + (static_cast<size_t>(blockIdx.x) * p.num_insts + i) * 4;
+      rec[0] = t_start;
+      rec[1] = s.ctl[2] ? s.t_wait : t_start;
+      rec[2] = wall_clock64();
+      rec[3] = static_cast<uint64_t>(opcode) | (static_cast<uint64_t>(static_cast<uint32_t>(s.inst[1])) << 8);
+      s.ctl[2] = 0;
+    }
+    __syncthreads();  // s.inst and s.x are reused by the next instruction
+  }
+  if (!ok || (p.flags & QMK_FLAG_KEEP_BARRIERS)) return;
+
+  // Retire.  The workgroup that arrives last owns the counters alone (every
+  // other queue is finished, so nobody polls any more) and clears them for the
+  // next step.  The arrival counter is the last word of layer 0's last row.
+  release_stores();  // our publishing atomics have landed before we say we are done
+  __syncthreads();
+  int32_t* done = counter_ptr(p, 0, p.num_layer_barriers - 1, p.barrier_slots - 1);
+  if (threadIdx.x == 0) {
+    const int prev = __hip_atomic_fetch_add(done, 1, __ATOMIC_ACQ_REL, __HIP_MEMORY_SCOPE_AGENT);
+    s.ctl[1] = (prev == static_cast<int>(gridDim.x) - 1);
+  }
+  __syncthreads();
+  if (s.ctl[1]) {
+    const int total = p.num_layers * p.num_layer_barriers * p.barrier_slots;
+    for (int i = threadIdx.x; i < total; i += kThreads)
+      __hip_atomic_store(p.barriers + i, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  }
+}
+
+struct DeviceInfo {
+  bool ready = false;
+  int cu_count = 0;
+  int max_queues = 0;
+  int32_t* status = nullptr;
+};
+DeviceInfo g_devices[kMaxDevices];
+std::mutex g_mutex;
+
+int device_info(DeviceInfo** out) {
+  int dev = -1;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) return QMK_ERR_NO_DEVICE;
+  std::lock_guard<std::mutex> lock(g_mutex);
+  DeviceInfo& d = g_devices[dev];
+  if (!d.ready) {
+    hipDeviceProp_t prop;
+    if (hipGetDeviceProperties(&prop, dev) != hipSuccess) return QMK_ERR_NO_DEVICE;
+    int per_cu = 0;
+    if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, decode_megakernel<Llama1B>, kThreads, 0) != hipSuccess)
+      return QMK_ERR_NO_DEVICE;
+    void* sym = nullptr;
+    if (hipGetSymbolAddress(&sym, HIP_SYMBOL(g_status)) != hipSuccess) return QMK_ERR_NO_DEVICE;
+    if (hipMemset(sym, 0, sizeof(int32_t) * kStatusWords) != hipSuccess) return QMK_ERR_NO_DEVICE;
+    d.cu_count = prop.multiProcessorCount;
+    d.max_queues = per_cu * prop.multiProcessorCount;
+    d.status = static_cast<int32_t*>(sym);
+    d.ready = true;
+  }
+  *out = &d;
+  return QMK_OK;
+}
+
+}  // namespace qmk
+
+using namespace qmk;
+
+extern "C" int qmk_decode_step(const QmkArgs* a) {
+  if (a == nullptr) return QMK_ERR_NULL_ARG;
+  if (a->struct_size != sizeof(QmkArgs)) return QMK_ERR_ABI;
+  if (a->model != QMK_MODEL_LLAMA_3_2_1B) return QMK_ERR_MODEL;
+  using M = Llama1B;
+  const void* required[] = {a->instructions, a->hidden_states, a->q_post_rope, a->k_cache, a->v_cache, a->attn_out,
+                            a->attn_lse_intermediates, a->attn_out_intermediates, a->silu_out, a->logits,
+                            a->attn_norm_weights, a->qkv_weights, a->rope_cos, a->rope_sin, a->o_proj_weights,
+                            a->mlp_norm_weights, a->up_proj_weights, a->gate_proj_weights, a->down_proj_weights,
+                            a->lm_head_norm_weights, a->lm_head_weights, a->barriers};
+  for (const void* ptr : required)
+    if (ptr == nullptr) return QMK_ERR_NULL_ARG;
+  if (a->num_queues < 1 || a->num_insts < 0 || a->num_layers < 1 || a->num_layer_barriers < 8 ||
+      a->barrier_slots < M::NQ + 2 * M::NKV || a->max_seq_len < 1 || a->max_splits < 1 || a->vocab_size < 1 ||
+      a->rope_rows < 1)
+    return QMK_ERR_SHAPE;
+  if (a->pos_id < 0 || a->pos_id >= a->max_seq_len || a->pos_id >= a->rope_rows) return QMK_ERR_POSITION;
+
+  DeviceInfo* dev = nullptr;
+  if (int rc = device_info(&dev); rc != QMK_OK) return rc;
+  if (a->num_queues > dev->max_queues) return QMK_ERR_TOO_MANY_QUEUES;
+  if (a->num_insts == 0) return QMK_OK;
+
+  Params p{};
+  p.instructions = a->instructions;
+  p.hidden = static_cast<u16*>(a->hidden_states);
+  p.q_post_rope = static_cast<u16*>(a->q_post_rope);
+  p.k_cache = static_cast<u16*>(a->k_cache);
+  p.v_cache = static_cast<u16*>(a->v_cache);
+  p.attn_out = static_cast<u16*>(a->attn_out);
+  p.attn_lse = a->attn_lse_intermediates;
+  p.attn_partial = a->attn_out_intermediates;
+  p.silu_out = static_cast<u16*>(a->silu_out);
+  p.logits = static_cast<u16*>(a->logits);
+  p.attn_norm = static_cast<const u16*>(a->attn_norm_weights);
+  p.qkv_w = static_cast<const u16*>(a->qkv_weights);
+  p.rope_cos = a->rope_cos;
+  p.rope_sin = a->rope_sin;
+  p.o_w = static_cast<const u16*>(a->o_proj_weights);
+  p.mlp_norm = static_cast<const u16*>(a->mlp_norm_weights);
+  p.up_w = static_cast<const u16*>(a->up_proj_weights);
+  p.gate_w = static_cast<const u16*>(a->gate_proj_weights);
+  p.down_w = static_cast<const u16*>(a->down_proj_weights);
+  p.lm_norm = static_cast<const u16*>(a->lm_head_norm_weights);
+  p.lm_w = static_cast<const u16*>(a->lm_head_weights);
+  p.barriers = a->barriers;
+  p.timeline = a->timeline;
+  p.status = dev->status;
+  p.num_insts = a->num_insts;
+  p.num_layers = a->num_layers;
+  p.num_layer_barriers = a->num_layer_barriers;
+  p.barrier_slots = a->barrier_slots;
+  p.max_seq_len = a->max_seq_len;
+  p.max_splits = a->max_splits;
+  p.vocab_size = a->vocab_size;
+  p.pos_id = a->pos_id;
+  p.attn_scale = a->attn_scale;
+  p.rms_norm_eps = a->rms_norm_eps;
+  // Reference geometry: 16-row tiles everywhere, down projection in 2048-wide K slices.
+  p.qkv_blocks_per_head = a->qkv_blocks_per_head > 0 ? a->qkv_blocks_per_head : M::D / 16;
+  p.oproj_blocks = a->oproj_blocks > 0 ? a->oproj_blocks : M::H / 16;
+  p.upgate_blocks_per_bucket = a->upgate_blocks_per_bucket > 0 ? a->upgate_blocks_per_bucket : 2048 / 16;
+  p.down_arrivals = a->down_arrivals > 0 ? a->down_arrivals : (M::H / 16) * (M::F / 2048);
+  p.spin_limit = a->spin_limit > 0 ? a->spin_limit : kDefaultSpinLimit;
+  p.flags = a->flags;
+
+  hipLaunchKernelGGL(decode_megakernel<M>, dim3(a->num_queues), dim3(kThreads), 0,
+                     static_cast<hipStream_t>(a->stream), p);
+  return hipGetLastError() == hipSuccess ? QMK_OK : QMK_ERR_LAUNCH;
+}
+
+extern "C" int qmk_query(int what) {
+  switch (what) {
+    case QMK_QUERY_ABI_VERSION: return QMK_ABI_VERSION;
+    case QMK_QUERY_THREADS: return kThreads;
+    case QMK_QUERY_LDS_BYTES: return static_cast<int>(sizeof(Smem<Llama1B>));
+    case QMK_QUERY_INSTRUCTION_WORDS: return kInstWords;
+    case QMK_QUERY_MAX_PARTIALS: return kMaxPartials;
+    default: break;
+  }
+  DeviceInfo* dev = nullptr;
+  if (device_info(&dev) != QMK_OK) return -QMK_ERR_NO_DEVICE;
+  if (what == QMK_QUERY_CU_COUNT) return dev->cu_count;
+  if (what == QMK_QUERY_MAX_QUEUES) return dev->max_queues;
+  return -QMK_ERR_SHAPE;
+}
+
+extern "C" int qmk_status_fetch(void* stream, int32_t detail[4]) {
+  DeviceInfo* dev = nullptr;
+  if (int rc = device_info(&dev); rc != QMK_OK) return rc;
+  if (hipStreamSynchronize(static_cast<hipStream_t>(stream)) != hipSuccess) return QMK_ERR_NO_DEVICE;
+  int32_t host[kStatusWords] = {0};
+  if (hipMemcpy(host, dev->status, sizeof(host), hipMemcpyDeviceToHost) != hipSuccess) return QMK_ERR_NO_DEVICE;
+  if (detail != nullptr)
+    for (int i = 0; i < 4; ++i) detail[i] = host[1 + i];
+  if (host[0] != 0 && hipMemset(dev->status, 0, sizeof(host)) != hipSuccess) return QMK_ERR_NO_DEVICE;
+  return host[0];
+}
+
+extern "C" const char* qmk_error_string(int code) {
+  switch (code) {
+    case QMK_OK: return "ok";
+    case QMK_ERR_NULL_ARG: return "null argument";
+    case QMK_ERR_ABI: return "QmkArgs.struct_size does not match the library";
+    case QMK_ERR_SHAPE: return "dimension out of range";
+    case QMK_ERR_POSITION: return "pos_id outside the KV cache or RoPE table";
+    case QMK_ERR_TOO_MANY_QUEUES: return "more instruction queues than co-resident workgroups";
+    case QMK_ERR_NO_DEVICE: return "no usable HIP device";
+    case QMK_ERR_LAUNCH: return "kernel launch failed";
+    case QMK_ERR_MODEL: return "unknown model id";
+    case QMK_DEV_BAD_OPCODE: return "device: opcode outside 0..7";
+    case QMK_DEV_BAD_OPERAND: return "device: instruction operand out of bounds";
+    case QMK_DEV_WAIT_TIMEOUT: return "device: counter wait ran out of polls";
+    default: return "unknown code";
+  }
+}

@@ -1,0 +1,179 @@
+// Device-side building blocks of the gfx950 decode megakernel: bf16 rounding,
+// wave/workgroup reductions, the inter-workgroup counter protocol and the
+// row-streaming GEMV primitives.  Wave size is 64 throughout.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "qmk.h"
+
+namespace qmk {
+
+constexpr int kThreads = 512;            // one workgroup per CU, 8 waves, 2 per SIMD
+constexpr int kWaveSize = 64;
+constexpr int kWaves = kThreads / kWaveSize;
+constexpr int kInstWords = QMK_INSTRUCTION_WORDS;
+constexpr int kMaxPartials = kInstWords - 7;   // reduction list capacity of one slot
+constexpr uint32_t kDefaultSpinLimit = 1u << 22;
+
+using u16 = uint16_t;
+typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
+typedef uint32_t v4u __attribute__((ext_vector_type(4)));  // 16 bytes = 8 bf16
+
+// Everything a workgroup needs; passed to the kernel by value.
+struct Params {
+  const int32_t* instructions;
+  u16* hidden;
+  u16* q_post_rope;
+  u16* k_cache;
+  u16* v_cache;
+  u16* attn_out;
+  float* attn_lse;
+  float* attn_partial;
+  u16* silu_out;
+  u16* logits;
+  const u16* attn_norm;
+  const u16* qkv_w;
+  const float* rope_cos;
+  const float* rope_sin;
+  const u16* o_w;
+  const u16* mlp_norm;
+  const u16* up_w;
+  const u16* gate_w;
+  const u16* down_w;
+  const u16* lm_norm;
+  const u16* lm_w;
+  int32_t* barriers;
+  uint64_t* timeline;
+  int32_t* status;      // device status words: {code, workgroup, inst, opcode, operand}
+  int32_t num_insts;
+  int32_t num_layers;
+  int32_t num_layer_barriers;
+  int32_t barrier_slots;
+  int32_t max_seq_len;
+  int32_t max_splits;
+  int32_t vocab_size;
+  int32_t pos_id;
+  float attn_scale;
+  float rms_norm_eps;
+  int32_t qkv_blocks_per_head;
+  int32_t oproj_blocks;
+  int32_t upgate_blocks_per_bucket;
+  int32_t down_arrivals;
+  uint32_t spin_limit;
+  uint32_t flags;
+};
+
+// ---------------------------------------------------------------- bf16 ----
+__device__ __forceinline__ float bf2f(u16 v) { return __uint_as_float(static_cast<uint32_t>(v) << 16); }
+
+// Round-to-nearest-even, the rounding torch applies on .to(bfloat16).
+__device__ __forceinline__ u16 f2bf(float f) {
+  uint32_t u = __float_as_uint(f);
+  if ((u & 0x7fffffffu) > 0x7f800000u) return static_cast<u16>((u >> 16) | 0x40u);  // quiet NaN
+  u += 0x7fffu + ((u >> 16) & 1u);
+  return static_cast<u16>(u >> 16);
+}
+__device__ __forceinline__ float round_bf16(float f) { return bf2f(f2bf(f)); }
+__device__ __forceinline__ float bf_lo(uint32_t w) { return __uint_as_float(w << 16); }
+__device__ __forceinline__ float bf_hi(uint32_t w) { return __uint_as_float(w & 0xffff0000u); }
+
+// 8 bf16 weights . 8 bf16 activations, fp32 accumulate (v_dot2c_f32_bf16).
+__device__ __forceinline__ float dot8(const v4u& w, const v4u& x, float acc) {
+  acc = __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2_t, w.x), __builtin_bit_cast(bf16x2_t, x.x), acc, false);
+  acc = __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2_t, w.y), __builtin_bit_cast(bf16x2_t, x.y), acc, false);
+  acc = __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2_t, w.z), __builtin_bit_cast(bf16x2_t, x.z), acc, false);
+  acc = __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2_t, w.w), __builtin_bit_cast(bf16x2_t, x.w), acc, false);
+  return acc;
+}
+
+// ---------------------------------------------------------- reductions ----
+__device__ __forceinline__ float wave_sum(float v) {
+#pragma unroll
+  for (int m = 32; m >= 1; m >>= 1) v += __shfl_xor(v, m, kWaveSize);
+  return v;
+}
+
+// Sum over the workgroup; `scratch` holds kWaves floats.  All threads get the total.
+__device__ __forceinline__ float block_sum(float v, float* scratch) {
+  v = wave_sum(v);
+  const int lane = threadIdx.x & (kWaveSize - 1), wave = threadIdx.x / kWaveSize;
+  __syncthreads();
+  if (lane == 0) scratch[wave] = v;
+  __syncthreads();
+  float t = 0.f;
+#pragma unroll
+  for (int w = 0; w < kWaves; ++w) t += scratch[w];
+  return t;
+}
+
+// ------------------------------------------------- counters ("barriers") ----
+__device__ __forceinline__ int32_t* counter_ptr(const Params& p, int layer, int row, int slot) {
+  return p.barriers + (static_cast<size_t>(layer) * p.num_layer_barriers + row) * p.barrier_slots + slot;
+}
+
+// Record the first device-side error; later ones are dropped.
+__device__ __forceinline__ void report_error(const Params& p, int code, int inst, int opcode, int operand) {
+  if (atomicCAS(p.status, 0, code) == 0) {
+    p.status[1] = blockIdx.x;
+    p.status[2] = inst;
+    p.status[3] = opcode;
+    p.status[4] = operand;
+  }
+}
+
+// One lane polls one counter until it reaches `expected`.  Returns false when
+// the poll budget runs out (the producer is gone): the caller retires the
+// workgroup so that the grid always drains.
+__device__ __forceinline__ bool poll_counter(const int32_t* ctr, int expected, uint32_t limit) {
+  uint32_t polls = 0;
+  while (__hip_atomic_load(ctr, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) < expected) {
+    if (++polls > limit) return false;
+    __builtin_amdgcn_s_sleep(2);
+  }
+  return true;
+}
+
+// Make every store of this thread visible device-wide; callers follow it with
+// __syncthreads() and one publishing atomic.
+__device__ __forceinline__ void release_stores() { __builtin_amdgcn_fence(__ATOMIC_RELEASE, "agent"); }
+// Drop stale cache lines after the counters were seen complete.
+__device__ __forceinline__ void acquire_loads() { __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent"); }
+
+__device__ __forceinline__ void publish(int32_t* ctr, int amount) {
+  __hip_atomic_fetch_add(ctr, amount, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+
+// ------------------------------------------------------- row streaming ----
+// A wave reads one weight row of CH*512 bf16 as CH fully coalesced 1 KiB loads;
+// lane l owns columns (j*64 + l)*8 .. +7 of chunk j.
+template <int CH>
+struct RowRegs {
+  v4u v[CH];
+};
+
+template <int CH>
+__device__ __forceinline__ void load_row(RowRegs<CH>& r, const u16* row, int lane) {
+  const v4u* p = reinterpret_cast<const v4u*>(row) + lane;
+#pragma unroll
+  for (int j = 0; j < CH; ++j) r.v[j] = __builtin_nontemporal_load(p + j * kWaveSize);
+}
+
+template <int CH>
+__device__ __forceinline__ float dot_row(const RowRegs<CH>& r, const v4u (&x)[CH]) {
+  float a = 0.f;
+#pragma unroll
+  for (int j = 0; j < CH; ++j) a = dot8(r.v[j], x[j], a);
+  return a;
+}
+
+// Lane l's activation chunks from a bf16 vector in LDS (same column ownership as load_row).
+template <int CH>
+__device__ __forceinline__ void load_x_from_lds(v4u (&x)[CH], const u16* lds_vec, int lane) {
+  const v4u* p = reinterpret_cast<const v4u*>(lds_vec) + lane;
+#pragma unroll
+  for (int j = 0; j < CH; ++j) x[j] = p[j * kWaveSize];
+}
+
+}  // namespace qmk

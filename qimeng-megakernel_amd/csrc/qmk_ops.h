@@ -1,0 +1,670 @@
+// The seven decode opcodes as workgroup-wide device functions.
+//
+// Semantics follow the reference's fused PyTorch route, including where it
+// rounds to bf16 (qimeng_megakernel/models/LLM/llama/llama3_2__1b/A100/
+// single_batch/decode_schedule/fused/operations.py:126-321); operand layout
+// and the counter protocol follow its instruction VM
+// (…/decode_schedule/instructions/python_vm.py:109-488).  The file is compiled
+// with -ffp-contract=off: where the fused route rounds between a multiply and
+// an add, so does this code; fused multiply-adds are written explicitly.
+#pragma once
+
+#include "qmk_device.h"
+
+namespace qmk {
+
+struct Llama1B {
+  static constexpr int H = 2048;    // hidden size
+  static constexpr int F = 8192;    // MLP intermediate size
+  static constexpr int D = 64;      // head dim
+  static constexpr int NQ = 32;     // query heads
+  static constexpr int NKV = 8;     // key/value heads
+  static constexpr int GQA = NQ / NKV;
+  static constexpr int QKV = (NQ + 2 * NKV) * D;
+  static constexpr int KV_BLOCK = 16;  // split-KV partition granularity in tokens
+};
+
+template <class M>
+struct Smem {
+  int32_t inst[kInstWords];
+  int32_t ctl[8];                       // [0] abort, [1] last workgroup to retire
+  float red[kWaves];
+  alignas(16) u16 x[M::F];              // activation vector handed to the GEMV lanes
+  float merge[kWaves][M::GQA][M::D + 2];  // per-wave attention state: acc[D], m, l
+  unsigned long long t_wait;            // timeline: when the last counter wait finished
+};
+
+enum Opcode {
+  OP_NOOP = 0,
+  OP_RMS_QKV_ROPE = 1,
+  OP_ATTN_SPLITKV = 2,
+  OP_ATTN_REDUCE = 3,
+  OP_OPROJ_RESIDUAL = 4,
+  OP_RMS_UPGATE_SILU = 5,
+  OP_DOWN_RESIDUAL = 6,
+  OP_RMS_LMHEAD = 7,
+};
+
+// Counter rows: opcode - 1.
+constexpr int ROW_QKV = 0, ROW_SPLITKV = 1, ROW_REDUCE = 2, ROW_OPROJ = 3, ROW_UPGATE = 4, ROW_DOWN = 5;
+
+struct Ctx {
+  int inst_idx;
+  int opcode;
+};
+
+template <class M>
+__device__ __forceinline__ bool bad_operand(const Params& p, Smem<M>& s, const Ctx& c, int operand) {
+  if (threadIdx.x == 0) report_error(p, QMK_DEV_BAD_OPERAND, c.inst_idx, c.opcode, operand);
+  return false;
+}
+
+// Lanes 0..n-1 each poll the counter `ctr_of(i)` up to `expected`; afterwards
+// every thread has acquired.  False (uniformly) when a poll ran out of budget.
+template <class M, class CtrOf>
+__device__ __forceinline__ bool wg_wait(const Params& p, Smem<M>& s, const Ctx& c, int n, CtrOf ctr_of, int expected) {
+  if (threadIdx.x < n) {
+    if (!poll_counter(ctr_of(threadIdx.x), expected, p.spin_limit)) {
+      s.ctl[0] = 1;
+      report_error(p, QMK_DEV_WAIT_TIMEOUT, c.inst_idx, c.opcode, threadIdx.x);
+    }
+  }
+  if (p.timeline != nullptr && threadIdx.x == 0) {
+    s.t_wait = wall_clock64();
+    s.ctl[2] = 1;
+  }
+  __syncthreads();
+  if (s.ctl[0]) return false;
+  acquire_loads();
+  return true;
+}
+
+// RMSNorm of the residual stream into s.x as bf16:
+//   n = bf16(x * rsqrt(mean(x^2) + eps));  y = bf16(w * n)
+// (fused/operations.py:126-131 — two roundings, the product taken on bf16 values).
+template <class M>
+__device__ __forceinline__ void rms_to_lds(const Params& p, Smem<M>& s, const u16* hidden, const u16* weight) {
+  static_assert(M::H == kThreads * 4, "one thread normalises four elements");
+  const int t = threadIdx.x;
+  const uint2 hv = *reinterpret_cast<const uint2*>(hidden + t * 4);
+  const float x0 = bf_lo(hv.x), x1 = bf_hi(hv.x), x2 = bf_lo(hv.y), x3 = bf_hi(hv.y);
+  float ss = __builtin_fmaf(x3, x3, __builtin_fmaf(x2, x2, __builtin_fmaf(x1, x1, x0 * x0)));
+  ss = block_sum(ss, s.red);
+  const float mean = ss / static_cast<float>(M::H);
+  const float rstd = 1.0f / sqrtf(mean + p.rms_norm_eps);
+  const uint2 wv = *reinterpret_cast<const uint2*>(weight + t * 4);
+  const u16 y0 = f2bf(bf_lo(wv.x) * round_bf16(x0 * rstd));
+  const u16 y1 = f2bf(bf_hi(wv.x) * round_bf16(x1 * rstd));
+  const u16 y2 = f2bf(bf_lo(wv.y) * round_bf16(x2 * rstd));
+  const u16 y3 = f2bf(bf_hi(wv.y) * round_bf16(x3 * rstd));
+  uint2 out;
+  out.x = static_cast<uint32_t>(y0) | (static_cast<uint32_t>(y1) << 16);
+  out.y = static_cast<uint32_t>(y2) | (static_cast<uint32_t>(y3) << 16);
+  *reinterpret_cast<uint2*>(s.x + t * 4) = out;
+  __syncthreads();
+}
+
+// Interleaved-pair RoPE on bf16-rounded inputs, evaluated in fp32 with a
+// rounding after every multiply and the add, then rounded to bf16
+// (fused/operations.py:134-148, 173-181).
+__device__ __forceinline__ uint32_t rope_pair(float v0, float v1, const float* cosr, const float* sinr, int d) {
+  const float o0 = v0 * cosr[d] + (-v1) * sinr[d];
+  const float o1 = v1 * cosr[d + 1] + v0 * sinr[d + 1];
+  return static_cast<uint32_t>(f2bf(o0)) | (static_cast<uint32_t>(f2bf(o1)) << 16);
+}
+
+// ===================================================================== 1 ==
+// [1, layer, tile_M, n_start, n_end, tile_M_g, tile_N_g]
+template <class M>
+__device__ bool op_rms_qkv_rope(const Params& p, Smem<M>& s, const Ctx& c) {
+  constexpr int CH = M::H / 512;
+  const int layer = s.inst[1], nstart = s.inst[3], nend = s.inst[4], tile = s.inst[6];
+  const int bph = p.qkv_blocks_per_head;
+  if (layer < 0 || layer >= p.num_layers) return bad_operand(p, s, c, 1);
+  if (tile <= 0 || (tile & 1) || tile * bph != M::D) return bad_operand(p, s, c, 6);
+  if (nstart < 0 || nend < nstart || static_cast<long>(nend) * tile > M::QKV) return bad_operand(p, s, c, 4);
+
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int rs = nstart * tile;
+  const int nunits = (nend - nstart) * tile / 2;
+  const u16* W = p.qkv_w + static_cast<size_t>(layer) * M::QKV * M::H;
+
+  RowRegs<CH> a0, a1, b0, b1;
+  int u = wave;
+  if (u < nunits) {  // in flight while the counter is polled
+    load_row(a0, W + static_cast<size_t>(rs + 2 * u) * M::H, lane);
+    load_row(a1, W + static_cast<size_t>(rs + 2 * u + 1) * M::H, lane);
+  }
+  if (layer > 0) {
+    if (!wg_wait(p, s, c, 1, [&](int) { return counter_ptr(p, layer - 1, ROW_DOWN, 0); }, p.down_arrivals)) return false;
+  }
+  rms_to_lds(p, s, p.hidden, p.attn_norm + static_cast<size_t>(layer) * M::H);
+  v4u x[CH];
+  load_x_from_lds(x, s.x, lane);
+
+  const float* cosr = p.rope_cos + static_cast<size_t>(p.pos_id) * M::D;
+  const float* sinr = p.rope_sin + static_cast<size_t>(p.pos_id) * M::D;
+  const size_t kv_row = (static_cast<size_t>(layer) * p.max_seq_len + p.pos_id) * (M::NKV * M::D);
+
+  auto finish = [&](int unit, float s0, float s1) {
+    if (lane != 0) return;
+    const int r = rs + 2 * unit;
+    const float v0 = round_bf16(s0), v1 = round_bf16(s1);  // the GEMV result is bf16 before RoPE
+    if (r < M::NQ * M::D) {
+      *reinterpret_cast<uint32_t*>(p.q_post_rope + r) = rope_pair(v0, v1, cosr, sinr, r % M::D);
+    } else if (r < (M::NQ + M::NKV) * M::D) {
+      const int i = r - M::NQ * M::D;
+      *reinterpret_cast<uint32_t*>(p.k_cache + kv_row + i) = rope_pair(v0, v1, cosr, sinr, i % M::D);
+    } else {
+      const int i = r - (M::NQ + M::NKV) * M::D;
+      *reinterpret_cast<uint32_t*>(p.v_cache + kv_row + i) =
+          static_cast<uint32_t>(f2bf(v0)) | (static_cast<uint32_t>(f2bf(v1)) << 16);
+    }
+  };
+
+  while (u < nunits) {
+    int un = u + kWaves;
+    if (un < nunits) {
+      load_row(b0, W + static_cast<size_t>(rs + 2 * un) * M::H, lane);
+      load_row(b1, W + static_cast<size_t>(rs + 2 * un + 1) * M::H, lane);
+    }
+    finish(u, wave_sum(dot_row(a0, x)), wave_sum(dot_row(a1, x)));
+    u = un;
+    if (u >= nunits) break;
+    un = u + kWaves;
+    if (un < nunits) {
+      load_row(a0, W + static_cast<size_t>(rs + 2 * un) * M::H, lane);
+      load_row(a1, W + static_cast<size_t>(rs + 2 * un + 1) * M::H, lane);
+    }
+    finish(u, wave_sum(dot_row(b0, x)), wave_sum(dot_row(b1, x)));
+    u = un;
+  }
+
+  release_stores();
+  __syncthreads();
+  // One arrival per tile, on the counter of the head the tile belongs to.
+  if (nend > nstart) {
+    const int slot0 = nstart / bph, slot1 = (nend - 1) / bph;
+    const int slot = slot0 + static_cast<int>(threadIdx.x);
+    if (slot <= slot1) {
+      const int lo = max(nstart, slot * bph), hi = min(nend, (slot + 1) * bph);
+      publish(counter_ptr(p, layer, ROW_QKV, slot), hi - lo);
+    }
+  }
+  return true;
+}
+
+// ===================================================================== 2 ==
+// [2, layer, kv_head, num_partials, partial_idx]
+// Flash-decoding over one contiguous slice of the context for the GQA group of
+// one KV head.  A wave handles 8 tokens per pass: lane group g = lane/8 owns a
+// token, lane c = lane%8 owns dims 8c..8c+7 of K and V.  Every lane group keeps
+// its own running (max, sum, acc) per query head; groups, then waves, are
+// merged once at the end.  Scores live in the log2 domain.
+template <class M>
+__device__ bool op_attn_splitkv(const Params& p, Smem<M>& s, const Ctx& c) {
+  static_assert(M::D == 64 && M::GQA == 4, "lane mapping assumes head_dim 64 and 4 query heads per KV head");
+  const int layer = s.inst[1], kvh = s.inst[2], P = s.inst[3], part = s.inst[4];
+  if (layer < 0 || layer >= p.num_layers) return bad_operand(p, s, c, 1);
+  if (kvh < 0 || kvh >= M::NKV) return bad_operand(p, s, c, 2);
+  if (P < 1 || P > p.max_splits || part < 0 || part >= P) return bad_operand(p, s, c, 3);
+
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int grp = lane >> 3, col = lane & 7;
+
+  if (!wg_wait(p, s, c, M::GQA + 2,
+               [&](int i) {
+                 const int slot = i < M::GQA ? kvh * M::GQA + i : (i == M::GQA ? M::NQ + kvh : M::NQ + M::NKV + kvh);
+                 return counter_ptr(p, layer, ROW_QKV, slot);
+               },
+               p.qkv_blocks_per_head))
+    return false;
+
+  // Context slice of this partial (python_vm.py:391-401).
+  const int seq_len = p.pos_id + 1;
+  const int total_blocks = (seq_len + M::KV_BLOCK - 1) / M::KV_BLOCK;
+  const int bpp = (total_blocks + P - 1) / P;
+  const int t0 = min(part * bpp, total_blocks) * M::KV_BLOCK;
+  const int t1 = min(min((part + 1) * bpp, total_blocks) * M::KV_BLOCK, seq_len);
+
+  // q[h][8]: this lane's dims of the four query heads, pre-scaled into the log2 domain.
+  const float qscale = p.attn_scale * 1.4426950408889634f;
+  float q[M::GQA][8];
+#pragma unroll
+  for (int h = 0; h < M::GQA; ++h) {
+    const v4u qv = *reinterpret_cast<const v4u*>(p.q_post_rope + (kvh * M::GQA + h) * M::D + col * 8);
+    q[h][0] = bf_lo(qv.x) * qscale; q[h][1] = bf_hi(qv.x) * qscale;
+    q[h][2] = bf_lo(qv.y) * qscale; q[h][3] = bf_hi(qv.y) * qscale;
+    q[h][4] = bf_lo(qv.z) * qscale; q[h][5] = bf_hi(qv.z) * qscale;
+    q[h][6] = bf_lo(qv.w) * qscale; q[h][7] = bf_hi(qv.w) * qscale;
+  }
+
+  float m[M::GQA], l[M::GQA], acc[M::GQA][8];
+#pragma unroll
+  for (int h = 0; h < M::GQA; ++h) {
+    m[h] = -INFINITY;
+    l[h] = 0.f;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) acc[h][i] = 0.f;
+  }
+
+  const size_t tok_stride = static_cast<size_t>(M::NKV) * M::D;
+  const size_t base = static_cast<size_t>(layer) * p.max_seq_len * tok_stride + static_cast<size_t>(kvh) * M::D + col * 8;
+  for (int t = t0 + wave * 8 + grp; t < t1; t += kWaves * 8) {
+    const size_t off = base + static_cast<size_t>(t) * tok_stride;
+    const v4u kv = *reinterpret_cast<const v4u*>(p.k_cache + off);
+    const v4u vv = *reinterpret_cast<const v4u*>(p.v_cache + off);
+    const float k[8] = {bf_lo(kv.x), bf_hi(kv.x), bf_lo(kv.y), bf_hi(kv.y), bf_lo(kv.z), bf_hi(kv.z), bf_lo(kv.w), bf_hi(kv.w)};
+    const float v[8] = {bf_lo(vv.x), bf_hi(vv.x), bf_lo(vv.y), bf_hi(vv.y), bf_lo(vv.z), bf_hi(vv.z), bf_lo(vv.w), bf_hi(vv.w)};
+#pragma unroll
+    for (int h = 0; h < M::GQA; ++h) {
+      float sc = 0.f;
+#pragma unroll
+      for (int i = 0; i < 8; ++i) sc = __builtin_fmaf(q[h][i], k[i], sc);
+      // The 8 lanes of a group always take the same branch, so the shuffles stay inside the group.
+      sc += __shfl_xor(sc, 1, kWaveSize);
+      sc += __shfl_xor(sc, 2, kWaveSize);
+      sc += __shfl_xor(sc, 4, kWaveSize);
+      const float mn = fmaxf(m[h], sc);
+      const float alpha = exp2f(m[h] - mn);   // 0 on the first token (m = -inf)
+      const float pr = exp2f(sc - mn);
+      l[h] = __builtin_fmaf(l[h], alpha, pr);
+#pragma unroll
+      for (int i = 0; i < 8; ++i) acc[h][i] = __builtin_fmaf(acc[h][i], alpha, pr * v[i]);
+      m[h] = mn;
+    }
+  }
+
+  // Merge the 8 token groups of the wave (lanes with equal `col`).
+#pragma unroll
+  for (int x = 8; x <= 32; x <<= 1) {
+#pragma unroll
+    for (int h = 0; h < M::GQA; ++h) {
+      const float mo = __shfl_xor(m[h], x, kWaveSize);
+      const float lo = __shfl_xor(l[h], x, kWaveSize);
+      const float mn = fmaxf(m[h], mo);
+      const float a = (m[h] == -INFINITY) ? 0.f : exp2f(m[h] - mn);
+      const float b = (mo == -INFINITY) ? 0.f : exp2f(mo - mn);
+      l[h] = l[h] * a + lo * b;
+#pragma unroll
+      for (int i = 0; i < 8; ++i) {
+        const float ao = __shfl_xor(acc[h][i], x, kWaveSize);
+        acc[h][i] = acc[h][i] * a + ao * b;
+      }
+      m[h] = mn;
+    }
+  }
+  if (grp == 0) {
+#pragma unroll
+    for (int h = 0; h < M::GQA; ++h) {
+#pragma unroll
+      for (int i = 0; i < 8; ++i) s.merge[wave][h][col * 8 + i] = acc[h][i];
+      if (col == 0) {
+        s.merge[wave][h][M::D] = m[h];
+        s.merge[wave][h][M::D + 1] = l[h];
+      }
+    }
+  }
+  __syncthreads();
+
+  // Merge the waves: thread (h, d) of the first 256 finishes one output element.
+  if (threadIdx.x < M::GQA * M::D) {
+    const int h = threadIdx.x / M::D, d = threadIdx.x % M::D;
+    float mx = -INFINITY;
+#pragma unroll
+    for (int w = 0; w < kWaves; ++w) mx = fmaxf(mx, s.merge[w][h][M::D]);
+    float num = 0.f, den = 0.f;
+#pragma unroll
+    for (int w = 0; w < kWaves; ++w) {
+      const float mw = s.merge[w][h][M::D];
+      const float f = (mw == -INFINITY) ? 0.f : exp2f(mw - mx);
+      num = __builtin_fmaf(s.merge[w][h][d], f, num);
+      den = __builtin_fmaf(s.merge[w][h][M::D + 1], f, den);
+    }
+    const int head = kvh * M::GQA + h;
+    const bool empty = !(den > 0.f);
+    // Normalised partial output and log2-sum-exp; an empty slice contributes (0, -inf).
+    p.attn_partial[(static_cast<size_t>(head) * p.max_splits + part) * M::D + d] = empty ? 0.f : num / den;
+    if (d == 0) p.attn_lse[static_cast<size_t>(head) * p.max_splits + part] = empty ? -INFINITY : mx + log2f(den);
+  }
+
+  release_stores();
+  __syncthreads();
+  if (threadIdx.x < M::GQA) publish(counter_ptr(p, layer, ROW_SPLITKV, kvh * M::GQA + threadIdx.x), 1);
+  return true;
+}
+
+// ===================================================================== 3 ==
+// [3, layer, head_start, num_partials, len, list..., is_terminal, output_partial]
+template <class M>
+__device__ bool op_attn_reduce(const Params& p, Smem<M>& s, const Ctx& c) {
+  const int layer = s.inst[1], head0 = s.inst[2], P = s.inst[3], n = s.inst[4];
+  if (layer < 0 || layer >= p.num_layers) return bad_operand(p, s, c, 1);
+  if (head0 < 0 || head0 + M::GQA > M::NQ) return bad_operand(p, s, c, 2);
+  if (n < 1 || n > kMaxPartials || P < 1) return bad_operand(p, s, c, 4);
+  for (int i = 0; i < n; ++i)
+    if (s.inst[5 + i] < 0 || s.inst[5 + i] >= p.max_splits) return bad_operand(p, s, c, 5 + i);
+  const bool terminal = s.inst[5 + n] != 0;
+  const int out_slot = s.inst[6 + n];
+  if (!terminal && (out_slot < 0 || out_slot >= p.max_splits)) return bad_operand(p, s, c, 6 + n);
+
+  if (!wg_wait(p, s, c, M::GQA, [&](int i) { return counter_ptr(p, layer, ROW_SPLITKV, head0 + i); }, P)) return false;
+
+  if (threadIdx.x < M::GQA * M::D) {
+    const int h = head0 + threadIdx.x / M::D, d = threadIdx.x % M::D;
+    const float* lse = p.attn_lse + static_cast<size_t>(h) * p.max_splits;
+    const float* part = p.attn_partial + static_cast<size_t>(h) * p.max_splits * M::D + d;
+    float mx = -INFINITY;
+    for (int i = 0; i < n; ++i) mx = fmaxf(mx, lse[s.inst[5 + i]]);
+    float num = 0.f, den = 0.f;
+    for (int i = 0; i < n; ++i) {
+      const int j = s.inst[5 + i];
+      const float e = lse[j];
+      const float f = (e == -INFINITY) ? 0.f : exp2f(e - mx);
+      num = __builtin_fmaf(part[static_cast<size_t>(j) * M::D], f, num);
+      den += f;
+    }
+    const float o = den > 0.f ? num / den : 0.f;
+    if (terminal) {
+      p.attn_out[h * M::D + d] = f2bf(o);
+    } else {
+      p.attn_partial[(static_cast<size_t>(h) * p.max_splits + out_slot) * M::D + d] = o;
+      if (d == 0) p.attn_lse[static_cast<size_t>(h) * p.max_splits + out_slot] = den > 0.f ? mx + log2f(den) : -INFINITY;
+    }
+  }
+  release_stores();
+  __syncthreads();
+  if (threadIdx.x == 0) publish(counter_ptr(p, layer, ROW_REDUCE, 0), M::GQA);
+  return true;
+}
+
+// ===================================================================== 4 ==
+// [4, layer, tile_M, n_start, n_end, reduction_block, tile_M_g, tile_N_g]
+// hidden[r] = bf16(hidden[r] + bf16(W_o[r] . attn_out))   (operations.py:251-262, 63-68)
+template <class M>
+__device__ bool op_oproj_residual(const Params& p, Smem<M>& s, const Ctx& c) {
+  constexpr int CH = M::H / 512;
+  static_assert(M::NQ * M::D == M::H, "attention output width equals the hidden size");
+  const int layer = s.inst[1], nstart = s.inst[3], nend = s.inst[4], tile = s.inst[7];
+  if (layer < 0 || layer >= p.num_layers) return bad_operand(p, s, c, 1);
+  if (tile <= 0 || (tile & 1)) return bad_operand(p, s, c, 7);
+  if (nstart < 0 || nend < nstart || static_cast<long>(nend) * tile > M::H) return bad_operand(p, s, c, 4);
+
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int rs = nstart * tile;
+  const int nunits = (nend - nstart) * tile / 2;
+  const u16* W = p.o_w + static_cast<size_t>(layer) * M::H * M::H;
+
+  RowRegs<CH> a0, a1, b0, b1;
+  int u = wave;
+  if (u < nunits) {
+    load_row(a0, W + static_cast<size_t>(rs + 2 * u) * M::H, lane);
+    load_row(a1, W + static_cast<size_t>(rs + 2 * u + 1) * M::H, lane);
+  }
+  if (!wg_wait(p, s, c, 1, [&](int) { return counter_ptr(p, layer, ROW_REDUCE, 0); }, M::NQ)) return false;
+
+  v4u x[CH];
+  {
+    const v4u* ap = reinterpret_cast<const v4u*>(p.attn_out) + lane;
+#pragma unroll
+    for (int j = 0; j < CH; ++j) x[j] = ap[j * kWaveSize];
+  }
+
+  auto finish = [&](int unit, float s0, float s1) {
+    if (lane != 0) return;
+    uint32_t* hp = reinterpret_cast<uint32_t*>(p.hidden + rs + 2 * unit);
+    const uint32_t old = *hp;
+    const u16 n0 = f2bf(bf_lo(old) + round_bf16(s0));
+    const u16 n1 = f2bf(bf_hi(old) + round_bf16(s1));
+    *hp = static_cast<uint32_t>(n0) | (static_cast<uint32_t>(n1) << 16);
+  };
+
+  while (u < nunits) {
+    int un = u + kWaves;
+    if (un < nunits) {
+      load_row(b0, W + static_cast<size_t>(rs + 2 * un) * M::H, lane);
+      load_row(b1, W + static_cast<size_t>(rs + 2 * un + 1) * M::H, lane);
+    }
+    finish(u, wave_sum(dot_row(a0, x)), wave_sum(dot_row(a1, x)));
+    u = un;
+    if (u >= nunits) break;
+    un = u + kWaves;
+    if (un < nunits) {
+      load_row(a0, W + static_cast<size_t>(rs + 2 * un) * M::H, lane);
+      load_row(a1, W + static_cast<size_t>(rs + 2 * un + 1) * M::H, lane);
+    }
+    finish(u, wave_sum(dot_row(b0, x)), wave_sum(dot_row(b1, x)));
+    u = un;
+  }
+
+  release_stores();
+  __syncthreads();
+  if (threadIdx.x == 0 && nend > nstart) publish(counter_ptr(p, layer, ROW_OPROJ, 0), nend - nstart);
+  return true;
+}
+
+// ===================================================================== 5 ==
+// [5, layer, tile_M, n, block_0..block_{n-1}, tile_M_g, tile_N_g]
+// up = bf16(W_u y), gate = bf16(W_g y), silu_out = bf16(bf16(silu(gate)) * up)   (operations.py:265-282)
+template <class M>
+__device__ bool op_rms_upgate_silu(const Params& p, Smem<M>& s, const Ctx& c) {
+  constexpr int CH = M::H / 512;
+  const int layer = s.inst[1], n = s.inst[3];
+  if (layer < 0 || layer >= p.num_layers) return bad_operand(p, s, c, 1);
+  if (n < 0 || n > kInstWords - 6) return bad_operand(p, s, c, 3);
+  const int tile = s.inst[5 + n];
+  if (tile <= 0) return bad_operand(p, s, c, 5 + n);
+  const int nblocks_total = M::F / tile;
+  for (int i = 0; i < n; ++i)
+    if (s.inst[4 + i] < 0 || s.inst[4 + i] >= nblocks_total) return bad_operand(p, s, c, 4 + i);
+
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int nunits = n * tile;  // one unit = one output element = an up row and a gate row
+  const u16* Wu = p.up_w + static_cast<size_t>(layer) * M::F * M::H;
+  const u16* Wg = p.gate_w + static_cast<size_t>(layer) * M::F * M::H;
+  auto row_of = [&](int unit) { return s.inst[4 + unit / tile] * tile + unit % tile; };
+
+  RowRegs<CH> a0, a1, b0, b1;
+  int u = wave;
+  if (u < nunits) {
+    const size_t r = row_of(u);
+    load_row(a0, Wu + r * M::H, lane);
+    load_row(a1, Wg + r * M::H, lane);
+  }
+  if (!wg_wait(p, s, c, 1, [&](int) { return counter_ptr(p, layer, ROW_OPROJ, 0); }, p.oproj_blocks)) return false;
+  rms_to_lds(p, s, p.hidden, p.mlp_norm + static_cast<size_t>(layer) * M::H);
+  v4u x[CH];
+  load_x_from_lds(x, s.x, lane);
+
+  auto finish = [&](int unit, float su, float sg) {
+    if (lane != 0) return;
+    const float up = round_bf16(su), gate = round_bf16(sg);
+    const float act = round_bf16(gate / (1.0f + expf(-gate)));
+    p.silu_out[row_of(unit)] = f2bf(act * up);
+  };
+
+  while (u < nunits) {
+    int un = u + kWaves;
+    if (un < nunits) {
+      const size_t r = row_of(un);
+      load_row(b0, Wu + r * M::H, lane);
+      load_row(b1, Wg + r * M::H, lane);
+    }
+    finish(u, wave_sum(dot_row(a0, x)), wave_sum(dot_row(a1, x)));
+    u = un;
+    if (u >= nunits) break;
+    un = u + kWaves;
+    if (un < nunits) {
+      const size_t r = row_of(un);
+      load_row(a0, Wu + r * M::H, lane);
+      load_row(a1, Wg + r * M::H, lane);
+    }
+    finish(u, wave_sum(dot_row(b0, x)), wave_sum(dot_row(b1, x)));
+    u = un;
+  }
+
+  release_stores();
+  __syncthreads();
+  // One arrival per block, on the bucket (= down-projection K slice) it belongs to.
+  if (static_cast<int>(threadIdx.x) < n)
+    publish(counter_ptr(p, layer, ROW_UPGATE, s.inst[4 + threadIdx.x] / p.upgate_blocks_per_bucket), 1);
+  return true;
+}
+
+// ===================================================================== 6 ==
+// bf16 add on one half of a 32-bit word, safe against concurrent adders of
+// other K slices (only needed when the down projection is split along K).
+__device__ __forceinline__ void atomic_add_bf16(u16* addr, float delta) {
+  uint32_t* word = reinterpret_cast<uint32_t*>(reinterpret_cast<uintptr_t>(addr) & ~uintptr_t(3));
+  const bool high = (reinterpret_cast<uintptr_t>(addr) & 2) != 0;
+  uint32_t seen = __hip_atomic_load(word, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  while (true) {
+    const u16 cur = high ? static_cast<u16>(seen >> 16) : static_cast<u16>(seen & 0xffffu);
+    const u16 nxt = f2bf(bf2f(cur) + delta);
+    const uint32_t want = high ? ((seen & 0x0000ffffu) | (static_cast<uint32_t>(nxt) << 16))
+                               : ((seen & 0xffff0000u) | nxt);
+    if (__hip_atomic_compare_exchange_strong(word, &seen, want, __ATOMIC_RELAXED, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT)) break;
+  }
+}
+
+// [6, layer, tile_M, n_start, n_end, split_K_idx, tile_M_g, tile_N_g, split_K_g]
+// hidden[r] = bf16(hidden[r] + bf16(W_d[r, slice] . silu_out[slice]))   (operations.py:285-295;
+// python_vm.py:137-171 for the sliced form).  With one slice this is the fused form exactly.
+template <class M, int G>
+__device__ __forceinline__ void down_rows(const Params& p, Smem<M>& s, const u16* W, int rs, int re, int ks, int kg,
+                                          RowRegs<G>& a, bool a_loaded, bool single_slice) {
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int groups = kg / (512 * G);  // G-chunk groups per row
+  const int nrows = re - rs;
+  // Flattened (row, group) sequence of this wave: row = rs + wave + 8*i, group g.
+  const int total = ((nrows - wave + kWaves - 1) / kWaves) * groups;  // may be <= 0
+  RowRegs<G> b;
+  auto src = [&](int idx) {
+    const int row = rs + wave + (idx / groups) * kWaves;
+    return W + static_cast<size_t>(row) * M::F + ks + (idx % groups) * (512 * G);
+  };
+  auto xs = [&](int idx, v4u (&x)[G]) { load_x_from_lds(x, s.x + (idx % groups) * (512 * G), lane); };
+  float acc = 0.f;
+  auto step = [&](const RowRegs<G>& r, int idx) {
+    v4u x[G];
+    xs(idx, x);
+#pragma unroll
+    for (int j = 0; j < G; ++j) acc = dot8(r.v[j], x[j], acc);
+    if (idx % groups == groups - 1) {
+      const float sum = wave_sum(acc);
+      acc = 0.f;
+      if (lane == 0) {
+        u16* hp = p.hidden + rs + wave + (idx / groups) * kWaves;
+        const float d = round_bf16(sum);
+        if (single_slice) *hp = f2bf(bf2f(*hp) + d);
+        else atomic_add_bf16(hp, d);
+      }
+    }
+  };
+  int i = 0;
+  if (total > 0 && !a_loaded) load_row(a, src(0), lane);
+  while (i < total) {
+    if (i + 1 < total) load_row(b, src(i + 1), lane);
+    step(a, i);
+    ++i;
+    if (i >= total) break;
+    if (i + 1 < total) load_row(a, src(i + 1), lane);
+    step(b, i);
+    ++i;
+  }
+}
+
+template <class M>
+__device__ bool op_down_residual(const Params& p, Smem<M>& s, const Ctx& c) {
+  const int layer = s.inst[1], nstart = s.inst[3], nend = s.inst[4], split = s.inst[5];
+  const int tile = s.inst[7], kg = s.inst[8];
+  if (layer < 0 || layer >= p.num_layers) return bad_operand(p, s, c, 1);
+  if (tile <= 0) return bad_operand(p, s, c, 7);
+  if (nstart < 0 || nend < nstart || static_cast<long>(nend) * tile > M::H) return bad_operand(p, s, c, 4);
+  if (kg <= 0 || kg % 2048 != 0 || kg > M::F) return bad_operand(p, s, c, 8);
+  if (split < 0 || static_cast<long>(split + 1) * kg > M::F) return bad_operand(p, s, c, 5);
+  if (split >= p.barrier_slots) return bad_operand(p, s, c, 5);
+
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int rs = nstart * tile, re = nend * tile, ks = split * kg;
+  const u16* W = p.down_w + static_cast<size_t>(layer) * M::H * M::F;
+  const bool wide = (kg % 4096) == 0;
+
+  RowRegs<8> a8;
+  RowRegs<4> a4;
+  const bool have_row = rs + wave < re;
+  if (have_row) {
+    const u16* first = W + static_cast<size_t>(rs + wave) * M::F + ks;
+    if (wide) load_row(a8, first, lane);
+    else load_row(a4, first, lane);
+  }
+  if (!wg_wait(p, s, c, 1, [&](int) { return counter_ptr(p, layer, ROW_UPGATE, split); }, p.upgate_blocks_per_bucket)) return false;
+
+  // The K slice of silu_out into LDS.
+  for (int i = threadIdx.x; i < kg / 8; i += kThreads)
+    reinterpret_cast<v4u*>(s.x)[i] = reinterpret_cast<const v4u*>(p.silu_out + ks)[i];
+  __syncthreads();
+
+  const bool single = kg == M::F;
+  if (wide) down_rows<M, 8>(p, s, W, rs, re, ks, kg, a8, have_row, single);
+  else down_rows<M, 4>(p, s, W, rs, re, ks, kg, a4, have_row, single);
+
+  release_stores();
+  __syncthreads();
+  if (threadIdx.x == 0 && nend > nstart) publish(counter_ptr(p, layer, ROW_DOWN, 0), nend - nstart);
+  return true;
+}
+
+// ===================================================================== 7 ==
+// [7, start_block, end_block, tile_M_g, tile_N_g]     logits = bf16(W_lm . rms(hidden))
+template <class M>
+__device__ bool op_rms_lmhead(const Params& p, Smem<M>& s, const Ctx& c) {
+  constexpr int CH = M::H / 512;
+  const int bstart = s.inst[1], bend = s.inst[2], tile = s.inst[4];
+  if (tile <= 0 || (tile & 1)) return bad_operand(p, s, c, 4);
+  if (bstart < 0 || bend < bstart || static_cast<long>(bend) * tile > p.vocab_size) return bad_operand(p, s, c, 2);
+  if (p.num_layers < 1) return bad_operand(p, s, c, 0);
+
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int rs = bstart * tile;
+  const int nunits = (bend - bstart) * tile / 2;
+  const u16* W = p.lm_w;
+
+  RowRegs<CH> a0, a1, b0, b1;
+  int u = wave;
+  if (u < nunits) {
+    load_row(a0, W + static_cast<size_t>(rs + 2 * u) * M::H, lane);
+    load_row(a1, W + static_cast<size_t>(rs + 2 * u + 1) * M::H, lane);
+  }
+  if (!wg_wait(p, s, c, 1, [&](int) { return counter_ptr(p, p.num_layers - 1, ROW_DOWN, 0); }, p.down_arrivals)) return false;
+  rms_to_lds(p, s, p.hidden, p.lm_norm);
+  v4u x[CH];
+  load_x_from_lds(x, s.x, lane);
+
+  auto finish = [&](int unit, float s0, float s1) {
+    if (lane != 0) return;
+    *reinterpret_cast<uint32_t*>(p.logits + rs + 2 * unit) =
+        static_cast<uint32_t>(f2bf(s0)) | (static_cast<uint32_t>(f2bf(s1)) << 16);
+  };
+
+  while (u < nunits) {
+    int un = u + kWaves;
+    if (un < nunits) {
+      load_row(b0, W + static_cast<size_t>(rs + 2 * un) * M::H, lane);
+      load_row(b1, W + static_cast<size_t>(rs + 2 * un + 1) * M::H, lane);
+    }
+    finish(u, wave_sum(dot_row(a0, x)), wave_sum(dot_row(a1, x)));
+    u = un;
+    if (u >= nunits) break;
+    un = u + kWaves;
+    if (un < nunits) {
+      load_row(a0, W + static_cast<size_t>(rs + 2 * un) * M::H, lane);
+      load_row(a1, W + static_cast<size_t>(rs + 2 * un + 1) * M::H, lane);
+    }
+    finish(u, wave_sum(dot_row(b0, x)), wave_sum(dot_row(b1, x)));
+    u = un;
+  }
+  return true;  // terminal: nothing waits on the logits inside the kernel
+}
+
+}  // namespace qmk

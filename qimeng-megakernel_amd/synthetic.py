@@ -1,0 +1,132 @@
+"""Seeded random-init weights and ``Globals`` allocation for the decode route.
+
+Stands in for the reference's checkpoint loader and buffer allocation when no
+checkpoint is available:
+
+* weight layout: per-layer matrices stacked ``[L, out, in]``, q/k rows of the
+  QKV matrix pair-interleaved per head (`LLM/llama/preprocess.py:21-83`);
+* RoPE tables: plain-theta ``cos/sin(pos * theta^(-2i/d))`` in fp32, columns
+  pair-interleaved the same way (`LLM/llama/load_weights.py:37-74`);
+* buffers: `…/A100/fused_prefill.py:38-160` (KV cache ``[L,1,S,Hkv,D]``, fp32
+  split-KV workspaces, int32 counters ``[L,10,48]``).
+
+Random weights are drawn on a CPU generator, so a seed names the same model on
+every machine.  A random-init matrix is its own interleaved version in
+distribution, so no row permutation is applied to it.
+"""
+from __future__ import annotations
+
+import dataclasses
+from typing import Any
+
+import torch
+
+from .decode_schedule.globs import Globals
+from .decode_schedule.model_config import DecodeShape, LlamaConfig
+
+BARRIER_ROWS = 10
+WEIGHT_STD = 0.02
+
+
+def interleave_indices(head_dim: int) -> torch.Tensor:
+    """Column order [0, d/2, 1, d/2+1, ...]: rotate-half partners become neighbours."""
+    half = head_dim // 2
+    return torch.stack((torch.arange(half), torch.arange(half) + half), dim=1).reshape(-1)
+
+
+def rope_tables(shape: DecodeShape, max_positions: int) -> tuple[torch.Tensor, torch.Tensor]:
+    """fp32 ``[max_positions, head_dim]`` cos/sin in the pair-interleaved layout."""
+    d = shape.head_dim
+    inv_freq = 1.0 / (shape.rope_theta ** (torch.arange(0, d, 2, dtype=torch.int64).float() / d))
+    freqs = torch.outer(torch.arange(max_positions, dtype=torch.float32), inv_freq)
+    emb = torch.cat((freqs, freqs), dim=-1)
+    idx = interleave_indices(d)
+    return emb.cos()[:, idx].contiguous(), emb.sin()[:, idx].contiguous()
+
+
+def _normal_bf16(gen: torch.Generator, *size: int) -> torch.Tensor:
+    # Drawn layer by layer in fp32, stored as bf16: peak host memory stays at one matrix.
+    return (torch.randn(*size, generator=gen, dtype=torch.float32) * WEIGHT_STD).to(torch.bfloat16)
+
+
+def random_weights(shape: DecodeShape, seed: int, max_positions: int) -> dict[str, torch.Tensor]:
+    """bf16 ~N(0, 0.02) projections and embeddings, unit norm weights, untied LM head (CPU tensors)."""
+    gen = torch.Generator(device="cpu")
+    gen.manual_seed(seed)
+    L, H, F, V = shape.num_hidden_layers, shape.hidden_size, shape.intermediate_size, shape.vocab_size
+    w: dict[str, torch.Tensor] = {}
+    w["embed_tokens"] = _normal_bf16(gen, V, H)
+    w["qkv_weights"] = torch.stack([_normal_bf16(gen, shape.qkv_out_dim, H) for _ in range(L)])
+    w["o_proj_weights"] = torch.stack([_normal_bf16(gen, H, shape.num_attention_heads * shape.head_dim) for _ in range(L)])
+    w["up_proj_weights"] = torch.stack([_normal_bf16(gen, F, H) for _ in range(L)])
+    w["gate_proj_weights"] = torch.stack([_normal_bf16(gen, F, H) for _ in range(L)])
+    w["down_proj_weights"] = torch.stack([_normal_bf16(gen, H, F) for _ in range(L)])
+    w["lm_head_weights"] = _normal_bf16(gen, V, H)
+    w["attn_norm_weights"] = torch.ones(L, H, dtype=torch.bfloat16)
+    w["mlp_norm_weights"] = torch.ones(L, H, dtype=torch.bfloat16)
+    w["lm_head_norm_weights"] = torch.ones(H, dtype=torch.bfloat16)
+    w["rope_cos"], w["rope_sin"] = rope_tables(shape, max_positions)
+    return w
+
+
+def random_prompt(shape: DecodeShape, seed: int, length: int) -> torch.Tensor:
+    gen = torch.Generator(device="cpu")
+    gen.manual_seed(seed + 1_000_003)
+    return torch.randint(0, shape.vocab_size, (length,), generator=gen, dtype=torch.long)
+
+
+def build_globals(
+    weights: dict[str, torch.Tensor],
+    shape: DecodeShape,
+    kv_capacity: int,
+    device: torch.device | str,
+    *,
+    max_partials: int = 32,
+    globals_cls: Any = Globals,
+) -> Any:
+    """Allocate every decode buffer on ``device`` and attach the weights (moved there)."""
+    device = torch.device(device)
+    bf16 = torch.bfloat16
+    L, H = shape.num_hidden_layers, shape.hidden_size
+    nq, nkv, d = shape.num_attention_heads, shape.num_key_value_heads, shape.head_dim
+
+    def zeros(*size: int, dtype: torch.dtype = bf16) -> torch.Tensor:
+        return torch.zeros(*size, dtype=dtype, device=device)
+
+    on_device = {k: v.to(device).contiguous() for k, v in weights.items()}
+    g = globals_cls(
+        position_id=0,
+        barriers=zeros(L, BARRIER_ROWS, shape.num_heads, dtype=torch.int32),
+        k_cache=zeros(L, 1, kv_capacity, nkv, d),
+        v_cache=zeros(L, 1, kv_capacity, nkv, d),
+        hidden_states=zeros(H),
+        q_post_rope=zeros(nq * d),
+        attn_out=zeros(nq * d),
+        attn_out_intermediates=zeros(nq, max_partials, d, dtype=torch.float32),
+        attn_lse_intermediates=zeros(nq, max_partials, dtype=torch.float32),
+        silu_out=zeros(shape.intermediate_size),
+        logits=zeros(shape.vocab_size),
+        **{k: v for k, v in on_device.items() if k != "embed_tokens"},
+    )
+    g.embed_tokens = on_device["embed_tokens"]
+    return g
+
+
+def build_synthetic_globals(
+    shape: DecodeShape | None = None,
+    *,
+    seed: int = 0,
+    kv_capacity: int = 136,
+    device: torch.device | str = "cuda",
+    max_partials: int = 32,
+) -> Any:
+    """Convenience: weights of ``seed`` + buffers; also points ``LlamaConfig`` at ``shape``."""
+    shape = shape or LlamaConfig.shape()
+    LlamaConfig.set_shape(shape)
+    weights = random_weights(shape, seed, max_positions=kv_capacity)
+    return build_globals(weights, shape, kv_capacity, device, max_partials=max_partials)
+
+
+def reduced_shape(num_layers: int = 2, vocab_size: int = 2048, **overrides: Any) -> DecodeShape:
+    """Llama-3.2-1B layer geometry with fewer layers and a small vocabulary (fast CPU checks)."""
+    return dataclasses.replace(LlamaConfig.shape().__class__(), num_hidden_layers=num_layers, vocab_size=vocab_size, **overrides)

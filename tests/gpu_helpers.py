@@ -1,0 +1,53 @@
+"""Helpers shared by the GPU parity tests (imported, not collected)."""
+from __future__ import annotations
+
+import copy
+
+import torch
+
+from pyvm_oracle import Counts, InstructionVM
+from qimeng_megakernel_amd import synthetic
+from qimeng_megakernel_amd.decode_schedule import mk_kernel
+from qimeng_megakernel_amd.decode_schedule.instructions import scheduler as S
+
+MUTABLE = ("hidden_states", "q_post_rope", "attn_out", "silu_out", "logits", "k_cache", "v_cache",
+           "attn_out_intermediates", "attn_lse_intermediates", "barriers")
+
+
+def sync_state(src, dst) -> None:
+    """Copy every mutable buffer of ``src`` onto ``dst`` (across devices)."""
+    for name in MUTABLE:
+        getattr(dst, name).copy_(getattr(src, name))
+    dst.position_id = src.position_id
+
+
+def pair(weights, shape, kv_capacity=96, max_partials=32):
+    cpu = synthetic.build_globals(weights, shape, kv_capacity, "cpu", max_partials=max_partials)
+    gpu = synthetic.build_globals(weights, shape, kv_capacity, "cuda:0", max_partials=max_partials)
+    return cpu, gpu
+
+
+def run_both(cpu, gpu, sched, instructions, *, sm_count=None):
+    """Execute the same instruction list on the CPU VM and on the kernel, counters kept."""
+    vm = InstructionVM(sched.shape, Counts(*sched.expected_counts()))
+    vm.run(cpu, copy.deepcopy(instructions))
+    mk = mk_kernel.get_mk(geometry=sched.geometry, reset_barriers=False)
+    mk_kernel.run_instructions(gpu, copy.deepcopy(instructions), mk=mk, sm_count=sm_count or sched.sm_count)
+    mk.check()
+    return mk
+
+
+def bf16_close(got: torch.Tensor, want: torch.Tensor, *, ulps: float = 1.0, frac: float = 0.02, name: str = "tensor"):
+    """bf16 tensors that come from fp32-accumulated dot products of the same inputs: equal except
+    where the exact value sits next to a rounding boundary; there, at most ``ulps`` bf16 ulps.
+    Tolerance: max |diff| <= ulps * 2^-7 * max(|want|, 2^-6) and at most ``frac`` of elements differ."""
+    got, want = got.detach().float().cpu().reshape(-1), want.detach().float().cpu().reshape(-1)
+    assert torch.isfinite(got).all(), f"{name}: non-finite values"
+    scale = torch.maximum(want.abs(), torch.tensor(2.0 ** -6))
+    ulp = torch.exp2(torch.floor(torch.log2(scale)) - 7)
+    diff = (got - want).abs()
+    worst = float((diff / ulp).max())
+    assert worst <= ulps * 1.001, f"{name}: {worst:.2f} ulps off (allowed {ulps})"
+    off = float((diff > 0).float().mean())
+    assert off <= frac, f"{name}: {off:.4f} of the elements differ (allowed {frac})"
+    return worst, off

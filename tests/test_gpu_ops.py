@@ -1,0 +1,155 @@
+"""Kernel vs sequential VM, one op at a time, with the counters pre-filled.
+
+Mirrors the reference's pyvm_to_megakernel stage
+(`qimeng_megakernel/verifier/LLM/llama/llama3_2__1b/A100/single_batch/pyvm_to_megakernel/`,
+barrier fills per `verifier/common/barrier_fill.py:67-119`): the same instruction
+list runs on the CPU VM and through the C ABI on the GPU; outputs must agree
+within bf16 rounding and the counters must be identical.
+"""
+import dataclasses
+
+import pytest
+import torch
+
+from gpu_helpers import bf16_close, pair, run_both, sync_state
+from qimeng_megakernel_amd import synthetic
+from qimeng_megakernel_amd.decode_schedule.instructions import instruction_defs as D
+from qimeng_megakernel_amd.decode_schedule.instructions import scheduler as S
+from qimeng_megakernel_amd.decode_schedule.model_config import LlamaConfig
+
+pytestmark = pytest.mark.gpu
+
+
+def _sched(shape, which, P=3):
+    if which == "mi355x":
+        return S.mi355x_scheduler(shape, sm_count=256, num_partials=P)
+    return S.DecodeScheduler(shape, D.REFERENCE_GEOMETRY, 108, P)
+
+
+@pytest.fixture()
+def state(small_model):
+    shape, w, _ = small_model
+    LlamaConfig.set_shape(shape)
+    cpu, gpu = pair(w, shape)
+    gen = torch.Generator().manual_seed(21)
+    cpu.hidden_states.copy_((torch.randn(shape.hidden_size, generator=gen) * 0.7).bfloat16())
+    cpu.attn_out.copy_(torch.randn(shape.hidden_size, generator=gen).bfloat16())
+    cpu.silu_out.copy_((torch.randn(shape.intermediate_size, generator=gen) * 0.3).bfloat16())
+    cpu.q_post_rope.copy_(torch.randn(shape.hidden_size, generator=gen).bfloat16())
+    cpu.k_cache.copy_(torch.randn(cpu.k_cache.shape, generator=gen).bfloat16())
+    cpu.v_cache.copy_(torch.randn(cpu.v_cache.shape, generator=gen).bfloat16())
+    cpu.position_id = 41
+    return shape, cpu, gpu
+
+
+@pytest.mark.parametrize("which", ["mi355x", "reference"])
+def test_op_qkv_rope(state, which):
+    shape, cpu, gpu = state
+    sched = _sched(shape, which)
+    sync_state(cpu, gpu)
+    run_both(cpu, gpu, sched, sched.qkvproj(0))
+    bf16_close(gpu.q_post_rope, cpu.q_post_rope, name="q_post_rope")
+    bf16_close(gpu.k_cache[0, 0, 41], cpu.k_cache[0, 0, 41], name="k row")
+    bf16_close(gpu.v_cache[0, 0, 41], cpu.v_cache[0, 0, 41], name="v row")
+    # only the row of this position was touched
+    assert torch.equal(gpu.k_cache[0, 0, :41].cpu(), cpu.k_cache[0, 0, :41])
+    assert torch.equal(gpu.k_cache[0, 0, 42:].cpu(), cpu.k_cache[0, 0, 42:])
+    assert torch.equal(gpu.barriers.cpu(), cpu.barriers)
+
+
+@pytest.mark.parametrize("which", ["mi355x", "reference"])
+@pytest.mark.parametrize("pos,P", [(0, 1), (0, 4), (15, 2), (16, 3), (41, 3), (80, 13), (95, 25)])
+def test_op_attention_split_and_reduce(state, which, pos, P):
+    shape, cpu, gpu = state
+    sched = _sched(shape, which, P)
+    cpu.position_id = pos
+    cpu.barriers[0, 0, :] = sched.expected_counts()[0]
+    cpu.attn_lse_intermediates.fill_(55.0)
+    cpu.attn_out_intermediates.fill_(-3.0)
+    sync_state(cpu, gpu)
+    run_both(cpu, gpu, sched, sched.attention_split_kv(0) + sched.attention_reduction(0))
+    lse_c, lse_g = cpu.attn_lse_intermediates[:, :P], gpu.attn_lse_intermediates[:, :P].cpu()
+    assert torch.equal(torch.isinf(lse_c), torch.isinf(lse_g))
+    fin = torch.isfinite(lse_c)
+    assert (lse_c[fin] - lse_g[fin]).abs().max() < 2e-4
+    assert (cpu.attn_out_intermediates[:, :P] - gpu.attn_out_intermediates[:, :P].cpu()).abs().max() < 2e-4
+    bf16_close(gpu.attn_out, cpu.attn_out, name="attn_out", frac=0.03)
+    assert torch.equal(gpu.barriers.cpu(), cpu.barriers)
+
+
+@pytest.mark.parametrize("which", ["mi355x", "reference"])
+def test_op_oproj(state, which):
+    shape, cpu, gpu = state
+    sched = _sched(shape, which)
+    cpu.barriers[0, 2, 0] = shape.num_attention_heads
+    sync_state(cpu, gpu)
+    run_both(cpu, gpu, sched, sched.oproj(0))
+    bf16_close(gpu.hidden_states, cpu.hidden_states, name="hidden")
+    assert torch.equal(gpu.barriers.cpu(), cpu.barriers)
+
+
+@pytest.mark.parametrize("which", ["mi355x", "reference"])
+def test_op_upgate(state, which):
+    shape, cpu, gpu = state
+    sched = _sched(shape, which)
+    cpu.barriers[0, 3, 0] = sched.expected_counts()[1]
+    sync_state(cpu, gpu)
+    run_both(cpu, gpu, sched, sched.upgate(0))
+    # silu_out = bf16(bf16(silu(gate)) * up): a 1-ulp difference in up or gate moves the product by up to 2 ulps
+    bf16_close(gpu.silu_out, cpu.silu_out, ulps=2.0, frac=0.03, name="silu_out")
+    assert torch.equal(gpu.barriers.cpu(), cpu.barriers)
+
+
+@pytest.mark.parametrize("which", ["mi355x", "reference"])
+def test_op_down(state, which):
+    shape, cpu, gpu = state
+    sched = _sched(shape, which)
+    cpu.barriers[0, 4, : sched.geometry.num_split_k(shape)] = sched.expected_counts()[2]
+    sync_state(cpu, gpu)
+    run_both(cpu, gpu, sched, sched.downproj(0))
+    if which == "mi355x":
+        bf16_close(gpu.hidden_states, cpu.hidden_states, name="hidden")
+    else:
+        # four K slices arrive in any order, each add rounds to bf16: the legal results span a few ulps
+        # (the reference gates this with an arrival-order envelope, verifier/common/reduction_order.py:161-243)
+        bf16_close(gpu.hidden_states, cpu.hidden_states, ulps=3.0, frac=0.5, name="hidden")
+    assert torch.equal(gpu.barriers.cpu(), cpu.barriers)
+
+
+@pytest.mark.parametrize("which", ["mi355x", "reference"])
+def test_op_lm_head(state, which):
+    shape, cpu, gpu = state
+    sched = _sched(shape, which)
+    cpu.barriers[shape.num_hidden_layers - 1, 5, 0] = sched.expected_counts()[3]
+    sync_state(cpu, gpu)
+    run_both(cpu, gpu, sched, sched.lmhead())
+    bf16_close(gpu.logits, cpu.logits, name="logits")
+    assert torch.equal(gpu.barriers.cpu(), cpu.barriers)
+
+
+@pytest.mark.parametrize("which", ["mi355x", "reference"])
+def test_whole_layer_and_counters(state, which):
+    shape, cpu, gpu = state
+    sched = _sched(shape, which, P=5)
+    sync_state(cpu, gpu)
+    run_both(cpu, gpu, sched, sched.instruction_list())
+    tol = dict(ulps=2.0, frac=0.2) if which == "mi355x" else dict(ulps=6.0, frac=0.7)
+    bf16_close(gpu.hidden_states, cpu.hidden_states, name="hidden", **tol)
+    assert (gpu.logits.float().cpu() - cpu.logits.float()).abs().max() < 0.1
+    assert torch.equal(gpu.barriers.cpu(), cpu.barriers)
+
+
+def test_single_queue_and_odd_queue_counts(state):
+    """The same stream dealt onto 1, 7 and 256 queues gives the same result (in-order queues, no deadlock)."""
+    shape, cpu, gpu = state
+    sched = S.mi355x_scheduler(shape, num_partials=2)
+    results = []
+    for sm in (1, 7, 256):
+        sync_state(cpu, gpu)
+        from qimeng_megakernel_amd.decode_schedule import mk_kernel
+        mk = mk_kernel.get_mk(geometry=sched.geometry, reset_barriers=False)
+        mk_kernel.run_instructions(gpu, sched.instruction_list(), mk=mk, sm_count=sm)
+        mk.check()
+        results.append((gpu.hidden_states.clone(), gpu.logits.clone()))
+    for h, l in results[1:]:
+        assert torch.equal(h, results[0][0]) and torch.equal(l, results[0][1])
