@@ -73,7 +73,7 @@ __global__ __launch_bounds__(kThreads, 1) void decode_megakernel(const Params p)
   __syncthreads();
   int32_t* done = counter_ptr(p, 0, p.num_layer_barriers - 1, p.barrier_slots - 1);
   if (threadIdx.x == 0) {
-    const int prev = __hip_atomic_fetch_add(done, 1, __ATOMIC_ACQ_REL, __HIP_MEMORY_SCOPE_AGENT);
+    const int prev = __hip_atomic_fetch_add(done, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     s.ctl[1] = (prev == static_cast<int>(gridDim.x) - 1);
   }
   __syncthreads();

@@ -79,12 +79,18 @@ __device__ __forceinline__ float round_bf16(float f) { return bf2f(f2bf(f)); }
 __device__ __forceinline__ float bf_lo(uint32_t w) { return __uint_as_float(w << 16); }
 __device__ __forceinline__ float bf_hi(uint32_t w) { return __uint_as_float(w & 0xffff0000u); }
 
-// 8 bf16 weights . 8 bf16 activations, fp32 accumulate (v_dot2c_f32_bf16).
+// 8 bf16 weights . 8 bf16 activations, fp32 accumulate (4 x v_dot2c_f32_bf16).
+// The pairs are taken with shufflevector from the whole 16-byte vector: extracting
+// one 32-bit lane first and bit-casting it to a bf16 pair makes this compiler
+// reuse lane 0 for all four dot products.
+typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
 __device__ __forceinline__ float dot8(const v4u& w, const v4u& x, float acc) {
-  acc = __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2_t, w.x), __builtin_bit_cast(bf16x2_t, x.x), acc, false);
-  acc = __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2_t, w.y), __builtin_bit_cast(bf16x2_t, x.y), acc, false);
-  acc = __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2_t, w.z), __builtin_bit_cast(bf16x2_t, x.z), acc, false);
-  acc = __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2_t, w.w), __builtin_bit_cast(bf16x2_t, x.w), acc, false);
+  const bf16x8_t a = __builtin_bit_cast(bf16x8_t, w);
+  const bf16x8_t b = __builtin_bit_cast(bf16x8_t, x);
+  acc = __builtin_amdgcn_fdot2_f32_bf16(__builtin_shufflevector(a, a, 0, 1), __builtin_shufflevector(b, b, 0, 1), acc, false);
+  acc = __builtin_amdgcn_fdot2_f32_bf16(__builtin_shufflevector(a, a, 2, 3), __builtin_shufflevector(b, b, 2, 3), acc, false);
+  acc = __builtin_amdgcn_fdot2_f32_bf16(__builtin_shufflevector(a, a, 4, 5), __builtin_shufflevector(b, b, 4, 5), acc, false);
+  acc = __builtin_amdgcn_fdot2_f32_bf16(__builtin_shufflevector(a, a, 6, 7), __builtin_shufflevector(b, b, 6, 7), acc, false);
   return acc;
 }
 
@@ -135,11 +141,49 @@ __device__ __forceinline__ bool poll_counter(const int32_t* ctr, int expected, u
   return true;
 }
 
-// Make every store of this thread visible device-wide; callers follow it with
-// __syncthreads() and one publishing atomic.
-__device__ __forceinline__ void release_stores() { __builtin_amdgcn_fence(__ATOMIC_RELEASE, "agent"); }
-// Drop stale cache lines after the counters were seen complete.
-__device__ __forceinline__ void acquire_loads() { __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent"); }
+// ---- data that one workgroup writes and another reads within the same launch ----
+// Each XCD has its own L2, so such data must not be served from (or parked in) a
+// local cache.  Instead of writing back / invalidating whole caches around every
+// counter, every access to the shared activation buffers is itself device-coherent:
+// relaxed agent-scope atomics compile to loads and stores with the sc1 bit, which
+// read from and write through to the memory side.  Weights and old KV rows, which no
+// workgroup writes during a launch, use ordinary (cached, non-temporal) loads.
+__device__ __forceinline__ uint32_t ld_shared32(const void* p) {
+  return __hip_atomic_load(static_cast<const uint32_t*>(p), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+__device__ __forceinline__ uint64_t ld_shared64(const void* p) {
+  return __hip_atomic_load(static_cast<const uint64_t*>(p), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+__device__ __forceinline__ float ld_shared_f32(const float* p) { return __uint_as_float(ld_shared32(p)); }
+__device__ __forceinline__ v4u ld_shared128(const void* p) {
+  const uint64_t lo = ld_shared64(p), hi = ld_shared64(static_cast<const char*>(p) + 8);
+  v4u r;
+  r.x = static_cast<uint32_t>(lo); r.y = static_cast<uint32_t>(lo >> 32);
+  r.z = static_cast<uint32_t>(hi); r.w = static_cast<uint32_t>(hi >> 32);
+  return r;
+}
+__device__ __forceinline__ void st_shared32(void* p, uint32_t v) {
+  __hip_atomic_store(static_cast<uint32_t*>(p), v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+__device__ __forceinline__ void st_shared_f32(float* p, float v) { st_shared32(p, __float_as_uint(v)); }
+// 16-bit stores have no atomic form; the neighbouring element belongs to the same
+// lane's next unit or to another wave, so the element is merged into its word by CAS.
+__device__ __forceinline__ void st_shared16(u16* p, u16 v) {
+  uint32_t* word = reinterpret_cast<uint32_t*>(reinterpret_cast<uintptr_t>(p) & ~uintptr_t(3));
+  const bool high = (reinterpret_cast<uintptr_t>(p) & 2) != 0;
+  uint32_t seen = ld_shared32(word);
+  while (true) {
+    const uint32_t want = high ? ((seen & 0x0000ffffu) | (static_cast<uint32_t>(v) << 16)) : ((seen & 0xffff0000u) | v);
+    if (__hip_atomic_compare_exchange_strong(word, &seen, want, __ATOMIC_RELAXED, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT)) break;
+  }
+}
+
+// All earlier vector-memory operations of this wave (the write-through stores above
+// included) have been acknowledged.  Callers follow it with __syncthreads() and one
+// publishing atomic.  s_waitcnt vmcnt(0), expcnt/lgkmcnt left alone.
+__device__ __forceinline__ void release_stores() { __builtin_amdgcn_s_waitcnt(0x0F70); }
+// Nothing to drop: consumers read shared data with device-coherent loads.
+__device__ __forceinline__ void acquire_loads() {}
 
 __device__ __forceinline__ void publish(int32_t* ctr, int amount) {
   __hip_atomic_fetch_add(ctr, amount, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);

@@ -24,12 +24,15 @@ struct Llama1B {
   static constexpr int KV_BLOCK = 16;  // split-KV partition granularity in tokens
 };
 
+constexpr int kResSlots = 4096;
+
 template <class M>
 struct Smem {
   int32_t inst[kInstWords];
   int32_t ctl[8];                       // [0] abort, [1] last workgroup to retire
   float red[kWaves];
   alignas(16) u16 x[M::F];              // activation vector handed to the GEMV lanes
+  float res[kResSlots];                 // per-row GEMV results awaiting the epilogue pass
   float merge[kWaves][M::GQA][M::D + 2];  // per-wave attention state: acc[D], m, l
   unsigned long long t_wait;            // timeline: when the last counter wait finished
 };
@@ -86,8 +89,9 @@ template <class M>
 __device__ __forceinline__ void rms_to_lds(const Params& p, Smem<M>& s, const u16* hidden, const u16* weight) {
   static_assert(M::H == kThreads * 4, "one thread normalises four elements");
   const int t = threadIdx.x;
-  const uint2 hv = *reinterpret_cast<const uint2*>(hidden + t * 4);
-  const float x0 = bf_lo(hv.x), x1 = bf_hi(hv.x), x2 = bf_lo(hv.y), x3 = bf_hi(hv.y);
+  const uint64_t hw = ld_shared64(hidden + t * 4);
+  const uint32_t hlo = static_cast<uint32_t>(hw), hhi = static_cast<uint32_t>(hw >> 32);
+  const float x0 = bf_lo(hlo), x1 = bf_hi(hlo), x2 = bf_lo(hhi), x3 = bf_hi(hhi);
   float ss = __builtin_fmaf(x3, x3, __builtin_fmaf(x2, x2, __builtin_fmaf(x1, x1, x0 * x0)));
   ss = block_sum(ss, s.red);
   const float mean = ss / static_cast<float>(M::H);
@@ -113,6 +117,45 @@ __device__ __forceinline__ uint32_t rope_pair(float v0, float v1, const float* c
   return static_cast<uint32_t>(f2bf(o0)) | (static_cast<uint32_t>(f2bf(o1)) << 16);
 }
 
+// Row-pair streaming shared by the K = hidden GEMVs: wave w takes units w, w+8, ...;
+// a unit is two weight rows (`rows(unit, r0, r1)`), double-buffered so that 16 loads
+// of 16 bytes per lane are in flight.  `a0/a1` may already hold unit `wave` (issued
+// before the counter wait).  Results go to `emit(unit, sum0, sum1)` on lane 0.
+template <int CH, class Rows, class Emit>
+__device__ __forceinline__ void stream_pairs(int nunits, Rows rows, const v4u (&x)[CH], RowRegs<CH>& a0, RowRegs<CH>& a1,
+                                             Emit emit) {
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  RowRegs<CH> b0, b1;
+  int u = wave;
+  while (u < nunits) {
+    int un = u + kWaves;
+    if (un < nunits) {
+      const u16 *r0, *r1;
+      rows(un, r0, r1);
+      load_row(b0, r0, lane);
+      load_row(b1, r1, lane);
+    }
+    {
+      const float s0 = wave_sum(dot_row(a0, x)), s1 = wave_sum(dot_row(a1, x));
+      if (lane == 0) emit(u, s0, s1);
+    }
+    u = un;
+    if (u >= nunits) break;
+    un = u + kWaves;
+    if (un < nunits) {
+      const u16 *r0, *r1;
+      rows(un, r0, r1);
+      load_row(a0, r0, lane);
+      load_row(a1, r1, lane);
+    }
+    {
+      const float s0 = wave_sum(dot_row(b0, x)), s1 = wave_sum(dot_row(b1, x));
+      if (lane == 0) emit(u, s0, s1);
+    }
+    u = un;
+  }
+}
+
 // ===================================================================== 1 ==
 // [1, layer, tile_M, n_start, n_end, tile_M_g, tile_N_g]
 template <class M>
@@ -123,17 +166,23 @@ __device__ bool op_rms_qkv_rope(const Params& p, Smem<M>& s, const Ctx& c) {
   if (layer < 0 || layer >= p.num_layers) return bad_operand(p, s, c, 1);
   if (tile <= 0 || (tile & 1) || tile * bph != M::D) return bad_operand(p, s, c, 6);
   if (nstart < 0 || nend < nstart || static_cast<long>(nend) * tile > M::QKV) return bad_operand(p, s, c, 4);
+  if ((nend - nstart) * tile > kResSlots) return bad_operand(p, s, c, 3);
 
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int rs = nstart * tile;
   const int nunits = (nend - nstart) * tile / 2;
   const u16* W = p.qkv_w + static_cast<size_t>(layer) * M::QKV * M::H;
+  auto rows = [&](int unit, const u16*& r0, const u16*& r1) {
+    r0 = W + static_cast<size_t>(rs + 2 * unit) * M::H;
+    r1 = r0 + M::H;
+  };
 
-  RowRegs<CH> a0, a1, b0, b1;
-  int u = wave;
-  if (u < nunits) {  // in flight while the counter is polled
-    load_row(a0, W + static_cast<size_t>(rs + 2 * u) * M::H, lane);
-    load_row(a1, W + static_cast<size_t>(rs + 2 * u + 1) * M::H, lane);
+  RowRegs<CH> a0, a1;
+  if (wave < nunits) {  // in flight while the counter is polled
+    const u16 *r0, *r1;
+    rows(wave, r0, r1);
+    load_row(a0, r0, lane);
+    load_row(a1, r1, lane);
   }
   if (layer > 0) {
     if (!wg_wait(p, s, c, 1, [&](int) { return counter_ptr(p, layer - 1, ROW_DOWN, 0); }, p.down_arrivals)) return false;
@@ -141,43 +190,28 @@ __device__ bool op_rms_qkv_rope(const Params& p, Smem<M>& s, const Ctx& c) {
   rms_to_lds(p, s, p.hidden, p.attn_norm + static_cast<size_t>(layer) * M::H);
   v4u x[CH];
   load_x_from_lds(x, s.x, lane);
+  stream_pairs<CH>(nunits, rows, x, a0, a1, [&](int unit, float s0, float s1) {
+    s.res[2 * unit] = s0;
+    s.res[2 * unit + 1] = s1;
+  });
+  __syncthreads();
 
+  // Epilogue: the GEMV result is bf16 before RoPE; q -> q_post_rope, k/v -> cache row of this position.
   const float* cosr = p.rope_cos + static_cast<size_t>(p.pos_id) * M::D;
   const float* sinr = p.rope_sin + static_cast<size_t>(p.pos_id) * M::D;
   const size_t kv_row = (static_cast<size_t>(layer) * p.max_seq_len + p.pos_id) * (M::NKV * M::D);
-
-  auto finish = [&](int unit, float s0, float s1) {
-    if (lane != 0) return;
+  for (int unit = threadIdx.x; unit < nunits; unit += kThreads) {
     const int r = rs + 2 * unit;
-    const float v0 = round_bf16(s0), v1 = round_bf16(s1);  // the GEMV result is bf16 before RoPE
+    const float v0 = round_bf16(s.res[2 * unit]), v1 = round_bf16(s.res[2 * unit + 1]);
     if (r < M::NQ * M::D) {
-      *reinterpret_cast<uint32_t*>(p.q_post_rope + r) = rope_pair(v0, v1, cosr, sinr, r % M::D);
+      st_shared32(p.q_post_rope + r, rope_pair(v0, v1, cosr, sinr, r % M::D));
     } else if (r < (M::NQ + M::NKV) * M::D) {
       const int i = r - M::NQ * M::D;
-      *reinterpret_cast<uint32_t*>(p.k_cache + kv_row + i) = rope_pair(v0, v1, cosr, sinr, i % M::D);
+      st_shared32(p.k_cache + kv_row + i, rope_pair(v0, v1, cosr, sinr, i % M::D));
     } else {
       const int i = r - (M::NQ + M::NKV) * M::D;
-      *reinterpret_cast<uint32_t*>(p.v_cache + kv_row + i) =
-          static_cast<uint32_t>(f2bf(v0)) | (static_cast<uint32_t>(f2bf(v1)) << 16);
+      st_shared32(p.v_cache + kv_row + i, static_cast<uint32_t>(f2bf(v0)) | (static_cast<uint32_t>(f2bf(v1)) << 16));
     }
-  };
-
-  while (u < nunits) {
-    int un = u + kWaves;
-    if (un < nunits) {
-      load_row(b0, W + static_cast<size_t>(rs + 2 * un) * M::H, lane);
-      load_row(b1, W + static_cast<size_t>(rs + 2 * un + 1) * M::H, lane);
-    }
-    finish(u, wave_sum(dot_row(a0, x)), wave_sum(dot_row(a1, x)));
-    u = un;
-    if (u >= nunits) break;
-    un = u + kWaves;
-    if (un < nunits) {
-      load_row(a0, W + static_cast<size_t>(rs + 2 * un) * M::H, lane);
-      load_row(a1, W + static_cast<size_t>(rs + 2 * un + 1) * M::H, lane);
-    }
-    finish(u, wave_sum(dot_row(b0, x)), wave_sum(dot_row(b1, x)));
-    u = un;
   }
 
   release_stores();
@@ -232,7 +266,7 @@ __device__ bool op_attn_splitkv(const Params& p, Smem<M>& s, const Ctx& c) {
   float q[M::GQA][8];
 #pragma unroll
   for (int h = 0; h < M::GQA; ++h) {
-    const v4u qv = *reinterpret_cast<const v4u*>(p.q_post_rope + (kvh * M::GQA + h) * M::D + col * 8);
+    const v4u qv = ld_shared128(p.q_post_rope + (kvh * M::GQA + h) * M::D + col * 8);
     q[h][0] = bf_lo(qv.x) * qscale; q[h][1] = bf_hi(qv.x) * qscale;
     q[h][2] = bf_lo(qv.y) * qscale; q[h][3] = bf_hi(qv.y) * qscale;
     q[h][4] = bf_lo(qv.z) * qscale; q[h][5] = bf_hi(qv.z) * qscale;
@@ -252,8 +286,14 @@ __device__ bool op_attn_splitkv(const Params& p, Smem<M>& s, const Ctx& c) {
   const size_t base = static_cast<size_t>(layer) * p.max_seq_len * tok_stride + static_cast<size_t>(kvh) * M::D + col * 8;
   for (int t = t0 + wave * 8 + grp; t < t1; t += kWaves * 8) {
     const size_t off = base + static_cast<size_t>(t) * tok_stride;
-    const v4u kv = *reinterpret_cast<const v4u*>(p.k_cache + off);
-    const v4u vv = *reinterpret_cast<const v4u*>(p.v_cache + off);
+    v4u kv, vv;
+    if (t == p.pos_id) {  // the row another workgroup appended during this launch
+      kv = ld_shared128(p.k_cache + off);
+      vv = ld_shared128(p.v_cache + off);
+    } else {
+      kv = *reinterpret_cast<const v4u*>(p.k_cache + off);
+      vv = *reinterpret_cast<const v4u*>(p.v_cache + off);
+    }
     const float k[8] = {bf_lo(kv.x), bf_hi(kv.x), bf_lo(kv.y), bf_hi(kv.y), bf_lo(kv.z), bf_hi(kv.z), bf_lo(kv.w), bf_hi(kv.w)};
     const float v[8] = {bf_lo(vv.x), bf_hi(vv.x), bf_lo(vv.y), bf_hi(vv.y), bf_lo(vv.z), bf_hi(vv.z), bf_lo(vv.w), bf_hi(vv.w)};
 #pragma unroll
@@ -324,8 +364,8 @@ __device__ bool op_attn_splitkv(const Params& p, Smem<M>& s, const Ctx& c) {
     const int head = kvh * M::GQA + h;
     const bool empty = !(den > 0.f);
     // Normalised partial output and log2-sum-exp; an empty slice contributes (0, -inf).
-    p.attn_partial[(static_cast<size_t>(head) * p.max_splits + part) * M::D + d] = empty ? 0.f : num / den;
-    if (d == 0) p.attn_lse[static_cast<size_t>(head) * p.max_splits + part] = empty ? -INFINITY : mx + log2f(den);
+    st_shared_f32(p.attn_partial + (static_cast<size_t>(head) * p.max_splits + part) * M::D + d, empty ? 0.f : num / den);
+    if (d == 0) st_shared_f32(p.attn_lse + static_cast<size_t>(head) * p.max_splits + part, empty ? -INFINITY : mx + log2f(den));
   }
 
   release_stores();
@@ -350,32 +390,45 @@ __device__ bool op_attn_reduce(const Params& p, Smem<M>& s, const Ctx& c) {
 
   if (!wg_wait(p, s, c, M::GQA, [&](int i) { return counter_ptr(p, layer, ROW_SPLITKV, head0 + i); }, P)) return false;
 
-  if (threadIdx.x < M::GQA * M::D) {
-    const int h = head0 + threadIdx.x / M::D, d = threadIdx.x % M::D;
+  // Thread (h, d/2) merges two neighbouring output dims so that it can store one 32-bit word.
+  if (threadIdx.x < M::GQA * M::D / 2) {
+    const int h = head0 + threadIdx.x / (M::D / 2), d = 2 * (threadIdx.x % (M::D / 2));
     const float* lse = p.attn_lse + static_cast<size_t>(h) * p.max_splits;
     const float* part = p.attn_partial + static_cast<size_t>(h) * p.max_splits * M::D + d;
     float mx = -INFINITY;
-    for (int i = 0; i < n; ++i) mx = fmaxf(mx, lse[s.inst[5 + i]]);
-    float num = 0.f, den = 0.f;
+    for (int i = 0; i < n; ++i) mx = fmaxf(mx, ld_shared_f32(lse + s.inst[5 + i]));
+    float num0 = 0.f, num1 = 0.f, den = 0.f;
     for (int i = 0; i < n; ++i) {
       const int j = s.inst[5 + i];
-      const float e = lse[j];
+      const float e = ld_shared_f32(lse + j);
       const float f = (e == -INFINITY) ? 0.f : exp2f(e - mx);
-      num = __builtin_fmaf(part[static_cast<size_t>(j) * M::D], f, num);
+      const uint64_t two = ld_shared64(part + static_cast<size_t>(j) * M::D);
+      num0 = __builtin_fmaf(__uint_as_float(static_cast<uint32_t>(two)), f, num0);
+      num1 = __builtin_fmaf(__uint_as_float(static_cast<uint32_t>(two >> 32)), f, num1);
       den += f;
     }
-    const float o = den > 0.f ? num / den : 0.f;
+    const float o0 = den > 0.f ? num0 / den : 0.f, o1 = den > 0.f ? num1 / den : 0.f;
     if (terminal) {
-      p.attn_out[h * M::D + d] = f2bf(o);
+      st_shared32(p.attn_out + h * M::D + d, static_cast<uint32_t>(f2bf(o0)) | (static_cast<uint32_t>(f2bf(o1)) << 16));
     } else {
-      p.attn_partial[(static_cast<size_t>(h) * p.max_splits + out_slot) * M::D + d] = o;
-      if (d == 0) p.attn_lse[static_cast<size_t>(h) * p.max_splits + out_slot] = den > 0.f ? mx + log2f(den) : -INFINITY;
+      float* dst = p.attn_partial + (static_cast<size_t>(h) * p.max_splits + out_slot) * M::D + d;
+      st_shared_f32(dst, o0);
+      st_shared_f32(dst + 1, o1);
+      if (d == 0) st_shared_f32(p.attn_lse + static_cast<size_t>(h) * p.max_splits + out_slot, den > 0.f ? mx + log2f(den) : -INFINITY);
     }
   }
   release_stores();
   __syncthreads();
   if (threadIdx.x == 0) publish(counter_ptr(p, layer, ROW_REDUCE, 0), M::GQA);
   return true;
+}
+
+// hidden[r0], hidden[r0+1] += bf16(delta): one coherent 32-bit read-modify-write.
+__device__ __forceinline__ void residual_pair(u16* hidden_pair, float d0, float d1) {
+  const uint32_t old = ld_shared32(hidden_pair);
+  const u16 n0 = f2bf(bf_lo(old) + round_bf16(d0));
+  const u16 n1 = f2bf(bf_hi(old) + round_bf16(d1));
+  st_shared32(hidden_pair, static_cast<uint32_t>(n0) | (static_cast<uint32_t>(n1) << 16));
 }
 
 // ===================================================================== 4 ==
@@ -389,53 +442,38 @@ __device__ bool op_oproj_residual(const Params& p, Smem<M>& s, const Ctx& c) {
   if (layer < 0 || layer >= p.num_layers) return bad_operand(p, s, c, 1);
   if (tile <= 0 || (tile & 1)) return bad_operand(p, s, c, 7);
   if (nstart < 0 || nend < nstart || static_cast<long>(nend) * tile > M::H) return bad_operand(p, s, c, 4);
+  if ((nend - nstart) * tile > kResSlots) return bad_operand(p, s, c, 3);
 
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int rs = nstart * tile;
   const int nunits = (nend - nstart) * tile / 2;
   const u16* W = p.o_w + static_cast<size_t>(layer) * M::H * M::H;
+  auto rows = [&](int unit, const u16*& r0, const u16*& r1) {
+    r0 = W + static_cast<size_t>(rs + 2 * unit) * M::H;
+    r1 = r0 + M::H;
+  };
 
-  RowRegs<CH> a0, a1, b0, b1;
-  int u = wave;
-  if (u < nunits) {
-    load_row(a0, W + static_cast<size_t>(rs + 2 * u) * M::H, lane);
-    load_row(a1, W + static_cast<size_t>(rs + 2 * u + 1) * M::H, lane);
+  RowRegs<CH> a0, a1;
+  if (wave < nunits) {
+    const u16 *r0, *r1;
+    rows(wave, r0, r1);
+    load_row(a0, r0, lane);
+    load_row(a1, r1, lane);
   }
   if (!wg_wait(p, s, c, 1, [&](int) { return counter_ptr(p, layer, ROW_REDUCE, 0); }, M::NQ)) return false;
 
+  static_assert(M::H == kThreads * 4, "one thread stages four elements");
+  *reinterpret_cast<uint64_t*>(s.x + threadIdx.x * 4) = ld_shared64(p.attn_out + threadIdx.x * 4);
+  __syncthreads();
   v4u x[CH];
-  {
-    const v4u* ap = reinterpret_cast<const v4u*>(p.attn_out) + lane;
-#pragma unroll
-    for (int j = 0; j < CH; ++j) x[j] = ap[j * kWaveSize];
-  }
-
-  auto finish = [&](int unit, float s0, float s1) {
-    if (lane != 0) return;
-    uint32_t* hp = reinterpret_cast<uint32_t*>(p.hidden + rs + 2 * unit);
-    const uint32_t old = *hp;
-    const u16 n0 = f2bf(bf_lo(old) + round_bf16(s0));
-    const u16 n1 = f2bf(bf_hi(old) + round_bf16(s1));
-    *hp = static_cast<uint32_t>(n0) | (static_cast<uint32_t>(n1) << 16);
-  };
-
-  while (u < nunits) {
-    int un = u + kWaves;
-    if (un < nunits) {
-      load_row(b0, W + static_cast<size_t>(rs + 2 * un) * M::H, lane);
-      load_row(b1, W + static_cast<size_t>(rs + 2 * un + 1) * M::H, lane);
-    }
-    finish(u, wave_sum(dot_row(a0, x)), wave_sum(dot_row(a1, x)));
-    u = un;
-    if (u >= nunits) break;
-    un = u + kWaves;
-    if (un < nunits) {
-      load_row(a0, W + static_cast<size_t>(rs + 2 * un) * M::H, lane);
-      load_row(a1, W + static_cast<size_t>(rs + 2 * un + 1) * M::H, lane);
-    }
-    finish(u, wave_sum(dot_row(b0, x)), wave_sum(dot_row(b1, x)));
-    u = un;
-  }
+  load_x_from_lds(x, s.x, lane);
+  stream_pairs<CH>(nunits, rows, x, a0, a1, [&](int unit, float s0, float s1) {
+    s.res[2 * unit] = s0;
+    s.res[2 * unit + 1] = s1;
+  });
+  __syncthreads();
+  for (int unit = threadIdx.x; unit < nunits; unit += kThreads)
+    residual_pair(p.hidden + rs + 2 * unit, s.res[2 * unit], s.res[2 * unit + 1]);
 
   release_stores();
   __syncthreads();
@@ -453,7 +491,8 @@ __device__ bool op_rms_upgate_silu(const Params& p, Smem<M>& s, const Ctx& c) {
   if (layer < 0 || layer >= p.num_layers) return bad_operand(p, s, c, 1);
   if (n < 0 || n > kInstWords - 6) return bad_operand(p, s, c, 3);
   const int tile = s.inst[5 + n];
-  if (tile <= 0) return bad_operand(p, s, c, 5 + n);
+  if (tile <= 0 || (tile & 1) || M::F % tile != 0) return bad_operand(p, s, c, 5 + n);
+  if (n * tile * 2 > kResSlots) return bad_operand(p, s, c, 3);
   const int nblocks_total = M::F / tile;
   for (int i = 0; i < n; ++i)
     if (s.inst[4 + i] < 0 || s.inst[4 + i] >= nblocks_total) return bad_operand(p, s, c, 4 + i);
@@ -463,44 +502,33 @@ __device__ bool op_rms_upgate_silu(const Params& p, Smem<M>& s, const Ctx& c) {
   const u16* Wu = p.up_w + static_cast<size_t>(layer) * M::F * M::H;
   const u16* Wg = p.gate_w + static_cast<size_t>(layer) * M::F * M::H;
   auto row_of = [&](int unit) { return s.inst[4 + unit / tile] * tile + unit % tile; };
+  auto rows = [&](int unit, const u16*& r0, const u16*& r1) {
+    const size_t r = row_of(unit);
+    r0 = Wu + r * M::H;
+    r1 = Wg + r * M::H;
+  };
 
-  RowRegs<CH> a0, a1, b0, b1;
-  int u = wave;
-  if (u < nunits) {
-    const size_t r = row_of(u);
-    load_row(a0, Wu + r * M::H, lane);
-    load_row(a1, Wg + r * M::H, lane);
+  RowRegs<CH> a0, a1;
+  if (wave < nunits) {
+    const u16 *r0, *r1;
+    rows(wave, r0, r1);
+    load_row(a0, r0, lane);
+    load_row(a1, r1, lane);
   }
   if (!wg_wait(p, s, c, 1, [&](int) { return counter_ptr(p, layer, ROW_OPROJ, 0); }, p.oproj_blocks)) return false;
   rms_to_lds(p, s, p.hidden, p.mlp_norm + static_cast<size_t>(layer) * M::H);
   v4u x[CH];
   load_x_from_lds(x, s.x, lane);
-
-  auto finish = [&](int unit, float su, float sg) {
-    if (lane != 0) return;
+  stream_pairs<CH>(nunits, rows, x, a0, a1, [&](int unit, float su, float sg) {
     const float up = round_bf16(su), gate = round_bf16(sg);
     const float act = round_bf16(gate / (1.0f + expf(-gate)));
-    p.silu_out[row_of(unit)] = f2bf(act * up);
-  };
-
-  while (u < nunits) {
-    int un = u + kWaves;
-    if (un < nunits) {
-      const size_t r = row_of(un);
-      load_row(b0, Wu + r * M::H, lane);
-      load_row(b1, Wg + r * M::H, lane);
-    }
-    finish(u, wave_sum(dot_row(a0, x)), wave_sum(dot_row(a1, x)));
-    u = un;
-    if (u >= nunits) break;
-    un = u + kWaves;
-    if (un < nunits) {
-      const size_t r = row_of(un);
-      load_row(a0, Wu + r * M::H, lane);
-      load_row(a1, Wg + r * M::H, lane);
-    }
-    finish(u, wave_sum(dot_row(b0, x)), wave_sum(dot_row(b1, x)));
-    u = un;
+    s.res[unit] = act * up;  // rounded to bf16 on the way out
+  });
+  __syncthreads();
+  // Two neighbouring outputs of a tile leave as one 32-bit word.
+  for (int pair = threadIdx.x; pair < nunits / 2; pair += kThreads) {
+    const uint32_t w = static_cast<uint32_t>(f2bf(s.res[2 * pair])) | (static_cast<uint32_t>(f2bf(s.res[2 * pair + 1])) << 16);
+    st_shared32(p.silu_out + row_of(2 * pair), w);
   }
 
   release_stores();
@@ -517,7 +545,7 @@ __device__ bool op_rms_upgate_silu(const Params& p, Smem<M>& s, const Ctx& c) {
 __device__ __forceinline__ void atomic_add_bf16(u16* addr, float delta) {
   uint32_t* word = reinterpret_cast<uint32_t*>(reinterpret_cast<uintptr_t>(addr) & ~uintptr_t(3));
   const bool high = (reinterpret_cast<uintptr_t>(addr) & 2) != 0;
-  uint32_t seen = __hip_atomic_load(word, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  uint32_t seen = ld_shared32(word);
   while (true) {
     const u16 cur = high ? static_cast<u16>(seen >> 16) : static_cast<u16>(seen & 0xffffu);
     const u16 nxt = f2bf(bf2f(cur) + delta);
@@ -530,35 +558,29 @@ __device__ __forceinline__ void atomic_add_bf16(u16* addr, float delta) {
 // [6, layer, tile_M, n_start, n_end, split_K_idx, tile_M_g, tile_N_g, split_K_g]
 // hidden[r] = bf16(hidden[r] + bf16(W_d[r, slice] . silu_out[slice]))   (operations.py:285-295;
 // python_vm.py:137-171 for the sliced form).  With one slice this is the fused form exactly.
+// Wave w streams rows rs+w, rs+w+8, ... in groups of G 1-KiB chunks, double-buffered.
 template <class M, int G>
-__device__ __forceinline__ void down_rows(const Params& p, Smem<M>& s, const u16* W, int rs, int re, int ks, int kg,
-                                          RowRegs<G>& a, bool a_loaded, bool single_slice) {
+__device__ __forceinline__ void down_rows(Smem<M>& s, const u16* W, int rs, int re, int ks, int kg, RowRegs<G>& a,
+                                          bool a_loaded) {
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-  const int groups = kg / (512 * G);  // G-chunk groups per row
+  const int groups = kg / (512 * G);
   const int nrows = re - rs;
-  // Flattened (row, group) sequence of this wave: row = rs + wave + 8*i, group g.
-  const int total = ((nrows - wave + kWaves - 1) / kWaves) * groups;  // may be <= 0
+  const int total = ((nrows - wave + kWaves - 1) / kWaves) * groups;  // (row, group) steps of this wave; <= 0 if none
   RowRegs<G> b;
   auto src = [&](int idx) {
     const int row = rs + wave + (idx / groups) * kWaves;
     return W + static_cast<size_t>(row) * M::F + ks + (idx % groups) * (512 * G);
   };
-  auto xs = [&](int idx, v4u (&x)[G]) { load_x_from_lds(x, s.x + (idx % groups) * (512 * G), lane); };
   float acc = 0.f;
   auto step = [&](const RowRegs<G>& r, int idx) {
     v4u x[G];
-    xs(idx, x);
+    load_x_from_lds(x, s.x + (idx % groups) * (512 * G), lane);
 #pragma unroll
     for (int j = 0; j < G; ++j) acc = dot8(r.v[j], x[j], acc);
     if (idx % groups == groups - 1) {
       const float sum = wave_sum(acc);
       acc = 0.f;
-      if (lane == 0) {
-        u16* hp = p.hidden + rs + wave + (idx / groups) * kWaves;
-        const float d = round_bf16(sum);
-        if (single_slice) *hp = f2bf(bf2f(*hp) + d);
-        else atomic_add_bf16(hp, d);
-      }
+      if (lane == 0) s.res[wave + (idx / groups) * kWaves] = sum;
     }
   };
   int i = 0;
@@ -579,8 +601,9 @@ __device__ bool op_down_residual(const Params& p, Smem<M>& s, const Ctx& c) {
   const int layer = s.inst[1], nstart = s.inst[3], nend = s.inst[4], split = s.inst[5];
   const int tile = s.inst[7], kg = s.inst[8];
   if (layer < 0 || layer >= p.num_layers) return bad_operand(p, s, c, 1);
-  if (tile <= 0) return bad_operand(p, s, c, 7);
+  if (tile <= 0 || (tile & 1)) return bad_operand(p, s, c, 7);
   if (nstart < 0 || nend < nstart || static_cast<long>(nend) * tile > M::H) return bad_operand(p, s, c, 4);
+  if ((nend - nstart) * tile > kResSlots) return bad_operand(p, s, c, 3);
   if (kg <= 0 || kg % 2048 != 0 || kg > M::F) return bad_operand(p, s, c, 8);
   if (split < 0 || static_cast<long>(split + 1) * kg > M::F) return bad_operand(p, s, c, 5);
   if (split >= p.barrier_slots) return bad_operand(p, s, c, 5);
@@ -601,13 +624,21 @@ __device__ bool op_down_residual(const Params& p, Smem<M>& s, const Ctx& c) {
   if (!wg_wait(p, s, c, 1, [&](int) { return counter_ptr(p, layer, ROW_UPGATE, split); }, p.upgate_blocks_per_bucket)) return false;
 
   // The K slice of silu_out into LDS.
-  for (int i = threadIdx.x; i < kg / 8; i += kThreads)
-    reinterpret_cast<v4u*>(s.x)[i] = reinterpret_cast<const v4u*>(p.silu_out + ks)[i];
+  for (int i = threadIdx.x; i < kg / 4; i += kThreads)
+    reinterpret_cast<uint64_t*>(s.x)[i] = ld_shared64(p.silu_out + ks + i * 4);
   __syncthreads();
 
-  const bool single = kg == M::F;
-  if (wide) down_rows<M, 8>(p, s, W, rs, re, ks, kg, a8, have_row, single);
-  else down_rows<M, 4>(p, s, W, rs, re, ks, kg, a4, have_row, single);
+  if (wide) down_rows<M, 8>(s, W, rs, re, ks, kg, a8, have_row);
+  else down_rows<M, 4>(s, W, rs, re, ks, kg, a4, have_row);
+  __syncthreads();
+
+  const int nrows = re - rs;
+  if (kg == M::F) {  // one slice: every row has a single writer
+    for (int pair = threadIdx.x; pair < nrows / 2; pair += kThreads)
+      residual_pair(p.hidden + rs + 2 * pair, s.res[2 * pair], s.res[2 * pair + 1]);
+  } else {           // other slices add to the same rows concurrently
+    for (int r = threadIdx.x; r < nrows; r += kThreads) atomic_add_bf16(p.hidden + rs + r, round_bf16(s.res[r]));
+  }
 
   release_stores();
   __syncthreads();
@@ -629,42 +660,28 @@ __device__ bool op_rms_lmhead(const Params& p, Smem<M>& s, const Ctx& c) {
   const int rs = bstart * tile;
   const int nunits = (bend - bstart) * tile / 2;
   const u16* W = p.lm_w;
+  auto rows = [&](int unit, const u16*& r0, const u16*& r1) {
+    r0 = W + static_cast<size_t>(rs + 2 * unit) * M::H;
+    r1 = r0 + M::H;
+  };
 
-  RowRegs<CH> a0, a1, b0, b1;
-  int u = wave;
-  if (u < nunits) {
-    load_row(a0, W + static_cast<size_t>(rs + 2 * u) * M::H, lane);
-    load_row(a1, W + static_cast<size_t>(rs + 2 * u + 1) * M::H, lane);
+  RowRegs<CH> a0, a1;
+  if (wave < nunits) {
+    const u16 *r0, *r1;
+    rows(wave, r0, r1);
+    load_row(a0, r0, lane);
+    load_row(a1, r1, lane);
   }
   if (!wg_wait(p, s, c, 1, [&](int) { return counter_ptr(p, p.num_layers - 1, ROW_DOWN, 0); }, p.down_arrivals)) return false;
   rms_to_lds(p, s, p.hidden, p.lm_norm);
   v4u x[CH];
   load_x_from_lds(x, s.x, lane);
-
-  auto finish = [&](int unit, float s0, float s1) {
-    if (lane != 0) return;
+  // Terminal op: nothing inside the launch reads the logits, so ordinary stores do.
+  stream_pairs<CH>(nunits, rows, x, a0, a1, [&](int unit, float s0, float s1) {
     *reinterpret_cast<uint32_t*>(p.logits + rs + 2 * unit) =
         static_cast<uint32_t>(f2bf(s0)) | (static_cast<uint32_t>(f2bf(s1)) << 16);
-  };
-
-  while (u < nunits) {
-    int un = u + kWaves;
-    if (un < nunits) {
-      load_row(b0, W + static_cast<size_t>(rs + 2 * un) * M::H, lane);
-      load_row(b1, W + static_cast<size_t>(rs + 2 * un + 1) * M::H, lane);
-    }
-    finish(u, wave_sum(dot_row(a0, x)), wave_sum(dot_row(a1, x)));
-    u = un;
-    if (u >= nunits) break;
-    un = u + kWaves;
-    if (un < nunits) {
-      load_row(a0, W + static_cast<size_t>(rs + 2 * un) * M::H, lane);
-      load_row(a1, W + static_cast<size_t>(rs + 2 * un + 1) * M::H, lane);
-    }
-    finish(u, wave_sum(dot_row(b0, x)), wave_sum(dot_row(b1, x)));
-    u = un;
-  }
-  return true;  // terminal: nothing waits on the logits inside the kernel
+  });
+  return true;
 }
 
 }  // namespace qmk

@@ -37,13 +37,16 @@ def run_both(cpu, gpu, sched, instructions, *, sm_count=None):
     return mk
 
 
-def bf16_close(got: torch.Tensor, want: torch.Tensor, *, ulps: float = 1.0, frac: float = 0.02, name: str = "tensor"):
+def bf16_close(got: torch.Tensor, want: torch.Tensor, *, ulps: float = 1.0, frac: float = 0.02,
+               floor: float = 2.0 ** -6, name: str = "tensor"):
     """bf16 tensors that come from fp32-accumulated dot products of the same inputs: equal except
     where the exact value sits next to a rounding boundary; there, at most ``ulps`` bf16 ulps.
-    Tolerance: max |diff| <= ulps * 2^-7 * max(|want|, 2^-6) and at most ``frac`` of elements differ."""
+    Tolerance: |diff| <= ulps * ulp_bf16(max(|want|, floor)); at most ``frac`` of the elements differ.
+    ``floor`` is the magnitude of the operands that were rounded on the way (for a residual add
+    the addends, not the possibly cancelled sum)."""
     got, want = got.detach().float().cpu().reshape(-1), want.detach().float().cpu().reshape(-1)
     assert torch.isfinite(got).all(), f"{name}: non-finite values"
-    scale = torch.maximum(want.abs(), torch.tensor(2.0 ** -6))
+    scale = torch.maximum(want.abs(), torch.tensor(float(floor)))
     ulp = torch.exp2(torch.floor(torch.log2(scale)) - 7)
     diff = (got - want).abs()
     worst = float((diff / ulp).max())
@@ -51,3 +54,18 @@ def bf16_close(got: torch.Tensor, want: torch.Tensor, *, ulps: float = 1.0, frac
     off = float((diff > 0).float().mean())
     assert off <= frac, f"{name}: {off:.4f} of the elements differ (allowed {frac})"
     return worst, off
+
+
+def rel_close(got: torch.Tensor, want: torch.Tensor, *, rel: float = 2e-2, name: str = "tensor"):
+    """The bf16 gate of the decode path: elementwise |diff| <= rel * max(|want_i|, rms(want)).
+
+    Relative error is taken against the element where it is large enough to carry a meaningful
+    ratio and against the tensor's RMS otherwise: the residual stream adds O(1) terms whose own
+    bf16 rounding (2^-8 relative) lands on elements that happen to cancel to nearly zero."""
+    got, want = got.detach().float().cpu().reshape(-1), want.detach().float().cpu().reshape(-1)
+    assert torch.isfinite(got).all(), f"{name}: non-finite values"
+    rms = float(want.pow(2).mean().sqrt())
+    bound = rel * torch.maximum(want.abs(), torch.tensor(rms))
+    ratio = float(((got - want).abs() / bound).max()) * rel
+    assert ratio <= rel, f"{name}: max rel err {ratio:.4g} > {rel} (rms {rms:.4g})"
+    return ratio

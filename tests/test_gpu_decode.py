@@ -3,35 +3,79 @@ import pytest
 import torch
 
 from fused_oracle import FusedOracle
-from gpu_helpers import bf16_close, pair
+from gpu_helpers import bf16_close, pair, rel_close
 from qimeng_megakernel_amd import decode, synthetic
 from qimeng_megakernel_amd.decode_schedule import mk_kernel
 from qimeng_megakernel_amd.decode_schedule.model_config import LlamaConfig
 
 pytestmark = pytest.mark.gpu
 
+# Gate for states that have run through several steps (the KV cache carries earlier rounding
+# differences forward): elementwise |diff| <= 4e-2 * max(|ref_i|, rms(ref)).  A single step from
+# identical state is held to 2e-2.  tests/test_oracle_noise_floor.py shows on the CPU that a second
+# fp32-accumulating implementation of the same reference sits at the same distance from the oracle.
+TRAJECTORY_REL = 4e-2
+
+
+def _margin_ulps(logits: torch.Tensor) -> float:
+    """top1 - top2 of bf16 logits, in bf16 ulps of the top logit."""
+    top = torch.topk(logits.float().cpu(), 2).values
+    return float((top[0] - top[1]) / 2.0 ** (torch.floor(torch.log2(top[0].abs())) - 7))
+
 
 def test_greedy_matches_oracle_teacher_forced(small_model):
+    """Every step is fed the oracle's token; the kernel's argmax must be the oracle's wherever the
+    oracle's own top-1 margin exceeds 2 bf16 ulps (below that, bf16 logits of two tokens are within
+    accumulation-order noise of each other and either is a valid greedy choice)."""
     shape, w, prompt = small_model
     LlamaConfig.set_shape(shape)
     cpu, gpu = pair(w, shape)
     oracle = FusedOracle(shape)
-    steps = 40
-    want = oracle.greedy(cpu, prompt, steps)
-    out = decode.decode(gpu, prompt, steps, decode_time=True)
-    got = out["new_tokens"][0].tolist()
-    assert got == want, f"first difference at {next(i for i, (a, b) in enumerate(zip(got, want)) if a != b)}"
-    # final state: residual stream and logits within bf16 rounding noise accumulated over 2 layers
-    assert (gpu.hidden_states.float().cpu() - cpu.hidden_states.float()).abs().max() <= 0.04
-    assert (gpu.logits.float().cpu() - cpu.logits.float()).abs().max() <= 0.06
-    # KV cache rows written for every position, untouched beyond
-    n = prompt.numel() + steps - 1
-    assert (gpu.k_cache[:, 0, :n].float().cpu() - cpu.k_cache[:, 0, :n].float()).abs().max() <= 0.07
+    mk = mk_kernel.get_mk()
+    seq = prompt.tolist()
+    steps, agree, close_calls = 60, 0, 0
+    for pos in range(len(seq) + steps - 1):
+        tok = seq[pos]
+        for g in (cpu, gpu):
+            g.hidden_states.copy_(g.embed_tokens[tok]); g.position_id = pos
+        oracle.decode_step(cpu)
+        mk_kernel.call_mk(gpu, mk)
+        want, got = int(cpu.logits.argmax()), int(gpu.logits.argmax())
+        if pos >= len(seq) - 1:
+            seq.append(want)
+            if got == want:
+                agree += 1
+            else:
+                close_calls += 1
+                assert _margin_ulps(cpu.logits) <= 2.0, f"step {pos}: kernel {got} vs oracle {want} at a clear margin"
+                # ... and the kernel's pick is the oracle's runner-up class: within 2 ulps of its top logit
+                top = float(cpu.logits[want]); ulp = 2.0 ** (torch.floor(torch.log2(torch.tensor(abs(top)))) - 7)
+                assert (top - float(cpu.logits[got])) / float(ulp) <= 2.0
+        rel_close(gpu.logits, cpu.logits, rel=TRAJECTORY_REL, name=f"logits@{pos}")
+    mk.check()
+    assert agree >= 0.85 * steps, (agree, close_calls)   # near-ties are ~15% of the steps at vocabulary 2048
+    rel_close(gpu.hidden_states, cpu.hidden_states, rel=TRAJECTORY_REL, name="hidden")
+    n = len(seq) - 1
+    rel_close(gpu.k_cache[:, 0, :n], cpu.k_cache[:, 0, :n], rel=TRAJECTORY_REL, name="k_cache")
+    rel_close(gpu.v_cache[:, 0, :n], cpu.v_cache[:, 0, :n], rel=TRAJECTORY_REL, name="v_cache")
     assert (gpu.k_cache[:, 0, n:] == 0).all() and (gpu.v_cache[:, 0, n:] == 0).all()
+    assert int(gpu.barriers.abs().sum()) == 0   # the kernel cleared its counters itself
+
+
+def test_decode_loop_timing_and_counters(small_model):
+    shape, w, prompt = small_model
+    LlamaConfig.set_shape(shape)
+    _, gpu = pair(w, shape)
+    steps = 24
+    out = decode.decode(gpu, prompt, steps, decode_time=True)
+    assert out["new_tokens"].shape == (1, steps)
     t = out["timing"]
     assert t["kernel_steps"] == steps - 1 and t["kernel_tok_s"] > 0 and t["decode_window_new_tokens"] == steps - 1
-    # the kernel cleared its counters itself
+    assert t["mk_kernel_gpu_s"] <= t["decode_gpu_s"] * 1.001
     assert int(gpu.barriers.abs().sum()) == 0
+    # the same request again gives the same tokens (the counters really were reset, no stale state)
+    again = decode.decode(gpu, prompt, steps, decode_time=False)
+    assert torch.equal(again["new_tokens"], out["new_tokens"])
 
 
 def test_rel_err_per_layer_and_top1(small_model):
@@ -56,13 +100,12 @@ def test_rel_err_per_layer_and_top1(small_model):
             gpu.hidden_states.copy_(start); gpu.k_cache.copy_(kv[0]); gpu.v_cache.copy_(kv[1])
             gpu.barriers.zero_()
             mk_kernel.run_instructions(gpu, sched.instruction_list(nl), mk=mk)
-            ref = per_layer[nl - 1].float()
-            got = gpu.hidden_states.float().cpu()
-            big = ref.abs() > 0.05
-            assert ((got - ref).abs()[big] / ref.abs()[big]).max() <= 2e-2
-            assert (got - ref).abs()[~big].max() <= 2e-3
+            rel_close(gpu.hidden_states, per_layer[nl - 1], rel=TRAJECTORY_REL if pos else 2e-2,
+                      name=f"hidden after layer {nl - 1} @pos {pos}")
         gpu.barriers.zero_()
-        assert int(gpu.logits.argmax()) == int(cpu.logits.argmax())
+        if _margin_ulps(cpu.logits) > 2.0:
+            assert int(gpu.logits.argmax()) == int(cpu.logits.argmax())
+        rel_close(gpu.logits, cpu.logits, rel=TRAJECTORY_REL, name=f"logits @pos {pos}")
         gpu.instructions = None
     mk.check()
 
@@ -84,6 +127,9 @@ def test_reference_built_instruction_stream_runs_unchanged(small_model):
             g.hidden_states.copy_(g.embed_tokens[tok]); g.position_id = pos
         oracle.decode_step(cpu)
         mk_kernel.call_mk(gpu, mk)
-        assert int(gpu.logits.argmax()) == int(cpu.logits.argmax())
+        if _margin_ulps(cpu.logits) > 2.0:
+            assert int(gpu.logits.argmax()) == int(cpu.logits.argmax())
+        # the K-sliced down projection rounds four times per row: a wider, but still bf16-sized, band
+        rel_close(gpu.logits, cpu.logits, rel=6e-2, name=f"logits @pos {pos}")
     mk.check()
-    assert (gpu.hidden_states.float().cpu() - cpu.hidden_states.float()).abs().max() <= 0.1
+    rel_close(gpu.hidden_states, cpu.hidden_states, rel=6e-2, name="hidden")

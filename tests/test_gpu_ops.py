@@ -11,7 +11,7 @@ import dataclasses
 import pytest
 import torch
 
-from gpu_helpers import bf16_close, pair, run_both, sync_state
+from gpu_helpers import bf16_close, pair, rel_close, run_both, sync_state
 from qimeng_megakernel_amd import synthetic
 from qimeng_megakernel_amd.decode_schedule.instructions import instruction_defs as D
 from qimeng_megakernel_amd.decode_schedule.instructions import scheduler as S
@@ -84,8 +84,14 @@ def test_op_oproj(state, which):
     cpu.barriers[0, 2, 0] = shape.num_attention_heads
     sync_state(cpu, gpu)
     run_both(cpu, gpu, sched, sched.oproj(0))
-    bf16_close(gpu.hidden_states, cpu.hidden_states, name="hidden")
+    # addends (hidden ~0.7, projection ~0.9) are O(1): 1 ulp at magnitude 1, wherever the sum lands
+    bf16_close(gpu.hidden_states, cpu.hidden_states, floor=1.0, name="hidden")
     assert torch.equal(gpu.barriers.cpu(), cpu.barriers)
+    # from a zero residual the result is the rounded projection itself: 1 ulp at its own magnitude
+    cpu.hidden_states.zero_(); cpu.barriers.zero_(); cpu.barriers[0, 2, 0] = shape.num_attention_heads
+    sync_state(cpu, gpu)
+    run_both(cpu, gpu, sched, sched.oproj(0))
+    bf16_close(gpu.hidden_states, cpu.hidden_states, name="projection")
 
 
 @pytest.mark.parametrize("which", ["mi355x", "reference"])
@@ -108,12 +114,19 @@ def test_op_down(state, which):
     sync_state(cpu, gpu)
     run_both(cpu, gpu, sched, sched.downproj(0))
     if which == "mi355x":
-        bf16_close(gpu.hidden_states, cpu.hidden_states, name="hidden")
+        bf16_close(gpu.hidden_states, cpu.hidden_states, floor=1.0, name="hidden")
     else:
-        # four K slices arrive in any order, each add rounds to bf16: the legal results span a few ulps
-        # (the reference gates this with an arrival-order envelope, verifier/common/reduction_order.py:161-243)
-        bf16_close(gpu.hidden_states, cpu.hidden_states, ulps=3.0, frac=0.5, name="hidden")
+        # four K slices arrive in any order and every add rounds to bf16: the legal results span a
+        # few ulps of the addends' magnitude (the reference gates this with an arrival-order
+        # envelope, verifier/common/reduction_order.py:161-243)
+        bf16_close(gpu.hidden_states, cpu.hidden_states, ulps=3.0, frac=0.6, floor=1.0, name="hidden")
     assert torch.equal(gpu.barriers.cpu(), cpu.barriers)
+    if which == "mi355x":
+        cpu.hidden_states.zero_(); cpu.barriers.zero_()
+        cpu.barriers[0, 4, : sched.geometry.num_split_k(shape)] = sched.expected_counts()[2]
+        sync_state(cpu, gpu)
+        run_both(cpu, gpu, sched, sched.downproj(0))
+        bf16_close(gpu.hidden_states, cpu.hidden_states, name="projection")
 
 
 @pytest.mark.parametrize("which", ["mi355x", "reference"])
@@ -133,9 +146,10 @@ def test_whole_layer_and_counters(state, which):
     sched = _sched(shape, which, P=5)
     sync_state(cpu, gpu)
     run_both(cpu, gpu, sched, sched.instruction_list())
-    tol = dict(ulps=2.0, frac=0.2) if which == "mi355x" else dict(ulps=6.0, frac=0.7)
-    bf16_close(gpu.hidden_states, cpu.hidden_states, name="hidden", **tol)
-    assert (gpu.logits.float().cpu() - cpu.logits.float()).abs().max() < 0.1
+    # one layer from identical state; the reference geometry's four rounded K slices widen the band
+    rel = 2e-2 if which == "mi355x" else 4e-2
+    rel_close(gpu.hidden_states, cpu.hidden_states, rel=rel, name="hidden")
+    rel_close(gpu.logits, cpu.logits, rel=rel, name="logits")
     assert torch.equal(gpu.barriers.cpu(), cpu.barriers)
 
 
