@@ -66,11 +66,24 @@ enum {
   QMK_QUERY_MAX_PARTIALS = 6       /* largest split-KV fan-out the kernel merges */
 };
 
+/* Rows of `barriers` per layer that QMK_FLAG_XCD_COUNTERS needs (with 48 slots). */
+#define QMK_XCD_COUNTER_ROWS 26
+
 /* Flags. */
 #define QMK_FLAG_KEEP_BARRIERS 1u  /* leave the final counter values in `barriers`
                                       (the reference's behaviour); by default the
                                       last workgroup to retire clears them so the
                                       host needs no barriers.zero_() per step.   */
+#define QMK_FLAG_XCD_COUNTERS 2u   /* the three all-to-all edges of a layer (O-proj -> up/gate,
+                                      up/gate -> down, down -> next QKV / LM head) count
+                                      arrivals on eight sub-counters, one 128-byte line per
+                                      XCD, kept in rows 10.. of each layer of `barriers`;
+                                      consumers poll the eight lines and sum them.  Needs
+                                      num_layer_barriers * barrier_slots >= 10 * barrier_slots
+                                      + 768 ints, a 128-byte aligned `barriers` with a layer
+                                      stride that is a multiple of 128 bytes, and a schedule
+                                      that does not split the down projection along K.  Rows
+                                      3..5 of the reference protocol stay zero in this mode. */
 
 /*
  * One decode step.  Tensor order and meaning follow mk(...) of the reference
@@ -125,9 +138,10 @@ typedef struct QmkArgs {
   int32_t upgate_blocks_per_bucket;/* split_k / upgate_tile_n                     */
   int32_t down_arrivals;           /* (H / down_tile_n) * (F / split_k)           */
 
-  uint64_t* timeline;              /* optional u64 [num_queues, num_insts, 4] device
-                                      buffer: start / after-wait / end timestamps
-                                      (100 MHz ticks) + opcode per instruction; NULL = off */
+  uint64_t* timeline;              /* optional u64 [num_queues, num_insts, 8] device
+                                      buffer, per instruction: start, after-wait, end
+                                      (100 MHz ticks), opcode | layer << 8, and four
+                                      op-specific intermediate stamps; NULL = off */
   void* stream;                    /* hipStream_t; NULL = the null stream         */
 } QmkArgs;
 

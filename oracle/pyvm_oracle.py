@@ -200,23 +200,31 @@ class InstructionVM:
         g.attn_lse_intermediates[h0:h1, ins.partial_idx] = lse2
         g.attn_out_intermediates[h0:h1, ins.partial_idx] = out
         g.barriers[ins.layer_idx, ROW_SPLITKV, h0:h1] += 1
+        # Extension of this build's schedules (operand word 5, zero in the reference's streams):
+        # the arrival that completes the head group merges all partials itself.
+        if getattr(ins, "merge_in_last", 0) and int(g.barriers[ins.layer_idx, ROW_SPLITKV, h0]) == ins.num_partials:
+            self._merge(g, ins.layer_idx, h0, list(range(ins.num_partials)), True, 0)
 
     # ---- 3 --------------------------------------------------------------------
     def decode_attention_reduction(self, g: Any, ins: Any) -> None:
         s = self.shape
         h0 = ins.head_start_idx
-        h1 = h0 + s.attn_reduction_size
         assert int(g.barriers[ins.layer_idx, ROW_SPLITKV, h0]) == ins.num_partials
-        idx = torch.tensor(ins.reduction_list, dtype=torch.long)
+        self._merge(g, ins.layer_idx, h0, ins.reduction_list, ins.is_terminal, ins.output_partial_idx)
+
+    def _merge(self, g: Any, layer: int, h0: int, reduction_list, is_terminal, output_partial_idx) -> None:
+        s = self.shape
+        h1 = h0 + s.attn_reduction_size
+        idx = torch.tensor(list(reduction_list), dtype=torch.long)
         lses = g.attn_lse_intermediates[h0:h1][:, idx]
         outs = g.attn_out_intermediates[h0:h1][:, idx]
         top = lses.max(dim=-1, keepdim=True).values
         factors = (lses - top).exp2()
         denom = factors.sum(dim=-1, keepdim=True)
         merged = (outs * factors.unsqueeze(-1)).sum(dim=1) / denom
-        if ins.is_terminal:
+        if is_terminal:
             g.attn_out.view(s.num_attention_heads, -1)[h0:h1] = merged
         else:
-            g.attn_lse_intermediates[h0:h1, ins.output_partial_idx] = (top + denom.log2()).squeeze(-1)
-            g.attn_out_intermediates[h0:h1, ins.output_partial_idx] = merged
-        g.barriers[ins.layer_idx, ROW_REDUCE, 0] += s.attn_reduction_size
+            g.attn_lse_intermediates[h0:h1, output_partial_idx] = (top + denom.log2()).squeeze(-1)
+            g.attn_out_intermediates[h0:h1, output_partial_idx] = merged
+        g.barriers[layer, ROW_REDUCE, 0] += s.attn_reduction_size

@@ -39,6 +39,7 @@ __global__ __launch_bounds__(kThreads, 1) void decode_megakernel(const Params p)
     unsigned long long t_start = 0;
     if (p.timeline != nullptr && threadIdx.x == 0) {
       t_start = wall_clock64();
+      for (int k = 0; k < 4; ++k) s.stamps[k] = t_start;
     }
     switch (opcode) {
       case OP_NOOP: break;
@@ -55,11 +56,12 @@ __global__ __launch_bounds__(kThreads, 1) void decode_megakernel(const Params p)
         break;
     }
     if (p.timeline != nullptr && threadIdx.x == 0) {
-      uint64_t* rec = p.timeline + (static_cast<size_t>(blockIdx.x) * p.num_insts + i) * 4;
+      uint64_t* rec = p.timeline + (static_cast<size_t>(blockIdx.x) * p.num_insts + i) * 8;
       rec[0] = t_start;
       rec[1] = s.ctl[2] ? s.t_wait : t_start;
       rec[2] = wall_clock64();
       rec[3] = static_cast<uint64_t>(opcode) | (static_cast<uint64_t>(static_cast<uint32_t>(s.inst[1])) << 8);
+      for (int k = 0; k < 4; ++k) rec[4 + k] = s.stamps[k];
       s.ctl[2] = 0;
     }
     __syncthreads();  // s.inst and s.x are reused by the next instruction
@@ -137,6 +139,13 @@ extern "C" int qmk_decode_step(const QmkArgs* a) {
       a->rope_rows < 1)
     return QMK_ERR_SHAPE;
   if (a->pos_id < 0 || a->pos_id >= a->max_seq_len || a->pos_id >= a->rope_rows) return QMK_ERR_POSITION;
+  if (a->flags & QMK_FLAG_XCD_COUNTERS) {
+    const long layer_ints = static_cast<long>(a->num_layer_barriers) * a->barrier_slots;
+    const long needed = static_cast<long>(kHierFirstRow) * a->barrier_slots + kHierEdges * kXcds * kLineInts;
+    const bool aligned = reinterpret_cast<uintptr_t>(a->barriers) % 128 == 0 && (layer_ints * 4) % 128 == 0 &&
+                         (static_cast<long>(kHierFirstRow) * a->barrier_slots * 4) % 128 == 0;
+    if (layer_ints < needed || !aligned) return QMK_ERR_SHAPE;
+  }
 
   DeviceInfo* dev = nullptr;
   if (int rc = device_info(&dev); rc != QMK_OK) return rc;

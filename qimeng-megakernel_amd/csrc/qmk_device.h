@@ -95,9 +95,49 @@ __device__ __forceinline__ float dot8(const v4u& w, const v4u& x, float acc) {
 }
 
 // ---------------------------------------------------------- reductions ----
+// Cross-lane reductions use DPP (data-parallel primitives on the VALU operand path), not
+// ds_bpermute shuffles: a shuffle is a round trip through the LDS crossbar (~100 cycles when the
+// result is needed at once), and six dependent ones per weight row add up.
+template <int kCtrl, int kRowMask = 0xf>
+__device__ __forceinline__ float dpp_f32(float identity, float v) {
+  return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(__builtin_bit_cast(int, identity), __builtin_bit_cast(int, v),
+                                                                kCtrl, kRowMask, 0xf, false));
+}
+constexpr int kDppQuadXor1 = 0xB1;       // quad_perm:[1,0,3,2]
+constexpr int kDppQuadXor2 = 0x4E;       // quad_perm:[2,3,0,1]
+constexpr int kDppHalfMirror = 0x141;    // row_half_mirror: lane i <-> 7-i within 8 lanes
+constexpr int kDppRowShr = 0x110;        // row_shr:n = 0x110 + n
+constexpr int kDppRowBcast15 = 0x142;    // lane 15 of a row -> every lane of the next row
+constexpr int kDppRowBcast31 = 0x143;    // lane 31 -> every lane of rows 2 and 3
+
+// Sum over the 64 lanes; every lane gets the total.
 __device__ __forceinline__ float wave_sum(float v) {
-#pragma unroll
-  for (int m = 32; m >= 1; m >>= 1) v += __shfl_xor(v, m, kWaveSize);
+  v += dpp_f32<kDppRowShr + 1>(0.f, v);
+  v += dpp_f32<kDppRowShr + 2>(0.f, v);
+  v += dpp_f32<kDppRowShr + 4>(0.f, v);
+  v += dpp_f32<kDppRowShr + 8>(0.f, v);           // lane 15 of each row: the row's total
+  v += dpp_f32<kDppRowBcast15, 0xa>(0.f, v);      // rows 1 and 3 add the row before them
+  v += dpp_f32<kDppRowBcast31, 0xc>(0.f, v);      // rows 2 and 3 add rows 0..1
+  return __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), 63));
+}
+
+// Maximum over the 64 lanes; every lane gets it.
+__device__ __forceinline__ float wave_max(float v) {
+  constexpr float kNegInf = -__builtin_huge_valf();
+  v = fmaxf(v, dpp_f32<kDppRowShr + 1>(kNegInf, v));
+  v = fmaxf(v, dpp_f32<kDppRowShr + 2>(kNegInf, v));
+  v = fmaxf(v, dpp_f32<kDppRowShr + 4>(kNegInf, v));
+  v = fmaxf(v, dpp_f32<kDppRowShr + 8>(kNegInf, v));
+  v = fmaxf(v, dpp_f32<kDppRowBcast15, 0xa>(kNegInf, v));
+  v = fmaxf(v, dpp_f32<kDppRowBcast31, 0xc>(kNegInf, v));
+  return __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), 63));
+}
+
+// Sum over each aligned group of 8 lanes; every lane of the group gets the group's total.
+__device__ __forceinline__ float group8_sum(float v) {
+  v += dpp_f32<kDppQuadXor1>(0.f, v);
+  v += dpp_f32<kDppQuadXor2>(0.f, v);
+  v += dpp_f32<kDppHalfMirror>(0.f, v);
   return v;
 }
 
@@ -187,6 +227,43 @@ __device__ __forceinline__ void acquire_loads() {}
 
 __device__ __forceinline__ void publish(int32_t* ctr, int amount) {
   __hip_atomic_fetch_add(ctr, amount, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+
+// ---- per-XCD sub-counters for the all-to-all edges (QMK_FLAG_XCD_COUNTERS) ----
+// 256 workgroups adding to one word make its cache line bounce between the eight
+// XCD-local L2s; a barrier through a single counter costs ~3.8 us on MI355X, through
+// eight per-XCD lines (one writer XCD each) ~1.5 us.  Workgroup b runs on XCD b % 8.
+constexpr int kXcds = 8;
+constexpr int kLineInts = 32;              // 128-byte line
+constexpr int kHierFirstRow = 10;          // first row of the sub-counter region of a layer
+constexpr int kHierEdges = 3;              // O-proj, up/gate, down  (counter rows 3, 4, 5)
+
+__device__ __forceinline__ bool xcd_counters(const Params& p) { return (p.flags & QMK_FLAG_XCD_COUNTERS) != 0; }
+
+__device__ __forceinline__ int32_t* sub_counter(const Params& p, int layer, int row, int xcd) {
+  return p.barriers + (static_cast<size_t>(layer) * p.num_layer_barriers + kHierFirstRow) * p.barrier_slots +
+         ((row - 3) * kXcds + xcd) * kLineInts;
+}
+
+// Arrival on an all-to-all edge (counter row 3, 4 or 5, slot 0).
+__device__ __forceinline__ void arrive_all(const Params& p, int layer, int row, int amount) {
+  publish(xcd_counters(p) ? sub_counter(p, layer, row, blockIdx.x & (kXcds - 1)) : counter_ptr(p, layer, row, 0), amount);
+}
+
+// Lanes 0..7 of a wave poll the eight sub-counters until their sum reaches `expected`.
+// Must be called by at least the first 8 lanes of the wave; returns the same value in all of them.
+__device__ __forceinline__ bool poll_sub_counters(const Params& p, int layer, int row, int expected, uint32_t limit) {
+  const int32_t* mine = sub_counter(p, layer, row, threadIdx.x & (kXcds - 1));
+  uint32_t polls = 0;
+  while (true) {
+    int v = __hip_atomic_load(mine, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    v += __shfl_xor(v, 1, kXcds);
+    v += __shfl_xor(v, 2, kXcds);
+    v += __shfl_xor(v, 4, kXcds);
+    if (v >= expected) return true;
+    if (++polls > limit) return false;
+    __builtin_amdgcn_s_sleep(1);
+  }
 }
 
 // ------------------------------------------------------- row streaming ----

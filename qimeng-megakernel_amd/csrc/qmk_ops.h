@@ -33,8 +33,9 @@ struct Smem {
   float red[kWaves];
   alignas(16) u16 x[M::F];              // activation vector handed to the GEMV lanes
   float res[kResSlots];                 // per-row GEMV results awaiting the epilogue pass
-  float merge[kWaves][M::GQA][M::D + 2];  // per-wave attention state: acc[D], m, l
+  float merge[kWaves * 8][M::GQA][M::D + 4];  // attention state per lane group: acc[D], m, l (+pad)
   unsigned long long t_wait;            // timeline: when the last counter wait finished
+  unsigned long long stamps[4];         // timeline: op-specific intermediate timestamps
 };
 
 enum Opcode {
@@ -55,6 +56,12 @@ struct Ctx {
   int inst_idx;
   int opcode;
 };
+
+// Optional intermediate timestamp k (0..3) of the running instruction, thread 0 only.
+#define QMK_STAMP(k)                                                        \
+  do {                                                                      \
+    if (p.timeline != nullptr && threadIdx.x == 0) s.stamps[k] = wall_clock64(); \
+  } while (0)
 
 template <class M>
 __device__ __forceinline__ bool bad_operand(const Params& p, Smem<M>& s, const Ctx& c, int operand) {
@@ -80,6 +87,26 @@ __device__ __forceinline__ bool wg_wait(const Params& p, Smem<M>& s, const Ctx& 
   if (s.ctl[0]) return false;
   acquire_loads();
   return true;
+}
+
+// Wait on an all-to-all edge (counter row 3, 4 or 5): slot 0 of the row, or the eight
+// per-XCD sub-counters of the edge when the launch uses them.
+template <class M>
+__device__ __forceinline__ bool wg_wait_all(const Params& p, Smem<M>& s, const Ctx& c, int layer, int row, int slot, int expected) {
+  if (!xcd_counters(p))
+    return wg_wait(p, s, c, 1, [&](int) { return counter_ptr(p, layer, row, slot); }, expected);
+  if (threadIdx.x < kXcds) {
+    if (!poll_sub_counters(p, layer, row, expected, p.spin_limit) && threadIdx.x == 0) {
+      s.ctl[0] = 1;
+      report_error(p, QMK_DEV_WAIT_TIMEOUT, c.inst_idx, c.opcode, row);
+    }
+  }
+  if (p.timeline != nullptr && threadIdx.x == 0) {
+    s.t_wait = wall_clock64();
+    s.ctl[2] = 1;
+  }
+  __syncthreads();
+  return s.ctl[0] == 0;
 }
 
 // RMSNorm of the residual stream into s.x as bf16:
@@ -117,42 +144,35 @@ __device__ __forceinline__ uint32_t rope_pair(float v0, float v1, const float* c
   return static_cast<uint32_t>(f2bf(o0)) | (static_cast<uint32_t>(f2bf(o1)) << 16);
 }
 
-// Row-pair streaming shared by the K = hidden GEMVs: wave w takes units w, w+8, ...;
-// a unit is two weight rows (`rows(unit, r0, r1)`), double-buffered so that 16 loads
-// of 16 bytes per lane are in flight.  `a0/a1` may already hold unit `wave` (issued
-// before the counter wait).  Results go to `emit(unit, sum0, sum1)` on lane 0.
-template <int CH, class Rows, class Emit>
-__device__ __forceinline__ void stream_pairs(int nunits, Rows rows, const v4u (&x)[CH], RowRegs<CH>& a0, RowRegs<CH>& a1,
-                                             Emit emit) {
+// ------------------------------------------------------------ streaming ----
+constexpr int kDepth = 4;  // row buffers per wave: 4 x CH x 16 B per lane in flight
+
+// Wave w consumes elements w, w+8, w+16, ... of a sequence of weight-row segments
+// (`src(e)` = address of CH*512 bf16).  `buf[k]` must already hold element w + 8k
+// (issued by `preload` before the counter wait); each buffer is refilled with the
+// element 32 further on as soon as it has been consumed.  `use(e, buf)` gets the
+// raw registers of element e.
+template <int CH, class Src>
+__device__ __forceinline__ void preload(int n, Src src, RowRegs<CH> (&buf)[kDepth]) {
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-  RowRegs<CH> b0, b1;
-  int u = wave;
-  while (u < nunits) {
-    int un = u + kWaves;
-    if (un < nunits) {
-      const u16 *r0, *r1;
-      rows(un, r0, r1);
-      load_row(b0, r0, lane);
-      load_row(b1, r1, lane);
+#pragma unroll
+  for (int k = 0; k < kDepth; ++k)
+    if (wave + k * kWaves < n) load_row(buf[k], src(wave + k * kWaves), lane);
+}
+
+template <int CH, class Src, class Use>
+__device__ __forceinline__ void stream(int n, Src src, RowRegs<CH> (&buf)[kDepth], Use use) {
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  for (int e = wave; e < n; e += kDepth * kWaves) {
+#pragma unroll
+    for (int k = 0; k < kDepth; ++k) {
+      const int ek = e + k * kWaves;
+      if (ek < n) {
+        use(ek, buf[k]);
+        const int nx = ek + kDepth * kWaves;
+        if (nx < n) load_row(buf[k], src(nx), lane);
+      }
     }
-    {
-      const float s0 = wave_sum(dot_row(a0, x)), s1 = wave_sum(dot_row(a1, x));
-      if (lane == 0) emit(u, s0, s1);
-    }
-    u = un;
-    if (u >= nunits) break;
-    un = u + kWaves;
-    if (un < nunits) {
-      const u16 *r0, *r1;
-      rows(un, r0, r1);
-      load_row(a0, r0, lane);
-      load_row(a1, r1, lane);
-    }
-    {
-      const float s0 = wave_sum(dot_row(b0, x)), s1 = wave_sum(dot_row(b1, x));
-      if (lane == 0) emit(u, s0, s1);
-    }
-    u = un;
   }
 }
 
@@ -168,31 +188,22 @@ __device__ bool op_rms_qkv_rope(const Params& p, Smem<M>& s, const Ctx& c) {
   if (nstart < 0 || nend < nstart || static_cast<long>(nend) * tile > M::QKV) return bad_operand(p, s, c, 4);
   if ((nend - nstart) * tile > kResSlots) return bad_operand(p, s, c, 3);
 
-  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-  const int rs = nstart * tile;
-  const int nunits = (nend - nstart) * tile / 2;
-  const u16* W = p.qkv_w + static_cast<size_t>(layer) * M::QKV * M::H;
-  auto rows = [&](int unit, const u16*& r0, const u16*& r1) {
-    r0 = W + static_cast<size_t>(rs + 2 * unit) * M::H;
-    r1 = r0 + M::H;
-  };
+  const int lane = threadIdx.x & 63;
+  const int rs = nstart * tile, nrows = (nend - nstart) * tile;
+  const u16* W = p.qkv_w + (static_cast<size_t>(layer) * M::QKV + rs) * M::H;
+  auto src = [&](int r) { return W + static_cast<size_t>(r) * M::H; };
 
-  RowRegs<CH> a0, a1;
-  if (wave < nunits) {  // in flight while the counter is polled
-    const u16 *r0, *r1;
-    rows(wave, r0, r1);
-    load_row(a0, r0, lane);
-    load_row(a1, r1, lane);
-  }
+  RowRegs<CH> buf[kDepth];
+  preload<CH>(nrows, src, buf);  // in flight while the counter is polled
   if (layer > 0) {
-    if (!wg_wait(p, s, c, 1, [&](int) { return counter_ptr(p, layer - 1, ROW_DOWN, 0); }, p.down_arrivals)) return false;
+    if (!wg_wait_all(p, s, c, layer - 1, ROW_DOWN, 0, p.down_arrivals)) return false;
   }
   rms_to_lds(p, s, p.hidden, p.attn_norm + static_cast<size_t>(layer) * M::H);
   v4u x[CH];
   load_x_from_lds(x, s.x, lane);
-  stream_pairs<CH>(nunits, rows, x, a0, a1, [&](int unit, float s0, float s1) {
-    s.res[2 * unit] = s0;
-    s.res[2 * unit + 1] = s1;
+  stream<CH>(nrows, src, buf, [&](int r, const RowRegs<CH>& w) {
+    const float sum = wave_sum(dot_row(w, x));
+    if (lane == 0) s.res[r] = sum;
   });
   __syncthreads();
 
@@ -200,9 +211,9 @@ __device__ bool op_rms_qkv_rope(const Params& p, Smem<M>& s, const Ctx& c) {
   const float* cosr = p.rope_cos + static_cast<size_t>(p.pos_id) * M::D;
   const float* sinr = p.rope_sin + static_cast<size_t>(p.pos_id) * M::D;
   const size_t kv_row = (static_cast<size_t>(layer) * p.max_seq_len + p.pos_id) * (M::NKV * M::D);
-  for (int unit = threadIdx.x; unit < nunits; unit += kThreads) {
-    const int r = rs + 2 * unit;
-    const float v0 = round_bf16(s.res[2 * unit]), v1 = round_bf16(s.res[2 * unit + 1]);
+  for (int pair = threadIdx.x; pair < nrows / 2; pair += kThreads) {
+    const int r = rs + 2 * pair;
+    const float v0 = round_bf16(s.res[2 * pair]), v1 = round_bf16(s.res[2 * pair + 1]);
     if (r < M::NQ * M::D) {
       st_shared32(p.q_post_rope + r, rope_pair(v0, v1, cosr, sinr, r % M::D));
     } else if (r < (M::NQ + M::NKV) * M::D) {
@@ -228,23 +239,93 @@ __device__ bool op_rms_qkv_rope(const Params& p, Smem<M>& s, const Ctx& c) {
   return true;
 }
 
+// Log-sum-exp merge of `n` split-KV partials (slot indices `list[i]`, or 0..n-1 when
+// list is null) for the GQA heads head0..head0+3 (python_vm.py:439-488).  Thread
+// (h, d/2) of the first 128 produces two neighbouring output dims.  All partial
+// reads are issued before the first use so that they overlap.
+template <class M>
+__device__ __forceinline__ void merge_partials(const Params& p, int head0, int n, const int32_t* list, bool terminal,
+                                               int out_slot) {
+  if (threadIdx.x >= M::GQA * M::D / 2) return;
+  const int h = head0 + threadIdx.x / (M::D / 2), d = 2 * (threadIdx.x % (M::D / 2));
+  const float* lse = p.attn_lse + static_cast<size_t>(h) * p.max_splits;
+  const float* part = p.attn_partial + static_cast<size_t>(h) * p.max_splits * M::D + d;
+  float e[kMaxPartials];
+  uint64_t two[kMaxPartials];
+#pragma unroll
+  for (int i = 0; i < kMaxPartials; ++i) {
+    if (i < n) {
+      const int j = list ? list[i] : i;
+      e[i] = ld_shared_f32(lse + j);
+      two[i] = ld_shared64(part + static_cast<size_t>(j) * M::D);
+    }
+  }
+  float mx = -INFINITY;
+#pragma unroll
+  for (int i = 0; i < kMaxPartials; ++i)
+    if (i < n) mx = fmaxf(mx, e[i]);
+  float num0 = 0.f, num1 = 0.f, den = 0.f;
+#pragma unroll
+  for (int i = 0; i < kMaxPartials; ++i) {
+    if (i < n) {
+      const float f = (e[i] == -INFINITY) ? 0.f : exp2f(e[i] - mx);
+      num0 = __builtin_fmaf(__uint_as_float(static_cast<uint32_t>(two[i])), f, num0);
+      num1 = __builtin_fmaf(__uint_as_float(static_cast<uint32_t>(two[i] >> 32)), f, num1);
+      den += f;
+    }
+  }
+  const float o0 = den > 0.f ? num0 / den : 0.f, o1 = den > 0.f ? num1 / den : 0.f;
+  if (terminal) {
+    st_shared32(p.attn_out + h * M::D + d, static_cast<uint32_t>(f2bf(o0)) | (static_cast<uint32_t>(f2bf(o1)) << 16));
+  } else {
+    float* dst = p.attn_partial + (static_cast<size_t>(h) * p.max_splits + out_slot) * M::D + d;
+    st_shared_f32(dst, o0);
+    st_shared_f32(dst + 1, o1);
+    if (d == 0) st_shared_f32(p.attn_lse + static_cast<size_t>(h) * p.max_splits + out_slot, den > 0.f ? mx + log2f(den) : -INFINITY);
+  }
+}
+
 // ===================================================================== 2 ==
-// [2, layer, kv_head, num_partials, partial_idx]
+// [2, layer, kv_head, num_partials, partial_idx, merge_in_last]
 // Flash-decoding over one contiguous slice of the context for the GQA group of
 // one KV head.  A wave handles 8 tokens per pass: lane group g = lane/8 owns a
 // token, lane c = lane%8 owns dims 8c..8c+7 of K and V.  Every lane group keeps
 // its own running (max, sum, acc) per query head; groups, then waves, are
 // merged once at the end.  Scores live in the log2 domain.
+//
+// merge_in_last (an extension; 0 in streams built by the reference scheduler): the
+// workgroup whose arrival completes the head group's counter merges all partials
+// itself and publishes on the reduction row, so no separate reduction instruction
+// (and no second wait) is needed.
 template <class M>
 __device__ bool op_attn_splitkv(const Params& p, Smem<M>& s, const Ctx& c) {
   static_assert(M::D == 64 && M::GQA == 4, "lane mapping assumes head_dim 64 and 4 query heads per KV head");
   const int layer = s.inst[1], kvh = s.inst[2], P = s.inst[3], part = s.inst[4];
+  const bool merge_in_last = s.inst[5] != 0;
   if (layer < 0 || layer >= p.num_layers) return bad_operand(p, s, c, 1);
   if (kvh < 0 || kvh >= M::NKV) return bad_operand(p, s, c, 2);
   if (P < 1 || P > p.max_splits || part < 0 || part >= P) return bad_operand(p, s, c, 3);
+  if (merge_in_last && P > kMaxPartials) return bad_operand(p, s, c, 3);
 
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int grp = lane >> 3, col = lane & 7;
+
+  // Context slice of this partial (python_vm.py:391-401).
+  const int seq_len = p.pos_id + 1;
+  const int total_blocks = (seq_len + M::KV_BLOCK - 1) / M::KV_BLOCK;
+  const int bpp = (total_blocks + P - 1) / P;
+  const int t0 = min(part * bpp, total_blocks) * M::KV_BLOCK;
+  const int t1 = min(min((part + 1) * bpp, total_blocks) * M::KV_BLOCK, seq_len);
+
+  // Rows of earlier positions do not depend on this step: fetch the first ones now.
+  const size_t tok_stride = static_cast<size_t>(M::NKV) * M::D;
+  const size_t base = static_cast<size_t>(layer) * p.max_seq_len * tok_stride + static_cast<size_t>(kvh) * M::D + col * 8;
+  int t = t0 + wave * 8 + grp;
+  v4u kv = {0, 0, 0, 0}, vv = {0, 0, 0, 0};
+  if (t < t1 && t != p.pos_id) {
+    kv = *reinterpret_cast<const v4u*>(p.k_cache + base + static_cast<size_t>(t) * tok_stride);
+    vv = *reinterpret_cast<const v4u*>(p.v_cache + base + static_cast<size_t>(t) * tok_stride);
+  }
 
   if (!wg_wait(p, s, c, M::GQA + 2,
                [&](int i) {
@@ -254,25 +335,27 @@ __device__ bool op_attn_splitkv(const Params& p, Smem<M>& s, const Ctx& c) {
                p.qkv_blocks_per_head))
     return false;
 
-  // Context slice of this partial (python_vm.py:391-401).
-  const int seq_len = p.pos_id + 1;
-  const int total_blocks = (seq_len + M::KV_BLOCK - 1) / M::KV_BLOCK;
-  const int bpp = (total_blocks + P - 1) / P;
-  const int t0 = min(part * bpp, total_blocks) * M::KV_BLOCK;
-  const int t1 = min(min((part + 1) * bpp, total_blocks) * M::KV_BLOCK, seq_len);
-
   // q[h][8]: this lane's dims of the four query heads, pre-scaled into the log2 domain.
   const float qscale = p.attn_scale * 1.4426950408889634f;
   float q[M::GQA][8];
+  {
+    v4u qv[M::GQA];
 #pragma unroll
-  for (int h = 0; h < M::GQA; ++h) {
-    const v4u qv = ld_shared128(p.q_post_rope + (kvh * M::GQA + h) * M::D + col * 8);
-    q[h][0] = bf_lo(qv.x) * qscale; q[h][1] = bf_hi(qv.x) * qscale;
-    q[h][2] = bf_lo(qv.y) * qscale; q[h][3] = bf_hi(qv.y) * qscale;
-    q[h][4] = bf_lo(qv.z) * qscale; q[h][5] = bf_hi(qv.z) * qscale;
-    q[h][6] = bf_lo(qv.w) * qscale; q[h][7] = bf_hi(qv.w) * qscale;
+    for (int h = 0; h < M::GQA; ++h) qv[h] = ld_shared128(p.q_post_rope + (kvh * M::GQA + h) * M::D + col * 8);
+    if (t < t1 && t == p.pos_id) {  // the row another workgroup appended during this launch
+      kv = ld_shared128(p.k_cache + base + static_cast<size_t>(t) * tok_stride);
+      vv = ld_shared128(p.v_cache + base + static_cast<size_t>(t) * tok_stride);
+    }
+#pragma unroll
+    for (int h = 0; h < M::GQA; ++h) {
+      q[h][0] = bf_lo(qv[h].x) * qscale; q[h][1] = bf_hi(qv[h].x) * qscale;
+      q[h][2] = bf_lo(qv[h].y) * qscale; q[h][3] = bf_hi(qv[h].y) * qscale;
+      q[h][4] = bf_lo(qv[h].z) * qscale; q[h][5] = bf_hi(qv[h].z) * qscale;
+      q[h][6] = bf_lo(qv[h].w) * qscale; q[h][7] = bf_hi(qv[h].w) * qscale;
+    }
   }
 
+  QMK_STAMP(0);  // q (and the appended row) have arrived
   float m[M::GQA], l[M::GQA], acc[M::GQA][8];
 #pragma unroll
   for (int h = 0; h < M::GQA; ++h) {
@@ -282,17 +365,19 @@ __device__ bool op_attn_splitkv(const Params& p, Smem<M>& s, const Ctx& c) {
     for (int i = 0; i < 8; ++i) acc[h][i] = 0.f;
   }
 
-  const size_t tok_stride = static_cast<size_t>(M::NKV) * M::D;
-  const size_t base = static_cast<size_t>(layer) * p.max_seq_len * tok_stride + static_cast<size_t>(kvh) * M::D + col * 8;
-  for (int t = t0 + wave * 8 + grp; t < t1; t += kWaves * 8) {
-    const size_t off = base + static_cast<size_t>(t) * tok_stride;
-    v4u kv, vv;
-    if (t == p.pos_id) {  // the row another workgroup appended during this launch
-      kv = ld_shared128(p.k_cache + off);
-      vv = ld_shared128(p.v_cache + off);
-    } else {
-      kv = *reinterpret_cast<const v4u*>(p.k_cache + off);
-      vv = *reinterpret_cast<const v4u*>(p.v_cache + off);
+  while (t < t1) {
+    // next token of this lane group, fetched while the current one is scored
+    const int tn = t + kWaves * 8;
+    v4u kn = {0, 0, 0, 0}, vn = {0, 0, 0, 0};
+    if (tn < t1) {
+      const size_t off = base + static_cast<size_t>(tn) * tok_stride;
+      if (tn == p.pos_id) {
+        kn = ld_shared128(p.k_cache + off);
+        vn = ld_shared128(p.v_cache + off);
+      } else {
+        kn = *reinterpret_cast<const v4u*>(p.k_cache + off);
+        vn = *reinterpret_cast<const v4u*>(p.v_cache + off);
+      }
     }
     const float k[8] = {bf_lo(kv.x), bf_hi(kv.x), bf_lo(kv.y), bf_hi(kv.y), bf_lo(kv.z), bf_hi(kv.z), bf_lo(kv.w), bf_hi(kv.w)};
     const float v[8] = {bf_lo(vv.x), bf_hi(vv.x), bf_lo(vv.y), bf_hi(vv.y), bf_lo(vv.z), bf_hi(vv.z), bf_lo(vv.w), bf_hi(vv.w)};
@@ -301,10 +386,7 @@ __device__ bool op_attn_splitkv(const Params& p, Smem<M>& s, const Ctx& c) {
       float sc = 0.f;
 #pragma unroll
       for (int i = 0; i < 8; ++i) sc = __builtin_fmaf(q[h][i], k[i], sc);
-      // The 8 lanes of a group always take the same branch, so the shuffles stay inside the group.
-      sc += __shfl_xor(sc, 1, kWaveSize);
-      sc += __shfl_xor(sc, 2, kWaveSize);
-      sc += __shfl_xor(sc, 4, kWaveSize);
+      sc = group8_sum(sc);  // the 8 lanes of a group always take the same branch
       const float mn = fmaxf(m[h], sc);
       const float alpha = exp2f(m[h] - mn);   // 0 on the first token (m = -inf)
       const float pr = exp2f(sc - mn);
@@ -313,64 +395,72 @@ __device__ bool op_attn_splitkv(const Params& p, Smem<M>& s, const Ctx& c) {
       for (int i = 0; i < 8; ++i) acc[h][i] = __builtin_fmaf(acc[h][i], alpha, pr * v[i]);
       m[h] = mn;
     }
+    t = tn;
+    kv = kn;
+    vv = vn;
   }
 
-  // Merge the 8 token groups of the wave (lanes with equal `col`).
-#pragma unroll
-  for (int x = 8; x <= 32; x <<= 1) {
-#pragma unroll
-    for (int h = 0; h < M::GQA; ++h) {
-      const float mo = __shfl_xor(m[h], x, kWaveSize);
-      const float lo = __shfl_xor(l[h], x, kWaveSize);
-      const float mn = fmaxf(m[h], mo);
-      const float a = (m[h] == -INFINITY) ? 0.f : exp2f(m[h] - mn);
-      const float b = (mo == -INFINITY) ? 0.f : exp2f(mo - mn);
-      l[h] = l[h] * a + lo * b;
-#pragma unroll
-      for (int i = 0; i < 8; ++i) {
-        const float ao = __shfl_xor(acc[h][i], x, kWaveSize);
-        acc[h][i] = acc[h][i] * a + ao * b;
-      }
-      m[h] = mn;
-    }
-  }
-  if (grp == 0) {
+  QMK_STAMP(1);  // tokens scored
+  // Every lane group (8 per wave, 64 per workgroup) parks its state in LDS; thread (h, d) of the
+  // first 256 then folds the 64 states of its head.  (Folding across lanes with shuffles costs
+  // ~120 dependent LDS-crossbar round trips per wave — several microseconds.)
+  {
+    const int g = wave * 8 + grp;
 #pragma unroll
     for (int h = 0; h < M::GQA; ++h) {
-#pragma unroll
-      for (int i = 0; i < 8; ++i) s.merge[wave][h][col * 8 + i] = acc[h][i];
+      float* dst = &s.merge[g][h][col * 8];
+      *reinterpret_cast<float4*>(dst) = make_float4(acc[h][0], acc[h][1], acc[h][2], acc[h][3]);
+      *reinterpret_cast<float4*>(dst + 4) = make_float4(acc[h][4], acc[h][5], acc[h][6], acc[h][7]);
       if (col == 0) {
-        s.merge[wave][h][M::D] = m[h];
-        s.merge[wave][h][M::D + 1] = l[h];
+        s.merge[g][h][M::D] = m[h];
+        s.merge[g][h][M::D + 1] = l[h];
       }
     }
   }
   __syncthreads();
 
-  // Merge the waves: thread (h, d) of the first 256 finishes one output element.
+  // Wave h of the first four folds head h.  Lane g first turns group g's (m, l) into its weight
+  // f = 2^(m - max) and l*f (max and the denominator are wave reductions), then lane d sums column d.
   if (threadIdx.x < M::GQA * M::D) {
-    const int h = threadIdx.x / M::D, d = threadIdx.x % M::D;
-    float mx = -INFINITY;
-#pragma unroll
-    for (int w = 0; w < kWaves; ++w) mx = fmaxf(mx, s.merge[w][h][M::D]);
-    float num = 0.f, den = 0.f;
-#pragma unroll
-    for (int w = 0; w < kWaves; ++w) {
-      const float mw = s.merge[w][h][M::D];
-      const float f = (mw == -INFINITY) ? 0.f : exp2f(mw - mx);
-      num = __builtin_fmaf(s.merge[w][h][d], f, num);
-      den = __builtin_fmaf(s.merge[w][h][M::D + 1], f, den);
-    }
-    const int head = kvh * M::GQA + h;
+    static_assert(kWaves * 8 == kWaveSize && M::D == kWaveSize, "one lane per group, then one lane per dim");
+    const int h = threadIdx.x / kWaveSize;
+    const float mg = s.merge[lane][h][M::D];
+    const float mx = wave_max(mg);
+    const float f = (mg == -INFINITY) ? 0.f : exp2f(mg - mx);
+    const float den = wave_sum(s.merge[lane][h][M::D + 1] * f);
+    s.merge[lane][h][M::D + 2] = f;
+    // wave-private rows of s.merge: written and read by this wave only, LDS ops of a wave stay in order
+    float num = 0.f;
+#pragma unroll 16
+    for (int g = 0; g < kWaves * 8; ++g) num = __builtin_fmaf(s.merge[g][h][lane], s.merge[g][h][M::D + 2], num);
+    const int head = kvh * M::GQA + h, d = lane;
     const bool empty = !(den > 0.f);
     // Normalised partial output and log2-sum-exp; an empty slice contributes (0, -inf).
     st_shared_f32(p.attn_partial + (static_cast<size_t>(head) * p.max_splits + part) * M::D + d, empty ? 0.f : num / den);
     if (d == 0) st_shared_f32(p.attn_lse + static_cast<size_t>(head) * p.max_splits + part, empty ? -INFINITY : mx + log2f(den));
   }
 
+  QMK_STAMP(2);  // partial merged and stored
   release_stores();
   __syncthreads();
-  if (threadIdx.x < M::GQA) publish(counter_ptr(p, layer, ROW_SPLITKV, kvh * M::GQA + threadIdx.x), 1);
+  QMK_STAMP(3);  // stores acknowledged
+  if (!merge_in_last) {
+    if (threadIdx.x < M::GQA) publish(counter_ptr(p, layer, ROW_SPLITKV, kvh * M::GQA + threadIdx.x), 1);
+    return true;
+  }
+  // Arrive on the four head counters; whoever sees P-1 earlier arrivals is last.
+  if (threadIdx.x < M::GQA) {
+    const int prev = __hip_atomic_fetch_add(counter_ptr(p, layer, ROW_SPLITKV, kvh * M::GQA + threadIdx.x), 1,
+                                            __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    if (threadIdx.x == 0) s.ctl[3] = (prev == P - 1);
+  }
+  __syncthreads();
+  if (s.ctl[3]) {  // uniform: every partial of this head group has been acknowledged in memory
+    merge_partials<M>(p, kvh * M::GQA, P, nullptr, true, 0);
+    release_stores();
+    __syncthreads();
+    if (threadIdx.x == 0) publish(counter_ptr(p, layer, ROW_REDUCE, 0), M::GQA);
+  }
   return true;
 }
 
@@ -389,34 +479,7 @@ __device__ bool op_attn_reduce(const Params& p, Smem<M>& s, const Ctx& c) {
   if (!terminal && (out_slot < 0 || out_slot >= p.max_splits)) return bad_operand(p, s, c, 6 + n);
 
   if (!wg_wait(p, s, c, M::GQA, [&](int i) { return counter_ptr(p, layer, ROW_SPLITKV, head0 + i); }, P)) return false;
-
-  // Thread (h, d/2) merges two neighbouring output dims so that it can store one 32-bit word.
-  if (threadIdx.x < M::GQA * M::D / 2) {
-    const int h = head0 + threadIdx.x / (M::D / 2), d = 2 * (threadIdx.x % (M::D / 2));
-    const float* lse = p.attn_lse + static_cast<size_t>(h) * p.max_splits;
-    const float* part = p.attn_partial + static_cast<size_t>(h) * p.max_splits * M::D + d;
-    float mx = -INFINITY;
-    for (int i = 0; i < n; ++i) mx = fmaxf(mx, ld_shared_f32(lse + s.inst[5 + i]));
-    float num0 = 0.f, num1 = 0.f, den = 0.f;
-    for (int i = 0; i < n; ++i) {
-      const int j = s.inst[5 + i];
-      const float e = ld_shared_f32(lse + j);
-      const float f = (e == -INFINITY) ? 0.f : exp2f(e - mx);
-      const uint64_t two = ld_shared64(part + static_cast<size_t>(j) * M::D);
-      num0 = __builtin_fmaf(__uint_as_float(static_cast<uint32_t>(two)), f, num0);
-      num1 = __builtin_fmaf(__uint_as_float(static_cast<uint32_t>(two >> 32)), f, num1);
-      den += f;
-    }
-    const float o0 = den > 0.f ? num0 / den : 0.f, o1 = den > 0.f ? num1 / den : 0.f;
-    if (terminal) {
-      st_shared32(p.attn_out + h * M::D + d, static_cast<uint32_t>(f2bf(o0)) | (static_cast<uint32_t>(f2bf(o1)) << 16));
-    } else {
-      float* dst = p.attn_partial + (static_cast<size_t>(h) * p.max_splits + out_slot) * M::D + d;
-      st_shared_f32(dst, o0);
-      st_shared_f32(dst + 1, o1);
-      if (d == 0) st_shared_f32(p.attn_lse + static_cast<size_t>(h) * p.max_splits + out_slot, den > 0.f ? mx + log2f(den) : -INFINITY);
-    }
-  }
+  merge_partials<M>(p, head0, n, &s.inst[5], terminal, out_slot);
   release_stores();
   __syncthreads();
   if (threadIdx.x == 0) publish(counter_ptr(p, layer, ROW_REDUCE, 0), M::GQA);
@@ -444,22 +507,13 @@ __device__ bool op_oproj_residual(const Params& p, Smem<M>& s, const Ctx& c) {
   if (nstart < 0 || nend < nstart || static_cast<long>(nend) * tile > M::H) return bad_operand(p, s, c, 4);
   if ((nend - nstart) * tile > kResSlots) return bad_operand(p, s, c, 3);
 
-  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-  const int rs = nstart * tile;
-  const int nunits = (nend - nstart) * tile / 2;
-  const u16* W = p.o_w + static_cast<size_t>(layer) * M::H * M::H;
-  auto rows = [&](int unit, const u16*& r0, const u16*& r1) {
-    r0 = W + static_cast<size_t>(rs + 2 * unit) * M::H;
-    r1 = r0 + M::H;
-  };
+  const int lane = threadIdx.x & 63;
+  const int rs = nstart * tile, nrows = (nend - nstart) * tile;
+  const u16* W = p.o_w + (static_cast<size_t>(layer) * M::H + rs) * M::H;
+  auto src = [&](int r) { return W + static_cast<size_t>(r) * M::H; };
 
-  RowRegs<CH> a0, a1;
-  if (wave < nunits) {
-    const u16 *r0, *r1;
-    rows(wave, r0, r1);
-    load_row(a0, r0, lane);
-    load_row(a1, r1, lane);
-  }
+  RowRegs<CH> buf[kDepth];
+  preload<CH>(nrows, src, buf);
   if (!wg_wait(p, s, c, 1, [&](int) { return counter_ptr(p, layer, ROW_REDUCE, 0); }, M::NQ)) return false;
 
   static_assert(M::H == kThreads * 4, "one thread stages four elements");
@@ -467,17 +521,17 @@ __device__ bool op_oproj_residual(const Params& p, Smem<M>& s, const Ctx& c) {
   __syncthreads();
   v4u x[CH];
   load_x_from_lds(x, s.x, lane);
-  stream_pairs<CH>(nunits, rows, x, a0, a1, [&](int unit, float s0, float s1) {
-    s.res[2 * unit] = s0;
-    s.res[2 * unit + 1] = s1;
+  stream<CH>(nrows, src, buf, [&](int r, const RowRegs<CH>& w) {
+    const float sum = wave_sum(dot_row(w, x));
+    if (lane == 0) s.res[r] = sum;
   });
   __syncthreads();
-  for (int unit = threadIdx.x; unit < nunits; unit += kThreads)
-    residual_pair(p.hidden + rs + 2 * unit, s.res[2 * unit], s.res[2 * unit + 1]);
+  for (int pair = threadIdx.x; pair < nrows / 2; pair += kThreads)
+    residual_pair(p.hidden + rs + 2 * pair, s.res[2 * pair], s.res[2 * pair + 1]);
 
   release_stores();
   __syncthreads();
-  if (threadIdx.x == 0 && nend > nstart) publish(counter_ptr(p, layer, ROW_OPROJ, 0), nend - nstart);
+  if (threadIdx.x == 0 && nend > nstart) arrive_all(p, layer, ROW_OPROJ, nend - nstart);
   return true;
 }
 
@@ -497,45 +551,46 @@ __device__ bool op_rms_upgate_silu(const Params& p, Smem<M>& s, const Ctx& c) {
   for (int i = 0; i < n; ++i)
     if (s.inst[4 + i] < 0 || s.inst[4 + i] >= nblocks_total) return bad_operand(p, s, c, 4 + i);
 
-  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-  const int nunits = n * tile;  // one unit = one output element = an up row and a gate row
+  const int lane = threadIdx.x & 63;
+  const int nout = n * tile;       // output elements of this instruction
+  const int nrows = 2 * nout;      // streamed rows: element 2i = up row i, 2i+1 = gate row i
   const u16* Wu = p.up_w + static_cast<size_t>(layer) * M::F * M::H;
   const u16* Wg = p.gate_w + static_cast<size_t>(layer) * M::F * M::H;
-  auto row_of = [&](int unit) { return s.inst[4 + unit / tile] * tile + unit % tile; };
-  auto rows = [&](int unit, const u16*& r0, const u16*& r1) {
-    const size_t r = row_of(unit);
-    r0 = Wu + r * M::H;
-    r1 = Wg + r * M::H;
-  };
+  auto row_of = [&](int i) { return s.inst[4 + i / tile] * tile + i % tile; };
+  auto src = [&](int e) { return ((e & 1) ? Wg : Wu) + static_cast<size_t>(row_of(e >> 1)) * M::H; };
 
-  RowRegs<CH> a0, a1;
-  if (wave < nunits) {
-    const u16 *r0, *r1;
-    rows(wave, r0, r1);
-    load_row(a0, r0, lane);
-    load_row(a1, r1, lane);
-  }
-  if (!wg_wait(p, s, c, 1, [&](int) { return counter_ptr(p, layer, ROW_OPROJ, 0); }, p.oproj_blocks)) return false;
+  RowRegs<CH> buf[kDepth];
+  preload<CH>(nrows, src, buf);
+  if (!wg_wait_all(p, s, c, layer, ROW_OPROJ, 0, p.oproj_blocks)) return false;
   rms_to_lds(p, s, p.hidden, p.mlp_norm + static_cast<size_t>(layer) * M::H);
   v4u x[CH];
   load_x_from_lds(x, s.x, lane);
-  stream_pairs<CH>(nunits, rows, x, a0, a1, [&](int unit, float su, float sg) {
-    const float up = round_bf16(su), gate = round_bf16(sg);
-    const float act = round_bf16(gate / (1.0f + expf(-gate)));
-    s.res[unit] = act * up;  // rounded to bf16 on the way out
+  stream<CH>(nrows, src, buf, [&](int e, const RowRegs<CH>& w) {
+    const float sum = wave_sum(dot_row(w, x));
+    if (lane == 0) s.res[e] = sum;
   });
   __syncthreads();
   // Two neighbouring outputs of a tile leave as one 32-bit word.
-  for (int pair = threadIdx.x; pair < nunits / 2; pair += kThreads) {
-    const uint32_t w = static_cast<uint32_t>(f2bf(s.res[2 * pair])) | (static_cast<uint32_t>(f2bf(s.res[2 * pair + 1])) << 16);
-    st_shared32(p.silu_out + row_of(2 * pair), w);
+  for (int pair = threadIdx.x; pair < nout / 2; pair += kThreads) {
+    uint32_t word = 0;
+#pragma unroll
+    for (int k = 0; k < 2; ++k) {
+      const int i = 2 * pair + k;
+      const float up = round_bf16(s.res[2 * i]), gate = round_bf16(s.res[2 * i + 1]);
+      const float act = round_bf16(gate / (1.0f + expf(-gate)));
+      word |= static_cast<uint32_t>(f2bf(act * up)) << (16 * k);
+    }
+    st_shared32(p.silu_out + row_of(2 * pair), word);
   }
 
   release_stores();
   __syncthreads();
   // One arrival per block, on the bucket (= down-projection K slice) it belongs to.
-  if (static_cast<int>(threadIdx.x) < n)
+  if (xcd_counters(p)) {
+    if (threadIdx.x == 0 && n > 0) arrive_all(p, layer, ROW_UPGATE, n);
+  } else if (static_cast<int>(threadIdx.x) < n) {
     publish(counter_ptr(p, layer, ROW_UPGATE, s.inst[4 + threadIdx.x] / p.upgate_blocks_per_bucket), 1);
+  }
   return true;
 }
 
@@ -558,81 +613,59 @@ __device__ __forceinline__ void atomic_add_bf16(u16* addr, float delta) {
 // [6, layer, tile_M, n_start, n_end, split_K_idx, tile_M_g, tile_N_g, split_K_g]
 // hidden[r] = bf16(hidden[r] + bf16(W_d[r, slice] . silu_out[slice]))   (operations.py:285-295;
 // python_vm.py:137-171 for the sliced form).  With one slice this is the fused form exactly.
-// Wave w streams rows rs+w, rs+w+8, ... in groups of G 1-KiB chunks, double-buffered.
-template <class M, int G>
-__device__ __forceinline__ void down_rows(Smem<M>& s, const u16* W, int rs, int re, int ks, int kg, RowRegs<G>& a,
-                                          bool a_loaded) {
-  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-  const int groups = kg / (512 * G);
-  const int nrows = re - rs;
-  const int total = ((nrows - wave + kWaves - 1) / kWaves) * groups;  // (row, group) steps of this wave; <= 0 if none
-  RowRegs<G> b;
-  auto src = [&](int idx) {
-    const int row = rs + wave + (idx / groups) * kWaves;
-    return W + static_cast<size_t>(row) * M::F + ks + (idx % groups) * (512 * G);
-  };
-  float acc = 0.f;
-  auto step = [&](const RowRegs<G>& r, int idx) {
-    v4u x[G];
-    load_x_from_lds(x, s.x + (idx % groups) * (512 * G), lane);
-#pragma unroll
-    for (int j = 0; j < G; ++j) acc = dot8(r.v[j], x[j], acc);
-    if (idx % groups == groups - 1) {
-      const float sum = wave_sum(acc);
-      acc = 0.f;
-      if (lane == 0) s.res[wave + (idx / groups) * kWaves] = sum;
-    }
-  };
-  int i = 0;
-  if (total > 0 && !a_loaded) load_row(a, src(0), lane);
-  while (i < total) {
-    if (i + 1 < total) load_row(b, src(i + 1), lane);
-    step(a, i);
-    ++i;
-    if (i >= total) break;
-    if (i + 1 < total) load_row(a, src(i + 1), lane);
-    step(b, i);
-    ++i;
-  }
-}
-
+// A row's K slice is streamed as 2048-column segments: element e = (row e / segs, segment e % segs).
 template <class M>
 __device__ bool op_down_residual(const Params& p, Smem<M>& s, const Ctx& c) {
+  constexpr int CH = 4;
   const int layer = s.inst[1], nstart = s.inst[3], nend = s.inst[4], split = s.inst[5];
   const int tile = s.inst[7], kg = s.inst[8];
   if (layer < 0 || layer >= p.num_layers) return bad_operand(p, s, c, 1);
   if (tile <= 0 || (tile & 1)) return bad_operand(p, s, c, 7);
   if (nstart < 0 || nend < nstart || static_cast<long>(nend) * tile > M::H) return bad_operand(p, s, c, 4);
   if ((nend - nstart) * tile > kResSlots) return bad_operand(p, s, c, 3);
-  if (kg <= 0 || kg % 2048 != 0 || kg > M::F) return bad_operand(p, s, c, 8);
+  if (kg <= 0 || kg % (512 * CH) != 0 || kg > M::F) return bad_operand(p, s, c, 8);
   if (split < 0 || static_cast<long>(split + 1) * kg > M::F) return bad_operand(p, s, c, 5);
   if (split >= p.barrier_slots) return bad_operand(p, s, c, 5);
 
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-  const int rs = nstart * tile, re = nend * tile, ks = split * kg;
-  const u16* W = p.down_w + static_cast<size_t>(layer) * M::H * M::F;
-  const bool wide = (kg % 4096) == 0;
+  const int rs = nstart * tile, nrows = (nend - nstart) * tile, ks = split * kg;
+  const int segs = kg / (512 * CH);
+  // Element order is chosen per wave so that a wave owns whole rows: wave w streams the
+  // segments of rows w, w+8, ...  Element index e (as seen by `stream`: e = w + 8*i) maps to
+  // step i of wave w: row = w + 8*(i / segs), segment = i % segs.
+  auto row_of = [&](int e) { return (e & (kWaves - 1)) + kWaves * ((e >> 3) / segs); };
+  auto seg_of = [&](int e) { return (e >> 3) % segs; };
+  const u16* W = p.down_w + (static_cast<size_t>(layer) * M::H + rs) * M::F + ks;
+  auto src = [&](int e) { return W + static_cast<size_t>(row_of(e)) * M::F + seg_of(e) * (512 * CH); };
+  // Number of stream elements: waves with fewer rows simply run out earlier; bound by the largest.
+  const int rows_w = (nrows - wave + kWaves - 1) / kWaves;          // rows owned by this wave (may be 0)
+  const int n_elems = wave + kWaves * (rows_w * segs - 1) + 1;      // last element index of this wave + 1 (<= wave if none)
 
-  RowRegs<8> a8;
-  RowRegs<4> a4;
-  const bool have_row = rs + wave < re;
-  if (have_row) {
-    const u16* first = W + static_cast<size_t>(rs + wave) * M::F + ks;
-    if (wide) load_row(a8, first, lane);
-    else load_row(a4, first, lane);
-  }
-  if (!wg_wait(p, s, c, 1, [&](int) { return counter_ptr(p, layer, ROW_UPGATE, split); }, p.upgate_blocks_per_bucket)) return false;
+  RowRegs<CH> buf[kDepth];
+  preload<CH>(rows_w > 0 ? n_elems : 0, src, buf);
+  if (xcd_counters(p) && (split != 0 || kg != M::F)) return bad_operand(p, s, c, 8);  // sub-counters cover one K slice
+  if (!wg_wait_all(p, s, c, layer, ROW_UPGATE, split, p.upgate_blocks_per_bucket)) return false;
 
   // The K slice of silu_out into LDS.
   for (int i = threadIdx.x; i < kg / 4; i += kThreads)
     reinterpret_cast<uint64_t*>(s.x)[i] = ld_shared64(p.silu_out + ks + i * 4);
   __syncthreads();
 
-  if (wide) down_rows<M, 8>(s, W, rs, re, ks, kg, a8, have_row);
-  else down_rows<M, 4>(s, W, rs, re, ks, kg, a4, have_row);
+  float acc = 0.f;
+  stream<CH>(rows_w > 0 ? n_elems : 0, src, buf, [&](int e, const RowRegs<CH>& w) {
+    const int seg = seg_of(e);
+    v4u x[CH];
+    load_x_from_lds(x, s.x + seg * (512 * CH), lane);
+#pragma unroll
+    for (int j = 0; j < CH; ++j) acc = dot8(w.v[j], x[j], acc);
+    if (seg == segs - 1) {
+      const float sum = wave_sum(acc);
+      acc = 0.f;
+      if (lane == 0) s.res[row_of(e)] = sum;
+    }
+  });
   __syncthreads();
 
-  const int nrows = re - rs;
   if (kg == M::F) {  // one slice: every row has a single writer
     for (int pair = threadIdx.x; pair < nrows / 2; pair += kThreads)
       residual_pair(p.hidden + rs + 2 * pair, s.res[2 * pair], s.res[2 * pair + 1]);
@@ -642,7 +675,7 @@ __device__ bool op_down_residual(const Params& p, Smem<M>& s, const Ctx& c) {
 
   release_stores();
   __syncthreads();
-  if (threadIdx.x == 0 && nend > nstart) publish(counter_ptr(p, layer, ROW_DOWN, 0), nend - nstart);
+  if (threadIdx.x == 0 && nend > nstart) arrive_all(p, layer, ROW_DOWN, nend - nstart);
   return true;
 }
 
@@ -652,34 +685,25 @@ template <class M>
 __device__ bool op_rms_lmhead(const Params& p, Smem<M>& s, const Ctx& c) {
   constexpr int CH = M::H / 512;
   const int bstart = s.inst[1], bend = s.inst[2], tile = s.inst[4];
-  if (tile <= 0 || (tile & 1)) return bad_operand(p, s, c, 4);
+  if (tile <= 0) return bad_operand(p, s, c, 4);
   if (bstart < 0 || bend < bstart || static_cast<long>(bend) * tile > p.vocab_size) return bad_operand(p, s, c, 2);
   if (p.num_layers < 1) return bad_operand(p, s, c, 0);
 
-  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-  const int rs = bstart * tile;
-  const int nunits = (bend - bstart) * tile / 2;
-  const u16* W = p.lm_w;
-  auto rows = [&](int unit, const u16*& r0, const u16*& r1) {
-    r0 = W + static_cast<size_t>(rs + 2 * unit) * M::H;
-    r1 = r0 + M::H;
-  };
+  const int lane = threadIdx.x & 63;
+  const int rs = bstart * tile, nrows = (bend - bstart) * tile;
+  const u16* W = p.lm_w + static_cast<size_t>(rs) * M::H;
+  auto src = [&](int r) { return W + static_cast<size_t>(r) * M::H; };
 
-  RowRegs<CH> a0, a1;
-  if (wave < nunits) {
-    const u16 *r0, *r1;
-    rows(wave, r0, r1);
-    load_row(a0, r0, lane);
-    load_row(a1, r1, lane);
-  }
-  if (!wg_wait(p, s, c, 1, [&](int) { return counter_ptr(p, p.num_layers - 1, ROW_DOWN, 0); }, p.down_arrivals)) return false;
+  RowRegs<CH> buf[kDepth];
+  preload<CH>(nrows, src, buf);
+  if (!wg_wait_all(p, s, c, p.num_layers - 1, ROW_DOWN, 0, p.down_arrivals)) return false;
   rms_to_lds(p, s, p.hidden, p.lm_norm);
   v4u x[CH];
   load_x_from_lds(x, s.x, lane);
   // Terminal op: nothing inside the launch reads the logits, so ordinary stores do.
-  stream_pairs<CH>(nunits, rows, x, a0, a1, [&](int unit, float s0, float s1) {
-    *reinterpret_cast<uint32_t*>(p.logits + rs + 2 * unit) =
-        static_cast<uint32_t>(f2bf(s0)) | (static_cast<uint32_t>(f2bf(s1)) << 16);
+  stream<CH>(nrows, src, buf, [&](int r, const RowRegs<CH>& w) {
+    const float sum = wave_sum(dot_row(w, x));
+    if (lane == 0) p.logits[rs + r] = f2bf(sum);
   });
   return true;
 }

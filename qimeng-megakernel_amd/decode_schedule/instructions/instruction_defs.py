@@ -139,7 +139,14 @@ class RMS_QKVProj_GEMV_RoPE(Instruction):
 
 @dataclass
 class DecodeAttentionSplitKV(Instruction):
-    """One KV head, one contiguous slice of the context, all query heads of the group."""
+    """One KV head, one contiguous slice of the context, all query heads of the group.
+
+    ``merge_in_last`` extends the reference's four operands (its word is 0 in any
+    stream the reference scheduler builds): when set, the workgroup whose arrival
+    completes the head group's split-KV counter also performs the log-sum-exp
+    merge of all partials and publishes on the reduction row, so the schedule
+    carries no separate reduction instruction for that head group.
+    """
 
     OPCODE: ClassVar[int] = 2
     PREV_OPCODES: ClassVar[tuple[int, ...]] = (1,)
@@ -147,6 +154,7 @@ class DecodeAttentionSplitKV(Instruction):
     kv_head_idx: int
     num_partials: int
     partial_idx: int
+    merge_in_last: int = 0
 
 
 @dataclass

@@ -16,6 +16,7 @@ tests check.
 from __future__ import annotations
 
 import dataclasses
+import os
 from dataclasses import dataclass
 from typing import Any, Iterable, Sequence
 
@@ -142,6 +143,8 @@ class DecodeScheduler:
     geometry: TileGeometry
     sm_count: int
     num_partials: int
+    #: fold the log-sum-exp merge into the last split-KV arrival (no reduction instructions)
+    fuse_attention_merge: bool = False
 
     def __post_init__(self) -> None:
         self.geometry.validate(self.shape)
@@ -160,12 +163,14 @@ class DecodeScheduler:
 
     def attention_split_kv(self, layer_idx: int) -> list[Instruction]:
         return [
-            DecodeAttentionSplitKV(layer_idx, kv_head, self.num_partials, p)
+            DecodeAttentionSplitKV(layer_idx, kv_head, self.num_partials, p, int(self.fuse_attention_merge))
             for kv_head in range(self.shape.num_key_value_heads)
             for p in range(self.num_partials)
         ]
 
     def attention_reduction(self, layer_idx: int) -> list[Instruction]:
+        if self.fuse_attention_merge:
+            return []
         step = self.shape.attn_reduction_size
         return [
             DecodeAttentionReduction(
@@ -261,11 +266,12 @@ def mi355x_scheduler(
     sm_count: int = MI355X_CU_COUNT,
     kv_capacity: int | None = None,
     num_partials: int | None = None,
+    fuse_attention_merge: bool = True,
 ) -> DecodeScheduler:
     shape = shape or LlamaConfig.shape()
     geometry = dataclasses.replace(MI355X_GEOMETRY, split_k=shape.intermediate_size)
     p = num_partials or pick_num_partials(sm_count, kv_capacity, shape=shape)
-    return DecodeScheduler(shape, geometry, sm_count, p)
+    return DecodeScheduler(shape, geometry, sm_count, p, fuse_attention_merge)
 
 
 def scheduler_for(globs: Any) -> DecodeScheduler:
@@ -279,6 +285,9 @@ def scheduler_for(globs: Any) -> DecodeScheduler:
     if lse is not None:
         max_p = min(max_p, int(lse.shape[-1]))
     p = pick_num_partials(sm_count, kv_capacity, max_partials=max_p)
+    override = os.environ.get("QMK_NUM_PARTIALS")  # tuning knob: force the split-KV fan-out
+    if override:
+        p = max(1, min(int(override), max_p))
     if cached is not None and (cached.sm_count, cached.num_partials, cached.shape) == (sm_count, p, LlamaConfig.shape()):
         return cached
     sched = mi355x_scheduler(sm_count=sm_count, num_partials=p)

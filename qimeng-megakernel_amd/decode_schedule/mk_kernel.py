@@ -29,6 +29,8 @@ from .model_config import LlamaConfig
 _LIBRARY_NAME = "libqmk_hip.so"
 
 QMK_FLAG_KEEP_BARRIERS = 1
+QMK_FLAG_XCD_COUNTERS = 2
+QMK_XCD_COUNTER_ROWS = 26
 QMK_MODEL_LLAMA_3_2_1B = 0
 QMK_QUERY_ABI_VERSION, QMK_QUERY_CU_COUNT, QMK_QUERY_THREADS, QMK_QUERY_LDS_BYTES = 0, 1, 2, 3
 QMK_QUERY_MAX_QUEUES, QMK_QUERY_INSTRUCTION_WORDS, QMK_QUERY_MAX_PARTIALS = 4, 5, 6
@@ -129,11 +131,13 @@ class MegaKernel:
     """
 
     def __init__(self, lib: ctypes.CDLL, geometry: TileGeometry | None = None, *, reset_barriers: bool = True,
-                 spin_limit: int = 0):
+                 spin_limit: int = 0, xcd_counters: bool = True):
         self._lib = lib
         self.geometry = geometry
         self.reset_barriers = reset_barriers
         self.spin_limit = int(spin_limit)
+        self.xcd_counters = xcd_counters   # use per-XCD sub-counters when `barriers` has room for them
+        self._xcd_counters = False
         self.timeline: torch.Tensor | None = None
         self._args = QmkArgs()
         self._args.struct_size = ctypes.sizeof(QmkArgs)
@@ -162,7 +166,8 @@ class MegaKernel:
     def with_options(self, **kw: Any) -> "MegaKernel":
         other = MegaKernel(self._lib, kw.pop("geometry", self.geometry),
                            reset_barriers=kw.pop("reset_barriers", self.reset_barriers),
-                           spin_limit=kw.pop("spin_limit", self.spin_limit))
+                           spin_limit=kw.pop("spin_limit", self.spin_limit),
+                           xcd_counters=kw.pop("xcd_counters", self.xcd_counters))
         if kw:
             raise TypeError(f"unknown options {sorted(kw)}")
         return other
@@ -224,6 +229,15 @@ class MegaKernel:
         a.max_seq_len, a.max_splits, a.vocab_size, a.rope_rows = S, P, V, int(cos.shape[0])
         geometry = self.geometry or REFERENCE_GEOMETRY
         (a.qkv_blocks_per_head, a.oproj_blocks, a.upgate_blocks_per_bucket, a.down_arrivals) = geometry.expected_counts(shape)
+        # Per-XCD sub-counters for the all-to-all edges need room in `barriers` (rows 10..25 of
+        # every layer) and a schedule with a single down-projection K slice.
+        self._xcd_counters = (
+            self.xcd_counters
+            and int(barriers.shape[1]) >= QMK_XCD_COUNTER_ROWS
+            and int(barriers.shape[2]) == 48
+            and barriers.data_ptr() % 128 == 0
+            and geometry.num_split_k(shape) == 1
+        )
 
     def __call__(self, *args: Any) -> None:
         if len(args) != 25:
@@ -238,7 +252,7 @@ class MegaKernel:
         a.pos_id = int(pos_id)
         a.attn_scale = float(attn_scale)
         a.rms_norm_eps = float(rms_norm_eps)
-        a.flags = 0 if self.reset_barriers else QMK_FLAG_KEEP_BARRIERS
+        a.flags = (0 if self.reset_barriers else QMK_FLAG_KEEP_BARRIERS) | (QMK_FLAG_XCD_COUNTERS if self._xcd_counters else 0)
         a.spin_limit = self.spin_limit
         a.timeline = self.timeline.data_ptr() if self.timeline is not None else None
         a.stream = torch.cuda.current_stream(tensors[1].device).cuda_stream
@@ -251,7 +265,7 @@ _LIB_CACHE: dict[Path, ctypes.CDLL] = {}
 
 
 def get_mk(mk_dir: Path | None = None, *, geometry: TileGeometry | None = None, reset_barriers: bool = True,
-           spin_limit: int = 0) -> MegaKernel:
+           spin_limit: int = 0, xcd_counters: bool = True) -> MegaKernel:
     """Return the ``mk`` callable bound to the prebuilt library in ``mk_dir``.
 
     ``geometry`` defaults to the MI355X schedule of this package; pass
@@ -264,7 +278,7 @@ def get_mk(mk_dir: Path | None = None, *, geometry: TileGeometry | None = None, 
         _LIB_CACHE[root] = lib
     if geometry is None:
         geometry = _scheduler.mi355x_scheduler(num_partials=1).geometry
-    return MegaKernel(lib, geometry, reset_barriers=reset_barriers, spin_limit=spin_limit)
+    return MegaKernel(lib, geometry, reset_barriers=reset_barriers, spin_limit=spin_limit, xcd_counters=xcd_counters)
 
 
 def call_mk(globs: Globals, mk: Any) -> None:

@@ -24,7 +24,8 @@ import torch
 from .decode_schedule.globs import Globals
 from .decode_schedule.model_config import DecodeShape, LlamaConfig
 
-BARRIER_ROWS = 10
+BARRIER_ROWS = 10          # the reference's allocation
+XCD_COUNTER_ROWS = 26      # rows 10..25 hold the per-XCD sub-counters of the all-to-all edges
 WEIGHT_STD = 0.02
 
 
@@ -83,6 +84,7 @@ def build_globals(
     *,
     max_partials: int = 32,
     globals_cls: Any = Globals,
+    barrier_rows: int = XCD_COUNTER_ROWS,
 ) -> Any:
     """Allocate every decode buffer on ``device`` and attach the weights (moved there)."""
     device = torch.device(device)
@@ -96,7 +98,7 @@ def build_globals(
     on_device = {k: v.to(device).contiguous() for k, v in weights.items()}
     g = globals_cls(
         position_id=0,
-        barriers=zeros(L, BARRIER_ROWS, shape.num_heads, dtype=torch.int32),
+        barriers=zeros(L, barrier_rows, shape.num_heads, dtype=torch.int32),
         k_cache=zeros(L, 1, kv_capacity, nkv, d),
         v_cache=zeros(L, 1, kv_capacity, nkv, d),
         hidden_states=zeros(H),

@@ -27,11 +27,14 @@ def pair(weights, shape, kv_capacity=96, max_partials=32):
     return cpu, gpu
 
 
-def run_both(cpu, gpu, sched, instructions, *, sm_count=None):
-    """Execute the same instruction list on the CPU VM and on the kernel, counters kept."""
+def run_both(cpu, gpu, sched, instructions, *, sm_count=None, xcd_counters=False):
+    """Execute the same instruction list on the CPU VM and on the kernel, counters kept.
+
+    By default the kernel counts on the reference protocol's rows, so the counter end state can be
+    compared word for word; ``xcd_counters=True`` exercises the per-XCD sub-counters instead."""
     vm = InstructionVM(sched.shape, Counts(*sched.expected_counts()))
     vm.run(cpu, copy.deepcopy(instructions))
-    mk = mk_kernel.get_mk(geometry=sched.geometry, reset_barriers=False)
+    mk = mk_kernel.get_mk(geometry=sched.geometry, reset_barriers=False, xcd_counters=xcd_counters)
     mk_kernel.run_instructions(gpu, copy.deepcopy(instructions), mk=mk, sm_count=sm_count or sched.sm_count)
     mk.check()
     return mk

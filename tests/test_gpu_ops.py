@@ -21,8 +21,10 @@ pytestmark = pytest.mark.gpu
 
 
 def _sched(shape, which, P=3):
-    if which == "mi355x":
+    if which == "mi355x":            # fused merge: the last split-KV arrival reduces
         return S.mi355x_scheduler(shape, sm_count=256, num_partials=P)
+    if which == "mi355x_unfused":    # MI355X tiles, separate reduction instructions
+        return S.mi355x_scheduler(shape, sm_count=256, num_partials=P, fuse_attention_merge=False)
     return S.DecodeScheduler(shape, D.REFERENCE_GEOMETRY, 108, P)
 
 
@@ -57,7 +59,7 @@ def test_op_qkv_rope(state, which):
     assert torch.equal(gpu.barriers.cpu(), cpu.barriers)
 
 
-@pytest.mark.parametrize("which", ["mi355x", "reference"])
+@pytest.mark.parametrize("which", ["mi355x", "mi355x_unfused", "reference"])
 @pytest.mark.parametrize("pos,P", [(0, 1), (0, 4), (15, 2), (16, 3), (41, 3), (80, 13), (95, 25)])
 def test_op_attention_split_and_reduce(state, which, pos, P):
     shape, cpu, gpu = state
@@ -151,6 +153,26 @@ def test_whole_layer_and_counters(state, which):
     rel_close(gpu.hidden_states, cpu.hidden_states, rel=rel, name="hidden")
     rel_close(gpu.logits, cpu.logits, rel=rel, name="logits")
     assert torch.equal(gpu.barriers.cpu(), cpu.barriers)
+
+
+def test_xcd_sub_counters(state):
+    """With room in `barriers`, the all-to-all edges count on eight per-XCD lines: same results,
+    rows 3..5 of the protocol untouched, the sub-counters of an edge summing to its final count."""
+    shape, cpu, gpu = state
+    sched = _sched(shape, "mi355x", P=4)
+    sync_state(cpu, gpu)
+    run_both(cpu, gpu, sched, sched.instruction_list(), xcd_counters=True)
+    rel_close(gpu.hidden_states, cpu.hidden_states, rel=2e-2, name="hidden")
+    rel_close(gpu.logits, cpu.logits, rel=2e-2, name="logits")
+    b = gpu.barriers.cpu()
+    assert torch.equal(b[:, :3], cpu.barriers[:, :3])          # per-head rows are the plain protocol
+    assert int(b[:, 3:6].abs().sum()) == 0
+    bph, opb, ubk, dwn = sched.expected_counts()
+    for layer in range(shape.num_hidden_layers):
+        region = b[layer, 10:26].reshape(3, 8, 32)
+        assert region[:, :, 0].sum(dim=1).tolist() == [opb, ubk, dwn]
+        assert (region[:, :, 0] > 0).all()                      # every XCD took part
+        assert int(region[:, :, 1:].abs().sum()) == 0
 
 
 def test_single_queue_and_odd_queue_counts(state):

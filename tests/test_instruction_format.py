@@ -20,7 +20,8 @@ from qimeng_megakernel_amd.decode_schedule.model_config import LLAMA_3_2_1B
 
 def test_serialize_known_words():
     assert D.RMS_QKVProj_GEMV_RoPE(3, 0, 10, 12).serialize() == [1, 3, 0, 10, 12, 1, 16]
-    assert D.DecodeAttentionSplitKV(2, 5, 13, 7).serialize() == [2, 2, 5, 13, 7]
+    assert D.DecodeAttentionSplitKV(2, 5, 13, 7).serialize() == [2, 2, 5, 13, 7, 0]
+    assert D.DecodeAttentionSplitKV(2, 5, 13, 7, 1).padded()[:7] == [2, 2, 5, 13, 7, 1, 0]
     assert D.DecodeAttentionReduction(1, 8, 3, [0, 1, 2]).serialize() == [3, 1, 8, 3, 3, 0, 1, 2, 1, 0]
     assert D.OProj_GEMV_Residual(0, 0, 4, 6, 0).serialize() == [4, 0, 0, 4, 6, 0, 1, 16]
     assert D.RMS_UpGateProj_GEMV_SiLU(0, 0, [7, 115, 223]).serialize() == [5, 0, 0, 3, 7, 115, 223, 1, 16]
@@ -187,6 +188,8 @@ def _simulate(sched, num_layers):
                 ctr[i.layer_idx, 0, b // bph] += 1
         elif op == 2:
             ctr[i.layer_idx, 1, i.kv_head_idx * ratio : (i.kv_head_idx + 1) * ratio] += 1
+            if i.merge_in_last and ctr[i.layer_idx, 1, i.kv_head_idx * ratio] == i.num_partials:
+                ctr[i.layer_idx, 2, 0] += ratio
         elif op == 3:
             ctr[i.layer_idx, 2, 0] += ratio
         elif op == 4:
