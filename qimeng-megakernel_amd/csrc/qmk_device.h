@@ -266,6 +266,35 @@ __device__ __forceinline__ bool poll_sub_counters(const Params& p, int layer, in
   }
 }
 
+// 2048 lanes polling eight lines that 256 producers are still updating slow the producers
+// down.  So only one workgroup per XCD (the "leader", workgroups 0..7) polls the sub-counters;
+// when the edge is complete it raises a flag in its own XCD's line (word 1), which the other
+// workgroups of that XCD poll out of their local L2.  A follower whose leader does not show up
+// (its queue may not contain a consumer of this edge) falls back to polling the sub-counters
+// itself after kFollowerPolls tries, and raises the flag for its neighbours too.
+constexpr uint32_t kFollowerPolls = 256;
+
+__device__ __forceinline__ bool wait_edge_xcd(const Params& p, int layer, int row, int expected, uint32_t limit) {
+  const int xcd = blockIdx.x & (kXcds - 1);
+  int32_t* flag = sub_counter(p, layer, row, xcd) + 1;
+  const bool leader = blockIdx.x < kXcds || gridDim.x < 2 * kXcds;
+  bool ready = false;
+  if (!leader) {
+    for (uint32_t k = 0; k < kFollowerPolls; ++k) {
+      if (__hip_atomic_load(flag, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != 0) {
+        ready = true;
+        break;
+      }
+      __builtin_amdgcn_s_sleep(1);
+    }
+  }
+  if (!ready) {
+    ready = poll_sub_counters(p, layer, row, expected, limit);
+    if (ready && (threadIdx.x & (kXcds - 1)) == 0) __hip_atomic_store(flag, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  }
+  return ready;
+}
+
 // ------------------------------------------------------- row streaming ----
 // A wave reads one weight row of CH*512 bf16 as CH fully coalesced 1 KiB loads;
 // lane l owns columns (j*64 + l)*8 .. +7 of chunk j.

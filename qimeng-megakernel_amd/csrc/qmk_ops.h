@@ -96,7 +96,7 @@ __device__ __forceinline__ bool wg_wait_all(const Params& p, Smem<M>& s, const C
   if (!xcd_counters(p))
     return wg_wait(p, s, c, 1, [&](int) { return counter_ptr(p, layer, row, slot); }, expected);
   if (threadIdx.x < kXcds) {
-    if (!poll_sub_counters(p, layer, row, expected, p.spin_limit) && threadIdx.x == 0) {
+    if (!wait_edge_xcd(p, layer, row, expected, p.spin_limit) && threadIdx.x == 0) {
       s.ctl[0] = 1;
       report_error(p, QMK_DEV_WAIT_TIMEOUT, c.inst_idx, c.opcode, row);
     }
@@ -145,7 +145,10 @@ __device__ __forceinline__ uint32_t rope_pair(float v0, float v1, const float* c
 }
 
 // ------------------------------------------------------------ streaming ----
-constexpr int kDepth = 4;  // row buffers per wave: 4 x CH x 16 B per lane in flight
+#ifndef QMK_DEPTH
+#define QMK_DEPTH 4
+#endif
+constexpr int kDepth = QMK_DEPTH;  // row buffers per wave: 4 x CH x 16 B per lane in flight
 
 // Wave w consumes elements w, w+8, w+16, ... of a sequence of weight-row segments
 // (`src(e)` = address of CH*512 bf16).  `buf[k]` must already hold element w + 8k

@@ -243,6 +243,8 @@ class MegaKernel:
         if len(args) != 25:
             raise TypeError(f"mk takes 22 tensors and 3 scalars (25 positional arguments), got {len(args)}")
         tensors, (pos_id, attn_scale, rms_norm_eps) = args[:22], args[22:]
+        if isinstance(tensors[0], torch.Tensor) and tensors[0].numel() == 0:
+            return  # empty queues: nothing to launch
         key = tuple((t.data_ptr(), tuple(t.shape)) if isinstance(t, torch.Tensor) else None for t in tensors) + (
             self.geometry, LlamaConfig.shape())
         if key != self._bound_key:

@@ -1,0 +1,115 @@
+"""The C-ABI library: it loads, exports what include/qmk.h declares, and the ctypes mirror matches the header.
+
+No GPU work here: only entry points that return before touching a device are called.
+"""
+import ctypes
+import re
+import subprocess
+import sys
+from pathlib import Path
+
+import pytest
+import torch
+
+from __graft_entry__ import LIBRARY, ROOT, build_library
+from qimeng_megakernel_amd.decode_schedule import mk_kernel
+
+HEADER = ROOT / "include" / "qmk.h"
+
+
+@pytest.fixture(scope="module")
+def lib():
+    if not LIBRARY.is_file():
+        build_library()
+    return mk_kernel.load_library()
+
+
+def test_every_declared_symbol_is_exported(lib):
+    text = HEADER.read_text()
+    declared = set(re.findall(r"^(?:int|const char\*)\s+(qmk_\w+)\s*\(", text, flags=re.M))
+    assert declared == {"qmk_decode_step", "qmk_query", "qmk_status_fetch", "qmk_error_string"}
+    for name in declared:
+        assert hasattr(lib, name), name
+
+
+def test_struct_layout_matches_header(tmp_path):
+    """Compile the header with gcc and compare sizeof/offsetof with the ctypes mirror."""
+    fields = [name for name, _ in mk_kernel.QmkArgs._fields_]
+    prog = tmp_path / "layout.c"
+    lines = ['#include <stdio.h>', '#include <stddef.h>', f'#include "{HEADER}"', "int main(void) {",
+             '  printf("%zu\\n", sizeof(QmkArgs));']
+    lines += [f'  printf("%zu\\n", offsetof(QmkArgs, {f}));' for f in fields]
+    lines += ["  return 0;", "}"]
+    prog.write_text("\n".join(lines))
+    exe = tmp_path / "layout"
+    subprocess.run(["gcc", "-std=c99", "-Wall", "-Werror", "-o", str(exe), str(prog)], check=True)
+    out = [int(x) for x in subprocess.run([str(exe)], check=True, capture_output=True, text=True).stdout.split()]
+    assert out[0] == ctypes.sizeof(mk_kernel.QmkArgs)
+    assert out[1:] == [getattr(mk_kernel.QmkArgs, f).offset for f in fields]
+    # every struct member of the header is mirrored, in order
+    body = HEADER.read_text().split("typedef struct QmkArgs {")[1].split("} QmkArgs;")[0]
+    body = re.sub(r"/\*.*?\*/", "", body, flags=re.S)
+    members = re.findall(r"(\w+)\s*;", body)
+    assert members == fields
+
+
+def test_constants_match_header():
+    text = HEADER.read_text()
+    def define(name):
+        return int(re.search(rf"#define {name} (\d+)", text).group(1))
+    assert define("QMK_FLAG_KEEP_BARRIERS") == mk_kernel.QMK_FLAG_KEEP_BARRIERS
+    assert define("QMK_FLAG_XCD_COUNTERS") == mk_kernel.QMK_FLAG_XCD_COUNTERS
+    assert define("QMK_XCD_COUNTER_ROWS") == mk_kernel.QMK_XCD_COUNTER_ROWS
+    assert define("QMK_INSTRUCTION_WORDS") == 32
+
+
+def test_host_side_argument_errors(lib):
+    assert lib.qmk_decode_step(None) == 1                                  # QMK_ERR_NULL_ARG
+    a = mk_kernel.QmkArgs()
+    a.struct_size = 12
+    assert lib.qmk_decode_step(ctypes.byref(a)) == 2                       # QMK_ERR_ABI
+    a.struct_size = ctypes.sizeof(mk_kernel.QmkArgs)
+    a.model = 99
+    assert lib.qmk_decode_step(ctypes.byref(a)) == 8                       # QMK_ERR_MODEL
+    a.model = 0
+    assert lib.qmk_decode_step(ctypes.byref(a)) == 1                       # all tensor pointers are NULL
+    assert lib.qmk_query(0) == 1 and lib.qmk_query(2) == 512 and lib.qmk_query(5) == 32 and lib.qmk_query(6) == 25
+    assert 0 < lib.qmk_query(3) <= 160 * 1024
+    assert lib.qmk_error_string(34).decode().startswith("device: counter wait")
+    assert lib.qmk_error_string(12345).decode() == "unknown code"
+
+
+def test_missing_library_is_an_import_error(tmp_path):
+    with pytest.raises(ImportError, match="missing prebuilt kernel"):
+        mk_kernel.get_mk(tmp_path)
+    (tmp_path / "libqmk_hip.so").write_bytes(b"not an ELF file")
+    with pytest.raises(ImportError, match="cannot load"):
+        mk_kernel.load_library(tmp_path)
+
+
+def test_mk_rejects_cpu_tensors_and_bad_dtypes(lib, small_model):
+    from qimeng_megakernel_amd import synthetic
+    from qimeng_megakernel_amd.decode_schedule.instructions import scheduler as S
+    from qimeng_megakernel_amd.decode_schedule.model_config import LlamaConfig
+
+    shape, w, _ = small_model
+    LlamaConfig.set_shape(shape)
+    g = synthetic.build_globals(w, shape, 16, "cpu")
+    S.build(g)
+    assert g.instructions.shape[0] == 1                                    # off-GPU: a single queue, as in the reference
+    mk = mk_kernel.get_mk()
+    with pytest.raises(ValueError, match="must live on the GPU"):
+        mk_kernel.call_mk(g, mk)
+    with pytest.raises(TypeError, match="25 positional"):
+        mk(g.instructions)
+    g.hidden_states = g.hidden_states.float()
+    with pytest.raises((TypeError, ValueError)):
+        mk_kernel.call_mk(g, mk)
+
+
+def test_product_code_never_imports_the_oracle():
+    """The shipped path must not route through the CPU oracle (or any CPU fallback)."""
+    pkg = ROOT / "qimeng-megakernel_amd"
+    for path in list(pkg.rglob("*.py")):
+        text = path.read_text()
+        assert "fused_oracle" not in text and "pyvm_oracle" not in text and "oracle/" not in text, path
