@@ -75,6 +75,8 @@ def main() -> None:
     ap.add_argument("--prompt-len", type=int, default=8)
     ap.add_argument("--cpu-steps", type=int, default=10)
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--copy-calibration", action="store_true",
+                    help="also run one 1 GiB device-to-device copy (a kernel of known traffic, for scaling rocprofv3 counters)")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         raise SystemExit("bench.py: this path runs on exactly one GPU (batch-1 decode does not shard; "
@@ -104,6 +106,12 @@ def main() -> None:
     globs = synthetic.build_globals(weights, shape, kv_capacity, device)
     mk = mk_kernel.get_mk()
 
+    if args.copy_calibration:
+        src = torch.empty(1 << 30, dtype=torch.uint8, device=device)
+        dst = torch.empty_like(src)
+        dst.copy_(src)                      # reads 1 GiB, writes 1 GiB
+        torch.cuda.synchronize(device)
+        del src, dst
     if args.warmup > 0:
         decode.decode(globs, prompt, min(args.warmup + 1, new_tokens), mk=mk, decode_time=False)
     globs.k_cache.zero_(); globs.v_cache.zero_()

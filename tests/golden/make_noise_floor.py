@@ -5,7 +5,8 @@ Teacher-forced replay of tests/golden/llama1b_seed0.* with this repository's CPU
 evaluated as an fp32 matmul instead of a bf16 einsum: the same bf16 rounding points as the reference,
 another fp32 accumulation order.  Writes tests/golden/noise_floor_llama1b_seed0.json: per-step distance
 of the top-8 logits from the fixture in bf16 ulps of the top logit, and the steps where the argmax
-differs.  The GPU parity gates are set against these numbers.
+differs, plus the deviation of the final residual stream at the recorded steps.  The GPU parity gates
+are set against these numbers.
 
 usage: python tests/golden/make_noise_floor.py [--steps 256]
 """
@@ -45,7 +46,7 @@ def main():
     oracle = fo.FusedOracle(shape)
     seq = meta["prompt"] + meta["tokens"]
     want = torch.from_numpy(arrays["topk_bits"].astype(np.int32)).to(torch.int16).view(torch.bfloat16).float()
-    dist, mismatches = [], []
+    dist, mismatches, hidden_dev = [], [], {}
     t0 = time.time()
     for pos in range(n_prompt + args.steps - 1):
         oracle.embed(g, seq[pos]); g.position_id = pos
@@ -58,13 +59,17 @@ def main():
         dist.append(float((g.logits[ids].float() - want[i]).abs().max()) / ulp)
         if int(g.logits.argmax()) != meta["tokens"][i]:
             mismatches.append({"step": i, "margin_ulps": meta["margins"][i] / ulp})
+        name = f"final_hidden_step{i - 1}"
+        if name in arrays:
+            ref = torch.from_numpy(arrays[name].astype(np.int32)).to(torch.int16).view(torch.bfloat16).float()
+            hidden_dev[f"step{i - 1}"] = float((g.hidden_states.float() - ref).abs().max() / ref.abs().max())
         if i % 16 == 0:
             print(f"step {i}: worst so far {max(dist):.2f} ulps, {len(mismatches)} argmax differences, {time.time() - t0:.0f}s", flush=True)
-            _write(args, dist, mismatches)
-    _write(args, dist, mismatches)
+            _write(args, dist, mismatches, hidden_dev)
+    _write(args, dist, mismatches, hidden_dev)
 
 
-def _write(args, dist, mismatches):
+def _write(args, dist, mismatches, hidden_dev):
     (OUT / "noise_floor_llama1b_seed0.json").write_text(json.dumps({
         "what": "CPU oracle with fp32-matmul GEMVs, teacher-forced on the golden tokens, vs the golden top-8 logits",
         "steps": len(dist),
@@ -72,6 +77,7 @@ def _write(args, dist, mismatches):
         "mean_ulps": sum(dist) / len(dist),
         "p99_ulps": float(np.quantile(np.array(dist), 0.99)),
         "argmax_differences": mismatches,
+        "final_hidden_max_diff_over_max_ref": hidden_dev,
         "per_step_max_ulps": dist,
         "torch": torch.__version__,
     }))

@@ -14,7 +14,7 @@ import pytest
 import torch
 
 from conftest import GOLDEN
-from gpu_helpers import rel_close
+from gpu_helpers import rel_close, tensor_rel_close
 from qimeng_megakernel_amd import decode, synthetic
 from qimeng_megakernel_amd.decode_schedule import mk_kernel
 from qimeng_megakernel_amd.decode_schedule.instructions import scheduler as S
@@ -111,8 +111,14 @@ def test_teacher_forced_1024_steps(golden, model):
     assert 1 - len(beyond) / int((~near).sum()) >= 0.99
     # 4. residual stream after the last layer and sampled logits at the recorded steps
     for name in record.values():
-        rel_close(hidden_at[name], _bf16(arrays[f"final_hidden_{name}"]), rel=4e-2, name=f"final hidden {name}")
-        rel_close(logits_at[name], _bf16(arrays[f"logit_samples_{name}"]), rel=4e-2, name=f"logit samples {name}")
+        # 16 layers deep a second CPU evaluation of the reference (tests/golden/noise_floor_*.json,
+        # final_hidden_max_diff_over_max_ref) sits at 2.0e-2 (step 0) .. 2.6e-2 (step 127) of the largest
+        # element; the gate is 1.5x that.
+        e = tensor_rel_close(hidden_at[name], _bf16(arrays[f"final_hidden_{name}"]), rel=4e-2, name=f"final hidden {name}")
+        want_l = _bf16(arrays[f"logit_samples_{name}"])
+        l_err = float((logits_at[name].float().cpu() - want_l).abs().max())
+        print(f"{name}: final hidden max|diff|/max|ref| {e:.4f}; 256 sampled logits off by <= {l_err:.4f}")
+        assert l_err <= LOGIT_ULPS * 2.0 ** -6      # LOGIT_ULPS ulps of a top logit in [2, 4)
 
 
 def test_per_layer_hidden_first_decode_step(golden, model):
@@ -132,8 +138,7 @@ def test_per_layer_hidden_first_decode_step(golden, model):
         g.position_id = pos
         g.barriers.zero_()
         mk_kernel.run_instructions(g, sched.instruction_list(nl), mk=mk)
-        rel_close(g.hidden_states[:: meta["sample_stride"]], want[nl - 1], rel=2e-2 if nl == 1 else 4e-2,
-                  name=f"hidden after layer {nl - 1}")
+        tensor_rel_close(g.hidden_states[:: meta["sample_stride"]], want[nl - 1], rel=2e-2, name=f"hidden after layer {nl - 1}")
         assert int(g.hidden_states.view(torch.int16).to(torch.int64).bitwise_and(0xFFFF).sum()) > 0
     g.barriers.zero_()
     g.instructions = None
