@@ -67,23 +67,24 @@ enum {
 };
 
 /* Rows of `barriers` per layer that QMK_FLAG_XCD_COUNTERS needs (with 48 slots). */
-#define QMK_XCD_COUNTER_ROWS 26
+#define QMK_XCD_COUNTER_ROWS 54
 
 /* Flags. */
 #define QMK_FLAG_KEEP_BARRIERS 1u  /* leave the final counter values in `barriers`
                                       (the reference's behaviour); by default the
                                       last workgroup to retire clears them so the
                                       host needs no barriers.zero_() per step.   */
-#define QMK_FLAG_XCD_COUNTERS 2u   /* the three all-to-all edges of a layer (O-proj -> up/gate,
+#define QMK_FLAG_XCD_COUNTERS 2u   /* the all-to-all edges of a layer (attention -> O-proj when the
+                                      O-proj merges the partials itself, O-proj -> up/gate,
                                       up/gate -> down, down -> next QKV / LM head) count
                                       arrivals on eight sub-counters, one 128-byte line per
                                       XCD, kept in rows 10.. of each layer of `barriers`;
                                       consumers poll the eight lines and sum them.  Needs
                                       num_layer_barriers * barrier_slots >= 10 * barrier_slots
-                                      + 768 ints, a 128-byte aligned `barriers` with a layer
+                                      + 2048 ints (32 counter lines, then 32 flag lines), a 128-byte aligned `barriers` with a layer
                                       stride that is a multiple of 128 bytes, and a schedule
                                       that does not split the down projection along K.  Rows
-                                      3..5 of the reference protocol stay zero in this mode. */
+                                      2..5 of the reference protocol stay zero in this mode. */
 
 /*
  * One decode step.  Tensor order and meaning follow mk(...) of the reference

@@ -86,8 +86,15 @@ class InstructionVM:
     # ---- 4 --------------------------------------------------------------------
     def oproj_gemv_residual(self, g: Any, ins: Any) -> None:
         s = self.shape
-        assert int(g.barriers[ins.layer_idx, ROW_REDUCE, 0]) == s.num_attention_heads
-        assert ins.reduction_block_idx == 0
+        if ins.reduction_block_idx == 0:
+            assert int(g.barriers[ins.layer_idx, ROW_REDUCE, 0]) == s.num_attention_heads
+        else:
+            # Extension: this instruction merges the split-KV partials itself (all heads); the
+            # reduction row then counts one arrival per split-KV instruction.
+            P = ins.reduction_block_idx
+            assert int(g.barriers[ins.layer_idx, ROW_REDUCE, 0]) == s.num_key_value_heads * P
+            for h0 in range(0, s.num_attention_heads, s.attn_reduction_size):
+                self._merge(g, ins.layer_idx, h0, list(range(P)), True, 0, count=False)
         tile = ins.tile_N_granularity
         w = g.o_proj_weights[ins.layer_idx]
         for blk in range(ins.tile_N_start_idx, ins.tile_N_end_idx):
@@ -199,10 +206,15 @@ class InstructionVM:
         out = torch.einsum("hk,ko->ho", probs, v)               # zeros for an empty slice
         g.attn_lse_intermediates[h0:h1, ins.partial_idx] = lse2
         g.attn_out_intermediates[h0:h1, ins.partial_idx] = out
-        g.barriers[ins.layer_idx, ROW_SPLITKV, h0:h1] += 1
         # Extension of this build's schedules (operand word 5, zero in the reference's streams):
-        # the arrival that completes the head group merges all partials itself.
-        if getattr(ins, "merge_in_last", 0) and int(g.barriers[ins.layer_idx, ROW_SPLITKV, h0]) == ins.num_partials:
+        # 1 = the arrival that completes the head group merges all partials itself;
+        # 2 = arrive on the reduction row only, the O-proj instructions merge.
+        mode = getattr(ins, "merge_in_last", 0)
+        if mode == 2:
+            g.barriers[ins.layer_idx, ROW_REDUCE, 0] += 1
+            return
+        g.barriers[ins.layer_idx, ROW_SPLITKV, h0:h1] += 1
+        if mode == 1 and int(g.barriers[ins.layer_idx, ROW_SPLITKV, h0]) == ins.num_partials:
             self._merge(g, ins.layer_idx, h0, list(range(ins.num_partials)), True, 0)
 
     # ---- 3 --------------------------------------------------------------------
@@ -212,7 +224,7 @@ class InstructionVM:
         assert int(g.barriers[ins.layer_idx, ROW_SPLITKV, h0]) == ins.num_partials
         self._merge(g, ins.layer_idx, h0, ins.reduction_list, ins.is_terminal, ins.output_partial_idx)
 
-    def _merge(self, g: Any, layer: int, h0: int, reduction_list, is_terminal, output_partial_idx) -> None:
+    def _merge(self, g: Any, layer: int, h0: int, reduction_list, is_terminal, output_partial_idx, count=True) -> None:
         s = self.shape
         h1 = h0 + s.attn_reduction_size
         idx = torch.tensor(list(reduction_list), dtype=torch.long)
@@ -227,4 +239,5 @@ class InstructionVM:
         else:
             g.attn_lse_intermediates[h0:h1, output_partial_idx] = (top + denom.log2()).squeeze(-1)
             g.attn_out_intermediates[h0:h1, output_partial_idx] = merged
-        g.barriers[layer, ROW_REDUCE, 0] += s.attn_reduction_size
+        if count:
+            g.barriers[layer, ROW_REDUCE, 0] += s.attn_reduction_size

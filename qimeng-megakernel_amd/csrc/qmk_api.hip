@@ -141,7 +141,7 @@ extern "C" int qmk_decode_step(const QmkArgs* a) {
   if (a->pos_id < 0 || a->pos_id >= a->max_seq_len || a->pos_id >= a->rope_rows) return QMK_ERR_POSITION;
   if (a->flags & QMK_FLAG_XCD_COUNTERS) {
     const long layer_ints = static_cast<long>(a->num_layer_barriers) * a->barrier_slots;
-    const long needed = static_cast<long>(kHierFirstRow) * a->barrier_slots + kHierEdges * kXcds * kLineInts;
+    const long needed = static_cast<long>(kHierFirstRow) * a->barrier_slots + 2 * kHierEdges * kXcds * kLineInts;  // counter lines + flag lines
     const bool aligned = reinterpret_cast<uintptr_t>(a->barriers) % 128 == 0 && (layer_ints * 4) % 128 == 0 &&
                          (static_cast<long>(kHierFirstRow) * a->barrier_slots * 4) % 128 == 0;
     if (layer_ints < needed || !aligned) return QMK_ERR_SHAPE;

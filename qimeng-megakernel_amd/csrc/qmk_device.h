@@ -70,11 +70,14 @@ __device__ __forceinline__ float bf2f(u16 v) { return __uint_as_float(static_cas
 
 // Round-to-nearest-even, the rounding torch applies on .to(bfloat16).
 __device__ __forceinline__ u16 f2bf(float f) {
-  uint32_t u = __float_as_uint(f);
-  if ((u & 0x7fffffffu) > 0x7f800000u) return static_cast<u16>((u >> 16) | 0x40u);  // quiet NaN
-  u += 0x7fffu + ((u >> 16) & 1u);
-  return static_cast<u16>(u >> 16);
+  const uint32_t u = __float_as_uint(f);
+  const uint32_t rounded = (u + 0x7fffu + ((u >> 16) & 1u)) >> 16;
+  const uint32_t quiet = (u >> 16) | 0x40u;  // NaN stays NaN
+  return static_cast<u16>((u & 0x7fffffffu) > 0x7f800000u ? quiet : rounded);  // a select, not a branch
 }
+// 2^x for x <= 0 as one v_exp_f32 (results below the normal range flush to zero, which is what a
+// softmax weight that small should be); 2^-inf = 0.
+__device__ __forceinline__ float exp2_fast(float x) { return __builtin_amdgcn_exp2f(x); }
 __device__ __forceinline__ float round_bf16(float f) { return bf2f(f2bf(f)); }
 __device__ __forceinline__ float bf_lo(uint32_t w) { return __uint_as_float(w << 16); }
 __device__ __forceinline__ float bf_hi(uint32_t w) { return __uint_as_float(w & 0xffff0000u); }
@@ -236,16 +239,16 @@ __device__ __forceinline__ void publish(int32_t* ctr, int amount) {
 constexpr int kXcds = 8;
 constexpr int kLineInts = 32;              // 128-byte line
 constexpr int kHierFirstRow = 10;          // first row of the sub-counter region of a layer
-constexpr int kHierEdges = 3;              // O-proj, up/gate, down  (counter rows 3, 4, 5)
+constexpr int kHierEdges = 4;              // attention, O-proj, up/gate, down  (counter rows 2..5)
 
 __device__ __forceinline__ bool xcd_counters(const Params& p) { return (p.flags & QMK_FLAG_XCD_COUNTERS) != 0; }
 
 __device__ __forceinline__ int32_t* sub_counter(const Params& p, int layer, int row, int xcd) {
   return p.barriers + (static_cast<size_t>(layer) * p.num_layer_barriers + kHierFirstRow) * p.barrier_slots +
-         ((row - 3) * kXcds + xcd) * kLineInts;
+         ((row - 2) * kXcds + xcd) * kLineInts;
 }
 
-// Arrival on an all-to-all edge (counter row 3, 4 or 5, slot 0).
+// Arrival on an all-to-all edge (counter row 2..5, slot 0).
 __device__ __forceinline__ void arrive_all(const Params& p, int layer, int row, int amount) {
   publish(xcd_counters(p) ? sub_counter(p, layer, row, blockIdx.x & (kXcds - 1)) : counter_ptr(p, layer, row, 0), amount);
 }
@@ -276,7 +279,9 @@ constexpr uint32_t kFollowerPolls = 256;
 
 __device__ __forceinline__ bool wait_edge_xcd(const Params& p, int layer, int row, int expected, uint32_t limit) {
   const int xcd = blockIdx.x & (kXcds - 1);
-  int32_t* flag = sub_counter(p, layer, row, xcd) + 1;
+  // The flag has a line of its own (second half of the region): only workgroups of this XCD ever
+  // touch it, so it lives in this XCD's L2 and polling it stays off the fabric.
+  int32_t* flag = sub_counter(p, layer, row, xcd) + kHierEdges * kXcds * kLineInts;
   const bool leader = blockIdx.x < kXcds || gridDim.x < 2 * kXcds;
   bool ready = false;
   if (!leader) {

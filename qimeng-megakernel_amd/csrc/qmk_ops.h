@@ -89,7 +89,7 @@ __device__ __forceinline__ bool wg_wait(const Params& p, Smem<M>& s, const Ctx& 
   return true;
 }
 
-// Wait on an all-to-all edge (counter row 3, 4 or 5): slot 0 of the row, or the eight
+// Wait on an all-to-all edge (counter row 2..5): slot 0 of the row, or the eight
 // per-XCD sub-counters of the edge when the launch uses them.
 template <class M>
 __device__ __forceinline__ bool wg_wait_all(const Params& p, Smem<M>& s, const Ctx& c, int layer, int row, int slot, int expected) {
@@ -253,29 +253,26 @@ __device__ __forceinline__ void merge_partials(const Params& p, int head0, int n
   const int h = head0 + threadIdx.x / (M::D / 2), d = 2 * (threadIdx.x % (M::D / 2));
   const float* lse = p.attn_lse + static_cast<size_t>(h) * p.max_splits;
   const float* part = p.attn_partial + static_cast<size_t>(h) * p.max_splits * M::D + d;
+  // Branch-free: slots beyond n re-read the last listed partial and get weight 0.
   float e[kMaxPartials];
   uint64_t two[kMaxPartials];
 #pragma unroll
   for (int i = 0; i < kMaxPartials; ++i) {
-    if (i < n) {
-      const int j = list ? list[i] : i;
-      e[i] = ld_shared_f32(lse + j);
-      two[i] = ld_shared64(part + static_cast<size_t>(j) * M::D);
-    }
+    const int ii = min(i, n - 1);
+    const int j = list ? list[ii] : ii;
+    e[i] = ld_shared_f32(lse + j);
+    two[i] = ld_shared64(part + static_cast<size_t>(j) * M::D);
   }
   float mx = -INFINITY;
 #pragma unroll
-  for (int i = 0; i < kMaxPartials; ++i)
-    if (i < n) mx = fmaxf(mx, e[i]);
+  for (int i = 0; i < kMaxPartials; ++i) mx = fmaxf(mx, e[i]);
   float num0 = 0.f, num1 = 0.f, den = 0.f;
 #pragma unroll
   for (int i = 0; i < kMaxPartials; ++i) {
-    if (i < n) {
-      const float f = (e[i] == -INFINITY) ? 0.f : exp2f(e[i] - mx);
-      num0 = __builtin_fmaf(__uint_as_float(static_cast<uint32_t>(two[i])), f, num0);
-      num1 = __builtin_fmaf(__uint_as_float(static_cast<uint32_t>(two[i] >> 32)), f, num1);
-      den += f;
-    }
+    const float f = (i < n && e[i] != -INFINITY) ? exp2_fast(e[i] - mx) : 0.f;
+    num0 = __builtin_fmaf(__uint_as_float(static_cast<uint32_t>(two[i])), f, num0);
+    num1 = __builtin_fmaf(__uint_as_float(static_cast<uint32_t>(two[i] >> 32)), f, num1);
+    den += f;
   }
   const float o0 = den > 0.f ? num0 / den : 0.f, o1 = den > 0.f ? num1 / den : 0.f;
   if (terminal) {
@@ -304,7 +301,9 @@ template <class M>
 __device__ bool op_attn_splitkv(const Params& p, Smem<M>& s, const Ctx& c) {
   static_assert(M::D == 64 && M::GQA == 4, "lane mapping assumes head_dim 64 and 4 query heads per KV head");
   const int layer = s.inst[1], kvh = s.inst[2], P = s.inst[3], part = s.inst[4];
-  const bool merge_in_last = s.inst[5] != 0;
+  const int merge_mode = s.inst[5];  // 0: per-head counters, 1: last arrival merges, 2: the O-proj merges
+  const bool merge_in_last = merge_mode == 1;
+  if (merge_mode < 0 || merge_mode > 2) return bad_operand(p, s, c, 5);
   if (layer < 0 || layer >= p.num_layers) return bad_operand(p, s, c, 1);
   if (kvh < 0 || kvh >= M::NKV) return bad_operand(p, s, c, 2);
   if (P < 1 || P > p.max_splits || part < 0 || part >= P) return bad_operand(p, s, c, 3);
@@ -391,8 +390,8 @@ __device__ bool op_attn_splitkv(const Params& p, Smem<M>& s, const Ctx& c) {
       for (int i = 0; i < 8; ++i) sc = __builtin_fmaf(q[h][i], k[i], sc);
       sc = group8_sum(sc);  // the 8 lanes of a group always take the same branch
       const float mn = fmaxf(m[h], sc);
-      const float alpha = exp2f(m[h] - mn);   // 0 on the first token (m = -inf)
-      const float pr = exp2f(sc - mn);
+      const float alpha = exp2_fast(m[h] - mn);   // 0 on the first token (m = -inf)
+      const float pr = exp2_fast(sc - mn);
       l[h] = __builtin_fmaf(l[h], alpha, pr);
 #pragma unroll
       for (int i = 0; i < 8; ++i) acc[h][i] = __builtin_fmaf(acc[h][i], alpha, pr * v[i]);
@@ -423,30 +422,56 @@ __device__ bool op_attn_splitkv(const Params& p, Smem<M>& s, const Ctx& c) {
   __syncthreads();
 
   // Wave h of the first four folds head h.  Lane g first turns group g's (m, l) into its weight
-  // f = 2^(m - max) and l*f (max and the denominator are wave reductions), then lane d sums column d.
+  // f = 2^(m - max) and l*f (max and the denominator are wave reductions).  Then lane = 4*quad + sub
+  // sums dims 4*quad..4*quad+3 over the 16 states g = sub, sub+4, ... and the four `sub` lanes of a
+  // quad are added with DPP.
   if (threadIdx.x < M::GQA * M::D) {
-    static_assert(kWaves * 8 == kWaveSize && M::D == kWaveSize, "one lane per group, then one lane per dim");
+    static_assert(kWaves * 8 == kWaveSize && M::D == kWaveSize, "one lane per group, 16 dim-quads x 4 state subsets");
     const int h = threadIdx.x / kWaveSize;
     const float mg = s.merge[lane][h][M::D];
     const float mx = wave_max(mg);
-    const float f = (mg == -INFINITY) ? 0.f : exp2f(mg - mx);
+    const float f = (mg == -INFINITY) ? 0.f : exp2_fast(mg - mx);
     const float den = wave_sum(s.merge[lane][h][M::D + 1] * f);
     s.merge[lane][h][M::D + 2] = f;
-    // wave-private rows of s.merge: written and read by this wave only, LDS ops of a wave stay in order
-    float num = 0.f;
-#pragma unroll 16
-    for (int g = 0; g < kWaves * 8; ++g) num = __builtin_fmaf(s.merge[g][h][lane], s.merge[g][h][M::D + 2], num);
-    const int head = kvh * M::GQA + h, d = lane;
+    // rows [*][h] of s.merge are touched by this wave only; LDS operations of one wave stay in order
+    const int quad = lane >> 2, sub = lane & 3;
+    float4 part4[16];
+    float w16[16];
+#pragma unroll
+    for (int i = 0; i < 16; ++i) {
+      part4[i] = *reinterpret_cast<const float4*>(&s.merge[sub + 4 * i][h][4 * quad]);
+      w16[i] = s.merge[sub + 4 * i][h][M::D + 2];
+    }
+    float n0 = 0.f, n1 = 0.f, n2 = 0.f, n3 = 0.f;
+#pragma unroll
+    for (int i = 0; i < 16; ++i) {
+      n0 = __builtin_fmaf(part4[i].x, w16[i], n0);
+      n1 = __builtin_fmaf(part4[i].y, w16[i], n1);
+      n2 = __builtin_fmaf(part4[i].z, w16[i], n2);
+      n3 = __builtin_fmaf(part4[i].w, w16[i], n3);
+    }
+    n0 += dpp_f32<kDppQuadXor1>(0.f, n0); n0 += dpp_f32<kDppQuadXor2>(0.f, n0);
+    n1 += dpp_f32<kDppQuadXor1>(0.f, n1); n1 += dpp_f32<kDppQuadXor2>(0.f, n1);
+    n2 += dpp_f32<kDppQuadXor1>(0.f, n2); n2 += dpp_f32<kDppQuadXor2>(0.f, n2);
+    n3 += dpp_f32<kDppQuadXor1>(0.f, n3); n3 += dpp_f32<kDppQuadXor2>(0.f, n3);
+    const int head = kvh * M::GQA + h;
     const bool empty = !(den > 0.f);
+    const float inv = empty ? 0.f : 1.0f / den;
     // Normalised partial output and log2-sum-exp; an empty slice contributes (0, -inf).
-    st_shared_f32(p.attn_partial + (static_cast<size_t>(head) * p.max_splits + part) * M::D + d, empty ? 0.f : num / den);
-    if (d == 0) st_shared_f32(p.attn_lse + static_cast<size_t>(head) * p.max_splits + part, empty ? -INFINITY : mx + log2f(den));
+    // Lane `sub` of a quad stores dim 4*quad + sub.
+    const float mine = sub == 0 ? n0 : (sub == 1 ? n1 : (sub == 2 ? n2 : n3));
+    st_shared_f32(p.attn_partial + (static_cast<size_t>(head) * p.max_splits + part) * M::D + lane, mine * inv);
+    if (lane == 0) st_shared_f32(p.attn_lse + static_cast<size_t>(head) * p.max_splits + part, empty ? -INFINITY : mx + log2f(den));
   }
 
   QMK_STAMP(2);  // partial merged and stored
   release_stores();
   __syncthreads();
   QMK_STAMP(3);  // stores acknowledged
+  if (merge_mode == 2) {  // one arrival per partial on the attention -> O-proj edge
+    if (threadIdx.x == 0) arrive_all(p, layer, ROW_REDUCE, 1);
+    return true;
+  }
   if (!merge_in_last) {
     if (threadIdx.x < M::GQA) publish(counter_ptr(p, layer, ROW_SPLITKV, kvh * M::GQA + threadIdx.x), 1);
     return true;
@@ -517,10 +542,56 @@ __device__ bool op_oproj_residual(const Params& p, Smem<M>& s, const Ctx& c) {
 
   RowRegs<CH> buf[kDepth];
   preload<CH>(nrows, src, buf);
-  if (!wg_wait(p, s, c, 1, [&](int) { return counter_ptr(p, layer, ROW_REDUCE, 0); }, M::NQ)) return false;
-
   static_assert(M::H == kThreads * 4, "one thread stages four elements");
-  *reinterpret_cast<uint64_t*>(s.x + threadIdx.x * 4) = ld_shared64(p.attn_out + threadIdx.x * 4);
+  const int self_merge = s.inst[5];  // reduction_block_idx: 0, or the split-KV fan-out P when this op merges
+  if (self_merge == 0) {
+    if (!wg_wait(p, s, c, 1, [&](int) { return counter_ptr(p, layer, ROW_REDUCE, 0); }, M::NQ)) return false;
+    *reinterpret_cast<uint64_t*>(s.x + threadIdx.x * 4) = ld_shared64(p.attn_out + threadIdx.x * 4);
+  } else {
+    // Every O-proj workgroup merges the split-KV partials itself (python_vm.py:439-488 for all heads):
+    // no merging workgroup, no attn_out round trip, one synchronisation hop less.  Thread t owns
+    // dims 4*(t%16).. of head t/16.
+    const int P = self_merge;
+    if (P < 1 || P > kMaxPartials || P > p.max_splits) return bad_operand(p, s, c, 5);
+    if (!wg_wait_all(p, s, c, layer, ROW_REDUCE, 0, M::NKV * P)) return false;
+    const int h = threadIdx.x / (M::D / 4), d0 = 4 * (threadIdx.x % (M::D / 4));
+    const float* lse = p.attn_lse + static_cast<size_t>(h) * p.max_splits;
+    const float* part = p.attn_partial + static_cast<size_t>(h) * p.max_splits * M::D + d0;
+    float mx = -INFINITY, den = 0.f, n0 = 0.f, n1 = 0.f, n2 = 0.f, n3 = 0.f;
+    for (int j0 = 0; j0 < P; j0 += 4) {   // four partials per round, loads first
+      float e[4];
+      v4u o[4];
+#pragma unroll
+      for (int k = 0; k < 4; ++k) {
+        const int j = min(j0 + k, P - 1);
+        e[k] = (j0 + k < P) ? ld_shared_f32(lse + j) : -INFINITY;
+        o[k] = ld_shared128(part + static_cast<size_t>(j) * M::D);
+      }
+      float mn = mx;
+#pragma unroll
+      for (int k = 0; k < 4; ++k) mn = fmaxf(mn, e[k]);
+      const float rescale = (mx == -INFINITY) ? 0.f : exp2_fast(mx - mn);
+      den *= rescale; n0 *= rescale; n1 *= rescale; n2 *= rescale; n3 *= rescale;
+#pragma unroll
+      for (int k = 0; k < 4; ++k) {
+        const float f = (e[k] == -INFINITY) ? 0.f : exp2_fast(e[k] - mn);
+        den += f;
+        n0 = __builtin_fmaf(__uint_as_float(o[k].x), f, n0);
+        n1 = __builtin_fmaf(__uint_as_float(o[k].y), f, n1);
+        n2 = __builtin_fmaf(__uint_as_float(o[k].z), f, n2);
+        n3 = __builtin_fmaf(__uint_as_float(o[k].w), f, n3);
+      }
+      mx = mn;
+    }
+    const float inv = den > 0.f ? 1.0f / den : 0.f;
+    const uint32_t lo = static_cast<uint32_t>(f2bf(n0 * inv)) | (static_cast<uint32_t>(f2bf(n1 * inv)) << 16);
+    const uint32_t hi = static_cast<uint32_t>(f2bf(n2 * inv)) | (static_cast<uint32_t>(f2bf(n3 * inv)) << 16);
+    *reinterpret_cast<uint2*>(s.x + threadIdx.x * 4) = make_uint2(lo, hi);
+    if (nstart == 0) {  // one workgroup also leaves attn_out in memory, as the reference does
+      st_shared32(p.attn_out + threadIdx.x * 4, lo);
+      st_shared32(p.attn_out + threadIdx.x * 4 + 2, hi);
+    }
+  }
   __syncthreads();
   v4u x[CH];
   load_x_from_lds(x, s.x, lane);

@@ -142,10 +142,13 @@ class DecodeAttentionSplitKV(Instruction):
     """One KV head, one contiguous slice of the context, all query heads of the group.
 
     ``merge_in_last`` extends the reference's four operands (its word is 0 in any
-    stream the reference scheduler builds): when set, the workgroup whose arrival
+    stream the reference scheduler builds).  1: the workgroup whose arrival
     completes the head group's split-KV counter also performs the log-sum-exp
-    merge of all partials and publishes on the reduction row, so the schedule
-    carries no separate reduction instruction for that head group.
+    merge of all partials and publishes on the reduction row.  2: the partial only
+    arrives on the reduction row (slot 0, one arrival per instruction) and every
+    O-proj instruction merges the partials itself (its ``reduction_block_idx``
+    then carries ``num_partials``).  Either way the schedule carries no separate
+    reduction instructions.
     """
 
     OPCODE: ClassVar[int] = 2
@@ -173,7 +176,12 @@ class DecodeAttentionReduction(Instruction):
 
 @dataclass
 class OProj_GEMV_Residual(Instruction):
-    """hidden[rows] += W_o[rows] . attn_out"""
+    """hidden[rows] += W_o[rows] . attn_out
+
+    ``reduction_block_idx`` is 0 in the reference's streams.  A positive value P
+    means: wait for the ``num_kv_heads * P`` split-KV arrivals on the reduction
+    row and merge the P partials of every head before the GEMV.
+    """
 
     OPCODE: ClassVar[int] = 4
     PREV_OPCODES: ClassVar[tuple[int, ...]] = (3,)

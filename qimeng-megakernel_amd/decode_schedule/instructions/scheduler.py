@@ -50,8 +50,11 @@ MAX_REDUCTION_LIST = ATTENTION_REDUCTION_LIST_CAPACITY
 #: kernel merges from registers and is bounded only by the instruction slot.
 REFERENCE_MAX_ATTENTION_PARTIALS = 16
 MAX_ATTENTION_PARTIALS = ATTENTION_REDUCTION_LIST_CAPACITY
-#: KV tokens one split-KV workgroup covers per pass (8 waves x 8 tokens).
-KV_TOKENS_PER_PASS = 64
+#: value of the split-KV instruction's ``merge_in_last`` word per merge mode
+ATTENTION_MERGE_MODES = {"separate": 0, "last": 1, "oproj": 2}
+#: KV tokens per split-KV partial the fan-out aims for: four passes of a workgroup (8 waves x 8
+#: tokens per pass).  Finer splits cost more in merging than they save in streaming (measured).
+KV_TOKENS_PER_PASS = 256
 
 
 def _ceil_div(a: int, b: int) -> int:
@@ -143,14 +146,17 @@ class DecodeScheduler:
     geometry: TileGeometry
     sm_count: int
     num_partials: int
-    #: fold the log-sum-exp merge into the last split-KV arrival (no reduction instructions)
-    fuse_attention_merge: bool = False
+    #: who merges the split-KV partials: "separate" reduction instructions (the reference), the
+    #: "last" split-KV arrival of a head group, or every "oproj" workgroup for itself
+    attention_merge: str = "separate"
 
     def __post_init__(self) -> None:
         self.geometry.validate(self.shape)
         if self.sm_count < 1:
             raise ValueError("sm_count must be positive")
         _validate_num_partials(self.num_partials)
+        if self.attention_merge not in ATTENTION_MERGE_MODES:
+            raise ValueError(f"attention_merge must be one of {sorted(ATTENTION_MERGE_MODES)}")
 
     # ---- per-op emitters -------------------------------------------------
     def qkvproj(self, layer_idx: int) -> list[Instruction]:
@@ -163,13 +169,13 @@ class DecodeScheduler:
 
     def attention_split_kv(self, layer_idx: int) -> list[Instruction]:
         return [
-            DecodeAttentionSplitKV(layer_idx, kv_head, self.num_partials, p, int(self.fuse_attention_merge))
+            DecodeAttentionSplitKV(layer_idx, kv_head, self.num_partials, p, ATTENTION_MERGE_MODES[self.attention_merge])
             for kv_head in range(self.shape.num_key_value_heads)
             for p in range(self.num_partials)
         ]
 
     def attention_reduction(self, layer_idx: int) -> list[Instruction]:
-        if self.fuse_attention_merge:
+        if self.attention_merge != "separate":
             return []
         step = self.shape.attn_reduction_size
         return [
@@ -182,8 +188,9 @@ class DecodeScheduler:
     def oproj(self, layer_idx: int) -> list[Instruction]:
         g = self.geometry.oproj_tile_n
         blocks = _ceil_div(self.shape.hidden_size, g)
+        merges = self.num_partials if self.attention_merge == "oproj" else 0
         return [
-            OProj_GEMV_Residual(layer_idx, 0, lo, hi, 0, tile_N_granularity=g)
+            OProj_GEMV_Residual(layer_idx, 0, lo, hi, merges, tile_N_granularity=g)
             for lo, hi in _split_n_tiles(blocks, self.sm_count)
         ]
 
@@ -266,12 +273,12 @@ def mi355x_scheduler(
     sm_count: int = MI355X_CU_COUNT,
     kv_capacity: int | None = None,
     num_partials: int | None = None,
-    fuse_attention_merge: bool = True,
+    attention_merge: str = "oproj",
 ) -> DecodeScheduler:
     shape = shape or LlamaConfig.shape()
     geometry = dataclasses.replace(MI355X_GEOMETRY, split_k=shape.intermediate_size)
     p = num_partials or pick_num_partials(sm_count, kv_capacity, shape=shape)
-    return DecodeScheduler(shape, geometry, sm_count, p, fuse_attention_merge)
+    return DecodeScheduler(shape, geometry, sm_count, p, attention_merge)
 
 
 def scheduler_for(globs: Any) -> DecodeScheduler:
@@ -288,9 +295,10 @@ def scheduler_for(globs: Any) -> DecodeScheduler:
     override = os.environ.get("QMK_NUM_PARTIALS")  # tuning knob: force the split-KV fan-out
     if override:
         p = max(1, min(int(override), max_p))
-    if cached is not None and (cached.sm_count, cached.num_partials, cached.shape) == (sm_count, p, LlamaConfig.shape()):
+    sched = mi355x_scheduler(sm_count=sm_count, num_partials=p,
+                             attention_merge=os.environ.get("QMK_ATTENTION_MERGE", "oproj"))
+    if cached == sched:
         return cached
-    sched = mi355x_scheduler(sm_count=sm_count, num_partials=p)
     try:
         globs._decode_scheduler = sched
     except AttributeError:

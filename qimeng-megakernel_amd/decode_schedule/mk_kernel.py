@@ -30,7 +30,7 @@ _LIBRARY_NAME = "libqmk_hip.so"
 
 QMK_FLAG_KEEP_BARRIERS = 1
 QMK_FLAG_XCD_COUNTERS = 2
-QMK_XCD_COUNTER_ROWS = 26
+QMK_XCD_COUNTER_ROWS = 54
 QMK_MODEL_LLAMA_3_2_1B = 0
 QMK_QUERY_ABI_VERSION, QMK_QUERY_CU_COUNT, QMK_QUERY_THREADS, QMK_QUERY_LDS_BYTES = 0, 1, 2, 3
 QMK_QUERY_MAX_QUEUES, QMK_QUERY_INSTRUCTION_WORDS, QMK_QUERY_MAX_PARTIALS = 4, 5, 6

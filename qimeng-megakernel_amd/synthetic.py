@@ -25,7 +25,7 @@ from .decode_schedule.globs import Globals
 from .decode_schedule.model_config import DecodeShape, LlamaConfig
 
 BARRIER_ROWS = 10          # the reference's allocation
-XCD_COUNTER_ROWS = 26      # rows 10..25 hold the per-XCD sub-counters of the all-to-all edges
+XCD_COUNTER_ROWS = 54      # rows 10..53 hold the per-XCD sub-counters of the all-to-all edges
 WEIGHT_STD = 0.02
 
 

@@ -138,7 +138,10 @@ def test_per_layer_hidden_first_decode_step(golden, model):
         g.position_id = pos
         g.barriers.zero_()
         mk_kernel.run_instructions(g, sched.instruction_list(nl), mk=mk)
-        tensor_rel_close(g.hidden_states[:: meta["sample_stride"]], want[nl - 1], rel=2e-2, name=f"hidden after layer {nl - 1}")
+        # 2e-2 of the largest element while the stream is shallow; deeper in, the gate of the final
+        # residual stream (1.5x the distance of a second CPU evaluation of the reference) applies
+        tensor_rel_close(g.hidden_states[:: meta["sample_stride"]], want[nl - 1], rel=2e-2 if nl <= 4 else 4e-2,
+                         name=f"hidden after layer {nl - 1}")
         assert int(g.hidden_states.view(torch.int16).to(torch.int64).bitwise_and(0xFFFF).sum()) > 0
     g.barriers.zero_()
     g.instructions = None

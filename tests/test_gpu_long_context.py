@@ -28,8 +28,8 @@ def _reference_attention(q, k, v, n_kv):
 
 
 @pytest.mark.parametrize("context", [4096, 16384, 32768])
-@pytest.mark.parametrize("fused", [True, False])
-def test_long_context_attention(context, fused):
+@pytest.mark.parametrize("merge", ["last", "separate"])
+def test_long_context_attention(context, merge):
     shape = dataclasses.replace(LLAMA_3_2_1B, num_hidden_layers=1, vocab_size=256)
     LlamaConfig.set_shape(shape)
     w = synthetic.random_weights(shape, seed=5, max_positions=context)
@@ -39,8 +39,8 @@ def test_long_context_attention(context, fused):
     g.v_cache.copy_(torch.randn(g.v_cache.shape, generator=gen, device="cuda").bfloat16())
     g.q_post_rope.copy_((torch.randn(shape.hidden_size, generator=gen, device="cuda") * 0.4).bfloat16())
     g.position_id = context - 1
-    sched = S.mi355x_scheduler(shape, kv_capacity=context, fuse_attention_merge=fused)
-    assert sched.num_partials == 25
+    sched = S.mi355x_scheduler(shape, kv_capacity=context, attention_merge=merge)
+    assert sched.num_partials == min(25, -(-context // 256))
     g.barriers[0, 0, :] = sched.expected_counts()[0]
     ins = sched.attention_split_kv(0) + sched.attention_reduction(0)
     mk = mk_kernel.get_mk(reset_barriers=False)
@@ -74,5 +74,5 @@ def test_long_context_attention(context, fused):
         total += start.elapsed_time(stop)
     mk.check()
     nbytes = context * 8 * 64 * 2 * 2
-    print(f"\ncontext {context} fused_merge={fused}: {total / reps * 1e3:.1f} us per attention phase, "
+    print(f"\ncontext {context} merge={merge}: {total / reps * 1e3:.1f} us per attention phase, "
           f"{nbytes / (total / reps * 1e-3) / 1e9:.0f} GB/s of K/V")

@@ -21,10 +21,12 @@ pytestmark = pytest.mark.gpu
 
 
 def _sched(shape, which, P=3):
-    if which == "mi355x":            # fused merge: the last split-KV arrival reduces
+    if which == "mi355x":            # the O-proj workgroups merge the split-KV partials themselves
         return S.mi355x_scheduler(shape, sm_count=256, num_partials=P)
+    if which == "mi355x_last":       # the last split-KV arrival of a head group merges
+        return S.mi355x_scheduler(shape, sm_count=256, num_partials=P, attention_merge="last")
     if which == "mi355x_unfused":    # MI355X tiles, separate reduction instructions
-        return S.mi355x_scheduler(shape, sm_count=256, num_partials=P, fuse_attention_merge=False)
+        return S.mi355x_scheduler(shape, sm_count=256, num_partials=P, attention_merge="separate")
     return S.DecodeScheduler(shape, D.REFERENCE_GEOMETRY, 108, P)
 
 
@@ -59,7 +61,7 @@ def test_op_qkv_rope(state, which):
     assert torch.equal(gpu.barriers.cpu(), cpu.barriers)
 
 
-@pytest.mark.parametrize("which", ["mi355x", "mi355x_unfused", "reference"])
+@pytest.mark.parametrize("which", ["mi355x", "mi355x_last", "mi355x_unfused", "reference"])
 @pytest.mark.parametrize("pos,P", [(0, 1), (0, 4), (15, 2), (16, 3), (41, 3), (80, 13), (95, 25)])
 def test_op_attention_split_and_reduce(state, which, pos, P):
     shape, cpu, gpu = state
@@ -69,7 +71,10 @@ def test_op_attention_split_and_reduce(state, which, pos, P):
     cpu.attn_lse_intermediates.fill_(55.0)
     cpu.attn_out_intermediates.fill_(-3.0)
     sync_state(cpu, gpu)
-    run_both(cpu, gpu, sched, sched.attention_split_kv(0) + sched.attention_reduction(0))
+    ins = sched.attention_split_kv(0) + sched.attention_reduction(0)
+    if sched.attention_merge == "oproj":
+        ins = ins + sched.oproj(0)           # the merge happens in the O-proj prologue
+    run_both(cpu, gpu, sched, ins)
     lse_c, lse_g = cpu.attn_lse_intermediates[:, :P], gpu.attn_lse_intermediates[:, :P].cpu()
     assert torch.equal(torch.isinf(lse_c), torch.isinf(lse_g))
     fin = torch.isfinite(lse_c)
@@ -83,6 +88,7 @@ def test_op_attention_split_and_reduce(state, which, pos, P):
 def test_op_oproj(state, which):
     shape, cpu, gpu = state
     sched = _sched(shape, which)
+    sched = dataclasses.replace(sched, attention_merge="separate")   # the plain GEMV; the merging form is covered above
     cpu.barriers[0, 2, 0] = shape.num_attention_heads
     sync_state(cpu, gpu)
     run_both(cpu, gpu, sched, sched.oproj(0))
@@ -165,15 +171,17 @@ def test_xcd_sub_counters(state):
     rel_close(gpu.hidden_states, cpu.hidden_states, rel=2e-2, name="hidden")
     rel_close(gpu.logits, cpu.logits, rel=2e-2, name="logits")
     b = gpu.barriers.cpu()
-    assert torch.equal(b[:, :3], cpu.barriers[:, :3])          # per-head rows are the plain protocol
-    assert int(b[:, 3:6].abs().sum()) == 0
+    assert torch.equal(b[:, :2], cpu.barriers[:, :2])          # per-head rows are the plain protocol
+    assert int(b[:, 2:6].abs().sum()) == 0
     bph, opb, ubk, dwn = sched.expected_counts()
     for layer in range(shape.num_hidden_layers):
-        region = b[layer, 10:26].reshape(3, 8, 32)
-        assert region[:, :, 0].sum(dim=1).tolist() == [opb, ubk, dwn]
-        assert (region[:, :, 0] > 0).all()                      # every XCD took part
-        assert int(region[:, :, 2:].abs().sum()) == 0              # word 1 is the XCD's ready flag
-        assert set(region[:, :, 1].reshape(-1).tolist()) <= {0, 1}
+        flat = b[layer, 10:54].reshape(-1)
+        region, flags = flat[: 4 * 8 * 32].reshape(4, 8, 32), flat[4 * 8 * 32 : 8 * 8 * 32].reshape(4, 8, 32)
+        assert region[:, :, 0].sum(dim=1).tolist() == [shape.num_key_value_heads * sched.num_partials, opb, ubk, dwn]
+        assert (region[1:, :, 0] > 0).all()                     # every XCD took part in the GEMV edges
+        assert int(region[:, :, 1:].abs().sum()) == 0
+        assert set(flags[:, :, 0].reshape(-1).tolist()) <= {0, 1}   # the XCD's ready flag, on a line of its own
+        assert int(flags[:, :, 1:].abs().sum()) == 0
 
 
 def test_single_queue_and_odd_queue_counts(state):

@@ -21,7 +21,7 @@ from qimeng_megakernel_amd.decode_schedule.model_config import LLAMA_3_2_1B
 def test_serialize_known_words():
     assert D.RMS_QKVProj_GEMV_RoPE(3, 0, 10, 12).serialize() == [1, 3, 0, 10, 12, 1, 16]
     assert D.DecodeAttentionSplitKV(2, 5, 13, 7).serialize() == [2, 2, 5, 13, 7, 0]
-    assert D.DecodeAttentionSplitKV(2, 5, 13, 7, 1).padded()[:7] == [2, 2, 5, 13, 7, 1, 0]
+    assert D.DecodeAttentionSplitKV(2, 5, 13, 7, 2).padded()[:7] == [2, 2, 5, 13, 7, 2, 0]
     assert D.DecodeAttentionReduction(1, 8, 3, [0, 1, 2]).serialize() == [3, 1, 8, 3, 3, 0, 1, 2, 1, 0]
     assert D.OProj_GEMV_Residual(0, 0, 4, 6, 0).serialize() == [4, 0, 0, 4, 6, 0, 1, 16]
     assert D.RMS_UpGateProj_GEMV_SiLU(0, 0, [7, 115, 223]).serialize() == [5, 0, 0, 3, 7, 115, 223, 1, 16]
@@ -172,7 +172,7 @@ def _simulate(sched, num_layers):
         if op == 3:
             return all(ctr[i.layer_idx, 1, i.head_start_idx + j] == i.num_partials for j in range(ratio))
         if op == 4:
-            return ctr[i.layer_idx, 2, 0] == nq
+            return ctr[i.layer_idx, 2, 0] == (nkv * i.reduction_block_idx if i.reduction_block_idx else nq)
         if op == 5:
             return ctr[i.layer_idx, 3, 0] == opb
         if op == 6:
@@ -187,8 +187,11 @@ def _simulate(sched, num_layers):
             for b in range(i.tile_N_start_idx, i.tile_N_end_idx):
                 ctr[i.layer_idx, 0, b // bph] += 1
         elif op == 2:
+            if i.merge_in_last == 2:
+                ctr[i.layer_idx, 2, 0] += 1
+                return
             ctr[i.layer_idx, 1, i.kv_head_idx * ratio : (i.kv_head_idx + 1) * ratio] += 1
-            if i.merge_in_last and ctr[i.layer_idx, 1, i.kv_head_idx * ratio] == i.num_partials:
+            if i.merge_in_last == 1 and ctr[i.layer_idx, 1, i.kv_head_idx * ratio] == i.num_partials:
                 ctr[i.layer_idx, 2, 0] += ratio
         elif op == 3:
             ctr[i.layer_idx, 2, 0] += ratio
@@ -216,7 +219,7 @@ def _simulate(sched, num_layers):
     return ctr
 
 
-@pytest.mark.parametrize("which", ["reference", "mi355x", "mi355x_97"])
+@pytest.mark.parametrize("which", ["reference", "mi355x", "mi355x_last", "mi355x_97"])
 def test_queues_drain_and_counters_end_state(which):
     import dataclasses
 
@@ -225,14 +228,20 @@ def test_queues_drain_and_counters_end_state(which):
         sched = S.reference_scheduler(shape)
     elif which == "mi355x":
         sched = S.mi355x_scheduler(shape, num_partials=16)
+    elif which == "mi355x_last":
+        sched = S.mi355x_scheduler(shape, num_partials=5, attention_merge="last")
     else:  # an awkward workgroup count must still be a valid schedule
         sched = S.mi355x_scheduler(shape, sm_count=97, num_partials=7)
     ctr = _simulate(sched, 3)
     bph, opb, ubk, dwn = sched.expected_counts()
     for layer in range(3):
         assert (ctr[layer, 0, : shape.num_heads] == bph).all()
-        assert (ctr[layer, 1, : shape.num_attention_heads] == sched.num_partials).all()
-        assert ctr[layer, 2, 0] == shape.num_attention_heads
+        if sched.attention_merge == "oproj":
+            assert ctr[layer, 1].sum() == 0
+            assert ctr[layer, 2, 0] == shape.num_key_value_heads * sched.num_partials
+        else:
+            assert (ctr[layer, 1, : shape.num_attention_heads] == sched.num_partials).all()
+            assert ctr[layer, 2, 0] == shape.num_attention_heads
         assert ctr[layer, 3, 0] == opb
         assert (ctr[layer, 4, : sched.geometry.num_split_k(shape)] == ubk).all()
         assert ctr[layer, 5, 0] == dwn
@@ -243,8 +252,8 @@ def test_pick_num_partials():
     assert S.pick_num_partials(108, max_partials=16) == 13            # the reference's A100 answer
     assert S.pick_num_partials(256) == S.MAX_ATTENTION_PARTIALS == 25
     assert S.pick_num_partials(256, kv_capacity=40) == 1
-    assert S.pick_num_partials(256, kv_capacity=136) == 3
-    assert S.pick_num_partials(256, kv_capacity=1032) == 17
+    assert S.pick_num_partials(256, kv_capacity=300) == 2
+    assert S.pick_num_partials(256, kv_capacity=1032) == 5
     assert S.pick_num_partials(4) == 1
     with pytest.raises(ValueError):
         S.schedule_attention_split_kv(0, 26)
