@@ -112,11 +112,13 @@ __device__ __forceinline__ bool wg_wait_all(const Params& p, Smem<M>& s, const C
 // RMSNorm of the residual stream into s.x as bf16:
 //   n = bf16(x * rsqrt(mean(x^2) + eps));  y = bf16(w * n)
 // (fused/operations.py:126-131 — two roundings, the product taken on bf16 values).
-template <class M>
-__device__ __forceinline__ void rms_to_lds(const Params& p, Smem<M>& s, const u16* hidden, const u16* weight) {
+template <class M, class AfterIssue>
+__device__ __forceinline__ void rms_to_lds(const Params& p, Smem<M>& s, const u16* hidden, const u16* weight, AfterIssue after_issue) {
   static_assert(M::H == kThreads * 4, "one thread normalises four elements");
   const int t = threadIdx.x;
   const uint64_t hw = ld_shared64(hidden + t * 4);
+  asm volatile("" ::: "memory");
+  after_issue();  // further loads queue up behind the residual stream, not in front of it
   const uint32_t hlo = static_cast<uint32_t>(hw), hhi = static_cast<uint32_t>(hw >> 32);
   const float x0 = bf_lo(hlo), x1 = bf_hi(hlo), x2 = bf_lo(hhi), x3 = bf_hi(hhi);
   float ss = __builtin_fmaf(x3, x3, __builtin_fmaf(x2, x2, __builtin_fmaf(x1, x1, x0 * x0)));
@@ -133,6 +135,10 @@ __device__ __forceinline__ void rms_to_lds(const Params& p, Smem<M>& s, const u1
   out.y = static_cast<uint32_t>(y2) | (static_cast<uint32_t>(y3) << 16);
   *reinterpret_cast<uint2*>(s.x + t * 4) = out;
   __syncthreads();
+}
+template <class M>
+__device__ __forceinline__ void rms_to_lds(const Params& p, Smem<M>& s, const u16* hidden, const u16* weight) {
+  rms_to_lds(p, s, hidden, weight, [] {});
 }
 
 // Interleaved-pair RoPE on bf16-rounded inputs, evaluated in fp32 with a
@@ -151,33 +157,54 @@ __device__ __forceinline__ uint32_t rope_pair(float v0, float v1, const float* c
 constexpr int kDepth = QMK_DEPTH;  // row buffers per wave: 4 x CH x 16 B per lane in flight
 
 // Wave w consumes elements w, w+8, w+16, ... of a sequence of weight-row segments
-// (`src(e)` = address of CH*512 bf16).  `buf[k]` must already hold element w + 8k
-// (issued by `preload` before the counter wait); each buffer is refilled with the
-// element 32 further on as soon as it has been consumed.  `use(e, buf)` gets the
-// raw registers of element e.
-template <int CH, class Src>
-__device__ __forceinline__ void preload(int n, Src src, RowRegs<CH> (&buf)[kDepth]) {
+// (`src(e)` = address of CH*512 bf16) through NB register buffers.  `buf[k]` must already hold
+// element w + 8k (issued by `preload` / `preload_range`); each buffer is refilled with the
+// element 8*NB further on as soon as it has been consumed.  `use(e, buf)` gets the raw
+// registers of element e.
+//
+// How much to ask for before the counter wait is a trade: what is in flight then lands while
+// the workgroup waits, but it also stands in the memory queues in front of the last producers'
+// stores and counter updates, and in front of this wave's own counter poll (loads return in
+// issue order).  So the big GEMVs ask for kEarly buffers up front and for the rest right after
+// the wait, behind the activation read.
+template <int K0, int K1, int CH, int NB, class Src>
+__device__ __forceinline__ void preload_range(int n, Src src, RowRegs<CH> (&buf)[NB]) {
+  static_assert(K0 >= 0 && K1 <= NB, "buffer range");
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
 #pragma unroll
-  for (int k = 0; k < kDepth; ++k)
+  for (int k = K0; k < K1; ++k)
     if (wave + k * kWaves < n) load_row(buf[k], src(wave + k * kWaves), lane);
 }
 
-template <int CH, class Src, class Use>
-__device__ __forceinline__ void stream(int n, Src src, RowRegs<CH> (&buf)[kDepth], Use use) {
+template <int CH, int NB, class Src>
+__device__ __forceinline__ void preload(int n, Src src, RowRegs<CH> (&buf)[NB]) {
+  preload_range<0, NB>(n, src, buf);
+}
+
+template <int CH, int NB, class Src, class Use>
+__device__ __forceinline__ void stream(int n, Src src, RowRegs<CH> (&buf)[NB], Use use) {
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-  for (int e = wave; e < n; e += kDepth * kWaves) {
+  for (int e = wave; e < n; e += NB * kWaves) {
 #pragma unroll
-    for (int k = 0; k < kDepth; ++k) {
+    for (int k = 0; k < NB; ++k) {
       const int ek = e + k * kWaves;
       if (ek < n) {
         use(ek, buf[k]);
-        const int nx = ek + kDepth * kWaves;
+        const int nx = ek + NB * kWaves;
         if (nx < n) load_row(buf[k], src(nx), lane);
       }
     }
   }
 }
+
+#ifndef QMK_EARLY
+#define QMK_EARLY 4
+#endif
+#ifndef QMK_UPGATE_BUFFERS
+#define QMK_UPGATE_BUFFERS 4
+#endif
+constexpr int kEarly = QMK_EARLY;                    // buffers of a big GEMV requested before its counter wait
+constexpr int kUpGateBuffers = QMK_UPGATE_BUFFERS;   // row buffers of the up/gate GEMV
 
 // ===================================================================== 1 ==
 // [1, layer, tile_M, n_start, n_end, tile_M_g, tile_N_g]
@@ -202,13 +229,16 @@ __device__ bool op_rms_qkv_rope(const Params& p, Smem<M>& s, const Ctx& c) {
     if (!wg_wait_all(p, s, c, layer - 1, ROW_DOWN, 0, p.down_arrivals)) return false;
   }
   rms_to_lds(p, s, p.hidden, p.attn_norm + static_cast<size_t>(layer) * M::H);
+  QMK_STAMP(0);
   v4u x[CH];
   load_x_from_lds(x, s.x, lane);
   stream<CH>(nrows, src, buf, [&](int r, const RowRegs<CH>& w) {
     const float sum = wave_sum(dot_row(w, x));
     if (lane == 0) s.res[r] = sum;
   });
+  QMK_STAMP(1);
   __syncthreads();
+  QMK_STAMP(2);
 
   // Epilogue: the GEMV result is bf16 before RoPE; q -> q_post_rope, k/v -> cache row of this position.
   const float* cosr = p.rope_cos + static_cast<size_t>(p.pos_id) * M::D;
@@ -593,13 +623,16 @@ __device__ bool op_oproj_residual(const Params& p, Smem<M>& s, const Ctx& c) {
     }
   }
   __syncthreads();
+  QMK_STAMP(0);
   v4u x[CH];
   load_x_from_lds(x, s.x, lane);
   stream<CH>(nrows, src, buf, [&](int r, const RowRegs<CH>& w) {
     const float sum = wave_sum(dot_row(w, x));
     if (lane == 0) s.res[r] = sum;
   });
+  QMK_STAMP(1);
   __syncthreads();
+  QMK_STAMP(2);
   for (int pair = threadIdx.x; pair < nrows / 2; pair += kThreads)
     residual_pair(p.hidden + rs + 2 * pair, s.res[2 * pair], s.res[2 * pair + 1]);
 
@@ -633,17 +666,21 @@ __device__ bool op_rms_upgate_silu(const Params& p, Smem<M>& s, const Ctx& c) {
   auto row_of = [&](int i) { return s.inst[4 + i / tile] * tile + i % tile; };
   auto src = [&](int e) { return ((e & 1) ? Wg : Wu) + static_cast<size_t>(row_of(e >> 1)) * M::H; };
 
-  RowRegs<CH> buf[kDepth];
-  preload<CH>(nrows, src, buf);
+  RowRegs<CH> buf[kUpGateBuffers];
+  preload_range<0, kEarly>(nrows, src, buf);
   if (!wg_wait_all(p, s, c, layer, ROW_OPROJ, 0, p.oproj_blocks)) return false;
-  rms_to_lds(p, s, p.hidden, p.mlp_norm + static_cast<size_t>(layer) * M::H);
+  rms_to_lds(p, s, p.hidden, p.mlp_norm + static_cast<size_t>(layer) * M::H,
+             [&] { preload_range<kEarly, kUpGateBuffers>(nrows, src, buf); });
+  QMK_STAMP(0);
   v4u x[CH];
   load_x_from_lds(x, s.x, lane);
   stream<CH>(nrows, src, buf, [&](int e, const RowRegs<CH>& w) {
     const float sum = wave_sum(dot_row(w, x));
     if (lane == 0) s.res[e] = sum;
   });
+  QMK_STAMP(1);
   __syncthreads();
+  QMK_STAMP(2);
   // Two neighbouring outputs of a tile leave as one 32-bit word.
   for (int pair = threadIdx.x; pair < nout / 2; pair += kThreads) {
     uint32_t word = 0;
@@ -716,13 +753,22 @@ __device__ bool op_down_residual(const Params& p, Smem<M>& s, const Ctx& c) {
   const int n_elems = wave + kWaves * (rows_w * segs - 1) + 1;      // last element index of this wave + 1 (<= wave if none)
 
   RowRegs<CH> buf[kDepth];
-  preload<CH>(rows_w > 0 ? n_elems : 0, src, buf);
+  static_assert(kEarly <= kDepth, "early buffers are a subset of the ring");
+  preload_range<0, kEarly>(rows_w > 0 ? n_elems : 0, src, buf);
   if (xcd_counters(p) && (split != 0 || kg != M::F)) return bad_operand(p, s, c, 8);  // sub-counters cover one K slice
   if (!wg_wait_all(p, s, c, layer, ROW_UPGATE, split, p.upgate_blocks_per_bucket)) return false;
 
-  // The K slice of silu_out into LDS.
-  for (int i = threadIdx.x; i < kg / 4; i += kThreads)
-    reinterpret_cast<uint64_t*>(s.x)[i] = ld_shared64(p.silu_out + ks + i * 4);
+  // The K slice of silu_out into LDS; the remaining row buffers are requested behind it.
+  static_assert(M::F / 4 == 4 * kThreads, "four 8-byte loads per thread cover the widest slice");
+  uint64_t act[4];
+#pragma unroll
+  for (int k = 0; k < 4; ++k)
+    if (static_cast<int>(threadIdx.x) + k * kThreads < kg / 4) act[k] = ld_shared64(p.silu_out + ks + (threadIdx.x + k * kThreads) * 4);
+  asm volatile("" ::: "memory");
+  preload_range<kEarly, kDepth>(rows_w > 0 ? n_elems : 0, src, buf);
+#pragma unroll
+  for (int k = 0; k < 4; ++k)
+    if (static_cast<int>(threadIdx.x) + k * kThreads < kg / 4) reinterpret_cast<uint64_t*>(s.x)[threadIdx.x + k * kThreads] = act[k];
   __syncthreads();
 
   float acc = 0.f;
@@ -738,7 +784,9 @@ __device__ bool op_down_residual(const Params& p, Smem<M>& s, const Ctx& c) {
       if (lane == 0) s.res[row_of(e)] = sum;
     }
   });
+  QMK_STAMP(1);
   __syncthreads();
+  QMK_STAMP(2);
 
   if (kg == M::F) {  // one slice: every row has a single writer
     for (int pair = threadIdx.x; pair < nrows / 2; pair += kThreads)

@@ -52,9 +52,10 @@ REFERENCE_MAX_ATTENTION_PARTIALS = 16
 MAX_ATTENTION_PARTIALS = ATTENTION_REDUCTION_LIST_CAPACITY
 #: value of the split-KV instruction's ``merge_in_last`` word per merge mode
 ATTENTION_MERGE_MODES = {"separate": 0, "last": 1, "oproj": 2}
-#: KV tokens per split-KV partial the fan-out aims for: four passes of a workgroup (8 waves x 8
-#: tokens per pass).  Finer splits cost more in merging than they save in streaming (measured).
-KV_TOKENS_PER_PASS = 256
+#: KV tokens per split-KV partial the fan-out aims for: five passes of a workgroup (8 waves x 8
+#: tokens per pass).  Finer splits cost more in merging than they save in streaming (measured:
+#: at a 1032-token capacity 4 partials per KV head beat 5 by 3 % and 3 by 2 %).
+KV_TOKENS_PER_PASS = 320
 
 
 def _ceil_div(a: int, b: int) -> int:

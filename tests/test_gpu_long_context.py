@@ -40,7 +40,7 @@ def test_long_context_attention(context, merge):
     g.q_post_rope.copy_((torch.randn(shape.hidden_size, generator=gen, device="cuda") * 0.4).bfloat16())
     g.position_id = context - 1
     sched = S.mi355x_scheduler(shape, kv_capacity=context, attention_merge=merge)
-    assert sched.num_partials == min(25, -(-context // 256))
+    assert sched.num_partials == min(25, -(-context // S.KV_TOKENS_PER_PASS))
     g.barriers[0, 0, :] = sched.expected_counts()[0]
     ins = sched.attention_split_kv(0) + sched.attention_reduction(0)
     mk = mk_kernel.get_mk(reset_barriers=False)

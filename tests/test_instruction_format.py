@@ -252,8 +252,9 @@ def test_pick_num_partials():
     assert S.pick_num_partials(108, max_partials=16) == 13            # the reference's A100 answer
     assert S.pick_num_partials(256) == S.MAX_ATTENTION_PARTIALS == 25
     assert S.pick_num_partials(256, kv_capacity=40) == 1
-    assert S.pick_num_partials(256, kv_capacity=300) == 2
-    assert S.pick_num_partials(256, kv_capacity=1032) == 5
+    assert S.pick_num_partials(256, kv_capacity=300) == 1
+    assert S.pick_num_partials(256, kv_capacity=400) == 2
+    assert S.pick_num_partials(256, kv_capacity=1032) == 4
     assert S.pick_num_partials(4) == 1
     with pytest.raises(ValueError):
         S.schedule_attention_split_kv(0, 26)
