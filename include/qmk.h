@@ -30,7 +30,7 @@
 extern "C" {
 #endif
 
-#define QMK_ABI_VERSION 1
+#define QMK_ABI_VERSION 2
 #define QMK_INSTRUCTION_WORDS 32
 
 /* Return / status codes. 0 is success; everything else is an error. */
@@ -70,6 +70,19 @@ enum {
 #define QMK_XCD_COUNTER_ROWS 54
 
 /* Flags. */
+#define QMK_FLAG_TAGGED 4u         /* the small vectors that every workgroup hands to others inside a
+                                      launch (q and the appended K/V row, the residual stream after
+                                      the O-proj and after the down projection) also travel through
+                                      `workspace` as 8-byte units {32-bit payload, 32-bit tag}, the
+                                      tag naming launch and layer.  A consumer polls the units it
+                                      needs until they carry the tag it expects, and the producer
+                                      neither waits for its stores to be acknowledged nor counts an
+                                      arrival: one memory round trip per hand-over instead of four.
+                                      Needs `workspace` (qmk_workspace_bytes), at most 63 layers and
+                                      a schedule whose down projection is not split along K; not
+                                      combinable with QMK_FLAG_KEEP_BARRIERS.  The caller's buffers
+                                      receive the same values as without the flag; counter rows 0,
+                                      3 and 5 stay zero.                                          */
 #define QMK_FLAG_KEEP_BARRIERS 1u  /* leave the final counter values in `barriers`
                                       (the reference's behaviour); by default the
                                       last workgroup to retire clears them so the
@@ -144,11 +157,19 @@ typedef struct QmkArgs {
                                       (100 MHz ticks), opcode | layer << 8, and four
                                       op-specific intermediate stamps; NULL = off */
   void* stream;                    /* hipStream_t; NULL = the null stream         */
+  void* workspace;                 /* QMK_FLAG_TAGGED: device buffer of workspace_bytes, 128-byte
+                                      aligned, zeroed once when allocated and then left to the
+                                      library (it carries a launch count from step to step); NULL
+                                      otherwise                                                  */
+  uint64_t workspace_bytes;        /* >= qmk_workspace_bytes(model)               */
 } QmkArgs;
 
 /* Launch one decode step asynchronously on args->stream.  Returns QMK_OK or a
  * host-side QMK_ERR_*.  Device-side errors surface through qmk_status_fetch. */
 int qmk_decode_step(const QmkArgs* args);
+
+/* Size of QmkArgs.workspace for QMK_FLAG_TAGGED; 0 for an unknown model. */
+uint64_t qmk_workspace_bytes(int model);
 
 /* Device/library properties (QMK_QUERY_*); negative on error. */
 int qmk_query(int what);

@@ -27,6 +27,7 @@ template <class M>
 __global__ __launch_bounds__(kThreads, 1) void decode_megakernel(const Params p) {
   __shared__ Smem<M> s;
   if (threadIdx.x < 8) s.ctl[threadIdx.x] = 0;
+  if (threadIdx.x == 0) s.generation = tagged(p) ? ld_shared32(p.ws + kWsGeneration) : 0u;
   __syncthreads();
 
   const int32_t* queue = p.instructions + static_cast<size_t>(blockIdx.x) * p.num_insts * kInstWords;
@@ -83,6 +84,8 @@ __global__ __launch_bounds__(kThreads, 1) void decode_megakernel(const Params p)
     const int total = p.num_layers * p.num_layer_barriers * p.barrier_slots;
     for (int i = threadIdx.x; i < total; i += kThreads)
       __hip_atomic_store(p.barriers + i, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    // The next launch tags its activations with the next count (26 bits: the tag keeps 6 for the layer).
+    if (tagged(p) && threadIdx.x == 0) st_shared32(p.ws + kWsGeneration, (s.generation + 1u) & 0x03ffffffu);
   }
 }
 
@@ -147,6 +150,13 @@ extern "C" int qmk_decode_step(const QmkArgs* a) {
     if (layer_ints < needed || !aligned) return QMK_ERR_SHAPE;
   }
 
+  if (a->flags & QMK_FLAG_TAGGED) {
+    if (a->workspace == nullptr) return QMK_ERR_NULL_ARG;
+    if ((a->flags & QMK_FLAG_KEEP_BARRIERS) || a->num_layers > 63 || reinterpret_cast<uintptr_t>(a->workspace) % 128 != 0 ||
+        a->workspace_bytes < qmk_workspace_bytes(static_cast<int>(a->model)))
+      return QMK_ERR_SHAPE;
+  }
+
   DeviceInfo* dev = nullptr;
   if (int rc = device_info(&dev); rc != QMK_OK) return rc;
   if (a->num_queues > dev->max_queues) return QMK_ERR_TOO_MANY_QUEUES;
@@ -175,6 +185,7 @@ extern "C" int qmk_decode_step(const QmkArgs* a) {
   p.lm_norm = static_cast<const u16*>(a->lm_head_norm_weights);
   p.lm_w = static_cast<const u16*>(a->lm_head_weights);
   p.barriers = a->barriers;
+  p.ws = (a->flags & QMK_FLAG_TAGGED) ? static_cast<uint64_t*>(a->workspace) : nullptr;
   p.timeline = a->timeline;
   p.status = dev->status;
   p.num_insts = a->num_insts;
@@ -198,6 +209,10 @@ extern "C" int qmk_decode_step(const QmkArgs* a) {
   hipLaunchKernelGGL(decode_megakernel<M>, dim3(a->num_queues), dim3(kThreads), 0,
                      static_cast<hipStream_t>(a->stream), p);
   return hipGetLastError() == hipSuccess ? QMK_OK : QMK_ERR_LAUNCH;
+}
+
+extern "C" uint64_t qmk_workspace_bytes(int model) {
+  return model == QMK_MODEL_LLAMA_3_2_1B ? static_cast<uint64_t>(kWsUnits) * sizeof(uint64_t) : 0;
 }
 
 extern "C" int qmk_query(int what) {

@@ -45,6 +45,7 @@ struct Params {
   const u16* lm_norm;
   const u16* lm_w;
   int32_t* barriers;
+  uint64_t* ws;         // tagged-activation workspace (QMK_FLAG_TAGGED), else null
   uint64_t* timeline;
   int32_t* status;      // device status words: {code, workgroup, inst, opcode, operand}
   int32_t num_insts;
@@ -205,6 +206,56 @@ __device__ __forceinline__ v4u ld_shared128(const void* p) {
   r.z = static_cast<uint32_t>(hi); r.w = static_cast<uint32_t>(hi >> 32);
   return r;
 }
+// ---- tagged activations (QMK_FLAG_TAGGED) ----
+// A hand-over through a counter costs four dependent trips to memory: the producer waits for its
+// stores to be acknowledged, adds to the counter, the consumer's poll sees the count, and only
+// then does the consumer fetch the data.  Here the data announces itself: every 8-byte unit of
+// the workspace is {32-bit payload, 32-bit tag}, written with one 64-bit store, and the tag
+// names the launch (a count kept in the workspace) and the layer.  The consumer polls the units
+// it needs until they carry the tag it expects: one trip.  A unit is never overwritten before
+// all its readers are done: its next writer depends, through the layer's data flow, on every one
+// of them.  Only the small vectors travel this way (every thread of every workgroup re-reading a
+// large one while it waits would flood the fabric).  Offsets below are in units of 8 bytes.
+constexpr int kWsGeneration = 0;            // launch count (first 128-byte line)
+constexpr int kWsQ = 512;                   // q after RoPE: NQ*D/2 units (two bf16 each)
+constexpr int kWsK = kWsQ + 1024;           // appended K row: NKV*D/2 units
+constexpr int kWsV = kWsK + 256;            // appended V row
+constexpr int kWsHiddenMid = kWsV + 256;    // residual stream after the O-proj: H/2 units
+constexpr int kWsHiddenOut = kWsHiddenMid + 1024;  // residual stream after the down projection
+constexpr int kWsUnits = kWsHiddenOut + 1024;
+
+__device__ __forceinline__ bool tagged(const Params& p) { return (p.flags & QMK_FLAG_TAGGED) != 0; }
+__device__ __forceinline__ uint32_t tag_of(uint32_t generation, int layer) { return (generation << 6) + static_cast<uint32_t>(layer) + 1u; }
+__device__ __forceinline__ void st_tagged(uint64_t* unit, uint32_t payload, uint32_t tag) {
+  __hip_atomic_store(unit, (static_cast<uint64_t>(tag) << 32) | payload, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+// Poll one unit / two neighbouring units until they carry `tag`; false when the budget runs out.
+__device__ __forceinline__ bool poll_tagged1(const uint64_t* unit, uint32_t tag, uint32_t limit, uint32_t& a) {
+  uint32_t polls = 0;
+  while (true) {
+    const uint64_t x = ld_shared64(unit);
+    if (static_cast<uint32_t>(x >> 32) == tag) {
+      a = static_cast<uint32_t>(x);
+      return true;
+    }
+    if (++polls > limit) return false;
+    __builtin_amdgcn_s_sleep(1);
+  }
+}
+__device__ __forceinline__ bool poll_tagged2(const uint64_t* units, uint32_t tag, uint32_t limit, uint32_t& a, uint32_t& b) {
+  uint32_t polls = 0;
+  while (true) {
+    const uint64_t x = ld_shared64(units), y = ld_shared64(units + 1);
+    if (static_cast<uint32_t>(x >> 32) == tag && static_cast<uint32_t>(y >> 32) == tag) {
+      a = static_cast<uint32_t>(x);
+      b = static_cast<uint32_t>(y);
+      return true;
+    }
+    if (++polls > limit) return false;
+    __builtin_amdgcn_s_sleep(1);
+  }
+}
+
 __device__ __forceinline__ void st_shared32(void* p, uint32_t v) {
   __hip_atomic_store(static_cast<uint32_t*>(p), v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }

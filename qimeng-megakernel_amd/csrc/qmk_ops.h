@@ -30,6 +30,7 @@ template <class M>
 struct Smem {
   int32_t inst[kInstWords];
   int32_t ctl[8];                       // [0] abort, [1] last workgroup to retire
+  uint32_t generation;                  // launch count of the tagged-activation workspace
   float red[kWaves];
   alignas(16) u16 x[M::F];              // activation vector handed to the GEMV lanes
   float res[kResSlots];                 // per-row GEMV results awaiting the epilogue pass
@@ -112,14 +113,32 @@ __device__ __forceinline__ bool wg_wait_all(const Params& p, Smem<M>& s, const C
 // RMSNorm of the residual stream into s.x as bf16:
 //   n = bf16(x * rsqrt(mean(x^2) + eps));  y = bf16(w * n)
 // (fused/operations.py:126-131 — two roundings, the product taken on bf16 values).
+// The residual stream comes from the caller's buffer (units == nullptr: a counter wait has made
+// it complete) or from its tagged copy, each thread polling its own two units.  False
+// (uniformly) when a tagged poll ran out of budget.
 template <class M, class AfterIssue>
-__device__ __forceinline__ void rms_to_lds(const Params& p, Smem<M>& s, const u16* hidden, const u16* weight, AfterIssue after_issue) {
+__device__ __forceinline__ bool rms_to_lds(const Params& p, Smem<M>& s, const Ctx& c, const uint64_t* units, uint32_t tag,
+                                           const u16* weight, AfterIssue after_issue) {
   static_assert(M::H == kThreads * 4, "one thread normalises four elements");
   const int t = threadIdx.x;
-  const uint64_t hw = ld_shared64(hidden + t * 4);
-  asm volatile("" ::: "memory");
-  after_issue();  // further loads queue up behind the residual stream, not in front of it
-  const uint32_t hlo = static_cast<uint32_t>(hw), hhi = static_cast<uint32_t>(hw >> 32);
+  uint32_t hlo, hhi;
+  if (units == nullptr) {
+    const uint64_t hw = ld_shared64(p.hidden + t * 4);
+    asm volatile("" ::: "memory");
+    after_issue();  // further loads queue up behind the residual stream, not in front of it
+    hlo = static_cast<uint32_t>(hw);
+    hhi = static_cast<uint32_t>(hw >> 32);
+  } else {
+    if (!poll_tagged2(units + 2 * t, tag, p.spin_limit, hlo, hhi)) {
+      s.ctl[0] = 1;
+      report_error(p, QMK_DEV_WAIT_TIMEOUT, c.inst_idx, c.opcode, t);
+    }
+    if (p.timeline != nullptr && t == 0) {
+      s.t_wait = wall_clock64();
+      s.ctl[2] = 1;
+    }
+    after_issue();
+  }
   const float x0 = bf_lo(hlo), x1 = bf_hi(hlo), x2 = bf_lo(hhi), x3 = bf_hi(hhi);
   float ss = __builtin_fmaf(x3, x3, __builtin_fmaf(x2, x2, __builtin_fmaf(x1, x1, x0 * x0)));
   ss = block_sum(ss, s.red);
@@ -135,10 +154,12 @@ __device__ __forceinline__ void rms_to_lds(const Params& p, Smem<M>& s, const u1
   out.y = static_cast<uint32_t>(y2) | (static_cast<uint32_t>(y3) << 16);
   *reinterpret_cast<uint2*>(s.x + t * 4) = out;
   __syncthreads();
+  return s.ctl[0] == 0;
 }
 template <class M>
-__device__ __forceinline__ void rms_to_lds(const Params& p, Smem<M>& s, const u16* hidden, const u16* weight) {
-  rms_to_lds(p, s, hidden, weight, [] {});
+__device__ __forceinline__ bool rms_to_lds(const Params& p, Smem<M>& s, const Ctx& c, const uint64_t* units, uint32_t tag,
+                                           const u16* weight) {
+  return rms_to_lds(p, s, c, units, tag, weight, [] {});
 }
 
 // Interleaved-pair RoPE on bf16-rounded inputs, evaluated in fp32 with a
@@ -203,7 +224,11 @@ __device__ __forceinline__ void stream(int n, Src src, RowRegs<CH> (&buf)[NB], U
 #ifndef QMK_UPGATE_BUFFERS
 #define QMK_UPGATE_BUFFERS 4
 #endif
-constexpr int kEarly = QMK_EARLY;                    // buffers of a big GEMV requested before its counter wait
+#ifndef QMK_EARLY_UPGATE
+#define QMK_EARLY_UPGATE QMK_EARLY
+#endif
+constexpr int kEarly = QMK_EARLY;                    // buffers of the down projection requested before its counter wait
+constexpr int kEarlyUpGate = QMK_EARLY_UPGATE;       // the same for the up/gate GEMV
 constexpr int kUpGateBuffers = QMK_UPGATE_BUFFERS;   // row buffers of the up/gate GEMV
 
 // ===================================================================== 1 ==
@@ -225,10 +250,13 @@ __device__ bool op_rms_qkv_rope(const Params& p, Smem<M>& s, const Ctx& c) {
 
   RowRegs<CH> buf[kDepth];
   preload<CH>(nrows, src, buf);  // in flight while the counter is polled
-  if (layer > 0) {
+  const bool tg = tagged(p);
+  const uint32_t tag = tag_of(s.generation, layer);
+  if (layer > 0 && !tg) {
     if (!wg_wait_all(p, s, c, layer - 1, ROW_DOWN, 0, p.down_arrivals)) return false;
   }
-  rms_to_lds(p, s, p.hidden, p.attn_norm + static_cast<size_t>(layer) * M::H);
+  if (!rms_to_lds(p, s, c, (tg && layer > 0) ? p.ws + kWsHiddenOut : nullptr, tag - 1, p.attn_norm + static_cast<size_t>(layer) * M::H))
+    return false;
   QMK_STAMP(0);
   v4u x[CH];
   load_x_from_lds(x, s.x, lane);
@@ -248,15 +276,22 @@ __device__ bool op_rms_qkv_rope(const Params& p, Smem<M>& s, const Ctx& c) {
     const int r = rs + 2 * pair;
     const float v0 = round_bf16(s.res[2 * pair]), v1 = round_bf16(s.res[2 * pair + 1]);
     if (r < M::NQ * M::D) {
-      st_shared32(p.q_post_rope + r, rope_pair(v0, v1, cosr, sinr, r % M::D));
+      const uint32_t w = rope_pair(v0, v1, cosr, sinr, r % M::D);
+      st_shared32(p.q_post_rope + r, w);
+      if (tg) st_tagged(p.ws + kWsQ + r / 2, w, tag);
     } else if (r < (M::NQ + M::NKV) * M::D) {
       const int i = r - M::NQ * M::D;
-      st_shared32(p.k_cache + kv_row + i, rope_pair(v0, v1, cosr, sinr, i % M::D));
+      const uint32_t w = rope_pair(v0, v1, cosr, sinr, i % M::D);
+      st_shared32(p.k_cache + kv_row + i, w);
+      if (tg) st_tagged(p.ws + kWsK + i / 2, w, tag);
     } else {
       const int i = r - (M::NQ + M::NKV) * M::D;
-      st_shared32(p.v_cache + kv_row + i, static_cast<uint32_t>(f2bf(v0)) | (static_cast<uint32_t>(f2bf(v1)) << 16));
+      const uint32_t w = static_cast<uint32_t>(f2bf(v0)) | (static_cast<uint32_t>(f2bf(v1)) << 16);
+      st_shared32(p.v_cache + kv_row + i, w);
+      if (tg) st_tagged(p.ws + kWsV + i / 2, w, tag);
     }
   }
+  if (tg) return true;  // the units announce themselves: nothing to wait for, nothing to count
 
   release_stores();
   __syncthreads();
@@ -359,13 +394,45 @@ __device__ bool op_attn_splitkv(const Params& p, Smem<M>& s, const Ctx& c) {
     vv = *reinterpret_cast<const v4u*>(p.v_cache + base + static_cast<size_t>(t) * tok_stride);
   }
 
-  if (!wg_wait(p, s, c, M::GQA + 2,
-               [&](int i) {
-                 const int slot = i < M::GQA ? kvh * M::GQA + i : (i == M::GQA ? M::NQ + kvh : M::NQ + M::NKV + kvh);
-                 return counter_ptr(p, layer, ROW_QKV, slot);
-               },
-               p.qkv_blocks_per_head))
+  const bool tg = tagged(p);
+  // Tagged mode: q of the four heads (128 units) is polled by threads 0..63, the K and V rows
+  // appended in this launch (32 units each, only when the slice holds this position) by threads
+  // 64..95; all of it is staged in LDS as words [0,128) q, [128,160) k, [160,192) v.
+  const v4u* stage = reinterpret_cast<const v4u*>(s.x);
+  if (tg) {
+    const uint32_t tag = tag_of(s.generation, layer);
+    uint32_t* words = reinterpret_cast<uint32_t*>(s.x);
+    const bool has_new = p.pos_id >= t0 && p.pos_id < t1;
+    bool arrived = true;
+    uint32_t a = 0, b = 0;
+    if (threadIdx.x < 64) {
+      arrived = poll_tagged2(p.ws + kWsQ + kvh * (M::GQA * M::D / 2) + 2 * threadIdx.x, tag, p.spin_limit, a, b);
+      words[2 * threadIdx.x] = a;
+      words[2 * threadIdx.x + 1] = b;
+    } else if (threadIdx.x < 96 && has_new) {
+      const int j = threadIdx.x - 64;
+      arrived = poll_tagged2(p.ws + (j < 16 ? kWsK : kWsV) + kvh * (M::D / 2) + 2 * (j & 15), tag, p.spin_limit, a, b);
+      words[128 + 2 * j] = a;
+      words[128 + 2 * j + 1] = b;
+    }
+    if (!arrived) {
+      s.ctl[0] = 1;
+      report_error(p, QMK_DEV_WAIT_TIMEOUT, c.inst_idx, c.opcode, threadIdx.x);
+    }
+    if (p.timeline != nullptr && threadIdx.x == 0) {
+      s.t_wait = wall_clock64();
+      s.ctl[2] = 1;
+    }
+    __syncthreads();
+    if (s.ctl[0]) return false;
+  } else if (!wg_wait(p, s, c, M::GQA + 2,
+                      [&](int i) {
+                        const int slot = i < M::GQA ? kvh * M::GQA + i : (i == M::GQA ? M::NQ + kvh : M::NQ + M::NKV + kvh);
+                        return counter_ptr(p, layer, ROW_QKV, slot);
+                      },
+                      p.qkv_blocks_per_head)) {
     return false;
+  }
 
   // q[h][8]: this lane's dims of the four query heads, pre-scaled into the log2 domain.
   const float qscale = p.attn_scale * 1.4426950408889634f;
@@ -373,10 +440,11 @@ __device__ bool op_attn_splitkv(const Params& p, Smem<M>& s, const Ctx& c) {
   {
     v4u qv[M::GQA];
 #pragma unroll
-    for (int h = 0; h < M::GQA; ++h) qv[h] = ld_shared128(p.q_post_rope + (kvh * M::GQA + h) * M::D + col * 8);
+    for (int h = 0; h < M::GQA; ++h)
+      qv[h] = tg ? stage[h * (M::D / 8) + col] : ld_shared128(p.q_post_rope + (kvh * M::GQA + h) * M::D + col * 8);
     if (t < t1 && t == p.pos_id) {  // the row another workgroup appended during this launch
-      kv = ld_shared128(p.k_cache + base + static_cast<size_t>(t) * tok_stride);
-      vv = ld_shared128(p.v_cache + base + static_cast<size_t>(t) * tok_stride);
+      kv = tg ? stage[32 + col] : ld_shared128(p.k_cache + base + static_cast<size_t>(t) * tok_stride);
+      vv = tg ? stage[40 + col] : ld_shared128(p.v_cache + base + static_cast<size_t>(t) * tok_stride);
     }
 #pragma unroll
     for (int h = 0; h < M::GQA; ++h) {
@@ -404,8 +472,8 @@ __device__ bool op_attn_splitkv(const Params& p, Smem<M>& s, const Ctx& c) {
     if (tn < t1) {
       const size_t off = base + static_cast<size_t>(tn) * tok_stride;
       if (tn == p.pos_id) {
-        kn = ld_shared128(p.k_cache + off);
-        vn = ld_shared128(p.v_cache + off);
+        kn = tg ? stage[32 + col] : ld_shared128(p.k_cache + off);
+        vn = tg ? stage[40 + col] : ld_shared128(p.v_cache + off);
       } else {
         kn = *reinterpret_cast<const v4u*>(p.k_cache + off);
         vn = *reinterpret_cast<const v4u*>(p.v_cache + off);
@@ -544,6 +612,23 @@ __device__ bool op_attn_reduce(const Params& p, Smem<M>& s, const Ctx& c) {
   return true;
 }
 
+// Two neighbouring residual-stream elements plus bf16(delta), as a bf16 pair.
+__device__ __forceinline__ uint32_t residual_word(uint32_t old, float d0, float d1) {
+  const u16 n0 = f2bf(bf_lo(old) + round_bf16(d0));
+  const u16 n1 = f2bf(bf_hi(old) + round_bf16(d1));
+  return static_cast<uint32_t>(n0) | (static_cast<uint32_t>(n1) << 16);
+}
+
+// The residual-stream pair `pair` of the rows [rs, ...) before this instruction adds to it: from
+// the caller's buffer, or from the tagged copy `units` (tag `tag`) of the previous writer.
+__device__ __forceinline__ bool residual_in(const Params& p, const uint64_t* units, uint32_t tag, int rs, int pair, uint32_t& old) {
+  if (units == nullptr) {
+    old = ld_shared32(p.hidden + rs + 2 * pair);
+    return true;
+  }
+  return poll_tagged1(units + (rs + 2 * pair) / 2, tag, p.spin_limit, old);
+}
+
 // hidden[r0], hidden[r0+1] += bf16(delta): one coherent 32-bit read-modify-write.
 __device__ __forceinline__ void residual_pair(u16* hidden_pair, float d0, float d1) {
   const uint32_t old = ld_shared32(hidden_pair);
@@ -573,6 +658,17 @@ __device__ bool op_oproj_residual(const Params& p, Smem<M>& s, const Ctx& c) {
   RowRegs<CH> buf[kDepth];
   preload<CH>(nrows, src, buf);
   static_assert(M::H == kThreads * 4, "one thread stages four elements");
+  // Tagged mode: the rows' residual values are those the previous layer's down projection
+  // announced (layer 0: the caller's buffer); they are fetched now, long before they are needed.
+  const bool tg = tagged(p);
+  const uint32_t tag = tag_of(s.generation, layer);
+  if (tg && nrows / 2 > kThreads) return bad_operand(p, s, c, 4);  // one residual pair per thread
+  uint32_t res_old = 0;
+  if (tg && static_cast<int>(threadIdx.x) < nrows / 2 &&
+      !residual_in(p, layer > 0 ? p.ws + kWsHiddenOut : nullptr, tag - 1, rs, threadIdx.x, res_old)) {
+    s.ctl[0] = 1;  // seen by everybody after the barrier inside the wait below
+    report_error(p, QMK_DEV_WAIT_TIMEOUT, c.inst_idx, c.opcode, threadIdx.x);
+  }
   const int self_merge = s.inst[5];  // reduction_block_idx: 0, or the split-KV fan-out P when this op merges
   if (self_merge == 0) {
     if (!wg_wait(p, s, c, 1, [&](int) { return counter_ptr(p, layer, ROW_REDUCE, 0); }, M::NQ)) return false;
@@ -633,6 +729,16 @@ __device__ bool op_oproj_residual(const Params& p, Smem<M>& s, const Ctx& c) {
   QMK_STAMP(1);
   __syncthreads();
   QMK_STAMP(2);
+  if (tg) {
+    // The new pair goes to the caller's buffer and, tagged, to the up/gate workgroups.
+    if (static_cast<int>(threadIdx.x) < nrows / 2) {
+      const int pair = threadIdx.x;
+      const uint32_t w = residual_word(res_old, s.res[2 * pair], s.res[2 * pair + 1]);
+      st_tagged(p.ws + kWsHiddenMid + (rs + 2 * pair) / 2, w, tag);
+      st_shared32(p.hidden + rs + 2 * pair, w);
+    }
+    return true;
+  }
   for (int pair = threadIdx.x; pair < nrows / 2; pair += kThreads)
     residual_pair(p.hidden + rs + 2 * pair, s.res[2 * pair], s.res[2 * pair + 1]);
 
@@ -667,10 +773,12 @@ __device__ bool op_rms_upgate_silu(const Params& p, Smem<M>& s, const Ctx& c) {
   auto src = [&](int e) { return ((e & 1) ? Wg : Wu) + static_cast<size_t>(row_of(e >> 1)) * M::H; };
 
   RowRegs<CH> buf[kUpGateBuffers];
-  preload_range<0, kEarly>(nrows, src, buf);
-  if (!wg_wait_all(p, s, c, layer, ROW_OPROJ, 0, p.oproj_blocks)) return false;
-  rms_to_lds(p, s, p.hidden, p.mlp_norm + static_cast<size_t>(layer) * M::H,
-             [&] { preload_range<kEarly, kUpGateBuffers>(nrows, src, buf); });
+  preload_range<0, kEarlyUpGate>(nrows, src, buf);
+  const bool tg = tagged(p);
+  if (!tg && !wg_wait_all(p, s, c, layer, ROW_OPROJ, 0, p.oproj_blocks)) return false;
+  if (!rms_to_lds(p, s, c, tg ? p.ws + kWsHiddenMid : nullptr, tag_of(s.generation, layer), p.mlp_norm + static_cast<size_t>(layer) * M::H,
+                  [&] { preload_range<kEarlyUpGate, kUpGateBuffers>(nrows, src, buf); }))
+    return false;
   QMK_STAMP(0);
   v4u x[CH];
   load_x_from_lds(x, s.x, lane);
@@ -755,7 +863,16 @@ __device__ bool op_down_residual(const Params& p, Smem<M>& s, const Ctx& c) {
   RowRegs<CH> buf[kDepth];
   static_assert(kEarly <= kDepth, "early buffers are a subset of the ring");
   preload_range<0, kEarly>(rows_w > 0 ? n_elems : 0, src, buf);
-  if (xcd_counters(p) && (split != 0 || kg != M::F)) return bad_operand(p, s, c, 8);  // sub-counters cover one K slice
+  const bool tg = tagged(p);
+  const uint32_t tag = tag_of(s.generation, layer);
+  if ((xcd_counters(p) || tg) && (split != 0 || kg != M::F)) return bad_operand(p, s, c, 8);  // one K slice only
+  if (tg && nrows / 2 > kThreads) return bad_operand(p, s, c, 4);  // one residual pair per thread
+  // Tagged mode: the rows' residual values as the O-proj announced them, fetched ahead of time.
+  uint32_t res_old = 0;
+  if (tg && static_cast<int>(threadIdx.x) < nrows / 2 && !residual_in(p, p.ws + kWsHiddenMid, tag, rs, threadIdx.x, res_old)) {
+    s.ctl[0] = 1;  // seen by everybody after the barrier inside the wait below
+    report_error(p, QMK_DEV_WAIT_TIMEOUT, c.inst_idx, c.opcode, threadIdx.x);
+  }
   if (!wg_wait_all(p, s, c, layer, ROW_UPGATE, split, p.upgate_blocks_per_bucket)) return false;
 
   // The K slice of silu_out into LDS; the remaining row buffers are requested behind it.
@@ -788,6 +905,15 @@ __device__ bool op_down_residual(const Params& p, Smem<M>& s, const Ctx& c) {
   __syncthreads();
   QMK_STAMP(2);
 
+  if (tg) {
+    if (static_cast<int>(threadIdx.x) < nrows / 2) {
+      const int pair = threadIdx.x;
+      const uint32_t w = residual_word(res_old, s.res[2 * pair], s.res[2 * pair + 1]);
+      st_tagged(p.ws + kWsHiddenOut + (rs + 2 * pair) / 2, w, tag);
+      st_shared32(p.hidden + rs + 2 * pair, w);
+    }
+    return true;
+  }
   if (kg == M::F) {  // one slice: every row has a single writer
     for (int pair = threadIdx.x; pair < nrows / 2; pair += kThreads)
       residual_pair(p.hidden + rs + 2 * pair, s.res[2 * pair], s.res[2 * pair + 1]);
@@ -818,8 +944,9 @@ __device__ bool op_rms_lmhead(const Params& p, Smem<M>& s, const Ctx& c) {
 
   RowRegs<CH> buf[kDepth];
   preload<CH>(nrows, src, buf);
-  if (!wg_wait_all(p, s, c, p.num_layers - 1, ROW_DOWN, 0, p.down_arrivals)) return false;
-  rms_to_lds(p, s, p.hidden, p.lm_norm);
+  const bool tg = tagged(p);
+  if (!tg && !wg_wait_all(p, s, c, p.num_layers - 1, ROW_DOWN, 0, p.down_arrivals)) return false;
+  if (!rms_to_lds(p, s, c, tg ? p.ws + kWsHiddenOut : nullptr, tag_of(s.generation, p.num_layers - 1), p.lm_norm)) return false;
   v4u x[CH];
   load_x_from_lds(x, s.x, lane);
   // Terminal op: nothing inside the launch reads the logits, so ordinary stores do.

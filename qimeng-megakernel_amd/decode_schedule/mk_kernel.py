@@ -30,6 +30,7 @@ _LIBRARY_NAME = "libqmk_hip.so"
 
 QMK_FLAG_KEEP_BARRIERS = 1
 QMK_FLAG_XCD_COUNTERS = 2
+QMK_FLAG_TAGGED = 4
 QMK_XCD_COUNTER_ROWS = 54
 QMK_MODEL_LLAMA_3_2_1B = 0
 QMK_QUERY_ABI_VERSION, QMK_QUERY_CU_COUNT, QMK_QUERY_THREADS, QMK_QUERY_LDS_BYTES = 0, 1, 2, 3
@@ -54,11 +55,11 @@ class QmkArgs(ctypes.Structure):
         ("barrier_slots", _I), ("max_seq_len", _I), ("max_splits", _I), ("vocab_size", _I), ("rope_rows", _I),
         ("pos_id", _I), ("attn_scale", ctypes.c_float), ("rms_norm_eps", ctypes.c_float),
         ("qkv_blocks_per_head", _I), ("oproj_blocks", _I), ("upgate_blocks_per_bucket", _I), ("down_arrivals", _I),
-        ("timeline", _P), ("stream", _P),
+        ("timeline", _P), ("stream", _P), ("workspace", _P), ("workspace_bytes", ctypes.c_uint64),
     ]
 
 
-_EXPORTS = ("qmk_decode_step", "qmk_query", "qmk_status_fetch", "qmk_error_string")
+_EXPORTS = ("qmk_decode_step", "qmk_query", "qmk_status_fetch", "qmk_error_string", "qmk_workspace_bytes")
 
 # (name, dtype, ndim) of the 22 tensors, in the positional order of mk(...).
 _TENSOR_ARGS: tuple[tuple[str, torch.dtype, int], ...] = (
@@ -112,6 +113,8 @@ def load_library(mk_dir: Path | None = None) -> ctypes.CDLL:
     lib.qmk_status_fetch.restype = ctypes.c_int
     lib.qmk_error_string.argtypes = [ctypes.c_int]
     lib.qmk_error_string.restype = ctypes.c_char_p
+    lib.qmk_workspace_bytes.argtypes = [ctypes.c_int]
+    lib.qmk_workspace_bytes.restype = ctypes.c_uint64
     return lib
 
 
@@ -127,17 +130,25 @@ class MegaKernel:
     ``geometry`` is the tile geometry the instruction tensor was scheduled with
     (it fixes the final counter values the kernel waits for); ``reset_barriers``
     selects whether the kernel clears the counters when it retires (default) or
-    leaves their final values in place like the reference kernel.
+    leaves their final values in place like the reference kernel.  ``tagged``
+    lets the small activation vectors travel between workgroups as
+    self-announcing tagged units (``QMK_FLAG_TAGGED``) whenever the schedule
+    allows it: the kernel clears its counters itself, the down projection is
+    not split along K and there are at most 63 layers.  The workspace that mode
+    needs belongs to this object.
     """
 
     def __init__(self, lib: ctypes.CDLL, geometry: TileGeometry | None = None, *, reset_barriers: bool = True,
-                 spin_limit: int = 0, xcd_counters: bool = True):
+                 spin_limit: int = 0, xcd_counters: bool = True, tagged: bool = True):
         self._lib = lib
         self.geometry = geometry
         self.reset_barriers = reset_barriers
         self.spin_limit = int(spin_limit)
         self.xcd_counters = xcd_counters   # use per-XCD sub-counters when `barriers` has room for them
         self._xcd_counters = False
+        self.tagged = tagged
+        self._tagged = False
+        self._workspace: torch.Tensor | None = None
         self.timeline: torch.Tensor | None = None
         self._args = QmkArgs()
         self._args.struct_size = ctypes.sizeof(QmkArgs)
@@ -157,6 +168,8 @@ class MegaKernel:
         handle = (stream or torch.cuda.current_stream()).cuda_stream
         code = int(self._lib.qmk_status_fetch(_P(handle), ctypes.byref(detail)))
         if code != 0:
+            if self._workspace is not None:
+                self._workspace.zero_()  # units of the aborted step must not pass for the next one's
             raise RuntimeError(
                 f"megakernel device error {code} ({self.error_string(code)}): workgroup={detail[0]} "
                 f"instruction={detail[1]} opcode={detail[2]} operand={detail[3]}; "
@@ -167,7 +180,8 @@ class MegaKernel:
         other = MegaKernel(self._lib, kw.pop("geometry", self.geometry),
                            reset_barriers=kw.pop("reset_barriers", self.reset_barriers),
                            spin_limit=kw.pop("spin_limit", self.spin_limit),
-                           xcd_counters=kw.pop("xcd_counters", self.xcd_counters))
+                           xcd_counters=kw.pop("xcd_counters", self.xcd_counters),
+                           tagged=kw.pop("tagged", self.tagged))
         if kw:
             raise TypeError(f"unknown options {sorted(kw)}")
         return other
@@ -238,6 +252,18 @@ class MegaKernel:
             and barriers.data_ptr() % 128 == 0
             and geometry.num_split_k(shape) == 1
         )
+        self._tagged = self.tagged and self.reset_barriers and geometry.num_split_k(shape) == 1 and L <= 63
+        if self._tagged:
+            nbytes = int(self._lib.qmk_workspace_bytes(QMK_MODEL_LLAMA_3_2_1B))
+            if self._workspace is None or self._workspace.device != device:
+                self._workspace = torch.zeros(nbytes, dtype=torch.uint8, device=device)
+            else:
+                self._workspace.zero_()
+            if self._workspace.data_ptr() % 128 != 0:
+                raise RuntimeError("torch returned a workspace that is not 128-byte aligned")
+            a.workspace, a.workspace_bytes = self._workspace.data_ptr(), nbytes
+        else:
+            a.workspace, a.workspace_bytes = None, 0
 
     def __call__(self, *args: Any) -> None:
         if len(args) != 25:
@@ -246,7 +272,7 @@ class MegaKernel:
         if isinstance(tensors[0], torch.Tensor) and tensors[0].numel() == 0:
             return  # empty queues: nothing to launch
         key = tuple((t.data_ptr(), tuple(t.shape)) if isinstance(t, torch.Tensor) else None for t in tensors) + (
-            self.geometry, LlamaConfig.shape())
+            self.geometry, LlamaConfig.shape(), self.tagged, self.reset_barriers, self.xcd_counters)
         if key != self._bound_key:
             self._bind(tensors)
             self._bound_key = key
@@ -254,7 +280,8 @@ class MegaKernel:
         a.pos_id = int(pos_id)
         a.attn_scale = float(attn_scale)
         a.rms_norm_eps = float(rms_norm_eps)
-        a.flags = (0 if self.reset_barriers else QMK_FLAG_KEEP_BARRIERS) | (QMK_FLAG_XCD_COUNTERS if self._xcd_counters else 0)
+        a.flags = ((0 if self.reset_barriers else QMK_FLAG_KEEP_BARRIERS) | (QMK_FLAG_XCD_COUNTERS if self._xcd_counters else 0)
+                   | (QMK_FLAG_TAGGED if self._tagged else 0))
         a.spin_limit = self.spin_limit
         a.timeline = self.timeline.data_ptr() if self.timeline is not None else None
         a.stream = torch.cuda.current_stream(tensors[1].device).cuda_stream
@@ -267,7 +294,7 @@ _LIB_CACHE: dict[Path, ctypes.CDLL] = {}
 
 
 def get_mk(mk_dir: Path | None = None, *, geometry: TileGeometry | None = None, reset_barriers: bool = True,
-           spin_limit: int = 0, xcd_counters: bool = True) -> MegaKernel:
+           spin_limit: int = 0, xcd_counters: bool = True, tagged: bool = True) -> MegaKernel:
     """Return the ``mk`` callable bound to the prebuilt library in ``mk_dir``.
 
     ``geometry`` defaults to the MI355X schedule of this package; pass
@@ -280,7 +307,8 @@ def get_mk(mk_dir: Path | None = None, *, geometry: TileGeometry | None = None, 
         _LIB_CACHE[root] = lib
     if geometry is None:
         geometry = _scheduler.mi355x_scheduler(num_partials=1).geometry
-    return MegaKernel(lib, geometry, reset_barriers=reset_barriers, spin_limit=spin_limit, xcd_counters=xcd_counters)
+    return MegaKernel(lib, geometry, reset_barriers=reset_barriers, spin_limit=spin_limit, xcd_counters=xcd_counters,
+                      tagged=tagged)
 
 
 def call_mk(globs: Globals, mk: Any) -> None:

@@ -26,8 +26,8 @@ def lib():
 
 def test_every_declared_symbol_is_exported(lib):
     text = HEADER.read_text()
-    declared = set(re.findall(r"^(?:int|const char\*)\s+(qmk_\w+)\s*\(", text, flags=re.M))
-    assert declared == {"qmk_decode_step", "qmk_query", "qmk_status_fetch", "qmk_error_string"}
+    declared = set(re.findall(r"^(?:int|uint64_t|const char\*)\s+(qmk_\w+)\s*\(", text, flags=re.M))
+    assert declared == {"qmk_decode_step", "qmk_query", "qmk_status_fetch", "qmk_error_string", "qmk_workspace_bytes"}
     for name in declared:
         assert hasattr(lib, name), name
 
@@ -59,6 +59,7 @@ def test_constants_match_header():
         return int(re.search(rf"#define {name} (\d+)", text).group(1))
     assert define("QMK_FLAG_KEEP_BARRIERS") == mk_kernel.QMK_FLAG_KEEP_BARRIERS
     assert define("QMK_FLAG_XCD_COUNTERS") == mk_kernel.QMK_FLAG_XCD_COUNTERS
+    assert define("QMK_FLAG_TAGGED") == mk_kernel.QMK_FLAG_TAGGED
     assert define("QMK_XCD_COUNTER_ROWS") == mk_kernel.QMK_XCD_COUNTER_ROWS
     assert define("QMK_INSTRUCTION_WORDS") == 32
 
@@ -73,7 +74,8 @@ def test_host_side_argument_errors(lib):
     assert lib.qmk_decode_step(ctypes.byref(a)) == 8                       # QMK_ERR_MODEL
     a.model = 0
     assert lib.qmk_decode_step(ctypes.byref(a)) == 1                       # all tensor pointers are NULL
-    assert lib.qmk_query(0) == 1 and lib.qmk_query(2) == 512 and lib.qmk_query(5) == 32 and lib.qmk_query(6) == 25
+    assert lib.qmk_workspace_bytes(0) == 8 * 4096 and lib.qmk_workspace_bytes(7) == 0
+    assert lib.qmk_query(0) == 2 and lib.qmk_query(2) == 512 and lib.qmk_query(5) == 32 and lib.qmk_query(6) == 25
     assert 0 < lib.qmk_query(3) <= 160 * 1024
     assert lib.qmk_error_string(34).decode().startswith("device: counter wait")
     assert lib.qmk_error_string(12345).decode() == "unknown code"
