@@ -32,6 +32,10 @@ ROOT = Path(__file__).resolve().parent
 sys.path.insert(0, str(ROOT))
 
 HBM_PEAK_GBPS = 8000.0
+# HBM bytes one launch moves, from the two rocprofv3 --pmc runs (FETCH_SIZE, WRITE_SIZE; each scaled by
+# what the same counter reads for a 1 GiB copy) summarised in profiles/decode_megakernel_llama1b_hbm_counters.txt:
+# 1.0050 x the algorithmic bytes of the profiled launches.  Not measured in this process.
+MEASURED_TRAFFIC_OVER_ALGORITHMIC = 1.0050
 
 
 def cpu_baseline(shape, weights, prompt, n_steps: int, cores: int) -> dict:
@@ -161,7 +165,7 @@ def main() -> None:
             "peak": HBM_PEAK_GBPS,
             "unit": "GB/s",
             "frac": achieved / HBM_PEAK_GBPS,
-            "traffic": None,
+            "traffic": MEASURED_TRAFFIC_OVER_ALGORITHMIC * t["algorithmic_bytes"] / max(args.steps, 1),
             "bytes_per_launch_avg": t["algorithmic_bytes"] / max(args.steps, 1),
             "kernel": "decode_megakernel<Llama1B>",
         },
