@@ -79,6 +79,10 @@ def main() -> None:
     ap.add_argument("--prompt-len", type=int, default=8)
     ap.add_argument("--cpu-steps", type=int, default=10)
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--host-sampling", action="store_true",
+                    help="argmax and embedding lookup on the host between launches, as the reference's loop does "
+                         "(default: inside the kernel)")
+    ap.add_argument("--no-graph-run", action="store_true", help="skip the extra untimed-per-step HIP-graph run")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also run one 1 GiB device-to-device copy (a kernel of known traffic, for scaling rocprofv3 counters)")
     args = ap.parse_args()
@@ -120,10 +124,18 @@ def main() -> None:
         decode.decode(globs, prompt, min(args.warmup + 1, new_tokens), mk=mk, decode_time=False)
     globs.k_cache.zero_(); globs.v_cache.zero_()
     torch.cuda.synchronize(device)
-    out = decode.decode(globs, prompt, new_tokens, mk=mk, decode_time=True)
+    out = decode.decode(globs, prompt, new_tokens, mk=mk, decode_time=True, device_sampling=not args.host_sampling)
     torch.cuda.synchronize(device)
     t = out["timing"]
     tokens = out["new_tokens"][0].tolist()
+    graph_tok_s = None
+    if not args.no_graph_run and not args.host_sampling:
+        # The same request once more as ONE HIP graph of all decode launches (no per-step events).
+        globs.k_cache.zero_(); globs.v_cache.zero_()
+        g_out = decode.decode(globs, prompt, new_tokens, mk=mk, decode_time=True, use_graph=True)
+        if g_out["new_tokens"][0].tolist() != tokens:
+            raise SystemExit("bench.py: the graph replay produced different tokens than the launch loop")
+        graph_tok_s = g_out["timing"]["effective_tok_s_gpu"]
 
     golden = ROOT / "tests" / "golden" / "llama1b_seed0.json"
     match = None
@@ -158,6 +170,8 @@ def main() -> None:
         "tok_s": t["effective_tok_s_wall"],
         "tok_s_gpu": t["effective_tok_s_gpu"],
         "kernel_tok_s": t["kernel_tok_s"],
+        "tok_s_gpu_graph": graph_tok_s,
+        "sampling": "host" if args.host_sampling else "device",
         "golden_token_prefix_match": match,
         "roofline": {
             "bound": "hbm",

@@ -30,7 +30,7 @@
 extern "C" {
 #endif
 
-#define QMK_ABI_VERSION 2
+#define QMK_ABI_VERSION 3
 #define QMK_INSTRUCTION_WORDS 32
 
 /* Return / status codes. 0 is success; everything else is an error. */
@@ -157,11 +157,20 @@ typedef struct QmkArgs {
                                       (100 MHz ticks), opcode | layer << 8, and four
                                       op-specific intermediate stamps; NULL = off */
   void* stream;                    /* hipStream_t; NULL = the null stream         */
-  void* workspace;                 /* QMK_FLAG_TAGGED: device buffer of workspace_bytes, 128-byte
-                                      aligned, zeroed once when allocated and then left to the
-                                      library (it carries a launch count from step to step); NULL
-                                      otherwise                                                  */
+  void* workspace;                 /* QMK_FLAG_TAGGED and/or token_out: device buffer of
+                                      workspace_bytes, 128-byte aligned, zeroed once when allocated
+                                      and then left to the library (it carries a launch count from
+                                      step to step); NULL otherwise                              */
   uint64_t workspace_bytes;        /* >= qmk_workspace_bytes(model)               */
+
+  /* Greedy step chaining on the device (both NULL = off, the reference's behaviour, where the host
+   * runs argmax and the embedding lookup between launches: models/LLM/decode.py:1386-1397).  With
+   * both set, the last workgroup to retire writes the index of the first maximal bf16 logit to
+   * *token_out and copies that token's embedding row into hidden_states, so the next step can be
+   * launched without any host work in between.  Needs `workspace`, at most 1024 queues, and is not
+   * combinable with QMK_FLAG_KEEP_BARRIERS. */
+  const void* embed_tokens;        /* bf16 [vocab_size, H]                        */
+  int64_t* token_out;              /* one element                                 */
 } QmkArgs;
 
 /* Launch one decode step asynchronously on args->stream.  Returns QMK_OK or a

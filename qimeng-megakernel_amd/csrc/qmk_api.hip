@@ -27,7 +27,11 @@ template <class M>
 __global__ __launch_bounds__(kThreads, 1) void decode_megakernel(const Params p) {
   __shared__ Smem<M> s;
   if (threadIdx.x < 8) s.ctl[threadIdx.x] = 0;
-  if (threadIdx.x == 0) s.generation = tagged(p) ? ld_shared32(p.ws + kWsGeneration) : 0u;
+  if (threadIdx.x == 0) {
+    s.generation = tagged(p) ? ld_shared32(p.ws + kWsGeneration) : 0u;
+    s.best_val = -INFINITY;
+    s.best_idx = 0x7fffffff;
+  }
   __syncthreads();
 
   const int32_t* queue = p.instructions + static_cast<size_t>(blockIdx.x) * p.num_insts * kInstWords;
@@ -72,6 +76,15 @@ __global__ __launch_bounds__(kThreads, 1) void decode_megakernel(const Params p)
   // Retire.  The workgroup that arrives last owns the counters alone (every
   // other queue is finished, so nobody polls any more) and clears them for the
   // next step.  The arrival counter is the last word of layer 0's last row.
+  // Greedy chaining: the workgroup's candidate {order-preserving logit bits, row} is in memory
+  // before the arrival below, so the last workgroup finds all of them.
+  const bool sampling = p.token_out != nullptr;
+  if (sampling && threadIdx.x == 0) {
+    const uint32_t bits = __float_as_uint(s.best_val);
+    const uint32_t key = (bits & 0x80000000u) ? ~bits : (bits | 0x80000000u);  // larger float <=> larger key
+    __hip_atomic_store(p.ws + kWsCandidates + blockIdx.x, (static_cast<uint64_t>(key) << 32) | static_cast<uint32_t>(s.best_idx),
+                       __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  }
   release_stores();  // our publishing atomics have landed before we say we are done
   __syncthreads();
   int32_t* done = counter_ptr(p, 0, p.num_layer_barriers - 1, p.barrier_slots - 1);
@@ -86,6 +99,33 @@ __global__ __launch_bounds__(kThreads, 1) void decode_megakernel(const Params p)
       __hip_atomic_store(p.barriers + i, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     // The next launch tags its activations with the next count (26 bits: the tag keeps 6 for the layer).
     if (tagged(p) && threadIdx.x == 0) st_shared32(p.ws + kWsGeneration, (s.generation + 1u) & 0x03ffffffu);
+    if (sampling) {
+      // Largest logit, smallest row among equals (torch.argmax's choice): the key orders by logit,
+      // the complemented row breaks ties towards the first row.
+      uint64_t mine = 0;
+      for (int q = threadIdx.x; q < static_cast<int>(gridDim.x); q += kThreads) {
+        const uint64_t cand = ld_shared64(p.ws + kWsCandidates + q);
+        const uint64_t ordered = (cand & 0xffffffff00000000ull) | (0xffffffffu - static_cast<uint32_t>(cand));
+        mine = ordered > mine ? ordered : mine;
+      }
+      for (int off = 1; off < kWaveSize; off <<= 1) {
+        const uint32_t lo = __shfl_xor(static_cast<uint32_t>(mine), off), hi = __shfl_xor(static_cast<uint32_t>(mine >> 32), off);
+        const uint64_t other = (static_cast<uint64_t>(hi) << 32) | lo;
+        mine = other > mine ? other : mine;
+      }
+      uint64_t* slots = reinterpret_cast<uint64_t*>(s.res);
+      if ((threadIdx.x & (kWaveSize - 1)) == 0) slots[threadIdx.x >> 6] = mine;
+      __syncthreads();
+      uint64_t best = slots[0];
+      for (int w = 1; w < kWaves; ++w) best = slots[w] > best ? slots[w] : best;
+      const uint32_t token = 0xffffffffu - static_cast<uint32_t>(best);
+      if (token < static_cast<uint32_t>(p.vocab_size)) {  // no LM-head instruction ran: leave both untouched
+        if (threadIdx.x == 0) *p.token_out = static_cast<long long>(token);
+        static_assert(M::H == kThreads * 4, "one thread copies four embedding elements");
+        const uint2 row = *reinterpret_cast<const uint2*>(p.embed + static_cast<size_t>(token) * M::H + threadIdx.x * 4);
+        *reinterpret_cast<uint2*>(p.hidden + threadIdx.x * 4) = row;
+      }
+    }
   }
 }
 
@@ -150,11 +190,15 @@ extern "C" int qmk_decode_step(const QmkArgs* a) {
     if (layer_ints < needed || !aligned) return QMK_ERR_SHAPE;
   }
 
-  if (a->flags & QMK_FLAG_TAGGED) {
+  const bool sampling = a->token_out != nullptr || a->embed_tokens != nullptr;
+  if (sampling && (a->token_out == nullptr || a->embed_tokens == nullptr)) return QMK_ERR_NULL_ARG;
+  if ((a->flags & QMK_FLAG_TAGGED) || sampling) {
     if (a->workspace == nullptr) return QMK_ERR_NULL_ARG;
-    if ((a->flags & QMK_FLAG_KEEP_BARRIERS) || a->num_layers > 63 || reinterpret_cast<uintptr_t>(a->workspace) % 128 != 0 ||
+    if ((a->flags & QMK_FLAG_KEEP_BARRIERS) || reinterpret_cast<uintptr_t>(a->workspace) % 128 != 0 ||
         a->workspace_bytes < qmk_workspace_bytes(static_cast<int>(a->model)))
       return QMK_ERR_SHAPE;
+    if ((a->flags & QMK_FLAG_TAGGED) && a->num_layers > 63) return QMK_ERR_SHAPE;
+    if (sampling && a->num_queues > kMaxSamplingQueues) return QMK_ERR_SHAPE;
   }
 
   DeviceInfo* dev = nullptr;
@@ -185,7 +229,9 @@ extern "C" int qmk_decode_step(const QmkArgs* a) {
   p.lm_norm = static_cast<const u16*>(a->lm_head_norm_weights);
   p.lm_w = static_cast<const u16*>(a->lm_head_weights);
   p.barriers = a->barriers;
-  p.ws = (a->flags & QMK_FLAG_TAGGED) ? static_cast<uint64_t*>(a->workspace) : nullptr;
+  p.ws = static_cast<uint64_t*>(a->workspace);
+  p.embed = static_cast<const u16*>(a->embed_tokens);
+  p.token_out = reinterpret_cast<long long*>(a->token_out);
   p.timeline = a->timeline;
   p.status = dev->status;
   p.num_insts = a->num_insts;

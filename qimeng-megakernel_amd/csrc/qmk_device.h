@@ -45,7 +45,9 @@ struct Params {
   const u16* lm_norm;
   const u16* lm_w;
   int32_t* barriers;
-  uint64_t* ws;         // tagged-activation workspace (QMK_FLAG_TAGGED), else null
+  uint64_t* ws;         // workspace (tagged units, greedy candidates), else null
+  const u16* embed;     // embedding table and destination of the greedy token, or null
+  long long* token_out;
   uint64_t* timeline;
   int32_t* status;      // device status words: {code, workgroup, inst, opcode, operand}
   int32_t num_insts;
@@ -222,7 +224,9 @@ constexpr int kWsK = kWsQ + 1024;           // appended K row: NKV*D/2 units
 constexpr int kWsV = kWsK + 256;            // appended V row
 constexpr int kWsHiddenMid = kWsV + 256;    // residual stream after the O-proj: H/2 units
 constexpr int kWsHiddenOut = kWsHiddenMid + 1024;  // residual stream after the down projection
-constexpr int kWsUnits = kWsHiddenOut + 1024;
+constexpr int kWsCandidates = kWsHiddenOut + 1024;  // one greedy candidate per workgroup: {logit bits, row}
+constexpr int kMaxSamplingQueues = 1024;
+constexpr int kWsUnits = kWsCandidates + kMaxSamplingQueues;
 
 __device__ __forceinline__ bool tagged(const Params& p) { return (p.flags & QMK_FLAG_TAGGED) != 0; }
 __device__ __forceinline__ uint32_t tag_of(uint32_t generation, int layer) { return (generation << 6) + static_cast<uint32_t>(layer) + 1u; }

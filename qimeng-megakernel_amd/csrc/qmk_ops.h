@@ -31,6 +31,9 @@ struct Smem {
   int32_t inst[kInstWords];
   int32_t ctl[8];                       // [0] abort, [1] last workgroup to retire
   uint32_t generation;                  // launch count of the tagged-activation workspace
+  float best_val;                       // greedy candidate of this workgroup: largest bf16 logit so far ...
+  int32_t best_idx;                     // ... and the first row that has it
+  int32_t wave_idx[kWaves];             // per-wave candidates on their way to best_val/best_idx
   float red[kWaves];
   alignas(16) u16 x[M::F];              // activation vector handed to the GEMV lanes
   float res[kResSlots];                 // per-row GEMV results awaiting the epilogue pass
@@ -949,11 +952,38 @@ __device__ bool op_rms_lmhead(const Params& p, Smem<M>& s, const Ctx& c) {
   if (!rms_to_lds(p, s, c, tg ? p.ws + kWsHiddenOut : nullptr, tag_of(s.generation, p.num_layers - 1), p.lm_norm)) return false;
   v4u x[CH];
   load_x_from_lds(x, s.x, lane);
-  // Terminal op: nothing inside the launch reads the logits, so ordinary stores do.
+  // Terminal op: nothing inside the launch reads the logits, so ordinary stores do.  A wave sees
+  // its rows in increasing order, so "strictly greater" keeps the first row of a tie.
+  float best = -INFINITY;
+  int best_row = 0x7fffffff;
   stream<CH>(nrows, src, buf, [&](int r, const RowRegs<CH>& w) {
     const float sum = wave_sum(dot_row(w, x));
-    if (lane == 0) p.logits[rs + r] = f2bf(sum);
+    const u16 logit = f2bf(sum);
+    if (lane == 0) p.logits[rs + r] = logit;
+    const float v = bf2f(logit);
+    if (v > best) {
+      best = v;
+      best_row = rs + r;
+    }
   });
+  if (p.token_out != nullptr) {  // greedy candidate of this workgroup (several LM-head instructions accumulate)
+    if (lane == 0) {
+      s.red[threadIdx.x >> 6] = best;
+      s.wave_idx[threadIdx.x >> 6] = best_row;
+    }
+    __syncthreads();
+    if (threadIdx.x == 0) {
+      float v = s.best_val;
+      int i = s.best_idx;
+      for (int w = 0; w < kWaves; ++w)
+        if (s.red[w] > v || (s.red[w] == v && s.wave_idx[w] < i)) {
+          v = s.red[w];
+          i = s.wave_idx[w];
+        }
+      s.best_val = v;
+      s.best_idx = i;
+    }
+  }
   return true;
 }
 

@@ -7,6 +7,9 @@ reference (`qimeng_megakernel/models/LLM/decode.py:536-796, 1340-1435`):
 * per step: embedding row -> ``hidden_states``, ``position_id = pos``, one kernel
   launch, ``argmax`` of the bf16 logits written straight into the token buffer;
   nothing synchronises inside the loop;
+* with ``device_sampling`` the kernel itself picks the greedy token and loads its
+  embedding row (``MegaKernel.greedy_into``): the loop is then nothing but launches,
+  optionally captured once into a HIP graph (``use_graph``);
 * timing: one pre-allocated event pair per step around the kernel call only
   (``mk_kernel_gpu_s``), one pair around the loop (``decode_gpu_s``) and
   ``perf_counter`` (``decode_wall_s``); the first new token comes from prefill
@@ -32,8 +35,11 @@ def _embed_into_hidden(globs: Any, token_ids: torch.Tensor) -> None:
     globs.hidden_states.copy_(emb.reshape(-1))
 
 
-def prefill_by_decode(globs: Any, mk: Any, prompt_ids: torch.Tensor) -> torch.Tensor:
-    """Fill the KV cache for ``prompt_ids`` one position at a time; returns the first new token (0-dim)."""
+def prefill_by_decode(globs: Any, mk: Any, prompt_ids: torch.Tensor, *, sample_into: tuple[torch.Tensor, int] | None = None) -> torch.Tensor:
+    """Fill the KV cache for ``prompt_ids`` one position at a time; returns the first new token (0-dim).
+
+    With ``sample_into=(tokens, index)`` the last launch picks that token on the device, stores it
+    in ``tokens.view(-1)[index]`` and leaves its embedding in ``hidden_states``."""
     if globs.instructions is None:
         _scheduler.build(globs)
     prompt_ids = prompt_ids.to(globs.hidden_states.device)
@@ -44,8 +50,43 @@ def prefill_by_decode(globs: Any, mk: Any, prompt_ids: torch.Tensor) -> torch.Te
     for pos in range(prompt_ids.numel()):
         _embed_into_hidden(globs, prompt_ids[pos : pos + 1])
         globs.position_id = pos
+        if sample_into is not None and pos == prompt_ids.numel() - 1:
+            mk.greedy_into(_embed_table(globs), sample_into[0], sample_into[1])
         _mk_kernel.call_mk(globs, mk)
+    if sample_into is not None:
+        return sample_into[0].view(-1)[sample_into[1]]
     return globs.logits.argmax()
+
+
+def _embed_table(globs: Any) -> torch.Tensor:
+    table = globs.embed_tokens
+    return table.data if isinstance(table, torch.nn.Parameter) else table
+
+
+def generate_greedy_on_device(
+    globs: Any,
+    output_tokens: torch.Tensor,
+    prompt_len: int,
+    ntok: int,
+    *,
+    mk: Any,
+    mk_step_events: list[tuple[torch.cuda.Event, torch.cuda.Event]] | None = None,
+) -> int:
+    """``ntok`` greedy steps with no host work between launches.
+
+    ``hidden_states`` must already hold the embedding of ``output_tokens[0, prompt_len]`` (the
+    previous launch put it there); step ``i`` writes ``output_tokens[0, prompt_len + i + 1]``."""
+    table = _embed_table(globs)
+    for i in range(ntok):
+        pos = prompt_len + i
+        globs.position_id = pos
+        mk.greedy_into(table, output_tokens, pos + 1)
+        if mk_step_events is not None:
+            mk_step_events[i][0].record()
+        _mk_kernel.call_mk(globs, mk)
+        if mk_step_events is not None:
+            mk_step_events[i][1].record()
+    return ntok
 
 
 def generate_greedy_fast(
@@ -82,8 +123,14 @@ def decode(
     *,
     mk: Any = None,
     decode_time: bool = True,
+    device_sampling: bool = False,
+    use_graph: bool = False,
 ) -> dict[str, Any]:
-    """Prefill + forced greedy decode to exactly ``max_new_tokens`` tokens (no EOS stop)."""
+    """Prefill + forced greedy decode to exactly ``max_new_tokens`` tokens (no EOS stop).
+
+    ``device_sampling``: argmax and embedding lookup run inside the kernel.  ``use_graph`` (implies
+    ``device_sampling``): the decode launches are captured into one HIP graph and replayed once;
+    per-step kernel times are then not available (``kernel_tok_s`` is reported as 0)."""
     device = globs.hidden_states.device
     prompt_len = int(prompt_ids.numel())
     if prompt_len + max_new_tokens > globs.k_cache.shape[2]:
@@ -93,21 +140,38 @@ def decode(
     _scheduler.build(globs)
     instruction_setup_wall_s = time.perf_counter() - t0
 
-    first = prefill_by_decode(globs, mk, prompt_ids)
+    device_sampling = device_sampling or use_graph
     output_tokens = torch.zeros(1, prompt_len + max(max_new_tokens, 1), dtype=torch.long, device=device)
     output_tokens[0, :prompt_len] = prompt_ids.to(device)
-    output_tokens[0, prompt_len] = first
+    if device_sampling:
+        prefill_by_decode(globs, mk, prompt_ids, sample_into=(output_tokens, prompt_len))
+    else:
+        output_tokens[0, prompt_len] = prefill_by_decode(globs, mk, prompt_ids)
     ntok = max(max_new_tokens - 1, 0)
+    graph = None
+    if use_graph and ntok > 0:
+        # Capture on a side stream (as torch requires); every launch carries its own position and
+        # token slot, so one replay is the whole request.  The graph starts from the state the
+        # prefill left: nothing it reads was produced by the capture itself.
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            generate_greedy_on_device(globs, output_tokens, prompt_len, ntok, mk=mk)
 
     events = None
     if decode_time:
-        events = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(ntok)]
+        events = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True))
+                  for _ in range(0 if graph is not None else ntok)]
         loop_start, loop_end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
         torch.cuda.synchronize(device)
         wall0 = time.perf_counter()
         loop_start.record()
-    generate_greedy_fast(globs, output_tokens, prompt_len, ntok, call_mk=lambda g: _mk_kernel.call_mk(g, mk),
-                         mk_step_events=events)
+    if graph is not None:
+        graph.replay()
+    elif device_sampling:
+        generate_greedy_on_device(globs, output_tokens, prompt_len, ntok, mk=mk, mk_step_events=events)
+    else:
+        generate_greedy_fast(globs, output_tokens, prompt_len, ntok, call_mk=lambda g: _mk_kernel.call_mk(g, mk),
+                             mk_step_events=events)
     result: dict[str, Any] = {"generated_ids": output_tokens, "new_tokens": output_tokens[:, prompt_len:]}
     if decode_time:
         loop_end.record()

@@ -56,6 +56,7 @@ class QmkArgs(ctypes.Structure):
         ("pos_id", _I), ("attn_scale", ctypes.c_float), ("rms_norm_eps", ctypes.c_float),
         ("qkv_blocks_per_head", _I), ("oproj_blocks", _I), ("upgate_blocks_per_bucket", _I), ("down_arrivals", _I),
         ("timeline", _P), ("stream", _P), ("workspace", _P), ("workspace_bytes", ctypes.c_uint64),
+        ("embed_tokens", _P), ("token_out", _P),
     ]
 
 
@@ -136,6 +137,12 @@ class MegaKernel:
     allows it: the kernel clears its counters itself, the down projection is
     not split along K and there are at most 63 layers.  The workspace that mode
     needs belongs to this object.
+
+    ``greedy_into(embed_tokens, tokens, index)`` arms device-side step chaining
+    for the next call: the kernel itself writes the greedy token to
+    ``tokens.view(-1)[index]`` and copies its embedding row into
+    ``hidden_states`` (the reference does both on the host between launches,
+    `models/LLM/decode.py:1386-1397`).
     """
 
     def __init__(self, lib: ctypes.CDLL, geometry: TileGeometry | None = None, *, reset_barriers: bool = True,
@@ -149,6 +156,7 @@ class MegaKernel:
         self.tagged = tagged
         self._tagged = False
         self._workspace: torch.Tensor | None = None
+        self._greedy: tuple[torch.Tensor, torch.Tensor, int] | None = None
         self.timeline: torch.Tensor | None = None
         self._args = QmkArgs()
         self._args.struct_size = ctypes.sizeof(QmkArgs)
@@ -185,6 +193,20 @@ class MegaKernel:
         if kw:
             raise TypeError(f"unknown options {sorted(kw)}")
         return other
+
+    def greedy_into(self, embed_tokens: torch.Tensor, tokens: torch.Tensor, index: int) -> None:
+        """The next call also samples: ``tokens.view(-1)[index] = argmax(logits)``, ``hidden_states = embed_tokens[that]``."""
+        if not self.reset_barriers:
+            raise ValueError("device-side sampling needs the self-clearing counters (reset_barriers=True)")
+        if embed_tokens.dtype != torch.bfloat16 or embed_tokens.dim() != 2 or not embed_tokens.is_contiguous():
+            raise TypeError("embed_tokens must be a contiguous bf16 [vocab, hidden] tensor")
+        if tokens.dtype != torch.int64 or not tokens.is_contiguous():
+            raise TypeError("tokens must be a contiguous int64 tensor")
+        if embed_tokens.device.type != "cuda" or tokens.device != embed_tokens.device:
+            raise ValueError("embed_tokens and tokens must live on the same GPU")
+        if not 0 <= index < tokens.numel():
+            raise IndexError(f"token index {index} outside a buffer of {tokens.numel()}")
+        self._greedy = (embed_tokens, tokens, int(index))
 
     # -- the call -------------------------------------------------------------
     def _bind(self, tensors: Sequence[torch.Tensor]) -> None:
@@ -253,7 +275,7 @@ class MegaKernel:
             and geometry.num_split_k(shape) == 1
         )
         self._tagged = self.tagged and self.reset_barriers and geometry.num_split_k(shape) == 1 and L <= 63
-        if self._tagged:
+        if self._tagged or self.reset_barriers:   # the workspace also carries the greedy candidates
             nbytes = int(self._lib.qmk_workspace_bytes(QMK_MODEL_LLAMA_3_2_1B))
             if self._workspace is None or self._workspace.device != device:
                 self._workspace = torch.zeros(nbytes, dtype=torch.uint8, device=device)
@@ -284,6 +306,15 @@ class MegaKernel:
                    | (QMK_FLAG_TAGGED if self._tagged else 0))
         a.spin_limit = self.spin_limit
         a.timeline = self.timeline.data_ptr() if self.timeline is not None else None
+        if self._greedy is not None:
+            embed, tokens, index = self._greedy
+            self._greedy = None
+            if tuple(embed.shape) != (a.vocab_size, LlamaConfig.shape().hidden_size) or embed.device != tensors[1].device:
+                raise ValueError(f"embed_tokens has shape {tuple(embed.shape)} on {embed.device}; the kernel needs "
+                                 f"({a.vocab_size}, {LlamaConfig.shape().hidden_size}) on {tensors[1].device}")
+            a.embed_tokens, a.token_out = embed.data_ptr(), tokens.data_ptr() + 8 * index
+        else:
+            a.embed_tokens, a.token_out = None, None
         a.stream = torch.cuda.current_stream(tensors[1].device).cuda_stream
         rc = int(self._lib.qmk_decode_step(ctypes.byref(a)))
         if rc != 0:
