@@ -87,8 +87,8 @@ def main() -> None:
                     help="also run one 1 GiB device-to-device copy (a kernel of known traffic, for scaling rocprofv3 counters)")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
-        raise SystemExit("bench.py: this path runs on exactly one GPU (batch-1 decode does not shard; "
-                         "see DESIGN.md 'More than one GPU'); run with --gpus 1")
+        raise SystemExit("bench.py: this path runs on exactly one GPU (a batch-1 decode step is one chain of "
+                         "GEMVs on one vector and does not shard); run with --gpus 1")
 
     import torch
 
