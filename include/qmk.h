@@ -30,7 +30,7 @@
 extern "C" {
 #endif
 
-#define QMK_ABI_VERSION 3
+#define QMK_ABI_VERSION 4
 #define QMK_INSTRUCTION_WORDS 32
 
 /* Return / status codes. 0 is success; everything else is an error. */
@@ -52,7 +52,10 @@ enum {
 
 /* Model shapes compiled into the library. */
 enum {
-  QMK_MODEL_LLAMA_3_2_1B = 0   /* H 2048, F 8192, 32 q / 8 kv heads, d 64 */
+  QMK_MODEL_LLAMA_3_2_1B = 0,  /* H 2048, F 8192, 32 q / 8 kv heads, d 64 */
+  QMK_MODEL_QWEN3_1_7B = 1     /* H 2048, F 6144, 16 q / 8 kv heads, d 128, per-head QK RMSNorm
+                                  (the Qwen3 op set: …/qwen/qwen3__0_6b/A100/single_batch/
+                                  decode_kernel/mk.h, decode_schedule/mk_kernel.py:52-110)     */
 };
 
 /* qmk_query selectors. */
@@ -171,6 +174,11 @@ typedef struct QmkArgs {
    * combinable with QMK_FLAG_KEEP_BARRIERS. */
   const void* embed_tokens;        /* bf16 [vocab_size, H]                        */
   int64_t* token_out;              /* one element                                 */
+
+  /* Qwen3 op set only (NULL for the Llama shape): the three tensors its mk(...) takes in addition. */
+  void* qkv_raw;                   /* bf16 [(Hq+2Hkv)*D]  QKV before norm and RoPE */
+  const void* q_norm_weights;      /* bf16 [L, D]  per-head RMSNorm of q, pair-interleaved like the q rows */
+  const void* k_norm_weights;      /* bf16 [L, D]                                 */
 } QmkArgs;
 
 /* Launch one decode step asynchronously on args->stream.  Returns QMK_OK or a

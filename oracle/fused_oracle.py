@@ -52,6 +52,14 @@ def rms_norm(x: Tensor, weight: Tensor, eps: float) -> Tensor:
     return weight * xf.to(dtype)
 
 
+def per_head_rms_norm(x: Tensor, weight: Tensor, eps: float) -> Tensor:
+    """RMSNorm over the last dim with one shared weight vector, all in fp32, ONE rounding at the end
+    (qwen3__0_6b/…/fused/operations.py:52-63 — unlike ``rms_norm``, which rounds before the weight)."""
+    xf = x.to(torch.float32)
+    xf = xf * torch.rsqrt(xf.pow(2).mean(-1, keepdim=True) + eps)
+    return (weight.to(torch.float32) * xf).to(x.dtype)
+
+
 def rotate_pairs(x: Tensor) -> Tensor:
     """(x0, x1, x2, x3, ...) -> (-x1, x0, -x3, x2, ...)."""
     even, odd = x[..., 0::2], x[..., 1::2]
@@ -73,6 +81,12 @@ class FusedOracle:
         q = qkv[:, : nq * d].view(1, nq, d)
         k = qkv[:, nq * d : (nq + nkv) * d].view(1, nkv, d)
         v = qkv[:, (nq + nkv) * d :].view(1, nkv, d)
+        if getattr(s, "qk_norm", False):
+            # Qwen3 op set: the raw vector is kept, q and k get a per-head RMSNorm before RoPE
+            # (qwen3__0_6b/…/fused/operations.py:65-120).
+            g.qkv_raw.copy_(qkv.reshape(-1).to(g.qkv_raw.dtype))
+            q = per_head_rms_norm(q, g.q_norm_weights[layer], s.rms_norm_eps)
+            k = per_head_rms_norm(k, g.k_norm_weights[layer], s.rms_norm_eps)
         pos = int(g.position_id or 0)
         cos = g.rope_cos[pos].view(1, 1, -1)  # fp32: the products below are fp32
         sin = g.rope_sin[pos].view(1, 1, -1)

@@ -165,11 +165,10 @@ int device_info(DeviceInfo** out) {
 
 using namespace qmk;
 
-extern "C" int qmk_decode_step(const QmkArgs* a) {
-  if (a == nullptr) return QMK_ERR_NULL_ARG;
-  if (a->struct_size != sizeof(QmkArgs)) return QMK_ERR_ABI;
-  if (a->model != QMK_MODEL_LLAMA_3_2_1B) return QMK_ERR_MODEL;
-  using M = Llama1B;
+namespace {
+
+template <class M>
+int decode_step(const QmkArgs* a) {
   const void* required[] = {a->instructions, a->hidden_states, a->q_post_rope, a->k_cache, a->v_cache, a->attn_out,
                             a->attn_lse_intermediates, a->attn_out_intermediates, a->silu_out, a->logits,
                             a->attn_norm_weights, a->qkv_weights, a->rope_cos, a->rope_sin, a->o_proj_weights,
@@ -177,6 +176,7 @@ extern "C" int qmk_decode_step(const QmkArgs* a) {
                             a->lm_head_norm_weights, a->lm_head_weights, a->barriers};
   for (const void* ptr : required)
     if (ptr == nullptr) return QMK_ERR_NULL_ARG;
+  if (M::QK_NORM && (a->qkv_raw == nullptr || a->q_norm_weights == nullptr || a->k_norm_weights == nullptr)) return QMK_ERR_NULL_ARG;
   if (a->num_queues < 1 || a->num_insts < 0 || a->num_layers < 1 || a->num_layer_barriers < 8 ||
       a->barrier_slots < M::NQ + 2 * M::NKV || a->max_seq_len < 1 || a->max_splits < 1 || a->vocab_size < 1 ||
       a->rope_rows < 1)
@@ -219,6 +219,9 @@ extern "C" int qmk_decode_step(const QmkArgs* a) {
   p.logits = static_cast<u16*>(a->logits);
   p.attn_norm = static_cast<const u16*>(a->attn_norm_weights);
   p.qkv_w = static_cast<const u16*>(a->qkv_weights);
+  p.qkv_raw = static_cast<u16*>(a->qkv_raw);
+  p.q_norm = static_cast<const u16*>(a->q_norm_weights);
+  p.k_norm = static_cast<const u16*>(a->k_norm_weights);
   p.rope_cos = a->rope_cos;
   p.rope_sin = a->rope_sin;
   p.o_w = static_cast<const u16*>(a->o_proj_weights);
@@ -257,8 +260,20 @@ extern "C" int qmk_decode_step(const QmkArgs* a) {
   return hipGetLastError() == hipSuccess ? QMK_OK : QMK_ERR_LAUNCH;
 }
 
+}  // namespace
+
+extern "C" int qmk_decode_step(const QmkArgs* a) {
+  if (a == nullptr) return QMK_ERR_NULL_ARG;
+  if (a->struct_size != sizeof(QmkArgs)) return QMK_ERR_ABI;
+  switch (a->model) {
+    case QMK_MODEL_LLAMA_3_2_1B: return decode_step<Llama1B>(a);
+    case QMK_MODEL_QWEN3_1_7B: return decode_step<Qwen3_1p7B>(a);
+    default: return QMK_ERR_MODEL;
+  }
+}
+
 extern "C" uint64_t qmk_workspace_bytes(int model) {
-  return model == QMK_MODEL_LLAMA_3_2_1B ? static_cast<uint64_t>(kWsUnits) * sizeof(uint64_t) : 0;
+  return (model == QMK_MODEL_LLAMA_3_2_1B || model == QMK_MODEL_QWEN3_1_7B) ? static_cast<uint64_t>(kWsUnits) * sizeof(uint64_t) : 0;
 }
 
 extern "C" int qmk_query(int what) {

@@ -34,6 +34,9 @@ struct Params {
   u16* silu_out;
   u16* logits;
   const u16* attn_norm;
+  u16* qkv_raw;         // Qwen3 op set only: QKV before the per-head norm and RoPE
+  const u16* q_norm;    // Qwen3 op set only: per-head RMSNorm weights [L, D]
+  const u16* k_norm;
   const u16* qkv_w;
   const float* rope_cos;
   const float* rope_sin;
@@ -221,8 +224,8 @@ __device__ __forceinline__ v4u ld_shared128(const void* p) {
 constexpr int kWsGeneration = 0;            // launch count (first 128-byte line)
 constexpr int kWsQ = 512;                   // q after RoPE: NQ*D/2 units (two bf16 each)
 constexpr int kWsK = kWsQ + 1024;           // appended K row: NKV*D/2 units
-constexpr int kWsV = kWsK + 256;            // appended V row
-constexpr int kWsHiddenMid = kWsV + 256;    // residual stream after the O-proj: H/2 units
+constexpr int kWsV = kWsK + 512;            // appended V row (regions sized for 8 KV heads of 128)
+constexpr int kWsHiddenMid = kWsV + 512;    // residual stream after the O-proj: H/2 units
 constexpr int kWsHiddenOut = kWsHiddenMid + 1024;  // residual stream after the down projection
 constexpr int kWsCandidates = kWsHiddenOut + 1024;  // one greedy candidate per workgroup: {logit bits, row}
 constexpr int kMaxSamplingQueues = 1024;

@@ -22,6 +22,22 @@ struct Llama1B {
   static constexpr int GQA = NQ / NKV;
   static constexpr int QKV = (NQ + 2 * NKV) * D;
   static constexpr int KV_BLOCK = 16;  // split-KV partition granularity in tokens
+  static constexpr bool QK_NORM = false;
+};
+
+// Qwen3-1.7B shape with the Qwen3 op set: opcode 1 leaves the raw QKV vector, the attention
+// prologue applies the per-head RMSNorm of q and k and RoPE
+// (qimeng_megakernel/models/LLM/qwen/qwen3__0_6b/A100/single_batch/decode_schedule/fused/operations.py:52-120).
+struct Qwen3_1p7B {
+  static constexpr int H = 2048;
+  static constexpr int F = 6144;
+  static constexpr int D = 128;
+  static constexpr int NQ = 16;
+  static constexpr int NKV = 8;
+  static constexpr int GQA = NQ / NKV;
+  static constexpr int QKV = (NQ + 2 * NKV) * D;
+  static constexpr int KV_BLOCK = 16;
+  static constexpr bool QK_NORM = true;
 };
 
 constexpr int kResSlots = 4096;
@@ -37,7 +53,7 @@ struct Smem {
   float red[kWaves];
   alignas(16) u16 x[M::F];              // activation vector handed to the GEMV lanes
   float res[kResSlots];                 // per-row GEMV results awaiting the epilogue pass
-  float merge[kWaves * 8][M::GQA][M::D + 4];  // attention state per lane group: acc[D], m, l (+pad)
+  float merge[kWaves * 8][M::GQA][M::D + 4];  // attention state per lane group: acc[D], m, l, fold weights
   unsigned long long t_wait;            // timeline: when the last counter wait finished
   unsigned long long stamps[4];         // timeline: op-specific intermediate timestamps
 };
@@ -278,7 +294,15 @@ __device__ bool op_rms_qkv_rope(const Params& p, Smem<M>& s, const Ctx& c) {
   for (int pair = threadIdx.x; pair < nrows / 2; pair += kThreads) {
     const int r = rs + 2 * pair;
     const float v0 = round_bf16(s.res[2 * pair]), v1 = round_bf16(s.res[2 * pair + 1]);
-    if (r < M::NQ * M::D) {
+    if constexpr (M::QK_NORM) {
+      // Qwen3 op set: the rounded GEMV result leaves as it is; norm and RoPE belong to the attention prologue.
+      const uint32_t w = static_cast<uint32_t>(f2bf(v0)) | (static_cast<uint32_t>(f2bf(v1)) << 16);
+      st_shared32(p.qkv_raw + r, w);
+      if (tg) {
+        const int kq = M::NQ * M::D, kk = (M::NQ + M::NKV) * M::D;
+        st_tagged(p.ws + (r < kq ? kWsQ + r / 2 : (r < kk ? kWsK + (r - kq) / 2 : kWsV + (r - kk) / 2)), w, tag);
+      }
+    } else if (r < M::NQ * M::D) {
       const uint32_t w = rope_pair(v0, v1, cosr, sinr, r % M::D);
       st_shared32(p.q_post_rope + r, w);
       if (tg) st_tagged(p.ws + kWsQ + r / 2, w, tag);
@@ -357,9 +381,16 @@ __device__ __forceinline__ void merge_partials(const Params& p, int head0, int n
 // [2, layer, kv_head, num_partials, partial_idx, merge_in_last]
 // Flash-decoding over one contiguous slice of the context for the GQA group of
 // one KV head.  A wave handles 8 tokens per pass: lane group g = lane/8 owns a
-// token, lane c = lane%8 owns dims 8c..8c+7 of K and V.  Every lane group keeps
+// token, lane c = lane%8 owns D/8 neighbouring dims of K and V.  Every lane group keeps
 // its own running (max, sum, acc) per query head; groups, then waves, are
 // merged once at the end.  Scores live in the log2 domain.
+//
+// The query heads and the K/V row appended in this launch are first staged in LDS (bf16:
+// [0, GQA*D) q, then k, then v) — from their tagged units, or after the per-head counters from
+// the caller's buffers.  With the Qwen3 op set (M::QK_NORM) what is staged is the raw QKV
+// vector; one wave per vector then applies the per-head RMSNorm and RoPE in place
+// (qwen3__0_6b/…/fused/operations.py:52-120), and the workgroup whose slice holds this position
+// also writes q_post_rope and the cache row.
 //
 // merge_in_last (an extension; 0 in streams built by the reference scheduler): the
 // workgroup whose arrival completes the head group's counter merges all partials
@@ -367,7 +398,11 @@ __device__ __forceinline__ void merge_partials(const Params& p, int head0, int n
 // (and no second wait) is needed.
 template <class M>
 __device__ bool op_attn_splitkv(const Params& p, Smem<M>& s, const Ctx& c) {
-  static_assert(M::D == 64 && M::GQA == 4, "lane mapping assumes head_dim 64 and 4 query heads per KV head");
+  constexpr int D = M::D, GQA = M::GQA;
+  constexpr int DPL = D / 8;   // dims of K and V one lane owns
+  constexpr int VPL = DPL / 8; // 16-byte vectors per lane and row
+  static_assert(D % 64 == 0 && GQA * D == 4 * kWaveSize, "four waves fold the GQA*D outputs; a lane owns whole 16-byte vectors");
+  static_assert(!M::QK_NORM || D == 2 * kWaveSize, "the per-head norm gives every lane one rotation pair");
   const int layer = s.inst[1], kvh = s.inst[2], P = s.inst[3], part = s.inst[4];
   const int merge_mode = s.inst[5];  // 0: per-head counters, 1: last arrival merges, 2: the O-proj merges
   const bool merge_in_last = merge_mode == 1;
@@ -386,37 +421,50 @@ __device__ bool op_attn_splitkv(const Params& p, Smem<M>& s, const Ctx& c) {
   const int bpp = (total_blocks + P - 1) / P;
   const int t0 = min(part * bpp, total_blocks) * M::KV_BLOCK;
   const int t1 = min(min((part + 1) * bpp, total_blocks) * M::KV_BLOCK, seq_len);
+  const bool has_new = p.pos_id >= t0 && p.pos_id < t1;
 
   // Rows of earlier positions do not depend on this step: fetch the first ones now.
-  const size_t tok_stride = static_cast<size_t>(M::NKV) * M::D;
-  const size_t base = static_cast<size_t>(layer) * p.max_seq_len * tok_stride + static_cast<size_t>(kvh) * M::D + col * 8;
+  const size_t tok_stride = static_cast<size_t>(M::NKV) * D;
+  const size_t row_of_kvh = static_cast<size_t>(layer) * p.max_seq_len * tok_stride + static_cast<size_t>(kvh) * D;
+  const size_t base = row_of_kvh + col * DPL;
   int t = t0 + wave * 8 + grp;
-  v4u kv = {0, 0, 0, 0}, vv = {0, 0, 0, 0};
+  v4u kv[VPL], vv[VPL];
+#pragma unroll
+  for (int j = 0; j < VPL; ++j) {
+    kv[j] = v4u{0, 0, 0, 0};
+    vv[j] = v4u{0, 0, 0, 0};
+  }
   if (t < t1 && t != p.pos_id) {
-    kv = *reinterpret_cast<const v4u*>(p.k_cache + base + static_cast<size_t>(t) * tok_stride);
-    vv = *reinterpret_cast<const v4u*>(p.v_cache + base + static_cast<size_t>(t) * tok_stride);
+#pragma unroll
+    for (int j = 0; j < VPL; ++j) {
+      kv[j] = reinterpret_cast<const v4u*>(p.k_cache + base + static_cast<size_t>(t) * tok_stride)[j];
+      vv[j] = reinterpret_cast<const v4u*>(p.v_cache + base + static_cast<size_t>(t) * tok_stride)[j];
+    }
   }
 
+  // ---- stage q (and the appended K/V row) in LDS --------------------------------------------
   const bool tg = tagged(p);
-  // Tagged mode: q of the four heads (128 units) is polled by threads 0..63, the K and V rows
-  // appended in this launch (32 units each, only when the slice holds this position) by threads
-  // 64..95; all of it is staged in LDS as words [0,128) q, [128,160) k, [160,192) v.
-  const v4u* stage = reinterpret_cast<const v4u*>(s.x);
+  u16* stage16 = s.x;
+  constexpr int kQ = 0, kK = GQA * D, kV = GQA * D + D;
+  const size_t new_row = row_of_kvh + static_cast<size_t>(p.pos_id) * tok_stride;
   if (tg) {
+    // q: GQA*D/2 = 128 units, two per thread of wave 0; K and V: D/2 units each, two per thread.
     const uint32_t tag = tag_of(s.generation, layer);
-    uint32_t* words = reinterpret_cast<uint32_t*>(s.x);
-    const bool has_new = p.pos_id >= t0 && p.pos_id < t1;
+    uint32_t* words = reinterpret_cast<uint32_t*>(stage16);
     bool arrived = true;
     uint32_t a = 0, b = 0;
-    if (threadIdx.x < 64) {
-      arrived = poll_tagged2(p.ws + kWsQ + kvh * (M::GQA * M::D / 2) + 2 * threadIdx.x, tag, p.spin_limit, a, b);
-      words[2 * threadIdx.x] = a;
-      words[2 * threadIdx.x + 1] = b;
-    } else if (threadIdx.x < 96 && has_new) {
-      const int j = threadIdx.x - 64;
-      arrived = poll_tagged2(p.ws + (j < 16 ? kWsK : kWsV) + kvh * (M::D / 2) + 2 * (j & 15), tag, p.spin_limit, a, b);
-      words[128 + 2 * j] = a;
-      words[128 + 2 * j + 1] = b;
+    const int tid = threadIdx.x;
+    if (tid < 64) {
+      arrived = poll_tagged2(p.ws + kWsQ + kvh * (GQA * D / 2) + 2 * tid, tag, p.spin_limit, a, b);
+      words[kQ / 2 + 2 * tid] = a;
+      words[kQ / 2 + 2 * tid + 1] = b;
+    } else if (tid < 64 + D / 2 && has_new) {
+      const int j = tid - 64;                              // [0, D/4): K, [D/4, D/2): V
+      const bool is_v = j >= D / 4;
+      const int u = 2 * (is_v ? j - D / 4 : j);
+      arrived = poll_tagged2(p.ws + (is_v ? kWsV : kWsK) + kvh * (D / 2) + u, tag, p.spin_limit, a, b);
+      words[(is_v ? kV : kK) / 2 + u] = a;
+      words[(is_v ? kV : kK) / 2 + u + 1] = b;
     }
     if (!arrived) {
       s.ctl[0] = 1;
@@ -426,122 +474,187 @@ __device__ bool op_attn_splitkv(const Params& p, Smem<M>& s, const Ctx& c) {
       s.t_wait = wall_clock64();
       s.ctl[2] = 1;
     }
+  } else {
+    if (!wg_wait(p, s, c, GQA + 2,
+                 [&](int i) {
+                   const int slot = i < GQA ? kvh * GQA + i : (i == GQA ? M::NQ + kvh : M::NQ + M::NKV + kvh);
+                   return counter_ptr(p, layer, ROW_QKV, slot);
+                 },
+                 p.qkv_blocks_per_head))
+      return false;
+    // 16-byte chunks: GQA*D/8 of q, then D/8 of K and of V (the row of this position only)
+    const int tid = threadIdx.x;
+    constexpr int kQChunks = GQA * D / 8, kRowChunks = D / 8;
+    const u16* q_src = M::QK_NORM ? p.qkv_raw + kvh * GQA * D : p.q_post_rope + kvh * GQA * D;
+    const u16* k_src = M::QK_NORM ? p.qkv_raw + M::NQ * D + kvh * D : p.k_cache + new_row;
+    const u16* v_src = M::QK_NORM ? p.qkv_raw + (M::NQ + M::NKV) * D + kvh * D : p.v_cache + new_row;
+    if (tid < kQChunks) {
+      reinterpret_cast<v4u*>(stage16 + kQ)[tid] = ld_shared128(q_src + tid * 8);
+    } else if (tid < kQChunks + kRowChunks && has_new) {
+      reinterpret_cast<v4u*>(stage16 + kK)[tid - kQChunks] = ld_shared128(k_src + (tid - kQChunks) * 8);
+    } else if (tid < kQChunks + 2 * kRowChunks && has_new) {
+      reinterpret_cast<v4u*>(stage16 + kV)[tid - kQChunks - kRowChunks] = ld_shared128(v_src + (tid - kQChunks - kRowChunks) * 8);
+    }
+  }
+  __syncthreads();
+  if (s.ctl[0]) return false;
+
+  if constexpr (M::QK_NORM) {
+    // Waves 0..GQA-1: the query heads; wave GQA: the new K row; wave GQA+1: the new V row goes
+    // to the cache as it is.  Lane l owns the rotation pair (2l, 2l+1).
+    //   n = bf16(w * (x * rsqrt(mean(x^2) + eps)))   — fp32 throughout, one rounding
+    uint32_t* words = reinterpret_cast<uint32_t*>(stage16);
+    if (wave <= GQA && (wave < GQA || has_new)) {
+      const bool is_k = wave == GQA;
+      const int at = is_k ? kK / 2 : (kQ + wave * D) / 2;
+      const uint32_t raw = words[at + lane];
+      const float x0 = bf_lo(raw), x1 = bf_hi(raw);
+      const float ss = wave_sum(__builtin_fmaf(x1, x1, x0 * x0));
+      const float rstd = 1.0f / sqrtf(ss / static_cast<float>(D) + p.rms_norm_eps);
+      const uint32_t wn = reinterpret_cast<const uint32_t*>((is_k ? p.k_norm : p.q_norm) + static_cast<size_t>(layer) * D)[lane];
+      const float n0 = round_bf16(bf_lo(wn) * (x0 * rstd)), n1 = round_bf16(bf_hi(wn) * (x1 * rstd));
+      const float* cosr = p.rope_cos + static_cast<size_t>(p.pos_id) * D;
+      const float* sinr = p.rope_sin + static_cast<size_t>(p.pos_id) * D;
+      const uint32_t out = rope_pair(n0, n1, cosr, sinr, 2 * lane);
+      words[at + lane] = out;
+      if (has_new) {  // exactly one partial of this KV head holds the position: it owns the caller's copies
+        if (is_k) st_shared32(p.k_cache + new_row + 2 * lane, out);
+        else st_shared32(p.q_post_rope + (kvh * GQA + wave) * D + 2 * lane, out);
+      }
+    } else if (wave == GQA + 1 && has_new) {
+      st_shared32(p.v_cache + new_row + 2 * lane, words[kV / 2 + lane]);
+    }
     __syncthreads();
-    if (s.ctl[0]) return false;
-  } else if (!wg_wait(p, s, c, M::GQA + 2,
-                      [&](int i) {
-                        const int slot = i < M::GQA ? kvh * M::GQA + i : (i == M::GQA ? M::NQ + kvh : M::NQ + M::NKV + kvh);
-                        return counter_ptr(p, layer, ROW_QKV, slot);
-                      },
-                      p.qkv_blocks_per_head)) {
-    return false;
   }
 
-  // q[h][8]: this lane's dims of the four query heads, pre-scaled into the log2 domain.
+  // q[h][DPL]: this lane's dims of the query heads, pre-scaled into the log2 domain.
   const float qscale = p.attn_scale * 1.4426950408889634f;
-  float q[M::GQA][8];
+  float q[GQA][DPL];
   {
-    v4u qv[M::GQA];
 #pragma unroll
-    for (int h = 0; h < M::GQA; ++h)
-      qv[h] = tg ? stage[h * (M::D / 8) + col] : ld_shared128(p.q_post_rope + (kvh * M::GQA + h) * M::D + col * 8);
-    if (t < t1 && t == p.pos_id) {  // the row another workgroup appended during this launch
-      kv = tg ? stage[32 + col] : ld_shared128(p.k_cache + base + static_cast<size_t>(t) * tok_stride);
-      vv = tg ? stage[40 + col] : ld_shared128(p.v_cache + base + static_cast<size_t>(t) * tok_stride);
+    for (int h = 0; h < GQA; ++h) {
+#pragma unroll
+      for (int j = 0; j < VPL; ++j) {
+        const v4u qv = reinterpret_cast<const v4u*>(stage16 + kQ + h * D + col * DPL)[j];
+        q[h][8 * j + 0] = bf_lo(qv.x) * qscale; q[h][8 * j + 1] = bf_hi(qv.x) * qscale;
+        q[h][8 * j + 2] = bf_lo(qv.y) * qscale; q[h][8 * j + 3] = bf_hi(qv.y) * qscale;
+        q[h][8 * j + 4] = bf_lo(qv.z) * qscale; q[h][8 * j + 5] = bf_hi(qv.z) * qscale;
+        q[h][8 * j + 6] = bf_lo(qv.w) * qscale; q[h][8 * j + 7] = bf_hi(qv.w) * qscale;
+      }
     }
+    if (t < t1 && t == p.pos_id) {  // the row appended during this launch
 #pragma unroll
-    for (int h = 0; h < M::GQA; ++h) {
-      q[h][0] = bf_lo(qv[h].x) * qscale; q[h][1] = bf_hi(qv[h].x) * qscale;
-      q[h][2] = bf_lo(qv[h].y) * qscale; q[h][3] = bf_hi(qv[h].y) * qscale;
-      q[h][4] = bf_lo(qv[h].z) * qscale; q[h][5] = bf_hi(qv[h].z) * qscale;
-      q[h][6] = bf_lo(qv[h].w) * qscale; q[h][7] = bf_hi(qv[h].w) * qscale;
+      for (int j = 0; j < VPL; ++j) {
+        kv[j] = reinterpret_cast<const v4u*>(stage16 + kK + col * DPL)[j];
+        vv[j] = reinterpret_cast<const v4u*>(stage16 + kV + col * DPL)[j];
+      }
     }
   }
 
   QMK_STAMP(0);  // q (and the appended row) have arrived
-  float m[M::GQA], l[M::GQA], acc[M::GQA][8];
+  float m[GQA], l[GQA], acc[GQA][DPL];
 #pragma unroll
-  for (int h = 0; h < M::GQA; ++h) {
+  for (int h = 0; h < GQA; ++h) {
     m[h] = -INFINITY;
     l[h] = 0.f;
 #pragma unroll
-    for (int i = 0; i < 8; ++i) acc[h][i] = 0.f;
+    for (int i = 0; i < DPL; ++i) acc[h][i] = 0.f;
   }
 
   while (t < t1) {
     // next token of this lane group, fetched while the current one is scored
     const int tn = t + kWaves * 8;
-    v4u kn = {0, 0, 0, 0}, vn = {0, 0, 0, 0};
+    v4u kn[VPL], vn[VPL];
+#pragma unroll
+    for (int j = 0; j < VPL; ++j) {
+      kn[j] = v4u{0, 0, 0, 0};
+      vn[j] = v4u{0, 0, 0, 0};
+    }
     if (tn < t1) {
       const size_t off = base + static_cast<size_t>(tn) * tok_stride;
-      if (tn == p.pos_id) {
-        kn = tg ? stage[32 + col] : ld_shared128(p.k_cache + off);
-        vn = tg ? stage[40 + col] : ld_shared128(p.v_cache + off);
-      } else {
-        kn = *reinterpret_cast<const v4u*>(p.k_cache + off);
-        vn = *reinterpret_cast<const v4u*>(p.v_cache + off);
+#pragma unroll
+      for (int j = 0; j < VPL; ++j) {
+        if (tn == p.pos_id) {
+          kn[j] = reinterpret_cast<const v4u*>(stage16 + kK + col * DPL)[j];
+          vn[j] = reinterpret_cast<const v4u*>(stage16 + kV + col * DPL)[j];
+        } else {
+          kn[j] = reinterpret_cast<const v4u*>(p.k_cache + off)[j];
+          vn[j] = reinterpret_cast<const v4u*>(p.v_cache + off)[j];
+        }
       }
     }
-    const float k[8] = {bf_lo(kv.x), bf_hi(kv.x), bf_lo(kv.y), bf_hi(kv.y), bf_lo(kv.z), bf_hi(kv.z), bf_lo(kv.w), bf_hi(kv.w)};
-    const float v[8] = {bf_lo(vv.x), bf_hi(vv.x), bf_lo(vv.y), bf_hi(vv.y), bf_lo(vv.z), bf_hi(vv.z), bf_lo(vv.w), bf_hi(vv.w)};
+    float k[DPL], v[DPL];
 #pragma unroll
-    for (int h = 0; h < M::GQA; ++h) {
+    for (int j = 0; j < VPL; ++j) {
+      k[8 * j + 0] = bf_lo(kv[j].x); k[8 * j + 1] = bf_hi(kv[j].x); k[8 * j + 2] = bf_lo(kv[j].y); k[8 * j + 3] = bf_hi(kv[j].y);
+      k[8 * j + 4] = bf_lo(kv[j].z); k[8 * j + 5] = bf_hi(kv[j].z); k[8 * j + 6] = bf_lo(kv[j].w); k[8 * j + 7] = bf_hi(kv[j].w);
+      v[8 * j + 0] = bf_lo(vv[j].x); v[8 * j + 1] = bf_hi(vv[j].x); v[8 * j + 2] = bf_lo(vv[j].y); v[8 * j + 3] = bf_hi(vv[j].y);
+      v[8 * j + 4] = bf_lo(vv[j].z); v[8 * j + 5] = bf_hi(vv[j].z); v[8 * j + 6] = bf_lo(vv[j].w); v[8 * j + 7] = bf_hi(vv[j].w);
+    }
+#pragma unroll
+    for (int h = 0; h < GQA; ++h) {
       float sc = 0.f;
 #pragma unroll
-      for (int i = 0; i < 8; ++i) sc = __builtin_fmaf(q[h][i], k[i], sc);
+      for (int i = 0; i < DPL; ++i) sc = __builtin_fmaf(q[h][i], k[i], sc);
       sc = group8_sum(sc);  // the 8 lanes of a group always take the same branch
       const float mn = fmaxf(m[h], sc);
       const float alpha = exp2_fast(m[h] - mn);   // 0 on the first token (m = -inf)
       const float pr = exp2_fast(sc - mn);
       l[h] = __builtin_fmaf(l[h], alpha, pr);
 #pragma unroll
-      for (int i = 0; i < 8; ++i) acc[h][i] = __builtin_fmaf(acc[h][i], alpha, pr * v[i]);
+      for (int i = 0; i < DPL; ++i) acc[h][i] = __builtin_fmaf(acc[h][i], alpha, pr * v[i]);
       m[h] = mn;
     }
     t = tn;
-    kv = kn;
-    vv = vn;
+#pragma unroll
+    for (int j = 0; j < VPL; ++j) {
+      kv[j] = kn[j];
+      vv[j] = vn[j];
+    }
   }
 
   QMK_STAMP(1);  // tokens scored
-  // Every lane group (8 per wave, 64 per workgroup) parks its state in LDS; thread (h, d) of the
-  // first 256 then folds the 64 states of its head.  (Folding across lanes with shuffles costs
-  // ~120 dependent LDS-crossbar round trips per wave — several microseconds.)
+  // Every lane group (8 per wave, 64 per workgroup) parks its state in LDS; the first four waves
+  // then fold the 64 states: wave f takes 64 neighbouring outputs of the GQA*D.  (Folding across
+  // lanes with shuffles costs ~120 dependent LDS-crossbar round trips per wave — several microseconds.)
   {
     const int g = wave * 8 + grp;
 #pragma unroll
-    for (int h = 0; h < M::GQA; ++h) {
-      float* dst = &s.merge[g][h][col * 8];
-      *reinterpret_cast<float4*>(dst) = make_float4(acc[h][0], acc[h][1], acc[h][2], acc[h][3]);
-      *reinterpret_cast<float4*>(dst + 4) = make_float4(acc[h][4], acc[h][5], acc[h][6], acc[h][7]);
+    for (int h = 0; h < GQA; ++h) {
+      float* dst = &s.merge[g][h][col * DPL];
+#pragma unroll
+      for (int i = 0; i < DPL; i += 4) *reinterpret_cast<float4*>(dst + i) = make_float4(acc[h][i], acc[h][i + 1], acc[h][i + 2], acc[h][i + 3]);
       if (col == 0) {
-        s.merge[g][h][M::D] = m[h];
-        s.merge[g][h][M::D + 1] = l[h];
+        s.merge[g][h][D] = m[h];
+        s.merge[g][h][D + 1] = l[h];
       }
     }
   }
   __syncthreads();
 
-  // Wave h of the first four folds head h.  Lane g first turns group g's (m, l) into its weight
-  // f = 2^(m - max) and l*f (max and the denominator are wave reductions).  Then lane = 4*quad + sub
-  // sums dims 4*quad..4*quad+3 over the 16 states g = sub, sub+4, ... and the four `sub` lanes of a
-  // quad are added with DPP.
-  if (threadIdx.x < M::GQA * M::D) {
-    static_assert(kWaves * 8 == kWaveSize && M::D == kWaveSize, "one lane per group, 16 dim-quads x 4 state subsets");
-    const int h = threadIdx.x / kWaveSize;
-    const float mg = s.merge[lane][h][M::D];
+  // Fold wave f handles head h = f / (D/64), dims dbase = 64 * (f % (D/64)) .. +63.  Lane g first
+  // turns group g's (m, l) into its weight w = 2^(m - max) and l*w (max and the denominator are
+  // wave reductions; with D = 128 the two waves of a head compute the same numbers).  Then
+  // lane = 4*quad + sub sums dims dbase + 4*quad..+3 over the 16 states g = sub, sub+4, ... and the
+  // four `sub` lanes of a quad are added with DPP.
+  if (threadIdx.x < GQA * D) {
+    static_assert(kWaves * 8 == kWaveSize, "one lane per lane group");
+    const int h = wave / (D / kWaveSize), dbase = kWaveSize * (wave % (D / kWaveSize));
+    const float mg = s.merge[lane][h][D];
     const float mx = wave_max(mg);
-    const float f = (mg == -INFINITY) ? 0.f : exp2_fast(mg - mx);
-    const float den = wave_sum(s.merge[lane][h][M::D + 1] * f);
-    s.merge[lane][h][M::D + 2] = f;
-    // rows [*][h] of s.merge are touched by this wave only; LDS operations of one wave stay in order
+    const float wgt = (mg == -INFINITY) ? 0.f : exp2_fast(mg - mx);
+    const float den = wave_sum(s.merge[lane][h][D + 1] * wgt);
+    // Each fold wave keeps its weights in a column of its own (D+2, D+3): no other wave reads or
+    // writes it; LDS operations of one wave stay in order.
+    const int wcol = D + 2 + wave % (D / kWaveSize);
+    s.merge[lane][h][wcol] = wgt;
     const int quad = lane >> 2, sub = lane & 3;
     float4 part4[16];
     float w16[16];
 #pragma unroll
     for (int i = 0; i < 16; ++i) {
-      part4[i] = *reinterpret_cast<const float4*>(&s.merge[sub + 4 * i][h][4 * quad]);
-      w16[i] = s.merge[sub + 4 * i][h][M::D + 2];
+      part4[i] = *reinterpret_cast<const float4*>(&s.merge[sub + 4 * i][h][dbase + 4 * quad]);
+      w16[i] = s.merge[sub + 4 * i][h][wcol];
     }
     float n0 = 0.f, n1 = 0.f, n2 = 0.f, n3 = 0.f;
 #pragma unroll
@@ -555,14 +668,15 @@ __device__ bool op_attn_splitkv(const Params& p, Smem<M>& s, const Ctx& c) {
     n1 += dpp_f32<kDppQuadXor1>(0.f, n1); n1 += dpp_f32<kDppQuadXor2>(0.f, n1);
     n2 += dpp_f32<kDppQuadXor1>(0.f, n2); n2 += dpp_f32<kDppQuadXor2>(0.f, n2);
     n3 += dpp_f32<kDppQuadXor1>(0.f, n3); n3 += dpp_f32<kDppQuadXor2>(0.f, n3);
-    const int head = kvh * M::GQA + h;
+    const int head = kvh * GQA + h;
     const bool empty = !(den > 0.f);
     const float inv = empty ? 0.f : 1.0f / den;
     // Normalised partial output and log2-sum-exp; an empty slice contributes (0, -inf).
-    // Lane `sub` of a quad stores dim 4*quad + sub.
+    // Lane `sub` of a quad stores dim dbase + 4*quad + sub.
     const float mine = sub == 0 ? n0 : (sub == 1 ? n1 : (sub == 2 ? n2 : n3));
-    st_shared_f32(p.attn_partial + (static_cast<size_t>(head) * p.max_splits + part) * M::D + lane, mine * inv);
-    if (lane == 0) st_shared_f32(p.attn_lse + static_cast<size_t>(head) * p.max_splits + part, empty ? -INFINITY : mx + log2f(den));
+    st_shared_f32(p.attn_partial + (static_cast<size_t>(head) * p.max_splits + part) * D + dbase + lane, mine * inv);
+    if (lane == 0 && dbase == 0)
+      st_shared_f32(p.attn_lse + static_cast<size_t>(head) * p.max_splits + part, empty ? -INFINITY : mx + log2f(den));
   }
 
   QMK_STAMP(2);  // partial merged and stored
@@ -879,15 +993,15 @@ __device__ bool op_down_residual(const Params& p, Smem<M>& s, const Ctx& c) {
   if (!wg_wait_all(p, s, c, layer, ROW_UPGATE, split, p.upgate_blocks_per_bucket)) return false;
 
   // The K slice of silu_out into LDS; the remaining row buffers are requested behind it.
-  static_assert(M::F / 4 == 4 * kThreads, "four 8-byte loads per thread cover the widest slice");
-  uint64_t act[4];
+  constexpr int kActLoads = (M::F / 4 + kThreads - 1) / kThreads;  // 8-byte loads per thread that cover the widest slice
+  uint64_t act[kActLoads];
 #pragma unroll
-  for (int k = 0; k < 4; ++k)
+  for (int k = 0; k < kActLoads; ++k)
     if (static_cast<int>(threadIdx.x) + k * kThreads < kg / 4) act[k] = ld_shared64(p.silu_out + ks + (threadIdx.x + k * kThreads) * 4);
   asm volatile("" ::: "memory");
   preload_range<kEarly, kDepth>(rows_w > 0 ? n_elems : 0, src, buf);
 #pragma unroll
-  for (int k = 0; k < 4; ++k)
+  for (int k = 0; k < kActLoads; ++k)
     if (static_cast<int>(threadIdx.x) + k * kThreads < kg / 4) reinterpret_cast<uint64_t*>(s.x)[threadIdx.x + k * kThreads] = act[k];
   __syncthreads();
 

@@ -19,7 +19,7 @@ _WEIGHT_FIELDS = frozenset(
     {
         "attn_norm_weights", "qkv_weights", "rope_cos", "rope_sin", "o_proj_weights",
         "mlp_norm_weights", "up_proj_weights", "gate_proj_weights", "down_proj_weights",
-        "lm_head_norm_weights", "lm_head_weights",
+        "lm_head_norm_weights", "lm_head_weights", "q_norm_weights", "k_norm_weights",
     }
 )
 
@@ -34,6 +34,8 @@ class Globals:
     # --- weights, in the order a layer consumes them ------------------------
     attn_norm_weights: Optional[Tensor] = None       # bf16 [L, H]
     qkv_weights: Optional[Tensor] = None             # bf16 [L, (Hq+2Hkv)*D, H], q/k rows pair-interleaved
+    q_norm_weights: Optional[Tensor] = None          # bf16 [L, D]  per-head RMSNorm of q (Qwen3 op set), pair-interleaved
+    k_norm_weights: Optional[Tensor] = None          # bf16 [L, D]  per-head RMSNorm of k
     rope_cos: Optional[Tensor] = None                # f32  [max_pos, D], pair-interleaved
     rope_sin: Optional[Tensor] = None                # f32  [max_pos, D]
     o_proj_weights: Optional[Tensor] = None          # bf16 [L, H, H]
@@ -48,6 +50,7 @@ class Globals:
     k_cache: Optional[Tensor] = None                 # bf16 [L, 1, S, Hkv, D]
     v_cache: Optional[Tensor] = None                 # bf16 [L, 1, S, Hkv, D]
     hidden_states: Optional[Tensor] = None           # bf16 [H]   residual stream, in/out
+    qkv_raw: Optional[Tensor] = None                 # bf16 [(Hq+2Hkv)*D]  QKV before QK-norm and RoPE (Qwen3 op set)
     q_post_rope: Optional[Tensor] = None             # bf16 [Hq*D]
     attn_out: Optional[Tensor] = None                # bf16 [Hq*D]
     attn_out_intermediates: Optional[Tensor] = None  # f32  [Hq, max_partials, D]

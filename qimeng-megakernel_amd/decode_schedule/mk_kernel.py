@@ -57,6 +57,7 @@ class QmkArgs(ctypes.Structure):
         ("qkv_blocks_per_head", _I), ("oproj_blocks", _I), ("upgate_blocks_per_bucket", _I), ("down_arrivals", _I),
         ("timeline", _P), ("stream", _P), ("workspace", _P), ("workspace_bytes", ctypes.c_uint64),
         ("embed_tokens", _P), ("token_out", _P),
+        ("qkv_raw", _P), ("q_norm_weights", _P), ("k_norm_weights", _P),
     ]
 
 

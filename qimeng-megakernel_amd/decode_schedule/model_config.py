@@ -28,6 +28,11 @@ class DecodeShape:
     # one reduction instruction merges this many query heads (= GQA ratio).
     attn_kv_block_size: int = 16
     attn_reduction_size: int = 4
+    # Qwen3 op set (`…/qwen/qwen3__0_6b/A100/single_batch/decode_schedule/fused/operations.py:52-120`):
+    # opcode 1 leaves the raw QKV vector, the attention prologue applies a per-head RMSNorm to q
+    # and k before RoPE; the LM head shares the embedding matrix.
+    qk_norm: bool = False
+    tie_word_embeddings: bool = False
 
     @property
     def num_heads(self) -> int:
@@ -45,6 +50,8 @@ class DecodeShape:
         """bf16 weight bytes one decode step has to stream (norm vectors included)."""
         h, f = self.hidden_size, self.intermediate_size
         per_layer = (self.qkv_out_dim * h + self.num_attention_heads * self.head_dim * h + 3 * f * h) * 2 + 2 * h * 2
+        if self.qk_norm:
+            per_layer += 2 * self.head_dim * 2
         return per_layer * self.num_hidden_layers + self.vocab_size * h * 2 + h * 2
 
     def kv_bytes_per_context_token(self) -> int:
@@ -57,6 +64,13 @@ class DecodeShape:
 
 
 LLAMA_3_2_1B = DecodeShape()
+
+#: Qwen3-1.7B shape: 28 layers, 16 query / 8 KV heads of 128, per-head QK RMSNorm, tied LM head.
+QWEN3_1_7B = DecodeShape(
+    num_hidden_layers=28, hidden_size=2048, intermediate_size=6144, head_dim=128, num_attention_heads=16,
+    num_key_value_heads=8, vocab_size=151936, rms_norm_eps=1e-6, rope_theta=1000000.0, attn_reduction_size=2,
+    qk_norm=True, tie_word_embeddings=True,
+)
 
 _FIELDS = tuple(f.name for f in dataclasses.fields(DecodeShape))
 

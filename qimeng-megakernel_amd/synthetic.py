@@ -62,7 +62,11 @@ def random_weights(shape: DecodeShape, seed: int, max_positions: int) -> dict[st
     w["up_proj_weights"] = torch.stack([_normal_bf16(gen, F, H) for _ in range(L)])
     w["gate_proj_weights"] = torch.stack([_normal_bf16(gen, F, H) for _ in range(L)])
     w["down_proj_weights"] = torch.stack([_normal_bf16(gen, H, F) for _ in range(L)])
-    w["lm_head_weights"] = _normal_bf16(gen, V, H)
+    w["lm_head_weights"] = w["embed_tokens"] if shape.tie_word_embeddings else _normal_bf16(gen, V, H)
+    if shape.qk_norm:
+        # Not all ones: a per-head norm whose weights do nothing would hide a wrong column order.
+        for name in ("q_norm_weights", "k_norm_weights"):
+            w[name] = (1.0 + 0.1 * torch.randn(L, shape.head_dim, generator=gen, dtype=torch.float32)).to(torch.bfloat16)
     w["attn_norm_weights"] = torch.ones(L, H, dtype=torch.bfloat16)
     w["mlp_norm_weights"] = torch.ones(L, H, dtype=torch.bfloat16)
     w["lm_head_norm_weights"] = torch.ones(H, dtype=torch.bfloat16)
@@ -111,6 +115,10 @@ def build_globals(
         **{k: v for k, v in on_device.items() if k != "embed_tokens"},
     )
     g.embed_tokens = on_device["embed_tokens"]
+    if shape.tie_word_embeddings:
+        g.lm_head_weights = g.embed_tokens          # one matrix on the device, as in the tied checkpoint
+    if shape.qk_norm:
+        g.qkv_raw = zeros(shape.qkv_out_dim)
     return g
 
 
