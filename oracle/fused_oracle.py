@@ -96,8 +96,45 @@ class FusedOracle:
         g.k_cache[layer, 0, pos].copy_(k_rot[0].to(g.k_cache.dtype))
         g.v_cache[layer, 0, pos].copy_(v[0].to(g.v_cache.dtype))
 
+    def attention_split_merge(self, g: Any, layer: int) -> None:
+        """The Qwen3 route's fused attention: always split into as many partials as the workspace
+        has columns and merged in the log2 domain (qwen3__0_6b/…/fused/operations.py:123-215)."""
+        s = self.shape
+        nq, nkv, d = s.num_attention_heads, s.num_key_value_heads, s.head_dim
+        ratio, block = nq // nkv, s.attn_kv_block_size
+        n = int(g.position_id or 0) + 1
+        parts = int(g.attn_lse_intermediates.shape[1])
+        total_blocks = math.ceil(n / block)
+        per_part = math.ceil(total_blocks / parts)
+        q = g.q_post_rope.view(nq, d).float()
+        k_full, v_full = g.k_cache[layer, 0, :n].float(), g.v_cache[layer, 0, :n].float()
+        scale = 1.0 / math.sqrt(d)
+        for h in range(nq):
+            k, v = k_full[:, h // ratio], v_full[:, h // ratio]
+            for p in range(parts):
+                t0 = p * per_part * block
+                t1 = min(min((p + 1) * per_part, total_blocks) * block, n)
+                if t0 >= t1:
+                    g.attn_lse_intermediates[h, p] = -float("inf")
+                    g.attn_out_intermediates[h, p] = 0.0
+                    continue
+                sc = torch.einsum("hi,ki->hk", q[h : h + 1], k[t0:t1]) * scale
+                g.attn_lse_intermediates[h, p] = torch.log2(torch.sum(torch.exp(sc), dim=-1) + 1e-12).squeeze(0)
+                g.attn_out_intermediates[h, p] = torch.einsum("hk,ko->ho", torch.softmax(sc, dim=-1), v[t0:t1]).squeeze(0)
+        step = s.attn_reduction_size  # the reference merges one reduction group of heads at a time
+        for h0 in range(0, nq, step):
+            lses, outs = g.attn_lse_intermediates[h0 : h0 + step], g.attn_out_intermediates[h0 : h0 + step]
+            lses = torch.where(torch.isposinf(lses), torch.full_like(lses, 1e10), lses)
+            top = torch.clamp(lses.max(dim=1, keepdim=True).values, min=-1e10)
+            weights = (lses - top).exp2()
+            denom = weights.sum(dim=1, keepdim=True).clamp(min=1e-12)
+            merged = (outs * weights.unsqueeze(-1)).sum(dim=1) / denom
+            g.attn_out.view(nq, d)[h0 : h0 + step] = merged.to(g.attn_out.dtype)
+
     def attention(self, g: Any, layer: int) -> None:
         s = self.shape
+        if getattr(s, "qk_norm", False):
+            return self.attention_split_merge(g, layer)
         nq, nkv, d = s.num_attention_heads, s.num_key_value_heads, s.head_dim
         ratio = nq // nkv
         n = int(g.position_id or 0) + 1

@@ -40,7 +40,7 @@ from typing import Any, Iterable
 import torch
 import torch.nn.functional as F
 
-from fused_oracle import rms_norm, rotate_pairs
+from fused_oracle import per_head_rms_norm, rms_norm, rotate_pairs
 
 Tensor = torch.Tensor
 
@@ -150,6 +150,14 @@ class InstructionVM:
             stop = min((row // d + 1) * d, end)
             seg = "q" if row < k_start else ("k" if row < v_start else "v")
             out = _tile_gemv(g.qkv_weights[layer], y, row, stop, 0, s.hidden_size)
+            if getattr(s, "qk_norm", False):
+                # Qwen3 op set (qwen3__0_6b/…/instructions/python_vm.py:110-141): the raw vector only;
+                # norm, RoPE and the cache write belong to the attention instruction.
+                g.qkv_raw[row:stop] = out.to(g.qkv_raw.dtype)
+                for blk in range(row // tile, (stop + tile - 1) // tile):
+                    g.barriers[layer, ROW_QKV, blk // blocks_per_head] += 1
+                row = stop
+                continue
             if seg != "v":
                 head = torch.zeros(1, d, dtype=out.dtype)
                 a = row % d
@@ -197,6 +205,19 @@ class InstructionVM:
         t0, t1 = b0 * block, min(b1 * block, seq_len)
 
         h0, h1 = ins.kv_head_idx * ratio, (ins.kv_head_idx + 1) * ratio
+        if getattr(s, "qk_norm", False):
+            # Qwen3 op set (qwen3__0_6b/…/instructions/python_vm.py:214-320): q and k of this KV head
+            # get their per-head RMSNorm and RoPE here; K/V of this position enter the cache.  Every
+            # partial computes the same values, so the sequential VM simply writes them each time.
+            pos = int(g.position_id or 0)
+            raw = g.qkv_raw
+            k_off, v_off = nq * d + ins.kv_head_idx * d, (nq + nkv) * d + ins.kv_head_idx * d
+            cos, sin = g.rope_cos[pos].unsqueeze(0), g.rope_sin[pos].unsqueeze(0)
+            qn = per_head_rms_norm(raw[h0 * d : h1 * d].view(ratio, d), g.q_norm_weights[ins.layer_idx], s.rms_norm_eps)
+            kn = per_head_rms_norm(raw[k_off : k_off + d].view(1, d), g.k_norm_weights[ins.layer_idx], s.rms_norm_eps)
+            g.q_post_rope.view(nq, d)[h0:h1] = ((qn * cos) + (rotate_pairs(qn) * sin)).to(g.q_post_rope.dtype)
+            g.k_cache[ins.layer_idx, 0, pos, ins.kv_head_idx] = ((kn * cos) + (rotate_pairs(kn) * sin)).view(-1).to(g.k_cache.dtype)
+            g.v_cache[ins.layer_idx, 0, pos, ins.kv_head_idx] = raw[v_off : v_off + d].to(g.v_cache.dtype)
         q = g.q_post_rope.view(nq, -1)[h0:h1].float()
         k = g.k_cache[ins.layer_idx, 0, t0:t1, ins.kv_head_idx].float()
         v = g.v_cache[ins.layer_idx, 0, t0:t1, ins.kv_head_idx].float()

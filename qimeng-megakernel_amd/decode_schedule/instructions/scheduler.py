@@ -278,6 +278,11 @@ def mi355x_scheduler(
 ) -> DecodeScheduler:
     shape = shape or LlamaConfig.shape()
     geometry = dataclasses.replace(MI355X_GEOMETRY, split_k=shape.intermediate_size)
+    # Up/gate blocks are dealt round-robin: halve the block when that is what makes every
+    # workgroup get the same number of them (intermediate 6144: 384 blocks of 16, 768 of 8).
+    blocks = shape.intermediate_size // geometry.upgate_tile_n
+    if blocks % sm_count != 0 and (2 * blocks) % sm_count == 0:
+        geometry = dataclasses.replace(geometry, upgate_tile_n=geometry.upgate_tile_n // 2)
     p = num_partials or pick_num_partials(sm_count, kv_capacity, shape=shape)
     return DecodeScheduler(shape, geometry, sm_count, p, attention_merge)
 

@@ -33,6 +33,7 @@ QMK_FLAG_XCD_COUNTERS = 2
 QMK_FLAG_TAGGED = 4
 QMK_XCD_COUNTER_ROWS = 54
 QMK_MODEL_LLAMA_3_2_1B = 0
+QMK_MODEL_QWEN3_1_7B = 1
 QMK_QUERY_ABI_VERSION, QMK_QUERY_CU_COUNT, QMK_QUERY_THREADS, QMK_QUERY_LDS_BYTES = 0, 1, 2, 3
 QMK_QUERY_MAX_QUEUES, QMK_QUERY_INSTRUCTION_WORDS, QMK_QUERY_MAX_PARTIALS = 4, 5, 6
 
@@ -88,6 +89,28 @@ _TENSOR_ARGS: tuple[tuple[str, torch.dtype, int], ...] = (
     ("lm_head_weights", torch.bfloat16, 2),
     ("barriers", torch.int32, 3),
 )
+
+
+# The Qwen3 op set's mk(...) takes three tensors more, in the reference's positional order
+# (`…/qwen/qwen3__0_6b/A100/single_batch/decode_schedule/mk_kernel.py:84-110`): qkv_raw after
+# hidden_states, the two per-head norm weights after qkv_weights.
+_QWEN3_TENSOR_ARGS: tuple[tuple[str, torch.dtype, int], ...] = (
+    _TENSOR_ARGS[:2] + (("qkv_raw", torch.bfloat16, 1),) + _TENSOR_ARGS[2:12]
+    + (("q_norm_weights", torch.bfloat16, 2), ("k_norm_weights", torch.bfloat16, 2)) + _TENSOR_ARGS[12:]
+)
+
+
+def _model_id(shape: Any) -> int:
+    """The compiled kernel instantiation for ``shape`` (layer count and vocabulary are run-time values)."""
+    key = (shape.hidden_size, shape.intermediate_size, shape.head_dim, shape.num_attention_heads,
+           shape.num_key_value_heads, bool(getattr(shape, "qk_norm", False)))
+    table = {
+        (2048, 8192, 64, 32, 8, False): QMK_MODEL_LLAMA_3_2_1B,
+        (2048, 6144, 128, 16, 8, True): QMK_MODEL_QWEN3_1_7B,
+    }
+    if key not in table:
+        raise ValueError(f"no kernel was compiled for the layer geometry {key}")
+    return table[key]
 
 
 def _default_mk_dir() -> Path:
@@ -213,7 +236,13 @@ class MegaKernel:
     def _bind(self, tensors: Sequence[torch.Tensor]) -> None:
         a = self._args
         device = tensors[1].device
-        for (name, dtype, ndim), t in zip(_TENSOR_ARGS, tensors):
+        shape = LlamaConfig.shape()
+        a.model = _model_id(shape)
+        qwen = a.model == QMK_MODEL_QWEN3_1_7B
+        if len(tensors) != (25 if qwen else 22):
+            raise TypeError(f"mk for this model takes {25 if qwen else 22} tensors, got {len(tensors)}")
+        spec = _QWEN3_TENSOR_ARGS if qwen else _TENSOR_ARGS
+        for (name, dtype, ndim), t in zip(spec, tensors):
             if not isinstance(t, torch.Tensor):
                 raise TypeError(f"{name} must be a torch.Tensor, got {type(t).__name__}")
             if t.device.type != "cuda":
@@ -227,9 +256,13 @@ class MegaKernel:
             if not t.is_contiguous():
                 raise ValueError(f"{name} must be contiguous")
             setattr(a, name, t.data_ptr())
+        if qwen:
+            expect_raw, expect_qn, expect_kn = tensors[2], tensors[13], tensors[14]
+            tensors = tuple(tensors[:2]) + tuple(tensors[3:13]) + tuple(tensors[15:])
+        else:
+            a.qkv_raw = a.q_norm_weights = a.k_norm_weights = None
         (instructions, hidden, _q, k_cache, v_cache, _ao, lse, part, silu, logits, attn_norm, qkv, cos, sin, o_w,
          mlp_norm, up, gate, down, lm_norm, lm_w, barriers) = tensors
-        shape = LlamaConfig.shape()
         L = int(barriers.shape[0])
         H, F = shape.hidden_size, shape.intermediate_size
 
@@ -240,6 +273,10 @@ class MegaKernel:
         if instructions.shape[2] != 32:
             raise ValueError("instructions must be [queues, length, 32]")
         expect("hidden_states", hidden, (H,))
+        if qwen:
+            expect("qkv_raw", expect_raw, (shape.qkv_out_dim,))
+            expect("q_norm_weights", expect_qn, (L, shape.head_dim))
+            expect("k_norm_weights", expect_kn, (L, shape.head_dim))
         expect("q_post_rope", tensors[2], (shape.num_attention_heads * shape.head_dim,))
         expect("attn_out", tensors[5], (shape.num_attention_heads * shape.head_dim,))
         expect("silu_out", silu, (F,))
@@ -277,7 +314,7 @@ class MegaKernel:
         )
         self._tagged = self.tagged and self.reset_barriers and geometry.num_split_k(shape) == 1 and L <= 63
         if self._tagged or self.reset_barriers:   # the workspace also carries the greedy candidates
-            nbytes = int(self._lib.qmk_workspace_bytes(QMK_MODEL_LLAMA_3_2_1B))
+            nbytes = int(self._lib.qmk_workspace_bytes(int(a.model)))
             if self._workspace is None or self._workspace.device != device:
                 self._workspace = torch.zeros(nbytes, dtype=torch.uint8, device=device)
             else:
@@ -289,9 +326,9 @@ class MegaKernel:
             a.workspace, a.workspace_bytes = None, 0
 
     def __call__(self, *args: Any) -> None:
-        if len(args) != 25:
-            raise TypeError(f"mk takes 22 tensors and 3 scalars (25 positional arguments), got {len(args)}")
-        tensors, (pos_id, attn_scale, rms_norm_eps) = args[:22], args[22:]
+        if len(args) not in (25, 28):
+            raise TypeError(f"mk takes 22 (Qwen3 op set: 25) tensors and 3 scalars, got {len(args)} positional arguments")
+        tensors, (pos_id, attn_scale, rms_norm_eps) = args[:-3], args[-3:]
         if isinstance(tensors[0], torch.Tensor) and tensors[0].numel() == 0:
             return  # empty queues: nothing to launch
         key = tuple((t.data_ptr(), tuple(t.shape)) if isinstance(t, torch.Tensor) else None for t in tensors) + (
@@ -348,9 +385,11 @@ def call_mk(globs: Globals, mk: Any) -> None:
     shape = LlamaConfig.shape()
     if globs.instructions is None:
         _scheduler.build(globs)
+    qwen = bool(getattr(shape, "qk_norm", False))
     mk(
         globs.instructions,
         globs.hidden_states,
+        *((globs.qkv_raw,) if qwen else ()),
         globs.q_post_rope,
         _tensor_for_mk(globs.k_cache),
         _tensor_for_mk(globs.v_cache),
@@ -361,6 +400,7 @@ def call_mk(globs: Globals, mk: Any) -> None:
         globs.logits,
         globs.attn_norm_weights,
         globs.qkv_weights,
+        *((_tensor_for_mk(globs.q_norm_weights), _tensor_for_mk(globs.k_norm_weights)) if qwen else ()),
         globs.rope_cos,
         globs.rope_sin,
         globs.o_proj_weights,

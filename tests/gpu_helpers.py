@@ -16,8 +16,9 @@ MUTABLE = ("hidden_states", "q_post_rope", "attn_out", "silu_out", "logits", "k_
 
 def sync_state(src, dst) -> None:
     """Copy every mutable buffer of ``src`` onto ``dst`` (across devices)."""
-    for name in MUTABLE:
-        getattr(dst, name).copy_(getattr(src, name))
+    for name in MUTABLE + ("qkv_raw",):
+        if getattr(src, name, None) is not None:
+            getattr(dst, name).copy_(getattr(src, name))
     dst.position_id = src.position_id
 
 
