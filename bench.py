@@ -79,6 +79,9 @@ def main() -> None:
     ap.add_argument("--prompt-len", type=int, default=8)
     ap.add_argument("--cpu-steps", type=int, default=10)
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--model", choices=("llama-3.2-1b", "qwen3-1.7b"), default="llama-3.2-1b",
+                    help="layer geometry: the headline Llama-3.2-1B shape, or the Qwen3-1.7B shape with the Qwen3 op set "
+                         "(28 layers, per-head QK RMSNorm, tied LM head)")
     ap.add_argument("--host-sampling", action="store_true",
                     help="argmax and embedding lookup on the host between launches, as the reference's loop does "
                          "(default: inside the kernel)")
@@ -101,9 +104,10 @@ def main() -> None:
     load_package()
     from qimeng_megakernel_amd import decode, synthetic
     from qimeng_megakernel_amd.decode_schedule import mk_kernel
-    from qimeng_megakernel_amd.decode_schedule.model_config import LLAMA_3_2_1B, LlamaConfig
+    from qimeng_megakernel_amd.decode_schedule.model_config import LLAMA_3_2_1B, QWEN3_1_7B, LlamaConfig
 
-    shape = LLAMA_3_2_1B
+    shape = LLAMA_3_2_1B if args.model == "llama-3.2-1b" else QWEN3_1_7B
+    model_name = "Llama-3.2-1B" if args.model == "llama-3.2-1b" else "Qwen3-1.7B"
     LlamaConfig.set_shape(shape)
     device = torch.device("cuda:0")
     torch.cuda.set_device(device)
@@ -139,7 +143,7 @@ def main() -> None:
 
     golden = ROOT / "tests" / "golden" / "llama1b_seed0.json"
     match = None
-    if args.seed == 0 and args.prompt_len == 8 and golden.is_file():
+    if args.model == "llama-3.2-1b" and args.seed == 0 and args.prompt_len == 8 and golden.is_file():
         want = json.loads(golden.read_text())["tokens"]
         n = min(len(want), len(tokens))
         match = next((i for i in range(n) if tokens[i] != want[i]), n)
@@ -160,7 +164,7 @@ def main() -> None:
         "dtype": "bf16",
         "data": "synthetic",
         "config": {
-            "workload": f"Llama-3.2-1B-shaped batch-1 greedy decode, {args.prompt_len}-token prompt, "
+            "workload": f"{model_name}-shaped batch-1 greedy decode, {args.prompt_len}-token prompt, "
                         f"{new_tokens} new tokens (context {ctx_first}..{ctx_last}), seeded random-init bf16 weights",
             "layers": shape.num_hidden_layers, "hidden": shape.hidden_size, "ffn": shape.intermediate_size,
             "q_heads": shape.num_attention_heads, "kv_heads": shape.num_key_value_heads, "head_dim": shape.head_dim,
@@ -181,7 +185,7 @@ def main() -> None:
             "frac": achieved / HBM_PEAK_GBPS,
             "traffic": MEASURED_TRAFFIC_OVER_ALGORITHMIC * t["algorithmic_bytes"] / max(args.steps, 1),
             "bytes_per_launch_avg": t["algorithmic_bytes"] / max(args.steps, 1),
-            "kernel": "decode_megakernel<Llama1B>",
+            "kernel": "decode_megakernel<Llama1B>" if args.model == "llama-3.2-1b" else "decode_megakernel<Qwen3_1p7B>",
         },
     }
     if not args.no_cpu_baseline:
