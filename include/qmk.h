@@ -73,9 +73,9 @@ enum {
 #define QMK_XCD_COUNTER_ROWS 54
 
 /* Flags. */
-#define QMK_FLAG_TAGGED 4u         /* the small vectors that every workgroup hands to others inside a
+#define QMK_FLAG_TAGGED 4u         /* the vectors that every workgroup hands to others inside a
                                       launch (q and the appended K/V row, the residual stream after
-                                      the O-proj and after the down projection) also travel through
+                                      the O-proj and after the down projection, silu_out) also travel through
                                       `workspace` as 8-byte units {32-bit payload, 32-bit tag}, the
                                       tag naming launch and layer.  A consumer polls the units it
                                       needs until they carry the tag it expects, and the producer
@@ -85,7 +85,8 @@ enum {
                                       a schedule whose down projection is not split along K; not
                                       combinable with QMK_FLAG_KEEP_BARRIERS.  The caller's buffers
                                       receive the same values as without the flag; counter rows 0,
-                                      3 and 5 stay zero.                                          */
+                                      3, 4 and 5 stay zero.  (The split-KV partials stay on
+                                      counters.)                                                  */
 #define QMK_FLAG_KEEP_BARRIERS 1u  /* leave the final counter values in `barriers`
                                       (the reference's behaviour); by default the
                                       last workgroup to retire clears them so the

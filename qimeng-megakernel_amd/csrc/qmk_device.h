@@ -219,15 +219,18 @@ __device__ __forceinline__ v4u ld_shared128(const void* p) {
 // names the launch (a count kept in the workspace) and the layer.  The consumer polls the units
 // it needs until they carry the tag it expects: one trip.  A unit is never overwritten before
 // all its readers are done: its next writer depends, through the layer's data flow, on every one
-// of them.  Only the small vectors travel this way (every thread of every workgroup re-reading a
-// large one while it waits would flood the fabric).  Offsets below are in units of 8 bytes.
+// of them.  The split-KV partials do not travel this way: 256 workgroups re-reading 40-200 KiB
+// each while they wait for the attention phase floods the fabric; for silu_out (16 KiB) the
+// waiting time is short, and not waiting for store acknowledgements behind the next GEMV's row
+// requests is worth more than the polling costs.  Offsets below are in units of 8 bytes.
 constexpr int kWsGeneration = 0;            // launch count (first 128-byte line)
 constexpr int kWsQ = 512;                   // q after RoPE: NQ*D/2 units (two bf16 each)
 constexpr int kWsK = kWsQ + 1024;           // appended K row: NKV*D/2 units
 constexpr int kWsV = kWsK + 512;            // appended V row (regions sized for 8 KV heads of 128)
 constexpr int kWsHiddenMid = kWsV + 512;    // residual stream after the O-proj: H/2 units
 constexpr int kWsHiddenOut = kWsHiddenMid + 1024;  // residual stream after the down projection
-constexpr int kWsCandidates = kWsHiddenOut + 1024;  // one greedy candidate per workgroup: {logit bits, row}
+constexpr int kWsSilu = kWsHiddenOut + 1024;        // silu_out: F/2 units (room for F = 8192)
+constexpr int kWsCandidates = kWsSilu + 4096;       // one greedy candidate per workgroup: {logit bits, row}
 constexpr int kMaxSamplingQueues = 1024;
 constexpr int kWsUnits = kWsCandidates + kMaxSamplingQueues;
 

@@ -917,7 +917,9 @@ __device__ bool op_rms_upgate_silu(const Params& p, Smem<M>& s, const Ctx& c) {
       word |= static_cast<uint32_t>(f2bf(act * up)) << (16 * k);
     }
     st_shared32(p.silu_out + row_of(2 * pair), word);
+    if (tg) st_tagged(p.ws + kWsSilu + row_of(2 * pair) / 2, word, tag_of(s.generation, layer));
   }
+  if (tg) return true;  // the down projection polls the units
 
   release_stores();
   __syncthreads();
@@ -990,6 +992,51 @@ __device__ bool op_down_residual(const Params& p, Smem<M>& s, const Ctx& c) {
     s.ctl[0] = 1;  // seen by everybody after the barrier inside the wait below
     report_error(p, QMK_DEV_WAIT_TIMEOUT, c.inst_idx, c.opcode, threadIdx.x);
   }
+  if (tg) {
+    // silu_out from its tagged units: thread t polls the unit pairs 2t + 1024k until they carry
+    // this layer's tag; pairs already staged are not fetched again.
+    static_assert(M::F % (4 * kThreads) == 0, "whole unit pairs per thread");
+    constexpr int kPairs = M::F / (4 * kThreads);
+    uint32_t* words = reinterpret_cast<uint32_t*>(s.x);
+    const uint64_t* mine = p.ws + kWsSilu + 2 * threadIdx.x;
+    uint32_t polls = 0;
+    bool have[kPairs];
+#pragma unroll
+    for (int k = 0; k < kPairs; ++k) have[k] = false;
+    while (true) {
+      uint64_t u[2 * kPairs];
+#pragma unroll
+      for (int k = 0; k < kPairs; ++k) {
+        if (!have[k]) {
+          u[2 * k] = ld_shared64(mine + 1024 * k);
+          u[2 * k + 1] = ld_shared64(mine + 1024 * k + 1);
+        }
+      }
+      bool all = true;
+#pragma unroll
+      for (int k = 0; k < kPairs; ++k) {
+        if (!have[k] && static_cast<uint32_t>(u[2 * k] >> 32) == tag && static_cast<uint32_t>(u[2 * k + 1] >> 32) == tag) {
+          words[2 * threadIdx.x + 1024 * k] = static_cast<uint32_t>(u[2 * k]);
+          words[2 * threadIdx.x + 1024 * k + 1] = static_cast<uint32_t>(u[2 * k + 1]);
+          have[k] = true;
+        }
+        all = all && have[k];
+      }
+      if (all) break;
+      if (++polls > p.spin_limit) {
+        s.ctl[0] = 1;
+        report_error(p, QMK_DEV_WAIT_TIMEOUT, c.inst_idx, c.opcode, threadIdx.x);
+        break;
+      }
+      __builtin_amdgcn_s_sleep(8);
+    }
+    if (p.timeline != nullptr && threadIdx.x == 0) {
+      s.t_wait = wall_clock64();
+      s.ctl[2] = 1;
+    }
+    __syncthreads();
+    if (s.ctl[0]) return false;
+  } else {
   if (!wg_wait_all(p, s, c, layer, ROW_UPGATE, split, p.upgate_blocks_per_bucket)) return false;
 
   // The K slice of silu_out into LDS; the remaining row buffers are requested behind it.
@@ -1004,6 +1051,7 @@ __device__ bool op_down_residual(const Params& p, Smem<M>& s, const Ctx& c) {
   for (int k = 0; k < kActLoads; ++k)
     if (static_cast<int>(threadIdx.x) + k * kThreads < kg / 4) reinterpret_cast<uint64_t*>(s.x)[threadIdx.x + k * kThreads] = act[k];
   __syncthreads();
+  }
 
   float acc = 0.f;
   stream<CH>(rows_w > 0 ? n_elems : 0, src, buf, [&](int e, const RowRegs<CH>& w) {

@@ -74,7 +74,7 @@ def test_host_side_argument_errors(lib):
     assert lib.qmk_decode_step(ctypes.byref(a)) == 8                       # QMK_ERR_MODEL
     a.model = 0
     assert lib.qmk_decode_step(ctypes.byref(a)) == 1                       # all tensor pointers are NULL
-    assert lib.qmk_workspace_bytes(0) == 8 * (4096 + 512 + 1024) and lib.qmk_workspace_bytes(1) == lib.qmk_workspace_bytes(0) and lib.qmk_workspace_bytes(7) == 0
+    assert lib.qmk_workspace_bytes(0) == 8 * (4096 + 512 + 4096 + 1024) and lib.qmk_workspace_bytes(1) == lib.qmk_workspace_bytes(0) and lib.qmk_workspace_bytes(7) == 0
     assert lib.qmk_query(0) == 4 and lib.qmk_query(2) == 512 and lib.qmk_query(5) == 32 and lib.qmk_query(6) == 25
     assert 0 < lib.qmk_query(3) <= 160 * 1024
     assert lib.qmk_error_string(34).decode().startswith("device: counter wait")
@@ -102,7 +102,7 @@ def test_mk_rejects_cpu_tensors_and_bad_dtypes(lib, small_model):
     mk = mk_kernel.get_mk()
     with pytest.raises(ValueError, match="must live on the GPU"):
         mk_kernel.call_mk(g, mk)
-    with pytest.raises(TypeError, match="25 positional"):
+    with pytest.raises(TypeError, match="3 scalars, got 1 positional"):
         mk(g.instructions)
     g.hidden_states = g.hidden_states.float()
     with pytest.raises((TypeError, ValueError)):
