@@ -583,23 +583,34 @@ __device__ bool op_attn_splitkv(const Params& p, Smem<M>& s, const Ctx& c) {
         }
       }
     }
-    float k[DPL], v[DPL];
+    // scores of all heads first (K live), then the accumulator updates (V live)
+    float sc[GQA];
+    {
+      float k[DPL];
+#pragma unroll
+      for (int j = 0; j < VPL; ++j) {
+        k[8 * j + 0] = bf_lo(kv[j].x); k[8 * j + 1] = bf_hi(kv[j].x); k[8 * j + 2] = bf_lo(kv[j].y); k[8 * j + 3] = bf_hi(kv[j].y);
+        k[8 * j + 4] = bf_lo(kv[j].z); k[8 * j + 5] = bf_hi(kv[j].z); k[8 * j + 6] = bf_lo(kv[j].w); k[8 * j + 7] = bf_hi(kv[j].w);
+      }
+#pragma unroll
+      for (int h = 0; h < GQA; ++h) {
+        float a = 0.f;
+#pragma unroll
+        for (int i = 0; i < DPL; ++i) a = __builtin_fmaf(q[h][i], k[i], a);
+        sc[h] = group8_sum(a);  // the 8 lanes of a group always take the same branch
+      }
+    }
+    float v[DPL];
 #pragma unroll
     for (int j = 0; j < VPL; ++j) {
-      k[8 * j + 0] = bf_lo(kv[j].x); k[8 * j + 1] = bf_hi(kv[j].x); k[8 * j + 2] = bf_lo(kv[j].y); k[8 * j + 3] = bf_hi(kv[j].y);
-      k[8 * j + 4] = bf_lo(kv[j].z); k[8 * j + 5] = bf_hi(kv[j].z); k[8 * j + 6] = bf_lo(kv[j].w); k[8 * j + 7] = bf_hi(kv[j].w);
       v[8 * j + 0] = bf_lo(vv[j].x); v[8 * j + 1] = bf_hi(vv[j].x); v[8 * j + 2] = bf_lo(vv[j].y); v[8 * j + 3] = bf_hi(vv[j].y);
       v[8 * j + 4] = bf_lo(vv[j].z); v[8 * j + 5] = bf_hi(vv[j].z); v[8 * j + 6] = bf_lo(vv[j].w); v[8 * j + 7] = bf_hi(vv[j].w);
     }
 #pragma unroll
     for (int h = 0; h < GQA; ++h) {
-      float sc = 0.f;
-#pragma unroll
-      for (int i = 0; i < DPL; ++i) sc = __builtin_fmaf(q[h][i], k[i], sc);
-      sc = group8_sum(sc);  // the 8 lanes of a group always take the same branch
-      const float mn = fmaxf(m[h], sc);
+      const float mn = fmaxf(m[h], sc[h]);
       const float alpha = exp2_fast(m[h] - mn);   // 0 on the first token (m = -inf)
-      const float pr = exp2_fast(sc - mn);
+      const float pr = exp2_fast(sc[h] - mn);
       l[h] = __builtin_fmaf(l[h], alpha, pr);
 #pragma unroll
       for (int i = 0; i < DPL; ++i) acc[h][i] = __builtin_fmaf(acc[h][i], alpha, pr * v[i]);
