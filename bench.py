@@ -38,7 +38,7 @@ HBM_PEAK_GBPS = 8000.0
 MEASURED_TRAFFIC_OVER_ALGORITHMIC = 1.0050
 
 
-def cpu_baseline(shape, weights, prompt, n_steps: int, cores: int) -> dict:
+def cpu_baseline(shape, weights, prompt, n_steps: int, cores: int, shape_name: str) -> dict:
     """Time the CPU oracle on single-token steps of the same request (bounded sample)."""
     import torch
 
@@ -64,8 +64,8 @@ def cpu_baseline(shape, weights, prompt, n_steps: int, cores: int) -> dict:
         "unit": "tok/s",
         "cores": cores,
         "kind": "port",
-        "sample": f"{n_steps} single-token decode steps (positions 0..{n_steps - 1}: the 8-token prompt through the "
-                  f"single-token path, then greedy steps) of the same seeded Llama-3.2-1B-shaped request, "
+        "sample": f"{n_steps} single-token decode steps (positions 0..{n_steps - 1}: the {prompt.numel()}-token prompt through "
+                  f"the single-token path, then greedy steps) of the same seeded {shape_name}-shaped request, "
                   f"torch {torch.__version__} bf16 on {cores} threads, {dt:.1f} s",
     }
 
@@ -183,14 +183,16 @@ def main() -> None:
             "peak": HBM_PEAK_GBPS,
             "unit": "GB/s",
             "frac": achieved / HBM_PEAK_GBPS,
-            "traffic": MEASURED_TRAFFIC_OVER_ALGORITHMIC * t["algorithmic_bytes"] / max(args.steps, 1),
+            # the counter runs were made on the Llama-shaped kernel only
+            "traffic": (MEASURED_TRAFFIC_OVER_ALGORITHMIC * t["algorithmic_bytes"] / max(args.steps, 1)
+                        if args.model == "llama-3.2-1b" else None),
             "bytes_per_launch_avg": t["algorithmic_bytes"] / max(args.steps, 1),
             "kernel": "decode_megakernel<Llama1B>" if args.model == "llama-3.2-1b" else "decode_megakernel<Qwen3_1p7B>",
         },
     }
     if not args.no_cpu_baseline:
         cores = min(os.cpu_count() or 1, 16)
-        line["cpu_baseline"] = cpu_baseline(shape, weights, prompt, args.cpu_steps, cores)
+        line["cpu_baseline"] = cpu_baseline(shape, weights, prompt, args.cpu_steps, cores, model_name)
     print(json.dumps(line))
 
 
