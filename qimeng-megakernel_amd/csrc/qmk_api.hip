@@ -40,7 +40,9 @@ __global__ __launch_bounds__(kThreads, 1) void decode_megakernel(const Params p)
     if (threadIdx.x < kInstWords) s.inst[threadIdx.x] = queue[i * kInstWords + threadIdx.x];
     __syncthreads();
     const int opcode = s.inst[0];
-    const Ctx c{i, opcode};
+    int tid = threadIdx.x;
+    asm volatile("" : "+v"(tid));
+    const Ctx c{i, opcode, tid};
     unsigned long long t_start = 0;
     if (p.timeline != nullptr && threadIdx.x == 0) {
       t_start = wall_clock64();

@@ -6,9 +6,20 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
+#include <type_traits>
+
 #include "qmk.h"
 
 namespace qmk {
+
+// f(integral_constant<I>), ..., f(integral_constant<N-1>): an unrolled loop whose index is a constant.
+template <int I, int N, class F>
+__device__ __forceinline__ void static_for(F&& f) {
+  if constexpr (I < N) {
+    f(std::integral_constant<int, I>{});
+    static_for<I + 1, N>(f);
+  }
+}
 
 constexpr int kThreads = 512;            // one workgroup per CU, 8 waves, 2 per SIMD
 constexpr int kWaveSize = 64;

@@ -11,6 +11,13 @@
 
 #include "qmk_device.h"
 
+#ifndef QMK_KV_AHEAD_LLAMA
+#define QMK_KV_AHEAD_LLAMA 1
+#endif
+#ifndef QMK_KV_AHEAD_QWEN
+#define QMK_KV_AHEAD_QWEN 1
+#endif
+
 namespace qmk {
 
 struct Llama1B {
@@ -22,6 +29,7 @@ struct Llama1B {
   static constexpr int GQA = NQ / NKV;
   static constexpr int QKV = (NQ + 2 * NKV) * D;
   static constexpr int KV_BLOCK = 16;  // split-KV partition granularity in tokens
+  static constexpr int KV_AHEAD = QMK_KV_AHEAD_LLAMA;  // cache rows a lane group asks for before it has q
   static constexpr bool QK_NORM = false;
 };
 
@@ -37,6 +45,7 @@ struct Qwen3_1p7B {
   static constexpr int GQA = NQ / NKV;
   static constexpr int QKV = (NQ + 2 * NKV) * D;
   static constexpr int KV_BLOCK = 16;
+  static constexpr int KV_AHEAD = QMK_KV_AHEAD_QWEN;
   static constexpr bool QK_NORM = true;
 };
 
@@ -75,17 +84,19 @@ constexpr int ROW_QKV = 0, ROW_SPLITKV = 1, ROW_REDUCE = 2, ROW_OPROJ = 3, ROW_U
 struct Ctx {
   int inst_idx;
   int opcode;
+  int tid;  // c.tid through an opaque copy made per instruction: what an op derives from it
+            // stays inside that op instead of being computed once for all ops and kept in registers
 };
 
 // Optional intermediate timestamp k (0..3) of the running instruction, thread 0 only.
 #define QMK_STAMP(k)                                                        \
   do {                                                                      \
-    if (p.timeline != nullptr && threadIdx.x == 0) s.stamps[k] = wall_clock64(); \
+    if (p.timeline != nullptr && c.tid == 0) s.stamps[k] = wall_clock64(); \
   } while (0)
 
 template <class M>
 __device__ __forceinline__ bool bad_operand(const Params& p, Smem<M>& s, const Ctx& c, int operand) {
-  if (threadIdx.x == 0) report_error(p, QMK_DEV_BAD_OPERAND, c.inst_idx, c.opcode, operand);
+  if (c.tid == 0) report_error(p, QMK_DEV_BAD_OPERAND, c.inst_idx, c.opcode, operand);
   return false;
 }
 
@@ -93,13 +104,13 @@ __device__ __forceinline__ bool bad_operand(const Params& p, Smem<M>& s, const C
 // every thread has acquired.  False (uniformly) when a poll ran out of budget.
 template <class M, class CtrOf>
 __device__ __forceinline__ bool wg_wait(const Params& p, Smem<M>& s, const Ctx& c, int n, CtrOf ctr_of, int expected) {
-  if (threadIdx.x < n) {
-    if (!poll_counter(ctr_of(threadIdx.x), expected, p.spin_limit)) {
+  if (c.tid < n) {
+    if (!poll_counter(ctr_of(c.tid), expected, p.spin_limit)) {
       s.ctl[0] = 1;
-      report_error(p, QMK_DEV_WAIT_TIMEOUT, c.inst_idx, c.opcode, threadIdx.x);
+      report_error(p, QMK_DEV_WAIT_TIMEOUT, c.inst_idx, c.opcode, c.tid);
     }
   }
-  if (p.timeline != nullptr && threadIdx.x == 0) {
+  if (p.timeline != nullptr && c.tid == 0) {
     s.t_wait = wall_clock64();
     s.ctl[2] = 1;
   }
@@ -115,13 +126,13 @@ template <class M>
 __device__ __forceinline__ bool wg_wait_all(const Params& p, Smem<M>& s, const Ctx& c, int layer, int row, int slot, int expected) {
   if (!xcd_counters(p))
     return wg_wait(p, s, c, 1, [&](int) { return counter_ptr(p, layer, row, slot); }, expected);
-  if (threadIdx.x < kXcds) {
-    if (!wait_edge_xcd(p, layer, row, expected, p.spin_limit) && threadIdx.x == 0) {
+  if (c.tid < kXcds) {
+    if (!wait_edge_xcd(p, layer, row, expected, p.spin_limit) && c.tid == 0) {
       s.ctl[0] = 1;
       report_error(p, QMK_DEV_WAIT_TIMEOUT, c.inst_idx, c.opcode, row);
     }
   }
-  if (p.timeline != nullptr && threadIdx.x == 0) {
+  if (p.timeline != nullptr && c.tid == 0) {
     s.t_wait = wall_clock64();
     s.ctl[2] = 1;
   }
@@ -135,35 +146,58 @@ __device__ __forceinline__ bool wg_wait_all(const Params& p, Smem<M>& s, const C
 // The residual stream comes from the caller's buffer (units == nullptr: a counter wait has made
 // it complete) or from its tagged copy, each thread polling its own two units.  False
 // (uniformly) when a tagged poll ran out of budget.
-template <class M, class AfterIssue>
+// `pace(k)`, k = 0..NP-1, issues the op's k-th group of weight-row requests.  With a tagged
+// residual stream they go out one group per look at the units: loads return in issue order, so a
+// look that stands behind all NP groups learns of the hand-over only when the last of them has
+// landed, while behind one group it costs one round trip and the rows still arrive in the
+// meantime.  Whatever has not been asked for when the units are complete goes out then.
+template <class M, int NP, class Pace, class Wait>
 __device__ __forceinline__ bool rms_to_lds(const Params& p, Smem<M>& s, const Ctx& c, const uint64_t* units, uint32_t tag,
-                                           const u16* weight, AfterIssue after_issue) {
+                                           const u16* weight, Pace pace, Wait wait) {
   static_assert(M::H == kThreads * 4, "one thread normalises four elements");
-  const int t = threadIdx.x;
-  uint32_t hlo, hhi;
+  const int t = c.tid;
+  uint32_t hlo = 0, hhi = 0;
+  // Asked for first: the norm weights are then in registers when the residual stream arrives,
+  // instead of costing a round trip of their own behind it.
+  const uint2 wv = *reinterpret_cast<const uint2*>(weight + t * 4);
+  const uint64_t* mine = units + 2 * t;
+  bool done = units == nullptr;
+  auto look = [&] {
+    const uint64_t x = ld_shared64(mine), y = ld_shared64(mine + 1);
+    hlo = static_cast<uint32_t>(x);
+    hhi = static_cast<uint32_t>(y);
+    const bool ok = static_cast<uint32_t>(x >> 32) == tag && static_cast<uint32_t>(y >> 32) == tag;
+    done = __builtin_amdgcn_ballot_w64(ok) == ~0ull;  // the wave moves on together: row requests are wave-wide
+  };
+  static_for<0, NP>([&](auto kk) {
+    pace(kk);
+    if (!done) look();
+  });
   if (units == nullptr) {
+    if (!wait()) return false;  // counters: the caller's wait, behind all row requests
     const uint64_t hw = ld_shared64(p.hidden + t * 4);
-    asm volatile("" ::: "memory");
-    after_issue();  // further loads queue up behind the residual stream, not in front of it
     hlo = static_cast<uint32_t>(hw);
     hhi = static_cast<uint32_t>(hw >> 32);
   } else {
-    if (!poll_tagged2(units + 2 * t, tag, p.spin_limit, hlo, hhi)) {
-      s.ctl[0] = 1;
-      report_error(p, QMK_DEV_WAIT_TIMEOUT, c.inst_idx, c.opcode, t);
+    for (uint32_t polls = 0; !done; ++polls) {
+      if (polls > p.spin_limit) {
+        s.ctl[0] = 1;
+        report_error(p, QMK_DEV_WAIT_TIMEOUT, c.inst_idx, c.opcode, t);
+        break;
+      }
+      if (polls) __builtin_amdgcn_s_sleep(1);
+      look();
     }
     if (p.timeline != nullptr && t == 0) {
       s.t_wait = wall_clock64();
       s.ctl[2] = 1;
     }
-    after_issue();
   }
   const float x0 = bf_lo(hlo), x1 = bf_hi(hlo), x2 = bf_lo(hhi), x3 = bf_hi(hhi);
   float ss = __builtin_fmaf(x3, x3, __builtin_fmaf(x2, x2, __builtin_fmaf(x1, x1, x0 * x0)));
   ss = block_sum(ss, s.red);
   const float mean = ss / static_cast<float>(M::H);
   const float rstd = 1.0f / sqrtf(mean + p.rms_norm_eps);
-  const uint2 wv = *reinterpret_cast<const uint2*>(weight + t * 4);
   const u16 y0 = f2bf(bf_lo(wv.x) * round_bf16(x0 * rstd));
   const u16 y1 = f2bf(bf_hi(wv.x) * round_bf16(x1 * rstd));
   const u16 y2 = f2bf(bf_lo(wv.y) * round_bf16(x2 * rstd));
@@ -178,16 +212,19 @@ __device__ __forceinline__ bool rms_to_lds(const Params& p, Smem<M>& s, const Ct
 template <class M>
 __device__ __forceinline__ bool rms_to_lds(const Params& p, Smem<M>& s, const Ctx& c, const uint64_t* units, uint32_t tag,
                                            const u16* weight) {
-  return rms_to_lds(p, s, c, units, tag, weight, [] {});
+  return rms_to_lds<M, 0>(p, s, c, units, tag, weight, [](auto) {}, [] { return true; });
 }
 
 // Interleaved-pair RoPE on bf16-rounded inputs, evaluated in fp32 with a
 // rounding after every multiply and the add, then rounded to bf16
 // (fused/operations.py:134-148, 173-181).
-__device__ __forceinline__ uint32_t rope_pair(float v0, float v1, const float* cosr, const float* sinr, int d) {
-  const float o0 = v0 * cosr[d] + (-v1) * sinr[d];
-  const float o1 = v1 * cosr[d + 1] + v0 * sinr[d + 1];
+__device__ __forceinline__ uint32_t rope_pair(float v0, float v1, float2 cs, float2 sn) {
+  const float o0 = v0 * cs.x + (-v1) * sn.x;
+  const float o1 = v1 * cs.y + v0 * sn.y;
   return static_cast<uint32_t>(f2bf(o0)) | (static_cast<uint32_t>(f2bf(o1)) << 16);
+}
+__device__ __forceinline__ uint32_t rope_pair(float v0, float v1, const float* cosr, const float* sinr, int d) {
+  return rope_pair(v0, v1, *reinterpret_cast<const float2*>(cosr + d), *reinterpret_cast<const float2*>(sinr + d));
 }
 
 // ------------------------------------------------------------ streaming ----
@@ -262,19 +299,29 @@ __device__ bool op_rms_qkv_rope(const Params& p, Smem<M>& s, const Ctx& c) {
   if (nstart < 0 || nend < nstart || static_cast<long>(nend) * tile > M::QKV) return bad_operand(p, s, c, 4);
   if ((nend - nstart) * tile > kResSlots) return bad_operand(p, s, c, 3);
 
-  const int lane = threadIdx.x & 63;
+  const int lane = c.tid & 63;
   const int rs = nstart * tile, nrows = (nend - nstart) * tile;
   const u16* W = p.qkv_w + (static_cast<size_t>(layer) * M::QKV + rs) * M::H;
   auto src = [&](int r) { return W + static_cast<size_t>(r) * M::H; };
 
+  // The RoPE factors of this thread's first output pair are asked for before anything else.
+  const float* cosr = p.rope_cos + static_cast<size_t>(p.pos_id) * M::D;
+  const float* sinr = p.rope_sin + static_cast<size_t>(p.pos_id) * M::D;
+  float2 cs0 = {0.0f, 0.0f}, sn0 = {0.0f, 0.0f};
+  if constexpr (!M::QK_NORM) {
+    const int r0 = rs + 2 * c.tid;
+    if (c.tid < nrows / 2 && r0 < (M::NQ + M::NKV) * M::D) {
+      cs0 = *reinterpret_cast<const float2*>(cosr + r0 % M::D);
+      sn0 = *reinterpret_cast<const float2*>(sinr + r0 % M::D);
+    }
+  }
   RowRegs<CH> buf[kDepth];
-  preload<CH>(nrows, src, buf);  // in flight while the counter is polled
   const bool tg = tagged(p);
   const uint32_t tag = tag_of(s.generation, layer);
-  if (layer > 0 && !tg) {
-    if (!wg_wait_all(p, s, c, layer - 1, ROW_DOWN, 0, p.down_arrivals)) return false;
-  }
-  if (!rms_to_lds(p, s, c, (tg && layer > 0) ? p.ws + kWsHiddenOut : nullptr, tag - 1, p.attn_norm + static_cast<size_t>(layer) * M::H))
+  if (!rms_to_lds<M, kDepth>(
+          p, s, c, (tg && layer > 0) ? p.ws + kWsHiddenOut : nullptr, tag - 1, p.attn_norm + static_cast<size_t>(layer) * M::H,
+          [&](auto k) { preload_range<decltype(k)::value, decltype(k)::value + 1>(nrows, src, buf); },
+          [&] { return layer == 0 || tg || wg_wait_all(p, s, c, layer - 1, ROW_DOWN, 0, p.down_arrivals); }))
     return false;
   QMK_STAMP(0);
   v4u x[CH];
@@ -288,11 +335,10 @@ __device__ bool op_rms_qkv_rope(const Params& p, Smem<M>& s, const Ctx& c) {
   QMK_STAMP(2);
 
   // Epilogue: the GEMV result is bf16 before RoPE; q -> q_post_rope, k/v -> cache row of this position.
-  const float* cosr = p.rope_cos + static_cast<size_t>(p.pos_id) * M::D;
-  const float* sinr = p.rope_sin + static_cast<size_t>(p.pos_id) * M::D;
   const size_t kv_row = (static_cast<size_t>(layer) * p.max_seq_len + p.pos_id) * (M::NKV * M::D);
-  for (int pair = threadIdx.x; pair < nrows / 2; pair += kThreads) {
+  for (int pair = c.tid; pair < nrows / 2; pair += kThreads) {
     const int r = rs + 2 * pair;
+    const bool first = pair == c.tid;
     const float v0 = round_bf16(s.res[2 * pair]), v1 = round_bf16(s.res[2 * pair + 1]);
     if constexpr (M::QK_NORM) {
       // Qwen3 op set: the rounded GEMV result leaves as it is; norm and RoPE belong to the attention prologue.
@@ -303,12 +349,12 @@ __device__ bool op_rms_qkv_rope(const Params& p, Smem<M>& s, const Ctx& c) {
         st_tagged(p.ws + (r < kq ? kWsQ + r / 2 : (r < kk ? kWsK + (r - kq) / 2 : kWsV + (r - kk) / 2)), w, tag);
       }
     } else if (r < M::NQ * M::D) {
-      const uint32_t w = rope_pair(v0, v1, cosr, sinr, r % M::D);
+      const uint32_t w = first ? rope_pair(v0, v1, cs0, sn0) : rope_pair(v0, v1, cosr, sinr, r % M::D);
       st_shared32(p.q_post_rope + r, w);
       if (tg) st_tagged(p.ws + kWsQ + r / 2, w, tag);
     } else if (r < (M::NQ + M::NKV) * M::D) {
       const int i = r - M::NQ * M::D;
-      const uint32_t w = rope_pair(v0, v1, cosr, sinr, i % M::D);
+      const uint32_t w = first ? rope_pair(v0, v1, cs0, sn0) : rope_pair(v0, v1, cosr, sinr, i % M::D);
       st_shared32(p.k_cache + kv_row + i, w);
       if (tg) st_tagged(p.ws + kWsK + i / 2, w, tag);
     } else {
@@ -325,7 +371,7 @@ __device__ bool op_rms_qkv_rope(const Params& p, Smem<M>& s, const Ctx& c) {
   // One arrival per tile, on the counter of the head the tile belongs to.
   if (nend > nstart) {
     const int slot0 = nstart / bph, slot1 = (nend - 1) / bph;
-    const int slot = slot0 + static_cast<int>(threadIdx.x);
+    const int slot = slot0 + c.tid;
     if (slot <= slot1) {
       const int lo = max(nstart, slot * bph), hi = min(nend, (slot + 1) * bph);
       publish(counter_ptr(p, layer, ROW_QKV, slot), hi - lo);
@@ -412,7 +458,7 @@ __device__ bool op_attn_splitkv(const Params& p, Smem<M>& s, const Ctx& c) {
   if (P < 1 || P > p.max_splits || part < 0 || part >= P) return bad_operand(p, s, c, 3);
   if (merge_in_last && P > kMaxPartials) return bad_operand(p, s, c, 3);
 
-  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int lane = c.tid & 63, wave = c.tid >> 6;
   const int grp = lane >> 3, col = lane & 7;
 
   // Context slice of this partial (python_vm.py:391-401).
@@ -427,18 +473,25 @@ __device__ bool op_attn_splitkv(const Params& p, Smem<M>& s, const Ctx& c) {
   const size_t tok_stride = static_cast<size_t>(M::NKV) * D;
   const size_t row_of_kvh = static_cast<size_t>(layer) * p.max_seq_len * tok_stride + static_cast<size_t>(kvh) * D;
   const size_t base = row_of_kvh + col * DPL;
+  // Lane group g of the workgroup takes tokens t0 + g, t0 + g + 64, ...; the first R of them are
+  // asked for here.  A short slice is then scored without a further trip to memory.
+  constexpr int R = M::KV_AHEAD, kStep = kWaves * 8;
   int t = t0 + wave * 8 + grp;
-  v4u kv[VPL], vv[VPL];
+  v4u kv[R][VPL], vv[R][VPL];
 #pragma unroll
-  for (int j = 0; j < VPL; ++j) {
-    kv[j] = v4u{0, 0, 0, 0};
-    vv[j] = v4u{0, 0, 0, 0};
-  }
-  if (t < t1 && t != p.pos_id) {
+  for (int r = 0; r < R; ++r) {
+    const int tr = t + r * kStep;
 #pragma unroll
     for (int j = 0; j < VPL; ++j) {
-      kv[j] = reinterpret_cast<const v4u*>(p.k_cache + base + static_cast<size_t>(t) * tok_stride)[j];
-      vv[j] = reinterpret_cast<const v4u*>(p.v_cache + base + static_cast<size_t>(t) * tok_stride)[j];
+      kv[r][j] = v4u{0, 0, 0, 0};
+      vv[r][j] = v4u{0, 0, 0, 0};
+    }
+    if (tr < t1 && tr != p.pos_id) {
+#pragma unroll
+      for (int j = 0; j < VPL; ++j) {
+        kv[r][j] = reinterpret_cast<const v4u*>(p.k_cache + base + static_cast<size_t>(tr) * tok_stride)[j];
+        vv[r][j] = reinterpret_cast<const v4u*>(p.v_cache + base + static_cast<size_t>(tr) * tok_stride)[j];
+      }
     }
   }
 
@@ -453,7 +506,7 @@ __device__ bool op_attn_splitkv(const Params& p, Smem<M>& s, const Ctx& c) {
     uint32_t* words = reinterpret_cast<uint32_t*>(stage16);
     bool arrived = true;
     uint32_t a = 0, b = 0;
-    const int tid = threadIdx.x;
+    const int tid = c.tid;
     if (tid < 64) {
       arrived = poll_tagged2(p.ws + kWsQ + kvh * (GQA * D / 2) + 2 * tid, tag, p.spin_limit, a, b);
       words[kQ / 2 + 2 * tid] = a;
@@ -468,9 +521,9 @@ __device__ bool op_attn_splitkv(const Params& p, Smem<M>& s, const Ctx& c) {
     }
     if (!arrived) {
       s.ctl[0] = 1;
-      report_error(p, QMK_DEV_WAIT_TIMEOUT, c.inst_idx, c.opcode, threadIdx.x);
+      report_error(p, QMK_DEV_WAIT_TIMEOUT, c.inst_idx, c.opcode, c.tid);
     }
-    if (p.timeline != nullptr && threadIdx.x == 0) {
+    if (p.timeline != nullptr && c.tid == 0) {
       s.t_wait = wall_clock64();
       s.ctl[2] = 1;
     }
@@ -483,7 +536,7 @@ __device__ bool op_attn_splitkv(const Params& p, Smem<M>& s, const Ctx& c) {
                  p.qkv_blocks_per_head))
       return false;
     // 16-byte chunks: GQA*D/8 of q, then D/8 of K and of V (the row of this position only)
-    const int tid = threadIdx.x;
+    const int tid = c.tid;
     constexpr int kQChunks = GQA * D / 8, kRowChunks = D / 8;
     const u16* q_src = M::QK_NORM ? p.qkv_raw + kvh * GQA * D : p.q_post_rope + kvh * GQA * D;
     const u16* k_src = M::QK_NORM ? p.qkv_raw + M::NQ * D + kvh * D : p.k_cache + new_row;
@@ -542,11 +595,14 @@ __device__ bool op_attn_splitkv(const Params& p, Smem<M>& s, const Ctx& c) {
         q[h][8 * j + 6] = bf_lo(qv.w) * qscale; q[h][8 * j + 7] = bf_hi(qv.w) * qscale;
       }
     }
-    if (t < t1 && t == p.pos_id) {  // the row appended during this launch
 #pragma unroll
-      for (int j = 0; j < VPL; ++j) {
-        kv[j] = reinterpret_cast<const v4u*>(stage16 + kK + col * DPL)[j];
-        vv[j] = reinterpret_cast<const v4u*>(stage16 + kV + col * DPL)[j];
+    for (int r = 0; r < R; ++r) {
+      if (t + r * kStep < t1 && t + r * kStep == p.pos_id) {  // the row appended during this launch
+#pragma unroll
+        for (int j = 0; j < VPL; ++j) {
+          kv[r][j] = reinterpret_cast<const v4u*>(stage16 + kK + col * DPL)[j];
+          vv[r][j] = reinterpret_cast<const v4u*>(stage16 + kV + col * DPL)[j];
+        }
       }
     }
   }
@@ -562,66 +618,63 @@ __device__ bool op_attn_splitkv(const Params& p, Smem<M>& s, const Ctx& c) {
   }
 
   while (t < t1) {
-    // next token of this lane group, fetched while the current one is scored
-    const int tn = t + kWaves * 8;
-    v4u kn[VPL], vn[VPL];
 #pragma unroll
-    for (int j = 0; j < VPL; ++j) {
-      kn[j] = v4u{0, 0, 0, 0};
-      vn[j] = v4u{0, 0, 0, 0};
-    }
-    if (tn < t1) {
-      const size_t off = base + static_cast<size_t>(tn) * tok_stride;
+    for (int r = 0; r < R; ++r) {
+      const int tr = t + r * kStep;
+      if (tr < t1) {  // the 8 lanes of a group always take the same branch
+        // scores of all heads first (K live), then the accumulator updates (V live)
+        float sc[GQA];
+        {
+          float k[DPL];
 #pragma unroll
-      for (int j = 0; j < VPL; ++j) {
-        if (tn == p.pos_id) {
-          kn[j] = reinterpret_cast<const v4u*>(stage16 + kK + col * DPL)[j];
-          vn[j] = reinterpret_cast<const v4u*>(stage16 + kV + col * DPL)[j];
-        } else {
-          kn[j] = reinterpret_cast<const v4u*>(p.k_cache + off)[j];
-          vn[j] = reinterpret_cast<const v4u*>(p.v_cache + off)[j];
+          for (int j = 0; j < VPL; ++j) {
+            const v4u kk = kv[r][j];
+            k[8 * j + 0] = bf_lo(kk.x); k[8 * j + 1] = bf_hi(kk.x); k[8 * j + 2] = bf_lo(kk.y); k[8 * j + 3] = bf_hi(kk.y);
+            k[8 * j + 4] = bf_lo(kk.z); k[8 * j + 5] = bf_hi(kk.z); k[8 * j + 6] = bf_lo(kk.w); k[8 * j + 7] = bf_hi(kk.w);
+          }
+#pragma unroll
+          for (int h = 0; h < GQA; ++h) {
+            float a = 0.f;
+#pragma unroll
+            for (int i = 0; i < DPL; ++i) a = __builtin_fmaf(q[h][i], k[i], a);
+            sc[h] = group8_sum(a);
+          }
+        }
+        float v[DPL];
+#pragma unroll
+        for (int j = 0; j < VPL; ++j) {
+          const v4u w = vv[r][j];
+          v[8 * j + 0] = bf_lo(w.x); v[8 * j + 1] = bf_hi(w.x); v[8 * j + 2] = bf_lo(w.y); v[8 * j + 3] = bf_hi(w.y);
+          v[8 * j + 4] = bf_lo(w.z); v[8 * j + 5] = bf_hi(w.z); v[8 * j + 6] = bf_lo(w.w); v[8 * j + 7] = bf_hi(w.w);
+        }
+        // the slot is free: ask for the token R steps further on
+        const int tn = tr + R * kStep;
+        if (tn < t1) {
+          const size_t off = base + static_cast<size_t>(tn) * tok_stride;
+#pragma unroll
+          for (int j = 0; j < VPL; ++j) {
+            if (tn == p.pos_id) {
+              kv[r][j] = reinterpret_cast<const v4u*>(stage16 + kK + col * DPL)[j];
+              vv[r][j] = reinterpret_cast<const v4u*>(stage16 + kV + col * DPL)[j];
+            } else {
+              kv[r][j] = reinterpret_cast<const v4u*>(p.k_cache + off)[j];
+              vv[r][j] = reinterpret_cast<const v4u*>(p.v_cache + off)[j];
+            }
+          }
+        }
+#pragma unroll
+        for (int h = 0; h < GQA; ++h) {
+          const float mn = fmaxf(m[h], sc[h]);
+          const float alpha = exp2_fast(m[h] - mn);   // 0 on the first token (m = -inf)
+          const float pr = exp2_fast(sc[h] - mn);
+          l[h] = __builtin_fmaf(l[h], alpha, pr);
+#pragma unroll
+          for (int i = 0; i < DPL; ++i) acc[h][i] = __builtin_fmaf(acc[h][i], alpha, pr * v[i]);
+          m[h] = mn;
         }
       }
     }
-    // scores of all heads first (K live), then the accumulator updates (V live)
-    float sc[GQA];
-    {
-      float k[DPL];
-#pragma unroll
-      for (int j = 0; j < VPL; ++j) {
-        k[8 * j + 0] = bf_lo(kv[j].x); k[8 * j + 1] = bf_hi(kv[j].x); k[8 * j + 2] = bf_lo(kv[j].y); k[8 * j + 3] = bf_hi(kv[j].y);
-        k[8 * j + 4] = bf_lo(kv[j].z); k[8 * j + 5] = bf_hi(kv[j].z); k[8 * j + 6] = bf_lo(kv[j].w); k[8 * j + 7] = bf_hi(kv[j].w);
-      }
-#pragma unroll
-      for (int h = 0; h < GQA; ++h) {
-        float a = 0.f;
-#pragma unroll
-        for (int i = 0; i < DPL; ++i) a = __builtin_fmaf(q[h][i], k[i], a);
-        sc[h] = group8_sum(a);  // the 8 lanes of a group always take the same branch
-      }
-    }
-    float v[DPL];
-#pragma unroll
-    for (int j = 0; j < VPL; ++j) {
-      v[8 * j + 0] = bf_lo(vv[j].x); v[8 * j + 1] = bf_hi(vv[j].x); v[8 * j + 2] = bf_lo(vv[j].y); v[8 * j + 3] = bf_hi(vv[j].y);
-      v[8 * j + 4] = bf_lo(vv[j].z); v[8 * j + 5] = bf_hi(vv[j].z); v[8 * j + 6] = bf_lo(vv[j].w); v[8 * j + 7] = bf_hi(vv[j].w);
-    }
-#pragma unroll
-    for (int h = 0; h < GQA; ++h) {
-      const float mn = fmaxf(m[h], sc[h]);
-      const float alpha = exp2_fast(m[h] - mn);   // 0 on the first token (m = -inf)
-      const float pr = exp2_fast(sc[h] - mn);
-      l[h] = __builtin_fmaf(l[h], alpha, pr);
-#pragma unroll
-      for (int i = 0; i < DPL; ++i) acc[h][i] = __builtin_fmaf(acc[h][i], alpha, pr * v[i]);
-      m[h] = mn;
-    }
-    t = tn;
-#pragma unroll
-    for (int j = 0; j < VPL; ++j) {
-      kv[j] = kn[j];
-      vv[j] = vn[j];
-    }
+    t += R * kStep;
   }
 
   QMK_STAMP(1);  // tokens scored
@@ -648,7 +701,7 @@ __device__ bool op_attn_splitkv(const Params& p, Smem<M>& s, const Ctx& c) {
   // wave reductions; with D = 128 the two waves of a head compute the same numbers).  Then
   // lane = 4*quad + sub sums dims dbase + 4*quad..+3 over the 16 states g = sub, sub+4, ... and the
   // four `sub` lanes of a quad are added with DPP.
-  if (threadIdx.x < GQA * D) {
+  if (c.tid < GQA * D) {
     static_assert(kWaves * 8 == kWaveSize, "one lane per lane group");
     const int h = wave / (D / kWaveSize), dbase = kWaveSize * (wave % (D / kWaveSize));
     const float mg = s.merge[lane][h][D];
@@ -695,25 +748,25 @@ __device__ bool op_attn_splitkv(const Params& p, Smem<M>& s, const Ctx& c) {
   __syncthreads();
   QMK_STAMP(3);  // stores acknowledged
   if (merge_mode == 2) {  // one arrival per partial on the attention -> O-proj edge
-    if (threadIdx.x == 0) arrive_all(p, layer, ROW_REDUCE, 1);
+    if (c.tid == 0) arrive_all(p, layer, ROW_REDUCE, 1);
     return true;
   }
   if (!merge_in_last) {
-    if (threadIdx.x < M::GQA) publish(counter_ptr(p, layer, ROW_SPLITKV, kvh * M::GQA + threadIdx.x), 1);
+    if (c.tid < M::GQA) publish(counter_ptr(p, layer, ROW_SPLITKV, kvh * M::GQA + c.tid), 1);
     return true;
   }
   // Arrive on the four head counters; whoever sees P-1 earlier arrivals is last.
-  if (threadIdx.x < M::GQA) {
-    const int prev = __hip_atomic_fetch_add(counter_ptr(p, layer, ROW_SPLITKV, kvh * M::GQA + threadIdx.x), 1,
+  if (c.tid < M::GQA) {
+    const int prev = __hip_atomic_fetch_add(counter_ptr(p, layer, ROW_SPLITKV, kvh * M::GQA + c.tid), 1,
                                             __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    if (threadIdx.x == 0) s.ctl[3] = (prev == P - 1);
+    if (c.tid == 0) s.ctl[3] = (prev == P - 1);
   }
   __syncthreads();
   if (s.ctl[3]) {  // uniform: every partial of this head group has been acknowledged in memory
     merge_partials<M>(p, kvh * M::GQA, P, nullptr, true, 0);
     release_stores();
     __syncthreads();
-    if (threadIdx.x == 0) publish(counter_ptr(p, layer, ROW_REDUCE, 0), M::GQA);
+    if (c.tid == 0) publish(counter_ptr(p, layer, ROW_REDUCE, 0), M::GQA);
   }
   return true;
 }
@@ -736,7 +789,7 @@ __device__ bool op_attn_reduce(const Params& p, Smem<M>& s, const Ctx& c) {
   merge_partials<M>(p, head0, n, &s.inst[5], terminal, out_slot);
   release_stores();
   __syncthreads();
-  if (threadIdx.x == 0) publish(counter_ptr(p, layer, ROW_REDUCE, 0), M::GQA);
+  if (c.tid == 0) publish(counter_ptr(p, layer, ROW_REDUCE, 0), M::GQA);
   return true;
 }
 
@@ -778,7 +831,7 @@ __device__ bool op_oproj_residual(const Params& p, Smem<M>& s, const Ctx& c) {
   if (nstart < 0 || nend < nstart || static_cast<long>(nend) * tile > M::H) return bad_operand(p, s, c, 4);
   if ((nend - nstart) * tile > kResSlots) return bad_operand(p, s, c, 3);
 
-  const int lane = threadIdx.x & 63;
+  const int lane = c.tid & 63;
   const int rs = nstart * tile, nrows = (nend - nstart) * tile;
   const u16* W = p.o_w + (static_cast<size_t>(layer) * M::H + rs) * M::H;
   auto src = [&](int r) { return W + static_cast<size_t>(r) * M::H; };
@@ -792,15 +845,15 @@ __device__ bool op_oproj_residual(const Params& p, Smem<M>& s, const Ctx& c) {
   const uint32_t tag = tag_of(s.generation, layer);
   if (tg && nrows / 2 > kThreads) return bad_operand(p, s, c, 4);  // one residual pair per thread
   uint32_t res_old = 0;
-  if (tg && static_cast<int>(threadIdx.x) < nrows / 2 &&
-      !residual_in(p, layer > 0 ? p.ws + kWsHiddenOut : nullptr, tag - 1, rs, threadIdx.x, res_old)) {
+  if (tg && c.tid < nrows / 2 &&
+      !residual_in(p, layer > 0 ? p.ws + kWsHiddenOut : nullptr, tag - 1, rs, c.tid, res_old)) {
     s.ctl[0] = 1;  // seen by everybody after the barrier inside the wait below
-    report_error(p, QMK_DEV_WAIT_TIMEOUT, c.inst_idx, c.opcode, threadIdx.x);
+    report_error(p, QMK_DEV_WAIT_TIMEOUT, c.inst_idx, c.opcode, c.tid);
   }
   const int self_merge = s.inst[5];  // reduction_block_idx: 0, or the split-KV fan-out P when this op merges
   if (self_merge == 0) {
     if (!wg_wait(p, s, c, 1, [&](int) { return counter_ptr(p, layer, ROW_REDUCE, 0); }, M::NQ)) return false;
-    *reinterpret_cast<uint64_t*>(s.x + threadIdx.x * 4) = ld_shared64(p.attn_out + threadIdx.x * 4);
+    *reinterpret_cast<uint64_t*>(s.x + c.tid * 4) = ld_shared64(p.attn_out + c.tid * 4);
   } else {
     // Every O-proj workgroup merges the split-KV partials itself (python_vm.py:439-488 for all heads):
     // no merging workgroup, no attn_out round trip, one synchronisation hop less.  Thread t owns
@@ -808,7 +861,7 @@ __device__ bool op_oproj_residual(const Params& p, Smem<M>& s, const Ctx& c) {
     const int P = self_merge;
     if (P < 1 || P > kMaxPartials || P > p.max_splits) return bad_operand(p, s, c, 5);
     if (!wg_wait_all(p, s, c, layer, ROW_REDUCE, 0, M::NKV * P)) return false;
-    const int h = threadIdx.x / (M::D / 4), d0 = 4 * (threadIdx.x % (M::D / 4));
+    const int h = c.tid / (M::D / 4), d0 = 4 * (c.tid % (M::D / 4));
     const float* lse = p.attn_lse + static_cast<size_t>(h) * p.max_splits;
     const float* part = p.attn_partial + static_cast<size_t>(h) * p.max_splits * M::D + d0;
     float mx = -INFINITY, den = 0.f, n0 = 0.f, n1 = 0.f, n2 = 0.f, n3 = 0.f;
@@ -840,10 +893,10 @@ __device__ bool op_oproj_residual(const Params& p, Smem<M>& s, const Ctx& c) {
     const float inv = den > 0.f ? 1.0f / den : 0.f;
     const uint32_t lo = static_cast<uint32_t>(f2bf(n0 * inv)) | (static_cast<uint32_t>(f2bf(n1 * inv)) << 16);
     const uint32_t hi = static_cast<uint32_t>(f2bf(n2 * inv)) | (static_cast<uint32_t>(f2bf(n3 * inv)) << 16);
-    *reinterpret_cast<uint2*>(s.x + threadIdx.x * 4) = make_uint2(lo, hi);
+    *reinterpret_cast<uint2*>(s.x + c.tid * 4) = make_uint2(lo, hi);
     if (nstart == 0) {  // one workgroup also leaves attn_out in memory, as the reference does
-      st_shared32(p.attn_out + threadIdx.x * 4, lo);
-      st_shared32(p.attn_out + threadIdx.x * 4 + 2, hi);
+      st_shared32(p.attn_out + c.tid * 4, lo);
+      st_shared32(p.attn_out + c.tid * 4 + 2, hi);
     }
   }
   __syncthreads();
@@ -859,20 +912,20 @@ __device__ bool op_oproj_residual(const Params& p, Smem<M>& s, const Ctx& c) {
   QMK_STAMP(2);
   if (tg) {
     // The new pair goes to the caller's buffer and, tagged, to the up/gate workgroups.
-    if (static_cast<int>(threadIdx.x) < nrows / 2) {
-      const int pair = threadIdx.x;
+    if (c.tid < nrows / 2) {
+      const int pair = c.tid;
       const uint32_t w = residual_word(res_old, s.res[2 * pair], s.res[2 * pair + 1]);
       st_tagged(p.ws + kWsHiddenMid + (rs + 2 * pair) / 2, w, tag);
       st_shared32(p.hidden + rs + 2 * pair, w);
     }
     return true;
   }
-  for (int pair = threadIdx.x; pair < nrows / 2; pair += kThreads)
+  for (int pair = c.tid; pair < nrows / 2; pair += kThreads)
     residual_pair(p.hidden + rs + 2 * pair, s.res[2 * pair], s.res[2 * pair + 1]);
 
   release_stores();
   __syncthreads();
-  if (threadIdx.x == 0 && nend > nstart) arrive_all(p, layer, ROW_OPROJ, nend - nstart);
+  if (c.tid == 0 && nend > nstart) arrive_all(p, layer, ROW_OPROJ, nend - nstart);
   return true;
 }
 
@@ -892,7 +945,7 @@ __device__ bool op_rms_upgate_silu(const Params& p, Smem<M>& s, const Ctx& c) {
   for (int i = 0; i < n; ++i)
     if (s.inst[4 + i] < 0 || s.inst[4 + i] >= nblocks_total) return bad_operand(p, s, c, 4 + i);
 
-  const int lane = threadIdx.x & 63;
+  const int lane = c.tid & 63;
   const int nout = n * tile;       // output elements of this instruction
   const int nrows = 2 * nout;      // streamed rows: element 2i = up row i, 2i+1 = gate row i
   const u16* Wu = p.up_w + static_cast<size_t>(layer) * M::F * M::H;
@@ -901,11 +954,11 @@ __device__ bool op_rms_upgate_silu(const Params& p, Smem<M>& s, const Ctx& c) {
   auto src = [&](int e) { return ((e & 1) ? Wg : Wu) + static_cast<size_t>(row_of(e >> 1)) * M::H; };
 
   RowRegs<CH> buf[kUpGateBuffers];
-  preload_range<0, kEarlyUpGate>(nrows, src, buf);
   const bool tg = tagged(p);
-  if (!tg && !wg_wait_all(p, s, c, layer, ROW_OPROJ, 0, p.oproj_blocks)) return false;
-  if (!rms_to_lds(p, s, c, tg ? p.ws + kWsHiddenMid : nullptr, tag_of(s.generation, layer), p.mlp_norm + static_cast<size_t>(layer) * M::H,
-                  [&] { preload_range<kEarlyUpGate, kUpGateBuffers>(nrows, src, buf); }))
+  if (!rms_to_lds<M, kUpGateBuffers>(
+          p, s, c, tg ? p.ws + kWsHiddenMid : nullptr, tag_of(s.generation, layer), p.mlp_norm + static_cast<size_t>(layer) * M::H,
+          [&](auto k) { preload_range<decltype(k)::value, decltype(k)::value + 1>(nrows, src, buf); },
+          [&] { return wg_wait_all(p, s, c, layer, ROW_OPROJ, 0, p.oproj_blocks); }))
     return false;
   QMK_STAMP(0);
   v4u x[CH];
@@ -918,7 +971,7 @@ __device__ bool op_rms_upgate_silu(const Params& p, Smem<M>& s, const Ctx& c) {
   __syncthreads();
   QMK_STAMP(2);
   // Two neighbouring outputs of a tile leave as one 32-bit word.
-  for (int pair = threadIdx.x; pair < nout / 2; pair += kThreads) {
+  for (int pair = c.tid; pair < nout / 2; pair += kThreads) {
     uint32_t word = 0;
 #pragma unroll
     for (int k = 0; k < 2; ++k) {
@@ -936,9 +989,9 @@ __device__ bool op_rms_upgate_silu(const Params& p, Smem<M>& s, const Ctx& c) {
   __syncthreads();
   // One arrival per block, on the bucket (= down-projection K slice) it belongs to.
   if (xcd_counters(p)) {
-    if (threadIdx.x == 0 && n > 0) arrive_all(p, layer, ROW_UPGATE, n);
-  } else if (static_cast<int>(threadIdx.x) < n) {
-    publish(counter_ptr(p, layer, ROW_UPGATE, s.inst[4 + threadIdx.x] / p.upgate_blocks_per_bucket), 1);
+    if (c.tid == 0 && n > 0) arrive_all(p, layer, ROW_UPGATE, n);
+  } else if (c.tid < n) {
+    publish(counter_ptr(p, layer, ROW_UPGATE, s.inst[4 + c.tid] / p.upgate_blocks_per_bucket), 1);
   }
   return true;
 }
@@ -976,7 +1029,7 @@ __device__ bool op_down_residual(const Params& p, Smem<M>& s, const Ctx& c) {
   if (split < 0 || static_cast<long>(split + 1) * kg > M::F) return bad_operand(p, s, c, 5);
   if (split >= p.barrier_slots) return bad_operand(p, s, c, 5);
 
-  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int lane = c.tid & 63, wave = c.tid >> 6;
   const int rs = nstart * tile, nrows = (nend - nstart) * tile, ks = split * kg;
   const int segs = kg / (512 * CH);
   // Element order is chosen per wave so that a wave owns whole rows: wave w streams the
@@ -999,9 +1052,9 @@ __device__ bool op_down_residual(const Params& p, Smem<M>& s, const Ctx& c) {
   if (tg && nrows / 2 > kThreads) return bad_operand(p, s, c, 4);  // one residual pair per thread
   // Tagged mode: the rows' residual values as the O-proj announced them, fetched ahead of time.
   uint32_t res_old = 0;
-  if (tg && static_cast<int>(threadIdx.x) < nrows / 2 && !residual_in(p, p.ws + kWsHiddenMid, tag, rs, threadIdx.x, res_old)) {
+  if (tg && c.tid < nrows / 2 && !residual_in(p, p.ws + kWsHiddenMid, tag, rs, c.tid, res_old)) {
     s.ctl[0] = 1;  // seen by everybody after the barrier inside the wait below
-    report_error(p, QMK_DEV_WAIT_TIMEOUT, c.inst_idx, c.opcode, threadIdx.x);
+    report_error(p, QMK_DEV_WAIT_TIMEOUT, c.inst_idx, c.opcode, c.tid);
   }
   if (tg) {
     // silu_out from its tagged units: thread t polls the unit pairs 2t + 1024k until they carry
@@ -1009,7 +1062,7 @@ __device__ bool op_down_residual(const Params& p, Smem<M>& s, const Ctx& c) {
     static_assert(M::F % (4 * kThreads) == 0, "whole unit pairs per thread");
     constexpr int kPairs = M::F / (4 * kThreads);
     uint32_t* words = reinterpret_cast<uint32_t*>(s.x);
-    const uint64_t* mine = p.ws + kWsSilu + 2 * threadIdx.x;
+    const uint64_t* mine = p.ws + kWsSilu + 2 * c.tid;
     uint32_t polls = 0;
     bool have[kPairs];
 #pragma unroll
@@ -1027,8 +1080,8 @@ __device__ bool op_down_residual(const Params& p, Smem<M>& s, const Ctx& c) {
 #pragma unroll
       for (int k = 0; k < kPairs; ++k) {
         if (!have[k] && static_cast<uint32_t>(u[2 * k] >> 32) == tag && static_cast<uint32_t>(u[2 * k + 1] >> 32) == tag) {
-          words[2 * threadIdx.x + 1024 * k] = static_cast<uint32_t>(u[2 * k]);
-          words[2 * threadIdx.x + 1024 * k + 1] = static_cast<uint32_t>(u[2 * k + 1]);
+          words[2 * c.tid + 1024 * k] = static_cast<uint32_t>(u[2 * k]);
+          words[2 * c.tid + 1024 * k + 1] = static_cast<uint32_t>(u[2 * k + 1]);
           have[k] = true;
         }
         all = all && have[k];
@@ -1036,12 +1089,12 @@ __device__ bool op_down_residual(const Params& p, Smem<M>& s, const Ctx& c) {
       if (all) break;
       if (++polls > p.spin_limit) {
         s.ctl[0] = 1;
-        report_error(p, QMK_DEV_WAIT_TIMEOUT, c.inst_idx, c.opcode, threadIdx.x);
+        report_error(p, QMK_DEV_WAIT_TIMEOUT, c.inst_idx, c.opcode, c.tid);
         break;
       }
       __builtin_amdgcn_s_sleep(8);
     }
-    if (p.timeline != nullptr && threadIdx.x == 0) {
+    if (p.timeline != nullptr && c.tid == 0) {
       s.t_wait = wall_clock64();
       s.ctl[2] = 1;
     }
@@ -1055,12 +1108,12 @@ __device__ bool op_down_residual(const Params& p, Smem<M>& s, const Ctx& c) {
   uint64_t act[kActLoads];
 #pragma unroll
   for (int k = 0; k < kActLoads; ++k)
-    if (static_cast<int>(threadIdx.x) + k * kThreads < kg / 4) act[k] = ld_shared64(p.silu_out + ks + (threadIdx.x + k * kThreads) * 4);
+    if (c.tid + k * kThreads < kg / 4) act[k] = ld_shared64(p.silu_out + ks + (c.tid + k * kThreads) * 4);
   asm volatile("" ::: "memory");
   preload_range<kEarly, kDepth>(rows_w > 0 ? n_elems : 0, src, buf);
 #pragma unroll
   for (int k = 0; k < kActLoads; ++k)
-    if (static_cast<int>(threadIdx.x) + k * kThreads < kg / 4) reinterpret_cast<uint64_t*>(s.x)[threadIdx.x + k * kThreads] = act[k];
+    if (c.tid + k * kThreads < kg / 4) reinterpret_cast<uint64_t*>(s.x)[c.tid + k * kThreads] = act[k];
   __syncthreads();
   }
 
@@ -1082,8 +1135,8 @@ __device__ bool op_down_residual(const Params& p, Smem<M>& s, const Ctx& c) {
   QMK_STAMP(2);
 
   if (tg) {
-    if (static_cast<int>(threadIdx.x) < nrows / 2) {
-      const int pair = threadIdx.x;
+    if (c.tid < nrows / 2) {
+      const int pair = c.tid;
       const uint32_t w = residual_word(res_old, s.res[2 * pair], s.res[2 * pair + 1]);
       st_tagged(p.ws + kWsHiddenOut + (rs + 2 * pair) / 2, w, tag);
       st_shared32(p.hidden + rs + 2 * pair, w);
@@ -1091,15 +1144,15 @@ __device__ bool op_down_residual(const Params& p, Smem<M>& s, const Ctx& c) {
     return true;
   }
   if (kg == M::F) {  // one slice: every row has a single writer
-    for (int pair = threadIdx.x; pair < nrows / 2; pair += kThreads)
+    for (int pair = c.tid; pair < nrows / 2; pair += kThreads)
       residual_pair(p.hidden + rs + 2 * pair, s.res[2 * pair], s.res[2 * pair + 1]);
   } else {           // other slices add to the same rows concurrently
-    for (int r = threadIdx.x; r < nrows; r += kThreads) atomic_add_bf16(p.hidden + rs + r, round_bf16(s.res[r]));
+    for (int r = c.tid; r < nrows; r += kThreads) atomic_add_bf16(p.hidden + rs + r, round_bf16(s.res[r]));
   }
 
   release_stores();
   __syncthreads();
-  if (threadIdx.x == 0 && nend > nstart) arrive_all(p, layer, ROW_DOWN, nend - nstart);
+  if (c.tid == 0 && nend > nstart) arrive_all(p, layer, ROW_DOWN, nend - nstart);
   return true;
 }
 
@@ -1113,7 +1166,7 @@ __device__ bool op_rms_lmhead(const Params& p, Smem<M>& s, const Ctx& c) {
   if (bstart < 0 || bend < bstart || static_cast<long>(bend) * tile > p.vocab_size) return bad_operand(p, s, c, 2);
   if (p.num_layers < 1) return bad_operand(p, s, c, 0);
 
-  const int lane = threadIdx.x & 63;
+  const int lane = c.tid & 63;
   const int rs = bstart * tile, nrows = (bend - bstart) * tile;
   const u16* W = p.lm_w + static_cast<size_t>(rs) * M::H;
   auto src = [&](int r) { return W + static_cast<size_t>(r) * M::H; };
@@ -1141,11 +1194,11 @@ __device__ bool op_rms_lmhead(const Params& p, Smem<M>& s, const Ctx& c) {
   });
   if (p.token_out != nullptr) {  // greedy candidate of this workgroup (several LM-head instructions accumulate)
     if (lane == 0) {
-      s.red[threadIdx.x >> 6] = best;
-      s.wave_idx[threadIdx.x >> 6] = best_row;
+      s.red[c.tid >> 6] = best;
+      s.wave_idx[c.tid >> 6] = best_row;
     }
     __syncthreads();
-    if (threadIdx.x == 0) {
+    if (c.tid == 0) {
       float v = s.best_val;
       int i = s.best_idx;
       for (int w = 0; w < kWaves; ++w)
