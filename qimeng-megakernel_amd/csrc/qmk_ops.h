@@ -239,11 +239,11 @@ constexpr int kDepth = QMK_DEPTH;  // row buffers per wave: 4 x CH x 16 B per la
 // element 8*NB further on as soon as it has been consumed.  `use(e, buf)` gets the raw
 // registers of element e.
 //
-// How much to ask for before the counter wait is a trade: what is in flight then lands while
-// the workgroup waits, but it also stands in the memory queues in front of the last producers'
-// stores and counter updates, and in front of this wave's own counter poll (loads return in
-// issue order).  So the big GEMVs ask for kEarly buffers up front and for the rest right after
-// the wait, behind the activation read.
+// How much to ask for before the wait is a trade: what is in flight then lands while the
+// workgroup waits, but it also stands in the memory queues in front of the last producers'
+// stores, and in front of this wave's own looks at the hand-over (loads return in issue order).
+// The ops that normalise the residual stream ask for one buffer per look; the down projection
+// asks for kEarly buffers up front and for the rest once silu_out is complete.
 template <int K0, int K1, int CH, int NB, class Src>
 __device__ __forceinline__ void preload_range(int n, Src src, RowRegs<CH> (&buf)[NB]) {
   static_assert(K0 >= 0 && K1 <= NB, "buffer range");
@@ -275,16 +275,12 @@ __device__ __forceinline__ void stream(int n, Src src, RowRegs<CH> (&buf)[NB], U
 }
 
 #ifndef QMK_EARLY
-#define QMK_EARLY 4
+#define QMK_EARLY 2
 #endif
 #ifndef QMK_UPGATE_BUFFERS
 #define QMK_UPGATE_BUFFERS 4
 #endif
-#ifndef QMK_EARLY_UPGATE
-#define QMK_EARLY_UPGATE QMK_EARLY
-#endif
-constexpr int kEarly = QMK_EARLY;                    // buffers of the down projection requested before its counter wait
-constexpr int kEarlyUpGate = QMK_EARLY_UPGATE;       // the same for the up/gate GEMV
+constexpr int kEarly = QMK_EARLY;                    // buffers of the down projection requested before its wait
 constexpr int kUpGateBuffers = QMK_UPGATE_BUFFERS;   // row buffers of the up/gate GEMV
 
 // ===================================================================== 1 ==
@@ -1094,6 +1090,7 @@ __device__ bool op_down_residual(const Params& p, Smem<M>& s, const Ctx& c) {
       }
       __builtin_amdgcn_s_sleep(8);
     }
+    preload_range<kEarly, kDepth>(rows_w > 0 ? n_elems : 0, src, buf);
     if (p.timeline != nullptr && c.tid == 0) {
       s.t_wait = wall_clock64();
       s.ctl[2] = 1;
