@@ -36,8 +36,13 @@ __global__ __launch_bounds__(kThreads, 1) void decode_megakernel(const Params p)
 
   const int32_t* queue = p.instructions + static_cast<size_t>(blockIdx.x) * p.num_insts * kInstWords;
   bool ok = true;
+  // The words of instruction i+1 are asked for while instruction i runs.
+  int32_t word = (threadIdx.x < kInstWords && p.num_insts > 0) ? queue[threadIdx.x] : 0;
   for (int i = 0; i < p.num_insts && ok; ++i) {
-    if (threadIdx.x < kInstWords) s.inst[threadIdx.x] = queue[i * kInstWords + threadIdx.x];
+    if (threadIdx.x < kInstWords) {
+      s.inst[threadIdx.x] = word;
+      if (i + 1 < p.num_insts) word = queue[(i + 1) * kInstWords + threadIdx.x];
+    }
     __syncthreads();
     const int opcode = s.inst[0];
     int tid = threadIdx.x;
