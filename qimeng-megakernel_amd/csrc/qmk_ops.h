@@ -455,7 +455,6 @@ __device__ bool op_attn_splitkv(const Params& p, Smem<M>& s, const Ctx& c) {
   if (merge_in_last && P > kMaxPartials) return bad_operand(p, s, c, 3);
 
   const int lane = c.tid & 63, wave = c.tid >> 6;
-  const int grp = lane >> 3, col = lane & 7;
 
   // Context slice of this partial (python_vm.py:391-401).
   const int seq_len = p.pos_id + 1;
@@ -465,31 +464,48 @@ __device__ bool op_attn_splitkv(const Params& p, Smem<M>& s, const Ctx& c) {
   const int t1 = min(min((part + 1) * bpp, total_blocks) * M::KV_BLOCK, seq_len);
   const bool has_new = p.pos_id >= t0 && p.pos_id < t1;
 
-  // Rows of earlier positions do not depend on this step: fetch the first ones now.
+  // A wave scores 16 tokens at a time on the matrix cores: S^T[token][head] = K[token][:] . q[head][:]
+  // (v_mfma_f32_16x16x16_bf16, K rows as the A operand, the GQA heads as GQA of the 16 B columns), then
+  // O[head][:] += P[head][token] . V[token][:] with P split into two bf16 terms so that it keeps 16
+  // mantissa bits.  Operand layout of the instruction: lane l holds A[l%16][4*(l/16)..+3],
+  // B[4*(l/16)..+3][l%16] and C[4*(l/16)..+3][l%16].  Which of the D dims sits in which k slot is free
+  // as long as q and K agree, and so is the order of the output columns: lane (c16, g4) reads K dims
+  // g4*D/4 .. +D/4 of token c16 and V dims c16*D/16 .. +D/16 of tokens 4*g4 .. +3, in 16- or 8-byte pieces.
+  // Rows of earlier positions do not depend on this step: the wave's first tile is fetched now.
+  constexpr int KV16 = D / 32;          // 16-byte vectors of a K row per lane
+  constexpr int NT = D / 16;            // k chunks of the score product = output column tiles of P.V
+  constexpr int kTile = 16, kStep = kWaves * kTile;
+  const int c16 = lane & 15, g4 = lane >> 4;
   const size_t tok_stride = static_cast<size_t>(M::NKV) * D;
   const size_t row_of_kvh = static_cast<size_t>(layer) * p.max_seq_len * tok_stride + static_cast<size_t>(kvh) * D;
-  const size_t base = row_of_kvh + col * DPL;
-  // Lane group g of the workgroup takes tokens t0 + g, t0 + g + 64, ...; the first R of them are
-  // asked for here.  A short slice is then scored without a further trip to memory.
-  constexpr int R = M::KV_AHEAD, kStep = kWaves * 8;
-  int t = t0 + wave * 8 + grp;
-  v4u kv[R][VPL], vv[R][VPL];
+  const u16* kbase = p.k_cache + row_of_kvh + g4 * (D / 4);
+  const u16* vbase = p.v_cache + row_of_kvh + c16 * NT;
+  struct Tile {
+    v4u k[KV16];         // K[token c16][g4*D/4 ..]
+    uint32_t v[4][NT / 2];  // V[token 4*g4 + j][c16*NT ..], two dims per word
+  };
+  // Tokens past the slice are fetched from its last row (finite data) and masked when scored.
+  auto fetch = [&](Tile& tl, int tb) {
+    const int tk = min(tb + c16, t1 - 1);
 #pragma unroll
-  for (int r = 0; r < R; ++r) {
-    const int tr = t + r * kStep;
+    for (int j = 0; j < KV16; ++j) tl.k[j] = reinterpret_cast<const v4u*>(kbase + static_cast<size_t>(tk) * tok_stride)[j];
 #pragma unroll
-    for (int j = 0; j < VPL; ++j) {
-      kv[r][j] = v4u{0, 0, 0, 0};
-      vv[r][j] = v4u{0, 0, 0, 0};
+    for (int j = 0; j < 4; ++j) {
+      const int tv = min(tb + 4 * g4 + j, t1 - 1);
+      const uint32_t* src = reinterpret_cast<const uint32_t*>(vbase + static_cast<size_t>(tv) * tok_stride);
+#pragma unroll
+      for (int i = 0; i < NT / 2; ++i) tl.v[j][i] = src[i];
     }
-    if (tr < t1 && tr != p.pos_id) {
+  };
+  int tb = t0 + wave * kTile;
+  Tile cur;
 #pragma unroll
-      for (int j = 0; j < VPL; ++j) {
-        kv[r][j] = reinterpret_cast<const v4u*>(p.k_cache + base + static_cast<size_t>(tr) * tok_stride)[j];
-        vv[r][j] = reinterpret_cast<const v4u*>(p.v_cache + base + static_cast<size_t>(tr) * tok_stride)[j];
-      }
-    }
-  }
+  for (int j = 0; j < KV16; ++j) cur.k[j] = v4u{0, 0, 0, 0};
+#pragma unroll
+  for (int j = 0; j < 4; ++j)
+#pragma unroll
+    for (int i = 0; i < NT / 2; ++i) cur.v[j][i] = 0;
+  if (tb < t1) fetch(cur, tb);
 
   // ---- stage q (and the appended K/V row) in LDS --------------------------------------------
   const bool tg = tagged(p);
@@ -576,167 +592,145 @@ __device__ bool op_attn_splitkv(const Params& p, Smem<M>& s, const Ctx& c) {
     __syncthreads();
   }
 
-  // q[h][DPL]: this lane's dims of the query heads, pre-scaled into the log2 domain.
-  const float qscale = p.attn_scale * 1.4426950408889634f;
-  float q[GQA][DPL];
-  {
+  // q as the B operand: column c16 is head c16 (zero beyond the GQA heads), k slots as for K.
+  typedef short bf4 __attribute__((ext_vector_type(4)));
+  typedef float f4 __attribute__((ext_vector_type(4)));
+  typedef uint32_t u2 __attribute__((ext_vector_type(2)));
+  const float qscale = p.attn_scale * 1.4426950408889634f;  // scores in the log2 domain
+  bf4 qb[NT];
 #pragma unroll
-    for (int h = 0; h < GQA; ++h) {
-#pragma unroll
-      for (int j = 0; j < VPL; ++j) {
-        const v4u qv = reinterpret_cast<const v4u*>(stage16 + kQ + h * D + col * DPL)[j];
-        q[h][8 * j + 0] = bf_lo(qv.x) * qscale; q[h][8 * j + 1] = bf_hi(qv.x) * qscale;
-        q[h][8 * j + 2] = bf_lo(qv.y) * qscale; q[h][8 * j + 3] = bf_hi(qv.y) * qscale;
-        q[h][8 * j + 4] = bf_lo(qv.z) * qscale; q[h][8 * j + 5] = bf_hi(qv.z) * qscale;
-        q[h][8 * j + 6] = bf_lo(qv.w) * qscale; q[h][8 * j + 7] = bf_hi(qv.w) * qscale;
-      }
-    }
-#pragma unroll
-    for (int r = 0; r < R; ++r) {
-      if (t + r * kStep < t1 && t + r * kStep == p.pos_id) {  // the row appended during this launch
-#pragma unroll
-        for (int j = 0; j < VPL; ++j) {
-          kv[r][j] = reinterpret_cast<const v4u*>(stage16 + kK + col * DPL)[j];
-          vv[r][j] = reinterpret_cast<const v4u*>(stage16 + kV + col * DPL)[j];
-        }
-      }
-    }
+  for (int j = 0; j < KV16; ++j) {
+    v4u qv = v4u{0, 0, 0, 0};
+    if (c16 < GQA) qv = reinterpret_cast<const v4u*>(stage16 + kQ + c16 * D + g4 * (D / 4))[j];
+    qb[2 * j] = __builtin_bit_cast(bf4, u2{qv.x, qv.y});
+    qb[2 * j + 1] = __builtin_bit_cast(bf4, u2{qv.z, qv.w});
   }
-
   QMK_STAMP(0);  // q (and the appended row) have arrived
-  float m[GQA], l[GQA], acc[GQA][DPL];
-#pragma unroll
-  for (int h = 0; h < GQA; ++h) {
-    m[h] = -INFINITY;
-    l[h] = 0.f;
-#pragma unroll
-    for (int i = 0; i < DPL; ++i) acc[h][i] = 0.f;
-  }
 
-  while (t < t1) {
+  // State of this wave: m (all four lanes of a column agree), this lane's share of l, and
+  // O[head i][dim c16*NT + tile] in acc[tile][i] of lanes 0..15.
+  float m_run = -INFINITY, l_run = 0.f;
+  f4 acc[NT];
 #pragma unroll
-    for (int r = 0; r < R; ++r) {
-      const int tr = t + r * kStep;
-      if (tr < t1) {  // the 8 lanes of a group always take the same branch
-        // scores of all heads first (K live), then the accumulator updates (V live)
-        float sc[GQA];
-        {
-          float k[DPL];
+  for (int i = 0; i < NT; ++i) acc[i] = f4{0.f, 0.f, 0.f, 0.f};
+
+  while (tb < t1) {
+    Tile nxt = cur;
+    if (tb + kStep < t1) fetch(nxt, tb + kStep);
+    if (p.pos_id >= tb && p.pos_id < tb + kTile) {  // the row appended during this launch comes from LDS
+      if (tb + c16 == p.pos_id) {
 #pragma unroll
-          for (int j = 0; j < VPL; ++j) {
-            const v4u kk = kv[r][j];
-            k[8 * j + 0] = bf_lo(kk.x); k[8 * j + 1] = bf_hi(kk.x); k[8 * j + 2] = bf_lo(kk.y); k[8 * j + 3] = bf_hi(kk.y);
-            k[8 * j + 4] = bf_lo(kk.z); k[8 * j + 5] = bf_hi(kk.z); k[8 * j + 6] = bf_lo(kk.w); k[8 * j + 7] = bf_hi(kk.w);
-          }
+        for (int j = 0; j < KV16; ++j) cur.k[j] = reinterpret_cast<const v4u*>(stage16 + kK + g4 * (D / 4))[j];
+      }
 #pragma unroll
-          for (int h = 0; h < GQA; ++h) {
-            float a = 0.f;
+      for (int j = 0; j < 4; ++j) {
+        if (tb + 4 * g4 + j == p.pos_id) {
 #pragma unroll
-            for (int i = 0; i < DPL; ++i) a = __builtin_fmaf(q[h][i], k[i], a);
-            sc[h] = group8_sum(a);
-          }
-        }
-        float v[DPL];
-#pragma unroll
-        for (int j = 0; j < VPL; ++j) {
-          const v4u w = vv[r][j];
-          v[8 * j + 0] = bf_lo(w.x); v[8 * j + 1] = bf_hi(w.x); v[8 * j + 2] = bf_lo(w.y); v[8 * j + 3] = bf_hi(w.y);
-          v[8 * j + 4] = bf_lo(w.z); v[8 * j + 5] = bf_hi(w.z); v[8 * j + 6] = bf_lo(w.w); v[8 * j + 7] = bf_hi(w.w);
-        }
-        // the slot is free: ask for the token R steps further on
-        const int tn = tr + R * kStep;
-        if (tn < t1) {
-          const size_t off = base + static_cast<size_t>(tn) * tok_stride;
-#pragma unroll
-          for (int j = 0; j < VPL; ++j) {
-            if (tn == p.pos_id) {
-              kv[r][j] = reinterpret_cast<const v4u*>(stage16 + kK + col * DPL)[j];
-              vv[r][j] = reinterpret_cast<const v4u*>(stage16 + kV + col * DPL)[j];
-            } else {
-              kv[r][j] = reinterpret_cast<const v4u*>(p.k_cache + off)[j];
-              vv[r][j] = reinterpret_cast<const v4u*>(p.v_cache + off)[j];
-            }
-          }
-        }
-#pragma unroll
-        for (int h = 0; h < GQA; ++h) {
-          const float mn = fmaxf(m[h], sc[h]);
-          const float alpha = exp2_fast(m[h] - mn);   // 0 on the first token (m = -inf)
-          const float pr = exp2_fast(sc[h] - mn);
-          l[h] = __builtin_fmaf(l[h], alpha, pr);
-#pragma unroll
-          for (int i = 0; i < DPL; ++i) acc[h][i] = __builtin_fmaf(acc[h][i], alpha, pr * v[i]);
-          m[h] = mn;
+          for (int i = 0; i < NT / 2; ++i) cur.v[j][i] = reinterpret_cast<const uint32_t*>(stage16 + kV + c16 * NT)[i];
         }
       }
     }
-    t += R * kStep;
+    // S^T[token 4*g4 + i][head c16]
+    f4 sc = f4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int j = 0; j < KV16; ++j) {
+      sc = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(__builtin_bit_cast(bf4, u2{cur.k[j].x, cur.k[j].y}), qb[2 * j], sc, 0, 0, 0);
+      sc = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(__builtin_bit_cast(bf4, u2{cur.k[j].z, cur.k[j].w}), qb[2 * j + 1], sc, 0, 0, 0);
+    }
+    float mt = -INFINITY;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      sc[i] = (tb + 4 * g4 + i < t1) ? sc[i] * qscale : -INFINITY;
+      mt = fmaxf(mt, sc[i]);
+    }
+    mt = fmaxf(mt, __shfl_xor(mt, 16));
+    mt = fmaxf(mt, __shfl_xor(mt, 32));      // the tile's maximum for head c16 (a tile has a valid token: finite)
+    const float mn = fmaxf(m_run, mt);
+    const float alpha = exp2_fast(m_run - mn);  // 0 on the first tile (m = -inf)
+    m_run = mn;
+    float pr[4], psum = 0.f;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      pr[i] = (c16 < GQA) ? exp2_fast(sc[i] - mn) : 0.f;
+      psum += pr[i];
+    }
+    l_run = __builtin_fmaf(l_run, alpha, psum);
+    // P = hi + lo, both bf16: A operand rows = heads, k slots = the lane's four tokens.
+    uint32_t hi[4], lo[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      hi[i] = f2bf(pr[i]);
+      lo[i] = f2bf(pr[i] - bf2f(static_cast<u16>(hi[i])));
+    }
+    const bf4 p_hi = __builtin_bit_cast(bf4, u2{hi[0] | (hi[1] << 16), hi[2] | (hi[3] << 16)});
+    const bf4 p_lo = __builtin_bit_cast(bf4, u2{lo[0] | (lo[1] << 16), lo[2] | (lo[3] << 16)});
+    // The accumulators of head i are scaled by that head's alpha (it lives in lane i).
+    float a_head[4];
+    bool rescale = false;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      a_head[i] = i < GQA ? __int_as_float(__builtin_amdgcn_readlane(__float_as_int(alpha), i)) : 1.f;
+      rescale = rescale || a_head[i] != 1.f;
+    }
+    if (rescale) {
+#pragma unroll
+      for (int tau = 0; tau < NT; ++tau)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) acc[tau][i] *= a_head[i];
+    }
+#pragma unroll
+    for (int tau = 0; tau < NT; ++tau) {
+      // B[token 4*g4 + j][column c16] = V[token][c16*NT + tau]
+      const int w = tau / 2;
+      uint32_t b0, b1;
+      if (tau & 1) {
+        b0 = (cur.v[0][w] >> 16) | (cur.v[1][w] & 0xffff0000u);
+        b1 = (cur.v[2][w] >> 16) | (cur.v[3][w] & 0xffff0000u);
+      } else {
+        b0 = (cur.v[0][w] & 0xffffu) | (cur.v[1][w] << 16);
+        b1 = (cur.v[2][w] & 0xffffu) | (cur.v[3][w] << 16);
+      }
+      const bf4 vb = __builtin_bit_cast(bf4, u2{b0, b1});
+      acc[tau] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(p_hi, vb, acc[tau], 0, 0, 0);
+      acc[tau] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(p_lo, vb, acc[tau], 0, 0, 0);
+    }
+    cur = nxt;
+    tb += kStep;
   }
 
   QMK_STAMP(1);  // tokens scored
-  // Every lane group (8 per wave, 64 per workgroup) parks its state in LDS; the first four waves
-  // then fold the 64 states: wave f takes 64 neighbouring outputs of the GQA*D.  (Folding across
-  // lanes with shuffles costs ~120 dependent LDS-crossbar round trips per wave — several microseconds.)
-  {
-    const int g = wave * 8 + grp;
+  // Every wave parks its state in LDS; GQA*D threads then merge the eight states, one output each.
+  l_run += __shfl_xor(l_run, 16);
+  l_run += __shfl_xor(l_run, 32);
+  if (lane < 16) {
 #pragma unroll
-    for (int h = 0; h < GQA; ++h) {
-      float* dst = &s.merge[g][h][col * DPL];
+    for (int tau = 0; tau < NT; ++tau)
 #pragma unroll
-      for (int i = 0; i < DPL; i += 4) *reinterpret_cast<float4*>(dst + i) = make_float4(acc[h][i], acc[h][i + 1], acc[h][i + 2], acc[h][i + 3]);
-      if (col == 0) {
-        s.merge[g][h][D] = m[h];
-        s.merge[g][h][D + 1] = l[h];
-      }
+      for (int i = 0; i < GQA; ++i) s.merge[wave][i][c16 * NT + tau] = acc[tau][i];
+    if (c16 < GQA) {
+      s.merge[wave][c16][D] = m_run;
+      s.merge[wave][c16][D + 1] = l_run;
     }
   }
   __syncthreads();
-
-  // Fold wave f handles head h = f / (D/64), dims dbase = 64 * (f % (D/64)) .. +63.  Lane g first
-  // turns group g's (m, l) into its weight w = 2^(m - max) and l*w (max and the denominator are
-  // wave reductions; with D = 128 the two waves of a head compute the same numbers).  Then
-  // lane = 4*quad + sub sums dims dbase + 4*quad..+3 over the 16 states g = sub, sub+4, ... and the
-  // four `sub` lanes of a quad are added with DPP.
   if (c.tid < GQA * D) {
-    static_assert(kWaves * 8 == kWaveSize, "one lane per lane group");
-    const int h = wave / (D / kWaveSize), dbase = kWaveSize * (wave % (D / kWaveSize));
-    const float mg = s.merge[lane][h][D];
-    const float mx = wave_max(mg);
-    const float wgt = (mg == -INFINITY) ? 0.f : exp2_fast(mg - mx);
-    const float den = wave_sum(s.merge[lane][h][D + 1] * wgt);
-    // Each fold wave keeps its weights in a column of its own (D+2, D+3): no other wave reads or
-    // writes it; LDS operations of one wave stay in order.
-    const int wcol = D + 2 + wave % (D / kWaveSize);
-    s.merge[lane][h][wcol] = wgt;
-    const int quad = lane >> 2, sub = lane & 3;
-    float4 part4[16];
-    float w16[16];
+    const int h = c.tid / D, d = c.tid % D;
+    float mx = -INFINITY;
 #pragma unroll
-    for (int i = 0; i < 16; ++i) {
-      part4[i] = *reinterpret_cast<const float4*>(&s.merge[sub + 4 * i][h][dbase + 4 * quad]);
-      w16[i] = s.merge[sub + 4 * i][h][wcol];
-    }
-    float n0 = 0.f, n1 = 0.f, n2 = 0.f, n3 = 0.f;
+    for (int w = 0; w < kWaves; ++w) mx = fmaxf(mx, s.merge[w][h][D]);
+    float den = 0.f, num = 0.f;
 #pragma unroll
-    for (int i = 0; i < 16; ++i) {
-      n0 = __builtin_fmaf(part4[i].x, w16[i], n0);
-      n1 = __builtin_fmaf(part4[i].y, w16[i], n1);
-      n2 = __builtin_fmaf(part4[i].z, w16[i], n2);
-      n3 = __builtin_fmaf(part4[i].w, w16[i], n3);
+    for (int w = 0; w < kWaves; ++w) {
+      const float mw = s.merge[w][h][D];
+      const float wgt = (mw == -INFINITY) ? 0.f : exp2_fast(mw - mx);
+      den = __builtin_fmaf(s.merge[w][h][D + 1], wgt, den);
+      num = __builtin_fmaf(s.merge[w][h][d], wgt, num);
     }
-    n0 += dpp_f32<kDppQuadXor1>(0.f, n0); n0 += dpp_f32<kDppQuadXor2>(0.f, n0);
-    n1 += dpp_f32<kDppQuadXor1>(0.f, n1); n1 += dpp_f32<kDppQuadXor2>(0.f, n1);
-    n2 += dpp_f32<kDppQuadXor1>(0.f, n2); n2 += dpp_f32<kDppQuadXor2>(0.f, n2);
-    n3 += dpp_f32<kDppQuadXor1>(0.f, n3); n3 += dpp_f32<kDppQuadXor2>(0.f, n3);
     const int head = kvh * GQA + h;
     const bool empty = !(den > 0.f);
-    const float inv = empty ? 0.f : 1.0f / den;
     // Normalised partial output and log2-sum-exp; an empty slice contributes (0, -inf).
-    // Lane `sub` of a quad stores dim dbase + 4*quad + sub.
-    const float mine = sub == 0 ? n0 : (sub == 1 ? n1 : (sub == 2 ? n2 : n3));
-    st_shared_f32(p.attn_partial + (static_cast<size_t>(head) * p.max_splits + part) * D + dbase + lane, mine * inv);
-    if (lane == 0 && dbase == 0)
-      st_shared_f32(p.attn_lse + static_cast<size_t>(head) * p.max_splits + part, empty ? -INFINITY : mx + log2f(den));
+    st_shared_f32(p.attn_partial + (static_cast<size_t>(head) * p.max_splits + part) * D + d, empty ? 0.f : num / den);
+    if (d == 0) st_shared_f32(p.attn_lse + static_cast<size_t>(head) * p.max_splits + part, empty ? -INFINITY : mx + log2f(den));
   }
 
   QMK_STAMP(2);  // partial merged and stored
