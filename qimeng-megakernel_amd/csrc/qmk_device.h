@@ -26,6 +26,7 @@ constexpr int kWaveSize = 64;
 constexpr int kWaves = kThreads / kWaveSize;
 constexpr int kInstWords = QMK_INSTRUCTION_WORDS;
 constexpr int kMaxPartials = kInstWords - 7;   // reduction list capacity of one slot
+constexpr int kMaxSelfMerge = 64;              // split-KV fan-out when every O-proj workgroup merges for itself
 constexpr uint32_t kDefaultSpinLimit = 1u << 22;
 
 using u16 = uint16_t;

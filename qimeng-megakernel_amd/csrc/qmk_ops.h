@@ -11,13 +11,6 @@
 
 #include "qmk_device.h"
 
-#ifndef QMK_KV_AHEAD_LLAMA
-#define QMK_KV_AHEAD_LLAMA 1
-#endif
-#ifndef QMK_KV_AHEAD_QWEN
-#define QMK_KV_AHEAD_QWEN 1
-#endif
-
 namespace qmk {
 
 struct Llama1B {
@@ -29,7 +22,6 @@ struct Llama1B {
   static constexpr int GQA = NQ / NKV;
   static constexpr int QKV = (NQ + 2 * NKV) * D;
   static constexpr int KV_BLOCK = 16;  // split-KV partition granularity in tokens
-  static constexpr int KV_AHEAD = QMK_KV_AHEAD_LLAMA;  // cache rows a lane group asks for before it has q
   static constexpr bool QK_NORM = false;
 };
 
@@ -45,7 +37,6 @@ struct Qwen3_1p7B {
   static constexpr int GQA = NQ / NKV;
   static constexpr int QKV = (NQ + 2 * NKV) * D;
   static constexpr int KV_BLOCK = 16;
-  static constexpr int KV_AHEAD = QMK_KV_AHEAD_QWEN;
   static constexpr bool QK_NORM = true;
 };
 
@@ -422,10 +413,9 @@ __device__ __forceinline__ void merge_partials(const Params& p, int head0, int n
 // ===================================================================== 2 ==
 // [2, layer, kv_head, num_partials, partial_idx, merge_in_last]
 // Flash-decoding over one contiguous slice of the context for the GQA group of
-// one KV head.  A wave handles 8 tokens per pass: lane group g = lane/8 owns a
-// token, lane c = lane%8 owns D/8 neighbouring dims of K and V.  Every lane group keeps
-// its own running (max, sum, acc) per query head; groups, then waves, are
-// merged once at the end.  Scores live in the log2 domain.
+// one KV head.  A wave takes 16 tokens at a time (tiles w, w+8, ... of the slice) and keeps one
+// running (max, sum, acc) per query head; the eight wave states are merged once at the end.
+// Scores live in the log2 domain.
 //
 // The query heads and the K/V row appended in this launch are first staged in LDS (bf16:
 // [0, GQA*D) q, then k, then v) — from their tagged units, or after the per-head counters from
@@ -441,9 +431,7 @@ __device__ __forceinline__ void merge_partials(const Params& p, int head0, int n
 template <class M>
 __device__ bool op_attn_splitkv(const Params& p, Smem<M>& s, const Ctx& c) {
   constexpr int D = M::D, GQA = M::GQA;
-  constexpr int DPL = D / 8;   // dims of K and V one lane owns
-  constexpr int VPL = DPL / 8; // 16-byte vectors per lane and row
-  static_assert(D % 64 == 0 && GQA * D == 4 * kWaveSize, "four waves fold the GQA*D outputs; a lane owns whole 16-byte vectors");
+  static_assert(D % 64 == 0 && GQA <= 4 && GQA * D <= kThreads, "a lane owns whole 16-byte vectors of K; one thread per merged output");
   static_assert(!M::QK_NORM || D == 2 * kWaveSize, "the per-head norm gives every lane one rotation pair");
   const int layer = s.inst[1], kvh = s.inst[2], P = s.inst[3], part = s.inst[4];
   const int merge_mode = s.inst[5];  // 0: per-head counters, 1: last arrival merges, 2: the O-proj merges
@@ -849,7 +837,7 @@ __device__ bool op_oproj_residual(const Params& p, Smem<M>& s, const Ctx& c) {
     // no merging workgroup, no attn_out round trip, one synchronisation hop less.  Thread t owns
     // dims 4*(t%16).. of head t/16.
     const int P = self_merge;
-    if (P < 1 || P > kMaxPartials || P > p.max_splits) return bad_operand(p, s, c, 5);
+    if (P < 1 || P > kMaxSelfMerge || P > p.max_splits) return bad_operand(p, s, c, 5);  // no list to fit: any fan-out the workspaces hold
     if (!wg_wait_all(p, s, c, layer, ROW_REDUCE, 0, M::NKV * P)) return false;
     const int h = c.tid / (M::D / 4), d0 = 4 * (c.tid % (M::D / 4));
     const float* lse = p.attn_lse + static_cast<size_t>(h) * p.max_splits;

@@ -50,6 +50,8 @@ MAX_REDUCTION_LIST = ATTENTION_REDUCTION_LIST_CAPACITY
 #: kernel merges from registers and is bounded only by the instruction slot.
 REFERENCE_MAX_ATTENTION_PARTIALS = 16
 MAX_ATTENTION_PARTIALS = ATTENTION_REDUCTION_LIST_CAPACITY
+#: with the merge done by the O-proj workgroups no instruction lists the partials
+MAX_SELF_MERGE_PARTIALS = 64
 #: value of the split-KV instruction's ``merge_in_last`` word per merge mode
 ATTENTION_MERGE_MODES = {"separate": 0, "last": 1, "oproj": 2}
 #: KV tokens per split-KV partial the fan-out aims for: five passes of a workgroup (8 waves x 8
@@ -155,7 +157,7 @@ class DecodeScheduler:
         self.geometry.validate(self.shape)
         if self.sm_count < 1:
             raise ValueError("sm_count must be positive")
-        _validate_num_partials(self.num_partials)
+        _validate_num_partials(self.num_partials, MAX_SELF_MERGE_PARTIALS if self.attention_merge == "oproj" else MAX_ATTENTION_PARTIALS)
         if self.attention_merge not in ATTENTION_MERGE_MODES:
             raise ValueError(f"attention_merge must be one of {sorted(ATTENTION_MERGE_MODES)}")
 
@@ -293,7 +295,8 @@ def scheduler_for(globs: Any) -> DecodeScheduler:
     device = _get_device(globs)
     sm_count = _get_sm_count(device)
     kv_capacity = int(globs.k_cache.shape[2]) if getattr(globs, "k_cache", None) is not None else None
-    max_p = MAX_ATTENTION_PARTIALS
+    merge = os.environ.get("QMK_ATTENTION_MERGE", "oproj")
+    max_p = MAX_SELF_MERGE_PARTIALS if merge == "oproj" else MAX_ATTENTION_PARTIALS
     lse = getattr(globs, "attn_lse_intermediates", None)
     if lse is not None:
         max_p = min(max_p, int(lse.shape[-1]))
@@ -302,7 +305,7 @@ def scheduler_for(globs: Any) -> DecodeScheduler:
     if override:
         p = max(1, min(int(override), max_p))
     sched = mi355x_scheduler(sm_count=sm_count, num_partials=p,
-                             attention_merge=os.environ.get("QMK_ATTENTION_MERGE", "oproj"))
+                             attention_merge=merge)
     if cached == sched:
         return cached
     try:
