@@ -36,12 +36,19 @@ __global__ __launch_bounds__(kThreads, 1) void decode_megakernel(const Params p)
 
   const int32_t* queue = p.instructions + static_cast<size_t>(blockIdx.x) * p.num_insts * kInstWords;
   bool ok = true;
-  // The words of instruction i+1 are asked for while instruction i runs.
+  // Two instructions are visible at a time (the second one for requests made on its behalf); the
+  // words of instruction i+2 are asked for while instruction i runs.
   int32_t word = (threadIdx.x < kInstWords && p.num_insts > 0) ? queue[threadIdx.x] : 0;
+  int32_t word1 = (threadIdx.x < kInstWords && p.num_insts > 1) ? queue[kInstWords + threadIdx.x] : 0;
+  Carried carry;
+  bool carried = false, after_attention = false;
+  forget(carry);
   for (int i = 0; i < p.num_insts && ok; ++i) {
     if (threadIdx.x < kInstWords) {
       s.inst[threadIdx.x] = word;
-      if (i + 1 < p.num_insts) word = queue[(i + 1) * kInstWords + threadIdx.x];
+      s.next[threadIdx.x] = word1;
+      word = word1;
+      word1 = (i + 2 < p.num_insts) ? queue[(i + 2) * kInstWords + threadIdx.x] : 0;
     }
     __syncthreads();
     const int opcode = s.inst[0];
@@ -53,20 +60,28 @@ __global__ __launch_bounds__(kThreads, 1) void decode_megakernel(const Params p)
       t_start = wall_clock64();
       for (int k = 0; k < 4; ++k) s.stamps[k] = t_start;
     }
+    // Only the O-proj hands rows to its successor: every other arm ends their life explicitly.
     switch (opcode) {
-      case OP_NOOP: break;
-      case OP_RMS_QKV_ROPE: ok = op_rms_qkv_rope<M>(p, s, c); break;
-      case OP_ATTN_SPLITKV: ok = op_attn_splitkv<M>(p, s, c); break;
-      case OP_ATTN_REDUCE: ok = op_attn_reduce<M>(p, s, c); break;
-      case OP_OPROJ_RESIDUAL: ok = op_oproj_residual<M>(p, s, c); break;
-      case OP_RMS_UPGATE_SILU: ok = op_rms_upgate_silu<M>(p, s, c); break;
-      case OP_DOWN_RESIDUAL: ok = op_down_residual<M>(p, s, c); break;
-      case OP_RMS_LMHEAD: ok = op_rms_lmhead<M>(p, s, c); break;
+      case OP_NOOP: forget(carry); break;
+      case OP_RMS_QKV_ROPE: ok = op_rms_qkv_rope<M>(p, s, c); forget(carry); break;
+      case OP_ATTN_SPLITKV: ok = op_attn_splitkv<M>(p, s, c); forget(carry); break;
+      case OP_ATTN_REDUCE: ok = op_attn_reduce<M>(p, s, c); forget(carry); break;
+      case OP_OPROJ_RESIDUAL:
+        carried = M::CARRY_AFTER_ATTENTION || !after_attention;
+        ok = op_oproj_residual<M>(p, s, c, carry, carried);
+        break;
+      case OP_RMS_UPGATE_SILU: ok = op_rms_upgate_silu<M>(p, s, c, carry, carried); forget(carry); break;
+      case OP_DOWN_RESIDUAL: ok = op_down_residual<M>(p, s, c); forget(carry); break;
+      case OP_RMS_LMHEAD: ok = op_rms_lmhead<M>(p, s, c); forget(carry); break;
       default:
         if (threadIdx.x == 0) report_error(p, QMK_DEV_BAD_OPCODE, i, opcode, 0);
         ok = false;
+        forget(carry);
         break;
     }
+    if (opcode != OP_OPROJ_RESIDUAL) carried = false;
+    after_attention = opcode == OP_ATTN_SPLITKV || opcode == OP_ATTN_REDUCE;
+
     if (p.timeline != nullptr && threadIdx.x == 0) {
       uint64_t* rec = p.timeline + (static_cast<size_t>(blockIdx.x) * p.num_insts + i) * 8;
       rec[0] = t_start;

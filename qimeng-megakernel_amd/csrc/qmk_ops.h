@@ -22,6 +22,8 @@ struct Llama1B {
   static constexpr int GQA = NQ / NKV;
   static constexpr int QKV = (NQ + 2 * NKV) * D;
   static constexpr int KV_BLOCK = 16;  // split-KV partition granularity in tokens
+  static constexpr int CARRY_ROWS = 2;  // up/gate rows per wave requested by the O-proj before it
+  static constexpr bool CARRY_AFTER_ATTENTION = false;  // ... also by a workgroup that has just run attention
   static constexpr bool QK_NORM = false;
 };
 
@@ -37,6 +39,8 @@ struct Qwen3_1p7B {
   static constexpr int GQA = NQ / NKV;
   static constexpr int QKV = (NQ + 2 * NKV) * D;
   static constexpr int KV_BLOCK = 16;
+  static constexpr int CARRY_ROWS = 3;
+  static constexpr bool CARRY_AFTER_ATTENTION = true;
   static constexpr bool QK_NORM = true;
 };
 
@@ -45,6 +49,7 @@ constexpr int kResSlots = 4096;
 template <class M>
 struct Smem {
   int32_t inst[kInstWords];
+  int32_t next[kInstWords];             // the instruction after this one (zeros behind the last)
   int32_t ctl[8];                       // [0] abort, [1] last workgroup to retire
   uint32_t generation;                  // launch count of the tagged-activation workspace
   float best_val;                       // greedy candidate of this workgroup: largest bf16 logit so far ...
@@ -273,6 +278,48 @@ __device__ __forceinline__ void stream(int n, Src src, RowRegs<CH> (&buf)[NB], U
 #endif
 constexpr int kEarly = QMK_EARLY;                    // buffers of the down projection requested before its wait
 constexpr int kUpGateBuffers = QMK_UPGATE_BUFFERS;   // row buffers of the up/gate GEMV
+
+// Rows that one instruction requests for the next one of its queue: the O-proj has three of its
+// four row buffers to spare and waits for the whole attention phase, in which the memory system
+// has little to do; it asks for the up/gate rows that would otherwise be requested behind that wait.
+// (Only there: anywhere else such requests would stand in front of the stores that hand the
+// instruction's own results over.)
+constexpr int kOprojBuffers = 2;  // row buffers of the O-proj (8 rows per workgroup: one per wave)
+constexpr int kCarried = kUpGateBuffers - 1;  // at most; a model asks for M::CARRY_ROWS of them (measured)
+struct Carried {
+  RowRegs<4> row[kCarried];  // element wave + 8 * (k + 1) of the up/gate instruction
+};
+// The registers hold nothing of interest from here on (no instruction is generated: this only
+// ends their live range, so that they are not kept across the ops that do not use them).
+__device__ __forceinline__ void forget(Carried& c) {
+#pragma unroll
+  for (int k = 0; k < kCarried; ++k)
+#pragma unroll
+    for (int j = 0; j < 4; ++j) asm volatile("" : "=v"(c.row[k].v[j]));
+}
+
+// Row of element e of an up/gate instruction (words w): element 2i is the up row of the
+// instruction's i-th output, 2i + 1 its gate row.
+template <class M>
+__device__ __forceinline__ const u16* upgate_row(const Params& p, const int32_t* w, int layer, int tile, int e) {
+  const int i = e >> 1;
+  const int row = w[4 + i / tile] * tile + i % tile;
+  const u16* base = (e & 1) ? p.gate_w : p.up_w;
+  return base + (static_cast<size_t>(layer) * M::F + row) * M::H;
+}
+// Operand checks of an up/gate instruction; the index of the offending word, or -1.
+template <class M>
+__device__ __forceinline__ int upgate_check(const Params& p, const int32_t* w) {
+  const int layer = w[1], n = w[3];
+  if (layer < 0 || layer >= p.num_layers) return 1;
+  if (n < 0 || n > kInstWords - 6) return 3;
+  const int tile = w[5 + n];
+  if (tile <= 0 || (tile & 1) || M::F % tile != 0) return 5 + n;
+  if (n * tile * 2 > kResSlots) return 3;
+  for (int i = 0; i < n; ++i)
+    if (w[4 + i] < 0 || w[4 + i] >= M::F / tile) return 4 + i;
+  return -1;
+}
 
 // ===================================================================== 1 ==
 // [1, layer, tile_M, n_start, n_end, tile_M_g, tile_N_g]
@@ -800,7 +847,7 @@ __device__ __forceinline__ void residual_pair(u16* hidden_pair, float d0, float 
 // [4, layer, tile_M, n_start, n_end, reduction_block, tile_M_g, tile_N_g]
 // hidden[r] = bf16(hidden[r] + bf16(W_o[r] . attn_out))   (operations.py:251-262, 63-68)
 template <class M>
-__device__ bool op_oproj_residual(const Params& p, Smem<M>& s, const Ctx& c) {
+__device__ bool op_oproj_residual(const Params& p, Smem<M>& s, const Ctx& c, Carried& carry, bool& carried) {
   constexpr int CH = M::H / 512;
   static_assert(M::NQ * M::D == M::H, "attention output width equals the hidden size");
   const int layer = s.inst[1], nstart = s.inst[3], nend = s.inst[4], tile = s.inst[7];
@@ -814,7 +861,7 @@ __device__ bool op_oproj_residual(const Params& p, Smem<M>& s, const Ctx& c) {
   const u16* W = p.o_w + (static_cast<size_t>(layer) * M::H + rs) * M::H;
   auto src = [&](int r) { return W + static_cast<size_t>(r) * M::H; };
 
-  RowRegs<CH> buf[kDepth];
+  RowRegs<CH> buf[kOprojBuffers];
   preload<CH>(nrows, src, buf);
   static_assert(M::H == kThreads * 4, "one thread stages four elements");
   // Tagged mode: the rows' residual values are those the previous layer's down projection
@@ -827,6 +874,22 @@ __device__ bool op_oproj_residual(const Params& p, Smem<M>& s, const Ctx& c) {
       !residual_in(p, layer > 0 ? p.ws + kWsHiddenOut : nullptr, tag - 1, rs, c.tid, res_old)) {
     s.ctl[0] = 1;  // seen by everybody after the barrier inside the wait below
     report_error(p, QMK_DEV_WAIT_TIMEOUT, c.inst_idx, c.opcode, c.tid);
+  }
+  // The next instruction's rows, if it is the up/gate GEMV of this layer (see Carried).
+  // (`carried` comes in as "may": a workgroup that has just run this layer's attention starts late,
+  // and its requests would stand in front of its own reads of the partials.)
+  carried = carried && s.next[0] == OP_RMS_UPGATE_SILU && s.next[1] == layer && upgate_check<M>(p, s.next) < 0;
+  if (carried) {
+    const int un = s.next[3], utile = s.next[5 + un];
+    const int wave = c.tid >> 6;
+    static_assert(M::CARRY_ROWS <= kCarried, "the carried rows fit the up/gate ring");
+#pragma unroll
+    for (int k = 0; k < M::CARRY_ROWS; ++k) {
+      const int e = wave + (k + 1) * kWaves;
+      if (e < 2 * un * utile) load_row(carry.row[k], upgate_row<M>(p, s.next, layer, utile, e), lane);
+    }
+  } else {
+    forget(carry);
   }
   const int self_merge = s.inst[5];  // reduction_block_idx: 0, or the split-KV fan-out P when this op merges
   if (self_merge == 0) {
@@ -911,17 +974,13 @@ __device__ bool op_oproj_residual(const Params& p, Smem<M>& s, const Ctx& c) {
 // [5, layer, tile_M, n, block_0..block_{n-1}, tile_M_g, tile_N_g]
 // up = bf16(W_u y), gate = bf16(W_g y), silu_out = bf16(bf16(silu(gate)) * up)   (operations.py:265-282)
 template <class M>
-__device__ bool op_rms_upgate_silu(const Params& p, Smem<M>& s, const Ctx& c) {
+__device__ bool op_rms_upgate_silu(const Params& p, Smem<M>& s, const Ctx& c, const Carried& carry, bool carried) {
   constexpr int CH = M::H / 512;
+  static_assert(CH == 4, "the carried rows are 4 KiB");
+  const int bad = upgate_check<M>(p, s.inst);
+  if (bad >= 0) return bad_operand(p, s, c, bad);
   const int layer = s.inst[1], n = s.inst[3];
-  if (layer < 0 || layer >= p.num_layers) return bad_operand(p, s, c, 1);
-  if (n < 0 || n > kInstWords - 6) return bad_operand(p, s, c, 3);
   const int tile = s.inst[5 + n];
-  if (tile <= 0 || (tile & 1) || M::F % tile != 0) return bad_operand(p, s, c, 5 + n);
-  if (n * tile * 2 > kResSlots) return bad_operand(p, s, c, 3);
-  const int nblocks_total = M::F / tile;
-  for (int i = 0; i < n; ++i)
-    if (s.inst[4 + i] < 0 || s.inst[4 + i] >= nblocks_total) return bad_operand(p, s, c, 4 + i);
 
   const int lane = c.tid & 63;
   const int nout = n * tile;       // output elements of this instruction
@@ -929,13 +988,20 @@ __device__ bool op_rms_upgate_silu(const Params& p, Smem<M>& s, const Ctx& c) {
   const u16* Wu = p.up_w + static_cast<size_t>(layer) * M::F * M::H;
   const u16* Wg = p.gate_w + static_cast<size_t>(layer) * M::F * M::H;
   auto row_of = [&](int i) { return s.inst[4 + i / tile] * tile + i % tile; };
-  auto src = [&](int e) { return ((e & 1) ? Wg : Wu) + static_cast<size_t>(row_of(e >> 1)) * M::H; };
+  auto src = [&](int e) { return upgate_row<M>(p, s.inst, layer, tile, e); };
 
   RowRegs<CH> buf[kUpGateBuffers];
+  if (carried) {  // the O-proj before this instruction has asked for the elements of buffers 1..
+#pragma unroll
+    for (int k = 0; k < M::CARRY_ROWS; ++k) buf[k + 1] = carry.row[k];
+  }
   const bool tg = tagged(p);
   if (!rms_to_lds<M, kUpGateBuffers>(
           p, s, c, tg ? p.ws + kWsHiddenMid : nullptr, tag_of(s.generation, layer), p.mlp_norm + static_cast<size_t>(layer) * M::H,
-          [&](auto k) { preload_range<decltype(k)::value, decltype(k)::value + 1>(nrows, src, buf); },
+          [&](auto k) {
+            constexpr int kk = decltype(k)::value;
+            if (kk == 0 || kk > M::CARRY_ROWS || !carried) preload_range<kk, kk + 1>(nrows, src, buf);
+          },
           [&] { return wg_wait_all(p, s, c, layer, ROW_OPROJ, 0, p.oproj_blocks); }))
     return false;
   QMK_STAMP(0);
