@@ -52,6 +52,8 @@ REFERENCE_MAX_ATTENTION_PARTIALS = 16
 MAX_ATTENTION_PARTIALS = ATTENTION_REDUCTION_LIST_CAPACITY
 #: with the merge done by the O-proj workgroups no instruction lists the partials
 MAX_SELF_MERGE_PARTIALS = 64
+#: the first XCD_COUNT workgroups lead the per-XCD waits of the kernel (qmk_device.h, wait_edge_xcd)
+XCD_COUNT = 8
 #: value of the split-KV instruction's ``merge_in_last`` word per merge mode
 ATTENTION_MERGE_MODES = {"separate": 0, "last": 1, "oproj": 2}
 #: KV tokens per split-KV partial the fan-out aims for: five passes of a workgroup (8 waves x 8
@@ -152,6 +154,9 @@ class DecodeScheduler:
     #: who merges the split-KV partials: "separate" reduction instructions (the reference), the
     #: "last" split-KV arrival of a head group, or every "oproj" workgroup for itself
     attention_merge: str = "separate"
+    #: give the queues that have just run a split-KV instruction no O-proj rows (their turn in the
+    #: round is a no-op): they start late and would otherwise finish the MLP behind everybody else
+    oproj_spares_attention: bool = False
 
     def __post_init__(self) -> None:
         self.geometry.validate(self.shape)
@@ -188,10 +193,29 @@ class DecodeScheduler:
             for head0 in range(0, self.shape.num_attention_heads, step)
         ]
 
-    def oproj(self, layer_idx: int) -> list[Instruction]:
+    def oproj(self, layer_idx: int, first_queue: int = 0) -> list[Instruction]:
+        """``first_queue``: the queue the first instruction of this round is dealt to."""
         g = self.geometry.oproj_tile_n
         blocks = _ceil_div(self.shape.hidden_size, g)
         merges = self.num_partials if self.attention_merge == "oproj" else 0
+        n_attn = self.shape.num_key_value_heads * self.num_partials
+        if self.oproj_spares_attention and self.attention_merge == "oproj" and 0 < n_attn < self.sm_count:
+            # The split-KV instructions directly precede this round: they went to the n_attn queues
+            # before first_queue.  The kernel's per-XCD wait on this edge is led by the first
+            # XCD_COUNT queues, which therefore always keep their rows.
+            sm = self.sm_count
+            attention = {(first_queue - 1 - k) % sm for k in range(n_attn)}
+            works = [((first_queue + j) % sm) not in attention or ((first_queue + j) % sm) < XCD_COUNT for j in range(sm)]
+            if sum(works) <= blocks:
+                spans = iter(_split_n_tiles(blocks, sum(works)))
+                out: list[Instruction] = []
+                for w in works:
+                    if w:
+                        lo, hi = next(spans)
+                        out.append(OProj_GEMV_Residual(layer_idx, 0, lo, hi, merges, tile_N_granularity=g))
+                    else:
+                        out.append(NoOp())
+                return out
         return [
             OProj_GEMV_Residual(layer_idx, 0, lo, hi, merges, tile_N_granularity=g)
             for lo, hi in _split_n_tiles(blocks, self.sm_count)
@@ -238,12 +262,16 @@ class DecodeScheduler:
         ]
 
     # ---- whole step ------------------------------------------------------
-    def layer(self, layer_idx: int) -> list[Instruction]:
-        return [
+    def layer(self, layer_idx: int, start: int = 0) -> list[Instruction]:
+        """``start``: instructions dealt before this layer's (the round-robin carries on from there)."""
+        head = [
             *self.qkvproj(layer_idx),
             *self.attention_split_kv(layer_idx),
             *self.attention_reduction(layer_idx),
-            *self.oproj(layer_idx),
+        ]
+        return [
+            *head,
+            *self.oproj(layer_idx, (start + len(head)) % self.sm_count),
             *self.upgate(layer_idx),
             *self.downproj(layer_idx),
         ]
@@ -252,7 +280,7 @@ class DecodeScheduler:
         layers = self.shape.num_hidden_layers if num_layers is None else num_layers
         out: list[Instruction] = []
         for layer_idx in range(layers):
-            out.extend(self.layer(layer_idx))
+            out.extend(self.layer(layer_idx, len(out)))
         if layers == self.shape.num_hidden_layers:
             out.extend(self.lmhead())
         return out
@@ -286,7 +314,8 @@ def mi355x_scheduler(
     if blocks % sm_count != 0 and (2 * blocks) % sm_count == 0:
         geometry = dataclasses.replace(geometry, upgate_tile_n=geometry.upgate_tile_n // 2)
     p = num_partials or pick_num_partials(sm_count, kv_capacity, shape=shape)
-    return DecodeScheduler(shape, geometry, sm_count, p, attention_merge)
+    return DecodeScheduler(shape, geometry, sm_count, p, attention_merge,
+                           oproj_spares_attention=os.environ.get("QMK_OPROJ_SPARES", "1") != "0")
 
 
 def scheduler_for(globs: Any) -> DecodeScheduler:
