@@ -34,8 +34,8 @@ sys.path.insert(0, str(ROOT))
 HBM_PEAK_GBPS = 8000.0
 # HBM bytes one launch moves, from the two rocprofv3 --pmc runs (FETCH_SIZE, WRITE_SIZE; each scaled by
 # what the same counter reads for a 1 GiB copy) summarised in profiles/decode_megakernel_llama1b_hbm_counters.txt:
-# 1.0064 x the algorithmic bytes of the profiled launches.  Not measured in this process.
-MEASURED_TRAFFIC_OVER_ALGORITHMIC = 1.0064
+# 1.0069 x the algorithmic bytes of the profiled launches.  Not measured in this process.
+MEASURED_TRAFFIC_OVER_ALGORITHMIC = 1.0069
 
 
 def cpu_baseline(shape, weights, prompt, n_steps: int, cores: int, shape_name: str) -> dict:
