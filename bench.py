@@ -70,6 +70,52 @@ def cpu_baseline(shape, weights, prompt, n_steps: int, cores: int, shape_name: s
     }
 
 
+def attention_stress(contexts=(4096, 16384, 32768)) -> dict:
+    """Split-KV attention at long contexts: one decode step per context on a 2-layer model of the
+    Llama-3.2-1B layer geometry with the KV cache filled with ~N(0,1) rows.  The phase is timed by
+    the kernel's own timeline records (100 MHz clock): from the end of the last QKV instruction of
+    layer 1 to the end of its last split-KV instruction.  K/V bytes of a layer = context x KV heads
+    x head_dim x 2 B x 2."""
+    import dataclasses
+
+    import numpy as np
+    import torch
+
+    from qimeng_megakernel_amd import synthetic
+    from qimeng_megakernel_amd.decode_schedule import mk_kernel
+    from qimeng_megakernel_amd.decode_schedule.instructions import scheduler as S
+    from qimeng_megakernel_amd.decode_schedule.model_config import LLAMA_3_2_1B, LlamaConfig
+
+    shape = dataclasses.replace(LLAMA_3_2_1B, num_hidden_layers=2, vocab_size=4096)
+    LlamaConfig.set_shape(shape)
+    out = {}
+    for ctx in contexts:
+        w = synthetic.random_weights(shape, 0, ctx)
+        g = synthetic.build_globals(w, shape, ctx, "cuda:0", max_partials=32)
+        g.k_cache.normal_(); g.v_cache.normal_()
+        S.build(g)
+        mk = mk_kernel.get_mk()
+        nq, ni = g.instructions.shape[:2]
+        timeline = torch.zeros(nq, ni, 8, dtype=torch.int64, device="cuda:0")
+        g.position_id = ctx - 1
+        for _ in range(2):
+            g.hidden_states.copy_(g.embed_tokens[5])
+            mk_kernel.call_mk(g, mk)
+        mk.timeline = timeline
+        g.hidden_states.copy_(g.embed_tokens[5])
+        mk_kernel.call_mk(g, mk)
+        torch.cuda.synchronize()
+        mk.check()
+        t = timeline.cpu().numpy().astype(np.int64)
+        op, layer = t[..., 3] & 0xFF, (t[..., 3] >> 8) & 0xFFFF
+        qkv_end = t[..., 2][(op == 1) & (layer == 1)].max()
+        attn_end = t[..., 2][(op == 2) & (layer == 1)].max()
+        us = (attn_end - qkv_end) / 100.0
+        kv_bytes = ctx * shape.num_key_value_heads * shape.head_dim * 2 * 2
+        out[str(ctx)] = {"partials": S.scheduler_for(g).num_partials, "phase_us": us, "GBps": kv_bytes / us / 1e3}
+    return out
+
+
 def main() -> None:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -86,6 +132,9 @@ def main() -> None:
                     help="argmax and embedding lookup on the host between launches, as the reference's loop does "
                          "(default: inside the kernel)")
     ap.add_argument("--no-graph-run", action="store_true", help="skip the extra untimed-per-step HIP-graph run")
+    ap.add_argument("--attention-stress", action="store_true",
+                    help="instead of the decode request: the split-KV attention phase at contexts 4096/16384/32768 "
+                         "(one JSON line, metric attention_phase_GBps)")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also run one 1 GiB device-to-device copy (a kernel of known traffic, for scaling rocprofv3 counters)")
     args = ap.parse_args()
@@ -106,6 +155,13 @@ def main() -> None:
     from qimeng_megakernel_amd.decode_schedule import mk_kernel
     from qimeng_megakernel_amd.decode_schedule.model_config import LLAMA_3_2_1B, QWEN3_1_7B, LlamaConfig
 
+    if args.attention_stress:
+        res = attention_stress()
+        print(json.dumps({"metric": "attention_phase_GBps", "unit": "GB/s", "n_gpus": 1, "higher_is_better": True,
+                          "dtype": "bf16", "data": "synthetic",
+                          "config": {"workload": "Llama-3.2-1B layer geometry, batch 1, one decode step, KV cache ~N(0,1)"},
+                          "value": res[max(res, key=int)]["GBps"], "contexts": res}))
+        return
     shape = LLAMA_3_2_1B if args.model == "llama-3.2-1b" else QWEN3_1_7B
     model_name = "Llama-3.2-1B" if args.model == "llama-3.2-1b" else "Qwen3-1.7B"
     LlamaConfig.set_shape(shape)
