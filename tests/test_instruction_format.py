@@ -288,3 +288,41 @@ def test_tensorize_pads_with_noops():
     t = S.tensorize_instructions(g, queues)
     assert t.shape == (2, 2, 32) and t.dtype == torch.int32 and g.instructions is t
     assert t[1, 1].tolist() == [0] * 32 and t[0, 1, :5].tolist() == [7, 1, 2, 1, 16]
+
+
+@pytest.mark.parametrize("shape_name,partials", [("llama", 4), ("llama", 32), ("qwen", 4)])
+def test_oproj_round_spares_the_queues_that_ran_attention(shape_name, partials):
+    """MI355X schedule: in every layer the queues that were dealt a split-KV instruction get a no-op
+    in the O-proj round, except queues 0..7 (they lead the kernel's per-XCD waits); the O-proj rows
+    are still covered exactly once, and nobody gets more than two 8-row tiles."""
+    from qimeng_megakernel_amd.decode_schedule.model_config import QWEN3_1_7B
+
+    shape = LLAMA_3_2_1B if shape_name == "llama" else QWEN3_1_7B
+    sched = S.mi355x_scheduler(shape, num_partials=partials)
+    queues = sched.queues(num_layers=10)          # the round-robin origin moves by 32 queues per layer
+    sm = sched.sm_count
+    for layer in range(10):
+        attention = {q for q in range(sm) if any(i.opcode() == 2 and i.layer_idx == layer for i in queues[q])}
+        assert len(attention) == shape.num_key_value_heads * partials
+        rows = []
+        for q in range(sm):
+            mine = [i for i in queues[q] if i.opcode() == 4 and i.layer_idx == layer]
+            if q in attention and q >= S.XCD_COUNT and len(attention) < sm:   # all queues in attention: nobody to spare
+                assert mine == []
+                # its slot in the round is a no-op right behind its split-KV instruction
+                at = next(k for k, i in enumerate(queues[q]) if i.opcode() == 2 and i.layer_idx == layer)
+                assert queues[q][at + 1].opcode() == 0
+            else:
+                assert len(mine) == 1 and 1 <= mine[0].tile_N_end_idx - mine[0].tile_N_start_idx <= 2
+                t = mine[0].tile_N_granularity
+                rows += range(mine[0].tile_N_start_idx * t, mine[0].tile_N_end_idx * t)
+        assert sorted(rows) == list(range(shape.hidden_size))
+    # switched off, every queue has O-proj rows again
+    plain = dataclasses_replace(sched, oproj_spares_attention=False)
+    assert all(i.opcode() == 4 for i in plain.oproj(0))
+
+
+def dataclasses_replace(obj, **kw):
+    import dataclasses
+
+    return dataclasses.replace(obj, **kw)
