@@ -84,6 +84,29 @@ def test_op_attention_split_and_reduce(state, which, pos, P):
     assert torch.equal(gpu.barriers.cpu(), cpu.barriers)
 
 
+@pytest.mark.parametrize("pos,P", [(95, 32), (33, 32), (7, 32), (64, 40)])
+def test_op_attention_fan_out_beyond_the_reduction_list(state, pos, P):
+    """With the O-proj workgroups merging the partials themselves no instruction lists them, so the
+    fan-out may exceed the 25 entries a reduction instruction holds (up to one workgroup per CU and
+    KV head); most slices are then shorter than one 16-token tile, many are empty."""
+    shape, cpu, gpu = state
+    cpu2, gpu2 = pair(synthetic.random_weights(shape, 0, 96), shape, max_partials=P)
+    for name in ("hidden_states", "q_post_rope", "k_cache", "v_cache"):
+        getattr(cpu2, name).copy_(getattr(cpu, name))
+    sched = _sched(shape, "mi355x", P)
+    cpu2.position_id = pos
+    cpu2.barriers[0, 0, :] = sched.expected_counts()[0]
+    sync_state(cpu2, gpu2)
+    run_both(cpu2, gpu2, sched, sched.attention_split_kv(0) + sched.oproj(0))
+    lse_c, lse_g = cpu2.attn_lse_intermediates[:, :P], gpu2.attn_lse_intermediates[:, :P].cpu()
+    assert torch.equal(torch.isinf(lse_c), torch.isinf(lse_g))
+    fin = torch.isfinite(lse_c)
+    assert (lse_c[fin] - lse_g[fin]).abs().max() < 2e-4
+    assert (cpu2.attn_out_intermediates[:, :P] - gpu2.attn_out_intermediates[:, :P].cpu()).abs().max() < 2e-4
+    bf16_close(gpu2.attn_out, cpu2.attn_out, name="attn_out", frac=0.03)
+    assert torch.equal(gpu2.barriers.cpu(), cpu2.barriers)
+
+
 @pytest.mark.parametrize("which", ["mi355x", "reference"])
 def test_op_oproj(state, which):
     shape, cpu, gpu = state
