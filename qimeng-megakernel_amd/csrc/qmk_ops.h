@@ -123,7 +123,8 @@ __device__ __forceinline__ bool wg_wait_all(const Params& p, Smem<M>& s, const C
   if (!xcd_counters(p))
     return wg_wait(p, s, c, 1, [&](int) { return counter_ptr(p, layer, row, slot); }, expected);
   if (c.tid < kXcds) {
-    if (!wait_edge_xcd(p, layer, row, expected, p.spin_limit) && c.tid == 0) {
+    // The attention edge has one producer per split-KV instruction: everybody polls it directly.
+    if (!wait_edge_xcd(p, layer, row, expected, p.spin_limit, row != ROW_REDUCE) && c.tid == 0) {
       s.ctl[0] = 1;
       report_error(p, QMK_DEV_WAIT_TIMEOUT, c.inst_idx, c.opcode, row);
     }

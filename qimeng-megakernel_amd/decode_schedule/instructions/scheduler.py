@@ -52,8 +52,6 @@ REFERENCE_MAX_ATTENTION_PARTIALS = 16
 MAX_ATTENTION_PARTIALS = ATTENTION_REDUCTION_LIST_CAPACITY
 #: with the merge done by the O-proj workgroups no instruction lists the partials
 MAX_SELF_MERGE_PARTIALS = 64
-#: the first XCD_COUNT workgroups lead the per-XCD waits of the kernel (qmk_device.h, wait_edge_xcd)
-XCD_COUNT = 8
 #: value of the split-KV instruction's ``merge_in_last`` word per merge mode
 ATTENTION_MERGE_MODES = {"separate": 0, "last": 1, "oproj": 2}
 #: KV tokens per split-KV partial the fan-out aims for: five passes of a workgroup (8 waves x 8
@@ -201,11 +199,10 @@ class DecodeScheduler:
         n_attn = self.shape.num_key_value_heads * self.num_partials
         if self.oproj_spares_attention and self.attention_merge == "oproj" and 0 < n_attn < self.sm_count:
             # The split-KV instructions directly precede this round: they went to the n_attn queues
-            # before first_queue.  The kernel's per-XCD wait on this edge is led by the first
-            # XCD_COUNT queues, which therefore always keep their rows.
+            # before first_queue.
             sm = self.sm_count
             attention = {(first_queue - 1 - k) % sm for k in range(n_attn)}
-            works = [((first_queue + j) % sm) not in attention or ((first_queue + j) % sm) < XCD_COUNT for j in range(sm)]
+            works = [((first_queue + j) % sm) not in attention for j in range(sm)]
             if sum(works) <= blocks:
                 spans = iter(_split_n_tiles(blocks, sum(works)))
                 out: list[Instruction] = []

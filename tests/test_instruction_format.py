@@ -293,8 +293,8 @@ def test_tensorize_pads_with_noops():
 @pytest.mark.parametrize("shape_name,partials", [("llama", 4), ("llama", 32), ("qwen", 4)])
 def test_oproj_round_spares_the_queues_that_ran_attention(shape_name, partials):
     """MI355X schedule: in every layer the queues that were dealt a split-KV instruction get a no-op
-    in the O-proj round, except queues 0..7 (they lead the kernel's per-XCD waits); the O-proj rows
-    are still covered exactly once, and nobody gets more than two 8-row tiles."""
+    in the O-proj round; the O-proj rows are still covered exactly once, and nobody gets more than
+    two 8-row tiles."""
     from qimeng_megakernel_amd.decode_schedule.model_config import QWEN3_1_7B
 
     shape = LLAMA_3_2_1B if shape_name == "llama" else QWEN3_1_7B
@@ -307,7 +307,7 @@ def test_oproj_round_spares_the_queues_that_ran_attention(shape_name, partials):
         rows = []
         for q in range(sm):
             mine = [i for i in queues[q] if i.opcode() == 4 and i.layer_idx == layer]
-            if q in attention and q >= S.XCD_COUNT and len(attention) < sm:   # all queues in attention: nobody to spare
+            if q in attention and len(attention) < sm:   # all queues in attention: nobody to spare
                 assert mine == []
                 # its slot in the round is a no-op right behind its split-KV instruction
                 at = next(k for k, i in enumerate(queues[q]) if i.opcode() == 2 and i.layer_idx == layer)
