@@ -1,0 +1,121 @@
+"""CPU oracle of the batch decode route (B rows) — TEST INFRASTRUCTURE, not product code.
+
+Only ``tests/`` may import this module, and only as the checker.
+
+The reference has no separate fused route for batch sizes above one: its single-batch fused
+operations work on ``[B, H]`` activations
+(``…/A100/multi_batch/decode_schedule/fused/__init__.py:1-18`` re-exports
+``…/A100/single_batch/decode_schedule/fused/operations.py``).  Restated here, per function:
+
+=========================  =====================================================
+``qkv_rope``               fused/operations.py:151-215  (per-row position, inactive rows write nothing)
+``attention``              fused/operations.py:218-248  (inactive rows: attn_out row zeroed)
+``oproj_residual``         fused/operations.py:251-262  (inactive rows add zero)
+``mlp_upgate``             fused/operations.py:265-282  (inactive rows: silu_out row zeroed)
+``mlp_down_residual``      fused/operations.py:285-295
+``lm_head``                fused/operations.py:303-321  (inactive rows: logits -1e9)
+=========================  =====================================================
+
+Pinning: tests/test_mb_oracle.py checks every row of a batch against the batch-1 oracle
+(``fused_oracle.FusedOracle``, itself pinned against closed forms and the imported reference) on
+the same weights — bit for bit where the reference's arithmetic is row-wise, which is everywhere
+except the accumulation order inside a GEMM with B columns, left unspecified by the reference — and
+against the fixture that tests/golden/make_fixtures_mb.py wrote from the imported reference while
+stepping this oracle in lock-step with it.
+"""
+from __future__ import annotations
+
+import math
+from typing import Any
+
+import torch
+import torch.nn.functional as F
+
+from fused_oracle import gemv, rms_norm, rotate_pairs
+
+Tensor = torch.Tensor
+
+
+def _row_active(g: Any, b: int) -> bool:
+    mask = getattr(g, "active_mask", None)
+    return True if mask is None else bool(mask[b])
+
+
+def _pos(g: Any, b: int) -> int:
+    ids = getattr(g, "position_ids", None)
+    return int(ids[b]) if ids is not None else int(g.position_id or 0)
+
+
+class FusedBatchOracle:
+    def __init__(self, shape: Any):
+        self.shape = shape
+
+    def qkv_rope(self, g: Any, layer: int) -> None:
+        s = self.shape
+        nq, nkv, d = s.num_attention_heads, s.num_key_value_heads, s.head_dim
+        y = rms_norm(g.hidden_states, g.attn_norm_weights[layer], s.rms_norm_eps)
+        qkv = gemv(g.qkv_weights[layer], y)                       # bf16 [B, (nq + 2 nkv) d]: rounded before RoPE
+        B = qkv.shape[0]
+        q = qkv[:, : nq * d].view(B, nq, d)
+        k = qkv[:, nq * d : (nq + nkv) * d].view(B, nkv, d)
+        v = qkv[:, (nq + nkv) * d :].view(B, nkv, d)
+        for b in range(B):
+            if not _row_active(g, b):
+                continue
+            pos = _pos(g, b)
+            cos, sin = g.rope_cos[pos].view(1, -1), g.rope_sin[pos].view(1, -1)   # fp32: the products are fp32
+            qr = q[b] * cos + rotate_pairs(q[b]) * sin
+            kr = k[b] * cos + rotate_pairs(k[b]) * sin
+            g.q_post_rope[b].copy_(qr.reshape(-1).to(g.q_post_rope.dtype))
+            g.k_cache[layer, b, pos].copy_(kr.to(g.k_cache.dtype))
+            g.v_cache[layer, b, pos].copy_(v[b].to(g.v_cache.dtype))
+
+    def attention(self, g: Any, layer: int) -> None:
+        s = self.shape
+        nq, d, ratio = s.num_attention_heads, s.head_dim, s.num_attention_heads // s.num_key_value_heads
+        for b in range(g.hidden_states.shape[0]):
+            if not _row_active(g, b):
+                g.attn_out[b].zero_()
+                continue
+            n = _pos(g, b) + 1
+            q = g.q_post_rope[b].view(nq, d).float()
+            k = g.k_cache[layer, b, :n].float().repeat_interleave(ratio, dim=1)   # [n, nq, d]
+            v = g.v_cache[layer, b, :n].float().repeat_interleave(ratio, dim=1)
+            scores = torch.einsum("hi,shi->hs", q, k) * (1 / math.sqrt(d))
+            out = torch.einsum("hs,sho->ho", torch.softmax(scores, dim=-1), v)
+            g.attn_out[b].copy_(out.reshape(-1).to(g.attn_out.dtype))
+
+    def _masked(self, g: Any, rows: Tensor, fill: float = 0.0) -> Tensor:
+        for b in range(rows.shape[0]):
+            if not _row_active(g, b):
+                rows[b] = fill
+        return rows
+
+    def oproj_residual(self, g: Any, layer: int) -> None:
+        g.hidden_states.add_(self._masked(g, gemv(g.o_proj_weights[layer], g.attn_out)).to(g.hidden_states.dtype))
+
+    def mlp_upgate(self, g: Any, layer: int) -> None:
+        y = rms_norm(g.hidden_states, g.mlp_norm_weights[layer], self.shape.rms_norm_eps)
+        up, gate = gemv(g.up_proj_weights[layer], y), gemv(g.gate_proj_weights[layer], y)
+        g.silu_out.copy_(self._masked(g, F.silu(gate) * up).to(g.silu_out.dtype))
+
+    def mlp_down_residual(self, g: Any, layer: int) -> None:
+        g.hidden_states.add_(self._masked(g, gemv(g.down_proj_weights[layer], g.silu_out)).to(g.hidden_states.dtype))
+
+    def lm_head(self, g: Any) -> None:
+        y = rms_norm(g.hidden_states, g.lm_head_norm_weights, self.shape.rms_norm_eps)
+        g.logits.copy_(self._masked(g, gemv(g.lm_head_weights, y).to(g.logits.dtype), -1e9))
+
+    def decode_layer(self, g: Any, layer: int) -> None:
+        self.qkv_rope(g, layer)
+        self.attention(g, layer)
+        self.oproj_residual(g, layer)
+        self.mlp_upgate(g, layer)
+        self.mlp_down_residual(g, layer)
+
+    def decode_step(self, g: Any, num_layers: int | None = None) -> None:
+        layers = self.shape.num_hidden_layers if num_layers is None else num_layers
+        for layer in range(layers):
+            self.decode_layer(g, layer)
+        if layers == self.shape.num_hidden_layers:
+            self.lm_head(g)

@@ -1,0 +1,231 @@
+"""Scheduler of the batch route (B <= 16: one M tile).
+
+Two layouts, both the reference's (`…/A100/multi_batch/decode_schedule/instructions/scheduler.py`):
+
+* ``instruction_list`` / ``queues``: the instructions of a step in dependency order, dealt
+  round-robin (`:399-440`); the split-KV instructions carry the context length and activity the
+  request has when the list is built.
+* ``runtime_queues``: a template built once per request (`:443-537`): every op starts on a fresh
+  round of the workers (short ops are padded with no-ops, the RMSNorm rows occupy the first B
+  workers of a round), and the attention instructions leave length and activity to the
+  ``position_ids`` / ``active_mask`` of the launch.
+
+``workers`` is the number of instruction queues: 2 per SM on the reference's A100 (216), one per
+CU on MI355X (256).
+"""
+from __future__ import annotations
+
+import dataclasses
+from dataclasses import dataclass
+from typing import Any, Sequence
+
+from ...decode_schedule.model_config import DecodeShape, LlamaConfig
+from ...instruction import INTS_PER_INSTRUCTION, Instruction
+from ..decode_state import decode_pos_id, row_active
+from .instruction_defs import (
+    MAX_BATCH,
+    TILE_N_GRANULARITY,
+    AttnRMS,
+    DecodeAttentionReduction,
+    DecodeAttentionSplitKV,
+    DownProj_GEMM_Residual,
+    LMHeadProj_GEMM,
+    LMHeadRMS,
+    MlpRMS,
+    NoOp,
+    OProj_GEMM_Residual,
+    QKVProj_GEMM_RoPE,
+    UpGateProj_GEMM_SiLU,
+)
+
+ATTN_REDUCTION_SIZE = 4
+MAX_TILE_BLOCKS_PER_INSTRUCTION = INTS_PER_INSTRUCTION - 6
+MAX_REDUCTION_LIST = INTS_PER_INSTRUCTION - 5
+A100_WORKERS = 108 * 2
+MI355X_WORKERS = 256
+
+
+def _ceil_div(a: int, b: int) -> int:
+    return -(-a // b)
+
+
+def _spans(n: int, parts: int) -> list[tuple[int, int]]:
+    """Contiguous, as-even-as-possible cut of n blocks into at most ``parts`` spans."""
+    if n <= 0:
+        return []
+    groups = min(n, parts)
+    small, extra = divmod(n, groups)
+    out, lo = [], 0
+    for g in range(groups):
+        hi = lo + small + (1 if g < extra else 0)
+        out.append((lo, hi))
+        lo = hi
+    return out
+
+
+def partials_for_blocks(active_rows: int, max_blocks: int, workers: int, kv_heads: int) -> int:
+    """Split-KV fan-out: about one split-KV instruction per worker, never more slices than 16-token
+    blocks, never more than a reduction instruction can list (`scheduler.py:351-376`)."""
+    if active_rows <= 0:
+        return 1
+    max_blocks = max(1, max_blocks)
+    target = min(workers, active_rows * kv_heads * max_blocks)
+    p = _ceil_div(target, active_rows * kv_heads)
+    return min(MAX_REDUCTION_LIST, max(1, min(p, max_blocks)))
+
+
+@dataclass
+class BatchScheduler:
+    shape: DecodeShape
+    workers: int
+    batch_size: int
+
+    def __post_init__(self) -> None:
+        if not 1 <= self.batch_size <= MAX_BATCH:
+            raise ValueError(f"batch size must be in [1, {MAX_BATCH}], got {self.batch_size}")
+        if self.workers < 1:
+            raise ValueError("workers must be positive")
+
+    # ---- per-op emitters ---------------------------------------------------
+    def attn_rms(self, layer: int) -> list[Instruction]:
+        return [AttnRMS(layer, self.batch_size, batch_row=r) for r in range(self.batch_size)]
+
+    def mlp_rms(self, layer: int) -> list[Instruction]:
+        return [MlpRMS(layer, self.batch_size, batch_row=r) for r in range(self.batch_size)]
+
+    def lmhead_rms(self) -> list[Instruction]:
+        return [LMHeadRMS(self.batch_size, batch_row=r) for r in range(self.batch_size)]
+
+    def qkvproj(self, layer: int) -> list[Instruction]:
+        blocks = _ceil_div(self.shape.qkv_out_dim, TILE_N_GRANULARITY)
+        return [QKVProj_GEMM_RoPE(layer, self.batch_size, 0, lo, hi) for lo, hi in _spans(blocks, self.workers)]
+
+    def oproj(self, layer: int) -> list[Instruction]:
+        blocks = _ceil_div(self.shape.hidden_size, TILE_N_GRANULARITY)
+        return [OProj_GEMM_Residual(layer, self.batch_size, 0, lo, hi, 0) for lo, hi in _spans(blocks, self.workers)]
+
+    def upgate(self, layer: int) -> list[Instruction]:
+        blocks = _ceil_div(self.shape.intermediate_size, TILE_N_GRANULARITY)
+        out: list[Instruction] = []
+        for lo, hi in _spans(blocks, self.workers):
+            mine = list(range(lo, hi))
+            for at in range(0, len(mine), MAX_TILE_BLOCKS_PER_INSTRUCTION):
+                out.append(UpGateProj_GEMM_SiLU(layer, self.batch_size, 0, mine[at : at + MAX_TILE_BLOCKS_PER_INSTRUCTION]))
+        return out
+
+    def downproj(self, layer: int) -> list[Instruction]:
+        blocks = _ceil_div(self.shape.hidden_size, TILE_N_GRANULARITY)
+        return [DownProj_GEMM_Residual(layer, self.batch_size, 0, lo, hi) for lo, hi in _spans(blocks, self.workers)]
+
+    def lmhead(self) -> list[Instruction]:
+        blocks = _ceil_div(self.shape.vocab_size, TILE_N_GRANULARITY)
+        return [LMHeadProj_GEMM(self.batch_size, lo, hi) for lo, hi in _spans(blocks, self.workers)]
+
+    def attention_split_kv(self, layer: int, num_partials: int, globs: Any = None) -> list[Instruction]:
+        """With ``globs``: length and activity fixed from the request's present state; without: left
+        to the launch (seq_len = is_active = -1)."""
+        kvb = self.shape.attn_kv_block_size
+        out: list[Instruction] = []
+        for b in range(self.batch_size):
+            if globs is not None:
+                on = row_active(globs, b)
+                lens = getattr(globs, "kv_lengths", None)
+                seq_len = int(lens[b]) if lens is not None else decode_pos_id(globs, b) + 1
+                total = max(1, _ceil_div(seq_len, kvb)) if on else 0
+                per = max(1, _ceil_div(total, num_partials)) if on else 1
+            for kvh in range(self.shape.num_key_value_heads):
+                for part in range(num_partials):
+                    if globs is None:
+                        out.append(DecodeAttentionSplitKV(layer, b, kvh, num_partials, part))
+                        continue
+                    t0 = part * per * kvb
+                    t1 = min(min(part * per + per, total) * kvb, seq_len)
+                    work = on and t0 < t1 and t1 > 0
+                    out.append(DecodeAttentionSplitKV(layer, b, kvh, num_partials, part, seq_len, 1 if work else 0))
+        return out
+
+    def attention_reduction(self, layer: int, num_partials: int, globs: Any = None) -> list[Instruction]:
+        out: list[Instruction] = []
+        for b in range(self.batch_size):
+            for head0 in range(0, self.shape.num_attention_heads, ATTN_REDUCTION_SIZE):
+                if globs is None:
+                    out.append(DecodeAttentionReduction(layer, b, head0, num_partials, list(range(num_partials))))
+                else:
+                    out.append(DecodeAttentionReduction(layer, b, head0, num_partials, list(range(num_partials)),
+                                                        valid_partials=num_partials, is_active=1 if row_active(globs, b) else 0))
+        return out
+
+    # ---- fan-out -------------------------------------------------------------
+    def partials_for_request(self, globs: Any) -> int:
+        kvb = self.shape.attn_kv_block_size
+        rows = [b for b in range(self.batch_size) if row_active(globs, b)]
+        lens = getattr(globs, "kv_lengths", None)
+        blocks = max([1] + [_ceil_div(int(lens[b]) if lens is not None else decode_pos_id(globs, b) + 1, kvb) for b in rows])
+        return partials_for_blocks(len(rows), blocks, self.workers, self.shape.num_key_value_heads)
+
+    def partials_for_capacity(self, kv_capacity: int) -> int:
+        blocks = max(1, _ceil_div(kv_capacity, self.shape.attn_kv_block_size))
+        return partials_for_blocks(self.batch_size, blocks, self.workers, self.shape.num_key_value_heads)
+
+    # ---- whole step: dependency order, dealt round-robin ---------------------
+    def instruction_list(self, globs: Any, num_layers: int | None = None) -> list[Instruction]:
+        layers = self.shape.num_hidden_layers if num_layers is None else num_layers
+        p = self.partials_for_request(globs)
+        out: list[Instruction] = []
+        for layer in range(layers):
+            out += self.attn_rms(layer) + self.qkvproj(layer)
+            out += self.attention_split_kv(layer, p, globs) + self.attention_reduction(layer, p, globs)
+            out += self.oproj(layer) + self.mlp_rms(layer) + self.upgate(layer) + self.downproj(layer)
+        if layers == self.shape.num_hidden_layers:
+            out += self.lmhead_rms() + self.lmhead()
+        return out
+
+    def queues(self, globs: Any, num_layers: int | None = None) -> list[list[Instruction]]:
+        return deal(self.instruction_list(globs, num_layers), self.workers)
+
+    # ---- whole step: a template for every step of a request ------------------
+    def runtime_instruction_list(self, kv_capacity: int, num_layers: int | None = None) -> list[Instruction]:
+        layers = self.shape.num_hidden_layers if num_layers is None else num_layers
+        p = self.partials_for_capacity(kv_capacity)
+        out: list[Instruction] = []
+
+        def rows_round(rows: Sequence[Instruction]) -> None:   # one instruction slot per worker
+            out.extend(list(rows) + [NoOp()] * (self.workers - len(rows)))
+
+        def rounds(segment: Sequence[Instruction]) -> None:    # whole rounds, the last one padded
+            for at in range(0, len(segment), self.workers):
+                chunk = list(segment[at : at + self.workers])
+                out.extend(chunk + [NoOp()] * (self.workers - len(chunk)))
+
+        for layer in range(layers):
+            rows_round(self.attn_rms(layer))
+            rounds(self.qkvproj(layer))
+            rounds(self.attention_split_kv(layer, p))
+            rounds(self.attention_reduction(layer, p))
+            rounds(self.oproj(layer))
+            rows_round(self.mlp_rms(layer))
+            rounds(self.upgate(layer))
+            rounds(self.downproj(layer))
+        if layers == self.shape.num_hidden_layers:
+            rows_round(self.lmhead_rms())
+            rounds(self.lmhead())
+        return out
+
+    def runtime_queues(self, kv_capacity: int, num_layers: int | None = None) -> list[list[Instruction]]:
+        return deal(self.runtime_instruction_list(kv_capacity, num_layers), self.workers)
+
+
+def deal(instructions: Sequence[Instruction], workers: int) -> list[list[Instruction]]:
+    queues: list[list[Instruction]] = [[] for _ in range(workers)]
+    for i, ins in enumerate(instructions):
+        queues[i % workers].append(ins)
+    return queues
+
+
+def reference_scheduler(batch_size: int, shape: DecodeShape | None = None) -> BatchScheduler:
+    """The A100 route's worker count: two queues per SM."""
+    return BatchScheduler(shape or LlamaConfig.shape(), A100_WORKERS, batch_size)
+
+
+def mi355x_scheduler(batch_size: int, shape: DecodeShape | None = None) -> BatchScheduler:
+    return BatchScheduler(shape or LlamaConfig.shape(), MI355X_WORKERS, batch_size)

@@ -122,6 +122,53 @@ def build_globals(
     return g
 
 
+def build_batch_globals(
+    weights: dict[str, torch.Tensor],
+    shape: DecodeShape,
+    kv_capacity: int,
+    batch_size: int,
+    device: torch.device | str,
+    *,
+    max_partials: int = 27,
+    globals_cls: Any = None,
+) -> Any:
+    """Buffers of the batch route for ``batch_size`` rows (allocation as the reference's
+    `…/A100/fused_prefill.py:93-160` for batch sizes above one); all rows active, positions 0."""
+    if globals_cls is None:
+        from .decode_schedule_mb.globs import Globals as globals_cls
+    device = torch.device(device)
+    bf16 = torch.bfloat16
+    L, H, B = shape.num_hidden_layers, shape.hidden_size, batch_size
+    nq, nkv, d = shape.num_attention_heads, shape.num_key_value_heads, shape.head_dim
+
+    def zeros(*size: int, dtype: torch.dtype = bf16) -> torch.Tensor:
+        return torch.zeros(*size, dtype=dtype, device=device)
+
+    on_device = {k: v.to(device).contiguous() for k, v in weights.items()}
+    g = globals_cls(
+        position_id=0,
+        barriers=zeros(L, 10, (nq + 2 * nkv) * B, dtype=torch.int32),
+        k_cache=zeros(L, B, kv_capacity, nkv, d),
+        v_cache=zeros(L, B, kv_capacity, nkv, d),
+        hidden_states=zeros(B, H),
+        q_post_rope=zeros(B, nq * d),
+        attn_out=zeros(B, nq * d),
+        attn_out_intermediates=zeros(B, nq, max_partials, d, dtype=torch.float32),
+        attn_lse_intermediates=zeros(B, nq, max_partials, dtype=torch.float32),
+        silu_out=zeros(B, shape.intermediate_size),
+        logits=zeros(B, shape.vocab_size),
+        position_ids=zeros(B, dtype=torch.int32),
+        active_mask=torch.ones(B, dtype=torch.bool, device=device),
+        attn_partial_valid=zeros(B, nq, max_partials, dtype=torch.bool),
+        attn_rms_out=zeros(B, H),
+        mlp_rms_out=zeros(B, H),
+        lm_head_rms_out=zeros(B, H),
+        **{k: v for k, v in on_device.items() if k != "embed_tokens"},
+    )
+    g.embed_tokens = on_device["embed_tokens"]
+    return g
+
+
 def build_synthetic_globals(
     shape: DecodeShape | None = None,
     *,

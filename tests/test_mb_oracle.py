@@ -1,0 +1,261 @@
+"""Batch decode route (2..16 rows): instruction set, scheduler, per-row state and the two CPU oracles.
+
+The gfx950 kernel of this route is not built yet; what is pinned here is everything it will be
+checked against.  Three independent anchors:
+
+* ``tests/golden/mb_reduced_seed0.json`` — written by ``make_fixtures_mb.py`` from the imported
+  reference while this repository's scheduler, VM and fused oracle ran in lock-step with the
+  reference's (bit-identical instruction words, buffers, counters and row state for six steps of a
+  ragged three-row request in which one row retires);
+* the batch-1 oracle (itself pinned elsewhere): the reference's arithmetic is row-wise, so every
+  row of a batch must reproduce what that row gives alone, bit for bit;
+* integer properties of the instruction streams (coverage, counters, round structure).
+"""
+import dataclasses
+import hashlib
+import json
+import sys
+
+import numpy as np
+import pytest
+import torch
+
+from conftest import GOLDEN, ROOT
+
+sys.path.insert(0, str(ROOT / "oracle"))
+from fused_mb_oracle import FusedBatchOracle  # noqa: E402
+from fused_oracle import FusedOracle  # noqa: E402
+from pyvm_mb_oracle import BatchInstructionVM  # noqa: E402
+from qimeng_megakernel_amd import synthetic  # noqa: E402
+from qimeng_megakernel_amd.decode_schedule.model_config import LLAMA_3_2_1B, LlamaConfig  # noqa: E402
+from qimeng_megakernel_amd.decode_schedule_mb import decode_state, mk_kernel  # noqa: E402
+from qimeng_megakernel_amd.decode_schedule_mb.globs import Globals  # noqa: E402
+from qimeng_megakernel_amd.decode_schedule_mb.instructions import instruction_defs as D  # noqa: E402
+from qimeng_megakernel_amd.decode_schedule_mb.instructions import scheduler as S  # noqa: E402
+
+FIX = json.loads((GOLDEN / "mb_reduced_seed0.json").read_text())
+MB_FULL = dataclasses.replace(LLAMA_3_2_1B, attn_kv_block_size=FIX["kv_block"])
+MB_SMALL = dataclasses.replace(MB_FULL, num_hidden_layers=FIX["layers"], vocab_size=FIX["vocab"])
+
+
+@pytest.fixture(autouse=True)
+def _no_grad_and_shape():
+    LlamaConfig.set_shape(MB_SMALL)
+    with torch.no_grad():
+        yield
+    LlamaConfig.set_shape(LLAMA_3_2_1B)
+
+
+def _words(instructions) -> np.ndarray:
+    return np.asarray([i.padded() for i in instructions], dtype=np.int32)
+
+
+def _bits(t: torch.Tensor) -> list:
+    return t.contiguous().view(torch.int16).to(torch.int32).bitwise_and(0xFFFF).tolist()
+
+
+def _request(weights):
+    g = synthetic.build_batch_globals(weights, MB_SMALL, FIX["kv_capacity"], FIX["rows"], "cpu")
+    gen = torch.Generator().manual_seed(FIX["seed"] + 1)
+    g.k_cache.copy_(torch.randn(g.k_cache.shape, generator=gen).bfloat16())
+    g.v_cache.copy_(torch.randn(g.v_cache.shape, generator=gen).bfloat16())
+    g.position_ids.copy_(torch.tensor(FIX["start_positions"], dtype=torch.int32))
+    decode_state.ensure_decode_state(g, FIX["rows"], torch.device("cpu"))
+    return g
+
+
+@pytest.fixture(scope="module")
+def weights():
+    return synthetic.random_weights(MB_SMALL, FIX["seed"], max_positions=FIX["kv_capacity"])
+
+
+# ---------------------------------------------------------------- wire format --
+def test_wire_format_known_words():
+    """Operand order and defaults of `…/multi_batch/…/instruction_defs.py:11-211`."""
+    assert D.AttnRMS(3, 5, batch_row=4).serialize() == [1, 3, 5, 0, 0, 0, 4]
+    assert D.QKVProj_GEMM_RoPE(2, 8, 0, 10, 12).serialize() == [2, 2, 8, 0, 10, 12, 16, 16]
+    assert D.DecodeAttentionSplitKV(1, 2, 7, 4, 3).serialize() == [3, 1, 2, 7, 4, 3, -1, -1]
+    assert D.DecodeAttentionSplitKV(1, 2, 7, 4, 3, 130, 1).serialize() == [3, 1, 2, 7, 4, 3, 130, 1]
+    assert D.DecodeAttentionReduction(1, 2, 4, 3, [0, 1, 2]).serialize() == [4, 1, 2, 4, 3, 3, 0, 1, 2, 1, 0, -1, -1]
+    assert D.OProj_GEMM_Residual(0, 8, 0, 4, 6, 0).serialize() == [5, 0, 8, 0, 4, 6, 0, 16, 16]
+    assert D.MlpRMS(9, 8, batch_row=7).serialize() == [6, 9, 8, 0, 0, 0, 7]
+    assert D.UpGateProj_GEMM_SiLU(0, 8, 0, [7, 8, 9]).serialize() == [7, 0, 8, 0, 3, 7, 8, 9, 16, 16]
+    assert D.DownProj_GEMM_Residual(9, 8, 0, 0, 5).serialize() == [8, 9, 8, 0, 0, 5, 16, 16]
+    assert D.LMHeadRMS(8, batch_row=2).serialize() == [9, 8, 0, 0, 0, 0, 2]
+    assert D.LMHeadProj_GEMM(8, 75, 150).serialize() == [10, 8, 75, 150, 16, 16]
+    assert sorted(D.OPCODE_TO_CLASS) == list(range(11))
+
+
+# ------------------------------------------------------------------ scheduler --
+def test_full_size_runtime_template_matches_the_reference_digest():
+    meta = FIX["full_size_runtime_template"]
+    LlamaConfig.set_shape(MB_FULL)
+    queues = S.reference_scheduler(meta["rows"], MB_FULL).runtime_queues(meta["kv_capacity"])
+    arr = np.stack([_words(q) for q in queues])
+    assert list(arr.shape) == meta["shape"]
+    assert hashlib.sha256(arr.tobytes()).hexdigest() == meta["sha256"]
+
+
+def test_runtime_template_is_made_of_whole_rounds():
+    sched = S.mi355x_scheduler(8, MB_FULL)
+    flat = sched.runtime_instruction_list(1024, num_layers=2)
+    assert len(flat) % sched.workers == 0
+    rounds = [flat[i : i + sched.workers] for i in range(0, len(flat), sched.workers)]
+    for r in rounds:   # a round holds one kind of instruction (and padding)
+        assert len({i.opcode() for i in r} - {0}) == 1
+    first = rounds[0]   # the RMSNorm rows sit in the first B slots of their round
+    assert [i.opcode() for i in first[:8]] == [1] * 8 and [i.batch_row for i in first[:8]] == list(range(8))
+    assert all(i.opcode() == 0 for i in first[8:])
+    # attention instructions leave length and activity to the launch
+    assert all(i.seq_len == -1 and i.is_active == -1 for i in flat if i.opcode() == 3)
+    assert all(i.valid_partials == -1 and i.is_active == -1 for i in flat if i.opcode() == 4)
+
+
+@pytest.mark.parametrize("make,rows", [(S.reference_scheduler, 3), (S.mi355x_scheduler, 8), (S.mi355x_scheduler, 16)])
+def test_every_output_once_and_final_counters(make, rows):
+    shape = MB_SMALL
+    sched = make(rows, shape)
+    flat = sched.runtime_instruction_list(256)
+    p = sched.partials_for_capacity(256)
+    out = {op: [] for op in (2, 5, 7, 8, 10)}
+    for i in flat:
+        if i.opcode() in (2, 5, 8):
+            out[i.opcode()] += range(i.tile_N_start_idx * 16, i.tile_N_end_idx * 16)
+        elif i.opcode() == 7:
+            for b in i.tile_N_block_idxs:
+                out[7] += range(b * 16, b * 16 + 16)
+        elif i.opcode() == 10:
+            out[10] += range(i.start_output_block_idx * 16, i.end_output_block_idx * 16)
+    L = shape.num_hidden_layers
+    assert sorted(out[2]) == sorted(list(range(shape.qkv_out_dim)) * L)
+    assert sorted(out[5]) == sorted(list(range(shape.hidden_size)) * L) == sorted(out[8])
+    assert sorted(out[7]) == sorted(list(range(shape.intermediate_size)) * L)
+    assert sorted(out[10]) == list(range(shape.vocab_size))
+    attn = [(i.layer_idx, i.batch_idx, i.kv_head_idx, i.partial_idx) for i in flat if i.opcode() == 3]
+    assert len(attn) == len(set(attn)) == L * rows * shape.num_key_value_heads * p
+    red = [(i.layer_idx, i.batch_idx, i.head_start_idx) for i in flat if i.opcode() == 4]
+    assert len(red) == len(set(red)) == L * rows * shape.num_attention_heads // 4
+    with pytest.raises(ValueError):
+        make(17, shape)
+
+
+def test_fan_out_policy():
+    """`scheduler.py:351-376`: about one split-KV instruction per worker, at most one per KV block,
+    at most what a reduction instruction lists."""
+    assert S.partials_for_blocks(8, 16, 216, 8) == 4        # ceil(216 / 64)
+    assert S.partials_for_blocks(1, 2, 216, 8) == 2         # two blocks: two slices
+    assert S.partials_for_blocks(2, 100, 216, 8) == 14      # ceil(216 / 16)
+    assert S.partials_for_blocks(1, 1000, 256, 8) == S.MAX_REDUCTION_LIST
+    assert S.partials_for_blocks(0, 5, 216, 8) == 1
+
+
+# -------------------------------------------------------------------- oracles --
+def test_request_of_the_reference_fixture(weights):
+    """Both oracles reproduce the six recorded steps: instruction words, tokens, top-4 logits, row state."""
+    vm_g, fu_g = _request(weights), _request(weights)
+    vm, fused = BatchInstructionVM(MB_SMALL), FusedBatchOracle(MB_SMALL)
+    sched = S.reference_scheduler(FIX["rows"], MB_SMALL)
+    toks = {"my_vm": list(FIX["start_tokens"]), "my_fused": list(FIX["start_tokens"])}
+    for step, want in enumerate(FIX["steps"]):
+        for name, g in (("my_vm", vm_g), ("my_fused", fu_g)):
+            for b in range(FIX["rows"]):
+                g.hidden_states[b].copy_(g.embed_tokens[toks[name][b]])
+            assert g.position_ids.tolist() == want["positions"] and g.active_mask.tolist() == want["active"]
+        vm_g.barriers.zero_()
+        flat = sched.instruction_list(vm_g)
+        assert hashlib.sha256(_words(flat).tobytes()).hexdigest() == FIX["instruction_list_sha256"][step]
+        vm.run(vm_g, flat)
+        fused.decode_step(fu_g)
+        assert _bits(vm_g.hidden_states[:, ::128]) == want["hidden_bits_sampled"]
+        for name, g in (("my_vm", vm_g), ("my_fused", fu_g)):
+            ids = torch.tensor(want[name]["top_ids"])
+            assert _bits(g.logits.gather(1, ids)) == want[name]["top_bits"], (step, name)
+            nxt = g.logits.float().argmax(dim=-1)
+            assert nxt.tolist() == want[name]["tokens"]
+            decode_state.advance_decode_state(g, nxt, [FIX["eos_token"]] if step >= 1 else [])
+            toks[name] = nxt.tolist()
+    assert vm_g.active_mask.tolist() == [True, False, True] and vm_g.eos_reached.tolist() == [False, True, False]
+
+
+def test_every_row_of_a_batch_equals_that_row_alone(weights):
+    """The fused batch oracle against the batch-1 oracle: bit for bit, at ragged positions."""
+    g = _request(weights)
+    tokens = (5, 900, 1234)
+    for b, t in enumerate(tokens):
+        g.hidden_states[b].copy_(g.embed_tokens[t])
+    before_k, before_v = g.k_cache.clone(), g.v_cache.clone()
+    FusedBatchOracle(MB_SMALL).decode_step(g)
+    one = FusedOracle(MB_SMALL)
+    for b, t in enumerate(tokens):
+        g1 = synthetic.build_globals(weights, MB_SMALL, FIX["kv_capacity"], "cpu")
+        g1.k_cache[:, 0].copy_(before_k[:, b]); g1.v_cache[:, 0].copy_(before_v[:, b])
+        g1.hidden_states.copy_(g1.embed_tokens[t]); g1.position_id = FIX["start_positions"][b]
+        one.decode_step(g1)
+        for name in ("hidden_states", "q_post_rope", "attn_out", "silu_out", "logits"):
+            assert torch.equal(getattr(g1, name), getattr(g, name)[b]), (b, name)
+        assert torch.equal(g1.k_cache[:, 0], g.k_cache[:, b]) and torch.equal(g1.v_cache[:, 0], g.v_cache[:, b])
+
+
+def test_inactive_row_is_frozen_and_forced(weights):
+    g = _request(weights)
+    g.active_mask[1] = False
+    for b in range(3):
+        g.hidden_states[b].copy_(g.embed_tokens[10 + b])
+    frozen = (g.hidden_states[1].clone(), g.k_cache[:, 1].clone(), g.q_post_rope[1].clone())
+    v = _request(weights); v.active_mask[1] = False
+    v.hidden_states.copy_(g.hidden_states)
+    FusedBatchOracle(MB_SMALL).decode_step(g)
+    BatchInstructionVM(MB_SMALL).run(v, S.mi355x_scheduler(3, MB_SMALL).instruction_list(v))
+    for x in (g, v):
+        assert torch.equal(x.hidden_states[1], frozen[0]) and torch.equal(x.k_cache[:, 1], frozen[1])
+        assert torch.equal(x.q_post_rope[1], frozen[2])
+        assert float(x.attn_out[1].abs().max()) == 0 and float(x.silu_out[1].abs().max()) == 0
+        assert bool((x.logits[1].float() == torch.tensor(-1e9).bfloat16().float()).all())
+    assert float(v.attn_rms_out[1].abs().max()) == 0 and not bool(v.attn_partial_valid[1].any())
+    assert bool(torch.isinf(v.attn_lse_intermediates[1, :, : S.mi355x_scheduler(3, MB_SMALL).partials_for_request(v)]).all())
+
+
+def test_vm_agrees_with_fused_and_counters_complete(weights):
+    f, v = _request(weights), _request(weights)
+    for b in range(3):
+        for g in (f, v):
+            g.hidden_states[b].copy_(g.embed_tokens[20 + b])
+    FusedBatchOracle(MB_SMALL).decode_step(f)
+    sched = S.mi355x_scheduler(3, MB_SMALL)
+    BatchInstructionVM(MB_SMALL).run(v, sched.runtime_instruction_list(FIX["kv_capacity"]))
+    for name in ("q_post_rope", "attn_out", "silu_out", "hidden_states", "logits"):
+        a, b_ = getattr(f, name).float(), getattr(v, name).float()
+        assert float((a - b_).abs().max()) <= 2.0 ** -5 * max(1.0, float(a.abs().max())), name
+    assert v.logits.float().argmax(-1).tolist() == f.logits.float().argmax(-1).tolist()
+    s, p = MB_SMALL, sched.partials_for_capacity(FIX["kv_capacity"])
+    stride = s.num_attention_heads + 2 * s.num_key_value_heads
+    for layer in range(s.num_hidden_layers):
+        bar = v.barriers[layer]
+        assert int(bar[0, 0]) == 3 and int(bar[5, 0]) == 3
+        assert bar[1, :stride].tolist() == [s.head_dim // 16] * stride
+        for b in range(3):
+            assert bar[2, b * stride : b * stride + s.num_attention_heads].tolist() == [p] * s.num_attention_heads
+            assert int(bar[3, b]) == s.num_attention_heads
+        assert int(bar[4, 0]) == s.hidden_size // 16 == int(bar[7, 0]) and int(bar[6, 0]) == s.intermediate_size // 16
+    assert int(v.barriers[s.num_hidden_layers - 1, 8, 0]) == 3
+
+
+# ---------------------------------------------------------------- row state ----
+def test_decode_state_advances_and_retires_rows():
+    g = Globals(hidden_states=torch.zeros(3, 4), position_ids=torch.tensor([5, 0, 9], dtype=torch.int32))
+    decode_state.ensure_decode_state(g, 3, torch.device("cpu"))
+    assert g.kv_lengths.tolist() == [6, 1, 10] and g.active_mask.tolist() == [True] * 3
+    decode_state.advance_decode_state(g, torch.tensor([7, 2, 8]), [2])
+    assert g.position_ids.tolist() == [6, 0, 10] and g.active_mask.tolist() == [True, False, True]
+    assert g.eos_reached.tolist() == [False, True, False] and g.kv_lengths.tolist() == [7, 1, 11]
+    decode_state.advance_decode_state(g, torch.tensor([2, 2, 3]), [2])      # a retired row stays retired
+    assert g.position_ids.tolist() == [6, 0, 11] and g.active_mask.tolist() == [False, False, True]
+    assert g.last_generated_tokens.tolist() == [2, 2, 3]
+    assert decode_state.instruction_active(0, g, 2) is False and decode_state.instruction_active(1, g, 0) is True
+    assert decode_state.instruction_active(-1, g, 2) is True and decode_state.instruction_active(-1, g, 0) is False
+    assert decode_state.batch_size(g) == 3 and decode_state.decode_pos_id(g, 2) == 11 and decode_state.kv_length(g, 2) == 12
+
+
+def test_batch_kernel_is_absent_and_says_so():
+    with pytest.raises(ImportError, match="not built"):
+        mk_kernel.get_mk()
