@@ -15,6 +15,11 @@
  *                        decode_kernel/mk.h:4-30, launcher decode_kernel/mk.cu:97-198,
  *                        python binding decode_kernel/pybind.cpp:8-39,
  *                        call site decode_schedule/mk_kernel.py:56-94
+ *   qmk_decode_step_batch <- void mk(22 x const torch::Tensor&, int pos_id, int batch_size,
+ *                        float attn_scale, float rms_norm_eps, optional position_ids, active_mask,
+ *                        attn_partial_valid, attn_rms_out, mlp_rms_out, lm_head_rms_out) of the batch route:
+ *                        …/A100/multi_batch/decode_kernel/mk.h:9-42, host checks mk.cu:52-216,
+ *                        call site …/multi_batch/decode_schedule/mk_kernel.py:56-111
  *   qmk_query         <- KernelConfig (NUM_SMS, NUM_THREADS, SHARED_MEMORY_SIZE,
  *                        INSTRUCTION_WIDTH) decode_kernel/kernel_config.cuh:6-14
  *   qmk_status_*      <- the reference only printf()s launch errors
@@ -30,7 +35,7 @@
 extern "C" {
 #endif
 
-#define QMK_ABI_VERSION 4
+#define QMK_ABI_VERSION 5
 #define QMK_INSTRUCTION_WORDS 32
 
 /* Return / status codes. 0 is success; everything else is an error. */
@@ -45,7 +50,7 @@ enum {
   QMK_ERR_LAUNCH = 7,          /* hipLaunchKernel failed                        */
   QMK_ERR_MODEL = 8,           /* unknown model id                              */
   /* device-side (reported through qmk_status_fetch) */
-  QMK_DEV_BAD_OPCODE = 32,     /* opcode outside 0..7                           */
+  QMK_DEV_BAD_OPCODE = 32,     /* opcode outside 0..7 (batch route: 0..10)      */
   QMK_DEV_BAD_OPERAND = 33,    /* an operand would index out of bounds          */
   QMK_DEV_WAIT_TIMEOUT = 34    /* a counter never reached its expected value    */
 };
@@ -185,6 +190,73 @@ typedef struct QmkArgs {
 /* Launch one decode step asynchronously on args->stream.  Returns QMK_OK or a
  * host-side QMK_ERR_*.  Device-side errors surface through qmk_status_fetch. */
 int qmk_decode_step(const QmkArgs* args);
+
+/*
+ * One decode step of the batch route: 2..16 rows decoded together (1 is accepted), each at its own
+ * position.  Ten opcodes (…/multi_batch/decode_schedule/instructions/instruction_defs.py:11-211):
+ * RMSNorm rows 1/6/9, GEMMs 2/5/7/8/10 over 16-row blocks on the matrix cores, split-KV attention 3 and
+ * its reduction 4 per batch row.  Tensors are the batch-1 ones with a leading batch dimension, in the
+ * order of mk(...) (…/multi_batch/decode_kernel/mk.h:9-42).  Only the Llama-3.2-1B layer geometry
+ * is compiled for this route.  Flags: QMK_FLAG_KEEP_BARRIERS only.
+ */
+typedef struct QmkBatchArgs {
+  uint32_t struct_size;            /* = sizeof(QmkBatchArgs)                      */
+  uint32_t model;                  /* QMK_MODEL_LLAMA_3_2_1B                      */
+  uint32_t flags;                  /* 0 or QMK_FLAG_KEEP_BARRIERS                 */
+  uint32_t spin_limit;             /* counter polls before QMK_DEV_WAIT_TIMEOUT; 0 = default */
+
+  const int32_t* instructions;     /* int32 [num_queues, num_insts, 32]           */
+  void* hidden_states;             /* bf16 [B, H]         in/out residual stream  */
+  void* q_post_rope;               /* bf16 [B, Hq*D]                              */
+  void* k_cache;                   /* bf16 [L, B, max_seq_len, Hkv, D]            */
+  void* v_cache;                   /* bf16 [L, B, max_seq_len, Hkv, D]            */
+  void* attn_out;                  /* bf16 [B, Hq*D]                              */
+  float* attn_lse_intermediates;   /* f32  [B, Hq, max_splits]   log2 domain      */
+  float* attn_out_intermediates;   /* f32  [B, Hq, max_splits, D]                 */
+  void* silu_out;                  /* bf16 [B, F]                                 */
+  void* logits;                    /* bf16 [B, vocab_size]                        */
+  const void* attn_norm_weights;   /* bf16 [L, H]                                 */
+  const void* qkv_weights;         /* bf16 [L, (Hq+2Hkv)*D, H]                    */
+  const float* rope_cos;           /* f32  [rope_rows, D]  pair-interleaved       */
+  const float* rope_sin;           /* f32  [rope_rows, D]                         */
+  const void* o_proj_weights;      /* bf16 [L, H, H]                              */
+  const void* mlp_norm_weights;    /* bf16 [L, H]                                 */
+  const void* up_proj_weights;     /* bf16 [L, F, H]                              */
+  const void* gate_proj_weights;   /* bf16 [L, F, H]                              */
+  const void* down_proj_weights;   /* bf16 [L, H, F]                              */
+  const void* lm_head_norm_weights;/* bf16 [H]                                    */
+  const void* lm_head_weights;     /* bf16 [vocab_size, H]                        */
+  int32_t* barriers;               /* int32 [num_layers, num_layer_barriers (>= 10), barrier_slots (>= B*(Hq+2Hkv))] */
+
+  int32_t num_queues;              /* instructions.size(0) = workgroups launched  */
+  int32_t num_insts;               /* instructions.size(1)                        */
+  int32_t num_layers;
+  int32_t num_layer_barriers;
+  int32_t barrier_slots;
+  int32_t max_seq_len;             /* k_cache.size(2)                             */
+  int32_t max_splits;              /* attn_lse_intermediates.size(2)              */
+  int32_t vocab_size;              /* logits.size(1)                              */
+  int32_t rope_rows;
+  int32_t pos_id;                  /* position of every row when position_ids is NULL */
+  int32_t batch_size;              /* B, 1..16                                    */
+  int32_t kv_block_size;           /* tokens per split-KV block (the scheduler's attn_kv_block_size) */
+  float attn_scale;
+  float rms_norm_eps;
+
+  const int32_t* position_ids;     /* int32 [B] or NULL                           */
+  const uint8_t* active_mask;      /* u8/bool [B] or NULL: every row is active    */
+  uint8_t* attn_partial_valid;     /* u8/bool [B, Hq, max_splits] or NULL         */
+  void* attn_rms_out;              /* bf16 [B, H]  RMSNorm rows for the QKV GEMM  */
+  void* mlp_rms_out;               /* bf16 [B, H]  ... for the up/gate GEMM       */
+  void* lm_head_rms_out;           /* bf16 [B, H]  ... for the LM head            */
+
+  uint64_t* timeline;              /* as in QmkArgs; NULL = off                   */
+  void* stream;                    /* hipStream_t; NULL = the null stream         */
+} QmkBatchArgs;
+
+/* Launch one step of the batch route asynchronously on args->stream.  Positions outside the KV
+ * cache or the RoPE table are found on the device (QMK_DEV_BAD_OPERAND, instruction -1). */
+int qmk_decode_step_batch(const QmkBatchArgs* args);
 
 /* Size of QmkArgs.workspace for QMK_FLAG_TAGGED; 0 for an unknown model. */
 uint64_t qmk_workspace_bytes(int model);

@@ -13,6 +13,7 @@
 #include <mutex>
 
 #include "qmk.h"
+#include "qmk_mb_ops.h"
 #include "qmk_ops.h"
 
 namespace qmk {
@@ -151,10 +152,100 @@ __global__ __launch_bounds__(kThreads, 1) void decode_megakernel(const Params p)
   }
 }
 
+// The batch route's interpreter: same queue walk, the ten opcodes of qmk_mb_ops.h, the reference's
+// counter protocol per batch row (…/A100/multi_batch/decode_kernel/mk.cu).  Per-row positions and
+// activity are read once per launch.
+template <class M>
+__global__ __launch_bounds__(kThreads, 1) void decode_megakernel_batch(const Params p) {
+  __shared__ mb::Smem<M> s;
+  if (threadIdx.x < 8) s.ctl[threadIdx.x] = 0;
+  if (threadIdx.x < mb::kMaxBatch) {   // one wave: the zeroing above has happened for all of them
+    const int b = threadIdx.x;
+    int pos = 0, on = 0;
+    if (b < p.batch) {
+      pos = p.position_ids != nullptr ? p.position_ids[b] : p.pos_id;
+      on = p.active_mask != nullptr ? (p.active_mask[b] != 0) : 1;
+      if (pos < 0 || pos >= p.max_seq_len || pos >= p.rope_rows) {
+        s.ctl[0] = 1;
+        report_error(p, QMK_DEV_BAD_OPERAND, -1, 0, b);
+        pos = 0;
+      }
+    }
+    s.pos[b] = pos;
+    s.active[b] = on;
+  }
+  __syncthreads();
+  bool ok = s.ctl[0] == 0;
+
+  const int32_t* queue = p.instructions + static_cast<size_t>(blockIdx.x) * p.num_insts * kInstWords;
+  int32_t word = (threadIdx.x < kInstWords && p.num_insts > 0) ? queue[threadIdx.x] : 0;
+  for (int i = 0; i < p.num_insts && ok; ++i) {
+    if (threadIdx.x < kInstWords) {
+      s.inst[threadIdx.x] = word;
+      word = (i + 1 < p.num_insts) ? queue[(i + 1) * kInstWords + threadIdx.x] : 0;
+    }
+    __syncthreads();
+    const int opcode = s.inst[0];
+    int tid = threadIdx.x;
+    asm volatile("" : "+v"(tid));
+    const Ctx c{i, opcode, tid};
+    unsigned long long t_start = 0;
+    if (p.timeline != nullptr && threadIdx.x == 0) {
+      t_start = wall_clock64();
+      for (int k = 0; k < 4; ++k) s.stamps[k] = t_start;
+    }
+    switch (opcode) {
+      case mb::OP_NOOP: break;
+      case mb::OP_ATTN_RMS:
+      case mb::OP_MLP_RMS:
+      case mb::OP_LM_RMS: ok = mb::op_rms_row<M>(p, s, c); break;
+      case mb::OP_QKV: ok = mb::op_qkv<M>(p, s, c); break;
+      case mb::OP_SPLITKV: ok = mb::op_splitkv<M>(p, s, c); break;
+      case mb::OP_REDUCE: ok = mb::op_reduce<M>(p, s, c); break;
+      case mb::OP_OPROJ: ok = mb::op_oproj<M>(p, s, c); break;
+      case mb::OP_UPGATE: ok = mb::op_upgate<M>(p, s, c); break;
+      case mb::OP_DOWN: ok = mb::op_down<M>(p, s, c); break;
+      case mb::OP_LMHEAD: ok = mb::op_lmhead<M>(p, s, c); break;
+      default:
+        if (threadIdx.x == 0) report_error(p, QMK_DEV_BAD_OPCODE, i, opcode, 0);
+        ok = false;
+        break;
+    }
+    if (p.timeline != nullptr && threadIdx.x == 0) {
+      uint64_t* rec = p.timeline + (static_cast<size_t>(blockIdx.x) * p.num_insts + i) * 8;
+      rec[0] = t_start;
+      rec[1] = s.ctl[2] ? s.t_wait : t_start;
+      rec[2] = wall_clock64();
+      rec[3] = static_cast<uint64_t>(opcode) | (static_cast<uint64_t>(static_cast<uint32_t>(s.inst[1])) << 8);
+      for (int k = 0; k < 4; ++k) rec[4 + k] = s.stamps[k];
+      s.ctl[2] = 0;
+    }
+    __syncthreads();  // s.inst and the staging areas are reused by the next instruction
+  }
+  if (!ok || (p.flags & QMK_FLAG_KEEP_BARRIERS)) return;
+
+  // Retire: the workgroup that arrives last owns the counters alone and clears them for the next
+  // step.  The arrival counter is the last word of layer 0's last row (row 9 carries no counter).
+  release_stores();
+  __syncthreads();
+  int32_t* done = counter_ptr(p, 0, p.num_layer_barriers - 1, p.barrier_slots - 1);
+  if (threadIdx.x == 0) {
+    const int prev = __hip_atomic_fetch_add(done, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    s.ctl[1] = (prev == static_cast<int>(gridDim.x) - 1);
+  }
+  __syncthreads();
+  if (s.ctl[1]) {
+    const int total = p.num_layers * p.num_layer_barriers * p.barrier_slots;
+    for (int i = threadIdx.x; i < total; i += kThreads)
+      __hip_atomic_store(p.barriers + i, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  }
+}
+
 struct DeviceInfo {
   bool ready = false;
   int cu_count = 0;
   int max_queues = 0;
+  int max_queues_batch = 0;
   int32_t* status = nullptr;
 };
 DeviceInfo g_devices[kMaxDevices];
@@ -171,11 +262,15 @@ int device_info(DeviceInfo** out) {
     int per_cu = 0;
     if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, decode_megakernel<Llama1B>, kThreads, 0) != hipSuccess)
       return QMK_ERR_NO_DEVICE;
+    int per_cu_batch = 0;
+    if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu_batch, decode_megakernel_batch<Llama1B>, kThreads, 0) != hipSuccess)
+      return QMK_ERR_NO_DEVICE;
     void* sym = nullptr;
     if (hipGetSymbolAddress(&sym, HIP_SYMBOL(g_status)) != hipSuccess) return QMK_ERR_NO_DEVICE;
     if (hipMemset(sym, 0, sizeof(int32_t) * kStatusWords) != hipSuccess) return QMK_ERR_NO_DEVICE;
     d.cu_count = prop.multiProcessorCount;
     d.max_queues = per_cu * prop.multiProcessorCount;
+    d.max_queues_batch = per_cu_batch * prop.multiProcessorCount;
     d.status = static_cast<int32_t*>(sym);
     d.ready = true;
   }
@@ -294,6 +389,83 @@ extern "C" int qmk_decode_step(const QmkArgs* a) {
   }
 }
 
+extern "C" int qmk_decode_step_batch(const QmkBatchArgs* a) {
+  using M = Llama1B;
+  if (a == nullptr) return QMK_ERR_NULL_ARG;
+  if (a->struct_size != sizeof(QmkBatchArgs)) return QMK_ERR_ABI;
+  if (a->model != QMK_MODEL_LLAMA_3_2_1B) return QMK_ERR_MODEL;
+  const void* required[] = {a->instructions, a->hidden_states, a->q_post_rope, a->k_cache, a->v_cache, a->attn_out,
+                            a->attn_lse_intermediates, a->attn_out_intermediates, a->silu_out, a->logits,
+                            a->attn_norm_weights, a->qkv_weights, a->rope_cos, a->rope_sin, a->o_proj_weights,
+                            a->mlp_norm_weights, a->up_proj_weights, a->gate_proj_weights, a->down_proj_weights,
+                            a->lm_head_norm_weights, a->lm_head_weights, a->barriers,
+                            a->attn_rms_out, a->mlp_rms_out, a->lm_head_rms_out};
+  for (const void* ptr : required)
+    if (ptr == nullptr) return QMK_ERR_NULL_ARG;
+  if (a->batch_size < 1 || a->batch_size > mb::kMaxBatch) return QMK_ERR_SHAPE;
+  if (a->num_queues < 1 || a->num_insts < 0 || a->num_layers < 1 || a->num_layer_barriers < 10 ||
+      a->barrier_slots < a->batch_size * (M::NQ + 2 * M::NKV) || a->max_seq_len < 1 || a->max_splits < 1 ||
+      a->vocab_size < 1 || a->rope_rows < 1 || a->kv_block_size < 1)
+    return QMK_ERR_SHAPE;
+  if (a->flags & ~QMK_FLAG_KEEP_BARRIERS) return QMK_ERR_SHAPE;
+  if (a->position_ids == nullptr && (a->pos_id < 0 || a->pos_id >= a->max_seq_len || a->pos_id >= a->rope_rows)) return QMK_ERR_POSITION;
+
+  DeviceInfo* dev = nullptr;
+  if (int rc = device_info(&dev); rc != QMK_OK) return rc;
+  if (a->num_queues > dev->max_queues_batch) return QMK_ERR_TOO_MANY_QUEUES;
+  if (a->num_insts == 0) return QMK_OK;
+
+  Params p{};
+  p.instructions = a->instructions;
+  p.hidden = static_cast<u16*>(a->hidden_states);
+  p.q_post_rope = static_cast<u16*>(a->q_post_rope);
+  p.k_cache = static_cast<u16*>(a->k_cache);
+  p.v_cache = static_cast<u16*>(a->v_cache);
+  p.attn_out = static_cast<u16*>(a->attn_out);
+  p.attn_lse = a->attn_lse_intermediates;
+  p.attn_partial = a->attn_out_intermediates;
+  p.silu_out = static_cast<u16*>(a->silu_out);
+  p.logits = static_cast<u16*>(a->logits);
+  p.attn_norm = static_cast<const u16*>(a->attn_norm_weights);
+  p.qkv_w = static_cast<const u16*>(a->qkv_weights);
+  p.rope_cos = a->rope_cos;
+  p.rope_sin = a->rope_sin;
+  p.o_w = static_cast<const u16*>(a->o_proj_weights);
+  p.mlp_norm = static_cast<const u16*>(a->mlp_norm_weights);
+  p.up_w = static_cast<const u16*>(a->up_proj_weights);
+  p.gate_w = static_cast<const u16*>(a->gate_proj_weights);
+  p.down_w = static_cast<const u16*>(a->down_proj_weights);
+  p.lm_norm = static_cast<const u16*>(a->lm_head_norm_weights);
+  p.lm_w = static_cast<const u16*>(a->lm_head_weights);
+  p.barriers = a->barriers;
+  p.timeline = a->timeline;
+  p.status = dev->status;
+  p.num_insts = a->num_insts;
+  p.num_layers = a->num_layers;
+  p.num_layer_barriers = a->num_layer_barriers;
+  p.barrier_slots = a->barrier_slots;
+  p.max_seq_len = a->max_seq_len;
+  p.max_splits = a->max_splits;
+  p.vocab_size = a->vocab_size;
+  p.pos_id = a->pos_id;
+  p.attn_scale = a->attn_scale;
+  p.rms_norm_eps = a->rms_norm_eps;
+  p.spin_limit = a->spin_limit > 0 ? a->spin_limit : kDefaultSpinLimit;
+  p.flags = a->flags;
+  p.batch = a->batch_size;
+  p.kv_block = a->kv_block_size;
+  p.position_ids = a->position_ids;
+  p.active_mask = a->active_mask;
+  p.partial_valid = a->attn_partial_valid;
+  p.attn_rms_out = static_cast<u16*>(a->attn_rms_out);
+  p.mlp_rms_out = static_cast<u16*>(a->mlp_rms_out);
+  p.lm_rms_out = static_cast<u16*>(a->lm_head_rms_out);
+  p.rope_rows = a->rope_rows;
+
+  hipLaunchKernelGGL(decode_megakernel_batch<M>, dim3(a->num_queues), dim3(kThreads), 0, static_cast<hipStream_t>(a->stream), p);
+  return hipGetLastError() == hipSuccess ? QMK_OK : QMK_ERR_LAUNCH;
+}
+
 extern "C" uint64_t qmk_workspace_bytes(int model) {
   return (model == QMK_MODEL_LLAMA_3_2_1B || model == QMK_MODEL_QWEN3_1_7B) ? static_cast<uint64_t>(kWsUnits) * sizeof(uint64_t) : 0;
 }
@@ -337,7 +509,7 @@ extern "C" const char* qmk_error_string(int code) {
     case QMK_ERR_NO_DEVICE: return "no usable HIP device";
     case QMK_ERR_LAUNCH: return "kernel launch failed";
     case QMK_ERR_MODEL: return "unknown model id";
-    case QMK_DEV_BAD_OPCODE: return "device: opcode outside 0..7";
+    case QMK_DEV_BAD_OPCODE: return "device: unknown opcode";
     case QMK_DEV_BAD_OPERAND: return "device: instruction operand out of bounds";
     case QMK_DEV_WAIT_TIMEOUT: return "device: counter wait ran out of polls";
     default: return "unknown code";

@@ -81,6 +81,16 @@ struct Params {
   int32_t down_arrivals;
   uint32_t spin_limit;
   uint32_t flags;
+  // Batch route only.
+  int32_t batch;                 // rows decoded together
+  int32_t kv_block;              // tokens per split-KV block
+  const int32_t* position_ids;   // [batch] or null: every row decodes pos_id
+  const uint8_t* active_mask;    // [batch] or null: every row is active
+  uint8_t* partial_valid;        // [batch, NQ, max_splits] or null
+  u16* attn_rms_out;             // [batch, H] each
+  u16* mlp_rms_out;
+  u16* lm_rms_out;
+  int32_t rope_rows;
 };
 
 // ---------------------------------------------------------------- bf16 ----

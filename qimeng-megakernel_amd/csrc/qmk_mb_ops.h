@@ -1,0 +1,752 @@
+// The ten opcodes of the batch decode route (2..16 rows decoded together) as workgroup-wide device
+// functions for gfx950.
+//
+// Semantics follow the reference's batch route: arithmetic and rounding points from its fused
+// PyTorch operations run on [B, H] activations
+// (qimeng_megakernel/models/LLM/llama/llama3_2__1b/A100/multi_batch/decode_schedule/fused/__init__.py,
+//  …/single_batch/decode_schedule/fused/operations.py:126-321), operand layout, per-row state and the
+// counter protocol from its instruction VM (…/multi_batch/decode_schedule/instructions/python_vm.py:139-730).
+//
+// The projections are GEMMs with a skinny activation side: a block is 16 weight rows, the batch
+// rows are the (at most 16) columns.  v_mfma_f32_16x16x32_bf16 takes the 16 weight rows as A and the
+// batch as B: lane l holds A[row l%16][k 8*(l/16)..+7], B[k 8*(l/16)..+7][column l%16] and
+// C[row 4*(l/16)..+3][column l%16].  Which 8 columns of a 32-column chunk sit in which k slot is
+// free as long as both operands agree, so a lane simply reads 16 contiguous bytes of its weight row
+// and of its batch row.  The eight waves of a workgroup split K: wave w owns a 256-column segment
+// (four of them for K = 8192) of the block, keeps its share of the activations in registers for the
+// whole instruction and streams weight segments through a register ring; the eight partial 16x16
+// tiles meet in LDS, where 128 threads add them up and apply the epilogue to two neighbouring
+// outputs each.  Weights cross the memory system once per step whatever the batch size: the bound
+// is still HBM.
+#pragma once
+
+#include "qmk_ops.h"
+
+namespace qmk {
+namespace mb {
+
+constexpr int kTile = 16;       // weight rows per block (the reference's tile_N_granularity)
+constexpr int kMaxBatch = 16;   // batch rows = columns of one matrix-core tile (tile_M_granularity)
+constexpr int kChunk = 32;      // K per matrix-core instruction
+constexpr int kSeg = 256;       // K columns of one segment: 8 chunks, 16 bytes per lane each
+constexpr int kSegChunks = kSeg / kChunk;
+constexpr int kMaxList = kInstWords - 10;  // reduction list: 6 leading and 4 trailing words
+constexpr float kNoContribution = -79.0f;  // without a validity buffer: partials at or below do not count
+
+enum Opcode {
+  OP_NOOP = 0,
+  OP_ATTN_RMS = 1,
+  OP_QKV = 2,
+  OP_SPLITKV = 3,
+  OP_REDUCE = 4,
+  OP_OPROJ = 5,
+  OP_MLP_RMS = 6,
+  OP_UPGATE = 7,
+  OP_DOWN = 8,
+  OP_LM_RMS = 9,
+  OP_LMHEAD = 10,
+};
+// Counter rows: opcode - 1.
+constexpr int ROW_ATTN_RMS = 0, ROW_QKV = 1, ROW_SPLITKV = 2, ROW_REDUCE = 3, ROW_OPROJ = 4, ROW_MLP_RMS = 5, ROW_UPGATE = 6,
+              ROW_DOWN = 7, ROW_LM_RMS = 8;
+
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef float f4 __attribute__((ext_vector_type(4)));
+
+// Validity flags are bytes that one workgroup writes and another reads within the launch.
+__device__ __forceinline__ void st_shared8(uint8_t* p, uint8_t v) { __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); }
+__device__ __forceinline__ uint8_t ld_shared8(const uint8_t* p) { return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); }
+
+template <class M>
+struct Smem {
+  int32_t inst[kInstWords];
+  int32_t ctl[8];                  // [0] abort, [1] last workgroup to retire, [2] a wait was timed
+  int32_t pos[kMaxBatch];          // position of the token each row decodes
+  int32_t active[kMaxBatch];       // rows that still generate
+  float red[kWaves];
+  float part[2][2][kWaves][kMaxBatch][kTile];  // [parity][unit][wave][batch row][weight row]: K-slice partial tiles
+  alignas(16) u16 stage[M::GQA * M::D + 2 * M::D];  // attention: q heads, then the K and V row of this step
+  float merge[kWaves][M::GQA][M::D + 4];
+  unsigned long long t_wait;
+  unsigned long long stamps[4];
+};
+
+#define QMK_MB_STAMP(k)                                                     \
+  do {                                                                      \
+    if (p.timeline != nullptr && c.tid == 0) s.stamps[k] = wall_clock64(); \
+  } while (0)
+
+template <class S>
+__device__ __forceinline__ bool bad_operand(const Params& p, S& s, const Ctx& c, int operand) {
+  if (c.tid == 0) report_error(p, QMK_DEV_BAD_OPERAND, c.inst_idx, c.opcode, operand);
+  return false;
+}
+
+// Lanes 0..n-1 each poll the counter `ctr_of(i)` up to `expected(i)`; false (uniformly) on a timeout.
+template <class S, class CtrOf, class Expected>
+__device__ __forceinline__ bool wait_counters(const Params& p, S& s, const Ctx& c, int n, CtrOf ctr_of, Expected expected) {
+  if (c.tid < n) {
+    if (!poll_counter(ctr_of(c.tid), expected(c.tid), p.spin_limit)) {
+      s.ctl[0] = 1;
+      report_error(p, QMK_DEV_WAIT_TIMEOUT, c.inst_idx, c.opcode, c.tid);
+    }
+  }
+  if (p.timeline != nullptr && c.tid == 0) {
+    s.t_wait = wall_clock64();
+    s.ctl[2] = 1;
+  }
+  __syncthreads();
+  return s.ctl[0] == 0;
+}
+template <class S>
+__device__ __forceinline__ bool wait_counter(const Params& p, S& s, const Ctx& c, int layer, int row, int expected) {
+  return wait_counters(p, s, c, 1, [&](int) { return counter_ptr(p, layer, row, 0); }, [&](int) { return expected; });
+}
+
+// All stores of the workgroup are in memory; then thread 0 adds `amount` to one counter.
+__device__ __forceinline__ void publish_after_stores(const Params& p, const Ctx& c, int layer, int row, int slot, int amount) {
+  release_stores();
+  __syncthreads();
+  if (c.tid == 0) publish(counter_ptr(p, layer, row, slot), amount);
+}
+
+// ================================================================ 1, 6, 9 ==
+// [op, layer, batch_size, -, -, -, batch_row]   (9: [op, batch_size, -, -, -, -, batch_row])
+// dst[row] = RMSNorm(hidden[row]) for an active row, zeros otherwise   (python_vm.py:139-160, 614-634, 668-690)
+template <class M>
+__device__ bool op_rms_row(const Params& p, Smem<M>& s, const Ctx& c) {
+  static_assert(M::H == kThreads * 4, "one thread normalises four elements");
+  const bool lm = c.opcode == OP_LM_RMS;
+  const int layer = lm ? p.num_layers - 1 : s.inst[1];
+  const int B = lm ? s.inst[1] : s.inst[2], row = s.inst[6];
+  if (layer < 0 || layer >= p.num_layers) return bad_operand(p, s, c, 1);
+  if (B != p.batch) return bad_operand(p, s, c, lm ? 1 : 2);
+  if (row < 0 || row >= B) return bad_operand(p, s, c, 6);
+  const u16* weight;
+  u16* dst;
+  int my_row, wait_layer = layer, wait_row;
+  if (c.opcode == OP_ATTN_RMS) {
+    weight = p.attn_norm + static_cast<size_t>(layer) * M::H, dst = p.attn_rms_out, my_row = ROW_ATTN_RMS;
+    wait_layer = layer - 1, wait_row = ROW_DOWN;
+  } else if (c.opcode == OP_MLP_RMS) {
+    weight = p.mlp_norm + static_cast<size_t>(layer) * M::H, dst = p.mlp_rms_out, my_row = ROW_MLP_RMS, wait_row = ROW_OPROJ;
+  } else {
+    weight = p.lm_norm, dst = p.lm_rms_out, my_row = ROW_LM_RMS, wait_row = ROW_DOWN;
+  }
+  const uint2 wv = *reinterpret_cast<const uint2*>(weight + c.tid * 4);
+  if (wait_layer >= 0 && !wait_counter(p, s, c, wait_layer, wait_row, M::H / kTile)) return false;
+  uint32_t lo = 0, hi = 0;
+  if (s.active[row]) {
+    const uint64_t hw = ld_shared64(p.hidden + static_cast<size_t>(row) * M::H + c.tid * 4);
+    const float x0 = bf_lo(static_cast<uint32_t>(hw)), x1 = bf_hi(static_cast<uint32_t>(hw));
+    const float x2 = bf_lo(static_cast<uint32_t>(hw >> 32)), x3 = bf_hi(static_cast<uint32_t>(hw >> 32));
+    float ss = __builtin_fmaf(x3, x3, __builtin_fmaf(x2, x2, __builtin_fmaf(x1, x1, x0 * x0)));
+    ss = block_sum(ss, s.red);
+    const float rstd = 1.0f / sqrtf(ss / static_cast<float>(M::H) + p.rms_norm_eps);
+    lo = static_cast<uint32_t>(f2bf(bf_lo(wv.x) * round_bf16(x0 * rstd))) | (static_cast<uint32_t>(f2bf(bf_hi(wv.x) * round_bf16(x1 * rstd))) << 16);
+    hi = static_cast<uint32_t>(f2bf(bf_lo(wv.y) * round_bf16(x2 * rstd))) | (static_cast<uint32_t>(f2bf(bf_hi(wv.y) * round_bf16(x3 * rstd))) << 16);
+  }
+  __hip_atomic_store(reinterpret_cast<uint64_t*>(dst + static_cast<size_t>(row) * M::H + c.tid * 4), (static_cast<uint64_t>(hi) << 32) | lo,
+                     __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  publish_after_stores(p, c, layer, my_row, 0, 1);
+  return true;
+}
+
+// ------------------------------------------------------------ GEMM core ----
+// One lane's share of a 16-row x 256-column weight segment: row l%16, 16 bytes of each 64-byte chunk.
+struct Seg {
+  v4u a[kSegChunks];
+};
+__device__ __forceinline__ void load_seg(Seg& sg, const u16* lane_ptr) {
+#pragma unroll
+  for (int j = 0; j < kSegChunks; ++j) sg.a[j] = __builtin_nontemporal_load(reinterpret_cast<const v4u*>(lane_ptr + j * kChunk));
+}
+__device__ __forceinline__ f4 mma_seg(const Seg& sg, const v4u (&x)[kSegChunks], f4 acc) {
+#pragma unroll
+  for (int j = 0; j < kSegChunks; ++j)
+    acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, sg.a[j]), __builtin_bit_cast(bf16x8, x[j]), acc, 0, 0, 0);
+  return acc;
+}
+// This lane's share of the activations [B, ld] for one segment: batch row l%16 (zeros beyond the
+// batch), the same 16 bytes of every chunk as the weights.  The buffers are written during the launch.
+__device__ __forceinline__ void load_x(v4u (&x)[kSegChunks], const u16* act, int ld, int B, int k0, int lane) {
+  const int n = lane & 15, g = lane >> 4;
+#pragma unroll
+  for (int j = 0; j < kSegChunks; ++j) {
+    x[j] = v4u{0, 0, 0, 0};
+    if (n < B) x[j] = ld_shared128(act + static_cast<size_t>(n) * ld + k0 + j * kChunk + g * 8);
+  }
+}
+// The wave's partial tile (C layout: rows 4*(l/16)..+3, column l%16) into its LDS slot.
+template <class M>
+__device__ __forceinline__ void park(Smem<M>& s, int parity, int unit, int wave, int lane, f4 acc) {
+  *reinterpret_cast<f4*>(&s.part[parity][unit][wave][lane & 15][4 * (lane >> 4)]) = acc;
+}
+// Outputs (2*rp, 2*rp + 1) of the block for batch row b: the eight K-slice partials added up.
+template <class M>
+__device__ __forceinline__ float2 gather(const Smem<M>& s, int parity, int unit, int b, int rp) {
+  float2 v = float2{0.f, 0.f};
+#pragma unroll
+  for (int w = 0; w < kWaves; ++w) {
+    const float2 t = *reinterpret_cast<const float2*>(&s.part[parity][unit][w][b][2 * rp]);
+    v.x += t.x;
+    v.y += t.y;
+  }
+  return v;
+}
+
+// Blocks 0..n-1 of NU weight matrices with K = 2048 (one segment per wave).  `src(j, u)` is the
+// address of row 0, column 0 of block j in matrix u (rows are `M::H` apart); `before(j)` runs on
+// all threads right after the block's tiles are parked (still before the barrier), `epi(j, parity,
+// b, rp)` on threads 0..127 after it.  The ring holds NB blocks; the first NB are requested at once
+// (the caller decides whether that is before or after its wait through `wait`).
+template <class M, int NU, int NB, class Src, class Wait, class Epi>
+__device__ __forceinline__ bool gemm_h(const Params& p, Smem<M>& s, const Ctx& c, int n, const u16* act, int B, Src src, Wait wait, Epi epi) {
+  static_assert(M::H == kWaves * kSeg, "one segment per wave");
+  const int lane = c.tid & 63, wave = c.tid >> 6;
+  const size_t lane_off = static_cast<size_t>(lane & 15) * M::H + wave * kSeg + (lane >> 4) * 8;
+  Seg ring[NB][NU];
+#pragma unroll
+  for (int k = 0; k < NB; ++k)
+    if (k < n)
+#pragma unroll
+      for (int u = 0; u < NU; ++u) load_seg(ring[k][u], src(k, u) + lane_off);
+  if (!wait()) return false;
+  v4u x[kSegChunks];
+  load_x(x, act, M::H, B, wave * kSeg, lane);
+  int parity = 0;
+  for (int j0 = 0; j0 < n; j0 += NB) {
+#pragma unroll
+    for (int k = 0; k < NB; ++k) {
+      const int j = j0 + k;
+      if (j < n) {  // uniform over the workgroup
+#pragma unroll
+        for (int u = 0; u < NU; ++u) {
+          const f4 acc = mma_seg(ring[k][u], x, f4{0.f, 0.f, 0.f, 0.f});
+          park(s, parity, u, wave, lane, acc);
+          if (j + NB < n) load_seg(ring[k][u], src(j + NB, u) + lane_off);
+        }
+        __syncthreads();
+        // Parity: a slot is written again two blocks later, behind the next barrier, which the
+        // reading threads reach only after they are done with it.
+        if (c.tid < 128) epi(j, parity, c.tid & 15, c.tid >> 4);
+        parity ^= 1;
+      }
+    }
+  }
+  return true;
+}
+
+// ===================================================================== 2 ==
+// [2, layer, batch_size, tile_M, n_start, n_end, tile_M_g, tile_N_g]
+// QKV rows of blocks [n_start, n_end) for every batch row from attn_rms_out; RoPE at the row's
+// position on q and k; q -> q_post_rope, k/v -> the row's cache line at its position
+// (python_vm.py:163-266).  One arrival per block on the counter of the block's head.
+template <class M>
+__device__ bool op_qkv(const Params& p, Smem<M>& s, const Ctx& c) {
+  const int layer = s.inst[1], B = s.inst[2], n0 = s.inst[4], n1 = s.inst[5];
+  if (layer < 0 || layer >= p.num_layers) return bad_operand(p, s, c, 1);
+  if (B != p.batch || s.inst[3] != 0) return bad_operand(p, s, c, 2);
+  if (n0 < 0 || n1 < n0 || n1 > M::QKV / kTile) return bad_operand(p, s, c, 4);
+  if (s.inst[6] != kMaxBatch || s.inst[7] != kTile) return bad_operand(p, s, c, 7);
+  const u16* w = p.qkv_w + static_cast<size_t>(layer) * M::QKV * M::H;
+  const size_t tok_stride = static_cast<size_t>(M::NKV) * M::D;
+  const bool ok = gemm_h<M, 1, 3>(
+      p, s, c, n1 - n0, p.attn_rms_out, B, [&](int j, int) { return w + static_cast<size_t>(n0 + j) * kTile * M::H; },
+      [&] { return wait_counter(p, s, c, layer, ROW_ATTN_RMS, B); },
+      [&](int j, int parity, int b, int rp) {
+        if (b >= B || !s.active[b]) return;
+        const float2 v = gather(s, parity, 0, b, rp);
+        const float v0 = round_bf16(v.x), v1 = round_bf16(v.y);
+        const int o = (n0 + j) * kTile + 2 * rp, d = o % M::D, pos = s.pos[b];
+        const size_t cache_row = ((static_cast<size_t>(layer) * B + b) * p.max_seq_len + pos) * tok_stride;
+        if (o < M::NQ * M::D) {
+          st_shared32(p.q_post_rope + static_cast<size_t>(b) * M::NQ * M::D + o,
+                      rope_pair(v0, v1, p.rope_cos + static_cast<size_t>(pos) * M::D, p.rope_sin + static_cast<size_t>(pos) * M::D, d));
+        } else if (o < (M::NQ + M::NKV) * M::D) {
+          st_shared32(p.k_cache + cache_row + (o - M::NQ * M::D),
+                      rope_pair(v0, v1, p.rope_cos + static_cast<size_t>(pos) * M::D, p.rope_sin + static_cast<size_t>(pos) * M::D, d));
+        } else {
+          st_shared32(p.v_cache + cache_row + (o - (M::NQ + M::NKV) * M::D), static_cast<uint32_t>(f2bf(v0)) | (static_cast<uint32_t>(f2bf(v1)) << 16));
+        }
+      });
+  if (!ok) return false;
+  release_stores();
+  __syncthreads();
+  if (c.tid < n1 - n0) publish(counter_ptr(p, layer, ROW_QKV, (n0 + c.tid) / (M::D / kTile)), 1);
+  return true;
+}
+
+// ===================================================================== 3 ==
+// [3, layer, batch_row, kv_head, num_partials, partial_idx, seq_len, is_active]
+// Flash-decoding over one slice of one batch row's context for the GQA group of one KV head
+// (python_vm.py:269-359).  seq_len < 0: the row's position + 1; is_active < 0: the row's flag.  The
+// slices are whole KV blocks of `kv_block` tokens.  An inactive row or an empty slice leaves
+// (0, -inf, not valid) and still counts.  Scoring as in the batch-1 kernel: a wave takes 16 tokens at
+// a time on the matrix cores and keeps one running (max, sum, acc) per query head.
+template <class M>
+__device__ bool op_splitkv(const Params& p, Smem<M>& s, const Ctx& c) {
+  constexpr int D = M::D, GQA = M::GQA;
+  static_assert(D % 64 == 0 && GQA <= 4 && GQA * D <= kThreads, "a lane owns whole 16-byte vectors of K; one thread per merged output");
+  const int layer = s.inst[1], b = s.inst[2], kvh = s.inst[3], P = s.inst[4], part = s.inst[5];
+  if (layer < 0 || layer >= p.num_layers) return bad_operand(p, s, c, 1);
+  if (b < 0 || b >= p.batch) return bad_operand(p, s, c, 2);
+  if (kvh < 0 || kvh >= M::NKV) return bad_operand(p, s, c, 3);
+  if (P < 1 || P > p.max_splits || part < 0 || part >= P) return bad_operand(p, s, c, 4);
+  const int pos = s.pos[b];
+  const int seq_len = s.inst[6] >= 0 ? s.inst[6] : pos + 1;
+  if (seq_len > p.max_seq_len) return bad_operand(p, s, c, 6);
+  const bool active = s.inst[7] == 0 ? false : (s.inst[7] == 1 ? true : s.active[b] != 0);
+  const int lane = c.tid & 63, wave = c.tid >> 6;
+  constexpr int kStride = M::NQ + 2 * M::NKV;   // counter slots per batch row
+
+  const int total = max(1, (seq_len + p.kv_block - 1) / p.kv_block);
+  const int per = max(1, (total + P - 1) / P);
+  const int t0 = part * per * p.kv_block;
+  const int t1 = min(min(part * per + per, total) * p.kv_block, seq_len);
+  const bool empty = !active || t0 >= t1;
+  const bool has_new = !empty && pos >= t0 && pos < t1;
+
+  constexpr int KV16 = D / 32, NT = D / 16, kTok = 16, kStep = kWaves * kTok;
+  const int c16 = lane & 15, g4 = lane >> 4;
+  const size_t tok_stride = static_cast<size_t>(M::NKV) * D;
+  const size_t row_of_kvh = (static_cast<size_t>(layer) * p.batch + b) * p.max_seq_len * tok_stride + static_cast<size_t>(kvh) * D;
+  const u16* kbase = p.k_cache + row_of_kvh + g4 * (D / 4);
+  const u16* vbase = p.v_cache + row_of_kvh + c16 * NT;
+  struct Tile {
+    v4u k[KV16];
+    uint32_t v[4][NT / 2];
+  };
+  // Rows of earlier positions do not depend on this step; tokens past the slice are fetched from
+  // its last row and masked when scored.
+  auto fetch = [&](Tile& tl, int tb) {
+    const int tk = min(tb + c16, t1 - 1);
+#pragma unroll
+    for (int j = 0; j < KV16; ++j) tl.k[j] = reinterpret_cast<const v4u*>(kbase + static_cast<size_t>(tk) * tok_stride)[j];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const int tv = min(tb + 4 * g4 + j, t1 - 1);
+      const uint32_t* src = reinterpret_cast<const uint32_t*>(vbase + static_cast<size_t>(tv) * tok_stride);
+#pragma unroll
+      for (int i = 0; i < NT / 2; ++i) tl.v[j][i] = src[i];
+    }
+  };
+  int tb = t0 + wave * kTok;
+  Tile cur;
+#pragma unroll
+  for (int j = 0; j < KV16; ++j) cur.k[j] = v4u{0, 0, 0, 0};
+#pragma unroll
+  for (int j = 0; j < 4; ++j)
+#pragma unroll
+    for (int i = 0; i < NT / 2; ++i) cur.v[j][i] = 0;
+  if (!empty && tb < t1) fetch(cur, tb);
+
+  if (!wait_counters(
+          p, s, c, GQA + 2,
+          [&](int i) {
+            const int slot = i < GQA ? kvh * GQA + i : (i == GQA ? M::NQ + kvh : M::NQ + M::NKV + kvh);
+            return counter_ptr(p, layer, ROW_QKV, slot);
+          },
+          [&](int) { return D / kTile; }))
+    return false;
+
+  const int head0 = kvh * GQA;
+  float* lse_out = p.attn_lse + (static_cast<size_t>(b) * M::NQ + head0) * p.max_splits + part;
+  float* part_out = p.attn_partial + ((static_cast<size_t>(b) * M::NQ + head0) * p.max_splits + part) * D;
+  uint8_t* valid_out = p.partial_valid ? p.partial_valid + (static_cast<size_t>(b) * M::NQ + head0) * p.max_splits + part : nullptr;
+  auto arrive = [&] {
+    release_stores();
+    __syncthreads();
+    if (c.tid < GQA) publish(counter_ptr(p, layer, ROW_SPLITKV, b * kStride + head0 + c.tid), 1);
+  };
+  if (empty) {  // uniform
+    if (c.tid < GQA * D) {
+      const int h = c.tid / D, d = c.tid % D;
+      st_shared_f32(part_out + static_cast<size_t>(h) * p.max_splits * D + d, 0.f);
+      if (d == 0) {
+        st_shared_f32(lse_out + static_cast<size_t>(h) * p.max_splits, -INFINITY);
+        if (valid_out) st_shared8(valid_out + static_cast<size_t>(h) * p.max_splits, 0);
+      }
+    }
+    arrive();
+    return true;
+  }
+
+  // q of the GQA group and, if the slice holds it, the K/V row this launch appended: bf16 in LDS.
+  u16* stage16 = s.stage;
+  constexpr int kQ = 0, kK = GQA * D, kV = GQA * D + D;
+  {
+    const size_t new_row = row_of_kvh + static_cast<size_t>(pos) * tok_stride;
+    constexpr int kQChunks = GQA * D / 8, kRowChunks = D / 8;
+    const int tid = c.tid;
+    if (tid < kQChunks) {
+      reinterpret_cast<v4u*>(stage16 + kQ)[tid] = ld_shared128(p.q_post_rope + static_cast<size_t>(b) * M::NQ * D + head0 * D + tid * 8);
+    } else if (tid < kQChunks + kRowChunks && has_new) {
+      reinterpret_cast<v4u*>(stage16 + kK)[tid - kQChunks] = ld_shared128(p.k_cache + new_row + (tid - kQChunks) * 8);
+    } else if (tid < kQChunks + 2 * kRowChunks && has_new) {
+      reinterpret_cast<v4u*>(stage16 + kV)[tid - kQChunks - kRowChunks] = ld_shared128(p.v_cache + new_row + (tid - kQChunks - kRowChunks) * 8);
+    }
+  }
+  __syncthreads();
+
+  typedef short bf4 __attribute__((ext_vector_type(4)));
+  typedef uint32_t u2 __attribute__((ext_vector_type(2)));
+  const float qscale = p.attn_scale * 1.4426950408889634f;  // scores in the log2 domain
+  bf4 qb[NT];
+#pragma unroll
+  for (int j = 0; j < KV16; ++j) {
+    v4u qv = v4u{0, 0, 0, 0};
+    if (c16 < GQA) qv = reinterpret_cast<const v4u*>(stage16 + kQ + c16 * D + g4 * (D / 4))[j];
+    qb[2 * j] = __builtin_bit_cast(bf4, u2{qv.x, qv.y});
+    qb[2 * j + 1] = __builtin_bit_cast(bf4, u2{qv.z, qv.w});
+  }
+  QMK_MB_STAMP(0);
+
+  float m_run = -INFINITY, l_run = 0.f;
+  f4 acc[NT];
+#pragma unroll
+  for (int i = 0; i < NT; ++i) acc[i] = f4{0.f, 0.f, 0.f, 0.f};
+
+  while (tb < t1) {
+    Tile nxt = cur;
+    if (tb + kStep < t1) fetch(nxt, tb + kStep);
+    if (pos >= tb && pos < tb + kTok) {  // the row appended during this launch comes from LDS
+      // (also where a token past the slice was redirected to this row: what the cache holds there is not defined yet)
+      if (min(tb + c16, t1 - 1) == pos) {
+#pragma unroll
+        for (int j = 0; j < KV16; ++j) cur.k[j] = reinterpret_cast<const v4u*>(stage16 + kK + g4 * (D / 4))[j];
+      }
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        if (min(tb + 4 * g4 + j, t1 - 1) == pos) {
+#pragma unroll
+          for (int i = 0; i < NT / 2; ++i) cur.v[j][i] = reinterpret_cast<const uint32_t*>(stage16 + kV + c16 * NT)[i];
+        }
+      }
+    }
+    f4 sc = f4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int j = 0; j < KV16; ++j) {
+      sc = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(__builtin_bit_cast(bf4, u2{cur.k[j].x, cur.k[j].y}), qb[2 * j], sc, 0, 0, 0);
+      sc = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(__builtin_bit_cast(bf4, u2{cur.k[j].z, cur.k[j].w}), qb[2 * j + 1], sc, 0, 0, 0);
+    }
+    float mt = -INFINITY;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      sc[i] = (tb + 4 * g4 + i < t1) ? sc[i] * qscale : -INFINITY;
+      mt = fmaxf(mt, sc[i]);
+    }
+    mt = fmaxf(mt, __shfl_xor(mt, 16));
+    mt = fmaxf(mt, __shfl_xor(mt, 32));
+    const float mn = fmaxf(m_run, mt);
+    const float alpha = exp2_fast(m_run - mn);
+    m_run = mn;
+    float pr[4], psum = 0.f;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      pr[i] = (c16 < GQA) ? exp2_fast(sc[i] - mn) : 0.f;
+      psum += pr[i];
+    }
+    l_run = __builtin_fmaf(l_run, alpha, psum);
+    uint32_t hi[4], lo[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      hi[i] = f2bf(pr[i]);
+      lo[i] = f2bf(pr[i] - bf2f(static_cast<u16>(hi[i])));
+    }
+    const bf4 p_hi = __builtin_bit_cast(bf4, u2{hi[0] | (hi[1] << 16), hi[2] | (hi[3] << 16)});
+    const bf4 p_lo = __builtin_bit_cast(bf4, u2{lo[0] | (lo[1] << 16), lo[2] | (lo[3] << 16)});
+    float a_head[4];
+    bool rescale = false;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      a_head[i] = i < GQA ? __int_as_float(__builtin_amdgcn_readlane(__float_as_int(alpha), i)) : 1.f;
+      rescale = rescale || a_head[i] != 1.f;
+    }
+    if (rescale) {
+#pragma unroll
+      for (int tau = 0; tau < NT; ++tau)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) acc[tau][i] *= a_head[i];
+    }
+#pragma unroll
+    for (int tau = 0; tau < NT; ++tau) {
+      const int w = tau / 2;
+      uint32_t b0, b1;
+      if (tau & 1) {
+        b0 = (cur.v[0][w] >> 16) | (cur.v[1][w] & 0xffff0000u);
+        b1 = (cur.v[2][w] >> 16) | (cur.v[3][w] & 0xffff0000u);
+      } else {
+        b0 = (cur.v[0][w] & 0xffffu) | (cur.v[1][w] << 16);
+        b1 = (cur.v[2][w] & 0xffffu) | (cur.v[3][w] << 16);
+      }
+      const bf4 vb = __builtin_bit_cast(bf4, u2{b0, b1});
+      acc[tau] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(p_hi, vb, acc[tau], 0, 0, 0);
+      acc[tau] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(p_lo, vb, acc[tau], 0, 0, 0);
+    }
+    cur = nxt;
+    tb += kStep;
+  }
+  QMK_MB_STAMP(1);
+
+  l_run += __shfl_xor(l_run, 16);
+  l_run += __shfl_xor(l_run, 32);
+  if (lane < 16) {
+#pragma unroll
+    for (int tau = 0; tau < NT; ++tau)
+#pragma unroll
+      for (int i = 0; i < GQA; ++i) s.merge[wave][i][c16 * NT + tau] = acc[tau][i];
+    if (c16 < GQA) {
+      s.merge[wave][c16][D] = m_run;
+      s.merge[wave][c16][D + 1] = l_run;
+    }
+  }
+  __syncthreads();
+  if (c.tid < GQA * D) {
+    const int h = c.tid / D, d = c.tid % D;
+    float mx = -INFINITY;
+#pragma unroll
+    for (int w = 0; w < kWaves; ++w) mx = fmaxf(mx, s.merge[w][h][D]);
+    float den = 0.f, num = 0.f;
+#pragma unroll
+    for (int w = 0; w < kWaves; ++w) {
+      const float mw = s.merge[w][h][D];
+      const float wgt = (mw == -INFINITY) ? 0.f : exp2_fast(mw - mx);
+      den = __builtin_fmaf(s.merge[w][h][D + 1], wgt, den);
+      num = __builtin_fmaf(s.merge[w][h][d], wgt, num);
+    }
+    const bool none = !(den > 0.f);
+    st_shared_f32(part_out + static_cast<size_t>(h) * p.max_splits * D + d, none ? 0.f : num / den);
+    if (d == 0) {
+      st_shared_f32(lse_out + static_cast<size_t>(h) * p.max_splits, none ? -INFINITY : mx + log2f(den));
+      if (valid_out) st_shared8(valid_out + static_cast<size_t>(h) * p.max_splits, none ? 0 : 1);
+    }
+  }
+  QMK_MB_STAMP(2);
+  arrive();
+  return true;
+}
+
+// ===================================================================== 4 ==
+// [4, layer, batch_row, head_start, num_partials, len, list..., is_terminal, output_partial, valid_partials, is_active]
+// Log-sum-exp merge (log2 domain) of the listed partials of four query heads of one batch row,
+// over the valid ones only (python_vm.py:442-551).  Thread t < GQA*D/2 produces two neighbouring dims.
+template <class M>
+__device__ bool op_reduce(const Params& p, Smem<M>& s, const Ctx& c) {
+  constexpr int D = M::D, R = M::GQA;
+  constexpr int kStride = M::NQ + 2 * M::NKV;
+  const int layer = s.inst[1], b = s.inst[2], head0 = s.inst[3], P = s.inst[4], n = s.inst[5];
+  if (layer < 0 || layer >= p.num_layers) return bad_operand(p, s, c, 1);
+  if (b < 0 || b >= p.batch) return bad_operand(p, s, c, 2);
+  if (head0 < 0 || head0 + R > M::NQ) return bad_operand(p, s, c, 3);
+  if (n < 1 || n > kMaxList || P < 1) return bad_operand(p, s, c, 5);
+  for (int i = 0; i < n; ++i)
+    if (s.inst[6 + i] < 0 || s.inst[6 + i] >= p.max_splits) return bad_operand(p, s, c, 6 + i);
+  const bool terminal = s.inst[6 + n] != 0;
+  const int out_slot = s.inst[7 + n];
+  if (!terminal && (out_slot < 0 || out_slot >= p.max_splits)) return bad_operand(p, s, c, 7 + n);
+  const int flag = s.inst[9 + n];
+  const bool active = flag == 0 ? false : (flag == 1 ? true : s.active[b] != 0);
+  const bool worker = c.tid < R * D / 2;
+  const int h = head0 + c.tid / (D / 2), d = 2 * (c.tid % (D / 2));
+  u16* out = p.attn_out + static_cast<size_t>(b) * M::NQ * D + static_cast<size_t>(h) * D + d;
+  if (!active) {
+    if (worker) st_shared32(out, 0u);
+    publish_after_stores(p, c, layer, ROW_REDUCE, b, R);
+    return true;
+  }
+  if (!wait_counters(p, s, c, R, [&](int i) { return counter_ptr(p, layer, ROW_SPLITKV, b * kStride + head0 + i); }, [&](int) { return P; }))
+    return false;
+  if (worker) {
+    const size_t row = (static_cast<size_t>(b) * M::NQ + h) * p.max_splits;
+    const float* lse = p.attn_lse + row;
+    const float* part = p.attn_partial + row * D + d;
+    const uint8_t* valid = p.partial_valid ? p.partial_valid + row : nullptr;
+    float e[kMaxList];
+    uint64_t two[kMaxList];
+    bool ok[kMaxList];
+#pragma unroll
+    for (int i = 0; i < kMaxList; ++i) {   // slots beyond n re-read the last listed partial and get weight 0
+      const int j = s.inst[6 + min(i, n - 1)];
+      e[i] = ld_shared_f32(lse + j);
+      two[i] = ld_shared64(part + static_cast<size_t>(j) * D);
+      ok[i] = valid ? ld_shared8(valid + j) != 0 : true;
+    }
+    float mx = -INFINITY;
+#pragma unroll
+    for (int i = 0; i < kMaxList; ++i) {
+      ok[i] = i < n && (valid ? ok[i] : (e[i] > kNoContribution && e[i] < INFINITY));
+      if (ok[i]) mx = fmaxf(mx, e[i]);
+    }
+    float num0 = 0.f, num1 = 0.f, den = 0.f;
+#pragma unroll
+    for (int i = 0; i < kMaxList; ++i) {
+      const float f = ok[i] ? exp2_fast(e[i] - mx) : 0.f;
+      num0 = __builtin_fmaf(__uint_as_float(static_cast<uint32_t>(two[i])), f, num0);
+      num1 = __builtin_fmaf(__uint_as_float(static_cast<uint32_t>(two[i] >> 32)), f, num1);
+      den += f;
+    }
+    const bool any = den > 0.f;
+    const float o0 = any ? num0 / den : 0.f, o1 = any ? num1 / den : 0.f;
+    if (terminal) {
+      st_shared32(out, static_cast<uint32_t>(f2bf(o0)) | (static_cast<uint32_t>(f2bf(o1)) << 16));
+    } else {
+      float* dst = p.attn_partial + (row + out_slot) * D + d;
+      st_shared_f32(dst, o0);
+      st_shared_f32(dst + 1, o1);
+      if (d == 0) {
+        st_shared_f32(p.attn_lse + row + out_slot, any ? mx + log2f(den) : (valid ? 0.f : kNoContribution - 1.0f));
+        if (p.partial_valid) st_shared8(p.partial_valid + row + out_slot, any ? 1 : 0);
+      }
+    }
+  }
+  publish_after_stores(p, c, layer, ROW_REDUCE, b, R);
+  return true;
+}
+
+// ===================================================================== 5 ==
+// [5, layer, batch_size, tile_M, n_start, n_end, reduction_block, tile_M_g, tile_N_g]
+// hidden[b, r] = bf16(hidden[b, r] + bf16(W_o[r] . attn_out[b])) for active rows   (python_vm.py:554-611)
+template <class M>
+__device__ bool op_oproj(const Params& p, Smem<M>& s, const Ctx& c) {
+  const int layer = s.inst[1], B = s.inst[2], n0 = s.inst[4], n1 = s.inst[5];
+  if (layer < 0 || layer >= p.num_layers) return bad_operand(p, s, c, 1);
+  if (B != p.batch || s.inst[3] != 0) return bad_operand(p, s, c, 2);
+  if (n0 < 0 || n1 < n0 || n1 > M::H / kTile) return bad_operand(p, s, c, 4);
+  if (s.inst[6] != 0) return bad_operand(p, s, c, 6);
+  if (s.inst[7] != kMaxBatch || s.inst[8] != kTile) return bad_operand(p, s, c, 8);
+  const u16* w = p.o_w + static_cast<size_t>(layer) * M::H * M::H;
+  const bool ok = gemm_h<M, 1, 3>(
+      p, s, c, n1 - n0, p.attn_out, B, [&](int j, int) { return w + static_cast<size_t>(n0 + j) * kTile * M::H; },
+      [&] {
+        return wait_counters(p, s, c, B, [&](int i) { return counter_ptr(p, layer, ROW_REDUCE, i); }, [&](int) { return M::NQ; });
+      },
+      [&](int j, int parity, int b, int rp) {
+        if (b >= B || !s.active[b]) return;
+        const float2 v = gather(s, parity, 0, b, rp);
+        residual_pair(p.hidden + static_cast<size_t>(b) * M::H + (n0 + j) * kTile + 2 * rp, v.x, v.y);
+      });
+  if (!ok) return false;
+  publish_after_stores(p, c, layer, ROW_OPROJ, 0, n1 - n0);
+  return true;
+}
+
+// ===================================================================== 7 ==
+// [7, layer, batch_size, tile_M, len, blocks..., tile_M_g, tile_N_g]
+// silu_out[b, r] = bf16(bf16(silu(bf16(W_g[r] . y_b))) * bf16(W_u[r] . y_b)), zero for inactive rows
+// (python_vm.py:637-665; operations.py:265-282)
+template <class M>
+__device__ bool op_upgate(const Params& p, Smem<M>& s, const Ctx& c) {
+  const int layer = s.inst[1], B = s.inst[2], n = s.inst[4];
+  if (layer < 0 || layer >= p.num_layers) return bad_operand(p, s, c, 1);
+  if (B != p.batch || s.inst[3] != 0) return bad_operand(p, s, c, 2);
+  if (n < 0 || n > kInstWords - 7) return bad_operand(p, s, c, 4);
+  for (int i = 0; i < n; ++i)
+    if (s.inst[5 + i] < 0 || s.inst[5 + i] >= M::F / kTile) return bad_operand(p, s, c, 5 + i);
+  if (s.inst[5 + n] != kMaxBatch || s.inst[6 + n] != kTile) return bad_operand(p, s, c, 6 + n);
+  const u16* wg = p.gate_w + static_cast<size_t>(layer) * M::F * M::H;
+  const u16* wu = p.up_w + static_cast<size_t>(layer) * M::F * M::H;
+  const bool ok = gemm_h<M, 2, 2>(
+      p, s, c, n, p.mlp_rms_out, B, [&](int j, int u) { return (u ? wu : wg) + static_cast<size_t>(s.inst[5 + j]) * kTile * M::H; },
+      [&] { return wait_counter(p, s, c, layer, ROW_MLP_RMS, B); },
+      [&](int j, int parity, int b, int rp) {
+        if (b >= B) return;
+        uint32_t word = 0;
+        if (s.active[b]) {
+          const float2 g = gather(s, parity, 0, b, rp), u = gather(s, parity, 1, b, rp);
+          const float g0 = round_bf16(g.x), g1 = round_bf16(g.y);
+          const float a0 = round_bf16(g0 / (1.0f + expf(-g0))), a1 = round_bf16(g1 / (1.0f + expf(-g1)));
+          word = static_cast<uint32_t>(f2bf(a0 * round_bf16(u.x))) | (static_cast<uint32_t>(f2bf(a1 * round_bf16(u.y))) << 16);
+        }
+        st_shared32(p.silu_out + static_cast<size_t>(b) * M::F + s.inst[5 + j] * kTile + 2 * rp, word);
+      });
+  if (!ok) return false;
+  publish_after_stores(p, c, layer, ROW_UPGATE, 0, n);
+  return true;
+}
+
+// ===================================================================== 8 ==
+// [8, layer, batch_size, tile_M, n_start, n_end, tile_M_g, tile_N_g]
+// hidden[b, r] = bf16(hidden[b, r] + bf16(W_d[r] . silu_out[b])) for active rows, the whole K in
+// one instruction (python_vm.py:554-611).  A wave owns F/8 columns: F/2048 segments per block, all
+// requested before the wait; its share of silu_out follows the wait, two segments at a time.
+template <class M>
+__device__ bool op_down(const Params& p, Smem<M>& s, const Ctx& c) {
+  constexpr int NS = M::F / (kWaves * kSeg);   // segments per wave and block
+  static_assert(M::F % (kWaves * kSeg) == 0, "whole segments");
+  const int layer = s.inst[1], B = s.inst[2], n0 = s.inst[4], n1 = s.inst[5];
+  if (layer < 0 || layer >= p.num_layers) return bad_operand(p, s, c, 1);
+  if (B != p.batch || s.inst[3] != 0) return bad_operand(p, s, c, 2);
+  if (n0 < 0 || n1 < n0 || n1 > M::H / kTile) return bad_operand(p, s, c, 4);
+  if (s.inst[6] != kMaxBatch || s.inst[7] != kTile) return bad_operand(p, s, c, 7);
+  const int lane = c.tid & 63, wave = c.tid >> 6;
+  const u16* w = p.down_w + static_cast<size_t>(layer) * M::H * M::F;
+  const int k0 = wave * NS * kSeg;
+  const size_t lane_off = static_cast<size_t>(lane & 15) * M::F + k0 + (lane >> 4) * 8;
+  Seg a[NS];
+  auto request = [&](int block) {
+#pragma unroll
+    for (int q = 0; q < NS; ++q) load_seg(a[q], w + static_cast<size_t>(block) * kTile * M::F + lane_off + q * kSeg);
+  };
+  if (n0 < n1) request(n0);
+  if (!wait_counter(p, s, c, layer, ROW_UPGATE, M::F / kTile)) return false;
+  int parity = 0;
+  for (int blk = n0; blk < n1; ++blk) {
+    f4 acc = f4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int q = 0; q < NS; ++q) {
+      v4u x[kSegChunks];
+      load_x(x, p.silu_out, M::F, B, k0 + q * kSeg, lane);
+      acc = mma_seg(a[q], x, acc);
+    }
+    park(s, parity, 0, wave, lane, acc);
+    if (blk + 1 < n1) request(blk + 1);
+    __syncthreads();
+    if (c.tid < 128) {
+      const int b = c.tid & 15, rp = c.tid >> 4;
+      if (b < B && s.active[b]) {
+        const float2 v = gather(s, parity, 0, b, rp);
+        residual_pair(p.hidden + static_cast<size_t>(b) * M::H + blk * kTile + 2 * rp, v.x, v.y);
+      }
+    }
+    parity ^= 1;
+  }
+  publish_after_stores(p, c, layer, ROW_DOWN, 0, n1 - n0);
+  return true;
+}
+
+// ==================================================================== 10 ==
+// [10, batch_size, start_block, end_block, tile_M_g, tile_N_g]
+// logits[b, r] = bf16(W_lm[r] . lm_head_rms_out[b]); -1e9 for inactive rows   (python_vm.py:693-715)
+template <class M>
+__device__ bool op_lmhead(const Params& p, Smem<M>& s, const Ctx& c) {
+  const int B = s.inst[1], n0 = s.inst[2], n1 = s.inst[3];
+  if (B != p.batch) return bad_operand(p, s, c, 1);
+  if (n0 < 0 || n1 < n0 || static_cast<long>(n1 - 1) * kTile >= p.vocab_size) return bad_operand(p, s, c, 3);
+  if (s.inst[4] != kMaxBatch || s.inst[5] != kTile) return bad_operand(p, s, c, 5);
+  const int last = p.vocab_size - 1;
+  const int lane_row = c.tid & 15;
+  // The last block may be ragged: its missing rows re-read the last row and are not stored.
+  return gemm_h<M, 1, 3>(
+      p, s, c, n1 - n0, p.lm_rms_out, B,
+      [&](int j, int) {
+        const int r0 = (n0 + j) * kTile;
+        return p.lm_w + static_cast<size_t>(min(r0 + lane_row, last) - lane_row) * M::H;
+      },
+      [&] { return wait_counter(p, s, c, p.num_layers - 1, ROW_LM_RMS, B); },
+      [&](int j, int parity, int b, int rp) {
+        if (b >= B) return;
+        const int o = (n0 + j) * kTile + 2 * rp;
+        const float2 v = s.active[b] ? gather(s, parity, 0, b, rp) : float2{-1e9f, -1e9f};
+        u16* dst = p.logits + static_cast<size_t>(b) * p.vocab_size + o;
+        if (o + 1 < p.vocab_size && (reinterpret_cast<uintptr_t>(dst) & 3) == 0) {
+          st_shared32(dst, static_cast<uint32_t>(f2bf(v.x)) | (static_cast<uint32_t>(f2bf(v.y)) << 16));
+        } else {
+          if (o < p.vocab_size) st_shared16(dst, f2bf(v.x));
+          if (o + 1 < p.vocab_size) st_shared16(dst + 1, f2bf(v.y));
+        }
+      });
+}
+
+}  // namespace mb
+}  // namespace qmk

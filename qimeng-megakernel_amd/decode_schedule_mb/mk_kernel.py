@@ -1,17 +1,328 @@
-"""Launcher of the batch route's kernel (`…/A100/multi_batch/decode_schedule/mk_kernel.py:41-111`).
+"""Load and call the gfx950 batch decode kernel through its C ABI.
 
-The gfx950 kernel for batch 2..16 does not exist yet.  Nothing else stands in for it: asking for
-it fails.
+Host-side counterpart of the reference's launcher of the batch route
+(`…/A100/multi_batch/decode_schedule/mk_kernel.py:41-111`): ``get_mk`` returns the ``mk``
+callable, ``call_mk(globs, mk)`` passes the 22 tensors, ``pos_id, batch_size, attn_scale,
+rms_norm_eps``, the three control tensors and the three RMSNorm scratch tensors in the
+reference's positional order, ``run_instructions`` executes an arbitrary instruction list.  The
+callable wraps ``qmk_decode_step_batch`` of ``libqmk_hip.so`` (``include/qmk.h``) with ctypes.
+
+There is no fallback: a missing library is an ``ImportError``, a non-GPU tensor a
+``ValueError`` and a device-side error a ``RuntimeError``.
 """
 from __future__ import annotations
 
-from typing import Any
+import ctypes
+import math
+from pathlib import Path
+from typing import Any, Sequence
+
+import torch
+
+from ..decode_schedule import mk_kernel as _single
+from ..decode_schedule.instructions.scheduler import tensorize_instructions
+from ..decode_schedule.model_config import LlamaConfig
+from ..instruction import Instruction
+from .decode_state import batch_size as _batch_size
+from .globs import Globals
+from .instructions import scheduler as _scheduler
+
+_P = ctypes.c_void_p
+_I = ctypes.c_int32
+MAX_BATCH = 16
 
 
-def get_mk(mk_dir: Any = None):
-    raise ImportError("the gfx950 decode kernel for batch sizes 2..16 is not built; "
-                      "only the batch-1 kernel (decode_schedule.mk_kernel) is available")
+class QmkBatchArgs(ctypes.Structure):
+    """Mirror of ``struct QmkBatchArgs`` in include/qmk.h (field order is the ABI)."""
+
+    _fields_ = [
+        ("struct_size", ctypes.c_uint32), ("model", ctypes.c_uint32),
+        ("flags", ctypes.c_uint32), ("spin_limit", ctypes.c_uint32),
+        ("instructions", _P), ("hidden_states", _P), ("q_post_rope", _P), ("k_cache", _P), ("v_cache", _P),
+        ("attn_out", _P), ("attn_lse_intermediates", _P), ("attn_out_intermediates", _P), ("silu_out", _P),
+        ("logits", _P), ("attn_norm_weights", _P), ("qkv_weights", _P), ("rope_cos", _P), ("rope_sin", _P),
+        ("o_proj_weights", _P), ("mlp_norm_weights", _P), ("up_proj_weights", _P), ("gate_proj_weights", _P),
+        ("down_proj_weights", _P), ("lm_head_norm_weights", _P), ("lm_head_weights", _P), ("barriers", _P),
+        ("num_queues", _I), ("num_insts", _I), ("num_layers", _I), ("num_layer_barriers", _I),
+        ("barrier_slots", _I), ("max_seq_len", _I), ("max_splits", _I), ("vocab_size", _I), ("rope_rows", _I),
+        ("pos_id", _I), ("batch_size", _I), ("kv_block_size", _I),
+        ("attn_scale", ctypes.c_float), ("rms_norm_eps", ctypes.c_float),
+        ("position_ids", _P), ("active_mask", _P), ("attn_partial_valid", _P),
+        ("attn_rms_out", _P), ("mlp_rms_out", _P), ("lm_head_rms_out", _P),
+        ("timeline", _P), ("stream", _P),
+    ]
 
 
-def call_mk(globs: Any, mk: Any) -> None:
-    raise ImportError("the gfx950 decode kernel for batch sizes 2..16 is not built")
+# (name, dtype, ndim) of the 22 tensors, in the positional order of mk(...).
+_TENSOR_ARGS: tuple[tuple[str, torch.dtype, int], ...] = (
+    ("instructions", torch.int32, 3),
+    ("hidden_states", torch.bfloat16, 2),
+    ("q_post_rope", torch.bfloat16, 2),
+    ("k_cache", torch.bfloat16, 5),
+    ("v_cache", torch.bfloat16, 5),
+    ("attn_out", torch.bfloat16, 2),
+    ("attn_lse_intermediates", torch.float32, 3),
+    ("attn_out_intermediates", torch.float32, 4),
+    ("silu_out", torch.bfloat16, 2),
+    ("logits", torch.bfloat16, 2),
+    ("attn_norm_weights", torch.bfloat16, 2),
+    ("qkv_weights", torch.bfloat16, 3),
+    ("rope_cos", torch.float32, 2),
+    ("rope_sin", torch.float32, 2),
+    ("o_proj_weights", torch.bfloat16, 3),
+    ("mlp_norm_weights", torch.bfloat16, 2),
+    ("up_proj_weights", torch.bfloat16, 3),
+    ("gate_proj_weights", torch.bfloat16, 3),
+    ("down_proj_weights", torch.bfloat16, 3),
+    ("lm_head_norm_weights", torch.bfloat16, 1),
+    ("lm_head_weights", torch.bfloat16, 2),
+    ("barriers", torch.int32, 3),
+)
+
+
+def _check(name: str, t: Any, device: torch.device, dtypes: tuple[torch.dtype, ...], shape: tuple[int, ...] | None, ndim: int) -> None:
+    if not isinstance(t, torch.Tensor):
+        raise TypeError(f"{name} must be a torch.Tensor, got {type(t).__name__}")
+    if t.device.type != "cuda" or t.device != device:
+        raise ValueError(f"{name} must live on {device}, got {t.device}")
+    if t.dtype not in dtypes:
+        raise TypeError(f"{name} must be {' or '.join(map(str, dtypes))}, got {t.dtype}")
+    if t.dim() != ndim:
+        raise ValueError(f"{name} must have {ndim} dims, got shape {tuple(t.shape)}")
+    if not t.is_contiguous():
+        raise ValueError(f"{name} must be contiguous")
+    if shape is not None and tuple(t.shape) != shape:
+        raise ValueError(f"{name} has shape {tuple(t.shape)}, the kernel needs {shape}")
+
+
+class BatchMegaKernel:
+    """The ``mk`` callable of the batch route.
+
+    ``reset_barriers``: the kernel clears the counters when it retires (default) or leaves their
+    final values in place like the reference kernel, whose host loop zeroes them before every step.
+    """
+
+    def __init__(self, lib: ctypes.CDLL, *, reset_barriers: bool = True, spin_limit: int = 0):
+        self._lib = lib
+        self.reset_barriers = reset_barriers
+        self.spin_limit = int(spin_limit)
+        self.timeline: torch.Tensor | None = None
+        self._args = QmkBatchArgs()
+        self._args.struct_size = ctypes.sizeof(QmkBatchArgs)
+        self._bound_key: tuple | None = None
+
+    def error_string(self, code: int) -> str:
+        return self._lib.qmk_error_string(int(code)).decode()
+
+    def check(self, stream: torch.cuda.Stream | None = None) -> None:
+        """Synchronise and raise if a kernel reported a device-side error."""
+        detail = (_I * 4)()
+        handle = (stream or torch.cuda.current_stream()).cuda_stream
+        code = int(self._lib.qmk_status_fetch(_P(handle), ctypes.byref(detail)))
+        if code != 0:
+            raise RuntimeError(
+                f"megakernel device error {code} ({self.error_string(code)}): workgroup={detail[0]} "
+                f"instruction={detail[1]} opcode={detail[2]} operand={detail[3]}; "
+                "the counters are undefined now — zero `barriers` before the next step"
+            )
+
+    def with_options(self, **kw: Any) -> "BatchMegaKernel":
+        other = BatchMegaKernel(self._lib, reset_barriers=kw.pop("reset_barriers", self.reset_barriers),
+                                spin_limit=kw.pop("spin_limit", self.spin_limit))
+        if kw:
+            raise TypeError(f"unknown options {sorted(kw)}")
+        return other
+
+    def _bind(self, tensors: Sequence[torch.Tensor], B: int, position_ids: Any, active_mask: Any, partial_valid: Any,
+              rms: Sequence[Any]) -> None:
+        a = self._args
+        shape = LlamaConfig.shape()
+        a.model = _single._model_id(shape)
+        if a.model != _single.QMK_MODEL_LLAMA_3_2_1B:
+            raise ValueError("the batch route is compiled for the Llama-3.2-1B layer geometry only")
+        if not 1 <= B <= MAX_BATCH:
+            raise ValueError(f"batch_size must be in [1, {MAX_BATCH}], got {B}")
+        device = tensors[1].device if isinstance(tensors[1], torch.Tensor) else None
+        for (name, dtype, ndim), t in zip(_TENSOR_ARGS, tensors):
+            _check(name, t, device, (dtype,), None, ndim)
+            setattr(a, name, t.data_ptr())
+        (instructions, hidden, q, k_cache, v_cache, ao, lse, part, silu, logits, attn_norm, qkv, cos, sin, o_w,
+         mlp_norm, up, gate, down, lm_norm, lm_w, barriers) = tensors
+        L = int(barriers.shape[0])
+        H, F = shape.hidden_size, shape.intermediate_size
+        nq, nkv, d = shape.num_attention_heads, shape.num_key_value_heads, shape.head_dim
+
+        def expect(name: str, t: torch.Tensor, want: tuple[int, ...]) -> None:
+            if tuple(t.shape) != want:
+                raise ValueError(f"{name} has shape {tuple(t.shape)}, the kernel needs {want}")
+
+        if instructions.shape[2] != 32:
+            raise ValueError("instructions must be [queues, length, 32]")
+        expect("hidden_states", hidden, (B, H))
+        expect("q_post_rope", q, (B, nq * d))
+        expect("attn_out", ao, (B, nq * d))
+        expect("silu_out", silu, (B, F))
+        S = int(k_cache.shape[2])
+        expect("k_cache", k_cache, (L, B, S, nkv, d))
+        expect("v_cache", v_cache, (L, B, S, nkv, d))
+        P = int(lse.shape[2])
+        expect("attn_lse_intermediates", lse, (B, nq, P))
+        expect("attn_out_intermediates", part, (B, nq, P, d))
+        V = int(logits.shape[1])
+        expect("logits", logits, (B, V))
+        expect("lm_head_weights", lm_w, (V, H))
+        expect("lm_head_norm_weights", lm_norm, (H,))
+        expect("attn_norm_weights", attn_norm, (L, H))
+        expect("mlp_norm_weights", mlp_norm, (L, H))
+        expect("qkv_weights", qkv, (L, shape.qkv_out_dim, H))
+        expect("o_proj_weights", o_w, (L, H, H))
+        expect("up_proj_weights", up, (L, F, H))
+        expect("gate_proj_weights", gate, (L, F, H))
+        expect("down_proj_weights", down, (L, H, F))
+        if cos.shape != sin.shape or cos.shape[1] != d:
+            raise ValueError("rope_cos/rope_sin must both be [positions, head_dim]")
+        if barriers.shape[1] < 10 or barriers.shape[2] < B * (nq + 2 * nkv):
+            raise ValueError(f"barriers must be [layers, >= 10, >= {B * (nq + 2 * nkv)}], got {tuple(barriers.shape)}")
+        # The control tensors (`…/multi_batch/decode_kernel/mk.cu:112-151`) and the RMSNorm scratch (`:199-216`).
+        if position_ids is not None:
+            _check("position_ids", position_ids, device, (torch.int32,), (B,), 1)
+        if active_mask is not None:
+            _check("active_mask", active_mask, device, (torch.uint8, torch.bool), (B,), 1)
+        if partial_valid is not None:
+            _check("attn_partial_valid", partial_valid, device, (torch.uint8, torch.bool), (B, nq, P), 3)
+        for name, t in zip(("attn_rms_out", "mlp_rms_out", "lm_head_rms_out"), rms):
+            if t is None:
+                raise ValueError(f"{name} must be provided")
+            _check(name, t, device, (torch.bfloat16,), (B, H), 2)
+            setattr(a, name, t.data_ptr())
+        a.position_ids = position_ids.data_ptr() if position_ids is not None else None
+        a.active_mask = active_mask.data_ptr() if active_mask is not None else None
+        a.attn_partial_valid = partial_valid.data_ptr() if partial_valid is not None else None
+        a.num_queues, a.num_insts = int(instructions.shape[0]), int(instructions.shape[1])
+        a.num_layers, a.num_layer_barriers, a.barrier_slots = L, int(barriers.shape[1]), int(barriers.shape[2])
+        a.max_seq_len, a.max_splits, a.vocab_size, a.rope_rows = S, P, V, int(cos.shape[0])
+        a.batch_size = B
+        a.kv_block_size = int(shape.attn_kv_block_size)
+
+    def __call__(self, *args: Any) -> None:
+        if len(args) != 32:
+            raise TypeError(f"mk of the batch route takes 22 tensors, 4 scalars and 6 tensors, got {len(args)} positional arguments")
+        tensors = args[:22]
+        pos_id, B, attn_scale, rms_norm_eps = args[22:26]
+        position_ids, active_mask, partial_valid = args[26:29]
+        rms = args[29:32]
+        if isinstance(tensors[0], torch.Tensor) and tensors[0].numel() == 0:
+            return
+        key = tuple((t.data_ptr(), tuple(t.shape)) if isinstance(t, torch.Tensor) else None for t in (*tensors, *args[26:32])) + (
+            int(B), LlamaConfig.shape())
+        if key != self._bound_key:
+            self._bind(tensors, int(B), position_ids, active_mask, partial_valid, rms)
+            self._bound_key = key
+        a = self._args
+        a.pos_id = int(pos_id)
+        a.attn_scale = float(attn_scale)
+        a.rms_norm_eps = float(rms_norm_eps)
+        a.flags = 0 if self.reset_barriers else _single.QMK_FLAG_KEEP_BARRIERS
+        a.spin_limit = self.spin_limit
+        a.timeline = self.timeline.data_ptr() if self.timeline is not None else None
+        a.stream = torch.cuda.current_stream(tensors[1].device).cuda_stream
+        rc = int(self._lib.qmk_decode_step_batch(ctypes.byref(a)))
+        if rc != 0:
+            raise RuntimeError(f"qmk_decode_step_batch failed with {rc}: {self.error_string(rc)}")
+
+
+def get_mk(mk_dir: Path | None = None, *, reset_barriers: bool = True, spin_limit: int = 0) -> BatchMegaKernel:
+    """Return the ``mk`` callable of the batch route bound to the prebuilt library in ``mk_dir``."""
+    root = (_single._default_mk_dir() if mk_dir is None else Path(mk_dir)).resolve()
+    lib = _single._LIB_CACHE.get(root)
+    if lib is None:
+        lib = _single.load_library(root)
+        _single._LIB_CACHE[root] = lib
+    if not hasattr(lib, "qmk_decode_step_batch"):
+        raise ImportError(f"{root / 'libqmk_hip.so'} does not export qmk_decode_step_batch")
+    lib.qmk_decode_step_batch.argtypes = [ctypes.POINTER(QmkBatchArgs)]
+    lib.qmk_decode_step_batch.restype = ctypes.c_int
+    return BatchMegaKernel(lib, reset_barriers=reset_barriers, spin_limit=spin_limit)
+
+
+def _mask_for_mk(t: torch.Tensor | None, device: torch.device) -> torch.Tensor | None:
+    """`…/multi_batch/decode_schedule/mk_launch_tensors.py:19-26`: on the device, u8 or bool, contiguous."""
+    if t is None:
+        return None
+    if t.device != device:
+        t = t.to(device)
+    if t.dtype not in (torch.uint8, torch.bool):
+        t = t.to(torch.uint8)
+    return t if t.is_contiguous() else t.contiguous()
+
+
+def call_mk(globs: Globals, mk: Any) -> None:
+    """One decode step with the current ``Globals`` (builds the request's instruction tensor on first use)."""
+    shape = LlamaConfig.shape()
+    B = _batch_size(globs)
+    device = globs.hidden_states.device
+    if globs.instructions is None:
+        build(globs)
+    position_ids = globs.position_ids
+    if position_ids is not None and position_ids.numel() == B:
+        if position_ids.device != device or position_ids.dtype != torch.int32:
+            position_ids = position_ids.to(device=device, dtype=torch.int32)
+        position_ids = position_ids.contiguous()
+    else:
+        position_ids = None
+    active = _mask_for_mk(globs.active_mask, device) if globs.active_mask is not None and globs.active_mask.numel() == B else None
+    mk(
+        globs.instructions,
+        globs.hidden_states,
+        globs.q_post_rope,
+        _single._tensor_for_mk(globs.k_cache),
+        _single._tensor_for_mk(globs.v_cache),
+        globs.attn_out,
+        globs.attn_lse_intermediates,
+        globs.attn_out_intermediates,
+        globs.silu_out,
+        globs.logits,
+        globs.attn_norm_weights,
+        globs.qkv_weights,
+        globs.rope_cos,
+        globs.rope_sin,
+        globs.o_proj_weights,
+        globs.mlp_norm_weights,
+        globs.up_proj_weights,
+        globs.gate_proj_weights,
+        globs.down_proj_weights,
+        globs.lm_head_norm_weights,
+        globs.lm_head_weights,
+        globs.barriers,
+        globs.position_id if globs.position_id is not None else 0,
+        B,
+        1.0 / math.sqrt(shape.head_dim),
+        shape.rms_norm_eps,
+        position_ids,
+        active,
+        _mask_for_mk(globs.attn_partial_valid, device),
+        globs.attn_rms_out,
+        globs.mlp_rms_out,
+        globs.lm_head_rms_out,
+    )
+
+
+def build(globs: Globals, kv_capacity: int | None = None) -> torch.Tensor:
+    """The request's instruction tensor: the run-time template of the MI355X scheduler (256 queues),
+    valid for every step of the request."""
+    sched = _scheduler.mi355x_scheduler(_batch_size(globs))
+    capacity = int(globs.k_cache.shape[2]) if kv_capacity is None else kv_capacity
+    if sched.partials_for_capacity(capacity) > int(globs.attn_lse_intermediates.shape[-1]):
+        raise ValueError("attn_lse_intermediates has fewer partial slots than the schedule's split-KV fan-out")
+    return tensorize_instructions(globs, sched.runtime_queues(capacity))
+
+
+def run_instructions(globs: Globals, instructions: list[Instruction], *, mk: Any = None, workers: int | None = None) -> None:
+    """Deal ``instructions`` round-robin onto the queues and execute them once.  The counters keep
+    their final values, so a caller can compare them with a sequential VM run."""
+    mk_call = get_mk() if mk is None else mk
+    if isinstance(mk_call, BatchMegaKernel) and mk_call.reset_barriers:
+        mk_call = mk_call.with_options(reset_barriers=False)
+    queues = _scheduler.deal(instructions, workers or _scheduler.MI355X_WORKERS)
+    tensorize_instructions(globs, queues)
+    call_mk(globs, mk_call)

@@ -13,6 +13,7 @@ import torch
 
 from __graft_entry__ import LIBRARY, ROOT, build_library
 from qimeng_megakernel_amd.decode_schedule import mk_kernel
+from qimeng_megakernel_amd.decode_schedule_mb import mk_kernel as mk_kernel_mb
 
 HEADER = ROOT / "include" / "qmk.h"
 
@@ -27,27 +28,29 @@ def lib():
 def test_every_declared_symbol_is_exported(lib):
     text = HEADER.read_text()
     declared = set(re.findall(r"^(?:int|uint64_t|const char\*)\s+(qmk_\w+)\s*\(", text, flags=re.M))
-    assert declared == {"qmk_decode_step", "qmk_query", "qmk_status_fetch", "qmk_error_string", "qmk_workspace_bytes"}
+    assert declared == {"qmk_decode_step", "qmk_decode_step_batch", "qmk_query", "qmk_status_fetch", "qmk_error_string",
+                        "qmk_workspace_bytes"}
     for name in declared:
         assert hasattr(lib, name), name
 
 
-def test_struct_layout_matches_header(tmp_path):
+@pytest.mark.parametrize("struct,mirror", [("QmkArgs", mk_kernel.QmkArgs), ("QmkBatchArgs", mk_kernel_mb.QmkBatchArgs)])
+def test_struct_layout_matches_header(tmp_path, struct, mirror):
     """Compile the header with gcc and compare sizeof/offsetof with the ctypes mirror."""
-    fields = [name for name, _ in mk_kernel.QmkArgs._fields_]
+    fields = [name for name, _ in mirror._fields_]
     prog = tmp_path / "layout.c"
     lines = ['#include <stdio.h>', '#include <stddef.h>', f'#include "{HEADER}"', "int main(void) {",
-             '  printf("%zu\\n", sizeof(QmkArgs));']
-    lines += [f'  printf("%zu\\n", offsetof(QmkArgs, {f}));' for f in fields]
+             f'  printf("%zu\\n", sizeof({struct}));']
+    lines += [f'  printf("%zu\\n", offsetof({struct}, {f}));' for f in fields]
     lines += ["  return 0;", "}"]
     prog.write_text("\n".join(lines))
     exe = tmp_path / "layout"
     subprocess.run(["gcc", "-std=c99", "-Wall", "-Werror", "-o", str(exe), str(prog)], check=True)
     out = [int(x) for x in subprocess.run([str(exe)], check=True, capture_output=True, text=True).stdout.split()]
-    assert out[0] == ctypes.sizeof(mk_kernel.QmkArgs)
-    assert out[1:] == [getattr(mk_kernel.QmkArgs, f).offset for f in fields]
+    assert out[0] == ctypes.sizeof(mirror)
+    assert out[1:] == [getattr(mirror, f).offset for f in fields]
     # every struct member of the header is mirrored, in order
-    body = HEADER.read_text().split("typedef struct QmkArgs {")[1].split("} QmkArgs;")[0]
+    body = HEADER.read_text().split("typedef struct " + struct + " {")[1].split("} " + struct + ";")[0]
     body = re.sub(r"/\*.*?\*/", "", body, flags=re.S)
     members = re.findall(r"(\w+)\s*;", body)
     assert members == fields
@@ -75,9 +78,19 @@ def test_host_side_argument_errors(lib):
     a.model = 0
     assert lib.qmk_decode_step(ctypes.byref(a)) == 1                       # all tensor pointers are NULL
     assert lib.qmk_workspace_bytes(0) == 8 * (4096 + 512 + 4096 + 1024) and lib.qmk_workspace_bytes(1) == lib.qmk_workspace_bytes(0) and lib.qmk_workspace_bytes(7) == 0
-    assert lib.qmk_query(0) == 4 and lib.qmk_query(2) == 512 and lib.qmk_query(5) == 32 and lib.qmk_query(6) == 25
+    assert lib.qmk_query(0) == 5 and lib.qmk_query(2) == 512 and lib.qmk_query(5) == 32 and lib.qmk_query(6) == 25
     assert 0 < lib.qmk_query(3) <= 160 * 1024
     assert lib.qmk_error_string(34).decode().startswith("device: counter wait")
+    mk_kernel_mb.get_mk()                                                  # declares the entry point's signature
+    assert lib.qmk_decode_step_batch(None) == 1
+    b = mk_kernel_mb.QmkBatchArgs()
+    b.struct_size = 12
+    assert lib.qmk_decode_step_batch(ctypes.byref(b)) == 2
+    b.struct_size = ctypes.sizeof(mk_kernel_mb.QmkBatchArgs)
+    b.model = 1
+    assert lib.qmk_decode_step_batch(ctypes.byref(b)) == 8                 # only the Llama geometry is compiled for this route
+    b.model = 0
+    assert lib.qmk_decode_step_batch(ctypes.byref(b)) == 1
     assert lib.qmk_error_string(12345).decode() == "unknown code"
 
 

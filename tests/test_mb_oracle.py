@@ -1,7 +1,7 @@
 """Batch decode route (2..16 rows): instruction set, scheduler, per-row state and the two CPU oracles.
 
-The gfx950 kernel of this route is not built yet; what is pinned here is everything it will be
-checked against.  Three independent anchors:
+What is pinned here is everything the gfx950 kernel of this route is checked against (its own
+parity tests need a GPU).  Three independent anchors:
 
 * ``tests/golden/mb_reduced_seed0.json`` — written by ``make_fixtures_mb.py`` from the imported
   reference while this repository's scheduler, VM and fused oracle ran in lock-step with the
@@ -256,6 +256,15 @@ def test_decode_state_advances_and_retires_rows():
     assert decode_state.batch_size(g) == 3 and decode_state.decode_pos_id(g, 2) == 11 and decode_state.kv_length(g, 2) == 12
 
 
-def test_batch_kernel_is_absent_and_says_so():
-    with pytest.raises(ImportError, match="not built"):
-        mk_kernel.get_mk()
+def test_mk_of_the_batch_route_checks_its_arguments(weights):
+    """The launcher refuses what the reference's host checks refuse (`…/multi_batch/decode_kernel/mk.cu:52-216`)
+    before anything reaches a device; a missing library is an ImportError."""
+    with pytest.raises(ImportError, match="missing prebuilt kernel"):
+        mk_kernel.get_mk(ROOT / "tests")
+    mk = mk_kernel.get_mk()
+    g = _request(weights)
+    g.instructions = torch.zeros(4, 1, 32, dtype=torch.int32)
+    with pytest.raises(ValueError, match="must live on"):
+        mk_kernel.call_mk(g, mk)
+    with pytest.raises(TypeError, match="positional arguments"):
+        mk(g.instructions, g.hidden_states)
