@@ -116,6 +116,79 @@ def attention_stress(contexts=(4096, 16384, 32768)) -> dict:
     return out
 
 
+def batch_decode(args) -> dict:
+    """B rows decoded together through the batch route's kernel: same request shape as the headline
+    (seeded random-init weights, one random prompt per row, greedy continuation past EOS)."""
+    import dataclasses
+
+    import torch
+
+    from qimeng_megakernel_amd import decode_batch, synthetic
+    from qimeng_megakernel_amd.decode_schedule.model_config import LLAMA_3_2_1B, LlamaConfig
+    from qimeng_megakernel_amd.decode_schedule_mb import mk_kernel
+
+    B = args.batch
+    shape = dataclasses.replace(LLAMA_3_2_1B, attn_kv_block_size=64)   # the batch route's split-KV block
+    LlamaConfig.set_shape(shape)
+    device = torch.device("cuda:0")
+    torch.cuda.set_device(device)
+    new_tokens = args.steps + 1
+    kv_capacity = args.prompt_len + new_tokens
+    weights = synthetic.random_weights(shape, args.seed, max_positions=kv_capacity)
+    prompts = torch.stack([synthetic.random_prompt(shape, args.seed + r, args.prompt_len) for r in range(B)])
+    globs = synthetic.build_batch_globals(weights, shape, kv_capacity, B, device)
+    mk = mk_kernel.get_mk()
+    if args.warmup > 0:
+        decode_batch.decode(globs, prompts, min(args.warmup + 1, new_tokens), mk=mk, decode_time=False)
+    globs.k_cache.zero_(); globs.v_cache.zero_()
+    out = decode_batch.decode(globs, prompts, new_tokens, mk=mk)
+    t = out["timing"]
+    line = {
+        "metric": "kernel_tok_s", "value": t["kernel_tok_s"], "unit": "tok/s", "n_gpus": 1, "steps": args.steps,
+        "warmup": args.warmup, "ms_per_step": t["kernel_ms_per_step"], "higher_is_better": True, "scaling": "weak",
+        "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
+        "config": {
+            "workload": f"Llama-3.2-1B-shaped batch-{B} greedy decode, {args.prompt_len}-token prompt per row, {new_tokens} new "
+                        f"tokens per row (context {args.prompt_len + 1}..{args.prompt_len + args.steps}), seeded random-init bf16 weights",
+            "batch": B, "seed": args.seed, "queues": int(globs.instructions.shape[0]),
+            "instructions_per_queue": int(globs.instructions.shape[1]),
+        },
+        "tok_s": t["effective_tok_s_wall"], "tok_s_gpu": t["effective_tok_s_gpu"], "kernel_tok_s": t["kernel_tok_s"],
+        "first_tokens": out["new_tokens"][:, :4].tolist(),
+        "roofline": {
+            "bound": "hbm", "achieved": t["achieved_GBps"], "peak": HBM_PEAK_GBPS, "unit": "GB/s",
+            "frac": t["achieved_GBps"] / HBM_PEAK_GBPS, "traffic": None,
+            "bytes_per_launch_avg": t["algorithmic_bytes"] / max(args.steps, 1), "kernel": "decode_megakernel_batch<Llama1B>",
+        },
+    }
+    if not args.no_cpu_baseline:
+        line["cpu_baseline"] = cpu_baseline_batch(shape, weights, prompts, args.cpu_steps, min(os.cpu_count() or 1, 16))
+    return line
+
+
+def cpu_baseline_batch(shape, weights, prompts, n_steps: int, cores: int) -> dict:
+    """The fused batch oracle on the host cores: ``n_steps`` steps of the same rows from position 0."""
+    import torch
+
+    sys.path.insert(0, str(ROOT / "oracle"))
+    from fused_mb_oracle import FusedBatchOracle
+    from qimeng_megakernel_amd import synthetic
+
+    torch.set_num_threads(cores)
+    B = int(prompts.shape[0])
+    g = synthetic.build_batch_globals(weights, shape, n_steps + 1, B, "cpu")
+    oracle = FusedBatchOracle(shape)
+    with torch.no_grad():
+        t0 = time.perf_counter()
+        for pos in range(n_steps):
+            g.hidden_states.copy_(g.embed_tokens[prompts[:, min(pos, prompts.shape[1] - 1)]])
+            g.position_ids.fill_(pos)
+            oracle.decode_step(g)
+        dt = time.perf_counter() - t0
+    return {"value": B * n_steps / dt, "unit": "tok/s", "cores": cores, "kind": "port",
+            "sample": f"{n_steps} steps of {B} rows (contexts 1..{n_steps}) of the Llama-3.2-1B-shaped workload through the fused batch oracle"}
+
+
 def main() -> None:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -135,6 +208,8 @@ def main() -> None:
     ap.add_argument("--attention-stress", action="store_true",
                     help="instead of the decode request: the split-KV attention phase at contexts 4096/16384/32768 "
                          "(one JSON line, metric attention_phase_GBps)")
+    ap.add_argument("--batch", type=int, default=1,
+                    help="rows decoded together (2..16: the batch route's kernel, Llama-3.2-1B shape; tokens/s counts all rows)")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also run one 1 GiB device-to-device copy (a kernel of known traffic, for scaling rocprofv3 counters)")
     args = ap.parse_args()
@@ -161,6 +236,11 @@ def main() -> None:
                           "dtype": "bf16", "data": "synthetic",
                           "config": {"workload": "Llama-3.2-1B layer geometry, batch 1, one decode step, KV cache ~N(0,1)"},
                           "value": res[max(res, key=int)]["GBps"], "contexts": res}))
+        return
+    if args.batch != 1:
+        if args.model != "llama-3.2-1b" or not 2 <= args.batch <= 16:
+            raise SystemExit("bench.py: --batch takes 2..16 and runs on the Llama-3.2-1B shape (the route the reference has)")
+        print(json.dumps(batch_decode(args)))
         return
     shape = LLAMA_3_2_1B if args.model == "llama-3.2-1b" else QWEN3_1_7B
     model_name = "Llama-3.2-1B" if args.model == "llama-3.2-1b" else "Qwen3-1.7B"

@@ -44,6 +44,14 @@ def _gemm(mat: Tensor, rows_bk: Tensor, r0: int, r1: int) -> Tensor:
     return torch.einsum("oi,bi->bo", mat[r0:r1], rows_bk)
 
 
+class _MergeAll:
+    """What a reduction instruction over all partials of a head group would say."""
+
+    def __init__(self, layer: int, b: int, h0: int, num_partials: int):
+        self.layer_idx, self.batch_idx, self.head_start_idx, self.num_partials = layer, b, h0, num_partials
+        self.reduction_list, self.is_terminal, self.output_partial_idx, self.is_active = list(range(num_partials)), True, 0, -1
+
+
 class BatchInstructionVM:
     def __init__(self, shape: Any):
         self.shape = shape
@@ -143,12 +151,18 @@ class BatchInstructionVM:
         mine = g.barriers[layer, 2, b * self.stride : (b + 1) * self.stride]
         seq_len = ins.seq_len if ins.seq_len >= 0 else self._pos(g, b) + 1
 
+        def arrive() -> None:
+            mine[h0:h1] += 1
+            # extension of this build: the arrival that completes the group merges it
+            if getattr(ins, "merge_in_last", 0) and int(mine[h0]) == ins.num_partials:
+                self.decode_attention_reduction(g, _MergeAll(layer, b, h0, ins.num_partials))   # the row's flag decides, not this slice's
+
         def leave_empty() -> None:
             g.attn_lse_intermediates[b, h0:h1, part] = INACTIVE_LSE
             g.attn_out_intermediates[b, h0:h1, part] = 0.0
             if g.attn_partial_valid is not None:
                 g.attn_partial_valid[b, h0:h1, part] = False
-            mine[h0:h1] += 1
+            arrive()
 
         if not self._instruction_active(ins.is_active, g, b):
             return leave_empty()
@@ -167,7 +181,7 @@ class BatchInstructionVM:
         g.attn_out_intermediates[b, h0:h1, part] = torch.einsum("hk,ko->ho", torch.softmax(scores, dim=-1), v)
         if g.attn_partial_valid is not None:
             g.attn_partial_valid[b, h0:h1, part] = True
-        mine[h0:h1] += 1
+        arrive()
 
     # ---- 4 -------------------------------------------------------------------------
     def decode_attention_reduction(self, g: Any, ins: Any) -> None:

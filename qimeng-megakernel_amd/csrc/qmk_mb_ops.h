@@ -277,13 +277,83 @@ __device__ bool op_qkv(const Params& p, Smem<M>& s, const Ctx& c) {
   return true;
 }
 
+// Log-sum-exp merge (log2 domain) of partials list[0..n) (null: 0..n-1) of the GQA query heads from
+// head0 of batch row b, over the valid ones only (python_vm.py:442-551).  Thread t < GQA*D/2
+// produces two neighbouring dims.  All reads are issued before the first use.
+template <class M>
+__device__ __forceinline__ void merge_heads(const Params& p, const Ctx& c, int b, int head0, int n, const int32_t* list, bool terminal,
+                                            int out_slot) {
+  constexpr int D = M::D;
+  if (c.tid >= M::GQA * D / 2) return;
+  const int h = head0 + c.tid / (D / 2), d = 2 * (c.tid % (D / 2));
+  const size_t row = (static_cast<size_t>(b) * M::NQ + h) * p.max_splits;
+  const float* lse = p.attn_lse + row;
+  const float* part = p.attn_partial + row * D + d;
+  const uint8_t* valid = p.partial_valid ? p.partial_valid + row : nullptr;
+  // Eight partials at a time (all eight reads in flight together; slots beyond n re-read the last
+  // listed partial and get weight 0), folded into a running (max, numerators, denominator).
+  constexpr int kGroup = 8;
+  float mx = -INFINITY, num0 = 0.f, num1 = 0.f, den = 0.f;
+  for (int base = 0; base < n; base += kGroup) {
+    float e[kGroup];
+    uint64_t two[kGroup];
+    bool ok[kGroup];
+#pragma unroll
+    for (int i = 0; i < kGroup; ++i) {
+      const int ii = min(base + i, n - 1);
+      const int j = list ? list[ii] : ii;
+      e[i] = ld_shared_f32(lse + j);
+      two[i] = ld_shared64(part + static_cast<size_t>(j) * D);
+      ok[i] = valid ? ld_shared8(valid + j) != 0 : true;
+    }
+    float gmx = mx;
+#pragma unroll
+    for (int i = 0; i < kGroup; ++i) {
+      ok[i] = base + i < n && (valid ? ok[i] : (e[i] > kNoContribution && e[i] < INFINITY));
+      if (ok[i]) gmx = fmaxf(gmx, e[i]);
+    }
+    const float keep = mx == -INFINITY ? 0.f : exp2_fast(mx - gmx);
+    num0 *= keep, num1 *= keep, den *= keep;
+    mx = gmx;
+#pragma unroll
+    for (int i = 0; i < kGroup; ++i) {
+      const float f = ok[i] ? exp2_fast(e[i] - mx) : 0.f;
+      num0 = __builtin_fmaf(__uint_as_float(static_cast<uint32_t>(two[i])), f, num0);
+      num1 = __builtin_fmaf(__uint_as_float(static_cast<uint32_t>(two[i] >> 32)), f, num1);
+      den += f;
+    }
+  }
+  const bool any = den > 0.f;
+  const float o0 = any ? num0 / den : 0.f, o1 = any ? num1 / den : 0.f;
+  if (terminal) {
+    st_shared32(p.attn_out + static_cast<size_t>(b) * M::NQ * D + static_cast<size_t>(h) * D + d,
+                static_cast<uint32_t>(f2bf(o0)) | (static_cast<uint32_t>(f2bf(o1)) << 16));
+  } else {
+    float* dst = p.attn_partial + (row + out_slot) * D + d;
+    st_shared_f32(dst, o0);
+    st_shared_f32(dst + 1, o1);
+    if (d == 0) {
+      st_shared_f32(p.attn_lse + row + out_slot, any ? mx + log2f(den) : (valid ? 0.f : kNoContribution - 1.0f));
+      if (p.partial_valid) st_shared8(p.partial_valid + row + out_slot, any ? 1 : 0);
+    }
+  }
+}
+// attn_out of the GQA heads from head0 of an inactive batch row.
+template <class M>
+__device__ __forceinline__ void zero_heads(const Params& p, const Ctx& c, int b, int head0) {
+  if (c.tid < M::GQA * M::D / 2) st_shared32(p.attn_out + static_cast<size_t>(b) * M::NQ * M::D + head0 * M::D + 2 * c.tid, 0u);
+}
+
 // ===================================================================== 3 ==
-// [3, layer, batch_row, kv_head, num_partials, partial_idx, seq_len, is_active]
+// [3, layer, batch_row, kv_head, num_partials, partial_idx, seq_len, is_active, merge_in_last]
 // Flash-decoding over one slice of one batch row's context for the GQA group of one KV head
 // (python_vm.py:269-359).  seq_len < 0: the row's position + 1; is_active < 0: the row's flag.  The
 // slices are whole KV blocks of `kv_block` tokens.  An inactive row or an empty slice leaves
 // (0, -inf, not valid) and still counts.  Scoring as in the batch-1 kernel: a wave takes 16 tokens at
 // a time on the matrix cores and keeps one running (max, sum, acc) per query head.
+// merge_in_last (an extension; 0 in streams built by the reference scheduler): the workgroup whose
+// arrival completes the head group's counters merges all partials itself (or zeroes the heads of an
+// inactive row) and counts on the reduction row, so no reduction instruction and no second wait is needed.
 template <class M>
 __device__ bool op_splitkv(const Params& p, Smem<M>& s, const Ctx& c) {
   constexpr int D = M::D, GQA = M::GQA;
@@ -297,6 +367,8 @@ __device__ bool op_splitkv(const Params& p, Smem<M>& s, const Ctx& c) {
   const int seq_len = s.inst[6] >= 0 ? s.inst[6] : pos + 1;
   if (seq_len > p.max_seq_len) return bad_operand(p, s, c, 6);
   const bool active = s.inst[7] == 0 ? false : (s.inst[7] == 1 ? true : s.active[b] != 0);
+  const bool merge_in_last = s.inst[8] != 0;
+  if (merge_in_last && P > kMaxList) return bad_operand(p, s, c, 8);
   const int lane = c.tid & 63, wave = c.tid >> 6;
   constexpr int kStride = M::NQ + 2 * M::NKV;   // counter slots per batch row
 
@@ -357,7 +429,22 @@ __device__ bool op_splitkv(const Params& p, Smem<M>& s, const Ctx& c) {
   auto arrive = [&] {
     release_stores();
     __syncthreads();
-    if (c.tid < GQA) publish(counter_ptr(p, layer, ROW_SPLITKV, b * kStride + head0 + c.tid), 1);
+    if (!merge_in_last) {
+      if (c.tid < GQA) publish(counter_ptr(p, layer, ROW_SPLITKV, b * kStride + head0 + c.tid), 1);
+      return;
+    }
+    if (c.tid < GQA) {   // whoever sees P-1 earlier arrivals is last: every partial of the group is in memory
+      const int prev = __hip_atomic_fetch_add(counter_ptr(p, layer, ROW_SPLITKV, b * kStride + head0 + c.tid), 1, __ATOMIC_RELAXED,
+                                              __HIP_MEMORY_SCOPE_AGENT);
+      if (c.tid == 0) s.ctl[3] = (prev == P - 1);
+    }
+    __syncthreads();
+    if (s.ctl[3]) {  // uniform
+      // the row's flag, not this slice's: an empty slice of a live row may well arrive last
+      if (s.active[b]) merge_heads<M>(p, c, b, head0, P, nullptr, true, 0);
+      else zero_heads<M>(p, c, b, head0);
+      publish_after_stores(p, c, layer, ROW_REDUCE, b, GQA);
+    }
   };
   if (empty) {  // uniform
     if (c.tid < GQA * D) {
@@ -547,59 +634,14 @@ __device__ bool op_reduce(const Params& p, Smem<M>& s, const Ctx& c) {
   if (!terminal && (out_slot < 0 || out_slot >= p.max_splits)) return bad_operand(p, s, c, 7 + n);
   const int flag = s.inst[9 + n];
   const bool active = flag == 0 ? false : (flag == 1 ? true : s.active[b] != 0);
-  const bool worker = c.tid < R * D / 2;
-  const int h = head0 + c.tid / (D / 2), d = 2 * (c.tid % (D / 2));
-  u16* out = p.attn_out + static_cast<size_t>(b) * M::NQ * D + static_cast<size_t>(h) * D + d;
   if (!active) {
-    if (worker) st_shared32(out, 0u);
+    zero_heads<M>(p, c, b, head0);
     publish_after_stores(p, c, layer, ROW_REDUCE, b, R);
     return true;
   }
   if (!wait_counters(p, s, c, R, [&](int i) { return counter_ptr(p, layer, ROW_SPLITKV, b * kStride + head0 + i); }, [&](int) { return P; }))
     return false;
-  if (worker) {
-    const size_t row = (static_cast<size_t>(b) * M::NQ + h) * p.max_splits;
-    const float* lse = p.attn_lse + row;
-    const float* part = p.attn_partial + row * D + d;
-    const uint8_t* valid = p.partial_valid ? p.partial_valid + row : nullptr;
-    float e[kMaxList];
-    uint64_t two[kMaxList];
-    bool ok[kMaxList];
-#pragma unroll
-    for (int i = 0; i < kMaxList; ++i) {   // slots beyond n re-read the last listed partial and get weight 0
-      const int j = s.inst[6 + min(i, n - 1)];
-      e[i] = ld_shared_f32(lse + j);
-      two[i] = ld_shared64(part + static_cast<size_t>(j) * D);
-      ok[i] = valid ? ld_shared8(valid + j) != 0 : true;
-    }
-    float mx = -INFINITY;
-#pragma unroll
-    for (int i = 0; i < kMaxList; ++i) {
-      ok[i] = i < n && (valid ? ok[i] : (e[i] > kNoContribution && e[i] < INFINITY));
-      if (ok[i]) mx = fmaxf(mx, e[i]);
-    }
-    float num0 = 0.f, num1 = 0.f, den = 0.f;
-#pragma unroll
-    for (int i = 0; i < kMaxList; ++i) {
-      const float f = ok[i] ? exp2_fast(e[i] - mx) : 0.f;
-      num0 = __builtin_fmaf(__uint_as_float(static_cast<uint32_t>(two[i])), f, num0);
-      num1 = __builtin_fmaf(__uint_as_float(static_cast<uint32_t>(two[i] >> 32)), f, num1);
-      den += f;
-    }
-    const bool any = den > 0.f;
-    const float o0 = any ? num0 / den : 0.f, o1 = any ? num1 / den : 0.f;
-    if (terminal) {
-      st_shared32(out, static_cast<uint32_t>(f2bf(o0)) | (static_cast<uint32_t>(f2bf(o1)) << 16));
-    } else {
-      float* dst = p.attn_partial + (row + out_slot) * D + d;
-      st_shared_f32(dst, o0);
-      st_shared_f32(dst + 1, o1);
-      if (d == 0) {
-        st_shared_f32(p.attn_lse + row + out_slot, any ? mx + log2f(den) : (valid ? 0.f : kNoContribution - 1.0f));
-        if (p.partial_valid) st_shared8(p.partial_valid + row + out_slot, any ? 1 : 0);
-      }
-    }
-  }
+  merge_heads<M>(p, c, b, head0, n, &s.inst[6], terminal, out_slot);
   publish_after_stores(p, c, layer, ROW_REDUCE, b, R);
   return true;
 }

@@ -1,0 +1,111 @@
+"""Host step loop of the batch ``mk`` route: B rows decoded together, each at its own position.
+
+Counterpart of the batch branch of the reference's decode loop
+(`qimeng_megakernel/models/LLM/decode.py:536-796`, per-row state `LLM/decode_state.py:46-138`):
+one instruction tensor per request (the scheduler's run-time template), per step the embedding
+rows of the last tokens -> ``hidden_states``, one kernel launch, ``argmax`` per row, then
+``advance_decode_state`` (rows that produced an EOS token retire, the others move one position
+on).  Timing as in the batch-1 loop: one event pair per step around the launch only.
+
+Prefill runs the same kernel once per prompt position with every row at that position.
+"""
+from __future__ import annotations
+
+import time
+from typing import Any, Sequence
+
+import torch
+
+from .decode_schedule_mb import decode_state as _state
+from .decode_schedule_mb import mk_kernel as _mk_kernel
+
+
+def step_bytes(shape: Any, contexts: Sequence[int]) -> int:
+    """Algorithmic HBM bytes of one batch step: the weights once, per active row its context's KV
+    rows read and one KV row written."""
+    kv = shape.kv_bytes_per_context_token()
+    return shape.weight_bytes_per_token() + sum(kv * c + kv for c in contexts)
+
+
+def _embed(globs: Any, tokens: torch.Tensor) -> None:
+    globs.hidden_states.copy_(globs.embed_tokens[tokens].to(globs.hidden_states.dtype))
+
+
+def prefill_by_decode(globs: Any, mk: Any, prompts: torch.Tensor) -> torch.Tensor:
+    """``prompts`` [B, T]: fill the KV cache one position at a time; returns the first new token of every row."""
+    B, T = prompts.shape
+    prompts = prompts.to(globs.hidden_states.device)
+    for pos in range(T):
+        _embed(globs, prompts[:, pos])
+        globs.position_ids.fill_(pos)
+        _mk_kernel.call_mk(globs, mk)
+    return globs.logits.float().argmax(dim=-1)
+
+
+def decode(globs: Any, prompts: torch.Tensor, max_new_tokens: int, *, mk: Any = None, eos_token_ids: Sequence[int] = (),
+           decode_time: bool = True) -> dict[str, Any]:
+    """Prefill + greedy decode of B rows to ``max_new_tokens`` tokens each (rows that hit an EOS token
+    of ``eos_token_ids`` retire; with none given every row runs to the end)."""
+    from .decode import globs_shape
+
+    device = globs.hidden_states.device
+    B, T = int(prompts.shape[0]), int(prompts.shape[1])
+    if B != _state.batch_size(globs):
+        raise ValueError(f"{B} prompts for buffers of {_state.batch_size(globs)} rows")
+    if T + max_new_tokens > globs.k_cache.shape[2]:
+        raise ValueError("prompt_len + max_new_tokens exceeds the KV cache capacity")
+    mk = mk or _mk_kernel.get_mk()
+    globs.active_mask.fill_(True)
+    _state.ensure_decode_state(globs, B, device)
+    if getattr(globs, "eos_reached", None) is not None:
+        globs.eos_reached.zero_()
+    globs.instructions = None
+    _mk_kernel.build(globs)
+    out = torch.zeros(B, T + max(max_new_tokens, 1), dtype=torch.long, device=device)
+    out[:, :T] = prompts.to(device)
+    out[:, T] = prefill_by_decode(globs, mk, prompts)
+    globs.position_ids.fill_(T)
+    _state.sync_kv_lengths(globs)
+    ntok = max(max_new_tokens - 1, 0)
+    events = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(ntok if decode_time else 0)]
+    loop_start, loop_end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    active_log = []
+    torch.cuda.synchronize(device)
+    wall0 = time.perf_counter()
+    loop_start.record()
+    for i in range(ntok):
+        _embed(globs, out[:, T + i])
+        if events:
+            events[i][0].record()
+        _mk_kernel.call_mk(globs, mk)
+        if events:
+            events[i][1].record()
+        nxt = globs.logits.float().argmax(dim=-1)
+        out[:, T + i + 1] = nxt
+        if eos_token_ids:
+            active_log.append(globs.active_mask.clone())
+        _state.advance_decode_state(globs, nxt, eos_token_ids)
+    loop_end.record()
+    torch.cuda.synchronize(device)
+    result: dict[str, Any] = {"generated_ids": out, "new_tokens": out[:, T:]}
+    if decode_time and ntok:
+        wall = time.perf_counter() - wall0
+        gpu_s = loop_start.elapsed_time(loop_end) / 1e3
+        per_step_ms = [a.elapsed_time(b) for a, b in events]
+        kernel_s = sum(per_step_ms) / 1e3
+        shape = globs_shape(globs)
+        if eos_token_ids:
+            rows = [int(m.sum()) for m in active_log]
+        else:
+            rows = [B] * ntok
+        produced = sum(rows)
+        nbytes = sum(step_bytes(shape, [T + i + 1] * rows[i]) for i in range(ntok))
+        result["timing"] = {
+            "decode_wall_s": wall, "decode_gpu_s": gpu_s, "mk_kernel_gpu_s": kernel_s,
+            "decode_window_new_tokens": produced,
+            "effective_tok_s_wall": produced / wall, "effective_tok_s_gpu": produced / gpu_s,
+            "kernel_tok_s": produced / kernel_s, "kernel_steps": ntok, "kernel_ms_per_step": kernel_s * 1e3 / ntok,
+            "algorithmic_bytes": nbytes, "achieved_GBps": nbytes / kernel_s / 1e9, "per_step_ms": per_step_ms,
+        }
+    mk.check()
+    return result

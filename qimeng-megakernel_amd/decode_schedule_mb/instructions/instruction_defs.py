@@ -87,6 +87,15 @@ class DecodeAttentionSplitKV(Instruction):
 
 
 @dataclass
+class DecodeAttentionSplitKVMerge(DecodeAttentionSplitKV):
+    """Extension of this build (same opcode, one more word): with ``merge_in_last`` set, the instruction
+    whose arrival completes the head group's counters also merges the group's partials into ``attn_out``
+    and counts on the reduction row; such a stream carries no reduction instructions."""
+
+    merge_in_last: int = 1
+
+
+@dataclass
 class DecodeAttentionReduction(Instruction):
     """Log-sum-exp merge of the listed partials for four query heads of one batch row."""
 

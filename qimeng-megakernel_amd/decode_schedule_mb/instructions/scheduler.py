@@ -28,6 +28,7 @@ from .instruction_defs import (
     AttnRMS,
     DecodeAttentionReduction,
     DecodeAttentionSplitKV,
+    DecodeAttentionSplitKVMerge,
     DownProj_GEMM_Residual,
     LMHeadProj_GEMM,
     LMHeadRMS,
@@ -79,6 +80,7 @@ class BatchScheduler:
     shape: DecodeShape
     workers: int
     batch_size: int
+    merge_in_last: bool = False   # the last split-KV arrival of a head group merges: no reduction instructions
 
     def __post_init__(self) -> None:
         if not 1 <= self.batch_size <= MAX_BATCH:
@@ -125,6 +127,7 @@ class BatchScheduler:
         """With ``globs``: length and activity fixed from the request's present state; without: left
         to the launch (seq_len = is_active = -1)."""
         kvb = self.shape.attn_kv_block_size
+        make = DecodeAttentionSplitKVMerge if self.merge_in_last else DecodeAttentionSplitKV
         out: list[Instruction] = []
         for b in range(self.batch_size):
             if globs is not None:
@@ -136,16 +139,18 @@ class BatchScheduler:
             for kvh in range(self.shape.num_key_value_heads):
                 for part in range(num_partials):
                     if globs is None:
-                        out.append(DecodeAttentionSplitKV(layer, b, kvh, num_partials, part))
+                        out.append(make(layer, b, kvh, num_partials, part))
                         continue
                     t0 = part * per * kvb
                     t1 = min(min(part * per + per, total) * kvb, seq_len)
                     work = on and t0 < t1 and t1 > 0
-                    out.append(DecodeAttentionSplitKV(layer, b, kvh, num_partials, part, seq_len, 1 if work else 0))
+                    out.append(make(layer, b, kvh, num_partials, part, seq_len, 1 if work else 0))
         return out
 
     def attention_reduction(self, layer: int, num_partials: int, globs: Any = None) -> list[Instruction]:
         out: list[Instruction] = []
+        if self.merge_in_last:
+            return out
         for b in range(self.batch_size):
             for head0 in range(0, self.shape.num_attention_heads, ATTN_REDUCTION_SIZE):
                 if globs is None:
@@ -227,5 +232,6 @@ def reference_scheduler(batch_size: int, shape: DecodeShape | None = None) -> Ba
     return BatchScheduler(shape or LlamaConfig.shape(), A100_WORKERS, batch_size)
 
 
-def mi355x_scheduler(batch_size: int, shape: DecodeShape | None = None) -> BatchScheduler:
-    return BatchScheduler(shape or LlamaConfig.shape(), MI355X_WORKERS, batch_size)
+def mi355x_scheduler(batch_size: int, shape: DecodeShape | None = None, *, merge_in_last: bool = True) -> BatchScheduler:
+    """One queue per CU; the split-KV partials are merged by the last arrival of each head group."""
+    return BatchScheduler(shape or LlamaConfig.shape(), MI355X_WORKERS, batch_size, merge_in_last=merge_in_last)

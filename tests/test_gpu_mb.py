@@ -104,6 +104,9 @@ STAGES = [
 ]
 
 
+CASES = {"ragged3": (3, (70, 3, 130), ()), "inactive_row": (4, (9, 64, 0, 127), (2,)), "batch16": (16, tuple(range(5, 150, 9))[:16], (7,))}
+
+
 def stage_instructions(sched, globs, name, layer=0):
     p = sched.partials_for_request(globs)
     if name == "attention_split_kv":
@@ -117,10 +120,9 @@ def stage_instructions(sched, globs, name, layer=0):
 @pytest.mark.parametrize("case", ["ragged3", "inactive_row", "batch16"])
 def test_one_op_against_the_vm(weights, stage, case):
     """Everything before the op runs on the VM; the op itself on both, from identical state."""
-    rows, positions, inactive = {"ragged3": (3, (70, 3, 130), ()), "inactive_row": (4, (9, 64, 0, 127), (2,)),
-                                 "batch16": (16, tuple(range(5, 150, 9))[:16], (7,))}[case]
+    rows, positions, inactive = CASES[case]
     cpu, gpu = make_pair(weights, rows, positions, inactive=inactive)
-    sched = S.mi355x_scheduler(rows, MB_SMALL)
+    sched = S.mi355x_scheduler(rows, MB_SMALL, merge_in_last=False)
     vm = BatchInstructionVM(MB_SMALL)
     for name, _ in STAGES[:stage]:
         vm.run(cpu, stage_instructions(sched, cpu, name))
@@ -140,6 +142,26 @@ def test_one_op_against_the_vm(weights, stage, case):
     for name in MUTABLE:
         if name not in STAGES[stage][1] and getattr(cpu, name).dtype == torch.bfloat16:
             assert torch.equal(getattr(gpu, name).cpu(), getattr(cpu, name)), name
+
+
+@pytest.mark.parametrize("case", list(CASES))
+@pytest.mark.parametrize("template", [False, True], ids=["static", "runtime"])
+def test_split_kv_whose_last_arrival_merges(weights, case, template):
+    """The MI355X stream: no reduction instructions; lengths and activity in the words or left to the launch."""
+    rows, positions, inactive = CASES[case]
+    cpu, gpu = make_pair(weights, rows, positions, inactive=inactive)
+    sched = S.mi355x_scheduler(rows, MB_SMALL)
+    vm = BatchInstructionVM(MB_SMALL)
+    vm.run(cpu, sched.attn_rms(0) + sched.qkvproj(0))
+    sync_state(cpu, gpu)
+    p = sched.partials_for_capacity(FIX["kv_capacity"]) if template else sched.partials_for_request(cpu)
+    mine = sched.attention_split_kv(0, p, None if template else cpu)
+    assert not sched.attention_reduction(0, p) and all(i.padded()[8] == 1 for i in mine)
+    vm.run(cpu, copy.deepcopy(mine))
+    run_kernel(gpu, mine)
+    bf16_close(gpu.attn_out, cpu.attn_out, name="attn_out")
+    compare(cpu, gpu, ("attn_out_intermediates", "attn_lse_intermediates", "attn_partial_valid"))
+    assert int(cpu.barriers[0, 3, 0]) == MB_SMALL.num_attention_heads
 
 
 def test_lm_head_ops_against_the_vm(weights):
