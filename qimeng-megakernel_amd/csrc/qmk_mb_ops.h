@@ -53,6 +53,19 @@ constexpr int ROW_ATTN_RMS = 0, ROW_QKV = 1, ROW_SPLITKV = 2, ROW_REDUCE = 3, RO
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef float f4 __attribute__((ext_vector_type(4)));
 
+// Two floats to a bf16 pair, round-to-nearest-even (v_cvt_pk_bf16_f32: the rounding torch applies on
+// .to(bfloat16)), low half first.
+typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+typedef float f32x2 __attribute__((ext_vector_type(2)));
+__device__ __forceinline__ uint32_t pack_bf16(float lo, float hi) {
+  return __builtin_bit_cast(uint32_t, __builtin_convertvector(f32x2{lo, hi}, bf16x2));
+}
+// old + bf16(delta) on a bf16 pair: the residual add of two neighbouring elements.
+__device__ __forceinline__ uint32_t residual_add(uint32_t old, float d0, float d1) {
+  const uint32_t d = pack_bf16(d0, d1);
+  return pack_bf16(bf_lo(old) + bf_lo(d), bf_hi(old) + bf_hi(d));
+}
+
 // Validity flags are bytes that one workgroup writes and another reads within the launch.
 __device__ __forceinline__ void st_shared8(uint8_t* p, uint8_t v) { __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); }
 __device__ __forceinline__ uint8_t ld_shared8(const uint8_t* p) { return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); }
@@ -154,12 +167,14 @@ __device__ bool op_rms_row(const Params& p, Smem<M>& s, const Ctx& c) {
 
 // ------------------------------------------------------------ GEMM core ----
 // One lane's share of a 16-row x 256-column weight segment: row l%16, 16 bytes of each 64-byte chunk.
+// Ordinary loads: an instruction takes 64 bytes of each of 16 rows, the next one the other half of the
+// same 128-byte lines; with the streaming hint the second half misses again (measured: LM head 101 -> 90 us).
 struct Seg {
   v4u a[kSegChunks];
 };
 __device__ __forceinline__ void load_seg(Seg& sg, const u16* lane_ptr) {
 #pragma unroll
-  for (int j = 0; j < kSegChunks; ++j) sg.a[j] = __builtin_nontemporal_load(reinterpret_cast<const v4u*>(lane_ptr + j * kChunk));
+  for (int j = 0; j < kSegChunks; ++j) sg.a[j] = *reinterpret_cast<const v4u*>(lane_ptr + j * kChunk);
 }
 __device__ __forceinline__ f4 mma_seg(const Seg& sg, const v4u (&x)[kSegChunks], f4 acc) {
 #pragma unroll
@@ -168,13 +183,22 @@ __device__ __forceinline__ f4 mma_seg(const Seg& sg, const v4u (&x)[kSegChunks],
   return acc;
 }
 // This lane's share of the activations [B, ld] for one segment: batch row l%16 (zeros beyond the
-// batch), the same 16 bytes of every chunk as the weights.  The buffers are written during the launch.
+// batch), the same 16 bytes of every chunk as the weights.  The buffers are written during the launch
+// by other workgroups, so the loads are device-coherent (sc1) like ld_shared128 — but as one 16-byte
+// buffer load per chunk instead of two 8-byte ones: half the requests for the same bytes.
 __device__ __forceinline__ void load_x(v4u (&x)[kSegChunks], const u16* act, int ld, int B, int k0, int lane) {
   const int n = lane & 15, g = lane >> 4;
+  constexpr int kDeviceCoherent = 16;   // the sc1 bit of the cache policy operand
+  // The descriptor is built where it is used: through an opaque copy of the pointer, so that the
+  // descriptors of all five activation tensors are not computed once for all ops and kept in registers.
+  u16* base = const_cast<u16*>(act);
+  asm volatile("" : "+s"(base));
+  const __amdgpu_buffer_rsrc_t rsrc = __builtin_amdgcn_make_buffer_rsrc(base, 0, 0x7fffffff, 0x00020000);
+  const uint32_t at = (static_cast<uint32_t>(n) * ld + k0 + g * 8) * 2;
 #pragma unroll
   for (int j = 0; j < kSegChunks; ++j) {
     x[j] = v4u{0, 0, 0, 0};
-    if (n < B) x[j] = ld_shared128(act + static_cast<size_t>(n) * ld + k0 + j * kChunk + g * 8);
+    if (n < B) x[j] = __builtin_bit_cast(v4u, __builtin_amdgcn_raw_buffer_load_b128(rsrc, at + j * kChunk * 2, 0, kDeviceCoherent));
   }
 }
 // The wave's partial tile (C layout: rows 4*(l/16)..+3, column l%16) into its LDS slot.
@@ -257,7 +281,8 @@ __device__ bool op_qkv(const Params& p, Smem<M>& s, const Ctx& c) {
       [&](int j, int parity, int b, int rp) {
         if (b >= B || !s.active[b]) return;
         const float2 v = gather(s, parity, 0, b, rp);
-        const float v0 = round_bf16(v.x), v1 = round_bf16(v.y);
+        const uint32_t vb = pack_bf16(v.x, v.y);
+        const float v0 = bf_lo(vb), v1 = bf_hi(vb);
         const int o = (n0 + j) * kTile + 2 * rp, d = o % M::D, pos = s.pos[b];
         const size_t cache_row = ((static_cast<size_t>(layer) * B + b) * p.max_seq_len + pos) * tok_stride;
         if (o < M::NQ * M::D) {
@@ -267,7 +292,7 @@ __device__ bool op_qkv(const Params& p, Smem<M>& s, const Ctx& c) {
           st_shared32(p.k_cache + cache_row + (o - M::NQ * M::D),
                       rope_pair(v0, v1, p.rope_cos + static_cast<size_t>(pos) * M::D, p.rope_sin + static_cast<size_t>(pos) * M::D, d));
         } else {
-          st_shared32(p.v_cache + cache_row + (o - (M::NQ + M::NKV) * M::D), static_cast<uint32_t>(f2bf(v0)) | (static_cast<uint32_t>(f2bf(v1)) << 16));
+          st_shared32(p.v_cache + cache_row + (o - (M::NQ + M::NKV) * M::D), vb);
         }
       });
   if (!ok) return false;
@@ -658,15 +683,22 @@ __device__ bool op_oproj(const Params& p, Smem<M>& s, const Ctx& c) {
   if (s.inst[6] != 0) return bad_operand(p, s, c, 6);
   if (s.inst[7] != kMaxBatch || s.inst[8] != kTile) return bad_operand(p, s, c, 8);
   const u16* w = p.o_w + static_cast<size_t>(layer) * M::H * M::H;
+  // The residual pair this thread adds to in the first block is asked for together with the activations.
+  u16* const mine = p.hidden + static_cast<size_t>(c.tid & 15) * M::H + 2 * (c.tid >> 4);
+  const bool adds = c.tid < 128 && (c.tid & 15) < B && s.active[c.tid & 15];
+  uint32_t old0 = 0;
   const bool ok = gemm_h<M, 1, 3>(
       p, s, c, n1 - n0, p.attn_out, B, [&](int j, int) { return w + static_cast<size_t>(n0 + j) * kTile * M::H; },
       [&] {
-        return wait_counters(p, s, c, B, [&](int i) { return counter_ptr(p, layer, ROW_REDUCE, i); }, [&](int) { return M::NQ; });
+        if (!wait_counters(p, s, c, B, [&](int i) { return counter_ptr(p, layer, ROW_REDUCE, i); }, [&](int) { return M::NQ; })) return false;
+        if (adds && n0 < n1) old0 = ld_shared32(mine + n0 * kTile);
+        return true;
       },
       [&](int j, int parity, int b, int rp) {
-        if (b >= B || !s.active[b]) return;
+        if (!adds) return;
         const float2 v = gather(s, parity, 0, b, rp);
-        residual_pair(p.hidden + static_cast<size_t>(b) * M::H + (n0 + j) * kTile + 2 * rp, v.x, v.y);
+        const uint32_t old = j == 0 ? old0 : ld_shared32(mine + (n0 + j) * kTile);
+        st_shared32(mine + (n0 + j) * kTile, residual_add(old, v.x, v.y));
       });
   if (!ok) return false;
   publish_after_stores(p, c, layer, ROW_OPROJ, 0, n1 - n0);
@@ -696,9 +728,10 @@ __device__ bool op_upgate(const Params& p, Smem<M>& s, const Ctx& c) {
         uint32_t word = 0;
         if (s.active[b]) {
           const float2 g = gather(s, parity, 0, b, rp), u = gather(s, parity, 1, b, rp);
-          const float g0 = round_bf16(g.x), g1 = round_bf16(g.y);
-          const float a0 = round_bf16(g0 / (1.0f + expf(-g0))), a1 = round_bf16(g1 / (1.0f + expf(-g1)));
-          word = static_cast<uint32_t>(f2bf(a0 * round_bf16(u.x))) | (static_cast<uint32_t>(f2bf(a1 * round_bf16(u.y))) << 16);
+          const uint32_t gb = pack_bf16(g.x, g.y), ub = pack_bf16(u.x, u.y);
+          const float g0 = bf_lo(gb), g1 = bf_hi(gb);
+          const uint32_t ab = pack_bf16(g0 / (1.0f + expf(-g0)), g1 / (1.0f + expf(-g1)));
+          word = pack_bf16(bf_lo(ab) * bf_lo(ub), bf_hi(ab) * bf_hi(ub));
         }
         st_shared32(p.silu_out + static_cast<size_t>(b) * M::F + s.inst[5 + j] * kTile + 2 * rp, word);
       });
@@ -710,8 +743,8 @@ __device__ bool op_upgate(const Params& p, Smem<M>& s, const Ctx& c) {
 // ===================================================================== 8 ==
 // [8, layer, batch_size, tile_M, n_start, n_end, tile_M_g, tile_N_g]
 // hidden[b, r] = bf16(hidden[b, r] + bf16(W_d[r] . silu_out[b])) for active rows, the whole K in
-// one instruction (python_vm.py:554-611).  A wave owns F/8 columns: F/2048 segments per block, all
-// requested before the wait; its share of silu_out follows the wait, two segments at a time.
+// one instruction (python_vm.py:554-611).  A wave owns F/8 columns: F/2048 segments per block; its
+// share of silu_out follows the wait, two segments at a time.
 template <class M>
 __device__ bool op_down(const Params& p, Smem<M>& s, const Ctx& c) {
   constexpr int NS = M::F / (kWaves * kSeg);   // segments per wave and block
@@ -725,32 +758,43 @@ __device__ bool op_down(const Params& p, Smem<M>& s, const Ctx& c) {
   const u16* w = p.down_w + static_cast<size_t>(layer) * M::H * M::F;
   const int k0 = wave * NS * kSeg;
   const size_t lane_off = static_cast<size_t>(lane & 15) * M::F + k0 + (lane >> 4) * 8;
-  Seg a[NS];
+  static_assert(NS == 4, "the segments below are handled by name");
+  // Three of the four weight segments of a block are requested before the wait and land during it; the
+  // fourth follows the first activations (all four beside two activation segments do not fit the registers).
+  Seg a0, a1, a2, a3;
+  auto wptr = [&](int block, int q) { return w + static_cast<size_t>(block) * kTile * M::F + lane_off + q * kSeg; };
   auto request = [&](int block) {
-#pragma unroll
-    for (int q = 0; q < NS; ++q) load_seg(a[q], w + static_cast<size_t>(block) * kTile * M::F + lane_off + q * kSeg);
+    load_seg(a0, wptr(block, 0));
+    load_seg(a1, wptr(block, 1));
+    load_seg(a2, wptr(block, 2));
   };
   if (n0 < n1) request(n0);
   if (!wait_counter(p, s, c, layer, ROW_UPGATE, M::F / kTile)) return false;
+  u16* const mine = p.hidden + static_cast<size_t>(c.tid & 15) * M::H + 2 * (c.tid >> 4);
+  const bool adds = c.tid < 128 && (c.tid & 15) < B && s.active[c.tid & 15];
   int parity = 0;
   for (int blk = n0; blk < n1; ++blk) {
-    f4 acc = f4{0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-    for (int q = 0; q < NS; ++q) {
-      v4u x[kSegChunks];
-      load_x(x, p.silu_out, M::F, B, k0 + q * kSeg, lane);
-      acc = mma_seg(a[q], x, acc);
-    }
+    v4u xa[kSegChunks], xb[kSegChunks];
+    load_x(xa, p.silu_out, M::F, B, k0, lane);
+    load_x(xb, p.silu_out, M::F, B, k0 + kSeg, lane);
+    load_seg(a3, wptr(blk, 3));
+    f4 acc = mma_seg(a0, xa, f4{0.f, 0.f, 0.f, 0.f});
+    load_x(xa, p.silu_out, M::F, B, k0 + 2 * kSeg, lane);
+    acc = mma_seg(a1, xb, acc);
+    load_x(xb, p.silu_out, M::F, B, k0 + 3 * kSeg, lane);
+    const uint32_t old = adds ? ld_shared32(mine + blk * kTile) : 0u;   // the pair this thread adds to, in time for the epilogue
+    acc = mma_seg(a2, xa, acc);
+    acc = mma_seg(a3, xb, acc);
     park(s, parity, 0, wave, lane, acc);
+    QMK_MB_STAMP(0);  // thread 0's weights and activations have all arrived
     if (blk + 1 < n1) request(blk + 1);
     __syncthreads();
-    if (c.tid < 128) {
-      const int b = c.tid & 15, rp = c.tid >> 4;
-      if (b < B && s.active[b]) {
-        const float2 v = gather(s, parity, 0, b, rp);
-        residual_pair(p.hidden + static_cast<size_t>(b) * M::H + blk * kTile + 2 * rp, v.x, v.y);
-      }
+    QMK_MB_STAMP(1);  // ... and everybody's
+    if (adds) {
+      const float2 v = gather(s, parity, 0, c.tid & 15, c.tid >> 4);
+      st_shared32(mine + blk * kTile, residual_add(old, v.x, v.y));
     }
+    QMK_MB_STAMP(2);
     parity ^= 1;
   }
   publish_after_stores(p, c, layer, ROW_DOWN, 0, n1 - n0);
@@ -782,7 +826,7 @@ __device__ bool op_lmhead(const Params& p, Smem<M>& s, const Ctx& c) {
         const float2 v = s.active[b] ? gather(s, parity, 0, b, rp) : float2{-1e9f, -1e9f};
         u16* dst = p.logits + static_cast<size_t>(b) * p.vocab_size + o;
         if (o + 1 < p.vocab_size && (reinterpret_cast<uintptr_t>(dst) & 3) == 0) {
-          st_shared32(dst, static_cast<uint32_t>(f2bf(v.x)) | (static_cast<uint32_t>(f2bf(v.y)) << 16));
+          st_shared32(dst, pack_bf16(v.x, v.y));
         } else {
           if (o < p.vocab_size) st_shared16(dst, f2bf(v.x));
           if (o + 1 < p.vocab_size) st_shared16(dst + 1, f2bf(v.y));
