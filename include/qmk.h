@@ -240,6 +240,10 @@ typedef struct QmkBatchArgs {
   int32_t pos_id;                  /* position of every row when position_ids is NULL */
   int32_t batch_size;              /* B, 1..16                                    */
   int32_t kv_block_size;           /* tokens per split-KV block (the scheduler's attn_kv_block_size) */
+  int32_t oproj_blocks;            /* final value of the O-proj counter = H / rows per O-proj block; 0 = H/16 */
+  int32_t down_blocks;             /* ... of the down-projection counter; 0 = H/16.  Blocks of 16 rows are
+                                      the reference's; this library also takes 8 (word tile_N_granularity
+                                      of opcodes 5 and 8), which gives each of 256 workgroups one block */
   float attn_scale;
   float rms_norm_eps;
 

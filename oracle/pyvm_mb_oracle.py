@@ -53,8 +53,11 @@ class _MergeAll:
 
 
 class BatchInstructionVM:
-    def __init__(self, shape: Any):
+    def __init__(self, shape: Any, oproj_tile: int = TILE, down_tile: int = TILE):
+        """``oproj_tile`` / ``down_tile``: rows per block of the two residual projections in the stream
+        (16 in the reference's; they fix the counter values the RMSNorm rows wait for)."""
         self.shape = shape
+        self.oproj_blocks, self.down_blocks = shape.hidden_size // oproj_tile, shape.hidden_size // down_tile
         self.stride = shape.num_attention_heads + 2 * shape.num_key_value_heads   # counter slots per batch row
 
     # ---- state ---------------------------------------------------------------
@@ -88,18 +91,18 @@ class BatchInstructionVM:
 
     def attn_rms(self, g: Any, ins: Any) -> None:
         if ins.layer_idx > 0:
-            assert int(g.barriers[ins.layer_idx - 1, 7, 0]) == self.shape.hidden_size // TILE
+            assert int(g.barriers[ins.layer_idx - 1, 7, 0]) == self.down_blocks
         self._rms_row(g, g.attn_rms_out, ins.batch_row, g.attn_norm_weights[ins.layer_idx])
         g.barriers[ins.layer_idx, 0, 0] += 1
 
     def mlp_rms(self, g: Any, ins: Any) -> None:
-        assert int(g.barriers[ins.layer_idx, 4, 0]) == self.shape.hidden_size // TILE
+        assert int(g.barriers[ins.layer_idx, 4, 0]) == self.oproj_blocks
         self._rms_row(g, g.mlp_rms_out, ins.batch_row, g.mlp_norm_weights[ins.layer_idx])
         g.barriers[ins.layer_idx, 5, 0] += 1
 
     def lmhead_rms(self, g: Any, ins: Any) -> None:
         last = self.shape.num_hidden_layers - 1
-        assert int(g.barriers[last, 7, 0]) == self.shape.hidden_size // TILE
+        assert int(g.barriers[last, 7, 0]) == self.down_blocks
         self._rms_row(g, g.lm_head_rms_out, ins.batch_row, g.lm_head_norm_weights)
         g.barriers[last, 8, 0] += 1
 
@@ -236,7 +239,7 @@ class BatchInstructionVM:
         self._gemm_residual(g, ins, g.o_proj_weights[ins.layer_idx], g.attn_out, 4)
 
     def down_proj_residual(self, g: Any, ins: Any) -> None:
-        assert int(g.barriers[ins.layer_idx, 6, 0]) == self.shape.intermediate_size // ins.tile_N_granularity
+        assert int(g.barriers[ins.layer_idx, 6, 0]) == self.shape.intermediate_size // TILE
         self._gemm_residual(g, ins, g.down_proj_weights[ins.layer_idx], g.silu_out, 7)
 
     # ---- 7 -------------------------------------------------------------------------

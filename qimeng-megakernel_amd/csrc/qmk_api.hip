@@ -405,7 +405,7 @@ extern "C" int qmk_decode_step_batch(const QmkBatchArgs* a) {
   if (a->batch_size < 1 || a->batch_size > mb::kMaxBatch) return QMK_ERR_SHAPE;
   if (a->num_queues < 1 || a->num_insts < 0 || a->num_layers < 1 || a->num_layer_barriers < 10 ||
       a->barrier_slots < a->batch_size * (M::NQ + 2 * M::NKV) || a->max_seq_len < 1 || a->max_splits < 1 ||
-      a->vocab_size < 1 || a->rope_rows < 1 || a->kv_block_size < 1)
+      a->vocab_size < 1 || a->rope_rows < 1 || a->kv_block_size < 1 || a->oproj_blocks < 0 || a->down_blocks < 0)
     return QMK_ERR_SHAPE;
   if (a->flags & ~QMK_FLAG_KEEP_BARRIERS) return QMK_ERR_SHAPE;
   if (a->position_ids == nullptr && (a->pos_id < 0 || a->pos_id >= a->max_seq_len || a->pos_id >= a->rope_rows)) return QMK_ERR_POSITION;
@@ -452,6 +452,8 @@ extern "C" int qmk_decode_step_batch(const QmkBatchArgs* a) {
   p.rms_norm_eps = a->rms_norm_eps;
   p.spin_limit = a->spin_limit > 0 ? a->spin_limit : kDefaultSpinLimit;
   p.flags = a->flags;
+  p.oproj_blocks = a->oproj_blocks > 0 ? a->oproj_blocks : M::H / mb::kTile;
+  p.down_arrivals = a->down_blocks > 0 ? a->down_blocks : M::H / mb::kTile;
   p.batch = a->batch_size;
   p.kv_block = a->kv_block_size;
   p.position_ids = a->position_ids;

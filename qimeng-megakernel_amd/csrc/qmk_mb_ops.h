@@ -147,7 +147,8 @@ __device__ bool op_rms_row(const Params& p, Smem<M>& s, const Ctx& c) {
     weight = p.lm_norm, dst = p.lm_rms_out, my_row = ROW_LM_RMS, wait_row = ROW_DOWN;
   }
   const uint2 wv = *reinterpret_cast<const uint2*>(weight + c.tid * 4);
-  if (wait_layer >= 0 && !wait_counter(p, s, c, wait_layer, wait_row, M::H / kTile)) return false;
+  const int produced = wait_row == ROW_OPROJ ? p.oproj_blocks : p.down_arrivals;   // blocks of the projection that completes the rows
+  if (wait_layer >= 0 && !wait_counter(p, s, c, wait_layer, wait_row, produced)) return false;
   uint32_t lo = 0, hi = 0;
   if (s.active[row]) {
     const uint64_t hw = ld_shared64(p.hidden + static_cast<size_t>(row) * M::H + c.tid * 4);
@@ -224,11 +225,14 @@ __device__ __forceinline__ float2 gather(const Smem<M>& s, int parity, int unit,
 // all threads right after the block's tiles are parked (still before the barrier), `epi(j, parity,
 // b, rp)` on threads 0..127 after it.  The ring holds NB blocks; the first NB are requested at once
 // (the caller decides whether that is before or after its wait through `wait`).
+// `rows` (16, or 8): weight rows per block; with 8 the upper half of the tile repeats the lower one
+// (the same addresses: no extra traffic) and only outputs 0..7 are used.
 template <class M, int NU, int NB, class Src, class Wait, class Epi>
-__device__ __forceinline__ bool gemm_h(const Params& p, Smem<M>& s, const Ctx& c, int n, const u16* act, int B, Src src, Wait wait, Epi epi) {
+__device__ __forceinline__ bool gemm_h(const Params& p, Smem<M>& s, const Ctx& c, int n, const u16* act, int B, Src src, Wait wait, Epi epi,
+                                       int rows = kTile) {
   static_assert(M::H == kWaves * kSeg, "one segment per wave");
   const int lane = c.tid & 63, wave = c.tid >> 6;
-  const size_t lane_off = static_cast<size_t>(lane & 15) * M::H + wave * kSeg + (lane >> 4) * 8;
+  const size_t lane_off = static_cast<size_t>(lane & (rows - 1)) * M::H + wave * kSeg + (lane >> 4) * 8;
   Seg ring[NB][NU];
 #pragma unroll
   for (int k = 0; k < NB; ++k)
@@ -253,7 +257,7 @@ __device__ __forceinline__ bool gemm_h(const Params& p, Smem<M>& s, const Ctx& c
         __syncthreads();
         // Parity: a slot is written again two blocks later, behind the next barrier, which the
         // reading threads reach only after they are done with it.
-        if (c.tid < 128) epi(j, parity, c.tid & 15, c.tid >> 4);
+        if (c.tid < 8 * rows) epi(j, parity, c.tid & 15, c.tid >> 4);
         parity ^= 1;
       }
     }
@@ -679,27 +683,29 @@ __device__ bool op_oproj(const Params& p, Smem<M>& s, const Ctx& c) {
   const int layer = s.inst[1], B = s.inst[2], n0 = s.inst[4], n1 = s.inst[5];
   if (layer < 0 || layer >= p.num_layers) return bad_operand(p, s, c, 1);
   if (B != p.batch || s.inst[3] != 0) return bad_operand(p, s, c, 2);
-  if (n0 < 0 || n1 < n0 || n1 > M::H / kTile) return bad_operand(p, s, c, 4);
+  const int R = s.inst[8];   // rows per block: 16 (the reference's), or 8 (one block per workgroup on 256 CUs)
+  if (s.inst[7] != kMaxBatch || (R != kTile && R != kTile / 2)) return bad_operand(p, s, c, 8);
+  if (n0 < 0 || n1 < n0 || n1 > M::H / R) return bad_operand(p, s, c, 4);
   if (s.inst[6] != 0) return bad_operand(p, s, c, 6);
-  if (s.inst[7] != kMaxBatch || s.inst[8] != kTile) return bad_operand(p, s, c, 8);
   const u16* w = p.o_w + static_cast<size_t>(layer) * M::H * M::H;
   // The residual pair this thread adds to in the first block is asked for together with the activations.
   u16* const mine = p.hidden + static_cast<size_t>(c.tid & 15) * M::H + 2 * (c.tid >> 4);
-  const bool adds = c.tid < 128 && (c.tid & 15) < B && s.active[c.tid & 15];
+  const bool adds = c.tid < 8 * R && (c.tid & 15) < B && s.active[c.tid & 15];
   uint32_t old0 = 0;
   const bool ok = gemm_h<M, 1, 3>(
-      p, s, c, n1 - n0, p.attn_out, B, [&](int j, int) { return w + static_cast<size_t>(n0 + j) * kTile * M::H; },
+      p, s, c, n1 - n0, p.attn_out, B, [&](int j, int) { return w + static_cast<size_t>(n0 + j) * R * M::H; },
       [&] {
         if (!wait_counters(p, s, c, B, [&](int i) { return counter_ptr(p, layer, ROW_REDUCE, i); }, [&](int) { return M::NQ; })) return false;
-        if (adds && n0 < n1) old0 = ld_shared32(mine + n0 * kTile);
+        if (adds && n0 < n1) old0 = ld_shared32(mine + n0 * R);
         return true;
       },
       [&](int j, int parity, int b, int rp) {
         if (!adds) return;
         const float2 v = gather(s, parity, 0, b, rp);
-        const uint32_t old = j == 0 ? old0 : ld_shared32(mine + (n0 + j) * kTile);
-        st_shared32(mine + (n0 + j) * kTile, residual_add(old, v.x, v.y));
-      });
+        const uint32_t old = j == 0 ? old0 : ld_shared32(mine + (n0 + j) * R);
+        st_shared32(mine + (n0 + j) * R, residual_add(old, v.x, v.y));
+      },
+      R);
   if (!ok) return false;
   publish_after_stores(p, c, layer, ROW_OPROJ, 0, n1 - n0);
   return true;
@@ -752,17 +758,18 @@ __device__ bool op_down(const Params& p, Smem<M>& s, const Ctx& c) {
   const int layer = s.inst[1], B = s.inst[2], n0 = s.inst[4], n1 = s.inst[5];
   if (layer < 0 || layer >= p.num_layers) return bad_operand(p, s, c, 1);
   if (B != p.batch || s.inst[3] != 0) return bad_operand(p, s, c, 2);
-  if (n0 < 0 || n1 < n0 || n1 > M::H / kTile) return bad_operand(p, s, c, 4);
-  if (s.inst[6] != kMaxBatch || s.inst[7] != kTile) return bad_operand(p, s, c, 7);
+  const int R = s.inst[7];   // rows per block: 16 (the reference's), or 8 (one block per workgroup on 256 CUs)
+  if (s.inst[6] != kMaxBatch || (R != kTile && R != kTile / 2)) return bad_operand(p, s, c, 7);
+  if (n0 < 0 || n1 < n0 || n1 > M::H / R) return bad_operand(p, s, c, 4);
   const int lane = c.tid & 63, wave = c.tid >> 6;
   const u16* w = p.down_w + static_cast<size_t>(layer) * M::H * M::F;
   const int k0 = wave * NS * kSeg;
-  const size_t lane_off = static_cast<size_t>(lane & 15) * M::F + k0 + (lane >> 4) * 8;
+  const size_t lane_off = static_cast<size_t>(lane & (R - 1)) * M::F + k0 + (lane >> 4) * 8;
   static_assert(NS == 4, "the segments below are handled by name");
   // Three of the four weight segments of a block are requested before the wait and land during it; the
   // fourth follows the first activations (all four beside two activation segments do not fit the registers).
   Seg a0, a1, a2, a3;
-  auto wptr = [&](int block, int q) { return w + static_cast<size_t>(block) * kTile * M::F + lane_off + q * kSeg; };
+  auto wptr = [&](int block, int q) { return w + static_cast<size_t>(block) * R * M::F + lane_off + q * kSeg; };
   auto request = [&](int block) {
     load_seg(a0, wptr(block, 0));
     load_seg(a1, wptr(block, 1));
@@ -771,7 +778,7 @@ __device__ bool op_down(const Params& p, Smem<M>& s, const Ctx& c) {
   if (n0 < n1) request(n0);
   if (!wait_counter(p, s, c, layer, ROW_UPGATE, M::F / kTile)) return false;
   u16* const mine = p.hidden + static_cast<size_t>(c.tid & 15) * M::H + 2 * (c.tid >> 4);
-  const bool adds = c.tid < 128 && (c.tid & 15) < B && s.active[c.tid & 15];
+  const bool adds = c.tid < 8 * R && (c.tid & 15) < B && s.active[c.tid & 15];
   int parity = 0;
   for (int blk = n0; blk < n1; ++blk) {
     v4u xa[kSegChunks], xb[kSegChunks];
@@ -782,7 +789,7 @@ __device__ bool op_down(const Params& p, Smem<M>& s, const Ctx& c) {
     load_x(xa, p.silu_out, M::F, B, k0 + 2 * kSeg, lane);
     acc = mma_seg(a1, xb, acc);
     load_x(xb, p.silu_out, M::F, B, k0 + 3 * kSeg, lane);
-    const uint32_t old = adds ? ld_shared32(mine + blk * kTile) : 0u;   // the pair this thread adds to, in time for the epilogue
+    const uint32_t old = adds ? ld_shared32(mine + blk * R) : 0u;   // the pair this thread adds to, in time for the epilogue
     acc = mma_seg(a2, xa, acc);
     acc = mma_seg(a3, xb, acc);
     park(s, parity, 0, wave, lane, acc);
@@ -792,7 +799,7 @@ __device__ bool op_down(const Params& p, Smem<M>& s, const Ctx& c) {
     QMK_MB_STAMP(1);  // ... and everybody's
     if (adds) {
       const float2 v = gather(s, parity, 0, c.tid & 15, c.tid >> 4);
-      st_shared32(mine + blk * kTile, residual_add(old, v.x, v.y));
+      st_shared32(mine + blk * R, residual_add(old, v.x, v.y));
     }
     QMK_MB_STAMP(2);
     parity ^= 1;

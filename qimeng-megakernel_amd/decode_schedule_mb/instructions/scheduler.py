@@ -81,6 +81,8 @@ class BatchScheduler:
     workers: int
     batch_size: int
     merge_in_last: bool = False   # the last split-KV arrival of a head group merges: no reduction instructions
+    oproj_tile: int = TILE_N_GRANULARITY   # rows per O-proj block: 16 (the reference's), or 8
+    down_tile: int = TILE_N_GRANULARITY    # rows per down-projection block
 
     def __post_init__(self) -> None:
         if not 1 <= self.batch_size <= MAX_BATCH:
@@ -103,8 +105,9 @@ class BatchScheduler:
         return [QKVProj_GEMM_RoPE(layer, self.batch_size, 0, lo, hi) for lo, hi in _spans(blocks, self.workers)]
 
     def oproj(self, layer: int) -> list[Instruction]:
-        blocks = _ceil_div(self.shape.hidden_size, TILE_N_GRANULARITY)
-        return [OProj_GEMM_Residual(layer, self.batch_size, 0, lo, hi, 0) for lo, hi in _spans(blocks, self.workers)]
+        blocks = _ceil_div(self.shape.hidden_size, self.oproj_tile)
+        return [OProj_GEMM_Residual(layer, self.batch_size, 0, lo, hi, 0, tile_N_granularity=self.oproj_tile)
+                for lo, hi in _spans(blocks, self.workers)]
 
     def upgate(self, layer: int) -> list[Instruction]:
         blocks = _ceil_div(self.shape.intermediate_size, TILE_N_GRANULARITY)
@@ -116,8 +119,9 @@ class BatchScheduler:
         return out
 
     def downproj(self, layer: int) -> list[Instruction]:
-        blocks = _ceil_div(self.shape.hidden_size, TILE_N_GRANULARITY)
-        return [DownProj_GEMM_Residual(layer, self.batch_size, 0, lo, hi) for lo, hi in _spans(blocks, self.workers)]
+        blocks = _ceil_div(self.shape.hidden_size, self.down_tile)
+        return [DownProj_GEMM_Residual(layer, self.batch_size, 0, lo, hi, tile_N_granularity=self.down_tile)
+                for lo, hi in _spans(blocks, self.workers)]
 
     def lmhead(self) -> list[Instruction]:
         blocks = _ceil_div(self.shape.vocab_size, TILE_N_GRANULARITY)
@@ -232,6 +236,13 @@ def reference_scheduler(batch_size: int, shape: DecodeShape | None = None) -> Ba
     return BatchScheduler(shape or LlamaConfig.shape(), A100_WORKERS, batch_size)
 
 
-def mi355x_scheduler(batch_size: int, shape: DecodeShape | None = None, *, merge_in_last: bool = True) -> BatchScheduler:
-    """One queue per CU; the split-KV partials are merged by the last arrival of each head group."""
-    return BatchScheduler(shape or LlamaConfig.shape(), MI355X_WORKERS, batch_size, merge_in_last=merge_in_last)
+def mi355x_scheduler(batch_size: int, shape: DecodeShape | None = None, *, merge_in_last: bool = True,
+                     residual_tile: int = 16) -> BatchScheduler:
+    """One queue per CU; the split-KV partials are merged by the last arrival of each head group.
+    ``residual_tile`` 8 gives the two projections that add to the residual stream one 8-row block per
+    workgroup instead of 16-row blocks on half the CUs; measured slower at batch 8 (every workgroup
+    reads all activations, so twice the workgroups read them twice: 7478 against 8015 tok/s)."""
+    if residual_tile not in (8, 16):
+        raise ValueError("blocks of the residual projections have 8 or 16 rows")
+    return BatchScheduler(shape or LlamaConfig.shape(), MI355X_WORKERS, batch_size, merge_in_last=merge_in_last,
+                          oproj_tile=residual_tile, down_tile=residual_tile)

@@ -45,7 +45,7 @@ class QmkBatchArgs(ctypes.Structure):
         ("down_proj_weights", _P), ("lm_head_norm_weights", _P), ("lm_head_weights", _P), ("barriers", _P),
         ("num_queues", _I), ("num_insts", _I), ("num_layers", _I), ("num_layer_barriers", _I),
         ("barrier_slots", _I), ("max_seq_len", _I), ("max_splits", _I), ("vocab_size", _I), ("rope_rows", _I),
-        ("pos_id", _I), ("batch_size", _I), ("kv_block_size", _I),
+        ("pos_id", _I), ("batch_size", _I), ("kv_block_size", _I), ("oproj_blocks", _I), ("down_blocks", _I),
         ("attn_scale", ctypes.c_float), ("rms_norm_eps", ctypes.c_float),
         ("position_ids", _P), ("active_mask", _P), ("attn_partial_valid", _P),
         ("attn_rms_out", _P), ("mlp_rms_out", _P), ("lm_head_rms_out", _P),
@@ -106,6 +106,7 @@ class BatchMegaKernel:
         self._lib = lib
         self.reset_barriers = reset_barriers
         self.spin_limit = int(spin_limit)
+        self.residual_tiles = (16, 16)   # rows per O-proj / down-projection block of the stream (set per call by call_mk)
         self.timeline: torch.Tensor | None = None
         self._args = QmkBatchArgs()
         self._args.struct_size = ctypes.sizeof(QmkBatchArgs)
@@ -224,6 +225,8 @@ class BatchMegaKernel:
         a.rms_norm_eps = float(rms_norm_eps)
         a.flags = 0 if self.reset_barriers else _single.QMK_FLAG_KEEP_BARRIERS
         a.spin_limit = self.spin_limit
+        hidden = LlamaConfig.shape().hidden_size
+        a.oproj_blocks, a.down_blocks = hidden // self.residual_tiles[0], hidden // self.residual_tiles[1]
         a.timeline = self.timeline.data_ptr() if self.timeline is not None else None
         a.stream = torch.cuda.current_stream(tensors[1].device).cuda_stream
         rc = int(self._lib.qmk_decode_step_batch(ctypes.byref(a)))
@@ -271,6 +274,8 @@ def call_mk(globs: Globals, mk: Any) -> None:
     else:
         position_ids = None
     active = _mask_for_mk(globs.active_mask, device) if globs.active_mask is not None and globs.active_mask.numel() == B else None
+    if isinstance(mk, BatchMegaKernel):
+        mk.residual_tiles = tuple(getattr(globs, "residual_tiles", (16, 16)))
     mk(
         globs.instructions,
         globs.hidden_states,
@@ -314,6 +319,7 @@ def build(globs: Globals, kv_capacity: int | None = None) -> torch.Tensor:
     capacity = int(globs.k_cache.shape[2]) if kv_capacity is None else kv_capacity
     if sched.partials_for_capacity(capacity) > int(globs.attn_lse_intermediates.shape[-1]):
         raise ValueError("attn_lse_intermediates has fewer partial slots than the schedule's split-KV fan-out")
+    globs.residual_tiles = (sched.oproj_tile, sched.down_tile)
     return tensorize_instructions(globs, sched.runtime_queues(capacity))
 
 
@@ -324,5 +330,11 @@ def run_instructions(globs: Globals, instructions: list[Instruction], *, mk: Any
     if isinstance(mk_call, BatchMegaKernel) and mk_call.reset_barriers:
         mk_call = mk_call.with_options(reset_barriers=False)
     queues = _scheduler.deal(instructions, workers or _scheduler.MI355X_WORKERS)
+    # rows per O-proj / down block: what the stream's own instructions say, else what the caller was built with
+    tiles = list(getattr(globs, "residual_tiles", (16, 16)))
+    for ins in instructions:
+        if ins.opcode() in (5, 8):
+            tiles[0 if ins.opcode() == 5 else 1] = ins.tile_N_granularity
+    globs.residual_tiles = tuple(tiles)
     tensorize_instructions(globs, queues)
     call_mk(globs, mk_call)

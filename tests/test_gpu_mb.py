@@ -70,6 +70,10 @@ def make_pair(weights, rows, positions, *, inactive=(), capacity=None, shape=MB_
     return cpu, gpu
 
 
+def vm_for(sched):
+    return BatchInstructionVM(sched.shape, sched.oproj_tile, sched.down_tile)
+
+
 def run_kernel(gpu, instructions, workers=256):
     mk = mk_kernel.get_mk(reset_barriers=False, spin_limit=1 << 18)
     mk_kernel.run_instructions(gpu, copy.deepcopy(instructions), mk=mk, workers=workers)
@@ -118,15 +122,19 @@ def stage_instructions(sched, globs, name, layer=0):
 
 @pytest.mark.parametrize("stage", range(len(STAGES)), ids=[s[0] for s in STAGES])
 @pytest.mark.parametrize("case", ["ragged3", "inactive_row", "batch16"])
-def test_one_op_against_the_vm(weights, stage, case):
+@pytest.mark.parametrize("tile", [16, 8], ids=["blocks16", "residual_blocks8"])
+def test_one_op_against_the_vm(weights, stage, case, tile):
     """Everything before the op runs on the VM; the op itself on both, from identical state."""
     rows, positions, inactive = CASES[case]
+    if tile == 8 and STAGES[stage][0] not in ("oproj", "mlp_rms", "downproj"):
+        pytest.skip("only the residual projections and what waits for them see the block size")
     cpu, gpu = make_pair(weights, rows, positions, inactive=inactive)
-    sched = S.mi355x_scheduler(rows, MB_SMALL, merge_in_last=False)
-    vm = BatchInstructionVM(MB_SMALL)
+    sched = S.mi355x_scheduler(rows, MB_SMALL, merge_in_last=False, residual_tile=tile)
+    vm = vm_for(sched)
     for name, _ in STAGES[:stage]:
         vm.run(cpu, stage_instructions(sched, cpu, name))
     sync_state(cpu, gpu)
+    gpu.residual_tiles = (sched.oproj_tile, sched.down_tile)
     mine = stage_instructions(sched, cpu, STAGES[stage][0])
     vm.run(cpu, copy.deepcopy(mine))
     run_kernel(gpu, mine)
@@ -151,7 +159,7 @@ def test_split_kv_whose_last_arrival_merges(weights, case, template):
     rows, positions, inactive = CASES[case]
     cpu, gpu = make_pair(weights, rows, positions, inactive=inactive)
     sched = S.mi355x_scheduler(rows, MB_SMALL)
-    vm = BatchInstructionVM(MB_SMALL)
+    vm = vm_for(sched)
     vm.run(cpu, sched.attn_rms(0) + sched.qkvproj(0))
     sync_state(cpu, gpu)
     p = sched.partials_for_capacity(FIX["kv_capacity"]) if template else sched.partials_for_request(cpu)
@@ -168,10 +176,11 @@ def test_lm_head_ops_against_the_vm(weights):
     cpu, gpu = make_pair(weights, 3, (70, 3, 130), inactive=(1,))
     sched = S.mi355x_scheduler(3, MB_SMALL)
     last = MB_SMALL.num_hidden_layers - 1
-    cpu.barriers[last, 7, 0] = MB_SMALL.hidden_size // 16     # the last down projection is complete
+    cpu.barriers[last, 7, 0] = MB_SMALL.hidden_size // sched.down_tile     # the last down projection is complete
     sync_state(cpu, gpu)
+    gpu.residual_tiles = (sched.oproj_tile, sched.down_tile)
     mine = sched.lmhead_rms() + sched.lmhead()
-    BatchInstructionVM(MB_SMALL).run(cpu, copy.deepcopy(mine))
+    vm_for(sched).run(cpu, copy.deepcopy(mine))
     run_kernel(gpu, mine)
     compare(cpu, gpu, ("lm_head_rms_out", "logits"))
     assert bool((gpu.logits[1].float() == torch.tensor(-1e9).bfloat16().float()).all())
@@ -183,7 +192,7 @@ def test_whole_step_static_list(weights, make, workers):
     cpu, gpu = make_pair(weights, 3, (70, 3, 130))
     sched = make(3, MB_SMALL)
     mine = sched.instruction_list(cpu)
-    BatchInstructionVM(MB_SMALL).run(cpu, copy.deepcopy(mine))
+    vm_for(sched).run(cpu, copy.deepcopy(mine))
     run_kernel(gpu, mine, workers=workers)
     assert torch.equal(gpu.barriers.cpu(), cpu.barriers)
     tensor_rel_close(gpu.hidden_states, cpu.hidden_states, name="hidden_states")
@@ -235,8 +244,9 @@ def test_full_size_layers_against_the_fused_oracle(full_weights, rows):
     cpu.hidden_states.copy_(cpu.embed_tokens[toks])
     fused, sched = FusedBatchOracle(MB_FULL), S.mi355x_scheduler(rows, MB_FULL)
     live = [r for r in range(rows) if bool(cpu.active_mask[r])]
-    done = MB_FULL.hidden_size // 16
+    done = MB_FULL.hidden_size // sched.down_tile
     p = sched.partials_for_request(cpu)
+    gpu.residual_tiles = (sched.oproj_tile, sched.down_tile)
     for layer in range(MB_FULL.num_hidden_layers):
         gpu.hidden_states.copy_(cpu.hidden_states)
         before = cpu.hidden_states.clone()

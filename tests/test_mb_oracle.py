@@ -120,7 +120,8 @@ def test_every_output_once_and_final_counters(make, rows):
     out = {op: [] for op in (2, 5, 7, 8, 10)}
     for i in flat:
         if i.opcode() in (2, 5, 8):
-            out[i.opcode()] += range(i.tile_N_start_idx * 16, i.tile_N_end_idx * 16)
+            out[i.opcode()] += range(i.tile_N_start_idx * i.tile_N_granularity, i.tile_N_end_idx * i.tile_N_granularity)
+            assert i.tile_N_granularity == (16 if i.opcode() == 2 else sched.oproj_tile if i.opcode() == 5 else sched.down_tile)
         elif i.opcode() == 7:
             for b in i.tile_N_block_idxs:
                 out[7] += range(b * 16, b * 16 + 16)
@@ -207,7 +208,7 @@ def test_inactive_row_is_frozen_and_forced(weights):
     v = _request(weights); v.active_mask[1] = False
     v.hidden_states.copy_(g.hidden_states)
     FusedBatchOracle(MB_SMALL).decode_step(g)
-    BatchInstructionVM(MB_SMALL).run(v, S.mi355x_scheduler(3, MB_SMALL).instruction_list(v))
+    BatchInstructionVM(MB_SMALL, 8, 8).run(v, S.mi355x_scheduler(3, MB_SMALL, residual_tile=8).instruction_list(v))
     for x in (g, v):
         assert torch.equal(x.hidden_states[1], frozen[0]) and torch.equal(x.k_cache[:, 1], frozen[1])
         assert torch.equal(x.q_post_rope[1], frozen[2])
@@ -223,8 +224,9 @@ def test_vm_agrees_with_fused_and_counters_complete(weights):
         for g in (f, v):
             g.hidden_states[b].copy_(g.embed_tokens[20 + b])
     FusedBatchOracle(MB_SMALL).decode_step(f)
-    sched = S.mi355x_scheduler(3, MB_SMALL)
-    BatchInstructionVM(MB_SMALL).run(v, sched.runtime_instruction_list(FIX["kv_capacity"]))
+    sched = S.mi355x_scheduler(3, MB_SMALL, residual_tile=8)
+    assert (sched.oproj_tile, sched.down_tile) == (8, 8) and S.mi355x_scheduler(3, MB_SMALL).down_tile == 16
+    BatchInstructionVM(MB_SMALL, sched.oproj_tile, sched.down_tile).run(v, sched.runtime_instruction_list(FIX["kv_capacity"]))
     for name in ("q_post_rope", "attn_out", "silu_out", "hidden_states", "logits"):
         a, b_ = getattr(f, name).float(), getattr(v, name).float()
         assert float((a - b_).abs().max()) <= 2.0 ** -5 * max(1.0, float(a.abs().max())), name
@@ -238,7 +240,7 @@ def test_vm_agrees_with_fused_and_counters_complete(weights):
         for b in range(3):
             assert bar[2, b * stride : b * stride + s.num_attention_heads].tolist() == [p] * s.num_attention_heads
             assert int(bar[3, b]) == s.num_attention_heads
-        assert int(bar[4, 0]) == s.hidden_size // 16 == int(bar[7, 0]) and int(bar[6, 0]) == s.intermediate_size // 16
+        assert int(bar[4, 0]) == s.hidden_size // 8 == int(bar[7, 0]) and int(bar[6, 0]) == s.intermediate_size // 16
     assert int(v.barriers[s.num_hidden_layers - 1, 8, 0]) == 3
 
 
