@@ -820,7 +820,7 @@ __device__ bool op_lmhead(const Params& p, Smem<M>& s, const Ctx& c) {
   const int last = p.vocab_size - 1;
   const int lane_row = c.tid & 15;
   // The last block may be ragged: its missing rows re-read the last row and are not stored.
-  return gemm_h<M, 1, 3>(
+  return gemm_h<M, 1, 4>(
       p, s, c, n1 - n0, p.lm_rms_out, B,
       [&](int j, int) {
         const int r0 = (n0 + j) * kTile;
