@@ -1,6 +1,7 @@
 """CPU oracle of the batch decode route (B rows) — TEST INFRASTRUCTURE, not product code.
 
-Only ``tests/`` may import this module, and only as the checker.
+Only ``tests/`` and the ``cpu_baseline`` leg of ``bench.py`` may import this module: as the checker and as
+the timed CPU baseline, never as part of the product path.
 
 The reference has no separate fused route for batch sizes above one: its single-batch fused
 operations work on ``[B, H]`` activations

@@ -39,7 +39,7 @@ def prefill_by_decode(globs: Any, mk: Any, prompts: torch.Tensor) -> torch.Tenso
         _embed(globs, prompts[:, pos])
         globs.position_ids.fill_(pos)
         _mk_kernel.call_mk(globs, mk)
-    return globs.logits.float().argmax(dim=-1)
+    return globs.logits.argmax(dim=-1)
 
 
 def decode(globs: Any, prompts: torch.Tensor, max_new_tokens: int, *, mk: Any = None, eos_token_ids: Sequence[int] = (),
@@ -80,7 +80,7 @@ def decode(globs: Any, prompts: torch.Tensor, max_new_tokens: int, *, mk: Any = 
         _mk_kernel.call_mk(globs, mk)
         if events:
             events[i][1].record()
-        nxt = globs.logits.float().argmax(dim=-1)
+        nxt = globs.logits.argmax(dim=-1)
         out[:, T + i + 1] = nxt
         if eos_token_ids:
             active_log.append(globs.active_mask.clone())
