@@ -1,0 +1,192 @@
+"""The twelve opcodes of the MoE decode route and their counter protocol.
+
+Opcodes, operand order and defaults are the reference's
+(`…/qwen1_5_moe_a2_7b/A100/single_batch/decode_schedule/instructions/instruction_defs.py:24-262`).
+Opcodes 1-4 and 7 are the dense route's attention and LM head (QKV with bias); 5 and 6 are unused;
+8-14 replace the dense MLP.
+
+Counters ``barriers[layer, opcode - 1, slot]`` (`…/instructions/python_vm.py:109-560`):
+
+=====  =============================  ==========================  ================================
+row    producer                       slot                        final count
+=====  =============================  ==========================  ================================
+0      1 RMS + QKV + bias + RoPE      q/k/v head index            head_dim / 16
+1      2 split-KV attention           query head                  num_partials
+2      3 attention reduction          0                           Hq
+3      4 O-proj + residual            0                           hidden / 16
+7      8 RMS + router logits          0: experts, 1: normed row   E, 1
+8      9 softmax + top-k              0                           1 (set, not added)
+9      10 shared up/gate + SiLU       0                           shared_intermediate / 16
+10     11 shared down (split K)       hidden block                num_downproj_split_k_shared
+11     12 routed up/gate + SiLU       0                           top_k * moe_intermediate / 16
+12     13 routed down                 hidden block                top_k
+13     14 combine + commit            0                           hidden / 16
+=====  =============================  ==========================  ================================
+"""
+from __future__ import annotations
+
+from dataclasses import dataclass
+from typing import ClassVar
+
+from ...instruction import Instruction
+
+TILE_M_GRANULARITY = 1
+TILE_N_GRANULARITY = 16
+ROUTER_TILE_N_GRANULARITY = 1
+SPLIT_K_GRANULARITY_SHARED = 5632 // 4   # default operand of opcode 11; schedulers pass the shape's
+
+
+@dataclass
+class NoOp(Instruction):
+    OPCODE: ClassVar[int] = 0
+
+
+@dataclass
+class RMS_QKVProj_GEMV_RoPE(Instruction):
+    OPCODE: ClassVar[int] = 1
+    PREV_OPCODES: ClassVar[tuple[int, ...]] = (14,)
+    layer_idx: int
+    tile_M_idx: int
+    tile_N_start_idx: int
+    tile_N_end_idx: int
+    tile_M_granularity: int = TILE_M_GRANULARITY
+    tile_N_granularity: int = TILE_N_GRANULARITY
+
+
+@dataclass
+class DecodeAttentionSplitKV(Instruction):
+    OPCODE: ClassVar[int] = 2
+    PREV_OPCODES: ClassVar[tuple[int, ...]] = (1,)
+    layer_idx: int
+    kv_head_idx: int
+    num_partials: int
+    partial_idx: int
+
+
+@dataclass
+class DecodeAttentionReduction(Instruction):
+    OPCODE: ClassVar[int] = 3
+    PREV_OPCODES: ClassVar[tuple[int, ...]] = (2,)
+    layer_idx: int
+    head_start_idx: int
+    num_partials: int
+    reduction_list: list[int]
+    is_terminal: int = 1
+    output_partial_idx: int = 0
+
+
+@dataclass
+class OProj_GEMV_Residual(Instruction):
+    OPCODE: ClassVar[int] = 4
+    PREV_OPCODES: ClassVar[tuple[int, ...]] = (3,)
+    layer_idx: int
+    tile_M_idx: int
+    tile_N_start_idx: int
+    tile_N_end_idx: int
+    reduction_block_idx: int
+    tile_M_granularity: int = TILE_M_GRANULARITY
+    tile_N_granularity: int = TILE_N_GRANULARITY
+
+
+@dataclass
+class RMS_LMHead_GEMV(Instruction):
+    OPCODE: ClassVar[int] = 7
+    PREV_OPCODES: ClassVar[tuple[int, ...]] = (14,)
+    start_output_block_idx: int
+    end_output_block_idx: int
+    tile_M_granularity: int = TILE_M_GRANULARITY
+    tile_N_granularity: int = TILE_N_GRANULARITY
+
+
+@dataclass
+class Router_GEMV(Instruction):
+    """RMSNorm + router logits of experts [start, end); one instruction also publishes the normalised row."""
+
+    OPCODE: ClassVar[int] = 8
+    PREV_OPCODES: ClassVar[tuple[int, ...]] = (4,)
+    layer_idx: int
+    tile_N_start_idx: int
+    tile_N_end_idx: int
+    write_normed_hidden: int = 0
+    tile_N_granularity: int = ROUTER_TILE_N_GRANULARITY
+
+
+@dataclass
+class Router_SoftmaxTopK(Instruction):
+    """softmax over all router logits, top-k: expert_indices / expert_weights."""
+
+    OPCODE: ClassVar[int] = 9
+    PREV_OPCODES: ClassVar[tuple[int, ...]] = (8,)
+    layer_idx: int
+
+
+@dataclass
+class SharedExpert_UpGate_SiLU(Instruction):
+    OPCODE: ClassVar[int] = 10
+    PREV_OPCODES: ClassVar[tuple[int, ...]] = (8,)
+    layer_idx: int
+    tile_M_idx: int
+    tile_N_start_idx: int
+    tile_N_end_idx: int
+    init_shared_out: int = 0
+    tile_M_granularity: int = TILE_M_GRANULARITY
+    tile_N_granularity: int = TILE_N_GRANULARITY
+
+
+@dataclass
+class SharedExpert_DownProj(Instruction):
+    OPCODE: ClassVar[int] = 11
+    PREV_OPCODES: ClassVar[tuple[int, ...]] = (10,)
+    layer_idx: int
+    tile_M_idx: int
+    tile_N_start_idx: int
+    tile_N_end_idx: int
+    split_K_idx: int
+    tile_M_granularity: int = TILE_M_GRANULARITY
+    tile_N_granularity: int = TILE_N_GRANULARITY
+    split_K_granularity: int = SPLIT_K_GRANULARITY_SHARED
+
+
+@dataclass
+class RoutedExpert_UpGate_SiLU(Instruction):
+    """``expert_idx`` is the slot 0..top_k-1; the physical expert is expert_indices[slot] at run time."""
+
+    OPCODE: ClassVar[int] = 12
+    PREV_OPCODES: ClassVar[tuple[int, ...]] = (9,)
+    layer_idx: int
+    expert_idx: int
+    tile_N_start_idx: int
+    tile_N_end_idx: int
+    tile_M_granularity: int = TILE_M_GRANULARITY
+    tile_N_granularity: int = TILE_N_GRANULARITY
+
+
+@dataclass
+class RoutedExpert_DownProj(Instruction):
+    OPCODE: ClassVar[int] = 13
+    PREV_OPCODES: ClassVar[tuple[int, ...]] = (12,)
+    layer_idx: int
+    expert_idx: int
+    tile_M_idx: int
+    tile_N_start_idx: int
+    tile_N_end_idx: int
+    tile_M_granularity: int = TILE_M_GRANULARITY
+    tile_N_granularity: int = TILE_N_GRANULARITY
+
+
+@dataclass
+class MoE_Combine_Commit(Instruction):
+    OPCODE: ClassVar[int] = 14
+    PREV_OPCODES: ClassVar[tuple[int, ...]] = (11, 13)
+    layer_idx: int
+    tile_N_start_idx: int
+    tile_N_end_idx: int
+    tile_N_granularity: int = TILE_N_GRANULARITY
+
+
+INSTRUCTION_BY_OPCODE = {
+    cls.OPCODE: cls
+    for cls in (NoOp, RMS_QKVProj_GEMV_RoPE, DecodeAttentionSplitKV, DecodeAttentionReduction, OProj_GEMV_Residual, RMS_LMHead_GEMV,
+                Router_GEMV, Router_SoftmaxTopK, SharedExpert_UpGate_SiLU, SharedExpert_DownProj, RoutedExpert_UpGate_SiLU,
+                RoutedExpert_DownProj, MoE_Combine_Commit)
+}

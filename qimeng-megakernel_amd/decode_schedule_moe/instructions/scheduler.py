@@ -1,0 +1,140 @@
+"""Scheduler of the MoE decode route: one step's instructions in dependency order, dealt round-robin.
+
+Emission order per layer 1 -> 2 -> 3 -> 4 -> 8 -> 9 -> 10 -> 11 -> 12 -> 13 -> 14, then 7
+(`…/qwen1_5_moe_a2_7b/A100/single_batch/decode_schedule/instructions/scheduler.py:139-370`).
+``sm_count`` is the number of instruction queues: 108 in the reference.
+"""
+from __future__ import annotations
+
+from dataclasses import dataclass
+from typing import Sequence
+
+from ...instruction import Instruction
+from ..model_config import A100_SM_COUNT, MoeShape, QwenMoeConfig, num_partials_for
+from .instruction_defs import (
+    TILE_N_GRANULARITY,
+    DecodeAttentionReduction,
+    DecodeAttentionSplitKV,
+    MoE_Combine_Commit,
+    OProj_GEMV_Residual,
+    RMS_LMHead_GEMV,
+    RMS_QKVProj_GEMV_RoPE,
+    RoutedExpert_DownProj,
+    RoutedExpert_UpGate_SiLU,
+    Router_GEMV,
+    Router_SoftmaxTopK,
+    SharedExpert_DownProj,
+    SharedExpert_UpGate_SiLU,
+)
+
+
+def _ceil_div(a: int, b: int) -> int:
+    return -(-a // b)
+
+
+def _spans(n: int, parts: int) -> list[tuple[int, int]]:
+    """Contiguous, as-even-as-possible cut of n tiles into at most ``parts`` spans."""
+    if n <= 0:
+        return []
+    groups = min(n, parts)
+    small, extra = divmod(n, groups)
+    out, lo = [], 0
+    for g in range(groups):
+        hi = lo + small + (1 if g < extra else 0)
+        out.append((lo, hi))
+        lo = hi
+    return out
+
+
+@dataclass
+class MoeScheduler:
+    shape: MoeShape
+    sm_count: int
+    num_partials: int
+
+    def qkvproj(self, layer: int) -> list[Instruction]:
+        tiles = _ceil_div(self.shape.qkv_out_dim, TILE_N_GRANULARITY)
+        return [RMS_QKVProj_GEMV_RoPE(layer, 0, lo, hi) for lo, hi in _spans(tiles, self.sm_count)]
+
+    def attention_split_kv(self, layer: int) -> list[Instruction]:
+        return [DecodeAttentionSplitKV(layer, kvh, self.num_partials, part)
+                for kvh in range(self.shape.num_key_value_heads) for part in range(self.num_partials)]
+
+    def attention_reduction(self, layer: int) -> list[Instruction]:
+        return [DecodeAttentionReduction(layer, h0, self.num_partials, list(range(self.num_partials)))
+                for h0 in range(0, self.shape.num_attention_heads, self.shape.attn_reduction_size)]
+
+    def oproj(self, layer: int) -> list[Instruction]:
+        return [OProj_GEMV_Residual(layer, 0, lo, hi, 0) for lo, hi in _spans(self.shape.num_hidden_blocks, self.sm_count)]
+
+    def router_gemv(self, layer: int) -> list[Instruction]:
+        """One instruction per expert: the top-k waits for all of them."""
+        e = self.shape.num_experts
+        return [Router_GEMV(layer, lo, hi, 1 if lo == 0 else 0) for lo, hi in _spans(e, e)]
+
+    def router_softmax_topk(self, layer: int) -> list[Instruction]:
+        return [Router_SoftmaxTopK(layer)]
+
+    def shared_upgate(self, layer: int) -> list[Instruction]:
+        tiles = _ceil_div(self.shape.intermediate_size, TILE_N_GRANULARITY)
+        return [SharedExpert_UpGate_SiLU(layer, 0, lo, hi, 1 if lo == 0 else 0) for lo, hi in _spans(tiles, self.sm_count)]
+
+    def shared_downproj(self, layer: int) -> list[Instruction]:
+        """K split into ``num_downproj_split_k_shared`` slices, each with its own share of the queues."""
+        k = self.shape.num_downproj_split_k_shared
+        per_group = max(1, self.sm_count // k)
+        out: list[Instruction] = []
+        for slice_idx in range(k):
+            first = slice_idx * per_group
+            last = min((slice_idx + 1) * per_group, self.sm_count) if slice_idx < k - 1 else self.sm_count
+            for lo, hi in _spans(self.shape.num_hidden_blocks, max(1, last - first)):
+                out.append(SharedExpert_DownProj(layer, 0, lo, hi, slice_idx, split_K_granularity=self.shape.split_k_granularity_shared))
+        return out
+
+    def routed_upgate(self, layer: int) -> list[Instruction]:
+        per_expert = max(1, self.sm_count // self.shape.num_experts_per_tok)
+        return [RoutedExpert_UpGate_SiLU(layer, slot, lo, hi)
+                for slot in range(self.shape.num_experts_per_tok)
+                for lo, hi in _spans(self.shape.num_moe_intermediate_blocks, per_expert)]
+
+    def routed_downproj(self, layer: int) -> list[Instruction]:
+        per_expert = max(1, self.sm_count // self.shape.num_experts_per_tok)
+        return [RoutedExpert_DownProj(layer, slot, 0, lo, hi)
+                for slot in range(self.shape.num_experts_per_tok)
+                for lo, hi in _spans(self.shape.num_hidden_blocks, per_expert)]
+
+    def combine_commit(self, layer: int) -> list[Instruction]:
+        return [MoE_Combine_Commit(layer, lo, hi) for lo, hi in _spans(self.shape.num_hidden_blocks, self.sm_count)]
+
+    def lmhead(self) -> list[Instruction]:
+        tiles = _ceil_div(self.shape.vocab_size, TILE_N_GRANULARITY)
+        return [RMS_LMHead_GEMV(lo, hi) for lo, hi in _spans(tiles, self.sm_count)]
+
+    def layer(self, layer: int) -> list[Instruction]:
+        return (self.qkvproj(layer) + self.attention_split_kv(layer) + self.attention_reduction(layer) + self.oproj(layer)
+                + self.router_gemv(layer) + self.router_softmax_topk(layer) + self.shared_upgate(layer) + self.shared_downproj(layer)
+                + self.routed_upgate(layer) + self.routed_downproj(layer) + self.combine_commit(layer))
+
+    def instruction_list(self, num_layers: int | None = None) -> list[Instruction]:
+        layers = self.shape.num_hidden_layers if num_layers is None else num_layers
+        out: list[Instruction] = []
+        for layer in range(layers):
+            out += self.layer(layer)
+        if layers == self.shape.num_hidden_layers:
+            out += self.lmhead()
+        return out
+
+    def queues(self, num_layers: int | None = None) -> list[list[Instruction]]:
+        return deal(self.instruction_list(num_layers), self.sm_count)
+
+
+def deal(instructions: Sequence[Instruction], queues: int) -> list[list[Instruction]]:
+    out: list[list[Instruction]] = [[] for _ in range(queues)]
+    for i, ins in enumerate(instructions):
+        out[i % queues].append(ins)
+    return out
+
+
+def reference_scheduler(shape: MoeShape | None = None, sm_count: int = A100_SM_COUNT) -> MoeScheduler:
+    shape = shape or QwenMoeConfig.shape()
+    return MoeScheduler(shape, sm_count, num_partials_for(sm_count, shape))

@@ -187,3 +187,76 @@ def build_synthetic_globals(
 def reduced_shape(num_layers: int = 2, vocab_size: int = 2048, **overrides: Any) -> DecodeShape:
     """Llama-3.2-1B layer geometry with fewer layers and a small vocabulary (fast CPU checks)."""
     return dataclasses.replace(LlamaConfig.shape().__class__(), num_hidden_layers=num_layers, vocab_size=vocab_size, **overrides)
+
+
+def random_moe_weights(shape: Any, seed: int, max_positions: int) -> dict[str, torch.Tensor]:
+    """Seeded random-init weights of the MoE route (``decode_schedule_moe.MoeShape``): bf16 ~N(0, 0.02)
+    projections, router and experts (gate rows first in ``expert_gate_up_proj_weights``), QKV bias
+    ~N(0, 0.02), norm weights near one (not all ones: the router and the shared gate read the
+    normalised row directly), untied LM head.  CPU tensors."""
+    gen = torch.Generator(device="cpu")
+    gen.manual_seed(seed)
+    L, H, V = shape.num_hidden_layers, shape.hidden_size, shape.vocab_size
+    F, Fm, E = shape.intermediate_size, shape.moe_intermediate_size, shape.num_experts
+    w: dict[str, torch.Tensor] = {}
+    w["embed_tokens"] = _normal_bf16(gen, V, H)
+    w["qkv_weights"] = torch.stack([_normal_bf16(gen, shape.qkv_out_dim, H) for _ in range(L)])
+    if shape.qkv_bias:
+        w["qkv_bias"] = torch.stack([_normal_bf16(gen, shape.qkv_out_dim) for _ in range(L)])
+    w["o_proj_weights"] = torch.stack([_normal_bf16(gen, H, shape.num_attention_heads * shape.head_dim) for _ in range(L)])
+    w["router_weights"] = torch.stack([_normal_bf16(gen, E, H) for _ in range(L)])
+    w["shared_expert_gate_proj_weights"] = torch.stack([_normal_bf16(gen, F, H) for _ in range(L)])
+    w["shared_expert_up_proj_weights"] = torch.stack([_normal_bf16(gen, F, H) for _ in range(L)])
+    w["shared_expert_down_proj_weights"] = torch.stack([_normal_bf16(gen, H, F) for _ in range(L)])
+    w["shared_expert_gate_weights"] = torch.stack([_normal_bf16(gen, 1, H) for _ in range(L)])
+    w["expert_gate_up_proj_weights"] = torch.stack([torch.stack([_normal_bf16(gen, 2 * Fm, H) for _ in range(E)]) for _ in range(L)])
+    w["expert_down_proj_weights"] = torch.stack([torch.stack([_normal_bf16(gen, H, Fm) for _ in range(E)]) for _ in range(L)])
+    w["lm_head_weights"] = _normal_bf16(gen, V, H)
+    for name, size in (("attn_norm_weights", (L, H)), ("mlp_norm_weights", (L, H)), ("lm_head_norm_weights", (H,))):
+        w[name] = (1.0 + 0.1 * torch.randn(*size, generator=gen, dtype=torch.float32)).to(torch.bfloat16)
+    rope_shape = DecodeShape(head_dim=shape.head_dim, rope_theta=shape.rope_theta)
+    w["rope_cos"], w["rope_sin"] = rope_tables(rope_shape, max_positions)
+    return w
+
+
+def build_moe_globals(weights: dict[str, torch.Tensor], shape: Any, kv_capacity: int, device: torch.device | str, *,
+                      max_partials: int = 27, globals_cls: Any = None) -> Any:
+    """Buffers of the MoE route (`…/qwen1_5_moe_a2_7b/A100/single_batch/decode_schedule/globs.py:79-120`)."""
+    if globals_cls is None:
+        from .decode_schedule_moe.globs import Globals as globals_cls
+    from .decode_schedule_moe.model_config import NUM_OPCODE_ROWS
+
+    device = torch.device(device)
+    bf16 = torch.bfloat16
+    L, H = shape.num_hidden_layers, shape.hidden_size
+    nq, nkv, d, k = shape.num_attention_heads, shape.num_key_value_heads, shape.head_dim, shape.num_experts_per_tok
+
+    def zeros(*size: int, dtype: torch.dtype = bf16) -> torch.Tensor:
+        return torch.zeros(*size, dtype=dtype, device=device)
+
+    on_device = {name: t.to(device).contiguous() for name, t in weights.items()}
+    g = globals_cls(
+        position_id=0,
+        barriers=zeros(L, NUM_OPCODE_ROWS, max(shape.barrier_slots, shape.num_heads), dtype=torch.int32),
+        k_cache=zeros(L, 1, kv_capacity, nkv, d),
+        v_cache=zeros(L, 1, kv_capacity, nkv, d),
+        hidden_states=zeros(H),
+        q_post_rope=zeros(nq * d),
+        attn_out=zeros(nq * d),
+        attn_out_intermediates=zeros(nq, max_partials, d, dtype=torch.float32),
+        attn_lse_intermediates=zeros(nq, max_partials, dtype=torch.float32),
+        router_logits_buf=zeros(shape.num_experts, dtype=torch.float32),
+        normed_hidden_states=zeros(H),
+        shared_expert_silu_out=zeros(shape.intermediate_size),
+        shared_out=zeros(H),
+        routed_out=zeros(H),
+        routed_out_f32=zeros(H, dtype=torch.float32),
+        routed_silu_buffer=zeros(k, shape.moe_intermediate_size),
+        expert_indices=zeros(k, dtype=torch.int64),
+        expert_weights=zeros(k, dtype=torch.float32),
+        silu_out=zeros(shape.moe_intermediate_size),
+        logits=zeros(shape.vocab_size),
+        **{name: t for name, t in on_device.items() if name != "embed_tokens"},
+    )
+    g.embed_tokens = on_device["embed_tokens"]
+    return g
