@@ -35,7 +35,7 @@
 extern "C" {
 #endif
 
-#define QMK_ABI_VERSION 5
+#define QMK_ABI_VERSION 6
 #define QMK_INSTRUCTION_WORDS 32
 
 /* Return / status codes. 0 is success; everything else is an error. */
@@ -58,6 +58,9 @@ enum {
 /* Model shapes compiled into the library. */
 enum {
   QMK_MODEL_LLAMA_3_2_1B = 0,  /* H 2048, F 8192, 32 q / 8 kv heads, d 64 */
+  QMK_MODEL_QWEN1_5_MOE_A2_7B = 2, /* H 2048, 16 q / 16 kv heads, d 128, QKV bias; the MoE op set
+                                  (…/qwen/qwen1_5_moe_a2_7b/A100/single_batch/decode_kernel/mk.h); expert
+                                  count, top-k and FFN widths are launch parameters (qmk_decode_step_moe) */
   QMK_MODEL_QWEN3_1_7B = 1     /* H 2048, F 6144, 16 q / 8 kv heads, d 128, per-head QK RMSNorm
                                   (the Qwen3 op set: …/qwen/qwen3__0_6b/A100/single_batch/
                                   decode_kernel/mk.h, decode_schedule/mk_kernel.py:52-110)     */
@@ -261,6 +264,88 @@ typedef struct QmkBatchArgs {
 /* Launch one step of the batch route asynchronously on args->stream.  Positions outside the KV
  * cache or the RoPE table are found on the device (QMK_DEV_BAD_OPERAND, instruction -1). */
 int qmk_decode_step_batch(const QmkBatchArgs* args);
+
+/*
+ * One decode step of the MoE route at batch 1: opcodes 1-4 and 7 of the dense route (QKV with bias) and
+ * 8-14 (…/qwen1_5_moe_a2_7b/A100/single_batch/decode_schedule/instructions/instruction_defs.py:24-151):
+ * router logits, softmax top-k, shared expert up/gate and K-split down, routed experts up/gate and down,
+ * combine + commit.  Tensors as in mk(...) of that route (decode_schedule/mk_kernel.py:95-205); its three
+ * unused dense-MLP positions have no field here.  Counters [L, >= 15, >= 128].
+ */
+typedef struct QmkMoeArgs {
+  uint32_t struct_size;            /* = sizeof(QmkMoeArgs)                        */
+  uint32_t model;                  /* QMK_MODEL_QWEN1_5_MOE_A2_7B                 */
+  uint32_t flags;                  /* 0 or QMK_FLAG_KEEP_BARRIERS                 */
+  uint32_t spin_limit;
+
+  const int32_t* instructions;     /* int32 [num_queues, num_insts, 32]           */
+  void* hidden_states;             /* bf16 [H]            in/out residual stream  */
+  void* normed_hidden_states;      /* bf16 [H]   RMSNorm row published by opcode 8 */
+  void* q_post_rope;               /* bf16 [Hq*D]                                 */
+  void* k_cache;                   /* bf16 [L, 1, max_seq_len, Hkv, D]            */
+  void* v_cache;
+  void* attn_out;                  /* bf16 [Hq*D]                                 */
+  float* attn_lse_intermediates;   /* f32  [Hq, max_splits]                       */
+  float* attn_out_intermediates;   /* f32  [Hq, max_splits, D]                    */
+  void* silu_out;                  /* bf16 [Fm]  what the last expert slot wrote  */
+  void* logits;                    /* bf16 [vocab_size]                           */
+  const void* attn_norm_weights;   /* bf16 [L, H]                                 */
+  const void* qkv_weights;         /* bf16 [L, (Hq+2Hkv)*D, H]                    */
+  const void* qkv_bias;            /* bf16 [L, (Hq+2Hkv)*D]                       */
+  const float* rope_cos;           /* f32  [rope_rows, D]                         */
+  const float* rope_sin;
+  const void* o_proj_weights;      /* bf16 [L, H, Hq*D]                           */
+  const void* mlp_norm_weights;    /* bf16 [L, H]                                 */
+  const void* lm_head_norm_weights;/* bf16 [H]                                    */
+  const void* lm_head_weights;     /* bf16 [vocab_size, H]                        */
+  const void* router_weights;      /* bf16 [L, E, H]                              */
+  float* router_logits_buf;        /* f32  [E]                                    */
+  int64_t* expert_indices;         /* i64  [top_k]                                */
+  float* expert_weights;           /* f32  [top_k]                                */
+  const void* shared_expert_gate_proj_weights; /* bf16 [L, Fs, H]                 */
+  const void* shared_expert_up_proj_weights;   /* bf16 [L, Fs, H]                 */
+  const void* shared_expert_down_proj_weights; /* bf16 [L, H, Fs]                 */
+  void* shared_expert_silu_out;    /* bf16 [Fs]                                   */
+  void* shared_out;                /* bf16 [H]                                    */
+  const void* shared_expert_gate_weights;      /* bf16 [L, H]  the sigmoid gate   */
+  const void* expert_gate_up_proj_weights;     /* bf16 [L, E, 2*Fm, H], gate rows first */
+  const void* expert_down_proj_weights;        /* bf16 [L, E, H, Fm]              */
+  void* routed_silu_buffer;        /* bf16 [top_k, Fm]                            */
+  float* routed_out_f32;           /* f32  [H]   left cleared, as by the reference */
+  void* routed_out;                /* bf16 [H]   unused by opcodes 8-14 (may be NULL) */
+  int32_t* barriers;               /* int32 [num_layers, num_layer_barriers, barrier_slots] */
+
+  int32_t num_queues;
+  int32_t num_insts;
+  int32_t num_layers;
+  int32_t num_layer_barriers;      /* >= 15                                       */
+  int32_t barrier_slots;           /* >= H/16 and >= Hq + 2 Hkv                   */
+  int32_t max_seq_len;
+  int32_t max_splits;
+  int32_t vocab_size;
+  int32_t rope_rows;
+  int32_t pos_id;
+  int32_t num_experts;             /* E, <= 512                                   */
+  int32_t top_k;                   /* experts per token, <= 8                     */
+  int32_t shared_ffn;              /* Fs, a multiple of 16                        */
+  int32_t moe_ffn;                 /* Fm, a multiple of 16, <= 2048               */
+  int32_t shared_k_slices;         /* K slices of the shared down projection (4 in the reference) */
+  float attn_scale;
+  float rms_norm_eps;
+
+  uint64_t* timeline;
+  void* stream;
+  void* workspace;                 /* qmk_moe_workspace_bytes(top_k, shared_k_slices) bytes, 128-byte aligned: the
+                                      terms of the two in-place accumulations of the reference (shared_out over
+                                      the K slices, routed_out_f32 over the expert slots), one slot per producer,
+                                      added by opcode 14 in the reference VM's order                            */
+  uint64_t workspace_bytes;
+} QmkMoeArgs;
+
+int qmk_decode_step_moe(const QmkMoeArgs* args);
+
+/* Size of QmkMoeArgs.workspace; 0 when an argument is out of range. */
+uint64_t qmk_moe_workspace_bytes(int top_k, int shared_k_slices);
 
 /* Size of QmkArgs.workspace for QMK_FLAG_TAGGED; 0 for an unknown model. */
 uint64_t qmk_workspace_bytes(int model);

@@ -14,6 +14,7 @@
 
 #include "qmk.h"
 #include "qmk_mb_ops.h"
+#include "qmk_moe_ops.h"
 #include "qmk_ops.h"
 
 namespace qmk {
@@ -241,11 +242,97 @@ __global__ __launch_bounds__(kThreads, 1) void decode_megakernel_batch(const Par
   }
 }
 
+// The MoE route's interpreter: the dense route's attention and LM head (opcodes 1-4, 7) and the MoE
+// block (8-14) on the reference's counters (…/qwen1_5_moe_a2_7b/A100/single_batch/decode_kernel/mk.cu).
+template <class M>
+__global__ __launch_bounds__(kThreads, 1) void decode_megakernel_moe(const Params p) {
+  __shared__ Smem<M> s;
+  if (threadIdx.x < 8) s.ctl[threadIdx.x] = 0;
+  if (threadIdx.x == 0) {
+    s.generation = 0u;
+    s.best_val = -INFINITY;
+    s.best_idx = 0x7fffffff;
+  }
+  __syncthreads();
+  const int32_t* queue = p.instructions + static_cast<size_t>(blockIdx.x) * p.num_insts * kInstWords;
+  bool ok = true;
+  int32_t word = (threadIdx.x < kInstWords && p.num_insts > 0) ? queue[threadIdx.x] : 0;
+  int32_t word1 = (threadIdx.x < kInstWords && p.num_insts > 1) ? queue[kInstWords + threadIdx.x] : 0;
+  Carried carry;
+  forget(carry);
+  for (int i = 0; i < p.num_insts && ok; ++i) {
+    if (threadIdx.x < kInstWords) {
+      s.inst[threadIdx.x] = word;
+      s.next[threadIdx.x] = word1;
+      word = word1;
+      word1 = (i + 2 < p.num_insts) ? queue[(i + 2) * kInstWords + threadIdx.x] : 0;
+    }
+    __syncthreads();
+    const int opcode = s.inst[0];
+    int tid = threadIdx.x;
+    asm volatile("" : "+v"(tid));
+    const Ctx c{i, opcode, tid};
+    unsigned long long t_start = 0;
+    if (p.timeline != nullptr && threadIdx.x == 0) {
+      t_start = wall_clock64();
+      for (int k = 0; k < 4; ++k) s.stamps[k] = t_start;
+    }
+    bool carried = false;
+    switch (opcode) {
+      case OP_NOOP: break;
+      case OP_RMS_QKV_ROPE: ok = op_rms_qkv_rope<M>(p, s, c); break;
+      case OP_ATTN_SPLITKV: ok = op_attn_splitkv<M>(p, s, c); break;
+      case OP_ATTN_REDUCE: ok = op_attn_reduce<M>(p, s, c); break;
+      case OP_OPROJ_RESIDUAL: ok = op_oproj_residual<M>(p, s, c, carry, carried); break;
+      case OP_RMS_LMHEAD: ok = op_rms_lmhead<M>(p, s, c); break;
+      case moe::OP_ROUTER: ok = moe::op_router<M>(p, s, c); break;
+      case moe::OP_TOPK: ok = moe::op_topk<M>(p, s, c); break;
+      case moe::OP_SHARED_UPGATE: ok = moe::op_shared_upgate<M>(p, s, c); break;
+      case moe::OP_SHARED_DOWN: ok = moe::op_shared_down<M>(p, s, c); break;
+      case moe::OP_ROUTED_UPGATE: ok = moe::op_routed_upgate<M>(p, s, c); break;
+      case moe::OP_ROUTED_DOWN: ok = moe::op_routed_down<M>(p, s, c); break;
+      case moe::OP_COMBINE: ok = moe::op_combine<M>(p, s, c); break;
+      default:
+        if (threadIdx.x == 0) report_error(p, QMK_DEV_BAD_OPCODE, i, opcode, 0);
+        ok = false;
+        break;
+    }
+    forget(carry);
+    if (p.timeline != nullptr && threadIdx.x == 0) {
+      uint64_t* rec = p.timeline + (static_cast<size_t>(blockIdx.x) * p.num_insts + i) * 8;
+      rec[0] = t_start;
+      rec[1] = s.ctl[2] ? s.t_wait : t_start;
+      rec[2] = wall_clock64();
+      rec[3] = static_cast<uint64_t>(opcode) | (static_cast<uint64_t>(static_cast<uint32_t>(s.inst[1])) << 8);
+      for (int k = 0; k < 4; ++k) rec[4 + k] = s.stamps[k];
+      s.ctl[2] = 0;
+    }
+    __syncthreads();
+  }
+  if (!ok || (p.flags & QMK_FLAG_KEEP_BARRIERS)) return;
+  // Retire: the last workgroup clears the counters (arrival counter: last word of layer 0's last row, which
+  // is row 14 and carries no counter of the protocol).
+  release_stores();
+  __syncthreads();
+  int32_t* done = counter_ptr(p, 0, p.num_layer_barriers - 1, p.barrier_slots - 1);
+  if (threadIdx.x == 0) {
+    const int prev = __hip_atomic_fetch_add(done, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    s.ctl[1] = (prev == static_cast<int>(gridDim.x) - 1);
+  }
+  __syncthreads();
+  if (s.ctl[1]) {
+    const int total = p.num_layers * p.num_layer_barriers * p.barrier_slots;
+    for (int i = threadIdx.x; i < total; i += kThreads)
+      __hip_atomic_store(p.barriers + i, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  }
+}
+
 struct DeviceInfo {
   bool ready = false;
   int cu_count = 0;
   int max_queues = 0;
   int max_queues_batch = 0;
+  int max_queues_moe = 0;
   int32_t* status = nullptr;
 };
 DeviceInfo g_devices[kMaxDevices];
@@ -265,12 +352,16 @@ int device_info(DeviceInfo** out) {
     int per_cu_batch = 0;
     if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu_batch, decode_megakernel_batch<Llama1B>, kThreads, 0) != hipSuccess)
       return QMK_ERR_NO_DEVICE;
+    int per_cu_moe = 0;
+    if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu_moe, decode_megakernel_moe<QwenMoeA2_7B>, kThreads, 0) != hipSuccess)
+      return QMK_ERR_NO_DEVICE;
     void* sym = nullptr;
     if (hipGetSymbolAddress(&sym, HIP_SYMBOL(g_status)) != hipSuccess) return QMK_ERR_NO_DEVICE;
     if (hipMemset(sym, 0, sizeof(int32_t) * kStatusWords) != hipSuccess) return QMK_ERR_NO_DEVICE;
     d.cu_count = prop.multiProcessorCount;
     d.max_queues = per_cu * prop.multiProcessorCount;
     d.max_queues_batch = per_cu_batch * prop.multiProcessorCount;
+    d.max_queues_moe = per_cu_moe * prop.multiProcessorCount;
     d.status = static_cast<int32_t*>(sym);
     d.ready = true;
   }
@@ -465,6 +556,112 @@ extern "C" int qmk_decode_step_batch(const QmkBatchArgs* a) {
   p.rope_rows = a->rope_rows;
 
   hipLaunchKernelGGL(decode_megakernel_batch<M>, dim3(a->num_queues), dim3(kThreads), 0, static_cast<hipStream_t>(a->stream), p);
+  return hipGetLastError() == hipSuccess ? QMK_OK : QMK_ERR_LAUNCH;
+}
+
+extern "C" uint64_t qmk_moe_workspace_bytes(int top_k, int shared_k_slices) {
+  if (top_k < 1 || top_k > moe::kMaxTopK || shared_k_slices < 0 || shared_k_slices > 16) return 0;
+  const uint64_t shared = static_cast<uint64_t>(shared_k_slices) * QwenMoeA2_7B::H * sizeof(u16);
+  return ((shared + 127) / 128) * 128 + static_cast<uint64_t>(top_k) * QwenMoeA2_7B::H * sizeof(float);
+}
+
+extern "C" int qmk_decode_step_moe(const QmkMoeArgs* a) {
+  using M = QwenMoeA2_7B;
+  if (a == nullptr) return QMK_ERR_NULL_ARG;
+  if (a->struct_size != sizeof(QmkMoeArgs)) return QMK_ERR_ABI;
+  if (a->model != QMK_MODEL_QWEN1_5_MOE_A2_7B) return QMK_ERR_MODEL;
+  const void* required[] = {a->instructions, a->hidden_states, a->normed_hidden_states, a->q_post_rope, a->k_cache, a->v_cache,
+                            a->attn_out, a->attn_lse_intermediates, a->attn_out_intermediates, a->silu_out, a->logits,
+                            a->attn_norm_weights, a->qkv_weights, a->qkv_bias, a->rope_cos, a->rope_sin, a->o_proj_weights,
+                            a->mlp_norm_weights, a->lm_head_norm_weights, a->lm_head_weights, a->router_weights,
+                            a->router_logits_buf, a->expert_indices, a->expert_weights, a->shared_expert_gate_proj_weights,
+                            a->shared_expert_up_proj_weights, a->shared_expert_down_proj_weights, a->shared_expert_silu_out,
+                            a->shared_out, a->shared_expert_gate_weights, a->expert_gate_up_proj_weights,
+                            a->expert_down_proj_weights, a->routed_silu_buffer, a->routed_out_f32, a->barriers, a->workspace};
+  for (const void* ptr : required)
+    if (ptr == nullptr) return QMK_ERR_NULL_ARG;
+  if (a->num_queues < 1 || a->num_insts < 0 || a->num_layers < 1 || a->num_layer_barriers < 15 ||
+      a->barrier_slots < M::H / 16 || a->barrier_slots < M::NQ + 2 * M::NKV || a->max_seq_len < 1 || a->max_splits < 1 ||
+      a->vocab_size < 1 || a->rope_rows < 1)
+    return QMK_ERR_SHAPE;
+  if (a->num_experts < 1 || a->num_experts > moe::kMaxExperts || a->top_k < 1 || a->top_k > moe::kMaxTopK || a->top_k > a->num_experts ||
+      a->shared_ffn < 16 || a->shared_ffn % 16 || a->moe_ffn < 16 || a->moe_ffn % 16 || a->moe_ffn > moe::kMaxK ||
+      a->shared_k_slices < 1 || a->shared_k_slices > 16)
+    return QMK_ERR_SHAPE;
+  if (a->flags & ~QMK_FLAG_KEEP_BARRIERS) return QMK_ERR_SHAPE;
+  if (a->pos_id < 0 || a->pos_id >= a->max_seq_len || a->pos_id >= a->rope_rows) return QMK_ERR_POSITION;
+  if (reinterpret_cast<uintptr_t>(a->workspace) % 128 != 0 || a->workspace_bytes < qmk_moe_workspace_bytes(a->top_k, a->shared_k_slices))
+    return QMK_ERR_SHAPE;
+
+  DeviceInfo* dev = nullptr;
+  if (int rc = device_info(&dev); rc != QMK_OK) return rc;
+  if (a->num_queues > dev->max_queues_moe) return QMK_ERR_TOO_MANY_QUEUES;
+  if (a->num_insts == 0) return QMK_OK;
+
+  Params p{};
+  p.instructions = a->instructions;
+  p.hidden = static_cast<u16*>(a->hidden_states);
+  p.q_post_rope = static_cast<u16*>(a->q_post_rope);
+  p.k_cache = static_cast<u16*>(a->k_cache);
+  p.v_cache = static_cast<u16*>(a->v_cache);
+  p.attn_out = static_cast<u16*>(a->attn_out);
+  p.attn_lse = a->attn_lse_intermediates;
+  p.attn_partial = a->attn_out_intermediates;
+  p.silu_out = static_cast<u16*>(a->silu_out);
+  p.logits = static_cast<u16*>(a->logits);
+  p.attn_norm = static_cast<const u16*>(a->attn_norm_weights);
+  p.qkv_w = static_cast<const u16*>(a->qkv_weights);
+  p.qkv_bias = static_cast<const u16*>(a->qkv_bias);
+  p.rope_cos = a->rope_cos;
+  p.rope_sin = a->rope_sin;
+  p.o_w = static_cast<const u16*>(a->o_proj_weights);
+  p.mlp_norm = static_cast<const u16*>(a->mlp_norm_weights);
+  p.lm_norm = static_cast<const u16*>(a->lm_head_norm_weights);
+  p.lm_w = static_cast<const u16*>(a->lm_head_weights);
+  p.barriers = a->barriers;
+  p.timeline = a->timeline;
+  p.status = dev->status;
+  p.num_insts = a->num_insts;
+  p.num_layers = a->num_layers;
+  p.num_layer_barriers = a->num_layer_barriers;
+  p.barrier_slots = a->barrier_slots;
+  p.max_seq_len = a->max_seq_len;
+  p.max_splits = a->max_splits;
+  p.vocab_size = a->vocab_size;
+  p.pos_id = a->pos_id;
+  p.attn_scale = a->attn_scale;
+  p.rms_norm_eps = a->rms_norm_eps;
+  p.qkv_blocks_per_head = M::D / 16;
+  p.oproj_blocks = M::H / 16;
+  p.down_arrivals = M::H / 16;           // what completes a layer here: the combine step's tiles
+  p.spin_limit = a->spin_limit > 0 ? a->spin_limit : kDefaultSpinLimit;
+  p.flags = a->flags;
+  p.router_w = static_cast<const u16*>(a->router_weights);
+  p.router_logits = a->router_logits_buf;
+  p.expert_indices = reinterpret_cast<long long*>(a->expert_indices);
+  p.expert_weights = a->expert_weights;
+  p.normed_hidden = static_cast<u16*>(a->normed_hidden_states);
+  p.shared_gate_w = static_cast<const u16*>(a->shared_expert_gate_proj_weights);
+  p.shared_up_w = static_cast<const u16*>(a->shared_expert_up_proj_weights);
+  p.shared_down_w = static_cast<const u16*>(a->shared_expert_down_proj_weights);
+  p.shared_scale_w = static_cast<const u16*>(a->shared_expert_gate_weights);
+  p.shared_silu = static_cast<u16*>(a->shared_expert_silu_out);
+  p.shared_out = static_cast<u16*>(a->shared_out);
+  p.expert_gate_up_w = static_cast<const u16*>(a->expert_gate_up_proj_weights);
+  p.expert_down_w = static_cast<const u16*>(a->expert_down_proj_weights);
+  p.routed_silu = static_cast<u16*>(a->routed_silu_buffer);
+  p.routed_out_f32 = a->routed_out_f32;
+  p.routed_out = static_cast<u16*>(a->routed_out);
+  p.shared_parts = static_cast<u16*>(a->workspace);
+  const uint64_t shared_bytes = ((static_cast<uint64_t>(a->shared_k_slices) * M::H * sizeof(u16) + 127) / 128) * 128;
+  p.routed_parts = reinterpret_cast<float*>(static_cast<char*>(a->workspace) + shared_bytes);
+  p.num_experts = a->num_experts;
+  p.top_k = a->top_k;
+  p.shared_ffn = a->shared_ffn;
+  p.moe_ffn = a->moe_ffn;
+  p.shared_k_slices = a->shared_k_slices;
+
+  hipLaunchKernelGGL(decode_megakernel_moe<M>, dim3(a->num_queues), dim3(kThreads), 0, static_cast<hipStream_t>(a->stream), p);
   return hipGetLastError() == hipSuccess ? QMK_OK : QMK_ERR_LAUNCH;
 }
 

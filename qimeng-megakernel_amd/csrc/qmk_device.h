@@ -91,6 +91,31 @@ struct Params {
   u16* mlp_rms_out;
   u16* lm_rms_out;
   int32_t rope_rows;
+  // MoE route only.
+  const u16* qkv_bias;           // [L, QKV]
+  const u16* router_w;           // [L, E, H]
+  float* router_logits;          // [E]
+  long long* expert_indices;     // [top_k]
+  float* expert_weights;         // [top_k]
+  u16* normed_hidden;            // [H]
+  const u16* shared_gate_w;      // [L, Fs, H]
+  const u16* shared_up_w;        // [L, Fs, H]
+  const u16* shared_down_w;      // [L, H, Fs]
+  const u16* shared_scale_w;     // [L, H]: the shared expert's sigmoid gate
+  u16* shared_silu;              // [Fs]
+  u16* shared_out;               // [H]
+  const u16* expert_gate_up_w;   // [L, E, 2 Fm, H], gate rows first
+  const u16* expert_down_w;      // [L, E, H, Fm]
+  u16* routed_silu;              // [top_k, Fm]
+  float* routed_out_f32;         // [H]
+  u16* routed_out;               // [H]
+  u16* shared_parts;             // workspace: [K slices, H] bf16 partial sums of the shared down projection
+  float* routed_parts;           // workspace: [top_k, H] weighted contributions of the routed experts
+  int32_t num_experts;
+  int32_t top_k;
+  int32_t shared_ffn;            // Fs
+  int32_t moe_ffn;               // Fm
+  int32_t shared_k_slices;
 };
 
 // ---------------------------------------------------------------- bf16 ----

@@ -1,0 +1,377 @@
+// Opcodes 8-14 of the MoE decode route (batch 1) as workgroup-wide device functions for gfx950, and
+// the layer geometry they are compiled for.  Opcodes 1-4 and 7 are the dense route's (qmk_ops.h), with
+// the QKV bias added in the projection's epilogue.
+//
+// Semantics follow the reference's instruction VM, which is also what its kernel does
+// (qimeng_megakernel/models/LLM/qwen/qwen1_5_moe_a2_7b/A100/single_batch/decode_schedule/instructions/
+// python_vm.py:331-530; decode_kernel/router_softmax_topk.cu, moe_combine_commit.cu): fp32 router logits,
+// softmax and top-k without renormalisation; silu(gate)*up evaluated in fp32 on the bf16-rounded GEMV
+// results with one rounding; the shared down projection split along K with bf16 partial sums; routed
+// contributions bf16(dot) * weight in fp32; hidden = bf16(hidden + routed + sigmoid(gate) * shared).
+//
+// Where the VM accumulates in place (shared_out over the K slices, routed_out_f32 over the expert
+// slots), concurrent workgroups would add in arrival order, and neither bf16 nor fp32 addition is
+// associative.  Here every producer leaves its term in a slot of its own in the caller's workspace and
+// the combine step adds the terms in the VM's order: same bits as the VM, every run.
+#pragma once
+
+#include "qmk_ops.h"
+
+namespace qmk {
+
+// Qwen1.5-MoE-A2.7B layer geometry.  Expert count, top-k and the two FFN widths are launch parameters.
+struct QwenMoeA2_7B {
+  static constexpr int H = 2048;
+  static constexpr int F = 8192;      // size of the LDS activation vector: >= every FFN width and H
+  static constexpr int D = 128;
+  static constexpr int NQ = 16;
+  static constexpr int NKV = 16;
+  static constexpr int GQA = NQ / NKV;
+  static constexpr int QKV = (NQ + 2 * NKV) * D;
+  static constexpr int KV_BLOCK = 16;
+  static constexpr int CARRY_ROWS = 0;
+  static constexpr bool CARRY_AFTER_ATTENTION = false;
+  static constexpr bool QK_NORM = false;
+  static constexpr bool QKV_BIAS = true;
+  static constexpr int REDUCE_HEADS = 4;   // attn_reduction_size of the route (model_config.py:27)
+  static constexpr int PREV_ROW = 13;      // a layer is complete when its combine step is
+};
+
+namespace moe {
+
+enum Opcode {
+  OP_ROUTER = 8,
+  OP_TOPK = 9,
+  OP_SHARED_UPGATE = 10,
+  OP_SHARED_DOWN = 11,
+  OP_ROUTED_UPGATE = 12,
+  OP_ROUTED_DOWN = 13,
+  OP_COMBINE = 14,
+};
+constexpr int ROW_ROUTER = 7, ROW_TOPK = 8, ROW_SHARED_UPGATE = 9, ROW_SHARED_DOWN = 10, ROW_ROUTED_UPGATE = 11, ROW_ROUTED_DOWN = 12,
+              ROW_COMBINE = 13;
+constexpr int kMaxK = 2048;       // longest dot product of these ops (a K slice, an expert's FFN width, H)
+constexpr int kMaxExperts = 512;
+constexpr int kMaxTopK = 8;
+constexpr int kTile = 16;
+
+// NR weight rows against the bf16 vector x in LDS, K (a multiple of 8, <= kMaxK) columns each: all
+// 16-byte pieces of all rows are requested before the first is used.  Every lane gets the sums.
+template <int NR>
+__device__ __forceinline__ void rows_dot(const u16* const (&rows)[NR], const u16* x, int K, int lane, float (&out)[NR]) {
+  constexpr int NI = kMaxK / 512;
+  v4u w[NR][NI];
+#pragma unroll
+  for (int r = 0; r < NR; ++r)
+#pragma unroll
+    for (int i = 0; i < NI; ++i) {
+      const int col = lane * 8 + i * 512;
+      w[r][i] = v4u{0, 0, 0, 0};
+      if (col < K) w[r][i] = __builtin_nontemporal_load(reinterpret_cast<const v4u*>(rows[r] + col));
+    }
+#pragma unroll
+  for (int r = 0; r < NR; ++r) {
+    float a = 0.f;
+#pragma unroll
+    for (int i = 0; i < NI; ++i) {
+      const int col = lane * 8 + i * 512;
+      if (col < K) a = dot8(w[r][i], *reinterpret_cast<const v4u*>(x + col), a);
+    }
+    out[r] = wave_sum(a);
+  }
+}
+
+// n bf16 elements (a multiple of 4) of a vector that another workgroup wrote during this launch, into s.x.
+template <class M>
+__device__ __forceinline__ void stage_vector(Smem<M>& s, const Ctx& c, const u16* src, int n) {
+  for (int i = c.tid * 4; i < n; i += kThreads * 4) *reinterpret_cast<uint64_t*>(s.x + i) = ld_shared64(src + i);
+  __syncthreads();
+}
+
+template <class M>
+__device__ __forceinline__ bool wait_one(const Params& p, Smem<M>& s, const Ctx& c, int layer, int row, int slot, int expected) {
+  return wg_wait(p, s, c, 1, [&](int) { return counter_ptr(p, layer, row, slot); }, expected);
+}
+
+__device__ __forceinline__ void publish_done(const Params& p, const Ctx& c, int layer, int row, int slot, int amount) {
+  release_stores();
+  __syncthreads();
+  if (c.tid == 0) publish(counter_ptr(p, layer, row, slot), amount);
+}
+
+// ===================================================================== 8 ==
+// [8, layer, e_start, e_end, write_normed_hidden, tile_N_g]
+// RMSNorm of the residual stream, fp32 router logits of experts [e_start, e_end); one instruction of a
+// layer also publishes the normalised row for opcodes 10, 12 and 14   (python_vm.py:331-357).
+template <class M>
+__device__ bool op_router(const Params& p, Smem<M>& s, const Ctx& c) {
+  const int layer = s.inst[1], g = s.inst[5], e0 = s.inst[2] * g, e1 = min(s.inst[3] * g, p.num_experts);
+  if (layer < 0 || layer >= p.num_layers) return bad_operand(p, s, c, 1);
+  if (g < 1 || e0 < 0 || e1 < e0) return bad_operand(p, s, c, 2);
+  if (!wait_one(p, s, c, layer, ROW_OPROJ, 0, p.oproj_blocks)) return false;
+  if (!rms_to_lds<M>(p, s, c, nullptr, 0u, p.mlp_norm + static_cast<size_t>(layer) * M::H)) return false;
+  const int lane = c.tid & 63, wave = c.tid >> 6;
+  const u16* w = p.router_w + static_cast<size_t>(layer) * p.num_experts * M::H;
+  for (int e = e0 + wave; e < e1; e += kWaves) {
+    const u16* const rows[1] = {w + static_cast<size_t>(e) * M::H};
+    float v[1];
+    rows_dot<1>(rows, s.x, M::H, lane, v);
+    if (lane == 0) st_shared_f32(p.router_logits + e, v[0]);
+  }
+  const bool publish_row = s.inst[4] != 0;
+  if (publish_row)
+    for (int i = c.tid * 2; i < M::H; i += kThreads * 2) st_shared32(p.normed_hidden + i, *reinterpret_cast<const uint32_t*>(s.x + i));
+  release_stores();
+  __syncthreads();
+  if (c.tid == 0) {
+    publish(counter_ptr(p, layer, ROW_ROUTER, 0), e1 - e0);
+    if (publish_row) publish(counter_ptr(p, layer, ROW_ROUTER, 1), 1);
+  }
+  return true;
+}
+
+// ===================================================================== 9 ==
+// [9, layer]   softmax over all router logits, the top_k largest probabilities and their experts, in
+// decreasing order (ties: the lower expert first), not renormalised   (python_vm.py:360-372).
+template <class M>
+__device__ bool op_topk(const Params& p, Smem<M>& s, const Ctx& c) {
+  const int layer = s.inst[1], E = p.num_experts;
+  if (layer < 0 || layer >= p.num_layers) return bad_operand(p, s, c, 1);
+  if (!wait_one(p, s, c, layer, ROW_ROUTER, 0, E)) return false;
+  for (int e = c.tid; e < E; e += kThreads) s.res[e] = ld_shared_f32(p.router_logits + e);
+  __syncthreads();
+  if (c.tid < kWaveSize) {
+    const int lane = c.tid;
+    float mx = -INFINITY;
+    for (int e = lane; e < E; e += kWaveSize) mx = fmaxf(mx, s.res[e]);
+    mx = wave_max(mx);
+    float sum = 0.f;
+    for (int e = lane; e < E; e += kWaveSize) {
+      const float x = expf(s.res[e] - mx);
+      s.res[e] = x;
+      sum += x;
+    }
+    sum = wave_sum(sum);
+    for (int j = 0; j < p.top_k; ++j) {
+      float best = -1.f;
+      int idx = 0x7fffffff;
+      for (int e = lane; e < E; e += kWaveSize)
+        if (s.res[e] > best) best = s.res[e], idx = e;   // ascending e: the first of equals stays
+      for (int off = 1; off < kWaveSize; off <<= 1) {
+        const float ob = __shfl_xor(best, off);
+        const int oi = __shfl_xor(idx, off);
+        if (ob > best || (ob == best && oi < idx)) best = ob, idx = oi;
+      }
+      if (lane == 0) {
+        __hip_atomic_store(p.expert_indices + j, static_cast<long long>(idx), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        st_shared_f32(p.expert_weights + j, best / sum);
+        s.res[idx] = -2.f;   // taken
+      }
+      __builtin_amdgcn_wave_barrier();
+    }
+  }
+  release_stores();
+  __syncthreads();
+  if (c.tid == 0) __hip_atomic_store(counter_ptr(p, layer, ROW_TOPK, 0), 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  return true;
+}
+
+// Gate and up rows [r0, r0 + n) of one FFN against the normalised row in s.x; out[i] =
+// bf16(silu(bf16(gate . x)) * bf16(up . x)), silu and the product in fp32 (python_vm.py:389-395, 455-459).
+// The results wait in s.res; two neighbouring ones leave as one word to every destination given.
+template <class M>
+__device__ __forceinline__ void upgate_rows(Smem<M>& s, const Ctx& c, const u16* gate_w, const u16* up_w, int r0, int n, u16* dst0, u16* dst1) {
+  const int lane = c.tid & 63, wave = c.tid >> 6;
+  for (int i = wave; i < n; i += 2 * kWaves) {
+    const int j = min(i + kWaves, n - 1);   // second output of this pass (repeats the first one's neighbour at the end)
+    const u16* const rows[4] = {gate_w + static_cast<size_t>(r0 + i) * M::H, up_w + static_cast<size_t>(r0 + i) * M::H,
+                                gate_w + static_cast<size_t>(r0 + j) * M::H, up_w + static_cast<size_t>(r0 + j) * M::H};
+    float v[4];
+    rows_dot<4>(rows, s.x, M::H, lane, v);
+    if (lane == 0) {
+      const float g0 = round_bf16(v[0]), g1 = round_bf16(v[2]);
+      s.res[i] = (g0 / (1.0f + expf(-g0))) * round_bf16(v[1]);
+      if (i + kWaves < n) s.res[i + kWaves] = (g1 / (1.0f + expf(-g1))) * round_bf16(v[3]);
+    }
+  }
+  __syncthreads();
+  for (int pair = c.tid; pair < n / 2; pair += kThreads) {
+    const uint32_t word = static_cast<uint32_t>(f2bf(s.res[2 * pair])) | (static_cast<uint32_t>(f2bf(s.res[2 * pair + 1])) << 16);
+    st_shared32(dst0 + r0 + 2 * pair, word);
+    if (dst1 != nullptr) st_shared32(dst1 + r0 + 2 * pair, word);
+  }
+}
+
+// ==================================================================== 10 ==
+// [10, layer, tile_M, n_start, n_end, init_shared_out, tile_M_g, tile_N_g]   (python_vm.py:375-396)
+// shared_out needs no clearing here: its K-slice terms have slots of their own until the combine step.
+template <class M>
+__device__ bool op_shared_upgate(const Params& p, Smem<M>& s, const Ctx& c) {
+  const int layer = s.inst[1], n0 = s.inst[3], n1 = s.inst[4], tile = s.inst[7];
+  if (layer < 0 || layer >= p.num_layers) return bad_operand(p, s, c, 1);
+  if (tile != kTile || n0 < 0 || n1 < n0 || n1 * tile > p.shared_ffn || (n1 - n0) * tile > kResSlots) return bad_operand(p, s, c, 4);
+  if (!wait_one(p, s, c, layer, ROW_ROUTER, 1, 1)) return false;
+  stage_vector(s, c, p.normed_hidden, M::H);
+  const size_t base = static_cast<size_t>(layer) * p.shared_ffn * M::H;
+  upgate_rows(s, c, p.shared_gate_w + base, p.shared_up_w + base, n0 * tile, (n1 - n0) * tile, p.shared_silu, nullptr);
+  publish_done(p, c, layer, ROW_SHARED_UPGATE, 0, n1 - n0);
+  return true;
+}
+
+// Rows [r0, r0 + n) of a down projection with K columns (row stride ld) against s.x[0..K); `leave(r, dot)`
+// runs on lane 0 of the wave that owns row r.
+template <class M, class Leave>
+__device__ __forceinline__ void down_rows(Smem<M>& s, const Ctx& c, const u16* w, size_t ld, int K, int r0, int n, Leave leave) {
+  const int lane = c.tid & 63, wave = c.tid >> 6;
+  for (int i = wave; i < n; i += 4 * kWaves) {
+    int r[4];
+    const u16* rows[4];
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+      r[k] = min(i + k * kWaves, n - 1);
+      rows[k] = w + static_cast<size_t>(r0 + r[k]) * ld;
+    }
+    float v[4];
+    rows_dot<4>(rows, s.x, K, lane, v);
+    if (lane == 0) {
+#pragma unroll
+      for (int k = 0; k < 4; ++k)
+        if (i + k * kWaves < n) leave(r0 + r[k], v[k]);
+    }
+  }
+}
+
+// ==================================================================== 11 ==
+// [11, layer, tile_M, n_start, n_end, split_K_idx, tile_M_g, tile_N_g, split_K_g]   (python_vm.py:399-418)
+// One K slice of the shared down projection: bf16(W[r, k0:k1] . silu[k0:k1]) into this slice's slot.
+template <class M>
+__device__ bool op_shared_down(const Params& p, Smem<M>& s, const Ctx& c) {
+  const int layer = s.inst[1], n0 = s.inst[3], n1 = s.inst[4], slice = s.inst[5], tile = s.inst[7], kg = s.inst[8];
+  if (layer < 0 || layer >= p.num_layers) return bad_operand(p, s, c, 1);
+  if (tile != kTile || n0 < 0 || n1 < n0 || n1 * tile > M::H) return bad_operand(p, s, c, 4);
+  if (slice < 0 || slice >= p.shared_k_slices || kg < 8 || (kg & 7) || kg > kMaxK || slice * kg >= p.shared_ffn) return bad_operand(p, s, c, 5);
+  if (!wait_one(p, s, c, layer, ROW_SHARED_UPGATE, 0, p.shared_ffn / kTile)) return false;
+  const int k0 = slice * kg, K = min(kg, p.shared_ffn - k0);
+  stage_vector(s, c, p.shared_silu + k0, K);
+  const u16* w = p.shared_down_w + static_cast<size_t>(layer) * M::H * p.shared_ffn + k0;
+  u16* mine = p.shared_parts + static_cast<size_t>(slice) * M::H;
+  down_rows(s, c, w, p.shared_ffn, K, n0 * tile, (n1 - n0) * tile, [&](int r, float dot) { s.res[r - n0 * tile] = dot; });
+  __syncthreads();
+  for (int pair = c.tid; pair < (n1 - n0) * tile / 2; pair += kThreads)
+    st_shared32(mine + n0 * tile + 2 * pair,
+                static_cast<uint32_t>(f2bf(s.res[2 * pair])) | (static_cast<uint32_t>(f2bf(s.res[2 * pair + 1])) << 16));
+  release_stores();
+  __syncthreads();
+  if (c.tid < n1 - n0) publish(counter_ptr(p, layer, ROW_SHARED_DOWN, n0 + c.tid), 1);
+  return true;
+}
+
+// The physical expert of a slot, read after the top-k edge; negative when it is not one.
+__device__ __forceinline__ int expert_of(const Params& p, int slot) {
+  const long long e = __hip_atomic_load(p.expert_indices + slot, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  return (e >= 0 && e < p.num_experts) ? static_cast<int>(e) : -1;
+}
+
+// ==================================================================== 12 ==
+// [12, layer, expert_slot, n_start, n_end, tile_M_g, tile_N_g]   (python_vm.py:421-464)
+// The single buffer silu_out keeps what the last slot wrote, as after the VM's sequential run.
+template <class M>
+__device__ bool op_routed_upgate(const Params& p, Smem<M>& s, const Ctx& c) {
+  const int layer = s.inst[1], slot = s.inst[2], n0 = s.inst[3], n1 = s.inst[4], tile = s.inst[6];
+  if (layer < 0 || layer >= p.num_layers) return bad_operand(p, s, c, 1);
+  if (slot < 0 || slot >= p.top_k) return bad_operand(p, s, c, 2);
+  if (tile != kTile || n0 < 0 || n1 < n0 || n1 * tile > p.moe_ffn || (n1 - n0) * tile > kResSlots) return bad_operand(p, s, c, 4);
+  if (!wait_one(p, s, c, layer, ROW_TOPK, 0, 1)) return false;
+  const int eid = expert_of(p, slot);
+  if (eid < 0) return bad_operand(p, s, c, 2);
+  stage_vector(s, c, p.normed_hidden, M::H);
+  const u16* w = p.expert_gate_up_w + (static_cast<size_t>(layer) * p.num_experts + eid) * 2 * p.moe_ffn * M::H;
+  upgate_rows(s, c, w, w + static_cast<size_t>(p.moe_ffn) * M::H, n0 * tile, (n1 - n0) * tile,
+              p.routed_silu + static_cast<size_t>(slot) * p.moe_ffn, slot == p.top_k - 1 ? p.silu_out : nullptr);
+  publish_done(p, c, layer, ROW_ROUTED_UPGATE, 0, n1 - n0);
+  return true;
+}
+
+// ==================================================================== 13 ==
+// [13, layer, expert_slot, tile_M, n_start, n_end, tile_M_g, tile_N_g]   (python_vm.py:467-489)
+// bf16(W_down[expert][r] . silu[slot]) * weight[slot], fp32, into the slot's own row of the workspace.
+template <class M>
+__device__ bool op_routed_down(const Params& p, Smem<M>& s, const Ctx& c) {
+  const int layer = s.inst[1], slot = s.inst[2], n0 = s.inst[4], n1 = s.inst[5], tile = s.inst[7];
+  if (layer < 0 || layer >= p.num_layers) return bad_operand(p, s, c, 1);
+  if (slot < 0 || slot >= p.top_k) return bad_operand(p, s, c, 2);
+  if (tile != kTile || n0 < 0 || n1 < n0 || n1 * tile > M::H) return bad_operand(p, s, c, 5);
+  if (!wait_one(p, s, c, layer, ROW_ROUTED_UPGATE, 0, p.top_k * (p.moe_ffn / kTile))) return false;
+  const int eid = expert_of(p, slot);
+  if (eid < 0) return bad_operand(p, s, c, 2);
+  const float weight = ld_shared_f32(p.expert_weights + slot);
+  stage_vector(s, c, p.routed_silu + static_cast<size_t>(slot) * p.moe_ffn, p.moe_ffn);
+  const u16* w = p.expert_down_w + (static_cast<size_t>(layer) * p.num_experts + eid) * M::H * p.moe_ffn;
+  float* mine = p.routed_parts + static_cast<size_t>(slot) * M::H;
+  down_rows(s, c, w, p.moe_ffn, p.moe_ffn, n0 * tile, (n1 - n0) * tile, [&](int r, float dot) { st_shared_f32(mine + r, round_bf16(dot) * weight); });
+  release_stores();
+  __syncthreads();
+  if (c.tid < n1 - n0) publish(counter_ptr(p, layer, ROW_ROUTED_DOWN, n0 + c.tid), 1);
+  return true;
+}
+
+// ==================================================================== 14 ==
+// [14, layer, n_start, n_end, tile_N_g]   (python_vm.py:492-530)
+// hidden[r] = bf16(hidden[r] + routed[r] + sigmoid(gate_w . normed) * shared[r]) for the rows of its tiles,
+// with shared = the K-slice terms added in bf16 in slice order and routed = the slots' terms added in
+// fp32 in slot order; leaves shared_out complete and routed_out_f32 cleared, as the VM does.
+template <class M>
+__device__ bool op_combine(const Params& p, Smem<M>& s, const Ctx& c) {
+  const int layer = s.inst[1], n0 = s.inst[2], n1 = s.inst[3], tile = s.inst[4];
+  if (layer < 0 || layer >= p.num_layers) return bad_operand(p, s, c, 1);
+  if (tile != kTile || n0 < 0 || n1 < n0 || n1 * tile > M::H || 2 * (n1 - n0) > kThreads) return bad_operand(p, s, c, 3);
+  const int nb = n1 - n0;
+  if (c.tid < 2 * nb) {
+    const bool routed = c.tid >= nb;
+    const int blk = n0 + (routed ? c.tid - nb : c.tid);
+    if (!poll_counter(counter_ptr(p, layer, routed ? ROW_ROUTED_DOWN : ROW_SHARED_DOWN, blk), routed ? p.top_k : p.shared_k_slices, p.spin_limit)) {
+      s.ctl[0] = 1;
+      report_error(p, QMK_DEV_WAIT_TIMEOUT, c.inst_idx, c.opcode, c.tid);
+    }
+  }
+  if (p.timeline != nullptr && c.tid == 0) {
+    s.t_wait = wall_clock64();
+    s.ctl[2] = 1;
+  }
+  __syncthreads();
+  if (s.ctl[0]) return false;
+  stage_vector(s, c, p.normed_hidden, M::H);
+  if (c.tid < kWaveSize) {
+    const u16* const rows[1] = {p.shared_scale_w + static_cast<size_t>(layer) * M::H};
+    float v[1];
+    rows_dot<1>(rows, s.x, M::H, c.tid, v);
+    if (c.tid == 0) s.red[0] = 1.0f / (1.0f + expf(-v[0]));
+  }
+  __syncthreads();
+  const float gate = s.red[0];
+  for (int pair = c.tid; pair < nb * tile / 2; pair += kThreads) {
+    const int r = n0 * tile + 2 * pair;
+    float sh0 = 0.f, sh1 = 0.f;
+    for (int k = 0; k < p.shared_k_slices; ++k) {
+      const uint32_t t = ld_shared32(p.shared_parts + static_cast<size_t>(k) * M::H + r);
+      sh0 = round_bf16(sh0 + bf_lo(t));
+      sh1 = round_bf16(sh1 + bf_hi(t));
+    }
+    float ro0 = 0.f, ro1 = 0.f;
+    for (int j = 0; j < p.top_k; ++j) {
+      ro0 += ld_shared_f32(p.routed_parts + static_cast<size_t>(j) * M::H + r);
+      ro1 += ld_shared_f32(p.routed_parts + static_cast<size_t>(j) * M::H + r + 1);
+    }
+    const uint32_t old = ld_shared32(p.hidden + r);
+    const float h0 = (bf_lo(old) + ro0) + gate * sh0, h1 = (bf_hi(old) + ro1) + gate * sh1;
+    st_shared32(p.hidden + r, static_cast<uint32_t>(f2bf(h0)) | (static_cast<uint32_t>(f2bf(h1)) << 16));
+    st_shared32(p.shared_out + r, static_cast<uint32_t>(f2bf(sh0)) | (static_cast<uint32_t>(f2bf(sh1)) << 16));
+    st_shared_f32(p.routed_out_f32 + r, 0.f);
+    st_shared_f32(p.routed_out_f32 + r + 1, 0.f);
+  }
+  publish_done(p, c, layer, ROW_COMBINE, 0, nb);
+  return true;
+}
+
+}  // namespace moe
+}  // namespace qmk

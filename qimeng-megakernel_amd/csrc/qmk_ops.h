@@ -25,6 +25,9 @@ struct Llama1B {
   static constexpr int CARRY_ROWS = 2;  // up/gate rows per wave requested by the O-proj before it
   static constexpr bool CARRY_AFTER_ATTENTION = false;  // ... also by a workgroup that has just run attention
   static constexpr bool QK_NORM = false;
+  static constexpr bool QKV_BIAS = false;
+  static constexpr int REDUCE_HEADS = GQA;  // query heads one reduction instruction merges
+  static constexpr int PREV_ROW = 5;        // counter row that completes a layer: the down projection's
 };
 
 // Qwen3-1.7B shape with the Qwen3 op set: opcode 1 leaves the raw QKV vector, the attention
@@ -42,6 +45,9 @@ struct Qwen3_1p7B {
   static constexpr int CARRY_ROWS = 3;
   static constexpr bool CARRY_AFTER_ATTENTION = true;
   static constexpr bool QK_NORM = true;
+  static constexpr bool QKV_BIAS = false;
+  static constexpr int REDUCE_HEADS = GQA;
+  static constexpr int PREV_ROW = 5;
 };
 
 constexpr int kResSlots = 4096;
@@ -356,7 +362,7 @@ __device__ bool op_rms_qkv_rope(const Params& p, Smem<M>& s, const Ctx& c) {
   if (!rms_to_lds<M, kDepth>(
           p, s, c, (tg && layer > 0) ? p.ws + kWsHiddenOut : nullptr, tag - 1, p.attn_norm + static_cast<size_t>(layer) * M::H,
           [&](auto k) { preload_range<decltype(k)::value, decltype(k)::value + 1>(nrows, src, buf); },
-          [&] { return layer == 0 || tg || wg_wait_all(p, s, c, layer - 1, ROW_DOWN, 0, p.down_arrivals); }))
+          [&] { return layer == 0 || tg || wg_wait_all(p, s, c, layer - 1, M::PREV_ROW, 0, p.down_arrivals); }))
     return false;
   QMK_STAMP(0);
   v4u x[CH];
@@ -374,7 +380,12 @@ __device__ bool op_rms_qkv_rope(const Params& p, Smem<M>& s, const Ctx& c) {
   for (int pair = c.tid; pair < nrows / 2; pair += kThreads) {
     const int r = rs + 2 * pair;
     const bool first = pair == c.tid;
-    const float v0 = round_bf16(s.res[2 * pair]), v1 = round_bf16(s.res[2 * pair + 1]);
+    float a0 = s.res[2 * pair], a1 = s.res[2 * pair + 1];
+    if constexpr (M::QKV_BIAS) {   // the bias belongs to the projection: added before its one rounding
+      const uint32_t bw = *reinterpret_cast<const uint32_t*>(p.qkv_bias + static_cast<size_t>(layer) * M::QKV + r);
+      a0 += bf_lo(bw), a1 += bf_hi(bw);
+    }
+    const float v0 = round_bf16(a0), v1 = round_bf16(a1);
     if constexpr (M::QK_NORM) {
       // Qwen3 op set: the rounded GEMV result leaves as it is; norm and RoPE belong to the attention prologue.
       const uint32_t w = static_cast<uint32_t>(f2bf(v0)) | (static_cast<uint32_t>(f2bf(v1)) << 16);
@@ -419,10 +430,11 @@ __device__ bool op_rms_qkv_rope(const Params& p, Smem<M>& s, const Ctx& c) {
 // list is null) for the GQA heads head0..head0+3 (python_vm.py:439-488).  Thread
 // (h, d/2) of the first 128 produces two neighbouring output dims.  All partial
 // reads are issued before the first use so that they overlap.
-template <class M>
+template <class M, int HEADS = M::GQA>
 __device__ __forceinline__ void merge_partials(const Params& p, int head0, int n, const int32_t* list, bool terminal,
                                                int out_slot) {
-  if (threadIdx.x >= M::GQA * M::D / 2) return;
+  static_assert(HEADS * M::D / 2 <= kThreads, "one thread per output pair");
+  if (threadIdx.x >= HEADS * M::D / 2) return;
   const int h = head0 + threadIdx.x / (M::D / 2), d = 2 * (threadIdx.x % (M::D / 2));
   const float* lse = p.attn_lse + static_cast<size_t>(h) * p.max_splits;
   const float* part = p.attn_partial + static_cast<size_t>(h) * p.max_splits * M::D + d;
@@ -803,7 +815,7 @@ template <class M>
 __device__ bool op_attn_reduce(const Params& p, Smem<M>& s, const Ctx& c) {
   const int layer = s.inst[1], head0 = s.inst[2], P = s.inst[3], n = s.inst[4];
   if (layer < 0 || layer >= p.num_layers) return bad_operand(p, s, c, 1);
-  if (head0 < 0 || head0 + M::GQA > M::NQ) return bad_operand(p, s, c, 2);
+  if (head0 < 0 || head0 + M::REDUCE_HEADS > M::NQ) return bad_operand(p, s, c, 2);
   if (n < 1 || n > kMaxPartials || P < 1) return bad_operand(p, s, c, 4);
   for (int i = 0; i < n; ++i)
     if (s.inst[5 + i] < 0 || s.inst[5 + i] >= p.max_splits) return bad_operand(p, s, c, 5 + i);
@@ -811,11 +823,11 @@ __device__ bool op_attn_reduce(const Params& p, Smem<M>& s, const Ctx& c) {
   const int out_slot = s.inst[6 + n];
   if (!terminal && (out_slot < 0 || out_slot >= p.max_splits)) return bad_operand(p, s, c, 6 + n);
 
-  if (!wg_wait(p, s, c, M::GQA, [&](int i) { return counter_ptr(p, layer, ROW_SPLITKV, head0 + i); }, P)) return false;
-  merge_partials<M>(p, head0, n, &s.inst[5], terminal, out_slot);
+  if (!wg_wait(p, s, c, M::REDUCE_HEADS, [&](int i) { return counter_ptr(p, layer, ROW_SPLITKV, head0 + i); }, P)) return false;
+  merge_partials<M, M::REDUCE_HEADS>(p, head0, n, &s.inst[5], terminal, out_slot);
   release_stores();
   __syncthreads();
-  if (c.tid == 0) publish(counter_ptr(p, layer, ROW_REDUCE, 0), M::GQA);
+  if (c.tid == 0) publish(counter_ptr(p, layer, ROW_REDUCE, 0), M::REDUCE_HEADS);
   return true;
 }
 
@@ -1220,7 +1232,7 @@ __device__ bool op_rms_lmhead(const Params& p, Smem<M>& s, const Ctx& c) {
   RowRegs<CH> buf[kDepth];
   preload<CH>(nrows, src, buf);
   const bool tg = tagged(p);
-  if (!tg && !wg_wait_all(p, s, c, p.num_layers - 1, ROW_DOWN, 0, p.down_arrivals)) return false;
+  if (!tg && !wg_wait_all(p, s, c, p.num_layers - 1, M::PREV_ROW, 0, p.down_arrivals)) return false;
   if (!rms_to_lds(p, s, c, tg ? p.ws + kWsHiddenOut : nullptr, tag_of(s.generation, p.num_layers - 1), p.lm_norm)) return false;
   v4u x[CH];
   load_x_from_lds(x, s.x, lane);

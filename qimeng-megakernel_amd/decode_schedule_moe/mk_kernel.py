@@ -1,16 +1,230 @@
-"""Launcher of the MoE route's kernel (`…/qwen1_5_moe_a2_7b/A100/single_batch/decode_schedule/mk_kernel.py`).
+"""Load and call the gfx950 MoE decode kernel through its C ABI.
 
-The gfx950 kernel for opcodes 8-14 does not exist yet.  Nothing else stands in for it: asking for it fails.
+Host-side counterpart of the reference's launcher of the MoE route
+(`…/qwen/qwen1_5_moe_a2_7b/A100/single_batch/decode_schedule/mk_kernel.py:63-205`): ``get_mk`` returns
+the ``mk`` callable, ``call_mk(globs, mk)`` passes the 39 tensors and 3 scalars in the reference's
+positional order (its three unused dense-MLP positions included), ``run_instructions`` executes an
+arbitrary instruction list.  The callable wraps ``qmk_decode_step_moe`` of ``libqmk_hip.so``
+(``include/qmk.h``) with ctypes.  There is no fallback: a missing library is an ``ImportError``, a
+non-GPU tensor a ``ValueError`` and a device-side error a ``RuntimeError``.
 """
 from __future__ import annotations
 
+import ctypes
+import math
+from pathlib import Path
 from typing import Any
 
+import torch
 
-def get_mk(mk_dir: Any = None):
-    raise ImportError("the gfx950 decode kernel for the MoE opcodes (8-14) is not built; "
-                      "only the dense routes (decode_schedule, decode_schedule_mb) are available")
+from ..decode_schedule import mk_kernel as _single
+from ..decode_schedule.instructions.scheduler import tensorize_instructions
+from ..instruction import Instruction
+from .globs import Globals
+from .instructions import scheduler as _scheduler
+from .model_config import QwenMoeConfig
+
+_P = ctypes.c_void_p
+_I = ctypes.c_int32
+QMK_MODEL_QWEN1_5_MOE_A2_7B = 2
+MI355X_QUEUES = 256
+
+# The positional order of mk(...): name in QmkMoeArgs, or None for the three unused dense-MLP positions.
+_TENSOR_ORDER = (
+    "instructions", "hidden_states", "normed_hidden_states", "q_post_rope", "k_cache", "v_cache", "attn_out",
+    "attn_lse_intermediates", "attn_out_intermediates", "silu_out", "logits", "attn_norm_weights", "qkv_weights", "qkv_bias",
+    "rope_cos", "rope_sin", "o_proj_weights", "mlp_norm_weights", None, None, None, "lm_head_norm_weights", "lm_head_weights",
+    "router_weights", "router_logits_buf", "expert_indices", "expert_weights", "shared_expert_gate_proj_weights",
+    "shared_expert_up_proj_weights", "shared_expert_down_proj_weights", "shared_expert_silu_out", "shared_out",
+    "shared_expert_gate_weights", "expert_gate_up_proj_weights", "expert_down_proj_weights", "routed_silu_buffer",
+    "routed_out_f32", "routed_out", "barriers",
+)
+_DTYPES = {"instructions": torch.int32, "attn_lse_intermediates": torch.float32, "attn_out_intermediates": torch.float32,
+           "rope_cos": torch.float32, "rope_sin": torch.float32, "router_logits_buf": torch.float32, "expert_indices": torch.int64,
+           "expert_weights": torch.float32, "routed_out_f32": torch.float32, "barriers": torch.int32}
 
 
-def call_mk(globs: Any, mk: Any) -> None:
-    raise ImportError("the gfx950 decode kernel for the MoE opcodes (8-14) is not built")
+class QmkMoeArgs(ctypes.Structure):
+    """Mirror of ``struct QmkMoeArgs`` in include/qmk.h (field order is the ABI)."""
+
+    _fields_ = (
+        [("struct_size", ctypes.c_uint32), ("model", ctypes.c_uint32), ("flags", ctypes.c_uint32), ("spin_limit", ctypes.c_uint32)]
+        + [(name, _P) for name in _TENSOR_ORDER if name is not None]
+        + [(name, _I) for name in ("num_queues", "num_insts", "num_layers", "num_layer_barriers", "barrier_slots", "max_seq_len",
+                                   "max_splits", "vocab_size", "rope_rows", "pos_id", "num_experts", "top_k", "shared_ffn", "moe_ffn",
+                                   "shared_k_slices")]
+        + [("attn_scale", ctypes.c_float), ("rms_norm_eps", ctypes.c_float), ("timeline", _P), ("stream", _P), ("workspace", _P),
+           ("workspace_bytes", ctypes.c_uint64)]
+    )
+
+
+class MoeMegaKernel:
+    """The ``mk`` callable of the MoE route.  ``reset_barriers``: the kernel clears the counters when it
+    retires (default), or leaves their final values like the reference kernel."""
+
+    def __init__(self, lib: ctypes.CDLL, *, reset_barriers: bool = True, spin_limit: int = 0):
+        self._lib = lib
+        self.reset_barriers = reset_barriers
+        self.spin_limit = int(spin_limit)
+        self.timeline: torch.Tensor | None = None
+        self._workspace: torch.Tensor | None = None
+        self._args = QmkMoeArgs()
+        self._args.struct_size = ctypes.sizeof(QmkMoeArgs)
+        self._args.model = QMK_MODEL_QWEN1_5_MOE_A2_7B
+        self._bound_key: tuple | None = None
+
+    def error_string(self, code: int) -> str:
+        return self._lib.qmk_error_string(int(code)).decode()
+
+    def check(self, stream: torch.cuda.Stream | None = None) -> None:
+        detail = (_I * 4)()
+        handle = (stream or torch.cuda.current_stream()).cuda_stream
+        code = int(self._lib.qmk_status_fetch(_P(handle), ctypes.byref(detail)))
+        if code != 0:
+            raise RuntimeError(
+                f"megakernel device error {code} ({self.error_string(code)}): workgroup={detail[0]} "
+                f"instruction={detail[1]} opcode={detail[2]} operand={detail[3]}; "
+                "the counters are undefined now — zero `barriers` before the next step"
+            )
+
+    def with_options(self, **kw: Any) -> "MoeMegaKernel":
+        other = MoeMegaKernel(self._lib, reset_barriers=kw.pop("reset_barriers", self.reset_barriers),
+                              spin_limit=kw.pop("spin_limit", self.spin_limit))
+        if kw:
+            raise TypeError(f"unknown options {sorted(kw)}")
+        return other
+
+    def _bind(self, tensors: dict[str, torch.Tensor]) -> None:
+        a, s = self._args, QwenMoeConfig.shape()
+        if (s.hidden_size, s.head_dim, s.num_attention_heads, s.num_key_value_heads) != (2048, 128, 16, 16):
+            raise ValueError("the MoE kernel is compiled for the Qwen1.5-MoE attention geometry (H 2048, 16/16 heads of 128)")
+        device = tensors["hidden_states"].device
+        for name, t in tensors.items():
+            if not isinstance(t, torch.Tensor):
+                raise TypeError(f"{name} must be a torch.Tensor, got {type(t).__name__}")
+            if t.device.type != "cuda" or t.device != device:
+                raise ValueError(f"{name} must live on the GPU of hidden_states, got {t.device}")
+            want = _DTYPES.get(name, torch.bfloat16)
+            if t.dtype != want:
+                raise TypeError(f"{name} must be {want}, got {t.dtype}")
+            if not t.is_contiguous():
+                raise ValueError(f"{name} must be contiguous")
+            setattr(a, name, t.data_ptr())
+        L, H = int(tensors["barriers"].shape[0]), s.hidden_size
+        E, k = int(tensors["router_weights"].shape[1]), int(tensors["expert_indices"].numel())
+        Fs, Fm = int(tensors["shared_expert_gate_proj_weights"].shape[1]), int(tensors["routed_silu_buffer"].shape[-1])
+        V = int(tensors["logits"].numel())
+
+        def numel(name: str, want: int) -> None:
+            if tensors[name].numel() != want:
+                raise ValueError(f"{name} has {tensors[name].numel()} elements ({tuple(tensors[name].shape)}), the kernel needs {want}")
+
+        if tensors["instructions"].dim() != 3 or tensors["instructions"].shape[2] != 32:
+            raise ValueError("instructions must be [queues, length, 32]")
+        S = int(tensors["k_cache"].shape[2])
+        P = int(tensors["attn_lse_intermediates"].shape[-1])
+        for name, want in (("hidden_states", H), ("normed_hidden_states", H), ("q_post_rope", H), ("attn_out", H), ("silu_out", Fm),
+                           ("k_cache", L * S * H), ("v_cache", L * S * H), ("attn_lse_intermediates", 16 * P),
+                           ("attn_out_intermediates", 16 * P * 128), ("attn_norm_weights", L * H), ("mlp_norm_weights", L * H),
+                           ("qkv_weights", L * 3 * H * H), ("qkv_bias", L * 3 * H), ("o_proj_weights", L * H * H),
+                           ("lm_head_norm_weights", H), ("lm_head_weights", V * H), ("router_weights", L * E * H),
+                           ("router_logits_buf", E), ("expert_weights", k), ("shared_expert_gate_proj_weights", L * Fs * H),
+                           ("shared_expert_up_proj_weights", L * Fs * H), ("shared_expert_down_proj_weights", L * H * Fs),
+                           ("shared_expert_silu_out", Fs), ("shared_out", H), ("shared_expert_gate_weights", L * H),
+                           ("expert_gate_up_proj_weights", L * E * 2 * Fm * H), ("expert_down_proj_weights", L * E * H * Fm),
+                           ("routed_silu_buffer", k * Fm), ("routed_out_f32", H), ("routed_out", H)):
+            numel(name, want)
+        if tensors["rope_cos"].shape != tensors["rope_sin"].shape or tensors["rope_cos"].shape[-1] != 128:
+            raise ValueError("rope_cos/rope_sin must both be [positions, head_dim]")
+        bar = tensors["barriers"]
+        if bar.dim() != 3 or bar.shape[1] < 15 or bar.shape[2] < 128:
+            raise ValueError(f"barriers must be [layers, >= 15, >= 128], got {tuple(bar.shape)}")
+        a.num_queues, a.num_insts = int(tensors["instructions"].shape[0]), int(tensors["instructions"].shape[1])
+        a.num_layers, a.num_layer_barriers, a.barrier_slots = L, int(bar.shape[1]), int(bar.shape[2])
+        a.max_seq_len, a.max_splits, a.vocab_size, a.rope_rows = S, P, V, int(tensors["rope_cos"].shape[0])
+        a.num_experts, a.top_k, a.shared_ffn, a.moe_ffn, a.shared_k_slices = E, k, Fs, Fm, int(s.num_downproj_split_k_shared)
+        nbytes = int(self._lib.qmk_moe_workspace_bytes(k, a.shared_k_slices))
+        if nbytes == 0:
+            raise ValueError(f"top_k {k} / {a.shared_k_slices} K slices are outside what the kernel supports")
+        if self._workspace is None or self._workspace.device != device or self._workspace.numel() < nbytes:
+            self._workspace = torch.zeros(nbytes, dtype=torch.uint8, device=device)
+        a.workspace, a.workspace_bytes = self._workspace.data_ptr(), nbytes
+
+    def __call__(self, *args: Any) -> None:
+        if len(args) != len(_TENSOR_ORDER) + 3:
+            raise TypeError(f"mk of the MoE route takes {len(_TENSOR_ORDER)} tensors and 3 scalars, got {len(args)} positional arguments")
+        tensors = {name: t for name, t in zip(_TENSOR_ORDER, args) if name is not None}
+        pos_id, attn_scale, rms_norm_eps = args[len(_TENSOR_ORDER):]
+        if isinstance(tensors["instructions"], torch.Tensor) and tensors["instructions"].numel() == 0:
+            return
+        key = tuple((t.data_ptr(), tuple(t.shape)) if isinstance(t, torch.Tensor) else None for t in tensors.values()) + (QwenMoeConfig.shape(),)
+        if key != self._bound_key:
+            self._bind(tensors)
+            self._bound_key = key
+        a = self._args
+        a.pos_id, a.attn_scale, a.rms_norm_eps = int(pos_id), float(attn_scale), float(rms_norm_eps)
+        a.flags = 0 if self.reset_barriers else _single.QMK_FLAG_KEEP_BARRIERS
+        a.spin_limit = self.spin_limit
+        a.timeline = self.timeline.data_ptr() if self.timeline is not None else None
+        a.stream = torch.cuda.current_stream(tensors["hidden_states"].device).cuda_stream
+        rc = int(self._lib.qmk_decode_step_moe(ctypes.byref(a)))
+        if rc != 0:
+            raise RuntimeError(f"qmk_decode_step_moe failed with {rc}: {self.error_string(rc)}")
+
+
+def get_mk(mk_dir: Path | None = None, *, reset_barriers: bool = True, spin_limit: int = 0) -> MoeMegaKernel:
+    """Return the ``mk`` callable of the MoE route bound to the prebuilt library in ``mk_dir``."""
+    root = (_single._default_mk_dir() if mk_dir is None else Path(mk_dir)).resolve()
+    lib = _single._LIB_CACHE.get(root)
+    if lib is None:
+        lib = _single.load_library(root)
+        _single._LIB_CACHE[root] = lib
+    for name in ("qmk_decode_step_moe", "qmk_moe_workspace_bytes"):
+        if not hasattr(lib, name):
+            raise ImportError(f"{root / 'libqmk_hip.so'} does not export {name}")
+    lib.qmk_decode_step_moe.argtypes = [ctypes.POINTER(QmkMoeArgs)]
+    lib.qmk_decode_step_moe.restype = ctypes.c_int
+    lib.qmk_moe_workspace_bytes.argtypes = [ctypes.c_int, ctypes.c_int]
+    lib.qmk_moe_workspace_bytes.restype = ctypes.c_uint64
+    return MoeMegaKernel(lib, reset_barriers=reset_barriers, spin_limit=spin_limit)
+
+
+def call_mk(globs: Globals, mk: Any) -> None:
+    """One decode step with the current ``Globals`` (builds the instruction tensor on first use)."""
+    s = QwenMoeConfig.shape()
+    if globs.instructions is None:
+        build(globs)
+    unused = globs.hidden_states          # the three dense-MLP positions of the reference's argument list
+    g = globs
+    mk(g.instructions, g.hidden_states, g.normed_hidden_states, g.q_post_rope, g.k_cache, g.v_cache, g.attn_out,
+       g.attn_lse_intermediates, g.attn_out_intermediates, g.silu_out, g.logits, g.attn_norm_weights, g.qkv_weights, g.qkv_bias,
+       g.rope_cos, g.rope_sin, g.o_proj_weights, g.mlp_norm_weights, unused, unused, unused, g.lm_head_norm_weights, g.lm_head_weights,
+       g.router_weights, g.router_logits_buf, g.expert_indices, g.expert_weights, g.shared_expert_gate_proj_weights,
+       g.shared_expert_up_proj_weights, g.shared_expert_down_proj_weights, g.shared_expert_silu_out, g.shared_out,
+       g.shared_expert_gate_weights, g.expert_gate_up_proj_weights, g.expert_down_proj_weights, g.routed_silu_buffer,
+       g.routed_out_f32, g.routed_out, g.barriers,
+       g.position_id if g.position_id is not None else 0, 1.0 / math.sqrt(s.head_dim), float(s.rms_norm_eps))
+
+
+def mi355x_scheduler(shape: Any = None) -> _scheduler.MoeScheduler:
+    """The reference's layout on one queue per CU."""
+    from .model_config import num_partials_for
+
+    shape = shape or QwenMoeConfig.shape()
+    return _scheduler.MoeScheduler(shape, MI355X_QUEUES, num_partials_for(MI355X_QUEUES, shape))
+
+
+def build(globs: Globals) -> torch.Tensor:
+    sched = mi355x_scheduler()
+    if sched.num_partials > int(globs.attn_lse_intermediates.shape[-1]):
+        raise ValueError("attn_lse_intermediates has fewer partial slots than the schedule's split-KV fan-out")
+    return tensorize_instructions(globs, sched.queues())
+
+
+def run_instructions(globs: Globals, instructions: list[Instruction], *, mk: Any = None, queues: int | None = None) -> None:
+    """Deal ``instructions`` round-robin onto the queues and execute them once, counters kept."""
+    mk_call = get_mk() if mk is None else mk
+    if isinstance(mk_call, MoeMegaKernel) and mk_call.reset_barriers:
+        mk_call = mk_call.with_options(reset_barriers=False)
+    tensorize_instructions(globs, _scheduler.deal(instructions, queues or MI355X_QUEUES))
+    call_mk(globs, mk_call)

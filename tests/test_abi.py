@@ -14,6 +14,7 @@ import torch
 from __graft_entry__ import LIBRARY, ROOT, build_library
 from qimeng_megakernel_amd.decode_schedule import mk_kernel
 from qimeng_megakernel_amd.decode_schedule_mb import mk_kernel as mk_kernel_mb
+from qimeng_megakernel_amd.decode_schedule_moe import mk_kernel as mk_kernel_moe
 
 HEADER = ROOT / "include" / "qmk.h"
 
@@ -28,13 +29,14 @@ def lib():
 def test_every_declared_symbol_is_exported(lib):
     text = HEADER.read_text()
     declared = set(re.findall(r"^(?:int|uint64_t|const char\*)\s+(qmk_\w+)\s*\(", text, flags=re.M))
-    assert declared == {"qmk_decode_step", "qmk_decode_step_batch", "qmk_query", "qmk_status_fetch", "qmk_error_string",
-                        "qmk_workspace_bytes"}
+    assert declared == {"qmk_decode_step", "qmk_decode_step_batch", "qmk_decode_step_moe", "qmk_moe_workspace_bytes", "qmk_query",
+                        "qmk_status_fetch", "qmk_error_string", "qmk_workspace_bytes"}
     for name in declared:
         assert hasattr(lib, name), name
 
 
-@pytest.mark.parametrize("struct,mirror", [("QmkArgs", mk_kernel.QmkArgs), ("QmkBatchArgs", mk_kernel_mb.QmkBatchArgs)])
+@pytest.mark.parametrize("struct,mirror", [("QmkArgs", mk_kernel.QmkArgs), ("QmkBatchArgs", mk_kernel_mb.QmkBatchArgs),
+                                           ("QmkMoeArgs", mk_kernel_moe.QmkMoeArgs)])
 def test_struct_layout_matches_header(tmp_path, struct, mirror):
     """Compile the header with gcc and compare sizeof/offsetof with the ctypes mirror."""
     fields = [name for name, _ in mirror._fields_]
@@ -78,7 +80,7 @@ def test_host_side_argument_errors(lib):
     a.model = 0
     assert lib.qmk_decode_step(ctypes.byref(a)) == 1                       # all tensor pointers are NULL
     assert lib.qmk_workspace_bytes(0) == 8 * (4096 + 512 + 4096 + 1024) and lib.qmk_workspace_bytes(1) == lib.qmk_workspace_bytes(0) and lib.qmk_workspace_bytes(7) == 0
-    assert lib.qmk_query(0) == 5 and lib.qmk_query(2) == 512 and lib.qmk_query(5) == 32 and lib.qmk_query(6) == 25
+    assert lib.qmk_query(0) == 6 and lib.qmk_query(2) == 512 and lib.qmk_query(5) == 32 and lib.qmk_query(6) == 25
     assert 0 < lib.qmk_query(3) <= 160 * 1024
     assert lib.qmk_error_string(34).decode().startswith("device: counter wait")
     mk_kernel_mb.get_mk()                                                  # declares the entry point's signature
@@ -91,6 +93,14 @@ def test_host_side_argument_errors(lib):
     assert lib.qmk_decode_step_batch(ctypes.byref(b)) == 8                 # only the Llama geometry is compiled for this route
     b.model = 0
     assert lib.qmk_decode_step_batch(ctypes.byref(b)) == 1
+    mk_kernel_moe.get_mk()
+    assert lib.qmk_decode_step_moe(None) == 1
+    m = mk_kernel_moe.QmkMoeArgs()
+    m.struct_size = ctypes.sizeof(mk_kernel_moe.QmkMoeArgs)
+    assert lib.qmk_decode_step_moe(ctypes.byref(m)) == 8                   # model 0 is not the MoE geometry
+    m.model = 2
+    assert lib.qmk_decode_step_moe(ctypes.byref(m)) == 1
+    assert lib.qmk_moe_workspace_bytes(4, 4) == 4 * 2048 * 2 + 4 * 2048 * 4 and lib.qmk_moe_workspace_bytes(9, 4) == 0
     assert lib.qmk_error_string(12345).decode() == "unknown code"
 
 

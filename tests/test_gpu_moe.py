@@ -1,0 +1,212 @@
+"""MoE decode route on the GPU: the kernel behind ``qmk_decode_step_moe`` against the CPU oracles.
+
+Mirrors the reference's verifier stages for this route
+(`qimeng_megakernel/verifier/LLM/qwen/qwen1_5_moe_a2_7b/A100/single_batch/{pyvm_to_megakernel,e2e_generate}`):
+the same instruction list runs on the sequential VM and through the C ABI; outputs agree within bf16
+rounding, routing decisions and counters exactly; a whole request reproduces the tokens and the routing
+recorded from the reference.
+"""
+import copy
+import dataclasses
+import json
+
+import pytest
+import torch
+
+from conftest import GOLDEN
+from gpu_helpers import bf16_close, rel_close, tensor_rel_close
+from pyvm_moe_oracle import MoeInstructionVM
+from qimeng_megakernel_amd import synthetic
+from qimeng_megakernel_amd.decode_schedule_moe import mk_kernel
+from qimeng_megakernel_amd.decode_schedule_moe.instructions import scheduler as S
+from qimeng_megakernel_amd.decode_schedule_moe.model_config import QWEN1_5_MOE_A2_7B, QwenMoeConfig, num_partials_for
+
+pytestmark = pytest.mark.gpu
+
+FIX = json.loads((GOLDEN / "moe_reduced_seed0.json").read_text())
+SMALL = dataclasses.replace(QWEN1_5_MOE_A2_7B, **FIX["shape"])
+MUTABLE = ("hidden_states", "q_post_rope", "attn_out", "logits", "k_cache", "v_cache", "attn_out_intermediates", "attn_lse_intermediates",
+           "barriers", "router_logits_buf", "normed_hidden_states", "shared_expert_silu_out", "shared_out", "routed_silu_buffer",
+           "routed_out_f32", "silu_out", "expert_indices", "expert_weights")
+
+
+@pytest.fixture(autouse=True)
+def _shape():
+    QwenMoeConfig.set_shape(SMALL)
+    with torch.no_grad():
+        yield
+    QwenMoeConfig.set_shape(QWEN1_5_MOE_A2_7B)
+
+
+@pytest.fixture(scope="module")
+def weights():
+    return synthetic.random_moe_weights(SMALL, FIX["seed"], FIX["kv_capacity"])
+
+
+def sync_state(src, dst):
+    for name in MUTABLE:
+        getattr(dst, name).copy_(getattr(src, name))
+    dst.position_id = src.position_id
+
+
+def make_pair(weights, shape=SMALL, position=41, token=99, capacity=None):
+    capacity = capacity or FIX["kv_capacity"]
+    cpu = synthetic.build_moe_globals(weights, shape, capacity, "cpu")
+    gpu = synthetic.build_moe_globals(weights, shape, capacity, "cuda:0")
+    gen = torch.Generator().manual_seed(5)
+    cpu.k_cache.copy_(torch.randn(cpu.k_cache.shape, generator=gen).bfloat16())
+    cpu.v_cache.copy_(torch.randn(cpu.v_cache.shape, generator=gen).bfloat16())
+    cpu.hidden_states.copy_(cpu.embed_tokens[token])
+    cpu.position_id = position
+    sync_state(cpu, gpu)
+    return cpu, gpu
+
+
+def run_kernel(gpu, instructions, queues=256):
+    mk = mk_kernel.get_mk(reset_barriers=False, spin_limit=1 << 18)
+    mk_kernel.run_instructions(gpu, copy.deepcopy(instructions), mk=mk, queues=queues)
+    mk.check()
+    return mk
+
+
+STAGES = ["qkvproj", "attention_split_kv", "attention_reduction", "oproj", "router_gemv", "router_softmax_topk", "shared_upgate",
+          "shared_downproj", "routed_upgate", "routed_downproj", "combine_commit"]
+BF16_OUT = {"qkvproj": ("q_post_rope", "k_cache", "v_cache"), "attention_reduction": ("attn_out",), "oproj": ("hidden_states",),
+            "router_gemv": ("normed_hidden_states",), "shared_upgate": ("shared_expert_silu_out",),
+            "routed_upgate": ("routed_silu_buffer", "silu_out"), "combine_commit": ("hidden_states", "shared_out")}
+
+
+@pytest.mark.parametrize("stage", range(len(STAGES)), ids=STAGES)
+@pytest.mark.parametrize("position", [41, 0, 95])
+def test_one_op_against_the_vm(weights, stage, position):
+    """Everything before the op runs on the VM; the op itself on both, from identical state."""
+    cpu, gpu = make_pair(weights, position=position)
+    sched = mk_kernel.mi355x_scheduler(SMALL)
+    vm = MoeInstructionVM(SMALL)
+    name = STAGES[stage]
+    # the combine step adds up terms that the two down projections left in the launcher's workspace: those run on both sides too
+    first = STAGES.index("shared_downproj") if name == "combine_commit" else stage
+    for earlier in STAGES[:first]:
+        vm.run(cpu, getattr(sched, earlier)(0))
+    sync_state(cpu, gpu)
+    mine = [ins for part in STAGES[first : stage + 1] for ins in getattr(sched, part)(0)]
+    vm.run(cpu, copy.deepcopy(mine))
+    mk = run_kernel(gpu, mine)
+    assert torch.equal(gpu.barriers.cpu(), cpu.barriers), "counters differ from the VM's"
+    for out in BF16_OUT.get(name, ()):
+        loose = out in ("q_post_rope", "k_cache", "shared_expert_silu_out", "routed_silu_buffer", "silu_out")
+        floor = 2.0 ** -1 if out == "hidden_states" else 2.0 ** -6
+        bf16_close(getattr(gpu, out), getattr(cpu, out), ulps=2.0 if loose else 1.0, floor=floor, name=out)
+    H = SMALL.hidden_size
+    if name == "attention_split_kv":
+        g, w = gpu.attn_lse_intermediates.cpu(), cpu.attn_lse_intermediates
+        assert torch.equal(torch.isinf(g), torch.isinf(w))
+        assert float((g[~torch.isinf(w)] - w[~torch.isinf(w)]).abs().max()) <= 2e-3
+        assert float((gpu.attn_out_intermediates.cpu() - cpu.attn_out_intermediates).abs().max()) <= 2e-3 * float(cpu.attn_out_intermediates.abs().max())
+    if name == "router_gemv":
+        assert torch.allclose(gpu.router_logits_buf.cpu(), cpu.router_logits_buf, rtol=1e-4, atol=1e-5)
+    if name == "router_softmax_topk":
+        assert gpu.expert_indices.tolist() == cpu.expert_indices.tolist()
+        assert torch.allclose(gpu.expert_weights.cpu(), cpu.expert_weights, rtol=1e-5)
+    if name == "shared_downproj":      # the K-slice terms wait in the workspace: added in slice order they are the VM's shared_out
+        parts = mk._workspace[: SMALL.num_downproj_split_k_shared * H * 2].view(torch.bfloat16).view(-1, H).cpu()
+        total = torch.zeros(H, dtype=torch.bfloat16)
+        for k in range(parts.shape[0]):
+            total = (total.float() + parts[k].float()).to(torch.bfloat16)
+        bf16_close(total, cpu.shared_out, ulps=2.0, name="shared_out from the K-slice terms")
+    if name == "routed_downproj":
+        off = ((SMALL.num_downproj_split_k_shared * H * 2 + 127) // 128) * 128
+        parts = mk._workspace[off : off + SMALL.num_experts_per_tok * H * 4].view(torch.float32).view(-1, H).cpu()
+        total = torch.zeros(H)
+        for j in range(parts.shape[0]):
+            total += parts[j]
+        assert float((total - cpu.routed_out_f32).abs().max()) <= 2.0 ** -8 * float(cpu.routed_out_f32.abs().max())
+    if name == "combine_commit":
+        assert float(gpu.routed_out_f32.abs().max()) == 0.0 == float(cpu.routed_out_f32.abs().max())
+
+
+def test_lm_head_against_the_vm(weights):
+    cpu, gpu = make_pair(weights)
+    sched = mk_kernel.mi355x_scheduler(SMALL)
+    cpu.barriers[SMALL.num_hidden_layers - 1, 13, 0] = SMALL.num_hidden_blocks
+    sync_state(cpu, gpu)
+    MoeInstructionVM(SMALL).run(cpu, sched.lmhead())
+    run_kernel(gpu, sched.lmhead())
+    bf16_close(gpu.logits, cpu.logits, name="logits")
+
+
+@pytest.mark.parametrize("queues", [256, 108])
+def test_whole_step(weights, queues):
+    """One step of both layers and the LM head: the reference's stream on 108 queues unchanged, and on 256."""
+    cpu, gpu = make_pair(weights)
+    sched = S.MoeScheduler(SMALL, queues, num_partials_for(queues, SMALL))
+    mine = sched.instruction_list()
+    MoeInstructionVM(SMALL).run(cpu, copy.deepcopy(mine))
+    run_kernel(gpu, mine, queues=queues)
+    assert torch.equal(gpu.barriers.cpu(), cpu.barriers)
+    assert gpu.expert_indices.tolist() == cpu.expert_indices.tolist()
+    tensor_rel_close(gpu.hidden_states, cpu.hidden_states, name="hidden_states")
+    rel_close(gpu.logits, cpu.logits, rel=4e-2, name="logits")
+    assert int(gpu.logits.float().argmax()) == int(cpu.logits.float().argmax())
+
+
+def test_request_of_the_reference_fixture(weights):
+    """Six greedy steps through call_mk with one instruction tensor and self-clearing counters: the tokens,
+    the last layer's routing and the top-4 logits recorded from the reference's VM."""
+    g = synthetic.build_moe_globals(weights, SMALL, FIX["kv_capacity"], "cuda:0")
+    gen = torch.Generator().manual_seed(FIX["seed"] + 1)
+    g.k_cache.copy_(torch.randn(g.k_cache.shape, generator=gen).bfloat16())
+    g.v_cache.copy_(torch.randn(g.v_cache.shape, generator=gen).bfloat16())
+    mk = mk_kernel.get_mk(spin_limit=1 << 18)
+    token = FIX["start_token"]
+    for step, want in enumerate(FIX["steps"]):
+        g.position_id = want["position"]
+        g.hidden_states.copy_(g.embed_tokens[token])
+        mk_kernel.call_mk(g, mk)
+        mk.check()
+        assert int(g.barriers.abs().sum()) == 0, "the last workgroup clears the counters"
+        rec = want["my_vm"]
+        if g.expert_indices.tolist() != rec["last_layer_experts"]["indices"]:
+            # A routing decision may flip where two experts are next to tied (the normalised row differs from the
+            # VM's in bf16 roundings): the disputed experts must then be that close, and the trajectories part here.
+            probs = torch.softmax(g.router_logits_buf.cpu(), dim=-1)
+            disputed = sorted(set(g.expert_indices.tolist()) ^ set(rec["last_layer_experts"]["indices"]))
+            assert len(disputed) == 2 and abs(float(probs[disputed[0]] - probs[disputed[1]])) <= 0.03 * float(probs[disputed].max()), (step, disputed, probs.tolist())
+            assert step >= 2, "the first steps of this request have clear routing margins"
+            break
+        assert torch.allclose(g.expert_weights.cpu(), torch.tensor(rec["last_layer_experts"]["weights"]), rtol=2e-2)
+        got = g.logits[torch.tensor(rec["top_ids"], device=g.logits.device)].view(torch.int16).to(torch.int32).cpu()
+        ref = torch.tensor(rec["top_bits"], dtype=torch.int32)
+        ref = torch.where(ref >= 32768, ref - 65536, ref)
+        assert int((got - ref).abs().max()) <= 8, (step, got.tolist(), ref.tolist())
+        token = int(g.logits.float().argmax())
+        assert token == rec["token"], step
+
+
+def test_full_geometry_layers_against_the_vm():
+    """Qwen1.5-MoE-A2.7B layer geometry (60 experts of 1408, top-4, shared 5632), two layers, small vocabulary:
+    layer by layer from the VM's residual stream, then the LM head."""
+    shape = dataclasses.replace(QWEN1_5_MOE_A2_7B, num_hidden_layers=2, vocab_size=2048)
+    QwenMoeConfig.set_shape(shape)
+    w = synthetic.random_moe_weights(shape, 4, 160)
+    cpu, gpu = make_pair(w, shape=shape, position=133, token=77, capacity=160)
+    sched = mk_kernel.mi355x_scheduler(shape)
+    vm = MoeInstructionVM(shape)
+    for layer in range(2):
+        gpu.hidden_states.copy_(cpu.hidden_states)
+        vm.run(cpu, sched.layer(layer))
+        gpu.barriers.zero_()
+        if layer:
+            gpu.barriers[layer - 1, 13, 0] = shape.num_hidden_blocks
+        run_kernel(gpu, sched.layer(layer))
+        assert gpu.expert_indices.tolist() == cpu.expert_indices.tolist(), layer
+        assert torch.allclose(gpu.expert_weights.cpu(), cpu.expert_weights, rtol=2e-2)   # the router reads a bf16 row that differs in roundings
+        rel_close(gpu.hidden_states, cpu.hidden_states, name=f"hidden_states after layer {layer}")
+        assert torch.equal(gpu.barriers[layer].cpu(), cpu.barriers[layer])
+    gpu.hidden_states.copy_(cpu.hidden_states)
+    vm.run(cpu, sched.lmhead())
+    gpu.barriers.zero_()
+    gpu.barriers[1, 13, 0] = shape.num_hidden_blocks
+    run_kernel(gpu, sched.lmhead())
+    rel_close(gpu.logits, cpu.logits, name="logits")
+    assert int(gpu.logits.float().argmax()) == int(cpu.logits.float().argmax())

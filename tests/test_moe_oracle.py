@@ -1,7 +1,7 @@
 """MoE decode route at batch 1: instruction set, scheduler and the two CPU oracles.
 
-The gfx950 kernel for opcodes 8-14 is not built yet; what is pinned here is everything it will be
-checked against.  Anchors:
+What is pinned here is everything the gfx950 kernel of this route is checked against (its own parity
+tests need a GPU).  Anchors:
 
 * ``tests/golden/moe_reduced_seed0.json`` — written by ``make_fixtures_moe.py`` from the imported
   reference while this repository's scheduler, VM and fused oracle ran in lock-step with the
@@ -220,6 +220,13 @@ def test_moe_block_closed_form(weights, route):
     assert float((before.float() + float(probs[5] + probs[2]) * one + shared - got).abs().max()) > 3e-2 * float(want.abs().max())
 
 
-def test_moe_kernel_is_absent_and_says_so():
-    with pytest.raises(ImportError, match="not built"):
-        mk_kernel.get_mk()
+def test_mk_of_the_moe_route_checks_its_arguments(weights):
+    with pytest.raises(ImportError, match="missing prebuilt kernel"):
+        mk_kernel.get_mk(ROOT / "tests")
+    mk = mk_kernel.get_mk()
+    g = _request(weights)
+    g.instructions = torch.zeros(4, 1, 32, dtype=torch.int32)
+    with pytest.raises(ValueError, match="must live on the GPU"):
+        mk_kernel.call_mk(g, mk)
+    with pytest.raises(TypeError, match="positional arguments"):
+        mk(g.instructions, g.hidden_states)
