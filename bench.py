@@ -166,6 +166,68 @@ def batch_decode(args) -> dict:
     return line
 
 
+def moe_decode(args) -> dict:
+    """Qwen1.5-MoE-A2.7B-shaped greedy decode at batch 1 through the MoE route's kernel."""
+    import torch
+
+    from qimeng_megakernel_amd import decode_moe, synthetic
+    from qimeng_megakernel_amd.decode_schedule_moe import mk_kernel
+    from qimeng_megakernel_amd.decode_schedule_moe.model_config import QWEN1_5_MOE_A2_7B, QwenMoeConfig
+
+    shape = QWEN1_5_MOE_A2_7B
+    QwenMoeConfig.set_shape(shape)
+    device = torch.device("cuda:0")
+    torch.cuda.set_device(device)
+    new_tokens = args.steps + 1
+    kv_capacity = args.prompt_len + new_tokens
+    weights = synthetic.random_moe_weights(shape, args.seed, kv_capacity)
+    gen = torch.Generator().manual_seed(args.seed + 1_000_003)
+    prompt = torch.randint(0, shape.vocab_size, (args.prompt_len,), generator=gen, dtype=torch.long)
+    globs = synthetic.build_moe_globals(weights, shape, kv_capacity, device)
+    mk = mk_kernel.get_mk()
+    if args.warmup > 0:
+        decode_moe.decode(globs, prompt, min(args.warmup + 1, new_tokens), mk=mk, decode_time=False)
+    globs.k_cache.zero_(); globs.v_cache.zero_()
+    out = decode_moe.decode(globs, prompt, new_tokens, mk=mk)
+    t = out["timing"]
+    line = {
+        "metric": "kernel_tok_s", "value": t["kernel_tok_s"], "unit": "tok/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": t["kernel_ms_per_step"], "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "bf16",
+        "data": "synthetic",
+        "config": {
+            "workload": f"Qwen1.5-MoE-A2.7B-shaped batch-1 greedy decode, {args.prompt_len}-token prompt, {new_tokens} new tokens "
+                        f"(context {args.prompt_len + 1}..{args.prompt_len + args.steps}), seeded random-init bf16 weights",
+            "layers": shape.num_hidden_layers, "experts": shape.num_experts, "experts_per_token": shape.num_experts_per_tok,
+            "expert_ffn": shape.moe_intermediate_size, "shared_ffn": shape.intermediate_size, "batch": 1, "seed": args.seed,
+            "queues": int(globs.instructions.shape[0]), "instructions_per_queue": int(globs.instructions.shape[1]),
+        },
+        "tok_s": t["effective_tok_s_wall"], "tok_s_gpu": t["effective_tok_s_gpu"], "kernel_tok_s": t["kernel_tok_s"],
+        "first_tokens": out["new_tokens"][:8].tolist(),
+        "roofline": {
+            "bound": "hbm", "achieved": t["achieved_GBps"], "peak": HBM_PEAK_GBPS, "unit": "GB/s", "frac": t["achieved_GBps"] / HBM_PEAK_GBPS,
+            "traffic": None, "bytes_per_launch_avg": t["algorithmic_bytes"] / max(args.steps, 1), "kernel": "decode_megakernel_moe<QwenMoeA2_7B>",
+        },
+    }
+    if not args.no_cpu_baseline:
+        sys.path.insert(0, str(ROOT / "oracle"))
+        from fused_moe_oracle import FusedMoeOracle
+
+        cores = min(os.cpu_count() or 1, 16)
+        torch.set_num_threads(cores)
+        g = synthetic.build_moe_globals(weights, shape, args.cpu_steps + 1, "cpu")
+        oracle = FusedMoeOracle(shape)
+        with torch.no_grad():
+            t0 = time.perf_counter()
+            for pos in range(args.cpu_steps):
+                g.hidden_states.copy_(g.embed_tokens[prompt[min(pos, len(prompt) - 1)]])
+                g.position_id = pos
+                oracle.decode_step(g)
+            dt = time.perf_counter() - t0
+        line["cpu_baseline"] = {"value": args.cpu_steps / dt, "unit": "tok/s", "cores": cores, "kind": "port",
+                                "sample": f"{args.cpu_steps} steps (contexts 1..{args.cpu_steps}) of the same workload through the fused MoE oracle"}
+    return line
+
+
 def cpu_baseline_batch(shape, weights, prompts, n_steps: int, cores: int) -> dict:
     """The fused batch oracle on the host cores: ``n_steps`` steps of the same rows from position 0."""
     import torch
@@ -198,9 +260,10 @@ def main() -> None:
     ap.add_argument("--prompt-len", type=int, default=8)
     ap.add_argument("--cpu-steps", type=int, default=10)
     ap.add_argument("--no-cpu-baseline", action="store_true")
-    ap.add_argument("--model", choices=("llama-3.2-1b", "qwen3-1.7b"), default="llama-3.2-1b",
-                    help="layer geometry: the headline Llama-3.2-1B shape, or the Qwen3-1.7B shape with the Qwen3 op set "
-                         "(28 layers, per-head QK RMSNorm, tied LM head)")
+    ap.add_argument("--model", choices=("llama-3.2-1b", "qwen3-1.7b", "qwen1.5-moe-a2.7b"), default="llama-3.2-1b",
+                    help="layer geometry: the headline Llama-3.2-1B shape, the Qwen3-1.7B shape with the Qwen3 op set "
+                         "(28 layers, per-head QK RMSNorm, tied LM head), or the Qwen1.5-MoE-A2.7B shape with the MoE op set "
+                         "(24 layers, 60 experts of 1408 with top-4 routing, shared expert of 5632)")
     ap.add_argument("--host-sampling", action="store_true",
                     help="argmax and embedding lookup on the host between launches, as the reference's loop does "
                          "(default: inside the kernel)")
@@ -236,6 +299,11 @@ def main() -> None:
                           "dtype": "bf16", "data": "synthetic",
                           "config": {"workload": "Llama-3.2-1B layer geometry, batch 1, one decode step, KV cache ~N(0,1)"},
                           "value": res[max(res, key=int)]["GBps"], "contexts": res}))
+        return
+    if args.model == "qwen1.5-moe-a2.7b":
+        if args.batch != 1:
+            raise SystemExit("bench.py: the MoE route runs at batch 1")
+        print(json.dumps(moe_decode(args)))
         return
     if args.batch != 1:
         if args.model != "llama-3.2-1b" or not 2 <= args.batch <= 16:

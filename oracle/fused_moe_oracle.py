@@ -1,6 +1,7 @@
 """CPU oracle of the MoE decode route (fused form) — TEST INFRASTRUCTURE, not product code.
 
-Only ``tests/`` may import this module, and only as the checker.
+Only ``tests/`` and the ``cpu_baseline`` leg of ``bench.py`` may import this module: as the checker and as
+the timed CPU baseline, never as part of the product path.
 
 Restates the reference's fused PyTorch operations
 (``…/qwen/qwen1_5_moe_a2_7b/A100/single_batch/decode_schedule/fused/operations.py``):

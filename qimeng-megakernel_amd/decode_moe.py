@@ -1,0 +1,67 @@
+"""Host step loop of the MoE ``mk`` route at batch 1: prefill-by-decode, greedy loop, timing.
+
+Same shape as the dense loop (``decode.py``; reference `qimeng_megakernel/models/LLM/decode.py:536-796`):
+one instruction tensor per request, per step the embedding row of the last token -> ``hidden_states``,
+``position_id = pos``, one kernel launch, ``argmax`` of the bf16 logits; one event pair per step around
+the launch only.
+"""
+from __future__ import annotations
+
+import time
+from typing import Any
+
+import torch
+
+from .decode_schedule_moe import mk_kernel as _mk_kernel
+from .decode_schedule_moe.model_config import QwenMoeConfig
+
+
+def decode(globs: Any, prompt_ids: torch.Tensor, max_new_tokens: int, *, mk: Any = None, decode_time: bool = True) -> dict[str, Any]:
+    """Prefill + forced greedy decode to exactly ``max_new_tokens`` tokens (no EOS stop)."""
+    device = globs.hidden_states.device
+    T = int(prompt_ids.numel())
+    if T + max_new_tokens > globs.k_cache.shape[2]:
+        raise ValueError("prompt_len + max_new_tokens exceeds the KV cache capacity")
+    mk = mk or _mk_kernel.get_mk()
+    globs.instructions = None
+    _mk_kernel.build(globs)
+    out = torch.zeros(T + max(max_new_tokens, 1), dtype=torch.long, device=device)
+    out[:T] = prompt_ids.to(device)
+    for pos in range(T):
+        globs.hidden_states.copy_(globs.embed_tokens[out[pos]])
+        globs.position_id = pos
+        _mk_kernel.call_mk(globs, mk)
+    out[T] = globs.logits.argmax()
+    ntok = max(max_new_tokens - 1, 0)
+    events = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(ntok if decode_time else 0)]
+    loop_start, loop_end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    torch.cuda.synchronize(device)
+    wall0 = time.perf_counter()
+    loop_start.record()
+    for i in range(ntok):
+        globs.hidden_states.copy_(globs.embed_tokens[out[T + i]])
+        globs.position_id = T + i
+        if events:
+            events[i][0].record()
+        _mk_kernel.call_mk(globs, mk)
+        if events:
+            events[i][1].record()
+        out[T + i + 1] = globs.logits.argmax()
+    loop_end.record()
+    torch.cuda.synchronize(device)
+    result: dict[str, Any] = {"generated_ids": out, "new_tokens": out[T:]}
+    if decode_time and ntok:
+        wall = time.perf_counter() - wall0
+        gpu_s = loop_start.elapsed_time(loop_end) / 1e3
+        per_step_ms = [a.elapsed_time(b) for a, b in events]
+        kernel_s = sum(per_step_ms) / 1e3
+        shape = QwenMoeConfig.shape()
+        nbytes = sum(shape.step_bytes(T + i + 1) for i in range(ntok))
+        result["timing"] = {
+            "decode_wall_s": wall, "decode_gpu_s": gpu_s, "mk_kernel_gpu_s": kernel_s,
+            "effective_tok_s_wall": ntok / wall, "effective_tok_s_gpu": ntok / gpu_s, "kernel_tok_s": ntok / kernel_s,
+            "kernel_steps": ntok, "kernel_ms_per_step": kernel_s * 1e3 / ntok, "algorithmic_bytes": nbytes,
+            "achieved_GBps": nbytes / kernel_s / 1e9, "per_step_ms": per_step_ms,
+        }
+    mk.check()
+    return result
