@@ -182,16 +182,24 @@ __device__ bool op_topk(const Params& p, Smem<M>& s, const Ctx& c) {
 template <class M>
 __device__ __forceinline__ void upgate_rows(Smem<M>& s, const Ctx& c, const u16* gate_w, const u16* up_w, int r0, int n, u16* dst0, u16* dst1) {
   const int lane = c.tid & 63, wave = c.tid >> 6;
-  for (int i = wave; i < n; i += 2 * kWaves) {
-    const int j = min(i + kWaves, n - 1);   // second output of this pass (repeats the first one's neighbour at the end)
-    const u16* const rows[4] = {gate_w + static_cast<size_t>(r0 + i) * M::H, up_w + static_cast<size_t>(r0 + i) * M::H,
-                                gate_w + static_cast<size_t>(r0 + j) * M::H, up_w + static_cast<size_t>(r0 + j) * M::H};
-    float v[4];
-    rows_dot<4>(rows, s.x, M::H, lane, v);
+  constexpr int kOut = 4;   // outputs (gate + up row each) of a wave in flight together: 32 KiB per wave
+  for (int i = wave; i < n; i += kOut * kWaves) {
+    int o[kOut];
+    const u16* rows[2 * kOut];
+#pragma unroll
+    for (int k = 0; k < kOut; ++k) {
+      o[k] = min(i + k * kWaves, n - 1);   // past the end: the last output once more, not stored
+      rows[2 * k] = gate_w + static_cast<size_t>(r0 + o[k]) * M::H;
+      rows[2 * k + 1] = up_w + static_cast<size_t>(r0 + o[k]) * M::H;
+    }
+    float v[2 * kOut];
+    rows_dot<2 * kOut>(rows, s.x, M::H, lane, v);
     if (lane == 0) {
-      const float g0 = round_bf16(v[0]), g1 = round_bf16(v[2]);
-      s.res[i] = (g0 / (1.0f + expf(-g0))) * round_bf16(v[1]);
-      if (i + kWaves < n) s.res[i + kWaves] = (g1 / (1.0f + expf(-g1))) * round_bf16(v[3]);
+#pragma unroll
+      for (int k = 0; k < kOut; ++k) {
+        const float g = round_bf16(v[2 * k]);
+        if (i + k * kWaves < n) s.res[o[k]] = (g / (1.0f + expf(-g))) * round_bf16(v[2 * k + 1]);
+      }
     }
   }
   __syncthreads();

@@ -51,6 +51,7 @@ class MoeScheduler:
     shape: MoeShape
     sm_count: int
     num_partials: int
+    interleave_experts: bool = False   # both up/gate phases before both down projections (the reference: 10, 11, 12, 13)
 
     def qkvproj(self, layer: int) -> list[Instruction]:
         tiles = _ceil_div(self.shape.qkv_out_dim, TILE_N_GRANULARITY)
@@ -111,9 +112,14 @@ class MoeScheduler:
         return [RMS_LMHead_GEMV(lo, hi) for lo, hi in _spans(tiles, self.sm_count)]
 
     def layer(self, layer: int) -> list[Instruction]:
-        return (self.qkvproj(layer) + self.attention_split_kv(layer) + self.attention_reduction(layer) + self.oproj(layer)
-                + self.router_gemv(layer) + self.router_softmax_topk(layer) + self.shared_upgate(layer) + self.shared_downproj(layer)
-                + self.routed_upgate(layer) + self.routed_downproj(layer) + self.combine_commit(layer))
+        head = (self.qkvproj(layer) + self.attention_split_kv(layer) + self.attention_reduction(layer) + self.oproj(layer)
+                + self.router_gemv(layer) + self.router_softmax_topk(layer))
+        if self.interleave_experts:
+            # the shared down projection's wait for all shared up/gate rows passes while the routed rows stream
+            experts = self.shared_upgate(layer) + self.routed_upgate(layer) + self.shared_downproj(layer) + self.routed_downproj(layer)
+        else:
+            experts = self.shared_upgate(layer) + self.shared_downproj(layer) + self.routed_upgate(layer) + self.routed_downproj(layer)
+        return head + experts + self.combine_commit(layer)
 
     def instruction_list(self, num_layers: int | None = None) -> list[Instruction]:
         layers = self.shape.num_hidden_layers if num_layers is None else num_layers

@@ -207,11 +207,11 @@ def call_mk(globs: Globals, mk: Any) -> None:
 
 
 def mi355x_scheduler(shape: Any = None) -> _scheduler.MoeScheduler:
-    """The reference's layout on one queue per CU."""
+    """The reference's tiles on one queue per CU, with both up/gate phases ahead of both down projections."""
     from .model_config import num_partials_for
 
     shape = shape or QwenMoeConfig.shape()
-    return _scheduler.MoeScheduler(shape, MI355X_QUEUES, num_partials_for(MI355X_QUEUES, shape))
+    return _scheduler.MoeScheduler(shape, MI355X_QUEUES, num_partials_for(MI355X_QUEUES, shape), interleave_experts=True)
 
 
 def build(globs: Globals) -> torch.Tensor:
