@@ -338,7 +338,7 @@ typedef struct QmkMoeArgs {
   void* workspace;                 /* qmk_moe_workspace_bytes(top_k, shared_k_slices) bytes, 128-byte aligned: the
                                       terms of the two in-place accumulations of the reference (shared_out over
                                       the K slices, routed_out_f32 over the expert slots), one slot per producer,
-                                      added by opcode 14 in the reference VM's order                            */
+                                      added by opcode 14 in the reference VM's order; and the layer's gate scalar */
   uint64_t workspace_bytes;
 } QmkMoeArgs;
 

@@ -126,6 +126,13 @@ class MoeInstructionVM:
         g.attn_lse_intermediates[h0:h1, ins.partial_idx] = lse
         g.attn_out_intermediates[h0:h1, ins.partial_idx] = out
         g.barriers[layer, 1][h0:h1] += 1
+        # extension of this build: the arrival that completes the KV head's counters merges its heads
+        if getattr(ins, "merge_in_last", 0) and int(g.barriers[layer, 1, h0]) == ins.num_partials:
+            idx = torch.arange(ins.num_partials)
+            lses, outs = g.attn_lse_intermediates[h0:h1][:, idx], g.attn_out_intermediates[h0:h1][:, idx]
+            wgt = (lses - lses.max(dim=-1, keepdim=True).values).exp2()
+            g.attn_out.view(s.num_attention_heads, -1)[h0:h1] = ((outs * wgt.unsqueeze(-1)).sum(dim=1) / wgt.sum(dim=-1, keepdim=True)).to(g.attn_out.dtype)
+            g.barriers[layer, 2, 0] += ratio
 
     def decode_attention_reduction(self, g: Any, ins: Any) -> None:
         s = self.shape

@@ -562,7 +562,7 @@ extern "C" int qmk_decode_step_batch(const QmkBatchArgs* a) {
 extern "C" uint64_t qmk_moe_workspace_bytes(int top_k, int shared_k_slices) {
   if (top_k < 1 || top_k > moe::kMaxTopK || shared_k_slices < 0 || shared_k_slices > 16) return 0;
   const uint64_t shared = static_cast<uint64_t>(shared_k_slices) * QwenMoeA2_7B::H * sizeof(u16);
-  return ((shared + 127) / 128) * 128 + static_cast<uint64_t>(top_k) * QwenMoeA2_7B::H * sizeof(float);
+  return ((shared + 127) / 128) * 128 + static_cast<uint64_t>(top_k) * QwenMoeA2_7B::H * sizeof(float) + 128;   // + the gate scalar's line
 }
 
 extern "C" int qmk_decode_step_moe(const QmkMoeArgs* a) {
@@ -655,6 +655,7 @@ extern "C" int qmk_decode_step_moe(const QmkMoeArgs* a) {
   p.shared_parts = static_cast<u16*>(a->workspace);
   const uint64_t shared_bytes = ((static_cast<uint64_t>(a->shared_k_slices) * M::H * sizeof(u16) + 127) / 128) * 128;
   p.routed_parts = reinterpret_cast<float*>(static_cast<char*>(a->workspace) + shared_bytes);
+  p.shared_gate = p.routed_parts + static_cast<size_t>(a->top_k) * M::H;
   p.num_experts = a->num_experts;
   p.top_k = a->top_k;
   p.shared_ffn = a->shared_ffn;

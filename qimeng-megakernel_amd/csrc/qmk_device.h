@@ -111,6 +111,7 @@ struct Params {
   u16* routed_out;               // [H]
   u16* shared_parts;             // workspace: [K slices, H] bf16 partial sums of the shared down projection
   float* routed_parts;           // workspace: [top_k, H] weighted contributions of the routed experts
+  float* shared_gate;            // workspace: the layer's sigmoid gate of the shared expert
   int32_t num_experts;
   int32_t top_k;
   int32_t shared_ffn;            // Fs

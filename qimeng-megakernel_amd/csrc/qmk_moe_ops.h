@@ -119,8 +119,17 @@ __device__ bool op_router(const Params& p, Smem<M>& s, const Ctx& c) {
     if (lane == 0) st_shared_f32(p.router_logits + e, v[0]);
   }
   const bool publish_row = s.inst[4] != 0;
-  if (publish_row)
+  if (publish_row) {
     for (int i = c.tid * 2; i < M::H; i += kThreads * 2) st_shared32(p.normed_hidden + i, *reinterpret_cast<const uint32_t*>(s.x + i));
+    // ... and the shared expert's gate, sigmoid(gate_w . normed) in fp32, which every combine instruction of the
+    // layer would otherwise recompute from the same row (python_vm.py:506-510)
+    if (wave == kWaves - 1) {
+      const u16* const rows[1] = {p.shared_scale_w + static_cast<size_t>(layer) * M::H};
+      float v[1];
+      rows_dot<1>(rows, s.x, M::H, lane, v);
+      if (lane == 0) st_shared_f32(p.shared_gate, 1.0f / (1.0f + expf(-v[0])));
+    }
+  }
   release_stores();
   __syncthreads();
   if (c.tid == 0) {
@@ -325,7 +334,7 @@ __device__ bool op_routed_down(const Params& p, Smem<M>& s, const Ctx& c) {
 
 // ==================================================================== 14 ==
 // [14, layer, n_start, n_end, tile_N_g]   (python_vm.py:492-530)
-// hidden[r] = bf16(hidden[r] + routed[r] + sigmoid(gate_w . normed) * shared[r]) for the rows of its tiles,
+// hidden[r] = bf16(hidden[r] + routed[r] + gate * shared[r]) for the rows of its tiles (gate: see opcode 8),
 // with shared = the K-slice terms added in bf16 in slice order and routed = the slots' terms added in
 // fp32 in slot order; leaves shared_out complete and routed_out_f32 cleared, as the VM does.
 template <class M>
@@ -348,15 +357,7 @@ __device__ bool op_combine(const Params& p, Smem<M>& s, const Ctx& c) {
   }
   __syncthreads();
   if (s.ctl[0]) return false;
-  stage_vector(s, c, p.normed_hidden, M::H);
-  if (c.tid < kWaveSize) {
-    const u16* const rows[1] = {p.shared_scale_w + static_cast<size_t>(layer) * M::H};
-    float v[1];
-    rows_dot<1>(rows, s.x, M::H, c.tid, v);
-    if (c.tid == 0) s.red[0] = 1.0f / (1.0f + expf(-v[0]));
-  }
-  __syncthreads();
-  const float gate = s.red[0];
+  const float gate = ld_shared_f32(p.shared_gate);   // left by the layer's publishing router instruction
   for (int pair = c.tid; pair < nb * tile / 2; pair += kThreads) {
     const int r = n0 * tile + 2 * pair;
     float sh0 = 0.f, sh1 = 0.f;

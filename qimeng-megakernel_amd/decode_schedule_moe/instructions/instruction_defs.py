@@ -64,6 +64,15 @@ class DecodeAttentionSplitKV(Instruction):
 
 
 @dataclass
+class DecodeAttentionSplitKVMerge(DecodeAttentionSplitKV):
+    """Extension of this build (same opcode, one more word): the instruction whose arrival completes its KV
+    head's counters also merges that head group's partials into ``attn_out`` and counts on the reduction row;
+    such a stream carries no reduction instructions."""
+
+    merge_in_last: int = 1
+
+
+@dataclass
 class DecodeAttentionReduction(Instruction):
     OPCODE: ClassVar[int] = 3
     PREV_OPCODES: ClassVar[tuple[int, ...]] = (2,)

@@ -15,6 +15,7 @@ from .instruction_defs import (
     TILE_N_GRANULARITY,
     DecodeAttentionReduction,
     DecodeAttentionSplitKV,
+    DecodeAttentionSplitKVMerge,
     MoE_Combine_Commit,
     OProj_GEMV_Residual,
     RMS_LMHead_GEMV,
@@ -52,16 +53,20 @@ class MoeScheduler:
     sm_count: int
     num_partials: int
     interleave_experts: bool = False   # both up/gate phases before both down projections (the reference: 10, 11, 12, 13)
+    merge_in_last: bool = False        # the last split-KV arrival of a KV head merges: no reduction instructions
 
     def qkvproj(self, layer: int) -> list[Instruction]:
         tiles = _ceil_div(self.shape.qkv_out_dim, TILE_N_GRANULARITY)
         return [RMS_QKVProj_GEMV_RoPE(layer, 0, lo, hi) for lo, hi in _spans(tiles, self.sm_count)]
 
     def attention_split_kv(self, layer: int) -> list[Instruction]:
-        return [DecodeAttentionSplitKV(layer, kvh, self.num_partials, part)
+        make = DecodeAttentionSplitKVMerge if self.merge_in_last else DecodeAttentionSplitKV
+        return [make(layer, kvh, self.num_partials, part)
                 for kvh in range(self.shape.num_key_value_heads) for part in range(self.num_partials)]
 
     def attention_reduction(self, layer: int) -> list[Instruction]:
+        if self.merge_in_last:
+            return []
         return [DecodeAttentionReduction(layer, h0, self.num_partials, list(range(self.num_partials)))
                 for h0 in range(0, self.shape.num_attention_heads, self.shape.attn_reduction_size)]
 

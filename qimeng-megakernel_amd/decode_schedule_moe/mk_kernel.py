@@ -207,11 +207,13 @@ def call_mk(globs: Globals, mk: Any) -> None:
 
 
 def mi355x_scheduler(shape: Any = None) -> _scheduler.MoeScheduler:
-    """The reference's tiles on one queue per CU, with both up/gate phases ahead of both down projections."""
+    """The reference's tiles on one queue per CU, with both up/gate phases ahead of both down projections and
+    the split-KV partials merged by the last arrival of each KV head (at most 25 partials)."""
     from .model_config import num_partials_for
 
     shape = shape or QwenMoeConfig.shape()
-    return _scheduler.MoeScheduler(shape, MI355X_QUEUES, num_partials_for(MI355X_QUEUES, shape), interleave_experts=True)
+    return _scheduler.MoeScheduler(shape, MI355X_QUEUES, min(25, num_partials_for(MI355X_QUEUES, shape)), interleave_experts=True,
+                                   merge_in_last=True)
 
 
 def build(globs: Globals) -> torch.Tensor:

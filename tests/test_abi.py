@@ -100,7 +100,7 @@ def test_host_side_argument_errors(lib):
     assert lib.qmk_decode_step_moe(ctypes.byref(m)) == 8                   # model 0 is not the MoE geometry
     m.model = 2
     assert lib.qmk_decode_step_moe(ctypes.byref(m)) == 1
-    assert lib.qmk_moe_workspace_bytes(4, 4) == 4 * 2048 * 2 + 4 * 2048 * 4 and lib.qmk_moe_workspace_bytes(9, 4) == 0
+    assert lib.qmk_moe_workspace_bytes(4, 4) == 4 * 2048 * 2 + 4 * 2048 * 4 + 128 and lib.qmk_moe_workspace_bytes(9, 4) == 0
     assert lib.qmk_error_string(12345).decode() == "unknown code"
 
 

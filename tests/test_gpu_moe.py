@@ -81,11 +81,12 @@ BF16_OUT = {"qkvproj": ("q_post_rope", "k_cache", "v_cache"), "attention_reducti
 def test_one_op_against_the_vm(weights, stage, position):
     """Everything before the op runs on the VM; the op itself on both, from identical state."""
     cpu, gpu = make_pair(weights, position=position)
-    sched = mk_kernel.mi355x_scheduler(SMALL)
+    sched = dataclasses.replace(mk_kernel.mi355x_scheduler(SMALL), merge_in_last=False)     # the reference's protocol, op by op
     vm = MoeInstructionVM(SMALL)
     name = STAGES[stage]
-    # the combine step adds up terms that the two down projections left in the launcher's workspace: those run on both sides too
-    first = STAGES.index("shared_downproj") if name == "combine_commit" else stage
+    # the combine step uses what the router (the gate) and the two down projections (their terms) left in the launcher's
+    # workspace: the whole MoE block runs on both sides then
+    first = STAGES.index("router_gemv") if name == "combine_commit" else stage
     for earlier in STAGES[:first]:
         vm.run(cpu, getattr(sched, earlier)(0))
     sync_state(cpu, gpu)
@@ -123,6 +124,23 @@ def test_one_op_against_the_vm(weights, stage, position):
         assert float((total - cpu.routed_out_f32).abs().max()) <= 2.0 ** -8 * float(cpu.routed_out_f32.abs().max())
     if name == "combine_commit":
         assert float(gpu.routed_out_f32.abs().max()) == 0.0 == float(cpu.routed_out_f32.abs().max())
+
+
+@pytest.mark.parametrize("position", [41, 0, 95])
+def test_split_kv_whose_last_arrival_merges(weights, position):
+    """The MI355X stream: no reduction instructions."""
+    cpu, gpu = make_pair(weights, position=position)
+    sched = mk_kernel.mi355x_scheduler(SMALL)
+    assert sched.merge_in_last and not sched.attention_reduction(0)
+    vm = MoeInstructionVM(SMALL)
+    vm.run(cpu, sched.qkvproj(0))
+    sync_state(cpu, gpu)
+    mine = sched.attention_split_kv(0)
+    assert all(i.padded()[5] == 1 for i in mine)
+    vm.run(cpu, copy.deepcopy(mine))
+    run_kernel(gpu, mine)
+    assert torch.equal(gpu.barriers.cpu(), cpu.barriers) and int(cpu.barriers[0, 2, 0]) == SMALL.num_attention_heads
+    bf16_close(gpu.attn_out, cpu.attn_out, name="attn_out")
 
 
 def test_lm_head_against_the_vm(weights):

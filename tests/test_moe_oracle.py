@@ -146,7 +146,10 @@ def test_vm_agrees_with_fused_and_counters_complete(weights):
         g.position_id = 41
         g.hidden_states.copy_(g.embed_tokens[99])
     FusedMoeOracle(SMALL).decode_step(f)
-    sched = S.MoeScheduler(SMALL, 256, num_partials_for(256, SMALL))          # any queue count: the VM is sequential
+    from qimeng_megakernel_amd.decode_schedule_moe.mk_kernel import mi355x_scheduler
+
+    sched = mi355x_scheduler(SMALL)          # 256 queues, expert phases interleaved, merge by the last split-KV arrival
+    assert not any(i.opcode() == 3 for i in sched.instruction_list())
     MoeInstructionVM(SMALL).run(v, sched.instruction_list())
     for name in ("q_post_rope", "attn_out", "hidden_states", "logits"):
         a, b = getattr(f, name).float(), getattr(v, name).float()
