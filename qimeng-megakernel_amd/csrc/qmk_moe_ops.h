@@ -227,8 +227,11 @@ __device__ bool op_shared_upgate(const Params& p, Smem<M>& s, const Ctx& c) {
   const int layer = s.inst[1], n0 = s.inst[3], n1 = s.inst[4], tile = s.inst[7];
   if (layer < 0 || layer >= p.num_layers) return bad_operand(p, s, c, 1);
   if (tile != kTile || n0 < 0 || n1 < n0 || n1 * tile > p.shared_ffn || (n1 - n0) * tile > kResSlots) return bad_operand(p, s, c, 4);
-  if (!wait_one(p, s, c, layer, ROW_ROUTER, 1, 1)) return false;
-  stage_vector(s, c, p.normed_hidden, M::H);
+  // The normalised row is recomputed here from the residual stream (the same function of the same values as
+  // the row opcode 8 publishes, bit for bit) instead of being waited for: the shared expert starts with the
+  // O-proj's last arrival, beside the router.
+  if (!wait_one(p, s, c, layer, ROW_OPROJ, 0, p.oproj_blocks)) return false;
+  if (!rms_to_lds<M>(p, s, c, nullptr, 0u, p.mlp_norm + static_cast<size_t>(layer) * M::H)) return false;
   const size_t base = static_cast<size_t>(layer) * p.shared_ffn * M::H;
   upgate_rows(s, c, p.shared_gate_w + base, p.shared_up_w + base, n0 * tile, (n1 - n0) * tile, p.shared_silu, nullptr);
   publish_done(p, c, layer, ROW_SHARED_UPGATE, 0, n1 - n0);
@@ -301,7 +304,7 @@ __device__ bool op_routed_upgate(const Params& p, Smem<M>& s, const Ctx& c) {
   if (!wait_one(p, s, c, layer, ROW_TOPK, 0, 1)) return false;
   const int eid = expert_of(p, slot);
   if (eid < 0) return bad_operand(p, s, c, 2);
-  stage_vector(s, c, p.normed_hidden, M::H);
+  if (!rms_to_lds<M>(p, s, c, nullptr, 0u, p.mlp_norm + static_cast<size_t>(layer) * M::H)) return false;   // as in opcode 10
   const u16* w = p.expert_gate_up_w + (static_cast<size_t>(layer) * p.num_experts + eid) * 2 * p.moe_ffn * M::H;
   upgate_rows(s, c, w, w + static_cast<size_t>(p.moe_ffn) * M::H, n0 * tile, (n1 - n0) * tile,
               p.routed_silu + static_cast<size_t>(slot) * p.moe_ffn, slot == p.top_k - 1 ? p.silu_out : nullptr);
