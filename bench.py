@@ -36,6 +36,8 @@ HBM_PEAK_GBPS = 8000.0
 # what the same counter reads for a 1 GiB copy) summarised in profiles/decode_megakernel_llama1b_hbm_counters.txt:
 # 1.0069 x the algorithmic bytes of the profiled launches.  Not measured in this process.
 MEASURED_TRAFFIC_OVER_ALGORITHMIC = 1.0069
+# The same for the batch route's kernel at batch 8 (profiles/decode_megakernel_batch_llama1b_hbm_counters.txt).
+MEASURED_TRAFFIC_OVER_ALGORITHMIC_BATCH8 = 1.0254
 
 
 def cpu_baseline(shape, weights, prompt, n_steps: int, cores: int, shape_name: str) -> dict:
@@ -116,6 +118,16 @@ def attention_stress(contexts=(4096, 16384, 32768)) -> dict:
     return out
 
 
+def copy_calibration(device) -> None:
+    """One 1 GiB device-to-device copy: a kernel of known traffic, for scaling rocprofv3's FETCH_SIZE / WRITE_SIZE."""
+    import torch
+
+    src = torch.empty(1 << 30, dtype=torch.uint8, device=device)
+    dst = torch.empty_like(src)
+    dst.copy_(src)
+    torch.cuda.synchronize(device)
+
+
 def batch_decode(args) -> dict:
     """B rows decoded together through the batch route's kernel: same request shape as the headline
     (seeded random-init weights, one random prompt per row, greedy continuation past EOS)."""
@@ -138,6 +150,8 @@ def batch_decode(args) -> dict:
     prompts = torch.stack([synthetic.random_prompt(shape, args.seed + r, args.prompt_len) for r in range(B)])
     globs = synthetic.build_batch_globals(weights, shape, kv_capacity, B, device)
     mk = mk_kernel.get_mk()
+    if args.copy_calibration:
+        copy_calibration(device)
     if args.warmup > 0:
         decode_batch.decode(globs, prompts, min(args.warmup + 1, new_tokens), mk=mk, decode_time=False)
     globs.k_cache.zero_(); globs.v_cache.zero_()
@@ -157,7 +171,9 @@ def batch_decode(args) -> dict:
         "first_tokens": out["new_tokens"][:, :4].tolist(),
         "roofline": {
             "bound": "hbm", "achieved": t["achieved_GBps"], "peak": HBM_PEAK_GBPS, "unit": "GB/s",
-            "frac": t["achieved_GBps"] / HBM_PEAK_GBPS, "traffic": None,
+            "frac": t["achieved_GBps"] / HBM_PEAK_GBPS,
+            # the counter runs were made at batch 8 only
+            "traffic": MEASURED_TRAFFIC_OVER_ALGORITHMIC_BATCH8 * t["algorithmic_bytes"] / max(args.steps, 1) if B == 8 else None,
             "bytes_per_launch_avg": t["algorithmic_bytes"] / max(args.steps, 1), "kernel": "decode_megakernel_batch<Llama1B>",
         },
     }
@@ -185,6 +201,8 @@ def moe_decode(args) -> dict:
     prompt = torch.randint(0, shape.vocab_size, (args.prompt_len,), generator=gen, dtype=torch.long)
     globs = synthetic.build_moe_globals(weights, shape, kv_capacity, device)
     mk = mk_kernel.get_mk()
+    if args.copy_calibration:
+        copy_calibration(device)
     if args.warmup > 0:
         decode_moe.decode(globs, prompt, min(args.warmup + 1, new_tokens), mk=mk, decode_time=False)
     globs.k_cache.zero_(); globs.v_cache.zero_()
