@@ -38,6 +38,8 @@ HBM_PEAK_GBPS = 8000.0
 MEASURED_TRAFFIC_OVER_ALGORITHMIC = 1.0069
 # The same for the batch route's kernel at batch 8 (profiles/decode_megakernel_batch_llama1b_hbm_counters.txt).
 MEASURED_TRAFFIC_OVER_ALGORITHMIC_BATCH8 = 1.0254
+# ... and for the MoE route's kernel (profiles/decode_megakernel_moe_qwen1p5_a2p7b_hbm_counters.txt).
+MEASURED_TRAFFIC_OVER_ALGORITHMIC_MOE = 1.0278
 
 
 def cpu_baseline(shape, weights, prompt, n_steps: int, cores: int, shape_name: str) -> dict:
@@ -223,7 +225,8 @@ def moe_decode(args) -> dict:
         "first_tokens": out["new_tokens"][:8].tolist(),
         "roofline": {
             "bound": "hbm", "achieved": t["achieved_GBps"], "peak": HBM_PEAK_GBPS, "unit": "GB/s", "frac": t["achieved_GBps"] / HBM_PEAK_GBPS,
-            "traffic": None, "bytes_per_launch_avg": t["algorithmic_bytes"] / max(args.steps, 1), "kernel": "decode_megakernel_moe<QwenMoeA2_7B>",
+            "traffic": MEASURED_TRAFFIC_OVER_ALGORITHMIC_MOE * t["algorithmic_bytes"] / max(args.steps, 1),
+            "bytes_per_launch_avg": t["algorithmic_bytes"] / max(args.steps, 1), "kernel": "decode_megakernel_moe<QwenMoeA2_7B>",
         },
     }
     if not args.no_cpu_baseline:
