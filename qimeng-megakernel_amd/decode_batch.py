@@ -42,10 +42,29 @@ def prefill_by_decode(globs: Any, mk: Any, prompts: torch.Tensor) -> torch.Tenso
     return globs.logits.argmax(dim=-1)
 
 
+def _argmax_rows(logits: torch.Tensor) -> torch.Tensor:
+    """First index of each row's maximum, in two short reductions (within runs of W columns, then over the
+    runs). One long reduction per row is spread over several workgroups by torch, with a counter that a memset
+    node clears, and such nodes have given wrong values on the replays of a captured graph after the first."""
+    rows, vocab = logits.shape
+    width = 1024
+    while width > 1 and vocab % width:
+        width //= 2
+    if width < 32:
+        return logits.argmax(dim=-1)
+    best, where = logits.view(rows, vocab // width, width).max(dim=-1)
+    run = best.argmax(dim=-1, keepdim=True)
+    return (run * width + where.gather(1, run)).squeeze(1)
+
+
 def decode(globs: Any, prompts: torch.Tensor, max_new_tokens: int, *, mk: Any = None, eos_token_ids: Sequence[int] = (),
-           decode_time: bool = True) -> dict[str, Any]:
+           decode_time: bool = True, use_graph: bool = False) -> dict[str, Any]:
     """Prefill + greedy decode of B rows to ``max_new_tokens`` tokens each (rows that hit an EOS token
-    of ``eos_token_ids`` retire; with none given every row runs to the end)."""
+    of ``eos_token_ids`` retire; with none given every row runs to the end).
+
+    ``use_graph``: the whole decode loop (embedding rows, kernel, argmax, row state) is captured into one
+    HIP graph and replayed once — the kernel reads positions and activity from device tensors, so nothing
+    in a step depends on the host.  Per-step kernel times are then not available."""
     from .decode import globs_shape
 
     device = globs.hidden_states.device
@@ -67,34 +86,69 @@ def decode(globs: Any, prompts: torch.Tensor, max_new_tokens: int, *, mk: Any = 
     globs.position_ids.fill_(T)
     _state.sync_kv_lengths(globs)
     ntok = max(max_new_tokens - 1, 0)
-    events = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(ntok if decode_time else 0)]
+    eos = None
+    if eos_token_ids:   # on the device before the loop: nothing inside a step comes from the host
+        eos = torch.tensor(list(eos_token_ids), dtype=torch.long, device=device)
+    timed = decode_time and not use_graph
+    events = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(ntok if timed else 0)]
     loop_start, loop_end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
     active_log = []
+
+    def steps() -> None:
+        for i in range(ntok):
+            _embed(globs, out[:, T + i])
+            if events:
+                events[i][0].record()
+            _mk_kernel.call_mk(globs, mk)
+            if events:
+                events[i][1].record()
+            nxt = _argmax_rows(globs.logits) if use_graph else globs.logits.argmax(dim=-1)
+            out[:, T + i + 1] = nxt
+            if eos is not None:
+                active_log.append(globs.active_mask.clone())
+            _state.advance_decode_state(globs, nxt, eos if eos is not None else ())
+
+    graph = None
+    first_token = out[:, T].clone()
+
+    def rewind() -> None:   # the state the prefill left: what a replay of the captured loop starts from
+        out[:, T] = first_token
+        globs.position_ids.fill_(T)
+        globs.active_mask.fill_(True)
+        globs.eos_reached.zero_()
+        _state.sync_kv_lengths(globs)
+
+    if use_graph and ntok:
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            steps()
+        rewind()   # capturing ran nothing, but the host-side bookkeeping of the loop did
     torch.cuda.synchronize(device)
     wall0 = time.perf_counter()
     loop_start.record()
-    for i in range(ntok):
-        _embed(globs, out[:, T + i])
-        if events:
-            events[i][0].record()
-        _mk_kernel.call_mk(globs, mk)
-        if events:
-            events[i][1].record()
-        nxt = globs.logits.argmax(dim=-1)
-        out[:, T + i + 1] = nxt
-        if eos_token_ids:
-            active_log.append(globs.active_mask.clone())
-        _state.advance_decode_state(globs, nxt, eos_token_ids)
+    if graph is not None:
+        graph.replay()
+    else:
+        steps()
     loop_end.record()
     torch.cuda.synchronize(device)
     result: dict[str, Any] = {"generated_ids": out, "new_tokens": out[:, T:]}
+    if graph is not None:
+        def replay(_inputs=(eos,)) -> torch.Tensor:
+            """The same request once more through the captured loop (the KV rows it wrote are simply written again).
+            ``_inputs`` keeps alive what the graph reads but was allocated outside its capture."""
+            rewind()
+            graph.replay()
+            return out[:, T:]
+
+        result["replay"] = replay
     if decode_time and ntok:
         wall = time.perf_counter() - wall0
         gpu_s = loop_start.elapsed_time(loop_end) / 1e3
         per_step_ms = [a.elapsed_time(b) for a, b in events]
-        kernel_s = sum(per_step_ms) / 1e3
+        kernel_s = sum(per_step_ms) / 1e3 if events else float("inf")
         shape = globs_shape(globs)
-        if eos_token_ids:
+        if eos is not None:
             rows = [int(m.sum()) for m in active_log]
         else:
             rows = [B] * ntok

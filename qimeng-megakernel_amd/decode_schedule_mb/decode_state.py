@@ -82,9 +82,9 @@ def advance_decode_state(globs: Any, next_tokens: torch.Tensor, eos_token_ids: S
     ensure_decode_state(globs, int(h.shape[0]), device)
     next_tokens = next_tokens.reshape(-1).to(device=device, dtype=torch.long)
     globs.last_generated_tokens.copy_(next_tokens)
-    if eos_token_ids:
-        eos = torch.tensor(list(eos_token_ids), dtype=torch.long, device=device)
-        hit = (next_tokens[:, None] == eos[None, :]).any(dim=1)
+    if isinstance(eos_token_ids, torch.Tensor) or eos_token_ids:
+        eos = eos_token_ids if isinstance(eos_token_ids, torch.Tensor) else torch.tensor(list(eos_token_ids), dtype=torch.long, device=device)
+        hit = (next_tokens[:, None] == eos.to(device=device, dtype=torch.long)[None, :]).any(dim=1)
     else:
         hit = torch.zeros_like(globs.active_mask)
     finished = globs.active_mask & hit

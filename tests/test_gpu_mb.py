@@ -300,6 +300,32 @@ def test_full_size_step_free_running(full_weights):
     assert int(gpu.barriers.abs().sum()) == 0
 
 
+def test_decode_loop_as_one_graph(weights):
+    """The whole loop of a request — embedding rows, kernel, argmax, row state with one row retiring on an EOS
+    token — captured into one HIP graph: the same tokens and row state as launch by launch, on three replays
+    with eager work between them."""
+    from qimeng_megakernel_amd import decode_batch
+
+    rows, new_tokens = 4, 12
+    g = synthetic.build_batch_globals(weights, MB_SMALL, FIX["kv_capacity"], rows, "cuda:0")
+    prompts = torch.stack([synthetic.random_prompt(MB_SMALL, 3 + r, 5) for r in range(rows)])
+    mk = mk_kernel.get_mk(spin_limit=1 << 18)
+    free = decode_batch.decode(g, prompts, new_tokens, mk=mk)["new_tokens"].clone()
+    eos = [int(free[2, 4])]                                  # row 2 retires after its fifth new token
+    eager = decode_batch.decode(g, prompts, new_tokens, mk=mk, eos_token_ids=eos)
+    want, want_active = eager["new_tokens"].clone(), g.active_mask.clone()
+    assert not bool(want_active[2]) and bool(want_active[0])
+    out = decode_batch.decode(g, prompts, new_tokens, mk=mk, eos_token_ids=eos, use_graph=True)
+    assert torch.equal(out["new_tokens"], want) and torch.equal(g.active_mask, want_active)
+    for _ in range(2):
+        g.logits.zero_()                                     # eager work between replays
+        torch.cuda.synchronize()
+        again = out["replay"]()
+        torch.cuda.synchronize()
+        mk.check()
+        assert torch.equal(again, want) and torch.equal(g.active_mask, want_active)
+
+
 def test_position_outside_the_cache_is_reported_not_executed(weights):
     cpu, gpu = make_pair(weights, 3, (70, 3, 130))
     gpu.position_ids[1] = FIX["kv_capacity"]          # one past the last cache row

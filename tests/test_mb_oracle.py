@@ -272,3 +272,16 @@ def test_mk_of_the_batch_route_checks_its_arguments(weights):
         mk_kernel.call_mk(g, mk)
     with pytest.raises(TypeError, match="positional arguments"):
         mk(g.instructions, g.hidden_states)
+
+
+def test_two_stage_argmax_is_the_first_maximum():
+    """The graph-safe argmax of the host loop returns what `argmax` does, ties included (first index wins)."""
+    from qimeng_megakernel_amd.decode_batch import _argmax_rows
+
+    gen = torch.Generator().manual_seed(11)
+    for vocab in (128256, 2048, 96, 1000):
+        logits = torch.randn(5, vocab, generator=gen).to(torch.bfloat16).float()
+        logits[1, 7] = logits[1, vocab - 3] = 9.0          # a tie across runs
+        logits[2, vocab // 2] = logits[2, vocab // 2 + 1] = 9.0   # a tie inside a run
+        want = torch.stack([torch.nonzero(r == r.max())[0, 0] for r in logits])
+        assert torch.equal(_argmax_rows(logits), want)
