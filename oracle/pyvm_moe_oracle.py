@@ -125,14 +125,22 @@ class MoeInstructionVM:
             out = torch.einsum("hk,ko->ho", torch.softmax(scores, dim=-1), v)
         g.attn_lse_intermediates[h0:h1, ins.partial_idx] = lse
         g.attn_out_intermediates[h0:h1, ins.partial_idx] = out
+        # extensions of this build (word 5; 0 in the reference's streams) --
+        mode = getattr(ins, "merge_in_last", 0)
+        if mode == 2:      # one arrival on the reduction row; the O-projection instructions merge
+            g.barriers[layer, 2, 0] += 1
+            return
         g.barriers[layer, 1][h0:h1] += 1
-        # extension of this build: the arrival that completes the KV head's counters merges its heads
-        if getattr(ins, "merge_in_last", 0) and int(g.barriers[layer, 1, h0]) == ins.num_partials:
-            idx = torch.arange(ins.num_partials)
-            lses, outs = g.attn_lse_intermediates[h0:h1][:, idx], g.attn_out_intermediates[h0:h1][:, idx]
-            wgt = (lses - lses.max(dim=-1, keepdim=True).values).exp2()
-            g.attn_out.view(s.num_attention_heads, -1)[h0:h1] = ((outs * wgt.unsqueeze(-1)).sum(dim=1) / wgt.sum(dim=-1, keepdim=True)).to(g.attn_out.dtype)
+        if mode == 1 and int(g.barriers[layer, 1, h0]) == ins.num_partials:   # the completing arrival merges its heads
+            self._merge_all(g, layer, h0, h1, ins.num_partials)
             g.barriers[layer, 2, 0] += ratio
+
+    def _merge_all(self, g: Any, layer: int, h0: int, h1: int, partials: int) -> None:
+        s = self.shape
+        idx = torch.arange(partials)
+        lses, outs = g.attn_lse_intermediates[h0:h1][:, idx], g.attn_out_intermediates[h0:h1][:, idx]
+        wgt = (lses - lses.max(dim=-1, keepdim=True).values).exp2()
+        g.attn_out.view(s.num_attention_heads, -1)[h0:h1] = ((outs * wgt.unsqueeze(-1)).sum(dim=1) / wgt.sum(dim=-1, keepdim=True)).to(g.attn_out.dtype)
 
     def decode_attention_reduction(self, g: Any, ins: Any) -> None:
         s = self.shape
@@ -154,7 +162,11 @@ class MoeInstructionVM:
     # ---- 4 -----------------------------------------------------------------------
     def oproj_gemv_residual(self, g: Any, ins: Any) -> None:
         s = self.shape
-        assert int(g.barriers[ins.layer_idx, 2, 0]) == s.num_attention_heads and ins.reduction_block_idx == 0
+        if ins.reduction_block_idx == 0:
+            assert int(g.barriers[ins.layer_idx, 2, 0]) == s.num_attention_heads
+        else:   # extension of this build: this instruction merges the split-KV partials of all heads itself
+            assert int(g.barriers[ins.layer_idx, 2, 0]) == s.num_key_value_heads * ins.reduction_block_idx
+            self._merge_all(g, ins.layer_idx, 0, s.num_attention_heads, ins.reduction_block_idx)
         hidden = g.hidden_states.reshape(-1)
         for blk in range(ins.tile_N_start_idx, ins.tile_N_end_idx):
             r0, r1 = blk * ins.tile_N_granularity, (blk + 1) * ins.tile_N_granularity

@@ -65,9 +65,11 @@ class DecodeAttentionSplitKV(Instruction):
 
 @dataclass
 class DecodeAttentionSplitKVMerge(DecodeAttentionSplitKV):
-    """Extension of this build (same opcode, one more word): the instruction whose arrival completes its KV
-    head's counters also merges that head group's partials into ``attn_out`` and counts on the reduction row;
-    such a stream carries no reduction instructions."""
+    """Extension of this build (same opcode, one more word), for streams without reduction instructions.
+    1: the instruction whose arrival completes its KV head's counters also merges that head group's partials
+    into ``attn_out`` and counts the heads on the reduction row.  2: the instruction counts one arrival on the
+    reduction row and nothing else; the O-projection instructions, whose ``reduction_block_idx`` then carries
+    the fan-out, merge the partials of all heads themselves."""
 
     merge_in_last: int = 1
 

@@ -54,29 +54,35 @@ class MoeScheduler:
     num_partials: int
     interleave_experts: bool = False   # both up/gate phases before both down projections (the reference: 10, 11, 12, 13)
     merge_in_last: bool = False        # the last split-KV arrival of a KV head merges: no reduction instructions
+    merge_in_oproj: bool = False       # every O-projection instruction merges all partials itself: no reduction instructions
+    router_span: int = 1               # experts per router instruction
 
     def qkvproj(self, layer: int) -> list[Instruction]:
         tiles = _ceil_div(self.shape.qkv_out_dim, TILE_N_GRANULARITY)
         return [RMS_QKVProj_GEMV_RoPE(layer, 0, lo, hi) for lo, hi in _spans(tiles, self.sm_count)]
 
     def attention_split_kv(self, layer: int) -> list[Instruction]:
-        make = DecodeAttentionSplitKVMerge if self.merge_in_last else DecodeAttentionSplitKV
+        if self.merge_in_oproj:
+            make = lambda *a: DecodeAttentionSplitKVMerge(*a, merge_in_last=2)
+        else:
+            make = DecodeAttentionSplitKVMerge if self.merge_in_last else DecodeAttentionSplitKV
         return [make(layer, kvh, self.num_partials, part)
                 for kvh in range(self.shape.num_key_value_heads) for part in range(self.num_partials)]
 
     def attention_reduction(self, layer: int) -> list[Instruction]:
-        if self.merge_in_last:
+        if self.merge_in_last or self.merge_in_oproj:
             return []
         return [DecodeAttentionReduction(layer, h0, self.num_partials, list(range(self.num_partials)))
                 for h0 in range(0, self.shape.num_attention_heads, self.shape.attn_reduction_size)]
 
     def oproj(self, layer: int) -> list[Instruction]:
-        return [OProj_GEMV_Residual(layer, 0, lo, hi, 0) for lo, hi in _spans(self.shape.num_hidden_blocks, self.sm_count)]
+        merges = self.num_partials if self.merge_in_oproj else 0
+        return [OProj_GEMV_Residual(layer, 0, lo, hi, merges) for lo, hi in _spans(self.shape.num_hidden_blocks, self.sm_count)]
 
     def router_gemv(self, layer: int) -> list[Instruction]:
         """One instruction per expert: the top-k waits for all of them."""
         e = self.shape.num_experts
-        return [Router_GEMV(layer, lo, hi, 1 if lo == 0 else 0) for lo, hi in _spans(e, e)]
+        return [Router_GEMV(layer, lo, hi, 1 if lo == 0 else 0) for lo, hi in _spans(e, _ceil_div(e, max(1, self.router_span)))]
 
     def router_softmax_topk(self, layer: int) -> list[Instruction]:
         return [Router_SoftmaxTopK(layer)]

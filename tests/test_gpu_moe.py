@@ -143,6 +143,27 @@ def test_split_kv_whose_last_arrival_merges(weights, position):
     bf16_close(gpu.attn_out, cpu.attn_out, name="attn_out")
 
 
+@pytest.mark.parametrize("position,partials", [(41, 3), (0, 2), (95, 6)])
+def test_oproj_that_merges_the_partials(weights, position, partials):
+    """The other stream without reduction instructions: split-KV instructions that only count their arrival,
+    O-projection instructions that merge the partials of all heads themselves."""
+    cpu, gpu = make_pair(weights, position=position)
+    sched = dataclasses.replace(mk_kernel.mi355x_scheduler(SMALL), merge_in_last=False, merge_in_oproj=True, num_partials=partials)
+    assert not sched.attention_reduction(0)
+    vm = MoeInstructionVM(SMALL)
+    vm.run(cpu, sched.qkvproj(0))
+    sync_state(cpu, gpu)
+    mine = sched.attention_split_kv(0) + sched.oproj(0)
+    assert all(i.padded()[5] == 2 for i in mine if i.opcode() == 2) and all(i.padded()[5] == partials for i in mine if i.opcode() == 4)
+    vm.run(cpu, copy.deepcopy(mine))
+    run_kernel(gpu, mine)
+    assert torch.equal(gpu.barriers.cpu(), cpu.barriers)
+    assert int(cpu.barriers[0, 2, 0]) == SMALL.num_key_value_heads * partials and int(cpu.barriers[0, 3, 0]) == SMALL.num_hidden_blocks
+    bf16_close(gpu.attn_out, cpu.attn_out, name="attn_out")
+    # each side multiplies its own merged attn_out (1 ulp apart at most) into the residual stream
+    bf16_close(gpu.hidden_states, cpu.hidden_states, ulps=2.0, frac=0.05, floor=2.0 ** -1, name="hidden_states")
+
+
 def test_lm_head_against_the_vm(weights):
     cpu, gpu = make_pair(weights)
     sched = mk_kernel.mi355x_scheduler(SMALL)
