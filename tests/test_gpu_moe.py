@@ -249,3 +249,90 @@ def test_full_geometry_layers_against_the_vm():
     run_kernel(gpu, sched.lmhead())
     rel_close(gpu.logits, cpu.logits, name="logits")
     assert int(gpu.logits.float().argmax()) == int(cpu.logits.float().argmax())
+
+
+# ---- error paths: forced from the host, every kernel still exits normally -----------------------------------------
+
+def _launch(gpu, instructions, **opts):
+    mk = mk_kernel.get_mk(reset_barriers=False, **opts)
+    mk_kernel.run_instructions(gpu, copy.deepcopy(instructions), mk=mk, queues=8)
+    return mk
+
+
+def test_wait_timeout_drains_the_grid_moe(weights):
+    """Routed up/gate instructions wait for a top-k that nobody runs: they run out of polls, say so and retire;
+    the next well-formed launch works (the reference hangs: decode_kernel/mk.cu has no bounded wait)."""
+    cpu, gpu = make_pair(weights)
+    sched = mk_kernel.mi355x_scheduler(SMALL)
+    mk = _launch(gpu, sched.routed_upgate(0)[:8], spin_limit=50)
+    with pytest.raises(RuntimeError, match="counter wait ran out of polls") as err:
+        mk.check()
+    assert "opcode=12" in str(err.value)
+    gpu.barriers.zero_()
+    vm = MoeInstructionVM(SMALL)
+    for stage in STAGES[: STAGES.index("oproj") + 1]:
+        vm.run(cpu, getattr(sched, stage)(0))
+    sync_state(cpu, gpu)
+    vm.run(cpu, sched.router_gemv(0))
+    run_kernel(gpu, sched.router_gemv(0))
+    assert torch.equal(gpu.barriers.cpu(), cpu.barriers)
+
+
+@pytest.mark.parametrize("bad, operand", [
+    (S.Router_GEMV(9, 0, 1, 0), 1),                                        # layer out of range
+    (S.Router_GEMV(0, 3, 2, 0), 2),                                        # experts end before they start
+    (S.Router_SoftmaxTopK(9), 1),
+    (S.SharedExpert_UpGate_SiLU(0, 0, 0, 4096, 0), 4),                     # rows beyond the shared expert's width
+    (S.SharedExpert_DownProj(0, 0, 0, 4096, 0), 4),                        # rows beyond the hidden size
+    (S.SharedExpert_DownProj(0, 0, 0, 1, 99), 5),                          # K slice beyond the launch's slices
+    (S.RoutedExpert_UpGate_SiLU(0, 8, 0, 1), 2),                           # expert slot beyond top-k
+    (S.RoutedExpert_UpGate_SiLU(0, 0, 0, 4096), 4),
+    (S.RoutedExpert_DownProj(0, 8, 0, 0, 1), 2),
+    (S.RoutedExpert_DownProj(0, 0, 0, 0, 4096), 5),
+    (S.MoE_Combine_Commit(0, 0, 4096), 3),
+])
+def test_bad_operands_are_rejected_on_the_device_moe(weights, bad, operand):
+    _, gpu = make_pair(weights)
+    before = {n: getattr(gpu, n).clone() for n in MUTABLE if n != "barriers"}
+    mk = _launch(gpu, [bad])
+    with pytest.raises(RuntimeError, match="operand out of bounds") as err:
+        mk.check()
+    assert f"opcode={bad.opcode()}" in str(err.value) and f"operand={operand}" in str(err.value)
+    for n, t in before.items():
+        assert torch.equal(getattr(gpu, n), t), n                           # nothing was written
+    assert int(gpu.barriers.abs().sum()) == 0
+
+
+def test_expert_index_outside_the_layer_is_rejected(weights):
+    """The routed ops take the physical expert from ``expert_indices`` at run time: a value no expert has
+    (a buffer the caller overwrote) is refused before any weight row is addressed."""
+    cpu, gpu = make_pair(weights)
+    gpu.expert_indices.fill_(SMALL.num_experts + 3)
+    gpu.barriers[0, 8, 0] = 1                                               # the top-k counts as done
+    gpu.barriers[0, 3, 0] = SMALL.num_hidden_blocks
+    before = gpu.routed_silu_buffer.clone()
+    mk = _launch(gpu, [S.RoutedExpert_UpGate_SiLU(0, 0, 0, 1)])
+    with pytest.raises(RuntimeError, match="operand out of bounds"):
+        mk.check()
+    assert torch.equal(gpu.routed_silu_buffer, before)
+
+
+def test_host_side_checks_moe(weights):
+    _, gpu = make_pair(weights)
+    mk = mk_kernel.get_mk()
+    mk_kernel.build(gpu)
+    gpu.position_id = FIX["kv_capacity"]
+    with pytest.raises(RuntimeError, match="pos_id outside"):
+        mk_kernel.call_mk(gpu, mk)
+    gpu.position_id = 3
+    keep = gpu.instructions
+    gpu.instructions = torch.zeros(4096, 1, 32, dtype=torch.int32, device="cuda:0")
+    with pytest.raises(RuntimeError, match="co-resident"):
+        mk_kernel.call_mk(gpu, mk)
+    gpu.instructions = keep
+    keep, gpu.barriers = gpu.barriers, gpu.barriers[:, :10].contiguous()    # the dense route's ten counter rows
+    with pytest.raises(ValueError, match="barriers must be"):
+        mk_kernel.call_mk(gpu, mk)
+    gpu.barriers = keep
+    mk_kernel.call_mk(gpu, mk)
+    mk.check()
