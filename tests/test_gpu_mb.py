@@ -336,3 +336,81 @@ def test_position_outside_the_cache_is_reported_not_executed(weights):
         mk.check()
     assert torch.equal(gpu.hidden_states, before)
     gpu.barriers.zero_()
+
+
+# ---- more error paths: forced from the host, every kernel still exits normally -------------------------------------
+
+def _launch(gpu, instructions, **opts):
+    mk = mk_kernel.get_mk(reset_barriers=False, **opts)
+    mk_kernel.run_instructions(gpu, copy.deepcopy(instructions), mk=mk, workers=8)
+    return mk
+
+
+def test_wait_timeout_drains_the_grid_batch(weights):
+    """O-projection tiles wait for attention heads that nobody merges: they run out of polls, say so and retire;
+    a well-formed launch afterwards works (the reference's kernel has no bounded wait)."""
+    cpu, gpu = make_pair(weights, 3, (70, 3, 130))
+    sched = S.mi355x_scheduler(3, MB_SMALL)
+    mk = _launch(gpu, sched.oproj(0)[:8], spin_limit=50)
+    with pytest.raises(RuntimeError, match="counter wait ran out of polls") as err:
+        mk.check()
+    assert "opcode=5" in str(err.value)
+    gpu.barriers.zero_()
+    first = sched.attn_rms(0)
+    vm_for(sched).run(cpu, copy.deepcopy(first))
+    run_kernel(gpu, first)
+    compare(cpu, gpu, ("attn_rms_out",))
+
+
+def _bad_batch_instructions():
+    from qimeng_megakernel_amd.decode_schedule_mb.instructions import instruction_defs as D
+
+    return [
+        (D.QKVProj_GEMM_RoPE(9, 3, 0, 0, 1), 1),                                   # layer out of range
+        (D.QKVProj_GEMM_RoPE(0, 5, 0, 0, 1), 2),                                   # not the launch's batch size
+        (D.QKVProj_GEMM_RoPE(0, 3, 0, 0, 4096), 4),                                # tiles beyond the QKV matrix
+        (D.QKVProj_GEMM_RoPE(0, 3, 0, 0, 1, tile_N_granularity=4), 7),             # a tile the kernel is not built for
+        (D.DecodeAttentionSplitKV(0, 7, 0, 1, 0), 2),                              # row beyond the batch
+        (D.DecodeAttentionSplitKV(0, 0, 99, 1, 0), 3),                             # kv head out of range
+        (D.DecodeAttentionSplitKV(0, 0, 0, 999, 0), 4),                            # more partials than the workspace holds
+        (D.DecodeAttentionReduction(0, 0, 999, 1, [0]), 3),                        # head group beyond the last head
+        (D.DecodeAttentionReduction(0, 0, 0, 1, [999]), 6),                        # partial index beyond the workspace
+        (D.OProj_GEMM_Residual(0, 3, 0, 0, 4096, 0), 4),
+        (D.UpGateProj_GEMM_SiLU(0, 3, 0, [1 << 20]), 5),                           # block beyond the intermediate size
+        (D.DownProj_GEMM_Residual(0, 3, 0, 0, 4096), 4),
+        (D.LMHeadProj_GEMM(3, 0, 1 << 20), 3),                                     # rows beyond the vocabulary
+    ]
+
+
+@pytest.mark.parametrize("case", range(13))
+def test_bad_operands_are_rejected_on_the_device_batch(weights, case):
+    bad, operand = _bad_batch_instructions()[case]
+    _, gpu = make_pair(weights, 3, (70, 3, 130))
+    names = ("hidden_states", "logits", "q_post_rope", "silu_out", "attn_out", "k_cache", "v_cache")
+    before = {n: getattr(gpu, n).clone() for n in names}
+    mk = _launch(gpu, [bad])
+    with pytest.raises(RuntimeError, match="operand out of bounds") as err:
+        mk.check()
+    assert f"opcode={bad.opcode()}" in str(err.value) and f"operand={operand}" in str(err.value)
+    for n, t in before.items():
+        assert torch.equal(getattr(gpu, n), t), n                                   # nothing was written
+    assert int(gpu.barriers.abs().sum()) == 0
+
+
+def test_host_side_checks_batch(weights):
+    _, gpu = make_pair(weights, 3, (70, 3, 130))
+    mk = mk_kernel.get_mk()
+    mk_kernel.build(gpu)
+    keep = gpu.instructions
+    gpu.instructions = torch.zeros(4096, 1, 32, dtype=torch.int32, device="cuda:0")
+    with pytest.raises(RuntimeError, match="co-resident"):
+        mk_kernel.call_mk(gpu, mk)
+    gpu.instructions = torch.zeros(4, 0, 32, dtype=torch.int32, device="cuda:0")
+    mk_kernel.call_mk(gpu, mk)                                                      # empty queues: nothing to launch
+    gpu.instructions = keep
+    keep, gpu.barriers = gpu.barriers, gpu.barriers[:, :7].contiguous()             # the batch-1 route's counter rows
+    with pytest.raises((RuntimeError, ValueError), match="barriers|dimension out of range"):
+        mk_kernel.call_mk(gpu, mk)
+    gpu.barriers = keep
+    mk_kernel.call_mk(gpu, mk)
+    mk.check()
