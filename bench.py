@@ -216,6 +216,9 @@ def moe_decode(args) -> dict:
     globs.k_cache.zero_(); globs.v_cache.zero_()
     out = decode_moe.decode(globs, prompt, new_tokens, mk=mk)
     t = out["timing"]
+    eager_tokens = out["new_tokens"].clone()
+    globs.k_cache.zero_(); globs.v_cache.zero_()
+    graphed = decode_moe.decode(globs, prompt, new_tokens, mk=mk, use_graph=True)   # the same loop as one HIP graph
     line = {
         "metric": "kernel_tok_s", "value": t["kernel_tok_s"], "unit": "tok/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": t["kernel_ms_per_step"], "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "bf16",
@@ -228,6 +231,8 @@ def moe_decode(args) -> dict:
             "queues": int(globs.instructions.shape[0]), "instructions_per_queue": int(globs.instructions.shape[1]),
         },
         "tok_s": t["effective_tok_s_wall"], "tok_s_gpu": t["effective_tok_s_gpu"], "kernel_tok_s": t["kernel_tok_s"],
+        "tok_s_gpu_graph": graphed["timing"]["effective_tok_s_gpu"],
+        "graph_tokens_equal": bool(torch.equal(graphed["new_tokens"], eager_tokens)),
         "first_tokens": out["new_tokens"][:8].tolist(),
         "roofline": {
             "bound": "hbm", "achieved": t["achieved_GBps"], "peak": HBM_PEAK_GBPS, "unit": "GB/s", "frac": t["achieved_GBps"] / HBM_PEAK_GBPS,

@@ -12,12 +12,18 @@ from typing import Any
 
 import torch
 
+from .decode_batch import _argmax_rows
 from .decode_schedule_moe import mk_kernel as _mk_kernel
 from .decode_schedule_moe.model_config import QwenMoeConfig
 
 
-def decode(globs: Any, prompt_ids: torch.Tensor, max_new_tokens: int, *, mk: Any = None, decode_time: bool = True) -> dict[str, Any]:
-    """Prefill + forced greedy decode to exactly ``max_new_tokens`` tokens (no EOS stop)."""
+def decode(globs: Any, prompt_ids: torch.Tensor, max_new_tokens: int, *, mk: Any = None, decode_time: bool = True,
+           use_graph: bool = False) -> dict[str, Any]:
+    """Prefill + forced greedy decode to exactly ``max_new_tokens`` tokens (no EOS stop).
+
+    ``use_graph``: the loop (embedding row, kernel, argmax, token write per step) is captured into one HIP graph
+    and replayed; the positions are launch arguments, so the graph belongs to this request.  The result then
+    carries ``replay``, which runs the same request once more through the graph."""
     device = globs.hidden_states.device
     T = int(prompt_ids.numel())
     if T + max_new_tokens > globs.k_cache.shape[2]:
@@ -33,28 +39,52 @@ def decode(globs: Any, prompt_ids: torch.Tensor, max_new_tokens: int, *, mk: Any
         _mk_kernel.call_mk(globs, mk)
     out[T] = globs.logits.argmax()
     ntok = max(max_new_tokens - 1, 0)
-    events = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(ntok if decode_time else 0)]
+    timed = decode_time and not use_graph
+    events = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(ntok if timed else 0)]
     loop_start, loop_end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+
+    def steps() -> None:
+        for i in range(ntok):
+            # a one-element index tensor: indexing with a 0-d tensor would read the token back to the host
+            globs.hidden_states.copy_(globs.embed_tokens.index_select(0, out[T + i : T + i + 1]).view(-1))
+            globs.position_id = T + i
+            if events:
+                events[i][0].record()
+            _mk_kernel.call_mk(globs, mk)
+            if events:
+                events[i][1].record()
+            # under capture: two short reductions instead of one long one, whose counter a memset node would clear
+            out[T + i + 1] = _argmax_rows(globs.logits.view(1, -1))[0] if use_graph else globs.logits.argmax()
+
+    graph = None
+    first_token = out[T].clone()
+    if use_graph and ntok:
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            steps()
     torch.cuda.synchronize(device)
     wall0 = time.perf_counter()
     loop_start.record()
-    for i in range(ntok):
-        globs.hidden_states.copy_(globs.embed_tokens[out[T + i]])
-        globs.position_id = T + i
-        if events:
-            events[i][0].record()
-        _mk_kernel.call_mk(globs, mk)
-        if events:
-            events[i][1].record()
-        out[T + i + 1] = globs.logits.argmax()
+    if graph is not None:
+        graph.replay()
+    else:
+        steps()
     loop_end.record()
     torch.cuda.synchronize(device)
     result: dict[str, Any] = {"generated_ids": out, "new_tokens": out[T:]}
+    if graph is not None:
+        def replay() -> torch.Tensor:
+            """The same request once more through the captured loop (the KV rows it wrote are written again)."""
+            out[T] = first_token
+            graph.replay()
+            return out[T:]
+
+        result["replay"] = replay
     if decode_time and ntok:
         wall = time.perf_counter() - wall0
         gpu_s = loop_start.elapsed_time(loop_end) / 1e3
         per_step_ms = [a.elapsed_time(b) for a, b in events]
-        kernel_s = sum(per_step_ms) / 1e3
+        kernel_s = sum(per_step_ms) / 1e3 if events else float("inf")
         shape = QwenMoeConfig.shape()
         nbytes = sum(shape.step_bytes(T + i + 1) for i in range(ntok))
         result["timing"] = {

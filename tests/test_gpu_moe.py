@@ -222,6 +222,28 @@ def test_request_of_the_reference_fixture(weights):
         assert token == rec["token"], step
 
 
+def test_decode_loop_as_one_graph_moe(weights):
+    """The request's loop (embedding row, kernel, argmax per step) as one HIP graph: the tokens of the loop run
+    launch by launch, on three replays with eager work between them."""
+    from qimeng_megakernel_amd import decode_moe
+
+    g = synthetic.build_moe_globals(weights, SMALL, FIX["kv_capacity"], "cuda:0")
+    gen = torch.Generator().manual_seed(17)
+    prompt = torch.randint(0, SMALL.vocab_size, (5,), generator=gen)
+    mk = mk_kernel.get_mk(spin_limit=1 << 18)
+    want = decode_moe.decode(g, prompt, 12, mk=mk)["new_tokens"].clone()
+    out = decode_moe.decode(g, prompt, 12, mk=mk, use_graph=True)
+    assert torch.equal(out["new_tokens"], want)
+    for _ in range(2):
+        g.logits.zero_()
+        g.hidden_states.zero_()
+        torch.cuda.synchronize()
+        again = out["replay"]()
+        torch.cuda.synchronize()
+        mk.check()
+        assert torch.equal(again, want)
+
+
 def test_full_geometry_layers_against_the_vm():
     """Qwen1.5-MoE-A2.7B layer geometry (60 experts of 1408, top-4, shared 5632), two layers, small vocabulary:
     layer by layer from the VM's residual stream, then the LM head."""
