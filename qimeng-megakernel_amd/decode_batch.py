@@ -42,7 +42,7 @@ def prefill_by_decode(globs: Any, mk: Any, prompts: torch.Tensor) -> torch.Tenso
     return globs.logits.argmax(dim=-1)
 
 
-def _argmax_rows(logits: torch.Tensor) -> torch.Tensor:
+def argmax_rows(logits: torch.Tensor) -> torch.Tensor:
     """First index of each row's maximum, in two short reductions (within runs of W columns, then over the
     runs). One long reduction per row is spread over several workgroups by torch, with a counter that a memset
     node clears, and such nodes have given wrong values on the replays of a captured graph after the first."""
@@ -102,7 +102,7 @@ def decode(globs: Any, prompts: torch.Tensor, max_new_tokens: int, *, mk: Any = 
             _mk_kernel.call_mk(globs, mk)
             if events:
                 events[i][1].record()
-            nxt = _argmax_rows(globs.logits) if use_graph else globs.logits.argmax(dim=-1)
+            nxt = argmax_rows(globs.logits) if use_graph else globs.logits.argmax(dim=-1)
             out[:, T + i + 1] = nxt
             if eos is not None:
                 active_log.append(globs.active_mask.clone())

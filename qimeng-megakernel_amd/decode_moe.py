@@ -12,7 +12,7 @@ from typing import Any
 
 import torch
 
-from .decode_batch import _argmax_rows
+from .decode_batch import argmax_rows
 from .decode_schedule_moe import mk_kernel as _mk_kernel
 from .decode_schedule_moe.model_config import QwenMoeConfig
 
@@ -54,7 +54,7 @@ def decode(globs: Any, prompt_ids: torch.Tensor, max_new_tokens: int, *, mk: Any
             if events:
                 events[i][1].record()
             # under capture: two short reductions instead of one long one, whose counter a memset node would clear
-            out[T + i + 1] = _argmax_rows(globs.logits.view(1, -1))[0] if use_graph else globs.logits.argmax()
+            out[T + i + 1] = argmax_rows(globs.logits.view(1, -1))[0] if use_graph else globs.logits.argmax()
 
     graph = None
     first_token = out[T].clone()

@@ -276,7 +276,7 @@ def test_mk_of_the_batch_route_checks_its_arguments(weights):
 
 def test_two_stage_argmax_is_the_first_maximum():
     """The graph-safe argmax of the host loop returns what `argmax` does, ties included (first index wins)."""
-    from qimeng_megakernel_amd.decode_batch import _argmax_rows
+    from qimeng_megakernel_amd.decode_batch import argmax_rows
 
     gen = torch.Generator().manual_seed(11)
     for vocab in (128256, 2048, 96, 1000):
@@ -284,4 +284,4 @@ def test_two_stage_argmax_is_the_first_maximum():
         logits[1, 7] = logits[1, vocab - 3] = 9.0          # a tie across runs
         logits[2, vocab // 2] = logits[2, vocab // 2 + 1] = 9.0   # a tie inside a run
         want = torch.stack([torch.nonzero(r == r.max())[0, 0] for r in logits])
-        assert torch.equal(_argmax_rows(logits), want)
+        assert torch.equal(argmax_rows(logits), want)
