@@ -275,7 +275,7 @@ int qmk_decode_step_batch(const QmkBatchArgs* args);
 typedef struct QmkMoeArgs {
   uint32_t struct_size;            /* = sizeof(QmkMoeArgs)                        */
   uint32_t model;                  /* QMK_MODEL_QWEN1_5_MOE_A2_7B                 */
-  uint32_t flags;                  /* 0 or QMK_FLAG_KEEP_BARRIERS                 */
+  uint32_t flags;                  /* QMK_FLAG_KEEP_BARRIERS, QMK_FLAG_TAGGED (whole steps, not with KEEP_BARRIERS) */
   uint32_t spin_limit;
 
   const int32_t* instructions;     /* int32 [num_queues, num_insts, 32]           */
@@ -338,7 +338,9 @@ typedef struct QmkMoeArgs {
   void* workspace;                 /* qmk_moe_workspace_bytes(top_k, shared_k_slices) bytes, 128-byte aligned: the
                                       terms of the two in-place accumulations of the reference (shared_out over
                                       the K slices, routed_out_f32 over the expert slots), one slot per producer,
-                                      added by opcode 14 in the reference VM's order; and the layer's gate scalar */
+                                      added by opcode 14 in the reference VM's order; the layer's gate scalar; and
+                                      the tagged units of QMK_FLAG_TAGGED (zeroed once when allocated, and again
+                                      after a launch that reported a device error)                              */
   uint64_t workspace_bytes;
 } QmkMoeArgs;
 

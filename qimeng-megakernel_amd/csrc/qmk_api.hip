@@ -249,7 +249,7 @@ __global__ __launch_bounds__(kThreads, 1) void decode_megakernel_moe(const Param
   __shared__ Smem<M> s;
   if (threadIdx.x < 8) s.ctl[threadIdx.x] = 0;
   if (threadIdx.x == 0) {
-    s.generation = 0u;
+    s.generation = tagged(p) ? ld_shared32(p.ws + kWsGeneration) : 0u;
     s.best_val = -INFINITY;
     s.best_idx = 0x7fffffff;
   }
@@ -324,6 +324,8 @@ __global__ __launch_bounds__(kThreads, 1) void decode_megakernel_moe(const Param
     const int total = p.num_layers * p.num_layer_barriers * p.barrier_slots;
     for (int i = threadIdx.x; i < total; i += kThreads)
       __hip_atomic_store(p.barriers + i, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    // The next launch tags its activations with the next count (26 bits: the tag keeps 6 for the layer).
+    if (tagged(p) && threadIdx.x == 0) st_shared32(p.ws + kWsGeneration, (s.generation + 1u) & 0x03ffffffu);
   }
 }
 
@@ -562,7 +564,9 @@ extern "C" int qmk_decode_step_batch(const QmkBatchArgs* a) {
 extern "C" uint64_t qmk_moe_workspace_bytes(int top_k, int shared_k_slices) {
   if (top_k < 1 || top_k > moe::kMaxTopK || shared_k_slices < 0 || shared_k_slices > 16) return 0;
   const uint64_t shared = static_cast<uint64_t>(shared_k_slices) * QwenMoeA2_7B::H * sizeof(u16);
-  return ((shared + 127) / 128) * 128 + static_cast<uint64_t>(top_k) * QwenMoeA2_7B::H * sizeof(float) + 128;   // + the gate scalar's line
+  // the down projections' terms, the gate scalar's line, then the tagged units of the residual stream and q/k/v
+  return ((shared + 127) / 128) * 128 + static_cast<uint64_t>(top_k) * QwenMoeA2_7B::H * sizeof(float) + 128 +
+         static_cast<uint64_t>(kWsUnits) * sizeof(uint64_t);
 }
 
 extern "C" int qmk_decode_step_moe(const QmkMoeArgs* a) {
@@ -588,7 +592,9 @@ extern "C" int qmk_decode_step_moe(const QmkMoeArgs* a) {
       a->shared_ffn < 16 || a->shared_ffn % 16 || a->moe_ffn < 16 || a->moe_ffn % 16 || a->moe_ffn > moe::kMaxK ||
       a->shared_k_slices < 1 || a->shared_k_slices > 16)
     return QMK_ERR_SHAPE;
-  if (a->flags & ~QMK_FLAG_KEEP_BARRIERS) return QMK_ERR_SHAPE;
+  if (a->flags & ~(QMK_FLAG_KEEP_BARRIERS | QMK_FLAG_TAGGED)) return QMK_ERR_SHAPE;
+  // tagged units carry the launch count, which the retiring launch advances, and six bits of layer
+  if ((a->flags & QMK_FLAG_TAGGED) && ((a->flags & QMK_FLAG_KEEP_BARRIERS) || a->num_layers > 63)) return QMK_ERR_SHAPE;
   if (a->pos_id < 0 || a->pos_id >= a->max_seq_len || a->pos_id >= a->rope_rows) return QMK_ERR_POSITION;
   if (reinterpret_cast<uintptr_t>(a->workspace) % 128 != 0 || a->workspace_bytes < qmk_moe_workspace_bytes(a->top_k, a->shared_k_slices))
     return QMK_ERR_SHAPE;
@@ -656,6 +662,7 @@ extern "C" int qmk_decode_step_moe(const QmkMoeArgs* a) {
   const uint64_t shared_bytes = ((static_cast<uint64_t>(a->shared_k_slices) * M::H * sizeof(u16) + 127) / 128) * 128;
   p.routed_parts = reinterpret_cast<float*>(static_cast<char*>(a->workspace) + shared_bytes);
   p.shared_gate = p.routed_parts + static_cast<size_t>(a->top_k) * M::H;
+  p.ws = reinterpret_cast<uint64_t*>(reinterpret_cast<char*>(p.shared_gate) + 128);
   p.num_experts = a->num_experts;
   p.top_k = a->top_k;
   p.shared_ffn = a->shared_ffn;

@@ -274,9 +274,9 @@ __device__ __forceinline__ v4u ld_shared128(const void* p) {
 constexpr int kWsGeneration = 0;            // launch count (first 128-byte line)
 constexpr int kWsQ = 512;                   // q after RoPE: NQ*D/2 units (two bf16 each)
 constexpr int kWsK = kWsQ + 1024;           // appended K row: NKV*D/2 units
-constexpr int kWsV = kWsK + 512;            // appended V row (regions sized for 8 KV heads of 128)
-constexpr int kWsHiddenMid = kWsV + 512;    // residual stream after the O-proj: H/2 units
-constexpr int kWsHiddenOut = kWsHiddenMid + 1024;  // residual stream after the down projection
+constexpr int kWsV = kWsK + 1024;           // appended V row (regions sized for 16 KV heads of 128)
+constexpr int kWsHiddenMid = kWsV + 1024;   // residual stream after the O-proj: H/2 units
+constexpr int kWsHiddenOut = kWsHiddenMid + 1024;  // residual stream after the down projection / the MoE combine step
 constexpr int kWsSilu = kWsHiddenOut + 1024;        // silu_out: F/2 units (room for F = 8192)
 constexpr int kWsCandidates = kWsSilu + 4096;       // one greedy candidate per workgroup: {logit bits, row}
 constexpr int kMaxSamplingQueues = 1024;

@@ -99,6 +99,18 @@ __device__ __forceinline__ void publish_done(const Params& p, const Ctx& c, int 
   if (c.tid == 0) publish(counter_ptr(p, layer, row, slot), amount);
 }
 
+// The layer's residual stream after the O-projection, normalised with the MLP norm weights, as bf16 in s.x.
+// With counters: after the O-projection's last arrival (`oproj_seen`: a counter the caller has waited on
+// already implies it), from the caller's buffer.  Tagged launch: from the units the O-projection workgroups
+// announce their rows in, each thread polling its own two.
+template <class M>
+__device__ __forceinline__ bool residual_to_lds(const Params& p, Smem<M>& s, const Ctx& c, int layer, bool oproj_seen = false) {
+  const u16* weight = p.mlp_norm + static_cast<size_t>(layer) * M::H;
+  if (tagged(p)) return rms_to_lds<M>(p, s, c, p.ws + kWsHiddenMid, tag_of(s.generation, layer), weight);
+  if (!oproj_seen && !wait_one(p, s, c, layer, ROW_OPROJ, 0, p.oproj_blocks)) return false;
+  return rms_to_lds<M>(p, s, c, nullptr, 0u, weight);
+}
+
 // ===================================================================== 8 ==
 // [8, layer, e_start, e_end, write_normed_hidden, tile_N_g]
 // RMSNorm of the residual stream, fp32 router logits of experts [e_start, e_end); one instruction of a
@@ -108,8 +120,7 @@ __device__ bool op_router(const Params& p, Smem<M>& s, const Ctx& c) {
   const int layer = s.inst[1], g = s.inst[5], e0 = s.inst[2] * g, e1 = min(s.inst[3] * g, p.num_experts);
   if (layer < 0 || layer >= p.num_layers) return bad_operand(p, s, c, 1);
   if (g < 1 || e0 < 0 || e1 < e0) return bad_operand(p, s, c, 2);
-  if (!wait_one(p, s, c, layer, ROW_OPROJ, 0, p.oproj_blocks)) return false;
-  if (!rms_to_lds<M>(p, s, c, nullptr, 0u, p.mlp_norm + static_cast<size_t>(layer) * M::H)) return false;
+  if (!residual_to_lds<M>(p, s, c, layer)) return false;
   const int lane = c.tid & 63, wave = c.tid >> 6;
   const u16* w = p.router_w + static_cast<size_t>(layer) * p.num_experts * M::H;
   for (int e = e0 + wave; e < e1; e += kWaves) {
@@ -230,8 +241,7 @@ __device__ bool op_shared_upgate(const Params& p, Smem<M>& s, const Ctx& c) {
   // The normalised row is recomputed here from the residual stream (the same function of the same values as
   // the row opcode 8 publishes, bit for bit) instead of being waited for: the shared expert starts with the
   // O-proj's last arrival, beside the router.
-  if (!wait_one(p, s, c, layer, ROW_OPROJ, 0, p.oproj_blocks)) return false;
-  if (!rms_to_lds<M>(p, s, c, nullptr, 0u, p.mlp_norm + static_cast<size_t>(layer) * M::H)) return false;
+  if (!residual_to_lds<M>(p, s, c, layer)) return false;
   const size_t base = static_cast<size_t>(layer) * p.shared_ffn * M::H;
   upgate_rows(s, c, p.shared_gate_w + base, p.shared_up_w + base, n0 * tile, (n1 - n0) * tile, p.shared_silu, nullptr);
   publish_done(p, c, layer, ROW_SHARED_UPGATE, 0, n1 - n0);
@@ -304,7 +314,7 @@ __device__ bool op_routed_upgate(const Params& p, Smem<M>& s, const Ctx& c) {
   if (!wait_one(p, s, c, layer, ROW_TOPK, 0, 1)) return false;
   const int eid = expert_of(p, slot);
   if (eid < 0) return bad_operand(p, s, c, 2);
-  if (!rms_to_lds<M>(p, s, c, nullptr, 0u, p.mlp_norm + static_cast<size_t>(layer) * M::H)) return false;   // as in opcode 10
+  if (!residual_to_lds<M>(p, s, c, layer, /*oproj_seen=*/true)) return false;   // as in opcode 10
   const u16* w = p.expert_gate_up_w + (static_cast<size_t>(layer) * p.num_experts + eid) * 2 * p.moe_ffn * M::H;
   upgate_rows(s, c, w, w + static_cast<size_t>(p.moe_ffn) * M::H, n0 * tile, (n1 - n0) * tile,
               p.routed_silu + static_cast<size_t>(slot) * p.moe_ffn, slot == p.top_k - 1 ? p.silu_out : nullptr);
@@ -360,6 +370,8 @@ __device__ bool op_combine(const Params& p, Smem<M>& s, const Ctx& c) {
   }
   __syncthreads();
   if (s.ctl[0]) return false;
+  const bool tg = tagged(p);
+  const uint32_t tag = tag_of(s.generation, layer);
   const float gate = ld_shared_f32(p.shared_gate);   // left by the layer's publishing router instruction
   for (int pair = c.tid; pair < nb * tile / 2; pair += kThreads) {
     const int r = n0 * tile + 2 * pair;
@@ -374,12 +386,22 @@ __device__ bool op_combine(const Params& p, Smem<M>& s, const Ctx& c) {
       ro0 += ld_shared_f32(p.routed_parts + static_cast<size_t>(j) * M::H + r);
       ro1 += ld_shared_f32(p.routed_parts + static_cast<size_t>(j) * M::H + r + 1);
     }
-    const uint32_t old = ld_shared32(p.hidden + r);
+    uint32_t old = 0;
+    if (!residual_in(p, tg ? p.ws + kWsHiddenMid : nullptr, tag, 0, r / 2, old)) {   // its tag has been seen by every up/gate workgroup
+      s.ctl[0] = 1;
+      report_error(p, QMK_DEV_WAIT_TIMEOUT, c.inst_idx, c.opcode, c.tid);
+    }
     const float h0 = (bf_lo(old) + ro0) + gate * sh0, h1 = (bf_hi(old) + ro1) + gate * sh1;
-    st_shared32(p.hidden + r, static_cast<uint32_t>(f2bf(h0)) | (static_cast<uint32_t>(f2bf(h1)) << 16));
+    const uint32_t word = static_cast<uint32_t>(f2bf(h0)) | (static_cast<uint32_t>(f2bf(h1)) << 16);
+    st_shared32(p.hidden + r, word);
+    if (tg) st_tagged(p.ws + kWsHiddenOut + r / 2, word, tag);   // the next layer's QKV and O-projection, the LM head
     st_shared32(p.shared_out + r, static_cast<uint32_t>(f2bf(sh0)) | (static_cast<uint32_t>(f2bf(sh1)) << 16));
     st_shared_f32(p.routed_out_f32 + r, 0.f);
     st_shared_f32(p.routed_out_f32 + r + 1, 0.f);
+  }
+  if (tg) {   // the units announce themselves: nothing to count
+    __syncthreads();
+    return s.ctl[0] == 0;
   }
   publish_done(p, c, layer, ROW_COMBINE, 0, nb);
   return true;

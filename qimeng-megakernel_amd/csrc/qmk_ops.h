@@ -561,18 +561,20 @@ __device__ bool op_attn_splitkv(const Params& p, Smem<M>& s, const Ctx& c) {
   constexpr int kQ = 0, kK = GQA * D, kV = GQA * D + D;
   const size_t new_row = row_of_kvh + static_cast<size_t>(p.pos_id) * tok_stride;
   if (tg) {
-    // q: GQA*D/2 = 128 units, two per thread of wave 0; K and V: D/2 units each, two per thread.
+    // q: GQA*D/2 units, two per thread of the first GQA*D/4 threads; K and V: D/2 units each, two per thread.
+    constexpr int kQThreads = GQA * D / 4;
+    static_assert(kQThreads + D / 2 <= kThreads, "one poller per unit pair");
     const uint32_t tag = tag_of(s.generation, layer);
     uint32_t* words = reinterpret_cast<uint32_t*>(stage16);
     bool arrived = true;
     uint32_t a = 0, b = 0;
     const int tid = c.tid;
-    if (tid < 64) {
+    if (tid < kQThreads) {
       arrived = poll_tagged2(p.ws + kWsQ + kvh * (GQA * D / 2) + 2 * tid, tag, p.spin_limit, a, b);
       words[kQ / 2 + 2 * tid] = a;
       words[kQ / 2 + 2 * tid + 1] = b;
-    } else if (tid < 64 + D / 2 && has_new) {
-      const int j = tid - 64;                              // [0, D/4): K, [D/4, D/2): V
+    } else if (tid < kQThreads + D / 2 && has_new) {
+      const int j = tid - kQThreads;                       // [0, D/4): K, [D/4, D/2): V
       const bool is_v = j >= D / 4;
       const int u = 2 * (is_v ? j - D / 4 : j);
       arrived = poll_tagged2(p.ws + (is_v ? kWsV : kWsK) + kvh * (D / 2) + u, tag, p.spin_limit, a, b);

@@ -222,6 +222,41 @@ def test_request_of_the_reference_fixture(weights):
         assert token == rec["token"], step
 
 
+def _request_both_ways(weights, shape, capacity, steps):
+    """The same greedy request on two sets of buffers: through counters only, then with tagged hand-over."""
+    from qimeng_megakernel_amd import decode_moe
+
+    gen = torch.Generator().manual_seed(23)
+    prompt = torch.randint(0, shape.vocab_size, (4,), generator=gen)
+    out = []
+    for tagged in (False, True):
+        g = synthetic.build_moe_globals(weights, shape, capacity, "cuda:0")
+        mk = mk_kernel.get_mk(tagged=tagged, spin_limit=1 << 18)
+        toks = decode_moe.decode(g, prompt, steps, mk=mk, decode_time=False)["new_tokens"].clone()
+        assert mk._tagged == tagged
+        out.append((g, toks))
+    return out
+
+
+def test_tagged_and_counter_modes_agree_bit_for_bit(weights):
+    """Tagged hand-over changes how values travel, not the values: every buffer of the request is identical."""
+    (plain, toks_p), (tagged, toks_t) = _request_both_ways(weights, SMALL, FIX["kv_capacity"], 24)
+    assert torch.equal(toks_p, toks_t)
+    for name in MUTABLE:
+        assert torch.equal(getattr(plain, name), getattr(tagged, name)), name
+    assert int(tagged.barriers.abs().sum()) == 0
+
+
+def test_tagged_and_counter_modes_agree_full_geometry():
+    shape = dataclasses.replace(QWEN1_5_MOE_A2_7B, num_hidden_layers=3, vocab_size=4096)
+    QwenMoeConfig.set_shape(shape)
+    w = synthetic.random_moe_weights(shape, 4, 40)
+    (plain, toks_p), (tagged, toks_t) = _request_both_ways(w, shape, 40, 10)
+    assert torch.equal(toks_p, toks_t)
+    for name in MUTABLE:
+        assert torch.equal(getattr(plain, name), getattr(tagged, name)), name
+
+
 def test_decode_loop_as_one_graph_moe(weights):
     """The request's loop (embedding row, kernel, argmax per step) as one HIP graph: the tokens of the loop run
     launch by launch, on three replays with eager work between them."""
