@@ -278,20 +278,22 @@ __global__ __launch_bounds__(kThreads, 1) void decode_megakernel_moe(const Param
       for (int k = 0; k < 4; ++k) s.stamps[k] = t_start;
     }
     bool carried = false;
+    // Every op inlined, whatever its size: an op left out of line takes `p` by reference, and the kernel
+    // arguments then live in private memory for all ops (vector loads from scratch instead of scalar loads).
     switch (opcode) {
       case OP_NOOP: break;
-      case OP_RMS_QKV_ROPE: ok = op_rms_qkv_rope<M>(p, s, c); break;
-      case OP_ATTN_SPLITKV: ok = op_attn_splitkv<M>(p, s, c); break;
-      case OP_ATTN_REDUCE: ok = op_attn_reduce<M>(p, s, c); break;
-      case OP_OPROJ_RESIDUAL: ok = op_oproj_residual<M>(p, s, c, carry, carried); break;
-      case OP_RMS_LMHEAD: ok = op_rms_lmhead<M>(p, s, c); break;
-      case moe::OP_ROUTER: ok = moe::op_router<M>(p, s, c); break;
-      case moe::OP_TOPK: ok = moe::op_topk<M>(p, s, c); break;
-      case moe::OP_SHARED_UPGATE: ok = moe::op_shared_upgate<M>(p, s, c); break;
-      case moe::OP_SHARED_DOWN: ok = moe::op_shared_down<M>(p, s, c); break;
-      case moe::OP_ROUTED_UPGATE: ok = moe::op_routed_upgate<M>(p, s, c); break;
-      case moe::OP_ROUTED_DOWN: ok = moe::op_routed_down<M>(p, s, c); break;
-      case moe::OP_COMBINE: ok = moe::op_combine<M>(p, s, c); break;
+      case OP_RMS_QKV_ROPE: [[clang::always_inline]] ok = op_rms_qkv_rope<M>(p, s, c); break;
+      case OP_ATTN_SPLITKV: [[clang::always_inline]] ok = op_attn_splitkv<M>(p, s, c); break;
+      case OP_ATTN_REDUCE: [[clang::always_inline]] ok = op_attn_reduce<M>(p, s, c); break;
+      case OP_OPROJ_RESIDUAL: [[clang::always_inline]] ok = op_oproj_residual<M>(p, s, c, carry, carried); break;
+      case OP_RMS_LMHEAD: [[clang::always_inline]] ok = op_rms_lmhead<M>(p, s, c); break;
+      case moe::OP_ROUTER: [[clang::always_inline]] ok = moe::op_router<M>(p, s, c); break;
+      case moe::OP_TOPK: [[clang::always_inline]] ok = moe::op_topk<M>(p, s, c); break;
+      case moe::OP_SHARED_UPGATE: [[clang::always_inline]] ok = moe::op_shared_upgate<M>(p, s, c); break;
+      case moe::OP_SHARED_DOWN: [[clang::always_inline]] ok = moe::op_shared_down<M>(p, s, c); break;
+      case moe::OP_ROUTED_UPGATE: [[clang::always_inline]] ok = moe::op_routed_upgate<M>(p, s, c); break;
+      case moe::OP_ROUTED_DOWN: [[clang::always_inline]] ok = moe::op_routed_down<M>(p, s, c); break;
+      case moe::OP_COMBINE: [[clang::always_inline]] ok = moe::op_combine<M>(p, s, c); break;
       default:
         if (threadIdx.x == 0) report_error(p, QMK_DEV_BAD_OPCODE, i, opcode, 0);
         ok = false;

@@ -60,25 +60,24 @@ constexpr int kTile = 16;
 template <int NR>
 __device__ __forceinline__ void rows_dot(const u16* const (&rows)[NR], const u16* x, int K, int lane, float (&out)[NR]) {
   constexpr int NI = kMaxK / 512;
+  // Indices that are constants already in the source (static_for, not unrolled loops): the pieces are
+  // registers however the optimiser treats the loops around this function.
   v4u w[NR][NI];
-#pragma unroll
-  for (int r = 0; r < NR; ++r)
-#pragma unroll
-    for (int i = 0; i < NI; ++i) {
+  static_for<0, NR>([&](auto r) {
+    static_for<0, NI>([&](auto i) {
       const int col = lane * 8 + i * 512;
       w[r][i] = v4u{0, 0, 0, 0};
       if (col < K) w[r][i] = __builtin_nontemporal_load(reinterpret_cast<const v4u*>(rows[r] + col));
-    }
-#pragma unroll
-  for (int r = 0; r < NR; ++r) {
+    });
+  });
+  static_for<0, NR>([&](auto r) {
     float a = 0.f;
-#pragma unroll
-    for (int i = 0; i < NI; ++i) {
+    static_for<0, NI>([&](auto i) {
       const int col = lane * 8 + i * 512;
       if (col < K) a = dot8(w[r][i], *reinterpret_cast<const v4u*>(x + col), a);
-    }
+    });
     out[r] = wave_sum(a);
-  }
+  });
 }
 
 // n bf16 elements (a multiple of 4) of a vector that another workgroup wrote during this launch, into s.x.
@@ -116,7 +115,7 @@ __device__ __forceinline__ bool residual_to_lds(const Params& p, Smem<M>& s, con
 // RMSNorm of the residual stream, fp32 router logits of experts [e_start, e_end); one instruction of a
 // layer also publishes the normalised row for opcodes 10, 12 and 14   (python_vm.py:331-357).
 template <class M>
-__device__ bool op_router(const Params& p, Smem<M>& s, const Ctx& c) {
+__device__ __forceinline__ bool op_router(const Params& p, Smem<M>& s, const Ctx& c) {
   const int layer = s.inst[1], g = s.inst[5], e0 = s.inst[2] * g, e1 = min(s.inst[3] * g, p.num_experts);
   if (layer < 0 || layer >= p.num_layers) return bad_operand(p, s, c, 1);
   if (g < 1 || e0 < 0 || e1 < e0) return bad_operand(p, s, c, 2);
@@ -154,7 +153,7 @@ __device__ bool op_router(const Params& p, Smem<M>& s, const Ctx& c) {
 // [9, layer]   softmax over all router logits, the top_k largest probabilities and their experts, in
 // decreasing order (ties: the lower expert first), not renormalised   (python_vm.py:360-372).
 template <class M>
-__device__ bool op_topk(const Params& p, Smem<M>& s, const Ctx& c) {
+__device__ __forceinline__ bool op_topk(const Params& p, Smem<M>& s, const Ctx& c) {
   const int layer = s.inst[1], E = p.num_experts;
   if (layer < 0 || layer >= p.num_layers) return bad_operand(p, s, c, 1);
   if (!wait_one(p, s, c, layer, ROW_ROUTER, 0, E)) return false;
@@ -234,7 +233,7 @@ __device__ __forceinline__ void upgate_rows(Smem<M>& s, const Ctx& c, const u16*
 // [10, layer, tile_M, n_start, n_end, init_shared_out, tile_M_g, tile_N_g]   (python_vm.py:375-396)
 // shared_out needs no clearing here: its K-slice terms have slots of their own until the combine step.
 template <class M>
-__device__ bool op_shared_upgate(const Params& p, Smem<M>& s, const Ctx& c) {
+__device__ __forceinline__ bool op_shared_upgate(const Params& p, Smem<M>& s, const Ctx& c) {
   const int layer = s.inst[1], n0 = s.inst[3], n1 = s.inst[4], tile = s.inst[7];
   if (layer < 0 || layer >= p.num_layers) return bad_operand(p, s, c, 1);
   if (tile != kTile || n0 < 0 || n1 < n0 || n1 * tile > p.shared_ffn || (n1 - n0) * tile > kResSlots) return bad_operand(p, s, c, 4);
@@ -275,7 +274,7 @@ __device__ __forceinline__ void down_rows(Smem<M>& s, const Ctx& c, const u16* w
 // [11, layer, tile_M, n_start, n_end, split_K_idx, tile_M_g, tile_N_g, split_K_g]   (python_vm.py:399-418)
 // One K slice of the shared down projection: bf16(W[r, k0:k1] . silu[k0:k1]) into this slice's slot.
 template <class M>
-__device__ bool op_shared_down(const Params& p, Smem<M>& s, const Ctx& c) {
+__device__ __forceinline__ bool op_shared_down(const Params& p, Smem<M>& s, const Ctx& c) {
   const int layer = s.inst[1], n0 = s.inst[3], n1 = s.inst[4], slice = s.inst[5], tile = s.inst[7], kg = s.inst[8];
   if (layer < 0 || layer >= p.num_layers) return bad_operand(p, s, c, 1);
   if (tile != kTile || n0 < 0 || n1 < n0 || n1 * tile > M::H) return bad_operand(p, s, c, 4);
@@ -306,7 +305,7 @@ __device__ __forceinline__ int expert_of(const Params& p, int slot) {
 // [12, layer, expert_slot, n_start, n_end, tile_M_g, tile_N_g]   (python_vm.py:421-464)
 // The single buffer silu_out keeps what the last slot wrote, as after the VM's sequential run.
 template <class M>
-__device__ bool op_routed_upgate(const Params& p, Smem<M>& s, const Ctx& c) {
+__device__ __forceinline__ bool op_routed_upgate(const Params& p, Smem<M>& s, const Ctx& c) {
   const int layer = s.inst[1], slot = s.inst[2], n0 = s.inst[3], n1 = s.inst[4], tile = s.inst[6];
   if (layer < 0 || layer >= p.num_layers) return bad_operand(p, s, c, 1);
   if (slot < 0 || slot >= p.top_k) return bad_operand(p, s, c, 2);
@@ -326,7 +325,7 @@ __device__ bool op_routed_upgate(const Params& p, Smem<M>& s, const Ctx& c) {
 // [13, layer, expert_slot, tile_M, n_start, n_end, tile_M_g, tile_N_g]   (python_vm.py:467-489)
 // bf16(W_down[expert][r] . silu[slot]) * weight[slot], fp32, into the slot's own row of the workspace.
 template <class M>
-__device__ bool op_routed_down(const Params& p, Smem<M>& s, const Ctx& c) {
+__device__ __forceinline__ bool op_routed_down(const Params& p, Smem<M>& s, const Ctx& c) {
   const int layer = s.inst[1], slot = s.inst[2], n0 = s.inst[4], n1 = s.inst[5], tile = s.inst[7];
   if (layer < 0 || layer >= p.num_layers) return bad_operand(p, s, c, 1);
   if (slot < 0 || slot >= p.top_k) return bad_operand(p, s, c, 2);
@@ -351,7 +350,7 @@ __device__ bool op_routed_down(const Params& p, Smem<M>& s, const Ctx& c) {
 // with shared = the K-slice terms added in bf16 in slice order and routed = the slots' terms added in
 // fp32 in slot order; leaves shared_out complete and routed_out_f32 cleared, as the VM does.
 template <class M>
-__device__ bool op_combine(const Params& p, Smem<M>& s, const Ctx& c) {
+__device__ __forceinline__ bool op_combine(const Params& p, Smem<M>& s, const Ctx& c) {
   const int layer = s.inst[1], n0 = s.inst[2], n1 = s.inst[3], tile = s.inst[4];
   if (layer < 0 || layer >= p.num_layers) return bad_operand(p, s, c, 1);
   if (tile != kTile || n0 < 0 || n1 < n0 || n1 * tile > M::H || 2 * (n1 - n0) > kThreads) return bad_operand(p, s, c, 3);
@@ -373,23 +372,34 @@ __device__ bool op_combine(const Params& p, Smem<M>& s, const Ctx& c) {
   const bool tg = tagged(p);
   const uint32_t tag = tag_of(s.generation, layer);
   const float gate = ld_shared_f32(p.shared_gate);   // left by the layer's publishing router instruction
+  constexpr int kMaxSlices = 16;   // the launcher's bound on shared_k_slices
   for (int pair = c.tid; pair < nb * tile / 2; pair += kThreads) {
     const int r = n0 * tile + 2 * pair;
+    // every term is asked for before the first one is used: one trip to memory, not one per term
+    uint32_t st[kMaxSlices];
+    uint64_t rt[kMaxTopK];
+#pragma unroll
+    for (int k = 0; k < kMaxSlices; ++k) st[k] = k < p.shared_k_slices ? ld_shared32(p.shared_parts + static_cast<size_t>(k) * M::H + r) : 0u;
+#pragma unroll
+    for (int j = 0; j < kMaxTopK; ++j) rt[j] = j < p.top_k ? ld_shared64(p.routed_parts + static_cast<size_t>(j) * M::H + r) : 0ull;
+    // Tagged launch: the unit the O-projection announced this pair in.  Every up/gate workgroup has seen its
+    // tag, and this instruction follows them through the counters of the down projections: no polling.
+    const uint32_t old = tg ? static_cast<uint32_t>(ld_shared64(p.ws + kWsHiddenMid + r / 2)) : ld_shared32(p.hidden + r);
     float sh0 = 0.f, sh1 = 0.f;
-    for (int k = 0; k < p.shared_k_slices; ++k) {
-      const uint32_t t = ld_shared32(p.shared_parts + static_cast<size_t>(k) * M::H + r);
-      sh0 = round_bf16(sh0 + bf_lo(t));
-      sh1 = round_bf16(sh1 + bf_hi(t));
+#pragma unroll
+    for (int k = 0; k < kMaxSlices; ++k) {
+      if (k < p.shared_k_slices) {
+        sh0 = round_bf16(sh0 + bf_lo(st[k]));
+        sh1 = round_bf16(sh1 + bf_hi(st[k]));
+      }
     }
     float ro0 = 0.f, ro1 = 0.f;
-    for (int j = 0; j < p.top_k; ++j) {
-      ro0 += ld_shared_f32(p.routed_parts + static_cast<size_t>(j) * M::H + r);
-      ro1 += ld_shared_f32(p.routed_parts + static_cast<size_t>(j) * M::H + r + 1);
-    }
-    uint32_t old = 0;
-    if (!residual_in(p, tg ? p.ws + kWsHiddenMid : nullptr, tag, 0, r / 2, old)) {   // its tag has been seen by every up/gate workgroup
-      s.ctl[0] = 1;
-      report_error(p, QMK_DEV_WAIT_TIMEOUT, c.inst_idx, c.opcode, c.tid);
+#pragma unroll
+    for (int j = 0; j < kMaxTopK; ++j) {
+      if (j < p.top_k) {
+        ro0 += __uint_as_float(static_cast<uint32_t>(rt[j]));
+        ro1 += __uint_as_float(static_cast<uint32_t>(rt[j] >> 32));
+      }
     }
     const float h0 = (bf_lo(old) + ro0) + gate * sh0, h1 = (bf_hi(old) + ro1) + gate * sh1;
     const uint32_t word = static_cast<uint32_t>(f2bf(h0)) | (static_cast<uint32_t>(f2bf(h1)) << 16);
@@ -398,10 +408,6 @@ __device__ bool op_combine(const Params& p, Smem<M>& s, const Ctx& c) {
     st_shared32(p.shared_out + r, static_cast<uint32_t>(f2bf(sh0)) | (static_cast<uint32_t>(f2bf(sh1)) << 16));
     st_shared_f32(p.routed_out_f32 + r, 0.f);
     st_shared_f32(p.routed_out_f32 + r + 1, 0.f);
-  }
-  if (tg) {   // the units announce themselves: nothing to count
-    __syncthreads();
-    return s.ctl[0] == 0;
   }
   publish_done(p, c, layer, ROW_COMBINE, 0, nb);
   return true;

@@ -63,11 +63,9 @@ class MoeMegaKernel:
     retires (default), or leaves their final values like the reference kernel.  ``tagged``: the residual stream
     (combine -> QKV / O-projection / LM head, O-projection -> router / up-gate ops / combine) and q, k, v travel
     as self-announcing tagged units instead of through counters, as on the dense route; whole steps only, so it
-    applies when the kernel also clears its counters.  Same values bit for bit; off by default, because here it
-    measures slower (515 against 597 tok/s): the O-projection gets 2.5 us shorter, but every streaming op of the
-    layer 20-30 % longer."""
+    applies when the kernel also clears its counters.  Same values bit for bit, 705 against 603 tok/s."""
 
-    def __init__(self, lib: ctypes.CDLL, *, reset_barriers: bool = True, spin_limit: int = 0, tagged: bool = False):
+    def __init__(self, lib: ctypes.CDLL, *, reset_barriers: bool = True, spin_limit: int = 0, tagged: bool = True):
         self._lib = lib
         self.reset_barriers = reset_barriers
         self.tagged = tagged
@@ -182,7 +180,7 @@ class MoeMegaKernel:
             raise RuntimeError(f"qmk_decode_step_moe failed with {rc}: {self.error_string(rc)}")
 
 
-def get_mk(mk_dir: Path | None = None, *, reset_barriers: bool = True, spin_limit: int = 0, tagged: bool = False) -> MoeMegaKernel:
+def get_mk(mk_dir: Path | None = None, *, reset_barriers: bool = True, spin_limit: int = 0, tagged: bool = True) -> MoeMegaKernel:
     """Return the ``mk`` callable of the MoE route bound to the prebuilt library in ``mk_dir``."""
     root = (_single._default_mk_dir() if mk_dir is None else Path(mk_dir)).resolve()
     lib = _single._LIB_CACHE.get(root)
