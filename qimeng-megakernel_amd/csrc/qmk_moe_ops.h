@@ -55,29 +55,40 @@ constexpr int kMaxExperts = 512;
 constexpr int kMaxTopK = 8;
 constexpr int kTile = 16;
 
-// NR weight rows against the bf16 vector x in LDS, K (a multiple of 8, <= kMaxK) columns each: all
-// 16-byte pieces of all rows are requested before the first is used.  Every lane gets the sums.
+// NR weight rows of K columns (a multiple of 8, <= kMaxK) as 16-byte pieces per lane.  `request_rows` asks
+// for all pieces of the first `live` rows (the others read as zeros); `reduce_rows` multiplies them with the
+// bf16 vector x in LDS and leaves every lane the sums.  Between the two a caller may wait for x: what it
+// asked for lands meanwhile.  Indices are constants already in the source (static_for, not unrolled loops).
 template <int NR>
-__device__ __forceinline__ void rows_dot(const u16* const (&rows)[NR], const u16* x, int K, int lane, float (&out)[NR]) {
-  constexpr int NI = kMaxK / 512;
-  // Indices that are constants already in the source (static_for, not unrolled loops): the pieces are
-  // registers however the optimiser treats the loops around this function.
-  v4u w[NR][NI];
+struct RowSet {
+  v4u w[NR][kMaxK / 512];
+};
+template <int NR>
+__device__ __forceinline__ void request_rows(RowSet<NR>& set, const u16* const (&rows)[NR], int K, int lane, int live = NR) {
   static_for<0, NR>([&](auto r) {
-    static_for<0, NI>([&](auto i) {
+    static_for<0, kMaxK / 512>([&](auto i) {
       const int col = lane * 8 + i * 512;
-      w[r][i] = v4u{0, 0, 0, 0};
-      if (col < K) w[r][i] = __builtin_nontemporal_load(reinterpret_cast<const v4u*>(rows[r] + col));
+      set.w[r][i] = v4u{0, 0, 0, 0};
+      if (r < live && col < K) set.w[r][i] = __builtin_nontemporal_load(reinterpret_cast<const v4u*>(rows[r] + col));
     });
   });
+}
+template <int NR>
+__device__ __forceinline__ void reduce_rows(const RowSet<NR>& set, const u16* x, int K, int lane, float (&out)[NR]) {
   static_for<0, NR>([&](auto r) {
     float a = 0.f;
-    static_for<0, NI>([&](auto i) {
+    static_for<0, kMaxK / 512>([&](auto i) {
       const int col = lane * 8 + i * 512;
-      if (col < K) a = dot8(w[r][i], *reinterpret_cast<const v4u*>(x + col), a);
+      if (col < K) a = dot8(set.w[r][i], *reinterpret_cast<const v4u*>(x + col), a);
     });
     out[r] = wave_sum(a);
   });
+}
+template <int NR>
+__device__ __forceinline__ void rows_dot(const u16* const (&rows)[NR], const u16* x, int K, int lane, float (&out)[NR]) {
+  RowSet<NR> set;
+  request_rows(set, rows, K, lane);
+  reduce_rows(set, x, K, lane, out);
 }
 
 // n bf16 elements (a multiple of 4) of a vector that another workgroup wrote during this launch, into s.x.
@@ -198,27 +209,35 @@ __device__ __forceinline__ bool op_topk(const Params& p, Smem<M>& s, const Ctx& 
 // Gate and up rows [r0, r0 + n) of one FFN against the normalised row in s.x; out[i] =
 // bf16(silu(bf16(gate . x)) * bf16(up . x)), silu and the product in fp32 (python_vm.py:389-395, 455-459).
 // The results wait in s.res; two neighbouring ones leave as one word to every destination given.
-template <class M>
-__device__ __forceinline__ void upgate_rows(Smem<M>& s, const Ctx& c, const u16* gate_w, const u16* up_w, int r0, int n, u16* dst0, u16* dst1) {
+// `ready()` makes s.x the normalised residual stream (false: give up); the rows of the wave's first round are
+// asked for before it is called.
+template <class M, class Ready>
+__device__ __forceinline__ bool upgate_rows(Smem<M>& s, const Ctx& c, const u16* gate_w, const u16* up_w, int r0, int n, u16* dst0, u16* dst1,
+                                            Ready ready) {
   const int lane = c.tid & 63, wave = c.tid >> 6;
   constexpr int kOut = 4;   // outputs (gate + up row each) of a wave in flight together: 32 KiB per wave
-  for (int i = wave; i < n; i += kOut * kWaves) {
-    int o[kOut];
+  RowSet<2 * kOut> set;
+  auto request = [&](int i) {
     const u16* rows[2 * kOut];
-#pragma unroll
-    for (int k = 0; k < kOut; ++k) {
-      o[k] = min(i + k * kWaves, n - 1);   // past the end: the last output once more, not stored
-      rows[2 * k] = gate_w + static_cast<size_t>(r0 + o[k]) * M::H;
-      rows[2 * k + 1] = up_w + static_cast<size_t>(r0 + o[k]) * M::H;
-    }
+    static_for<0, kOut>([&](auto k) {
+      const int o = min(i + k * kWaves, n - 1);   // past the end: not asked for
+      rows[2 * k] = gate_w + static_cast<size_t>(r0 + o) * M::H;
+      rows[2 * k + 1] = up_w + static_cast<size_t>(r0 + o) * M::H;
+    });
+    const int left = i < n ? (n - 1 - i) / kWaves + 1 : 0;   // outputs of this round that exist
+    request_rows(set, rows, M::H, lane, 2 * min(left, kOut));
+  };
+  request(wave);
+  if (!ready()) return false;
+  for (int i = wave; i < n; i += kOut * kWaves) {
     float v[2 * kOut];
-    rows_dot<2 * kOut>(rows, s.x, M::H, lane, v);
+    reduce_rows(set, s.x, M::H, lane, v);
+    if (i + kOut * kWaves < n) request(i + kOut * kWaves);
     if (lane == 0) {
-#pragma unroll
-      for (int k = 0; k < kOut; ++k) {
+      static_for<0, kOut>([&](auto k) {
         const float g = round_bf16(v[2 * k]);
-        if (i + k * kWaves < n) s.res[o[k]] = (g / (1.0f + expf(-g))) * round_bf16(v[2 * k + 1]);
-      }
+        if (i + k * kWaves < n) s.res[i + k * kWaves] = (g / (1.0f + expf(-g))) * round_bf16(v[2 * k + 1]);
+      });
     }
   }
   __syncthreads();
@@ -227,6 +246,7 @@ __device__ __forceinline__ void upgate_rows(Smem<M>& s, const Ctx& c, const u16*
     st_shared32(dst0 + r0 + 2 * pair, word);
     if (dst1 != nullptr) st_shared32(dst1 + r0 + 2 * pair, word);
   }
+  return true;
 }
 
 // ==================================================================== 10 ==
@@ -240,34 +260,40 @@ __device__ __forceinline__ bool op_shared_upgate(const Params& p, Smem<M>& s, co
   // The normalised row is recomputed here from the residual stream (the same function of the same values as
   // the row opcode 8 publishes, bit for bit) instead of being waited for: the shared expert starts with the
   // O-proj's last arrival, beside the router.
-  if (!residual_to_lds<M>(p, s, c, layer)) return false;
   const size_t base = static_cast<size_t>(layer) * p.shared_ffn * M::H;
-  upgate_rows(s, c, p.shared_gate_w + base, p.shared_up_w + base, n0 * tile, (n1 - n0) * tile, p.shared_silu, nullptr);
+  if (!upgate_rows(s, c, p.shared_gate_w + base, p.shared_up_w + base, n0 * tile, (n1 - n0) * tile, p.shared_silu, nullptr,
+                   [&] { return residual_to_lds<M>(p, s, c, layer); }))
+    return false;
   publish_done(p, c, layer, ROW_SHARED_UPGATE, 0, n1 - n0);
   return true;
 }
 
 // Rows [r0, r0 + n) of a down projection with K columns (row stride ld) against s.x[0..K); `leave(r, dot)`
-// runs on lane 0 of the wave that owns row r.
-template <class M, class Leave>
-__device__ __forceinline__ void down_rows(Smem<M>& s, const Ctx& c, const u16* w, size_t ld, int K, int r0, int n, Leave leave) {
+// runs on lane 0 of the wave that owns row r.  `ready()` fills s.x (false: give up); the rows of the wave's
+// first round are asked for before it is called.
+template <class M, class Ready, class Leave>
+__device__ __forceinline__ bool down_rows(Smem<M>& s, const Ctx& c, const u16* w, size_t ld, int K, int r0, int n, Ready ready, Leave leave) {
   const int lane = c.tid & 63, wave = c.tid >> 6;
-  for (int i = wave; i < n; i += 4 * kWaves) {
-    int r[4];
-    const u16* rows[4];
-#pragma unroll
-    for (int k = 0; k < 4; ++k) {
-      r[k] = min(i + k * kWaves, n - 1);
-      rows[k] = w + static_cast<size_t>(r0 + r[k]) * ld;
-    }
-    float v[4];
-    rows_dot<4>(rows, s.x, K, lane, v);
+  constexpr int kRows = 4;
+  RowSet<kRows> set;
+  auto request = [&](int i) {
+    const u16* rows[kRows];
+    static_for<0, kRows>([&](auto k) { rows[k] = w + static_cast<size_t>(r0 + min(i + k * kWaves, n - 1)) * ld; });
+    request_rows(set, rows, K, lane, i < n ? min((n - 1 - i) / kWaves + 1, kRows) : 0);
+  };
+  request(wave);
+  if (!ready()) return false;
+  for (int i = wave; i < n; i += kRows * kWaves) {
+    float v[kRows];
+    reduce_rows(set, s.x, K, lane, v);
+    if (i + kRows * kWaves < n) request(i + kRows * kWaves);
     if (lane == 0) {
-#pragma unroll
-      for (int k = 0; k < 4; ++k)
-        if (i + k * kWaves < n) leave(r0 + r[k], v[k]);
+      static_for<0, kRows>([&](auto k) {
+        if (i + k * kWaves < n) leave(r0 + i + k * kWaves, v[k]);
+      });
     }
   }
+  return true;
 }
 
 // ==================================================================== 11 ==
@@ -279,12 +305,18 @@ __device__ __forceinline__ bool op_shared_down(const Params& p, Smem<M>& s, cons
   if (layer < 0 || layer >= p.num_layers) return bad_operand(p, s, c, 1);
   if (tile != kTile || n0 < 0 || n1 < n0 || n1 * tile > M::H) return bad_operand(p, s, c, 4);
   if (slice < 0 || slice >= p.shared_k_slices || kg < 8 || (kg & 7) || kg > kMaxK || slice * kg >= p.shared_ffn) return bad_operand(p, s, c, 5);
-  if (!wait_one(p, s, c, layer, ROW_SHARED_UPGATE, 0, p.shared_ffn / kTile)) return false;
   const int k0 = slice * kg, K = min(kg, p.shared_ffn - k0);
-  stage_vector(s, c, p.shared_silu + k0, K);
   const u16* w = p.shared_down_w + static_cast<size_t>(layer) * M::H * p.shared_ffn + k0;
   u16* mine = p.shared_parts + static_cast<size_t>(slice) * M::H;
-  down_rows(s, c, w, p.shared_ffn, K, n0 * tile, (n1 - n0) * tile, [&](int r, float dot) { s.res[r - n0 * tile] = dot; });
+  if (!down_rows(
+          s, c, w, p.shared_ffn, K, n0 * tile, (n1 - n0) * tile,
+          [&] {
+            if (!wait_one(p, s, c, layer, ROW_SHARED_UPGATE, 0, p.shared_ffn / kTile)) return false;
+            stage_vector(s, c, p.shared_silu + k0, K);
+            return true;
+          },
+          [&](int r, float dot) { s.res[r - n0 * tile] = dot; }))
+    return false;
   __syncthreads();
   for (int pair = c.tid; pair < (n1 - n0) * tile / 2; pair += kThreads)
     st_shared32(mine + n0 * tile + 2 * pair,
@@ -313,10 +345,11 @@ __device__ __forceinline__ bool op_routed_upgate(const Params& p, Smem<M>& s, co
   if (!wait_one(p, s, c, layer, ROW_TOPK, 0, 1)) return false;
   const int eid = expert_of(p, slot);
   if (eid < 0) return bad_operand(p, s, c, 2);
-  if (!residual_to_lds<M>(p, s, c, layer, /*oproj_seen=*/true)) return false;   // as in opcode 10
   const u16* w = p.expert_gate_up_w + (static_cast<size_t>(layer) * p.num_experts + eid) * 2 * p.moe_ffn * M::H;
-  upgate_rows(s, c, w, w + static_cast<size_t>(p.moe_ffn) * M::H, n0 * tile, (n1 - n0) * tile,
-              p.routed_silu + static_cast<size_t>(slot) * p.moe_ffn, slot == p.top_k - 1 ? p.silu_out : nullptr);
+  if (!upgate_rows(s, c, w, w + static_cast<size_t>(p.moe_ffn) * M::H, n0 * tile, (n1 - n0) * tile,
+                   p.routed_silu + static_cast<size_t>(slot) * p.moe_ffn, slot == p.top_k - 1 ? p.silu_out : nullptr,
+                   [&] { return residual_to_lds<M>(p, s, c, layer, /*oproj_seen=*/true); }))   // as in opcode 10
+    return false;
   publish_done(p, c, layer, ROW_ROUTED_UPGATE, 0, n1 - n0);
   return true;
 }
@@ -330,14 +363,23 @@ __device__ __forceinline__ bool op_routed_down(const Params& p, Smem<M>& s, cons
   if (layer < 0 || layer >= p.num_layers) return bad_operand(p, s, c, 1);
   if (slot < 0 || slot >= p.top_k) return bad_operand(p, s, c, 2);
   if (tile != kTile || n0 < 0 || n1 < n0 || n1 * tile > M::H) return bad_operand(p, s, c, 5);
-  if (!wait_one(p, s, c, layer, ROW_ROUTED_UPGATE, 0, p.top_k * (p.moe_ffn / kTile))) return false;
+  // The expert is known with the top-k edge, long before the routed up/gate rows are complete: its rows are
+  // asked for in between.
+  if (!wait_one(p, s, c, layer, ROW_TOPK, 0, 1)) return false;
   const int eid = expert_of(p, slot);
   if (eid < 0) return bad_operand(p, s, c, 2);
   const float weight = ld_shared_f32(p.expert_weights + slot);
-  stage_vector(s, c, p.routed_silu + static_cast<size_t>(slot) * p.moe_ffn, p.moe_ffn);
   const u16* w = p.expert_down_w + (static_cast<size_t>(layer) * p.num_experts + eid) * M::H * p.moe_ffn;
   float* mine = p.routed_parts + static_cast<size_t>(slot) * M::H;
-  down_rows(s, c, w, p.moe_ffn, p.moe_ffn, n0 * tile, (n1 - n0) * tile, [&](int r, float dot) { st_shared_f32(mine + r, round_bf16(dot) * weight); });
+  if (!down_rows(
+          s, c, w, p.moe_ffn, p.moe_ffn, n0 * tile, (n1 - n0) * tile,
+          [&] {
+            if (!wait_one(p, s, c, layer, ROW_ROUTED_UPGATE, 0, p.top_k * (p.moe_ffn / kTile))) return false;
+            stage_vector(s, c, p.routed_silu + static_cast<size_t>(slot) * p.moe_ffn, p.moe_ffn);
+            return true;
+          },
+          [&](int r, float dot) { st_shared_f32(mine + r, round_bf16(dot) * weight); }))
+    return false;
   release_stores();
   __syncthreads();
   if (c.tid < n1 - n0) publish(counter_ptr(p, layer, ROW_ROUTED_DOWN, n0 + c.tid), 1);

@@ -1,4 +1,5 @@
-"""Scheduler of the MoE decode route: one step's instructions in dependency order, dealt round-robin.
+"""Scheduler of the MoE decode route: one step's instructions in dependency order, dealt round-robin
+(the reference's way) or placed queue by queue (``placed=True``: the MI355X stream).
 
 Emission order per layer 1 -> 2 -> 3 -> 4 -> 8 -> 9 -> 10 -> 11 -> 12 -> 13 -> 14, then 7
 (`…/qwen1_5_moe_a2_7b/A100/single_batch/decode_schedule/instructions/scheduler.py:139-370`).
@@ -56,6 +57,7 @@ class MoeScheduler:
     merge_in_last: bool = False        # the last split-KV arrival of a KV head merges: no reduction instructions
     merge_in_oproj: bool = False       # every O-projection instruction merges all partials itself: no reduction instructions
     router_span: int = 1               # experts per router instruction
+    placed: bool = False               # queues() places the instructions of a layer by role instead of dealing them
 
     def qkvproj(self, layer: int) -> list[Instruction]:
         tiles = _ceil_div(self.shape.qkv_out_dim, TILE_N_GRANULARITY)
@@ -88,6 +90,8 @@ class MoeScheduler:
         return [Router_SoftmaxTopK(layer)]
 
     def shared_upgate(self, layer: int) -> list[Instruction]:
+        if self.placed:
+            return [ins for _, ins in self._placed_shared_upgate(layer)]
         tiles = _ceil_div(self.shape.intermediate_size, TILE_N_GRANULARITY)
         return [SharedExpert_UpGate_SiLU(layer, 0, lo, hi, 1 if lo == 0 else 0) for lo, hi in _spans(tiles, self.sm_count)]
 
@@ -104,6 +108,8 @@ class MoeScheduler:
         return out
 
     def routed_upgate(self, layer: int) -> list[Instruction]:
+        if self.placed:
+            return [ins for _, ins in self._placed_routed_upgate(layer)]
         per_expert = max(1, self.sm_count // self.shape.num_experts_per_tok)
         return [RoutedExpert_UpGate_SiLU(layer, slot, lo, hi)
                 for slot in range(self.shape.num_experts_per_tok)
@@ -132,6 +138,85 @@ class MoeScheduler:
             experts = self.shared_upgate(layer) + self.shared_downproj(layer) + self.routed_upgate(layer) + self.routed_downproj(layer)
         return head + experts + self.combine_commit(layer)
 
+    # ---- placement by role (``placed=True``) -------------------------------------------------------------
+    # With the stream dealt round-robin, the queues that run the router and the top-k of a layer start that
+    # layer's expert phases one or two hand-overs after everybody else, with the same amount of work ahead of
+    # them, and the down projections wait for the slowest queue.  Placed: the last queues of the device take the
+    # router and the top-k and no shared up/gate rows; the O-projection queues take one shared up/gate tile and
+    # the queues that only wait during the O-projection two; the routed up/gate tiles go where the shared ones
+    # left room (three tiles of the two phases per queue at most).
+
+    def _roles(self) -> tuple[list[int], list[int], int]:
+        """(queues of the O-projection and the expert phases, queues of the router and the top-k, O-proj count)."""
+        n = self.sm_count
+        side = len(self.router_gemv(0)) + 1
+        if side * 4 > n:                       # a device too small to set queues aside
+            return list(range(n)), list(range(n)), min(n, self.shape.num_hidden_blocks)
+        return list(range(n - side)), list(range(n - side, n)), min(n - side, self.shape.num_hidden_blocks)
+
+    @staticmethod
+    def _weighted_sizes(tiles: int, weights: Sequence[int]) -> list[int]:
+        """``tiles`` cut in proportion to ``weights`` (largest remainders first, earlier entries on ties)."""
+        total = sum(weights)
+        raw = [tiles * w / total for w in weights]
+        sizes = [int(r) for r in raw]
+        order = sorted(range(len(weights)), key=lambda i: (-(raw[i] - sizes[i]), i))
+        for i in order[: tiles - sum(sizes)]:
+            sizes[i] += 1
+        return sizes
+
+    def _shared_sizes(self) -> dict[int, int]:
+        main, _, oproj_queues = self._roles()
+        tiles = _ceil_div(self.shape.intermediate_size, TILE_N_GRANULARITY)
+        weights = [1 if i < oproj_queues else 2 for i in range(len(main))]
+        return dict(zip(main, self._weighted_sizes(tiles, weights)))
+
+    def _placed_shared_upgate(self, layer: int) -> list[tuple[int, Instruction]]:
+        out, lo = [], 0
+        for queue, size in self._shared_sizes().items():
+            if size:
+                out.append((queue, SharedExpert_UpGate_SiLU(layer, 0, lo, lo + size, 1 if lo == 0 else 0)))
+                lo += size
+        return out
+
+    def _placed_routed_upgate(self, layer: int) -> list[tuple[int, Instruction]]:
+        shared = self._shared_sizes()
+        blocks, slots = self.shape.num_moe_intermediate_blocks, self.shape.num_experts_per_tok
+        most = max(shared.values()) + 1
+        queues = list(range(self.sm_count))
+        sizes = self._weighted_sizes(blocks * slots, [most - shared.get(q, most - 2) for q in queues])
+        out, slot, lo = [], 0, 0
+        for queue, size in zip(queues, sizes):
+            while size:                          # a span ends with its expert slot: the rest goes to the next slot
+                take = min(size, blocks - lo)
+                out.append((queue, RoutedExpert_UpGate_SiLU(layer, slot, lo, lo + take)))
+                size, lo = size - take, lo + take
+                if lo == blocks:
+                    slot, lo = slot + 1, 0
+        return out
+
+    def _place_layer(self, out: list[list[Instruction]], layer: int) -> None:
+        n = self.sm_count
+        main, side, _ = self._roles()
+
+        def spread(instructions: Sequence[Instruction], queues: Sequence[int]) -> None:
+            for i, ins in enumerate(instructions):
+                out[queues[i % len(queues)]].append(ins)
+
+        everyone = list(range(n))
+        spread(self.qkvproj(layer), everyone)
+        spread(self.attention_split_kv(layer), everyone)
+        spread(self.attention_reduction(layer), everyone)
+        spread(self.oproj(layer), main)
+        router = self.router_gemv(layer)
+        spread(router, side)
+        out[side[len(router) % len(side)]] += self.router_softmax_topk(layer)
+        for queue, ins in self._placed_shared_upgate(layer) + self._placed_routed_upgate(layer):
+            out[queue].append(ins)
+        spread(self.shared_downproj(layer), everyone)
+        spread(self.routed_downproj(layer), everyone)
+        spread(self.combine_commit(layer), everyone[::-1])   # not on the O-projection's queues
+
     def instruction_list(self, num_layers: int | None = None) -> list[Instruction]:
         layers = self.shape.num_hidden_layers if num_layers is None else num_layers
         out: list[Instruction] = []
@@ -142,7 +227,18 @@ class MoeScheduler:
         return out
 
     def queues(self, num_layers: int | None = None) -> list[list[Instruction]]:
-        return deal(self.instruction_list(num_layers), self.sm_count)
+        if not self.placed:
+            return deal(self.instruction_list(num_layers), self.sm_count)
+        if not self.interleave_experts:
+            raise ValueError("the placed stream runs both up/gate phases ahead of both down projections")
+        layers = self.shape.num_hidden_layers if num_layers is None else num_layers
+        out: list[list[Instruction]] = [[] for _ in range(self.sm_count)]
+        for layer in range(layers):
+            self._place_layer(out, layer)
+        if layers == self.shape.num_hidden_layers:
+            for i, ins in enumerate(self.lmhead()):
+                out[i % self.sm_count].append(ins)
+        return out
 
 
 def deal(instructions: Sequence[Instruction], queues: int) -> list[list[Instruction]]:

@@ -215,13 +215,16 @@ def call_mk(globs: Globals, mk: Any) -> None:
 
 
 def mi355x_scheduler(shape: Any = None) -> _scheduler.MoeScheduler:
-    """The reference's tiles on one queue per CU, with both up/gate phases ahead of both down projections and
-    the split-KV partials merged by the last arrival of each KV head (at most 25 partials)."""
+    """One queue per CU; both up/gate phases ahead of both down projections; the instructions of a layer placed
+    by role (the queues of the router and the top-k take no shared up/gate rows); eight experts per router
+    instruction; at most 8 split-KV partials per KV head, merged by the O-projection workgroups themselves
+    (measured at contexts up to 263: 753 tok/s, against 728 with 16 partials and 719 with the merge by the last
+    split-KV arrival)."""
     from .model_config import num_partials_for
 
     shape = shape or QwenMoeConfig.shape()
-    return _scheduler.MoeScheduler(shape, MI355X_QUEUES, min(25, num_partials_for(MI355X_QUEUES, shape)), interleave_experts=True,
-                                   merge_in_last=True)
+    return _scheduler.MoeScheduler(shape, MI355X_QUEUES, min(8, num_partials_for(MI355X_QUEUES, shape)), interleave_experts=True,
+                                   merge_in_oproj=True, router_span=8, placed=True)
 
 
 def build(globs: Globals) -> torch.Tensor:

@@ -81,7 +81,7 @@ BF16_OUT = {"qkvproj": ("q_post_rope", "k_cache", "v_cache"), "attention_reducti
 def test_one_op_against_the_vm(weights, stage, position):
     """Everything before the op runs on the VM; the op itself on both, from identical state."""
     cpu, gpu = make_pair(weights, position=position)
-    sched = dataclasses.replace(mk_kernel.mi355x_scheduler(SMALL), merge_in_last=False)     # the reference's protocol, op by op
+    sched = dataclasses.replace(mk_kernel.mi355x_scheduler(SMALL), merge_in_last=False, merge_in_oproj=False)     # the reference's protocol, op by op
     vm = MoeInstructionVM(SMALL)
     name = STAGES[stage]
     # the combine step uses what the router (the gate) and the two down projections (their terms) left in the launcher's
@@ -128,10 +128,10 @@ def test_one_op_against_the_vm(weights, stage, position):
 
 @pytest.mark.parametrize("position", [41, 0, 95])
 def test_split_kv_whose_last_arrival_merges(weights, position):
-    """The MI355X stream: no reduction instructions."""
+    """A stream without reduction instructions: the last split-KV arrival of a KV head merges."""
     cpu, gpu = make_pair(weights, position=position)
-    sched = mk_kernel.mi355x_scheduler(SMALL)
-    assert sched.merge_in_last and not sched.attention_reduction(0)
+    sched = dataclasses.replace(mk_kernel.mi355x_scheduler(SMALL), merge_in_last=True, merge_in_oproj=False, num_partials=16)
+    assert not sched.attention_reduction(0)
     vm = MoeInstructionVM(SMALL)
     vm.run(cpu, sched.qkvproj(0))
     sync_state(cpu, gpu)
@@ -148,7 +148,8 @@ def test_oproj_that_merges_the_partials(weights, position, partials):
     """The other stream without reduction instructions: split-KV instructions that only count their arrival,
     O-projection instructions that merge the partials of all heads themselves."""
     cpu, gpu = make_pair(weights, position=position)
-    sched = dataclasses.replace(mk_kernel.mi355x_scheduler(SMALL), merge_in_last=False, merge_in_oproj=True, num_partials=partials)
+    sched = dataclasses.replace(mk_kernel.mi355x_scheduler(SMALL), num_partials=partials)
+    assert sched.merge_in_oproj and not sched.merge_in_last
     assert not sched.attention_reduction(0)
     vm = MoeInstructionVM(SMALL)
     vm.run(cpu, sched.qkvproj(0))

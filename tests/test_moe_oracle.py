@@ -140,7 +140,8 @@ def test_request_of_the_reference_fixture(weights):
             assert tok[name] == want[name]["token"]
 
 
-def test_vm_agrees_with_fused_and_counters_complete(weights):
+@pytest.mark.parametrize("merge", ["oproj", "last"])
+def test_vm_agrees_with_fused_and_counters_complete(weights, merge):
     f, v = _request(weights), _request(weights)
     for g in (f, v):
         g.position_id = 41
@@ -148,7 +149,10 @@ def test_vm_agrees_with_fused_and_counters_complete(weights):
     FusedMoeOracle(SMALL).decode_step(f)
     from qimeng_megakernel_amd.decode_schedule_moe.mk_kernel import mi355x_scheduler
 
-    sched = mi355x_scheduler(SMALL)          # 256 queues, expert phases interleaved, merge by the last split-KV arrival
+    sched = mi355x_scheduler(SMALL)          # 256 queues placed by role, expert phases interleaved, the O-projection merges
+    assert sched.merge_in_oproj and sched.placed
+    if merge == "last":                      # the other stream without reduction instructions
+        sched = dataclasses.replace(sched, merge_in_oproj=False, merge_in_last=True, num_partials=16)
     assert not any(i.opcode() == 3 for i in sched.instruction_list())
     MoeInstructionVM(SMALL).run(v, sched.instruction_list())
     for name in ("q_post_rope", "attn_out", "hidden_states", "logits"):
@@ -159,13 +163,42 @@ def test_vm_agrees_with_fused_and_counters_complete(weights):
     for layer in range(s.num_hidden_layers):
         bar = v.barriers[layer]
         assert bar[0, : s.num_heads].tolist() == [s.head_dim // 16] * s.num_heads
-        assert bar[1, : s.num_attention_heads].tolist() == [sched.num_partials] * s.num_attention_heads
-        assert int(bar[2, 0]) == s.num_attention_heads and int(bar[3, 0]) == s.num_hidden_blocks == int(bar[13, 0])
+        if merge == "last":
+            assert bar[1, : s.num_attention_heads].tolist() == [sched.num_partials] * s.num_attention_heads
+        else:                                # split-KV instructions count on the reduction row only
+            assert int(bar[1].abs().sum()) == 0
+        assert int(bar[2, 0]) == (s.num_attention_heads if merge == "last" else s.num_key_value_heads * sched.num_partials)
+        assert int(bar[3, 0]) == s.num_hidden_blocks == int(bar[13, 0])
         assert bar[7, :2].tolist() == [s.num_experts, 1] and int(bar[8, 0]) == 1
         assert int(bar[9, 0]) == s.intermediate_size // 16 and int(bar[11, 0]) == s.num_experts_per_tok * s.num_moe_intermediate_blocks
         assert bar[10, : s.num_hidden_blocks].tolist() == [s.num_downproj_split_k_shared] * s.num_hidden_blocks
         assert bar[12, : s.num_hidden_blocks].tolist() == [s.num_experts_per_tok] * s.num_hidden_blocks
     assert float(v.routed_out_f32.abs().max()) == 0.0      # the combine step hands the accumulator back cleared
+
+
+def test_placed_stream_is_the_same_instructions_by_role():
+    """The MI355X stream at full size: the queues hold exactly the instruction list, every queue runs its layer's
+    phases in dependency order, the queues of the router and the top-k take no shared up/gate rows, and no queue
+    takes more than three up/gate tiles of a layer."""
+    from collections import Counter
+
+    from qimeng_megakernel_amd.decode_schedule_moe.mk_kernel import mi355x_scheduler
+    from qimeng_megakernel_amd.decode_schedule_moe.model_config import QWEN1_5_MOE_A2_7B as FULL
+
+    sched = mi355x_scheduler(FULL)
+    queues = sched.queues()
+    assert len(queues) == 256 and sched.placed
+    key = lambda ins: tuple(ins.padded())
+    assert Counter(key(i) for q in queues for i in q) == Counter(key(i) for i in sched.instruction_list())
+    phase = {1: 0, 2: 1, 3: 2, 4: 3, 8: 4, 9: 5, 10: 6, 12: 7, 11: 8, 13: 9, 14: 10, 7: 11}
+    for q in queues:
+        order = [(10 ** 6 if i.opcode() == 7 else i.padded()[1], phase[i.opcode()]) for i in q]
+        assert order == sorted(order)
+    layer0 = [[i for i in q if i.opcode() != 7 and i.padded()[1] == 0] for q in queues]
+    side = [q for q in layer0 if any(i.opcode() in (8, 9) for i in q)]
+    assert len(side) == 9 and not any(i.opcode() in (4, 10) for q in side for i in q)
+    tiles = [sum(i.padded()[4] - i.padded()[3] for i in q if i.opcode() in (10, 12)) for q in layer0]
+    assert max(tiles) == 3 and sum(tiles) == 2 * 352
 
 
 def _crafted(weights, layer=0):
