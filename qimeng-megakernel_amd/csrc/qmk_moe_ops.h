@@ -342,13 +342,16 @@ __device__ __forceinline__ bool op_routed_upgate(const Params& p, Smem<M>& s, co
   if (layer < 0 || layer >= p.num_layers) return bad_operand(p, s, c, 1);
   if (slot < 0 || slot >= p.top_k) return bad_operand(p, s, c, 2);
   if (tile != kTile || n0 < 0 || n1 < n0 || n1 * tile > p.moe_ffn || (n1 - n0) * tile > kResSlots) return bad_operand(p, s, c, 4);
+  // The normalised row first (as in opcode 10; a tagged launch has it long before the top-k is known), then the
+  // expert: its rows are the only thing left to wait for.
+  if (tagged(p) && !residual_to_lds<M>(p, s, c, layer)) return false;
   if (!wait_one(p, s, c, layer, ROW_TOPK, 0, 1)) return false;
   const int eid = expert_of(p, slot);
   if (eid < 0) return bad_operand(p, s, c, 2);
   const u16* w = p.expert_gate_up_w + (static_cast<size_t>(layer) * p.num_experts + eid) * 2 * p.moe_ffn * M::H;
   if (!upgate_rows(s, c, w, w + static_cast<size_t>(p.moe_ffn) * M::H, n0 * tile, (n1 - n0) * tile,
                    p.routed_silu + static_cast<size_t>(slot) * p.moe_ffn, slot == p.top_k - 1 ? p.silu_out : nullptr,
-                   [&] { return residual_to_lds<M>(p, s, c, layer, /*oproj_seen=*/true); }))   // as in opcode 10
+                   [&] { return tagged(p) || residual_to_lds<M>(p, s, c, layer, /*oproj_seen=*/true); }))
     return false;
   publish_done(p, c, layer, ROW_ROUTED_UPGATE, 0, n1 - n0);
   return true;

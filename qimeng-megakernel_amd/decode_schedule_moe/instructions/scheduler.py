@@ -211,9 +211,14 @@ class MoeScheduler:
         router = self.router_gemv(layer)
         spread(router, side)
         out[side[len(router) % len(side)]] += self.router_softmax_topk(layer)
-        for queue, ins in self._placed_shared_upgate(layer) + self._placed_routed_upgate(layer):
+        for queue, ins in self._placed_shared_upgate(layer):
             out[queue].append(ins)
-        spread(self.shared_downproj(layer), everyone)
+        if not self.interleave_experts:
+            spread(self.shared_downproj(layer), everyone)
+        for queue, ins in self._placed_routed_upgate(layer):
+            out[queue].append(ins)
+        if self.interleave_experts:
+            spread(self.shared_downproj(layer), everyone)
         spread(self.routed_downproj(layer), everyone)
         spread(self.combine_commit(layer), everyone[::-1])   # not on the O-projection's queues
 
@@ -229,8 +234,6 @@ class MoeScheduler:
     def queues(self, num_layers: int | None = None) -> list[list[Instruction]]:
         if not self.placed:
             return deal(self.instruction_list(num_layers), self.sm_count)
-        if not self.interleave_experts:
-            raise ValueError("the placed stream runs both up/gate phases ahead of both down projections")
         layers = self.shape.num_hidden_layers if num_layers is None else num_layers
         out: list[list[Instruction]] = [[] for _ in range(self.sm_count)]
         for layer in range(layers):
