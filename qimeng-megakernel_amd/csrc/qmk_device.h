@@ -280,7 +280,8 @@ constexpr int kWsHiddenOut = kWsHiddenMid + 1024;  // residual stream after the 
 constexpr int kWsSilu = kWsHiddenOut + 1024;        // silu_out: F/2 units (room for F = 8192)
 constexpr int kWsCandidates = kWsSilu + 4096;       // one greedy candidate per workgroup: {logit bits, row}
 constexpr int kMaxSamplingQueues = 1024;
-constexpr int kWsUnits = kWsCandidates + kMaxSamplingQueues;
+constexpr int kWsExperts = kWsCandidates + kMaxSamplingQueues;   // MoE route: the top-k's experts, then their weights (8 units each)
+constexpr int kWsUnits = kWsExperts + 16;
 
 __device__ __forceinline__ bool tagged(const Params& p) { return (p.flags & QMK_FLAG_TAGGED) != 0; }
 __device__ __forceinline__ uint32_t tag_of(uint32_t generation, int layer) { return (generation << 6) + static_cast<uint32_t>(layer) + 1u; }

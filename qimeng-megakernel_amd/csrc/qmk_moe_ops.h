@@ -195,6 +195,10 @@ __device__ __forceinline__ bool op_topk(const Params& p, Smem<M>& s, const Ctx& 
       if (lane == 0) {
         __hip_atomic_store(p.expert_indices + j, static_cast<long long>(idx), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         st_shared_f32(p.expert_weights + j, best / sum);
+        if (tagged(p)) {   // the routed ops poll these instead of the counter below: one trip, no drain in between
+          st_tagged(p.ws + kWsExperts + j, static_cast<uint32_t>(idx), tag_of(s.generation, layer));
+          st_tagged(p.ws + kWsExperts + kMaxTopK + j, __float_as_uint(best / sum), tag_of(s.generation, layer));
+        }
         s.res[idx] = -2.f;   // taken
       }
       __builtin_amdgcn_wave_barrier();
@@ -333,6 +337,37 @@ __device__ __forceinline__ int expert_of(const Params& p, int slot) {
   return (e >= 0 && e < p.num_experts) ? static_cast<int>(e) : -1;
 }
 
+// Wait for the layer's top-k and fetch a slot's expert (negative: not an expert of the layer) and weight:
+// through the counter and the caller's buffers, or, in a tagged launch, from the two units the top-k
+// instruction announces them in.  False (uniformly) when the wait ran out of polls.
+template <class M>
+__device__ __forceinline__ bool routed_expert(const Params& p, Smem<M>& s, const Ctx& c, int layer, int slot, int& eid, float& weight) {
+  if (!tagged(p)) {
+    if (!wait_one(p, s, c, layer, ROW_TOPK, 0, 1)) return false;
+    eid = expert_of(p, slot);
+    weight = ld_shared_f32(p.expert_weights + slot);
+    return true;
+  }
+  if (c.tid == 0) {
+    uint32_t e = 0, w = 0;
+    const uint32_t tag = tag_of(s.generation, layer);
+    if (!poll_tagged1(p.ws + kWsExperts + slot, tag, p.spin_limit, e) || !poll_tagged1(p.ws + kWsExperts + kMaxTopK + slot, tag, p.spin_limit, w)) {
+      s.ctl[0] = 1;
+      report_error(p, QMK_DEV_WAIT_TIMEOUT, c.inst_idx, c.opcode, slot);
+    }
+    s.ctl[4] = e < static_cast<uint32_t>(p.num_experts) ? static_cast<int>(e) : -1;
+    s.ctl[5] = static_cast<int>(w);
+    if (p.timeline != nullptr) {
+      s.t_wait = wall_clock64();
+      s.ctl[2] = 1;
+    }
+  }
+  __syncthreads();
+  eid = s.ctl[4];
+  weight = __uint_as_float(static_cast<uint32_t>(s.ctl[5]));
+  return s.ctl[0] == 0;
+}
+
 // ==================================================================== 12 ==
 // [12, layer, expert_slot, n_start, n_end, tile_M_g, tile_N_g]   (python_vm.py:421-464)
 // The single buffer silu_out keeps what the last slot wrote, as after the VM's sequential run.
@@ -345,8 +380,9 @@ __device__ __forceinline__ bool op_routed_upgate(const Params& p, Smem<M>& s, co
   // The normalised row first (as in opcode 10; a tagged launch has it long before the top-k is known), then the
   // expert: its rows are the only thing left to wait for.
   if (tagged(p) && !residual_to_lds<M>(p, s, c, layer)) return false;
-  if (!wait_one(p, s, c, layer, ROW_TOPK, 0, 1)) return false;
-  const int eid = expert_of(p, slot);
+  int eid;
+  float unused;
+  if (!routed_expert<M>(p, s, c, layer, slot, eid, unused)) return false;
   if (eid < 0) return bad_operand(p, s, c, 2);
   const u16* w = p.expert_gate_up_w + (static_cast<size_t>(layer) * p.num_experts + eid) * 2 * p.moe_ffn * M::H;
   if (!upgate_rows(s, c, w, w + static_cast<size_t>(p.moe_ffn) * M::H, n0 * tile, (n1 - n0) * tile,
@@ -368,10 +404,10 @@ __device__ __forceinline__ bool op_routed_down(const Params& p, Smem<M>& s, cons
   if (tile != kTile || n0 < 0 || n1 < n0 || n1 * tile > M::H) return bad_operand(p, s, c, 5);
   // The expert is known with the top-k edge, long before the routed up/gate rows are complete: its rows are
   // asked for in between.
-  if (!wait_one(p, s, c, layer, ROW_TOPK, 0, 1)) return false;
-  const int eid = expert_of(p, slot);
+  int eid;
+  float weight;
+  if (!routed_expert<M>(p, s, c, layer, slot, eid, weight)) return false;
   if (eid < 0) return bad_operand(p, s, c, 2);
-  const float weight = ld_shared_f32(p.expert_weights + slot);
   const u16* w = p.expert_down_w + (static_cast<size_t>(layer) * p.num_experts + eid) * M::H * p.moe_ffn;
   float* mine = p.routed_parts + static_cast<size_t>(slot) * M::H;
   if (!down_rows(
