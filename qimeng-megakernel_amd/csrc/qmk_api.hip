@@ -65,16 +65,16 @@ __global__ __launch_bounds__(kThreads, 1) void decode_megakernel(const Params p)
     // Only the O-proj hands rows to its successor: every other arm ends their life explicitly.
     switch (opcode) {
       case OP_NOOP: forget(carry); break;
-      case OP_RMS_QKV_ROPE: ok = op_rms_qkv_rope<M>(p, s, c); forget(carry); break;
-      case OP_ATTN_SPLITKV: ok = op_attn_splitkv<M>(p, s, c); forget(carry); break;
-      case OP_ATTN_REDUCE: ok = op_attn_reduce<M>(p, s, c); forget(carry); break;
+      case OP_RMS_QKV_ROPE: [[clang::always_inline]] ok = op_rms_qkv_rope<M>(p, s, c); forget(carry); break;
+      case OP_ATTN_SPLITKV: [[clang::always_inline]] ok = op_attn_splitkv<M>(p, s, c); forget(carry); break;
+      case OP_ATTN_REDUCE: [[clang::always_inline]] ok = op_attn_reduce<M>(p, s, c); forget(carry); break;
       case OP_OPROJ_RESIDUAL:
         carried = M::CARRY_AFTER_ATTENTION || !after_attention;
-        ok = op_oproj_residual<M>(p, s, c, carry, carried);
+        [[clang::always_inline]] ok = op_oproj_residual<M>(p, s, c, carry, carried);
         break;
-      case OP_RMS_UPGATE_SILU: ok = op_rms_upgate_silu<M>(p, s, c, carry, carried); forget(carry); break;
-      case OP_DOWN_RESIDUAL: ok = op_down_residual<M>(p, s, c); forget(carry); break;
-      case OP_RMS_LMHEAD: ok = op_rms_lmhead<M>(p, s, c); forget(carry); break;
+      case OP_RMS_UPGATE_SILU: [[clang::always_inline]] ok = op_rms_upgate_silu<M>(p, s, c, carry, carried); forget(carry); break;
+      case OP_DOWN_RESIDUAL: [[clang::always_inline]] ok = op_down_residual<M>(p, s, c); forget(carry); break;
+      case OP_RMS_LMHEAD: [[clang::always_inline]] ok = op_rms_lmhead<M>(p, s, c); forget(carry); break;
       default:
         if (threadIdx.x == 0) report_error(p, QMK_DEV_BAD_OPCODE, i, opcode, 0);
         ok = false;
@@ -199,14 +199,14 @@ __global__ __launch_bounds__(kThreads, 1) void decode_megakernel_batch(const Par
       case mb::OP_NOOP: break;
       case mb::OP_ATTN_RMS:
       case mb::OP_MLP_RMS:
-      case mb::OP_LM_RMS: ok = mb::op_rms_row<M>(p, s, c); break;
-      case mb::OP_QKV: ok = mb::op_qkv<M>(p, s, c); break;
-      case mb::OP_SPLITKV: ok = mb::op_splitkv<M>(p, s, c); break;
-      case mb::OP_REDUCE: ok = mb::op_reduce<M>(p, s, c); break;
-      case mb::OP_OPROJ: ok = mb::op_oproj<M>(p, s, c); break;
-      case mb::OP_UPGATE: ok = mb::op_upgate<M>(p, s, c); break;
-      case mb::OP_DOWN: ok = mb::op_down<M>(p, s, c); break;
-      case mb::OP_LMHEAD: ok = mb::op_lmhead<M>(p, s, c); break;
+      case mb::OP_LM_RMS: [[clang::always_inline]] ok = mb::op_rms_row<M>(p, s, c); break;
+      case mb::OP_QKV: [[clang::always_inline]] ok = mb::op_qkv<M>(p, s, c); break;
+      case mb::OP_SPLITKV: [[clang::always_inline]] ok = mb::op_splitkv<M>(p, s, c); break;
+      case mb::OP_REDUCE: [[clang::always_inline]] ok = mb::op_reduce<M>(p, s, c); break;
+      case mb::OP_OPROJ: [[clang::always_inline]] ok = mb::op_oproj<M>(p, s, c); break;
+      case mb::OP_UPGATE: [[clang::always_inline]] ok = mb::op_upgate<M>(p, s, c); break;
+      case mb::OP_DOWN: [[clang::always_inline]] ok = mb::op_down<M>(p, s, c); break;
+      case mb::OP_LMHEAD: [[clang::always_inline]] ok = mb::op_lmhead<M>(p, s, c); break;
       default:
         if (threadIdx.x == 0) report_error(p, QMK_DEV_BAD_OPCODE, i, opcode, 0);
         ok = false;
