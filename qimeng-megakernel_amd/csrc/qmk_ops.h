@@ -955,9 +955,6 @@ __device__ bool op_oproj_residual(const Params& p, Smem<M>& s, const Ctx& c, Car
       st_shared32(p.attn_out + c.tid * 4 + 2, hi);
     }
   }
-  // Counter mode: the attention of this layer is complete, so the previous layer is, and these rows of the
-  // residual stream have no other writer now: asked for here, they arrive behind the dot products.
-  if (!tg && c.tid < nrows / 2) res_old = ld_shared32(p.hidden + rs + 2 * c.tid);
   __syncthreads();
   QMK_STAMP(0);
   v4u x[CH];
@@ -979,8 +976,7 @@ __device__ bool op_oproj_residual(const Params& p, Smem<M>& s, const Ctx& c, Car
     }
     return true;
   }
-  if (c.tid < nrows / 2) st_shared32(p.hidden + rs + 2 * c.tid, residual_word(res_old, s.res[2 * c.tid], s.res[2 * c.tid + 1]));
-  for (int pair = c.tid + kThreads; pair < nrows / 2; pair += kThreads)
+  for (int pair = c.tid; pair < nrows / 2; pair += kThreads)
     residual_pair(p.hidden + rs + 2 * pair, s.res[2 * pair], s.res[2 * pair + 1]);
 
   release_stores();
