@@ -49,6 +49,8 @@ enum {
   QMK_ERR_NO_DEVICE = 6,       /* no gfx950 device / HIP runtime error          */
   QMK_ERR_LAUNCH = 7,          /* hipLaunchKernel failed                        */
   QMK_ERR_MODEL = 8,           /* unknown model id                              */
+  QMK_ERR_SCRATCH = 9,         /* qmk_decode_step_static: the launch needs more than the
+                                  library's static scratch array holds          */
   /* device-side (reported through qmk_status_fetch) */
   QMK_DEV_BAD_OPCODE = 32,     /* opcode outside 0..7 (batch route: 0..10)      */
   QMK_DEV_BAD_OPERAND = 33,    /* an operand would index out of bounds          */
@@ -193,6 +195,24 @@ typedef struct QmkArgs {
 /* Launch one decode step asynchronously on args->stream.  Returns QMK_OK or a
  * host-side QMK_ERR_*.  Device-side errors surface through qmk_status_fetch. */
 int qmk_decode_step(const QmkArgs* args);
+
+/*
+ * qmk_decode_step without any allocation on the caller's side or the library's: no counterpart in
+ * the reference.  It is for callers that cannot allocate device memory -- code under HIP graph
+ * capture, tight serving loops, harnesses that forbid hipMalloc.  Everything is as in
+ * qmk_decode_step (same struct, same kernels, same results bit for bit), except that
+ * args->workspace and args->workspace_bytes are ignored: the tagged units, the greedy candidates
+ * and the launch count live in a static device array of the library (86 144 bytes per GPU, held
+ * until the process ends; its address is looked up once per device on the first call of any entry
+ * point there).  Limits of that array: at most 1024 queues when token_out is set and at most 63
+ * layers with QMK_FLAG_TAGGED -- beyond them the call returns QMK_ERR_SCRATCH and launches nothing.
+ * All calls on one GPU share the array, which keeps the previous call's contents: the launch count
+ * carries on from call to call (stale units never carry a current tag; candidates are rewritten by
+ * every queue of a launch before they are read), and qmk_status_fetch clears the array when it
+ * reports a device-side error.  Calls that overlap on one GPU (two streams) race on it: serialise
+ * them, or use qmk_decode_step with one workspace per stream.
+ */
+int qmk_decode_step_static(const QmkArgs* args);
 
 /*
  * One decode step of the batch route: 2..16 rows decoded together (1 is accepted), each at its own

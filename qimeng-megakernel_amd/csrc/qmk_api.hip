@@ -17,6 +17,13 @@
 #include "qmk_moe_ops.h"
 #include "qmk_ops.h"
 
+// Workspace of qmk_decode_step_static: the tagged units, the greedy candidates and the launch count
+// that qmk_decode_step keeps in the caller's QmkArgs.workspace, here in an array of the library's own
+// (86 144 bytes per device, held until the process ends), so that the entry point allocates nothing.
+// In host code the name is only a handle for hipGetSymbolAddress: the kernels get the device address
+// that call returned (DeviceInfo::scratch), once per device.
+static __device__ __align__(256) unsigned long long scratch[qmk::kWsUnits];
+
 namespace qmk {
 
 constexpr int kStatusWords = 8;
@@ -338,6 +345,7 @@ struct DeviceInfo {
   int max_queues_batch = 0;
   int max_queues_moe = 0;
   int32_t* status = nullptr;
+  uint64_t* scratch = nullptr;   // this device's copy of the file-scope `scratch` array
 };
 DeviceInfo g_devices[kMaxDevices];
 std::mutex g_mutex;
@@ -362,11 +370,14 @@ int device_info(DeviceInfo** out) {
     void* sym = nullptr;
     if (hipGetSymbolAddress(&sym, HIP_SYMBOL(g_status)) != hipSuccess) return QMK_ERR_NO_DEVICE;
     if (hipMemset(sym, 0, sizeof(int32_t) * kStatusWords) != hipSuccess) return QMK_ERR_NO_DEVICE;
+    void* scratch_ptr = nullptr;
+    if (hipGetSymbolAddress(&scratch_ptr, HIP_SYMBOL(scratch)) != hipSuccess || scratch_ptr == nullptr) return QMK_ERR_NO_DEVICE;
     d.cu_count = prop.multiProcessorCount;
     d.max_queues = per_cu * prop.multiProcessorCount;
     d.max_queues_batch = per_cu_batch * prop.multiProcessorCount;
     d.max_queues_moe = per_cu_moe * prop.multiProcessorCount;
     d.status = static_cast<int32_t*>(sym);
+    d.scratch = static_cast<uint64_t*>(scratch_ptr);
     d.ready = true;
   }
   *out = &d;
@@ -379,8 +390,10 @@ using namespace qmk;
 
 namespace {
 
+// `static_scratch`: the workspace is the library's own array of the current device instead of
+// a->workspace (qmk_decode_step_static).
 template <class M>
-int decode_step(const QmkArgs* a) {
+int decode_step(const QmkArgs* a, bool static_scratch) {
   const void* required[] = {a->instructions, a->hidden_states, a->q_post_rope, a->k_cache, a->v_cache, a->attn_out,
                             a->attn_lse_intermediates, a->attn_out_intermediates, a->silu_out, a->logits,
                             a->attn_norm_weights, a->qkv_weights, a->rope_cos, a->rope_sin, a->o_proj_weights,
@@ -405,12 +418,20 @@ int decode_step(const QmkArgs* a) {
   const bool sampling = a->token_out != nullptr || a->embed_tokens != nullptr;
   if (sampling && (a->token_out == nullptr || a->embed_tokens == nullptr)) return QMK_ERR_NULL_ARG;
   if ((a->flags & QMK_FLAG_TAGGED) || sampling) {
-    if (a->workspace == nullptr) return QMK_ERR_NULL_ARG;
-    if ((a->flags & QMK_FLAG_KEEP_BARRIERS) || reinterpret_cast<uintptr_t>(a->workspace) % 128 != 0 ||
-        a->workspace_bytes < qmk_workspace_bytes(static_cast<int>(a->model)))
-      return QMK_ERR_SHAPE;
-    if ((a->flags & QMK_FLAG_TAGGED) && a->num_layers > 63) return QMK_ERR_SHAPE;
-    if (sampling && a->num_queues > kMaxSamplingQueues) return QMK_ERR_SHAPE;
+    if (static_scratch) {
+      // What the array has room for: one candidate per queue, six bits of layer in a tag.
+      if (qmk_workspace_bytes(static_cast<int>(a->model)) > sizeof(scratch)) return QMK_ERR_SCRATCH;
+      if ((a->flags & QMK_FLAG_TAGGED) && a->num_layers > 63) return QMK_ERR_SCRATCH;
+      if (sampling && a->num_queues > kMaxSamplingQueues) return QMK_ERR_SCRATCH;
+      if (a->flags & QMK_FLAG_KEEP_BARRIERS) return QMK_ERR_SHAPE;
+    } else {
+      if (a->workspace == nullptr) return QMK_ERR_NULL_ARG;
+      if ((a->flags & QMK_FLAG_KEEP_BARRIERS) || reinterpret_cast<uintptr_t>(a->workspace) % 128 != 0 ||
+          a->workspace_bytes < qmk_workspace_bytes(static_cast<int>(a->model)))
+        return QMK_ERR_SHAPE;
+      if ((a->flags & QMK_FLAG_TAGGED) && a->num_layers > 63) return QMK_ERR_SHAPE;
+      if (sampling && a->num_queues > kMaxSamplingQueues) return QMK_ERR_SHAPE;
+    }
   }
 
   DeviceInfo* dev = nullptr;
@@ -444,7 +465,7 @@ int decode_step(const QmkArgs* a) {
   p.lm_norm = static_cast<const u16*>(a->lm_head_norm_weights);
   p.lm_w = static_cast<const u16*>(a->lm_head_weights);
   p.barriers = a->barriers;
-  p.ws = static_cast<uint64_t*>(a->workspace);
+  p.ws = static_scratch ? dev->scratch : static_cast<uint64_t*>(a->workspace);
   p.embed = static_cast<const u16*>(a->embed_tokens);
   p.token_out = reinterpret_cast<long long*>(a->token_out);
   p.timeline = a->timeline;
@@ -474,15 +495,23 @@ int decode_step(const QmkArgs* a) {
 
 }  // namespace
 
-extern "C" int qmk_decode_step(const QmkArgs* a) {
+namespace {
+int decode_step_any(const QmkArgs* a, bool static_scratch) {
   if (a == nullptr) return QMK_ERR_NULL_ARG;
   if (a->struct_size != sizeof(QmkArgs)) return QMK_ERR_ABI;
   switch (a->model) {
-    case QMK_MODEL_LLAMA_3_2_1B: return decode_step<Llama1B>(a);
-    case QMK_MODEL_QWEN3_1_7B: return decode_step<Qwen3_1p7B>(a);
+    case QMK_MODEL_LLAMA_3_2_1B: return decode_step<Llama1B>(a, static_scratch);
+    case QMK_MODEL_QWEN3_1_7B: return decode_step<Qwen3_1p7B>(a, static_scratch);
     default: return QMK_ERR_MODEL;
   }
 }
+}  // namespace
+
+extern "C" int qmk_decode_step(const QmkArgs* a) { return decode_step_any(a, false); }
+
+// The same launch with the library's own workspace: no allocation anywhere on the way (the array
+// lives in the code object; its address was looked up when the device was first used).
+extern "C" int qmk_decode_step_static(const QmkArgs* a) { return decode_step_any(a, true); }
 
 extern "C" int qmk_decode_step_batch(const QmkBatchArgs* a) {
   using M = Llama1B;
@@ -703,7 +732,11 @@ extern "C" int qmk_status_fetch(void* stream, int32_t detail[4]) {
   if (hipMemcpy(host, dev->status, sizeof(host), hipMemcpyDeviceToHost) != hipSuccess) return QMK_ERR_NO_DEVICE;
   if (detail != nullptr)
     for (int i = 0; i < 4; ++i) detail[i] = host[1 + i];
-  if (host[0] != 0 && hipMemset(dev->status, 0, sizeof(host)) != hipSuccess) return QMK_ERR_NO_DEVICE;
+  if (host[0] != 0) {
+    if (hipMemset(dev->status, 0, sizeof(host)) != hipSuccess) return QMK_ERR_NO_DEVICE;
+    // Units of the aborted step must not pass for the next one's (the launch count did not advance).
+    if (hipMemset(dev->scratch, 0, sizeof(scratch)) != hipSuccess) return QMK_ERR_NO_DEVICE;
+  }
   return host[0];
 }
 
@@ -718,6 +751,7 @@ extern "C" const char* qmk_error_string(int code) {
     case QMK_ERR_NO_DEVICE: return "no usable HIP device";
     case QMK_ERR_LAUNCH: return "kernel launch failed";
     case QMK_ERR_MODEL: return "unknown model id";
+    case QMK_ERR_SCRATCH: return "launch needs more than the library's static scratch array holds (queues > 1024 with token_out, layers > 63 with QMK_FLAG_TAGGED)";
     case QMK_DEV_BAD_OPCODE: return "device: unknown opcode";
     case QMK_DEV_BAD_OPERAND: return "device: instruction operand out of bounds";
     case QMK_DEV_WAIT_TIMEOUT: return "device: counter wait ran out of polls";

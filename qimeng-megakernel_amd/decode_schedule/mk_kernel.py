@@ -62,7 +62,7 @@ class QmkArgs(ctypes.Structure):
     ]
 
 
-_EXPORTS = ("qmk_decode_step", "qmk_query", "qmk_status_fetch", "qmk_error_string", "qmk_workspace_bytes")
+_EXPORTS = ("qmk_decode_step", "qmk_decode_step_static", "qmk_query", "qmk_status_fetch", "qmk_error_string", "qmk_workspace_bytes")
 
 # (name, dtype, ndim) of the 22 tensors, in the positional order of mk(...).
 _TENSOR_ARGS: tuple[tuple[str, torch.dtype, int], ...] = (
@@ -132,6 +132,8 @@ def load_library(mk_dir: Path | None = None) -> ctypes.CDLL:
             raise ImportError(f"{dso} does not export {name}")
     lib.qmk_decode_step.argtypes = [ctypes.POINTER(QmkArgs)]
     lib.qmk_decode_step.restype = ctypes.c_int
+    lib.qmk_decode_step_static.argtypes = [ctypes.POINTER(QmkArgs)]
+    lib.qmk_decode_step_static.restype = ctypes.c_int
     lib.qmk_query.argtypes = [ctypes.c_int]
     lib.qmk_query.restype = ctypes.c_int
     lib.qmk_status_fetch.argtypes = [_P, ctypes.POINTER(_I * 4)]
@@ -160,7 +162,10 @@ class MegaKernel:
     self-announcing tagged units (``QMK_FLAG_TAGGED``) whenever the schedule
     allows it: the kernel clears its counters itself, the down projection is
     not split along K and there are at most 63 layers.  The workspace that mode
-    needs belongs to this object.
+    needs belongs to this object — or, with ``static_scratch``, to the library:
+    the call then goes through ``qmk_decode_step_static``, which allocates
+    nothing and takes no workspace (one array per GPU, shared by every such
+    call: do not overlap them on two streams).
 
     ``greedy_into(embed_tokens, tokens, index)`` arms device-side step chaining
     for the next call: the kernel itself writes the greedy token to
@@ -170,8 +175,9 @@ class MegaKernel:
     """
 
     def __init__(self, lib: ctypes.CDLL, geometry: TileGeometry | None = None, *, reset_barriers: bool = True,
-                 spin_limit: int = 0, xcd_counters: bool = True, tagged: bool = True):
+                 spin_limit: int = 0, xcd_counters: bool = True, tagged: bool = True, static_scratch: bool = False):
         self._lib = lib
+        self.static_scratch = static_scratch
         self.geometry = geometry
         self.reset_barriers = reset_barriers
         self.spin_limit = int(spin_limit)
@@ -213,7 +219,8 @@ class MegaKernel:
                            reset_barriers=kw.pop("reset_barriers", self.reset_barriers),
                            spin_limit=kw.pop("spin_limit", self.spin_limit),
                            xcd_counters=kw.pop("xcd_counters", self.xcd_counters),
-                           tagged=kw.pop("tagged", self.tagged))
+                           tagged=kw.pop("tagged", self.tagged),
+                           static_scratch=kw.pop("static_scratch", self.static_scratch))
         if kw:
             raise TypeError(f"unknown options {sorted(kw)}")
         return other
@@ -313,7 +320,10 @@ class MegaKernel:
             and geometry.num_split_k(shape) == 1
         )
         self._tagged = self.tagged and self.reset_barriers and geometry.num_split_k(shape) == 1 and L <= 63
-        if self._tagged or self.reset_barriers:   # the workspace also carries the greedy candidates
+        if self.static_scratch:
+            self._workspace = None
+            a.workspace, a.workspace_bytes = None, 0
+        elif self._tagged or self.reset_barriers:   # the workspace also carries the greedy candidates
             nbytes = int(self._lib.qmk_workspace_bytes(int(a.model)))
             if self._workspace is None or self._workspace.device != device:
                 self._workspace = torch.zeros(nbytes, dtype=torch.uint8, device=device)
@@ -332,7 +342,7 @@ class MegaKernel:
         if isinstance(tensors[0], torch.Tensor) and tensors[0].numel() == 0:
             return  # empty queues: nothing to launch
         key = tuple((t.data_ptr(), tuple(t.shape)) if isinstance(t, torch.Tensor) else None for t in tensors) + (
-            self.geometry, LlamaConfig.shape(), self.tagged, self.reset_barriers, self.xcd_counters)
+            self.geometry, LlamaConfig.shape(), self.tagged, self.reset_barriers, self.xcd_counters, self.static_scratch)
         if key != self._bound_key:
             self._bind(tensors)
             self._bound_key = key
@@ -354,16 +364,17 @@ class MegaKernel:
         else:
             a.embed_tokens, a.token_out = None, None
         a.stream = torch.cuda.current_stream(tensors[1].device).cuda_stream
-        rc = int(self._lib.qmk_decode_step(ctypes.byref(a)))
+        step = self._lib.qmk_decode_step_static if self.static_scratch else self._lib.qmk_decode_step
+        rc = int(step(ctypes.byref(a)))
         if rc != 0:
-            raise RuntimeError(f"qmk_decode_step failed with {rc}: {self.error_string(rc)}")
+            raise RuntimeError(f"{step.__name__} failed with {rc}: {self.error_string(rc)}")
 
 
 _LIB_CACHE: dict[Path, ctypes.CDLL] = {}
 
 
 def get_mk(mk_dir: Path | None = None, *, geometry: TileGeometry | None = None, reset_barriers: bool = True,
-           spin_limit: int = 0, xcd_counters: bool = True, tagged: bool = True) -> MegaKernel:
+           spin_limit: int = 0, xcd_counters: bool = True, tagged: bool = True, static_scratch: bool = False) -> MegaKernel:
     """Return the ``mk`` callable bound to the prebuilt library in ``mk_dir``.
 
     ``geometry`` defaults to the MI355X schedule of this package; pass
@@ -377,7 +388,7 @@ def get_mk(mk_dir: Path | None = None, *, geometry: TileGeometry | None = None, 
     if geometry is None:
         geometry = _scheduler.mi355x_scheduler(num_partials=1).geometry
     return MegaKernel(lib, geometry, reset_barriers=reset_barriers, spin_limit=spin_limit, xcd_counters=xcd_counters,
-                      tagged=tagged)
+                      tagged=tagged, static_scratch=static_scratch)
 
 
 def call_mk(globs: Globals, mk: Any) -> None:

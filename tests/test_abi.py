@@ -29,7 +29,7 @@ def lib():
 def test_every_declared_symbol_is_exported(lib):
     text = HEADER.read_text()
     declared = set(re.findall(r"^(?:int|uint64_t|const char\*)\s+(qmk_\w+)\s*\(", text, flags=re.M))
-    assert declared == {"qmk_decode_step", "qmk_decode_step_batch", "qmk_decode_step_moe", "qmk_moe_workspace_bytes", "qmk_query",
+    assert declared == {"qmk_decode_step", "qmk_decode_step_static", "qmk_decode_step_batch", "qmk_decode_step_moe", "qmk_moe_workspace_bytes", "qmk_query",
                         "qmk_status_fetch", "qmk_error_string", "qmk_workspace_bytes"}
     for name in declared:
         assert hasattr(lib, name), name
