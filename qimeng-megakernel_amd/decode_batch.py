@@ -4,8 +4,7 @@ Counterpart of the batch branch of the reference's decode loop
 (`qimeng_megakernel/models/LLM/decode.py:536-796`, per-row state `LLM/decode_state.py:46-138`):
 one instruction tensor per request (the scheduler's run-time template), per step the embedding
 rows of the last tokens -> ``hidden_states``, one kernel launch, ``argmax`` per row, then
-``advance_decode_state`` (rows that produced an EOS token retire, the others move one position
-on).  Timing as in the batch-1 loop: one event pair per step around the launch only.
+``RowState.advance`` (rows that produced an EOS token retire, the others move one position on).  Timing as in the batch-1 loop: one event pair per step around the launch only.
 
 Prefill runs the same kernel once per prompt position with every row at that position.
 """
@@ -16,7 +15,7 @@ from typing import Any, Sequence
 
 import torch
 
-from .decode_schedule_mb import decode_state as _state
+from .decode_schedule_mb.row_state import RowState, rows_of
 from .decode_schedule_mb import mk_kernel as _mk_kernel
 
 
@@ -69,22 +68,19 @@ def decode(globs: Any, prompts: torch.Tensor, max_new_tokens: int, *, mk: Any = 
 
     device = globs.hidden_states.device
     B, T = int(prompts.shape[0]), int(prompts.shape[1])
-    if B != _state.batch_size(globs):
-        raise ValueError(f"{B} prompts for buffers of {_state.batch_size(globs)} rows")
+    if B != rows_of(globs):
+        raise ValueError(f"{B} prompts for buffers of {rows_of(globs)} rows")
     if T + max_new_tokens > globs.k_cache.shape[2]:
         raise ValueError("prompt_len + max_new_tokens exceeds the KV cache capacity")
     mk = mk or _mk_kernel.get_mk()
-    globs.active_mask.fill_(True)
-    _state.ensure_decode_state(globs, B, device)
-    if getattr(globs, "eos_reached", None) is not None:
-        globs.eos_reached.zero_()
+    state = RowState.of(globs)
+    state.restart(0)
     globs.instructions = None
     _mk_kernel.build(globs)
     out = torch.zeros(B, T + max(max_new_tokens, 1), dtype=torch.long, device=device)
     out[:, :T] = prompts.to(device)
     out[:, T] = prefill_by_decode(globs, mk, prompts)
-    globs.position_ids.fill_(T)
-    _state.sync_kv_lengths(globs)
+    state.restart(T)
     ntok = max(max_new_tokens - 1, 0)
     eos = None
     if eos_token_ids:   # on the device before the loop: nothing inside a step comes from the host
@@ -106,17 +102,14 @@ def decode(globs: Any, prompts: torch.Tensor, max_new_tokens: int, *, mk: Any = 
             out[:, T + i + 1] = nxt
             if eos is not None:
                 active_log.append(globs.active_mask.clone())
-            _state.advance_decode_state(globs, nxt, eos if eos is not None else ())
+            state.advance(nxt, eos)
 
     graph = None
     first_token = out[:, T].clone()
 
     def rewind() -> None:   # the state the prefill left: what a replay of the captured loop starts from
         out[:, T] = first_token
-        globs.position_ids.fill_(T)
-        globs.active_mask.fill_(True)
-        globs.eos_reached.zero_()
-        _state.sync_kv_lengths(globs)
+        state.restart(T)
 
     if use_graph and ntok:
         graph = torch.cuda.CUDAGraph()

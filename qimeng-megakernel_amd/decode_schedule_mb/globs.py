@@ -9,7 +9,7 @@ Shapes for batch B (Llama-3.2-1B geometry): ``hidden_states/q_post_rope/attn_out
 from __future__ import annotations
 
 from dataclasses import dataclass
-from typing import Optional
+from typing import Any, Optional
 
 import torch
 
@@ -21,10 +21,8 @@ Tensor = torch.Tensor
 @dataclass
 class Globals(_SingleBatchGlobals):
     position_ids: Optional[Tensor] = None            # int32 [B]  index of the token each row decodes
-    kv_lengths: Optional[Tensor] = None              # int64 [B]  position_ids + 1
     active_mask: Optional[Tensor] = None             # bool  [B]  rows that still generate
-    eos_reached: Optional[Tensor] = None             # bool  [B]
-    last_generated_tokens: Optional[Tensor] = None   # int64 [B]
+    row_state: Optional[Any] = None                  # the RowState bound to the two tensors above (row_state.py)
     eos_token_id: Optional[int] = None
     attn_partial_valid: Optional[Tensor] = None      # bool  [B, Hq, P]  which split-KV partials hold data
     attn_rms_out: Optional[Tensor] = None            # bf16  [B, H]  RMSNorm rows for the QKV GEMM

@@ -21,7 +21,7 @@ from typing import Any, Sequence
 
 from ...decode_schedule.model_config import DecodeShape, LlamaConfig
 from ...instruction import INTS_PER_INSTRUCTION, Instruction
-from ..decode_state import decode_pos_id, row_active
+from ..row_state import RowState
 from .instruction_defs import (
     MAX_BATCH,
     TILE_N_GRANULARITY,
@@ -135,9 +135,8 @@ class BatchScheduler:
         out: list[Instruction] = []
         for b in range(self.batch_size):
             if globs is not None:
-                on = row_active(globs, b)
-                lens = getattr(globs, "kv_lengths", None)
-                seq_len = int(lens[b]) if lens is not None else decode_pos_id(globs, b) + 1
+                state = RowState.of(globs)
+                on, seq_len = state.is_active(b), state.position(b) + 1
                 total = max(1, _ceil_div(seq_len, kvb)) if on else 0
                 per = max(1, _ceil_div(total, num_partials)) if on else 1
             for kvh in range(self.shape.num_key_value_heads):
@@ -161,15 +160,15 @@ class BatchScheduler:
                     out.append(DecodeAttentionReduction(layer, b, head0, num_partials, list(range(num_partials))))
                 else:
                     out.append(DecodeAttentionReduction(layer, b, head0, num_partials, list(range(num_partials)),
-                                                        valid_partials=num_partials, is_active=1 if row_active(globs, b) else 0))
+                                                        valid_partials=num_partials, is_active=1 if RowState.of(globs).is_active(b) else 0))
         return out
 
     # ---- fan-out -------------------------------------------------------------
     def partials_for_request(self, globs: Any) -> int:
         kvb = self.shape.attn_kv_block_size
-        rows = [b for b in range(self.batch_size) if row_active(globs, b)]
-        lens = getattr(globs, "kv_lengths", None)
-        blocks = max([1] + [_ceil_div(int(lens[b]) if lens is not None else decode_pos_id(globs, b) + 1, kvb) for b in rows])
+        state = RowState.of(globs)
+        rows = [b for b in range(self.batch_size) if state.is_active(b)]
+        blocks = max([1] + [_ceil_div(state.position(b) + 1, kvb) for b in rows])
         return partials_for_blocks(len(rows), blocks, self.workers, self.shape.num_key_value_heads)
 
     def partials_for_capacity(self, kv_capacity: int) -> int:

@@ -23,7 +23,7 @@ from ..decode_schedule import mk_kernel as _single
 from ..decode_schedule.instructions.scheduler import tensorize_instructions
 from ..decode_schedule.model_config import LlamaConfig
 from ..instruction import Instruction
-from .decode_state import batch_size as _batch_size
+from .row_state import rows_of as _batch_size
 from .globs import Globals
 from .instructions import scheduler as _scheduler
 
@@ -111,6 +111,7 @@ class BatchMegaKernel:
         self._args = QmkBatchArgs()
         self._args.struct_size = ctypes.sizeof(QmkBatchArgs)
         self._bound_key: tuple | None = None
+        self._barriers: torch.Tensor | None = None   # the counters of the bound launch: cleared by check() after an error
 
     def error_string(self, code: int) -> str:
         return self._lib.qmk_error_string(int(code)).decode()
@@ -121,10 +122,12 @@ class BatchMegaKernel:
         handle = (stream or torch.cuda.current_stream()).cuda_stream
         code = int(self._lib.qmk_status_fetch(_P(handle), ctypes.byref(detail)))
         if code != 0:
+            if self._barriers is not None:   # a workgroup that gives up does not retire: the counters are those of an unfinished step
+                self._barriers.zero_()
             raise RuntimeError(
                 f"megakernel device error {code} ({self.error_string(code)}): workgroup={detail[0]} "
                 f"instruction={detail[1]} opcode={detail[2]} operand={detail[3]}; "
-                "the counters are undefined now — zero `barriers` before the next step"
+                "the counters of the aborted step have been cleared"
             )
 
     def with_options(self, **kw: Any) -> "BatchMegaKernel":
@@ -150,6 +153,7 @@ class BatchMegaKernel:
         (instructions, hidden, q, k_cache, v_cache, ao, lse, part, silu, logits, attn_norm, qkv, cos, sin, o_w,
          mlp_norm, up, gate, down, lm_norm, lm_w, barriers) = tensors
         L = int(barriers.shape[0])
+        self._barriers = barriers
         H, F = shape.hidden_size, shape.intermediate_size
         nq, nkv, d = shape.num_attention_heads, shape.num_key_value_heads, shape.head_dim
 

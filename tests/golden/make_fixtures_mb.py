@@ -70,7 +70,7 @@ def main() -> None:
     from pyvm_mb_oracle import BatchInstructionVM
     from qimeng_megakernel_amd import synthetic
     from qimeng_megakernel_amd.decode_schedule.model_config import LLAMA_3_2_1B, LlamaConfig
-    from qimeng_megakernel_amd.decode_schedule_mb import decode_state as my_state
+    from qimeng_megakernel_amd.decode_schedule_mb.row_state import RowState
     from qimeng_megakernel_amd.decode_schedule_mb.instructions import scheduler as my_sched
 
     ref_sched = importlib.import_module(A100 + ".multi_batch.decode_schedule.instructions.scheduler")
@@ -118,7 +118,10 @@ def main() -> None:
         g.k_cache.copy_(torch.randn(g.k_cache.shape, generator=gen).bfloat16())
         g.v_cache.copy_(torch.randn(g.v_cache.shape, generator=gen).bfloat16())
         g.position_ids.copy_(torch.tensor(START_POS, dtype=torch.int32))
-        my_state.ensure_decode_state(g, ROWS, torch.device("cpu"))
+        if cls is MyGlobals:
+            RowState.of(g)
+        else:
+            ref_state.ensure_decode_state(g, ROWS, device=torch.device("cpu"))
         return g
 
     from qimeng_megakernel_amd.decode_schedule_mb.globs import Globals as MyGlobals
@@ -165,12 +168,17 @@ def main() -> None:
             eos = [int(record["my_vm"]["tokens"][1])]
         for name, g in routes.items():
             nxt = g.logits.float().argmax(dim=-1)
-            (ref_state if name.startswith("ref") else my_state).advance_decode_state(g, nxt, eos)
+            if name.startswith("ref"):
+                ref_state.advance_decode_state(g, nxt, eos)
+            else:
+                RowState.of(g).advance(nxt, eos)
             toks[name] = [int(t) for t in nxt]
-        for name in ("position_ids", "active_mask", "eos_reached", "kv_lengths", "last_generated_tokens"):
-            for a, b in (("ref_vm", "my_vm"), ("ref_fused", "my_fused")):
-                if not torch.equal(getattr(routes[a], name), getattr(routes[b], name)):
-                    raise SystemExit(f"step {step}: {name} differs after advance_decode_state")
+        for a, b in (("ref_vm", "my_vm"), ("ref_fused", "my_fused")):
+            mine = RowState.of(routes[b])
+            for name, got in (("position_ids", mine.position_ids), ("active_mask", mine.active_mask), ("eos_reached", mine.finished),
+                              ("kv_lengths", mine.kv_lengths()), ("last_generated_tokens", mine.last_tokens)):
+                if not torch.equal(getattr(routes[a], name), got):
+                    raise SystemExit(f"step {step}: {name} differs after the row state advanced")
     if all(steps[-1]["active"]):
         raise SystemExit("no row retired: the fixture would not cover inactive rows")
 

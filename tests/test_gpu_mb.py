@@ -18,7 +18,8 @@ from gpu_helpers import bf16_close, rel_close, tensor_rel_close
 from pyvm_mb_oracle import BatchInstructionVM
 from qimeng_megakernel_amd import synthetic
 from qimeng_megakernel_amd.decode_schedule.model_config import LLAMA_3_2_1B, LlamaConfig
-from qimeng_megakernel_amd.decode_schedule_mb import decode_state, mk_kernel
+from qimeng_megakernel_amd.decode_schedule_mb import mk_kernel
+from qimeng_megakernel_amd.decode_schedule_mb.row_state import RowState
 from qimeng_megakernel_amd.decode_schedule_mb.instructions import scheduler as S
 
 pytestmark = pytest.mark.gpu
@@ -65,7 +66,7 @@ def make_pair(weights, rows, positions, *, inactive=(), capacity=None, shape=MB_
     cpu.position_ids.copy_(torch.tensor(positions, dtype=torch.int32))
     for r in inactive:
         cpu.active_mask[r] = False
-    decode_state.ensure_decode_state(cpu, rows, torch.device("cpu"))
+    RowState.of(cpu)
     sync_state(cpu, gpu)
     return cpu, gpu
 
@@ -209,7 +210,7 @@ def test_request_of_the_reference_fixture(weights):
     g.k_cache.copy_(torch.randn(g.k_cache.shape, generator=gen).bfloat16())
     g.v_cache.copy_(torch.randn(g.v_cache.shape, generator=gen).bfloat16())
     g.position_ids.copy_(torch.tensor(FIX["start_positions"], dtype=torch.int32))
-    decode_state.ensure_decode_state(g, FIX["rows"], g.hidden_states.device)
+    state = RowState.of(g)
     mk = mk_kernel.get_mk(spin_limit=1 << 18)
     tokens = list(FIX["start_tokens"])
     for step, want in enumerate(FIX["steps"]):
@@ -225,7 +226,7 @@ def test_request_of_the_reference_fixture(weights):
         assert int((got - ref).abs().max()) <= 8, (step, got.tolist(), ref.tolist())
         nxt = g.logits.float().argmax(dim=-1)
         assert nxt.tolist() == want["my_vm"]["tokens"], step
-        decode_state.advance_decode_state(g, nxt, [FIX["eos_token"]] if step >= 1 else [])
+        state.advance(nxt, [FIX["eos_token"]] if step >= 1 else [])
         tokens = nxt.tolist()
     assert g.active_mask.tolist() == [True, False, True]
 

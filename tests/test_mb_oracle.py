@@ -28,7 +28,8 @@ from fused_oracle import FusedOracle  # noqa: E402
 from pyvm_mb_oracle import BatchInstructionVM  # noqa: E402
 from qimeng_megakernel_amd import synthetic  # noqa: E402
 from qimeng_megakernel_amd.decode_schedule.model_config import LLAMA_3_2_1B, LlamaConfig  # noqa: E402
-from qimeng_megakernel_amd.decode_schedule_mb import decode_state, mk_kernel  # noqa: E402
+from qimeng_megakernel_amd.decode_schedule_mb import mk_kernel  # noqa: E402
+from qimeng_megakernel_amd.decode_schedule_mb.row_state import RowState, rows_of  # noqa: E402
 from qimeng_megakernel_amd.decode_schedule_mb.globs import Globals  # noqa: E402
 from qimeng_megakernel_amd.decode_schedule_mb.instructions import instruction_defs as D  # noqa: E402
 from qimeng_megakernel_amd.decode_schedule_mb.instructions import scheduler as S  # noqa: E402
@@ -60,7 +61,7 @@ def _request(weights):
     g.k_cache.copy_(torch.randn(g.k_cache.shape, generator=gen).bfloat16())
     g.v_cache.copy_(torch.randn(g.v_cache.shape, generator=gen).bfloat16())
     g.position_ids.copy_(torch.tensor(FIX["start_positions"], dtype=torch.int32))
-    decode_state.ensure_decode_state(g, FIX["rows"], torch.device("cpu"))
+    RowState.of(g)
     return g
 
 
@@ -175,9 +176,9 @@ def test_request_of_the_reference_fixture(weights):
             assert _bits(g.logits.gather(1, ids)) == want[name]["top_bits"], (step, name)
             nxt = g.logits.float().argmax(dim=-1)
             assert nxt.tolist() == want[name]["tokens"]
-            decode_state.advance_decode_state(g, nxt, [FIX["eos_token"]] if step >= 1 else [])
+            RowState.of(g).advance(nxt, [FIX["eos_token"]] if step >= 1 else [])
             toks[name] = nxt.tolist()
-    assert vm_g.active_mask.tolist() == [True, False, True] and vm_g.eos_reached.tolist() == [False, True, False]
+    assert vm_g.active_mask.tolist() == [True, False, True] and RowState.of(vm_g).finished.tolist() == [False, True, False]
 
 
 def test_every_row_of_a_batch_equals_that_row_alone(weights):
@@ -245,19 +246,27 @@ def test_vm_agrees_with_fused_and_counters_complete(weights):
 
 
 # ---------------------------------------------------------------- row state ----
-def test_decode_state_advances_and_retires_rows():
+def test_row_state_advances_and_retires_rows():
     g = Globals(hidden_states=torch.zeros(3, 4), position_ids=torch.tensor([5, 0, 9], dtype=torch.int32))
-    decode_state.ensure_decode_state(g, 3, torch.device("cpu"))
-    assert g.kv_lengths.tolist() == [6, 1, 10] and g.active_mask.tolist() == [True] * 3
-    decode_state.advance_decode_state(g, torch.tensor([7, 2, 8]), [2])
+    state = RowState.of(g)
+    assert RowState.of(g) is state and g.active_mask is state.active_mask and g.position_ids is state.position_ids
+    assert state.kv_lengths().tolist() == [6, 1, 10] and g.active_mask.tolist() == [True] * 3
+    state.advance(torch.tensor([7, 2, 8]), [2])
     assert g.position_ids.tolist() == [6, 0, 10] and g.active_mask.tolist() == [True, False, True]
-    assert g.eos_reached.tolist() == [False, True, False] and g.kv_lengths.tolist() == [7, 1, 11]
-    decode_state.advance_decode_state(g, torch.tensor([2, 2, 3]), [2])      # a retired row stays retired
+    assert state.finished.tolist() == [False, True, False] and state.kv_lengths().tolist() == [7, 1, 11]
+    state.advance(torch.tensor([2, 2, 3]), torch.tensor([2]))      # a retired row stays retired
     assert g.position_ids.tolist() == [6, 0, 11] and g.active_mask.tolist() == [False, False, True]
-    assert g.last_generated_tokens.tolist() == [2, 2, 3]
-    assert decode_state.instruction_active(0, g, 2) is False and decode_state.instruction_active(1, g, 0) is True
-    assert decode_state.instruction_active(-1, g, 2) is True and decode_state.instruction_active(-1, g, 0) is False
-    assert decode_state.batch_size(g) == 3 and decode_state.decode_pos_id(g, 2) == 11 and decode_state.kv_length(g, 2) == 12
+    assert state.finished.tolist() == [True, True, False] and state.last_tokens.tolist() == [2, 2, 3]
+    state.advance(torch.tensor([4, 4, 4]))                         # no end-of-sequence tokens: only the live row moves
+    assert g.position_ids.tolist() == [6, 0, 12]
+    assert state.follows(0, 2) is False and state.follows(1, 0) is True
+    assert state.follows(-1, 2) is True and state.follows(-1, 0) is False
+    assert rows_of(g) == 3 and state.rows == 3 and state.position(2) == 12
+    state.restart(4)
+    assert g.position_ids.tolist() == [4, 4, 4] and g.active_mask.tolist() == [True] * 3 and not state.finished.any()
+    # a caller that replaces one of the two boundary tensors gets a fresh state bound to the new one
+    g.active_mask = torch.tensor([True, False, True])
+    assert RowState.of(g) is not state and RowState.of(g).active_mask is g.active_mask
 
 
 def test_mk_of_the_batch_route_checks_its_arguments(weights):
