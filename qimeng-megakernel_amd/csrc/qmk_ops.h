@@ -231,10 +231,7 @@ __device__ __forceinline__ uint32_t rope_pair(float v0, float v1, const float* c
 }
 
 // ------------------------------------------------------------ streaming ----
-#ifndef QMK_DEPTH
-#define QMK_DEPTH 4
-#endif
-constexpr int kDepth = QMK_DEPTH;  // row buffers per wave: 4 x CH x 16 B per lane in flight
+constexpr int kDepth = 4;  // row buffers per wave: 4 x CH x 16 B per lane in flight
 
 // Wave w consumes elements w, w+8, w+16, ... of a sequence of weight-row segments
 // (`src(e)` = address of CH*512 bf16) through NB register buffers.  `buf[k]` must already hold
@@ -277,14 +274,8 @@ __device__ __forceinline__ void stream(int n, Src src, RowRegs<CH> (&buf)[NB], U
   }
 }
 
-#ifndef QMK_EARLY
-#define QMK_EARLY 2
-#endif
-#ifndef QMK_UPGATE_BUFFERS
-#define QMK_UPGATE_BUFFERS 4
-#endif
-constexpr int kEarly = QMK_EARLY;                    // buffers of the down projection requested before its wait
-constexpr int kUpGateBuffers = QMK_UPGATE_BUFFERS;   // row buffers of the up/gate GEMV
+constexpr int kEarly = 2;           // buffers of the down projection requested before its wait
+constexpr int kUpGateBuffers = 4;   // row buffers of the up/gate GEMV
 
 // Rows that one instruction requests for the next one of its queue: the O-proj has three of its
 // four row buffers to spare and waits for the whole attention phase, in which the memory system

@@ -16,7 +16,6 @@ tests check.
 from __future__ import annotations
 
 import dataclasses
-import os
 from dataclasses import dataclass
 from typing import Any, Iterable, Sequence
 
@@ -302,6 +301,7 @@ def mi355x_scheduler(
     kv_capacity: int | None = None,
     num_partials: int | None = None,
     attention_merge: str = "oproj",
+    oproj_spares_attention: bool = True,
 ) -> DecodeScheduler:
     shape = shape or LlamaConfig.shape()
     geometry = dataclasses.replace(MI355X_GEOMETRY, split_k=shape.intermediate_size)
@@ -311,8 +311,7 @@ def mi355x_scheduler(
     if blocks % sm_count != 0 and (2 * blocks) % sm_count == 0:
         geometry = dataclasses.replace(geometry, upgate_tile_n=geometry.upgate_tile_n // 2)
     p = num_partials or pick_num_partials(sm_count, kv_capacity, shape=shape)
-    return DecodeScheduler(shape, geometry, sm_count, p, attention_merge,
-                           oproj_spares_attention=os.environ.get("QMK_OPROJ_SPARES", "1") != "0")
+    return DecodeScheduler(shape, geometry, sm_count, p, attention_merge, oproj_spares_attention=oproj_spares_attention)
 
 
 def scheduler_for(globs: Any) -> DecodeScheduler:
@@ -321,17 +320,12 @@ def scheduler_for(globs: Any) -> DecodeScheduler:
     device = _get_device(globs)
     sm_count = _get_sm_count(device)
     kv_capacity = int(globs.k_cache.shape[2]) if getattr(globs, "k_cache", None) is not None else None
-    merge = os.environ.get("QMK_ATTENTION_MERGE", "oproj")
-    max_p = MAX_SELF_MERGE_PARTIALS if merge == "oproj" else MAX_ATTENTION_PARTIALS
+    max_p = MAX_SELF_MERGE_PARTIALS
     lse = getattr(globs, "attn_lse_intermediates", None)
     if lse is not None:
         max_p = min(max_p, int(lse.shape[-1]))
     p = pick_num_partials(sm_count, kv_capacity, max_partials=max_p)
-    override = os.environ.get("QMK_NUM_PARTIALS")  # tuning knob: force the split-KV fan-out
-    if override:
-        p = max(1, min(int(override), max_p))
-    sched = mi355x_scheduler(sm_count=sm_count, num_partials=p,
-                             attention_merge=merge)
+    sched = mi355x_scheduler(sm_count=sm_count, num_partials=p)
     if cached == sched:
         return cached
     try:
