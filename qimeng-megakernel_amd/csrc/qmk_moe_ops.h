@@ -192,6 +192,13 @@ __device__ __forceinline__ bool op_topk(const Params& p, Smem<M>& s, const Ctx& 
         const int oi = __shfl_xor(idx, off);
         if (ob > best || (ob == best && oi < idx)) best = ob, idx = oi;
       }
+      if (idx < 0 || idx >= E) {   // no logit compares greater than "nothing": NaNs from a broken router row
+        if (lane == 0) {
+          s.ctl[0] = 1;
+          report_error(p, QMK_DEV_BAD_OPERAND, c.inst_idx, c.opcode, j);
+        }
+        break;   // uniform: every lane holds the same idx
+      }
       if (lane == 0) {
         __hip_atomic_store(p.expert_indices + j, static_cast<long long>(idx), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         st_shared_f32(p.expert_weights + j, best / sum);
@@ -206,6 +213,7 @@ __device__ __forceinline__ bool op_topk(const Params& p, Smem<M>& s, const Ctx& 
   }
   release_stores();
   __syncthreads();
+  if (s.ctl[0]) return false;
   if (c.tid == 0) __hip_atomic_store(counter_ptr(p, layer, ROW_TOPK, 0), 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
   return true;
 }

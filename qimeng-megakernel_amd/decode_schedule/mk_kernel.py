@@ -186,6 +186,7 @@ class MegaKernel:
         self.tagged = tagged
         self._tagged = False
         self._workspace: torch.Tensor | None = None
+        self._barriers: torch.Tensor | None = None   # the counters of the bound launch: cleared by check() after an error
         self._greedy: tuple[torch.Tensor, torch.Tensor, int] | None = None
         self.timeline: torch.Tensor | None = None
         self._args = QmkArgs()
@@ -206,12 +207,16 @@ class MegaKernel:
         handle = (stream or torch.cuda.current_stream()).cuda_stream
         code = int(self._lib.qmk_status_fetch(_P(handle), ctypes.byref(detail)))
         if code != 0:
+            # A workgroup that gives up does not retire: the counters, the arrival word and the tagged units are
+            # those of a step that never finished, and the next launch would take them for its own.
             if self._workspace is not None:
-                self._workspace.zero_()  # units of the aborted step must not pass for the next one's
+                self._workspace.zero_()
+            if self._barriers is not None:
+                self._barriers.zero_()
             raise RuntimeError(
                 f"megakernel device error {code} ({self.error_string(code)}): workgroup={detail[0]} "
                 f"instruction={detail[1]} opcode={detail[2]} operand={detail[3]}; "
-                "the counters are undefined now — zero `barriers` before the next step"
+                "the counters (and the workspace) of the aborted step have been cleared"
             )
 
     def with_options(self, **kw: Any) -> "MegaKernel":
@@ -271,6 +276,7 @@ class MegaKernel:
         (instructions, hidden, _q, k_cache, v_cache, _ao, lse, part, silu, logits, attn_norm, qkv, cos, sin, o_w,
          mlp_norm, up, gate, down, lm_norm, lm_w, barriers) = tensors
         L = int(barriers.shape[0])
+        self._barriers = barriers
         H, F = shape.hidden_size, shape.intermediate_size
 
         def expect(name: str, t: torch.Tensor, want: tuple[int, ...]) -> None:

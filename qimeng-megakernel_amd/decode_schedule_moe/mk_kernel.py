@@ -72,6 +72,7 @@ class MoeMegaKernel:
         self.spin_limit = int(spin_limit)
         self.timeline: torch.Tensor | None = None
         self._workspace: torch.Tensor | None = None
+        self._barriers: torch.Tensor | None = None   # the counters of the bound launch: cleared by check() after an error
         self._args = QmkMoeArgs()
         self._args.struct_size = ctypes.sizeof(QmkMoeArgs)
         self._args.model = QMK_MODEL_QWEN1_5_MOE_A2_7B
@@ -86,12 +87,15 @@ class MoeMegaKernel:
         handle = (stream or torch.cuda.current_stream()).cuda_stream
         code = int(self._lib.qmk_status_fetch(_P(handle), ctypes.byref(detail)))
         if code != 0:
+            # A workgroup that gives up does not retire: counters and tagged units are those of an unfinished step.
             if self._workspace is not None:
-                self._workspace.zero_()  # units of the aborted step must not pass for the next one's
+                self._workspace.zero_()
+            if self._barriers is not None:
+                self._barriers.zero_()
             raise RuntimeError(
                 f"megakernel device error {code} ({self.error_string(code)}): workgroup={detail[0]} "
                 f"instruction={detail[1]} opcode={detail[2]} operand={detail[3]}; "
-                "the counters are undefined now — zero `barriers` before the next step"
+                "the counters (and the workspace) of the aborted step have been cleared"
             )
 
     def with_options(self, **kw: Any) -> "MoeMegaKernel":
@@ -144,6 +148,7 @@ class MoeMegaKernel:
         if tensors["rope_cos"].shape != tensors["rope_sin"].shape or tensors["rope_cos"].shape[-1] != 128:
             raise ValueError("rope_cos/rope_sin must both be [positions, head_dim]")
         bar = tensors["barriers"]
+        self._barriers = bar
         if bar.dim() != 3 or bar.shape[1] < 15 or bar.shape[2] < 128:
             raise ValueError(f"barriers must be [layers, >= 15, >= 128], got {tuple(bar.shape)}")
         a.num_queues, a.num_insts = int(tensors["instructions"].shape[0]), int(tensors["instructions"].shape[1])

@@ -49,6 +49,38 @@ def test_wait_timeout_drains_the_grid(gpu):
     assert int(g.barriers[0, 3, 0]) == sched.expected_counts()[1]
 
 
+def test_a_failed_step_leaves_nothing_behind_for_the_next_one(small_model):
+    """A whole step that aborts half way (its wait budget is too small for the real waits) leaves counters, an
+    arrival word and tagged units of a step that never finished; check() clears them, so the same request
+    simply carries on and ends where an undisturbed one ends."""
+    shape, w, _ = small_model
+    LlamaConfig.set_shape(shape)
+
+    def request(fail_at):
+        g = synthetic.build_globals(w, shape, 32, "cuda:0")
+        S.build(g)
+        mk, tok = mk_kernel.get_mk(), 7
+        for pos in range(6):
+            g.hidden_states.copy_(g.embed_tokens[tok]); g.position_id = pos
+            if pos == fail_at:
+                keep = (g.hidden_states.clone(), g.k_cache.clone(), g.v_cache.clone())
+                broken = mk.with_options(spin_limit=1)
+                mk_kernel.call_mk(g, broken)
+                with pytest.raises(RuntimeError, match="ran out of polls|cleared"):
+                    broken.check()
+                assert int(g.barriers.abs().sum()) == 0
+                g.hidden_states.copy_(keep[0]); g.k_cache.copy_(keep[1]); g.v_cache.copy_(keep[2])
+            mk_kernel.call_mk(g, mk)
+            tok = int(g.logits.argmax())
+        mk.check()
+        return g, tok
+
+    (plain, tok_plain), (hurt, tok_hurt) = request(None), request(3)
+    assert tok_plain == tok_hurt
+    for name in ("hidden_states", "logits", "k_cache", "v_cache", "attn_out", "silu_out"):
+        assert torch.equal(getattr(plain, name), getattr(hurt, name)), name
+
+
 def test_xcd_edge_wait_timeout(gpu):
     shape, g = gpu
     sched = S.mi355x_scheduler(shape, num_partials=1)
