@@ -6,13 +6,18 @@ output length 1024): seeded random-init weights, 8-token random prompt, KV prefi
 through the decode kernel, then forced greedy continuation.  One "step" is one
 decode step = one megakernel launch = one new token.
 
-  python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu-baseline]
+  python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu-baseline] [--lengths 128,256,512,1024]
 
-W untimed steps run as a separate short request first; then a fresh request is
-prefilled and exactly K decode steps are timed the way the reference times them
-(`qimeng_megakernel/models/LLM/decode.py:719-792`): one HIP event pair per step
-around the kernel launch only -> kernel_tok_s (the metric), one pair around the
-loop -> tok_s_gpu, perf_counter -> tok_s.  Prints ONE JSON line.
+W untimed steps run as a separate short request first; then the request of the
+metric's configuration is run — prompt, prefill, 1024 new tokens (contexts up to
+prompt + 1023) — and exactly its LAST K decode steps are timed (all 1023 by
+default; the steps before them run untimed, then the device is synchronised), the
+way the reference times them (`qimeng_megakernel/models/LLM/decode.py:719-792`):
+one HIP event pair per step around the kernel launch only -> kernel_tok_s (the
+metric), one pair around the loop -> tok_s_gpu, perf_counter -> tok_s.  Prints
+ONE JSON line.  `--lengths` adds the reference's output-length matrix
+(`benchmarks/llm_decode.py:36-43, 195-254`: warm-up iterations, then the mean of
+the bench iterations per length) under the key "lengths".
 
 `roofline.achieved` = algorithmic bytes of the K timed launches (bf16 weights +
 KV rows read + KV row written, see DecodeShape.step_bytes) / summed launch time.
@@ -43,7 +48,8 @@ MEASURED_TRAFFIC_OVER_ALGORITHMIC_MOE = 1.0134
 
 
 def cpu_baseline(shape, weights, prompt, n_steps: int, cores: int, shape_name: str) -> dict:
-    """Time the CPU oracle on single-token steps of the same request (bounded sample)."""
+    """BASELINE config 1 on the host: the prompt is prefilled through the single-token path (untimed), then
+    ``n_steps`` greedy decode steps of the same seeded request are timed (a bounded sample of its 128)."""
     import torch
 
     sys.path.insert(0, str(ROOT / "oracle"))
@@ -51,26 +57,29 @@ def cpu_baseline(shape, weights, prompt, n_steps: int, cores: int, shape_name: s
     from qimeng_megakernel_amd import synthetic
 
     torch.set_num_threads(cores)
-    g = synthetic.build_globals(weights, shape, prompt.numel() + n_steps + 1, "cpu")
+    T = int(prompt.numel())
+    g = synthetic.build_globals(weights, shape, T + n_steps + 1, "cpu")
     oracle = FusedOracle(shape)
     toks = prompt.tolist()
-    # one untimed step pages the weights in
-    oracle.embed(g, toks[0]); g.position_id = 0; oracle.decode_step(g)
-    t0 = time.perf_counter()
-    for pos in range(n_steps):
+    for pos in range(T):      # prefill; also pages the weights in
         oracle.embed(g, toks[pos]); g.position_id = pos
         oracle.decode_step(g)
-        if pos + 1 >= len(toks):
-            toks.append(int(g.logits.argmax()))
+    toks.append(int(g.logits.argmax()))
+    t0 = time.perf_counter()
+    for pos in range(T, T + n_steps):
+        oracle.embed(g, toks[pos]); g.position_id = pos
+        oracle.decode_step(g)
+        toks.append(int(g.logits.argmax()))
     dt = time.perf_counter() - t0
     return {
         "value": n_steps / dt,
         "unit": "tok/s",
         "cores": cores,
+        "host_cpu_count": os.cpu_count(),
         "kind": "port",
-        "sample": f"{n_steps} single-token decode steps (positions 0..{n_steps - 1}: the {prompt.numel()}-token prompt through "
-                  f"the single-token path, then greedy steps) of the same seeded {shape_name}-shaped request, "
-                  f"torch {torch.__version__} bf16 on {cores} threads, {dt:.1f} s",
+        "sample": f"{n_steps} greedy decode steps (contexts {T + 1}..{T + n_steps}) behind the {T}-token prompt of the same seeded "
+                  f"{shape_name}-shaped request (the prompt prefilled through the single-token path, untimed), "
+                  f"torch {torch.__version__} bf16 on {cores} threads of {os.cpu_count()} host CPUs, {dt:.1f} s",
     }
 
 
@@ -290,7 +299,15 @@ def main() -> None:
     ap.add_argument("--warmup", type=int, default=16)
     ap.add_argument("--seed", type=int, default=0)
     ap.add_argument("--prompt-len", type=int, default=8)
-    ap.add_argument("--cpu-steps", type=int, default=10)
+    ap.add_argument("--new-tokens", type=int, default=1024,
+                    help="output length of the request (the metric's configuration: 1024); the last --steps of its "
+                         "decode steps are timed")
+    ap.add_argument("--lengths", default="",
+                    help="comma-separated output lengths (the reference's matrix: 128,256,512,1024): each is run "
+                         "--length-warmup-iters + --length-bench-iters times and the mean tok_s / tok_s_gpu / kernel_tok_s reported")
+    ap.add_argument("--length-warmup-iters", type=int, default=2)
+    ap.add_argument("--length-bench-iters", type=int, default=5)
+    ap.add_argument("--cpu-steps", type=int, default=16)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--model", choices=("llama-3.2-1b", "qwen3-1.7b", "qwen1.5-moe-a2.7b"), default="llama-3.2-1b",
                     help="layer geometry: the headline Llama-3.2-1B shape, the Qwen3-1.7B shape with the Qwen3 op set "
@@ -347,8 +364,10 @@ def main() -> None:
     LlamaConfig.set_shape(shape)
     device = torch.device("cuda:0")
     torch.cuda.set_device(device)
-    new_tokens = args.steps + 1
-    kv_capacity = args.prompt_len + new_tokens
+    lengths = [int(x) for x in args.lengths.split(",") if x.strip()]
+    new_tokens = max(args.new_tokens, args.steps + 1)
+    timed = min(args.steps, new_tokens - 1)
+    kv_capacity = args.prompt_len + max([new_tokens] + lengths)
     weights = synthetic.random_weights(shape, args.seed, max_positions=kv_capacity)
     prompt = synthetic.random_prompt(shape, args.seed, args.prompt_len)
     globs = synthetic.build_globals(weights, shape, kv_capacity, device)
@@ -364,18 +383,35 @@ def main() -> None:
         decode.decode(globs, prompt, min(args.warmup + 1, new_tokens), mk=mk, decode_time=False)
     globs.k_cache.zero_(); globs.v_cache.zero_()
     torch.cuda.synchronize(device)
-    out = decode.decode(globs, prompt, new_tokens, mk=mk, decode_time=True, device_sampling=not args.host_sampling)
+    out = decode.decode(globs, prompt, new_tokens, mk=mk, decode_time=True, device_sampling=not args.host_sampling,
+                        timed_steps=timed)
     torch.cuda.synchronize(device)
     t = out["timing"]
     tokens = out["new_tokens"][0].tolist()
     graph_tok_s = None
     if not args.no_graph_run and not args.host_sampling:
-        # The same request once more as ONE HIP graph of all decode launches (no per-step events).
+        # The same request once more with the timed launches as ONE HIP graph (no per-step events).
         globs.k_cache.zero_(); globs.v_cache.zero_()
-        g_out = decode.decode(globs, prompt, new_tokens, mk=mk, decode_time=True, use_graph=True)
+        g_out = decode.decode(globs, prompt, new_tokens, mk=mk, decode_time=True, use_graph=True, timed_steps=timed)
         if g_out["new_tokens"][0].tolist() != tokens:
             raise SystemExit("bench.py: the graph replay produced different tokens than the launch loop")
         graph_tok_s = g_out["timing"]["effective_tok_s_gpu"]
+
+    matrix = {}
+    for n in lengths:   # the reference's output-length matrix: warm-up runs, then the mean over the bench runs
+        samples = []
+        for it in range(args.length_warmup_iters + args.length_bench_iters):
+            globs.k_cache.zero_(); globs.v_cache.zero_()
+            r = decode.decode(globs, prompt, n, mk=mk, decode_time=True, device_sampling=not args.host_sampling)
+            if it >= args.length_warmup_iters:
+                samples.append((r["timing"], r["new_tokens"][0].tolist()))
+        mean = lambda key: sum(tm[key] for tm, _ in samples) / len(samples)
+        matrix[f"b1_t{n}"] = {
+            "max_new_tokens": n, "eos_policy": "forced_continuation", "bench_iters": len(samples), "warmup_iters": args.length_warmup_iters,
+            "tok_s": mean("effective_tok_s_wall"), "tok_s_gpu": mean("effective_tok_s_gpu"), "kernel_tok_s": mean("kernel_tok_s"),
+            "achieved_GBps": mean("achieved_GBps"), "hbm_frac": mean("achieved_GBps") / HBM_PEAK_GBPS,
+            "greedy_rerun_match": all(tk == samples[0][1] for _, tk in samples[1:]),
+        }
 
     golden = ROOT / "tests" / "golden" / "llama1b_seed0.json"
     match = None
@@ -384,14 +420,14 @@ def main() -> None:
         n = min(len(want), len(tokens))
         match = next((i for i in range(n) if tokens[i] != want[i]), n)
 
-    ctx_first, ctx_last = args.prompt_len + 1, args.prompt_len + args.steps
+    ctx_first, ctx_last = t["first_timed_context"], t["last_timed_context"]
     achieved = t["achieved_GBps"]
     line = {
         "metric": "kernel_tok_s",
         "value": t["kernel_tok_s"],
         "unit": "tok/s",
         "n_gpus": 1,
-        "steps": args.steps,
+        "steps": timed,
         "warmup": args.warmup,
         "ms_per_step": t["kernel_ms_per_step"],
         "higher_is_better": True,
@@ -401,7 +437,8 @@ def main() -> None:
         "data": "synthetic",
         "config": {
             "workload": f"{model_name}-shaped batch-1 greedy decode, {args.prompt_len}-token prompt, "
-                        f"{new_tokens} new tokens (context {ctx_first}..{ctx_last}), seeded random-init bf16 weights",
+                        f"{new_tokens} new tokens; timed: the last {timed} decode steps (contexts {ctx_first}..{ctx_last}), "
+                        f"seeded random-init bf16 weights",
             "layers": shape.num_hidden_layers, "hidden": shape.hidden_size, "ffn": shape.intermediate_size,
             "q_heads": shape.num_attention_heads, "kv_heads": shape.num_key_value_heads, "head_dim": shape.head_dim,
             "vocab": shape.vocab_size, "batch": 1, "seed": args.seed,
@@ -420,14 +457,16 @@ def main() -> None:
             "unit": "GB/s",
             "frac": achieved / HBM_PEAK_GBPS,
             # the counter runs were made on the Llama-shaped kernel only
-            "traffic": (MEASURED_TRAFFIC_OVER_ALGORITHMIC * t["algorithmic_bytes"] / max(args.steps, 1)
+            "traffic": (MEASURED_TRAFFIC_OVER_ALGORITHMIC * t["algorithmic_bytes"] / max(timed, 1)
                         if args.model == "llama-3.2-1b" else None),
-            "bytes_per_launch_avg": t["algorithmic_bytes"] / max(args.steps, 1),
+            "bytes_per_launch_avg": t["algorithmic_bytes"] / max(timed, 1),
             "kernel": "decode_megakernel<Llama1B>" if args.model == "llama-3.2-1b" else "decode_megakernel<Qwen3_1p7B>",
         },
     }
+    if matrix:
+        line["lengths"] = matrix
     if not args.no_cpu_baseline:
-        cores = min(os.cpu_count() or 1, 16)
+        cores = min(os.cpu_count() or 1, 16)   # a GPU box gives one job 16 cores, whatever it reports
         line["cpu_baseline"] = cpu_baseline(shape, weights, prompt, args.cpu_steps, cores, model_name)
     print(json.dumps(line))
 

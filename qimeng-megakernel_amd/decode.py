@@ -125,12 +125,15 @@ def decode(
     decode_time: bool = True,
     device_sampling: bool = False,
     use_graph: bool = False,
+    timed_steps: int | None = None,
 ) -> dict[str, Any]:
     """Prefill + forced greedy decode to exactly ``max_new_tokens`` tokens (no EOS stop).
 
     ``device_sampling``: argmax and embedding lookup run inside the kernel.  ``use_graph`` (implies
     ``device_sampling``): the decode launches are captured into one HIP graph and replayed once;
-    per-step kernel times are then not available (``kernel_tok_s`` is reported as 0)."""
+    per-step kernel times are then not available (``kernel_tok_s`` is reported as 0).
+    ``timed_steps``: only the last that many decode steps of the request are timed (and captured);
+    the steps before them run untimed, followed by a device synchronisation.  Default: all of them."""
     device = globs.hidden_states.device
     prompt_len = int(prompt_ids.numel())
     if prompt_len + max_new_tokens > globs.k_cache.shape[2]:
@@ -147,7 +150,15 @@ def decode(
         prefill_by_decode(globs, mk, prompt_ids, sample_into=(output_tokens, prompt_len))
     else:
         output_tokens[0, prompt_len] = prefill_by_decode(globs, mk, prompt_ids)
-    ntok = max(max_new_tokens - 1, 0)
+    total = max(max_new_tokens - 1, 0)
+    ntok = total if timed_steps is None else max(0, min(int(timed_steps), total))
+    lead = total - ntok
+    if lead:   # the untimed head of the request
+        if device_sampling:
+            generate_greedy_on_device(globs, output_tokens, prompt_len, lead, mk=mk)
+        else:
+            generate_greedy_fast(globs, output_tokens, prompt_len, lead, call_mk=lambda g: _mk_kernel.call_mk(g, mk))
+        prompt_len += lead
     graph = None
     if use_graph and ntok > 0:
         # Capture on a side stream (as torch requires); every launch carries its own position and
@@ -172,7 +183,7 @@ def decode(
     else:
         generate_greedy_fast(globs, output_tokens, prompt_len, ntok, call_mk=lambda g: _mk_kernel.call_mk(g, mk),
                              mk_step_events=events)
-    result: dict[str, Any] = {"generated_ids": output_tokens, "new_tokens": output_tokens[:, prompt_len:]}
+    result: dict[str, Any] = {"generated_ids": output_tokens, "new_tokens": output_tokens[:, prompt_len - lead:]}
     if decode_time:
         loop_end.record()
         torch.cuda.synchronize(device)
@@ -189,7 +200,9 @@ def decode(
             "decode_gpu_s": decode_gpu_s,
             "mk_kernel_gpu_s": mk_kernel_gpu_s,
             "non_kernel_gpu_s": max(decode_gpu_s - mk_kernel_gpu_s, 0.0),
-            "effective_new_tokens": ntok + 1,
+            "effective_new_tokens": total + 1,
+            "first_timed_context": prompt_len + 1,
+            "last_timed_context": prompt_len + ntok,
             "decode_window_new_tokens": window,
             "effective_tok_s_wall": window / decode_wall_s if window and decode_wall_s > 0 else 0.0,
             "effective_tok_s_gpu": window / decode_gpu_s if window and decode_gpu_s > 0 else 0.0,
