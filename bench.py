@@ -200,43 +200,54 @@ def batch_decode(args) -> dict:
 
 
 def moe_decode(args) -> dict:
-    """Qwen1.5-MoE-A2.7B-shaped greedy decode at batch 1 through the MoE route's kernel."""
+    """Greedy decode at batch 1 through the MoE route's kernel: the Qwen1.5-MoE-A2.7B shape (the reference's route) or
+    the Qwen3-30B-A3B shape (BASELINE config 5: 48 layers, 128 experts of 768, renormalised top-8, no shared expert,
+    32 query / 4 KV heads of 128 with the Qwen3 op set's attention; 61 GB of bf16 weights, drawn on the GPU)."""
+    import dataclasses
+
     import torch
 
     from qimeng_megakernel_amd import decode_moe, synthetic
     from qimeng_megakernel_amd.decode_schedule_moe import mk_kernel
-    from qimeng_megakernel_amd.decode_schedule_moe.model_config import QWEN1_5_MOE_A2_7B, QwenMoeConfig
+    from qimeng_megakernel_amd.decode_schedule_moe.model_config import QWEN1_5_MOE_A2_7B, QWEN3_30B_A3B, QwenMoeConfig
 
-    shape = QWEN1_5_MOE_A2_7B
+    a3b = args.model == "qwen3-30b-a3b"
+    shape = QWEN3_30B_A3B if a3b else QWEN1_5_MOE_A2_7B
+    name = "Qwen3-30B-A3B" if a3b else "Qwen1.5-MoE-A2.7B"
     QwenMoeConfig.set_shape(shape)
     device = torch.device("cuda:0")
     torch.cuda.set_device(device)
-    new_tokens = args.steps + 1
+    # config 5 is quoted on 512 greedy steps; the reference's own shape keeps the length the steps ask for
+    new_tokens = max(args.new_tokens if args.new_tokens != 1024 else 512, args.steps + 1) if a3b else args.steps + 1
+    timed = min(args.steps, new_tokens - 1)
     kv_capacity = args.prompt_len + new_tokens
-    weights = synthetic.random_moe_weights(shape, args.seed, kv_capacity)
+    weights = synthetic.random_moe_weights(shape, args.seed, kv_capacity, device=device if a3b else "cpu")
     gen = torch.Generator().manual_seed(args.seed + 1_000_003)
     prompt = torch.randint(0, shape.vocab_size, (args.prompt_len,), generator=gen, dtype=torch.long)
-    globs = synthetic.build_moe_globals(weights, shape, kv_capacity, device)
+    globs = synthetic.build_moe_globals(weights, shape, kv_capacity, device, max_partials=8 if a3b else 27)
     mk = mk_kernel.get_mk()
     if args.copy_calibration:
         copy_calibration(device)
     if args.warmup > 0:
         decode_moe.decode(globs, prompt, min(args.warmup + 1, new_tokens), mk=mk, decode_time=False)
     globs.k_cache.zero_(); globs.v_cache.zero_()
-    out = decode_moe.decode(globs, prompt, new_tokens, mk=mk)
+    out = decode_moe.decode(globs, prompt, new_tokens, mk=mk, timed_steps=timed)
     t = out["timing"]
     eager_tokens = out["new_tokens"].clone()
     globs.k_cache.zero_(); globs.v_cache.zero_()
-    graphed = decode_moe.decode(globs, prompt, new_tokens, mk=mk, use_graph=True)   # the same loop as one HIP graph
+    graphed = decode_moe.decode(globs, prompt, new_tokens, mk=mk, use_graph=True, timed_steps=timed)   # the timed launches as one HIP graph
     line = {
-        "metric": "kernel_tok_s", "value": t["kernel_tok_s"], "unit": "tok/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "metric": "kernel_tok_s", "value": t["kernel_tok_s"], "unit": "tok/s", "n_gpus": 1, "steps": timed, "warmup": args.warmup,
         "ms_per_step": t["kernel_ms_per_step"], "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "bf16",
         "data": "synthetic",
         "config": {
-            "workload": f"Qwen1.5-MoE-A2.7B-shaped batch-1 greedy decode, {args.prompt_len}-token prompt, {new_tokens} new tokens "
-                        f"(context {args.prompt_len + 1}..{args.prompt_len + args.steps}), seeded random-init bf16 weights",
+            "workload": f"{name}-shaped batch-1 greedy decode, {args.prompt_len}-token prompt, {new_tokens} new tokens; timed: the last "
+                        f"{timed} decode steps (contexts {t['first_timed_context']}..{t['last_timed_context']}), seeded random-init bf16 "
+                        f"weights" + (" drawn on the GPU" if a3b else ""),
             "layers": shape.num_hidden_layers, "experts": shape.num_experts, "experts_per_token": shape.num_experts_per_tok,
-            "expert_ffn": shape.moe_intermediate_size, "shared_ffn": shape.intermediate_size, "batch": 1, "seed": args.seed,
+            "expert_ffn": shape.moe_intermediate_size, "shared_ffn": shape.intermediate_size, "renormalised_top_k": bool(shape.norm_topk_prob),
+            "q_heads": shape.num_attention_heads, "kv_heads": shape.num_key_value_heads, "head_dim": shape.head_dim, "qk_norm": bool(shape.qk_norm),
+            "batch": 1, "seed": args.seed, "weight_bytes": shape.weight_bytes_per_token(),
             "queues": int(globs.instructions.shape[0]), "instructions_per_queue": int(globs.instructions.shape[1]),
         },
         "tok_s": t["effective_tok_s_wall"], "tok_s_gpu": t["effective_tok_s_gpu"], "kernel_tok_s": t["kernel_tok_s"],
@@ -245,8 +256,10 @@ def moe_decode(args) -> dict:
         "first_tokens": out["new_tokens"][:8].tolist(),
         "roofline": {
             "bound": "hbm", "achieved": t["achieved_GBps"], "peak": HBM_PEAK_GBPS, "unit": "GB/s", "frac": t["achieved_GBps"] / HBM_PEAK_GBPS,
-            "traffic": MEASURED_TRAFFIC_OVER_ALGORITHMIC_MOE * t["algorithmic_bytes"] / max(args.steps, 1),
-            "bytes_per_launch_avg": t["algorithmic_bytes"] / max(args.steps, 1), "kernel": "decode_megakernel_moe<QwenMoeA2_7B>",
+            # the counter runs were made on the Qwen1.5-shaped kernel only
+            "traffic": None if a3b else MEASURED_TRAFFIC_OVER_ALGORITHMIC_MOE * t["algorithmic_bytes"] / max(timed, 1),
+            "bytes_per_launch_avg": t["algorithmic_bytes"] / max(timed, 1),
+            "kernel": "decode_megakernel_moe<Qwen3MoeA3B>" if a3b else "decode_megakernel_moe<QwenMoeA2_7B>",
         },
     }
     if not args.no_cpu_baseline:
@@ -255,17 +268,46 @@ def moe_decode(args) -> dict:
 
         cores = min(os.cpu_count() or 1, 16)
         torch.set_num_threads(cores)
-        g = synthetic.build_moe_globals(weights, shape, args.cpu_steps + 1, "cpu")
-        oracle = FusedMoeOracle(shape)
-        with torch.no_grad():
-            t0 = time.perf_counter()
-            for pos in range(args.cpu_steps):
-                g.hidden_states.copy_(g.embed_tokens[prompt[min(pos, len(prompt) - 1)]])
-                g.position_id = pos
-                oracle.decode_step(g)
-            dt = time.perf_counter() - t0
-        line["cpu_baseline"] = {"value": args.cpu_steps / dt, "unit": "tok/s", "cores": cores, "kind": "port",
-                                "sample": f"{args.cpu_steps} steps (contexts 1..{args.cpu_steps}) of the same workload through the fused MoE oracle"}
+        if a3b:
+            # 61 GB of weights do not go through host memory for a reported baseline: the fused oracle is timed on a
+            # 2-layer model of the same layer geometry (its own seeded weights) plus the LM head, and the step time of
+            # the 48-layer model is put together from the per-layer and the LM-head time.
+            small = dataclasses.replace(shape, num_hidden_layers=2)
+            w = synthetic.random_moe_weights(small, args.seed, args.cpu_steps + 1)
+            g = synthetic.build_moe_globals(w, small, args.cpu_steps + 1, "cpu", max_partials=8)
+            oracle = FusedMoeOracle(small)
+            t_layers = t_head = 0.0
+            with torch.no_grad():
+                for pos in range(args.cpu_steps + 1):
+                    g.hidden_states.copy_(g.embed_tokens[prompt[min(pos, len(prompt) - 1)]])
+                    g.position_id = pos
+                    t0 = time.perf_counter()
+                    for layer in range(2):
+                        oracle.decode_layer(g, layer)
+                    t1 = time.perf_counter()
+                    oracle.lm_head(g)
+                    if pos:   # the first step pages the weights in
+                        t_layers += t1 - t0
+                        t_head += time.perf_counter() - t1
+            per_layer, head = t_layers / (2 * args.cpu_steps), t_head / args.cpu_steps
+            line["cpu_baseline"] = {
+                "value": 1.0 / (shape.num_hidden_layers * per_layer + head), "unit": "tok/s", "cores": cores, "host_cpu_count": os.cpu_count(),
+                "kind": "port",
+                "sample": f"{args.cpu_steps} steps (contexts 2..{args.cpu_steps + 1}) of a 2-layer model of the same layer geometry through the "
+                          f"fused MoE oracle: {per_layer * 1e3:.1f} ms per layer, {head * 1e3:.1f} ms for the LM head; value = 1 / (48 layers + LM head)",
+            }
+        else:
+            g = synthetic.build_moe_globals(weights, shape, args.cpu_steps + 1, "cpu")
+            oracle = FusedMoeOracle(shape)
+            with torch.no_grad():
+                t0 = time.perf_counter()
+                for pos in range(args.cpu_steps):
+                    g.hidden_states.copy_(g.embed_tokens[prompt[min(pos, len(prompt) - 1)]])
+                    g.position_id = pos
+                    oracle.decode_step(g)
+                dt = time.perf_counter() - t0
+            line["cpu_baseline"] = {"value": args.cpu_steps / dt, "unit": "tok/s", "cores": cores, "host_cpu_count": os.cpu_count(), "kind": "port",
+                                    "sample": f"{args.cpu_steps} steps (contexts 1..{args.cpu_steps}) of the same workload through the fused MoE oracle"}
     return line
 
 
@@ -309,10 +351,11 @@ def main() -> None:
     ap.add_argument("--length-bench-iters", type=int, default=5)
     ap.add_argument("--cpu-steps", type=int, default=16)
     ap.add_argument("--no-cpu-baseline", action="store_true")
-    ap.add_argument("--model", choices=("llama-3.2-1b", "qwen3-1.7b", "qwen1.5-moe-a2.7b"), default="llama-3.2-1b",
+    ap.add_argument("--model", choices=("llama-3.2-1b", "qwen3-1.7b", "qwen1.5-moe-a2.7b", "qwen3-30b-a3b"), default="llama-3.2-1b",
                     help="layer geometry: the headline Llama-3.2-1B shape, the Qwen3-1.7B shape with the Qwen3 op set "
-                         "(28 layers, per-head QK RMSNorm, tied LM head), or the Qwen1.5-MoE-A2.7B shape with the MoE op set "
-                         "(24 layers, 60 experts of 1408 with top-4 routing, shared expert of 5632)")
+                         "(28 layers, per-head QK RMSNorm, tied LM head), the Qwen1.5-MoE-A2.7B shape with the MoE op set "
+                         "(24 layers, 60 experts of 1408 with top-4 routing, shared expert of 5632), or the Qwen3-30B-A3B shape "
+                         "(48 layers, 128 experts of 768 with renormalised top-8 routing, 32/4 heads of 128; 512 new tokens)")
     ap.add_argument("--host-sampling", action="store_true",
                     help="argmax and embedding lookup on the host between launches, as the reference's loop does "
                          "(default: inside the kernel)")
@@ -349,7 +392,7 @@ def main() -> None:
                           "config": {"workload": "Llama-3.2-1B layer geometry, batch 1, one decode step, KV cache ~N(0,1)"},
                           "value": res[max(res, key=int)]["GBps"], "contexts": res}))
         return
-    if args.model == "qwen1.5-moe-a2.7b":
+    if args.model in ("qwen1.5-moe-a2.7b", "qwen3-30b-a3b"):
         if args.batch != 1:
             raise SystemExit("bench.py: the MoE route runs at batch 1")
         print(json.dumps(moe_decode(args)))

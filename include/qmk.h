@@ -35,7 +35,7 @@
 extern "C" {
 #endif
 
-#define QMK_ABI_VERSION 6
+#define QMK_ABI_VERSION 7
 #define QMK_INSTRUCTION_WORDS 32
 
 /* Return / status codes. 0 is success; everything else is an error. */
@@ -63,9 +63,15 @@ enum {
   QMK_MODEL_QWEN1_5_MOE_A2_7B = 2, /* H 2048, 16 q / 16 kv heads, d 128, QKV bias; the MoE op set
                                   (…/qwen/qwen1_5_moe_a2_7b/A100/single_batch/decode_kernel/mk.h); expert
                                   count, top-k and FFN widths are launch parameters (qmk_decode_step_moe) */
-  QMK_MODEL_QWEN3_1_7B = 1     /* H 2048, F 6144, 16 q / 8 kv heads, d 128, per-head QK RMSNorm
+  QMK_MODEL_QWEN3_1_7B = 1,    /* H 2048, F 6144, 16 q / 8 kv heads, d 128, per-head QK RMSNorm
                                   (the Qwen3 op set: …/qwen/qwen3__0_6b/A100/single_batch/
                                   decode_kernel/mk.h, decode_schedule/mk_kernel.py:52-110)     */
+  QMK_MODEL_QWEN3_30B_A3B = 3  /* H 2048, 32 q / 4 kv heads, d 128 (attention output 4096 wide), per-head QK
+                                  RMSNorm, no QKV bias: the Qwen3 op set's attention in front of the MoE op
+                                  set (qmk_decode_step_moe), without a shared expert and with renormalised
+                                  top-k weights (norm_topk_prob: …/qwen1_5_moe_a2_7b/A100/single_batch/
+                                  decode_schedule/fused/operations.py:405).  The reference has no route
+                                  for this shape: it is its two routes put together                  */
 };
 
 /* qmk_query selectors. */
@@ -202,7 +208,7 @@ int qmk_decode_step(const QmkArgs* args);
  * capture, tight serving loops, harnesses that forbid hipMalloc.  Everything is as in
  * qmk_decode_step (same struct, same kernels, same results bit for bit), except that
  * args->workspace and args->workspace_bytes are ignored: the tagged units, the greedy candidates
- * and the launch count live in a static device array of the library (86 144 bytes per GPU, held
+ * and the launch count live in a static device array of the library (94 336 bytes per GPU, held
  * until the process ends; its address is looked up once per device on the first call of any entry
  * point there).  Limits of that array: at most 1024 queues when token_out is set and at most 63
  * layers with QMK_FLAG_TAGGED -- beyond them the call returns QMK_ERR_SCRATCH and launches nothing.
@@ -294,7 +300,7 @@ int qmk_decode_step_batch(const QmkBatchArgs* args);
  */
 typedef struct QmkMoeArgs {
   uint32_t struct_size;            /* = sizeof(QmkMoeArgs)                        */
-  uint32_t model;                  /* QMK_MODEL_QWEN1_5_MOE_A2_7B                 */
+  uint32_t model;                  /* QMK_MODEL_QWEN1_5_MOE_A2_7B or QMK_MODEL_QWEN3_30B_A3B */
   uint32_t flags;                  /* QMK_FLAG_KEEP_BARRIERS, QMK_FLAG_TAGGED (whole steps, not with KEEP_BARRIERS) */
   uint32_t spin_limit;
 
@@ -311,7 +317,7 @@ typedef struct QmkMoeArgs {
   void* logits;                    /* bf16 [vocab_size]                           */
   const void* attn_norm_weights;   /* bf16 [L, H]                                 */
   const void* qkv_weights;         /* bf16 [L, (Hq+2Hkv)*D, H]                    */
-  const void* qkv_bias;            /* bf16 [L, (Hq+2Hkv)*D]                       */
+  const void* qkv_bias;            /* bf16 [L, (Hq+2Hkv)*D]; NULL for QMK_MODEL_QWEN3_30B_A3B */
   const float* rope_cos;           /* f32  [rope_rows, D]                         */
   const float* rope_sin;
   const void* o_proj_weights;      /* bf16 [L, H, Hq*D]                           */
@@ -322,6 +328,7 @@ typedef struct QmkMoeArgs {
   float* router_logits_buf;        /* f32  [E]                                    */
   int64_t* expert_indices;         /* i64  [top_k]                                */
   float* expert_weights;           /* f32  [top_k]                                */
+  /* the six shared-expert tensors: NULL for a model without a shared expert (shared_ffn = 0) */
   const void* shared_expert_gate_proj_weights; /* bf16 [L, Fs, H]                 */
   const void* shared_expert_up_proj_weights;   /* bf16 [L, Fs, H]                 */
   const void* shared_expert_down_proj_weights; /* bf16 [L, H, Fs]                 */
@@ -347,9 +354,10 @@ typedef struct QmkMoeArgs {
   int32_t pos_id;
   int32_t num_experts;             /* E, <= 512                                   */
   int32_t top_k;                   /* experts per token, <= 8                     */
-  int32_t shared_ffn;              /* Fs, a multiple of 16                        */
+  int32_t shared_ffn;              /* Fs, a multiple of 16; 0 = no shared expert: the stream then holds no opcodes 10/11
+                                      and opcode 14 adds the routed experts only                                   */
   int32_t moe_ffn;                 /* Fm, a multiple of 16, <= 2048               */
-  int32_t shared_k_slices;         /* K slices of the shared down projection (4 in the reference) */
+  int32_t shared_k_slices;         /* K slices of the shared down projection (4 in the reference); 0 with shared_ffn = 0 */
   float attn_scale;
   float rms_norm_eps;
 
@@ -362,6 +370,15 @@ typedef struct QmkMoeArgs {
                                       the tagged units of QMK_FLAG_TAGGED (zeroed once when allocated, and again
                                       after a launch that reported a device error)                              */
   uint64_t workspace_bytes;
+
+  /* Qwen3 op set only (QMK_MODEL_QWEN3_30B_A3B; NULL otherwise), as in QmkArgs. */
+  void* qkv_raw;                   /* bf16 [(Hq+2Hkv)*D]  QKV before norm and RoPE */
+  const void* q_norm_weights;      /* bf16 [L, D]                                 */
+  const void* k_norm_weights;      /* bf16 [L, D]                                 */
+  int32_t norm_topk_prob;          /* 1: opcode 9 divides the top-k probabilities by their sum (fp32, added in slot
+                                      order); 0: raw probabilities, as the reference's decode route leaves them   */
+  int32_t routed_upgate_tile;      /* outputs per tile of opcode 12 (its tile_N_granularity word): 16 (0 = 16), or 8
+                                      where that deals the tiles evenly (Fm = 768: 768 tiles for 256 queues)        */
 } QmkMoeArgs;
 
 int qmk_decode_step_moe(const QmkMoeArgs* args);

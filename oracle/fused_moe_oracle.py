@@ -17,6 +17,14 @@ Restates the reference's fused PyTorch operations
 ``lm_head``                  :141-152
 ===========================  ================================================================
 
+A shape with ``qk_norm`` (Qwen3-30B-A3B) has no route in the reference; its step is the reference's two routes
+put together: the attention half is the Qwen3 route's (``FusedOracle.qkv_rope`` / ``attention_split_merge`` /
+``oproj_residual`` of oracle/fused_oracle.py, restating …/qwen/qwen3__0_6b/A100/single_batch/decode_schedule/
+fused/operations.py:52-215), the MoE half is the block above with the two switches that shape sets:
+``norm_topk_prob`` — the top-k probabilities divided by their sum in fp32, the one line the reference has for it
+(…/qwen1_5_moe_a2_7b/…/fused/operations.py:405, in its prefill block) — and no shared expert (the block's shared
+terms dropped; with all-zero shared weights the reference's block computes the same bits).
+
 Pinning: tests/test_moe_oracle.py — closed forms (a router whose logits are given, experts that
 are multiples of each other), the instruction VM of oracle/pyvm_moe_oracle.py on the same inputs,
 and the fixture written by tests/golden/make_fixtures_moe.py from the imported reference while
@@ -30,7 +38,7 @@ from typing import Any
 import torch
 import torch.nn.functional as F
 
-from fused_oracle import rms_norm, rotate_pairs
+from fused_oracle import FusedOracle, rms_norm, rotate_pairs
 
 Tensor = torch.Tensor
 
@@ -38,9 +46,12 @@ Tensor = torch.Tensor
 class FusedMoeOracle:
     def __init__(self, shape: Any):
         self.shape = shape
+        self._qwen3 = FusedOracle(shape) if getattr(shape, "qk_norm", False) else None   # the Qwen3 route's attention half
 
     def qkv_rope(self, g: Any, layer: int) -> None:
         s = self.shape
+        if self._qwen3 is not None:
+            return self._qwen3.qkv_rope(g, layer)
         nq, nkv, d, pos = s.num_attention_heads, s.num_key_value_heads, s.head_dim, int(g.position_id or 0)
         y = rms_norm(g.hidden_states, g.attn_norm_weights[layer], s.rms_norm_eps)
         bias = None if g.qkv_bias is None else g.qkv_bias[layer]
@@ -56,6 +67,8 @@ class FusedMoeOracle:
     def attention(self, g: Any, layer: int) -> None:
         """torch's scaled-dot-product attention on fp32 copies, grouped heads, no mask (`:90-131`)."""
         s = self.shape
+        if self._qwen3 is not None:
+            return self._qwen3.attention_split_merge(g, layer)
         nq, d, n = s.num_attention_heads, s.head_dim, int(g.position_id or 0) + 1
         q = g.q_post_rope.view(1, nq, 1, d).float()
         k = g.k_cache[layer, 0, :n].permute(1, 0, 2).unsqueeze(0).float()
@@ -64,6 +77,8 @@ class FusedMoeOracle:
         g.attn_out.copy_(out.squeeze(0).squeeze(1).reshape(-1).to(g.attn_out.dtype))
 
     def oproj_residual(self, g: Any, layer: int) -> None:
+        if self._qwen3 is not None:
+            return self._qwen3.oproj_residual(g, layer)
         g.hidden_states += F.linear(g.attn_out.unsqueeze(0), g.o_proj_weights[layer]).squeeze(0).to(g.hidden_states.dtype)
 
     def shared_mlp(self, g: Any, layer: int, normed: Tensor) -> None:
@@ -75,6 +90,8 @@ class FusedMoeOracle:
     def router(self, g: Any, layer: int, normed: Tensor) -> None:
         logits = F.linear(normed.float().unsqueeze(0), g.router_weights[layer].float()).squeeze(0)
         top_p, top_i = torch.topk(F.softmax(logits, dim=-1), self.shape.num_experts_per_tok, dim=-1)
+        if getattr(self.shape, "norm_topk_prob", False):
+            top_p = top_p / top_p.sum(dim=-1, keepdim=True)
         g.expert_indices.copy_(top_i.to(g.expert_indices.dtype))
         g.expert_weights.copy_(top_p.to(g.expert_weights.dtype))
 
@@ -89,12 +106,17 @@ class FusedMoeOracle:
     def moe_block(self, g: Any, layer: int) -> None:
         s = self.shape
         normed = rms_norm(g.hidden_states, g.mlp_norm_weights[layer], s.rms_norm_eps)
-        self.shared_mlp(g, layer, normed)
+        shared = getattr(s, "has_shared_expert", True)
+        if shared:
+            self.shared_mlp(g, layer, normed)
         self.router(g, layer, normed)
         accum = torch.zeros(g.routed_out.shape, dtype=torch.float32)
         for slot in range(s.num_experts_per_tok):
             self.routed_expert(g, layer, slot, normed, accum)
         g.routed_out.copy_(accum.to(g.routed_out.dtype))
+        if not shared:
+            g.hidden_states.add_(g.routed_out)
+            return
         gate_logit = (g.shared_expert_gate_weights[layer].squeeze(0).float() * normed.float()).sum()
         gate_scale = torch.sigmoid(gate_logit).to(g.hidden_states.dtype)
         g.hidden_states.add_(g.routed_out)

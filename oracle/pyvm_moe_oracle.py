@@ -24,6 +24,12 @@ projection is split along K and accumulates bf16 partial sums, and the combine s
 ``rms_lmhead_gemv``              python_vm.py:533-546
 ===============================  =====================
 
+A shape with ``qk_norm`` takes the Qwen3 route's protocol for opcodes 1 and 2 (…/qwen/qwen3__0_6b/A100/
+single_batch/decode_schedule/instructions/python_vm.py:110-141, 214-320): opcode 1 leaves the raw QKV vector, every
+split-KV instruction normalises and rotates the q heads and the K row of its KV head and writes the cache rows.
+``norm_topk_prob`` divides the top-k probabilities by their sum (…/fused/operations.py:405); a shape without a
+shared expert has no opcodes 10/11 and opcode 14 adds the routed experts only.
+
 Pinning: tests/test_moe_oracle.py — against the fused MoE oracle within bf16 tolerance, final
 counter values, and the fixture written by tests/golden/make_fixtures_moe.py from the imported
 reference, which ran the reference's VM on the same instruction list in lock-step with this one.
@@ -36,7 +42,7 @@ from typing import Any, Iterable
 import torch
 import torch.nn.functional as F
 
-from fused_oracle import rms_norm, rotate_pairs
+from fused_oracle import per_head_rms_norm, rms_norm, rotate_pairs
 
 Tensor = torch.Tensor
 TILE = 16
@@ -80,6 +86,12 @@ class MoeInstructionVM:
             seg = "q" if row < k_start else ("k" if row < v_start else "v")
             bias = None if g.qkv_bias is None else g.qkv_bias[layer, row:stop].to(g.qkv_weights.dtype)
             out = F.linear(y, g.qkv_weights[layer, row:stop], bias)
+            if getattr(s, "qk_norm", False):   # the raw vector only; norm, RoPE and the cache write belong to opcode 2
+                g.qkv_raw[row:stop] = out.to(g.qkv_raw.dtype)
+                for blk in range(row // tile, (stop + tile - 1) // tile):
+                    bar[blk // (d // tile)] += 1
+                row = stop
+                continue
             if seg != "v":
                 # RoPE on a head-sized row that is zero outside the chunk: pairs are neighbours
                 head = torch.zeros(1, d, dtype=out.dtype)
@@ -113,6 +125,16 @@ class MoeInstructionVM:
         b0 = ins.partial_idx * per
         t0, t1 = b0 * s.attn_kv_block_size, min(min(b0 + per, total) * s.attn_kv_block_size, seq_len)
         h0, h1 = kvh * ratio, (kvh + 1) * ratio
+        if getattr(s, "qk_norm", False):
+            # every partial computes the same values, so the sequential VM simply writes them each time
+            nq, nkv, pos, raw = s.num_attention_heads, s.num_key_value_heads, int(g.position_id or 0), g.qkv_raw
+            k_off, v_off = nq * d + kvh * d, (nq + nkv) * d + kvh * d
+            cos, sin = g.rope_cos[pos].unsqueeze(0), g.rope_sin[pos].unsqueeze(0)
+            qn = per_head_rms_norm(raw[h0 * d : h1 * d].view(ratio, d), g.q_norm_weights[layer], s.rms_norm_eps)
+            kn = per_head_rms_norm(raw[k_off : k_off + d].view(1, d), g.k_norm_weights[layer], s.rms_norm_eps)
+            g.q_post_rope.view(nq, d)[h0:h1] = ((qn * cos) + (rotate_pairs(qn) * sin)).to(g.q_post_rope.dtype)
+            g.k_cache[layer, 0, pos, kvh] = ((kn * cos) + (rotate_pairs(kn) * sin)).view(-1).to(g.k_cache.dtype)
+            g.v_cache[layer, 0, pos, kvh] = raw[v_off : v_off + d].to(g.v_cache.dtype)
         if t1 <= t0:
             lse = torch.full((ratio,), float("-inf"), dtype=torch.float32)
             out = torch.zeros(ratio, d, dtype=g.attn_out_intermediates.dtype)
@@ -192,6 +214,8 @@ class MoeInstructionVM:
         s, layer = self.shape, ins.layer_idx
         assert int(g.barriers[layer, 7, 0]) == s.num_experts
         top_p, top_i = torch.topk(F.softmax(g.router_logits_buf, dim=-1), s.num_experts_per_tok, dim=-1)
+        if getattr(s, "norm_topk_prob", False):
+            top_p = top_p / top_p.sum(dim=-1, keepdim=True)
         g.expert_indices.copy_(top_i.to(g.expert_indices.dtype))
         g.expert_weights.copy_(top_p.to(g.expert_weights.dtype))
         g.barriers[layer, 8, 0] = 1
@@ -239,7 +263,7 @@ class MoeInstructionVM:
 
     def routed_expert_downproj(self, g: Any, ins: Any) -> None:
         s, layer = self.shape, ins.layer_idx
-        assert int(g.barriers[layer, 11, 0]) == s.num_experts_per_tok * s.num_moe_intermediate_blocks
+        assert int(g.barriers[layer, 11, 0]) == s.num_experts_per_tok * (s.moe_intermediate_size // getattr(s, "routed_upgate_tile", TILE))
         eid = int(g.expert_indices[ins.expert_idx])
         w = g.expert_weights[ins.expert_idx].to(torch.float32)
         mat = g.expert_down_proj_weights[layer, eid].contiguous()
@@ -253,13 +277,17 @@ class MoeInstructionVM:
     # ---- 14 ----------------------------------------------------------------------
     def moe_combine_commit(self, g: Any, ins: Any) -> None:
         s, layer = self.shape, ins.layer_idx
+        has_shared = getattr(s, "has_shared_expert", True)
         for blk in range(ins.tile_N_start_idx, ins.tile_N_end_idx):
-            assert int(g.barriers[layer, 10, blk]) == s.num_downproj_split_k_shared
+            assert int(g.barriers[layer, 10, blk]) == (s.num_downproj_split_k_shared if has_shared else 0)
             assert int(g.barriers[layer, 12, blk]) == s.num_experts_per_tok
-        gate = torch.sigmoid((g.shared_expert_gate_weights[layer].reshape(-1).float() * g.normed_hidden_states.reshape(-1).float()).sum())
         r0, r1 = ins.tile_N_start_idx * ins.tile_N_granularity, ins.tile_N_end_idx * ins.tile_N_granularity
-        hidden, routed, shared = g.hidden_states.reshape(-1), g.routed_out_f32.reshape(-1), g.shared_out.reshape(-1)
-        hidden[r0:r1] = (hidden[r0:r1].float() + routed[r0:r1] + gate * shared[r0:r1].float()).to(hidden.dtype)
+        hidden, routed = g.hidden_states.reshape(-1), g.routed_out_f32.reshape(-1)
+        if has_shared:
+            gate = torch.sigmoid((g.shared_expert_gate_weights[layer].reshape(-1).float() * g.normed_hidden_states.reshape(-1).float()).sum())
+            hidden[r0:r1] = (hidden[r0:r1].float() + routed[r0:r1] + gate * g.shared_out.reshape(-1)[r0:r1].float()).to(hidden.dtype)
+        else:
+            hidden[r0:r1] = (hidden[r0:r1].float() + routed[r0:r1]).to(hidden.dtype)
         routed[r0:r1] = 0.0
         g.barriers[layer, 13, 0] += ins.tile_N_end_idx - ins.tile_N_start_idx
 

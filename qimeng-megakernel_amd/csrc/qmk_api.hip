@@ -19,7 +19,7 @@
 
 // Workspace of qmk_decode_step_static: the tagged units, the greedy candidates and the launch count
 // that qmk_decode_step keeps in the caller's QmkArgs.workspace, here in an array of the library's own
-// (86 144 bytes per device, held until the process ends), so that the entry point allocates nothing.
+// (94 336 bytes per device, held until the process ends), so that the entry point allocates nothing.
 // In host code the name is only a handle for hipGetSymbolAddress: the kernels get the device address
 // that call returned (DeviceInfo::scratch), once per device.
 static __device__ __align__(256) unsigned long long scratch[qmk::kWsUnits];
@@ -367,6 +367,10 @@ int device_info(DeviceInfo** out) {
     int per_cu_moe = 0;
     if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu_moe, decode_megakernel_moe<QwenMoeA2_7B>, kThreads, 0) != hipSuccess)
       return QMK_ERR_NO_DEVICE;
+    int per_cu_moe3 = 0;
+    if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu_moe3, decode_megakernel_moe<Qwen3MoeA3B>, kThreads, 0) != hipSuccess)
+      return QMK_ERR_NO_DEVICE;
+    per_cu_moe = per_cu_moe3 < per_cu_moe ? per_cu_moe3 : per_cu_moe;
     void* sym = nullptr;
     if (hipGetSymbolAddress(&sym, HIP_SYMBOL(g_status)) != hipSuccess) return QMK_ERR_NO_DEVICE;
     if (hipMemset(sym, 0, sizeof(int32_t) * kStatusWords) != hipSuccess) return QMK_ERR_NO_DEVICE;
@@ -593,36 +597,45 @@ extern "C" int qmk_decode_step_batch(const QmkBatchArgs* a) {
 }
 
 extern "C" uint64_t qmk_moe_workspace_bytes(int top_k, int shared_k_slices) {
-  if (top_k < 1 || top_k > moe::kMaxTopK || shared_k_slices < 0 || shared_k_slices > 16) return 0;
+  if (top_k < 1 || top_k > moe::kMaxTopK || shared_k_slices < 0 || shared_k_slices > 16) return 0;   // 0 slices: no shared expert
   const uint64_t shared = static_cast<uint64_t>(shared_k_slices) * QwenMoeA2_7B::H * sizeof(u16);
   // the down projections' terms, the gate scalar's line, then the tagged units of the residual stream and q/k/v
   return ((shared + 127) / 128) * 128 + static_cast<uint64_t>(top_k) * QwenMoeA2_7B::H * sizeof(float) + 128 +
          static_cast<uint64_t>(kWsUnits) * sizeof(uint64_t);
 }
 
-extern "C" int qmk_decode_step_moe(const QmkMoeArgs* a) {
-  using M = QwenMoeA2_7B;
-  if (a == nullptr) return QMK_ERR_NULL_ARG;
-  if (a->struct_size != sizeof(QmkMoeArgs)) return QMK_ERR_ABI;
-  if (a->model != QMK_MODEL_QWEN1_5_MOE_A2_7B) return QMK_ERR_MODEL;
+namespace {
+
+template <class M>
+int decode_step_moe(const QmkMoeArgs* a) {
   const void* required[] = {a->instructions, a->hidden_states, a->normed_hidden_states, a->q_post_rope, a->k_cache, a->v_cache,
                             a->attn_out, a->attn_lse_intermediates, a->attn_out_intermediates, a->silu_out, a->logits,
-                            a->attn_norm_weights, a->qkv_weights, a->qkv_bias, a->rope_cos, a->rope_sin, a->o_proj_weights,
+                            a->attn_norm_weights, a->qkv_weights, a->rope_cos, a->rope_sin, a->o_proj_weights,
                             a->mlp_norm_weights, a->lm_head_norm_weights, a->lm_head_weights, a->router_weights,
-                            a->router_logits_buf, a->expert_indices, a->expert_weights, a->shared_expert_gate_proj_weights,
-                            a->shared_expert_up_proj_weights, a->shared_expert_down_proj_weights, a->shared_expert_silu_out,
-                            a->shared_out, a->shared_expert_gate_weights, a->expert_gate_up_proj_weights,
+                            a->router_logits_buf, a->expert_indices, a->expert_weights, a->expert_gate_up_proj_weights,
                             a->expert_down_proj_weights, a->routed_silu_buffer, a->routed_out_f32, a->barriers, a->workspace};
   for (const void* ptr : required)
     if (ptr == nullptr) return QMK_ERR_NULL_ARG;
+  if (M::QKV_BIAS && a->qkv_bias == nullptr) return QMK_ERR_NULL_ARG;
+  if (M::QK_NORM && (a->qkv_raw == nullptr || a->q_norm_weights == nullptr || a->k_norm_weights == nullptr)) return QMK_ERR_NULL_ARG;
+  const bool shared = a->shared_ffn != 0;   // a model without a shared expert: shared_ffn = shared_k_slices = 0, no opcodes 10/11
+  if (shared && (a->shared_expert_gate_proj_weights == nullptr || a->shared_expert_up_proj_weights == nullptr ||
+                 a->shared_expert_down_proj_weights == nullptr || a->shared_expert_silu_out == nullptr || a->shared_out == nullptr ||
+                 a->shared_expert_gate_weights == nullptr))
+    return QMK_ERR_NULL_ARG;
   if (a->num_queues < 1 || a->num_insts < 0 || a->num_layers < 1 || a->num_layer_barriers < 15 ||
       a->barrier_slots < M::H / 16 || a->barrier_slots < M::NQ + 2 * M::NKV || a->max_seq_len < 1 || a->max_splits < 1 ||
       a->vocab_size < 1 || a->rope_rows < 1)
     return QMK_ERR_SHAPE;
   if (a->num_experts < 1 || a->num_experts > moe::kMaxExperts || a->top_k < 1 || a->top_k > moe::kMaxTopK || a->top_k > a->num_experts ||
-      a->shared_ffn < 16 || a->shared_ffn % 16 || a->moe_ffn < 16 || a->moe_ffn % 16 || a->moe_ffn > moe::kMaxK ||
-      a->shared_k_slices < 1 || a->shared_k_slices > 16)
+      a->moe_ffn < 16 || a->moe_ffn % 16 || a->moe_ffn > moe::kMaxK)
     return QMK_ERR_SHAPE;
+  if (shared ? (a->shared_ffn < 16 || a->shared_ffn % 16 || a->shared_k_slices < 1 || a->shared_k_slices > 16)
+             : (a->shared_ffn != 0 || a->shared_k_slices != 0))
+    return QMK_ERR_SHAPE;
+  const int routed_tile = a->routed_upgate_tile == 0 ? moe::kTile : a->routed_upgate_tile;
+  if ((routed_tile != 8 && routed_tile != 16) || a->moe_ffn % routed_tile) return QMK_ERR_SHAPE;
+  if (a->norm_topk_prob != 0 && a->norm_topk_prob != 1) return QMK_ERR_SHAPE;
   if (a->flags & ~(QMK_FLAG_KEEP_BARRIERS | QMK_FLAG_TAGGED)) return QMK_ERR_SHAPE;
   // tagged units carry the launch count, which the retiring launch advances, and six bits of layer
   if ((a->flags & QMK_FLAG_TAGGED) && ((a->flags & QMK_FLAG_KEEP_BARRIERS) || a->num_layers > 63)) return QMK_ERR_SHAPE;
@@ -649,6 +662,9 @@ extern "C" int qmk_decode_step_moe(const QmkMoeArgs* a) {
   p.attn_norm = static_cast<const u16*>(a->attn_norm_weights);
   p.qkv_w = static_cast<const u16*>(a->qkv_weights);
   p.qkv_bias = static_cast<const u16*>(a->qkv_bias);
+  p.qkv_raw = static_cast<u16*>(a->qkv_raw);
+  p.q_norm = static_cast<const u16*>(a->q_norm_weights);
+  p.k_norm = static_cast<const u16*>(a->k_norm_weights);
   p.rope_cos = a->rope_cos;
   p.rope_sin = a->rope_sin;
   p.o_w = static_cast<const u16*>(a->o_proj_weights);
@@ -699,9 +715,23 @@ extern "C" int qmk_decode_step_moe(const QmkMoeArgs* a) {
   p.shared_ffn = a->shared_ffn;
   p.moe_ffn = a->moe_ffn;
   p.shared_k_slices = a->shared_k_slices;
+  p.norm_topk = a->norm_topk_prob;
+  p.routed_tile = routed_tile;
 
   hipLaunchKernelGGL(decode_megakernel_moe<M>, dim3(a->num_queues), dim3(kThreads), 0, static_cast<hipStream_t>(a->stream), p);
   return hipGetLastError() == hipSuccess ? QMK_OK : QMK_ERR_LAUNCH;
+}
+
+}  // namespace
+
+extern "C" int qmk_decode_step_moe(const QmkMoeArgs* a) {
+  if (a == nullptr) return QMK_ERR_NULL_ARG;
+  if (a->struct_size != sizeof(QmkMoeArgs)) return QMK_ERR_ABI;
+  switch (a->model) {
+    case QMK_MODEL_QWEN1_5_MOE_A2_7B: return decode_step_moe<QwenMoeA2_7B>(a);
+    case QMK_MODEL_QWEN3_30B_A3B: return decode_step_moe<Qwen3MoeA3B>(a);
+    default: return QMK_ERR_MODEL;
+  }
 }
 
 extern "C" uint64_t qmk_workspace_bytes(int model) {

@@ -117,6 +117,8 @@ struct Params {
   int32_t shared_ffn;            // Fs
   int32_t moe_ffn;               // Fm
   int32_t shared_k_slices;
+  int32_t norm_topk;             // 1: the top-k weights are divided by their sum
+  int32_t routed_tile;           // outputs per tile of the routed up/gate instructions (16, or 8)
 };
 
 // ---------------------------------------------------------------- bf16 ----
@@ -272,8 +274,8 @@ __device__ __forceinline__ v4u ld_shared128(const void* p) {
 // waiting time is short, and not waiting for store acknowledgements behind the next GEMV's row
 // requests is worth more than the polling costs.  Offsets below are in units of 8 bytes.
 constexpr int kWsGeneration = 0;            // launch count (first 128-byte line)
-constexpr int kWsQ = 512;                   // q after RoPE: NQ*D/2 units (two bf16 each)
-constexpr int kWsK = kWsQ + 1024;           // appended K row: NKV*D/2 units
+constexpr int kWsQ = 512;                   // q after RoPE: NQ*D/2 units (two bf16 each; room for 32 heads of 128)
+constexpr int kWsK = kWsQ + 2048;           // appended K row: NKV*D/2 units
 constexpr int kWsV = kWsK + 1024;           // appended V row (regions sized for 16 KV heads of 128)
 constexpr int kWsHiddenMid = kWsV + 1024;   // residual stream after the O-proj: H/2 units
 constexpr int kWsHiddenOut = kWsHiddenMid + 1024;  // residual stream after the down projection / the MoE combine step

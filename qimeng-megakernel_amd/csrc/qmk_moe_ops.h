@@ -28,6 +28,7 @@ struct QwenMoeA2_7B {
   static constexpr int NKV = 16;
   static constexpr int GQA = NQ / NKV;
   static constexpr int QKV = (NQ + 2 * NKV) * D;
+  static constexpr int AW = NQ * D;
   static constexpr int KV_BLOCK = 16;
   static constexpr int CARRY_ROWS = 0;
   static constexpr bool CARRY_AFTER_ATTENTION = false;
@@ -35,6 +36,29 @@ struct QwenMoeA2_7B {
   static constexpr bool QKV_BIAS = true;
   static constexpr int REDUCE_HEADS = 4;   // attn_reduction_size of the route (model_config.py:27)
   static constexpr int PREV_ROW = 13;      // a layer is complete when its combine step is
+};
+
+// Qwen3-30B-A3B layer geometry: 32 query heads over 4 KV heads of 128 (the attention output is twice as
+// wide as the residual stream), the Qwen3 op set's attention (opcode 1 leaves the raw QKV vector, the
+// split-KV prologue applies the per-head RMSNorm of q and k and RoPE; no QKV bias) in front of the MoE
+// block.  Expert count, top-k, FFN width, the absence of a shared expert and the renormalisation of the
+// top-k weights are launch parameters.
+struct Qwen3MoeA3B {
+  static constexpr int H = 2048;
+  static constexpr int F = 8192;      // size of the LDS activation vector: >= AW, every FFN width and H
+  static constexpr int D = 128;
+  static constexpr int NQ = 32;
+  static constexpr int NKV = 4;
+  static constexpr int GQA = NQ / NKV;
+  static constexpr int QKV = (NQ + 2 * NKV) * D;
+  static constexpr int AW = NQ * D;
+  static constexpr int KV_BLOCK = 16;
+  static constexpr int CARRY_ROWS = 0;
+  static constexpr bool CARRY_AFTER_ATTENTION = false;
+  static constexpr bool QK_NORM = true;
+  static constexpr bool QKV_BIAS = false;
+  static constexpr int REDUCE_HEADS = GQA;
+  static constexpr int PREV_ROW = 13;
 };
 
 namespace moe {
@@ -144,7 +168,7 @@ __device__ __forceinline__ bool op_router(const Params& p, Smem<M>& s, const Ctx
     for (int i = c.tid * 2; i < M::H; i += kThreads * 2) st_shared32(p.normed_hidden + i, *reinterpret_cast<const uint32_t*>(s.x + i));
     // ... and the shared expert's gate, sigmoid(gate_w . normed) in fp32, which every combine instruction of the
     // layer would otherwise recompute from the same row (python_vm.py:506-510)
-    if (wave == kWaves - 1) {
+    if (wave == kWaves - 1 && p.shared_ffn > 0) {
       const u16* const rows[1] = {p.shared_scale_w + static_cast<size_t>(layer) * M::H};
       float v[1];
       rows_dot<1>(rows, s.x, M::H, lane, v);
@@ -182,6 +206,8 @@ __device__ __forceinline__ bool op_topk(const Params& p, Smem<M>& s, const Ctx& 
       sum += x;
     }
     sum = wave_sum(sum);
+    float* picked = &s.merge[0][0][0];   // the probabilities of the picks, in slot order; their experts behind them
+    bool complete = true;
     for (int j = 0; j < p.top_k; ++j) {
       float best = -1.f;
       int idx = 0x7fffffff;
@@ -197,18 +223,30 @@ __device__ __forceinline__ bool op_topk(const Params& p, Smem<M>& s, const Ctx& 
           s.ctl[0] = 1;
           report_error(p, QMK_DEV_BAD_OPERAND, c.inst_idx, c.opcode, j);
         }
+        complete = false;
         break;   // uniform: every lane holds the same idx
       }
       if (lane == 0) {
-        __hip_atomic_store(p.expert_indices + j, static_cast<long long>(idx), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        st_shared_f32(p.expert_weights + j, best / sum);
-        if (tagged(p)) {   // the routed ops poll these instead of the counter below: one trip, no drain in between
-          st_tagged(p.ws + kWsExperts + j, static_cast<uint32_t>(idx), tag_of(s.generation, layer));
-          st_tagged(p.ws + kWsExperts + kMaxTopK + j, __float_as_uint(best / sum), tag_of(s.generation, layer));
-        }
+        picked[j] = best / sum;
+        picked[kMaxTopK + j] = __int_as_float(idx);
         s.res[idx] = -2.f;   // taken
       }
       __builtin_amdgcn_wave_barrier();
+    }
+    if (complete && lane == 0) {
+      // norm_topk_prob: the picks' probabilities divided by their sum, added up in slot order (fp32)
+      float total = 0.f;
+      for (int j = 0; j < p.top_k; ++j) total += picked[j];
+      for (int j = 0; j < p.top_k; ++j) {
+        const int idx = __float_as_int(picked[kMaxTopK + j]);
+        const float w = p.norm_topk ? picked[j] / total : picked[j];
+        __hip_atomic_store(p.expert_indices + j, static_cast<long long>(idx), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        st_shared_f32(p.expert_weights + j, w);
+        if (tagged(p)) {   // the routed ops poll these instead of the counter below: one trip, no drain in between
+          st_tagged(p.ws + kWsExperts + j, static_cast<uint32_t>(idx), tag_of(s.generation, layer));
+          st_tagged(p.ws + kWsExperts + kMaxTopK + j, __float_as_uint(w), tag_of(s.generation, layer));
+        }
+      }
     }
   }
   release_stores();
@@ -384,7 +422,7 @@ __device__ __forceinline__ bool op_routed_upgate(const Params& p, Smem<M>& s, co
   const int layer = s.inst[1], slot = s.inst[2], n0 = s.inst[3], n1 = s.inst[4], tile = s.inst[6];
   if (layer < 0 || layer >= p.num_layers) return bad_operand(p, s, c, 1);
   if (slot < 0 || slot >= p.top_k) return bad_operand(p, s, c, 2);
-  if (tile != kTile || n0 < 0 || n1 < n0 || n1 * tile > p.moe_ffn || (n1 - n0) * tile > kResSlots) return bad_operand(p, s, c, 4);
+  if (tile != p.routed_tile || n0 < 0 || n1 < n0 || n1 * tile > p.moe_ffn || (n1 - n0) * tile > kResSlots) return bad_operand(p, s, c, 4);
   // The normalised row first (as in opcode 10; a tagged launch has it long before the top-k is known), then the
   // expert: its rows are the only thing left to wait for.
   if (tagged(p) && !residual_to_lds<M>(p, s, c, layer)) return false;
@@ -421,7 +459,7 @@ __device__ __forceinline__ bool op_routed_down(const Params& p, Smem<M>& s, cons
   if (!down_rows(
           s, c, w, p.moe_ffn, p.moe_ffn, n0 * tile, (n1 - n0) * tile,
           [&] {
-            if (!wait_one(p, s, c, layer, ROW_ROUTED_UPGATE, 0, p.top_k * (p.moe_ffn / kTile))) return false;
+            if (!wait_one(p, s, c, layer, ROW_ROUTED_UPGATE, 0, p.top_k * (p.moe_ffn / p.routed_tile))) return false;
             stage_vector(s, c, p.routed_silu + static_cast<size_t>(slot) * p.moe_ffn, p.moe_ffn);
             return true;
           },
@@ -447,6 +485,7 @@ __device__ __forceinline__ bool op_combine(const Params& p, Smem<M>& s, const Ct
   if (c.tid < 2 * nb) {
     const bool routed = c.tid >= nb;
     const int blk = n0 + (routed ? c.tid - nb : c.tid);
+    // (without a shared expert shared_k_slices is 0 and that half of the pollers passes at once)
     if (!poll_counter(counter_ptr(p, layer, routed ? ROW_ROUTED_DOWN : ROW_SHARED_DOWN, blk), routed ? p.top_k : p.shared_k_slices, p.spin_limit)) {
       s.ctl[0] = 1;
       report_error(p, QMK_DEV_WAIT_TIMEOUT, c.inst_idx, c.opcode, c.tid);
@@ -460,7 +499,7 @@ __device__ __forceinline__ bool op_combine(const Params& p, Smem<M>& s, const Ct
   if (s.ctl[0]) return false;
   const bool tg = tagged(p);
   const uint32_t tag = tag_of(s.generation, layer);
-  const float gate = ld_shared_f32(p.shared_gate);   // left by the layer's publishing router instruction
+  const float gate = p.shared_k_slices > 0 ? ld_shared_f32(p.shared_gate) : 0.f;   // left by the layer's publishing router instruction
   constexpr int kMaxSlices = 16;   // the launcher's bound on shared_k_slices
   for (int pair = c.tid; pair < nb * tile / 2; pair += kThreads) {
     const int r = n0 * tile + 2 * pair;
@@ -494,7 +533,7 @@ __device__ __forceinline__ bool op_combine(const Params& p, Smem<M>& s, const Ct
     const uint32_t word = static_cast<uint32_t>(f2bf(h0)) | (static_cast<uint32_t>(f2bf(h1)) << 16);
     st_shared32(p.hidden + r, word);
     if (tg) st_tagged(p.ws + kWsHiddenOut + r / 2, word, tag);   // the next layer's QKV and O-projection, the LM head
-    st_shared32(p.shared_out + r, static_cast<uint32_t>(f2bf(sh0)) | (static_cast<uint32_t>(f2bf(sh1)) << 16));
+    if (p.shared_k_slices > 0) st_shared32(p.shared_out + r, static_cast<uint32_t>(f2bf(sh0)) | (static_cast<uint32_t>(f2bf(sh1)) << 16));
     st_shared_f32(p.routed_out_f32 + r, 0.f);
     st_shared_f32(p.routed_out_f32 + r + 1, 0.f);
   }

@@ -21,6 +21,7 @@ struct Llama1B {
   static constexpr int NKV = 8;     // key/value heads
   static constexpr int GQA = NQ / NKV;
   static constexpr int QKV = (NQ + 2 * NKV) * D;
+  static constexpr int AW = NQ * D;    // width of the attention output = columns of the O-projection
   static constexpr int KV_BLOCK = 16;  // split-KV partition granularity in tokens
   static constexpr int CARRY_ROWS = 2;  // up/gate rows per wave requested by the O-proj before it
   static constexpr bool CARRY_AFTER_ATTENTION = false;  // ... also by a workgroup that has just run attention
@@ -41,6 +42,7 @@ struct Qwen3_1p7B {
   static constexpr int NKV = 8;
   static constexpr int GQA = NQ / NKV;
   static constexpr int QKV = (NQ + 2 * NKV) * D;
+  static constexpr int AW = NQ * D;
   static constexpr int KV_BLOCK = 16;
   static constexpr int CARRY_ROWS = 3;
   static constexpr bool CARRY_AFTER_ATTENTION = true;
@@ -64,7 +66,7 @@ struct Smem {
   float red[kWaves];
   alignas(16) u16 x[M::F];              // activation vector handed to the GEMV lanes
   float res[kResSlots];                 // per-row GEMV results awaiting the epilogue pass
-  float merge[kWaves * 8][M::GQA][M::D + 4];  // attention state per lane group: acc[D], m, l, fold weights
+  float merge[kWaves][M::GQA][M::D + 4];  // attention state per wave and head: acc[D], m, l
   unsigned long long t_wait;            // timeline: when the last counter wait finished
   unsigned long long stamps[4];         // timeline: op-specific intermediate timestamps
 };
@@ -461,6 +463,37 @@ __device__ __forceinline__ void merge_partials(const Params& p, int head0, int n
   }
 }
 
+// One role of the Qwen3 op set's attention prologue, run by one wave on the staged vectors (`words`: q heads
+// from 0, then the new K row, then the new V row; lane l owns the rotation pair (2l, 2l+1)).  Roles 0..GQA-1:
+// a query head; GQA: the K row — per-head RMSNorm, n = bf16(w * (x * rsqrt(mean(x^2) + eps))) in fp32 with one
+// rounding, then RoPE, in place; GQA+1: the V row, which goes to the cache as it is.  The one partial of the KV
+// head whose slice holds this position (`has_new`) also writes the caller's copies.
+template <class M>
+__device__ __forceinline__ void qk_norm_rope_role(const Params& p, uint32_t* words, int role, int lane, int layer, int kvh,
+                                                  bool has_new, size_t new_row) {
+  constexpr int D = M::D, GQA = M::GQA, kQ = 0, kK = GQA * D, kV = GQA * D + D;
+  if (role <= GQA && (role < GQA || has_new)) {
+    const bool is_k = role == GQA;
+    const int at = is_k ? kK / 2 : (kQ + role * D) / 2;
+    const uint32_t raw = words[at + lane];
+    const float x0 = bf_lo(raw), x1 = bf_hi(raw);
+    const float ss = wave_sum(__builtin_fmaf(x1, x1, x0 * x0));
+    const float rstd = 1.0f / sqrtf(ss / static_cast<float>(D) + p.rms_norm_eps);
+    const uint32_t wn = reinterpret_cast<const uint32_t*>((is_k ? p.k_norm : p.q_norm) + static_cast<size_t>(layer) * D)[lane];
+    const float n0 = round_bf16(bf_lo(wn) * (x0 * rstd)), n1 = round_bf16(bf_hi(wn) * (x1 * rstd));
+    const float* cosr = p.rope_cos + static_cast<size_t>(p.pos_id) * D;
+    const float* sinr = p.rope_sin + static_cast<size_t>(p.pos_id) * D;
+    const uint32_t out = rope_pair(n0, n1, cosr, sinr, 2 * lane);
+    words[at + lane] = out;
+    if (has_new) {
+      if (is_k) st_shared32(p.k_cache + new_row + 2 * lane, out);
+      else st_shared32(p.q_post_rope + (kvh * GQA + role) * D + 2 * lane, out);
+    }
+  } else if (role == GQA + 1 && has_new) {
+    st_shared32(p.v_cache + new_row + 2 * lane, words[kV / 2 + lane]);
+  }
+}
+
 // ===================================================================== 2 ==
 // [2, layer, kv_head, num_partials, partial_idx, merge_in_last]
 // Flash-decoding over one contiguous slice of the context for the GQA group of
@@ -482,7 +515,7 @@ __device__ __forceinline__ void merge_partials(const Params& p, int head0, int n
 template <class M>
 __device__ bool op_attn_splitkv(const Params& p, Smem<M>& s, const Ctx& c) {
   constexpr int D = M::D, GQA = M::GQA;
-  static_assert(D % 64 == 0 && GQA <= 4 && GQA * D <= kThreads, "a lane owns whole 16-byte vectors of K; one thread per merged output");
+  static_assert(D % 64 == 0 && GQA <= 8 && GQA * D <= 2 * kThreads, "a lane owns whole 16-byte vectors of K; heads 4g..4g+3 live in lane group g");
   static_assert(!M::QK_NORM || D == 2 * kWaveSize, "the per-head norm gives every lane one rotation pair");
   const int layer = s.inst[1], kvh = s.inst[2], P = s.inst[3], part = s.inst[4];
   const int merge_mode = s.inst[5];  // 0: per-head counters, 1: last arrival merges, 2: the O-proj merges
@@ -606,29 +639,37 @@ __device__ bool op_attn_splitkv(const Params& p, Smem<M>& s, const Ctx& c) {
   if (s.ctl[0]) return false;
 
   if constexpr (M::QK_NORM) {
-    // Waves 0..GQA-1: the query heads; wave GQA: the new K row; wave GQA+1: the new V row goes
-    // to the cache as it is.  Lane l owns the rotation pair (2l, 2l+1).
+    // One wave per vector: roles 0..GQA-1 are the query heads, role GQA the new K row; the new V row
+    // (role GQA+1) goes to the cache as it is.  Lane l owns the rotation pair (2l, 2l+1).
     //   n = bf16(w * (x * rsqrt(mean(x^2) + eps)))   — fp32 throughout, one rounding
     uint32_t* words = reinterpret_cast<uint32_t*>(stage16);
-    if (wave <= GQA && (wave < GQA || has_new)) {
-      const bool is_k = wave == GQA;
-      const int at = is_k ? kK / 2 : (kQ + wave * D) / 2;
-      const uint32_t raw = words[at + lane];
-      const float x0 = bf_lo(raw), x1 = bf_hi(raw);
-      const float ss = wave_sum(__builtin_fmaf(x1, x1, x0 * x0));
-      const float rstd = 1.0f / sqrtf(ss / static_cast<float>(D) + p.rms_norm_eps);
-      const uint32_t wn = reinterpret_cast<const uint32_t*>((is_k ? p.k_norm : p.q_norm) + static_cast<size_t>(layer) * D)[lane];
-      const float n0 = round_bf16(bf_lo(wn) * (x0 * rstd)), n1 = round_bf16(bf_hi(wn) * (x1 * rstd));
-      const float* cosr = p.rope_cos + static_cast<size_t>(p.pos_id) * D;
-      const float* sinr = p.rope_sin + static_cast<size_t>(p.pos_id) * D;
-      const uint32_t out = rope_pair(n0, n1, cosr, sinr, 2 * lane);
-      words[at + lane] = out;
-      if (has_new) {  // exactly one partial of this KV head holds the position: it owns the caller's copies
-        if (is_k) st_shared32(p.k_cache + new_row + 2 * lane, out);
-        else st_shared32(p.q_post_rope + (kvh * GQA + wave) * D + 2 * lane, out);
+    // A pass gives every wave one role; two passes cover the ten roles of a group of eight heads.
+    if constexpr (GQA + 2 <= kWaves) {
+      // (the helper's body, in place: called as a function — even a forced-inline one — this compiler allocates
+      // the registers of the whole op differently and the dense Qwen3 kernel loses 1.3 %)
+      if (wave <= GQA && (wave < GQA || has_new)) {
+        const bool is_k = wave == GQA;
+        const int at = is_k ? kK / 2 : (kQ + wave * D) / 2;
+        const uint32_t raw = words[at + lane];
+        const float x0 = bf_lo(raw), x1 = bf_hi(raw);
+        const float ss = wave_sum(__builtin_fmaf(x1, x1, x0 * x0));
+        const float rstd = 1.0f / sqrtf(ss / static_cast<float>(D) + p.rms_norm_eps);
+        const uint32_t wn = reinterpret_cast<const uint32_t*>((is_k ? p.k_norm : p.q_norm) + static_cast<size_t>(layer) * D)[lane];
+        const float n0 = round_bf16(bf_lo(wn) * (x0 * rstd)), n1 = round_bf16(bf_hi(wn) * (x1 * rstd));
+        const float* cosr = p.rope_cos + static_cast<size_t>(p.pos_id) * D;
+        const float* sinr = p.rope_sin + static_cast<size_t>(p.pos_id) * D;
+        const uint32_t out = rope_pair(n0, n1, cosr, sinr, 2 * lane);
+        words[at + lane] = out;
+        if (has_new) {  // exactly one partial of this KV head holds the position: it owns the caller's copies
+          if (is_k) st_shared32(p.k_cache + new_row + 2 * lane, out);
+          else st_shared32(p.q_post_rope + (kvh * GQA + wave) * D + 2 * lane, out);
+        }
+      } else if (wave == GQA + 1 && has_new) {
+        st_shared32(p.v_cache + new_row + 2 * lane, words[kV / 2 + lane]);
       }
-    } else if (wave == GQA + 1 && has_new) {
-      st_shared32(p.v_cache + new_row + 2 * lane, words[kV / 2 + lane]);
+    } else {
+      qk_norm_rope_role<M>(p, words, wave, lane, layer, kvh, has_new, new_row);
+      qk_norm_rope_role<M>(p, words, wave + kWaves, lane, layer, kvh, has_new, new_row);
     }
     __syncthreads();
   }
@@ -649,7 +690,7 @@ __device__ bool op_attn_splitkv(const Params& p, Smem<M>& s, const Ctx& c) {
   QMK_STAMP(0);  // q (and the appended row) have arrived
 
   // State of this wave: m (all four lanes of a column agree), this lane's share of l, and
-  // O[head i][dim c16*NT + tile] in acc[tile][i] of lanes 0..15.
+  // O[head 4*g4 + i][dim c16*NT + tile] in acc[tile][i] (lane groups beyond the GQA heads hold nothing).
   float m_run = -INFINITY, l_run = 0.f;
   f4 acc[NT];
 #pragma unroll
@@ -705,12 +746,17 @@ __device__ bool op_attn_splitkv(const Params& p, Smem<M>& s, const Ctx& c) {
     }
     const bf4 p_hi = __builtin_bit_cast(bf4, u2{hi[0] | (hi[1] << 16), hi[2] | (hi[3] << 16)});
     const bf4 p_lo = __builtin_bit_cast(bf4, u2{lo[0] | (lo[1] << 16), lo[2] | (lo[3] << 16)});
-    // The accumulators of head i are scaled by that head's alpha (it lives in lane i).
+    // The accumulators of head h are scaled by that head's alpha (it lives in lane h); this lane
+    // holds the heads 4*g4 .. 4*g4 + 3.
     float a_head[4];
     bool rescale = false;
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
       a_head[i] = i < GQA ? __int_as_float(__builtin_amdgcn_readlane(__float_as_int(alpha), i)) : 1.f;
+      if constexpr (GQA > 4) {
+        const float upper = 4 + i < GQA ? __int_as_float(__builtin_amdgcn_readlane(__float_as_int(alpha), 4 + i)) : 1.f;
+        a_head[i] = g4 == 1 ? upper : a_head[i];
+      }
       rescale = rescale || a_head[i] != 1.f;
     }
     if (rescale) {
@@ -743,19 +789,32 @@ __device__ bool op_attn_splitkv(const Params& p, Smem<M>& s, const Ctx& c) {
   // Every wave parks its state in LDS; GQA*D threads then merge the eight states, one output each.
   l_run += __shfl_xor(l_run, 16);
   l_run += __shfl_xor(l_run, 32);
-  if (lane < 16) {
+  if constexpr (GQA <= 4) {
+    if (lane < 16) {
+#pragma unroll
+      for (int tau = 0; tau < NT; ++tau)
+#pragma unroll
+        for (int i = 0; i < GQA; ++i) s.merge[wave][i][c16 * NT + tau] = acc[tau][i];
+      if (c16 < GQA) {
+        s.merge[wave][c16][D] = m_run;
+        s.merge[wave][c16][D + 1] = l_run;
+      }
+    }
+  } else if (lane < 32) {   // two lane groups hold the rows of heads 0..3 and 4..7
 #pragma unroll
     for (int tau = 0; tau < NT; ++tau)
 #pragma unroll
-      for (int i = 0; i < GQA; ++i) s.merge[wave][i][c16 * NT + tau] = acc[tau][i];
-    if (c16 < GQA) {
+      for (int i = 0; i < 4; ++i)
+        if (4 * g4 + i < GQA) s.merge[wave][4 * g4 + i][c16 * NT + tau] = acc[tau][i];
+    if (g4 == 0 && c16 < GQA) {
       s.merge[wave][c16][D] = m_run;
       s.merge[wave][c16][D + 1] = l_run;
     }
   }
   __syncthreads();
-  if (c.tid < GQA * D) {
-    const int h = c.tid / D, d = c.tid % D;
+  auto merge_output = [&](int o) {   // output o = (head, dim) of the partial: the eight wave states folded
+    if (o >= GQA * D) return;
+    const int h = o / D, d = o % D;
     float mx = -INFINITY;
 #pragma unroll
     for (int w = 0; w < kWaves; ++w) mx = fmaxf(mx, s.merge[w][h][D]);
@@ -772,6 +831,12 @@ __device__ bool op_attn_splitkv(const Params& p, Smem<M>& s, const Ctx& c) {
     // Normalised partial output and log2-sum-exp; an empty slice contributes (0, -inf).
     st_shared_f32(p.attn_partial + (static_cast<size_t>(head) * p.max_splits + part) * D + d, empty ? 0.f : num / den);
     if (d == 0) st_shared_f32(p.attn_lse + static_cast<size_t>(head) * p.max_splits + part, empty ? -INFINITY : mx + log2f(den));
+  };
+  if constexpr (GQA * D <= kThreads) {
+    if (c.tid < GQA * D) merge_output(c.tid);
+  } else {
+    merge_output(c.tid);
+    merge_output(c.tid + kThreads);
   }
 
   QMK_STAMP(2);  // partial merged and stored
@@ -854,8 +919,9 @@ __device__ __forceinline__ void residual_pair(u16* hidden_pair, float d0, float 
 // hidden[r] = bf16(hidden[r] + bf16(W_o[r] . attn_out))   (operations.py:251-262, 63-68)
 template <class M>
 __device__ bool op_oproj_residual(const Params& p, Smem<M>& s, const Ctx& c, Carried& carry, bool& carried) {
-  constexpr int CH = M::H / 512;
-  static_assert(M::NQ * M::D == M::H, "attention output width equals the hidden size");
+  constexpr int AW = M::AW;          // columns of W_o: all query heads side by side (= H for the dense models)
+  constexpr int CH = AW / 512;
+  static_assert(AW % (kThreads * 4) == 0 && AW <= M::F, "whole 8-byte pieces per thread; the vector fits the LDS buffer");
   const int layer = s.inst[1], nstart = s.inst[3], nend = s.inst[4], tile = s.inst[7];
   if (layer < 0 || layer >= p.num_layers) return bad_operand(p, s, c, 1);
   if (tile <= 0 || (tile & 1)) return bad_operand(p, s, c, 7);
@@ -864,12 +930,11 @@ __device__ bool op_oproj_residual(const Params& p, Smem<M>& s, const Ctx& c, Car
 
   const int lane = c.tid & 63;
   const int rs = nstart * tile, nrows = (nend - nstart) * tile;
-  const u16* W = p.o_w + (static_cast<size_t>(layer) * M::H + rs) * M::H;
-  auto src = [&](int r) { return W + static_cast<size_t>(r) * M::H; };
+  const u16* W = p.o_w + (static_cast<size_t>(layer) * M::H + rs) * AW;
+  auto src = [&](int r) { return W + static_cast<size_t>(r) * AW; };
 
   RowRegs<CH> buf[kOprojBuffers];
   preload<CH>(nrows, src, buf);
-  static_assert(M::H == kThreads * 4, "one thread stages four elements");
   // Tagged mode: the rows' residual values are those the previous layer's down projection
   // announced (layer 0: the caller's buffer); they are fetched now, long before they are needed.
   const bool tg = tagged(p);
@@ -900,50 +965,56 @@ __device__ bool op_oproj_residual(const Params& p, Smem<M>& s, const Ctx& c, Car
   const int self_merge = s.inst[5];  // reduction_block_idx: 0, or the split-KV fan-out P when this op merges
   if (self_merge == 0) {
     if (!wg_wait(p, s, c, 1, [&](int) { return counter_ptr(p, layer, ROW_REDUCE, 0); }, M::NQ)) return false;
-    *reinterpret_cast<uint64_t*>(s.x + c.tid * 4) = ld_shared64(p.attn_out + c.tid * 4);
+#pragma unroll
+    for (int k = 0; k < AW / (kThreads * 4); ++k)
+      *reinterpret_cast<uint64_t*>(s.x + (c.tid + k * kThreads) * 4) = ld_shared64(p.attn_out + (c.tid + k * kThreads) * 4);
   } else {
     // Every O-proj workgroup merges the split-KV partials itself (python_vm.py:439-488 for all heads):
-    // no merging workgroup, no attn_out round trip, one synchronisation hop less.  Thread t owns
-    // dims 4*(t%16).. of head t/16.
+    // no merging workgroup, no attn_out round trip, one synchronisation hop less.  Item t (one or two
+    // per thread) is dims 4*(t % (D/4)).. of head t / (D/4).
     const int P = self_merge;
     if (P < 1 || P > kMaxSelfMerge || P > p.max_splits) return bad_operand(p, s, c, 5);  // no list to fit: any fan-out the workspaces hold
     if (!wg_wait_all(p, s, c, layer, ROW_REDUCE, 0, M::NKV * P)) return false;
-    const int h = c.tid / (M::D / 4), d0 = 4 * (c.tid % (M::D / 4));
-    const float* lse = p.attn_lse + static_cast<size_t>(h) * p.max_splits;
-    const float* part = p.attn_partial + static_cast<size_t>(h) * p.max_splits * M::D + d0;
-    float mx = -INFINITY, den = 0.f, n0 = 0.f, n1 = 0.f, n2 = 0.f, n3 = 0.f;
-    for (int j0 = 0; j0 < P; j0 += 4) {   // four partials per round, loads first
-      float e[4];
-      v4u o[4];
 #pragma unroll
-      for (int k = 0; k < 4; ++k) {
-        const int j = min(j0 + k, P - 1);
-        e[k] = (j0 + k < P) ? ld_shared_f32(lse + j) : -INFINITY;
-        o[k] = ld_shared128(part + static_cast<size_t>(j) * M::D);
+    for (int k = 0; k < AW / (kThreads * 4); ++k) {
+      const int item = c.tid + k * kThreads;
+      const int h = item / (M::D / 4), d0 = 4 * (item % (M::D / 4));
+      const float* lse = p.attn_lse + static_cast<size_t>(h) * p.max_splits;
+      const float* part = p.attn_partial + static_cast<size_t>(h) * p.max_splits * M::D + d0;
+      float mx = -INFINITY, den = 0.f, n0 = 0.f, n1 = 0.f, n2 = 0.f, n3 = 0.f;
+      for (int j0 = 0; j0 < P; j0 += 4) {   // four partials per round, loads first
+        float e[4];
+        v4u o[4];
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+          const int j = min(j0 + q, P - 1);
+          e[q] = (j0 + q < P) ? ld_shared_f32(lse + j) : -INFINITY;
+          o[q] = ld_shared128(part + static_cast<size_t>(j) * M::D);
+        }
+        float mn = mx;
+#pragma unroll
+        for (int q = 0; q < 4; ++q) mn = fmaxf(mn, e[q]);
+        const float rescale = (mx == -INFINITY) ? 0.f : exp2_fast(mx - mn);
+        den *= rescale; n0 *= rescale; n1 *= rescale; n2 *= rescale; n3 *= rescale;
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+          const float f = (e[q] == -INFINITY) ? 0.f : exp2_fast(e[q] - mn);
+          den += f;
+          n0 = __builtin_fmaf(__uint_as_float(o[q].x), f, n0);
+          n1 = __builtin_fmaf(__uint_as_float(o[q].y), f, n1);
+          n2 = __builtin_fmaf(__uint_as_float(o[q].z), f, n2);
+          n3 = __builtin_fmaf(__uint_as_float(o[q].w), f, n3);
+        }
+        mx = mn;
       }
-      float mn = mx;
-#pragma unroll
-      for (int k = 0; k < 4; ++k) mn = fmaxf(mn, e[k]);
-      const float rescale = (mx == -INFINITY) ? 0.f : exp2_fast(mx - mn);
-      den *= rescale; n0 *= rescale; n1 *= rescale; n2 *= rescale; n3 *= rescale;
-#pragma unroll
-      for (int k = 0; k < 4; ++k) {
-        const float f = (e[k] == -INFINITY) ? 0.f : exp2_fast(e[k] - mn);
-        den += f;
-        n0 = __builtin_fmaf(__uint_as_float(o[k].x), f, n0);
-        n1 = __builtin_fmaf(__uint_as_float(o[k].y), f, n1);
-        n2 = __builtin_fmaf(__uint_as_float(o[k].z), f, n2);
-        n3 = __builtin_fmaf(__uint_as_float(o[k].w), f, n3);
+      const float inv = den > 0.f ? 1.0f / den : 0.f;
+      const uint32_t lo = static_cast<uint32_t>(f2bf(n0 * inv)) | (static_cast<uint32_t>(f2bf(n1 * inv)) << 16);
+      const uint32_t hi = static_cast<uint32_t>(f2bf(n2 * inv)) | (static_cast<uint32_t>(f2bf(n3 * inv)) << 16);
+      *reinterpret_cast<uint2*>(s.x + item * 4) = make_uint2(lo, hi);
+      if (nstart == 0) {  // one workgroup also leaves attn_out in memory, as the reference does
+        st_shared32(p.attn_out + item * 4, lo);
+        st_shared32(p.attn_out + item * 4 + 2, hi);
       }
-      mx = mn;
-    }
-    const float inv = den > 0.f ? 1.0f / den : 0.f;
-    const uint32_t lo = static_cast<uint32_t>(f2bf(n0 * inv)) | (static_cast<uint32_t>(f2bf(n1 * inv)) << 16);
-    const uint32_t hi = static_cast<uint32_t>(f2bf(n2 * inv)) | (static_cast<uint32_t>(f2bf(n3 * inv)) << 16);
-    *reinterpret_cast<uint2*>(s.x + c.tid * 4) = make_uint2(lo, hi);
-    if (nstart == 0) {  // one workgroup also leaves attn_out in memory, as the reference does
-      st_shared32(p.attn_out + c.tid * 4, lo);
-      st_shared32(p.attn_out + c.tid * 4 + 2, hi);
     }
   }
   __syncthreads();

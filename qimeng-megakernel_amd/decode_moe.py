@@ -18,8 +18,11 @@ from .decode_schedule_moe.model_config import QwenMoeConfig
 
 
 def decode(globs: Any, prompt_ids: torch.Tensor, max_new_tokens: int, *, mk: Any = None, decode_time: bool = True,
-           use_graph: bool = False) -> dict[str, Any]:
+           use_graph: bool = False, timed_steps: int | None = None) -> dict[str, Any]:
     """Prefill + forced greedy decode to exactly ``max_new_tokens`` tokens (no EOS stop).
+
+    ``timed_steps``: only the last that many decode steps are timed (and captured); the steps before them run
+    untimed and the device is synchronised in between.  Default: all of them.
 
     ``use_graph``: the loop (embedding row, kernel, argmax, token write per step) is captured into one HIP graph
     and replayed; the positions are launch arguments, so the graph belongs to this request.  The result then
@@ -38,7 +41,15 @@ def decode(globs: Any, prompt_ids: torch.Tensor, max_new_tokens: int, *, mk: Any
         globs.position_id = pos
         _mk_kernel.call_mk(globs, mk)
     out[T] = globs.logits.argmax()
-    ntok = max(max_new_tokens - 1, 0)
+    total = max(max_new_tokens - 1, 0)
+    ntok = total if timed_steps is None else max(0, min(int(timed_steps), total))
+    T0 = T
+    for i in range(total - ntok):   # the untimed head of the request
+        globs.hidden_states.copy_(globs.embed_tokens.index_select(0, out[T + i : T + i + 1]).view(-1))
+        globs.position_id = T + i
+        _mk_kernel.call_mk(globs, mk)
+        out[T + i + 1] = globs.logits.argmax()
+    T += total - ntok
     timed = decode_time and not use_graph
     events = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(ntok if timed else 0)]
     loop_start, loop_end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
@@ -71,13 +82,13 @@ def decode(globs: Any, prompt_ids: torch.Tensor, max_new_tokens: int, *, mk: Any
         steps()
     loop_end.record()
     torch.cuda.synchronize(device)
-    result: dict[str, Any] = {"generated_ids": out, "new_tokens": out[T:]}
+    result: dict[str, Any] = {"generated_ids": out, "new_tokens": out[T0:]}
     if graph is not None:
         def replay() -> torch.Tensor:
             """The same request once more through the captured loop (the KV rows it wrote are written again)."""
             out[T] = first_token
             graph.replay()
-            return out[T:]
+            return out[T0:]
 
         result["replay"] = replay
     if decode_time and ntok:
@@ -91,6 +102,7 @@ def decode(globs: Any, prompt_ids: torch.Tensor, max_new_tokens: int, *, mk: Any
             "decode_wall_s": wall, "decode_gpu_s": gpu_s, "mk_kernel_gpu_s": kernel_s,
             "effective_tok_s_wall": ntok / wall, "effective_tok_s_gpu": ntok / gpu_s, "kernel_tok_s": ntok / kernel_s,
             "kernel_steps": ntok, "kernel_ms_per_step": kernel_s * 1e3 / ntok, "algorithmic_bytes": nbytes,
+            "first_timed_context": T + 1, "last_timed_context": T + ntok,
             "achieved_GBps": nbytes / kernel_s / 1e9, "per_step_ms": per_step_ms,
         }
     mk.check()

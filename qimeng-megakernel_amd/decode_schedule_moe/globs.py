@@ -7,7 +7,9 @@ Shapes (Qwen1.5-MoE-A2.7B): ``qkv_weights [L, 6144, 2048]`` + ``qkv_bias [L, 614
 ``shared_expert_gate_weights [L, 1, H]``; buffers ``router_logits_buf [E]`` f32,
 ``expert_indices [k]`` int64, ``expert_weights [k]`` f32, ``normed_hidden_states [H]``,
 ``shared_expert_silu_out [5632]``, ``shared_out [H]``, ``routed_silu_buffer [k, 1408]``,
-``routed_out_f32 [H]`` f32, ``barriers [L, 15, 128]``.
+``routed_out_f32 [H]`` f32, ``barriers [L, 15, 128]``.  A shape without a shared expert (Qwen3-30B-A3B) leaves the
+six shared-expert fields ``None``; a shape with the Qwen3 op set's attention adds ``qkv_raw`` and the two per-head
+norm weights, as the dense Qwen3 route does (`…/qwen/qwen3__0_6b/A100/single_batch/decode_schedule/globs.py`).
 """
 from __future__ import annotations
 
@@ -27,6 +29,9 @@ class Globals:
     attn_norm_weights: Optional[Tensor] = None
     qkv_weights: Optional[Tensor] = None
     qkv_bias: Optional[Tensor] = None
+    qkv_raw: Optional[Tensor] = None                 # Qwen3 op set: bf16 [(Hq+2Hkv)*D], QKV before norm and RoPE
+    q_norm_weights: Optional[Tensor] = None          # Qwen3 op set: bf16 [L, D]
+    k_norm_weights: Optional[Tensor] = None
     rope_cos: Optional[Tensor] = None
     rope_sin: Optional[Tensor] = None
     o_proj_weights: Optional[Tensor] = None

@@ -90,6 +90,8 @@ class MoeScheduler:
         return [Router_SoftmaxTopK(layer)]
 
     def shared_upgate(self, layer: int) -> list[Instruction]:
+        if not self.shape.has_shared_expert:
+            return []
         if self.placed:
             return [ins for _, ins in self._placed_shared_upgate(layer)]
         tiles = _ceil_div(self.shape.intermediate_size, TILE_N_GRANULARITY)
@@ -98,6 +100,8 @@ class MoeScheduler:
     def shared_downproj(self, layer: int) -> list[Instruction]:
         """K split into ``num_downproj_split_k_shared`` slices, each with its own share of the queues."""
         k = self.shape.num_downproj_split_k_shared
+        if not self.shape.has_shared_expert or k < 1:
+            return []
         per_group = max(1, self.sm_count // k)
         out: list[Instruction] = []
         for slice_idx in range(k):
@@ -111,9 +115,10 @@ class MoeScheduler:
         if self.placed:
             return [ins for _, ins in self._placed_routed_upgate(layer)]
         per_expert = max(1, self.sm_count // self.shape.num_experts_per_tok)
-        return [RoutedExpert_UpGate_SiLU(layer, slot, lo, hi)
+        tile = self.shape.routed_upgate_tile
+        return [RoutedExpert_UpGate_SiLU(layer, slot, lo, hi, tile_N_granularity=tile)
                 for slot in range(self.shape.num_experts_per_tok)
-                for lo, hi in _spans(self.shape.num_moe_intermediate_blocks, per_expert)]
+                for lo, hi in _spans(self.shape.num_routed_upgate_blocks, per_expert)]
 
     def routed_downproj(self, layer: int) -> list[Instruction]:
         per_expert = max(1, self.sm_count // self.shape.num_experts_per_tok)
@@ -167,6 +172,8 @@ class MoeScheduler:
 
     def _shared_sizes(self) -> dict[int, int]:
         main, _, oproj_queues = self._roles()
+        if not self.shape.has_shared_expert:
+            return {q: 0 for q in main}
         tiles = _ceil_div(self.shape.intermediate_size, TILE_N_GRANULARITY)
         weights = [1 if i < oproj_queues else 2 for i in range(len(main))]
         return dict(zip(main, self._weighted_sizes(tiles, weights)))
@@ -181,15 +188,19 @@ class MoeScheduler:
 
     def _placed_routed_upgate(self, layer: int) -> list[tuple[int, Instruction]]:
         shared = self._shared_sizes()
-        blocks, slots = self.shape.num_moe_intermediate_blocks, self.shape.num_experts_per_tok
-        most = max(shared.values()) + 1
+        blocks, slots, tile = self.shape.num_routed_upgate_blocks, self.shape.num_experts_per_tok, self.shape.routed_upgate_tile
         queues = list(range(self.sm_count))
-        sizes = self._weighted_sizes(blocks * slots, [most - shared.get(q, most - 2) for q in queues])
+        if self.shape.has_shared_expert:
+            most = max(shared.values()) + 1
+            weights = [most - shared.get(q, most - 2) for q in queues]
+        else:                                    # nothing else in the phase: the tiles evenly on all queues
+            weights = [1] * len(queues)
+        sizes = self._weighted_sizes(blocks * slots, weights)
         out, slot, lo = [], 0, 0
         for queue, size in zip(queues, sizes):
             while size:                          # a span ends with its expert slot: the rest goes to the next slot
                 take = min(size, blocks - lo)
-                out.append((queue, RoutedExpert_UpGate_SiLU(layer, slot, lo, lo + take)))
+                out.append((queue, RoutedExpert_UpGate_SiLU(layer, slot, lo, lo + take, tile_N_granularity=tile)))
                 size, lo = size - take, lo + take
                 if lo == blocks:
                     slot, lo = slot + 1, 0

@@ -1,4 +1,4 @@
-"""Load and call the gfx950 MoE decode kernel through its C ABI.
+"""Load and call the gfx950 MoE decode kernels through their C ABI.
 
 Host-side counterpart of the reference's launcher of the MoE route
 (`…/qwen/qwen1_5_moe_a2_7b/A100/single_batch/decode_schedule/mk_kernel.py:63-205`): ``get_mk`` returns
@@ -7,6 +7,11 @@ positional order (its three unused dense-MLP positions included), ``run_instruct
 arbitrary instruction list.  The callable wraps ``qmk_decode_step_moe`` of ``libqmk_hip.so``
 (``include/qmk.h``) with ctypes.  There is no fallback: a missing library is an ``ImportError``, a
 non-GPU tensor a ``ValueError`` and a device-side error a ``RuntimeError``.
+
+Two layer geometries are compiled: Qwen1.5-MoE-A2.7B (the reference's route) and Qwen3-30B-A3B, for which the
+reference has no route: its ``mk`` here takes the same positional list with ``None`` in the places of the
+tensors the model does not have (QKV bias, the six shared-expert tensors) and the three tensors of the Qwen3
+op set (``qkv_raw``, ``q_norm_weights``, ``k_norm_weights``) appended behind ``barriers``.
 """
 from __future__ import annotations
 
@@ -27,7 +32,13 @@ from .model_config import QwenMoeConfig
 _P = ctypes.c_void_p
 _I = ctypes.c_int32
 QMK_MODEL_QWEN1_5_MOE_A2_7B = 2
+QMK_MODEL_QWEN3_30B_A3B = 3
 MI355X_QUEUES = 256
+# (hidden, head_dim, query heads, KV heads, QK norm) -> compiled kernel
+_MODELS = {(2048, 128, 16, 16, False): QMK_MODEL_QWEN1_5_MOE_A2_7B, (2048, 128, 32, 4, True): QMK_MODEL_QWEN3_30B_A3B}
+_QWEN3_EXTRA = ("qkv_raw", "q_norm_weights", "k_norm_weights")
+_SHARED = ("shared_expert_gate_proj_weights", "shared_expert_up_proj_weights", "shared_expert_down_proj_weights",
+           "shared_expert_silu_out", "shared_out", "shared_expert_gate_weights")
 
 # The positional order of mk(...): name in QmkMoeArgs, or None for the three unused dense-MLP positions.
 _TENSOR_ORDER = (
@@ -55,6 +66,7 @@ class QmkMoeArgs(ctypes.Structure):
                                    "shared_k_slices")]
         + [("attn_scale", ctypes.c_float), ("rms_norm_eps", ctypes.c_float), ("timeline", _P), ("stream", _P), ("workspace", _P),
            ("workspace_bytes", ctypes.c_uint64)]
+        + [(name, _P) for name in _QWEN3_EXTRA] + [("norm_topk_prob", _I), ("routed_upgate_tile", _I)]
     )
 
 
@@ -75,7 +87,7 @@ class MoeMegaKernel:
         self._barriers: torch.Tensor | None = None   # the counters of the bound launch: cleared by check() after an error
         self._args = QmkMoeArgs()
         self._args.struct_size = ctypes.sizeof(QmkMoeArgs)
-        self._args.model = QMK_MODEL_QWEN1_5_MOE_A2_7B
+        self._args.model = QMK_MODEL_QWEN1_5_MOE_A2_7B   # rebound per call from the shape
         self._bound_key: tuple | None = None
         self._tagged = False
 
@@ -105,12 +117,24 @@ class MoeMegaKernel:
             raise TypeError(f"unknown options {sorted(kw)}")
         return other
 
-    def _bind(self, tensors: dict[str, torch.Tensor]) -> None:
+    def _bind(self, tensors: dict[str, torch.Tensor | None]) -> None:
         a, s = self._args, QwenMoeConfig.shape()
-        if (s.hidden_size, s.head_dim, s.num_attention_heads, s.num_key_value_heads) != (2048, 128, 16, 16):
-            raise ValueError("the MoE kernel is compiled for the Qwen1.5-MoE attention geometry (H 2048, 16/16 heads of 128)")
+        key = (s.hidden_size, s.head_dim, s.num_attention_heads, s.num_key_value_heads, bool(s.qk_norm))
+        if key not in _MODELS:
+            raise ValueError(f"no MoE kernel was compiled for the attention geometry {key} (hidden, head_dim, query heads, KV heads, QK norm)")
+        a.model = _MODELS[key]
+        absent = set() if s.has_shared_expert else set(_SHARED)
+        if not s.qkv_bias:
+            absent.add("qkv_bias")
+        if not s.qk_norm:
+            absent.update(_QWEN3_EXTRA)
         device = tensors["hidden_states"].device
         for name, t in tensors.items():
+            if name in absent:
+                if t is not None:
+                    raise ValueError(f"{name} must be None for this model")
+                setattr(a, name, None)
+                continue
             if not isinstance(t, torch.Tensor):
                 raise TypeError(f"{name} must be a torch.Tensor, got {type(t).__name__}")
             if t.device.type != "cuda" or t.device != device:
@@ -122,8 +146,11 @@ class MoeMegaKernel:
                 raise ValueError(f"{name} must be contiguous")
             setattr(a, name, t.data_ptr())
         L, H = int(tensors["barriers"].shape[0]), s.hidden_size
+        nq, nkv, d = s.num_attention_heads, s.num_key_value_heads, s.head_dim
+        AW, QKV = nq * d, (nq + 2 * nkv) * d
         E, k = int(tensors["router_weights"].shape[1]), int(tensors["expert_indices"].numel())
-        Fs, Fm = int(tensors["shared_expert_gate_proj_weights"].shape[1]), int(tensors["routed_silu_buffer"].shape[-1])
+        Fs = int(tensors["shared_expert_gate_proj_weights"].shape[1]) if s.has_shared_expert else 0
+        Fm = int(tensors["routed_silu_buffer"].shape[-1])
         V = int(tensors["logits"].numel())
 
         def numel(name: str, want: int) -> None:
@@ -134,18 +161,25 @@ class MoeMegaKernel:
             raise ValueError("instructions must be [queues, length, 32]")
         S = int(tensors["k_cache"].shape[2])
         P = int(tensors["attn_lse_intermediates"].shape[-1])
-        for name, want in (("hidden_states", H), ("normed_hidden_states", H), ("q_post_rope", H), ("attn_out", H), ("silu_out", Fm),
-                           ("k_cache", L * S * H), ("v_cache", L * S * H), ("attn_lse_intermediates", 16 * P),
-                           ("attn_out_intermediates", 16 * P * 128), ("attn_norm_weights", L * H), ("mlp_norm_weights", L * H),
-                           ("qkv_weights", L * 3 * H * H), ("qkv_bias", L * 3 * H), ("o_proj_weights", L * H * H),
-                           ("lm_head_norm_weights", H), ("lm_head_weights", V * H), ("router_weights", L * E * H),
-                           ("router_logits_buf", E), ("expert_weights", k), ("shared_expert_gate_proj_weights", L * Fs * H),
-                           ("shared_expert_up_proj_weights", L * Fs * H), ("shared_expert_down_proj_weights", L * H * Fs),
-                           ("shared_expert_silu_out", Fs), ("shared_out", H), ("shared_expert_gate_weights", L * H),
-                           ("expert_gate_up_proj_weights", L * E * 2 * Fm * H), ("expert_down_proj_weights", L * E * H * Fm),
-                           ("routed_silu_buffer", k * Fm), ("routed_out_f32", H), ("routed_out", H)):
+        sizes = [("hidden_states", H), ("normed_hidden_states", H), ("q_post_rope", AW), ("attn_out", AW), ("silu_out", Fm),
+                 ("k_cache", L * S * nkv * d), ("v_cache", L * S * nkv * d), ("attn_lse_intermediates", nq * P),
+                 ("attn_out_intermediates", nq * P * d), ("attn_norm_weights", L * H), ("mlp_norm_weights", L * H),
+                 ("qkv_weights", L * QKV * H), ("o_proj_weights", L * H * AW),
+                 ("lm_head_norm_weights", H), ("lm_head_weights", V * H), ("router_weights", L * E * H),
+                 ("router_logits_buf", E), ("expert_weights", k),
+                 ("expert_gate_up_proj_weights", L * E * 2 * Fm * H), ("expert_down_proj_weights", L * E * H * Fm),
+                 ("routed_silu_buffer", k * Fm), ("routed_out_f32", H), ("routed_out", H)]
+        if s.qkv_bias:
+            sizes.append(("qkv_bias", L * QKV))
+        if s.has_shared_expert:
+            sizes += [("shared_expert_gate_proj_weights", L * Fs * H), ("shared_expert_up_proj_weights", L * Fs * H),
+                      ("shared_expert_down_proj_weights", L * H * Fs), ("shared_expert_silu_out", Fs), ("shared_out", H),
+                      ("shared_expert_gate_weights", L * H)]
+        if s.qk_norm:
+            sizes += [("qkv_raw", QKV), ("q_norm_weights", L * d), ("k_norm_weights", L * d)]
+        for name, want in sizes:
             numel(name, want)
-        if tensors["rope_cos"].shape != tensors["rope_sin"].shape or tensors["rope_cos"].shape[-1] != 128:
+        if tensors["rope_cos"].shape != tensors["rope_sin"].shape or tensors["rope_cos"].shape[-1] != d:
             raise ValueError("rope_cos/rope_sin must both be [positions, head_dim]")
         bar = tensors["barriers"]
         self._barriers = bar
@@ -154,7 +188,9 @@ class MoeMegaKernel:
         a.num_queues, a.num_insts = int(tensors["instructions"].shape[0]), int(tensors["instructions"].shape[1])
         a.num_layers, a.num_layer_barriers, a.barrier_slots = L, int(bar.shape[1]), int(bar.shape[2])
         a.max_seq_len, a.max_splits, a.vocab_size, a.rope_rows = S, P, V, int(tensors["rope_cos"].shape[0])
-        a.num_experts, a.top_k, a.shared_ffn, a.moe_ffn, a.shared_k_slices = E, k, Fs, Fm, int(s.num_downproj_split_k_shared)
+        a.num_experts, a.top_k, a.shared_ffn, a.moe_ffn = E, k, Fs, Fm
+        a.shared_k_slices = int(s.num_downproj_split_k_shared) if s.has_shared_expert else 0
+        a.norm_topk_prob, a.routed_upgate_tile = int(bool(s.norm_topk_prob)), int(s.routed_upgate_tile)
         nbytes = int(self._lib.qmk_moe_workspace_bytes(k, a.shared_k_slices))
         if nbytes == 0:
             raise ValueError(f"top_k {k} / {a.shared_k_slices} K slices are outside what the kernel supports")
@@ -163,10 +199,14 @@ class MoeMegaKernel:
         a.workspace, a.workspace_bytes = self._workspace.data_ptr(), nbytes
 
     def __call__(self, *args: Any) -> None:
-        if len(args) != len(_TENSOR_ORDER) + 3:
-            raise TypeError(f"mk of the MoE route takes {len(_TENSOR_ORDER)} tensors and 3 scalars, got {len(args)} positional arguments")
-        tensors = {name: t for name, t in zip(_TENSOR_ORDER, args) if name is not None}
-        pos_id, attn_scale, rms_norm_eps = args[len(_TENSOR_ORDER):]
+        order = _TENSOR_ORDER + (_QWEN3_EXTRA if len(args) == len(_TENSOR_ORDER) + 3 + len(_QWEN3_EXTRA) else ())
+        if len(args) != len(order) + 3:
+            raise TypeError(f"mk of the MoE route takes {len(_TENSOR_ORDER)} tensors (with the Qwen3 op set's attention "
+                            f"{len(_TENSOR_ORDER) + len(_QWEN3_EXTRA)}) and 3 scalars, got {len(args)} positional arguments")
+        tensors = {name: t for name, t in zip(order, args) if name is not None}
+        for name in _QWEN3_EXTRA:
+            tensors.setdefault(name, None)
+        pos_id, attn_scale, rms_norm_eps = args[len(order):]
         if isinstance(tensors["instructions"], torch.Tensor) and tensors["instructions"].numel() == 0:
             return
         key = tuple((t.data_ptr(), tuple(t.shape)) if isinstance(t, torch.Tensor) else None for t in tensors.values()) + (QwenMoeConfig.shape(),)
@@ -216,6 +256,7 @@ def call_mk(globs: Globals, mk: Any) -> None:
        g.shared_expert_up_proj_weights, g.shared_expert_down_proj_weights, g.shared_expert_silu_out, g.shared_out,
        g.shared_expert_gate_weights, g.expert_gate_up_proj_weights, g.expert_down_proj_weights, g.routed_silu_buffer,
        g.routed_out_f32, g.routed_out, g.barriers,
+       *((g.qkv_raw, g.q_norm_weights, g.k_norm_weights) if s.qk_norm else ()),
        g.position_id if g.position_id is not None else 0, 1.0 / math.sqrt(s.head_dim), float(s.rms_norm_eps))
 
 

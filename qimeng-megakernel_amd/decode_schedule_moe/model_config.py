@@ -1,4 +1,5 @@
-"""Shape and schedule constants of the MoE decode route (Qwen1.5-MoE-A2.7B by default).
+"""Shape and schedule constants of the MoE decode route (Qwen1.5-MoE-A2.7B by default; ``QWEN3_30B_A3B`` is
+the second compiled geometry: the Qwen3 op set's attention in front of a MoE block without a shared expert).
 
 ``QwenMoeConfig`` keeps the reference's access pattern — class attributes read at call time,
 ``update_from_dict`` (`…/qwen1_5_moe_a2_7b/A100/single_batch/decode_schedule/model_config.py:8-180`)
@@ -24,12 +25,18 @@ class MoeShape:
     moe_intermediate_size: int = 1408       # one routed expert
     num_experts: int = 60
     num_experts_per_tok: int = 4
-    norm_topk_prob: bool = False
+    norm_topk_prob: bool = False            # top-k weights divided by their sum (`…/fused/operations.py:405`)
     qkv_bias: bool = True
+    qk_norm: bool = False                   # the Qwen3 op set's attention: raw QKV, per-head RMSNorm of q and k, RoPE
     attn_kv_block_size: int = 16
     attn_reduction_size: int = 4
     tile_n_granularity: int = 16
     num_downproj_split_k_shared: int = 4
+    routed_upgate_tile: int = 16            # outputs per tile of the routed up/gate instructions (16, or 8)
+
+    @property
+    def has_shared_expert(self) -> bool:
+        return self.intermediate_size > 0
 
     @property
     def num_heads(self) -> int:
@@ -48,8 +55,12 @@ class MoeShape:
         return self.moe_intermediate_size // self.tile_n_granularity
 
     @property
+    def num_routed_upgate_blocks(self) -> int:
+        return self.moe_intermediate_size // self.routed_upgate_tile
+
+    @property
     def split_k_granularity_shared(self) -> int:
-        return self.intermediate_size // self.num_downproj_split_k_shared
+        return self.intermediate_size // max(1, self.num_downproj_split_k_shared)
 
     @property
     def barrier_slots(self) -> int:
@@ -60,10 +71,10 @@ class MoeShape:
         ``num_experts_per_tok`` routed experts it selects, norms, LM head."""
         h = self.hidden_size
         attn = (self.qkv_out_dim * h + self.num_attention_heads * self.head_dim * h) * 2 + (self.qkv_out_dim * 2 if self.qkv_bias else 0)
-        shared = 3 * self.intermediate_size * h * 2 + h * 2
+        shared = (3 * self.intermediate_size * h * 2 + h * 2) if self.has_shared_expert else 0
         routed = self.num_experts_per_tok * 3 * self.moe_intermediate_size * h * 2
         router = self.num_experts * h * 2
-        per_layer = attn + shared + routed + router + 2 * h * 2
+        per_layer = attn + shared + routed + router + 2 * h * 2 + (2 * self.head_dim * 2 if self.qk_norm else 0)
         return per_layer * self.num_hidden_layers + self.vocab_size * h * 2 + h * 2
 
     def kv_bytes_per_context_token(self) -> int:
@@ -75,6 +86,15 @@ class MoeShape:
 
 
 QWEN1_5_MOE_A2_7B = MoeShape()
+
+#: Qwen3-30B-A3B shape: 48 layers, 32 query / 4 KV heads of 128 (attention output 4096 wide), per-head QK RMSNorm,
+#: no QKV bias, 128 experts of 768 with renormalised top-8 routing, no shared expert, untied LM head; 61 GB in bf16.
+#: Routed up/gate tiles of 8 outputs: 8 x 96 = 768 tiles, three per queue of a 256-CU device.
+QWEN3_30B_A3B = MoeShape(
+    num_hidden_layers=48, num_attention_heads=32, num_key_value_heads=4, intermediate_size=0, moe_intermediate_size=768,
+    num_experts=128, num_experts_per_tok=8, norm_topk_prob=True, qkv_bias=False, qk_norm=True, attn_reduction_size=8,
+    num_downproj_split_k_shared=0, routed_upgate_tile=8,
+)
 
 MAX_OPCODE = 14
 NUM_OPCODE_ROWS = MAX_OPCODE + 1
@@ -133,6 +153,8 @@ class QwenMoeConfig(metaclass=_ConfigMeta):
             num_experts_per_tok=int(config.get("num_experts_per_tok", 4)),
             norm_topk_prob=bool(config.get("norm_topk_prob", False)),
         )
+        if changes["intermediate_size"] == 0:    # no shared expert: nothing to split
+            changes["num_downproj_split_k_shared"] = 0
         cls.set_shape(dataclasses.replace(cls._shape, **changes))
 
 

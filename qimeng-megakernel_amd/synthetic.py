@@ -189,33 +189,60 @@ def reduced_shape(num_layers: int = 2, vocab_size: int = 2048, **overrides: Any)
     return dataclasses.replace(LlamaConfig.shape().__class__(), num_hidden_layers=num_layers, vocab_size=vocab_size, **overrides)
 
 
-def random_moe_weights(shape: Any, seed: int, max_positions: int) -> dict[str, torch.Tensor]:
+def random_moe_weights(shape: Any, seed: int, max_positions: int, device: torch.device | str = "cpu") -> dict[str, torch.Tensor]:
     """Seeded random-init weights of the MoE route (``decode_schedule_moe.MoeShape``): bf16 ~N(0, 0.02)
     projections, router and experts (gate rows first in ``expert_gate_up_proj_weights``), QKV bias
-    ~N(0, 0.02), norm weights near one (not all ones: the router and the shared gate read the
-    normalised row directly), untied LM head.  CPU tensors."""
-    gen = torch.Generator(device="cpu")
+    ~N(0, 0.02) where the shape has one, norm weights near one (not all ones: the router and the shared
+    gate read the normalised row directly), untied LM head; the tensors of a shared expert and of the
+    per-head QK norm only for shapes that have them.
+
+    ``device`` "cpu" (default): drawn on a CPU generator, so a seed names the same model on every machine.
+    On a GPU the draws come from that device's generator, one layer of experts at a time — for models
+    whose weights (61 GB for the Qwen3-30B-A3B shape) should not pass through host memory."""
+    device = torch.device(device)
+    gen = torch.Generator(device=device)
     gen.manual_seed(seed)
+
+    def normal(*size: int) -> torch.Tensor:
+        return (torch.randn(*size, generator=gen, dtype=torch.float32, device=device) * WEIGHT_STD).to(torch.bfloat16)
+
+    def stacked(count: int, *size: int) -> torch.Tensor:
+        out = torch.empty(count, *size, dtype=torch.bfloat16, device=device)
+        for i in range(count):
+            out[i] = normal(*size)
+        return out
+
     L, H, V = shape.num_hidden_layers, shape.hidden_size, shape.vocab_size
     F, Fm, E = shape.intermediate_size, shape.moe_intermediate_size, shape.num_experts
     w: dict[str, torch.Tensor] = {}
-    w["embed_tokens"] = _normal_bf16(gen, V, H)
-    w["qkv_weights"] = torch.stack([_normal_bf16(gen, shape.qkv_out_dim, H) for _ in range(L)])
+    w["embed_tokens"] = normal(V, H)
+    w["qkv_weights"] = stacked(L, shape.qkv_out_dim, H)
     if shape.qkv_bias:
-        w["qkv_bias"] = torch.stack([_normal_bf16(gen, shape.qkv_out_dim) for _ in range(L)])
-    w["o_proj_weights"] = torch.stack([_normal_bf16(gen, H, shape.num_attention_heads * shape.head_dim) for _ in range(L)])
-    w["router_weights"] = torch.stack([_normal_bf16(gen, E, H) for _ in range(L)])
-    w["shared_expert_gate_proj_weights"] = torch.stack([_normal_bf16(gen, F, H) for _ in range(L)])
-    w["shared_expert_up_proj_weights"] = torch.stack([_normal_bf16(gen, F, H) for _ in range(L)])
-    w["shared_expert_down_proj_weights"] = torch.stack([_normal_bf16(gen, H, F) for _ in range(L)])
-    w["shared_expert_gate_weights"] = torch.stack([_normal_bf16(gen, 1, H) for _ in range(L)])
-    w["expert_gate_up_proj_weights"] = torch.stack([torch.stack([_normal_bf16(gen, 2 * Fm, H) for _ in range(E)]) for _ in range(L)])
-    w["expert_down_proj_weights"] = torch.stack([torch.stack([_normal_bf16(gen, H, Fm) for _ in range(E)]) for _ in range(L)])
-    w["lm_head_weights"] = _normal_bf16(gen, V, H)
-    for name, size in (("attn_norm_weights", (L, H)), ("mlp_norm_weights", (L, H)), ("lm_head_norm_weights", (H,))):
-        w[name] = (1.0 + 0.1 * torch.randn(*size, generator=gen, dtype=torch.float32)).to(torch.bfloat16)
+        w["qkv_bias"] = stacked(L, shape.qkv_out_dim)
+    w["o_proj_weights"] = stacked(L, H, shape.num_attention_heads * shape.head_dim)
+    w["router_weights"] = stacked(L, E, H)
+    if shape.has_shared_expert:
+        w["shared_expert_gate_proj_weights"] = stacked(L, F, H)
+        w["shared_expert_up_proj_weights"] = stacked(L, F, H)
+        w["shared_expert_down_proj_weights"] = stacked(L, H, F)
+        w["shared_expert_gate_weights"] = stacked(L, 1, H)
+    w["expert_gate_up_proj_weights"] = torch.empty(L, E, 2 * Fm, H, dtype=torch.bfloat16, device=device)
+    for layer in range(L):
+        for e in range(E):
+            w["expert_gate_up_proj_weights"][layer, e] = normal(2 * Fm, H)
+    w["expert_down_proj_weights"] = torch.empty(L, E, H, Fm, dtype=torch.bfloat16, device=device)
+    for layer in range(L):
+        for e in range(E):
+            w["expert_down_proj_weights"][layer, e] = normal(H, Fm)
+    w["lm_head_weights"] = normal(V, H)
+    norms = [("attn_norm_weights", (L, H)), ("mlp_norm_weights", (L, H)), ("lm_head_norm_weights", (H,))]
+    if shape.qk_norm:
+        norms += [("q_norm_weights", (L, shape.head_dim)), ("k_norm_weights", (L, shape.head_dim))]
+    for name, size in norms:
+        w[name] = (1.0 + 0.1 * torch.randn(*size, generator=gen, dtype=torch.float32, device=device)).to(torch.bfloat16)
     rope_shape = DecodeShape(head_dim=shape.head_dim, rope_theta=shape.rope_theta)
-    w["rope_cos"], w["rope_sin"] = rope_tables(rope_shape, max_positions)
+    cos, sin = rope_tables(rope_shape, max_positions)
+    w["rope_cos"], w["rope_sin"] = cos.to(device), sin.to(device)
     return w
 
 
@@ -247,8 +274,8 @@ def build_moe_globals(weights: dict[str, torch.Tensor], shape: Any, kv_capacity:
         attn_lse_intermediates=zeros(nq, max_partials, dtype=torch.float32),
         router_logits_buf=zeros(shape.num_experts, dtype=torch.float32),
         normed_hidden_states=zeros(H),
-        shared_expert_silu_out=zeros(shape.intermediate_size),
-        shared_out=zeros(H),
+        **(dict(shared_expert_silu_out=zeros(shape.intermediate_size), shared_out=zeros(H)) if shape.has_shared_expert else {}),
+        **(dict(qkv_raw=zeros(shape.qkv_out_dim)) if shape.qk_norm else {}),
         routed_out=zeros(H),
         routed_out_f32=zeros(H, dtype=torch.float32),
         routed_silu_buffer=zeros(k, shape.moe_intermediate_size),

@@ -79,8 +79,8 @@ def test_host_side_argument_errors(lib):
     assert lib.qmk_decode_step(ctypes.byref(a)) == 8                       # QMK_ERR_MODEL
     a.model = 0
     assert lib.qmk_decode_step(ctypes.byref(a)) == 1                       # all tensor pointers are NULL
-    assert lib.qmk_workspace_bytes(0) == 8 * (4096 + 1024 + 512 + 4096 + 1024 + 16) and lib.qmk_workspace_bytes(1) == lib.qmk_workspace_bytes(0) and lib.qmk_workspace_bytes(7) == 0
-    assert lib.qmk_query(0) == 6 and lib.qmk_query(2) == 512 and lib.qmk_query(5) == 32 and lib.qmk_query(6) == 25
+    assert lib.qmk_workspace_bytes(0) == 8 * (512 + 2048 + 4 * 1024 + 4096 + 1024 + 16) and lib.qmk_workspace_bytes(1) == lib.qmk_workspace_bytes(0) and lib.qmk_workspace_bytes(7) == 0
+    assert lib.qmk_query(0) == 7 and lib.qmk_query(2) == 512 and lib.qmk_query(5) == 32 and lib.qmk_query(6) == 25
     assert 0 < lib.qmk_query(3) <= 160 * 1024
     assert lib.qmk_error_string(34).decode().startswith("device: counter wait")
     mk_kernel_mb.get_mk()                                                  # declares the entry point's signature
