@@ -379,6 +379,10 @@ typedef struct QmkMoeArgs {
                                       order); 0: raw probabilities, as the reference's decode route leaves them   */
   int32_t routed_upgate_tile;      /* outputs per tile of opcode 12 (its tile_N_granularity word): 16 (0 = 16), or 8
                                       where that deals the tiles evenly (Fm = 768: 768 tiles for 256 queues)        */
+  int32_t oproj_tile;              /* rows per tile of opcode 4 (its tile_N_granularity word): 16 (0 = 16), or 8, which
+                                      gives each of 256 queues one tile of the 2048 rows; fixes the final value of the
+                                      O-projection counter (H / oproj_tile)                                          */
+  int32_t reserved;                /* 0 */
 } QmkMoeArgs;
 
 int qmk_decode_step_moe(const QmkMoeArgs* args);

@@ -199,7 +199,7 @@ class MoeInstructionVM:
     # ---- 8, 9 --------------------------------------------------------------------
     def router_gemv(self, g: Any, ins: Any) -> None:
         s, layer = self.shape, ins.layer_idx
-        assert int(g.barriers[layer, 3, 0]) == s.num_hidden_blocks
+        assert int(g.barriers[layer, 3, 0]) == s.hidden_size // getattr(s, "oproj_tile", TILE)
         normed = rms_norm(g.hidden_states.reshape(-1), g.mlp_norm_weights[layer], s.rms_norm_eps)
         e0 = ins.tile_N_start_idx * ins.tile_N_granularity
         e1 = min(ins.tile_N_end_idx * ins.tile_N_granularity, s.num_experts)
@@ -260,10 +260,15 @@ class MoeInstructionVM:
             g.silu_out.reshape(-1)[r0:r1] = piece            # the single buffer of the fused route is kept up to date too
             g.routed_silu_buffer[ins.expert_idx, r0:r1] = piece
         g.barriers[layer, 11, 0] += ins.tile_N_end_idx - ins.tile_N_start_idx
+        g.barriers[layer, 14, ins.expert_idx] += ins.tile_N_end_idx - ins.tile_N_start_idx   # this build's per-slot count
 
     def routed_expert_downproj(self, g: Any, ins: Any) -> None:
         s, layer = self.shape, ins.layer_idx
-        assert int(g.barriers[layer, 11, 0]) == s.num_experts_per_tok * (s.moe_intermediate_size // getattr(s, "routed_upgate_tile", TILE))
+        per_slot = s.moe_intermediate_size // getattr(s, "routed_upgate_tile", TILE)
+        if ins.tile_M_idx == 1:     # this build's streams: the slot's own tiles are enough
+            assert int(g.barriers[layer, 14, ins.expert_idx]) == per_slot
+        else:
+            assert int(g.barriers[layer, 11, 0]) == s.num_experts_per_tok * per_slot
         eid = int(g.expert_indices[ins.expert_idx])
         w = g.expert_weights[ins.expert_idx].to(torch.float32)
         mat = g.expert_down_proj_weights[layer, eid].contiguous()

@@ -600,8 +600,9 @@ extern "C" uint64_t qmk_moe_workspace_bytes(int top_k, int shared_k_slices) {
   if (top_k < 1 || top_k > moe::kMaxTopK || shared_k_slices < 0 || shared_k_slices > 16) return 0;   // 0 slices: no shared expert
   const uint64_t shared = static_cast<uint64_t>(shared_k_slices) * QwenMoeA2_7B::H * sizeof(u16);
   // the down projections' terms, the gate scalar's line, then the tagged units of the residual stream and q/k/v
+  static_assert(QwenMoeA2_7B::H <= 2048 && Qwen3MoeA3B::H <= 2048 && moe::kMaxTopK <= 8 && moe::kMaxK <= 2048, "the tagged MoE regions");
   return ((shared + 127) / 128) * 128 + static_cast<uint64_t>(top_k) * QwenMoeA2_7B::H * sizeof(float) + 128 +
-         static_cast<uint64_t>(kWsUnits) * sizeof(uint64_t);
+         static_cast<uint64_t>(kWsMoeUnits) * sizeof(uint64_t);
 }
 
 namespace {
@@ -636,6 +637,8 @@ int decode_step_moe(const QmkMoeArgs* a) {
   const int routed_tile = a->routed_upgate_tile == 0 ? moe::kTile : a->routed_upgate_tile;
   if ((routed_tile != 8 && routed_tile != 16) || a->moe_ffn % routed_tile) return QMK_ERR_SHAPE;
   if (a->norm_topk_prob != 0 && a->norm_topk_prob != 1) return QMK_ERR_SHAPE;
+  const int oproj_tile = a->oproj_tile == 0 ? moe::kTile : a->oproj_tile;
+  if ((oproj_tile != 8 && oproj_tile != 16) || a->reserved != 0) return QMK_ERR_SHAPE;
   if (a->flags & ~(QMK_FLAG_KEEP_BARRIERS | QMK_FLAG_TAGGED)) return QMK_ERR_SHAPE;
   // tagged units carry the launch count, which the retiring launch advances, and six bits of layer
   if ((a->flags & QMK_FLAG_TAGGED) && ((a->flags & QMK_FLAG_KEEP_BARRIERS) || a->num_layers > 63)) return QMK_ERR_SHAPE;
@@ -685,7 +688,7 @@ int decode_step_moe(const QmkMoeArgs* a) {
   p.attn_scale = a->attn_scale;
   p.rms_norm_eps = a->rms_norm_eps;
   p.qkv_blocks_per_head = M::D / 16;
-  p.oproj_blocks = M::H / 16;
+  p.oproj_blocks = M::H / oproj_tile;
   p.down_arrivals = M::H / 16;           // what completes a layer here: the combine step's tiles
   p.spin_limit = a->spin_limit > 0 ? a->spin_limit : kDefaultSpinLimit;
   p.flags = a->flags;

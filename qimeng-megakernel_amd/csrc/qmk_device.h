@@ -192,6 +192,22 @@ __device__ __forceinline__ float wave_max(float v) {
   return __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), 63));
 }
 
+// Minimum of a signed integer over the 64 lanes; every lane gets it.
+template <int kCtrl, int kRowMask = 0xf>
+__device__ __forceinline__ int dpp_i32(int identity, int v) {
+  return __builtin_amdgcn_update_dpp(identity, v, kCtrl, kRowMask, 0xf, false);
+}
+__device__ __forceinline__ int wave_min_i32(int v) {
+  constexpr int kMax = 0x7fffffff;
+  v = min(v, dpp_i32<kDppRowShr + 1>(kMax, v));
+  v = min(v, dpp_i32<kDppRowShr + 2>(kMax, v));
+  v = min(v, dpp_i32<kDppRowShr + 4>(kMax, v));
+  v = min(v, dpp_i32<kDppRowShr + 8>(kMax, v));
+  v = min(v, dpp_i32<kDppRowBcast15, 0xa>(kMax, v));
+  v = min(v, dpp_i32<kDppRowBcast31, 0xc>(kMax, v));
+  return __builtin_amdgcn_readlane(v, 63);
+}
+
 // Sum over each aligned group of 8 lanes; every lane of the group gets the group's total.
 __device__ __forceinline__ float group8_sum(float v) {
   v += dpp_f32<kDppQuadXor1>(0.f, v);
@@ -210,6 +226,19 @@ __device__ __forceinline__ float block_sum(float v, float* scratch) {
   float t = 0.f;
 #pragma unroll
   for (int w = 0; w < kWaves; ++w) t += scratch[w];
+  return t;
+}
+
+// Maximum over the workgroup; `scratch` holds kWaves floats.  All threads get it.
+__device__ __forceinline__ float block_max(float v, float* scratch) {
+  v = wave_max(v);
+  const int lane = threadIdx.x & (kWaveSize - 1), wave = threadIdx.x / kWaveSize;
+  __syncthreads();
+  if (lane == 0) scratch[wave] = v;
+  __syncthreads();
+  float t = scratch[0];
+#pragma unroll
+  for (int w = 1; w < kWaves; ++w) t = fmaxf(t, scratch[w]);
   return t;
 }
 
@@ -284,6 +313,11 @@ constexpr int kWsCandidates = kWsSilu + 4096;       // one greedy candidate per 
 constexpr int kMaxSamplingQueues = 1024;
 constexpr int kWsExperts = kWsCandidates + kMaxSamplingQueues;   // MoE route: the top-k's experts, then their weights (8 units each)
 constexpr int kWsUnits = kWsExperts + 16;
+// MoE route only, behind the regions above (its workspace is sized by qmk_moe_workspace_bytes):
+constexpr int kWsLogits = kWsUnits;                   // router logits, one fp32 per unit (room for 512 experts)
+constexpr int kWsRoutedSilu = kWsLogits + 512;        // silu vectors of the routed experts: 1024 units (2048 values) per slot
+constexpr int kWsRoutedParts = kWsRoutedSilu + 8 * 1024;   // weighted down-projection rows of the routed experts: H fp32 units per slot
+constexpr int kWsMoeUnits = kWsRoutedParts + 8 * 2048;
 
 __device__ __forceinline__ bool tagged(const Params& p) { return (p.flags & QMK_FLAG_TAGGED) != 0; }
 __device__ __forceinline__ uint32_t tag_of(uint32_t generation, int layer) { return (generation << 6) + static_cast<uint32_t>(layer) + 1u; }

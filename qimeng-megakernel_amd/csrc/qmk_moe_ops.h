@@ -36,6 +36,7 @@ struct QwenMoeA2_7B {
   static constexpr bool QKV_BIAS = true;
   static constexpr int REDUCE_HEADS = 4;   // attn_reduction_size of the route (model_config.py:27)
   static constexpr int PREV_ROW = 13;      // a layer is complete when its combine step is
+  static constexpr int UPGATE_OUTPUTS_IN_FLIGHT = 4;   // per wave, in the expert up/gate ops (2 measured the same here)
 };
 
 // Qwen3-30B-A3B layer geometry: 32 query heads over 4 KV heads of 128 (the attention output is twice as
@@ -59,6 +60,9 @@ struct Qwen3MoeA3B {
   static constexpr bool QKV_BIAS = false;
   static constexpr int REDUCE_HEADS = GQA;
   static constexpr int PREV_ROW = 13;
+  // One output (two rows) per wave in flight: a queue has 24 outputs of a phase, and with all of a wave's rows
+  // requested at once the hand-overs behind them wait for the whole burst (measured: 395 against 381 tok/s with 4).
+  static constexpr int UPGATE_OUTPUTS_IN_FLIGHT = 1;
 };
 
 namespace moe {
@@ -74,6 +78,10 @@ enum Opcode {
 };
 constexpr int ROW_ROUTER = 7, ROW_TOPK = 8, ROW_SHARED_UPGATE = 9, ROW_SHARED_DOWN = 10, ROW_ROUTED_UPGATE = 11, ROW_ROUTED_DOWN = 12,
               ROW_COMBINE = 13;
+// An extension of this build, in the row behind the reference's fourteen: the routed up/gate tiles counted per expert
+// slot as well, so that a slot's down projection can start when its own silu vector is complete (word tile_M_idx of
+// opcode 13 = 1) instead of when all slots' are.
+constexpr int ROW_ROUTED_UPGATE_SLOT = 14;
 constexpr int kMaxK = 2048;       // longest dot product of these ops (a K slice, an expert's FFN width, H)
 constexpr int kMaxExperts = 512;
 constexpr int kMaxTopK = 8;
@@ -161,7 +169,11 @@ __device__ __forceinline__ bool op_router(const Params& p, Smem<M>& s, const Ctx
     const u16* const rows[1] = {w + static_cast<size_t>(e) * M::H};
     float v[1];
     rows_dot<1>(rows, s.x, M::H, lane, v);
-    if (lane == 0) st_shared_f32(p.router_logits + e, v[0]);
+    if (lane == 0) {
+      st_shared_f32(p.router_logits + e, v[0]);
+      // tagged launch: the routed up/gate workgroups take the routing decision themselves from these
+      if (tagged(p)) st_tagged(p.ws + kWsLogits + e, __float_as_uint(v[0]), tag_of(s.generation, layer));
+    }
   }
   const bool publish_row = s.inst[4] != 0;
   if (publish_row) {
@@ -186,72 +198,104 @@ __device__ __forceinline__ bool op_router(const Params& p, Smem<M>& s, const Ctx
 
 // ===================================================================== 9 ==
 // [9, layer]   softmax over all router logits, the top_k largest probabilities and their experts, in
-// decreasing order (ties: the lower expert first), not renormalised   (python_vm.py:360-372).
+// decreasing order (ties: the lower expert first)   (python_vm.py:360-372); renormalised to sum 1 when the
+// launch asks for it (fused/operations.py:405).
+// Softmax over the E router logits (thread t brings expert t's; threads beyond E bring nothing) and the top_k picks:
+// afterwards, for every slot j < top_k, picked[j] is the pick's probability and picked[kMaxTopK + j] its expert (as
+// int bits), in decreasing order of probability, the lower expert first among equals — the order repeated arg-max
+// with first-index ties produces.  Instead of top_k dependent sweeps every expert counts the experts that go before
+// it; a count below top_k is the pick's slot.  False (uniformly) when a logit is NaN or infinite: no order to pick by.
+// Uses s.res[0 .. 2 * kMaxExperts) and s.red.
+template <class M>
+__device__ __forceinline__ bool rank_experts(const Params& p, Smem<M>& s, const Ctx& c, float logit, float* picked) {
+  const int t = c.tid, E = p.num_experts;
+  const bool live = t < E;
+  const float mx = block_max(live ? logit : -INFINITY, s.red);
+  const float x = live ? expf(logit - mx) : 0.f;
+  const int padded = (E + 3) & ~3;
+  int* counts = reinterpret_cast<int*>(s.res) + kMaxExperts;      // behind the probabilities
+  if (t < padded) {
+    s.res[t] = live ? x : -1.f;   // padded to whole groups of four with values nobody goes behind
+    counts[t] = 0;
+  }
+  const float sum = block_sum(x, s.red);   // its barriers also make s.res complete
+  const bool ok = sum > 0.f && sum < INFINITY;
+  QMK_STAMP(2);
+  // The E x E comparisons are spread over the whole workgroup (one wave alone would spend 3-4 us on them): thread t
+  // compares expert t % E' with a slice of the others and adds its count to the expert's.
+  int parts = 1;
+  while (2 * parts * padded <= kThreads) parts *= 2;
+  const int mine = t % padded, part = t / padded;
+  if (ok && part < parts && mine < E) {
+    const float xm = s.res[mine];
+    const int per = ((padded / 4 + parts - 1) / parts) * 4;        // a slice is whole groups of four
+    const int e0 = part * per, e1 = min(e0 + per, padded);
+    int before = 0;
+    const float4* all = reinterpret_cast<const float4*>(s.res);
+#pragma unroll 4
+    for (int e = e0; e < e1; e += 4) {
+      const float4 v = all[e >> 2];
+      before += (v.x > xm || (v.x == xm && e < mine)) ? 1 : 0;
+      before += (v.y > xm || (v.y == xm && e + 1 < mine)) ? 1 : 0;
+      before += (v.z > xm || (v.z == xm && e + 2 < mine)) ? 1 : 0;
+      before += (v.w > xm || (v.w == xm && e + 3 < mine)) ? 1 : 0;
+    }
+    if (before) atomicAdd(&counts[mine], before);
+  }
+  QMK_STAMP(3);
+  __syncthreads();
+  if (ok && live && counts[t] < p.top_k) {
+    picked[counts[t]] = x / sum;
+    picked[kMaxTopK + counts[t]] = __int_as_float(t);
+  }
+  __syncthreads();
+  return ok;
+}
+
 template <class M>
 __device__ __forceinline__ bool op_topk(const Params& p, Smem<M>& s, const Ctx& c) {
   const int layer = s.inst[1], E = p.num_experts;
+  static_assert(kMaxExperts <= kThreads, "one thread per expert");
   if (layer < 0 || layer >= p.num_layers) return bad_operand(p, s, c, 1);
-  if (!wait_one(p, s, c, layer, ROW_ROUTER, 0, E)) return false;
-  for (int e = c.tid; e < E; e += kThreads) s.res[e] = ld_shared_f32(p.router_logits + e);
-  __syncthreads();
-  if (c.tid < kWaveSize) {
-    const int lane = c.tid;
-    float mx = -INFINITY;
-    for (int e = lane; e < E; e += kWaveSize) mx = fmaxf(mx, s.res[e]);
-    mx = wave_max(mx);
-    float sum = 0.f;
-    for (int e = lane; e < E; e += kWaveSize) {
-      const float x = expf(s.res[e] - mx);
-      s.res[e] = x;
-      sum += x;
+  const int t = c.tid;
+  const bool tg = tagged(p);
+  float logit = 0.f;
+  if (tg) {
+    // Tagged launch: the logits from their units, like every consumer of the routing decision; nobody inside the
+    // launch reads what this instruction writes, so it neither drains its stores nor counts.
+    uint32_t bits = 0;
+    if (t < E && !poll_tagged1(p.ws + kWsLogits + t, tag_of(s.generation, layer), p.spin_limit, bits)) {
+      s.ctl[0] = 1;
+      report_error(p, QMK_DEV_WAIT_TIMEOUT, c.inst_idx, c.opcode, t);
     }
-    sum = wave_sum(sum);
-    float* picked = &s.merge[0][0][0];   // the probabilities of the picks, in slot order; their experts behind them
-    bool complete = true;
+    logit = __uint_as_float(bits);
+    QMK_STAMP(0);
+  } else {
+    if (!wait_one(p, s, c, layer, ROW_ROUTER, 0, E)) return false;
+    if (t < E) logit = ld_shared_f32(p.router_logits + t);
+  }
+  float* picked = &s.merge[0][0][0];
+  const bool ranked = rank_experts<M>(p, s, c, logit, picked);   // (its barriers publish s.ctl[0])
+  QMK_STAMP(1);
+  if (s.ctl[0]) return false;
+  if (!ranked) return bad_operand(p, s, c, 0);
+  if (t == 0) {
+    // norm_topk_prob: the picks' probabilities divided by their sum, added up in slot order (fp32)
+    float total = 0.f;
+    for (int j = 0; j < p.top_k; ++j) total += picked[j];
     for (int j = 0; j < p.top_k; ++j) {
-      float best = -1.f;
-      int idx = 0x7fffffff;
-      for (int e = lane; e < E; e += kWaveSize)
-        if (s.res[e] > best) best = s.res[e], idx = e;   // ascending e: the first of equals stays
-      for (int off = 1; off < kWaveSize; off <<= 1) {
-        const float ob = __shfl_xor(best, off);
-        const int oi = __shfl_xor(idx, off);
-        if (ob > best || (ob == best && oi < idx)) best = ob, idx = oi;
-      }
-      if (idx < 0 || idx >= E) {   // no logit compares greater than "nothing": NaNs from a broken router row
-        if (lane == 0) {
-          s.ctl[0] = 1;
-          report_error(p, QMK_DEV_BAD_OPERAND, c.inst_idx, c.opcode, j);
-        }
-        complete = false;
-        break;   // uniform: every lane holds the same idx
-      }
-      if (lane == 0) {
-        picked[j] = best / sum;
-        picked[kMaxTopK + j] = __int_as_float(idx);
-        s.res[idx] = -2.f;   // taken
-      }
-      __builtin_amdgcn_wave_barrier();
+      const int idx = __float_as_int(picked[kMaxTopK + j]);
+      const float w = p.norm_topk ? picked[j] / total : picked[j];
+      __hip_atomic_store(p.expert_indices + j, static_cast<long long>(idx), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      st_shared_f32(p.expert_weights + j, w);
     }
-    if (complete && lane == 0) {
-      // norm_topk_prob: the picks' probabilities divided by their sum, added up in slot order (fp32)
-      float total = 0.f;
-      for (int j = 0; j < p.top_k; ++j) total += picked[j];
-      for (int j = 0; j < p.top_k; ++j) {
-        const int idx = __float_as_int(picked[kMaxTopK + j]);
-        const float w = p.norm_topk ? picked[j] / total : picked[j];
-        __hip_atomic_store(p.expert_indices + j, static_cast<long long>(idx), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        st_shared_f32(p.expert_weights + j, w);
-        if (tagged(p)) {   // the routed ops poll these instead of the counter below: one trip, no drain in between
-          st_tagged(p.ws + kWsExperts + j, static_cast<uint32_t>(idx), tag_of(s.generation, layer));
-          st_tagged(p.ws + kWsExperts + kMaxTopK + j, __float_as_uint(w), tag_of(s.generation, layer));
-        }
-      }
-    }
+  }
+  if (tg) {
+    __syncthreads();   // picked is read: s.merge and s.res may be reused
+    return true;
   }
   release_stores();
   __syncthreads();
-  if (s.ctl[0]) return false;
   if (c.tid == 0) __hip_atomic_store(counter_ptr(p, layer, ROW_TOPK, 0), 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
   return true;
 }
@@ -263,9 +307,9 @@ __device__ __forceinline__ bool op_topk(const Params& p, Smem<M>& s, const Ctx& 
 // asked for before it is called.
 template <class M, class Ready>
 __device__ __forceinline__ bool upgate_rows(Smem<M>& s, const Ctx& c, const u16* gate_w, const u16* up_w, int r0, int n, u16* dst0, u16* dst1,
-                                            Ready ready) {
+                                            Ready ready, uint64_t* units = nullptr, uint32_t tag = 0) {
   const int lane = c.tid & 63, wave = c.tid >> 6;
-  constexpr int kOut = 4;   // outputs (gate + up row each) of a wave in flight together: 32 KiB per wave
+  constexpr int kOut = M::UPGATE_OUTPUTS_IN_FLIGHT;   // outputs (gate + up row each) of a wave in flight together: 8 KiB each
   RowSet<2 * kOut> set;
   auto request = [&](int i) {
     const u16* rows[2 * kOut];
@@ -295,6 +339,7 @@ __device__ __forceinline__ bool upgate_rows(Smem<M>& s, const Ctx& c, const u16*
     const uint32_t word = static_cast<uint32_t>(f2bf(s.res[2 * pair])) | (static_cast<uint32_t>(f2bf(s.res[2 * pair + 1])) << 16);
     st_shared32(dst0 + r0 + 2 * pair, word);
     if (dst1 != nullptr) st_shared32(dst1 + r0 + 2 * pair, word);
+    if (units != nullptr) st_tagged(units + (r0 + 2 * pair) / 2, word, tag);
   }
   return true;
 }
@@ -414,6 +459,35 @@ __device__ __forceinline__ bool routed_expert(const Params& p, Smem<M>& s, const
   return s.ctl[0] == 0;
 }
 
+// Tagged launch: the routing decision taken by the consumer itself, from the router's logits as they announce
+// themselves — the top-k instruction's own function of the same 32-bit values (rank_experts, then the same
+// renormalisation in the same order), so the same experts and weights, bit for bit — instead of waiting for that
+// instruction to announce it: one hand-over less between the O-projection and the expert rows, during which the
+// whole device has nothing else to do.  The top-k instruction still leaves expert_indices / expert_weights for the
+// caller, off the critical path.  False (uniformly) when the wait ran out of polls or the logits have no order.
+template <class M>
+__device__ __forceinline__ bool routing_decision(const Params& p, Smem<M>& s, const Ctx& c, int layer, int slot, int& eid, float& weight) {
+  uint32_t bits = 0;
+  if (c.tid < p.num_experts && !poll_tagged1(p.ws + kWsLogits + c.tid, tag_of(s.generation, layer), p.spin_limit, bits)) {
+    s.ctl[0] = 1;
+    report_error(p, QMK_DEV_WAIT_TIMEOUT, c.inst_idx, c.opcode, c.tid);
+  }
+  if (p.timeline != nullptr && c.tid == 0) {
+    s.t_wait = wall_clock64();
+    s.ctl[2] = 1;
+  }
+  float* picked = &s.merge[0][0][0];
+  const bool ranked = rank_experts<M>(p, s, c, __uint_as_float(bits), picked);   // (its barriers publish s.ctl[0])
+  if (s.ctl[0]) return false;
+  if (!ranked) return bad_operand(p, s, c, 2);
+  float total = 0.f;
+  for (int j = 0; j < p.top_k; ++j) total += picked[j];
+  eid = __float_as_int(picked[kMaxTopK + slot]);
+  weight = p.norm_topk ? picked[slot] / total : picked[slot];
+  __syncthreads();   // picked is read: s.merge and s.res may be reused
+  return true;
+}
+
 // ==================================================================== 12 ==
 // [12, layer, expert_slot, n_start, n_end, tile_M_g, tile_N_g]   (python_vm.py:421-464)
 // The single buffer silu_out keeps what the last slot wrote, as after the VM's sequential run.
@@ -421,21 +495,30 @@ template <class M>
 __device__ __forceinline__ bool op_routed_upgate(const Params& p, Smem<M>& s, const Ctx& c) {
   const int layer = s.inst[1], slot = s.inst[2], n0 = s.inst[3], n1 = s.inst[4], tile = s.inst[6];
   if (layer < 0 || layer >= p.num_layers) return bad_operand(p, s, c, 1);
-  if (slot < 0 || slot >= p.top_k) return bad_operand(p, s, c, 2);
+  if (slot < 0 || slot >= p.top_k || slot >= p.barrier_slots - 1) return bad_operand(p, s, c, 2);
   if (tile != p.routed_tile || n0 < 0 || n1 < n0 || n1 * tile > p.moe_ffn || (n1 - n0) * tile > kResSlots) return bad_operand(p, s, c, 4);
-  // The normalised row first (as in opcode 10; a tagged launch has it long before the top-k is known), then the
-  // expert: its rows are the only thing left to wait for.
-  if (tagged(p) && !residual_to_lds<M>(p, s, c, layer)) return false;
+  const bool tg = tagged(p);
+  const uint32_t tag = tag_of(s.generation, layer);
   int eid;
   float unused;
-  if (!routed_expert<M>(p, s, c, layer, slot, eid, unused)) return false;
+  // A tagged launch has the normalised row long before the experts are known.
+  if (tg && !residual_to_lds<M>(p, s, c, layer)) return false;
+  if (!(tg ? routing_decision<M>(p, s, c, layer, slot, eid, unused) : routed_expert<M>(p, s, c, layer, slot, eid, unused))) return false;
   if (eid < 0) return bad_operand(p, s, c, 2);
   const u16* w = p.expert_gate_up_w + (static_cast<size_t>(layer) * p.num_experts + eid) * 2 * p.moe_ffn * M::H;
+  // tagged launch: the slot's down projections poll the silu values as units of their own
+  uint64_t* units = tg ? p.ws + kWsRoutedSilu + slot * 1024 : nullptr;
   if (!upgate_rows(s, c, w, w + static_cast<size_t>(p.moe_ffn) * M::H, n0 * tile, (n1 - n0) * tile,
                    p.routed_silu + static_cast<size_t>(slot) * p.moe_ffn, slot == p.top_k - 1 ? p.silu_out : nullptr,
-                   [&] { return tagged(p) || residual_to_lds<M>(p, s, c, layer, /*oproj_seen=*/true); }))
+                   [&] { return tg || residual_to_lds<M>(p, s, c, layer, /*oproj_seen=*/true); }, units, tag))
     return false;
-  publish_done(p, c, layer, ROW_ROUTED_UPGATE, 0, n1 - n0);
+  if (tg) return true;   // nothing to wait for, nothing to count
+  release_stores();
+  __syncthreads();
+  if (c.tid == 0) {
+    publish(counter_ptr(p, layer, ROW_ROUTED_UPGATE_SLOT, slot), n1 - n0);
+    publish(counter_ptr(p, layer, ROW_ROUTED_UPGATE, 0), n1 - n0);
+  }
   return true;
 }
 
@@ -445,26 +528,60 @@ __device__ __forceinline__ bool op_routed_upgate(const Params& p, Smem<M>& s, co
 template <class M>
 __device__ __forceinline__ bool op_routed_down(const Params& p, Smem<M>& s, const Ctx& c) {
   const int layer = s.inst[1], slot = s.inst[2], n0 = s.inst[4], n1 = s.inst[5], tile = s.inst[7];
+  const bool own_slot_only = s.inst[3] == 1;   // tile_M_idx: 0 in the reference's streams
   if (layer < 0 || layer >= p.num_layers) return bad_operand(p, s, c, 1);
-  if (slot < 0 || slot >= p.top_k) return bad_operand(p, s, c, 2);
+  if (slot < 0 || slot >= p.top_k || slot >= p.barrier_slots - 1) return bad_operand(p, s, c, 2);
+  if (s.inst[3] != 0 && s.inst[3] != 1) return bad_operand(p, s, c, 3);
   if (tile != kTile || n0 < 0 || n1 < n0 || n1 * tile > M::H) return bad_operand(p, s, c, 5);
+  if (tagged(p) && (p.moe_ffn & 3)) return bad_operand(p, s, c, 0);   // whole unit pairs
   // The expert is known with the top-k edge, long before the routed up/gate rows are complete: its rows are
   // asked for in between.
   int eid;
   float weight;
-  if (!routed_expert<M>(p, s, c, layer, slot, eid, weight)) return false;
+  if (!(tagged(p) ? routing_decision<M>(p, s, c, layer, slot, eid, weight) : routed_expert<M>(p, s, c, layer, slot, eid, weight))) return false;
   if (eid < 0) return bad_operand(p, s, c, 2);
   const u16* w = p.expert_down_w + (static_cast<size_t>(layer) * p.num_experts + eid) * M::H * p.moe_ffn;
   float* mine = p.routed_parts + static_cast<size_t>(slot) * M::H;
+  const bool tg = tagged(p);
+  const uint32_t tag = tag_of(s.generation, layer);
+  uint64_t* out_units = p.ws + kWsRoutedParts + slot * 2048;
   if (!down_rows(
           s, c, w, p.moe_ffn, p.moe_ffn, n0 * tile, (n1 - n0) * tile,
           [&] {
-            if (!wait_one(p, s, c, layer, ROW_ROUTED_UPGATE, 0, p.top_k * (p.moe_ffn / p.routed_tile))) return false;
+            if (tg) {
+              // the slot's silu vector from the units its up/gate workgroups announce it in: two units per poller
+              const uint64_t* units = p.ws + kWsRoutedSilu + slot * 1024;
+              uint32_t* words = reinterpret_cast<uint32_t*>(s.x);
+              for (int u = 2 * c.tid; u < p.moe_ffn / 2; u += 2 * kThreads) {
+                uint32_t a = 0, b = 0;
+                if (!poll_tagged2(units + u, tag, p.spin_limit, a, b)) {
+                  s.ctl[0] = 1;
+                  report_error(p, QMK_DEV_WAIT_TIMEOUT, c.inst_idx, c.opcode, c.tid);
+                }
+                words[u] = a;
+                words[u + 1] = b;
+              }
+              if (p.timeline != nullptr && c.tid == 0) {
+                s.t_wait = wall_clock64();
+                s.ctl[2] = 1;
+              }
+              __syncthreads();
+              return s.ctl[0] == 0;
+            }
+            const int per_slot = p.moe_ffn / p.routed_tile;
+            if (!(own_slot_only ? wait_one(p, s, c, layer, ROW_ROUTED_UPGATE_SLOT, slot, per_slot)
+                                : wait_one(p, s, c, layer, ROW_ROUTED_UPGATE, 0, p.top_k * per_slot)))
+              return false;
             stage_vector(s, c, p.routed_silu + static_cast<size_t>(slot) * p.moe_ffn, p.moe_ffn);
             return true;
           },
-          [&](int r, float dot) { st_shared_f32(mine + r, round_bf16(dot) * weight); }))
+          [&](int r, float dot) {
+            const float term = round_bf16(dot) * weight;
+            if (tg) st_tagged(out_units + r, __float_as_uint(term), tag);   // the combine step polls these
+            else st_shared_f32(mine + r, term);
+          }))
     return false;
+  if (tg) return true;
   release_stores();
   __syncthreads();
   if (c.tid < n1 - n0) publish(counter_ptr(p, layer, ROW_ROUTED_DOWN, n0 + c.tid), 1);
@@ -482,7 +599,11 @@ __device__ __forceinline__ bool op_combine(const Params& p, Smem<M>& s, const Ct
   if (layer < 0 || layer >= p.num_layers) return bad_operand(p, s, c, 1);
   if (tile != kTile || n0 < 0 || n1 < n0 || n1 * tile > M::H || 2 * (n1 - n0) > kThreads) return bad_operand(p, s, c, 3);
   const int nb = n1 - n0;
-  if (c.tid < 2 * nb) {
+  const bool tg = tagged(p);
+  const uint32_t tag = tag_of(s.generation, layer);
+  // Counters: the down projections of the instruction's blocks.  In a tagged launch the routed experts' rows are
+  // units that announce themselves (polled below), so only the shared expert's K-slice counters are waited for.
+  if (c.tid < 2 * nb && (!tg || c.tid < nb)) {
     const bool routed = c.tid >= nb;
     const int blk = n0 + (routed ? c.tid - nb : c.tid);
     // (without a shared expert shared_k_slices is 0 and that half of the pollers passes at once)
@@ -497,8 +618,6 @@ __device__ __forceinline__ bool op_combine(const Params& p, Smem<M>& s, const Ct
   }
   __syncthreads();
   if (s.ctl[0]) return false;
-  const bool tg = tagged(p);
-  const uint32_t tag = tag_of(s.generation, layer);
   const float gate = p.shared_k_slices > 0 ? ld_shared_f32(p.shared_gate) : 0.f;   // left by the layer's publishing router instruction
   constexpr int kMaxSlices = 16;   // the launcher's bound on shared_k_slices
   for (int pair = c.tid; pair < nb * tile / 2; pair += kThreads) {
@@ -508,10 +627,40 @@ __device__ __forceinline__ bool op_combine(const Params& p, Smem<M>& s, const Ct
     uint64_t rt[kMaxTopK];
 #pragma unroll
     for (int k = 0; k < kMaxSlices; ++k) st[k] = k < p.shared_k_slices ? ld_shared32(p.shared_parts + static_cast<size_t>(k) * M::H + r) : 0u;
+    if (tg) {
+      // two units per slot, all slots in flight together, looked at until every one carries this layer's tag
+      const uint64_t* units = p.ws + kWsRoutedParts + r;
+      bool have[kMaxTopK];
 #pragma unroll
-    for (int j = 0; j < kMaxTopK; ++j) rt[j] = j < p.top_k ? ld_shared64(p.routed_parts + static_cast<size_t>(j) * M::H + r) : 0ull;
+      for (int j = 0; j < kMaxTopK; ++j) have[j] = j >= p.top_k, rt[j] = 0ull;
+      for (uint32_t polls = 0;; ++polls) {
+        uint64_t a[kMaxTopK], b[kMaxTopK];
+#pragma unroll
+        for (int j = 0; j < kMaxTopK; ++j)
+          if (!have[j]) a[j] = ld_shared64(units + j * 2048), b[j] = ld_shared64(units + j * 2048 + 1);
+        bool all = true;
+#pragma unroll
+        for (int j = 0; j < kMaxTopK; ++j) {
+          if (!have[j] && static_cast<uint32_t>(a[j] >> 32) == tag && static_cast<uint32_t>(b[j] >> 32) == tag) {
+            rt[j] = (a[j] & 0xffffffffull) | (b[j] << 32);
+            have[j] = true;
+          }
+          all = all && have[j];
+        }
+        if (all) break;
+        if (polls > p.spin_limit) {
+          s.ctl[0] = 1;
+          report_error(p, QMK_DEV_WAIT_TIMEOUT, c.inst_idx, c.opcode, c.tid);
+          break;
+        }
+        __builtin_amdgcn_s_sleep(2);
+      }
+    } else {
+#pragma unroll
+      for (int j = 0; j < kMaxTopK; ++j) rt[j] = j < p.top_k ? ld_shared64(p.routed_parts + static_cast<size_t>(j) * M::H + r) : 0ull;
+    }
     // Tagged launch: the unit the O-projection announced this pair in.  Every up/gate workgroup has seen its
-    // tag, and this instruction follows them through the counters of the down projections: no polling.
+    // tag, and this instruction follows them through the down projections: no polling.
     const uint32_t old = tg ? static_cast<uint32_t>(ld_shared64(p.ws + kWsHiddenMid + r / 2)) : ld_shared32(p.hidden + r);
     float sh0 = 0.f, sh1 = 0.f;
 #pragma unroll
@@ -536,6 +685,10 @@ __device__ __forceinline__ bool op_combine(const Params& p, Smem<M>& s, const Ct
     if (p.shared_k_slices > 0) st_shared32(p.shared_out + r, static_cast<uint32_t>(f2bf(sh0)) | (static_cast<uint32_t>(f2bf(sh1)) << 16));
     st_shared_f32(p.routed_out_f32 + r, 0.f);
     st_shared_f32(p.routed_out_f32 + r + 1, 0.f);
+  }
+  if (tg) {   // uniform: a poller that gave up has said so
+    __syncthreads();
+    if (s.ctl[0]) return false;
   }
   publish_done(p, c, layer, ROW_COMBINE, 0, nb);
   return true;

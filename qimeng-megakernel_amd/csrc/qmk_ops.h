@@ -65,7 +65,7 @@ struct Smem {
   int32_t wave_idx[kWaves];             // per-wave candidates on their way to best_val/best_idx
   float red[kWaves];
   alignas(16) u16 x[M::F];              // activation vector handed to the GEMV lanes
-  float res[kResSlots];                 // per-row GEMV results awaiting the epilogue pass
+  alignas(16) float res[kResSlots];     // per-row GEMV results awaiting the epilogue pass
   float merge[kWaves][M::GQA][M::D + 4];  // attention state per wave and head: acc[D], m, l
   unsigned long long t_wait;            // timeline: when the last counter wait finished
   unsigned long long stamps[4];         // timeline: op-specific intermediate timestamps
@@ -975,41 +975,55 @@ __device__ bool op_oproj_residual(const Params& p, Smem<M>& s, const Ctx& c, Car
     const int P = self_merge;
     if (P < 1 || P > kMaxSelfMerge || P > p.max_splits) return bad_operand(p, s, c, 5);  // no list to fit: any fan-out the workspaces hold
     if (!wg_wait_all(p, s, c, layer, ROW_REDUCE, 0, M::NKV * P)) return false;
+    constexpr int kItems = AW / (kThreads * 4);
+    const float* lse[kItems];
+    const float* part[kItems];
+    float mx[kItems], den[kItems], n0[kItems], n1[kItems], n2[kItems], n3[kItems];
 #pragma unroll
-    for (int k = 0; k < AW / (kThreads * 4); ++k) {
+    for (int k = 0; k < kItems; ++k) {
       const int item = c.tid + k * kThreads;
       const int h = item / (M::D / 4), d0 = 4 * (item % (M::D / 4));
-      const float* lse = p.attn_lse + static_cast<size_t>(h) * p.max_splits;
-      const float* part = p.attn_partial + static_cast<size_t>(h) * p.max_splits * M::D + d0;
-      float mx = -INFINITY, den = 0.f, n0 = 0.f, n1 = 0.f, n2 = 0.f, n3 = 0.f;
-      for (int j0 = 0; j0 < P; j0 += 4) {   // four partials per round, loads first
-        float e[4];
-        v4u o[4];
+      lse[k] = p.attn_lse + static_cast<size_t>(h) * p.max_splits;
+      part[k] = p.attn_partial + static_cast<size_t>(h) * p.max_splits * M::D + d0;
+      mx[k] = -INFINITY;
+      den[k] = n0[k] = n1[k] = n2[k] = n3[k] = 0.f;
+    }
+    for (int j0 = 0; j0 < P; j0 += 4) {   // four partials of every item per round, all loads first
+      float e[kItems][4];
+      v4u o[kItems][4];
+#pragma unroll
+      for (int k = 0; k < kItems; ++k)
 #pragma unroll
         for (int q = 0; q < 4; ++q) {
           const int j = min(j0 + q, P - 1);
-          e[q] = (j0 + q < P) ? ld_shared_f32(lse + j) : -INFINITY;
-          o[q] = ld_shared128(part + static_cast<size_t>(j) * M::D);
+          e[k][q] = (j0 + q < P) ? ld_shared_f32(lse[k] + j) : -INFINITY;
+          o[k][q] = ld_shared128(part[k] + static_cast<size_t>(j) * M::D);
         }
-        float mn = mx;
 #pragma unroll
-        for (int q = 0; q < 4; ++q) mn = fmaxf(mn, e[q]);
-        const float rescale = (mx == -INFINITY) ? 0.f : exp2_fast(mx - mn);
-        den *= rescale; n0 *= rescale; n1 *= rescale; n2 *= rescale; n3 *= rescale;
+      for (int k = 0; k < kItems; ++k) {
+        float mn = mx[k];
+#pragma unroll
+        for (int q = 0; q < 4; ++q) mn = fmaxf(mn, e[k][q]);
+        const float rescale = (mx[k] == -INFINITY) ? 0.f : exp2_fast(mx[k] - mn);
+        den[k] *= rescale; n0[k] *= rescale; n1[k] *= rescale; n2[k] *= rescale; n3[k] *= rescale;
 #pragma unroll
         for (int q = 0; q < 4; ++q) {
-          const float f = (e[q] == -INFINITY) ? 0.f : exp2_fast(e[q] - mn);
-          den += f;
-          n0 = __builtin_fmaf(__uint_as_float(o[q].x), f, n0);
-          n1 = __builtin_fmaf(__uint_as_float(o[q].y), f, n1);
-          n2 = __builtin_fmaf(__uint_as_float(o[q].z), f, n2);
-          n3 = __builtin_fmaf(__uint_as_float(o[q].w), f, n3);
+          const float f = (e[k][q] == -INFINITY) ? 0.f : exp2_fast(e[k][q] - mn);
+          den[k] += f;
+          n0[k] = __builtin_fmaf(__uint_as_float(o[k][q].x), f, n0[k]);
+          n1[k] = __builtin_fmaf(__uint_as_float(o[k][q].y), f, n1[k]);
+          n2[k] = __builtin_fmaf(__uint_as_float(o[k][q].z), f, n2[k]);
+          n3[k] = __builtin_fmaf(__uint_as_float(o[k][q].w), f, n3[k]);
         }
-        mx = mn;
+        mx[k] = mn;
       }
-      const float inv = den > 0.f ? 1.0f / den : 0.f;
-      const uint32_t lo = static_cast<uint32_t>(f2bf(n0 * inv)) | (static_cast<uint32_t>(f2bf(n1 * inv)) << 16);
-      const uint32_t hi = static_cast<uint32_t>(f2bf(n2 * inv)) | (static_cast<uint32_t>(f2bf(n3 * inv)) << 16);
+    }
+#pragma unroll
+    for (int k = 0; k < kItems; ++k) {
+      const int item = c.tid + k * kThreads;
+      const float inv = den[k] > 0.f ? 1.0f / den[k] : 0.f;
+      const uint32_t lo = static_cast<uint32_t>(f2bf(n0[k] * inv)) | (static_cast<uint32_t>(f2bf(n1[k] * inv)) << 16);
+      const uint32_t hi = static_cast<uint32_t>(f2bf(n2[k] * inv)) | (static_cast<uint32_t>(f2bf(n3[k] * inv)) << 16);
       *reinterpret_cast<uint2*>(s.x + item * 4) = make_uint2(lo, hi);
       if (nstart == 0) {  // one workgroup also leaves attn_out in memory, as the reference does
         st_shared32(p.attn_out + item * 4, lo);

@@ -33,7 +33,7 @@ def decode(globs: Any, prompt_ids: torch.Tensor, max_new_tokens: int, *, mk: Any
         raise ValueError("prompt_len + max_new_tokens exceeds the KV cache capacity")
     mk = mk or _mk_kernel.get_mk()
     globs.instructions = None
-    _mk_kernel.build(globs)
+    _mk_kernel.build(globs, mk)
     out = torch.zeros(T + max(max_new_tokens, 1), dtype=torch.long, device=device)
     out[:T] = prompt_ids.to(device)
     for pos in range(T):

@@ -21,7 +21,12 @@ row    producer                       slot                        final count
 11     12 routed up/gate + SiLU       0                           top_k * moe_intermediate / 16
 12     13 routed down                 hidden block                top_k
 13     14 combine + commit            0                           hidden / 16
+14     12 routed up/gate (this build)  expert slot                 moe_intermediate / tile
 =====  =============================  ==========================  ================================
+
+Row 14 is this build's: the reference counts the routed up/gate tiles of all slots on one word (row 11), and a routed
+down projection whose ``tile_M_idx`` is 1 (0 in the reference's streams) waits for the row-14 word of its own slot
+instead.  The last word of layer 0's row 14 is the kernel's retirement count.
 """
 from __future__ import annotations
 

@@ -58,6 +58,9 @@ class MoeScheduler:
     merge_in_oproj: bool = False       # every O-projection instruction merges all partials itself: no reduction instructions
     router_span: int = 1               # experts per router instruction
     placed: bool = False               # queues() places the instructions of a layer by role instead of dealing them
+    down_per_slot: bool = False        # a routed down projection waits for its own slot's up/gate tiles only (tile_M_idx = 1)
+    topk_late: bool = False            # placed streams for tagged launches: the consumers take the routing decision themselves,
+                                       # the top-k instruction runs behind its queue's up/gate tiles (it only reports the routing)
 
     def qkvproj(self, layer: int) -> list[Instruction]:
         tiles = _ceil_div(self.shape.qkv_out_dim, TILE_N_GRANULARITY)
@@ -79,7 +82,8 @@ class MoeScheduler:
 
     def oproj(self, layer: int) -> list[Instruction]:
         merges = self.num_partials if self.merge_in_oproj else 0
-        return [OProj_GEMV_Residual(layer, 0, lo, hi, merges) for lo, hi in _spans(self.shape.num_hidden_blocks, self.sm_count)]
+        return [OProj_GEMV_Residual(layer, 0, lo, hi, merges, tile_N_granularity=self.shape.oproj_tile)
+                for lo, hi in _spans(self.shape.num_oproj_blocks, self.sm_count)]
 
     def router_gemv(self, layer: int) -> list[Instruction]:
         """One instruction per expert: the top-k waits for all of them."""
@@ -122,7 +126,7 @@ class MoeScheduler:
 
     def routed_downproj(self, layer: int) -> list[Instruction]:
         per_expert = max(1, self.sm_count // self.shape.num_experts_per_tok)
-        return [RoutedExpert_DownProj(layer, slot, 0, lo, hi)
+        return [RoutedExpert_DownProj(layer, slot, 1 if self.down_per_slot else 0, lo, hi)
                 for slot in range(self.shape.num_experts_per_tok)
                 for lo, hi in _spans(self.shape.num_hidden_blocks, per_expert)]
 
@@ -156,8 +160,8 @@ class MoeScheduler:
         n = self.sm_count
         side = len(self.router_gemv(0)) + 1
         if side * 4 > n:                       # a device too small to set queues aside
-            return list(range(n)), list(range(n)), min(n, self.shape.num_hidden_blocks)
-        return list(range(n - side)), list(range(n - side, n)), min(n - side, self.shape.num_hidden_blocks)
+            return list(range(n)), list(range(n)), min(n, self.shape.num_oproj_blocks)
+        return list(range(n - side)), list(range(n - side, n)), min(n - side, self.shape.num_oproj_blocks)
 
     @staticmethod
     def _weighted_sizes(tiles: int, weights: Sequence[int]) -> list[int]:
@@ -218,16 +222,21 @@ class MoeScheduler:
         spread(self.qkvproj(layer), everyone)
         spread(self.attention_split_kv(layer), everyone)
         spread(self.attention_reduction(layer), everyone)
-        spread(self.oproj(layer), main)
+        # without a shared expert nothing runs beside the router: its queues take O-projection rows like everybody else
+        spread(self.oproj(layer), main if self.shape.has_shared_expert else everyone)
         router = self.router_gemv(layer)
         spread(router, side)
-        out[side[len(router) % len(side)]] += self.router_softmax_topk(layer)
+        topk_queue = side[len(router) % len(side)]
+        if not self.topk_late:
+            out[topk_queue] += self.router_softmax_topk(layer)
         for queue, ins in self._placed_shared_upgate(layer):
             out[queue].append(ins)
         if not self.interleave_experts:
             spread(self.shared_downproj(layer), everyone)
         for queue, ins in self._placed_routed_upgate(layer):
             out[queue].append(ins)
+        if self.topk_late:    # behind the queue's up/gate tiles, where it would otherwise wait for its slot's silu vector
+            out[topk_queue] += self.router_softmax_topk(layer)
         if self.interleave_experts:
             spread(self.shared_downproj(layer), everyone)
         spread(self.routed_downproj(layer), everyone)

@@ -66,7 +66,7 @@ class QmkMoeArgs(ctypes.Structure):
                                    "shared_k_slices")]
         + [("attn_scale", ctypes.c_float), ("rms_norm_eps", ctypes.c_float), ("timeline", _P), ("stream", _P), ("workspace", _P),
            ("workspace_bytes", ctypes.c_uint64)]
-        + [(name, _P) for name in _QWEN3_EXTRA] + [("norm_topk_prob", _I), ("routed_upgate_tile", _I)]
+        + [(name, _P) for name in _QWEN3_EXTRA] + [("norm_topk_prob", _I), ("routed_upgate_tile", _I), ("oproj_tile", _I), ("reserved", _I)]
     )
 
 
@@ -190,7 +190,7 @@ class MoeMegaKernel:
         a.max_seq_len, a.max_splits, a.vocab_size, a.rope_rows = S, P, V, int(tensors["rope_cos"].shape[0])
         a.num_experts, a.top_k, a.shared_ffn, a.moe_ffn = E, k, Fs, Fm
         a.shared_k_slices = int(s.num_downproj_split_k_shared) if s.has_shared_expert else 0
-        a.norm_topk_prob, a.routed_upgate_tile = int(bool(s.norm_topk_prob)), int(s.routed_upgate_tile)
+        a.norm_topk_prob, a.routed_upgate_tile, a.oproj_tile = int(bool(s.norm_topk_prob)), int(s.routed_upgate_tile), int(s.oproj_tile)
         nbytes = int(self._lib.qmk_moe_workspace_bytes(k, a.shared_k_slices))
         if nbytes == 0:
             raise ValueError(f"top_k {k} / {a.shared_k_slices} K slices are outside what the kernel supports")
@@ -246,7 +246,7 @@ def call_mk(globs: Globals, mk: Any) -> None:
     """One decode step with the current ``Globals`` (builds the instruction tensor on first use)."""
     s = QwenMoeConfig.shape()
     if globs.instructions is None:
-        build(globs)
+        build(globs, mk)
     unused = globs.hidden_states          # the three dense-MLP positions of the reference's argument list
     g = globs
     mk(g.instructions, g.hidden_states, g.normed_hidden_states, g.q_post_rope, g.k_cache, g.v_cache, g.attn_out,
@@ -260,21 +260,30 @@ def call_mk(globs: Globals, mk: Any) -> None:
        g.position_id if g.position_id is not None else 0, 1.0 / math.sqrt(s.head_dim), float(s.rms_norm_eps))
 
 
-def mi355x_scheduler(shape: Any = None) -> _scheduler.MoeScheduler:
+def mi355x_scheduler(shape: Any = None, *, tagged: bool = True) -> _scheduler.MoeScheduler:
     """One queue per CU; both up/gate phases ahead of both down projections; the instructions of a layer placed
     by role (the queues of the router and the top-k take no shared up/gate rows); eight experts per router
-    instruction; at most 8 split-KV partials per KV head, merged by the O-projection workgroups themselves
-    (measured at contexts up to 263: 753 tok/s, against 728 with 16 partials and 719 with the merge by the last
-    split-KV arrival)."""
+    instruction; few split-KV partials per KV head, merged by the O-projection workgroups themselves
+    (Qwen1.5 shape, contexts up to 263: 753 tok/s with 8 partials, against 728 with 16 and 719 with the merge by the
+    last split-KV arrival; Qwen3-30B-A3B shape, 4 KV heads, contexts up to 528: 2 partials); a routed down projection
+    waits for its own slot only.  ``tagged``: the stream is for launches with QMK_FLAG_TAGGED, where the consumers of
+    the routing decision take it themselves and the top-k instruction runs late in its queue; a launch on counters
+    needs the stream built with ``tagged=False``, whose top-k instruction stands in front of its consumers."""
     from .model_config import num_partials_for
 
     shape = shape or QwenMoeConfig.shape()
-    return _scheduler.MoeScheduler(shape, MI355X_QUEUES, min(8, num_partials_for(MI355X_QUEUES, shape)), interleave_experts=True,
-                                   merge_in_oproj=True, router_span=8, placed=True)
+    partials = min(8 if shape.num_key_value_heads > 4 else 2, num_partials_for(MI355X_QUEUES, shape))
+    return _scheduler.MoeScheduler(shape, MI355X_QUEUES, partials, interleave_experts=True, merge_in_oproj=True, router_span=8,
+                                   placed=True, down_per_slot=True, topk_late=tagged)
 
 
-def build(globs: Globals) -> torch.Tensor:
-    sched = mi355x_scheduler()
+def build(globs: Globals, mk: Any = None) -> torch.Tensor:
+    """The instruction tensor of a request; ``mk``: the callable it is built for (a launch on counters gets a stream
+    whose top-k instruction precedes its consumers)."""
+    tagged = True
+    if isinstance(mk, MoeMegaKernel):
+        tagged = mk.tagged and mk.reset_barriers and QwenMoeConfig.shape().num_hidden_layers <= 63
+    sched = mi355x_scheduler(tagged=tagged)
     if sched.num_partials > int(globs.attn_lse_intermediates.shape[-1]):
         raise ValueError("attn_lse_intermediates has fewer partial slots than the schedule's split-KV fan-out")
     return tensorize_instructions(globs, sched.queues())

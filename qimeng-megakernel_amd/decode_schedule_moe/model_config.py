@@ -33,6 +33,7 @@ class MoeShape:
     tile_n_granularity: int = 16
     num_downproj_split_k_shared: int = 4
     routed_upgate_tile: int = 16            # outputs per tile of the routed up/gate instructions (16, or 8)
+    oproj_tile: int = 16                    # rows per tile of the O-projection instructions (16, or 8: one tile per queue of 256)
 
     @property
     def has_shared_expert(self) -> bool:
@@ -53,6 +54,10 @@ class MoeShape:
     @property
     def num_moe_intermediate_blocks(self) -> int:
         return self.moe_intermediate_size // self.tile_n_granularity
+
+    @property
+    def num_oproj_blocks(self) -> int:
+        return self.hidden_size // self.oproj_tile
 
     @property
     def num_routed_upgate_blocks(self) -> int:
@@ -93,7 +98,7 @@ QWEN1_5_MOE_A2_7B = MoeShape()
 QWEN3_30B_A3B = MoeShape(
     num_hidden_layers=48, num_attention_heads=32, num_key_value_heads=4, intermediate_size=0, moe_intermediate_size=768,
     num_experts=128, num_experts_per_tok=8, norm_topk_prob=True, qkv_bias=False, qk_norm=True, attn_reduction_size=8,
-    num_downproj_split_k_shared=0, routed_upgate_tile=8,
+    num_downproj_split_k_shared=0, routed_upgate_tile=8, oproj_tile=8,
 )
 
 MAX_OPCODE = 14

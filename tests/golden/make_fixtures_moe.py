@@ -140,7 +140,10 @@ def main() -> None:
             ref_ops.fused_rms_lmhead_gemv(routes["ref_fused"]); my_fused.lm_head(routes["my_fused"])
             for a, b, names in (("ref_vm", "my_vm", BUFFERS + VM_ONLY), ("ref_fused", "my_fused", BUFFERS + FUSED_ONLY)):
                 for name in names:
-                    assert same(getattr(routes[a], name), getattr(routes[b], name)), f"step {step}: {a} and {b} differ in {name}"
+                    x, y = getattr(routes[a], name), getattr(routes[b], name)
+                    if name == "barriers":      # row 14 is this repository's own (per-slot counts): the reference's fourteen rows
+                        x, y = x[:, :14], y[:, :14]
+                    assert same(x, y), f"step {step}: {a} and {b} differ in {name}"
             for name in ("my_vm", "my_fused"):
                 g = routes[name]
                 top = g.logits.float().topk(4)

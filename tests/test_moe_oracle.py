@@ -185,9 +185,16 @@ def test_placed_stream_is_the_same_instructions_by_role():
     from qimeng_megakernel_amd.decode_schedule_moe.mk_kernel import mi355x_scheduler
     from qimeng_megakernel_amd.decode_schedule_moe.model_config import QWEN1_5_MOE_A2_7B as FULL
 
-    sched = mi355x_scheduler(FULL)
+    sched = mi355x_scheduler(FULL, tagged=False)    # the stream for launches on counters: every queue in dependency order
     queues = sched.queues()
     assert len(queues) == 256 and sched.placed
+    # the stream for tagged launches differs in one thing: the top-k instruction stands behind its queue's routed up/gate tiles
+    late = mi355x_scheduler(FULL).queues()
+    for q, ql in zip(queues, late):
+        assert sorted(tuple(i.padded()) for i in q) == sorted(tuple(i.padded()) for i in ql)
+        if any(i.opcode() == 9 for i in ql):
+            ops = [i.opcode() for i in ql if i.opcode() != 7 and i.padded()[1] == 0]
+            assert ops.index(9) == max(k for k, o in enumerate(ops) if o == 12) + 1
     key = lambda ins: tuple(ins.padded())
     assert Counter(key(i) for q in queues for i in q) == Counter(key(i) for i in sched.instruction_list())
     phase = {1: 0, 2: 1, 3: 2, 4: 3, 8: 4, 9: 5, 10: 6, 12: 7, 11: 8, 13: 9, 14: 10, 7: 11}
