@@ -382,7 +382,12 @@ typedef struct QmkMoeArgs {
   int32_t oproj_tile;              /* rows per tile of opcode 4 (its tile_N_granularity word): 16 (0 = 16), or 8, which
                                       gives each of 256 queues one tile of the 2048 rows; fixes the final value of the
                                       O-projection counter (H / oproj_tile)                                          */
-  int32_t reserved;                /* 0 */
+  int32_t local_routing;           /* QMK_FLAG_TAGGED only.  0: the routed ops (12, 13) wait for the experts and weights that
+                                      opcode 9 announces.  1: they take the routing decision themselves from the router's
+                                      logits (the same function of the same values: the same experts and weights), and
+                                      opcode 9 only reports it — for streams in which nothing runs beside the router and the
+                                      top-k (no shared expert), where that hand-over would leave the whole device waiting;
+                                      such a stream may place opcode 9 behind its queue's routed up/gate tiles          */
 } QmkMoeArgs;
 
 int qmk_decode_step_moe(const QmkMoeArgs* args);

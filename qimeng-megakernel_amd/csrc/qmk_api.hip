@@ -638,7 +638,7 @@ int decode_step_moe(const QmkMoeArgs* a) {
   if ((routed_tile != 8 && routed_tile != 16) || a->moe_ffn % routed_tile) return QMK_ERR_SHAPE;
   if (a->norm_topk_prob != 0 && a->norm_topk_prob != 1) return QMK_ERR_SHAPE;
   const int oproj_tile = a->oproj_tile == 0 ? moe::kTile : a->oproj_tile;
-  if ((oproj_tile != 8 && oproj_tile != 16) || a->reserved != 0) return QMK_ERR_SHAPE;
+  if ((oproj_tile != 8 && oproj_tile != 16) || (a->local_routing != 0 && a->local_routing != 1)) return QMK_ERR_SHAPE;
   if (a->flags & ~(QMK_FLAG_KEEP_BARRIERS | QMK_FLAG_TAGGED)) return QMK_ERR_SHAPE;
   // tagged units carry the launch count, which the retiring launch advances, and six bits of layer
   if ((a->flags & QMK_FLAG_TAGGED) && ((a->flags & QMK_FLAG_KEEP_BARRIERS) || a->num_layers > 63)) return QMK_ERR_SHAPE;
@@ -720,6 +720,7 @@ int decode_step_moe(const QmkMoeArgs* a) {
   p.shared_k_slices = a->shared_k_slices;
   p.norm_topk = a->norm_topk_prob;
   p.routed_tile = routed_tile;
+  p.local_routing = a->local_routing;
 
   hipLaunchKernelGGL(decode_megakernel_moe<M>, dim3(a->num_queues), dim3(kThreads), 0, static_cast<hipStream_t>(a->stream), p);
   return hipGetLastError() == hipSuccess ? QMK_OK : QMK_ERR_LAUNCH;

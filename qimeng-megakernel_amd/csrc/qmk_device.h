@@ -119,6 +119,7 @@ struct Params {
   int32_t shared_k_slices;
   int32_t norm_topk;             // 1: the top-k weights are divided by their sum
   int32_t routed_tile;           // outputs per tile of the routed up/gate instructions (16, or 8)
+  int32_t local_routing;         // tagged launches: 1 = the routed ops take the routing decision themselves from the logits
 };
 
 // ---------------------------------------------------------------- bf16 ----

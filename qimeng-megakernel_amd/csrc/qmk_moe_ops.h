@@ -288,6 +288,10 @@ __device__ __forceinline__ bool op_topk(const Params& p, Smem<M>& s, const Ctx& 
       const float w = p.norm_topk ? picked[j] / total : picked[j];
       __hip_atomic_store(p.expert_indices + j, static_cast<long long>(idx), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
       st_shared_f32(p.expert_weights + j, w);
+      if (tg && !p.local_routing) {   // the routed ops poll these: one trip, no drain in between
+        st_tagged(p.ws + kWsExperts + j, static_cast<uint32_t>(idx), tag_of(s.generation, layer));
+        st_tagged(p.ws + kWsExperts + kMaxTopK + j, __float_as_uint(w), tag_of(s.generation, layer));
+      }
     }
   }
   if (tg) {
@@ -503,7 +507,7 @@ __device__ __forceinline__ bool op_routed_upgate(const Params& p, Smem<M>& s, co
   float unused;
   // A tagged launch has the normalised row long before the experts are known.
   if (tg && !residual_to_lds<M>(p, s, c, layer)) return false;
-  if (!(tg ? routing_decision<M>(p, s, c, layer, slot, eid, unused) : routed_expert<M>(p, s, c, layer, slot, eid, unused))) return false;
+  if (!(tg && p.local_routing ? routing_decision<M>(p, s, c, layer, slot, eid, unused) : routed_expert<M>(p, s, c, layer, slot, eid, unused))) return false;
   if (eid < 0) return bad_operand(p, s, c, 2);
   const u16* w = p.expert_gate_up_w + (static_cast<size_t>(layer) * p.num_experts + eid) * 2 * p.moe_ffn * M::H;
   // tagged launch: the slot's down projections poll the silu values as units of their own
@@ -538,7 +542,7 @@ __device__ __forceinline__ bool op_routed_down(const Params& p, Smem<M>& s, cons
   // asked for in between.
   int eid;
   float weight;
-  if (!(tagged(p) ? routing_decision<M>(p, s, c, layer, slot, eid, weight) : routed_expert<M>(p, s, c, layer, slot, eid, weight))) return false;
+  if (!(tagged(p) && p.local_routing ? routing_decision<M>(p, s, c, layer, slot, eid, weight) : routed_expert<M>(p, s, c, layer, slot, eid, weight))) return false;
   if (eid < 0) return bad_operand(p, s, c, 2);
   const u16* w = p.expert_down_w + (static_cast<size_t>(layer) * p.num_experts + eid) * M::H * p.moe_ffn;
   float* mine = p.routed_parts + static_cast<size_t>(slot) * M::H;

@@ -66,7 +66,7 @@ class QmkMoeArgs(ctypes.Structure):
                                    "shared_k_slices")]
         + [("attn_scale", ctypes.c_float), ("rms_norm_eps", ctypes.c_float), ("timeline", _P), ("stream", _P), ("workspace", _P),
            ("workspace_bytes", ctypes.c_uint64)]
-        + [(name, _P) for name in _QWEN3_EXTRA] + [("norm_topk_prob", _I), ("routed_upgate_tile", _I), ("oproj_tile", _I), ("reserved", _I)]
+        + [(name, _P) for name in _QWEN3_EXTRA] + [("norm_topk_prob", _I), ("routed_upgate_tile", _I), ("oproj_tile", _I), ("local_routing", _I)]
     )
 
 
@@ -77,8 +77,12 @@ class MoeMegaKernel:
     as self-announcing tagged units instead of through counters, as on the dense route; whole steps only, so it
     applies when the kernel also clears its counters.  Same values bit for bit, 705 against 603 tok/s."""
 
-    def __init__(self, lib: ctypes.CDLL, *, reset_barriers: bool = True, spin_limit: int = 0, tagged: bool = True):
+    def __init__(self, lib: ctypes.CDLL, *, reset_barriers: bool = True, spin_limit: int = 0, tagged: bool = True,
+                 local_routing: bool | None = None):
         self._lib = lib
+        #: tagged launches: the routed ops take the routing decision themselves (None: where the model has no shared expert,
+        #: i.e. where nothing runs beside the router and the top-k)
+        self.local_routing = local_routing
         self.reset_barriers = reset_barriers
         self.tagged = tagged
         self.spin_limit = int(spin_limit)
@@ -112,7 +116,8 @@ class MoeMegaKernel:
 
     def with_options(self, **kw: Any) -> "MoeMegaKernel":
         other = MoeMegaKernel(self._lib, reset_barriers=kw.pop("reset_barriers", self.reset_barriers),
-                              spin_limit=kw.pop("spin_limit", self.spin_limit), tagged=kw.pop("tagged", self.tagged))
+                              spin_limit=kw.pop("spin_limit", self.spin_limit), tagged=kw.pop("tagged", self.tagged),
+                              local_routing=kw.pop("local_routing", self.local_routing))
         if kw:
             raise TypeError(f"unknown options {sorted(kw)}")
         return other
@@ -191,6 +196,7 @@ class MoeMegaKernel:
         a.num_experts, a.top_k, a.shared_ffn, a.moe_ffn = E, k, Fs, Fm
         a.shared_k_slices = int(s.num_downproj_split_k_shared) if s.has_shared_expert else 0
         a.norm_topk_prob, a.routed_upgate_tile, a.oproj_tile = int(bool(s.norm_topk_prob)), int(s.routed_upgate_tile), int(s.oproj_tile)
+        a.local_routing = int(self.local_routing if self.local_routing is not None else not s.has_shared_expert)
         nbytes = int(self._lib.qmk_moe_workspace_bytes(k, a.shared_k_slices))
         if nbytes == 0:
             raise ValueError(f"top_k {k} / {a.shared_k_slices} K slices are outside what the kernel supports")
@@ -225,7 +231,8 @@ class MoeMegaKernel:
             raise RuntimeError(f"qmk_decode_step_moe failed with {rc}: {self.error_string(rc)}")
 
 
-def get_mk(mk_dir: Path | None = None, *, reset_barriers: bool = True, spin_limit: int = 0, tagged: bool = True) -> MoeMegaKernel:
+def get_mk(mk_dir: Path | None = None, *, reset_barriers: bool = True, spin_limit: int = 0, tagged: bool = True,
+           local_routing: bool | None = None) -> MoeMegaKernel:
     """Return the ``mk`` callable of the MoE route bound to the prebuilt library in ``mk_dir``."""
     root = (_single._default_mk_dir() if mk_dir is None else Path(mk_dir)).resolve()
     lib = _single._LIB_CACHE.get(root)
@@ -239,7 +246,7 @@ def get_mk(mk_dir: Path | None = None, *, reset_barriers: bool = True, spin_limi
     lib.qmk_decode_step_moe.restype = ctypes.c_int
     lib.qmk_moe_workspace_bytes.argtypes = [ctypes.c_int, ctypes.c_int]
     lib.qmk_moe_workspace_bytes.restype = ctypes.c_uint64
-    return MoeMegaKernel(lib, reset_barriers=reset_barriers, spin_limit=spin_limit, tagged=tagged)
+    return MoeMegaKernel(lib, reset_barriers=reset_barriers, spin_limit=spin_limit, tagged=tagged, local_routing=local_routing)
 
 
 def call_mk(globs: Globals, mk: Any) -> None:
@@ -274,7 +281,7 @@ def mi355x_scheduler(shape: Any = None, *, tagged: bool = True) -> _scheduler.Mo
     shape = shape or QwenMoeConfig.shape()
     partials = min(8 if shape.num_key_value_heads > 4 else 2, num_partials_for(MI355X_QUEUES, shape))
     return _scheduler.MoeScheduler(shape, MI355X_QUEUES, partials, interleave_experts=True, merge_in_oproj=True, router_span=8,
-                                   placed=True, down_per_slot=True, topk_late=tagged)
+                                   placed=True, down_per_slot=True, topk_late=tagged and not shape.has_shared_expert)
 
 
 def build(globs: Globals, mk: Any = None) -> torch.Tensor:
@@ -282,7 +289,7 @@ def build(globs: Globals, mk: Any = None) -> torch.Tensor:
     whose top-k instruction precedes its consumers)."""
     tagged = True
     if isinstance(mk, MoeMegaKernel):
-        tagged = mk.tagged and mk.reset_barriers and QwenMoeConfig.shape().num_hidden_layers <= 63
+        tagged = mk.tagged and mk.reset_barriers and QwenMoeConfig.shape().num_hidden_layers <= 63 and mk.local_routing is not False
     sched = mi355x_scheduler(tagged=tagged)
     if sched.num_partials > int(globs.attn_lse_intermediates.shape[-1]):
         raise ValueError("attn_lse_intermediates has fewer partial slots than the schedule's split-KV fan-out")

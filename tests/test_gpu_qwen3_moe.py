@@ -229,6 +229,49 @@ def test_teacher_forced_request_against_the_fused_oracle(weights):
     rel_close(gpu.k_cache[:, 0, :steps], cpu.k_cache[:, 0, :steps], rel=4e-2, name="k_cache")
 
 
+def test_request_of_the_reference_fixture():
+    """The request recorded from the reference's own functions put together (tests/golden/make_fixtures_qwen3_moe.py),
+    teacher-forced through call_mk: the last layer's routing, the top-4 logits within 8 bf16 ulps, the greedy token
+    wherever the reference's margin is clear.  A routing decision may flip only where the reference has the two
+    experts within 3 % of each other."""
+    fix = json.loads((GOLDEN / "qwen3_moe_reduced_seed0.json").read_text())
+    shape = dataclasses.replace(QWEN3_30B_A3B, **fix["shape"])
+    QwenMoeConfig.set_shape(shape)
+    w = synthetic.random_moe_weights(shape, fix["seed"], fix["kv_capacity"])
+    g = synthetic.build_moe_globals(w, shape, fix["kv_capacity"], "cuda:0", max_partials=fix["max_partials"])
+    gen = torch.Generator().manual_seed(fix["seed"] + 1)
+    g.k_cache.copy_(torch.randn(g.k_cache.shape, generator=gen).bfloat16())
+    g.v_cache.copy_(torch.randn(g.v_cache.shape, generator=gen).bfloat16())
+    mk = mk_kernel.get_mk(spin_limit=1 << 18)
+    token, agree = fix["start_token"], 0
+    for step, want in enumerate(fix["steps"]):
+        g.position_id = want["position"]
+        g.hidden_states.copy_(g.embed_tokens[token])
+        mk_kernel.call_mk(g, mk)
+        mk.check()
+        assert int(g.barriers.abs().sum()) == 0, "the last workgroup clears the counters"
+        got_experts, ref_experts = g.expert_indices.tolist(), want["experts_per_layer"][-1]
+        if sorted(got_experts) != sorted(ref_experts):
+            probs = torch.softmax(g.router_logits_buf.cpu(), dim=-1)
+            disputed = sorted(set(got_experts) ^ set(ref_experts))
+            assert len(disputed) == 2 and abs(float(probs[disputed[0]] - probs[disputed[1]])) <= 0.03 * float(probs[disputed].max()), (step, disputed)
+        else:
+            ref_w = dict(zip(ref_experts, want["weights_per_layer"][-1]))
+            assert torch.allclose(g.expert_weights.cpu(), torch.tensor([ref_w[e] for e in got_experts]), rtol=2e-2)
+            assert abs(float(g.expert_weights.sum()) - 1.0) < 1e-6
+        got = g.logits[torch.tensor(want["top_ids"], device=g.logits.device)].view(torch.int16).to(torch.int32).cpu()
+        ref = torch.tensor(want["top_bits"], dtype=torch.int32)
+        ref = torch.where(ref >= 32768, ref - 65536, ref)
+        assert int((got - ref).abs().max()) <= 8, (step, got.tolist(), ref.tolist())
+        mine = int(g.logits.float().argmax())
+        if mine == want["token"]:
+            agree += 1
+        else:
+            assert int(ref[0] - ref[1]) <= 8, f"step {step}: different pick at a clear margin"
+        token = want["token"]
+    assert mk._tagged and agree >= len(fix["steps"]) - 1
+
+
 def test_tagged_and_counter_modes_agree_bit_for_bit(weights):
     out = []
     for tagged in (False, True):

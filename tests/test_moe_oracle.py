@@ -189,8 +189,9 @@ def test_placed_stream_is_the_same_instructions_by_role():
     queues = sched.queues()
     assert len(queues) == 256 and sched.placed
     # the stream for tagged launches differs in one thing: the top-k instruction stands behind its queue's routed up/gate tiles
-    late = mi355x_scheduler(FULL).queues()
-    for q, ql in zip(queues, late):
+    from qimeng_megakernel_amd.decode_schedule_moe.model_config import QWEN3_30B_A3B
+    assert [tuple(i.padded()) for q in mi355x_scheduler(FULL).queues() for i in q] == [tuple(i.padded()) for q in queues for i in q]   # a shared expert: no late top-k
+    for q, ql in zip(mi355x_scheduler(QWEN3_30B_A3B, tagged=False).queues(1), mi355x_scheduler(QWEN3_30B_A3B).queues(1)):
         assert sorted(tuple(i.padded()) for i in q) == sorted(tuple(i.padded()) for i in ql)
         if any(i.opcode() == 9 for i in ql):
             ops = [i.opcode() for i in ql if i.opcode() != 7 and i.padded()[1] == 0]
