@@ -147,15 +147,20 @@ def batch_decode(args) -> dict:
     import torch
 
     from qimeng_megakernel_amd import decode_batch, synthetic
-    from qimeng_megakernel_amd.decode_schedule.model_config import LLAMA_3_2_1B, LlamaConfig
+    from qimeng_megakernel_amd.decode_schedule.model_config import LLAMA_3_2_1B, QWEN3_1_7B, LlamaConfig
     from qimeng_megakernel_amd.decode_schedule_mb import mk_kernel
 
     B = args.batch
-    shape = dataclasses.replace(LLAMA_3_2_1B, attn_kv_block_size=64)   # the batch route's split-KV block
+    if args.model == "qwen3-1.7b":
+        name, kernel, shape = "Qwen3-1.7B", "decode_megakernel_batch<Qwen3_1p7B>", QWEN3_1_7B
+    else:
+        name, kernel = "Llama-3.2-1B", "decode_megakernel_batch<Llama1B>"
+        shape = dataclasses.replace(LLAMA_3_2_1B, attn_kv_block_size=64)   # the batch route's split-KV block
     LlamaConfig.set_shape(shape)
     device = torch.device("cuda:0")
     torch.cuda.set_device(device)
-    new_tokens = args.steps + 1
+    new_tokens = max(args.new_tokens, args.steps + 1)
+    timed = min(args.steps, new_tokens - 1)
     kv_capacity = args.prompt_len + new_tokens
     weights = synthetic.random_weights(shape, args.seed, max_positions=kv_capacity)
     prompts = torch.stack([synthetic.random_prompt(shape, args.seed + r, args.prompt_len) for r in range(B)])
@@ -166,19 +171,20 @@ def batch_decode(args) -> dict:
     if args.warmup > 0:
         decode_batch.decode(globs, prompts, min(args.warmup + 1, new_tokens), mk=mk, decode_time=False)
     globs.k_cache.zero_(); globs.v_cache.zero_()
-    out = decode_batch.decode(globs, prompts, new_tokens, mk=mk)
+    out = decode_batch.decode(globs, prompts, new_tokens, mk=mk, timed_steps=timed)
     t = out["timing"]
     eager_tokens = out["new_tokens"].clone()
     # the same request with the whole loop (embedding rows, kernel, argmax, row state) as one HIP graph
     globs.k_cache.zero_(); globs.v_cache.zero_()
     graphed = decode_batch.decode(globs, prompts, new_tokens, mk=mk, use_graph=True)
     line = {
-        "metric": "kernel_tok_s", "value": t["kernel_tok_s"], "unit": "tok/s", "n_gpus": 1, "steps": args.steps,
+        "metric": "kernel_tok_s", "value": t["kernel_tok_s"], "unit": "tok/s", "n_gpus": 1, "steps": timed,
         "warmup": args.warmup, "ms_per_step": t["kernel_ms_per_step"], "higher_is_better": True, "scaling": "weak",
         "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
         "config": {
-            "workload": f"Llama-3.2-1B-shaped batch-{B} greedy decode, {args.prompt_len}-token prompt per row, {new_tokens} new "
-                        f"tokens per row (context {args.prompt_len + 1}..{args.prompt_len + args.steps}), seeded random-init bf16 weights",
+            "workload": f"{name}-shaped batch-{B} greedy decode, {args.prompt_len}-token prompt per row, {new_tokens} new "
+                        f"tokens per row; timed: the last {timed} decode steps (context {t['first_timed_context']}.."
+                        f"{t['last_timed_context']}), seeded random-init bf16 weights",
             "batch": B, "seed": args.seed, "queues": int(globs.instructions.shape[0]),
             "instructions_per_queue": int(globs.instructions.shape[1]),
         },
@@ -189,13 +195,14 @@ def batch_decode(args) -> dict:
         "roofline": {
             "bound": "hbm", "achieved": t["achieved_GBps"], "peak": HBM_PEAK_GBPS, "unit": "GB/s",
             "frac": t["achieved_GBps"] / HBM_PEAK_GBPS,
-            # the counter runs were made at batch 8 only
-            "traffic": MEASURED_TRAFFIC_OVER_ALGORITHMIC_BATCH8 * t["algorithmic_bytes"] / max(args.steps, 1) if B == 8 else None,
-            "bytes_per_launch_avg": t["algorithmic_bytes"] / max(args.steps, 1), "kernel": "decode_megakernel_batch<Llama1B>",
+            # the counter runs were made on the Llama shape at batch 8 only
+            "traffic": (MEASURED_TRAFFIC_OVER_ALGORITHMIC_BATCH8 * t["algorithmic_bytes"] / max(timed, 1)
+                        if B == 8 and args.model == "llama-3.2-1b" else None),
+            "bytes_per_launch_avg": t["algorithmic_bytes"] / max(timed, 1), "kernel": kernel,
         },
     }
     if not args.no_cpu_baseline:
-        line["cpu_baseline"] = cpu_baseline_batch(shape, weights, prompts, args.cpu_steps, min(os.cpu_count() or 1, 16))
+        line["cpu_baseline"] = cpu_baseline_batch(shape, weights, prompts, args.cpu_steps, min(os.cpu_count() or 1, 16), name)
     return line
 
 
@@ -311,7 +318,7 @@ def moe_decode(args) -> dict:
     return line
 
 
-def cpu_baseline_batch(shape, weights, prompts, n_steps: int, cores: int) -> dict:
+def cpu_baseline_batch(shape, weights, prompts, n_steps: int, cores: int, shape_name: str) -> dict:
     """The fused batch oracle on the host cores: ``n_steps`` steps of the same rows from position 0."""
     import torch
 
@@ -321,7 +328,8 @@ def cpu_baseline_batch(shape, weights, prompts, n_steps: int, cores: int) -> dic
 
     torch.set_num_threads(cores)
     B = int(prompts.shape[0])
-    g = synthetic.build_batch_globals(weights, shape, n_steps + 1, B, "cpu")
+    # the Qwen3 route's fused attention walks its partial slots in Python: the route's own 8 slots, not the kernel's fan-out
+    g = synthetic.build_batch_globals(weights, shape, n_steps + 1, B, "cpu", max_partials=8 if shape.qk_norm else 27)
     oracle = FusedBatchOracle(shape)
     with torch.no_grad():
         t0 = time.perf_counter()
@@ -331,7 +339,8 @@ def cpu_baseline_batch(shape, weights, prompts, n_steps: int, cores: int) -> dic
             oracle.decode_step(g)
         dt = time.perf_counter() - t0
     return {"value": B * n_steps / dt, "unit": "tok/s", "cores": cores, "kind": "port",
-            "sample": f"{n_steps} steps of {B} rows (contexts 1..{n_steps}) of the Llama-3.2-1B-shaped workload through the fused batch oracle"}
+            "host_cpu_count": os.cpu_count(),
+            "sample": f"{n_steps} steps of {B} rows (contexts 1..{n_steps}) of the {shape_name}-shaped workload through the fused batch oracle"}
 
 
 def main() -> None:
@@ -364,7 +373,7 @@ def main() -> None:
                     help="instead of the decode request: the split-KV attention phase at contexts 4096/16384/32768 "
                          "(one JSON line, metric attention_phase_GBps)")
     ap.add_argument("--batch", type=int, default=1,
-                    help="rows decoded together (2..16: the batch route's kernel, Llama-3.2-1B shape; tokens/s counts all rows)")
+                    help="rows decoded together (2..16: the batch route's kernel, Llama-3.2-1B or Qwen3-1.7B shape; tokens/s counts all rows)")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also run one 1 GiB device-to-device copy (a kernel of known traffic, for scaling rocprofv3 counters)")
     args = ap.parse_args()
@@ -398,8 +407,8 @@ def main() -> None:
         print(json.dumps(moe_decode(args)))
         return
     if args.batch != 1:
-        if args.model != "llama-3.2-1b" or not 2 <= args.batch <= 16:
-            raise SystemExit("bench.py: --batch takes 2..16 and runs on the Llama-3.2-1B shape (the route the reference has)")
+        if args.model not in ("llama-3.2-1b", "qwen3-1.7b") or not 2 <= args.batch <= 16:
+            raise SystemExit("bench.py: --batch takes 2..16 and runs on the Llama-3.2-1B or the Qwen3-1.7B shape")
         print(json.dumps(batch_decode(args)))
         return
     shape = LLAMA_3_2_1B if args.model == "llama-3.2-1b" else QWEN3_1_7B

@@ -35,7 +35,7 @@
 extern "C" {
 #endif
 
-#define QMK_ABI_VERSION 7
+#define QMK_ABI_VERSION 8
 #define QMK_INSTRUCTION_WORDS 32
 
 /* Return / status codes. 0 is success; everything else is an error. */
@@ -225,12 +225,14 @@ int qmk_decode_step_static(const QmkArgs* args);
  * position.  Ten opcodes (…/multi_batch/decode_schedule/instructions/instruction_defs.py:11-211):
  * RMSNorm rows 1/6/9, GEMMs 2/5/7/8/10 over 16-row blocks on the matrix cores, split-KV attention 3 and
  * its reduction 4 per batch row.  Tensors are the batch-1 ones with a leading batch dimension, in the
- * order of mk(...) (…/multi_batch/decode_kernel/mk.h:9-42).  Only the Llama-3.2-1B layer geometry
- * is compiled for this route.  Flags: QMK_FLAG_KEEP_BARRIERS only.
+ * order of mk(...) (…/multi_batch/decode_kernel/mk.h:9-42).  Two layer geometries are compiled for this
+ * route: Llama-3.2-1B, and Qwen3-1.7B with the Qwen3 op set (opcode 2 leaves the raw QKV rows, opcode 3
+ * applies the per-head RMSNorm and RoPE to its row's q and k and appends the cache row).
+ * Flags: QMK_FLAG_KEEP_BARRIERS only.
  */
 typedef struct QmkBatchArgs {
   uint32_t struct_size;            /* = sizeof(QmkBatchArgs)                      */
-  uint32_t model;                  /* QMK_MODEL_LLAMA_3_2_1B                      */
+  uint32_t model;                  /* QMK_MODEL_LLAMA_3_2_1B or QMK_MODEL_QWEN3_1_7B */
   uint32_t flags;                  /* 0 or QMK_FLAG_KEEP_BARRIERS                 */
   uint32_t spin_limit;             /* counter polls before QMK_DEV_WAIT_TIMEOUT; 0 = default */
 
@@ -285,6 +287,12 @@ typedef struct QmkBatchArgs {
 
   uint64_t* timeline;              /* as in QmkArgs; NULL = off                   */
   void* stream;                    /* hipStream_t; NULL = the null stream         */
+
+  /* Qwen3 op set only (QMK_MODEL_QWEN3_1_7B; NULL otherwise): as in QmkArgs, with a leading batch dimension
+   * (…/qwen/qwen3__0_6b/A100/single_batch/decode_schedule/fused/operations.py:52-120 run per row). */
+  void* qkv_raw;                   /* bf16 [B, (Hq+2Hkv)*D]  QKV before the per-head norm and RoPE */
+  const void* q_norm_weights;      /* bf16 [L, D]  pair-interleaved like the q rows of qkv_weights */
+  const void* k_norm_weights;      /* bf16 [L, D]                                 */
 } QmkBatchArgs;
 
 /* Launch one step of the batch route asynchronously on args->stream.  Positions outside the KV

@@ -10,8 +10,8 @@ first checks that its producers' counters are complete and then adds to its own.
 =============================  ==========================
 ``attn_rms / mlp_rms``         python_vm.py:139-160, 614-634
 ``lmhead_rms``                 python_vm.py:668-690
-``qkvproj_gemm_rope``          python_vm.py:163-266
-``decode_attention_split_kv``  python_vm.py:269-359
+``qkvproj_gemm_rope``          python_vm.py:163-266   (Qwen3 op set: the raw rows only)
+``decode_attention_split_kv``  python_vm.py:269-359   (Qwen3 op set: per-head norm, RoPE and cache rows first)
 ``decode_attention_reduction`` python_vm.py:442-551
 ``oproj / down``               python_vm.py:554-611
 ``upgate``                     python_vm.py:637-665
@@ -31,7 +31,7 @@ from typing import Any, Iterable
 import torch
 import torch.nn.functional as F
 
-from fused_oracle import rms_norm, rotate_pairs
+from fused_oracle import per_head_rms_norm, rms_norm, rotate_pairs
 
 Tensor = torch.Tensor
 TILE = 16                      # output rows per GEMM block
@@ -124,6 +124,11 @@ class BatchInstructionVM:
                 if not self._active(g, b):
                     continue
                 pos, mine = self._pos(g, b), out[b]
+                if getattr(s, "qk_norm", False):
+                    # Qwen3 op set (qwen3__0_6b/…/instructions/python_vm.py:110-141, per row): the raw vector
+                    # only; norm, RoPE and the cache rows belong to the attention instruction.
+                    g.qkv_raw[b, row:stop] = mine.to(g.qkv_raw.dtype)
+                    continue
                 if seg != "v":
                     # RoPE pairs are neighbours, so a chunk that starts on an even column is closed under it
                     h0 = row % d
@@ -176,6 +181,19 @@ class BatchInstructionVM:
         t1 = min(min(part * per + per, total) * kvb, seq_len)
         if t0 >= t1:
             return leave_empty()
+        if getattr(s, "qk_norm", False):
+            # Qwen3 op set (qwen3__0_6b/…/instructions/python_vm.py:214-320, per row): q and k of this KV head get
+            # their per-head RMSNorm and RoPE here and K/V of the row's position enter the cache.  Every slice
+            # with work computes the same values, so the sequential VM simply writes them each time.
+            nq, nkv, pos = s.num_attention_heads, s.num_key_value_heads, self._pos(g, b)
+            raw = g.qkv_raw[b]
+            k_off, v_off = (nq + kvh) * d, (nq + nkv + kvh) * d
+            cos, sin = g.rope_cos[pos].unsqueeze(0), g.rope_sin[pos].unsqueeze(0)
+            qn = per_head_rms_norm(raw[h0 * d : h1 * d].view(ratio, d), g.q_norm_weights[layer], s.rms_norm_eps)
+            kn = per_head_rms_norm(raw[k_off : k_off + d].view(1, d), g.k_norm_weights[layer], s.rms_norm_eps)
+            g.q_post_rope[b].view(nq, d)[h0:h1] = ((qn * cos) + (rotate_pairs(qn) * sin)).to(g.q_post_rope.dtype)
+            g.k_cache[layer, b, pos, kvh] = ((kn * cos) + (rotate_pairs(kn) * sin)).view(-1).to(g.k_cache.dtype)
+            g.v_cache[layer, b, pos, kvh] = raw[v_off : v_off + d].to(g.v_cache.dtype)
         k = g.k_cache[layer, b, t0:t1, kvh].float()
         v = g.v_cache[layer, b, t0:t1, kvh].float()
         q = g.q_post_rope[b].view(s.num_attention_heads, d)[h0:h1].float()

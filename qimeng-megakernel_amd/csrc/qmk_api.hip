@@ -343,6 +343,7 @@ struct DeviceInfo {
   int cu_count = 0;
   int max_queues = 0;
   int max_queues_batch = 0;
+  int max_queues_batch_qwen3 = 0;
   int max_queues_moe = 0;
   int32_t* status = nullptr;
   uint64_t* scratch = nullptr;   // this device's copy of the file-scope `scratch` array
@@ -364,6 +365,9 @@ int device_info(DeviceInfo** out) {
     int per_cu_batch = 0;
     if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu_batch, decode_megakernel_batch<Llama1B>, kThreads, 0) != hipSuccess)
       return QMK_ERR_NO_DEVICE;
+    int per_cu_batch3 = 0;
+    if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu_batch3, decode_megakernel_batch<Qwen3_1p7B>, kThreads, 0) != hipSuccess)
+      return QMK_ERR_NO_DEVICE;
     int per_cu_moe = 0;
     if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu_moe, decode_megakernel_moe<QwenMoeA2_7B>, kThreads, 0) != hipSuccess)
       return QMK_ERR_NO_DEVICE;
@@ -379,6 +383,7 @@ int device_info(DeviceInfo** out) {
     d.cu_count = prop.multiProcessorCount;
     d.max_queues = per_cu * prop.multiProcessorCount;
     d.max_queues_batch = per_cu_batch * prop.multiProcessorCount;
+    d.max_queues_batch_qwen3 = per_cu_batch3 * prop.multiProcessorCount;
     d.max_queues_moe = per_cu_moe * prop.multiProcessorCount;
     d.status = static_cast<int32_t*>(sym);
     d.scratch = static_cast<uint64_t*>(scratch_ptr);
@@ -517,11 +522,8 @@ extern "C" int qmk_decode_step(const QmkArgs* a) { return decode_step_any(a, fal
 // lives in the code object; its address was looked up when the device was first used).
 extern "C" int qmk_decode_step_static(const QmkArgs* a) { return decode_step_any(a, true); }
 
-extern "C" int qmk_decode_step_batch(const QmkBatchArgs* a) {
-  using M = Llama1B;
-  if (a == nullptr) return QMK_ERR_NULL_ARG;
-  if (a->struct_size != sizeof(QmkBatchArgs)) return QMK_ERR_ABI;
-  if (a->model != QMK_MODEL_LLAMA_3_2_1B) return QMK_ERR_MODEL;
+template <class M>
+static int decode_step_batch(const QmkBatchArgs* a) {
   const void* required[] = {a->instructions, a->hidden_states, a->q_post_rope, a->k_cache, a->v_cache, a->attn_out,
                             a->attn_lse_intermediates, a->attn_out_intermediates, a->silu_out, a->logits,
                             a->attn_norm_weights, a->qkv_weights, a->rope_cos, a->rope_sin, a->o_proj_weights,
@@ -530,6 +532,7 @@ extern "C" int qmk_decode_step_batch(const QmkBatchArgs* a) {
                             a->attn_rms_out, a->mlp_rms_out, a->lm_head_rms_out};
   for (const void* ptr : required)
     if (ptr == nullptr) return QMK_ERR_NULL_ARG;
+  if (M::QK_NORM && (a->qkv_raw == nullptr || a->q_norm_weights == nullptr || a->k_norm_weights == nullptr)) return QMK_ERR_NULL_ARG;
   if (a->batch_size < 1 || a->batch_size > mb::kMaxBatch) return QMK_ERR_SHAPE;
   if (a->num_queues < 1 || a->num_insts < 0 || a->num_layers < 1 || a->num_layer_barriers < 10 ||
       a->barrier_slots < a->batch_size * (M::NQ + 2 * M::NKV) || a->max_seq_len < 1 || a->max_splits < 1 ||
@@ -540,7 +543,7 @@ extern "C" int qmk_decode_step_batch(const QmkBatchArgs* a) {
 
   DeviceInfo* dev = nullptr;
   if (int rc = device_info(&dev); rc != QMK_OK) return rc;
-  if (a->num_queues > dev->max_queues_batch) return QMK_ERR_TOO_MANY_QUEUES;
+  if (a->num_queues > (M::QK_NORM ? dev->max_queues_batch_qwen3 : dev->max_queues_batch)) return QMK_ERR_TOO_MANY_QUEUES;
   if (a->num_insts == 0) return QMK_OK;
 
   Params p{};
@@ -591,9 +594,20 @@ extern "C" int qmk_decode_step_batch(const QmkBatchArgs* a) {
   p.mlp_rms_out = static_cast<u16*>(a->mlp_rms_out);
   p.lm_rms_out = static_cast<u16*>(a->lm_head_rms_out);
   p.rope_rows = a->rope_rows;
+  p.qkv_raw = static_cast<u16*>(a->qkv_raw);
+  p.q_norm = static_cast<const u16*>(a->q_norm_weights);
+  p.k_norm = static_cast<const u16*>(a->k_norm_weights);
 
   hipLaunchKernelGGL(decode_megakernel_batch<M>, dim3(a->num_queues), dim3(kThreads), 0, static_cast<hipStream_t>(a->stream), p);
   return hipGetLastError() == hipSuccess ? QMK_OK : QMK_ERR_LAUNCH;
+}
+
+extern "C" int qmk_decode_step_batch(const QmkBatchArgs* a) {
+  if (a == nullptr) return QMK_ERR_NULL_ARG;
+  if (a->struct_size != sizeof(QmkBatchArgs)) return QMK_ERR_ABI;
+  if (a->model == QMK_MODEL_LLAMA_3_2_1B) return decode_step_batch<Llama1B>(a);
+  if (a->model == QMK_MODEL_QWEN3_1_7B) return decode_step_batch<Qwen3_1p7B>(a);
+  return QMK_ERR_MODEL;
 }
 
 extern "C" uint64_t qmk_moe_workspace_bytes(int top_k, int shared_k_slices) {

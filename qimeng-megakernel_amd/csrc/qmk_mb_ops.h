@@ -288,6 +288,10 @@ __device__ bool op_qkv(const Params& p, Smem<M>& s, const Ctx& c) {
         const uint32_t vb = pack_bf16(v.x, v.y);
         const float v0 = bf_lo(vb), v1 = bf_hi(vb);
         const int o = (n0 + j) * kTile + 2 * rp, d = o % M::D, pos = s.pos[b];
+        if constexpr (M::QK_NORM) {   // Qwen3 op set: the raw vector; norm, RoPE and the cache rows belong to the attention prologue
+          st_shared32(p.qkv_raw + static_cast<size_t>(b) * M::QKV + o, vb);
+          return;
+        }
         const size_t cache_row = ((static_cast<size_t>(layer) * B + b) * p.max_seq_len + pos) * tok_stride;
         if (o < M::NQ * M::D) {
           st_shared32(p.q_post_rope + static_cast<size_t>(b) * M::NQ * M::D + o,
@@ -387,6 +391,7 @@ template <class M>
 __device__ bool op_splitkv(const Params& p, Smem<M>& s, const Ctx& c) {
   constexpr int D = M::D, GQA = M::GQA;
   static_assert(D % 64 == 0 && GQA <= 4 && GQA * D <= kThreads, "a lane owns whole 16-byte vectors of K; one thread per merged output");
+  static_assert(M::AW == M::H, "the O-projection of this route reads an attention output as wide as the hidden state");
   const int layer = s.inst[1], b = s.inst[2], kvh = s.inst[3], P = s.inst[4], part = s.inst[5];
   if (layer < 0 || layer >= p.num_layers) return bad_operand(p, s, c, 1);
   if (b < 0 || b >= p.batch) return bad_operand(p, s, c, 2);
@@ -495,7 +500,41 @@ __device__ bool op_splitkv(const Params& p, Smem<M>& s, const Ctx& c) {
     const size_t new_row = row_of_kvh + static_cast<size_t>(pos) * tok_stride;
     constexpr int kQChunks = GQA * D / 8, kRowChunks = D / 8;
     const int tid = c.tid;
-    if (tid < kQChunks) {
+    if constexpr (M::QK_NORM) {
+      // Qwen3 op set (qwen3__0_6b/…/fused/operations.py:52-120): the raw vectors are staged; then one wave per
+      // vector applies the per-head RMSNorm and RoPE in place (every lane one rotation pair), and the workgroup
+      // whose slice holds the row's position also writes q_post_rope and the cache row.
+      static_assert(D == 2 * kWaveSize && GQA + 2 <= kWaves, "one wave per vector, one rotation pair per lane");
+      const u16* raw = p.qkv_raw + static_cast<size_t>(b) * M::QKV;
+      if (tid < kQChunks) {
+        reinterpret_cast<v4u*>(stage16 + kQ)[tid] = ld_shared128(raw + head0 * D + tid * 8);
+      } else if (tid < kQChunks + kRowChunks && has_new) {
+        reinterpret_cast<v4u*>(stage16 + kK)[tid - kQChunks] = ld_shared128(raw + (M::NQ + kvh) * D + (tid - kQChunks) * 8);
+      } else if (tid < kQChunks + 2 * kRowChunks && has_new) {
+        reinterpret_cast<v4u*>(stage16 + kV)[tid - kQChunks - kRowChunks] =
+            ld_shared128(raw + (M::NQ + M::NKV + kvh) * D + (tid - kQChunks - kRowChunks) * 8);
+      }
+      __syncthreads();
+      uint32_t* words = reinterpret_cast<uint32_t*>(stage16);
+      if (wave <= GQA && (wave < GQA || has_new)) {
+        const bool is_k = wave == GQA;
+        const int at = is_k ? kK / 2 : (kQ + wave * D) / 2;
+        const uint32_t rw = words[at + lane];
+        const float x0 = bf_lo(rw), x1 = bf_hi(rw);
+        const float ss = wave_sum(__builtin_fmaf(x1, x1, x0 * x0));
+        const float rstd = 1.0f / sqrtf(ss / static_cast<float>(D) + p.rms_norm_eps);
+        const uint32_t wn = reinterpret_cast<const uint32_t*>((is_k ? p.k_norm : p.q_norm) + static_cast<size_t>(layer) * D)[lane];
+        const float n0 = round_bf16(bf_lo(wn) * (x0 * rstd)), n1 = round_bf16(bf_hi(wn) * (x1 * rstd));
+        const uint32_t out = rope_pair(n0, n1, p.rope_cos + static_cast<size_t>(pos) * D, p.rope_sin + static_cast<size_t>(pos) * D, 2 * lane);
+        words[at + lane] = out;
+        if (has_new) {
+          if (is_k) st_shared32(p.k_cache + new_row + 2 * lane, out);
+          else st_shared32(p.q_post_rope + static_cast<size_t>(b) * M::NQ * D + (head0 + wave) * D + 2 * lane, out);
+        }
+      } else if (wave == GQA + 1 && has_new) {
+        st_shared32(p.v_cache + new_row + 2 * lane, words[kV / 2 + lane]);
+      }
+    } else if (tid < kQChunks) {
       reinterpret_cast<v4u*>(stage16 + kQ)[tid] = ld_shared128(p.q_post_rope + static_cast<size_t>(b) * M::NQ * D + head0 * D + tid * 8);
     } else if (tid < kQChunks + kRowChunks && has_new) {
       reinterpret_cast<v4u*>(stage16 + kK)[tid - kQChunks] = ld_shared128(p.k_cache + new_row + (tid - kQChunks) * 8);
@@ -749,8 +788,8 @@ __device__ bool op_upgate(const Params& p, Smem<M>& s, const Ctx& c) {
 // ===================================================================== 8 ==
 // [8, layer, batch_size, tile_M, n_start, n_end, tile_M_g, tile_N_g]
 // hidden[b, r] = bf16(hidden[b, r] + bf16(W_d[r] . silu_out[b])) for active rows, the whole K in
-// one instruction (python_vm.py:554-611).  A wave owns F/8 columns: F/2048 segments per block; its
-// share of silu_out follows the wait, two segments at a time.
+// one instruction (python_vm.py:554-611).  A wave owns F/8 columns: F/2048 segments per block (four for
+// F = 8192, three for 6144); its share of silu_out follows the wait, two segments at a time.
 template <class M>
 __device__ bool op_down(const Params& p, Smem<M>& s, const Ctx& c) {
   constexpr int NS = M::F / (kWaves * kSeg);   // segments per wave and block
@@ -765,9 +804,9 @@ __device__ bool op_down(const Params& p, Smem<M>& s, const Ctx& c) {
   const u16* w = p.down_w + static_cast<size_t>(layer) * M::H * M::F;
   const int k0 = wave * NS * kSeg;
   const size_t lane_off = static_cast<size_t>(lane & (R - 1)) * M::F + k0 + (lane >> 4) * 8;
-  static_assert(NS == 4, "the segments below are handled by name");
-  // Three of the four weight segments of a block are requested before the wait and land during it; the
-  // fourth follows the first activations (all four beside two activation segments do not fit the registers).
+  static_assert(NS == 3 || NS == 4, "the segments below are handled by name");
+  // Three weight segments of a block are requested before the wait and land during it; with four segments
+  // the last follows the first activations (all four beside two activation segments do not fit the registers).
   Seg a0, a1, a2, a3;
   auto wptr = [&](int block, int q) { return w + static_cast<size_t>(block) * R * M::F + lane_off + q * kSeg; };
   auto request = [&](int block) {
@@ -784,14 +823,14 @@ __device__ bool op_down(const Params& p, Smem<M>& s, const Ctx& c) {
     v4u xa[kSegChunks], xb[kSegChunks];
     load_x(xa, p.silu_out, M::F, B, k0, lane);
     load_x(xb, p.silu_out, M::F, B, k0 + kSeg, lane);
-    load_seg(a3, wptr(blk, 3));
+    if constexpr (NS == 4) load_seg(a3, wptr(blk, 3));
     f4 acc = mma_seg(a0, xa, f4{0.f, 0.f, 0.f, 0.f});
     load_x(xa, p.silu_out, M::F, B, k0 + 2 * kSeg, lane);
     acc = mma_seg(a1, xb, acc);
-    load_x(xb, p.silu_out, M::F, B, k0 + 3 * kSeg, lane);
+    if constexpr (NS == 4) load_x(xb, p.silu_out, M::F, B, k0 + 3 * kSeg, lane);
     const uint32_t old = adds ? ld_shared32(mine + blk * R) : 0u;   // the pair this thread adds to, in time for the epilogue
     acc = mma_seg(a2, xa, acc);
-    acc = mma_seg(a3, xb, acc);
+    if constexpr (NS == 4) acc = mma_seg(a3, xb, acc);
     park(s, parity, 0, wave, lane, acc);
     QMK_MB_STAMP(0);  // thread 0's weights and activations have all arrived
     if (blk + 1 < n1) request(blk + 1);

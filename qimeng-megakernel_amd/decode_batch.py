@@ -57,9 +57,12 @@ def argmax_rows(logits: torch.Tensor) -> torch.Tensor:
 
 
 def decode(globs: Any, prompts: torch.Tensor, max_new_tokens: int, *, mk: Any = None, eos_token_ids: Sequence[int] = (),
-           decode_time: bool = True, use_graph: bool = False) -> dict[str, Any]:
+           decode_time: bool = True, use_graph: bool = False, timed_steps: int | None = None) -> dict[str, Any]:
     """Prefill + greedy decode of B rows to ``max_new_tokens`` tokens each (rows that hit an EOS token
     of ``eos_token_ids`` retire; with none given every row runs to the end).
+
+    ``timed_steps``: time only the last so many decode steps of the request (the longest contexts); the steps
+    before them run untimed.  Default: all of them.
 
     ``use_graph``: the whole decode loop (embedding rows, kernel, argmax, row state) is captured into one
     HIP graph and replayed once — the kernel reads positions and activity from device tensors, so nothing
@@ -86,18 +89,19 @@ def decode(globs: Any, prompts: torch.Tensor, max_new_tokens: int, *, mk: Any = 
     if eos_token_ids:   # on the device before the loop: nothing inside a step comes from the host
         eos = torch.tensor(list(eos_token_ids), dtype=torch.long, device=device)
     timed = decode_time and not use_graph
-    events = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(ntok if timed else 0)]
+    lead_in = 0 if timed_steps is None or use_graph else max(ntok - max(int(timed_steps), 0), 0)
+    events = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(ntok - lead_in if timed else 0)]
     loop_start, loop_end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
     active_log = []
 
-    def steps() -> None:
-        for i in range(ntok):
+    def steps(first: int = 0, last: int = ntok) -> None:
+        for i in range(first, last):
             _embed(globs, out[:, T + i])
-            if events:
-                events[i][0].record()
+            if events and i >= lead_in:
+                events[i - lead_in][0].record()
             _mk_kernel.call_mk(globs, mk)
-            if events:
-                events[i][1].record()
+            if events and i >= lead_in:
+                events[i - lead_in][1].record()
             nxt = argmax_rows(globs.logits) if use_graph else globs.logits.argmax(dim=-1)
             out[:, T + i + 1] = nxt
             if eos is not None:
@@ -116,13 +120,15 @@ def decode(globs: Any, prompts: torch.Tensor, max_new_tokens: int, *, mk: Any = 
         with torch.cuda.graph(graph):
             steps()
         rewind()   # capturing ran nothing, but the host-side bookkeeping of the loop did
+    if graph is None and lead_in:
+        steps(0, lead_in)
     torch.cuda.synchronize(device)
     wall0 = time.perf_counter()
     loop_start.record()
     if graph is not None:
         graph.replay()
     else:
-        steps()
+        steps(lead_in, ntok)
     loop_end.record()
     torch.cuda.synchronize(device)
     result: dict[str, Any] = {"generated_ids": out, "new_tokens": out[:, T:]}
@@ -145,14 +151,17 @@ def decode(globs: Any, prompts: torch.Tensor, max_new_tokens: int, *, mk: Any = 
             rows = [int(m.sum()) for m in active_log]
         else:
             rows = [B] * ntok
-        produced = sum(rows)
-        nbytes = sum(step_bytes(shape, [T + i + 1] * rows[i]) for i in range(ntok))
+        window = range(lead_in, ntok)          # the steps between the loop's two events
+        produced = sum(rows[i] for i in window)
+        nbytes = sum(step_bytes(shape, [T + i + 1] * rows[i]) for i in window)
+        nsteps = max(len(window), 1)
         result["timing"] = {
             "decode_wall_s": wall, "decode_gpu_s": gpu_s, "mk_kernel_gpu_s": kernel_s,
             "decode_window_new_tokens": produced,
             "effective_tok_s_wall": produced / wall, "effective_tok_s_gpu": produced / gpu_s,
-            "kernel_tok_s": produced / kernel_s, "kernel_steps": ntok, "kernel_ms_per_step": kernel_s * 1e3 / ntok,
+            "kernel_tok_s": produced / kernel_s, "kernel_steps": len(window), "kernel_ms_per_step": kernel_s * 1e3 / nsteps,
             "algorithmic_bytes": nbytes, "achieved_GBps": nbytes / kernel_s / 1e9, "per_step_ms": per_step_ms,
+            "first_timed_context": T + lead_in + 1, "last_timed_context": T + ntok,
         }
     mk.check()
     return result

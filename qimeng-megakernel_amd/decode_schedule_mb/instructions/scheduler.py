@@ -39,7 +39,6 @@ from .instruction_defs import (
     UpGateProj_GEMM_SiLU,
 )
 
-ATTN_REDUCTION_SIZE = 4
 MAX_TILE_BLOCKS_PER_INSTRUCTION = INTS_PER_INSTRUCTION - 6
 MAX_REDUCTION_LIST = INTS_PER_INSTRUCTION - 5
 A100_WORKERS = 108 * 2
@@ -155,7 +154,7 @@ class BatchScheduler:
         if self.merge_in_last:
             return out
         for b in range(self.batch_size):
-            for head0 in range(0, self.shape.num_attention_heads, ATTN_REDUCTION_SIZE):
+            for head0 in range(0, self.shape.num_attention_heads, self.shape.attn_reduction_size):
                 if globs is None:
                     out.append(DecodeAttentionReduction(layer, b, head0, num_partials, list(range(num_partials))))
                 else:

@@ -7,6 +7,11 @@ rms_norm_eps``, the three control tensors and the three RMSNorm scratch tensors 
 reference's positional order, ``run_instructions`` executes an arbitrary instruction list.  The
 callable wraps ``qmk_decode_step_batch`` of ``libqmk_hip.so`` (``include/qmk.h``) with ctypes.
 
+A shape with the Qwen3 op set (``qk_norm``: Qwen3-1.7B) has no batch route in the reference; its
+``mk`` takes three more tensors behind the 32 arguments — ``qkv_raw [B, QKV]``, ``q_norm_weights``,
+``k_norm_weights`` — the ones the reference's Qwen3 launcher adds to the batch-1 call
+(`…/qwen/qwen3__0_6b/A100/single_batch/decode_schedule/mk_kernel.py`).
+
 There is no fallback: a missing library is an ``ImportError``, a non-GPU tensor a
 ``ValueError`` and a device-side error a ``RuntimeError``.
 """
@@ -50,6 +55,7 @@ class QmkBatchArgs(ctypes.Structure):
         ("position_ids", _P), ("active_mask", _P), ("attn_partial_valid", _P),
         ("attn_rms_out", _P), ("mlp_rms_out", _P), ("lm_head_rms_out", _P),
         ("timeline", _P), ("stream", _P),
+        ("qkv_raw", _P), ("q_norm_weights", _P), ("k_norm_weights", _P),
     ]
 
 
@@ -138,12 +144,12 @@ class BatchMegaKernel:
         return other
 
     def _bind(self, tensors: Sequence[torch.Tensor], B: int, position_ids: Any, active_mask: Any, partial_valid: Any,
-              rms: Sequence[Any]) -> None:
+              rms: Sequence[Any], qwen3: Sequence[Any] = ()) -> None:
         a = self._args
         shape = LlamaConfig.shape()
         a.model = _single._model_id(shape)
-        if a.model != _single.QMK_MODEL_LLAMA_3_2_1B:
-            raise ValueError("the batch route is compiled for the Llama-3.2-1B layer geometry only")
+        if a.model not in (_single.QMK_MODEL_LLAMA_3_2_1B, _single.QMK_MODEL_QWEN3_1_7B):
+            raise ValueError("the batch route is compiled for the Llama-3.2-1B and Qwen3-1.7B layer geometries only")
         if not 1 <= B <= MAX_BATCH:
             raise ValueError(f"batch_size must be in [1, {MAX_BATCH}], got {B}")
         device = tensors[1].device if isinstance(tensors[1], torch.Tensor) else None
@@ -200,6 +206,16 @@ class BatchMegaKernel:
                 raise ValueError(f"{name} must be provided")
             _check(name, t, device, (torch.bfloat16,), (B, H), 2)
             setattr(a, name, t.data_ptr())
+        a.qkv_raw = a.q_norm_weights = a.k_norm_weights = None
+        if shape.qk_norm:
+            if len(qwen3) != 3 or any(t is None for t in qwen3):
+                raise ValueError("the Qwen3 op set needs qkv_raw, q_norm_weights and k_norm_weights behind the 32 arguments")
+            _check("qkv_raw", qwen3[0], device, (torch.bfloat16,), (B, shape.qkv_out_dim), 2)
+            _check("q_norm_weights", qwen3[1], device, (torch.bfloat16,), (L, d), 2)
+            _check("k_norm_weights", qwen3[2], device, (torch.bfloat16,), (L, d), 2)
+            a.qkv_raw, a.q_norm_weights, a.k_norm_weights = (t.data_ptr() for t in qwen3)
+        elif qwen3:
+            raise TypeError("qkv_raw / q_norm_weights / k_norm_weights belong to the Qwen3 op set only")
         a.position_ids = position_ids.data_ptr() if position_ids is not None else None
         a.active_mask = active_mask.data_ptr() if active_mask is not None else None
         a.attn_partial_valid = partial_valid.data_ptr() if partial_valid is not None else None
@@ -210,18 +226,20 @@ class BatchMegaKernel:
         a.kv_block_size = int(shape.attn_kv_block_size)
 
     def __call__(self, *args: Any) -> None:
-        if len(args) != 32:
-            raise TypeError(f"mk of the batch route takes 22 tensors, 4 scalars and 6 tensors, got {len(args)} positional arguments")
+        want = 35 if LlamaConfig.shape().qk_norm else 32
+        if len(args) != want:
+            raise TypeError(f"mk of the batch route takes 22 tensors, 4 scalars and {want - 26} tensors for this shape, "
+                            f"got {len(args)} positional arguments")
         tensors = args[:22]
         pos_id, B, attn_scale, rms_norm_eps = args[22:26]
         position_ids, active_mask, partial_valid = args[26:29]
         rms = args[29:32]
         if isinstance(tensors[0], torch.Tensor) and tensors[0].numel() == 0:
             return
-        key = tuple((t.data_ptr(), tuple(t.shape)) if isinstance(t, torch.Tensor) else None for t in (*tensors, *args[26:32])) + (
+        key = tuple((t.data_ptr(), tuple(t.shape)) if isinstance(t, torch.Tensor) else None for t in (*tensors, *args[26:])) + (
             int(B), LlamaConfig.shape())
         if key != self._bound_key:
-            self._bind(tensors, int(B), position_ids, active_mask, partial_valid, rms)
+            self._bind(tensors, int(B), position_ids, active_mask, partial_valid, rms, args[32:])
             self._bound_key = key
         a = self._args
         a.pos_id = int(pos_id)
@@ -313,6 +331,7 @@ def call_mk(globs: Globals, mk: Any) -> None:
         globs.attn_rms_out,
         globs.mlp_rms_out,
         globs.lm_head_rms_out,
+        *((globs.qkv_raw, globs.q_norm_weights, globs.k_norm_weights) if shape.qk_norm else ()),
     )
 
 

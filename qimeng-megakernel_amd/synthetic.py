@@ -166,6 +166,8 @@ def build_batch_globals(
         **{k: v for k, v in on_device.items() if k != "embed_tokens"},
     )
     g.embed_tokens = on_device["embed_tokens"]
+    if shape.qk_norm:
+        g.qkv_raw = zeros(B, shape.qkv_out_dim)
     return g
 
 

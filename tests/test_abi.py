@@ -80,7 +80,7 @@ def test_host_side_argument_errors(lib):
     a.model = 0
     assert lib.qmk_decode_step(ctypes.byref(a)) == 1                       # all tensor pointers are NULL
     assert lib.qmk_workspace_bytes(0) == 8 * (512 + 2048 + 4 * 1024 + 4096 + 1024 + 16) and lib.qmk_workspace_bytes(1) == lib.qmk_workspace_bytes(0) and lib.qmk_workspace_bytes(7) == 0
-    assert lib.qmk_query(0) == 7 and lib.qmk_query(2) == 512 and lib.qmk_query(5) == 32 and lib.qmk_query(6) == 25
+    assert lib.qmk_query(0) == 8 and lib.qmk_query(2) == 512 and lib.qmk_query(5) == 32 and lib.qmk_query(6) == 25
     assert 0 < lib.qmk_query(3) <= 160 * 1024
     assert lib.qmk_error_string(34).decode().startswith("device: counter wait")
     mk_kernel_mb.get_mk()                                                  # declares the entry point's signature
@@ -89,10 +89,11 @@ def test_host_side_argument_errors(lib):
     b.struct_size = 12
     assert lib.qmk_decode_step_batch(ctypes.byref(b)) == 2
     b.struct_size = ctypes.sizeof(mk_kernel_mb.QmkBatchArgs)
-    b.model = 1
-    assert lib.qmk_decode_step_batch(ctypes.byref(b)) == 8                 # only the Llama geometry is compiled for this route
-    b.model = 0
-    assert lib.qmk_decode_step_batch(ctypes.byref(b)) == 1
+    b.model = 2
+    assert lib.qmk_decode_step_batch(ctypes.byref(b)) == 8                 # the MoE geometries are not compiled for this route
+    for model in (0, 1):                                                   # Llama-3.2-1B, Qwen3-1.7B: all tensor pointers are NULL
+        b.model = model
+        assert lib.qmk_decode_step_batch(ctypes.byref(b)) == 1
     mk_kernel_moe.get_mk()
     assert lib.qmk_decode_step_moe(None) == 1
     m = mk_kernel_moe.QmkMoeArgs()
