@@ -1,4 +1,5 @@
-"""Host step loop of the MoE ``mk`` route at batch 1: prefill-by-decode, greedy loop, timing.
+"""Host step loops of the MoE ``mk`` route: prefill-by-decode, greedy loop, timing — one request (``decode``) or
+several rows side by side (``decode_rows``).
 
 Same shape as the dense loop (``decode.py``; reference `qimeng_megakernel/models/LLM/decode.py:536-796`):
 one instruction tensor per request, per step the embedding row of the last token -> ``hidden_states``,
@@ -8,7 +9,7 @@ the launch only.
 from __future__ import annotations
 
 import time
-from typing import Any
+from typing import Any, Sequence
 
 import torch
 
@@ -106,4 +107,93 @@ def decode(globs: Any, prompt_ids: torch.Tensor, max_new_tokens: int, *, mk: Any
             "achieved_GBps": nbytes / kernel_s / 1e9, "per_step_ms": per_step_ms,
         }
     mk.check()
+    return result
+
+
+def share_weights(globs: Any, shape: Any, kv_capacity: int, rows: int, *, max_partials: int) -> list[Any]:
+    """``rows`` sets of buffers (KV cache, activations, counters) over ONE copy of ``globs``' weights: what a batch
+    of requests on the batch-1 kernel needs.  Row 0 is ``globs`` itself."""
+    from . import synthetic
+
+    weights = {name: getattr(globs, name) for name in synthetic.MOE_WEIGHT_NAMES if getattr(globs, name, None) is not None}
+    weights["embed_tokens"] = globs.embed_tokens
+    out = [globs]
+    for _ in range(1, rows):
+        out.append(synthetic.build_moe_globals(weights, shape, kv_capacity, globs.hidden_states.device, max_partials=max_partials))
+    return out
+
+
+def decode_rows(rows: Sequence[Any], prompts: torch.Tensor, max_new_tokens: int, *, mks: Sequence[Any] | None = None,
+                decode_time: bool = True, timed_steps: int | None = None) -> dict[str, Any]:
+    """Greedy decode of ``len(rows)`` requests side by side on the batch-1 kernel: every step launches the kernel
+    once per row, back to back on one stream (each row has its own buffers and its own launcher, hence its own
+    workspace; the weights exist once).  Nothing is shared between the rows' launches but the weights' place in
+    memory: a step moves every row's weight bytes again.  The reference has no MoE route for batch sizes above
+    one; its batch loop (`qimeng_megakernel/models/LLM/decode.py:536-796`) is what the step order follows.
+
+    ``prompts`` [B, T]; ``timed_steps`` as in ``decode``.  Timing: one event pair around each launch; a step's time
+    is the sum over its rows."""
+    B, T = int(prompts.shape[0]), int(prompts.shape[1])
+    if B != len(rows):
+        raise ValueError(f"{B} prompts for {len(rows)} rows of buffers")
+    device = rows[0].hidden_states.device
+    if any(T + max_new_tokens > int(g.k_cache.shape[2]) for g in rows):
+        raise ValueError("prompt_len + max_new_tokens exceeds the KV cache capacity")
+    mks = list(mks) if mks is not None else [_mk_kernel.get_mk() for _ in rows]
+    for g, mk in zip(rows, mks):
+        g.instructions = None
+        _mk_kernel.build(g, mk)
+    out = torch.zeros(B, T + max(max_new_tokens, 1), dtype=torch.long, device=device)
+    out[:, :T] = prompts.to(device)
+
+    def step(pos: int, column: int, events: list | None) -> None:
+        for r, (g, mk) in enumerate(zip(rows, mks)):
+            g.hidden_states.copy_(g.embed_tokens.index_select(0, out[r, column : column + 1]).view(-1))
+            g.position_id = pos
+            if events is not None:
+                pair = (torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True))
+                pair[0].record()
+            _mk_kernel.call_mk(g, mk)
+            if events is not None:
+                pair[1].record()
+                events.append(pair)
+            out[r, column + 1] = g.logits.argmax()
+
+    for pos in range(T - 1):           # prompt positions whose prediction is not needed
+        for r, (g, mk) in enumerate(zip(rows, mks)):
+            g.hidden_states.copy_(g.embed_tokens.index_select(0, out[r, pos : pos + 1]).view(-1))
+            g.position_id = pos
+            _mk_kernel.call_mk(g, mk)
+    step(T - 1, T - 1, None)           # the last prompt position predicts the first new token
+    total = max(max_new_tokens - 1, 0)
+    ntok = total if timed_steps is None else max(0, min(int(timed_steps), total))
+    for i in range(total - ntok):
+        step(T + i, T + i, None)
+    first = T + total - ntok
+    events: list = []
+    loop_start, loop_end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    torch.cuda.synchronize(device)
+    wall0 = time.perf_counter()
+    loop_start.record()
+    for i in range(ntok):
+        step(first + i, first + i, events if decode_time else None)
+    loop_end.record()
+    torch.cuda.synchronize(device)
+    result: dict[str, Any] = {"generated_ids": out, "new_tokens": out[:, T:]}
+    if decode_time and ntok:
+        wall = time.perf_counter() - wall0
+        gpu_s = loop_start.elapsed_time(loop_end) / 1e3
+        launch_ms = [a.elapsed_time(b) for a, b in events]
+        kernel_s = sum(launch_ms) / 1e3
+        shape = QwenMoeConfig.shape()
+        nbytes = B * sum(shape.step_bytes(first + i + 1) for i in range(ntok))
+        result["timing"] = {
+            "decode_wall_s": wall, "decode_gpu_s": gpu_s, "mk_kernel_gpu_s": kernel_s,
+            "effective_tok_s_wall": B * ntok / wall, "effective_tok_s_gpu": B * ntok / gpu_s, "kernel_tok_s": B * ntok / kernel_s,
+            "kernel_steps": ntok, "kernel_launches": len(launch_ms), "kernel_ms_per_step": kernel_s * 1e3 / ntok,
+            "kernel_ms_per_launch": kernel_s * 1e3 / len(launch_ms), "algorithmic_bytes": nbytes,
+            "first_timed_context": first + 1, "last_timed_context": first + ntok, "achieved_GBps": nbytes / kernel_s / 1e9,
+        }
+    for mk in mks:
+        mk.check()
     return result

@@ -191,6 +191,13 @@ def reduced_shape(num_layers: int = 2, vocab_size: int = 2048, **overrides: Any)
     return dataclasses.replace(LlamaConfig.shape().__class__(), num_hidden_layers=num_layers, vocab_size=vocab_size, **overrides)
 
 
+#: what ``random_moe_weights`` may return beside ``embed_tokens`` (the read-only tensors of the MoE route's ``Globals``)
+MOE_WEIGHT_NAMES = ("qkv_weights", "qkv_bias", "o_proj_weights", "router_weights", "shared_expert_gate_proj_weights",
+                    "shared_expert_up_proj_weights", "shared_expert_down_proj_weights", "shared_expert_gate_weights",
+                    "expert_gate_up_proj_weights", "expert_down_proj_weights", "lm_head_weights", "attn_norm_weights",
+                    "mlp_norm_weights", "lm_head_norm_weights", "q_norm_weights", "k_norm_weights", "rope_cos", "rope_sin")
+
+
 def random_moe_weights(shape: Any, seed: int, max_positions: int, device: torch.device | str = "cpu") -> dict[str, torch.Tensor]:
     """Seeded random-init weights of the MoE route (``decode_schedule_moe.MoeShape``): bf16 ~N(0, 0.02)
     projections, router and experts (gate rows first in ``expert_gate_up_proj_weights``), QKV bias

@@ -306,6 +306,28 @@ def test_decode_loop_and_graph(weights):
     mk.check()
 
 
+def test_rows_side_by_side_equal_the_rows_alone(weights):
+    """Four requests side by side over one copy of the weights (BASELINE's batch 4 on this route: one launch per row and
+    step): every row's tokens, logits and cache equal that request decoded alone, and the first row's step follows the
+    fused oracle teacher-forced like the batch-1 request does."""
+    rows_n, new = 4, 10
+    first = synthetic.build_moe_globals(weights, SMALL, 64, "cuda:0", max_partials=8)
+    rows = decode_moe.share_weights(first, SMALL, 64, rows_n, max_partials=8)
+    assert all(g.qkv_weights.data_ptr() == first.qkv_weights.data_ptr() for g in rows)          # one copy of the weights
+    assert len({g.k_cache.data_ptr() for g in rows}) == rows_n                                   # ... and a cache per row
+    prompts = torch.tensor([[3, 99, 1024, 7], [5, 5, 5, 5], [2047, 0, 1, 2], [77, 1500, 300, 9]])
+    together = decode_moe.decode_rows(rows, prompts, new, timed_steps=4)
+    t = together["timing"]
+    assert t["kernel_steps"] == 4 and t["kernel_launches"] == 4 * rows_n and t["first_timed_context"] == 4 + (new - 1 - 4) + 1
+    assert t["algorithmic_bytes"] == rows_n * sum(SMALL.step_bytes(c) for c in range(t["first_timed_context"], t["last_timed_context"] + 1))
+    for r in range(rows_n):
+        alone = synthetic.build_moe_globals(weights, SMALL, 64, "cuda:0", max_partials=8)
+        want = decode_moe.decode(alone, prompts[r], new, decode_time=False)["new_tokens"]
+        assert torch.equal(together["new_tokens"][r], want), r
+        assert torch.equal(rows[r].logits, alone.logits) and torch.equal(rows[r].k_cache, alone.k_cache), r
+    assert len({tuple(x) for x in together["new_tokens"].tolist()}) == rows_n                    # four different requests
+
+
 @pytest.mark.slow
 def test_full_layer_geometry_layer_by_layer():
     """128 experts of 768, top-8 renormalised, 32/4 heads of 128 — the benchmarked layer, three of them and a reduced
