@@ -82,6 +82,7 @@ class BatchScheduler:
     merge_in_last: bool = False   # the last split-KV arrival of a head group merges: no reduction instructions
     oproj_tile: int = TILE_N_GRANULARITY   # rows per O-proj block: 16 (the reference's), or 8
     down_tile: int = TILE_N_GRANULARITY    # rows per down-projection block
+    skew_upgate: bool = False     # run-time template: workers that have just run an O-proj block get fewer up/gate blocks
 
     def __post_init__(self) -> None:
         if not 1 <= self.batch_size <= MAX_BATCH:
@@ -115,6 +116,28 @@ class BatchScheduler:
             mine = list(range(lo, hi))
             for at in range(0, len(mine), MAX_TILE_BLOCKS_PER_INSTRUCTION):
                 out.append(UpGateProj_GEMM_SiLU(layer, self.batch_size, 0, mine[at : at + MAX_TILE_BLOCKS_PER_INSTRUCTION]))
+        return out
+
+    def upgate_skewed(self, layer: int) -> list[Instruction]:
+        """One instruction (or no-op) per worker, in worker order.  The workers of the O-proj round start their
+        up/gate weights a phase later than the idle ones, whose first blocks stream during that round: they get one
+        block less than an even deal would give them, the others share the rest."""
+        blocks = _ceil_div(self.shape.intermediate_size, TILE_N_GRANULARITY)
+        busy = min(self.workers, len(self.oproj(layer)))
+        idle = self.workers - busy
+        even = blocks // self.workers
+        light = max(even - 1, 0) if idle > 0 else even
+        rest = blocks - light * busy
+        if idle <= 0 or rest > idle * MAX_TILE_BLOCKS_PER_INSTRUCTION:
+            return self.upgate(layer)
+        heavy, extra = divmod(rest, idle)
+        out: list[Instruction] = []
+        at = 0
+        for worker in range(self.workers):
+            n = light if worker < busy else heavy + (1 if worker - busy < extra else 0)
+            out.append(UpGateProj_GEMM_SiLU(layer, self.batch_size, 0, list(range(at, at + n))) if n else NoOp())
+            at += n
+        assert at == blocks
         return out
 
     def downproj(self, layer: int) -> list[Instruction]:
@@ -211,7 +234,7 @@ class BatchScheduler:
             rounds(self.attention_reduction(layer, p))
             rounds(self.oproj(layer))
             rows_round(self.mlp_rms(layer))
-            rounds(self.upgate(layer))
+            rounds(self.upgate_skewed(layer) if self.skew_upgate else self.upgate(layer))
             rounds(self.downproj(layer))
         if layers == self.shape.num_hidden_layers:
             rows_round(self.lmhead_rms())
@@ -235,7 +258,7 @@ def reference_scheduler(batch_size: int, shape: DecodeShape | None = None) -> Ba
 
 
 def mi355x_scheduler(batch_size: int, shape: DecodeShape | None = None, *, merge_in_last: bool = True,
-                     residual_tile: int = 16) -> BatchScheduler:
+                     residual_tile: int = 16, skew_upgate: bool = True) -> BatchScheduler:
     """One queue per CU; the split-KV partials are merged by the last arrival of each head group.
     ``residual_tile`` 8 gives the two projections that add to the residual stream one 8-row block per
     workgroup instead of 16-row blocks on half the CUs; measured slower at batch 8 (every workgroup
@@ -243,4 +266,4 @@ def mi355x_scheduler(batch_size: int, shape: DecodeShape | None = None, *, merge
     if residual_tile not in (8, 16):
         raise ValueError("blocks of the residual projections have 8 or 16 rows")
     return BatchScheduler(shape or LlamaConfig.shape(), MI355X_WORKERS, batch_size, merge_in_last=merge_in_last,
-                          oproj_tile=residual_tile, down_tile=residual_tile)
+                          oproj_tile=residual_tile, down_tile=residual_tile, skew_upgate=skew_upgate)

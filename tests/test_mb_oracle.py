@@ -112,6 +112,22 @@ def test_runtime_template_is_made_of_whole_rounds():
     assert all(i.valid_partials == -1 and i.is_active == -1 for i in flat if i.opcode() == 4)
 
 
+def test_up_gate_blocks_follow_the_o_proj_round():
+    """MI355X template: the workers that ran an O-proj block get one up/gate block less than an even deal, the idle ones
+    share the rest; the reference's deal stays even."""
+    sched = S.mi355x_scheduler(8, MB_FULL)
+    mine = sched.upgate_skewed(0)
+    counts = [len(i.tile_N_block_idxs) if i.opcode() == 7 else 0 for i in mine]
+    busy = len(sched.oproj(0))
+    assert len(mine) == sched.workers and busy == 128
+    assert set(counts[:busy]) == {1} and set(counts[busy:]) == {3} and sum(counts) == MB_FULL.intermediate_size // 16
+    flat = [b for i in mine if i.opcode() == 7 for b in i.tile_N_block_idxs]
+    assert flat == list(range(MB_FULL.intermediate_size // 16))
+    even = [len(i.tile_N_block_idxs) for i in S.reference_scheduler(8, MB_FULL).upgate(0)]
+    assert max(even) - min(even) <= 1
+    assert not S.mi355x_scheduler(8, MB_FULL, skew_upgate=False).skew_upgate
+
+
 @pytest.mark.parametrize("make,rows", [(S.reference_scheduler, 3), (S.mi355x_scheduler, 8), (S.mi355x_scheduler, 16)])
 def test_every_output_once_and_final_counters(make, rows):
     shape = MB_SMALL
