@@ -256,6 +256,7 @@ __global__ __launch_bounds__(kThreads, 1) void decode_megakernel_moe(const Param
   __shared__ Smem<M> s;
   if (threadIdx.x < 8) s.ctl[threadIdx.x] = 0;
   if (threadIdx.x == 0) {
+    s.route_layer = -1;
     s.generation = tagged(p) ? ld_shared32(p.ws + kWsGeneration) : 0u;
     s.best_val = -INFINITY;
     s.best_idx = 0x7fffffff;

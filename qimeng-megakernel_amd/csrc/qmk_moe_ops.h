@@ -469,8 +469,20 @@ __device__ __forceinline__ bool routed_expert(const Params& p, Smem<M>& s, const
 // instruction to announce it: one hand-over less between the O-projection and the expert rows, during which the
 // whole device has nothing else to do.  The top-k instruction still leaves expert_indices / expert_weights for the
 // caller, off the critical path.  False (uniformly) when the wait ran out of polls or the logits have no order.
+// A workgroup takes the decision once per layer: its routed down-projection instruction finds what its routed
+// up/gate instruction of the same layer left in LDS.
 template <class M>
 __device__ __forceinline__ bool routing_decision(const Params& p, Smem<M>& s, const Ctx& c, int layer, int slot, int& eid, float& weight) {
+  static_assert(kMaxTopK <= 8, "the decision kept in LDS has eight slots");
+  if (s.route_layer == layer) {   // (written before the barrier that ended an earlier instruction)
+    eid = s.route_expert[slot];
+    weight = s.route_weight[slot];
+    if (p.timeline != nullptr && c.tid == 0) {
+      s.t_wait = wall_clock64();
+      s.ctl[2] = 1;
+    }
+    return true;
+  }
   uint32_t bits = 0;
   if (c.tid < p.num_experts && !poll_tagged1(p.ws + kWsLogits + c.tid, tag_of(s.generation, layer), p.spin_limit, bits)) {
     s.ctl[0] = 1;
@@ -488,6 +500,11 @@ __device__ __forceinline__ bool routing_decision(const Params& p, Smem<M>& s, co
   for (int j = 0; j < p.top_k; ++j) total += picked[j];
   eid = __float_as_int(picked[kMaxTopK + slot]);
   weight = p.norm_topk ? picked[slot] / total : picked[slot];
+  if (c.tid < p.top_k) {
+    s.route_expert[c.tid] = __float_as_int(picked[kMaxTopK + c.tid]);
+    s.route_weight[c.tid] = p.norm_topk ? picked[c.tid] / total : picked[c.tid];
+  }
+  if (c.tid == 0) s.route_layer = layer;
   __syncthreads();   // picked is read: s.merge and s.res may be reused
   return true;
 }

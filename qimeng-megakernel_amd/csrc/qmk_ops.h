@@ -69,6 +69,10 @@ struct Smem {
   float merge[kWaves][M::GQA][M::D + 4];  // attention state per wave and head: acc[D], m, l
   unsigned long long t_wait;            // timeline: when the last counter wait finished
   unsigned long long stamps[4];         // timeline: op-specific intermediate timestamps
+  // MoE route, tagged launches: the routing decision this workgroup last took from a layer's logits (-1: none yet)
+  int32_t route_layer;
+  int32_t route_expert[8];
+  float route_weight[8];
 };
 
 enum Opcode {

@@ -60,7 +60,7 @@ class MoeScheduler:
     placed: bool = False               # queues() places the instructions of a layer by role instead of dealing them
     down_per_slot: bool = False        # a routed down projection waits for its own slot's up/gate tiles only (tile_M_idx = 1)
     topk_late: bool = False            # placed streams for tagged launches: the consumers take the routing decision themselves,
-                                       # the top-k instruction runs behind its queue's up/gate tiles (it only reports the routing)
+                                       # the top-k instruction runs last in its layer on a queue without a combine instruction (it only reports the routing)
 
     def qkvproj(self, layer: int) -> list[Instruction]:
         tiles = _ceil_div(self.shape.qkv_out_dim, TILE_N_GRANULARITY)
@@ -235,12 +235,17 @@ class MoeScheduler:
             spread(self.shared_downproj(layer), everyone)
         for queue, ins in self._placed_routed_upgate(layer):
             out[queue].append(ins)
-        if self.topk_late:    # behind the queue's up/gate tiles, where it would otherwise wait for its slot's silu vector
-            out[topk_queue] += self.router_softmax_topk(layer)
         if self.interleave_experts:
             spread(self.shared_downproj(layer), everyone)
         spread(self.routed_downproj(layer), everyone)
-        spread(self.combine_commit(layer), everyone[::-1])   # not on the O-projection's queues
+        combine = self.combine_commit(layer)
+        spread(combine, everyone[::-1])   # not on the O-projection's queues
+        if self.topk_late:
+            # Nobody inside the launch waits for it: behind the routed down projection of a queue that has no combine
+            # instruction, where it runs while the others combine (behind the up/gate tiles it held its queue's down
+            # projection back, and with it every combine instruction: 3 us per layer).
+            spare = everyone[0] if len(combine) < len(everyone) else topk_queue
+            out[spare] += self.router_softmax_topk(layer)
 
     def instruction_list(self, num_layers: int | None = None) -> list[Instruction]:
         layers = self.shape.num_hidden_layers if num_layers is None else num_layers
