@@ -162,13 +162,20 @@ __device__ __forceinline__ bool op_router(const Params& p, Smem<M>& s, const Ctx
   const int layer = s.inst[1], g = s.inst[5], e0 = s.inst[2] * g, e1 = min(s.inst[3] * g, p.num_experts);
   if (layer < 0 || layer >= p.num_layers) return bad_operand(p, s, c, 1);
   if (g < 1 || e0 < 0 || e1 < e0) return bad_operand(p, s, c, 2);
-  if (!residual_to_lds<M>(p, s, c, layer)) return false;
   const int lane = c.tid & 63, wave = c.tid >> 6;
   const u16* w = p.router_w + static_cast<size_t>(layer) * p.num_experts * M::H;
+  // The wave's first expert row is asked for before the residual stream is looked at: it lands during the wait.
+  RowSet<1> first;
+  {
+    const u16* const rows[1] = {w + static_cast<size_t>(min(e0 + wave, max(e1 - 1, 0))) * M::H};
+    request_rows<1>(first, rows, M::H, lane, e0 + wave < e1 ? 1 : 0);
+  }
+  if (!residual_to_lds<M>(p, s, c, layer)) return false;
   for (int e = e0 + wave; e < e1; e += kWaves) {
     const u16* const rows[1] = {w + static_cast<size_t>(e) * M::H};
     float v[1];
-    rows_dot<1>(rows, s.x, M::H, lane, v);
+    if (e == e0 + wave) reduce_rows<1>(first, s.x, M::H, lane, v);
+    else rows_dot<1>(rows, s.x, M::H, lane, v);
     if (lane == 0) {
       st_shared_f32(p.router_logits + e, v[0]);
       // tagged launch: the routed up/gate workgroups take the routing decision themselves from these
@@ -648,6 +655,10 @@ __device__ __forceinline__ bool op_combine(const Params& p, Smem<M>& s, const Ct
     uint64_t rt[kMaxTopK];
 #pragma unroll
     for (int k = 0; k < kMaxSlices; ++k) st[k] = k < p.shared_k_slices ? ld_shared32(p.shared_parts + static_cast<size_t>(k) * M::H + r) : 0u;
+    // Tagged launch: the unit the O-projection announced this pair in.  Every up/gate workgroup has seen its
+    // tag, and this instruction follows them through the down projections: no polling — and asked for before the
+    // looks at the routed rows below, so that it does not cost a trip of its own behind them.
+    const uint32_t old = tg ? static_cast<uint32_t>(ld_shared64(p.ws + kWsHiddenMid + r / 2)) : ld_shared32(p.hidden + r);
     if (tg) {
       // two units per slot, all slots in flight together, looked at until every one carries this layer's tag
       const uint64_t* units = p.ws + kWsRoutedParts + r;
@@ -680,9 +691,6 @@ __device__ __forceinline__ bool op_combine(const Params& p, Smem<M>& s, const Ct
 #pragma unroll
       for (int j = 0; j < kMaxTopK; ++j) rt[j] = j < p.top_k ? ld_shared64(p.routed_parts + static_cast<size_t>(j) * M::H + r) : 0ull;
     }
-    // Tagged launch: the unit the O-projection announced this pair in.  Every up/gate workgroup has seen its
-    // tag, and this instruction follows them through the down projections: no polling.
-    const uint32_t old = tg ? static_cast<uint32_t>(ld_shared64(p.ws + kWsHiddenMid + r / 2)) : ld_shared32(p.hidden + r);
     float sh0 = 0.f, sh1 = 0.f;
 #pragma unroll
     for (int k = 0; k < kMaxSlices; ++k) {
