@@ -243,8 +243,9 @@ class MoeScheduler:
         if self.topk_late:
             # Nobody inside the launch waits for it: behind the routed down projection of a queue that has no combine
             # instruction, where it runs while the others combine (behind the up/gate tiles it held its queue's down
-            # projection back, and with it every combine instruction: 3 us per layer).
-            spare = everyone[0] if len(combine) < len(everyone) else topk_queue
+            # projection back, and with it every combine instruction: 3 us per layer) — the last such queue, away from
+            # the first queues, whose next instruction is the next layer's split-KV slice.
+            spare = everyone[len(everyone) - len(combine) - 1] if len(combine) < len(everyone) else topk_queue
             out[spare] += self.router_softmax_topk(layer)
 
     def instruction_list(self, num_layers: int | None = None) -> list[Instruction]:
