@@ -72,7 +72,7 @@ class MoeInstructionVM:
         s = self.shape
         layer, d, tile = ins.layer_idx, s.head_dim, ins.tile_N_granularity
         if layer > 0:
-            assert int(g.barriers[layer - 1, 13, 0]) == s.num_hidden_blocks
+            assert self._layer_complete(g, layer - 1)
         y = rms_norm(g.hidden_states.reshape(-1), g.attn_norm_weights[layer], s.rms_norm_eps).reshape(-1)
         pos = int(g.position_id or 0)
         k_start = s.num_attention_heads * d
@@ -265,6 +265,25 @@ class MoeInstructionVM:
     def routed_expert_downproj(self, g: Any, ins: Any) -> None:
         s, layer = self.shape, ins.layer_idx
         per_slot = s.moe_intermediate_size // getattr(s, "routed_upgate_tile", TILE)
+        if ins.tile_M_idx == 2:
+            # This build's streams for tagged launches without a shared expert: all expert slots of the instruction's
+            # rows and the commit in one — the handler below for every slot in slot order, then opcode 14's arithmetic
+            # on the same rows (`:467-530`).  Such a launch keeps no counters; here the rows committed are counted in
+            # slot 1 of the combine row, in tiles of the instruction's granularity.
+            assert not getattr(s, "has_shared_expert", True) and ins.expert_idx == 0
+            assert int(g.barriers[layer, 11, 0]) == s.num_experts_per_tok * per_slot
+            r0, r1 = ins.tile_N_start_idx * ins.tile_N_granularity, ins.tile_N_end_idx * ins.tile_N_granularity
+            acc = torch.zeros(r1 - r0, dtype=torch.float32)
+            for slot in range(s.num_experts_per_tok):
+                mat = g.expert_down_proj_weights[layer, int(g.expert_indices[slot])].contiguous()
+                vec = g.routed_silu_buffer[slot].reshape(-1).contiguous()
+                acc += _rows(mat, vec, r0, r1).float() * g.expert_weights[slot].to(torch.float32)
+            hidden = g.hidden_states.reshape(-1)
+            hidden[r0:r1] = (hidden[r0:r1].float() + acc).to(hidden.dtype)
+            g.routed_out_f32.reshape(-1)[r0:r1] = 0.0
+            g.barriers[layer, 13, 1] += (r1 - r0) // ins.tile_N_granularity
+            self._commit_tile = ins.tile_N_granularity
+            return
         if ins.tile_M_idx == 1:     # this build's streams: the slot's own tiles are enough
             assert int(g.barriers[layer, 14, ins.expert_idx]) == per_slot
         else:
@@ -278,6 +297,15 @@ class MoeInstructionVM:
             r0, r1 = blk * ins.tile_N_granularity, (blk + 1) * ins.tile_N_granularity
             acc[r0:r1] += _rows(mat, vec, r0, r1).float() * w
             g.barriers[layer, 12, blk] += 1
+
+    def _layer_complete(self, g: Any, layer: int) -> bool:
+        """Every row of the residual stream committed: by opcode 14 (16-row tiles, slot 0 of its counter row) or by
+        opcode 13's committing form (tiles of its own granularity, slot 1)."""
+        s = self.shape
+        if int(g.barriers[layer, 13, 0]) == s.num_hidden_blocks:
+            return True
+        tile = getattr(self, "_commit_tile", TILE)
+        return int(g.barriers[layer, 13, 1]) == s.hidden_size // tile
 
     # ---- 14 ----------------------------------------------------------------------
     def moe_combine_commit(self, g: Any, ins: Any) -> None:
@@ -299,7 +327,7 @@ class MoeInstructionVM:
     # ---- 7 -----------------------------------------------------------------------
     def rms_lmhead_gemv(self, g: Any, ins: Any) -> None:
         s = self.shape
-        assert int(g.barriers[s.num_hidden_layers - 1, 13, 0]) == s.num_hidden_blocks
+        assert self._layer_complete(g, s.num_hidden_layers - 1)
         y = rms_norm(g.hidden_states.reshape(-1), g.lm_head_norm_weights, s.rms_norm_eps)
         for blk in range(ins.start_output_block_idx, ins.end_output_block_idx):
             r0, r1 = blk * ins.tile_N_granularity, (blk + 1) * ins.tile_N_granularity

@@ -179,7 +179,7 @@ __device__ __forceinline__ bool op_router(const Params& p, Smem<M>& s, const Ctx
     if (lane == 0) {
       st_shared_f32(p.router_logits + e, v[0]);
       // tagged launch: the routed up/gate workgroups take the routing decision themselves from these
-      if (tagged(p)) st_tagged(p.ws + kWsLogits + e, __float_as_uint(v[0]), tag_of(s.generation, layer));
+      if (tagged(p)) st_tagged(p.ws + kWsLogits + e * kLogitStride, __float_as_uint(v[0]), tag_of(s.generation, layer));
     }
   }
   const bool publish_row = s.inst[4] != 0;
@@ -271,7 +271,7 @@ __device__ __forceinline__ bool op_topk(const Params& p, Smem<M>& s, const Ctx& 
     // Tagged launch: the logits from their units, like every consumer of the routing decision; nobody inside the
     // launch reads what this instruction writes, so it neither drains its stores nor counts.
     uint32_t bits = 0;
-    if (t < E && !poll_tagged1(p.ws + kWsLogits + t, tag_of(s.generation, layer), p.spin_limit, bits)) {
+    if (t < E && !poll_tagged1(p.ws + kWsLogits + t * kLogitStride, tag_of(s.generation, layer), p.spin_limit, bits)) {
       s.ctl[0] = 1;
       report_error(p, QMK_DEV_WAIT_TIMEOUT, c.inst_idx, c.opcode, t);
     }
@@ -491,7 +491,7 @@ __device__ __forceinline__ bool routing_decision(const Params& p, Smem<M>& s, co
     return true;
   }
   uint32_t bits = 0;
-  if (c.tid < p.num_experts && !poll_tagged1(p.ws + kWsLogits + c.tid, tag_of(s.generation, layer), p.spin_limit, bits)) {
+  if (c.tid < p.num_experts && !poll_tagged1(p.ws + kWsLogits + c.tid * kLogitStride, tag_of(s.generation, layer), p.spin_limit, bits)) {
     s.ctl[0] = 1;
     report_error(p, QMK_DEV_WAIT_TIMEOUT, c.inst_idx, c.opcode, c.tid);
   }
@@ -550,6 +550,107 @@ __device__ __forceinline__ bool op_routed_upgate(const Params& p, Smem<M>& s, co
   return true;
 }
 
+// Opcode 13 with tile_M_idx = 2, an extension of this build for tagged launches of a model without a shared
+// expert: ALL expert slots of the rows [r0, r0 + n) and the combine step in one instruction — the terms
+// bf16(W_down[expert_j][r] . silu_j) * weight_j are added in slot order in fp32 and committed as opcode 14 commits
+// them, hidden[r] = bf16(hidden[r] + routed[r])  (python_vm.py:467-530), so the stream needs no opcode 14 and the
+// routed rows no hand-over of their own.  The decision of every slot comes from the workgroup's own ranking of the
+// router's logits (local routing).
+// Wave j takes expert slot j: it asks for its rows (kRows of kChunks x 512 columns per round: 8 x 2 holds all of an
+// 8-row instruction for an expert width up to 1024; wider experts take 4 x 4 and more rounds), then every lane looks
+// at exactly the units of silu_j its pieces of the rows multiply, all of them in one trip, and keeps them in
+// registers: no LDS copy of the vectors, no barrier between the looks and the dot products, and a wave whose slot
+// was finished early is not held up by a later one.
+template <class M, int kRows, int kChunks>
+__device__ __forceinline__ bool routed_down_commit(const Params& p, Smem<M>& s, const Ctx& c, int layer, int r0, int n) {
+  const int lane = c.tid & 63, wave = c.tid >> 6;
+  const int K = p.moe_ffn;
+  const uint32_t tag = tag_of(s.generation, layer);
+  int first_expert;
+  float first_weight;
+  if (!routing_decision<M>(p, s, c, layer, 0, first_expert, first_weight)) return false;   // leaves all slots in s.route_*
+  const bool live = wave < p.top_k;
+  const u16* const rows = p.expert_down_w + ((static_cast<size_t>(layer) * p.num_experts + (live ? s.route_expert[wave] : 0)) * M::H + r0) * K + lane * 8;
+  v4u w[kRows][kChunks];
+  auto request = [&](int r) {
+    static_for<0, kRows>([&](auto k) {
+      static_for<0, kChunks>([&](auto q) {
+        w[k][q] = v4u{0, 0, 0, 0};
+        if (live && r + k < n && lane * 8 + q * 512 < K)
+          w[k][q] = __builtin_nontemporal_load(reinterpret_cast<const v4u*>(rows + static_cast<size_t>(r + k) * K + q * 512));
+      });
+    });
+  };
+  request(0);
+  // the residual pair this thread commits, from the unit the O-projection announced it in (every up/gate workgroup
+  // has seen its tag): asked for before the looks at the silu vector, not behind them
+  uint32_t old = 0;
+  if (c.tid < n / 2) old = static_cast<uint32_t>(ld_shared64(p.ws + kWsHiddenMid + (r0 + 2 * c.tid) / 2));
+  v4u x[kChunks];   // columns lane*8 + q*512 .. +7 of silu_j: four units of two bf16 each; zeros past the row's end
+  static_for<0, kChunks>([&](auto q) { x[q] = v4u{0, 0, 0, 0}; });
+  if (live) {
+    const uint64_t* units = p.ws + kWsRoutedSilu + wave * 1024 + lane * 4;
+    uint32_t polls = 0;
+    while (true) {
+      uint64_t u[kChunks][4];
+      static_for<0, kChunks>([&](auto q) {
+        static_for<0, 4>([&](auto j) {
+          u[q][j] = static_cast<uint64_t>(tag) << 32;
+          if (lane * 8 + q * 512 < K) u[q][j] = ld_shared64(units + q * 256 + j);
+        });
+      });
+      bool all = true;
+      static_for<0, kChunks>([&](auto q) {
+        static_for<0, 4>([&](auto j) { all = all && static_cast<uint32_t>(u[q][j] >> 32) == tag; });
+        x[q] = v4u{static_cast<uint32_t>(u[q][0]), static_cast<uint32_t>(u[q][1]), static_cast<uint32_t>(u[q][2]), static_cast<uint32_t>(u[q][3])};
+      });
+      if (all) break;
+      if (++polls > p.spin_limit) {
+        s.ctl[0] = 1;   // seen by everybody after the barrier in front of the commit
+        report_error(p, QMK_DEV_WAIT_TIMEOUT, c.inst_idx, c.opcode, wave);
+        break;
+      }
+      __builtin_amdgcn_s_sleep(1);
+    }
+  }
+  if (p.timeline != nullptr && c.tid == 0) {
+    s.t_wait = wall_clock64();
+    s.ctl[2] = 1;
+  }
+  for (int r = 0; r < n; r += kRows) {
+    float v[kRows];
+    static_for<0, kRows>([&](auto k) {
+      float a = 0.f;
+      static_for<0, kChunks>([&](auto q) { a = dot8(w[k][q], x[q], a); });
+      v[k] = wave_sum(a);
+    });
+    if (r + kRows < n) request(r + kRows);
+    if (lane == 0 && live) {
+      const float weight = s.route_weight[wave];
+      static_for<0, kRows>([&](auto k) {
+        if (r + k < n) s.res[wave * n + r + k] = round_bf16(v[k]) * weight;
+      });
+    }
+  }
+  __syncthreads();
+  if (s.ctl[0]) return false;
+  if (c.tid < n / 2) {
+    const int pair = c.tid, r = r0 + 2 * pair;
+    float ro0 = 0.f, ro1 = 0.f;
+    for (int j = 0; j < p.top_k; ++j) {
+      ro0 += s.res[j * n + 2 * pair];
+      ro1 += s.res[j * n + 2 * pair + 1];
+    }
+    const float h0 = (bf_lo(old) + ro0) + 0.f, h1 = (bf_hi(old) + ro1) + 0.f;   // opcode 14's expression without a shared term
+    const uint32_t word = static_cast<uint32_t>(f2bf(h0)) | (static_cast<uint32_t>(f2bf(h1)) << 16);
+    st_shared32(p.hidden + r, word);
+    st_tagged(p.ws + kWsHiddenOut + r / 2, word, tag);
+    st_shared_f32(p.routed_out_f32 + r, 0.f);
+    st_shared_f32(p.routed_out_f32 + r + 1, 0.f);
+  }
+  return true;
+}
+
 // ==================================================================== 13 ==
 // [13, layer, expert_slot, tile_M, n_start, n_end, tile_M_g, tile_N_g]   (python_vm.py:467-489)
 // bf16(W_down[expert][r] . silu[slot]) * weight[slot], fp32, into the slot's own row of the workspace.
@@ -559,6 +660,13 @@ __device__ __forceinline__ bool op_routed_down(const Params& p, Smem<M>& s, cons
   const bool own_slot_only = s.inst[3] == 1;   // tile_M_idx: 0 in the reference's streams
   if (layer < 0 || layer >= p.num_layers) return bad_operand(p, s, c, 1);
   if (slot < 0 || slot >= p.top_k || slot >= p.barrier_slots - 1) return bad_operand(p, s, c, 2);
+  if (s.inst[3] == 2) {   // all slots of the rows and the commit: tagged launches with local routing, no shared expert
+    if (!tagged(p) || !p.local_routing || p.shared_k_slices != 0 || slot != 0) return bad_operand(p, s, c, 3);
+    if ((tile != kTile && tile != kTile / 2) || n0 < 0 || n1 <= n0 || n1 * tile > M::H || (n1 - n0) * tile > kTile) return bad_operand(p, s, c, 5);
+    if ((p.moe_ffn & 7) || p.moe_ffn > kMaxK || p.top_k > kWaves) return bad_operand(p, s, c, 0);   // a wave per slot, <= 4 x 512 columns
+    if (p.moe_ffn <= 1024) return routed_down_commit<M, 8, 2>(p, s, c, layer, n0 * tile, (n1 - n0) * tile);
+    return routed_down_commit<M, 4, 4>(p, s, c, layer, n0 * tile, (n1 - n0) * tile);
+  }
   if (s.inst[3] != 0 && s.inst[3] != 1) return bad_operand(p, s, c, 3);
   if (tile != kTile || n0 < 0 || n1 < n0 || n1 * tile > M::H) return bad_operand(p, s, c, 5);
   if (tagged(p) && (p.moe_ffn & 3)) return bad_operand(p, s, c, 0);   // whole unit pairs

@@ -59,6 +59,8 @@ class MoeScheduler:
     router_span: int = 1               # experts per router instruction
     placed: bool = False               # queues() places the instructions of a layer by role instead of dealing them
     down_per_slot: bool = False        # a routed down projection waits for its own slot's up/gate tiles only (tile_M_idx = 1)
+    commit_in_down: bool = False       # tagged launches without a shared expert: opcode 13 with tile_M_idx = 2 takes all expert slots
+                                       # of 8 rows and commits them (the combine step's arithmetic): no opcode 14 in the stream
     topk_late: bool = False            # placed streams for tagged launches: the consumers take the routing decision themselves,
                                        # the top-k instruction runs last in its layer on a queue without a combine instruction (it only reports the routing)
 
@@ -125,12 +127,18 @@ class MoeScheduler:
                 for lo, hi in _spans(self.shape.num_routed_upgate_blocks, per_expert)]
 
     def routed_downproj(self, layer: int) -> list[Instruction]:
+        if self.commit_in_down:
+            rows = TILE_N_GRANULARITY // 2
+            return [RoutedExpert_DownProj(layer, 0, 2, lo, hi, tile_N_granularity=rows)
+                    for lo, hi in _spans(self.shape.hidden_size // rows, self.sm_count)]
         per_expert = max(1, self.sm_count // self.shape.num_experts_per_tok)
         return [RoutedExpert_DownProj(layer, slot, 1 if self.down_per_slot else 0, lo, hi)
                 for slot in range(self.shape.num_experts_per_tok)
                 for lo, hi in _spans(self.shape.num_hidden_blocks, per_expert)]
 
     def combine_commit(self, layer: int) -> list[Instruction]:
+        if self.commit_in_down:
+            return []
         return [MoE_Combine_Commit(layer, lo, hi) for lo, hi in _spans(self.shape.num_hidden_blocks, self.sm_count)]
 
     def lmhead(self) -> list[Instruction]:
@@ -162,6 +170,10 @@ class MoeScheduler:
         if side * 4 > n:                       # a device too small to set queues aside
             return list(range(n)), list(range(n)), min(n, self.shape.num_oproj_blocks)
         return list(range(n - side)), list(range(n - side, n)), min(n - side, self.shape.num_oproj_blocks)
+
+    def _late_topk_queue(self) -> int:
+        """A queue in the middle: the first ones run the split-KV slices, the last ones the router."""
+        return max(self.sm_count // 2 - 1, 0)
 
     @staticmethod
     def _weighted_sizes(tiles: int, weights: Sequence[int]) -> list[int]:
@@ -222,6 +234,11 @@ class MoeScheduler:
         spread(self.qkvproj(layer), everyone)
         spread(self.attention_split_kv(layer), everyone)
         spread(self.attention_reduction(layer), everyone)
+        if self.topk_late and layer > 0:
+            # The previous layer's reporting top-k: nobody inside the launch waits for it, and this is where a queue
+            # has time — between its QKV rows and its O-projection rows, while the few split-KV workgroups work.
+            # (The router that overwrites the logits it reads cannot start before this queue's O-projection rows.)
+            out[self._late_topk_queue()] += self.router_softmax_topk(layer - 1)
         # without a shared expert nothing runs beside the router: its queues take O-projection rows like everybody else
         spread(self.oproj(layer), main if self.shape.has_shared_expert else everyone)
         router = self.router_gemv(layer)
@@ -238,15 +255,7 @@ class MoeScheduler:
         if self.interleave_experts:
             spread(self.shared_downproj(layer), everyone)
         spread(self.routed_downproj(layer), everyone)
-        combine = self.combine_commit(layer)
-        spread(combine, everyone[::-1])   # not on the O-projection's queues
-        if self.topk_late:
-            # Nobody inside the launch waits for it: behind the routed down projection of a queue that has no combine
-            # instruction, where it runs while the others combine (behind the up/gate tiles it held its queue's down
-            # projection back, and with it every combine instruction: 3 us per layer) — the last such queue, away from
-            # the first queues, whose next instruction is the next layer's split-KV slice.
-            spare = everyone[len(everyone) - len(combine) - 1] if len(combine) < len(everyone) else topk_queue
-            out[spare] += self.router_softmax_topk(layer)
+        spread(self.combine_commit(layer), everyone[::-1])   # not on the O-projection's queues
 
     def instruction_list(self, num_layers: int | None = None) -> list[Instruction]:
         layers = self.shape.num_hidden_layers if num_layers is None else num_layers
@@ -267,6 +276,8 @@ class MoeScheduler:
         if layers == self.shape.num_hidden_layers:
             for i, ins in enumerate(self.lmhead()):
                 out[i % self.sm_count].append(ins)
+        if self.topk_late and layers > 0:      # the last layer's report: the last instruction of its queue
+            out[self._late_topk_queue()] += self.router_softmax_topk(layers - 1)
         return out
 
 

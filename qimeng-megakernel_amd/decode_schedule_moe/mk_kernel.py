@@ -274,14 +274,17 @@ def mi355x_scheduler(shape: Any = None, *, tagged: bool = True) -> _scheduler.Mo
     (Qwen1.5 shape, contexts up to 263: 753 tok/s with 8 partials, against 728 with 16 and 719 with the merge by the
     last split-KV arrival; Qwen3-30B-A3B shape, 4 KV heads, contexts up to 528: 2 partials); a routed down projection
     waits for its own slot only.  ``tagged``: the stream is for launches with QMK_FLAG_TAGGED, where the consumers of
-    the routing decision take it themselves and the top-k instruction runs late in its queue; a launch on counters
-    needs the stream built with ``tagged=False``, whose top-k instruction stands in front of its consumers."""
+    the routing decision take it themselves, the top-k instruction (a report for the caller) runs in the next layer's
+    attention phase, and — without a shared expert — one routed down-projection instruction takes all expert slots of
+    its 8 rows and commits them, so the stream has no combine instructions; a launch on counters needs the stream
+    built with ``tagged=False``: top-k in front of its consumers, down projections per slot, combine instructions."""
     from .model_config import num_partials_for
 
     shape = shape or QwenMoeConfig.shape()
     partials = min(8 if shape.num_key_value_heads > 4 else 2, num_partials_for(MI355X_QUEUES, shape))
     return _scheduler.MoeScheduler(shape, MI355X_QUEUES, partials, interleave_experts=True, merge_in_oproj=True, router_span=8,
-                                   placed=True, down_per_slot=True, topk_late=tagged and not shape.has_shared_expert)
+                                   placed=True, down_per_slot=True, topk_late=tagged and not shape.has_shared_expert,
+                                   commit_in_down=tagged and not shape.has_shared_expert)
 
 
 def build(globs: Globals, mk: Any = None) -> torch.Tensor:

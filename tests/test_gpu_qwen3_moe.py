@@ -82,7 +82,8 @@ BF16_OUT = {"qkvproj": ("qkv_raw",), "attention_split_kv": ("q_post_rope", "k_ca
 def test_the_stream_has_no_shared_expert_instructions():
     for sched in (S.reference_scheduler(SMALL), mk_kernel.mi355x_scheduler(SMALL), mk_kernel.mi355x_scheduler(QWEN3_30B_A3B)):
         opcodes = {ins.opcode() for ins in sched.instruction_list(1)}
-        assert opcodes == {1, 2, 4, 8, 9, 12, 13, 14} | ({3} if not (sched.merge_in_last or sched.merge_in_oproj) else set())
+        # (a stream for tagged launches commits in its routed down projections: no opcode 14)
+        assert opcodes == {1, 2, 4, 8, 9, 12, 13} | (set() if sched.commit_in_down else {14}) | ({3} if not (sched.merge_in_last or sched.merge_in_oproj) else set())
     full = mk_kernel.mi355x_scheduler(QWEN3_30B_A3B)
     tiles = [ins.tile_N_end_idx - ins.tile_N_start_idx for ins in full.routed_upgate(0)]
     per_queue = [sum(i.tile_N_end_idx - i.tile_N_start_idx for i in q if i.opcode() == 12) for q in full.queues(1)]
@@ -94,7 +95,7 @@ def test_the_stream_has_no_shared_expert_instructions():
 def test_one_op_against_the_vm(weights, stage, position):
     """Everything before the op runs on the VM; the op itself on both, from identical state."""
     cpu, gpu = make_pair(weights, position=position)
-    sched = dataclasses.replace(mk_kernel.mi355x_scheduler(SMALL), merge_in_last=False, merge_in_oproj=False)
+    sched = dataclasses.replace(mk_kernel.mi355x_scheduler(SMALL, tagged=False), merge_in_last=False, merge_in_oproj=False)
     vm = MoeInstructionVM(SMALL)
     name = STAGES[stage]
     # the combine step adds what the routed down projections left in the launcher's workspace: both run on both sides then
@@ -144,7 +145,7 @@ def test_streams_without_reduction_instructions(weights, position, partials, mod
     """The O-projection instructions merge the partials of all 32 heads themselves (two items per thread), or the
     last split-KV arrival of a KV head merges its eight heads."""
     cpu, gpu = make_pair(weights, position=position)
-    sched = dataclasses.replace(mk_kernel.mi355x_scheduler(SMALL), num_partials=partials, merge_in_oproj=mode == "oproj",
+    sched = dataclasses.replace(mk_kernel.mi355x_scheduler(SMALL, tagged=False), num_partials=partials, merge_in_oproj=mode == "oproj",
                                 merge_in_last=mode == "last")
     assert not sched.attention_reduction(0)
     vm = MoeInstructionVM(SMALL)
@@ -162,7 +163,7 @@ def test_streams_without_reduction_instructions(weights, position, partials, mod
 
 def test_lm_head_against_the_vm(weights):
     cpu, gpu = make_pair(weights)
-    sched = mk_kernel.mi355x_scheduler(SMALL)
+    sched = mk_kernel.mi355x_scheduler(SMALL, tagged=False)
     cpu.barriers[SMALL.num_hidden_layers - 1, 13, 0] = SMALL.num_hidden_blocks
     sync_state(cpu, gpu)
     MoeInstructionVM(SMALL).run(cpu, sched.lmhead())

@@ -188,18 +188,25 @@ def test_placed_stream_is_the_same_instructions_by_role():
     sched = mi355x_scheduler(FULL, tagged=False)    # the stream for launches on counters: every queue in dependency order
     queues = sched.queues()
     assert len(queues) == 256 and sched.placed
-    # the stream for tagged launches differs in one thing: the top-k instruction, which nobody inside such a launch waits
-    # for, is the last instruction of its layer on a queue that has no combine instruction
+    # The stream for tagged launches of a shape without a shared expert differs in two things: the top-k instruction,
+    # which nobody inside such a launch waits for, runs in the NEXT layer's attention phase (between its queue's QKV rows
+    # and O-projection rows; the last layer's is the queue's last instruction), and one routed down-projection
+    # instruction per 8 rows takes all expert slots and commits them, so there are no combine instructions.
     from qimeng_megakernel_amd.decode_schedule_moe.model_config import QWEN3_30B_A3B
-    assert [tuple(i.padded()) for q in mi355x_scheduler(FULL).queues() for i in q] == [tuple(i.padded()) for q in queues for i in q]   # a shared expert: no late top-k
-    counters, tagged_stream = mi355x_scheduler(QWEN3_30B_A3B, tagged=False).queues(1), mi355x_scheduler(QWEN3_30B_A3B).queues(1)
-    assert Counter(tuple(i.padded()) for q in counters for i in q) == Counter(tuple(i.padded()) for q in tagged_stream for i in q)
+    assert [tuple(i.padded()) for q in mi355x_scheduler(FULL).queues() for i in q] == [tuple(i.padded()) for q in queues for i in q]   # a shared expert: neither
+    counters, tagged_stream = mi355x_scheduler(QWEN3_30B_A3B, tagged=False).queues(2), mi355x_scheduler(QWEN3_30B_A3B).queues(2)
+    same = lambda qs: Counter(tuple(i.padded()) for q in qs for i in q if i.opcode() not in (13, 14))
+    assert same(counters) == same(tagged_stream)
+    assert not any(i.opcode() == 14 for q in tagged_stream for i in q) and sum(i.opcode() == 14 for q in counters for i in q) == 2 * 128
+    down = [i for q in tagged_stream for i in q if i.opcode() == 13]
+    assert len(down) == 2 * 256 and all(i.tile_M_idx == 2 and i.expert_idx == 0 and i.tile_N_granularity == 8 for i in down)
+    assert sorted((i.layer_idx, r) for i in down for r in range(i.tile_N_start_idx * 8, i.tile_N_end_idx * 8)) == \
+        [(layer, r) for layer in range(2) for r in range(QWEN3_30B_A3B.hidden_size)]
     holders = [ql for ql in tagged_stream if any(i.opcode() == 9 for i in ql)]
     assert len(holders) == 1
-    ops = [i.opcode() for i in holders[0] if i.opcode() != 7 and i.padded()[1] == 0]
-    assert ops[-1] == 9 and 13 in ops and 14 not in ops
-    for q, ql in zip(counters, tagged_stream):
-        assert [tuple(i.padded()) for i in q if i.opcode() != 9] == [tuple(i.padded()) for i in ql if i.opcode() != 9]
+    ops = [(i.opcode(), i.padded()[1]) for i in holders[0]]
+    at = ops.index((9, 0))                         # layer 0's report: behind layer 1's QKV rows, ahead of its O-projection rows
+    assert ops[at - 1] == (1, 1) and ops[at + 1] == (4, 1) and ops[-1] == (9, 1)
     key = lambda ins: tuple(ins.padded())
     assert Counter(key(i) for q in queues for i in q) == Counter(key(i) for i in sched.instruction_list())
     phase = {1: 0, 2: 1, 3: 2, 4: 3, 8: 4, 9: 5, 10: 6, 12: 7, 11: 8, 13: 9, 14: 10, 7: 11}

@@ -160,6 +160,24 @@ def test_vm_against_fused_and_final_counters(weights, stream):
     assert float(v.routed_out_f32.abs().max()) == 0.0
 
 
+def test_committing_down_projection_equals_down_projections_plus_combine(weights):
+    """The stream for tagged launches (opcode 13 with tile_M_idx = 2: all expert slots of 8 rows and the commit, no
+    opcode 14; the reporting top-k one layer late) through the VM: every buffer bit for bit what the stream on
+    counters (down projection per slot, combine instructions) leaves, and the rows committed are counted."""
+    a, b = _globs(weights), _globs(weights)
+    classic, fused = mk_kernel.mi355x_scheduler(SMALL, tagged=False), mk_kernel.mi355x_scheduler(SMALL)
+    assert fused.commit_in_down and fused.topk_late and not classic.commit_in_down
+    flat = fused.instruction_list()
+    assert 14 not in {i.opcode() for i in flat} and all(i.tile_M_idx == 2 for i in flat if i.opcode() == 13)
+    MoeInstructionVM(SMALL).run(a, copy.deepcopy(classic.instruction_list()))
+    MoeInstructionVM(SMALL).run(b, copy.deepcopy(flat))
+    for name in ("hidden_states", "logits", "k_cache", "v_cache", "expert_indices", "expert_weights", "routed_out_f32", "attn_out"):
+        assert torch.equal(getattr(a, name), getattr(b, name)), name
+    for layer in range(SMALL.num_hidden_layers):
+        assert int(b.barriers[layer, 13, 0]) == 0 and int(b.barriers[layer, 13, 1]) == SMALL.hidden_size // 8
+    assert sum(1 for q in fused.queues() for i in q if i.opcode() == 9) == SMALL.num_hidden_layers
+
+
 def test_full_size_stream():
     """The stream a request of the full shape runs: 48 layers on 256 queues, 768 routed up/gate tiles of 8 outputs per
     layer dealt three to a queue, one O-projection tile of 8 rows per queue, every queue in dependency order."""
