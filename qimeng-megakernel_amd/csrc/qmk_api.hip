@@ -32,8 +32,22 @@ constexpr int kMaxDevices = 16;
 // {code, workgroup, instruction, opcode, operand}; written only on errors.
 __device__ int32_t g_status[kStatusWords];
 
+// The launch's Params as an instruction sees them: read from the kernel-argument segment through a pointer the
+// compiler cannot look behind, so what an op needs of them is loaded (scalar loads) inside that op and forgotten
+// after it.  Read through the kernel's own by-value parameter, every field is loaded once at the top, outlives the
+// whole instruction loop, and — 100 pointers against 100 scalar registers — is parked in vector-register lanes:
+// one v_readlane per use, an eighth of all instructions of the MoE kernels (Qwen1.5-MoE shape +4.1 % tok/s,
+// Qwen3-30B-A3B +3 %, Qwen3-1.7B +1.8 %; the Llama-3.2-1B kernel, whose by-value form parks a quarter as many,
+// loses 1.7 % and keeps that form: M::PARAMS_PER_INSTRUCTION).
+__device__ __forceinline__ const Params& params_of_this_instruction() {
+  auto args = __builtin_amdgcn_kernarg_segment_ptr();   // (a pointer into the constant address space)
+  asm volatile("" : "+s"(args));
+  return *(const Params*)args;   // the only kernel argument: offset 0 of the segment
+}
+
 template <class M>
-__global__ __launch_bounds__(kThreads, 1) void decode_megakernel(const Params p) {
+__global__ __launch_bounds__(kThreads, 1) void decode_megakernel(const Params p_launch) {
+  const Params& p = p_launch;
   __shared__ Smem<M> s;
   if (threadIdx.x < 8) s.ctl[threadIdx.x] = 0;
   if (threadIdx.x == 0) {
@@ -52,14 +66,16 @@ __global__ __launch_bounds__(kThreads, 1) void decode_megakernel(const Params p)
   Carried carry;
   bool carried = false, after_attention = false;
   forget(carry);
-  for (int i = 0; i < p.num_insts && ok; ++i) {
+  const int num_insts = p.num_insts;
+  for (int i = 0; i < num_insts && ok; ++i) {
     if (threadIdx.x < kInstWords) {
       s.inst[threadIdx.x] = word;
       s.next[threadIdx.x] = word1;
       word = word1;
-      word1 = (i + 2 < p.num_insts) ? queue[(i + 2) * kInstWords + threadIdx.x] : 0;
+      word1 = (i + 2 < num_insts) ? queue[(i + 2) * kInstWords + threadIdx.x] : 0;
     }
     __syncthreads();
+    const Params& p = M::PARAMS_PER_INSTRUCTION ? params_of_this_instruction() : p_launch;
     const int opcode = s.inst[0];
     int tid = threadIdx.x;
     asm volatile("" : "+v"(tid));
@@ -252,7 +268,8 @@ __global__ __launch_bounds__(kThreads, 1) void decode_megakernel_batch(const Par
 // The MoE route's interpreter: the dense route's attention and LM head (opcodes 1-4, 7) and the MoE
 // block (8-14) on the reference's counters (…/qwen1_5_moe_a2_7b/A100/single_batch/decode_kernel/mk.cu).
 template <class M>
-__global__ __launch_bounds__(kThreads, 1) void decode_megakernel_moe(const Params p) {
+__global__ __launch_bounds__(kThreads, 1) void decode_megakernel_moe(const Params p_launch) {
+  const Params& p = p_launch;
   __shared__ Smem<M> s;
   if (threadIdx.x < 8) s.ctl[threadIdx.x] = 0;
   if (threadIdx.x == 0) {
@@ -268,14 +285,16 @@ __global__ __launch_bounds__(kThreads, 1) void decode_megakernel_moe(const Param
   int32_t word1 = (threadIdx.x < kInstWords && p.num_insts > 1) ? queue[kInstWords + threadIdx.x] : 0;
   Carried carry;
   forget(carry);
-  for (int i = 0; i < p.num_insts && ok; ++i) {
+  const int num_insts = p.num_insts;
+  for (int i = 0; i < num_insts && ok; ++i) {
     if (threadIdx.x < kInstWords) {
       s.inst[threadIdx.x] = word;
       s.next[threadIdx.x] = word1;
       word = word1;
-      word1 = (i + 2 < p.num_insts) ? queue[(i + 2) * kInstWords + threadIdx.x] : 0;
+      word1 = (i + 2 < num_insts) ? queue[(i + 2) * kInstWords + threadIdx.x] : 0;
     }
     __syncthreads();
+    const Params& p = params_of_this_instruction();
     const int opcode = s.inst[0];
     int tid = threadIdx.x;
     asm volatile("" : "+v"(tid));

@@ -324,7 +324,8 @@ constexpr int kWsLogits = kWsUnits;                   // router logits, one fp32
 constexpr int kLogitStride = 16;
 constexpr int kWsRoutedSilu = kWsLogits + 512 * kLogitStride;        // silu vectors of the routed experts: 1024 units (2048 values) per slot
 constexpr int kWsRoutedParts = kWsRoutedSilu + 8 * 1024;   // weighted down-projection rows of the routed experts: H fp32 units per slot
-constexpr int kWsMoeUnits = kWsRoutedParts + 8 * 2048;
+constexpr int kWsSharedGate = kWsRoutedParts + 8 * 2048;   // the shared expert's sigmoid gate, fp32 (a line of its own)
+constexpr int kWsMoeUnits = kWsSharedGate + 16;
 
 __device__ __forceinline__ bool tagged(const Params& p) { return (p.flags & QMK_FLAG_TAGGED) != 0; }
 __device__ __forceinline__ uint32_t tag_of(uint32_t generation, int layer) { return (generation << 6) + static_cast<uint32_t>(layer) + 1u; }

@@ -191,7 +191,11 @@ __device__ __forceinline__ bool op_router(const Params& p, Smem<M>& s, const Ctx
       const u16* const rows[1] = {p.shared_scale_w + static_cast<size_t>(layer) * M::H};
       float v[1];
       rows_dot<1>(rows, s.x, M::H, lane, v);
-      if (lane == 0) st_shared_f32(p.shared_gate, 1.0f / (1.0f + expf(-v[0])));
+      if (lane == 0) {
+        const float gate = 1.0f / (1.0f + expf(-v[0]));
+        st_shared_f32(p.shared_gate, gate);
+        if (tagged(p)) st_tagged(p.ws + kWsSharedGate, __float_as_uint(gate), tag_of(s.generation, layer));
+      }
     }
   }
   release_stores();
@@ -754,7 +758,21 @@ __device__ __forceinline__ bool op_combine(const Params& p, Smem<M>& s, const Ct
   }
   __syncthreads();
   if (s.ctl[0]) return false;
-  const float gate = p.shared_k_slices > 0 ? ld_shared_f32(p.shared_gate) : 0.f;   // left by the layer's publishing router instruction
+  // left by the layer's publishing router instruction: behind the router counter that the top-k instruction waited
+  // for, or, in a tagged launch, in a unit of its own
+  float gate = 0.f;
+  if (p.shared_k_slices > 0) {
+    if (tg) {
+      uint32_t bits = 0;
+      if (!poll_tagged1(p.ws + kWsSharedGate, tag, p.spin_limit, bits)) {
+        s.ctl[0] = 1;   // seen by everybody behind the barrier below
+        report_error(p, QMK_DEV_WAIT_TIMEOUT, c.inst_idx, c.opcode, c.tid);
+      }
+      gate = __uint_as_float(bits);
+    } else {
+      gate = ld_shared_f32(p.shared_gate);
+    }
+  }
   constexpr int kMaxSlices = 16;   // the launcher's bound on shared_k_slices
   for (int pair = c.tid; pair < nb * tile / 2; pair += kThreads) {
     const int r = n0 * tile + 2 * pair;

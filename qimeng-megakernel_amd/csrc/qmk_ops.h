@@ -29,6 +29,7 @@ struct Llama1B {
   static constexpr bool QKV_BIAS = false;
   static constexpr int REDUCE_HEADS = GQA;  // query heads one reduction instruction merges
   static constexpr int PREV_ROW = 5;        // counter row that completes a layer: the down projection's
+  static constexpr bool PARAMS_PER_INSTRUCTION = false;  // launch parameters re-read from the argument segment by every instruction (measured)
 };
 
 // Qwen3-1.7B shape with the Qwen3 op set: opcode 1 leaves the raw QKV vector, the attention
@@ -50,6 +51,7 @@ struct Qwen3_1p7B {
   static constexpr bool QKV_BIAS = false;
   static constexpr int REDUCE_HEADS = GQA;
   static constexpr int PREV_ROW = 5;
+  static constexpr bool PARAMS_PER_INSTRUCTION = true;
 };
 
 constexpr int kResSlots = 4096;

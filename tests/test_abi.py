@@ -102,8 +102,8 @@ def test_host_side_argument_errors(lib):
     m.model = 2
     assert lib.qmk_decode_step_moe(ctypes.byref(m)) == 1
     # the shared expert's K-slice terms, the routed experts' rows, the gate's line, the dense route's units, then the MoE route's
-    # own units (router logits, one per 128-byte line; routed silu vectors; routed rows)
-    moe_units = 8 * (512 * 16 + 8 * 1024 + 8 * 2048)
+    # own units (router logits, one per 128-byte line; routed silu vectors; routed rows; the shared expert's gate)
+    moe_units = 8 * (512 * 16 + 8 * 1024 + 8 * 2048 + 16)
     assert lib.qmk_moe_workspace_bytes(4, 4) == 4 * 2048 * 2 + 4 * 2048 * 4 + 128 + lib.qmk_workspace_bytes(0) + moe_units
     assert lib.qmk_moe_workspace_bytes(8, 0) == 8 * 2048 * 4 + 128 + lib.qmk_workspace_bytes(0) + moe_units     # no shared expert
     assert lib.qmk_moe_workspace_bytes(9, 4) == 0
