@@ -267,12 +267,14 @@ def call_mk(globs: Globals, mk: Any) -> None:
        g.position_id if g.position_id is not None else 0, 1.0 / math.sqrt(s.head_dim), float(s.rms_norm_eps))
 
 
-def mi355x_scheduler(shape: Any = None, *, tagged: bool = True) -> _scheduler.MoeScheduler:
+def mi355x_scheduler(shape: Any = None, *, tagged: bool = True, kv_capacity: int | None = None) -> _scheduler.MoeScheduler:
     """One queue per CU; both up/gate phases ahead of both down projections; the instructions of a layer placed
     by role (the queues of the router and the top-k take no shared up/gate rows); eight experts per router
     instruction; few split-KV partials per KV head, merged by the O-projection workgroups themselves
     (Qwen1.5 shape, contexts up to 263: 753 tok/s with 8 partials, against 728 with 16 and 719 with the merge by the
-    last split-KV arrival; Qwen3-30B-A3B shape, 4 KV heads, contexts up to 528: 2 partials); a routed down projection
+    last split-KV arrival; Qwen3-30B-A3B shape, 4 KV heads: 2 partials, 4 when the request's cache holds more than 256
+    tokens — a 512-token request: 492 against 487 tok/s, 3 % at its long end; 6 and 8 cost the O-projection a second
+    round of partial reads); a routed down projection
     waits for its own slot only.  ``tagged``: the stream is for launches with QMK_FLAG_TAGGED, where the consumers of
     the routing decision take it themselves, the top-k instruction (a report for the caller) runs in the next layer's
     attention phase, and — without a shared expert — one routed down-projection instruction takes all expert slots of
@@ -281,7 +283,8 @@ def mi355x_scheduler(shape: Any = None, *, tagged: bool = True) -> _scheduler.Mo
     from .model_config import num_partials_for
 
     shape = shape or QwenMoeConfig.shape()
-    partials = min(8 if shape.num_key_value_heads > 4 else 2, num_partials_for(MI355X_QUEUES, shape))
+    few = 2 if kv_capacity is None or kv_capacity <= 256 else 4
+    partials = min(8 if shape.num_key_value_heads > 4 else few, num_partials_for(MI355X_QUEUES, shape))
     return _scheduler.MoeScheduler(shape, MI355X_QUEUES, partials, interleave_experts=True, merge_in_oproj=True, router_span=8,
                                    placed=True, down_per_slot=True, topk_late=tagged and not shape.has_shared_expert,
                                    commit_in_down=tagged and not shape.has_shared_expert)
@@ -293,7 +296,7 @@ def build(globs: Globals, mk: Any = None) -> torch.Tensor:
     tagged = True
     if isinstance(mk, MoeMegaKernel):
         tagged = mk.tagged and mk.reset_barriers and QwenMoeConfig.shape().num_hidden_layers <= 63 and mk.local_routing is not False
-    sched = mi355x_scheduler(tagged=tagged)
+    sched = mi355x_scheduler(tagged=tagged, kv_capacity=int(globs.k_cache.shape[2]))
     if sched.num_partials > int(globs.attn_lse_intermediates.shape[-1]):
         raise ValueError("attn_lse_intermediates has fewer partial slots than the schedule's split-KV fan-out")
     return tensorize_instructions(globs, sched.queues())
