@@ -129,8 +129,10 @@ class MoeScheduler:
     def routed_downproj(self, layer: int) -> list[Instruction]:
         if self.commit_in_down:
             rows = TILE_N_GRANULARITY // 2
+            tiles = self.shape.hidden_size // rows
+            # an instruction commits at most 16 rows: with fewer than tiles / 2 queues a queue gets several
             return [RoutedExpert_DownProj(layer, 0, 2, lo, hi, tile_N_granularity=rows)
-                    for lo, hi in _spans(self.shape.hidden_size // rows, self.sm_count)]
+                    for lo, hi in _spans(tiles, max(self.sm_count, _ceil_div(tiles, 2)))]
         per_expert = max(1, self.sm_count // self.shape.num_experts_per_tok)
         return [RoutedExpert_DownProj(layer, slot, 1 if self.down_per_slot else 0, lo, hi)
                 for slot in range(self.shape.num_experts_per_tok)

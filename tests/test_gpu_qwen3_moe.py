@@ -291,6 +291,32 @@ def test_tagged_and_counter_modes_agree_bit_for_bit(weights):
         assert torch.equal(getattr(out[0][0], name), getattr(out[1][0], name)), name
 
 
+def test_committing_down_projection_of_sixteen_rows(weights):
+    """The tagged stream on 128 queues: every committing down-projection instruction takes two tiles of 8 rows (the
+    most the op accepts).  Same bits as the 256-queue stream, whose instructions take one."""
+    from qimeng_megakernel_amd.decode_schedule.instructions.scheduler import tensorize_instructions
+
+    out = []
+    for queues in (256, 128):
+        g = synthetic.build_moe_globals(weights, SMALL, 64, "cuda:0", max_partials=8)
+        sched = dataclasses.replace(mk_kernel.mi355x_scheduler(SMALL), sm_count=queues)
+        rows = {i.tile_N_granularity * (i.tile_N_end_idx - i.tile_N_start_idx) for q in sched.queues() for i in q if i.opcode() == 13}
+        assert rows == ({8} if queues == 256 else {16})
+        tensorize_instructions(g, sched.queues())
+        mk = mk_kernel.get_mk(spin_limit=1 << 18)
+        tok, toks = 7, []
+        for pos in range(12):
+            g.hidden_states.copy_(g.embed_tokens[tok]); g.position_id = pos
+            mk_kernel.call_mk(g, mk)
+            tok = int(g.logits.argmax()); toks.append(tok)
+        mk.check()
+        assert mk._tagged and int(g.instructions.shape[0]) == queues
+        out.append((g, toks))
+    assert out[0][1] == out[1][1]
+    for name in ("hidden_states", "logits", "k_cache", "v_cache", "expert_indices", "expert_weights"):
+        assert torch.equal(getattr(out[0][0], name), getattr(out[1][0], name)), name
+
+
 def test_decode_loop_and_graph(weights):
     g = synthetic.build_moe_globals(weights, SMALL, 64, "cuda:0", max_partials=8)
     prompt = torch.tensor([3, 99, 1024, 7])

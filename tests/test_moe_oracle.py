@@ -202,6 +202,11 @@ def test_placed_stream_is_the_same_instructions_by_role():
     assert len(down) == 2 * 256 and all(i.tile_M_idx == 2 and i.expert_idx == 0 and i.tile_N_granularity == 8 for i in down)
     assert sorted((i.layer_idx, r) for i in down for r in range(i.tile_N_start_idx * 8, i.tile_N_end_idx * 8)) == \
         [(layer, r) for layer in range(2) for r in range(QWEN3_30B_A3B.hidden_size)]
+    import dataclasses
+    for fewer in (128, 100):                       # fewer queues: one or two tiles of 8 rows per committing instruction, never more
+        spans = [i.tile_N_end_idx - i.tile_N_start_idx for q in dataclasses.replace(mi355x_scheduler(QWEN3_30B_A3B), sm_count=fewer).queues(1)
+                 for i in q if i.opcode() == 13]
+        assert sum(spans) == QWEN3_30B_A3B.hidden_size // 8 and set(spans) <= {1, 2}
     # split-KV slices per KV head of that shape: 2, 4 for a request whose cache holds more than 256 tokens
     assert [mi355x_scheduler(QWEN3_30B_A3B, kv_capacity=c).num_partials for c in (None, 64, 256, 257, 528)] == [2, 2, 2, 4, 4]
     assert mi355x_scheduler(FULL, kv_capacity=1040).num_partials == 8
