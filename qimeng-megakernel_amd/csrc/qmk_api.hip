@@ -37,8 +37,10 @@ __device__ int32_t g_status[kStatusWords];
 // after it.  Read through the kernel's own by-value parameter, every field is loaded once at the top, outlives the
 // whole instruction loop, and — 100 pointers against 100 scalar registers — is parked in vector-register lanes:
 // one v_readlane per use, an eighth of all instructions of the MoE kernels (Qwen1.5-MoE shape +4.1 % tok/s,
-// Qwen3-30B-A3B +3 %, Qwen3-1.7B +1.8 %; the Llama-3.2-1B kernel, whose by-value form parks a quarter as many,
-// loses 1.7 % and keeps that form: M::PARAMS_PER_INSTRUCTION).
+// Qwen3-30B-A3B +3 %).  The dense kernels park a quarter as many, and there it depends on the op: the up/gate GEMV
+// loses 2 % this way (its first row requests wait for the scalar loads), the O-projection gains; which ops of a
+// dense kernel read the segment is M::PARAMS_FROM_SEGMENT, measured op by op (Llama-3.2-1B +0.7 %, Qwen3-1.7B +2.7 %
+// against all by value).
 __device__ __forceinline__ const Params& params_of_this_instruction() {
   auto args = __builtin_amdgcn_kernarg_segment_ptr();   // (a pointer into the constant address space)
   asm volatile("" : "+s"(args));
@@ -75,7 +77,8 @@ __global__ __launch_bounds__(kThreads, 1) void decode_megakernel(const Params p_
       word1 = (i + 2 < num_insts) ? queue[(i + 2) * kInstWords + threadIdx.x] : 0;
     }
     __syncthreads();
-    const Params& p = M::PARAMS_PER_INSTRUCTION ? params_of_this_instruction() : p_launch;
+    const Params& from_segment = params_of_this_instruction();
+    auto params_for = [&](int op) -> const Params& { return (M::PARAMS_FROM_SEGMENT & op) ? from_segment : p; };
     const int opcode = s.inst[0];
     int tid = threadIdx.x;
     asm volatile("" : "+v"(tid));
@@ -88,16 +91,16 @@ __global__ __launch_bounds__(kThreads, 1) void decode_megakernel(const Params p_
     // Only the O-proj hands rows to its successor: every other arm ends their life explicitly.
     switch (opcode) {
       case OP_NOOP: forget(carry); break;
-      case OP_RMS_QKV_ROPE: [[clang::always_inline]] ok = op_rms_qkv_rope<M>(p, s, c); forget(carry); break;
-      case OP_ATTN_SPLITKV: [[clang::always_inline]] ok = op_attn_splitkv<M>(p, s, c); forget(carry); break;
+      case OP_RMS_QKV_ROPE: [[clang::always_inline]] ok = op_rms_qkv_rope<M>(params_for(kSegmentQkv), s, c); forget(carry); break;
+      case OP_ATTN_SPLITKV: [[clang::always_inline]] ok = op_attn_splitkv<M>(params_for(kSegmentAttention), s, c); forget(carry); break;
       case OP_ATTN_REDUCE: [[clang::always_inline]] ok = op_attn_reduce<M>(p, s, c); forget(carry); break;
       case OP_OPROJ_RESIDUAL:
         carried = M::CARRY_AFTER_ATTENTION || !after_attention;
-        [[clang::always_inline]] ok = op_oproj_residual<M>(p, s, c, carry, carried);
+        [[clang::always_inline]] ok = op_oproj_residual<M>(params_for(kSegmentOproj), s, c, carry, carried);
         break;
-      case OP_RMS_UPGATE_SILU: [[clang::always_inline]] ok = op_rms_upgate_silu<M>(p, s, c, carry, carried); forget(carry); break;
-      case OP_DOWN_RESIDUAL: [[clang::always_inline]] ok = op_down_residual<M>(p, s, c); forget(carry); break;
-      case OP_RMS_LMHEAD: [[clang::always_inline]] ok = op_rms_lmhead<M>(p, s, c); forget(carry); break;
+      case OP_RMS_UPGATE_SILU: [[clang::always_inline]] ok = op_rms_upgate_silu<M>(params_for(kSegmentUpGate), s, c, carry, carried); forget(carry); break;
+      case OP_DOWN_RESIDUAL: [[clang::always_inline]] ok = op_down_residual<M>(params_for(kSegmentDown), s, c); forget(carry); break;
+      case OP_RMS_LMHEAD: [[clang::always_inline]] ok = op_rms_lmhead<M>(params_for(kSegmentLmHead), s, c); forget(carry); break;
       default:
         if (threadIdx.x == 0) report_error(p, QMK_DEV_BAD_OPCODE, i, opcode, 0);
         ok = false;
