@@ -208,7 +208,7 @@ int qmk_decode_step(const QmkArgs* args);
  * capture, tight serving loops, harnesses that forbid hipMalloc.  Everything is as in
  * qmk_decode_step (same struct, same kernels, same results bit for bit), except that
  * args->workspace and args->workspace_bytes are ignored: the tagged units, the greedy candidates
- * and the launch count live in a static device array of the library (94 336 bytes per GPU, held
+ * and the launch count live in a static device array of the library (94 208 bytes per GPU, held
  * until the process ends; its address is looked up once per device on the first call of any entry
  * point there).  Limits of that array: at most 1024 queues when token_out is set and at most 63
  * layers with QMK_FLAG_TAGGED -- beyond them the call returns QMK_ERR_SCRATCH and launches nothing.

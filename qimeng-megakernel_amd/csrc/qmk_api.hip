@@ -19,7 +19,7 @@
 
 // Workspace of qmk_decode_step_static: the tagged units, the greedy candidates and the launch count
 // that qmk_decode_step keeps in the caller's QmkArgs.workspace, here in an array of the library's own
-// (94 336 bytes per device, held until the process ends), so that the entry point allocates nothing.
+// (94 208 bytes per device, held until the process ends), so that the entry point allocates nothing.
 // In host code the name is only a handle for hipGetSymbolAddress: the kernels get the device address
 // that call returned (DeviceInfo::scratch), once per device.
 static __device__ __align__(256) unsigned long long scratch[qmk::kWsUnits];

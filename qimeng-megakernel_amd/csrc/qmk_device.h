@@ -312,8 +312,7 @@ constexpr int kWsHiddenOut = kWsHiddenMid + 1024;  // residual stream after the 
 constexpr int kWsSilu = kWsHiddenOut + 1024;        // silu_out: F/2 units (room for F = 8192)
 constexpr int kWsCandidates = kWsSilu + 4096;       // one greedy candidate per workgroup: {logit bits, row}
 constexpr int kMaxSamplingQueues = 1024;
-constexpr int kWsExperts = kWsCandidates + kMaxSamplingQueues;   // MoE route: the top-k's experts, then their weights (8 units each)
-constexpr int kWsUnits = kWsExperts + 16;
+constexpr int kWsUnits = kWsCandidates + kMaxSamplingQueues;
 // MoE route only, behind the regions above (its workspace is sized by qmk_moe_workspace_bytes):
 constexpr int kWsLogits = kWsUnits;                   // router logits, one fp32 per unit (room for 512 experts)
 // One router logit per 128-byte line: 128 threads of every workgroup look at the logits from the end of the
@@ -325,7 +324,8 @@ constexpr int kLogitStride = 16;
 constexpr int kWsRoutedSilu = kWsLogits + 512 * kLogitStride;        // silu vectors of the routed experts: 1024 units (2048 values) per slot
 constexpr int kWsRoutedParts = kWsRoutedSilu + 8 * 1024;   // weighted down-projection rows of the routed experts: H fp32 units per slot
 constexpr int kWsSharedGate = kWsRoutedParts + 8 * 2048;   // the shared expert's sigmoid gate, fp32 (a line of its own)
-constexpr int kWsMoeUnits = kWsSharedGate + 16;
+constexpr int kWsTopK = kWsSharedGate + 16;                // the top-k's picks: slot j's expert and weight side by side at 16 j (a line per slot)
+constexpr int kWsMoeUnits = kWsTopK + 8 * 16;
 
 __device__ __forceinline__ bool tagged(const Params& p) { return (p.flags & QMK_FLAG_TAGGED) != 0; }
 __device__ __forceinline__ uint32_t tag_of(uint32_t generation, int layer) { return (generation << 6) + static_cast<uint32_t>(layer) + 1u; }

@@ -300,8 +300,8 @@ __device__ __forceinline__ bool op_topk(const Params& p, Smem<M>& s, const Ctx& 
       __hip_atomic_store(p.expert_indices + j, static_cast<long long>(idx), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
       st_shared_f32(p.expert_weights + j, w);
       if (tg && !p.local_routing) {   // the routed ops poll these: one trip, no drain in between
-        st_tagged(p.ws + kWsExperts + j, static_cast<uint32_t>(idx), tag_of(s.generation, layer));
-        st_tagged(p.ws + kWsExperts + kMaxTopK + j, __float_as_uint(w), tag_of(s.generation, layer));
+        st_tagged(p.ws + kWsTopK + 16 * j, static_cast<uint32_t>(idx), tag_of(s.generation, layer));
+        st_tagged(p.ws + kWsTopK + 16 * j + 1, __float_as_uint(w), tag_of(s.generation, layer));
       }
     }
   }
@@ -444,8 +444,8 @@ __device__ __forceinline__ int expert_of(const Params& p, int slot) {
 }
 
 // Wait for the layer's top-k and fetch a slot's expert (negative: not an expert of the layer) and weight:
-// through the counter and the caller's buffers, or, in a tagged launch, from the two units the top-k
-// instruction announces them in.  False (uniformly) when the wait ran out of polls.
+// through the counter and the caller's buffers, or, in a tagged launch, from the two neighbouring units the top-k
+// instruction announces them in (one look for both; a line per slot).  False (uniformly) when the wait ran out of polls.
 template <class M>
 __device__ __forceinline__ bool routed_expert(const Params& p, Smem<M>& s, const Ctx& c, int layer, int slot, int& eid, float& weight) {
   if (!tagged(p)) {
@@ -457,7 +457,7 @@ __device__ __forceinline__ bool routed_expert(const Params& p, Smem<M>& s, const
   if (c.tid == 0) {
     uint32_t e = 0, w = 0;
     const uint32_t tag = tag_of(s.generation, layer);
-    if (!poll_tagged1(p.ws + kWsExperts + slot, tag, p.spin_limit, e) || !poll_tagged1(p.ws + kWsExperts + kMaxTopK + slot, tag, p.spin_limit, w)) {
+    if (!poll_tagged2(p.ws + kWsTopK + 16 * slot, tag, p.spin_limit, e, w)) {   // expert and weight in one trip
       s.ctl[0] = 1;
       report_error(p, QMK_DEV_WAIT_TIMEOUT, c.inst_idx, c.opcode, slot);
     }

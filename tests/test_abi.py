@@ -79,7 +79,7 @@ def test_host_side_argument_errors(lib):
     assert lib.qmk_decode_step(ctypes.byref(a)) == 8                       # QMK_ERR_MODEL
     a.model = 0
     assert lib.qmk_decode_step(ctypes.byref(a)) == 1                       # all tensor pointers are NULL
-    assert lib.qmk_workspace_bytes(0) == 8 * (512 + 2048 + 4 * 1024 + 4096 + 1024 + 16) and lib.qmk_workspace_bytes(1) == lib.qmk_workspace_bytes(0) and lib.qmk_workspace_bytes(7) == 0
+    assert lib.qmk_workspace_bytes(0) == 8 * (512 + 2048 + 4 * 1024 + 4096 + 1024) and lib.qmk_workspace_bytes(1) == lib.qmk_workspace_bytes(0) and lib.qmk_workspace_bytes(7) == 0
     assert lib.qmk_query(0) == 8 and lib.qmk_query(2) == 512 and lib.qmk_query(5) == 32 and lib.qmk_query(6) == 25
     assert 0 < lib.qmk_query(3) <= 160 * 1024
     assert lib.qmk_error_string(34).decode().startswith("device: counter wait")
@@ -102,8 +102,9 @@ def test_host_side_argument_errors(lib):
     m.model = 2
     assert lib.qmk_decode_step_moe(ctypes.byref(m)) == 1
     # the shared expert's K-slice terms, the routed experts' rows, the gate's line, the dense route's units, then the MoE route's
-    # own units (router logits, one per 128-byte line; routed silu vectors; routed rows; the shared expert's gate)
-    moe_units = 8 * (512 * 16 + 8 * 1024 + 8 * 2048 + 16)
+    # own units (router logits, one per 128-byte line; routed silu vectors; routed rows; the shared expert's gate; the top-k's
+    # picks, a line per slot)
+    moe_units = 8 * (512 * 16 + 8 * 1024 + 8 * 2048 + 16 + 8 * 16)
     assert lib.qmk_moe_workspace_bytes(4, 4) == 4 * 2048 * 2 + 4 * 2048 * 4 + 128 + lib.qmk_workspace_bytes(0) + moe_units
     assert lib.qmk_moe_workspace_bytes(8, 0) == 8 * 2048 * 4 + 128 + lib.qmk_workspace_bytes(0) + moe_units     # no shared expert
     assert lib.qmk_moe_workspace_bytes(9, 4) == 0
