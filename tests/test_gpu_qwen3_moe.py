@@ -317,6 +317,31 @@ def test_committing_down_projection_of_sixteen_rows(weights):
         assert torch.equal(getattr(out[0][0], name), getattr(out[1][0], name)), name
 
 
+@pytest.mark.parametrize("bad, operand, tagged", [
+    (S.RoutedExpert_DownProj(0, 0, 2, 0, 1, tile_N_granularity=8), 3, False),     # the committing form in a launch on counters
+    (S.RoutedExpert_DownProj(0, 1, 2, 0, 1, tile_N_granularity=8), 3, True),      # ... names a slot: it takes all of them
+    (S.RoutedExpert_DownProj(0, 0, 2, 0, 3, tile_N_granularity=8), 5, True),      # more than 16 rows
+    (S.RoutedExpert_DownProj(0, 0, 2, 0, 1, tile_N_granularity=4), 5, True),      # tiles of 8 or 16 rows only
+    (S.RoutedExpert_DownProj(0, 0, 2, 256, 257, tile_N_granularity=8), 5, True),  # rows beyond the hidden size
+    (S.RoutedExpert_DownProj(0, 0, 3, 0, 1), 3, True),                            # no such form
+])
+def test_bad_committing_instructions_are_rejected_on_the_device(weights, bad, operand, tagged):
+    """Error paths forced from the host: the kernel refuses the instruction before it writes anything and exits normally."""
+    _, gpu = make_pair(weights)
+    names = ("hidden_states", "routed_out_f32", "routed_silu_buffer", "k_cache", "logits")
+    before = {n: getattr(gpu, n).clone() for n in names}
+    from qimeng_megakernel_amd.decode_schedule.instructions.scheduler import tensorize_instructions
+
+    tensorize_instructions(gpu, S.deal([copy.deepcopy(bad)], 8))
+    mk = mk_kernel.get_mk(spin_limit=1 << 10) if tagged else mk_kernel.get_mk(reset_barriers=False, spin_limit=1 << 10)
+    mk_kernel.call_mk(gpu, mk)
+    with pytest.raises(RuntimeError, match="operand out of bounds") as err:
+        mk.check()
+    assert mk._tagged == tagged and "opcode=13" in str(err.value) and f"operand={operand}" in str(err.value)
+    for n, t in before.items():
+        assert torch.equal(getattr(gpu, n), t), n
+
+
 def test_decode_loop_and_graph(weights):
     g = synthetic.build_moe_globals(weights, SMALL, 64, "cuda:0", max_partials=8)
     prompt = torch.tensor([3, 99, 1024, 7])
