@@ -342,6 +342,27 @@ def test_bad_committing_instructions_are_rejected_on_the_device(weights, bad, op
         assert torch.equal(getattr(gpu, n), t), n
 
 
+def test_committing_instruction_whose_inputs_never_arrive_runs_out_of_polls(weights):
+    """Nobody runs the router: the committing instruction's looks at the logits run out of polls, it says so and the
+    grid drains; the launcher clears the workspace, and the next well-formed step works."""
+    from qimeng_megakernel_amd.decode_schedule.instructions.scheduler import tensorize_instructions
+
+    _, gpu = make_pair(weights)
+    before = gpu.hidden_states.clone()
+    tensorize_instructions(gpu, S.deal([S.RoutedExpert_DownProj(0, 0, 2, 0, 1, tile_N_granularity=8)], 8))
+    mk = mk_kernel.get_mk(spin_limit=64)
+    mk_kernel.call_mk(gpu, mk)
+    with pytest.raises(RuntimeError, match="ran out of polls") as err:
+        mk.check()
+    assert "opcode=13" in str(err.value) and torch.equal(gpu.hidden_states, before)
+    assert int(mk._workspace.view(torch.int32).abs().sum()) == 0 and int(gpu.barriers.abs().sum()) == 0
+    gpu.instructions = None
+    mk = mk_kernel.get_mk(spin_limit=1 << 18)
+    mk_kernel.call_mk(gpu, mk)                      # a whole step on the same buffers
+    mk.check()
+    assert torch.isfinite(gpu.logits.float()).all()
+
+
 def test_decode_loop_and_graph(weights):
     g = synthetic.build_moe_globals(weights, SMALL, 64, "cuda:0", max_partials=8)
     prompt = torch.tensor([3, 99, 1024, 7])
