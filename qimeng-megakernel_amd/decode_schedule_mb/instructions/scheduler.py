@@ -83,6 +83,7 @@ class BatchScheduler:
     oproj_tile: int = TILE_N_GRANULARITY   # rows per O-proj block: 16 (the reference's), or 8
     down_tile: int = TILE_N_GRANULARITY    # rows per down-projection block
     skew_upgate: bool = False     # run-time template: workers that have just run an O-proj block get fewer up/gate blocks
+    split_kv_per_worker: float = 1.0   # split-KV instructions of a step per worker that the fan-out aims at (the reference: one)
 
     def __post_init__(self) -> None:
         if not 1 <= self.batch_size <= MAX_BATCH:
@@ -191,11 +192,14 @@ class BatchScheduler:
         state = RowState.of(globs)
         rows = [b for b in range(self.batch_size) if state.is_active(b)]
         blocks = max([1] + [_ceil_div(state.position(b) + 1, kvb) for b in rows])
-        return partials_for_blocks(len(rows), blocks, self.workers, self.shape.num_key_value_heads)
+        return partials_for_blocks(len(rows), blocks, self._split_kv_workers(), self.shape.num_key_value_heads)
+
+    def _split_kv_workers(self) -> int:
+        return max(1, int(self.workers * self.split_kv_per_worker))
 
     def partials_for_capacity(self, kv_capacity: int) -> int:
         blocks = max(1, _ceil_div(kv_capacity, self.shape.attn_kv_block_size))
-        return partials_for_blocks(self.batch_size, blocks, self.workers, self.shape.num_key_value_heads)
+        return partials_for_blocks(self.batch_size, blocks, self._split_kv_workers(), self.shape.num_key_value_heads)
 
     # ---- whole step: dependency order, dealt round-robin ---------------------
     def instruction_list(self, globs: Any, num_layers: int | None = None) -> list[Instruction]:
@@ -262,8 +266,14 @@ def mi355x_scheduler(batch_size: int, shape: DecodeShape | None = None, *, merge
     """One queue per CU; the split-KV partials are merged by the last arrival of each head group.
     ``residual_tile`` 8 gives the two projections that add to the residual stream one 8-row block per
     workgroup instead of 16-row blocks on half the CUs; measured slower at batch 8 (every workgroup
-    reads all activations, so twice the workgroups read them twice: 7478 against 8015 tok/s)."""
+    reads all activations, so twice the workgroups read them twice: 7478 against 8015 tok/s).
+    Split-KV fan-out: with heads of 64 half as many slices as the reference's one-instruction-per-worker rule gives —
+    what a slice saves in scores the merge by the last arrival (a counted arrival, a second read of the partials,
+    a second hand-over) costs again: Llama shape, contexts 500 / 1000, step time with the reference's fan-out against
+    half of it: B=2 938/947 -> 853/856 us, B=4 938/947 -> 881/905, B=8 1021/1048 -> 972/1009, B=16 1187/1233 ->
+    1108/1176.  With heads of 128 (Qwen3-1.7B shape, B=8: 1566/1636 us with 4 slices, 1591/1721 with 2) the rule stays."""
     if residual_tile not in (8, 16):
         raise ValueError("blocks of the residual projections have 8 or 16 rows")
-    return BatchScheduler(shape or LlamaConfig.shape(), MI355X_WORKERS, batch_size, merge_in_last=merge_in_last,
-                          oproj_tile=residual_tile, down_tile=residual_tile, skew_upgate=skew_upgate)
+    shape = shape or LlamaConfig.shape()
+    return BatchScheduler(shape, MI355X_WORKERS, batch_size, merge_in_last=merge_in_last, oproj_tile=residual_tile,
+                          down_tile=residual_tile, skew_upgate=skew_upgate, split_kv_per_worker=0.5 if shape.head_dim <= 64 else 1.0)
