@@ -170,7 +170,7 @@ def test_fan_out_policy():
     # this build's stream: half that fan-out for heads of 64 (the merge by the last arrival costs what a slice saves), the rule itself for heads of 128
     from qimeng_megakernel_amd.decode_schedule.model_config import QWEN3_1_7B
     assert [S.mi355x_scheduler(b, dataclasses.replace(LLAMA_3_2_1B, attn_kv_block_size=64)).partials_for_capacity(1040) for b in (2, 4, 8, 16)] == [8, 4, 2, 1]
-    assert S.mi355x_scheduler(8, QWEN3_1_7B).partials_for_capacity(1040) == 4
+    assert [S.mi355x_scheduler(b, QWEN3_1_7B).partials_for_capacity(1040) for b in (2, 4, 8, 16)] == [8, 8, 4, 2]    # ... capped at 8
 
 
 # -------------------------------------------------------------------- oracles --
