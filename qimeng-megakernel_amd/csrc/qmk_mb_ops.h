@@ -437,15 +437,23 @@ __device__ bool op_splitkv(const Params& p, Smem<M>& s, const Ctx& c) {
       for (int i = 0; i < NT / 2; ++i) tl.v[j][i] = src[i];
     }
   };
+  // A wave's next kDepth tiles are in flight at any time, the first of them from before the wait below: a tile
+  // costs a trip to memory and 16 tokens of arithmetic, so with one tile ahead every round paid most of the trip.
+#ifndef QMK_MB_KV_DEPTH
+#define QMK_MB_KV_DEPTH 2
+#endif
+  constexpr int kDepth = QMK_MB_KV_DEPTH;
   int tb = t0 + wave * kTok;
-  Tile cur;
+  Tile ring[kDepth];
+  static_for<0, kDepth>([&](auto i) {
 #pragma unroll
-  for (int j = 0; j < KV16; ++j) cur.k[j] = v4u{0, 0, 0, 0};
+    for (int j = 0; j < KV16; ++j) ring[i].k[j] = v4u{0, 0, 0, 0};
 #pragma unroll
-  for (int j = 0; j < 4; ++j)
+    for (int j = 0; j < 4; ++j)
 #pragma unroll
-    for (int i = 0; i < NT / 2; ++i) cur.v[j][i] = 0;
-  if (!empty && tb < t1) fetch(cur, tb);
+      for (int e = 0; e < NT / 2; ++e) ring[i].v[j][e] = 0;
+    if (!empty && tb + i * kStep < t1) fetch(ring[i], tb + i * kStep);
+  });
 
   if (!wait_counters(
           p, s, c, GQA + 2,
@@ -480,6 +488,7 @@ __device__ bool op_splitkv(const Params& p, Smem<M>& s, const Ctx& c) {
       publish_after_stores(p, c, layer, ROW_REDUCE, b, GQA);
     }
   };
+  const bool alone = merge_in_last && P == 1 && !empty;
   if (empty) {  // uniform
     if (c.tid < GQA * D) {
       const int h = c.tid / D, d = c.tid % D;
@@ -562,9 +571,7 @@ __device__ bool op_splitkv(const Params& p, Smem<M>& s, const Ctx& c) {
 #pragma unroll
   for (int i = 0; i < NT; ++i) acc[i] = f4{0.f, 0.f, 0.f, 0.f};
 
-  while (tb < t1) {
-    Tile nxt = cur;
-    if (tb + kStep < t1) fetch(nxt, tb + kStep);
+  auto round = [&](Tile& cur) {
     if (pos >= tb && pos < tb + kTok) {  // the row appended during this launch comes from LDS
       // (also where a token past the slice was redirected to this row: what the cache holds there is not defined yet)
       if (min(tb + c16, t1 - 1) == pos) {
@@ -603,14 +610,11 @@ __device__ bool op_splitkv(const Params& p, Smem<M>& s, const Ctx& c) {
       psum += pr[i];
     }
     l_run = __builtin_fmaf(l_run, alpha, psum);
-    uint32_t hi[4], lo[4];
-#pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      hi[i] = f2bf(pr[i]);
-      lo[i] = f2bf(pr[i] - bf2f(static_cast<u16>(hi[i])));
-    }
-    const bf4 p_hi = __builtin_bit_cast(bf4, u2{hi[0] | (hi[1] << 16), hi[2] | (hi[3] << 16)});
-    const bf4 p_lo = __builtin_bit_cast(bf4, u2{lo[0] | (lo[1] << 16), lo[2] | (lo[3] << 16)});
+    // the weights as bf16 pairs hi + lo (lo = what the rounding of hi left): two conversions per pair
+    const u2 hi = u2{pack_bf16(pr[0], pr[1]), pack_bf16(pr[2], pr[3])};
+    const u2 lo = u2{pack_bf16(pr[0] - bf_lo(hi.x), pr[1] - bf_hi(hi.x)), pack_bf16(pr[2] - bf_lo(hi.y), pr[3] - bf_hi(hi.y))};
+    const bf4 p_hi = __builtin_bit_cast(bf4, hi);
+    const bf4 p_lo = __builtin_bit_cast(bf4, lo);
     float a_head[4];
     bool rescale = false;
 #pragma unroll
@@ -639,8 +643,13 @@ __device__ bool op_splitkv(const Params& p, Smem<M>& s, const Ctx& c) {
       acc[tau] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(p_hi, vb, acc[tau], 0, 0, 0);
       acc[tau] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(p_lo, vb, acc[tau], 0, 0, 0);
     }
-    cur = nxt;
+    if (tb + kDepth * kStep < t1) fetch(cur, tb + kDepth * kStep);   // the tile that takes this one's place
     tb += kStep;
+  };
+  while (tb < t1) {
+    static_for<0, kDepth>([&](auto i) {
+      if (tb < t1) round(ring[i]);
+    });
   }
   QMK_MB_STAMP(1);
 
@@ -672,12 +681,21 @@ __device__ bool op_splitkv(const Params& p, Smem<M>& s, const Ctx& c) {
     }
     const bool none = !(den > 0.f);
     st_shared_f32(part_out + static_cast<size_t>(h) * p.max_splits * D + d, none ? 0.f : num / den);
+    // the only slice of its heads: what the merge of one partial leaves (weight 2^0, denominator 1) is the partial itself
+    if (alone) st_shared16(p.attn_out + static_cast<size_t>(b) * M::NQ * D + static_cast<size_t>(head0 + h) * D + d, f2bf(none ? 0.f : num / den));
     if (d == 0) {
       st_shared_f32(lse_out + static_cast<size_t>(h) * p.max_splits, none ? -INFINITY : mx + log2f(den));
       if (valid_out) st_shared8(valid_out + static_cast<size_t>(h) * p.max_splits, none ? 0 : 1);
     }
   }
   QMK_MB_STAMP(2);
+  if (alone) {   // no trip for the count of arrivals, none to read the partial back
+    release_stores();
+    __syncthreads();
+    if (c.tid < GQA) publish(counter_ptr(p, layer, ROW_SPLITKV, b * kStride + head0 + c.tid), 1);
+    if (c.tid == 0) publish(counter_ptr(p, layer, ROW_REDUCE, b), GQA);
+    return true;
+  }
   arrive();
   return true;
 }
