@@ -682,7 +682,10 @@ __device__ bool op_splitkv(const Params& p, Smem<M>& s, const Ctx& c) {
     const bool none = !(den > 0.f);
     st_shared_f32(part_out + static_cast<size_t>(h) * p.max_splits * D + d, none ? 0.f : num / den);
     // the only slice of its heads: what the merge of one partial leaves (weight 2^0, denominator 1) is the partial itself
-    if (alone) st_shared16(p.attn_out + static_cast<size_t>(b) * M::NQ * D + static_cast<size_t>(head0 + h) * D + d, f2bf(none ? 0.f : num / den));
+    // (whole waves are here: GQA * D is a multiple of the wave size, and the even lane stores its neighbour's half too)
+    const uint32_t half = f2bf(none ? 0.f : num / den);
+    const uint32_t next = __shfl_down(half, 1);
+    if (alone && !(d & 1)) st_shared32(p.attn_out + static_cast<size_t>(b) * M::NQ * D + static_cast<size_t>(head0 + h) * D + d, half | (next << 16));
     if (d == 0) {
       st_shared_f32(lse_out + static_cast<size_t>(h) * p.max_splits, none ? -INFINITY : mx + log2f(den));
       if (valid_out) st_shared8(valid_out + static_cast<size_t>(h) * p.max_splits, none ? 0 : 1);

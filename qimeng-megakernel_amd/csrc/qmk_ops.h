@@ -845,8 +845,30 @@ __device__ bool op_attn_splitkv(const Params& p, Smem<M>& s, const Ctx& c) {
   if constexpr (GQA * D <= kThreads) {
     if (c.tid < GQA * D) merge_output(c.tid);
   } else {
-    merge_output(c.tid);
-    merge_output(c.tid + kThreads);
+    // Two neighbouring dims of one head per thread: the head's maximum, weights and denominator once for both.
+    static_assert(GQA * D == 2 * kThreads && D % 2 == 0, "one pair per thread");
+    const int h = (2 * c.tid) / D, d = (2 * c.tid) % D;
+    float mx = -INFINITY;
+#pragma unroll
+    for (int w = 0; w < kWaves; ++w) mx = fmaxf(mx, s.merge[w][h][D]);
+    float den = 0.f, num0 = 0.f, num1 = 0.f;
+#pragma unroll
+    for (int w = 0; w < kWaves; ++w) {
+      const float mw = s.merge[w][h][D];
+      const float wgt = (mw == -INFINITY) ? 0.f : exp2_fast(mw - mx);
+      const float2 a = *reinterpret_cast<const float2*>(&s.merge[w][h][d]);
+      den = __builtin_fmaf(s.merge[w][h][D + 1], wgt, den);
+      num0 = __builtin_fmaf(a.x, wgt, num0);
+      num1 = __builtin_fmaf(a.y, wgt, num1);
+    }
+    const int head = kvh * GQA + h;
+    const bool empty = !(den > 0.f);
+    float* dst = p.attn_partial + (static_cast<size_t>(head) * p.max_splits + part) * D + d;
+    __hip_atomic_store(reinterpret_cast<uint64_t*>(dst),
+                       static_cast<uint64_t>(__float_as_uint(empty ? 0.f : num0 / den)) |
+                           (static_cast<uint64_t>(__float_as_uint(empty ? 0.f : num1 / den)) << 32),
+                       __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    if (d == 0) st_shared_f32(p.attn_lse + static_cast<size_t>(head) * p.max_splits + part, empty ? -INFINITY : mx + log2f(den));
   }
 
   QMK_STAMP(2);  // partial merged and stored

@@ -85,6 +85,8 @@ class BatchScheduler:
     skew_upgate: bool = False     # run-time template: workers that have just run an O-proj block get fewer up/gate blocks
     split_kv_per_worker: float = 1.0   # split-KV instructions of a step per worker that the fan-out aims at (the reference: one)
     split_kv_cap: int = MAX_REDUCTION_LIST   # ... and never more slices per KV head than this
+    lone_slice_tokens: int = 0         # where the rule gives two slices and the slices' tokens are at most this many: one slice
+                                       # (the only slice of its heads writes attn_out itself: no counted arrival, no merge)
 
     def __post_init__(self) -> None:
         if not 1 <= self.batch_size <= MAX_BATCH:
@@ -193,14 +195,20 @@ class BatchScheduler:
         state = RowState.of(globs)
         rows = [b for b in range(self.batch_size) if state.is_active(b)]
         blocks = max([1] + [_ceil_div(state.position(b) + 1, kvb) for b in rows])
-        return min(self.split_kv_cap, partials_for_blocks(len(rows), blocks, self._split_kv_workers(), self.shape.num_key_value_heads))
+        return self._fan_out(len(rows), blocks)
 
     def _split_kv_workers(self) -> int:
         return max(1, int(self.workers * self.split_kv_per_worker))
 
+    def _fan_out(self, rows: int, blocks: int) -> int:
+        p = min(self.split_kv_cap, partials_for_blocks(rows, blocks, self._split_kv_workers(), self.shape.num_key_value_heads))
+        if p == 2 and self.merge_in_last and blocks * self.shape.attn_kv_block_size <= self.lone_slice_tokens:
+            return 1
+        return p
+
     def partials_for_capacity(self, kv_capacity: int) -> int:
         blocks = max(1, _ceil_div(kv_capacity, self.shape.attn_kv_block_size))
-        return min(self.split_kv_cap, partials_for_blocks(self.batch_size, blocks, self._split_kv_workers(), self.shape.num_key_value_heads))
+        return self._fan_out(self.batch_size, blocks)
 
     # ---- whole step: dependency order, dealt round-robin ---------------------
     def instruction_list(self, globs: Any, num_layers: int | None = None) -> list[Instruction]:
@@ -272,11 +280,14 @@ def mi355x_scheduler(batch_size: int, shape: DecodeShape | None = None, *, merge
     what a slice saves in scores the merge by the last arrival (a counted arrival, a second read of the partials,
     a second hand-over) costs again: Llama shape, contexts 500 / 1000, step time with the reference's fan-out against
     half of it: B=2 938/947 -> 853/856 us, B=4 938/947 -> 881/905, B=8 1021/1048 -> 972/1009, B=16 1187/1233 ->
-    1108/1176.  With heads of 128 (Qwen3-1.7B shape, B=8: 1566/1636 us with 4 slices, 1591/1721 with 2) the rule stays,
-    but never more than 8 slices (that shape at B=2: 1360/1360 us with 8, 1443/1448 with the rule's 16)."""
+    1108/1176.  With heads of 128 (Qwen3-1.7B shape, B=8: 1566/1636 us with 4 slices, 1591/1721 with 2) the rule stays.
+    Never more than 4 slices (mean step time at contexts 250 / 500 / 1000 with 4 against 8 slices: Llama shape B=2
+    843 against 856 us; Qwen3 shape B=2 1345 against 1362, B=4 1432 against 1433).  With heads of 64 and a cache of at
+    most 2048 tokens one slice where the rule gives two: the only slice of its heads writes attn_out itself (Llama
+    shape B=8: 963 against 980 us; the second slice halves a loop of 0.9 us per 128 tokens and costs a merge of 4 us)."""
     if residual_tile not in (8, 16):
         raise ValueError("blocks of the residual projections have 8 or 16 rows")
     shape = shape or LlamaConfig.shape()
     return BatchScheduler(shape, MI355X_WORKERS, batch_size, merge_in_last=merge_in_last, oproj_tile=residual_tile,
                           down_tile=residual_tile, skew_upgate=skew_upgate, split_kv_per_worker=0.5 if shape.head_dim <= 64 else 1.0,
-                          split_kv_cap=8)
+                          split_kv_cap=4, lone_slice_tokens=2048 if shape.head_dim <= 64 else 0)

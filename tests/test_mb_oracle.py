@@ -167,10 +167,15 @@ def test_fan_out_policy():
     assert S.partials_for_blocks(2, 100, 216, 8) == 14      # ceil(216 / 16)
     assert S.partials_for_blocks(1, 1000, 256, 8) == S.MAX_REDUCTION_LIST
     assert S.partials_for_blocks(0, 5, 216, 8) == 1
-    # this build's stream: half that fan-out for heads of 64 (the merge by the last arrival costs what a slice saves), the rule itself for heads of 128
+    # this build's stream: half that fan-out for heads of 64 (the merge by the last arrival costs what a slice saves), the rule
+    # itself for heads of 128; never more than 4 slices; with heads of 64 one slice instead of two while the cache is small
     from qimeng_megakernel_amd.decode_schedule.model_config import QWEN3_1_7B
-    assert [S.mi355x_scheduler(b, dataclasses.replace(LLAMA_3_2_1B, attn_kv_block_size=64)).partials_for_capacity(1040) for b in (2, 4, 8, 16)] == [8, 4, 2, 1]
-    assert [S.mi355x_scheduler(b, QWEN3_1_7B).partials_for_capacity(1040) for b in (2, 4, 8, 16)] == [8, 8, 4, 2]    # ... capped at 8
+    llama = dataclasses.replace(LLAMA_3_2_1B, attn_kv_block_size=64)
+    assert [S.mi355x_scheduler(b, llama).partials_for_capacity(1040) for b in (2, 4, 8, 16)] == [4, 4, 1, 1]
+    assert [S.mi355x_scheduler(b, llama).partials_for_capacity(4096) for b in (2, 4, 8, 16)] == [4, 4, 2, 1]
+    assert [S.mi355x_scheduler(b, QWEN3_1_7B).partials_for_capacity(1040) for b in (2, 4, 8, 16)] == [4, 4, 4, 2]
+    # streams with a reduction instruction keep both slices
+    assert S.mi355x_scheduler(8, llama, merge_in_last=False).partials_for_capacity(1040) == 2
 
 
 # -------------------------------------------------------------------- oracles --

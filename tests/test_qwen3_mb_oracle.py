@@ -62,7 +62,7 @@ def test_request_of_the_reference_fixture(weights, route):
     """Six steps: greedy tokens, row state, top-4 logits bit for bit and samples of the hidden state."""
     g = _request(weights, FIX["max_partials"] if route == "fused" else 27)
     # the stream the fixture's VM leg was recorded with: this build's placement, the reference's split-KV fan-out rule
-    sched = dataclasses.replace(S.mi355x_scheduler(FIX["rows"], SMALL), split_kv_per_worker=1.0, split_kv_cap=S.MAX_REDUCTION_LIST)
+    sched = dataclasses.replace(S.mi355x_scheduler(FIX["rows"], SMALL), split_kv_per_worker=1.0, split_kv_cap=S.MAX_REDUCTION_LIST, lone_slice_tokens=0)
     fused, vm = FusedBatchOracle(SMALL), BatchInstructionVM(SMALL)
     tokens = list(FIX["start_tokens"])
     for step, want in enumerate(FIX["steps"]):
