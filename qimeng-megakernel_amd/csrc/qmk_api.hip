@@ -66,7 +66,7 @@ __global__ __launch_bounds__(kThreads, 1) void decode_megakernel(const Params p_
   int32_t word = (threadIdx.x < kInstWords && p.num_insts > 0) ? queue[threadIdx.x] : 0;
   int32_t word1 = (threadIdx.x < kInstWords && p.num_insts > 1) ? queue[kInstWords + threadIdx.x] : 0;
   Carried carry;
-  bool carried = false, after_attention = false;
+  bool carried = false, parked = false, after_attention = false;
   forget(carry);
   const int num_insts = p.num_insts;
   for (int i = 0; i < num_insts && ok; ++i) {
@@ -96,9 +96,10 @@ __global__ __launch_bounds__(kThreads, 1) void decode_megakernel(const Params p_
       case OP_ATTN_REDUCE: [[clang::always_inline]] ok = op_attn_reduce<M>(p, s, c); forget(carry); break;
       case OP_OPROJ_RESIDUAL:
         carried = M::CARRY_AFTER_ATTENTION || !after_attention;
-        [[clang::always_inline]] ok = op_oproj_residual<M>(params_for(kSegmentOproj), s, c, carry, carried);
+        parked = !after_attention;   // a workgroup that has just run the attention has no wait to fill
+        [[clang::always_inline]] ok = op_oproj_residual<M>(params_for(kSegmentOproj), s, c, carry, carried, parked);
         break;
-      case OP_RMS_UPGATE_SILU: [[clang::always_inline]] ok = op_rms_upgate_silu<M>(params_for(kSegmentUpGate), s, c, carry, carried); forget(carry); break;
+      case OP_RMS_UPGATE_SILU: [[clang::always_inline]] ok = op_rms_upgate_silu<M>(params_for(kSegmentUpGate), s, c, carry, carried, parked); forget(carry); break;
       case OP_DOWN_RESIDUAL: [[clang::always_inline]] ok = op_down_residual<M>(params_for(kSegmentDown), s, c); forget(carry); break;
       case OP_RMS_LMHEAD: [[clang::always_inline]] ok = op_rms_lmhead<M>(params_for(kSegmentLmHead), s, c); forget(carry); break;
       default:
@@ -107,7 +108,7 @@ __global__ __launch_bounds__(kThreads, 1) void decode_megakernel(const Params p_
         forget(carry);
         break;
     }
-    if (opcode != OP_OPROJ_RESIDUAL) carried = false;
+    if (opcode != OP_OPROJ_RESIDUAL) carried = parked = false;
     after_attention = opcode == OP_ATTN_SPLITKV || opcode == OP_ATTN_REDUCE;
 
     if (p.timeline != nullptr && threadIdx.x == 0) {
@@ -307,7 +308,7 @@ __global__ __launch_bounds__(kThreads, 1) void decode_megakernel_moe(const Param
       t_start = wall_clock64();
       for (int k = 0; k < 4; ++k) s.stamps[k] = t_start;
     }
-    bool carried = false;
+    bool carried = false, parked = false;
     // Every op inlined, whatever its size: an op left out of line takes `p` by reference, and the kernel
     // arguments then live in private memory for all ops (vector loads from scratch instead of scalar loads).
     switch (opcode) {
@@ -315,7 +316,7 @@ __global__ __launch_bounds__(kThreads, 1) void decode_megakernel_moe(const Param
       case OP_RMS_QKV_ROPE: [[clang::always_inline]] ok = op_rms_qkv_rope<M>(p, s, c); break;
       case OP_ATTN_SPLITKV: [[clang::always_inline]] ok = op_attn_splitkv<M>(p, s, c); break;
       case OP_ATTN_REDUCE: [[clang::always_inline]] ok = op_attn_reduce<M>(p, s, c); break;
-      case OP_OPROJ_RESIDUAL: [[clang::always_inline]] ok = op_oproj_residual<M>(p, s, c, carry, carried); break;
+      case OP_OPROJ_RESIDUAL: [[clang::always_inline]] ok = op_oproj_residual<M>(p, s, c, carry, carried, parked); break;
       case OP_RMS_LMHEAD: [[clang::always_inline]] ok = op_rms_lmhead<M>(p, s, c); break;
       case moe::OP_ROUTER: [[clang::always_inline]] ok = moe::op_router<M>(p, s, c); break;
       case moe::OP_TOPK: [[clang::always_inline]] ok = moe::op_topk<M>(p, s, c); break;

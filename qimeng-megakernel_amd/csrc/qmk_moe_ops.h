@@ -31,6 +31,7 @@ struct QwenMoeA2_7B {
   static constexpr int AW = NQ * D;
   static constexpr int KV_BLOCK = 16;
   static constexpr int CARRY_ROWS = 0;
+  static constexpr int PARK_ROWS = 0;
   static constexpr bool CARRY_AFTER_ATTENTION = false;
   static constexpr bool QK_NORM = false;
   static constexpr bool QKV_BIAS = true;
@@ -55,6 +56,7 @@ struct Qwen3MoeA3B {
   static constexpr int AW = NQ * D;
   static constexpr int KV_BLOCK = 16;
   static constexpr int CARRY_ROWS = 0;
+  static constexpr int PARK_ROWS = 0;
   static constexpr bool CARRY_AFTER_ATTENTION = false;
   static constexpr bool QK_NORM = true;
   static constexpr bool QKV_BIAS = false;
