@@ -82,6 +82,9 @@ struct Smem {
   float merge[kWaves][M::GQA][M::D + 4];
   unsigned long long t_wait;
   unsigned long long stamps[4];
+  // One weight segment per wave ([wave][chunk][lane]) fetched before a wait that the registers have no room for: the
+  // gate segment of an up/gate instruction's third block, the fourth segment of a down projection's first block.
+  alignas(16) v4u seg_park[kWaves][kSegChunks][64];
 };
 
 #define QMK_MB_STAMP(k)                                                     \
@@ -227,7 +230,9 @@ __device__ __forceinline__ float2 gather(const Smem<M>& s, int parity, int unit,
 // (the caller decides whether that is before or after its wait through `wait`).
 // `rows` (16, or 8): weight rows per block; with 8 the upper half of the tile repeats the lower one
 // (the same addresses: no extra traffic) and only outputs 0..7 are used.
-template <class M, int NU, int NB, class Src, class Wait, class Epi>
+// `PARK`: the first matrix's segment of block NB — the first one the ring has no room for — is fetched before the wait
+// as well and waits in LDS (s.seg_park) until the ring's first slot is free.
+template <class M, int NU, int NB, bool PARK = false, class Src, class Wait, class Epi>
 __device__ __forceinline__ bool gemm_h(const Params& p, Smem<M>& s, const Ctx& c, int n, const u16* act, int B, Src src, Wait wait, Epi epi,
                                        int rows = kTile) {
   static_assert(M::H == kWaves * kSeg, "one segment per wave");
@@ -239,6 +244,14 @@ __device__ __forceinline__ bool gemm_h(const Params& p, Smem<M>& s, const Ctx& c
     if (k < n)
 #pragma unroll
       for (int u = 0; u < NU; ++u) load_seg(ring[k][u], src(k, u) + lane_off);
+  if constexpr (PARK) {
+    if (n > NB) {
+      Seg extra;
+      load_seg(extra, src(NB, 0) + lane_off);
+#pragma unroll
+      for (int j = 0; j < kSegChunks; ++j) s.seg_park[wave][j][lane] = extra.a[j];
+    }
+  }
   if (!wait()) return false;
   v4u x[kSegChunks];
   load_x(x, act, M::H, B, wave * kSeg, lane);
@@ -252,7 +265,14 @@ __device__ __forceinline__ bool gemm_h(const Params& p, Smem<M>& s, const Ctx& c
         for (int u = 0; u < NU; ++u) {
           const f4 acc = mma_seg(ring[k][u], x, f4{0.f, 0.f, 0.f, 0.f});
           park(s, parity, u, wave, lane, acc);
-          if (j + NB < n) load_seg(ring[k][u], src(j + NB, u) + lane_off);
+          if (j + NB < n) {
+            if (PARK && j == 0 && u == 0) {
+#pragma unroll
+              for (int q = 0; q < kSegChunks; ++q) ring[k][u].a[q] = s.seg_park[wave][q][lane];
+            } else {
+              load_seg(ring[k][u], src(j + NB, u) + lane_off);
+            }
+          }
         }
         __syncthreads();
         // Parity: a slot is written again two blocks later, behind the next barrier, which the
@@ -786,7 +806,7 @@ __device__ bool op_upgate(const Params& p, Smem<M>& s, const Ctx& c) {
   if (s.inst[5 + n] != kMaxBatch || s.inst[6 + n] != kTile) return bad_operand(p, s, c, 6 + n);
   const u16* wg = p.gate_w + static_cast<size_t>(layer) * M::F * M::H;
   const u16* wu = p.up_w + static_cast<size_t>(layer) * M::F * M::H;
-  const bool ok = gemm_h<M, 2, 2>(
+  const bool ok = gemm_h<M, 2, 2, true>(
       p, s, c, n, p.mlp_rms_out, B, [&](int j, int u) { return (u ? wu : wg) + static_cast<size_t>(s.inst[5 + j]) * kTile * M::H; },
       [&] { return wait_counter(p, s, c, layer, ROW_MLP_RMS, B); },
       [&](int j, int parity, int b, int rp) {
@@ -835,23 +855,44 @@ __device__ bool op_down(const Params& p, Smem<M>& s, const Ctx& c) {
     load_seg(a1, wptr(block, 1));
     load_seg(a2, wptr(block, 2));
   };
-  if (n0 < n1) request(n0);
+  if (n0 < n1) {
+    request(n0);
+    if constexpr (NS == 4) {
+      // The fourth segment of the first block goes to LDS through a3's registers: it lands during the wait instead of
+      // behind the first activations (the registers hold three weight and two activation segments, not four and two).
+      load_seg(a3, wptr(n0, 3));
+#pragma unroll
+      for (int j = 0; j < kSegChunks; ++j) s.seg_park[wave][j][lane] = a3.a[j];
+    }
+  }
   if (!wait_counter(p, s, c, layer, ROW_UPGATE, M::F / kTile)) return false;
   u16* const mine = p.hidden + static_cast<size_t>(c.tid & 15) * M::H + 2 * (c.tid >> 4);
   const bool adds = c.tid < 8 * R && (c.tid & 15) < B && s.active[c.tid & 15];
   int parity = 0;
   for (int blk = n0; blk < n1; ++blk) {
-    v4u xa[kSegChunks], xb[kSegChunks];
-    load_x(xa, p.silu_out, M::F, B, k0, lane);
-    load_x(xb, p.silu_out, M::F, B, k0 + kSeg, lane);
-    if constexpr (NS == 4) load_seg(a3, wptr(blk, 3));
-    f4 acc = mma_seg(a0, xa, f4{0.f, 0.f, 0.f, 0.f});
-    load_x(xa, p.silu_out, M::F, B, k0 + 2 * kSeg, lane);
-    acc = mma_seg(a1, xb, acc);
-    if constexpr (NS == 4) load_x(xb, p.silu_out, M::F, B, k0 + 3 * kSeg, lane);
-    const uint32_t old = adds ? ld_shared32(mine + blk * R) : 0u;   // the pair this thread adds to, in time for the epilogue
-    acc = mma_seg(a2, xa, acc);
-    if constexpr (NS == 4) acc = mma_seg(a3, xb, acc);
+    f4 acc = f4{0.f, 0.f, 0.f, 0.f};
+    uint32_t old = 0u;
+    {
+      v4u xa[kSegChunks], xb[kSegChunks];
+      load_x(xa, p.silu_out, M::F, B, k0, lane);
+      load_x(xb, p.silu_out, M::F, B, k0 + kSeg, lane);
+      if constexpr (NS == 4) {
+        if (blk != n0) load_seg(a3, wptr(blk, 3));
+      }
+      acc = mma_seg(a0, xa, acc);
+      load_x(xa, p.silu_out, M::F, B, k0 + 2 * kSeg, lane);
+      acc = mma_seg(a1, xb, acc);
+      if constexpr (NS == 4) load_x(xb, p.silu_out, M::F, B, k0 + 3 * kSeg, lane);
+      old = adds ? ld_shared32(mine + blk * R) : 0u;   // the pair this thread adds to, in time for the epilogue
+      acc = mma_seg(a2, xa, acc);
+      if constexpr (NS == 4) {
+        if (blk == n0) {
+#pragma unroll
+          for (int j = 0; j < kSegChunks; ++j) a3.a[j] = s.seg_park[wave][j][lane];
+        }
+        acc = mma_seg(a3, xb, acc);
+      }
+    }
     park(s, parity, 0, wave, lane, acc);
     QMK_MB_STAMP(0);  // thread 0's weights and activations have all arrived
     if (blk + 1 < n1) request(blk + 1);
