@@ -221,3 +221,35 @@ def test_single_queue_and_odd_queue_counts(state):
         results.append((gpu.hidden_states.clone(), gpu.logits.clone()))
     for h, l in results[1:]:
         assert torch.equal(h, results[0][0]) and torch.equal(l, results[0][1])
+
+
+def test_parked_upgate_rows_with_ragged_instructions(state):
+    """An O-proj that has a wait ahead leaves rows of the up/gate instruction behind it in LDS.  Up/gate instructions
+    whose rows are not whole rounds of the eight waves (blocks of 2 outputs dealt for 100 queues: 104, 60 and 56 rows
+    per instruction, so the parked rows and the ring's refills exist for some waves only), on few queues so that every
+    queue has O-proj instructions in front of its up/gate instructions: the silu vector equals the VM's, and 7 and 13
+    queues give bit for bit what 256 give."""
+    shape, cpu, gpu = state
+    start_hidden, start_silu = cpu.hidden_states.clone(), cpu.silu_out.clone()
+    base = S.mi355x_scheduler(shape, sm_count=100, num_partials=2)
+    sched = dataclasses.replace(base, geometry=dataclasses.replace(base.geometry, upgate_tile_n=2),
+                                attention_merge="separate")   # the plain O-proj GEMV: attn_out is given
+    rows = sorted({4 * len(i.tile_N_block_idxs) for i in sched.upgate(0)})
+    assert any(r % 8 for r in rows) and max(rows) > 8 * 6      # ragged, and longer than ring + parked rows
+    from qimeng_megakernel_amd.decode_schedule import mk_kernel
+    first = None
+    for sm in (7, 13, 256):
+        cpu.barriers.zero_(); cpu.barriers[0, 2, 0] = shape.num_attention_heads
+        sync_state(cpu, gpu)
+        if first is None:
+            run_both(cpu, gpu, sched, [*sched.oproj(0), *sched.upgate(0)], sm_count=sm)
+            bf16_close(gpu.silu_out, cpu.silu_out, ulps=2.0, frac=0.03, name="silu_out")
+            bf16_close(gpu.hidden_states, cpu.hidden_states, floor=1.0, name="hidden after the O-proj")
+            first = (gpu.silu_out.clone(), gpu.hidden_states.clone())
+            # the VM has advanced the CPU state: put back what the runs start from
+            cpu.hidden_states.copy_(start_hidden); cpu.silu_out.copy_(start_silu)
+        else:
+            mk = mk_kernel.get_mk(geometry=sched.geometry, reset_barriers=False)
+            mk_kernel.run_instructions(gpu, [*sched.oproj(0), *sched.upgate(0)], mk=mk, sm_count=sm)
+            mk.check()
+            assert torch.equal(gpu.silu_out, first[0]) and torch.equal(gpu.hidden_states, first[1])
