@@ -388,5 +388,48 @@ def tensorize_instructions(globs: Any, instruction_queues: list[list[Instruction
     return tensor
 
 
+#: Heads of 128: tokens of context per split-KV slice beyond which a request's later steps get a wider fan-out
+#: (Qwen3-1.7B shape, step time at contexts ~64 / ~512 / ~1000 with 4, 8, 12 slices per KV head: 838/853/932,
+#: 854/856/903, 869/870/882 us).  Heads of 64 keep one stream per request: there the attention phase hides behind
+#: the rows the O-proj workgroups fetch for the up/gate GEMV, and the one fan-out of the capacity rule is the best one.
+LONG_CONTEXT_TOKENS_PER_SLICE = 80
+LONG_CONTEXT_FAN_OUT_STEP = 4
+
+
+def fan_out_plan(sm_count: int, kv_capacity: int | None, *, shape: DecodeShape | None = None,
+                 max_partials: int = MAX_ATTENTION_PARTIALS) -> list[tuple[int, int]]:
+    """``[(first position, fan-out), ...]``: the split-KV fan-out of a request's decode steps by position.
+    The first entry (position 0) is the fan-out ``pick_num_partials`` gives; the fan-out only ever grows."""
+    shape = shape or LlamaConfig.shape()
+    base = pick_num_partials(sm_count, kv_capacity, shape=shape, max_partials=max_partials)
+    plan = [(0, base)]
+    if shape.head_dim <= 64 or kv_capacity is None:
+        return plan
+    cap = min(max_partials, max(1, sm_count // shape.num_key_value_heads))
+    p = base
+    while True:
+        p += LONG_CONTEXT_FAN_OUT_STEP
+        first = (p - LONG_CONTEXT_FAN_OUT_STEP // 2) * LONG_CONTEXT_TOKENS_PER_SLICE   # 8 slices from context 480 on, 12 from 800 on
+        if p > cap or first >= int(kv_capacity):
+            return plan
+        plan.append((first, p))
+
+
 def build(globs: Any, num_layers: int | None = None) -> torch.Tensor:
-    return tensorize_instructions(globs, build_instruction_queues(globs, num_layers))
+    """The request's instruction tensor on ``globs.instructions``; where the fan-out plan has later entries, their
+    tensors wait in ``globs.instruction_plan`` (``call_mk`` picks by ``position_id``)."""
+    base = tensorize_instructions(globs, build_instruction_queues(globs, num_layers))
+    globs.instruction_plan = None
+    sched = scheduler_for(globs)
+    kv_capacity = int(globs.k_cache.shape[2]) if getattr(globs, "k_cache", None) is not None else None
+    lse = getattr(globs, "attn_lse_intermediates", None)
+    max_p = MAX_SELF_MERGE_PARTIALS if lse is None else min(MAX_SELF_MERGE_PARTIALS, int(lse.shape[-1]))
+    plan = fan_out_plan(sched.sm_count, kv_capacity, shape=sched.shape, max_partials=max_p)
+    if len(plan) > 1 and plan[0][1] == sched.num_partials:
+        later = []
+        for first, p in plan[1:]:
+            tensorize_instructions(globs, dataclasses.replace(sched, num_partials=p).queues(num_layers))
+            later.append((first, globs.instructions))
+        globs.instructions = base
+        globs.instruction_plan = (base, later)
+    return base

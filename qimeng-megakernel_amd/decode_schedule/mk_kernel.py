@@ -403,8 +403,15 @@ def call_mk(globs: Globals, mk: Any) -> None:
     if globs.instructions is None:
         _scheduler.build(globs)
     qwen = bool(getattr(shape, "qk_norm", False))
+    instructions = globs.instructions
+    plan = getattr(globs, "instruction_plan", None)
+    if plan is not None and plan[0] is instructions:   # streams with a wider split-KV fan-out for the request's later positions
+        position = globs.position_id if globs.position_id is not None else 0
+        for first, tensor in plan[1]:
+            if position >= first:
+                instructions = tensor
     mk(
-        globs.instructions,
+        instructions,
         globs.hidden_states,
         *((globs.qkv_raw,) if qwen else ()),
         globs.q_post_rope,

@@ -214,3 +214,36 @@ def test_full_size_model_layer_by_layer():
     # 28 layers of rounding differences deep, so the gate is on the tensor's scale (as for the Llama shape)
     err = tensor_rel_close(gpu.logits, cpu2.logits, rel=5e-2, name="free-running logits")
     print(f"free-running step: logits {err:.4f} of the tensor maximum")
+
+
+def test_later_positions_of_a_request_run_a_wider_fan_out(qwen):
+    """Heads of 128: `build` leaves streams with 8 and 12 split-KV slices per KV head beside the request's first one, and
+    `call_mk` takes them from positions 480 and 800 on.  One free-running step at a position of each stream against
+    the fused oracle from the same state: logits within the trajectory gate, the same pick at a clear margin."""
+    shape, _ = qwen
+    LlamaConfig.set_shape(shape)
+    capacity = 1040
+    w = synthetic.random_weights(shape, 5, capacity)
+    gpu = synthetic.build_globals(w, shape, capacity, "cuda:0")
+    S.build(gpu)
+    base, later = gpu.instruction_plan
+    assert base is gpu.instructions and [first for first, _ in later] == [480, 800]
+    widths = [int((t[:, :, 0] == 2).sum()) // shape.num_hidden_layers // shape.num_key_value_heads for t in (base, later[0][1], later[1][1])]
+    assert widths == [4, 8, 12]
+    oracle = FusedOracle(shape)
+    mk = mk_kernel.get_mk()
+    gen = torch.Generator().manual_seed(11)
+    cpu = synthetic.build_globals(w, shape, capacity, "cpu")
+    cpu.k_cache.copy_(torch.randn(cpu.k_cache.shape, generator=gen).bfloat16())
+    cpu.v_cache.copy_(torch.randn(cpu.v_cache.shape, generator=gen).bfloat16())
+    for pos in (100, 479, 480, 700, 1000):
+        cpu.hidden_states.copy_(cpu.embed_tokens[17 + pos]); cpu.position_id = pos
+        sync_state(cpu, gpu)
+        gpu.barriers.zero_()
+        oracle.decode_step(cpu)
+        mk_kernel.call_mk(gpu, mk)
+        mk.check()
+        tensor_rel_close(gpu.logits, cpu.logits, rel=TRAJECTORY_REL, name=f"logits at position {pos}")
+        if _margin_ulps(cpu.logits) > 2.0:
+            assert int(gpu.logits.argmax()) == int(cpu.logits.argmax())
+        bf16_close(gpu.k_cache[0, 0, pos], cpu.k_cache[0, 0, pos], ulps=2.0, frac=0.03, name=f"k row at {pos}")

@@ -260,6 +260,20 @@ def test_pick_num_partials():
         S.schedule_attention_split_kv(0, 26)
 
 
+def test_fan_out_plan_by_position():
+    """One stream per request for heads of 64; heads of 128 get 4 more slices per KV head every 320 tokens of context
+    (8 from position 480 on, 12 from 800 on, ...), never beyond one workgroup per slice or the partial slots."""
+    from qimeng_megakernel_amd.decode_schedule.model_config import QWEN3_1_7B
+    assert S.fan_out_plan(256, 1040, shape=LLAMA_3_2_1B, max_partials=32) == [(0, 4)]
+    assert S.fan_out_plan(256, None, shape=QWEN3_1_7B, max_partials=32) == [(0, 32)]
+    assert S.fan_out_plan(256, 1040, shape=QWEN3_1_7B, max_partials=32) == [(0, 4), (480, 8), (800, 12)]
+    assert S.fan_out_plan(256, 1040, shape=QWEN3_1_7B, max_partials=8) == [(0, 4), (480, 8)]
+    assert S.fan_out_plan(256, 200, shape=QWEN3_1_7B, max_partials=32) == [(0, 1)]
+    assert S.fan_out_plan(256, 600, shape=QWEN3_1_7B, max_partials=32) == [(0, 2), (320, 6)]
+    plan = S.fan_out_plan(256, 4096, shape=QWEN3_1_7B, max_partials=32)
+    assert plan[0] == (0, 13) and plan[-1] == (2160, 29) and all(b[1] - a[1] == 4 for a, b in zip(plan, plan[1:]))
+
+
 def test_geometry_validation():
     with pytest.raises(ValueError):
         D.TileGeometry(qkv_tile_n=3).validate(LLAMA_3_2_1B)
