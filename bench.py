@@ -45,11 +45,15 @@ MEASURED_TRAFFIC_OVER_ALGORITHMIC = 1.0069
 MEASURED_TRAFFIC_OVER_ALGORITHMIC_BATCH8 = 1.0233
 # ... and for the MoE route's kernel (profiles/decode_megakernel_moe_qwen1p5_a2p7b_hbm_counters.txt).
 MEASURED_TRAFFIC_OVER_ALGORITHMIC_MOE = 1.0111
+# What `roofline.traffic` is: not a counter read in this process, but the algorithmic bytes of the timed launches times
+# the ratio the counter runs of the same kernel measured (their contexts are named in the profiles/ file).
+TRAFFIC_SOURCE = "constant ratio from the rocprofv3 FETCH_SIZE/WRITE_SIZE runs of this kernel (profiles/*_hbm_counters.txt) x algorithmic bytes"
 
 
 def cpu_baseline(shape, weights, prompt, n_steps: int, cores: int, shape_name: str) -> dict:
     """BASELINE config 1 on the host: the prompt is prefilled through the single-token path (untimed), then
-    ``n_steps`` greedy decode steps of the same seeded request are timed (a bounded sample of its 128)."""
+    ``n_steps`` greedy decode steps of the same seeded request are timed: a bounded sample of the configuration's 128
+    (``--cpu-steps 128`` times all of them, about 80 s)."""
     import torch
 
     sys.path.insert(0, str(ROOT / "oracle"))
@@ -77,7 +81,7 @@ def cpu_baseline(shape, weights, prompt, n_steps: int, cores: int, shape_name: s
         "cores": cores,
         "host_cpu_count": os.cpu_count(),
         "kind": "port",
-        "sample": f"{n_steps} greedy decode steps (contexts {T + 1}..{T + n_steps}) behind the {T}-token prompt of the same seeded "
+        "sample": f"{n_steps} of the configuration's 128 greedy decode steps (contexts {T + 1}..{T + n_steps}) behind the {T}-token prompt of the same seeded "
                   f"{shape_name}-shaped request (the prompt prefilled through the single-token path, untimed), "
                   f"torch {torch.__version__} bf16 on {cores} threads of {os.cpu_count()} host CPUs, {dt:.1f} s",
     }
@@ -198,6 +202,7 @@ def batch_decode(args) -> dict:
             # the counter runs were made on the Llama shape at batch 8 only
             "traffic": (MEASURED_TRAFFIC_OVER_ALGORITHMIC_BATCH8 * t["algorithmic_bytes"] / max(timed, 1)
                         if B == 8 and args.model == "llama-3.2-1b" else None),
+            "traffic_source": TRAFFIC_SOURCE if B == 8 and args.model == "llama-3.2-1b" else None,
             "bytes_per_launch_avg": t["algorithmic_bytes"] / max(timed, 1), "kernel": kernel,
         },
     }
@@ -267,6 +272,7 @@ def moe_decode(args) -> dict:
             "bound": "hbm", "achieved": t["achieved_GBps"], "peak": HBM_PEAK_GBPS, "unit": "GB/s", "frac": t["achieved_GBps"] / HBM_PEAK_GBPS,
             # the counter runs were made on the Qwen1.5-shaped kernel only
             "traffic": None if a3b else MEASURED_TRAFFIC_OVER_ALGORITHMIC_MOE * t["algorithmic_bytes"] / max(timed, 1),
+            "traffic_source": None if a3b else TRAFFIC_SOURCE,
             "bytes_per_launch_avg": t["algorithmic_bytes"] / max(timed, 1),
             "kernel": "decode_megakernel_moe<Qwen3MoeA3B>" if a3b else "decode_megakernel_moe<QwenMoeA2_7B>",
         },
@@ -560,6 +566,7 @@ def main() -> None:
             # the counter runs were made on the Llama-shaped kernel only
             "traffic": (MEASURED_TRAFFIC_OVER_ALGORITHMIC * t["algorithmic_bytes"] / max(timed, 1)
                         if args.model == "llama-3.2-1b" else None),
+            "traffic_source": TRAFFIC_SOURCE if args.model == "llama-3.2-1b" else None,
             "bytes_per_launch_avg": t["algorithmic_bytes"] / max(timed, 1),
             "kernel": "decode_megakernel<Llama1B>" if args.model == "llama-3.2-1b" else "decode_megakernel<Qwen3_1p7B>",
         },

@@ -217,6 +217,10 @@ int qmk_decode_step(const QmkArgs* args);
  * every queue of a launch before they are read), and qmk_status_fetch clears the array when it
  * reports a device-side error.  Calls that overlap on one GPU (two streams) race on it: serialise
  * them, or use qmk_decode_step with one workspace per stream.
+ * Under HIP graph capture: the first call of any entry point on a device looks the device up (occupancy
+ * queries, hipGetSymbolAddress, a blocking clear of the status words), none of which may be captured, so
+ * call qmk_query(QMK_QUERY_MAX_QUEUES) once per device before the capture begins; from then on a call
+ * is one kernel launch and nothing else.
  */
 int qmk_decode_step_static(const QmkArgs* args);
 

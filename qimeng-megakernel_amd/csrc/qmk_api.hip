@@ -41,6 +41,12 @@ __device__ int32_t g_status[kStatusWords];
 // loses 2 % this way (its first row requests wait for the scalar loads), the O-projection gains; which ops of a
 // dense kernel read the segment is M::PARAMS_FROM_SEGMENT, measured op by op (Llama-3.2-1B +0.7 %, Qwen3-1.7B +2.7 %
 // against all by value).
+// What this rests on, checked where it can be: every interpreter kernel takes exactly one argument, a trivially
+// copyable Params by value, so the explicit-argument part of the kernel-argument segment is that struct at offset 0
+// (explicit arguments come first in the segment, in declaration order, at their natural alignment; the hidden
+// arguments follow).  The launcher passes the same struct type, so sizeof agrees by construction.
+static_assert(std::is_trivially_copyable<Params>::value && std::is_standard_layout<Params>::value, "Params is copied byte for byte into the kernel-argument segment");
+static_assert(alignof(Params) <= 16, "the segment's base alignment covers the struct's");
 __device__ __forceinline__ const Params& params_of_this_instruction() {
   auto args = __builtin_amdgcn_kernarg_segment_ptr();   // (a pointer into the constant address space)
   asm volatile("" : "+s"(args));
@@ -362,6 +368,12 @@ __global__ __launch_bounds__(kThreads, 1) void decode_megakernel_moe(const Param
   }
 }
 
+static_assert(std::is_same<decltype(&decode_megakernel<Llama1B>), void (*)(const Params)>::value &&
+                  std::is_same<decltype(&decode_megakernel<Qwen3_1p7B>), void (*)(const Params)>::value &&
+                  std::is_same<decltype(&decode_megakernel_moe<QwenMoeA2_7B>), void (*)(const Params)>::value &&
+                  std::is_same<decltype(&decode_megakernel_moe<Qwen3MoeA3B>), void (*)(const Params)>::value,
+              "the kernels that read the kernel-argument segment have one by-value Params argument and nothing else");
+
 struct DeviceInfo {
   bool ready = false;
   int cu_count = 0;
@@ -371,6 +383,7 @@ struct DeviceInfo {
   int max_queues_moe = 0;
   int32_t* status = nullptr;
   uint64_t* scratch = nullptr;   // this device's copy of the file-scope `scratch` array
+  bool static_in_use = false;    // a launch since the last status fetch used that array as its workspace
 };
 DeviceInfo g_devices[kMaxDevices];
 std::mutex g_mutex;
@@ -499,6 +512,10 @@ int decode_step(const QmkArgs* a, bool static_scratch) {
   p.lm_w = static_cast<const u16*>(a->lm_head_weights);
   p.barriers = a->barriers;
   p.ws = static_scratch ? dev->scratch : static_cast<uint64_t*>(a->workspace);
+  if (static_scratch) {
+    std::lock_guard<std::mutex> lock(g_mutex);
+    dev->static_in_use = true;
+  }
   p.embed = static_cast<const u16*>(a->embed_tokens);
   p.token_out = reinterpret_cast<long long*>(a->token_out);
   p.timeline = a->timeline;
@@ -804,10 +821,20 @@ extern "C" int qmk_status_fetch(void* stream, int32_t detail[4]) {
   if (hipMemcpy(host, dev->status, sizeof(host), hipMemcpyDeviceToHost) != hipSuccess) return QMK_ERR_NO_DEVICE;
   if (detail != nullptr)
     for (int i = 0; i < 4; ++i) detail[i] = host[1 + i];
+  bool static_used;
+  {
+    std::lock_guard<std::mutex> lock(g_mutex);
+    static_used = dev->static_in_use;
+    dev->static_in_use = false;
+  }
   if (host[0] != 0) {
-    if (hipMemset(dev->status, 0, sizeof(host)) != hipSuccess) return QMK_ERR_NO_DEVICE;
-    // Units of the aborted step must not pass for the next one's (the launch count did not advance).
-    if (hipMemset(dev->scratch, 0, sizeof(scratch)) != hipSuccess) return QMK_ERR_NO_DEVICE;
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    if (hipMemsetAsync(dev->status, 0, sizeof(host), st) != hipSuccess) return QMK_ERR_NO_DEVICE;
+    // Units of the aborted step must not pass for the next one's (the launch count did not advance).  Only when a
+    // launch behind the last fetch used the library's own array, and on the caller's stream: a launch of another
+    // route on another stream has a workspace of its own and is not disturbed.
+    if (static_used && hipMemsetAsync(dev->scratch, 0, sizeof(scratch), st) != hipSuccess) return QMK_ERR_NO_DEVICE;
+    if (hipStreamSynchronize(st) != hipSuccess) return QMK_ERR_NO_DEVICE;
   }
   return host[0];
 }

@@ -84,3 +84,64 @@ def test_static_scratch_rejects_what_the_array_cannot_hold(small_model):
     a.num_layers = 2
     assert mk._lib.qmk_decode_step_static(ctypes.byref(a)) == 0
     mk.check()
+
+
+def _chained_request(shape, weights, *, static, steps, tagged=True, capture=False, replays=1, kv_capacity=48):
+    """``steps`` chained greedy launches (the kernel writes each token and the next embedding row itself), eager or
+    captured into one HIP graph that is replayed ``replays`` times with eager work in between."""
+    LlamaConfig.set_shape(shape)
+    g = synthetic.build_globals(weights, shape, kv_capacity, "cuda:0")
+    sched = S.mi355x_scheduler(shape, sm_count=256, kv_capacity=kv_capacity)
+    S.tensorize_instructions(g, sched.queues())
+    mk = mk_kernel.get_mk(geometry=sched.geometry, static_scratch=static, tagged=tagged)
+    assert mk.query(4) > 0        # QMK_QUERY_MAX_QUEUES: the device is looked up here, outside any capture
+    tokens = torch.zeros(steps + 1, dtype=torch.long, device="cuda:0")
+    first = g.embed_tokens[7].clone()
+
+    def launches():
+        for pos in range(steps):
+            g.position_id = pos
+            mk.greedy_into(g.embed_tokens, tokens, pos + 1)
+            mk_kernel.call_mk(g, mk)
+
+    g.hidden_states.copy_(first)
+    if not capture:
+        launches()
+        mk.check()
+        return g, [tokens.tolist()]
+    launches()                    # binds the argument block before the capture
+    mk.check()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        launches()
+    seen = []
+    for _ in range(replays):
+        g.hidden_states.copy_(first)
+        tokens.zero_()
+        graph.replay()
+        torch.cuda.synchronize()
+        mk.check()
+        seen.append(tokens.tolist())
+        torch.randn(1024, device="cuda:0").sum().item()   # eager work and a synchronisation between replays
+    return g, seen
+
+
+def test_static_entry_point_under_graph_capture_replays_like_the_eager_loop(small_model):
+    shape, w, _ = small_model
+    want, (toks,) = _chained_request(shape, w, static=False, steps=8)
+    got, seen = _chained_request(shape, w, static=True, steps=8, capture=True, replays=3)
+    assert all(t == toks for t in seen), (toks, seen)
+    _same(got, want)
+    assert len(set(toks[1:])) > 1
+
+
+def test_static_entry_point_sampling_only_without_tagged_units(small_model):
+    """Counters carry the hand-overs; only the greedy candidates live in the library's array."""
+    shape, w, _ = small_model
+    want, (toks,) = _chained_request(shape, w, static=False, steps=6, tagged=False)
+    got, (toks_static,) = _chained_request(shape, w, static=True, steps=6, tagged=False)
+    assert toks_static == toks
+    _same(got, want)
+    again, (toks_tagged,) = _chained_request(shape, w, static=True, steps=6, tagged=True)
+    assert toks_tagged == toks     # tagged and counter launches agree bit for bit, also through the array
+    _same(again, want)
