@@ -237,8 +237,11 @@ def moe_decode(args) -> dict:
     gen = torch.Generator().manual_seed(args.seed + 1_000_003)
     prompt = torch.randint(0, shape.vocab_size, (args.prompt_len,), generator=gen, dtype=torch.long)
     globs = synthetic.build_moe_globals(weights, shape, kv_capacity, device, max_partials=8 if a3b else 27)
-    if args.batch > 1:
+    if args.batch > 1 and (args.rows_side_by_side or shape.has_shared_expert or args.batch > 4):
         return moe_decode_rows(args, shape, name, globs, kv_capacity, new_tokens, timed)
+    if args.batch > 1:
+        del globs
+        return moe_decode_batch(args, shape, name, weights, kv_capacity, new_tokens, timed)
     mk = mk_kernel.get_mk()
     if args.copy_calibration:
         copy_calibration(device)
@@ -324,6 +327,55 @@ def moe_decode(args) -> dict:
             line["cpu_baseline"] = {"value": args.cpu_steps / dt, "unit": "tok/s", "cores": cores, "host_cpu_count": os.cpu_count(), "kind": "port",
                                     "sample": f"{args.cpu_steps} steps (contexts 1..{args.cpu_steps}) of the same workload through the fused MoE oracle"}
     return line
+
+
+def moe_decode_batch(args, shape, name: str, weights, kv_capacity: int, new_tokens: int, timed: int) -> dict:
+    """``--batch B`` (2..4) on a MoE shape without a shared expert: the B requests in ONE launch per step
+    (qmk_decode_step_moe_rows).  Attention weights, router and LM head are read once per step, every expert once for
+    all the rows that picked it; the roofline is taken on those algorithmic bytes, the distinct experts counted by
+    the kernel per layer and step."""
+    import torch
+
+    from qimeng_megakernel_amd import decode_moe
+    from qimeng_megakernel_amd.decode_schedule_moe import rows_kernel
+
+    B = args.batch
+    device = torch.device("cuda:0")
+    globs = rows_kernel.build_rows_globals(weights, shape, kv_capacity, B, device, max_partials=8)
+    gen = torch.Generator().manual_seed(args.seed + 1_000_003)
+    prompts = torch.randint(0, shape.vocab_size, (B, args.prompt_len), generator=gen, dtype=torch.long)
+    mk = rows_kernel.get_mk()
+    if args.copy_calibration:
+        copy_calibration(device)
+    if args.warmup > 0:
+        decode_moe.decode_batch(globs, prompts, min(args.warmup + 1, new_tokens), mk=mk, decode_time=False)
+    globs.k_cache.zero_(); globs.v_cache.zero_()
+    out = decode_moe.decode_batch(globs, prompts, new_tokens, mk=mk, timed_steps=timed)
+    t = out["timing"]
+    return {
+        "metric": "kernel_tok_s", "value": t["kernel_tok_s"], "unit": "tok/s", "n_gpus": 1, "steps": timed, "warmup": args.warmup,
+        "ms_per_step": t["kernel_ms_per_step"], "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "bf16",
+        "data": "synthetic",
+        "config": {
+            "workload": f"{name}-shaped greedy decode of {B} requests in one launch per step, {args.prompt_len}-token prompts, "
+                        f"{new_tokens} new tokens per row; timed: the last {timed} decode steps (contexts {t['first_timed_context']}.."
+                        f"{t['last_timed_context']}), seeded random-init bf16 weights drawn on the GPU",
+            "layers": shape.num_hidden_layers, "experts": shape.num_experts, "experts_per_token": shape.num_experts_per_tok,
+            "batch": B, "seed": args.seed, "weight_bytes_per_row": shape.weight_bytes_per_token(),
+            "distinct_experts_per_layer": t["distinct_experts_per_layer"],
+            "queues": int(globs.instructions.shape[0]), "instructions_per_queue": int(globs.instructions.shape[1]),
+        },
+        "tok_s": t["effective_tok_s_wall"], "tok_s_gpu": t["effective_tok_s_gpu"], "kernel_tok_s": t["kernel_tok_s"],
+        "first_tokens": out["new_tokens"][:, :4].tolist(),
+        "roofline": {
+            "bound": "hbm", "achieved": t["achieved_GBps"], "peak": HBM_PEAK_GBPS, "unit": "GB/s", "frac": t["achieved_GBps"] / HBM_PEAK_GBPS,
+            "traffic": None, "traffic_source": None, "bytes_per_launch_avg": t["algorithmic_bytes"] / max(timed, 1),
+            "bytes_if_rows_alone_avg": t["moved_if_rows_alone"] / max(timed, 1),
+            "kernel": "decode_megakernel_moe_rows<Qwen3MoeA3B>",
+            "note": "algorithmic bytes = attention, router, LM head once + every row's KV rows + each DISTINCT expert of a layer once",
+        },
+        "cpu_baseline": None,
+    }
 
 
 def moe_decode_rows(args, shape, name: str, globs, kv_capacity: int, new_tokens: int, timed: int) -> dict:
@@ -427,6 +479,9 @@ def main() -> None:
                          "(one JSON line, metric attention_phase_GBps)")
     ap.add_argument("--batch", type=int, default=1,
                     help="rows decoded together (2..16: the batch route's kernel, Llama-3.2-1B or Qwen3-1.7B shape; tokens/s counts all rows)")
+    ap.add_argument("--rows-side-by-side", action="store_true",
+                    help="MoE shapes with --batch B: one batch-1 launch per row and step (the only way for a shape with a shared "
+                         "expert or more than 4 rows) instead of the B requests in one launch")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also run one 1 GiB device-to-device copy (a kernel of known traffic, for scaling rocprofv3 counters)")
     args = ap.parse_args()

@@ -407,6 +407,41 @@ int qmk_decode_step_moe(const QmkMoeArgs* args);
 /* Size of QmkMoeArgs.workspace; 0 when an argument is out of range. */
 uint64_t qmk_moe_workspace_bytes(int top_k, int shared_k_slices);
 
+/*
+ * One decode step of the MoE route for 1..4 requests ("rows") in ONE launch.  The reference has no MoE route for
+ * batch sizes above one (its batch route, …/llama3_2__1b/A100/multi_batch/decode_kernel/mk.h:9-42, is dense); a step
+ * is defined as the batch-1 route above run for every row on that row's own buffers, and every row's results are
+ * those of the row decoded alone, bit for bit.  What the launch saves is traffic: attention weights, router and LM
+ * head are read once per step, and each expert once for all the rows that picked it.
+ *
+ * `step` is a QmkMoeArgs in which every per-request buffer carries a leading row dimension — hidden_states [B, H],
+ * k_cache [B, L, 1, S, Hkv, D], logits [B, vocab], expert_indices [B, top_k], routed_silu_buffer [B, top_k, Fm], … —
+ * so row r's slice is a batch-1 buffer set; the weights, the RoPE tables, `instructions` and `barriers` exist once.
+ * step.pos_id is ignored: row r decodes position_ids[r].  Models without a shared expert only (shared_ffn = 0:
+ * QMK_MODEL_QWEN3_30B_A3B), QMK_FLAG_TAGGED required, Fm <= 1024, B x (E rounded up to 64) <= 512.
+ * step.workspace: qmk_moe_rows_workspace_bytes(B) bytes (one set of tagged units per row), zeroed once.
+ *
+ * Instruction stream: opcodes 1, 4, 7, 8 as above, each for all rows; 2 and 9 with the row in the word behind
+ * their batch-1 operands; and instead of 12/13/14
+ *   [15, layer, part, nparts, tile]     gate/up rows of the layer's DISTINCT experts (the rows' picks merged on the
+ *                                       device, ascending), dealt over the instruction's waves at run time
+ *   [16, layer, n_start, n_end, tile]   down-projection rows [n_start*tile, n_end*tile) of every distinct expert and
+ *                                       the commit of those rows for every request (tile 8 or 16, at most 16 rows).
+ */
+typedef struct QmkMoeRowsArgs {
+  uint32_t struct_size;            /* = sizeof(QmkMoeRowsArgs)                    */
+  int32_t batch_size;              /* B, 1..4                                     */
+  const int32_t* position_ids;     /* int32 [B] on the device                     */
+  int32_t* distinct_experts;       /* int32 [num_layers] on the device, or NULL: the number of distinct experts each
+                                      layer streamed in this launch (what a step's algorithmic bytes are counted from) */
+  QmkMoeArgs step;                 /* step.struct_size = sizeof(QmkMoeArgs)       */
+} QmkMoeRowsArgs;
+
+int qmk_decode_step_moe_rows(const QmkMoeRowsArgs* args);
+
+/* Size of QmkMoeRowsArgs.step.workspace; 0 when batch_size is out of range. */
+uint64_t qmk_moe_rows_workspace_bytes(int batch_size);
+
 /* Size of QmkArgs.workspace for QMK_FLAG_TAGGED; 0 for an unknown model. */
 uint64_t qmk_workspace_bytes(int model);
 

@@ -16,6 +16,7 @@
 #include "qmk_mb_ops.h"
 #include "qmk_moe_ops.h"
 #include "qmk_ops.h"
+#include "qmk_rows_ops.h"
 
 // Workspace of qmk_decode_step_static: the tagged units, the greedy candidates and the launch count
 // that qmk_decode_step keeps in the caller's QmkArgs.workspace, here in an array of the library's own
@@ -368,6 +369,120 @@ __global__ __launch_bounds__(kThreads, 1) void decode_megakernel_moe(const Param
   }
 }
 
+
+// The MoE route for several requests in one launch (qmk_rows_ops.h): the same queue walk; opcodes 1, 4, 7, 8 for all
+// rows at once, 2 and 9 as the batch-1 ops on a row's view of the buffers, 15 and 16 over the layer's distinct experts.
+// The parameters are the kernel's by-value argument throughout.
+template <class M>
+__global__ __launch_bounds__(kThreads, 1) void decode_megakernel_moe_rows(const Params p) {
+  __shared__ rows::Smem<M> s;
+  if (threadIdx.x < 8) s.b.ctl[threadIdx.x] = 0;
+  if (threadIdx.x < rows::kMaxRows) {
+    const int b = threadIdx.x;
+    int pos = 0;
+    if (b < p.batch) {
+      pos = p.position_ids[b];
+      if (pos < 0 || pos >= p.max_seq_len || pos >= p.rope_rows) {
+        s.b.ctl[0] = 1;
+        report_error(p, QMK_DEV_BAD_OPERAND, -1, 0, b);
+        pos = 0;
+      }
+    }
+    s.pos[b] = pos;
+  }
+  if (threadIdx.x == 0) {
+    s.route_layer = -1;
+    s.n_list = 0;
+    s.b.route_layer = -1;
+    s.b.generation = ld_shared32(p.ws + kWsGeneration);   // row 0's workspace keeps the launch count for all rows
+    s.b.best_val = -INFINITY;
+    s.b.best_idx = 0x7fffffff;
+  }
+  __syncthreads();
+  bool ok = s.b.ctl[0] == 0;
+  const int32_t* queue = p.instructions + static_cast<size_t>(blockIdx.x) * p.num_insts * kInstWords;
+  int32_t word = (threadIdx.x < kInstWords && p.num_insts > 0) ? queue[threadIdx.x] : 0;
+  int32_t word1 = (threadIdx.x < kInstWords && p.num_insts > 1) ? queue[kInstWords + threadIdx.x] : 0;
+  const int num_insts = p.num_insts;
+  for (int i = 0; i < num_insts && ok; ++i) {
+    if (threadIdx.x < kInstWords) {
+      s.b.inst[threadIdx.x] = word;
+      s.b.next[threadIdx.x] = word1;
+      word = word1;
+      word1 = (i + 2 < num_insts) ? queue[(i + 2) * kInstWords + threadIdx.x] : 0;
+    }
+    __syncthreads();
+    const int opcode = s.b.inst[0];
+    int tid = threadIdx.x;
+    asm volatile("" : "+v"(tid));
+    const Ctx c{i, opcode, tid};
+    unsigned long long t_start = 0;
+    if (p.timeline != nullptr && threadIdx.x == 0) {
+      t_start = wall_clock64();
+      for (int k = 0; k < 4; ++k) s.b.stamps[k] = t_start;
+    }
+    switch (opcode) {
+      case OP_NOOP: break;
+      case OP_RMS_QKV_ROPE: [[clang::always_inline]] ok = rows::op_qkv<M>(p, s, c); break;
+      case OP_ATTN_SPLITKV: {
+        const int row = s.b.inst[6];   // the word behind the batch-1 operands
+        if (row < 0 || row >= p.batch) {
+          ok = rows::bad_operand(p, s, c, 6);
+        } else {
+          const Params pr = rows::row_view<M>(p, row, s.pos[row]);
+          [[clang::always_inline]] ok = op_attn_splitkv<M>(pr, s.b, c);
+        }
+        break;
+      }
+      case OP_OPROJ_RESIDUAL: [[clang::always_inline]] ok = rows::op_oproj<M>(p, s, c); break;
+      case OP_RMS_LMHEAD: [[clang::always_inline]] ok = rows::op_lmhead<M>(p, s, c); break;
+      case moe::OP_ROUTER: [[clang::always_inline]] ok = rows::op_router<M>(p, s, c); break;
+      case moe::OP_TOPK: {
+        const int row = s.b.inst[2];
+        if (row < 0 || row >= p.batch) {
+          ok = rows::bad_operand(p, s, c, 2);
+        } else {
+          const Params pr = rows::row_view<M>(p, row, s.pos[row]);
+          [[clang::always_inline]] ok = moe::op_topk<M>(pr, s.b, c);
+        }
+        break;
+      }
+      case rows::OP_ROUTED_UPGATE_ROWS: [[clang::always_inline]] ok = rows::op_routed_upgate<M>(p, s, c); break;
+      case rows::OP_ROUTED_DOWN_COMMIT_ROWS: [[clang::always_inline]] ok = rows::op_routed_down_commit<M>(p, s, c); break;
+      default:
+        if (threadIdx.x == 0) report_error(p, QMK_DEV_BAD_OPCODE, i, opcode, 0);
+        ok = false;
+        break;
+    }
+    if (p.timeline != nullptr && threadIdx.x == 0) {
+      uint64_t* rec = p.timeline + (static_cast<size_t>(blockIdx.x) * p.num_insts + i) * 8;
+      rec[0] = t_start;
+      rec[1] = s.b.ctl[2] ? s.b.t_wait : t_start;
+      rec[2] = wall_clock64();
+      rec[3] = static_cast<uint64_t>(opcode) | (static_cast<uint64_t>(static_cast<uint32_t>(s.b.inst[1])) << 8);
+      for (int k = 0; k < 4; ++k) rec[4 + k] = s.b.stamps[k];
+      s.b.ctl[2] = 0;
+    }
+    __syncthreads();
+  }
+  if (!ok) return;
+  // Retire: the last workgroup clears the counters and advances the launch count the tags are derived from.
+  release_stores();
+  __syncthreads();
+  int32_t* done = counter_ptr(p, 0, p.num_layer_barriers - 1, p.barrier_slots - 1);
+  if (threadIdx.x == 0) {
+    const int prev = __hip_atomic_fetch_add(done, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    s.b.ctl[1] = (prev == static_cast<int>(gridDim.x) - 1);
+  }
+  __syncthreads();
+  if (s.b.ctl[1]) {
+    const int total = p.num_layers * p.num_layer_barriers * p.barrier_slots;
+    for (int i = threadIdx.x; i < total; i += kThreads)
+      __hip_atomic_store(p.barriers + i, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    if (threadIdx.x == 0) st_shared32(p.ws + kWsGeneration, (s.b.generation + 1u) & 0x03ffffffu);
+  }
+}
+
 static_assert(std::is_same<decltype(&decode_megakernel<Llama1B>), void (*)(const Params)>::value &&
                   std::is_same<decltype(&decode_megakernel<Qwen3_1p7B>), void (*)(const Params)>::value &&
                   std::is_same<decltype(&decode_megakernel_moe<QwenMoeA2_7B>), void (*)(const Params)>::value &&
@@ -381,6 +496,7 @@ struct DeviceInfo {
   int max_queues_batch = 0;
   int max_queues_batch_qwen3 = 0;
   int max_queues_moe = 0;
+  int max_queues_moe_rows = 0;
   int32_t* status = nullptr;
   uint64_t* scratch = nullptr;   // this device's copy of the file-scope `scratch` array
   bool static_in_use = false;    // a launch since the last status fetch used that array as its workspace
@@ -412,6 +528,9 @@ int device_info(DeviceInfo** out) {
     if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu_moe3, decode_megakernel_moe<Qwen3MoeA3B>, kThreads, 0) != hipSuccess)
       return QMK_ERR_NO_DEVICE;
     per_cu_moe = per_cu_moe3 < per_cu_moe ? per_cu_moe3 : per_cu_moe;
+    int per_cu_rows = 0;
+    if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu_rows, decode_megakernel_moe_rows<Qwen3MoeA3B>, kThreads, 0) != hipSuccess)
+      return QMK_ERR_NO_DEVICE;
     void* sym = nullptr;
     if (hipGetSymbolAddress(&sym, HIP_SYMBOL(g_status)) != hipSuccess) return QMK_ERR_NO_DEVICE;
     if (hipMemset(sym, 0, sizeof(int32_t) * kStatusWords) != hipSuccess) return QMK_ERR_NO_DEVICE;
@@ -422,6 +541,7 @@ int device_info(DeviceInfo** out) {
     d.max_queues_batch = per_cu_batch * prop.multiProcessorCount;
     d.max_queues_batch_qwen3 = per_cu_batch3 * prop.multiProcessorCount;
     d.max_queues_moe = per_cu_moe * prop.multiProcessorCount;
+    d.max_queues_moe_rows = per_cu_rows * prop.multiProcessorCount;
     d.status = static_cast<int32_t*>(sym);
     d.scratch = static_cast<uint64_t*>(scratch_ptr);
     d.ready = true;
@@ -663,6 +783,9 @@ extern "C" uint64_t qmk_moe_workspace_bytes(int top_k, int shared_k_slices) {
 namespace {
 
 template <class M>
+void fill_moe_params(const QmkMoeArgs* a, DeviceInfo* dev, Params& p);
+
+template <class M>
 int decode_step_moe(const QmkMoeArgs* a) {
   const void* required[] = {a->instructions, a->hidden_states, a->normed_hidden_states, a->q_post_rope, a->k_cache, a->v_cache,
                             a->attn_out, a->attn_lse_intermediates, a->attn_out_intermediates, a->silu_out, a->logits,
@@ -707,6 +830,22 @@ int decode_step_moe(const QmkMoeArgs* a) {
   if (a->num_insts == 0) return QMK_OK;
 
   Params p{};
+  fill_moe_params<M>(a, dev, p);
+  const uint64_t shared_bytes = ((static_cast<uint64_t>(a->shared_k_slices) * M::H * sizeof(u16) + 127) / 128) * 128;
+  p.shared_parts = static_cast<u16*>(a->workspace);
+  p.routed_parts = reinterpret_cast<float*>(static_cast<char*>(a->workspace) + shared_bytes);
+  p.shared_gate = p.routed_parts + static_cast<size_t>(a->top_k) * M::H;
+  p.ws = reinterpret_cast<uint64_t*>(reinterpret_cast<char*>(p.shared_gate) + 128);
+
+  hipLaunchKernelGGL(decode_megakernel_moe<M>, dim3(a->num_queues), dim3(kThreads), 0, static_cast<hipStream_t>(a->stream), p);
+  return hipGetLastError() == hipSuccess ? QMK_OK : QMK_ERR_LAUNCH;
+}
+
+// The fields of Params that come straight from a QmkMoeArgs (everything but the workspace's regions).
+template <class M>
+void fill_moe_params(const QmkMoeArgs* a, DeviceInfo* dev, Params& p) {
+  const int routed_tile = a->routed_upgate_tile == 0 ? moe::kTile : a->routed_upgate_tile;
+  const int oproj_tile = a->oproj_tile == 0 ? moe::kTile : a->oproj_tile;
   p.instructions = a->instructions;
   p.hidden = static_cast<u16*>(a->hidden_states);
   p.q_post_rope = static_cast<u16*>(a->q_post_rope);
@@ -763,11 +902,6 @@ int decode_step_moe(const QmkMoeArgs* a) {
   p.routed_silu = static_cast<u16*>(a->routed_silu_buffer);
   p.routed_out_f32 = a->routed_out_f32;
   p.routed_out = static_cast<u16*>(a->routed_out);
-  p.shared_parts = static_cast<u16*>(a->workspace);
-  const uint64_t shared_bytes = ((static_cast<uint64_t>(a->shared_k_slices) * M::H * sizeof(u16) + 127) / 128) * 128;
-  p.routed_parts = reinterpret_cast<float*>(static_cast<char*>(a->workspace) + shared_bytes);
-  p.shared_gate = p.routed_parts + static_cast<size_t>(a->top_k) * M::H;
-  p.ws = reinterpret_cast<uint64_t*>(reinterpret_cast<char*>(p.shared_gate) + 128);
   p.num_experts = a->num_experts;
   p.top_k = a->top_k;
   p.shared_ffn = a->shared_ffn;
@@ -776,8 +910,57 @@ int decode_step_moe(const QmkMoeArgs* a) {
   p.norm_topk = a->norm_topk_prob;
   p.routed_tile = routed_tile;
   p.local_routing = a->local_routing;
+}
 
-  hipLaunchKernelGGL(decode_megakernel_moe<M>, dim3(a->num_queues), dim3(kThreads), 0, static_cast<hipStream_t>(a->stream), p);
+// Units from one row's tagged workspace to the next in a launch of several rows: a batch-1 launch's units, in whole lines.
+constexpr int kWsRowUnits = ((kWsMoeUnits + 15) / 16) * 16;
+
+template <class M>
+int decode_step_moe_rows(const QmkMoeRowsArgs* r) {
+  const QmkMoeArgs* a = &r->step;
+  const int B = r->batch_size;
+  if (B < 1 || B > rows::kMaxRows) return QMK_ERR_SHAPE;
+  const void* required[] = {a->instructions, a->hidden_states, a->normed_hidden_states, a->q_post_rope, a->k_cache, a->v_cache,
+                            a->attn_out, a->attn_lse_intermediates, a->attn_out_intermediates, a->silu_out, a->logits,
+                            a->attn_norm_weights, a->qkv_weights, a->rope_cos, a->rope_sin, a->o_proj_weights,
+                            a->mlp_norm_weights, a->lm_head_norm_weights, a->lm_head_weights, a->router_weights,
+                            a->router_logits_buf, a->expert_indices, a->expert_weights, a->expert_gate_up_proj_weights,
+                            a->expert_down_proj_weights, a->routed_silu_buffer, a->routed_out_f32, a->routed_out, a->barriers,
+                            a->workspace, r->position_ids};
+  for (const void* ptr : required)
+    if (ptr == nullptr) return QMK_ERR_NULL_ARG;
+  if (M::QKV_BIAS && a->qkv_bias == nullptr) return QMK_ERR_NULL_ARG;
+  if (M::QK_NORM && (a->qkv_raw == nullptr || a->q_norm_weights == nullptr || a->k_norm_weights == nullptr)) return QMK_ERR_NULL_ARG;
+  if (a->shared_ffn != 0 || a->shared_k_slices != 0) return QMK_ERR_SHAPE;   // the committing stream has no shared expert
+  if (a->num_queues < 1 || a->num_insts < 0 || a->num_layers < 1 || a->num_layers > 63 || a->num_layer_barriers < 15 ||
+      a->barrier_slots < 8 || a->max_seq_len < 1 || a->max_splits < 1 || a->vocab_size < 1 || a->rope_rows < 1)
+    return QMK_ERR_SHAPE;
+  // a wave per expert slot of a row's softmax, the rows side by side: rows x (experts in whole waves) threads
+  if (a->num_experts < 1 || a->num_experts > moe::kMaxExperts || ((a->num_experts + kWaveSize - 1) / kWaveSize) * kWaveSize * B > kThreads ||
+      a->top_k < 1 || a->top_k > moe::kMaxTopK || a->top_k > a->num_experts || a->moe_ffn < 16 || a->moe_ffn % 16 || a->moe_ffn > 1024)
+    return QMK_ERR_SHAPE;
+  if (a->norm_topk_prob != 0 && a->norm_topk_prob != 1) return QMK_ERR_SHAPE;
+  const int oproj_tile = a->oproj_tile == 0 ? moe::kTile : a->oproj_tile;
+  if (oproj_tile != 8 && oproj_tile != 16) return QMK_ERR_SHAPE;
+  if (a->flags != QMK_FLAG_TAGGED) return QMK_ERR_SHAPE;   // tagged hand-over, self-clearing counters: nothing else is built
+  if (reinterpret_cast<uintptr_t>(a->workspace) % 128 != 0 || a->workspace_bytes < qmk_moe_rows_workspace_bytes(B)) return QMK_ERR_SHAPE;
+
+  DeviceInfo* dev = nullptr;
+  if (int rc = device_info(&dev); rc != QMK_OK) return rc;
+  if (a->num_queues > dev->max_queues_moe_rows) return QMK_ERR_TOO_MANY_QUEUES;
+  if (a->num_insts == 0) return QMK_OK;
+
+  Params p{};
+  fill_moe_params<M>(a, dev, p);
+  p.local_routing = 1;
+  p.ws = static_cast<uint64_t*>(a->workspace);
+  p.ws_row_units = kWsRowUnits;
+  p.batch = B;
+  p.position_ids = r->position_ids;
+  p.distinct_out = r->distinct_experts;
+  p.rope_rows = a->rope_rows;
+  p.pos_id = 0;
+  hipLaunchKernelGGL(decode_megakernel_moe_rows<M>, dim3(a->num_queues), dim3(kThreads), 0, static_cast<hipStream_t>(a->stream), p);
   return hipGetLastError() == hipSuccess ? QMK_OK : QMK_ERR_LAUNCH;
 }
 
@@ -789,6 +972,20 @@ extern "C" int qmk_decode_step_moe(const QmkMoeArgs* a) {
   switch (a->model) {
     case QMK_MODEL_QWEN1_5_MOE_A2_7B: return decode_step_moe<QwenMoeA2_7B>(a);
     case QMK_MODEL_QWEN3_30B_A3B: return decode_step_moe<Qwen3MoeA3B>(a);
+    default: return QMK_ERR_MODEL;
+  }
+}
+
+extern "C" uint64_t qmk_moe_rows_workspace_bytes(int batch_size) {
+  if (batch_size < 1 || batch_size > rows::kMaxRows) return 0;
+  return static_cast<uint64_t>(batch_size) * kWsRowUnits * sizeof(uint64_t);
+}
+
+extern "C" int qmk_decode_step_moe_rows(const QmkMoeRowsArgs* r) {
+  if (r == nullptr) return QMK_ERR_NULL_ARG;
+  if (r->struct_size != sizeof(QmkMoeRowsArgs) || r->step.struct_size != sizeof(QmkMoeArgs)) return QMK_ERR_ABI;
+  switch (r->step.model) {
+    case QMK_MODEL_QWEN3_30B_A3B: return decode_step_moe_rows<Qwen3MoeA3B>(r);
     default: return QMK_ERR_MODEL;
   }
 }

@@ -120,6 +120,9 @@ struct Params {
   int32_t norm_topk;             // 1: the top-k weights are divided by their sum
   int32_t routed_tile;           // outputs per tile of the routed up/gate instructions (16, or 8)
   int32_t local_routing;         // tagged launches: 1 = the routed ops take the routing decision themselves from the logits
+  // MoE route, several requests in one launch (qmk_rows_ops.h): every per-request buffer above is [batch, ...].
+  int32_t ws_row_units;          // 8-byte units from one row's tagged workspace to the next
+  int32_t* distinct_out;         // [L] or null: distinct experts each layer streamed in this launch
 };
 
 // ---------------------------------------------------------------- bf16 ----

@@ -1,0 +1,763 @@
+// The MoE decode route for 2..4 requests ("rows") in ONE launch per step, on the batch-1 kernel's row-streaming
+// engine: a wave still reads whole weight rows as coalesced 16-byte pieces, but multiplies each piece with the
+// activation vectors of all rows, so the attention half, the router and the LM head cross the memory system once
+// per step instead of once per row, and every selected expert once for all the rows that chose it.
+//
+// The reference has no MoE route for batch sizes above one.  A step here is DEFINED as its batch-1 route
+// (qimeng_megakernel/models/LLM/qwen/qwen1_5_moe_a2_7b/A100/single_batch/decode_schedule/instructions/python_vm.py:331-530,
+// with the Qwen3 op set's attention, …/qwen/qwen3__0_6b/A100/single_batch/decode_schedule/fused/operations.py:52-120)
+// run for every row on that row's own buffers, and every row keeps the batch-1 kernel's bits: each dot product is
+// accumulated over the same pieces in the same order, the routed terms of a row are added in its own slot order.
+//
+// Layout: every per-request buffer of the batch-1 route gets a leading row dimension ([B, ...], KV cache
+// [B, L, 1, S, NKV, D]), so row r's slice IS a batch-1 buffer set; weights exist once.  Hand-over between
+// workgroups is the tagged one throughout (one workspace of self-announcing units per row); the only counters
+// are the split-KV arrivals in front of the O-projection and the retirement count.
+//
+// Opcodes: 1, 4, 7, 8 as on the batch-1 route but for all rows at once; 2 (split-KV) and 9 (the reporting top-k)
+// are the batch-1 ops run on a row's view of the buffers (the row is an extra operand word); 15 and 16 replace the
+// per-slot instructions 12/13 — the rows' picks are merged, in every workgroup alike, into the list of DISTINCT
+// experts in ascending order, and the routed work is dealt over that list at run time.
+#pragma once
+
+#include "qmk_moe_ops.h"
+
+namespace qmk {
+namespace rows {
+
+constexpr int kMaxRows = 4;
+constexpr int kMaxList = kMaxRows * moe::kMaxTopK;   // distinct experts of a layer at most
+constexpr int kRowRes = 256;                         // GEMV results per row awaiting an epilogue
+constexpr int kCommitRows = 16;                      // residual-stream rows one committing instruction takes at most
+
+enum Opcode {
+  OP_ROUTED_UPGATE_ROWS = 15,
+  OP_ROUTED_DOWN_COMMIT_ROWS = 16,
+};
+
+template <class M>
+struct Smem {
+  qmk::Smem<M> b;                       // what the batch-1 ops use when they run on a row's view (attention, top-k report)
+  int32_t pos[kMaxRows];                // position each row decodes
+  float red[2][kMaxRows][kWaves];
+  alignas(16) u16 x[kMaxRows][M::AW > M::H ? M::AW : M::H];   // the rows' activation vectors
+  float res[kMaxRows][kRowRes];
+  // the routing decision this workgroup last took (layer, -1: none yet), per row and slot, and the distinct experts
+  int32_t route_layer;
+  int32_t n_list;
+  int32_t route_expert[kMaxRows][moe::kMaxTopK];
+  float route_weight[kMaxRows][moe::kMaxTopK];
+  int32_t list_expert[kMaxList];
+  int32_t list_slot[kMaxList][kMaxRows];   // the slot in which row r picked list entry u, or -1
+  alignas(16) float prob[kMaxRows][moe::kMaxExperts];  // ranking: the rows' softmax numerators (read four at a time)
+  float picked_p[kMaxRows][moe::kMaxTopK];
+  int32_t picked_e[kMaxRows][moe::kMaxTopK];
+  int32_t wave_count[kWaves];
+  float terms[kMaxRows][moe::kMaxTopK][kCommitRows];   // committing instruction: weighted rows per (row, slot)
+};
+
+#define QMK_ROWS_STAMP(k)                                                     \
+  do {                                                                        \
+    if (p.timeline != nullptr && c.tid == 0) s.b.stamps[k] = wall_clock64(); \
+  } while (0)
+
+template <class M>
+__device__ __forceinline__ bool bad_operand(const Params& p, Smem<M>& s, const Ctx& c, int operand) {
+  return qmk::bad_operand(p, s.b, c, operand);
+}
+
+// Row r's tagged-unit workspace.
+__device__ __forceinline__ uint64_t* ws_of(const Params& p, int r) { return p.ws + static_cast<size_t>(r) * p.ws_row_units; }
+
+// The launch parameters as row r's batch-1 launch would have them: every per-request pointer moved to the row's
+// slice, the position the row's own.
+template <class M>
+__device__ __forceinline__ Params row_view(const Params& p, int r, int pos) {
+  Params q = p;
+  const size_t R = static_cast<size_t>(r);
+  const size_t cache = static_cast<size_t>(p.num_layers) * p.max_seq_len * M::NKV * M::D;
+  q.pos_id = pos;
+  q.hidden = p.hidden + R * M::H;
+  q.q_post_rope = p.q_post_rope + R * M::AW;
+  q.attn_out = p.attn_out + R * M::AW;
+  q.k_cache = p.k_cache + R * cache;
+  q.v_cache = p.v_cache + R * cache;
+  q.attn_lse = p.attn_lse + R * M::NQ * p.max_splits;
+  q.attn_partial = p.attn_partial + R * M::NQ * p.max_splits * M::D;
+  q.silu_out = p.silu_out + R * p.moe_ffn;
+  q.logits = p.logits + R * p.vocab_size;
+  q.qkv_raw = p.qkv_raw != nullptr ? p.qkv_raw + R * M::QKV : nullptr;
+  q.router_logits = p.router_logits + R * p.num_experts;
+  q.expert_indices = p.expert_indices + R * p.top_k;
+  q.expert_weights = p.expert_weights + R * p.top_k;
+  q.normed_hidden = p.normed_hidden + R * M::H;
+  q.routed_silu = p.routed_silu + R * p.top_k * p.moe_ffn;
+  q.routed_out_f32 = p.routed_out_f32 + R * M::H;
+  q.routed_out = p.routed_out + R * M::H;
+  q.ws = ws_of(p, r);
+  return q;
+}
+
+// RMSNorm of every row's residual stream into s.x[row] (the batch-1 kernel's rms_to_lds per row: the same sums in
+// the same order).  `region` >= 0: the rows' tagged units at that offset of their workspaces, each thread polling
+// its own two per row, all rows in one trip; < 0: the caller's buffers (layer 0).  `pace(k)` issues the op's k-th
+// group of weight-row requests, one group per look at the units.
+template <class M, int NP, class Pace>
+__device__ __forceinline__ bool rms_rows(const Params& p, Smem<M>& s, const Ctx& c, int region, uint32_t tag, const u16* weight, Pace pace) {
+  static_assert(M::H == kThreads * 4, "one thread normalises four elements of every row");
+  const int t = c.tid, B = p.batch;
+  const uint2 wv = *reinterpret_cast<const uint2*>(weight + t * 4);
+  uint32_t lo[kMaxRows], hi[kMaxRows];
+  static_for<0, kMaxRows>([&](auto b) { lo[b] = hi[b] = 0u; });
+  bool done = region < 0;
+  auto look = [&] {
+    uint64_t xx[kMaxRows], yy[kMaxRows];
+    static_for<0, kMaxRows>([&](auto b) {
+      xx[b] = yy[b] = static_cast<uint64_t>(tag) << 32;
+      if (b < B) {
+        const uint64_t* mine = ws_of(p, b) + region + 2 * t;
+        xx[b] = ld_shared64(mine);
+        yy[b] = ld_shared64(mine + 1);
+      }
+    });
+    bool ok = true;
+    static_for<0, kMaxRows>([&](auto b) {
+      lo[b] = static_cast<uint32_t>(xx[b]);
+      hi[b] = static_cast<uint32_t>(yy[b]);
+      ok = ok && static_cast<uint32_t>(xx[b] >> 32) == tag && static_cast<uint32_t>(yy[b] >> 32) == tag;
+    });
+    done = __builtin_amdgcn_ballot_w64(ok) == ~0ull;   // the wave moves on together: row requests are wave-wide
+  };
+  static_for<0, NP>([&](auto kk) {
+    pace(kk);
+    if (!done) look();
+  });
+  if (region < 0) {
+    static_for<0, kMaxRows>([&](auto b) {
+      if (b < B) {
+        const uint64_t hw = ld_shared64(p.hidden + static_cast<size_t>(b) * M::H + t * 4);
+        lo[b] = static_cast<uint32_t>(hw);
+        hi[b] = static_cast<uint32_t>(hw >> 32);
+      }
+    });
+  } else {
+    for (uint32_t polls = 0; !done; ++polls) {
+      if (polls > p.spin_limit) {
+        s.b.ctl[0] = 1;
+        report_error(p, QMK_DEV_WAIT_TIMEOUT, c.inst_idx, c.opcode, t);
+        break;
+      }
+      if (polls) __builtin_amdgcn_s_sleep(1);
+      look();
+    }
+    if (p.timeline != nullptr && t == 0) {
+      s.b.t_wait = wall_clock64();
+      s.b.ctl[2] = 1;
+    }
+  }
+  float ss[kMaxRows];
+  static_for<0, kMaxRows>([&](auto b) {
+    const float x0 = bf_lo(lo[b]), x1 = bf_hi(lo[b]), x2 = bf_lo(hi[b]), x3 = bf_hi(hi[b]);
+    ss[b] = wave_sum(__builtin_fmaf(x3, x3, __builtin_fmaf(x2, x2, __builtin_fmaf(x1, x1, x0 * x0))));
+  });
+  const int lane = t & 63, wave = t >> 6;
+  __syncthreads();
+  if (lane == 0) static_for<0, kMaxRows>([&](auto b) { s.red[0][b][wave] = ss[b]; });
+  __syncthreads();
+  static_for<0, kMaxRows>([&](auto b) {
+    if (b < B) {
+      float total = 0.f;
+#pragma unroll
+      for (int w = 0; w < kWaves; ++w) total += s.red[0][b][w];
+      const float mean = total / static_cast<float>(M::H);
+      const float rstd = 1.0f / sqrtf(mean + p.rms_norm_eps);
+      const float x0 = bf_lo(lo[b]), x1 = bf_hi(lo[b]), x2 = bf_lo(hi[b]), x3 = bf_hi(hi[b]);
+      const u16 y0 = f2bf(bf_lo(wv.x) * round_bf16(x0 * rstd));
+      const u16 y1 = f2bf(bf_hi(wv.x) * round_bf16(x1 * rstd));
+      const u16 y2 = f2bf(bf_lo(wv.y) * round_bf16(x2 * rstd));
+      const u16 y3 = f2bf(bf_hi(wv.y) * round_bf16(x3 * rstd));
+      uint2 out;
+      out.x = static_cast<uint32_t>(y0) | (static_cast<uint32_t>(y1) << 16);
+      out.y = static_cast<uint32_t>(y2) | (static_cast<uint32_t>(y3) << 16);
+      *reinterpret_cast<uint2*>(&s.x[b][t * 4]) = out;
+    }
+  });
+  __syncthreads();
+  return s.b.ctl[0] == 0;
+}
+
+// The rows' activation vectors of H elements from s.x into registers (lane l: columns (j*64 + l)*8 .. +7 of chunk j).
+template <class M, int CH>
+__device__ __forceinline__ void load_x_rows(const Smem<M>& s, v4u (&x)[kMaxRows][CH], int lane) {
+  static_for<0, kMaxRows>([&](auto b) { load_x_from_lds(x[b], &s.x[b][0], lane); });
+}
+
+// ===================================================================== 1 ==
+// [1, layer, tile_M, n_start, n_end, tile_M_g, tile_N_g]   the QKV rows of the instruction for every row of the batch
+template <class M>
+__device__ bool op_qkv(const Params& p, Smem<M>& s, const Ctx& c) {
+  constexpr int CH = M::H / 512;
+  const int layer = s.b.inst[1], nstart = s.b.inst[3], nend = s.b.inst[4], tile = s.b.inst[6];
+  const int bph = p.qkv_blocks_per_head, B = p.batch;
+  if (layer < 0 || layer >= p.num_layers) return bad_operand(p, s, c, 1);
+  if (tile <= 0 || (tile & 1) || tile * bph != M::D) return bad_operand(p, s, c, 6);
+  if (nstart < 0 || nend < nstart || static_cast<long>(nend) * tile > M::QKV) return bad_operand(p, s, c, 4);
+  if ((nend - nstart) * tile > kRowRes) return bad_operand(p, s, c, 3);
+  const int lane = c.tid & 63;
+  const int rs = nstart * tile, nrows = (nend - nstart) * tile;
+  const u16* W = p.qkv_w + (static_cast<size_t>(layer) * M::QKV + rs) * M::H;
+  auto src = [&](int r) { return W + static_cast<size_t>(r) * M::H; };
+  RowRegs<CH> buf[kDepth];
+  const uint32_t tag = tag_of(s.b.generation, layer);
+  if (!rms_rows<M, kDepth>(p, s, c, layer > 0 ? kWsHiddenOut : -1, tag - 1, p.attn_norm + static_cast<size_t>(layer) * M::H,
+                           [&](auto k) { preload_range<decltype(k)::value, decltype(k)::value + 1>(nrows, src, buf); }))
+    return false;
+  QMK_ROWS_STAMP(0);
+  v4u x[kMaxRows][CH];
+  load_x_rows<M, CH>(s, x, lane);
+  stream<CH>(nrows, src, buf, [&](int r, const RowRegs<CH>& w) {
+    float sum[kMaxRows];
+    static_for<0, kMaxRows>([&](auto b) { sum[b] = wave_sum(dot_row(w, x[b])); });
+    if (lane == 0) static_for<0, kMaxRows>([&](auto b) { s.res[b][r] = sum[b]; });
+  });
+  QMK_ROWS_STAMP(1);
+  __syncthreads();
+  // Epilogue per (row, output pair): the GEMV result is bf16 before anything else happens to it.
+  const int pairs = nrows / 2;
+  const size_t cache = static_cast<size_t>(p.num_layers) * p.max_seq_len * M::NKV * M::D;
+  for (int item = c.tid; item < B * pairs; item += kThreads) {
+    const int b = item / pairs, pair = item % pairs;
+    const int r = rs + 2 * pair;
+    float a0 = s.res[b][2 * pair], a1 = s.res[b][2 * pair + 1];
+    if constexpr (M::QKV_BIAS) {
+      const uint32_t bw = *reinterpret_cast<const uint32_t*>(p.qkv_bias + static_cast<size_t>(layer) * M::QKV + r);
+      a0 += bf_lo(bw), a1 += bf_hi(bw);
+    }
+    const float v0 = round_bf16(a0), v1 = round_bf16(a1);
+    uint64_t* ws = ws_of(p, b);
+    constexpr int kq = M::NQ * M::D, kk = (M::NQ + M::NKV) * M::D;
+    if constexpr (M::QK_NORM) {
+      const uint32_t w = static_cast<uint32_t>(f2bf(v0)) | (static_cast<uint32_t>(f2bf(v1)) << 16);
+      st_shared32(p.qkv_raw + static_cast<size_t>(b) * M::QKV + r, w);
+      st_tagged(ws + (r < kq ? kWsQ + r / 2 : (r < kk ? kWsK + (r - kq) / 2 : kWsV + (r - kk) / 2)), w, tag);
+    } else {
+      const int pos = s.pos[b];
+      const float* cosr = p.rope_cos + static_cast<size_t>(pos) * M::D;
+      const float* sinr = p.rope_sin + static_cast<size_t>(pos) * M::D;
+      const size_t kv_row = static_cast<size_t>(b) * cache + (static_cast<size_t>(layer) * p.max_seq_len + pos) * (M::NKV * M::D);
+      if (r < kq) {
+        const uint32_t w = rope_pair(v0, v1, cosr, sinr, r % M::D);
+        st_shared32(p.q_post_rope + static_cast<size_t>(b) * M::AW + r, w);
+        st_tagged(ws + kWsQ + r / 2, w, tag);
+      } else if (r < kk) {
+        const int i = r - kq;
+        const uint32_t w = rope_pair(v0, v1, cosr, sinr, i % M::D);
+        st_shared32(p.k_cache + kv_row + i, w);
+        st_tagged(ws + kWsK + i / 2, w, tag);
+      } else {
+        const int i = r - kk;
+        const uint32_t w = static_cast<uint32_t>(f2bf(v0)) | (static_cast<uint32_t>(f2bf(v1)) << 16);
+        st_shared32(p.v_cache + kv_row + i, w);
+        st_tagged(ws + kWsV + i / 2, w, tag);
+      }
+    }
+  }
+  return true;   // the units announce themselves
+}
+
+// ===================================================================== 4 ==
+// [4, layer, tile_M, n_start, n_end, P, tile_M_g, tile_N_g]
+// Every row's split-KV partials merged by this workgroup itself (P per KV head: the batch-1 op's self-merge, row by
+// row), then hidden[b][r] = bf16(hidden[b][r] + bf16(W_o[r] . attn_out[b])) for the instruction's rows r.
+template <class M>
+__device__ bool op_oproj(const Params& p, Smem<M>& s, const Ctx& c) {
+  constexpr int AW = M::AW, CH = AW / 512;
+  static_assert(AW % (kThreads * 4) == 0, "whole 8-byte pieces per thread");
+  const int layer = s.b.inst[1], nstart = s.b.inst[3], nend = s.b.inst[4], P = s.b.inst[5], tile = s.b.inst[7];
+  const int B = p.batch;
+  if (layer < 0 || layer >= p.num_layers) return bad_operand(p, s, c, 1);
+  if (tile <= 0 || (tile & 1)) return bad_operand(p, s, c, 7);
+  if (nstart < 0 || nend < nstart || static_cast<long>(nend) * tile > M::H) return bad_operand(p, s, c, 4);
+  if ((nend - nstart) * tile > kRowRes || B * (nend - nstart) * tile / 2 > kThreads) return bad_operand(p, s, c, 3);
+  if (P < 1 || P > kMaxSelfMerge || P > p.max_splits) return bad_operand(p, s, c, 5);
+  const int lane = c.tid & 63;
+  const int rs = nstart * tile, nrows = (nend - nstart) * tile, pairs = nrows / 2;
+  const u16* W = p.o_w + (static_cast<size_t>(layer) * M::H + rs) * AW;
+  auto src = [&](int r) { return W + static_cast<size_t>(r) * AW; };
+  RowRegs<CH> buf[kOprojBuffers];
+  preload<CH>(nrows, src, buf);
+  const uint32_t tag = tag_of(s.b.generation, layer);
+  // the residual values this thread adds to: those the previous layer's commit announced (layer 0: the caller's buffer)
+  const int my_b = c.tid / max(pairs, 1), my_pair = c.tid % max(pairs, 1);
+  const bool adds = c.tid < B * pairs;
+  uint32_t res_old = 0;
+  if (adds) {
+    if (layer == 0) {
+      res_old = ld_shared32(p.hidden + static_cast<size_t>(my_b) * M::H + rs + 2 * my_pair);
+    } else if (!poll_tagged1(ws_of(p, my_b) + kWsHiddenOut + (rs + 2 * my_pair) / 2, tag - 1, p.spin_limit, res_old)) {
+      s.b.ctl[0] = 1;   // seen by everybody after the barrier inside the wait below
+      report_error(p, QMK_DEV_WAIT_TIMEOUT, c.inst_idx, c.opcode, c.tid);
+    }
+  }
+  if (!wg_wait(p, s.b, c, 1, [&](int) { return counter_ptr(p, layer, ROW_REDUCE, 0); }, B * M::NKV * P)) return false;
+  // Item t (one or two per thread) is dims 4*(t % (D/4)).. of head t / (D/4); four partials of every item per round,
+  // all loads first — the batch-1 op's arithmetic, one row of the batch after the other.
+  constexpr int kItems = AW / (kThreads * 4);
+  for (int b = 0; b < B; ++b) {
+    const float* lse_b = p.attn_lse + static_cast<size_t>(b) * M::NQ * p.max_splits;
+    const float* part_b = p.attn_partial + static_cast<size_t>(b) * M::NQ * p.max_splits * M::D;
+    const float* lse[kItems];
+    const float* part[kItems];
+    float mx[kItems], den[kItems], n0[kItems], n1[kItems], n2[kItems], n3[kItems];
+#pragma unroll
+    for (int k = 0; k < kItems; ++k) {
+      const int item = c.tid + k * kThreads;
+      const int h = item / (M::D / 4), d0 = 4 * (item % (M::D / 4));
+      lse[k] = lse_b + static_cast<size_t>(h) * p.max_splits;
+      part[k] = part_b + static_cast<size_t>(h) * p.max_splits * M::D + d0;
+      mx[k] = -INFINITY;
+      den[k] = n0[k] = n1[k] = n2[k] = n3[k] = 0.f;
+    }
+    for (int j0 = 0; j0 < P; j0 += 4) {
+      float e[kItems][4];
+      v4u o[kItems][4];
+#pragma unroll
+      for (int k = 0; k < kItems; ++k)
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+          const int j = min(j0 + q, P - 1);
+          e[k][q] = (j0 + q < P) ? ld_shared_f32(lse[k] + j) : -INFINITY;
+          o[k][q] = ld_shared128(part[k] + static_cast<size_t>(j) * M::D);
+        }
+#pragma unroll
+      for (int k = 0; k < kItems; ++k) {
+        float mn = mx[k];
+#pragma unroll
+        for (int q = 0; q < 4; ++q) mn = fmaxf(mn, e[k][q]);
+        const float rescale = (mx[k] == -INFINITY) ? 0.f : exp2_fast(mx[k] - mn);
+        den[k] *= rescale; n0[k] *= rescale; n1[k] *= rescale; n2[k] *= rescale; n3[k] *= rescale;
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+          const float f = (e[k][q] == -INFINITY) ? 0.f : exp2_fast(e[k][q] - mn);
+          den[k] += f;
+          n0[k] = __builtin_fmaf(__uint_as_float(o[k][q].x), f, n0[k]);
+          n1[k] = __builtin_fmaf(__uint_as_float(o[k][q].y), f, n1[k]);
+          n2[k] = __builtin_fmaf(__uint_as_float(o[k][q].z), f, n2[k]);
+          n3[k] = __builtin_fmaf(__uint_as_float(o[k][q].w), f, n3[k]);
+        }
+        mx[k] = mn;
+      }
+    }
+#pragma unroll
+    for (int k = 0; k < kItems; ++k) {
+      const int item = c.tid + k * kThreads;
+      const float inv = den[k] > 0.f ? 1.0f / den[k] : 0.f;
+      const uint32_t lo = static_cast<uint32_t>(f2bf(n0[k] * inv)) | (static_cast<uint32_t>(f2bf(n1[k] * inv)) << 16);
+      const uint32_t hi = static_cast<uint32_t>(f2bf(n2[k] * inv)) | (static_cast<uint32_t>(f2bf(n3[k] * inv)) << 16);
+      *reinterpret_cast<uint2*>(&s.x[b][item * 4]) = make_uint2(lo, hi);
+      if (nstart == 0) {  // one workgroup also leaves attn_out in memory, as the reference does
+        u16* out = p.attn_out + static_cast<size_t>(b) * AW + item * 4;
+        st_shared32(out, lo);
+        st_shared32(out + 2, hi);
+      }
+    }
+  }
+  __syncthreads();
+  QMK_ROWS_STAMP(0);
+  // The activation pieces come from LDS as they are used (CH * rows of them do not fit the registers beside the rows).
+  stream<CH>(nrows, src, buf, [&](int r, const RowRegs<CH>& w) {
+    static_for<0, kMaxRows>([&](auto b) {
+      float a = 0.f;
+#pragma unroll
+      for (int j = 0; j < CH; ++j) a = dot8(w.v[j], *reinterpret_cast<const v4u*>(&s.x[b][(j * kWaveSize + lane) * 8]), a);
+      const float sum = wave_sum(a);
+      if (lane == 0) s.res[b][r] = sum;
+    });
+  });
+  QMK_ROWS_STAMP(1);
+  __syncthreads();
+  if (adds) {
+    const uint32_t w = residual_word(res_old, s.res[my_b][2 * my_pair], s.res[my_b][2 * my_pair + 1]);
+    st_tagged(ws_of(p, my_b) + kWsHiddenMid + (rs + 2 * my_pair) / 2, w, tag);
+    st_shared32(p.hidden + static_cast<size_t>(my_b) * M::H + rs + 2 * my_pair, w);
+  }
+  return true;
+}
+
+// ===================================================================== 8 ==
+// [8, layer, e_start, e_end, write_normed_hidden, tile_N_g]   router logits of the instruction's experts for every row
+template <class M>
+__device__ bool op_router(const Params& p, Smem<M>& s, const Ctx& c) {
+  constexpr int CH = M::H / 512;
+  const int layer = s.b.inst[1], g = s.b.inst[5], e0 = s.b.inst[2] * g, e1 = min(s.b.inst[3] * g, p.num_experts);
+  const int B = p.batch;
+  if (layer < 0 || layer >= p.num_layers) return bad_operand(p, s, c, 1);
+  if (g < 1 || e0 < 0 || e1 < e0) return bad_operand(p, s, c, 2);
+  const int lane = c.tid & 63, wave = c.tid >> 6;
+  const u16* w = p.router_w + static_cast<size_t>(layer) * p.num_experts * M::H;
+  const uint32_t tag = tag_of(s.b.generation, layer);
+  RowRegs<CH> first;   // the wave's first expert row lands during the wait for the residual stream
+#pragma unroll
+  for (int j = 0; j < CH; ++j) first.v[j] = v4u{0, 0, 0, 0};
+  if (e0 + wave < e1) load_row(first, w + static_cast<size_t>(e0 + wave) * M::H, lane);
+  if (!rms_rows<M, 0>(p, s, c, kWsHiddenMid, tag, p.mlp_norm + static_cast<size_t>(layer) * M::H, [](auto) {})) return false;
+  v4u x[kMaxRows][CH];
+  load_x_rows<M, CH>(s, x, lane);
+  for (int e = e0 + wave; e < e1; e += kWaves) {
+    RowRegs<CH> row = first;
+    if (e != e0 + wave) load_row(row, w + static_cast<size_t>(e) * M::H, lane);
+    float v[kMaxRows];
+    static_for<0, kMaxRows>([&](auto b) { v[b] = wave_sum(dot_row(row, x[b])); });
+    static_for<0, kMaxRows>([&](auto b) {
+      if (lane == b && b < B) {
+        st_shared_f32(p.router_logits + static_cast<size_t>(b) * p.num_experts + e, v[b]);
+        st_tagged(ws_of(p, b) + kWsLogits + e * kLogitStride, __float_as_uint(v[b]), tag);
+      }
+    });
+  }
+  if (s.b.inst[4] != 0)   // one instruction of a layer also leaves the normalised rows, as opcode 8 of the batch-1 route does
+    for (int i = c.tid * 2; i < B * M::H; i += kThreads * 2)
+      st_shared32(p.normed_hidden + i, *reinterpret_cast<const uint32_t*>(&s.x[i / M::H][i % M::H]));
+  return true;
+}
+
+// The routing decision of every row, taken by the consumer itself from the router's logits as they announce
+// themselves (the batch-1 kernel's rank_experts and renormalisation per row: the same function of the same 32-bit
+// values, the sums added in the same order), then the rows' picks merged into the list of distinct experts in
+// ascending order — the same list in every workgroup.  Thread t works for row t / per, expert t % per, where per is
+// the expert count rounded up to whole waves (the launcher checks rows * per <= threads), so that a row's softmax sums
+// are added up wave by wave exactly as the batch-1 kernel adds them.  Taken once per layer and workgroup.
+template <class M>
+__device__ __forceinline__ bool route_rows(const Params& p, Smem<M>& s, const Ctx& c, int layer) {
+  if (s.route_layer == layer) {
+    if (p.timeline != nullptr && c.tid == 0) {
+      s.b.t_wait = wall_clock64();
+      s.b.ctl[2] = 1;
+    }
+    return true;
+  }
+  const int E = p.num_experts, B = p.batch, K = p.top_k;
+  const int per = ((E + kWaveSize - 1) / kWaveSize) * kWaveSize, waves_per_row = per / kWaveSize;
+  const int t = c.tid, lane = t & 63, wave = t >> 6;
+  const int r = t / per, e = t % per;
+  const bool live = r < B && e < E;
+  const uint32_t tag = tag_of(s.b.generation, layer);
+  uint32_t bits = 0;
+  if (live && !poll_tagged1(ws_of(p, r) + kWsLogits + e * kLogitStride, tag, p.spin_limit, bits)) {
+    s.b.ctl[0] = 1;
+    report_error(p, QMK_DEV_WAIT_TIMEOUT, c.inst_idx, c.opcode, t);
+  }
+  if (p.timeline != nullptr && t == 0) {
+    s.b.t_wait = wall_clock64();
+    s.b.ctl[2] = 1;
+  }
+  const float logit = __uint_as_float(bits);
+  const float wmax = wave_max(live ? logit : -INFINITY);
+  __syncthreads();
+  if (lane == 0) s.red[0][0][wave] = wmax;
+  if (t < kMaxRows * moe::kMaxTopK) {
+    s.picked_p[t / moe::kMaxTopK][t % moe::kMaxTopK] = 0.f;
+    s.picked_e[t / moe::kMaxTopK][t % moe::kMaxTopK] = -1;
+  }
+  __syncthreads();
+  if (s.b.ctl[0]) return false;
+  float mx = -INFINITY;
+  if (r < B)
+    for (int w = 0; w < waves_per_row; ++w) mx = fmaxf(mx, s.red[0][0][r * waves_per_row + w]);
+  const float x = live ? expf(logit - mx) : 0.f;
+  const int padded = (E + 3) & ~3;
+  if (r < B && e < padded) s.prob[r][e] = live ? x : -1.f;   // padded to whole groups of four with values nobody goes behind
+  const float wsum = wave_sum(x);
+  if (lane == 0) s.red[1][0][wave] = wsum;
+  __syncthreads();
+  float sum = 0.f;
+  if (r < B)
+    for (int w = 0; w < waves_per_row; ++w) sum += s.red[1][0][r * waves_per_row + w];
+  const bool ok = !(r < B) || (sum > 0.f && sum < INFINITY);
+  if (!ok) s.b.ctl[3] = 1;   // a logit is NaN or infinite: no order to pick by (ctl[3] is cleared below)
+  if (live && ok) {
+    const float xm = s.prob[r][e];
+    const float4* all = reinterpret_cast<const float4*>(&s.prob[r][0]);
+    int before = 0;
+#pragma unroll 4
+    for (int k = 0; k < padded; k += 4) {
+      const float4 v = all[k >> 2];
+      before += (v.x > xm || (v.x == xm && k < e)) ? 1 : 0;
+      before += (v.y > xm || (v.y == xm && k + 1 < e)) ? 1 : 0;
+      before += (v.z > xm || (v.z == xm && k + 2 < e)) ? 1 : 0;
+      before += (v.w > xm || (v.w == xm && k + 3 < e)) ? 1 : 0;
+    }
+    if (before < K) {
+      s.picked_p[r][before] = x / sum;
+      s.picked_e[r][before] = e;
+    }
+  }
+  __syncthreads();
+  if (s.b.ctl[3]) {
+    __syncthreads();
+    if (t == 0) s.b.ctl[3] = 0;
+    return bad_operand(p, s, c, 2);
+  }
+  if (t < B * K) {   // norm_topk_prob: the picks' probabilities divided by their sum, added up in slot order (fp32)
+    const int rr = t / K, j = t % K;
+    float total = 0.f;
+    for (int q = 0; q < K; ++q) total += s.picked_p[rr][q];
+    s.route_expert[rr][j] = s.picked_e[rr][j];
+    s.route_weight[rr][j] = p.norm_topk ? s.picked_p[rr][j] / total : s.picked_p[rr][j];
+  }
+  __syncthreads();
+  // distinct experts in ascending order: thread e (< E) knows whether anybody picked expert e and in which slots
+  int slot_of[kMaxRows];
+  bool present = false;
+  static_for<0, kMaxRows>([&](auto b) {
+    slot_of[b] = -1;
+    if (t < E && b < B)
+      for (int j = 0; j < K; ++j)
+        if (s.route_expert[b][j] == t) slot_of[b] = j;
+    present = present || slot_of[b] >= 0;
+  });
+  const uint64_t mask = __builtin_amdgcn_ballot_w64(present);
+  if (lane == 0) s.wave_count[wave] = __builtin_popcountll(mask);
+  __syncthreads();
+  int offset = 0, total = 0;
+  for (int w = 0; w < kWaves; ++w) {
+    offset += w < wave ? s.wave_count[w] : 0;
+    total += s.wave_count[w];
+  }
+  if (present) {
+    const int u = offset + __builtin_popcountll(mask & ((1ull << lane) - 1ull));
+    if (u < kMaxList) {
+      s.list_expert[u] = t;
+      static_for<0, kMaxRows>([&](auto b) { s.list_slot[u][b] = slot_of[b]; });
+    }
+  }
+  if (t == 0) {
+    s.n_list = min(total, kMaxList);
+    s.route_layer = layer;
+  }
+  __syncthreads();
+  return true;
+}
+
+// ==================================================================== 15 ==
+// [15, layer, part, nparts, tile_N_g]
+// The gate and up rows of every DISTINCT expert the rows of the batch picked in this layer, streamed once against the
+// normalised residual streams of all rows: item g = (list entry g / (F/2), output pair g % (F/2)); wave w of the
+// instruction takes the items part*8 + w, + nparts*8, ... (dealt at run time: the length of the list is not known
+// to the scheduler).  silu = bf16(silu(bf16(gate . x)) * bf16(up . x)) as in opcode 12 (python_vm.py:421-464), for every
+// row that picked the expert, into that row's slot: routed_silu[row][slot] and the slot's tagged units.  A wave owns
+// both outputs of a pair (four weight rows, 16 KiB in flight), so nothing is exchanged between waves.
+template <class M>
+__device__ bool op_routed_upgate(const Params& p, Smem<M>& s, const Ctx& c) {
+  constexpr int CH = M::H / 512;
+  const int layer = s.b.inst[1], part = s.b.inst[2], nparts = s.b.inst[3];
+  const int B = p.batch, F = p.moe_ffn, K = p.top_k;
+  if (layer < 0 || layer >= p.num_layers) return bad_operand(p, s, c, 1);
+  if (nparts < 1 || part < 0 || part >= nparts) return bad_operand(p, s, c, 2);
+  const int lane = c.tid & 63, wave = c.tid >> 6;
+  const uint32_t tag = tag_of(s.b.generation, layer);
+  // the normalised rows long before the experts are known
+  if (!rms_rows<M, 0>(p, s, c, kWsHiddenMid, tag, p.mlp_norm + static_cast<size_t>(layer) * M::H, [](auto) {})) return false;
+  QMK_ROWS_STAMP(0);
+  if (!route_rows<M>(p, s, c, layer)) return false;
+  QMK_ROWS_STAMP(1);
+  const int ppe = F / 2, total = s.n_list * ppe, stride = nparts * kWaves;
+  const u16* base = p.expert_gate_up_w + static_cast<size_t>(layer) * p.num_experts * 2 * F * M::H;
+  RowRegs<CH> w[4];   // gate o, gate o+1, up o, up o+1
+  auto request = [&](int g) {
+    if (g >= total) return;
+    const int u = g / ppe, o = 2 * (g % ppe);
+    const u16* ex = base + static_cast<size_t>(s.list_expert[u]) * 2 * F * M::H;
+    load_row(w[0], ex + static_cast<size_t>(o) * M::H, lane);
+    load_row(w[1], ex + static_cast<size_t>(o + 1) * M::H, lane);
+    load_row(w[2], ex + static_cast<size_t>(F + o) * M::H, lane);
+    load_row(w[3], ex + static_cast<size_t>(F + o + 1) * M::H, lane);
+  };
+  int g = part * kWaves + wave;
+  request(g);
+  v4u x[kMaxRows][CH];
+  load_x_rows<M, CH>(s, x, lane);
+  for (; g < total; g += stride) {
+    float v[4][kMaxRows];
+    static_for<0, 4>([&](auto k) { static_for<0, kMaxRows>([&](auto b) { v[k][b] = wave_sum(dot_row(w[k], x[b])); }); });
+    const int u = g / ppe, o = 2 * (g % ppe);
+    request(g + stride);
+    static_for<0, kMaxRows>([&](auto b) {
+      if (lane == b && b < B) {
+        const int j = s.list_slot[u][b];
+        if (j >= 0) {
+          const float g0 = round_bf16(v[0][b]), g1 = round_bf16(v[1][b]);
+          const float a0 = (g0 / (1.0f + expf(-g0))) * round_bf16(v[2][b]);
+          const float a1 = (g1 / (1.0f + expf(-g1))) * round_bf16(v[3][b]);
+          const uint32_t word = static_cast<uint32_t>(f2bf(a0)) | (static_cast<uint32_t>(f2bf(a1)) << 16);
+          st_shared32(p.routed_silu + (static_cast<size_t>(b) * K + j) * F + o, word);
+          if (j == K - 1) st_shared32(p.silu_out + static_cast<size_t>(b) * F + o, word);   // what the last slot leaves, as after the VM's run
+          st_tagged(ws_of(p, b) + kWsRoutedSilu + j * 1024 + o / 2, word, tag);
+        }
+      }
+    });
+  }
+  return true;
+}
+
+// ==================================================================== 16 ==
+// [16, layer, n_start, n_end, tile_N_g]
+// ALL distinct experts of the rows [r0, r0 + n) of the residual stream and the commit, for every row of the batch:
+// wave w takes the list entries w, w + 8, ...; for each it streams the expert's n down-projection rows once (in halves
+// of four rows through a ring of two buffers) and multiplies them with the silu vector of every row that picked the
+// expert (looked at as tagged units, straight into registers: exactly the units its pieces multiply), leaving
+// bf16(W_down[e][r] . silu) * weight in the (row, slot) the expert has there.  Then, per row, the slots' terms are
+// added in slot order in fp32 and committed, hidden[b][r] = bf16(hidden[b][r] + routed[b][r])  (python_vm.py:467-530
+// without a shared expert): the batch-1 route's committing instruction for every row.
+template <class M>
+__device__ bool op_routed_down_commit(const Params& p, Smem<M>& s, const Ctx& c) {
+  constexpr int kChunks = 2, kHalf = 4;   // an expert's width is at most 1024: two 512-column chunks per row
+  const int layer = s.b.inst[1], n0 = s.b.inst[2], n1 = s.b.inst[3], tile = s.b.inst[4];
+  const int B = p.batch, K = p.moe_ffn, TK = p.top_k;
+  if (layer < 0 || layer >= p.num_layers) return bad_operand(p, s, c, 1);
+  if ((tile != 8 && tile != 16) || n0 < 0 || n1 <= n0 || n1 * tile > M::H || (n1 - n0) * tile > kCommitRows) return bad_operand(p, s, c, 3);
+  const int lane = c.tid & 63, wave = c.tid >> 6;
+  const int r0 = n0 * tile, n = (n1 - n0) * tile, pairs = n / 2;
+  const uint32_t tag = tag_of(s.b.generation, layer);
+  if (!route_rows<M>(p, s, c, layer)) return false;
+  const int halves = n / kHalf;                       // 2 or 4
+  const int mine = s.n_list > wave ? (s.n_list - wave + kWaves - 1) / kWaves : 0;   // list entries of this wave
+  const int nsteps = mine * halves;
+  const u16* base = p.expert_down_w + static_cast<size_t>(layer) * p.num_experts * M::H * K;
+  v4u ring[2][kHalf][kChunks];
+  auto request = [&](auto slot, int step) {
+    static_for<0, kHalf>([&](auto i) { static_for<0, kChunks>([&](auto q) { ring[slot][i][q] = v4u{0, 0, 0, 0}; }); });
+    if (step >= nsteps) return;
+    const int u = wave + kWaves * (step / halves), h = step % halves;
+    const u16* rows = base + (static_cast<size_t>(s.list_expert[u]) * M::H + r0 + h * kHalf) * K + lane * 8;
+    static_for<0, kHalf>([&](auto i) {
+      static_for<0, kChunks>([&](auto q) {
+        if (lane * 8 + q * 512 < K) ring[slot][i][q] = __builtin_nontemporal_load(reinterpret_cast<const v4u*>(rows + static_cast<size_t>(i) * K + q * 512));
+      });
+    });
+  };
+  request(std::integral_constant<int, 0>{}, 0);
+  request(std::integral_constant<int, 1>{}, 1);
+  // the residual pair this thread commits, from the unit the O-projection announced it in
+  const int my_b = c.tid / pairs, my_pair = c.tid % pairs;
+  const bool commits = c.tid < B * pairs;
+  uint32_t old = 0;
+  if (commits && !poll_tagged1(ws_of(p, my_b) + kWsHiddenMid + (r0 + 2 * my_pair) / 2, tag, p.spin_limit, old)) {
+    s.b.ctl[0] = 1;   // seen by everybody after the barrier in front of the commit
+    report_error(p, QMK_DEV_WAIT_TIMEOUT, c.inst_idx, c.opcode, c.tid);
+  }
+  v4u x[kMaxRows][kChunks];   // columns lane*8 + q*512 .. +7 of the silu vector of (row, its slot for the entry)
+  auto step_of = [&](auto slot, int step) {
+    if (step >= nsteps) return;
+    const int u = wave + kWaves * (step / halves), h = step % halves;
+    if (h == 0) {   // a new list entry: the silu vectors of the rows that picked it
+      static_for<0, kMaxRows>([&](auto b) { static_for<0, kChunks>([&](auto q) { x[b][q] = v4u{0, 0, 0, 0}; }); });
+      uint32_t polls = 0;
+      while (true) {
+        bool all = true;
+        static_for<0, kMaxRows>([&](auto b) {
+          const int j = b < B ? s.list_slot[u][b] : -1;
+          if (j >= 0) {   // uniform over the wave
+            const uint64_t* units = ws_of(p, b) + kWsRoutedSilu + j * 1024 + lane * 4;
+            uint64_t un[kChunks][4];
+            static_for<0, kChunks>([&](auto q) {
+              static_for<0, 4>([&](auto k) {
+                un[q][k] = static_cast<uint64_t>(tag) << 32;
+                if (lane * 8 + q * 512 < K) un[q][k] = ld_shared64(units + q * 256 + k);
+              });
+            });
+            static_for<0, kChunks>([&](auto q) {
+              static_for<0, 4>([&](auto k) { all = all && static_cast<uint32_t>(un[q][k] >> 32) == tag; });
+              x[b][q] = v4u{static_cast<uint32_t>(un[q][0]), static_cast<uint32_t>(un[q][1]), static_cast<uint32_t>(un[q][2]), static_cast<uint32_t>(un[q][3])};
+            });
+          }
+        });
+        if (__builtin_amdgcn_ballot_w64(all) == ~0ull) break;
+        if (++polls > p.spin_limit) {
+          s.b.ctl[0] = 1;
+          report_error(p, QMK_DEV_WAIT_TIMEOUT, c.inst_idx, c.opcode, u);
+          break;
+        }
+        __builtin_amdgcn_s_sleep(1);
+      }
+    }
+    static_for<0, kMaxRows>([&](auto b) {
+      const int j = b < B ? s.list_slot[u][b] : -1;
+      if (j >= 0) {
+        float v[kHalf];
+        static_for<0, kHalf>([&](auto i) {
+          float a = 0.f;
+          static_for<0, kChunks>([&](auto q) { a = dot8(ring[slot][i][q], x[b][q], a); });
+          v[i] = wave_sum(a);
+        });
+        if (lane == 0) {
+          const float weight = s.route_weight[b][j];
+          static_for<0, kHalf>([&](auto i) { s.terms[b][j][h * kHalf + i] = round_bf16(v[i]) * weight; });
+        }
+      }
+    });
+    request(slot, step + 2);
+  };
+  if (p.timeline != nullptr && c.tid == 0) {
+    s.b.t_wait = wall_clock64();
+    s.b.ctl[2] = 1;
+  }
+  for (int step = 0; step < nsteps; step += 2) {
+    step_of(std::integral_constant<int, 0>{}, step);
+    step_of(std::integral_constant<int, 1>{}, step + 1);
+  }
+  QMK_ROWS_STAMP(1);
+  __syncthreads();
+  if (s.b.ctl[0]) return false;
+  if (commits) {
+    const int r = r0 + 2 * my_pair;
+    float ro0 = 0.f, ro1 = 0.f;
+    for (int j = 0; j < TK; ++j) {
+      ro0 += s.terms[my_b][j][2 * my_pair];
+      ro1 += s.terms[my_b][j][2 * my_pair + 1];
+    }
+    const float h0 = (bf_lo(old) + ro0) + 0.f, h1 = (bf_hi(old) + ro1) + 0.f;   // opcode 14's expression without a shared term
+    const uint32_t word = static_cast<uint32_t>(f2bf(h0)) | (static_cast<uint32_t>(f2bf(h1)) << 16);
+    st_shared32(p.hidden + static_cast<size_t>(my_b) * M::H + r, word);
+    st_tagged(ws_of(p, my_b) + kWsHiddenOut + r / 2, word, tag);
+    st_shared_f32(p.routed_out_f32 + static_cast<size_t>(my_b) * M::H + r, 0.f);
+    st_shared_f32(p.routed_out_f32 + static_cast<size_t>(my_b) * M::H + r + 1, 0.f);
+  }
+  // how many distinct experts the layer streamed: what the step's algorithmic bytes are counted from
+  if (n0 == 0 && c.tid == 0 && p.distinct_out != nullptr) p.distinct_out[layer] = s.n_list;
+  __syncthreads();   // s.terms is read: the next instruction may write it
+  return true;
+}
+
+// ===================================================================== 7 ==
+// [7, start_block, end_block, tile_M_g, tile_N_g]     logits[b] = bf16(W_lm . rms(hidden[b])) for every row
+template <class M>
+__device__ bool op_lmhead(const Params& p, Smem<M>& s, const Ctx& c) {
+  constexpr int CH = M::H / 512;
+  const int bstart = s.b.inst[1], bend = s.b.inst[2], tile = s.b.inst[4];
+  const int B = p.batch;
+  if (tile <= 0) return bad_operand(p, s, c, 4);
+  if (bstart < 0 || bend < bstart || static_cast<long>(bend) * tile > p.vocab_size) return bad_operand(p, s, c, 2);
+  if (p.num_layers < 1) return bad_operand(p, s, c, 0);
+  const int lane = c.tid & 63;
+  const int rs = bstart * tile, nrows = (bend - bstart) * tile;
+  const u16* W = p.lm_w + static_cast<size_t>(rs) * M::H;
+  auto src = [&](int r) { return W + static_cast<size_t>(r) * M::H; };
+  RowRegs<CH> buf[kDepth];
+  preload<CH>(nrows, src, buf);
+  if (!rms_rows<M, 0>(p, s, c, kWsHiddenOut, tag_of(s.b.generation, p.num_layers - 1), p.lm_norm, [](auto) {})) return false;
+  v4u x[kMaxRows][CH];
+  load_x_rows<M, CH>(s, x, lane);
+  // Terminal op: nothing inside the launch reads the logits, so ordinary stores do.
+  stream<CH>(nrows, src, buf, [&](int r, const RowRegs<CH>& w) {
+    float sum[kMaxRows];
+    static_for<0, kMaxRows>([&](auto b) { sum[b] = wave_sum(dot_row(w, x[b])); });
+    static_for<0, kMaxRows>([&](auto b) {
+      if (lane == b && b < B) p.logits[static_cast<size_t>(b) * p.vocab_size + rs + r] = f2bf(sum[b]);
+    });
+  });
+  return true;
+}
+
+}  // namespace rows
+}  // namespace qmk

@@ -197,3 +197,85 @@ def decode_rows(rows: Sequence[Any], prompts: torch.Tensor, max_new_tokens: int,
     for mk in mks:
         mk.check()
     return result
+
+
+def decode_batch(globs: Any, prompts: torch.Tensor, max_new_tokens: int, *, mk: Any = None, decode_time: bool = True,
+                 timed_steps: int | None = None) -> dict[str, Any]:
+    """Greedy decode of ``prompts.shape[0]`` requests in ONE launch per step (``decode_schedule_moe.rows_kernel``):
+    ``globs`` holds the requests' buffers with a leading row dimension over one copy of the weights.  Per step: the
+    rows' embedding rows -> ``hidden_states``, their positions -> ``position_ids``, one launch, ``argmax`` per row.
+    The reference has no MoE route for batch sizes above one; the step order is its batch loop's
+    (`qimeng_megakernel/models/LLM/decode.py:536-796`).
+
+    Timing: one event pair per step around the launch.  ``algorithmic_bytes`` counts what a step has to move: the
+    attention weights, the router and the LM head once, each row's KV rows, and every DISTINCT expert the rows picked
+    once (counted by the kernel, per layer and step); ``moved_if_rows_alone`` is what the same rows cost as B launches."""
+    from .decode_schedule_moe import rows_kernel
+
+    B, T = int(prompts.shape[0]), int(prompts.shape[1])
+    if B != int(globs.hidden_states.shape[0]):
+        raise ValueError(f"{B} prompts for {int(globs.hidden_states.shape[0])} rows of buffers")
+    device = globs.hidden_states.device
+    if T + max_new_tokens > int(globs.k_cache.shape[3]):
+        raise ValueError("prompt_len + max_new_tokens exceeds the KV cache capacity")
+    mk = mk or rows_kernel.get_mk()
+    globs.instructions = None
+    rows_kernel.build(globs)
+    out = torch.zeros(B, T + max(max_new_tokens, 1), dtype=torch.long, device=device)
+    out[:, :T] = prompts.to(device)
+    distinct = torch.zeros((), dtype=torch.int64, device=device)
+
+    def step(column: int, events: list | None, count: bool) -> None:
+        globs.hidden_states.copy_(globs.embed_tokens.index_select(0, out[:, column]))
+        globs.position_ids.fill_(column)
+        if events is not None:
+            pair = (torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True))
+            pair[0].record()
+        mk(globs)
+        if events is not None:
+            pair[1].record()
+            events.append(pair)
+        if count:
+            distinct.add_(globs.distinct_experts.sum())
+        if column + 1 >= T:            # a prompt position's prediction is needed only behind the last one
+            out[:, column + 1] = globs.logits.argmax(dim=-1)
+
+    for pos in range(T):
+        step(pos, None, False)
+    total = max(max_new_tokens - 1, 0)
+    ntok = total if timed_steps is None else max(0, min(int(timed_steps), total))
+    for i in range(total - ntok):
+        step(T + i, None, False)
+    first = T + total - ntok
+    events: list = []
+    loop_start, loop_end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    torch.cuda.synchronize(device)
+    wall0 = time.perf_counter()
+    loop_start.record()
+    for i in range(ntok):
+        step(first + i, events if decode_time else None, True)
+    loop_end.record()
+    torch.cuda.synchronize(device)
+    result: dict[str, Any] = {"generated_ids": out, "new_tokens": out[:, T:]}
+    if decode_time and ntok:
+        wall = time.perf_counter() - wall0
+        gpu_s = loop_start.elapsed_time(loop_end) / 1e3
+        launch_ms = [a.elapsed_time(b) for a, b in events]
+        kernel_s = sum(launch_ms) / 1e3
+        shape = QwenMoeConfig.shape()
+        experts = int(distinct.item())
+        expert_bytes = 3 * shape.moe_intermediate_size * shape.hidden_size * 2
+        alone = sum(shape.step_bytes(first + i + 1) for i in range(ntok))            # one row's bytes per step, summed
+        shared = alone - ntok * shape.num_hidden_layers * shape.num_experts_per_tok * expert_bytes
+        kv = sum(shape.step_bytes(first + i + 1) - shape.weight_bytes_per_token() for i in range(ntok))   # one row's KV rows read + appended
+        nbytes = shared + (B - 1) * kv + experts * expert_bytes
+        result["timing"] = {
+            "decode_wall_s": wall, "decode_gpu_s": gpu_s, "mk_kernel_gpu_s": kernel_s,
+            "effective_tok_s_wall": B * ntok / wall, "effective_tok_s_gpu": B * ntok / gpu_s, "kernel_tok_s": B * ntok / kernel_s,
+            "kernel_steps": ntok, "kernel_launches": len(launch_ms), "kernel_ms_per_step": kernel_s * 1e3 / ntok,
+            "algorithmic_bytes": nbytes, "moved_if_rows_alone": B * alone,
+            "distinct_experts_per_layer": experts / (ntok * shape.num_hidden_layers),
+            "first_timed_context": first + 1, "last_timed_context": first + ntok, "achieved_GBps": nbytes / kernel_s / 1e9,
+        }
+    mk.check()
+    return result

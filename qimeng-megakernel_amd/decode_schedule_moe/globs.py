@@ -64,3 +64,6 @@ class Globals:
     silu_out: Optional[Tensor] = None
     logits: Optional[Tensor] = None
     embed_tokens: Optional[Tensor] = None
+    # several requests in one launch (rows_kernel.py): every per-request buffer above then has a leading row dimension
+    position_ids: Optional[Tensor] = None            # int32 [rows]
+    distinct_experts: Optional[Tensor] = None        # int32 [L]: distinct experts each layer streamed in the last launch

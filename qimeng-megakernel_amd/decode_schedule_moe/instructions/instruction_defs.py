@@ -200,6 +200,57 @@ class MoE_Combine_Commit(Instruction):
     tile_N_granularity: int = TILE_N_GRANULARITY
 
 
+# ---- several requests ("rows") in one launch: this build's stream, the reference has no MoE route for batch sizes
+# above one.  Opcodes 1, 4, 7, 8 keep their words and act on all rows; 2 and 9 name their row in the word behind the
+# batch-1 operands; 15 and 16 take the place of 12, 13 and 14.
+
+@dataclass
+class DecodeAttentionSplitKVRow(DecodeAttentionSplitKVMerge):
+    """Opcode 2 for one row of the batch: the batch-1 instruction on that row's buffers at that row's position."""
+
+    batch_row: int = 0
+
+
+@dataclass
+class Router_SoftmaxTopKRow(Router_SoftmaxTopK):
+    """Opcode 9 for one row of the batch (the report of that row's routing for the caller)."""
+
+    batch_row: int = 0
+
+
+@dataclass
+class RoutedExperts_UpGate_Rows(Instruction):
+    """Gate/up rows of the layer's distinct experts (the rows' picks merged on the device, ascending expert index):
+    item g = (list entry g // (Fm/2), output pair g % (Fm/2)); wave w of part ``part_idx`` takes the items
+    ``part_idx*8 + w + k * num_parts*8``.  The parts of a layer must cover 0..num_parts-1 exactly once."""
+
+    OPCODE: ClassVar[int] = 15
+    PREV_OPCODES: ClassVar[tuple[int, ...]] = (8,)
+    layer_idx: int
+    part_idx: int
+    num_parts: int
+    tile_N_granularity: int = 2
+
+
+@dataclass
+class RoutedExperts_DownCommit_Rows(Instruction):
+    """Down-projection rows [start*tile, end*tile) of every distinct expert against the silu vectors of the rows that
+    picked it, the rows' terms added per request in slot order, and the commit of those rows for every request."""
+
+    OPCODE: ClassVar[int] = 16
+    PREV_OPCODES: ClassVar[tuple[int, ...]] = (15,)
+    layer_idx: int
+    tile_N_start_idx: int
+    tile_N_end_idx: int
+    tile_N_granularity: int = 8
+
+
+ROWS_INSTRUCTION_BY_OPCODE = {
+    cls.OPCODE: cls
+    for cls in (NoOp, RMS_QKVProj_GEMV_RoPE, DecodeAttentionSplitKVRow, OProj_GEMV_Residual, RMS_LMHead_GEMV, Router_GEMV,
+                Router_SoftmaxTopKRow, RoutedExperts_UpGate_Rows, RoutedExperts_DownCommit_Rows)
+}
+
 INSTRUCTION_BY_OPCODE = {
     cls.OPCODE: cls
     for cls in (NoOp, RMS_QKVProj_GEMV_RoPE, DecodeAttentionSplitKV, DecodeAttentionReduction, OProj_GEMV_Residual, RMS_LMHead_GEMV,

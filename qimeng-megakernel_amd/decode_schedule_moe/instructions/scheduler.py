@@ -17,14 +17,18 @@ from .instruction_defs import (
     DecodeAttentionReduction,
     DecodeAttentionSplitKV,
     DecodeAttentionSplitKVMerge,
+    DecodeAttentionSplitKVRow,
     MoE_Combine_Commit,
     OProj_GEMV_Residual,
     RMS_LMHead_GEMV,
     RMS_QKVProj_GEMV_RoPE,
     RoutedExpert_DownProj,
     RoutedExpert_UpGate_SiLU,
+    RoutedExperts_DownCommit_Rows,
+    RoutedExperts_UpGate_Rows,
     Router_GEMV,
     Router_SoftmaxTopK,
+    Router_SoftmaxTopKRow,
     SharedExpert_DownProj,
     SharedExpert_UpGate_SiLU,
 )
@@ -281,6 +285,80 @@ class MoeScheduler:
         if self.topk_late and layers > 0:      # the last layer's report: the last instruction of its queue
             out[self._late_topk_queue()] += self.router_softmax_topk(layers - 1)
         return out
+
+
+@dataclass
+class MoeRowsScheduler:
+    """One step of ``rows`` requests in one launch (a model without a shared expert, tagged hand-over): per layer the QKV
+    rows, one split-KV instruction per (row, KV head, slice), the O-projection tiles (each merges every row's partials
+    itself), the router (``router_span`` experts per instruction), one part of the distinct experts' gate/up rows per
+    queue, the committing down-projection tiles; the rows' reporting top-k instructions of layer l run behind layer
+    l + 1's QKV rows, where their queue waits for the attention anyway; then the LM head."""
+
+    shape: MoeShape
+    sm_count: int
+    num_partials: int
+    rows: int
+    router_span: int = 8
+    commit_tile: int = 8
+
+    def __post_init__(self) -> None:
+        if self.shape.has_shared_expert:
+            raise ValueError("the rows stream is built for models without a shared expert")
+        if not 1 <= self.rows <= 4:
+            raise ValueError("1..4 rows")
+        self._one = MoeScheduler(self.shape, self.sm_count, self.num_partials, merge_in_oproj=True, router_span=self.router_span)
+
+    def attention_split_kv(self, layer: int) -> list[Instruction]:
+        return [DecodeAttentionSplitKVRow(layer, kvh, self.num_partials, part, merge_in_last=2, batch_row=row)
+                for row in range(self.rows) for kvh in range(self.shape.num_key_value_heads) for part in range(self.num_partials)]
+
+    def topk_reports(self, layer: int) -> list[Instruction]:
+        return [Router_SoftmaxTopKRow(layer, batch_row=row) for row in range(self.rows)]
+
+    def routed_upgate(self, layer: int) -> list[Instruction]:
+        return [RoutedExperts_UpGate_Rows(layer, part, self.sm_count) for part in range(self.sm_count)]
+
+    def routed_down_commit(self, layer: int) -> list[Instruction]:
+        tiles = self.shape.hidden_size // self.commit_tile
+        per = max(1, 16 // self.commit_tile)       # an instruction commits at most 16 rows
+        return [RoutedExperts_DownCommit_Rows(layer, lo, hi, self.commit_tile)
+                for lo, hi in _spans(tiles, max(self.sm_count, _ceil_div(tiles, per)))]
+
+    def _report_queues(self) -> list[int]:
+        """Queues in the middle of the device: the first ones run the split-KV slices, the last ones the router."""
+        mid = max(self.sm_count // 2 - 1, 0)
+        return [(mid + i) % self.sm_count for i in range(self.rows)]
+
+    def queues(self, num_layers: int | None = None) -> list[list[Instruction]]:
+        layers = self.shape.num_hidden_layers if num_layers is None else num_layers
+        n = self.sm_count
+        out: list[list[Instruction]] = [[] for _ in range(n)]
+
+        def spread(instructions: Sequence[Instruction], queues: Sequence[int]) -> None:
+            for i, ins in enumerate(instructions):
+                out[queues[i % len(queues)]].append(ins)
+
+        everyone = list(range(n))
+        for layer in range(layers):
+            spread(self._one.qkvproj(layer), everyone)
+            spread(self.attention_split_kv(layer), everyone)
+            if layer > 0:
+                for queue, ins in zip(self._report_queues(), self.topk_reports(layer - 1)):
+                    out[queue].append(ins)
+            spread(self._one.oproj(layer), everyone)
+            spread(self._one.router_gemv(layer), everyone[::-1])    # the last queues: the first ones ran the attention
+            spread(self.routed_upgate(layer), everyone)
+            spread(self.routed_down_commit(layer), everyone)
+        if layers == self.shape.num_hidden_layers:
+            spread(self._one.lmhead(), everyone)
+        if layers > 0:
+            for queue, ins in zip(self._report_queues(), self.topk_reports(layers - 1)):
+                out[queue].append(ins)
+        return out
+
+    def instruction_list(self, num_layers: int | None = None) -> list[Instruction]:
+        return [ins for q in self.queues(num_layers) for ins in q]
 
 
 def deal(instructions: Sequence[Instruction], queues: int) -> list[list[Instruction]]:
