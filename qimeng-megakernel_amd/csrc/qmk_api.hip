@@ -933,7 +933,7 @@ int decode_step_moe_rows(const QmkMoeRowsArgs* r) {
   if (M::QK_NORM && (a->qkv_raw == nullptr || a->q_norm_weights == nullptr || a->k_norm_weights == nullptr)) return QMK_ERR_NULL_ARG;
   if (a->shared_ffn != 0 || a->shared_k_slices != 0) return QMK_ERR_SHAPE;   // the committing stream has no shared expert
   if (a->num_queues < 1 || a->num_insts < 0 || a->num_layers < 1 || a->num_layers > 63 || a->num_layer_barriers < 15 ||
-      a->barrier_slots < 8 || a->max_seq_len < 1 || a->max_splits < 1 || a->vocab_size < 1 || a->rope_rows < 1)
+      a->barrier_slots < B * M::NQ || a->max_seq_len < 1 || a->max_splits < 1 || a->vocab_size < 1 || a->rope_rows < 1)
     return QMK_ERR_SHAPE;
   // a wave per expert slot of a row's softmax, the rows side by side: rows x (experts in whole waves) threads
   if (a->num_experts < 1 || a->num_experts > moe::kMaxExperts || ((a->num_experts + kWaveSize - 1) / kWaveSize) * kWaveSize * B > kThreads ||

@@ -45,12 +45,13 @@ struct Smem {
   // the routing decision this workgroup last took (layer, -1: none yet), per row and slot, and the distinct experts
   int32_t route_layer;
   int32_t n_list;
-  int32_t route_expert[kMaxRows][moe::kMaxTopK];
+  int32_t no_order;                     // ranking: a row's logits have no order (NaN or infinite)
+  alignas(16) int32_t route_expert[kMaxRows][moe::kMaxTopK];
   float route_weight[kMaxRows][moe::kMaxTopK];
   int32_t list_expert[kMaxList];
   int32_t list_slot[kMaxList][kMaxRows];   // the slot in which row r picked list entry u, or -1
-  alignas(16) float prob[kMaxRows][moe::kMaxExperts];  // ranking: the rows' softmax numerators (read four at a time)
-  float picked_p[kMaxRows][moe::kMaxTopK];
+  alignas(16) uint64_t key[kMaxRows][moe::kMaxExperts];  // ranking: {softmax numerator bits, ~expert} per row and expert (read two at a time)
+  alignas(16) float picked_p[kMaxRows][moe::kMaxTopK];
   int32_t picked_e[kMaxRows][moe::kMaxTopK];
   int32_t wave_count[kWaves];
   float terms[kMaxRows][moe::kMaxTopK][kCommitRows];   // committing instruction: weighted rows per (row, slot)
@@ -95,6 +96,9 @@ __device__ __forceinline__ Params row_view(const Params& p, int r, int pos) {
   q.routed_out_f32 = p.routed_out_f32 + R * M::H;
   q.routed_out = p.routed_out + R * M::H;
   q.ws = ws_of(p, r);
+  // the per-head counters of a row's split-KV instructions (and the row's word on the reduction row) behind those of
+  // the rows before it: NQ slots per row (the launcher checks that a counter row has room for all rows)
+  q.barriers = p.barriers + r * M::NQ;
   return q;
 }
 
@@ -279,7 +283,7 @@ __device__ bool op_oproj(const Params& p, Smem<M>& s, const Ctx& c) {
   if (tile <= 0 || (tile & 1)) return bad_operand(p, s, c, 7);
   if (nstart < 0 || nend < nstart || static_cast<long>(nend) * tile > M::H) return bad_operand(p, s, c, 4);
   if ((nend - nstart) * tile > kRowRes || B * (nend - nstart) * tile / 2 > kThreads) return bad_operand(p, s, c, 3);
-  if (P < 1 || P > kMaxSelfMerge || P > p.max_splits) return bad_operand(p, s, c, 5);
+  if (P < 0 || P > kMaxSelfMerge || P > p.max_splits) return bad_operand(p, s, c, 5);
   const int lane = c.tid & 63;
   const int rs = nstart * tile, nrows = (nend - nstart) * tile, pairs = nrows / 2;
   const u16* W = p.o_w + (static_cast<size_t>(layer) * M::H + rs) * AW;
@@ -299,7 +303,26 @@ __device__ bool op_oproj(const Params& p, Smem<M>& s, const Ctx& c) {
       report_error(p, QMK_DEV_WAIT_TIMEOUT, c.inst_idx, c.opcode, c.tid);
     }
   }
-  if (!wg_wait(p, s.b, c, 1, [&](int) { return counter_ptr(p, layer, ROW_REDUCE, 0); }, B * M::NKV * P)) return false;
+  if (P == 0) {
+    // The rows' attention outputs are complete in memory: the last split-KV arrival of every (row, KV head) merged its
+    // group's partials and counted the group's heads on the row's word of the reduction row.  All rows in one trip.
+    if (!wg_wait(p, s.b, c, B, [&](int i) { return counter_ptr(p, layer, ROW_REDUCE, i * M::NQ); }, M::NQ)) return false;
+    constexpr int kPieces = kMaxRows * AW / (kThreads * 8);   // 16-byte pieces per thread
+    v4u piece[kPieces];
+#pragma unroll
+    for (int k = 0; k < kPieces; ++k) {
+      const int at = (c.tid + k * kThreads) * 8;            // element index in [B, AW]
+      piece[k] = v4u{0, 0, 0, 0};
+      if (at < B * AW) piece[k] = ld_shared128(p.attn_out + at);
+    }
+#pragma unroll
+    for (int k = 0; k < kPieces; ++k) {
+      const int at = (c.tid + k * kThreads) * 8;
+      if (at < B * AW) *reinterpret_cast<v4u*>(&s.x[at / AW][at % AW]) = piece[k];
+    }
+  } else {
+  // one arrival per split-KV instruction, on its row's word of the reduction row
+  if (!wg_wait(p, s.b, c, B, [&](int i) { return counter_ptr(p, layer, ROW_REDUCE, i * M::NQ); }, M::NKV * P)) return false;
   // Item t (one or two per thread) is dims 4*(t % (D/4)).. of head t / (D/4); four partials of every item per round,
   // all loads first — the batch-1 op's arithmetic, one row of the batch after the other.
   constexpr int kItems = AW / (kThreads * 4);
@@ -361,6 +384,7 @@ __device__ bool op_oproj(const Params& p, Smem<M>& s, const Ctx& c) {
         st_shared32(out + 2, hi);
       }
     }
+  }
   }
   __syncthreads();
   QMK_ROWS_STAMP(0);
@@ -454,7 +478,9 @@ __device__ __forceinline__ bool route_rows(const Params& p, Smem<M>& s, const Ct
   const float logit = __uint_as_float(bits);
   const float wmax = wave_max(live ? logit : -INFINITY);
   __syncthreads();
+  QMK_ROWS_STAMP(2);   // every thread has its logit
   if (lane == 0) s.red[0][0][wave] = wmax;
+  if (t == 0) s.no_order = 0;
   if (t < kMaxRows * moe::kMaxTopK) {
     s.picked_p[t / moe::kMaxTopK][t % moe::kMaxTopK] = 0.f;
     s.picked_e[t / moe::kMaxTopK][t % moe::kMaxTopK] = -1;
@@ -465,8 +491,11 @@ __device__ __forceinline__ bool route_rows(const Params& p, Smem<M>& s, const Ct
   if (r < B)
     for (int w = 0; w < waves_per_row; ++w) mx = fmaxf(mx, s.red[0][0][r * waves_per_row + w]);
   const float x = live ? expf(logit - mx) : 0.f;
-  const int padded = (E + 3) & ~3;
-  if (r < B && e < padded) s.prob[r][e] = live ? x : -1.f;   // padded to whole groups of four with values nobody goes behind
+  // An expert goes before another when its probability is larger, or equal with the lower index: one unsigned compare
+  // of {numerator bits (not negative: ordered like the floats), ~index}.  Padded to pairs with keys nobody goes behind.
+  const int padded = (E + 1) & ~1;
+  const uint64_t my_key = (static_cast<uint64_t>(__float_as_uint(x)) << 32) | (0xffffffffu - static_cast<uint32_t>(e));
+  if (r < B && e < padded) s.key[r][e] = live ? my_key : 0ull;
   const float wsum = wave_sum(x);
   if (lane == 0) s.red[1][0][wave] = wsum;
   __syncthreads();
@@ -474,18 +503,16 @@ __device__ __forceinline__ bool route_rows(const Params& p, Smem<M>& s, const Ct
   if (r < B)
     for (int w = 0; w < waves_per_row; ++w) sum += s.red[1][0][r * waves_per_row + w];
   const bool ok = !(r < B) || (sum > 0.f && sum < INFINITY);
-  if (!ok) s.b.ctl[3] = 1;   // a logit is NaN or infinite: no order to pick by (ctl[3] is cleared below)
+  if (!ok) s.no_order = 1;   // a logit is NaN or infinite: no order to pick by
   if (live && ok) {
-    const float xm = s.prob[r][e];
-    const float4* all = reinterpret_cast<const float4*>(&s.prob[r][0]);
+    typedef uint64_t u64x2 __attribute__((ext_vector_type(2)));
+    const u64x2* all = reinterpret_cast<const u64x2*>(&s.key[r][0]);
     int before = 0;
-#pragma unroll 4
-    for (int k = 0; k < padded; k += 4) {
-      const float4 v = all[k >> 2];
-      before += (v.x > xm || (v.x == xm && k < e)) ? 1 : 0;
-      before += (v.y > xm || (v.y == xm && k + 1 < e)) ? 1 : 0;
-      before += (v.z > xm || (v.z == xm && k + 2 < e)) ? 1 : 0;
-      before += (v.w > xm || (v.w == xm && k + 3 < e)) ? 1 : 0;
+#pragma unroll 8
+    for (int k = 0; k < padded; k += 2) {
+      const u64x2 v = all[k >> 1];
+      before += v.x > my_key ? 1 : 0;
+      before += v.y > my_key ? 1 : 0;
     }
     if (before < K) {
       s.picked_p[r][before] = x / sum;
@@ -493,15 +520,15 @@ __device__ __forceinline__ bool route_rows(const Params& p, Smem<M>& s, const Ct
     }
   }
   __syncthreads();
-  if (s.b.ctl[3]) {
-    __syncthreads();
-    if (t == 0) s.b.ctl[3] = 0;
-    return bad_operand(p, s, c, 2);
-  }
+  if (s.no_order) return bad_operand(p, s, c, 2);
   if (t < B * K) {   // norm_topk_prob: the picks' probabilities divided by their sum, added up in slot order (fp32)
     const int rr = t / K, j = t % K;
+    float pk[moe::kMaxTopK];
+    *reinterpret_cast<float4*>(&pk[0]) = *reinterpret_cast<const float4*>(&s.picked_p[rr][0]);
+    *reinterpret_cast<float4*>(&pk[4]) = *reinterpret_cast<const float4*>(&s.picked_p[rr][4]);
     float total = 0.f;
-    for (int q = 0; q < K; ++q) total += s.picked_p[rr][q];
+#pragma unroll
+    for (int q = 0; q < moe::kMaxTopK; ++q) total += q < K ? pk[q] : 0.f;
     s.route_expert[rr][j] = s.picked_e[rr][j];
     s.route_weight[rr][j] = p.norm_topk ? s.picked_p[rr][j] / total : s.picked_p[rr][j];
   }
@@ -511,9 +538,14 @@ __device__ __forceinline__ bool route_rows(const Params& p, Smem<M>& s, const Ct
   bool present = false;
   static_for<0, kMaxRows>([&](auto b) {
     slot_of[b] = -1;
-    if (t < E && b < B)
-      for (int j = 0; j < K; ++j)
-        if (s.route_expert[b][j] == t) slot_of[b] = j;
+    if (t < E && b < B) {
+      int picks[moe::kMaxTopK];
+      *reinterpret_cast<int4*>(&picks[0]) = *reinterpret_cast<const int4*>(&s.route_expert[b][0]);
+      *reinterpret_cast<int4*>(&picks[4]) = *reinterpret_cast<const int4*>(&s.route_expert[b][4]);
+#pragma unroll
+      for (int j = 0; j < moe::kMaxTopK; ++j)
+        if (j < K && picks[j] == t) slot_of[b] = j;
+    }
     present = present || slot_of[b] >= 0;
   });
   const uint64_t mask = __builtin_amdgcn_ballot_w64(present);
@@ -536,6 +568,7 @@ __device__ __forceinline__ bool route_rows(const Params& p, Smem<M>& s, const Ct
     s.route_layer = layer;
   }
   __syncthreads();
+  QMK_ROWS_STAMP(3);   // the list of distinct experts is complete
   return true;
 }
 
@@ -624,7 +657,8 @@ __device__ bool op_routed_down_commit(const Params& p, Smem<M>& s, const Ctx& c)
   const int mine = s.n_list > wave ? (s.n_list - wave + kWaves - 1) / kWaves : 0;   // list entries of this wave
   const int nsteps = mine * halves;
   const u16* base = p.expert_down_w + static_cast<size_t>(layer) * p.num_experts * M::H * K;
-  v4u ring[2][kHalf][kChunks];
+  constexpr int kRing = 3;   // half tiles of a wave in flight (6 KiB each for an expert width of 768)
+  v4u ring[kRing][kHalf][kChunks];
   auto request = [&](auto slot, int step) {
     static_for<0, kHalf>([&](auto i) { static_for<0, kChunks>([&](auto q) { ring[slot][i][q] = v4u{0, 0, 0, 0}; }); });
     if (step >= nsteps) return;
@@ -636,8 +670,7 @@ __device__ bool op_routed_down_commit(const Params& p, Smem<M>& s, const Ctx& c)
       });
     });
   };
-  request(std::integral_constant<int, 0>{}, 0);
-  request(std::integral_constant<int, 1>{}, 1);
+  static_for<0, kRing>([&](auto k) { request(k, k); });
   // the residual pair this thread commits, from the unit the O-projection announced it in
   const int my_b = c.tid / pairs, my_pair = c.tid % pairs;
   const bool commits = c.tid < B * pairs;
@@ -696,16 +729,13 @@ __device__ bool op_routed_down_commit(const Params& p, Smem<M>& s, const Ctx& c)
         }
       }
     });
-    request(slot, step + 2);
+    request(slot, step + kRing);
   };
   if (p.timeline != nullptr && c.tid == 0) {
     s.b.t_wait = wall_clock64();
     s.b.ctl[2] = 1;
   }
-  for (int step = 0; step < nsteps; step += 2) {
-    step_of(std::integral_constant<int, 0>{}, step);
-    step_of(std::integral_constant<int, 1>{}, step + 1);
-  }
+  for (int step = 0; step < nsteps; step += kRing) static_for<0, kRing>([&](auto k) { step_of(k, step + k); });
   QMK_ROWS_STAMP(1);
   __syncthreads();
   if (s.b.ctl[0]) return false;

@@ -200,7 +200,7 @@ def decode_rows(rows: Sequence[Any], prompts: torch.Tensor, max_new_tokens: int,
 
 
 def decode_batch(globs: Any, prompts: torch.Tensor, max_new_tokens: int, *, mk: Any = None, decode_time: bool = True,
-                 timed_steps: int | None = None) -> dict[str, Any]:
+                 timed_steps: int | None = None, merge_in_oproj: bool = False) -> dict[str, Any]:
     """Greedy decode of ``prompts.shape[0]`` requests in ONE launch per step (``decode_schedule_moe.rows_kernel``):
     ``globs`` holds the requests' buffers with a leading row dimension over one copy of the weights.  Per step: the
     rows' embedding rows -> ``hidden_states``, their positions -> ``position_ids``, one launch, ``argmax`` per row.
@@ -209,7 +209,11 @@ def decode_batch(globs: Any, prompts: torch.Tensor, max_new_tokens: int, *, mk: 
 
     Timing: one event pair per step around the launch.  ``algorithmic_bytes`` counts what a step has to move: the
     attention weights, the router and the LM head once, each row's KV rows, and every DISTINCT expert the rows picked
-    once (counted by the kernel, per layer and step); ``moved_if_rows_alone`` is what the same rows cost as B launches."""
+    once (counted by the kernel, per layer and step); ``moved_if_rows_alone`` is what the same rows cost as B launches.
+    ``merge_in_oproj``: the batch-1 stream's way of merging the split-KV partials (see ``rows_kernel.mi355x_scheduler``);
+    with it a row's bits are those of the default batch-1 request, without it those of the batch-1 request whose
+    stream merges by the last arrival (``MoeScheduler(merge_in_last=True)``) — the two differ by what
+    ``num / den`` and ``num * (1 / den)`` differ by in the attention output."""
     from .decode_schedule_moe import rows_kernel
 
     B, T = int(prompts.shape[0]), int(prompts.shape[1])
@@ -220,7 +224,7 @@ def decode_batch(globs: Any, prompts: torch.Tensor, max_new_tokens: int, *, mk: 
         raise ValueError("prompt_len + max_new_tokens exceeds the KV cache capacity")
     mk = mk or rows_kernel.get_mk()
     globs.instructions = None
-    rows_kernel.build(globs)
+    rows_kernel.build(globs, merge_in_oproj=merge_in_oproj)
     out = torch.zeros(B, T + max(max_new_tokens, 1), dtype=torch.long, device=device)
     out[:, :T] = prompts.to(device)
     distinct = torch.zeros((), dtype=torch.int64, device=device)

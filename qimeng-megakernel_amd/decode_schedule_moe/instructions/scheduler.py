@@ -301,16 +301,20 @@ class MoeRowsScheduler:
     rows: int
     router_span: int = 8
     commit_tile: int = 8
+    merge_in_oproj: bool = False     # True: every O-projection workgroup merges every row's split-KV partials itself (the
+                                     # batch-1 stream's way); False: the last split-KV arrival of a (row, KV head) merges its
+                                     # group, and the O-projection reads the rows' finished attention outputs in one trip
 
     def __post_init__(self) -> None:
         if self.shape.has_shared_expert:
             raise ValueError("the rows stream is built for models without a shared expert")
         if not 1 <= self.rows <= 4:
             raise ValueError("1..4 rows")
-        self._one = MoeScheduler(self.shape, self.sm_count, self.num_partials, merge_in_oproj=True, router_span=self.router_span)
+        self._one = MoeScheduler(self.shape, self.sm_count, self.num_partials, merge_in_oproj=self.merge_in_oproj,
+                                 merge_in_last=not self.merge_in_oproj, router_span=self.router_span)
 
     def attention_split_kv(self, layer: int) -> list[Instruction]:
-        return [DecodeAttentionSplitKVRow(layer, kvh, self.num_partials, part, merge_in_last=2, batch_row=row)
+        return [DecodeAttentionSplitKVRow(layer, kvh, self.num_partials, part, merge_in_last=2 if self.merge_in_oproj else 1, batch_row=row)
                 for row in range(self.rows) for kvh in range(self.shape.num_key_value_heads) for part in range(self.num_partials)]
 
     def topk_reports(self, layer: int) -> list[Instruction]:

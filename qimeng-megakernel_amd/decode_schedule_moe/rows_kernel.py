@@ -164,8 +164,8 @@ class MoeRowsMegaKernel:
         if g.rope_cos.shape != g.rope_sin.shape or g.rope_cos.shape[-1] != d:
             raise ValueError("rope_cos/rope_sin must both be [positions, head_dim]")
         bar = g.barriers
-        if bar.dim() != 3 or bar.shape[1] < 15 or bar.shape[2] < 8:
-            raise ValueError(f"barriers must be [layers, >= 15, >= 8], got {tuple(bar.shape)}")
+        if bar.dim() != 3 or bar.shape[1] < 15 or bar.shape[2] < B * nq:
+            raise ValueError(f"barriers must be [layers, >= 15, >= rows x query heads = {B * nq}], got {tuple(bar.shape)}")
         self._barriers = bar
         a.num_queues, a.num_insts = int(g.instructions.shape[0]), int(g.instructions.shape[1])
         a.num_layers, a.num_layer_barriers, a.barrier_slots = L, int(bar.shape[1]), int(bar.shape[2])
@@ -221,20 +221,23 @@ def get_mk(mk_dir: Path | None = None, *, spin_limit: int = 0) -> MoeRowsMegaKer
 
 
 def mi355x_scheduler(rows: int, shape: Any = None, *, kv_capacity: int | None = None, queues: int = _moe.MI355X_QUEUES,
-                     num_partials: int | None = None) -> _scheduler.MoeRowsScheduler:
+                     num_partials: int | None = None, merge_in_oproj: bool = False) -> _scheduler.MoeRowsScheduler:
     """One queue per CU.  Split-KV fan-out: the batch-1 stream's (2 slices per KV head, 4 when the request's cache holds
-    more than 256 tokens) as long as rows x KV heads x slices stays within a quarter of the queues."""
+    more than 256 tokens) as long as rows x KV heads x slices stays within a quarter of the queues.  The partials of a
+    (row, KV head) are merged by the group's last arrival (``merge_in_oproj=True``: by every O-projection workgroup, as
+    in the batch-1 stream — with several rows that is four trips to memory per workgroup instead of one)."""
     shape = shape or QwenMoeConfig.shape()
     if num_partials is None:
         few = 2 if kv_capacity is None or kv_capacity <= 256 else 4
         num_partials = max(1, min(few, queues // (4 * rows * shape.num_key_value_heads)))
-    return _scheduler.MoeRowsScheduler(shape, queues, num_partials, rows)
+    return _scheduler.MoeRowsScheduler(shape, queues, num_partials, rows, merge_in_oproj=merge_in_oproj)
 
 
-def build(globs: Globals, *, queues: int = _moe.MI355X_QUEUES, num_partials: int | None = None) -> torch.Tensor:
+def build(globs: Globals, *, queues: int = _moe.MI355X_QUEUES, num_partials: int | None = None, merge_in_oproj: bool = False) -> torch.Tensor:
     """The instruction tensor of a batch of requests."""
     rows = int(globs.hidden_states.shape[0])
-    sched = mi355x_scheduler(rows, kv_capacity=int(globs.k_cache.shape[3]), queues=queues, num_partials=num_partials)
+    sched = mi355x_scheduler(rows, kv_capacity=int(globs.k_cache.shape[3]), queues=queues, num_partials=num_partials,
+                             merge_in_oproj=merge_in_oproj)
     if sched.num_partials > int(globs.attn_lse_intermediates.shape[-1]):
         raise ValueError("attn_lse_intermediates has fewer partial slots than the schedule's split-KV fan-out")
     return tensorize_instructions(globs, sched.queues())

@@ -54,8 +54,10 @@ def _fill_state(g, rows, seed):
     g.hidden_states.copy_(g.embed_tokens[tokens.to(g.embed_tokens.device)])
 
 
-def _rows_alone(g, shape, positions, partials):
-    """Every row of ``g`` stepped once by the batch-1 kernel on a copy of the row's buffers; the copies."""
+def _rows_alone(g, shape, positions, partials, merge_in_oproj):
+    """Every row of ``g`` stepped once by the batch-1 kernel on a copy of the row's buffers; the copies.  The batch-1
+    stream merges the split-KV partials where the rows stream does (in the O-projection workgroups, or by the last arrival
+    of a KV head: ``num * (1 / den)`` there, ``num / den`` here)."""
     out = []
     for r, pos in enumerate(positions):
         view = rows_kernel.row_view(g, r)
@@ -63,7 +65,8 @@ def _rows_alone(g, shape, positions, partials):
         for name in ROW_STATE:
             setattr(alone, name, getattr(view, name).clone())
         alone.position_id = pos
-        sched = dataclasses.replace(mk_kernel.mi355x_scheduler(shape, kv_capacity=int(g.k_cache.shape[3])), num_partials=partials)
+        sched = dataclasses.replace(mk_kernel.mi355x_scheduler(shape, kv_capacity=int(g.k_cache.shape[3])), num_partials=partials,
+                                    merge_in_oproj=merge_in_oproj, merge_in_last=not merge_in_oproj)
         tensorize_instructions(alone, sched.queues())
         mk = mk_kernel.get_mk(spin_limit=1 << 20)
         mk_kernel.call_mk(alone, mk)
@@ -73,15 +76,16 @@ def _rows_alone(g, shape, positions, partials):
     return out
 
 
+@pytest.mark.parametrize("merge_in_oproj", [False, True])
 @pytest.mark.parametrize("positions", [(41, 41, 41, 41), (70, 3, 41), (0, 95), (17,)])
-def test_one_step_of_ragged_rows_equals_each_row_alone(weights, positions):
+def test_one_step_of_ragged_rows_equals_each_row_alone(weights, positions, merge_in_oproj):
     """Rows at different positions over random pasts: one launch for all of them against one batch-1 launch per row."""
     rows = len(positions)
     g = rows_kernel.build_rows_globals(weights, SMALL, 96, rows, "cuda:0", max_partials=8)
     _fill_state(g, rows, seed=3 + rows)
     g.position_ids.copy_(torch.tensor(positions, dtype=torch.int32))
-    alone = _rows_alone(g, SMALL, positions, partials=2)
-    rows_kernel.build(g, num_partials=2)
+    alone = _rows_alone(g, SMALL, positions, partials=2, merge_in_oproj=merge_in_oproj)
+    rows_kernel.build(g, num_partials=2, merge_in_oproj=merge_in_oproj)
     mk = rows_kernel.get_mk(spin_limit=1 << 20)
     mk(g)
     mk.check()
@@ -102,7 +106,7 @@ def test_requests_decoded_together_equal_the_requests_alone(weights):
     new = 10
     prompts = torch.tensor([[3, 99, 1024, 7], [5, 5, 5, 5], [2047, 0, 1, 2], [77, 1500, 300, 9]])
     g = rows_kernel.build_rows_globals(weights, SMALL, 64, 4, "cuda:0", max_partials=8)
-    together = decode_moe.decode_batch(g, prompts, new, timed_steps=4)
+    together = decode_moe.decode_batch(g, prompts, new, timed_steps=4, merge_in_oproj=True)   # the default batch-1 request's bits
     t = together["timing"]
     assert t["kernel_steps"] == 4 and t["kernel_launches"] == 4 and t["first_timed_context"] == 4 + (new - 1 - 4) + 1
     assert 1.0 <= t["distinct_experts_per_layer"] <= 16.0
@@ -116,7 +120,7 @@ def test_requests_decoded_together_equal_the_requests_alone(weights):
     # identical requests pick identical experts: the list of distinct experts is as long as one row's picks
     same = torch.tensor([[3, 99, 1024, 7]] * 3)
     g3 = rows_kernel.build_rows_globals(weights, SMALL, 64, 3, "cuda:0", max_partials=8)
-    out = decode_moe.decode_batch(g3, same, 6, timed_steps=2)
+    out = decode_moe.decode_batch(g3, same, 6, timed_steps=2, merge_in_oproj=True)
     assert out["timing"]["distinct_experts_per_layer"] == SMALL.num_experts_per_tok
     assert torch.equal(out["new_tokens"][0], out["new_tokens"][1]) and torch.equal(out["new_tokens"][0], out["new_tokens"][2])
     assert torch.equal(out["new_tokens"][0], together["new_tokens"][0][:6])
@@ -180,7 +184,7 @@ def test_teacher_forced_rows_follow_the_fused_oracle(weights):
     (D.RoutedExperts_UpGate_Rows(0, 8, 8), 15, 2),                                   # part 8 of 8
     (D.RoutedExperts_DownCommit_Rows(0, 0, 3, 8), 16, 3),                            # more than 16 rows
     (D.RoutedExperts_DownCommit_Rows(0, 0, 1, 4), 16, 3),                            # tiles of 8 or 16 rows only
-    (D.OProj_GEMV_Residual(0, 0, 0, 1, 0, tile_N_granularity=8), 4, 5),              # no fan-out to merge
+    (D.OProj_GEMV_Residual(0, 0, 0, 1, 65, tile_N_granularity=8), 4, 5),             # a fan-out beyond what a workgroup merges
 ])
 def test_bad_instructions_are_rejected_on_the_device(weights, bad, opcode, operand):
     """Error paths forced from the host: the kernel refuses the instruction before it writes anything and exits normally."""
@@ -254,7 +258,7 @@ def test_full_layer_geometry_four_rows_equal_the_rows_alone():
     g = rows_kernel.build_rows_globals(w, shape, 300, 4, "cuda:0", max_partials=8)
     _fill_state(g, 4, seed=11)
     g.position_ids.copy_(torch.tensor(positions, dtype=torch.int32))
-    alone = _rows_alone(g, shape, positions, partials=4)
+    alone = _rows_alone(g, shape, positions, partials=4, merge_in_oproj=False)
     rows_kernel.build(g)
     assert int((g.instructions[..., 0] == 2).sum()) == 3 * 4 * 4 * 4        # layers x rows x KV heads x slices
     mk = rows_kernel.get_mk(spin_limit=1 << 20)

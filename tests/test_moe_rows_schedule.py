@@ -15,10 +15,10 @@ from qimeng_megakernel_amd.decode_schedule_moe.model_config import QWEN1_5_MOE_A
 from qimeng_megakernel_amd.instruction import decode_words
 
 
-@pytest.mark.parametrize("rows, queues, partials", [(4, 256, 4), (2, 256, 2), (1, 64, 2), (3, 108, 1)])
-def test_every_piece_of_a_step_is_scheduled_once(rows, queues, partials):
+@pytest.mark.parametrize("rows, queues, partials, merge_in_oproj", [(4, 256, 4, False), (2, 256, 2, True), (1, 64, 2, False), (3, 108, 1, True)])
+def test_every_piece_of_a_step_is_scheduled_once(rows, queues, partials, merge_in_oproj):
     shape = dataclasses.replace(QWEN3_30B_A3B, num_hidden_layers=3)
-    sched = S.MoeRowsScheduler(shape, queues, partials, rows)
+    sched = S.MoeRowsScheduler(shape, queues, partials, rows, merge_in_oproj=merge_in_oproj)
     qs = sched.queues()
     assert len(qs) == queues
     flat = [ins for q in qs for ins in q]
@@ -31,11 +31,12 @@ def test_every_piece_of_a_step_is_scheduled_once(rows, queues, partials):
             assert covered[0][0] == 0 and covered[-1][1] == total
             assert all(a[1] == b[0] for a, b in zip(covered, covered[1:]))
         assert all((i.tile_N_end_idx - i.tile_N_start_idx) * i.tile_N_granularity <= 16 for i in of(16))
-        assert all(i.reduction_block_idx == partials for i in of(4))
+        # who merges the split-KV partials: every O-projection workgroup (its word carries the fan-out), or the last arrival
+        assert all(i.reduction_block_idx == (partials if merge_in_oproj else 0) for i in of(4))
         # one split-KV instruction per (row, KV head, slice), merged by the O-projection workgroups
         assert sorted((i.batch_row, i.kv_head_idx, i.partial_idx) for i in of(2)) == [
             (r, h, p) for r in range(rows) for h in range(shape.num_key_value_heads) for p in range(partials)]
-        assert all(i.merge_in_last == 2 and i.num_partials == partials for i in of(2))
+        assert all(i.merge_in_last == (2 if merge_in_oproj else 1) and i.num_partials == partials for i in of(2))
         # the router's experts once; one report per row
         experts = sorted((i.tile_N_start_idx, i.tile_N_end_idx) for i in of(8))
         assert experts[0][0] == 0 and experts[-1][1] == shape.num_experts and all(a[1] == b[0] for a, b in zip(experts, experts[1:]))
