@@ -169,7 +169,15 @@ def batch_decode(args) -> dict:
     weights = synthetic.random_weights(shape, args.seed, max_positions=kv_capacity)
     prompts = torch.stack([synthetic.random_prompt(shape, args.seed + r, args.prompt_len) for r in range(B)])
     globs = synthetic.build_batch_globals(weights, shape, kv_capacity, B, device)
-    mk = mk_kernel.get_mk()
+    # up to four rows: the batch-1 kernel's row-streaming engine (--batch-engine tiles: the batch kernel's matrix-core tiles)
+    rows_engine = args.batch_engine == "rows" or (args.batch_engine == "auto" and B <= decode_batch.ROWS_ENGINE_MAX_BATCH)
+    if rows_engine:
+        from qimeng_megakernel_amd.decode_schedule_mb import rows_kernel
+
+        mk = rows_kernel.get_mk()
+        kernel = kernel.replace("decode_megakernel_batch<", "decode_megakernel_rows<").replace(">", "Rows>")
+    else:
+        mk = mk_kernel.get_mk()
     if args.copy_calibration:
         copy_calibration(device)
     if args.warmup > 0:
@@ -190,7 +198,7 @@ def batch_decode(args) -> dict:
                         f"tokens per row; timed: the last {timed} decode steps (context {t['first_timed_context']}.."
                         f"{t['last_timed_context']}), seeded random-init bf16 weights",
             "batch": B, "seed": args.seed, "queues": int(globs.instructions.shape[0]),
-            "instructions_per_queue": int(globs.instructions.shape[1]),
+            "instructions_per_queue": int(globs.instructions.shape[1]), "engine": t["engine"],
         },
         "tok_s": t["effective_tok_s_wall"], "tok_s_gpu": t["effective_tok_s_gpu"], "kernel_tok_s": t["kernel_tok_s"],
         "tok_s_gpu_graph": graphed["timing"]["effective_tok_s_gpu"],
@@ -479,6 +487,9 @@ def main() -> None:
                          "(one JSON line, metric attention_phase_GBps)")
     ap.add_argument("--batch", type=int, default=1,
                     help="rows decoded together (2..16: the batch route's kernel, Llama-3.2-1B or Qwen3-1.7B shape; tokens/s counts all rows)")
+    ap.add_argument("--batch-engine", choices=("auto", "rows", "tiles"), default="auto",
+                    help="dense shapes with --batch B: 'rows' = the batch-1 kernel's row-streaming engine with every row's activation "
+                         "vector (1..4 rows), 'tiles' = the batch kernel's matrix-core tiles (2..16), 'auto' = rows up to four rows")
     ap.add_argument("--rows-side-by-side", action="store_true",
                     help="MoE shapes with --batch B: one batch-1 launch per row and step (the only way for a shape with a shared "
                          "expert or more than 4 rows) instead of the B requests in one launch")

@@ -304,6 +304,33 @@ typedef struct QmkBatchArgs {
 int qmk_decode_step_batch(const QmkBatchArgs* args);
 
 /*
+ * One decode step of 1..4 requests ("rows") on the batch-1 kernel's row-streaming engine, for the batch sizes at which
+ * the matrix-core tiles of qmk_decode_step_batch are mostly empty.  Same buffers as qmk_decode_step_batch (`step` is a
+ * QmkBatchArgs: [B, ...] activations, KV cache [L, B, S, Hkv, D], position_ids, active_mask; its three RMSNorm row
+ * buffers, attn_partial_valid, kv_block_size, oproj_blocks and down_blocks are not used, step.flags must be 0), but the
+ * instruction stream is the BATCH-1 route's (…/single_batch/decode_schedule/instructions/instruction_defs.py:39-177):
+ * opcodes 1, 4, 5, 6, 7 act on all rows at once — every weight row is streamed once and multiplied with every row's
+ * activation vector — and opcode 2 names its row in the word behind its batch-1 operands (word 6).  The reference's batch
+ * route (…/multi_batch/decode_kernel/mk.h:9-42) has no counterpart of this stream; a step is the batch-1 route run for
+ * every active row, whose results it reproduces bit for bit.  Hand-over is the tagged one (one set of units per row in
+ * `workspace`, qmk_rows_workspace_bytes(B) bytes, 128-byte aligned, zeroed once); the split-KV partials of a (row, KV
+ * head) are merged by the group's last arrival (merge word 1, O-projection word 5 = 0) or by every O-projection
+ * workgroup (merge word 2, word 5 = fan-out).  A row whose active flag is off is left alone; its logits are set to -1e9.
+ */
+typedef struct QmkRowsArgs {
+  uint32_t struct_size;            /* = sizeof(QmkRowsArgs)                       */
+  int32_t qkv_blocks_per_head;     /* final value of a head's QKV counter = D / rows per QKV tile; 0 = D/16 */
+  void* workspace;
+  uint64_t workspace_bytes;
+  QmkBatchArgs step;               /* step.struct_size = sizeof(QmkBatchArgs); batch_size 1..4 */
+} QmkRowsArgs;
+
+int qmk_decode_step_rows(const QmkRowsArgs* args);
+
+/* Size of QmkRowsArgs.workspace; 0 when batch_size is out of range. */
+uint64_t qmk_rows_workspace_bytes(int batch_size);
+
+/*
  * One decode step of the MoE route at batch 1: opcodes 1-4 and 7 of the dense route (QKV with bias) and
  * 8-14 (…/qwen1_5_moe_a2_7b/A100/single_batch/decode_schedule/instructions/instruction_defs.py:24-151):
  * router logits, softmax top-k, shared expert up/gate and K-split down, routed experts up/gate and down,

@@ -389,6 +389,7 @@ __global__ __launch_bounds__(kThreads, 1) void decode_megakernel_moe_rows(const 
       }
     }
     s.pos[b] = pos;
+    s.live[b] = b < p.batch;
   }
   if (threadIdx.x == 0) {
     s.route_layer = -1;
@@ -483,6 +484,109 @@ __global__ __launch_bounds__(kThreads, 1) void decode_megakernel_moe_rows(const 
   }
 }
 
+// The dense route for 1..4 requests in one launch on the batch-1 row-streaming engine (qmk_rows_ops.h): opcodes 1, 4, 5,
+// 6, 7 of the batch-1 route for all rows at once, 2 as the batch-1 op on a row's view of the buffers.  Buffers in the
+// batch route's layout ([B, ...]; KV cache [L, B, S, Hkv, D]); a row whose active flag is off is a hole: nothing of it is
+// read or written but its logits, which are set to -1e9 as the batch route does.
+template <class M>
+__global__ __launch_bounds__(kThreads, 1) void decode_megakernel_rows(const Params p) {
+  __shared__ rows::Smem<M> s;
+  if (threadIdx.x < 8) s.b.ctl[threadIdx.x] = 0;
+  if (threadIdx.x < rows::kMaxRows) {
+    const int b = threadIdx.x;
+    int pos = 0, on = 0;
+    if (b < p.batch) {
+      pos = p.position_ids != nullptr ? p.position_ids[b] : p.pos_id;
+      on = p.active_mask != nullptr ? (p.active_mask[b] != 0) : 1;
+      if (on && (pos < 0 || pos >= p.kv_row_tokens || pos >= p.rope_rows)) {
+        s.b.ctl[0] = 1;
+        report_error(p, QMK_DEV_BAD_OPERAND, -1, 0, b);
+      }
+      if (pos < 0 || pos >= p.kv_row_tokens || pos >= p.rope_rows) pos = 0;
+    }
+    s.pos[b] = pos;
+    s.live[b] = on;
+  }
+  if (threadIdx.x == 0) {
+    s.route_layer = -1;
+    s.n_list = 0;
+    s.b.generation = ld_shared32(p.ws + kWsGeneration);
+    s.b.best_val = -INFINITY;
+    s.b.best_idx = 0x7fffffff;
+  }
+  __syncthreads();
+  bool ok = s.b.ctl[0] == 0;
+  const int32_t* queue = p.instructions + static_cast<size_t>(blockIdx.x) * p.num_insts * kInstWords;
+  int32_t word = (threadIdx.x < kInstWords && p.num_insts > 0) ? queue[threadIdx.x] : 0;
+  int32_t word1 = (threadIdx.x < kInstWords && p.num_insts > 1) ? queue[kInstWords + threadIdx.x] : 0;
+  const int num_insts = p.num_insts;
+  for (int i = 0; i < num_insts && ok; ++i) {
+    if (threadIdx.x < kInstWords) {
+      s.b.inst[threadIdx.x] = word;
+      s.b.next[threadIdx.x] = word1;
+      word = word1;
+      word1 = (i + 2 < num_insts) ? queue[(i + 2) * kInstWords + threadIdx.x] : 0;
+    }
+    __syncthreads();
+    const int opcode = s.b.inst[0];
+    int tid = threadIdx.x;
+    asm volatile("" : "+v"(tid));
+    const Ctx c{i, opcode, tid};
+    unsigned long long t_start = 0;
+    if (p.timeline != nullptr && threadIdx.x == 0) {
+      t_start = wall_clock64();
+      for (int k = 0; k < 4; ++k) s.b.stamps[k] = t_start;
+    }
+    switch (opcode) {
+      case OP_NOOP: break;
+      case OP_RMS_QKV_ROPE: [[clang::always_inline]] ok = rows::op_qkv<M>(p, s, c); break;
+      case OP_ATTN_SPLITKV: {
+        const int row = s.b.inst[6];   // the word behind the batch-1 operands
+        if (row < 0 || row >= p.batch) {
+          ok = rows::bad_operand(p, s, c, 6);
+        } else if (s.live[row]) {
+          const Params pr = rows::row_view<M>(p, row, s.pos[row]);
+          [[clang::always_inline]] ok = op_attn_splitkv<M>(pr, s.b, c);
+        }
+        break;
+      }
+      case OP_OPROJ_RESIDUAL: [[clang::always_inline]] ok = rows::op_oproj<M>(p, s, c); break;
+      case OP_RMS_UPGATE_SILU: [[clang::always_inline]] ok = rows::op_upgate<M>(p, s, c); break;
+      case OP_DOWN_RESIDUAL: [[clang::always_inline]] ok = rows::op_down<M>(p, s, c); break;
+      case OP_RMS_LMHEAD: [[clang::always_inline]] ok = rows::op_lmhead<M>(p, s, c); break;
+      default:
+        if (threadIdx.x == 0) report_error(p, QMK_DEV_BAD_OPCODE, i, opcode, 0);
+        ok = false;
+        break;
+    }
+    if (p.timeline != nullptr && threadIdx.x == 0) {
+      uint64_t* rec = p.timeline + (static_cast<size_t>(blockIdx.x) * p.num_insts + i) * 8;
+      rec[0] = t_start;
+      rec[1] = s.b.ctl[2] ? s.b.t_wait : t_start;
+      rec[2] = wall_clock64();
+      rec[3] = static_cast<uint64_t>(opcode) | (static_cast<uint64_t>(static_cast<uint32_t>(s.b.inst[1])) << 8);
+      for (int k = 0; k < 4; ++k) rec[4 + k] = s.b.stamps[k];
+      s.b.ctl[2] = 0;
+    }
+    __syncthreads();
+  }
+  if (!ok) return;
+  release_stores();
+  __syncthreads();
+  int32_t* done = counter_ptr(p, 0, p.num_layer_barriers - 1, p.barrier_slots - 1);
+  if (threadIdx.x == 0) {
+    const int prev = __hip_atomic_fetch_add(done, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    s.b.ctl[1] = (prev == static_cast<int>(gridDim.x) - 1);
+  }
+  __syncthreads();
+  if (s.b.ctl[1]) {
+    const int total = p.num_layers * p.num_layer_barriers * p.barrier_slots;
+    for (int i = threadIdx.x; i < total; i += kThreads)
+      __hip_atomic_store(p.barriers + i, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    if (threadIdx.x == 0) st_shared32(p.ws + kWsGeneration, (s.b.generation + 1u) & 0x03ffffffu);
+  }
+}
+
 static_assert(std::is_same<decltype(&decode_megakernel<Llama1B>), void (*)(const Params)>::value &&
                   std::is_same<decltype(&decode_megakernel<Qwen3_1p7B>), void (*)(const Params)>::value &&
                   std::is_same<decltype(&decode_megakernel_moe<QwenMoeA2_7B>), void (*)(const Params)>::value &&
@@ -497,6 +601,7 @@ struct DeviceInfo {
   int max_queues_batch_qwen3 = 0;
   int max_queues_moe = 0;
   int max_queues_moe_rows = 0;
+  int max_queues_rows = 0;
   int32_t* status = nullptr;
   uint64_t* scratch = nullptr;   // this device's copy of the file-scope `scratch` array
   bool static_in_use = false;    // a launch since the last status fetch used that array as its workspace
@@ -542,6 +647,11 @@ int device_info(DeviceInfo** out) {
     d.max_queues_batch_qwen3 = per_cu_batch3 * prop.multiProcessorCount;
     d.max_queues_moe = per_cu_moe * prop.multiProcessorCount;
     d.max_queues_moe_rows = per_cu_rows * prop.multiProcessorCount;
+    int per_cu_dense_rows = 0, per_cu_dense_rows3 = 0;
+    if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu_dense_rows, decode_megakernel_rows<rows::Llama1BRows>, kThreads, 0) != hipSuccess ||
+        hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu_dense_rows3, decode_megakernel_rows<rows::Qwen3_1p7BRows>, kThreads, 0) != hipSuccess)
+      return QMK_ERR_NO_DEVICE;
+    d.max_queues_rows = (per_cu_dense_rows3 < per_cu_dense_rows ? per_cu_dense_rows3 : per_cu_dense_rows) * prop.multiProcessorCount;
     d.status = static_cast<int32_t*>(sym);
     d.scratch = static_cast<uint64_t*>(scratch_ptr);
     d.ready = true;
@@ -959,6 +1069,8 @@ int decode_step_moe_rows(const QmkMoeRowsArgs* r) {
   p.position_ids = r->position_ids;
   p.distinct_out = r->distinct_experts;
   p.rope_rows = a->rope_rows;
+  p.kv_row_tokens = a->num_layers * a->max_seq_len;   // caches [B, L, 1, S, Hkv, D]
+  p.kv_layer_tokens = a->max_seq_len;
   p.pos_id = 0;
   hipLaunchKernelGGL(decode_megakernel_moe_rows<M>, dim3(a->num_queues), dim3(kThreads), 0, static_cast<hipStream_t>(a->stream), p);
   return hipGetLastError() == hipSuccess ? QMK_OK : QMK_ERR_LAUNCH;
@@ -974,6 +1086,100 @@ extern "C" int qmk_decode_step_moe(const QmkMoeArgs* a) {
     case QMK_MODEL_QWEN3_30B_A3B: return decode_step_moe<Qwen3MoeA3B>(a);
     default: return QMK_ERR_MODEL;
   }
+}
+
+// Units from one row's tagged workspace to the next in a dense launch of several rows.
+constexpr int kWsDenseRowUnits = ((kWsUnits + 15) / 16) * 16;
+
+extern "C" uint64_t qmk_rows_workspace_bytes(int batch_size) {
+  if (batch_size < 1 || batch_size > rows::kMaxRows) return 0;
+  return static_cast<uint64_t>(batch_size) * kWsDenseRowUnits * sizeof(uint64_t);
+}
+
+template <class M>
+static int decode_step_rows(const QmkRowsArgs* r) {
+  const QmkBatchArgs* a = &r->step;
+  const int B = a->batch_size;
+  if (B < 1 || B > rows::kMaxRows) return QMK_ERR_SHAPE;
+  const void* required[] = {a->instructions, a->hidden_states, a->q_post_rope, a->k_cache, a->v_cache, a->attn_out,
+                            a->attn_lse_intermediates, a->attn_out_intermediates, a->silu_out, a->logits,
+                            a->attn_norm_weights, a->qkv_weights, a->rope_cos, a->rope_sin, a->o_proj_weights,
+                            a->mlp_norm_weights, a->up_proj_weights, a->gate_proj_weights, a->down_proj_weights,
+                            a->lm_head_norm_weights, a->lm_head_weights, a->barriers, r->workspace};
+  for (const void* ptr : required)
+    if (ptr == nullptr) return QMK_ERR_NULL_ARG;
+  if (M::QK_NORM && (a->qkv_raw == nullptr || a->q_norm_weights == nullptr || a->k_norm_weights == nullptr)) return QMK_ERR_NULL_ARG;
+  if (a->num_queues < 1 || a->num_insts < 0 || a->num_layers < 1 || a->num_layers > 63 || a->num_layer_barriers < 8 ||
+      a->barrier_slots < B * M::NQ || a->max_seq_len < 1 || a->max_splits < 1 || a->vocab_size < 1 || a->rope_rows < 1)
+    return QMK_ERR_SHAPE;
+  if (a->flags != 0) return QMK_ERR_SHAPE;   // tagged hand-over and self-clearing counters always
+  if (a->position_ids == nullptr && (a->pos_id < 0 || a->pos_id >= a->max_seq_len || a->pos_id >= a->rope_rows)) return QMK_ERR_POSITION;
+  if (reinterpret_cast<uintptr_t>(r->workspace) % 128 != 0 || r->workspace_bytes < qmk_rows_workspace_bytes(B)) return QMK_ERR_SHAPE;
+
+  DeviceInfo* dev = nullptr;
+  if (int rc = device_info(&dev); rc != QMK_OK) return rc;
+  if (a->num_queues > dev->max_queues_rows) return QMK_ERR_TOO_MANY_QUEUES;
+  if (a->num_insts == 0) return QMK_OK;
+
+  Params p{};
+  p.instructions = a->instructions;
+  p.hidden = static_cast<u16*>(a->hidden_states);
+  p.q_post_rope = static_cast<u16*>(a->q_post_rope);
+  p.k_cache = static_cast<u16*>(a->k_cache);
+  p.v_cache = static_cast<u16*>(a->v_cache);
+  p.attn_out = static_cast<u16*>(a->attn_out);
+  p.attn_lse = a->attn_lse_intermediates;
+  p.attn_partial = a->attn_out_intermediates;
+  p.silu_out = static_cast<u16*>(a->silu_out);
+  p.logits = static_cast<u16*>(a->logits);
+  p.attn_norm = static_cast<const u16*>(a->attn_norm_weights);
+  p.qkv_w = static_cast<const u16*>(a->qkv_weights);
+  p.qkv_raw = static_cast<u16*>(a->qkv_raw);
+  p.q_norm = static_cast<const u16*>(a->q_norm_weights);
+  p.k_norm = static_cast<const u16*>(a->k_norm_weights);
+  p.rope_cos = a->rope_cos;
+  p.rope_sin = a->rope_sin;
+  p.o_w = static_cast<const u16*>(a->o_proj_weights);
+  p.mlp_norm = static_cast<const u16*>(a->mlp_norm_weights);
+  p.up_w = static_cast<const u16*>(a->up_proj_weights);
+  p.gate_w = static_cast<const u16*>(a->gate_proj_weights);
+  p.down_w = static_cast<const u16*>(a->down_proj_weights);
+  p.lm_norm = static_cast<const u16*>(a->lm_head_norm_weights);
+  p.lm_w = static_cast<const u16*>(a->lm_head_weights);
+  p.barriers = a->barriers;
+  p.ws = static_cast<uint64_t*>(r->workspace);
+  p.ws_row_units = kWsDenseRowUnits;
+  p.timeline = a->timeline;
+  p.status = dev->status;
+  p.num_insts = a->num_insts;
+  p.num_layers = a->num_layers;
+  p.num_layer_barriers = a->num_layer_barriers;
+  p.barrier_slots = a->barrier_slots;
+  p.max_seq_len = a->max_seq_len;
+  p.max_splits = a->max_splits;
+  p.vocab_size = a->vocab_size;
+  p.pos_id = a->pos_id;
+  p.attn_scale = a->attn_scale;
+  p.rms_norm_eps = a->rms_norm_eps;
+  p.qkv_blocks_per_head = r->qkv_blocks_per_head > 0 ? r->qkv_blocks_per_head : M::D / 16;
+  p.spin_limit = a->spin_limit > 0 ? a->spin_limit : kDefaultSpinLimit;
+  p.flags = QMK_FLAG_TAGGED;
+  p.batch = B;
+  p.position_ids = a->position_ids;
+  p.active_mask = a->active_mask;
+  p.rope_rows = a->rope_rows;
+  p.kv_row_tokens = a->max_seq_len;            // caches [L, B, S, Hkv, D]
+  p.kv_layer_tokens = B * a->max_seq_len;
+  hipLaunchKernelGGL(decode_megakernel_rows<M>, dim3(a->num_queues), dim3(kThreads), 0, static_cast<hipStream_t>(a->stream), p);
+  return hipGetLastError() == hipSuccess ? QMK_OK : QMK_ERR_LAUNCH;
+}
+
+extern "C" int qmk_decode_step_rows(const QmkRowsArgs* r) {
+  if (r == nullptr) return QMK_ERR_NULL_ARG;
+  if (r->struct_size != sizeof(QmkRowsArgs) || r->step.struct_size != sizeof(QmkBatchArgs)) return QMK_ERR_ABI;
+  if (r->step.model == QMK_MODEL_LLAMA_3_2_1B) return decode_step_rows<rows::Llama1BRows>(r);
+  if (r->step.model == QMK_MODEL_QWEN3_1_7B) return decode_step_rows<rows::Qwen3_1p7BRows>(r);
+  return QMK_ERR_MODEL;
 }
 
 extern "C" uint64_t qmk_moe_rows_workspace_bytes(int batch_size) {

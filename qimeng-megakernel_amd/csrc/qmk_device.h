@@ -123,6 +123,8 @@ struct Params {
   // MoE route, several requests in one launch (qmk_rows_ops.h): every per-request buffer above is [batch, ...].
   int32_t ws_row_units;          // 8-byte units from one row's tagged workspace to the next
   int32_t* distinct_out;         // [L] or null: distinct experts each layer streamed in this launch
+  int32_t kv_row_tokens;         // KV-cache tokens from one row's cache to the next ([B, L, 1, S, ..]: L*S; [L, B, S, ..]: S)
+  int32_t kv_layer_tokens;       // ... from one layer to the next within a row's cache (S, or B*S)
 };
 
 // ---------------------------------------------------------------- bf16 ----

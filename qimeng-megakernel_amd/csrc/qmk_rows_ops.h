@@ -35,12 +35,36 @@ enum Opcode {
   OP_ROUTED_DOWN_COMMIT_ROWS = 16,
 };
 
+// Width of a row's activation vector in LDS: the widest vector an op of the route stages (the attention output; for the
+// dense models, whose geometries say so with DENSE_ROWS, the MLP's intermediate vector).
+template <class M, class = void>
+struct XWidth {
+  static constexpr int value = M::AW > M::H ? M::AW : M::H;
+};
+template <class M>
+struct XWidth<M, std::enable_if_t<M::DENSE_ROWS>> {
+  static constexpr int value = M::F;
+};
+
+// The dense geometries as the rows kernel uses them: nothing carried or parked between instructions.
+struct Llama1BRows : Llama1B {
+  static constexpr int CARRY_ROWS = 0;
+  static constexpr int PARK_ROWS = 0;
+  static constexpr bool DENSE_ROWS = true;
+};
+struct Qwen3_1p7BRows : Qwen3_1p7B {
+  static constexpr int CARRY_ROWS = 0;
+  static constexpr int PARK_ROWS = 0;
+  static constexpr bool DENSE_ROWS = true;
+};
+
 template <class M>
 struct Smem {
   qmk::Smem<M> b;                       // what the batch-1 ops use when they run on a row's view (attention, top-k report)
   int32_t pos[kMaxRows];                // position each row decodes
+  int32_t live[kMaxRows];               // the row exists and is active: a row that is not is a hole every op steps over
   float red[2][kMaxRows][kWaves];
-  alignas(16) u16 x[kMaxRows][M::AW > M::H ? M::AW : M::H];   // the rows' activation vectors
+  alignas(16) u16 x[kMaxRows][XWidth<M>::value];   // the rows' activation vectors
   float res[kMaxRows][kRowRes];
   // the routing decision this workgroup last took (layer, -1: none yet), per row and slot, and the distinct experts
   int32_t route_layer;
@@ -76,8 +100,9 @@ template <class M>
 __device__ __forceinline__ Params row_view(const Params& p, int r, int pos) {
   Params q = p;
   const size_t R = static_cast<size_t>(r);
-  const size_t cache = static_cast<size_t>(p.num_layers) * p.max_seq_len * M::NKV * M::D;
+  const size_t cache = static_cast<size_t>(p.kv_row_tokens) * M::NKV * M::D;
   q.pos_id = pos;
+  q.max_seq_len = p.kv_layer_tokens;   // (the batch-1 ops use it for nothing but the distance between two layers' rows)
   q.hidden = p.hidden + R * M::H;
   q.q_post_rope = p.q_post_rope + R * M::AW;
   q.attn_out = p.attn_out + R * M::AW;
@@ -85,7 +110,7 @@ __device__ __forceinline__ Params row_view(const Params& p, int r, int pos) {
   q.v_cache = p.v_cache + R * cache;
   q.attn_lse = p.attn_lse + R * M::NQ * p.max_splits;
   q.attn_partial = p.attn_partial + R * M::NQ * p.max_splits * M::D;
-  q.silu_out = p.silu_out + R * p.moe_ffn;
+  q.silu_out = p.silu_out + R * (p.moe_ffn > 0 ? p.moe_ffn : M::F);
   q.logits = p.logits + R * p.vocab_size;
   q.qkv_raw = p.qkv_raw != nullptr ? p.qkv_raw + R * M::QKV : nullptr;
   q.router_logits = p.router_logits + R * p.num_experts;
@@ -118,7 +143,7 @@ __device__ __forceinline__ bool rms_rows(const Params& p, Smem<M>& s, const Ctx&
     uint64_t xx[kMaxRows], yy[kMaxRows];
     static_for<0, kMaxRows>([&](auto b) {
       xx[b] = yy[b] = static_cast<uint64_t>(tag) << 32;
-      if (b < B) {
+      if (s.live[b]) {
         const uint64_t* mine = ws_of(p, b) + region + 2 * t;
         xx[b] = ld_shared64(mine);
         yy[b] = ld_shared64(mine + 1);
@@ -138,7 +163,7 @@ __device__ __forceinline__ bool rms_rows(const Params& p, Smem<M>& s, const Ctx&
   });
   if (region < 0) {
     static_for<0, kMaxRows>([&](auto b) {
-      if (b < B) {
+      if (s.live[b]) {
         const uint64_t hw = ld_shared64(p.hidden + static_cast<size_t>(b) * M::H + t * 4);
         lo[b] = static_cast<uint32_t>(hw);
         hi[b] = static_cast<uint32_t>(hw >> 32);
@@ -228,9 +253,9 @@ __device__ bool op_qkv(const Params& p, Smem<M>& s, const Ctx& c) {
   __syncthreads();
   // Epilogue per (row, output pair): the GEMV result is bf16 before anything else happens to it.
   const int pairs = nrows / 2;
-  const size_t cache = static_cast<size_t>(p.num_layers) * p.max_seq_len * M::NKV * M::D;
   for (int item = c.tid; item < B * pairs; item += kThreads) {
     const int b = item / pairs, pair = item % pairs;
+    if (!s.live[b]) continue;
     const int r = rs + 2 * pair;
     float a0 = s.res[b][2 * pair], a1 = s.res[b][2 * pair + 1];
     if constexpr (M::QKV_BIAS) {
@@ -248,7 +273,7 @@ __device__ bool op_qkv(const Params& p, Smem<M>& s, const Ctx& c) {
       const int pos = s.pos[b];
       const float* cosr = p.rope_cos + static_cast<size_t>(pos) * M::D;
       const float* sinr = p.rope_sin + static_cast<size_t>(pos) * M::D;
-      const size_t kv_row = static_cast<size_t>(b) * cache + (static_cast<size_t>(layer) * p.max_seq_len + pos) * (M::NKV * M::D);
+      const size_t kv_row = (static_cast<size_t>(b) * p.kv_row_tokens + static_cast<size_t>(layer) * p.kv_layer_tokens + pos) * (M::NKV * M::D);
       if (r < kq) {
         const uint32_t w = rope_pair(v0, v1, cosr, sinr, r % M::D);
         st_shared32(p.q_post_rope + static_cast<size_t>(b) * M::AW + r, w);
@@ -267,6 +292,21 @@ __device__ bool op_qkv(const Params& p, Smem<M>& s, const Ctx& c) {
     }
   }
   return true;   // the units announce themselves
+}
+
+// Every live row's word on the reduction row has reached `expected` (lane r polls row r's).  False (uniformly) on a timeout.
+template <class M>
+__device__ __forceinline__ bool wait_rows(const Params& p, Smem<M>& s, const Ctx& c, int layer, int expected) {
+  if (c.tid < p.batch && s.live[c.tid] && !poll_counter(counter_ptr(p, layer, ROW_REDUCE, c.tid * M::NQ), expected, p.spin_limit)) {
+    s.b.ctl[0] = 1;
+    report_error(p, QMK_DEV_WAIT_TIMEOUT, c.inst_idx, c.opcode, c.tid);
+  }
+  if (p.timeline != nullptr && c.tid == 0) {
+    s.b.t_wait = wall_clock64();
+    s.b.ctl[2] = 1;
+  }
+  __syncthreads();
+  return s.b.ctl[0] == 0;
 }
 
 // ===================================================================== 4 ==
@@ -293,7 +333,7 @@ __device__ bool op_oproj(const Params& p, Smem<M>& s, const Ctx& c) {
   const uint32_t tag = tag_of(s.b.generation, layer);
   // the residual values this thread adds to: those the previous layer's commit announced (layer 0: the caller's buffer)
   const int my_b = c.tid / max(pairs, 1), my_pair = c.tid % max(pairs, 1);
-  const bool adds = c.tid < B * pairs;
+  const bool adds = c.tid < B * pairs && s.live[my_b];
   uint32_t res_old = 0;
   if (adds) {
     if (layer == 0) {
@@ -306,7 +346,7 @@ __device__ bool op_oproj(const Params& p, Smem<M>& s, const Ctx& c) {
   if (P == 0) {
     // The rows' attention outputs are complete in memory: the last split-KV arrival of every (row, KV head) merged its
     // group's partials and counted the group's heads on the row's word of the reduction row.  All rows in one trip.
-    if (!wg_wait(p, s.b, c, B, [&](int i) { return counter_ptr(p, layer, ROW_REDUCE, i * M::NQ); }, M::NQ)) return false;
+    if (!wait_rows(p, s, c, layer, M::NQ)) return false;
     constexpr int kPieces = kMaxRows * AW / (kThreads * 8);   // 16-byte pieces per thread
     v4u piece[kPieces];
 #pragma unroll
@@ -322,7 +362,7 @@ __device__ bool op_oproj(const Params& p, Smem<M>& s, const Ctx& c) {
     }
   } else {
   // one arrival per split-KV instruction, on its row's word of the reduction row
-  if (!wg_wait(p, s.b, c, B, [&](int i) { return counter_ptr(p, layer, ROW_REDUCE, i * M::NQ); }, M::NKV * P)) return false;
+  if (!wait_rows(p, s, c, layer, M::NKV * P)) return false;
   // Item t (one or two per thread) is dims 4*(t % (D/4)).. of head t / (D/4); four partials of every item per round,
   // all loads first — the batch-1 op's arithmetic, one row of the batch after the other.
   constexpr int kItems = AW / (kThreads * 4);
@@ -759,6 +799,163 @@ __device__ bool op_routed_down_commit(const Params& p, Smem<M>& s, const Ctx& c)
   return true;
 }
 
+// ===================================================================== 5 ==
+// [5, layer, tile_M, n, block_0..block_{n-1}, tile_M_g, tile_N_g]   dense MLP, every row of the batch:
+// silu_out[b] = bf16(bf16(silu(bf16(W_g y_b))) * bf16(W_u y_b))  (operations.py:265-282; the batch-1 op's arithmetic per row)
+template <class M>
+__device__ bool op_upgate(const Params& p, Smem<M>& s, const Ctx& c) {
+  constexpr int CH = M::H / 512;
+  const int bad = upgate_check<M>(p, s.b.inst);
+  if (bad >= 0) return bad_operand(p, s, c, bad);
+  const int layer = s.b.inst[1], n = s.b.inst[3], B = p.batch;
+  const int tile = s.b.inst[5 + n];
+  const int lane = c.tid & 63;
+  const int nout = n * tile, nrows = 2 * nout;     // streamed rows: element 2i = up row i, 2i+1 = gate row i
+  if (nrows > kRowRes) return bad_operand(p, s, c, 3);
+  auto row_of = [&](int i) { return s.b.inst[4 + i / tile] * tile + i % tile; };
+  auto src = [&](int e) { return upgate_row<M>(p, s.b.inst, layer, tile, e); };
+  RowRegs<CH> buf[kUpGateBuffers];
+  const uint32_t tag = tag_of(s.b.generation, layer);
+  if (!rms_rows<M, kUpGateBuffers>(p, s, c, kWsHiddenMid, tag, p.mlp_norm + static_cast<size_t>(layer) * M::H,
+                                   [&](auto k) { preload_range<decltype(k)::value, decltype(k)::value + 1>(nrows, src, buf); }))
+    return false;
+  QMK_ROWS_STAMP(0);
+  v4u x[kMaxRows][CH];
+  load_x_rows<M, CH>(s, x, lane);
+  stream<CH>(nrows, src, buf, [&](int e, const RowRegs<CH>& w) {
+    float sum[kMaxRows];
+    static_for<0, kMaxRows>([&](auto b) { sum[b] = wave_sum(dot_row(w, x[b])); });
+    if (lane == 0) static_for<0, kMaxRows>([&](auto b) { s.res[b][e] = sum[b]; });
+  });
+  QMK_ROWS_STAMP(1);
+  __syncthreads();
+  const int pairs = nout / 2;
+  for (int item = c.tid; item < B * pairs; item += kThreads) {
+    const int b = item / pairs, pair = item % pairs;
+    uint32_t word = 0;
+    if (s.live[b]) {
+#pragma unroll
+      for (int k = 0; k < 2; ++k) {
+        const int i = 2 * pair + k;
+        const float up = round_bf16(s.res[b][2 * i]), gate = round_bf16(s.res[b][2 * i + 1]);
+        const float act = round_bf16(gate / (1.0f + expf(-gate)));
+        word |= static_cast<uint32_t>(f2bf(act * up)) << (16 * k);
+      }
+      st_tagged(ws_of(p, b) + kWsSilu + row_of(2 * pair) / 2, word, tag);
+    }
+    st_shared32(p.silu_out + static_cast<size_t>(b) * M::F + row_of(2 * pair), word);   // zeros for a row that is not decoded
+  }
+  return true;
+}
+
+// ===================================================================== 6 ==
+// [6, layer, tile_M, n_start, n_end, split_K_idx, tile_M_g, tile_N_g, split_K_g]   one K slice over the whole F only:
+// hidden[b][r] = bf16(hidden[b][r] + bf16(W_d[r] . silu_out[b])) for every row of the batch  (operations.py:285-295)
+template <class M>
+__device__ bool op_down(const Params& p, Smem<M>& s, const Ctx& c) {
+  constexpr int CH = 4;
+  static_assert(M::F % (4 * kThreads) == 0 && M::F <= XWidth<M>::value, "whole unit pairs per thread; the vectors fit");
+  const int layer = s.b.inst[1], nstart = s.b.inst[3], nend = s.b.inst[4], split = s.b.inst[5];
+  const int tile = s.b.inst[7], kg = s.b.inst[8], B = p.batch;
+  if (layer < 0 || layer >= p.num_layers) return bad_operand(p, s, c, 1);
+  if (tile <= 0 || (tile & 1)) return bad_operand(p, s, c, 7);
+  if (nstart < 0 || nend < nstart || static_cast<long>(nend) * tile > M::H) return bad_operand(p, s, c, 4);
+  if ((nend - nstart) * tile > kRowRes || B * (nend - nstart) * tile / 2 > kThreads) return bad_operand(p, s, c, 3);
+  if (split != 0 || kg != M::F) return bad_operand(p, s, c, 8);
+  const int lane = c.tid & 63, wave = c.tid >> 6;
+  const int rs = nstart * tile, nrows = (nend - nstart) * tile, pairs = nrows / 2;
+  constexpr int segs = M::F / (512 * CH);
+  auto row_of = [&](int e) { return (e & (kWaves - 1)) + kWaves * ((e >> 3) / segs); };
+  auto seg_of = [&](int e) { return (e >> 3) % segs; };
+  const u16* W = p.down_w + (static_cast<size_t>(layer) * M::H + rs) * M::F;
+  auto src = [&](int e) { return W + static_cast<size_t>(row_of(e)) * M::F + seg_of(e) * (512 * CH); };
+  const int rows_w = (nrows - wave + kWaves - 1) / kWaves;
+  const int n_elems = rows_w > 0 ? wave + kWaves * (rows_w * segs - 1) + 1 : 0;
+  RowRegs<CH> buf[kDepth];
+  preload_range<0, kEarly>(n_elems, src, buf);
+  const uint32_t tag = tag_of(s.b.generation, layer);
+  const int my_b = c.tid / max(pairs, 1), my_pair = c.tid % max(pairs, 1);
+  const bool adds = c.tid < B * pairs && s.live[my_b];
+  uint32_t res_old = 0;
+  if (adds && !poll_tagged1(ws_of(p, my_b) + kWsHiddenMid + (rs + 2 * my_pair) / 2, tag, p.spin_limit, res_old)) {
+    s.b.ctl[0] = 1;
+    report_error(p, QMK_DEV_WAIT_TIMEOUT, c.inst_idx, c.opcode, c.tid);
+  }
+  // silu_out of every live row from its tagged units: thread t looks at the unit pairs 2t + 1024k of every row until
+  // they carry this layer's tag; what has been staged is not fetched again.
+  {
+    constexpr int kPairs = M::F / (4 * kThreads);
+    bool have[kMaxRows][kPairs];
+    static_for<0, kMaxRows>([&](auto b) {
+#pragma unroll
+      for (int k = 0; k < kPairs; ++k) have[b][k] = !s.live[b];
+    });
+    for (uint32_t polls = 0;; ++polls) {
+      bool all = true;
+      static_for<0, kMaxRows>([&](auto b) {
+        if (s.live[b]) {
+          const uint64_t* mine = ws_of(p, b) + kWsSilu + 2 * c.tid;
+          uint32_t* words = reinterpret_cast<uint32_t*>(&s.x[b][0]);
+          uint64_t u[2 * kPairs];
+#pragma unroll
+          for (int k = 0; k < kPairs; ++k)
+            if (!have[b][k]) {
+              u[2 * k] = ld_shared64(mine + 1024 * k);
+              u[2 * k + 1] = ld_shared64(mine + 1024 * k + 1);
+            }
+#pragma unroll
+          for (int k = 0; k < kPairs; ++k) {
+            if (!have[b][k] && static_cast<uint32_t>(u[2 * k] >> 32) == tag && static_cast<uint32_t>(u[2 * k + 1] >> 32) == tag) {
+              words[2 * c.tid + 1024 * k] = static_cast<uint32_t>(u[2 * k]);
+              words[2 * c.tid + 1024 * k + 1] = static_cast<uint32_t>(u[2 * k + 1]);
+              have[b][k] = true;
+            }
+            all = all && have[b][k];
+          }
+        }
+      });
+      if (all) break;
+      if (polls > p.spin_limit) {
+        s.b.ctl[0] = 1;
+        report_error(p, QMK_DEV_WAIT_TIMEOUT, c.inst_idx, c.opcode, c.tid);
+        break;
+      }
+      __builtin_amdgcn_s_sleep(8);
+    }
+  }
+  preload_range<kEarly, kDepth>(n_elems, src, buf);
+  if (p.timeline != nullptr && c.tid == 0) {
+    s.b.t_wait = wall_clock64();
+    s.b.ctl[2] = 1;
+  }
+  __syncthreads();
+  if (s.b.ctl[0]) return false;
+  float acc[kMaxRows];
+  static_for<0, kMaxRows>([&](auto b) { acc[b] = 0.f; });
+  stream<CH>(n_elems, src, buf, [&](int e, const RowRegs<CH>& w) {
+    const int seg = seg_of(e);
+    static_for<0, kMaxRows>([&](auto b) {
+#pragma unroll
+      for (int j = 0; j < CH; ++j) acc[b] = dot8(w.v[j], *reinterpret_cast<const v4u*>(&s.x[b][seg * (512 * CH) + (j * kWaveSize + lane) * 8]), acc[b]);
+    });
+    if (seg == segs - 1) {
+      static_for<0, kMaxRows>([&](auto b) {
+        const float sum = wave_sum(acc[b]);
+        acc[b] = 0.f;
+        if (lane == 0) s.res[b][row_of(e)] = sum;
+      });
+    }
+  });
+  QMK_ROWS_STAMP(1);
+  __syncthreads();
+  if (adds) {
+    const uint32_t w = residual_word(res_old, s.res[my_b][2 * my_pair], s.res[my_b][2 * my_pair + 1]);
+    st_tagged(ws_of(p, my_b) + kWsHiddenOut + (rs + 2 * my_pair) / 2, w, tag);
+    st_shared32(p.hidden + static_cast<size_t>(my_b) * M::H + rs + 2 * my_pair, w);
+  }
+  return true;
+}
+
 // ===================================================================== 7 ==
 // [7, start_block, end_block, tile_M_g, tile_N_g]     logits[b] = bf16(W_lm . rms(hidden[b])) for every row
 template <class M>
@@ -783,7 +980,7 @@ __device__ bool op_lmhead(const Params& p, Smem<M>& s, const Ctx& c) {
     float sum[kMaxRows];
     static_for<0, kMaxRows>([&](auto b) { sum[b] = wave_sum(dot_row(w, x[b])); });
     static_for<0, kMaxRows>([&](auto b) {
-      if (lane == b && b < B) p.logits[static_cast<size_t>(b) * p.vocab_size + rs + r] = f2bf(sum[b]);
+      if (lane == b && b < B) p.logits[static_cast<size_t>(b) * p.vocab_size + rs + r] = f2bf(s.live[b] ? sum[b] : -1e9f);   // (a row that is not decoded: as the batch route leaves it)
     });
   });
   return true;

@@ -17,6 +17,24 @@ import torch
 
 from .decode_schedule_mb.row_state import RowState, rows_of
 from .decode_schedule_mb import mk_kernel as _mk_kernel
+from .decode_schedule_mb import rows_kernel as _rows_kernel
+
+#: up to this many rows the batch-1 kernel's row-streaming engine decodes a batch faster than the matrix-core tiles
+ROWS_ENGINE_MAX_BATCH = _rows_kernel.MAX_ROWS
+
+
+def _route(mk: Any, rows: int, engine: str):
+    """(launcher module, mk) for ``engine``: "rows" (1..4 rows on the row-streaming engine), "tiles" (the batch kernel's
+    matrix-core tiles), or "auto": what ``mk`` was made for, else rows up to four rows and tiles beyond."""
+    if engine not in ("auto", "rows", "tiles"):
+        raise ValueError("engine must be 'auto', 'rows' or 'tiles'")
+    if engine == "auto":
+        if mk is not None:
+            engine = "rows" if isinstance(mk, _rows_kernel.RowsMegaKernel) else "tiles"
+        else:
+            engine = "rows" if rows <= ROWS_ENGINE_MAX_BATCH else "tiles"
+    module = _rows_kernel if engine == "rows" else _mk_kernel
+    return module, (mk or module.get_mk())
 
 
 def step_bytes(shape: Any, contexts: Sequence[int]) -> int:
@@ -34,10 +52,11 @@ def prefill_by_decode(globs: Any, mk: Any, prompts: torch.Tensor) -> torch.Tenso
     """``prompts`` [B, T]: fill the KV cache one position at a time; returns the first new token of every row."""
     B, T = prompts.shape
     prompts = prompts.to(globs.hidden_states.device)
+    launcher = _rows_kernel if isinstance(mk, _rows_kernel.RowsMegaKernel) else _mk_kernel
     for pos in range(T):
         _embed(globs, prompts[:, pos])
         globs.position_ids.fill_(pos)
-        _mk_kernel.call_mk(globs, mk)
+        launcher.call_mk(globs, mk)
     return globs.logits.argmax(dim=-1)
 
 
@@ -57,7 +76,7 @@ def argmax_rows(logits: torch.Tensor) -> torch.Tensor:
 
 
 def decode(globs: Any, prompts: torch.Tensor, max_new_tokens: int, *, mk: Any = None, eos_token_ids: Sequence[int] = (),
-           decode_time: bool = True, use_graph: bool = False, timed_steps: int | None = None) -> dict[str, Any]:
+           decode_time: bool = True, use_graph: bool = False, timed_steps: int | None = None, engine: str = "auto") -> dict[str, Any]:
     """Prefill + greedy decode of B rows to ``max_new_tokens`` tokens each (rows that hit an EOS token
     of ``eos_token_ids`` retire; with none given every row runs to the end).
 
@@ -66,7 +85,11 @@ def decode(globs: Any, prompts: torch.Tensor, max_new_tokens: int, *, mk: Any = 
 
     ``use_graph``: the whole decode loop (embedding rows, kernel, argmax, row state) is captured into one
     HIP graph and replayed once — the kernel reads positions and activity from device tensors, so nothing
-    in a step depends on the host.  Per-step kernel times are then not available."""
+    in a step depends on the host.  Per-step kernel times are then not available.
+
+    ``engine``: "tiles" = the batch kernel (matrix-core tiles, 2..16 rows), "rows" = the batch-1 kernel's row-streaming
+    engine with every row's activation vector (1..4 rows: `decode_schedule_mb.rows_kernel`), "auto" = what ``mk`` was
+    made for, else rows up to four rows.  Both decode every active row as the batch-1 route would decode it alone."""
     from .decode import globs_shape
 
     device = globs.hidden_states.device
@@ -75,11 +98,11 @@ def decode(globs: Any, prompts: torch.Tensor, max_new_tokens: int, *, mk: Any = 
         raise ValueError(f"{B} prompts for buffers of {rows_of(globs)} rows")
     if T + max_new_tokens > globs.k_cache.shape[2]:
         raise ValueError("prompt_len + max_new_tokens exceeds the KV cache capacity")
-    mk = mk or _mk_kernel.get_mk()
+    launcher, mk = _route(mk, B, engine)
     state = RowState.of(globs)
     state.restart(0)
     globs.instructions = None
-    _mk_kernel.build(globs)
+    launcher.build(globs)
     out = torch.zeros(B, T + max(max_new_tokens, 1), dtype=torch.long, device=device)
     out[:, :T] = prompts.to(device)
     out[:, T] = prefill_by_decode(globs, mk, prompts)
@@ -99,7 +122,7 @@ def decode(globs: Any, prompts: torch.Tensor, max_new_tokens: int, *, mk: Any = 
             _embed(globs, out[:, T + i])
             if events and i >= lead_in:
                 events[i - lead_in][0].record()
-            _mk_kernel.call_mk(globs, mk)
+            launcher.call_mk(globs, mk)
             if events and i >= lead_in:
                 events[i - lead_in][1].record()
             nxt = argmax_rows(globs.logits) if use_graph else globs.logits.argmax(dim=-1)
@@ -162,6 +185,7 @@ def decode(globs: Any, prompts: torch.Tensor, max_new_tokens: int, *, mk: Any = 
             "kernel_tok_s": produced / kernel_s, "kernel_steps": len(window), "kernel_ms_per_step": kernel_s * 1e3 / nsteps,
             "algorithmic_bytes": nbytes, "achieved_GBps": nbytes / kernel_s / 1e9, "per_step_ms": per_step_ms,
             "first_timed_context": T + lead_in + 1, "last_timed_context": T + ntok,
+            "engine": "rows" if launcher is _rows_kernel else "tiles",
         }
     mk.check()
     return result

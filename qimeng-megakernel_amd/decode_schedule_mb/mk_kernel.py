@@ -251,7 +251,10 @@ class BatchMegaKernel:
         a.oproj_blocks, a.down_blocks = hidden // self.residual_tiles[0], hidden // self.residual_tiles[1]
         a.timeline = self.timeline.data_ptr() if self.timeline is not None else None
         a.stream = torch.cuda.current_stream(tensors[1].device).cuda_stream
-        rc = int(self._lib.qmk_decode_step_batch(ctypes.byref(a)))
+        self._launch(tensors[1].device)
+
+    def _launch(self, device: torch.device) -> None:
+        rc = int(self._lib.qmk_decode_step_batch(ctypes.byref(self._args)))
         if rc != 0:
             raise RuntimeError(f"qmk_decode_step_batch failed with {rc}: {self.error_string(rc)}")
 

@@ -15,6 +15,7 @@ from __graft_entry__ import LIBRARY, ROOT, build_library
 from qimeng_megakernel_amd.decode_schedule import mk_kernel
 from qimeng_megakernel_amd.decode_schedule_mb import mk_kernel as mk_kernel_mb
 from qimeng_megakernel_amd.decode_schedule_moe import mk_kernel as mk_kernel_moe
+from qimeng_megakernel_amd.decode_schedule_mb import rows_kernel as rows_kernel_mb
 from qimeng_megakernel_amd.decode_schedule_moe import rows_kernel
 
 HEADER = ROOT / "include" / "qmk.h"
@@ -31,14 +32,16 @@ def test_every_declared_symbol_is_exported(lib):
     text = HEADER.read_text()
     declared = set(re.findall(r"^(?:int|uint64_t|const char\*)\s+(qmk_\w+)\s*\(", text, flags=re.M))
     assert declared == {"qmk_decode_step", "qmk_decode_step_static", "qmk_decode_step_batch", "qmk_decode_step_moe", "qmk_moe_workspace_bytes",
-                        "qmk_decode_step_moe_rows", "qmk_moe_rows_workspace_bytes", "qmk_query",
+                        "qmk_decode_step_moe_rows", "qmk_moe_rows_workspace_bytes",
+                        "qmk_decode_step_rows", "qmk_rows_workspace_bytes", "qmk_query",
                         "qmk_status_fetch", "qmk_error_string", "qmk_workspace_bytes"}
     for name in declared:
         assert hasattr(lib, name), name
 
 
 @pytest.mark.parametrize("struct,mirror", [("QmkArgs", mk_kernel.QmkArgs), ("QmkBatchArgs", mk_kernel_mb.QmkBatchArgs),
-                                           ("QmkMoeArgs", mk_kernel_moe.QmkMoeArgs), ("QmkMoeRowsArgs", rows_kernel.QmkMoeRowsArgs)])
+                                           ("QmkMoeArgs", mk_kernel_moe.QmkMoeArgs), ("QmkMoeRowsArgs", rows_kernel.QmkMoeRowsArgs),
+                                           ("QmkRowsArgs", rows_kernel_mb.QmkRowsArgs)])
 def test_struct_layout_matches_header(tmp_path, struct, mirror):
     """Compile the header with gcc and compare sizeof/offsetof with the ctypes mirror."""
     fields = [name for name, _ in mirror._fields_]
@@ -111,6 +114,20 @@ def test_host_side_argument_errors(lib):
     assert lib.qmk_moe_workspace_bytes(8, 0) == 8 * 2048 * 4 + 128 + lib.qmk_workspace_bytes(0) + moe_units     # no shared expert
     assert lib.qmk_moe_workspace_bytes(9, 4) == 0
     assert lib.qmk_error_string(12345).decode() == "unknown code"
+    # the dense route at 1..4 rows on the row-streaming engine: a set of the dense route's units per row
+    rows_kernel_mb.get_mk()
+    assert [lib.qmk_rows_workspace_bytes(b) for b in (0, 1, 4, 5)] == [0, lib.qmk_workspace_bytes(0), 4 * lib.qmk_workspace_bytes(0), 0]
+    assert lib.qmk_decode_step_rows(None) == 1
+    d = rows_kernel_mb.QmkRowsArgs()
+    d.struct_size = ctypes.sizeof(rows_kernel_mb.QmkRowsArgs)
+    assert lib.qmk_decode_step_rows(ctypes.byref(d)) == 2                    # the nested step carries its own size
+    d.step.struct_size = ctypes.sizeof(mk_kernel_mb.QmkBatchArgs)
+    d.step.model = 2
+    assert lib.qmk_decode_step_rows(ctypes.byref(d)) == 8
+    d.step.model = 0
+    assert lib.qmk_decode_step_rows(ctypes.byref(d)) == 3                    # batch_size 0
+    d.step.batch_size = 4
+    assert lib.qmk_decode_step_rows(ctypes.byref(d)) == 1                    # all tensor pointers are NULL
     # several requests in one launch: a set of the MoE route's units per row, in whole 128-byte lines
     rows_kernel.get_mk()
     per_row = lib.qmk_moe_workspace_bytes(8, 0) - 8 * 2048 * 4 - 128
