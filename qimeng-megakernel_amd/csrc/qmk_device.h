@@ -136,6 +136,12 @@ __device__ __forceinline__ float bf2f(u16 v) { return __uint_as_float(static_cas
 // norms, epilogues and merges round thousands of values per layer between two streaming phases, where instruction
 // count is time: +1.4 % tok/s on the Llama-3.2-1B shape, +2.1 % Qwen3-1.7B, +2.1 % Qwen1.5-MoE, same bits.
 __device__ __forceinline__ u16 f2bf(float f) { return __builtin_bit_cast(u16, static_cast<__bf16>(f)); }
+// Two at once, low half first (the instruction converts a pair; written as two f2bf the compiler issues it twice).
+typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
+typedef float f32x2_t __attribute__((ext_vector_type(2)));
+__device__ __forceinline__ uint32_t f2bf2(float lo, float hi) {
+  return __builtin_bit_cast(uint32_t, __builtin_convertvector(f32x2_t{lo, hi}, bf16x2_t));
+}
 // 2^x for x <= 0 as one v_exp_f32 (results below the normal range flush to zero, which is what a
 // softmax weight that small should be); 2^-inf = 0.
 __device__ __forceinline__ float exp2_fast(float x) { return __builtin_amdgcn_exp2f(x); }

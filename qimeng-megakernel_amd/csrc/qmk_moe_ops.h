@@ -353,7 +353,7 @@ __device__ __forceinline__ bool upgate_rows(Smem<M>& s, const Ctx& c, const u16*
   }
   __syncthreads();
   for (int pair = c.tid; pair < n / 2; pair += kThreads) {
-    const uint32_t word = static_cast<uint32_t>(f2bf(s.res[2 * pair])) | (static_cast<uint32_t>(f2bf(s.res[2 * pair + 1])) << 16);
+    const uint32_t word = f2bf2(s.res[2 * pair], s.res[2 * pair + 1]);
     st_shared32(dst0 + r0 + 2 * pair, word);
     if (dst1 != nullptr) st_shared32(dst1 + r0 + 2 * pair, word);
     if (units != nullptr) st_tagged(units + (r0 + 2 * pair) / 2, word, tag);
@@ -432,7 +432,7 @@ __device__ __forceinline__ bool op_shared_down(const Params& p, Smem<M>& s, cons
   __syncthreads();
   for (int pair = c.tid; pair < (n1 - n0) * tile / 2; pair += kThreads)
     st_shared32(mine + n0 * tile + 2 * pair,
-                static_cast<uint32_t>(f2bf(s.res[2 * pair])) | (static_cast<uint32_t>(f2bf(s.res[2 * pair + 1])) << 16));
+                f2bf2(s.res[2 * pair], s.res[2 * pair + 1]));
   release_stores();
   __syncthreads();
   if (c.tid < n1 - n0) publish(counter_ptr(p, layer, ROW_SHARED_DOWN, n0 + c.tid), 1);
@@ -648,7 +648,7 @@ __device__ __forceinline__ bool routed_down_commit(const Params& p, Smem<M>& s, 
       ro1 += s.res[j * n + 2 * pair + 1];
     }
     const float h0 = (bf_lo(old) + ro0) + 0.f, h1 = (bf_hi(old) + ro1) + 0.f;   // opcode 14's expression without a shared term
-    const uint32_t word = static_cast<uint32_t>(f2bf(h0)) | (static_cast<uint32_t>(f2bf(h1)) << 16);
+    const uint32_t word = f2bf2(h0, h1);
     st_shared32(p.hidden + r, word);
     st_tagged(p.ws + kWsHiddenOut + r / 2, word, tag);
     st_shared_f32(p.routed_out_f32 + r, 0.f);
@@ -836,10 +836,10 @@ __device__ __forceinline__ bool op_combine(const Params& p, Smem<M>& s, const Ct
       }
     }
     const float h0 = (bf_lo(old) + ro0) + gate * sh0, h1 = (bf_hi(old) + ro1) + gate * sh1;
-    const uint32_t word = static_cast<uint32_t>(f2bf(h0)) | (static_cast<uint32_t>(f2bf(h1)) << 16);
+    const uint32_t word = f2bf2(h0, h1);
     st_shared32(p.hidden + r, word);
     if (tg) st_tagged(p.ws + kWsHiddenOut + r / 2, word, tag);   // the next layer's QKV and O-projection, the LM head
-    if (p.shared_k_slices > 0) st_shared32(p.shared_out + r, static_cast<uint32_t>(f2bf(sh0)) | (static_cast<uint32_t>(f2bf(sh1)) << 16));
+    if (p.shared_k_slices > 0) st_shared32(p.shared_out + r, f2bf2(sh0, sh1));
     st_shared_f32(p.routed_out_f32 + r, 0.f);
     st_shared_f32(p.routed_out_f32 + r + 1, 0.f);
   }

@@ -224,13 +224,10 @@ __device__ __forceinline__ bool rms_to_lds(const Params& p, Smem<M>& s, const Ct
   ss = block_sum(ss, s.red);
   const float mean = ss / static_cast<float>(M::H);
   const float rstd = 1.0f / sqrtf(mean + p.rms_norm_eps);
-  const u16 y0 = f2bf(bf_lo(wv.x) * round_bf16(x0 * rstd));
-  const u16 y1 = f2bf(bf_hi(wv.x) * round_bf16(x1 * rstd));
-  const u16 y2 = f2bf(bf_lo(wv.y) * round_bf16(x2 * rstd));
-  const u16 y3 = f2bf(bf_hi(wv.y) * round_bf16(x3 * rstd));
+  const uint32_t n01 = f2bf2(x0 * rstd, x1 * rstd), n23 = f2bf2(x2 * rstd, x3 * rstd);   // bf16(x * rstd) ...
   uint2 out;
-  out.x = static_cast<uint32_t>(y0) | (static_cast<uint32_t>(y1) << 16);
-  out.y = static_cast<uint32_t>(y2) | (static_cast<uint32_t>(y3) << 16);
+  out.x = f2bf2(bf_lo(wv.x) * bf_lo(n01), bf_hi(wv.x) * bf_hi(n01));                     // ... times the weight, rounded again
+  out.y = f2bf2(bf_lo(wv.y) * bf_lo(n23), bf_hi(wv.y) * bf_hi(n23));
   *reinterpret_cast<uint2*>(s.x + t * 4) = out;
   __syncthreads();
   return s.ctl[0] == 0;
@@ -247,7 +244,7 @@ __device__ __forceinline__ bool rms_to_lds(const Params& p, Smem<M>& s, const Ct
 __device__ __forceinline__ uint32_t rope_pair(float v0, float v1, float2 cs, float2 sn) {
   const float o0 = v0 * cs.x + (-v1) * sn.x;
   const float o1 = v1 * cs.y + v0 * sn.y;
-  return static_cast<uint32_t>(f2bf(o0)) | (static_cast<uint32_t>(f2bf(o1)) << 16);
+  return f2bf2(o0, o1);
 }
 __device__ __forceinline__ uint32_t rope_pair(float v0, float v1, const float* cosr, const float* sinr, int d) {
   return rope_pair(v0, v1, *reinterpret_cast<const float2*>(cosr + d), *reinterpret_cast<const float2*>(sinr + d));
@@ -402,7 +399,7 @@ __device__ bool op_rms_qkv_rope(const Params& p, Smem<M>& s, const Ctx& c) {
     const float v0 = round_bf16(a0), v1 = round_bf16(a1);
     if constexpr (M::QK_NORM) {
       // Qwen3 op set: the rounded GEMV result leaves as it is; norm and RoPE belong to the attention prologue.
-      const uint32_t w = static_cast<uint32_t>(f2bf(v0)) | (static_cast<uint32_t>(f2bf(v1)) << 16);
+      const uint32_t w = f2bf2(v0, v1);
       st_shared32(p.qkv_raw + r, w);
       if (tg) {
         const int kq = M::NQ * M::D, kk = (M::NQ + M::NKV) * M::D;
@@ -419,11 +416,12 @@ __device__ bool op_rms_qkv_rope(const Params& p, Smem<M>& s, const Ctx& c) {
       if (tg) st_tagged(p.ws + kWsK + i / 2, w, tag);
     } else {
       const int i = r - (M::NQ + M::NKV) * M::D;
-      const uint32_t w = static_cast<uint32_t>(f2bf(v0)) | (static_cast<uint32_t>(f2bf(v1)) << 16);
+      const uint32_t w = f2bf2(v0, v1);
       st_shared32(p.v_cache + kv_row + i, w);
       if (tg) st_tagged(p.ws + kWsV + i / 2, w, tag);
     }
   }
+  QMK_STAMP(3);
   if (tg) return true;  // the units announce themselves: nothing to wait for, nothing to count
 
   release_stores();
@@ -475,7 +473,7 @@ __device__ __forceinline__ void merge_partials(const Params& p, int head0, int n
   }
   const float o0 = den > 0.f ? num0 / den : 0.f, o1 = den > 0.f ? num1 / den : 0.f;
   if (terminal) {
-    st_shared32(p.attn_out + h * M::D + d, static_cast<uint32_t>(f2bf(o0)) | (static_cast<uint32_t>(f2bf(o1)) << 16));
+    st_shared32(p.attn_out + h * M::D + d, f2bf2(o0, o1));
   } else {
     float* dst = p.attn_partial + (static_cast<size_t>(h) * p.max_splits + out_slot) * M::D + d;
     st_shared_f32(dst, o0);
@@ -759,14 +757,10 @@ __device__ bool op_attn_splitkv(const Params& p, Smem<M>& s, const Ctx& c) {
     }
     l_run = __builtin_fmaf(l_run, alpha, psum);
     // P = hi + lo, both bf16: A operand rows = heads, k slots = the lane's four tokens.
-    uint32_t hi[4], lo[4];
-#pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      hi[i] = f2bf(pr[i]);
-      lo[i] = f2bf(pr[i] - bf2f(static_cast<u16>(hi[i])));
-    }
-    const bf4 p_hi = __builtin_bit_cast(bf4, u2{hi[0] | (hi[1] << 16), hi[2] | (hi[3] << 16)});
-    const bf4 p_lo = __builtin_bit_cast(bf4, u2{lo[0] | (lo[1] << 16), lo[2] | (lo[3] << 16)});
+    const uint32_t h01 = f2bf2(pr[0], pr[1]), h23 = f2bf2(pr[2], pr[3]);
+    const uint32_t l01 = f2bf2(pr[0] - bf_lo(h01), pr[1] - bf_hi(h01)), l23 = f2bf2(pr[2] - bf_lo(h23), pr[3] - bf_hi(h23));
+    const bf4 p_hi = __builtin_bit_cast(bf4, u2{h01, h23});
+    const bf4 p_lo = __builtin_bit_cast(bf4, u2{l01, l23});
     // The accumulators of head h are scaled by that head's alpha (it lives in lane h); this lane
     // holds the heads 4*g4 .. 4*g4 + 3.
     float a_head[4];
@@ -934,9 +928,8 @@ __device__ bool op_attn_reduce(const Params& p, Smem<M>& s, const Ctx& c) {
 
 // Two neighbouring residual-stream elements plus bf16(delta), as a bf16 pair.
 __device__ __forceinline__ uint32_t residual_word(uint32_t old, float d0, float d1) {
-  const u16 n0 = f2bf(bf_lo(old) + round_bf16(d0));
-  const u16 n1 = f2bf(bf_hi(old) + round_bf16(d1));
-  return static_cast<uint32_t>(n0) | (static_cast<uint32_t>(n1) << 16);
+  const uint32_t d = f2bf2(d0, d1);
+  return f2bf2(bf_lo(old) + bf_lo(d), bf_hi(old) + bf_hi(d));
 }
 
 // The residual-stream pair `pair` of the rows [rs, ...) before this instruction adds to it: from
@@ -952,9 +945,8 @@ __device__ __forceinline__ bool residual_in(const Params& p, const uint64_t* uni
 // hidden[r0], hidden[r0+1] += bf16(delta): one coherent 32-bit read-modify-write.
 __device__ __forceinline__ void residual_pair(u16* hidden_pair, float d0, float d1) {
   const uint32_t old = ld_shared32(hidden_pair);
-  const u16 n0 = f2bf(bf_lo(old) + round_bf16(d0));
-  const u16 n1 = f2bf(bf_hi(old) + round_bf16(d1));
-  st_shared32(hidden_pair, static_cast<uint32_t>(n0) | (static_cast<uint32_t>(n1) << 16));
+  const uint32_t d = f2bf2(d0, d1);
+  st_shared32(hidden_pair, f2bf2(bf_lo(old) + bf_lo(d), bf_hi(old) + bf_hi(d)));
 }
 
 // Rows kUpGateBuffers .. kUpGateBuffers + PARK_ROWS - 1 of every wave of the up/gate instruction `words` into LDS,
@@ -1090,8 +1082,8 @@ __device__ bool op_oproj_residual(const Params& p, Smem<M>& s, const Ctx& c, Car
     for (int k = 0; k < kItems; ++k) {
       const int item = c.tid + k * kThreads;
       const float inv = den[k] > 0.f ? 1.0f / den[k] : 0.f;
-      const uint32_t lo = static_cast<uint32_t>(f2bf(n0[k] * inv)) | (static_cast<uint32_t>(f2bf(n1[k] * inv)) << 16);
-      const uint32_t hi = static_cast<uint32_t>(f2bf(n2[k] * inv)) | (static_cast<uint32_t>(f2bf(n3[k] * inv)) << 16);
+      const uint32_t lo = f2bf2(n0[k] * inv, n1[k] * inv);
+      const uint32_t hi = f2bf2(n2[k] * inv, n3[k] * inv);
       *reinterpret_cast<uint2*>(s.x + item * 4) = make_uint2(lo, hi);
       if (nstart == 0) {  // one workgroup also leaves attn_out in memory, as the reference does
         st_shared32(p.attn_out + item * 4, lo);
@@ -1118,6 +1110,7 @@ __device__ bool op_oproj_residual(const Params& p, Smem<M>& s, const Ctx& c, Car
       st_tagged(p.ws + kWsHiddenMid + (rs + 2 * pair) / 2, w, tag);
       st_shared32(p.hidden + rs + 2 * pair, w);
     }
+    QMK_STAMP(3);
     return true;
   }
   for (int pair = c.tid; pair < nrows / 2; pair += kThreads)
@@ -1205,17 +1198,15 @@ __device__ bool op_rms_upgate_silu(const Params& p, Smem<M>& s, const Ctx& c, co
   QMK_STAMP(2);
   // Two neighbouring outputs of a tile leave as one 32-bit word.
   for (int pair = c.tid; pair < nout / 2; pair += kThreads) {
-    uint32_t word = 0;
-#pragma unroll
-    for (int k = 0; k < 2; ++k) {
-      const int i = 2 * pair + k;
-      const float up = round_bf16(s.res[2 * i]), gate = round_bf16(s.res[2 * i + 1]);
-      const float act = round_bf16(gate / (1.0f + expf(-gate)));
-      word |= static_cast<uint32_t>(f2bf(act * up)) << (16 * k);
-    }
+    // elements 4 pair .. 4 pair + 3: up and gate of the pair's two outputs
+    const uint32_t ug0 = f2bf2(s.res[4 * pair], s.res[4 * pair + 1]), ug1 = f2bf2(s.res[4 * pair + 2], s.res[4 * pair + 3]);
+    const float g0 = bf_hi(ug0), g1 = bf_hi(ug1);
+    const uint32_t act = f2bf2(g0 / (1.0f + expf(-g0)), g1 / (1.0f + expf(-g1)));
+    const uint32_t word = f2bf2(bf_lo(act) * bf_lo(ug0), bf_hi(act) * bf_lo(ug1));
     st_shared32(p.silu_out + row_of(2 * pair), word);
     if (tg) st_tagged(p.ws + kWsSilu + row_of(2 * pair) / 2, word, tag_of(s.generation, layer));
   }
+  QMK_STAMP(3);
   if (tg) return true;  // the down projection polls the units
 
   release_stores();
@@ -1375,6 +1366,7 @@ __device__ bool op_down_residual(const Params& p, Smem<M>& s, const Ctx& c) {
       st_tagged(p.ws + kWsHiddenOut + (rs + 2 * pair) / 2, w, tag);
       st_shared32(p.hidden + rs + 2 * pair, w);
     }
+    QMK_STAMP(3);
     return true;
   }
   if (kg == M::F) {  // one slice: every row has a single writer

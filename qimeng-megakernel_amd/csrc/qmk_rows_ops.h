@@ -201,13 +201,10 @@ __device__ __forceinline__ bool rms_rows(const Params& p, Smem<M>& s, const Ctx&
       const float mean = total / static_cast<float>(M::H);
       const float rstd = 1.0f / sqrtf(mean + p.rms_norm_eps);
       const float x0 = bf_lo(lo[b]), x1 = bf_hi(lo[b]), x2 = bf_lo(hi[b]), x3 = bf_hi(hi[b]);
-      const u16 y0 = f2bf(bf_lo(wv.x) * round_bf16(x0 * rstd));
-      const u16 y1 = f2bf(bf_hi(wv.x) * round_bf16(x1 * rstd));
-      const u16 y2 = f2bf(bf_lo(wv.y) * round_bf16(x2 * rstd));
-      const u16 y3 = f2bf(bf_hi(wv.y) * round_bf16(x3 * rstd));
+      const uint32_t n01 = f2bf2(x0 * rstd, x1 * rstd), n23 = f2bf2(x2 * rstd, x3 * rstd);
       uint2 out;
-      out.x = static_cast<uint32_t>(y0) | (static_cast<uint32_t>(y1) << 16);
-      out.y = static_cast<uint32_t>(y2) | (static_cast<uint32_t>(y3) << 16);
+      out.x = f2bf2(bf_lo(wv.x) * bf_lo(n01), bf_hi(wv.x) * bf_hi(n01));
+      out.y = f2bf2(bf_lo(wv.y) * bf_lo(n23), bf_hi(wv.y) * bf_hi(n23));
       *reinterpret_cast<uint2*>(&s.x[b][t * 4]) = out;
     }
   });
@@ -266,7 +263,7 @@ __device__ bool op_qkv(const Params& p, Smem<M>& s, const Ctx& c) {
     uint64_t* ws = ws_of(p, b);
     constexpr int kq = M::NQ * M::D, kk = (M::NQ + M::NKV) * M::D;
     if constexpr (M::QK_NORM) {
-      const uint32_t w = static_cast<uint32_t>(f2bf(v0)) | (static_cast<uint32_t>(f2bf(v1)) << 16);
+      const uint32_t w = f2bf2(v0, v1);
       st_shared32(p.qkv_raw + static_cast<size_t>(b) * M::QKV + r, w);
       st_tagged(ws + (r < kq ? kWsQ + r / 2 : (r < kk ? kWsK + (r - kq) / 2 : kWsV + (r - kk) / 2)), w, tag);
     } else {
@@ -285,7 +282,7 @@ __device__ bool op_qkv(const Params& p, Smem<M>& s, const Ctx& c) {
         st_tagged(ws + kWsK + i / 2, w, tag);
       } else {
         const int i = r - kk;
-        const uint32_t w = static_cast<uint32_t>(f2bf(v0)) | (static_cast<uint32_t>(f2bf(v1)) << 16);
+        const uint32_t w = f2bf2(v0, v1);
         st_shared32(p.v_cache + kv_row + i, w);
         st_tagged(ws + kWsV + i / 2, w, tag);
       }
@@ -415,8 +412,8 @@ __device__ bool op_oproj(const Params& p, Smem<M>& s, const Ctx& c) {
     for (int k = 0; k < kItems; ++k) {
       const int item = c.tid + k * kThreads;
       const float inv = den[k] > 0.f ? 1.0f / den[k] : 0.f;
-      const uint32_t lo = static_cast<uint32_t>(f2bf(n0[k] * inv)) | (static_cast<uint32_t>(f2bf(n1[k] * inv)) << 16);
-      const uint32_t hi = static_cast<uint32_t>(f2bf(n2[k] * inv)) | (static_cast<uint32_t>(f2bf(n3[k] * inv)) << 16);
+      const uint32_t lo = f2bf2(n0[k] * inv, n1[k] * inv);
+      const uint32_t hi = f2bf2(n2[k] * inv, n3[k] * inv);
       *reinterpret_cast<uint2*>(&s.x[b][item * 4]) = make_uint2(lo, hi);
       if (nstart == 0) {  // one workgroup also leaves attn_out in memory, as the reference does
         u16* out = p.attn_out + static_cast<size_t>(b) * AW + item * 4;
@@ -662,7 +659,7 @@ __device__ bool op_routed_upgate(const Params& p, Smem<M>& s, const Ctx& c) {
           const float g0 = round_bf16(v[0][b]), g1 = round_bf16(v[1][b]);
           const float a0 = (g0 / (1.0f + expf(-g0))) * round_bf16(v[2][b]);
           const float a1 = (g1 / (1.0f + expf(-g1))) * round_bf16(v[3][b]);
-          const uint32_t word = static_cast<uint32_t>(f2bf(a0)) | (static_cast<uint32_t>(f2bf(a1)) << 16);
+          const uint32_t word = f2bf2(a0, a1);
           st_shared32(p.routed_silu + (static_cast<size_t>(b) * K + j) * F + o, word);
           if (j == K - 1) st_shared32(p.silu_out + static_cast<size_t>(b) * F + o, word);   // what the last slot leaves, as after the VM's run
           st_tagged(ws_of(p, b) + kWsRoutedSilu + j * 1024 + o / 2, word, tag);
@@ -787,7 +784,7 @@ __device__ bool op_routed_down_commit(const Params& p, Smem<M>& s, const Ctx& c)
       ro1 += s.terms[my_b][j][2 * my_pair + 1];
     }
     const float h0 = (bf_lo(old) + ro0) + 0.f, h1 = (bf_hi(old) + ro1) + 0.f;   // opcode 14's expression without a shared term
-    const uint32_t word = static_cast<uint32_t>(f2bf(h0)) | (static_cast<uint32_t>(f2bf(h1)) << 16);
+    const uint32_t word = f2bf2(h0, h1);
     st_shared32(p.hidden + static_cast<size_t>(my_b) * M::H + r, word);
     st_tagged(ws_of(p, my_b) + kWsHiddenOut + r / 2, word, tag);
     st_shared_f32(p.routed_out_f32 + static_cast<size_t>(my_b) * M::H + r, 0.f);
@@ -834,13 +831,10 @@ __device__ bool op_upgate(const Params& p, Smem<M>& s, const Ctx& c) {
     const int b = item / pairs, pair = item % pairs;
     uint32_t word = 0;
     if (s.live[b]) {
-#pragma unroll
-      for (int k = 0; k < 2; ++k) {
-        const int i = 2 * pair + k;
-        const float up = round_bf16(s.res[b][2 * i]), gate = round_bf16(s.res[b][2 * i + 1]);
-        const float act = round_bf16(gate / (1.0f + expf(-gate)));
-        word |= static_cast<uint32_t>(f2bf(act * up)) << (16 * k);
-      }
+      const uint32_t ug0 = f2bf2(s.res[b][4 * pair], s.res[b][4 * pair + 1]), ug1 = f2bf2(s.res[b][4 * pair + 2], s.res[b][4 * pair + 3]);
+      const float g0 = bf_hi(ug0), g1 = bf_hi(ug1);
+      const uint32_t act = f2bf2(g0 / (1.0f + expf(-g0)), g1 / (1.0f + expf(-g1)));
+      word = f2bf2(bf_lo(act) * bf_lo(ug0), bf_hi(act) * bf_lo(ug1));
       st_tagged(ws_of(p, b) + kWsSilu + row_of(2 * pair) / 2, word, tag);
     }
     st_shared32(p.silu_out + static_cast<size_t>(b) * M::F + row_of(2 * pair), word);   // zeros for a row that is not decoded
