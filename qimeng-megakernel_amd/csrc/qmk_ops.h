@@ -321,7 +321,8 @@ __device__ __forceinline__ void forget(Carried& c) {
 template <class M>
 __device__ __forceinline__ const u16* upgate_row(const Params& p, const int32_t* w, int layer, int tile, int e) {
   const int i = e >> 1;
-  const int row = w[4 + i / tile] * tile + i % tile;
+  const int sh = __builtin_ctz(static_cast<unsigned>(tile));   // tiles are powers of two (upgate_check): no integer division per row request
+  const int row = w[4 + (i >> sh)] * tile + (i & (tile - 1));
   const u16* base = (e & 1) ? p.gate_w : p.up_w;
   return base + (static_cast<size_t>(layer) * M::F + row) * M::H;
 }
@@ -332,10 +333,10 @@ __device__ __forceinline__ int upgate_check(const Params& p, const int32_t* w) {
   if (layer < 0 || layer >= p.num_layers) return 1;
   if (n < 0 || n > kInstWords - 6) return 3;
   const int tile = w[5 + n];
-  if (tile <= 0 || (tile & 1) || M::F % tile != 0) return 5 + n;
+  if (tile < 2 || (tile & (tile - 1)) || M::F % tile != 0) return 5 + n;   // an even power of two
   if (n * tile * 2 > kResSlots) return 3;
   for (int i = 0; i < n; ++i)
-    if (w[4 + i] < 0 || w[4 + i] >= M::F / tile) return 4 + i;
+    if (w[4 + i] < 0 || static_cast<long>(w[4 + i] + 1) * tile > M::F) return 4 + i;
   return -1;
 }
 
@@ -1139,7 +1140,7 @@ __device__ bool op_rms_upgate_silu(const Params& p, Smem<M>& s, const Ctx& c, co
   const int nrows = 2 * nout;      // streamed rows: element 2i = up row i, 2i+1 = gate row i
   const u16* Wu = p.up_w + static_cast<size_t>(layer) * M::F * M::H;
   const u16* Wg = p.gate_w + static_cast<size_t>(layer) * M::F * M::H;
-  auto row_of = [&](int i) { return s.inst[4 + i / tile] * tile + i % tile; };
+  auto row_of = [&](int i) { return s.inst[4 + (i >> __builtin_ctz(static_cast<unsigned>(tile)))] * tile + (i & (tile - 1)); };
   auto src = [&](int e) { return upgate_row<M>(p, s.inst, layer, tile, e); };
 
   bool in_lds = false;   // the O-proj before this instruction has left rows kUpGateBuffers.. of every wave in LDS
@@ -1259,8 +1260,11 @@ __device__ bool op_down_residual(const Params& p, Smem<M>& s, const Ctx& c) {
   // Element order is chosen per wave so that a wave owns whole rows: wave w streams the
   // segments of rows w, w+8, ...  Element index e (as seen by `stream`: e = w + 8*i) maps to
   // step i of wave w: row = w + 8*(i / segs), segment = i % segs.
-  auto row_of = [&](int e) { return (e & (kWaves - 1)) + kWaves * ((e >> 3) / segs); };
-  auto seg_of = [&](int e) { return (e >> 3) % segs; };
+  // (i / segs as a multiplication: exact for the few steps a wave has, and an integer division costs forty instructions)
+  const int inv_segs = (65536 + segs - 1) / segs;
+  auto step_row = [&](int e) { return ((e >> 3) * inv_segs) >> 16; };
+  auto row_of = [&](int e) { return (e & (kWaves - 1)) + kWaves * step_row(e); };
+  auto seg_of = [&](int e) { return (e >> 3) - step_row(e) * segs; };
   const u16* W = p.down_w + (static_cast<size_t>(layer) * M::H + rs) * M::F + ks;
   auto src = [&](int e) { return W + static_cast<size_t>(row_of(e)) * M::F + seg_of(e) * (512 * CH); };
   // Number of stream elements: waves with fewer rows simply run out earlier; bound by the largest.
