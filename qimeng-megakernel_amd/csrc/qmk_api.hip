@@ -1177,8 +1177,13 @@ static int decode_step_rows(const QmkRowsArgs* r) {
 extern "C" int qmk_decode_step_rows(const QmkRowsArgs* r) {
   if (r == nullptr) return QMK_ERR_NULL_ARG;
   if (r->struct_size != sizeof(QmkRowsArgs) || r->step.struct_size != sizeof(QmkBatchArgs)) return QMK_ERR_ABI;
-  if (r->step.model == QMK_MODEL_LLAMA_3_2_1B) return decode_step_rows<rows::Llama1BRows>(r);
-  if (r->step.model == QMK_MODEL_QWEN3_1_7B) return decode_step_rows<rows::Qwen3_1p7BRows>(r);
+  // the ops compiled for the smallest row count that holds the batch (same LDS and registers at every count: the
+  // occupancy found for four holds)
+  const int B = r->step.batch_size;
+  if (r->step.model == QMK_MODEL_LLAMA_3_2_1B)
+    return B <= 2 ? decode_step_rows<rows::Llama1BRowsN<2>>(r) : (B == 3 ? decode_step_rows<rows::Llama1BRowsN<3>>(r) : decode_step_rows<rows::Llama1BRows>(r));
+  if (r->step.model == QMK_MODEL_QWEN3_1_7B)
+    return B <= 2 ? decode_step_rows<rows::Qwen3_1p7BRowsN<2>>(r) : (B == 3 ? decode_step_rows<rows::Qwen3_1p7BRowsN<3>>(r) : decode_step_rows<rows::Qwen3_1p7BRows>(r));
   return QMK_ERR_MODEL;
 }
 

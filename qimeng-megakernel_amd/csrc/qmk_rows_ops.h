@@ -46,16 +46,33 @@ struct XWidth<M, std::enable_if_t<M::DENSE_ROWS>> {
   static constexpr int value = M::F;
 };
 
-// The dense geometries as the rows kernel uses them: nothing carried or parked between instructions.
-struct Llama1BRows : Llama1B {
+// The dense geometries as the rows kernel uses them: nothing carried or parked between instructions, and the number of
+// rows the ops are compiled for (ROWS: 2, 3 or 4 — a launch of B rows runs on the smallest that holds them, so that two
+// rows do not pay the norms, dot products and epilogues of four).
+template <int NR>
+struct Llama1BRowsN : Llama1B {
   static constexpr int CARRY_ROWS = 0;
   static constexpr int PARK_ROWS = 0;
   static constexpr bool DENSE_ROWS = true;
+  static constexpr int ROWS = NR;
 };
-struct Qwen3_1p7BRows : Qwen3_1p7B {
+template <int NR>
+struct Qwen3_1p7BRowsN : Qwen3_1p7B {
   static constexpr int CARRY_ROWS = 0;
   static constexpr int PARK_ROWS = 0;
   static constexpr bool DENSE_ROWS = true;
+  static constexpr int ROWS = NR;
+};
+using Llama1BRows = Llama1BRowsN<kMaxRows>;
+using Qwen3_1p7BRows = Qwen3_1p7BRowsN<kMaxRows>;
+// Rows the ops of a geometry are compiled for (kMaxRows unless the geometry says otherwise).
+template <class M, class = void>
+struct RowsOf {
+  static constexpr int value = kMaxRows;
+};
+template <class M>
+struct RowsOf<M, std::void_t<decltype(M::ROWS)>> {
+  static constexpr int value = M::ROWS;
 };
 
 template <class M>
@@ -133,15 +150,16 @@ __device__ __forceinline__ Params row_view(const Params& p, int r, int pos) {
 // group of weight-row requests, one group per look at the units.
 template <class M, int NP, class Pace>
 __device__ __forceinline__ bool rms_rows(const Params& p, Smem<M>& s, const Ctx& c, int region, uint32_t tag, const u16* weight, Pace pace) {
+  constexpr int NR = RowsOf<M>::value;
   static_assert(M::H == kThreads * 4, "one thread normalises four elements of every row");
   const int t = c.tid, B = p.batch;
   const uint2 wv = *reinterpret_cast<const uint2*>(weight + t * 4);
-  uint32_t lo[kMaxRows], hi[kMaxRows];
-  static_for<0, kMaxRows>([&](auto b) { lo[b] = hi[b] = 0u; });
+  uint32_t lo[NR], hi[NR];
+  static_for<0, NR>([&](auto b) { lo[b] = hi[b] = 0u; });
   bool done = region < 0;
   auto look = [&] {
-    uint64_t xx[kMaxRows], yy[kMaxRows];
-    static_for<0, kMaxRows>([&](auto b) {
+    uint64_t xx[NR], yy[NR];
+    static_for<0, NR>([&](auto b) {
       xx[b] = yy[b] = static_cast<uint64_t>(tag) << 32;
       if (s.live[b]) {
         const uint64_t* mine = ws_of(p, b) + region + 2 * t;
@@ -150,7 +168,7 @@ __device__ __forceinline__ bool rms_rows(const Params& p, Smem<M>& s, const Ctx&
       }
     });
     bool ok = true;
-    static_for<0, kMaxRows>([&](auto b) {
+    static_for<0, NR>([&](auto b) {
       lo[b] = static_cast<uint32_t>(xx[b]);
       hi[b] = static_cast<uint32_t>(yy[b]);
       ok = ok && static_cast<uint32_t>(xx[b] >> 32) == tag && static_cast<uint32_t>(yy[b] >> 32) == tag;
@@ -162,7 +180,7 @@ __device__ __forceinline__ bool rms_rows(const Params& p, Smem<M>& s, const Ctx&
     if (!done) look();
   });
   if (region < 0) {
-    static_for<0, kMaxRows>([&](auto b) {
+    static_for<0, NR>([&](auto b) {
       if (s.live[b]) {
         const uint64_t hw = ld_shared64(p.hidden + static_cast<size_t>(b) * M::H + t * 4);
         lo[b] = static_cast<uint32_t>(hw);
@@ -184,22 +202,28 @@ __device__ __forceinline__ bool rms_rows(const Params& p, Smem<M>& s, const Ctx&
       s.b.ctl[2] = 1;
     }
   }
-  float ss[kMaxRows];
-  static_for<0, kMaxRows>([&](auto b) {
+  float ss[NR];
+  static_for<0, NR>([&](auto b) {
     const float x0 = bf_lo(lo[b]), x1 = bf_hi(lo[b]), x2 = bf_lo(hi[b]), x3 = bf_hi(hi[b]);
     ss[b] = wave_sum(__builtin_fmaf(x3, x3, __builtin_fmaf(x2, x2, __builtin_fmaf(x1, x1, x0 * x0))));
   });
   const int lane = t & 63, wave = t >> 6;
   __syncthreads();
-  if (lane == 0) static_for<0, kMaxRows>([&](auto b) { s.red[0][b][wave] = ss[b]; });
+  if (lane == 0) static_for<0, NR>([&](auto b) { s.red[0][b][wave] = ss[b]; });
   __syncthreads();
-  static_for<0, kMaxRows>([&](auto b) {
-    if (b < B) {
-      float total = 0.f;
+  // A row's scale by one thread (the wave sums added in the batch-1 kernel's order): every thread adding up every row's
+  // sums and taking its root is thirty instructions per row and thread in front of every GEMV.
+  if (t < NR) {
+    float total = 0.f;
 #pragma unroll
-      for (int w = 0; w < kWaves; ++w) total += s.red[0][b][w];
-      const float mean = total / static_cast<float>(M::H);
-      const float rstd = 1.0f / sqrtf(mean + p.rms_norm_eps);
+    for (int w = 0; w < kWaves; ++w) total += s.red[0][t][w];
+    const float mean = total / static_cast<float>(M::H);
+    s.red[1][t][0] = 1.0f / sqrtf(mean + p.rms_norm_eps);
+  }
+  __syncthreads();
+  static_for<0, NR>([&](auto b) {
+    if (b < B) {
+      const float rstd = s.red[1][b][0];
       const float x0 = bf_lo(lo[b]), x1 = bf_hi(lo[b]), x2 = bf_lo(hi[b]), x3 = bf_hi(hi[b]);
       const uint32_t n01 = f2bf2(x0 * rstd, x1 * rstd), n23 = f2bf2(x2 * rstd, x3 * rstd);
       uint2 out;
@@ -213,15 +237,16 @@ __device__ __forceinline__ bool rms_rows(const Params& p, Smem<M>& s, const Ctx&
 }
 
 // The rows' activation vectors of H elements from s.x into registers (lane l: columns (j*64 + l)*8 .. +7 of chunk j).
-template <class M, int CH>
-__device__ __forceinline__ void load_x_rows(const Smem<M>& s, v4u (&x)[kMaxRows][CH], int lane) {
-  static_for<0, kMaxRows>([&](auto b) { load_x_from_lds(x[b], &s.x[b][0], lane); });
+template <class M, int CH, int NR>
+__device__ __forceinline__ void load_x_rows(const Smem<M>& s, v4u (&x)[NR][CH], int lane) {
+  static_for<0, NR>([&](auto b) { load_x_from_lds(x[b], &s.x[b][0], lane); });
 }
 
 // ===================================================================== 1 ==
 // [1, layer, tile_M, n_start, n_end, tile_M_g, tile_N_g]   the QKV rows of the instruction for every row of the batch
 template <class M>
 __device__ bool op_qkv(const Params& p, Smem<M>& s, const Ctx& c) {
+  constexpr int NR = RowsOf<M>::value;
   constexpr int CH = M::H / 512;
   const int layer = s.b.inst[1], nstart = s.b.inst[3], nend = s.b.inst[4], tile = s.b.inst[6];
   const int bph = p.qkv_blocks_per_head, B = p.batch;
@@ -239,12 +264,12 @@ __device__ bool op_qkv(const Params& p, Smem<M>& s, const Ctx& c) {
                            [&](auto k) { preload_range<decltype(k)::value, decltype(k)::value + 1>(nrows, src, buf); }))
     return false;
   QMK_ROWS_STAMP(0);
-  v4u x[kMaxRows][CH];
+  v4u x[NR][CH];
   load_x_rows<M, CH>(s, x, lane);
   stream<CH>(nrows, src, buf, [&](int r, const RowRegs<CH>& w) {
-    float sum[kMaxRows];
-    static_for<0, kMaxRows>([&](auto b) { sum[b] = wave_sum(dot_row(w, x[b])); });
-    if (lane == 0) static_for<0, kMaxRows>([&](auto b) { s.res[b][r] = sum[b]; });
+    float sum[NR];
+    static_for<0, NR>([&](auto b) { sum[b] = wave_sum(dot_row(w, x[b])); });
+    if (lane == 0) static_for<0, NR>([&](auto b) { s.res[b][r] = sum[b]; });
   });
   QMK_ROWS_STAMP(1);
   __syncthreads();
@@ -312,6 +337,7 @@ __device__ __forceinline__ bool wait_rows(const Params& p, Smem<M>& s, const Ctx
 // row), then hidden[b][r] = bf16(hidden[b][r] + bf16(W_o[r] . attn_out[b])) for the instruction's rows r.
 template <class M>
 __device__ bool op_oproj(const Params& p, Smem<M>& s, const Ctx& c) {
+  constexpr int NR = RowsOf<M>::value;
   constexpr int AW = M::AW, CH = AW / 512;
   static_assert(AW % (kThreads * 4) == 0, "whole 8-byte pieces per thread");
   const int layer = s.b.inst[1], nstart = s.b.inst[3], nend = s.b.inst[4], P = s.b.inst[5], tile = s.b.inst[7];
@@ -344,7 +370,7 @@ __device__ bool op_oproj(const Params& p, Smem<M>& s, const Ctx& c) {
     // The rows' attention outputs are complete in memory: the last split-KV arrival of every (row, KV head) merged its
     // group's partials and counted the group's heads on the row's word of the reduction row.  All rows in one trip.
     if (!wait_rows(p, s, c, layer, M::NQ)) return false;
-    constexpr int kPieces = kMaxRows * AW / (kThreads * 8);   // 16-byte pieces per thread
+    constexpr int kPieces = (NR * AW + kThreads * 8 - 1) / (kThreads * 8);   // 16-byte pieces per thread
     v4u piece[kPieces];
 #pragma unroll
     for (int k = 0; k < kPieces; ++k) {
@@ -427,7 +453,7 @@ __device__ bool op_oproj(const Params& p, Smem<M>& s, const Ctx& c) {
   QMK_ROWS_STAMP(0);
   // The activation pieces come from LDS as they are used (CH * rows of them do not fit the registers beside the rows).
   stream<CH>(nrows, src, buf, [&](int r, const RowRegs<CH>& w) {
-    static_for<0, kMaxRows>([&](auto b) {
+    static_for<0, NR>([&](auto b) {
       float a = 0.f;
 #pragma unroll
       for (int j = 0; j < CH; ++j) a = dot8(w.v[j], *reinterpret_cast<const v4u*>(&s.x[b][(j * kWaveSize + lane) * 8]), a);
@@ -801,6 +827,7 @@ __device__ bool op_routed_down_commit(const Params& p, Smem<M>& s, const Ctx& c)
 // silu_out[b] = bf16(bf16(silu(bf16(W_g y_b))) * bf16(W_u y_b))  (operations.py:265-282; the batch-1 op's arithmetic per row)
 template <class M>
 __device__ bool op_upgate(const Params& p, Smem<M>& s, const Ctx& c) {
+  constexpr int NR = RowsOf<M>::value;
   constexpr int CH = M::H / 512;
   const int bad = upgate_check<M>(p, s.b.inst);
   if (bad >= 0) return bad_operand(p, s, c, bad);
@@ -817,12 +844,12 @@ __device__ bool op_upgate(const Params& p, Smem<M>& s, const Ctx& c) {
                                    [&](auto k) { preload_range<decltype(k)::value, decltype(k)::value + 1>(nrows, src, buf); }))
     return false;
   QMK_ROWS_STAMP(0);
-  v4u x[kMaxRows][CH];
+  v4u x[NR][CH];
   load_x_rows<M, CH>(s, x, lane);
   stream<CH>(nrows, src, buf, [&](int e, const RowRegs<CH>& w) {
-    float sum[kMaxRows];
-    static_for<0, kMaxRows>([&](auto b) { sum[b] = wave_sum(dot_row(w, x[b])); });
-    if (lane == 0) static_for<0, kMaxRows>([&](auto b) { s.res[b][e] = sum[b]; });
+    float sum[NR];
+    static_for<0, NR>([&](auto b) { sum[b] = wave_sum(dot_row(w, x[b])); });
+    if (lane == 0) static_for<0, NR>([&](auto b) { s.res[b][e] = sum[b]; });
   });
   QMK_ROWS_STAMP(1);
   __syncthreads();
@@ -847,6 +874,7 @@ __device__ bool op_upgate(const Params& p, Smem<M>& s, const Ctx& c) {
 // hidden[b][r] = bf16(hidden[b][r] + bf16(W_d[r] . silu_out[b])) for every row of the batch  (operations.py:285-295)
 template <class M>
 __device__ bool op_down(const Params& p, Smem<M>& s, const Ctx& c) {
+  constexpr int NR = RowsOf<M>::value;
   constexpr int CH = 4;
   static_assert(M::F % (4 * kThreads) == 0 && M::F <= XWidth<M>::value, "whole unit pairs per thread; the vectors fit");
   const int layer = s.b.inst[1], nstart = s.b.inst[3], nend = s.b.inst[4], split = s.b.inst[5];
@@ -879,14 +907,14 @@ __device__ bool op_down(const Params& p, Smem<M>& s, const Ctx& c) {
   // they carry this layer's tag; what has been staged is not fetched again.
   {
     constexpr int kPairs = M::F / (4 * kThreads);
-    bool have[kMaxRows][kPairs];
-    static_for<0, kMaxRows>([&](auto b) {
+    bool have[NR][kPairs];
+    static_for<0, NR>([&](auto b) {
 #pragma unroll
       for (int k = 0; k < kPairs; ++k) have[b][k] = !s.live[b];
     });
     for (uint32_t polls = 0;; ++polls) {
       bool all = true;
-      static_for<0, kMaxRows>([&](auto b) {
+      static_for<0, NR>([&](auto b) {
         if (s.live[b]) {
           const uint64_t* mine = ws_of(p, b) + kWsSilu + 2 * c.tid;
           uint32_t* words = reinterpret_cast<uint32_t*>(&s.x[b][0]);
@@ -924,16 +952,16 @@ __device__ bool op_down(const Params& p, Smem<M>& s, const Ctx& c) {
   }
   __syncthreads();
   if (s.b.ctl[0]) return false;
-  float acc[kMaxRows];
-  static_for<0, kMaxRows>([&](auto b) { acc[b] = 0.f; });
+  float acc[NR];
+  static_for<0, NR>([&](auto b) { acc[b] = 0.f; });
   stream<CH>(n_elems, src, buf, [&](int e, const RowRegs<CH>& w) {
     const int seg = seg_of(e);
-    static_for<0, kMaxRows>([&](auto b) {
+    static_for<0, NR>([&](auto b) {
 #pragma unroll
       for (int j = 0; j < CH; ++j) acc[b] = dot8(w.v[j], *reinterpret_cast<const v4u*>(&s.x[b][seg * (512 * CH) + (j * kWaveSize + lane) * 8]), acc[b]);
     });
     if (seg == segs - 1) {
-      static_for<0, kMaxRows>([&](auto b) {
+      static_for<0, NR>([&](auto b) {
         const float sum = wave_sum(acc[b]);
         acc[b] = 0.f;
         if (lane == 0) s.res[b][row_of(e)] = sum;
@@ -954,6 +982,7 @@ __device__ bool op_down(const Params& p, Smem<M>& s, const Ctx& c) {
 // [7, start_block, end_block, tile_M_g, tile_N_g]     logits[b] = bf16(W_lm . rms(hidden[b])) for every row
 template <class M>
 __device__ bool op_lmhead(const Params& p, Smem<M>& s, const Ctx& c) {
+  constexpr int NR = RowsOf<M>::value;
   constexpr int CH = M::H / 512;
   const int bstart = s.b.inst[1], bend = s.b.inst[2], tile = s.b.inst[4];
   const int B = p.batch;
@@ -967,13 +996,13 @@ __device__ bool op_lmhead(const Params& p, Smem<M>& s, const Ctx& c) {
   RowRegs<CH> buf[kDepth];
   preload<CH>(nrows, src, buf);
   if (!rms_rows<M, 0>(p, s, c, kWsHiddenOut, tag_of(s.b.generation, p.num_layers - 1), p.lm_norm, [](auto) {})) return false;
-  v4u x[kMaxRows][CH];
+  v4u x[NR][CH];
   load_x_rows<M, CH>(s, x, lane);
   // Terminal op: nothing inside the launch reads the logits, so ordinary stores do.
   stream<CH>(nrows, src, buf, [&](int r, const RowRegs<CH>& w) {
-    float sum[kMaxRows];
-    static_for<0, kMaxRows>([&](auto b) { sum[b] = wave_sum(dot_row(w, x[b])); });
-    static_for<0, kMaxRows>([&](auto b) {
+    float sum[NR];
+    static_for<0, NR>([&](auto b) { sum[b] = wave_sum(dot_row(w, x[b])); });
+    static_for<0, NR>([&](auto b) {
       if (lane == b && b < B) p.logits[static_cast<size_t>(b) * p.vocab_size + rs + r] = f2bf(s.live[b] ? sum[b] : -1e9f);   // (a row that is not decoded: as the batch route leaves it)
     });
   });
