@@ -43,6 +43,8 @@ HBM_PEAK_GBPS = 8000.0
 MEASURED_TRAFFIC_OVER_ALGORITHMIC = 1.0069
 # The same for the batch route's kernel at batch 8 (profiles/decode_megakernel_batch_llama1b_hbm_counters.txt).
 MEASURED_TRAFFIC_OVER_ALGORITHMIC_BATCH8 = 1.0233
+# ... for the rows engine at 4 rows (profiles/decode_megakernel_rows_llama1b_batch4_hbm_counters.txt)
+MEASURED_TRAFFIC_OVER_ALGORITHMIC_ROWS4 = 1.0172
 # ... and for the MoE route's kernel (profiles/decode_megakernel_moe_qwen1p5_a2p7b_hbm_counters.txt).
 MEASURED_TRAFFIC_OVER_ALGORITHMIC_MOE = 1.0111
 # What `roofline.traffic` is: not a counter read in this process, but the algorithmic bytes of the timed launches times
@@ -189,6 +191,11 @@ def batch_decode(args) -> dict:
     # the same request with the whole loop (embedding rows, kernel, argmax, row state) as one HIP graph
     globs.k_cache.zero_(); globs.v_cache.zero_()
     graphed = decode_batch.decode(globs, prompts, new_tokens, mk=mk, use_graph=True)
+    traffic_ratio = None
+    if args.model == "llama-3.2-1b" and B == 8 and t["engine"] == "tiles":
+        traffic_ratio = MEASURED_TRAFFIC_OVER_ALGORITHMIC_BATCH8
+    elif args.model == "llama-3.2-1b" and B == 4 and t["engine"] == "rows":
+        traffic_ratio = MEASURED_TRAFFIC_OVER_ALGORITHMIC_ROWS4
     line = {
         "metric": "kernel_tok_s", "value": t["kernel_tok_s"], "unit": "tok/s", "n_gpus": 1, "steps": timed,
         "warmup": args.warmup, "ms_per_step": t["kernel_ms_per_step"], "higher_is_better": True, "scaling": "weak",
@@ -207,10 +214,9 @@ def batch_decode(args) -> dict:
         "roofline": {
             "bound": "hbm", "achieved": t["achieved_GBps"], "peak": HBM_PEAK_GBPS, "unit": "GB/s",
             "frac": t["achieved_GBps"] / HBM_PEAK_GBPS,
-            # the counter runs were made on the Llama shape at batch 8 only
-            "traffic": (MEASURED_TRAFFIC_OVER_ALGORITHMIC_BATCH8 * t["algorithmic_bytes"] / max(timed, 1)
-                        if B == 8 and args.model == "llama-3.2-1b" else None),
-            "traffic_source": TRAFFIC_SOURCE if B == 8 and args.model == "llama-3.2-1b" else None,
+            # the counter runs were made on the Llama shape at batch 8 (tiles engine) and batch 4 (rows engine) only
+            "traffic": (traffic_ratio * t["algorithmic_bytes"] / max(timed, 1) if traffic_ratio else None),
+            "traffic_source": TRAFFIC_SOURCE if traffic_ratio else None,
             "bytes_per_launch_avg": t["algorithmic_bytes"] / max(timed, 1), "kernel": kernel,
         },
     }
