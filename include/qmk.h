@@ -297,6 +297,14 @@ typedef struct QmkBatchArgs {
   void* qkv_raw;                   /* bf16 [B, (Hq+2Hkv)*D]  QKV before the per-head norm and RoPE */
   const void* q_norm_weights;      /* bf16 [L, D]  pair-interleaved like the q rows of qkv_weights */
   const void* k_norm_weights;      /* bf16 [L, D]                                 */
+
+  /* Column window (…/multi_batch/decode_kernel/mk.h:44-115: mk_step runs the one column inst_idx of the instruction
+   * tensor per launch, mk_step_loop all columns one launch after the other): the launch runs the columns
+   * [first_inst, first_inst + inst_count) of `instructions`; inst_count = 0 runs all of them (first_inst must then
+   * be 0).  A window that is not the whole tensor needs QMK_FLAG_KEEP_BARRIERS: the counters carry the step from one
+   * launch to the next and the caller zeroes them before the first column, as the reference's callers do. */
+  int32_t first_inst;
+  int32_t inst_count;
 } QmkBatchArgs;
 
 /* Launch one step of the batch route asynchronously on args->stream.  Positions outside the KV

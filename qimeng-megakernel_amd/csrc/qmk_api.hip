@@ -213,11 +213,13 @@ __global__ __launch_bounds__(kThreads, 1) void decode_megakernel_batch(const Par
   bool ok = s.ctl[0] == 0;
 
   const int32_t* queue = p.instructions + static_cast<size_t>(blockIdx.x) * p.num_insts * kInstWords;
-  int32_t word = (threadIdx.x < kInstWords && p.num_insts > 0) ? queue[threadIdx.x] : 0;
-  for (int i = 0; i < p.num_insts && ok; ++i) {
+  // A launch runs the columns [first_inst, end_inst) of the tensor: all of them, or the window of a column-by-column run
+  // (…/multi_batch/decode_kernel/mk.h:44-115: mk_step, mk_step_loop).
+  int32_t word = (threadIdx.x < kInstWords && p.first_inst < p.end_inst) ? queue[p.first_inst * kInstWords + threadIdx.x] : 0;
+  for (int i = p.first_inst; i < p.end_inst && ok; ++i) {
     if (threadIdx.x < kInstWords) {
       s.inst[threadIdx.x] = word;
-      word = (i + 1 < p.num_insts) ? queue[(i + 1) * kInstWords + threadIdx.x] : 0;
+      word = (i + 1 < p.end_inst) ? queue[(i + 1) * kInstWords + threadIdx.x] : 0;
     }
     __syncthreads();
     const int opcode = s.inst[0];
@@ -811,6 +813,12 @@ static int decode_step_batch(const QmkBatchArgs* a) {
     return QMK_ERR_SHAPE;
   if (a->flags & ~QMK_FLAG_KEEP_BARRIERS) return QMK_ERR_SHAPE;
   if (a->position_ids == nullptr && (a->pos_id < 0 || a->pos_id >= a->max_seq_len || a->pos_id >= a->rope_rows)) return QMK_ERR_POSITION;
+  // the column window: all columns, or a part of them with counters that outlive the launch
+  if (a->first_inst < 0 || a->inst_count < 0 || (a->inst_count == 0 && a->first_inst != 0) ||
+      static_cast<long>(a->first_inst) + a->inst_count > a->num_insts)
+    return QMK_ERR_SHAPE;
+  const bool whole = a->inst_count == 0 || (a->first_inst == 0 && a->inst_count == a->num_insts);
+  if (!whole && !(a->flags & QMK_FLAG_KEEP_BARRIERS)) return QMK_ERR_SHAPE;
 
   DeviceInfo* dev = nullptr;
   if (int rc = device_info(&dev); rc != QMK_OK) return rc;
@@ -843,6 +851,8 @@ static int decode_step_batch(const QmkBatchArgs* a) {
   p.timeline = a->timeline;
   p.status = dev->status;
   p.num_insts = a->num_insts;
+  p.first_inst = a->first_inst;
+  p.end_inst = whole ? a->num_insts : a->first_inst + a->inst_count;
   p.num_layers = a->num_layers;
   p.num_layer_barriers = a->num_layer_barriers;
   p.barrier_slots = a->barrier_slots;
@@ -1112,7 +1122,7 @@ static int decode_step_rows(const QmkRowsArgs* r) {
   if (a->num_queues < 1 || a->num_insts < 0 || a->num_layers < 1 || a->num_layers > 63 || a->num_layer_barriers < 8 ||
       a->barrier_slots < B * M::NQ || a->max_seq_len < 1 || a->max_splits < 1 || a->vocab_size < 1 || a->rope_rows < 1)
     return QMK_ERR_SHAPE;
-  if (a->flags != 0) return QMK_ERR_SHAPE;   // tagged hand-over and self-clearing counters always
+  if (a->flags != 0 || a->first_inst != 0 || a->inst_count != 0) return QMK_ERR_SHAPE;   // tagged hand-over and self-clearing counters always: whole steps only
   if (a->position_ids == nullptr && (a->pos_id < 0 || a->pos_id >= a->max_seq_len || a->pos_id >= a->rope_rows)) return QMK_ERR_POSITION;
   if (reinterpret_cast<uintptr_t>(r->workspace) % 128 != 0 || r->workspace_bytes < qmk_rows_workspace_bytes(B)) return QMK_ERR_SHAPE;
 

@@ -66,6 +66,7 @@ struct Params {
   uint64_t* timeline;
   int32_t* status;      // device status words: {code, workgroup, inst, opcode, operand}
   int32_t num_insts;
+  int32_t first_inst, end_inst;   // batch route: the columns [first_inst, end_inst) of the instruction tensor run in this launch
   int32_t num_layers;
   int32_t num_layer_barriers;
   int32_t barrier_slots;

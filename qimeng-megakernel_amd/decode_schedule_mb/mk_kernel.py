@@ -56,6 +56,7 @@ class QmkBatchArgs(ctypes.Structure):
         ("attn_rms_out", _P), ("mlp_rms_out", _P), ("lm_head_rms_out", _P),
         ("timeline", _P), ("stream", _P),
         ("qkv_raw", _P), ("q_norm_weights", _P), ("k_norm_weights", _P),
+        ("first_inst", _I), ("inst_count", _I),
     ]
 
 
@@ -118,6 +119,7 @@ class BatchMegaKernel:
         self._args.struct_size = ctypes.sizeof(QmkBatchArgs)
         self._bound_key: tuple | None = None
         self._barriers: torch.Tensor | None = None   # the counters of the bound launch: cleared by check() after an error
+        self._window = (0, 0)            # (first column, columns) of the launch; (0, 0): the whole tensor
 
     def error_string(self, code: int) -> str:
         return self._lib.qmk_error_string(int(code)).decode()
@@ -251,7 +253,30 @@ class BatchMegaKernel:
         a.oproj_blocks, a.down_blocks = hidden // self.residual_tiles[0], hidden // self.residual_tiles[1]
         a.timeline = self.timeline.data_ptr() if self.timeline is not None else None
         a.stream = torch.cuda.current_stream(tensors[1].device).cuda_stream
+        a.first_inst, a.inst_count = self._window
         self._launch(tensors[1].device)
+
+    # ---- one instruction column per launch (`…/multi_batch/decode_kernel/mk.h:44-115`) ----
+    def mk_step(self, *args: Any) -> None:
+        """The reference's ``mk_step``: the 22 tensors, then ``inst_idx``, then the arguments of ``mk`` from ``pos_id``
+        on; runs column ``inst_idx`` of the instruction tensor.  The counters carry the step from one column to the
+        next, so this object must have been made with ``reset_barriers=False`` and the caller zeroes them before
+        column 0, as the reference's callers do."""
+        if self.reset_barriers:
+            raise ValueError("mk_step needs counters that outlive a launch: get_mk(reset_barriers=False)")
+        inst_idx = int(args[22])
+        if not 0 <= inst_idx < int(args[0].shape[1]):
+            raise ValueError("mk_step: inst_idx out of range")
+        self._window = (inst_idx, 1)
+        try:
+            self(*args[:22], *args[23:])
+        finally:
+            self._window = (0, 0)
+
+    def mk_step_loop(self, *args: Any) -> None:
+        """The reference's ``mk_step_loop``: the arguments of ``mk``; every column in its own launch, one after the other."""
+        for inst_idx in range(int(args[0].shape[1])):
+            self.mk_step(*args[:22], inst_idx, *args[22:])
 
     def _launch(self, device: torch.device) -> None:
         rc = int(self._lib.qmk_decode_step_batch(ctypes.byref(self._args)))
@@ -284,8 +309,10 @@ def _mask_for_mk(t: torch.Tensor | None, device: torch.device) -> torch.Tensor |
     return t if t.is_contiguous() else t.contiguous()
 
 
-def call_mk(globs: Globals, mk: Any) -> None:
-    """One decode step with the current ``Globals`` (builds the request's instruction tensor on first use)."""
+def call_mk(globs: Globals, mk: Any, *, column_by_column: bool = False) -> None:
+    """One decode step with the current ``Globals`` (builds the request's instruction tensor on first use).
+    ``column_by_column``: through ``mk.mk_step_loop`` — one launch per instruction column, for bisecting a step; the
+    caller zeroes ``globs.barriers`` first and ``mk`` keeps the counters (``reset_barriers=False``)."""
     shape = LlamaConfig.shape()
     B = _batch_size(globs)
     device = globs.hidden_states.device
@@ -301,7 +328,8 @@ def call_mk(globs: Globals, mk: Any) -> None:
     active = _mask_for_mk(globs.active_mask, device) if globs.active_mask is not None and globs.active_mask.numel() == B else None
     if isinstance(mk, BatchMegaKernel):
         mk.residual_tiles = tuple(getattr(globs, "residual_tiles", (16, 16)))
-    mk(
+    launch = mk.mk_step_loop if column_by_column else mk
+    launch(
         globs.instructions,
         globs.hidden_states,
         globs.q_post_rope,

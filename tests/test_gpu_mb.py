@@ -6,6 +6,7 @@ the same instruction list runs on the sequential VM and through the C ABI; outpu
 rounding, the counters word for word; whole requests reproduce the tokens recorded from the reference.
 """
 import copy
+import ctypes
 import dataclasses
 import json
 
@@ -200,6 +201,39 @@ def test_whole_step_static_list(weights, make, workers):
     rel_close(gpu.logits, cpu.logits, rel=4e-2, name="logits")
     assert gpu.logits.float().argmax(-1).tolist() == cpu.logits.float().argmax(-1).tolist()
     assert torch.equal(gpu.attn_partial_valid.cpu(), cpu.attn_partial_valid)
+
+
+def test_step_run_column_by_column_equals_the_step_run_whole(weights):
+    """`mk_step` / `mk_step_loop` (…/multi_batch/decode_kernel/mk.h:44-115): the step's instruction tensor one column per
+    launch, the counters carrying the step from launch to launch, against the same tensor in one launch: every buffer and
+    every counter bit for bit; a window without lasting counters and a column outside the tensor are refused."""
+    sched = S.mi355x_scheduler(3, MB_SMALL)
+    results = []
+    for by_column in (False, True):
+        cpu, gpu = make_pair(weights, 3, (70, 3, 130), inactive=(1,))
+        mk = mk_kernel.get_mk(reset_barriers=False, spin_limit=1 << 18)
+        mk_kernel.tensorize_instructions(gpu, S.deal(sched.instruction_list(cpu), 64))   # 64 queues: a couple of dozen columns
+        gpu.residual_tiles = (sched.oproj_tile, sched.down_tile)
+        gpu.barriers.zero_()
+        mk_kernel.call_mk(gpu, mk, column_by_column=by_column)
+        mk.check()
+        results.append(gpu)
+    whole, cols = results
+    assert int(whole.instructions.shape[1]) > 10
+    for f in dataclasses.fields(whole):
+        a, b = getattr(whole, f.name), getattr(cols, f.name)
+        if isinstance(a, torch.Tensor):
+            assert torch.equal(a, b), f.name
+    assert int(whole.barriers.abs().sum()) > 0
+    clearing = mk_kernel.get_mk(spin_limit=1 << 18)
+    with pytest.raises(ValueError):
+        mk_kernel.call_mk(cols, clearing, column_by_column=True)
+    args = mk_kernel.QmkBatchArgs()
+    ctypes.memmove(ctypes.byref(args), ctypes.byref(mk._args), ctypes.sizeof(args))
+    args.first_inst, args.inst_count = int(whole.instructions.shape[1]) - 1, 2      # past the last column
+    assert mk._lib.qmk_decode_step_batch(ctypes.byref(args)) != 0
+    args.first_inst, args.inst_count, args.flags = 1, 1, 0                           # a window, but counters that are cleared
+    assert mk._lib.qmk_decode_step_batch(ctypes.byref(args)) != 0
 
 
 def test_request_of_the_reference_fixture(weights):
