@@ -135,6 +135,67 @@ def attention_stress(contexts=(4096, 16384, 32768)) -> dict:
     return out
 
 
+def phase_table(contexts=(64, 1000)) -> dict:
+    """Where a decode step of the headline configuration spends its time, by phase: one step per context on the full
+    Llama-3.2-1B shape with the KV cache filled with ~N(0,1) rows, timed by the kernel's own timeline records (100 MHz
+    clock).  A phase lasts from the end of the previous phase's last instruction to the end of its own last one, averaged
+    over layers 1..15; its bytes are the weights its instructions stream (attention: the K/V rows of the context); the
+    achieved rate is bytes / duration.  The records cost the kernel 1-2 % of a step."""
+    import numpy as np
+    import torch
+
+    from qimeng_megakernel_amd import synthetic
+    from qimeng_megakernel_amd.decode_schedule import mk_kernel
+    from qimeng_megakernel_amd.decode_schedule.instructions import scheduler as S
+    from qimeng_megakernel_amd.decode_schedule.model_config import LLAMA_3_2_1B, LlamaConfig
+
+    shape = LLAMA_3_2_1B
+    LlamaConfig.set_shape(shape)
+    H, F, L = shape.hidden_size, shape.intermediate_size, shape.num_hidden_layers
+    g = synthetic.build_synthetic_globals(shape, seed=0, kv_capacity=1032, device=torch.device("cuda:0"))
+    g.k_cache.normal_(); g.v_cache.normal_()
+    S.build(g)
+    mk = mk_kernel.get_mk()
+    nq, ni = g.instructions.shape[:2]
+    timeline = torch.zeros(nq, ni, 8, dtype=torch.int64, device="cuda:0")
+    order = [(1, "qkv"), (2, "attention"), (4, "o_proj"), (5, "up_gate"), (6, "down")]
+    out = {}
+    for ctx in contexts:
+        g.position_id = ctx
+        mk.timeline = None
+        for _ in range(3):
+            g.hidden_states.copy_(g.embed_tokens[5])
+            mk_kernel.call_mk(g, mk)
+        mk.timeline = timeline
+        g.hidden_states.copy_(g.embed_tokens[5])
+        mk_kernel.call_mk(g, mk)
+        torch.cuda.synchronize()
+        mk.check()
+        t = timeline.cpu().numpy().astype(np.int64)
+        op, layer = t[..., 3] & 0xFF, (t[..., 3] >> 8) & 0xFFFF
+        end_of = lambda o, l: t[..., 2][(op == o) & (layer == l)].max()
+        nbytes = {"qkv": shape.qkv_out_dim * H * 2, "attention": (ctx + 1) * shape.num_key_value_heads * shape.head_dim * 2 * 2,
+                  "o_proj": H * H * 2, "up_gate": 2 * F * H * 2, "down": H * F * 2}
+        rows = {}
+        for k, (o, name) in enumerate(order):
+            us = []
+            for l in range(1, L):
+                prev = end_of(6, l - 1) if k == 0 else end_of(order[k - 1][0], l)
+                us.append((end_of(o, l) - prev) / 100.0)
+            d = float(np.mean(us))
+            rows[name] = {"us": d, "MB": nbytes[name] / 1e6, "GBps": nbytes[name] / d / 1e3}
+        layer_us = float(np.mean([(end_of(6, l) - end_of(6, l - 1)) / 100.0 for l in range(1, L)]))
+        lm = op == 7
+        lm_us = float((t[..., 2][lm].max() - end_of(6, L - 1)) / 100.0)
+        lm_bytes = shape.vocab_size * H * 2
+        rows["lm_head"] = {"us": lm_us, "MB": lm_bytes / 1e6, "GBps": lm_bytes / lm_us / 1e3}
+        layer_bytes = sum(nbytes.values())
+        out[str(ctx)] = {"phases": rows, "layer_us": layer_us, "layer_MB": layer_bytes / 1e6, "layer_GBps": layer_bytes / layer_us / 1e3,
+                         "step_us_with_records": float((t[..., 2][op > 0].max() - t[..., 0][op > 0].min()) / 100.0)}
+    mk.timeline = None
+    return out
+
+
 def copy_calibration(device) -> None:
     """One 1 GiB device-to-device copy: a kernel of known traffic, for scaling rocprofv3's FETCH_SIZE / WRITE_SIZE."""
     import torch
@@ -499,6 +560,8 @@ def main() -> None:
     ap.add_argument("--rows-side-by-side", action="store_true",
                     help="MoE shapes with --batch B: one batch-1 launch per row and step (the only way for a shape with a shared "
                          "expert or more than 4 rows) instead of the B requests in one launch")
+    ap.add_argument("--phase-table", action="store_true",
+                    help="one decode step of the headline shape at contexts 64 and 1000 with timeline records: time, bytes and achieved GB/s per phase")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also run one 1 GiB device-to-device copy (a kernel of known traffic, for scaling rocprofv3 counters)")
     args = ap.parse_args()
@@ -521,6 +584,12 @@ def main() -> None:
     from qimeng_megakernel_amd.decode_schedule import mk_kernel
     from qimeng_megakernel_amd.decode_schedule.model_config import LLAMA_3_2_1B, QWEN3_1_7B, LlamaConfig
 
+    if args.phase_table:
+        res = phase_table()
+        print(json.dumps({"metric": "phase_GBps", "unit": "GB/s", "n_gpus": 1, "higher_is_better": True, "dtype": "bf16", "data": "synthetic",
+                          "config": {"workload": "Llama-3.2-1B shape, batch 1, one decode step per context, KV cache ~N(0,1); per-phase time from the kernel's timeline records"},
+                          "value": res[max(res, key=int)]["layer_GBps"], "contexts": res}))
+        return
     if args.attention_stress:
         res = attention_stress()
         print(json.dumps({"metric": "attention_phase_GBps", "unit": "GB/s", "n_gpus": 1, "higher_is_better": True,
