@@ -433,7 +433,7 @@ __global__ __launch_bounds__(kThreads, 1) void decode_megakernel_moe_rows(const 
           ok = rows::bad_operand(p, s, c, 6);
         } else {
           const Params pr = rows::row_view<M>(p, row, s.pos[row]);
-          [[clang::always_inline]] ok = op_attn_splitkv<M>(pr, s.b, c);
+          [[clang::always_inline]] ok = op_attn_splitkv<rows::Inner<M>>(pr, s.b, c);
         }
         break;
       }
@@ -446,7 +446,7 @@ __global__ __launch_bounds__(kThreads, 1) void decode_megakernel_moe_rows(const 
           ok = rows::bad_operand(p, s, c, 2);
         } else {
           const Params pr = rows::row_view<M>(p, row, s.pos[row]);
-          [[clang::always_inline]] ok = moe::op_topk<M>(pr, s.b, c);
+          [[clang::always_inline]] ok = moe::op_topk<rows::Inner<M>>(pr, s.b, c);
         }
         break;
       }
@@ -522,6 +522,9 @@ __global__ __launch_bounds__(kThreads, 1) void decode_megakernel_rows(const Para
   int32_t word = (threadIdx.x < kInstWords && p.num_insts > 0) ? queue[threadIdx.x] : 0;
   int32_t word1 = (threadIdx.x < kInstWords && p.num_insts > 1) ? queue[kInstWords + threadIdx.x] : 0;
   const int num_insts = p.num_insts;
+  Carried carry;
+  bool carried = false, parked = false, after_attention = false;
+  forget(carry);
   for (int i = 0; i < num_insts && ok; ++i) {
     if (threadIdx.x < kInstWords) {
       s.b.inst[threadIdx.x] = word;
@@ -540,27 +543,36 @@ __global__ __launch_bounds__(kThreads, 1) void decode_megakernel_rows(const Para
       for (int k = 0; k < 4; ++k) s.b.stamps[k] = t_start;
     }
     switch (opcode) {
-      case OP_NOOP: break;
-      case OP_RMS_QKV_ROPE: [[clang::always_inline]] ok = rows::op_qkv<M>(p, s, c); break;
+      // Only the O-projection hands rows to its successor: every other arm ends their life explicitly.
+      case OP_NOOP: forget(carry); break;
+      case OP_RMS_QKV_ROPE: [[clang::always_inline]] ok = rows::op_qkv<M>(p, s, c); forget(carry); break;
       case OP_ATTN_SPLITKV: {
         const int row = s.b.inst[6];   // the word behind the batch-1 operands
         if (row < 0 || row >= p.batch) {
           ok = rows::bad_operand(p, s, c, 6);
         } else if (s.live[row]) {
           const Params pr = rows::row_view<M>(p, row, s.pos[row]);
-          [[clang::always_inline]] ok = op_attn_splitkv<M>(pr, s.b, c);
+          [[clang::always_inline]] ok = op_attn_splitkv<rows::Inner<M>>(pr, s.b, c);
         }
+        forget(carry);
         break;
       }
-      case OP_OPROJ_RESIDUAL: [[clang::always_inline]] ok = rows::op_oproj<M>(p, s, c); break;
-      case OP_RMS_UPGATE_SILU: [[clang::always_inline]] ok = rows::op_upgate<M>(p, s, c); break;
-      case OP_DOWN_RESIDUAL: [[clang::always_inline]] ok = rows::op_down<M>(p, s, c); break;
-      case OP_RMS_LMHEAD: [[clang::always_inline]] ok = rows::op_lmhead<M>(p, s, c); break;
+      case OP_OPROJ_RESIDUAL:
+        carried = M::CARRY_AFTER_ATTENTION || !after_attention;
+        parked = !after_attention;   // a workgroup that has just run the attention has no wait to fill
+        [[clang::always_inline]] ok = rows::op_oproj<M, rows::AsksAhead<M>::value>(p, s, c, carry, carried, parked);
+        break;
+      case OP_RMS_UPGATE_SILU: [[clang::always_inline]] ok = rows::op_upgate<M>(p, s, c, carry, carried, parked); forget(carry); break;
+      case OP_DOWN_RESIDUAL: [[clang::always_inline]] ok = rows::op_down<M>(p, s, c); forget(carry); break;
+      case OP_RMS_LMHEAD: [[clang::always_inline]] ok = rows::op_lmhead<M>(p, s, c); forget(carry); break;
       default:
         if (threadIdx.x == 0) report_error(p, QMK_DEV_BAD_OPCODE, i, opcode, 0);
         ok = false;
+        forget(carry);
         break;
     }
+    if (opcode != OP_OPROJ_RESIDUAL) carried = parked = false;
+    after_attention = opcode == OP_ATTN_SPLITKV;
     if (p.timeline != nullptr && threadIdx.x == 0) {
       uint64_t* rec = p.timeline + (static_cast<size_t>(blockIdx.x) * p.num_insts + i) * 8;
       rec[0] = t_start;

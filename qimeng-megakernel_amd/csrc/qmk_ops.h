@@ -61,6 +61,15 @@ struct Qwen3_1p7B {
 };
 
 constexpr int kResSlots = 4096;
+// A geometry whose kernel parks no GEMV results in Smem::res says how few slots it needs (M::RES_SLOTS).
+template <class M, class = void>
+struct ResSlotsOf {
+  static constexpr int value = kResSlots;
+};
+template <class M>
+struct ResSlotsOf<M, std::void_t<decltype(M::RES_SLOTS)>> {
+  static constexpr int value = M::RES_SLOTS;
+};
 
 // Up/gate rows that the O-proj before them leaves in LDS: [row][wave][chunk][lane], 4 KiB per row and wave.
 template <int N>
@@ -81,7 +90,7 @@ struct Smem {
   int32_t wave_idx[kWaves];             // per-wave candidates on their way to best_val/best_idx
   float red[kWaves];
   alignas(16) u16 x[M::F];              // activation vector handed to the GEMV lanes
-  alignas(16) float res[kResSlots];     // per-row GEMV results awaiting the epilogue pass
+  alignas(16) float res[ResSlotsOf<M>::value];   // per-row GEMV results awaiting the epilogue pass
   float merge[kWaves][M::GQA][M::D + 4];  // attention state per wave and head: acc[D], m, l
   unsigned long long t_wait;            // timeline: when the last counter wait finished
   unsigned long long stamps[4];         // timeline: op-specific intermediate timestamps

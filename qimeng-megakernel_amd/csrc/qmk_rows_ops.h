@@ -46,15 +46,22 @@ struct XWidth<M, std::enable_if_t<M::DENSE_ROWS>> {
   static constexpr int value = M::F;
 };
 
-// The dense geometries as the rows kernel uses them: nothing carried or parked between instructions, and the number of
-// rows the ops are compiled for (ROWS: 2, 3 or 4 — a launch of B rows runs on the smallest that holds them, so that two
-// rows do not pay the norms, dot products and epilogues of four).
+// The dense geometries as the rows kernel uses them: the number of rows the ops are compiled for (ROWS: 2, 3 or 4 — a
+// launch of B rows runs on the smallest that holds them, so that two rows do not pay the norms, dot products and
+// epilogues of four), and, as in the batch-1 kernel, the rows of the up/gate instruction behind it that an O-projection
+// workgroup asks for while it waits through the attention phase and leaves in LDS (PARK_ROWS per wave; the batch-1 ops'
+// result slots are not used here and make room for them).  Llama shape, last 200 steps of the 1024-token request, ms per
+// step at 2 / 3 / 4 rows: none parked 0.645 / 0.690 / 0.738, two parked 0.629 / 0.677 / 0.736 (three at 2 rows: 0.625);
+// rows also carried in registers, as the batch-1 kernel does (CARRY_ROWS): one 0.638 / 0.677 / 0.739, two 0.677 at 2 rows
+// — beside the rows' activation vectors they cost more registers than they save time.  The Qwen3-1.7B shape, whose
+// O-projection waits less, gains nothing from either (1.053 against 1.049 ms at 2 rows) and parks none.
 template <int NR>
 struct Llama1BRowsN : Llama1B {
   static constexpr int CARRY_ROWS = 0;
-  static constexpr int PARK_ROWS = 0;
+  static constexpr int PARK_ROWS = 2;
   static constexpr bool DENSE_ROWS = true;
   static constexpr int ROWS = NR;
+  static constexpr int RES_SLOTS = 16;
 };
 template <int NR>
 struct Qwen3_1p7BRowsN : Qwen3_1p7B {
@@ -75,13 +82,34 @@ struct RowsOf<M, std::void_t<decltype(M::ROWS)>> {
   static constexpr int value = M::ROWS;
 };
 
+// The geometry as the batch-1 ops called from here see it: their LDS holds no parked rows (this kernel keeps its own).
+template <class M>
+struct Inner : M {
+  static constexpr int PARK_ROWS = 0;
+};
+template <class M, class = void>
+struct IsDense : std::false_type {};
+template <class M>
+struct IsDense<M, std::enable_if_t<M::DENSE_ROWS>> : std::true_type {};
+// A dense geometry whose O-projection asks for rows of the up/gate instruction behind it.
+template <class M>
+struct AsksAhead {
+  static constexpr bool value = IsDense<M>::value && (M::PARK_ROWS > 0 || M::CARRY_ROWS > 0);
+};
+// What only the MoE ops keep in LDS (absent from the dense kernels).
+struct RoutingScratch {
+  alignas(16) uint64_t key[kMaxRows][moe::kMaxExperts];  // ranking: {softmax numerator bits, ~expert} per row and expert (read two at a time)
+  float terms[kMaxRows][moe::kMaxTopK][kCommitRows];     // committing instruction: weighted rows per (row, slot)
+};
+struct NoRoutingScratch {};
+
 template <class M>
 struct Smem {
-  qmk::Smem<M> b;                       // what the batch-1 ops use when they run on a row's view (attention, top-k report)
+  qmk::Smem<Inner<M>> b;                // what the batch-1 ops use when they run on a row's view (attention, top-k report)
   int32_t pos[kMaxRows];                // position each row decodes
   int32_t live[kMaxRows];               // the row exists and is active: a row that is not is a hole every op steps over
   float red[2][kMaxRows][kWaves];
-  alignas(16) u16 x[kMaxRows][XWidth<M>::value];   // the rows' activation vectors
+  alignas(16) u16 x[AsksAhead<M>::value ? RowsOf<M>::value : kMaxRows][XWidth<M>::value];   // the rows' activation vectors (no more of them than the ops are compiled for where LDS is short)
   float res[kMaxRows][kRowRes];
   // the routing decision this workgroup last took (layer, -1: none yet), per row and slot, and the distinct experts
   int32_t route_layer;
@@ -91,11 +119,11 @@ struct Smem {
   float route_weight[kMaxRows][moe::kMaxTopK];
   int32_t list_expert[kMaxList];
   int32_t list_slot[kMaxList][kMaxRows];   // the slot in which row r picked list entry u, or -1
-  alignas(16) uint64_t key[kMaxRows][moe::kMaxExperts];  // ranking: {softmax numerator bits, ~expert} per row and expert (read two at a time)
   alignas(16) float picked_p[kMaxRows][moe::kMaxTopK];
   int32_t picked_e[kMaxRows][moe::kMaxTopK];
   int32_t wave_count[kWaves];
-  float terms[kMaxRows][moe::kMaxTopK][kCommitRows];   // committing instruction: weighted rows per (row, slot)
+  alignas(16) std::conditional_t<IsDense<M>::value, NoRoutingScratch, RoutingScratch> moe;
+  alignas(16) ParkedRows<IsDense<M>::value ? M::PARK_ROWS : 0> park;   // up/gate rows an O-projection leaves for the instruction behind it
 };
 
 #define QMK_ROWS_STAMP(k)                                                     \
@@ -335,8 +363,11 @@ __device__ __forceinline__ bool wait_rows(const Params& p, Smem<M>& s, const Ctx
 // [4, layer, tile_M, n_start, n_end, P, tile_M_g, tile_N_g]
 // Every row's split-KV partials merged by this workgroup itself (P per KV head: the batch-1 op's self-merge, row by
 // row), then hidden[b][r] = bf16(hidden[b][r] + bf16(W_o[r] . attn_out[b])) for the instruction's rows r.
-template <class M>
-__device__ bool op_oproj(const Params& p, Smem<M>& s, const Ctx& c) {
+// `carry` / `carried` / `parked` (dense kernels): as in the batch-1 op, the first rows of the up/gate instruction behind
+// this one are asked for in front of the wait for the attention phase — CARRY_ROWS per wave handed over in registers,
+// PARK_ROWS more left in LDS.
+template <class M, bool kCarry>
+__device__ bool op_oproj(const Params& p, Smem<M>& s, const Ctx& c, Carried& carry, bool& carried, bool& parked) {
   constexpr int NR = RowsOf<M>::value;
   constexpr int AW = M::AW, CH = AW / 512;
   static_assert(AW % (kThreads * 4) == 0, "whole 8-byte pieces per thread");
@@ -367,6 +398,37 @@ __device__ bool op_oproj(const Params& p, Smem<M>& s, const Ctx& c) {
     }
   }
   if (P == 0) {
+    if constexpr (kCarry) {
+      carried = carried && s.b.next[0] == OP_RMS_UPGATE_SILU && s.b.next[1] == layer && upgate_check<M>(p, s.b.next) < 0;
+      if (carried) {
+        const int un = s.b.next[3], utile = s.b.next[5 + un];
+        const int wave = c.tid >> 6;
+        static_assert(M::CARRY_ROWS <= kCarried, "the carried rows fit the up/gate ring");
+#pragma unroll
+        for (int k = 0; k < M::CARRY_ROWS; ++k) {
+          const int e = wave + (k + 1) * kWaves;
+          if (e < 2 * un * utile) load_row(carry.row[k], upgate_row<M>(p, s.b.next, layer, utile, e), lane);
+        }
+      } else {
+        forget(carry);
+      }
+      parked = parked && carried && M::PARK_ROWS > 0;
+      if constexpr (M::PARK_ROWS > 0) {
+        if (parked) {   // (the batch-1 kernel's park_upgate_rows on this kernel's LDS)
+          const int un = s.b.next[3], utile = s.b.next[5 + un], wave = c.tid >> 6;
+#pragma unroll 1
+          for (int k = 0; k < M::PARK_ROWS; ++k) {
+            const int e = wave + (kUpGateBuffers + k) * kWaves;
+            if (e < 2 * un * utile) {
+              RowRegs<4> r;
+              load_row(r, upgate_row<M>(p, s.b.next, layer, utile, e), lane);
+#pragma unroll
+              for (int j = 0; j < 4; ++j) s.park.v[k][wave][j][lane] = r.v[j];
+            }
+          }
+        }
+      }
+    }
     // The rows' attention outputs are complete in memory: the last split-KV arrival of every (row, KV head) merged its
     // group's partials and counted the group's heads on the row's word of the reduction row.  All rows in one trip.
     if (!wait_rows(p, s, c, layer, M::NQ)) return false;
@@ -384,6 +446,7 @@ __device__ bool op_oproj(const Params& p, Smem<M>& s, const Ctx& c) {
       if (at < B * AW) *reinterpret_cast<v4u*>(&s.x[at / AW][at % AW]) = piece[k];
     }
   } else {
+  if constexpr (kCarry) carried = parked = false;   // (this mode's merge needs the registers)
   // one arrival per split-KV instruction, on its row's word of the reduction row
   if (!wait_rows(p, s, c, layer, M::NKV * P)) return false;
   // Item t (one or two per thread) is dims 4*(t % (D/4)).. of head t / (D/4); four partials of every item per round,
@@ -448,6 +511,7 @@ __device__ bool op_oproj(const Params& p, Smem<M>& s, const Ctx& c) {
       }
     }
   }
+  if constexpr (kCarry) forget(carry);
   }
   __syncthreads();
   QMK_ROWS_STAMP(0);
@@ -469,6 +533,13 @@ __device__ bool op_oproj(const Params& p, Smem<M>& s, const Ctx& c) {
     st_shared32(p.hidden + static_cast<size_t>(my_b) * M::H + rs + 2 * my_pair, w);
   }
   return true;
+}
+
+template <class M>
+__device__ __forceinline__ bool op_oproj(const Params& p, Smem<M>& s, const Ctx& c) {
+  Carried none;
+  bool no = false, neither = false;
+  return op_oproj<M, false>(p, s, c, none, no, neither);
 }
 
 // ===================================================================== 8 ==
@@ -558,7 +629,7 @@ __device__ __forceinline__ bool route_rows(const Params& p, Smem<M>& s, const Ct
   // of {numerator bits (not negative: ordered like the floats), ~index}.  Padded to pairs with keys nobody goes behind.
   const int padded = (E + 1) & ~1;
   const uint64_t my_key = (static_cast<uint64_t>(__float_as_uint(x)) << 32) | (0xffffffffu - static_cast<uint32_t>(e));
-  if (r < B && e < padded) s.key[r][e] = live ? my_key : 0ull;
+  if (r < B && e < padded) s.moe.key[r][e] = live ? my_key : 0ull;
   const float wsum = wave_sum(x);
   if (lane == 0) s.red[1][0][wave] = wsum;
   __syncthreads();
@@ -569,7 +640,7 @@ __device__ __forceinline__ bool route_rows(const Params& p, Smem<M>& s, const Ct
   if (!ok) s.no_order = 1;   // a logit is NaN or infinite: no order to pick by
   if (live && ok) {
     typedef uint64_t u64x2 __attribute__((ext_vector_type(2)));
-    const u64x2* all = reinterpret_cast<const u64x2*>(&s.key[r][0]);
+    const u64x2* all = reinterpret_cast<const u64x2*>(&s.moe.key[r][0]);
     int before = 0;
 #pragma unroll 8
     for (int k = 0; k < padded; k += 2) {
@@ -788,7 +859,7 @@ __device__ bool op_routed_down_commit(const Params& p, Smem<M>& s, const Ctx& c)
         });
         if (lane == 0) {
           const float weight = s.route_weight[b][j];
-          static_for<0, kHalf>([&](auto i) { s.terms[b][j][h * kHalf + i] = round_bf16(v[i]) * weight; });
+          static_for<0, kHalf>([&](auto i) { s.moe.terms[b][j][h * kHalf + i] = round_bf16(v[i]) * weight; });
         }
       }
     });
@@ -806,8 +877,8 @@ __device__ bool op_routed_down_commit(const Params& p, Smem<M>& s, const Ctx& c)
     const int r = r0 + 2 * my_pair;
     float ro0 = 0.f, ro1 = 0.f;
     for (int j = 0; j < TK; ++j) {
-      ro0 += s.terms[my_b][j][2 * my_pair];
-      ro1 += s.terms[my_b][j][2 * my_pair + 1];
+      ro0 += s.moe.terms[my_b][j][2 * my_pair];
+      ro1 += s.moe.terms[my_b][j][2 * my_pair + 1];
     }
     const float h0 = (bf_lo(old) + ro0) + 0.f, h1 = (bf_hi(old) + ro1) + 0.f;   // opcode 14's expression without a shared term
     const uint32_t word = f2bf2(h0, h1);
@@ -818,7 +889,7 @@ __device__ bool op_routed_down_commit(const Params& p, Smem<M>& s, const Ctx& c)
   }
   // how many distinct experts the layer streamed: what the step's algorithmic bytes are counted from
   if (n0 == 0 && c.tid == 0 && p.distinct_out != nullptr) p.distinct_out[layer] = s.n_list;
-  __syncthreads();   // s.terms is read: the next instruction may write it
+  __syncthreads();   // s.moe.terms is read: the next instruction may write it
   return true;
 }
 
@@ -826,31 +897,66 @@ __device__ bool op_routed_down_commit(const Params& p, Smem<M>& s, const Ctx& c)
 // [5, layer, tile_M, n, block_0..block_{n-1}, tile_M_g, tile_N_g]   dense MLP, every row of the batch:
 // silu_out[b] = bf16(bf16(silu(bf16(W_g y_b))) * bf16(W_u y_b))  (operations.py:265-282; the batch-1 op's arithmetic per row)
 template <class M>
-__device__ bool op_upgate(const Params& p, Smem<M>& s, const Ctx& c) {
+__device__ bool op_upgate(const Params& p, Smem<M>& s, const Ctx& c, const Carried& carry, bool carried, bool parked) {
   constexpr int NR = RowsOf<M>::value;
   constexpr int CH = M::H / 512;
+  static_assert(CH == 4, "the carried rows are 4 KiB");
   const int bad = upgate_check<M>(p, s.b.inst);
   if (bad >= 0) return bad_operand(p, s, c, bad);
   const int layer = s.b.inst[1], n = s.b.inst[3], B = p.batch;
   const int tile = s.b.inst[5 + n];
-  const int lane = c.tid & 63;
+  const int lane = c.tid & 63, wave = c.tid >> 6;
   const int nout = n * tile, nrows = 2 * nout;     // streamed rows: element 2i = up row i, 2i+1 = gate row i
   if (nrows > kRowRes) return bad_operand(p, s, c, 3);
   auto row_of = [&](int i) { return s.b.inst[4 + i / tile] * tile + i % tile; };
   auto src = [&](int e) { return upgate_row<M>(p, s.b.inst, layer, tile, e); };
+  bool in_lds = false;   // the O-projection before this instruction has left rows kUpGateBuffers.. of every wave in LDS
+  if constexpr (M::PARK_ROWS > 0) in_lds = parked && carried;
   RowRegs<CH> buf[kUpGateBuffers];
+  if (carried) {  // ... and has asked for the elements of buffers 1..
+#pragma unroll
+    for (int k = 0; k < M::CARRY_ROWS; ++k) buf[k + 1] = carry.row[k];
+  }
   const uint32_t tag = tag_of(s.b.generation, layer);
-  if (!rms_rows<M, kUpGateBuffers>(p, s, c, kWsHiddenMid, tag, p.mlp_norm + static_cast<size_t>(layer) * M::H,
-                                   [&](auto k) { preload_range<decltype(k)::value, decltype(k)::value + 1>(nrows, src, buf); }))
+  if (!rms_rows<M, kUpGateBuffers>(p, s, c, kWsHiddenMid, tag, p.mlp_norm + static_cast<size_t>(layer) * M::H, [&](auto k) {
+        constexpr int kk = decltype(k)::value;
+        if (kk == 0 || kk > M::CARRY_ROWS || !carried) preload_range<kk, kk + 1>(nrows, src, buf);
+      }))
     return false;
   QMK_ROWS_STAMP(0);
   v4u x[NR][CH];
   load_x_rows<M, CH>(s, x, lane);
-  stream<CH>(nrows, src, buf, [&](int e, const RowRegs<CH>& w) {
+  auto use = [&](int e, const RowRegs<CH>& w) {
     float sum[NR];
     static_for<0, NR>([&](auto b) { sum[b] = wave_sum(dot_row(w, x[b])); });
     if (lane == 0) static_for<0, NR>([&](auto b) { s.res[b][e] = sum[b]; });
-  });
+  };
+  // The ring holds the wave's first kUpGateBuffers rows and, when they were parked, LDS the PARK_ROWS behind them: a ring
+  // buffer is refilled with the row behind those, and the parked rows are used while the refills are on their way.
+  int pk = 0;
+  if constexpr (M::PARK_ROWS > 0) pk = in_lds ? M::PARK_ROWS : 0;
+  const int shift = (kUpGateBuffers + pk) * kWaves;
+#pragma unroll
+  for (int k = 0; k < kUpGateBuffers; ++k) {
+    const int e = wave + k * kWaves;
+    if (e < nrows) {
+      use(e, buf[k]);
+      if (e + shift < nrows) load_row(buf[k], src(e + shift), lane);
+    }
+  }
+  if constexpr (M::PARK_ROWS > 0) {
+#pragma unroll 1
+    for (int k = 0; k < pk; ++k) {
+      const int e = wave + (kUpGateBuffers + k) * kWaves;
+      if (e < nrows) {
+        RowRegs<CH> r;
+#pragma unroll
+        for (int q = 0; q < CH; ++q) r.v[q] = s.park.v[k][wave][q][lane];
+        use(e, r);
+      }
+    }
+  }
+  stream<CH>(nrows - shift, [&](int e) { return src(e + shift); }, buf, [&](int e, const RowRegs<CH>& w) { use(e + shift, w); });
   QMK_ROWS_STAMP(1);
   __syncthreads();
   const int pairs = nout / 2;
