@@ -515,16 +515,27 @@ __device__ bool op_oproj(const Params& p, Smem<M>& s, const Ctx& c, Carried& car
   }
   __syncthreads();
   QMK_ROWS_STAMP(0);
-  // The activation pieces come from LDS as they are used (CH * rows of them do not fit the registers beside the rows).
-  stream<CH>(nrows, src, buf, [&](int r, const RowRegs<CH>& w) {
-    static_for<0, NR>([&](auto b) {
-      float a = 0.f;
-#pragma unroll
-      for (int j = 0; j < CH; ++j) a = dot8(w.v[j], *reinterpret_cast<const v4u*>(&s.x[b][(j * kWaveSize + lane) * 8]), a);
-      const float sum = wave_sum(a);
-      if (lane == 0) s.res[b][r] = sum;
+  if constexpr (CH <= 4) {
+    // (an attention output as wide as the hidden state: the rows' vectors fit the registers beside this op's two row buffers)
+    v4u x[NR][CH];
+    load_x_rows<M, CH>(s, x, lane);
+    stream<CH>(nrows, src, buf, [&](int r, const RowRegs<CH>& w) {
+      float sum[NR];
+      static_for<0, NR>([&](auto b) { sum[b] = wave_sum(dot_row(w, x[b])); });
+      if (lane == 0) static_for<0, NR>([&](auto b) { s.res[b][r] = sum[b]; });
     });
-  });
+  } else {
+    // The activation pieces come from LDS as they are used (CH * rows of them do not fit the registers beside the rows).
+    stream<CH>(nrows, src, buf, [&](int r, const RowRegs<CH>& w) {
+      static_for<0, NR>([&](auto b) {
+        float a = 0.f;
+#pragma unroll
+        for (int j = 0; j < CH; ++j) a = dot8(w.v[j], *reinterpret_cast<const v4u*>(&s.x[b][(j * kWaveSize + lane) * 8]), a);
+        const float sum = wave_sum(a);
+        if (lane == 0) s.res[b][r] = sum;
+      });
+    });
+  }
   QMK_ROWS_STAMP(1);
   __syncthreads();
   if (adds) {
