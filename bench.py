@@ -39,8 +39,11 @@ sys.path.insert(0, str(ROOT))
 HBM_PEAK_GBPS = 8000.0
 # HBM bytes one launch moves, from the two rocprofv3 --pmc runs (FETCH_SIZE, WRITE_SIZE; each scaled by
 # what the same counter reads for a 1 GiB copy) summarised in profiles/decode_megakernel_llama1b_hbm_counters.txt:
-# 1.0069 x the algorithmic bytes of the profiled launches.  Not measured in this process.
-MEASURED_TRAFFIC_OVER_ALGORITHMIC = 1.0069
+# 1.0082 x the algorithmic bytes over the launches this file times by default with `--steps 20` (contexts 1012..1031);
+# 1.0068 over a 64-token request.  Not measured in this process.
+MEASURED_TRAFFIC_OVER_ALGORITHMIC = 1.0082
+# The same kernel template on the Qwen3-1.7B shape, contexts 1020..1039 (profiles/decode_megakernel_qwen3_1p7b_hbm_counters.txt).
+MEASURED_TRAFFIC_OVER_ALGORITHMIC_QWEN3_1P7B = 1.0139
 # The same for the batch route's kernel at batch 8 (profiles/decode_megakernel_batch_llama1b_hbm_counters.txt).
 MEASURED_TRAFFIC_OVER_ALGORITHMIC_BATCH8 = 1.0233
 # ... for the rows engine at 4 rows (profiles/decode_megakernel_rows_llama1b_batch4_hbm_counters.txt)
@@ -704,10 +707,9 @@ def main() -> None:
             "peak": HBM_PEAK_GBPS,
             "unit": "GB/s",
             "frac": achieved / HBM_PEAK_GBPS,
-            # the counter runs were made on the Llama-shaped kernel only
-            "traffic": (MEASURED_TRAFFIC_OVER_ALGORITHMIC * t["algorithmic_bytes"] / max(timed, 1)
-                        if args.model == "llama-3.2-1b" else None),
-            "traffic_source": TRAFFIC_SOURCE if args.model == "llama-3.2-1b" else None,
+            "traffic": ((MEASURED_TRAFFIC_OVER_ALGORITHMIC if args.model == "llama-3.2-1b" else MEASURED_TRAFFIC_OVER_ALGORITHMIC_QWEN3_1P7B)
+                        * t["algorithmic_bytes"] / max(timed, 1)),
+            "traffic_source": TRAFFIC_SOURCE,
             "bytes_per_launch_avg": t["algorithmic_bytes"] / max(timed, 1),
             "kernel": "decode_megakernel<Llama1B>" if args.model == "llama-3.2-1b" else "decode_megakernel<Qwen3_1p7B>",
         },
