@@ -232,12 +232,16 @@ int qmk_decode_step_static(const QmkArgs* args);
  * order of mk(...) (…/multi_batch/decode_kernel/mk.h:9-42).  Two layer geometries are compiled for this
  * route: Llama-3.2-1B, and Qwen3-1.7B with the Qwen3 op set (opcode 2 leaves the raw QKV rows, opcode 3
  * applies the per-head RMSNorm and RoPE to its row's q and k and appends the cache row).
- * Flags: QMK_FLAG_KEEP_BARRIERS only.
+ * Flags: QMK_FLAG_KEEP_BARRIERS, and QMK_FLAG_XCD_COUNTERS in this route's form: the blocks of the
+ * O-projection, the up/gate and the down projection (counter rows 4, 6, 7) are counted on words 32, 64 .. 256 of
+ * their row (the sender's workgroup index modulo 8 chooses: one 128-byte line per XCD) instead of on word 0, and
+ * the instructions that wait for them add the eight words up; needs barrier_slots >= 288.  Hundreds of arrivals
+ * from eight XCDs on one line are seen 2 us later than on eight.  No counterpart in the reference.
  */
 typedef struct QmkBatchArgs {
   uint32_t struct_size;            /* = sizeof(QmkBatchArgs)                      */
   uint32_t model;                  /* QMK_MODEL_LLAMA_3_2_1B or QMK_MODEL_QWEN3_1_7B */
-  uint32_t flags;                  /* 0 or QMK_FLAG_KEEP_BARRIERS                 */
+  uint32_t flags;                  /* QMK_FLAG_KEEP_BARRIERS, QMK_FLAG_XCD_COUNTERS */
   uint32_t spin_limit;             /* counter polls before QMK_DEV_WAIT_TIMEOUT; 0 = default */
 
   const int32_t* instructions;     /* int32 [num_queues, num_insts, 32]           */

@@ -126,6 +126,47 @@ __device__ __forceinline__ void publish_after_stores(const Params& p, const Ctx&
   if (c.tid == 0) publish(counter_ptr(p, layer, row, slot), amount);
 }
 
+// ---- the all-to-all edges' arrivals on eight lines (QMK_FLAG_XCD_COUNTERS) ----
+// The O-projection, the up/gate and the down projection each count 128..512 blocks on word 0 of their counter row, and
+// every one of those arrivals is a read-modify-write of the same line from another XCD: the last of them is seen
+// microseconds after it was sent.  With the flag an arrival goes to the sub-counter of the sender's XCD (workgroup % 8:
+// word 32 * (1 + xcd) of the same row, a line of its own; the rows have no other user beyond word 0), and a waiting
+// workgroup's first eight lanes read the eight words and add them up.
+constexpr int kSpread = kXcds;
+__device__ __forceinline__ bool spread_counters(const Params& p) { return (p.flags & QMK_FLAG_XCD_COUNTERS) != 0; }
+__device__ __forceinline__ void publish_edge_after_stores(const Params& p, const Ctx& c, int layer, int row, int amount) {
+  publish_after_stores(p, c, layer, row, spread_counters(p) ? kLineInts * (1 + static_cast<int>(blockIdx.x & (kSpread - 1))) : 0, amount);
+}
+template <class S>
+__device__ __forceinline__ bool wait_edge(const Params& p, S& s, const Ctx& c, int layer, int row, int expected) {
+  if (!spread_counters(p)) return wait_counter(p, s, c, layer, row, expected);
+  if (c.tid < kSpread) {
+    const int32_t* mine = counter_ptr(p, layer, row, kLineInts * (1 + c.tid));
+    uint32_t polls = 0;
+    while (true) {
+      int v = __hip_atomic_load(mine, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      v += __shfl_xor(v, 1, kSpread);
+      v += __shfl_xor(v, 2, kSpread);
+      v += __shfl_xor(v, 4, kSpread);
+      if (v >= expected) break;
+      if (++polls > p.spin_limit) {   // the same for all eight lanes
+        if (c.tid == 0) {
+          s.ctl[0] = 1;
+          report_error(p, QMK_DEV_WAIT_TIMEOUT, c.inst_idx, c.opcode, 0);
+        }
+        break;
+      }
+      __builtin_amdgcn_s_sleep(2);
+    }
+  }
+  if (p.timeline != nullptr && c.tid == 0) {
+    s.t_wait = wall_clock64();
+    s.ctl[2] = 1;
+  }
+  __syncthreads();
+  return s.ctl[0] == 0;
+}
+
 // ================================================================ 1, 6, 9 ==
 // [op, layer, batch_size, -, -, -, batch_row]   (9: [op, batch_size, -, -, -, -, batch_row])
 // dst[row] = RMSNorm(hidden[row]) for an active row, zeros otherwise   (python_vm.py:139-160, 614-634, 668-690)
@@ -151,7 +192,7 @@ __device__ bool op_rms_row(const Params& p, Smem<M>& s, const Ctx& c) {
   }
   const uint2 wv = *reinterpret_cast<const uint2*>(weight + c.tid * 4);
   const int produced = wait_row == ROW_OPROJ ? p.oproj_blocks : p.down_arrivals;   // blocks of the projection that completes the rows
-  if (wait_layer >= 0 && !wait_counter(p, s, c, wait_layer, wait_row, produced)) return false;
+  if (wait_layer >= 0 && !wait_edge(p, s, c, wait_layer, wait_row, produced)) return false;
   uint32_t lo = 0, hi = 0;
   if (s.active[row]) {
     const uint64_t hw = ld_shared64(p.hidden + static_cast<size_t>(row) * M::H + c.tid * 4);
@@ -784,7 +825,7 @@ __device__ bool op_oproj(const Params& p, Smem<M>& s, const Ctx& c) {
       },
       R);
   if (!ok) return false;
-  publish_after_stores(p, c, layer, ROW_OPROJ, 0, n1 - n0);
+  publish_edge_after_stores(p, c, layer, ROW_OPROJ, n1 - n0);
   return true;
 }
 
@@ -819,7 +860,7 @@ __device__ bool op_upgate(const Params& p, Smem<M>& s, const Ctx& c) {
         st_shared32(p.silu_out + static_cast<size_t>(b) * M::F + s.inst[5 + j] * kTile + 2 * rp, word);
       });
   if (!ok) return false;
-  publish_after_stores(p, c, layer, ROW_UPGATE, 0, n);
+  publish_edge_after_stores(p, c, layer, ROW_UPGATE, n);
   return true;
 }
 
@@ -862,7 +903,7 @@ __device__ bool op_down(const Params& p, Smem<M>& s, const Ctx& c) {
       for (int j = 0; j < kSegChunks; ++j) s.seg_park[wave][j][lane] = a3.a[j];
     }
   }
-  if (!wait_counter(p, s, c, layer, ROW_UPGATE, M::F / kTile)) return false;
+  if (!wait_edge(p, s, c, layer, ROW_UPGATE, M::F / kTile)) return false;
   u16* const mine = p.hidden + static_cast<size_t>(c.tid & 15) * M::H + 2 * (c.tid >> 4);
   const bool adds = c.tid < 8 * R && (c.tid & 15) < B && s.active[c.tid & 15];
   int parity = 0;
@@ -902,7 +943,7 @@ __device__ bool op_down(const Params& p, Smem<M>& s, const Ctx& c) {
     QMK_MB_STAMP(2);
     parity ^= 1;
   }
-  publish_after_stores(p, c, layer, ROW_DOWN, 0, n1 - n0);
+  publish_edge_after_stores(p, c, layer, ROW_DOWN, n1 - n0);
   return true;
 }
 

@@ -107,11 +107,18 @@ class BatchMegaKernel:
 
     ``reset_barriers``: the kernel clears the counters when it retires (default) or leaves their
     final values in place like the reference kernel, whose host loop zeroes them before every step.
+    ``xcd_counters``: the blocks of the O-projection, the up/gate and the down projection are counted on eight
+    sub-counters (words 32, 64, .. 256 of their counter row, one 128-byte line per XCD) instead of on word 0, where
+    hundreds of arrivals from eight XCDs queue on one line.  Taken when the kernel clears the counters itself and
+    a row has the 288 words (batches of 6 and more); a launch that keeps the counters leaves the reference's words.
     """
 
-    def __init__(self, lib: ctypes.CDLL, *, reset_barriers: bool = True, spin_limit: int = 0):
+    XCD_COUNTER_WORDS = 32 * 9
+
+    def __init__(self, lib: ctypes.CDLL, *, reset_barriers: bool = True, spin_limit: int = 0, xcd_counters: bool = True):
         self._lib = lib
         self.reset_barriers = reset_barriers
+        self.xcd_counters = xcd_counters
         self.spin_limit = int(spin_limit)
         self.residual_tiles = (16, 16)   # rows per O-proj / down-projection block of the stream (set per call by call_mk)
         self.timeline: torch.Tensor | None = None
@@ -140,7 +147,8 @@ class BatchMegaKernel:
 
     def with_options(self, **kw: Any) -> "BatchMegaKernel":
         other = BatchMegaKernel(self._lib, reset_barriers=kw.pop("reset_barriers", self.reset_barriers),
-                                spin_limit=kw.pop("spin_limit", self.spin_limit))
+                                spin_limit=kw.pop("spin_limit", self.spin_limit),
+                                xcd_counters=kw.pop("xcd_counters", self.xcd_counters))
         if kw:
             raise TypeError(f"unknown options {sorted(kw)}")
         return other
@@ -248,6 +256,8 @@ class BatchMegaKernel:
         a.attn_scale = float(attn_scale)
         a.rms_norm_eps = float(rms_norm_eps)
         a.flags = 0 if self.reset_barriers else _single.QMK_FLAG_KEEP_BARRIERS
+        if self.xcd_counters and self.reset_barriers and a.barrier_slots >= self.XCD_COUNTER_WORDS:
+            a.flags |= _single.QMK_FLAG_XCD_COUNTERS
         a.spin_limit = self.spin_limit
         hidden = LlamaConfig.shape().hidden_size
         a.oproj_blocks, a.down_blocks = hidden // self.residual_tiles[0], hidden // self.residual_tiles[1]
@@ -284,7 +294,7 @@ class BatchMegaKernel:
             raise RuntimeError(f"qmk_decode_step_batch failed with {rc}: {self.error_string(rc)}")
 
 
-def get_mk(mk_dir: Path | None = None, *, reset_barriers: bool = True, spin_limit: int = 0) -> BatchMegaKernel:
+def get_mk(mk_dir: Path | None = None, *, reset_barriers: bool = True, spin_limit: int = 0, xcd_counters: bool = True) -> BatchMegaKernel:
     """Return the ``mk`` callable of the batch route bound to the prebuilt library in ``mk_dir``."""
     root = (_single._default_mk_dir() if mk_dir is None else Path(mk_dir)).resolve()
     lib = _single._LIB_CACHE.get(root)
@@ -295,7 +305,7 @@ def get_mk(mk_dir: Path | None = None, *, reset_barriers: bool = True, spin_limi
         raise ImportError(f"{root / 'libqmk_hip.so'} does not export qmk_decode_step_batch")
     lib.qmk_decode_step_batch.argtypes = [ctypes.POINTER(QmkBatchArgs)]
     lib.qmk_decode_step_batch.restype = ctypes.c_int
-    return BatchMegaKernel(lib, reset_barriers=reset_barriers, spin_limit=spin_limit)
+    return BatchMegaKernel(lib, reset_barriers=reset_barriers, spin_limit=spin_limit, xcd_counters=xcd_counters)
 
 
 def _mask_for_mk(t: torch.Tensor | None, device: torch.device) -> torch.Tensor | None:

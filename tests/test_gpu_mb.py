@@ -236,6 +236,43 @@ def test_step_run_column_by_column_equals_the_step_run_whole(weights):
     assert mk._lib.qmk_decode_step_batch(ctypes.byref(args)) != 0
 
 
+def test_arrivals_counted_per_xcd_change_no_result(weights):
+    """The blocks of the O-projection, the up/gate and the down projection counted on eight sub-counters of their rows
+    (QMK_FLAG_XCD_COUNTERS; taken by default when the kernel clears the counters and a row has 288 words) against the
+    same step counted on word 0: every buffer bit for bit, the counters cleared; a launch that keeps the counters
+    stays with the reference's words, and rows too short for the sub-counters are refused."""
+    rows = 8
+    sched = S.mi355x_scheduler(rows, MB_SMALL)
+    results = []
+    for per_xcd in (False, True):
+        cpu, gpu = make_pair(weights, rows, (70, 3, 130, 64, 0, 17, 150, 99), inactive=(2,))
+        mk = mk_kernel.get_mk(spin_limit=1 << 18, xcd_counters=per_xcd)
+        mk_kernel.tensorize_instructions(gpu, sched.runtime_queues(int(gpu.k_cache.shape[2])))
+        gpu.residual_tiles = (sched.oproj_tile, sched.down_tile)
+        mk_kernel.call_mk(gpu, mk)
+        mk.check()
+        assert bool(mk._args.flags & 2) == per_xcd
+        assert int(gpu.barriers.abs().sum()) == 0
+        results.append((gpu, mk))
+    (plain, _), (spread, mk) = results
+    for f in dataclasses.fields(plain):
+        a, b = getattr(plain, f.name), getattr(spread, f.name)
+        if isinstance(a, torch.Tensor):
+            assert torch.equal(a, b), f.name
+    keeping = mk_kernel.get_mk(reset_barriers=False, spin_limit=1 << 18)
+    spread.barriers.zero_()
+    mk_kernel.call_mk(spread, keeping)
+    keeping.check()
+    assert keeping._args.flags == 1
+    blocks = MB_SMALL.intermediate_size // 16
+    assert spread.barriers[:, 6, 0].tolist() == [blocks] * MB_SMALL.num_hidden_layers and int(spread.barriers[:, 6, 1:].abs().sum()) == 0
+    args = mk_kernel.QmkBatchArgs()
+    ctypes.memmove(ctypes.byref(args), ctypes.byref(mk._args), ctypes.sizeof(args))
+    assert args.flags & 2 and args.barrier_slots >= 288
+    args.barrier_slots = 287
+    assert mk._lib.qmk_decode_step_batch(ctypes.byref(args)) != 0
+
+
 def test_request_of_the_reference_fixture(weights):
     """Six steps of the recorded request through call_mk with one instruction tensor for the whole request
     and self-clearing counters: tokens, row state and the recorded top-4 logits."""

@@ -112,20 +112,43 @@ def test_runtime_template_is_made_of_whole_rounds():
     assert all(i.valid_partials == -1 and i.is_active == -1 for i in flat if i.opcode() == 4)
 
 
-def test_up_gate_blocks_follow_the_o_proj_round():
-    """MI355X template: the workers that ran an O-proj block get one up/gate block less than an even deal, the idle ones
-    share the rest; the reference's deal stays even."""
+def test_up_gate_blocks_stay_off_the_down_projection_workers():
+    """MI355X template: the workers of the down projection's round get no up/gate block, the others share all of
+    them; the reference's deal stays even."""
     sched = S.mi355x_scheduler(8, MB_FULL)
     mine = sched.upgate_skewed(0)
     counts = [len(i.tile_N_block_idxs) if i.opcode() == 7 else 0 for i in mine]
-    busy = len(sched.oproj(0))
+    busy = len(sched.downproj(0))
     assert len(mine) == sched.workers and busy == 128
-    assert set(counts[:busy]) == {1} and set(counts[busy:]) == {3} and sum(counts) == MB_FULL.intermediate_size // 16
+    assert set(counts[:busy]) == {0} and set(counts[busy:]) == {4} and sum(counts) == MB_FULL.intermediate_size // 16
     flat = [b for i in mine if i.opcode() == 7 for b in i.tile_N_block_idxs]
     assert flat == list(range(MB_FULL.intermediate_size // 16))
     even = [len(i.tile_N_block_idxs) for i in S.reference_scheduler(8, MB_FULL).upgate(0)]
     assert max(even) - min(even) <= 1
     assert not S.mi355x_scheduler(8, MB_FULL, skew_upgate=False).skew_upgate
+    # 8-row blocks put a down-projection block on every worker: nobody is left to take the up/gate blocks alone
+    assert [i.opcode() for i in S.mi355x_scheduler(8, MB_FULL, residual_tile=8).upgate_skewed(0)] == [7] * 256
+
+
+def test_o_proj_blocks_go_beside_the_attention_workers():
+    """MI355X template: where the split-KV round leaves at least half of the down-projection workers free, the
+    O-projection's blocks go to those, two to a worker; otherwise (and in the reference's template) one block per
+    worker from worker 0 on."""
+    sched = S.mi355x_scheduler(8, MB_FULL)
+    p = sched.partials_for_capacity(1024)
+    slices = len(sched.attention_split_kv(0, p))
+    assert slices == 64
+    placed = sched.oproj_round(0, p)
+    assert len(placed) == sched.workers
+    assert all(i.opcode() == 0 for i in placed[:slices] + placed[128:])
+    spans = [(i.tile_N_start_idx, i.tile_N_end_idx) for i in placed[slices:128]]
+    assert spans == [(2 * k, 2 * k + 2) for k in range(64)]
+    full = S.mi355x_scheduler(16, MB_FULL)   # 128 slices: no down-projection worker is free
+    plain = full.oproj_round(0, full.partials_for_capacity(1024))
+    assert [i.opcode() for i in plain] == [5] * 128 + [0] * 128
+    assert [(i.tile_N_start_idx, i.tile_N_end_idx) for i in plain[:128]] == [(k, k + 1) for k in range(128)]
+    ref = S.reference_scheduler(8, MB_FULL)
+    assert ref.oproj_round(0, 4)[: len(ref.oproj(0))] == ref.oproj(0)
 
 
 @pytest.mark.parametrize("make,rows", [(S.reference_scheduler, 3), (S.mi355x_scheduler, 8), (S.mi355x_scheduler, 16)])
