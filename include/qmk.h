@@ -112,7 +112,9 @@ enum {
                                       up/gate -> down, down -> next QKV / LM head) count
                                       arrivals on eight sub-counters, one 128-byte line per
                                       XCD, kept in rows 10.. of each layer of `barriers`;
-                                      consumers poll the eight lines and sum them.  Needs
+                                      consumers poll the eight lines and sum them (the attention
+                                      edge: every arrival goes to all eight lines and a consumer
+                                      polls the line of its own XCD).  Needs
                                       num_layer_barriers * barrier_slots >= 10 * barrier_slots
                                       + 2048 ints (32 counter lines, then 32 flag lines), a 128-byte aligned `barriers` with a layer
                                       stride that is a multiple of 128 bytes, and a schedule

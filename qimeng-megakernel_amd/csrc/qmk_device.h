@@ -442,14 +442,12 @@ __device__ __forceinline__ bool poll_sub_counters(const Params& p, int layer, in
 // itself after kFollowerPolls tries, and raises the flag for its neighbours too.
 constexpr uint32_t kFollowerPolls = 256;
 
-// `relay` = false: every workgroup polls the sub-counters itself (an edge with few producers, where
-// the relay through the leader's flag costs more than the polling disturbs).
-__device__ __forceinline__ bool wait_edge_xcd(const Params& p, int layer, int row, int expected, uint32_t limit, bool relay = true) {
+__device__ __forceinline__ bool wait_edge_xcd(const Params& p, int layer, int row, int expected, uint32_t limit) {
   const int xcd = blockIdx.x & (kXcds - 1);
   // The flag has a line of its own (second half of the region): only workgroups of this XCD ever
   // touch it, so it lives in this XCD's L2 and polling it stays off the fabric.
   int32_t* flag = sub_counter(p, layer, row, xcd) + kHierEdges * kXcds * kLineInts;
-  const bool leader = blockIdx.x < kXcds || gridDim.x < 2 * kXcds || !relay;
+  const bool leader = blockIdx.x < kXcds || gridDim.x < 2 * kXcds;
   bool ready = false;
   if (!leader) {
     for (uint32_t k = 0; k < kFollowerPolls; ++k) {

@@ -186,7 +186,8 @@ def test_whole_layer_and_counters(state, which):
 
 def test_xcd_sub_counters(state):
     """With room in `barriers`, the all-to-all edges count on eight per-XCD lines: same results,
-    rows 3..5 of the protocol untouched, the sub-counters of an edge summing to its final count."""
+    rows 3..5 of the protocol untouched, the sub-counters of a GEMV edge summing to its final count, each of the
+    attention edge's holding all of it."""
     shape, cpu, gpu = state
     sched = _sched(shape, "mi355x", P=4)
     sync_state(cpu, gpu)
@@ -200,7 +201,9 @@ def test_xcd_sub_counters(state):
     for layer in range(shape.num_hidden_layers):
         flat = b[layer, 10:54].reshape(-1)
         region, flags = flat[: 4 * 8 * 32].reshape(4, 8, 32), flat[4 * 8 * 32 : 8 * 8 * 32].reshape(4, 8, 32)
-        assert region[:, :, 0].sum(dim=1).tolist() == [shape.num_key_value_heads * sched.num_partials, opb, ubk, dwn]
+        # the GEMV edges: an arrival on the sender's XCD's line; the attention edge: every arrival on all eight lines
+        assert region[1:, :, 0].sum(dim=1).tolist() == [opb, ubk, dwn]
+        assert region[0, :, 0].tolist() == [shape.num_key_value_heads * sched.num_partials] * 8
         assert (region[1:, :, 0] > 0).all()                     # every XCD took part in the GEMV edges
         assert int(region[:, :, 1:].abs().sum()) == 0
         assert set(flags[:, :, 0].reshape(-1).tolist()) <= {0, 1}   # the XCD's ready flag, on a line of its own
