@@ -101,8 +101,13 @@ enum {
                                       a schedule whose down projection is not split along K; not
                                       combinable with QMK_FLAG_KEEP_BARRIERS.  The caller's buffers
                                       receive the same values as without the flag; counter rows 0,
-                                      3, 4 and 5 stay zero.  (The split-KV partials stay on
-                                      counters.)                                                  */
+                                      3, 4 and 5 carry no count.  (The split-KV partials stay on
+                                      counters.  Where the O-projection merges them itself, the
+                                      model has at most 8 KV heads, QMK_FLAG_XCD_COUNTERS is not
+                                      set and rows 2..5 hold 256 words, their arrivals go to eight
+                                      128-byte lines from word 0 of row 2 on, every arrival to all
+                                      eight, and an O-projection workgroup polls the line of its
+                                      own XCD: rows 3.. are then written in part.)                */
 #define QMK_FLAG_KEEP_BARRIERS 1u  /* leave the final counter values in `barriers`
                                       (the reference's behaviour); by default the
                                       last workgroup to retire clears them so the

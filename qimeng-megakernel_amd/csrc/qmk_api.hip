@@ -780,7 +780,7 @@ int decode_step(const QmkArgs* a, bool static_scratch) {
   p.upgate_blocks_per_bucket = a->upgate_blocks_per_bucket > 0 ? a->upgate_blocks_per_bucket : 2048 / 16;
   p.down_arrivals = a->down_arrivals > 0 ? a->down_arrivals : (M::H / 16) * (M::F / 2048);
   p.spin_limit = a->spin_limit > 0 ? a->spin_limit : kDefaultSpinLimit;
-  p.flags = a->flags;
+  p.flags = a->flags | attention_lines_flag(a->flags, a->num_layer_barriers, a->barrier_slots, M::NKV);
 
   hipLaunchKernelGGL(decode_megakernel<M>, dim3(a->num_queues), dim3(kThreads), 0,
                      static_cast<hipStream_t>(a->stream), p);
@@ -965,6 +965,7 @@ int decode_step_moe(const QmkMoeArgs* a) {
 
   Params p{};
   fill_moe_params<M>(a, dev, p);
+  p.flags |= attention_lines_flag(a->flags, a->num_layer_barriers, a->barrier_slots, M::NKV);
   const uint64_t shared_bytes = ((static_cast<uint64_t>(a->shared_k_slices) * M::H * sizeof(u16) + 127) / 128) * 128;
   p.shared_parts = static_cast<u16*>(a->workspace);
   p.routed_parts = reinterpret_cast<float*>(static_cast<char*>(a->workspace) + shared_bytes);

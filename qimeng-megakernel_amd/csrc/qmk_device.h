@@ -413,6 +413,23 @@ __device__ __forceinline__ int32_t* sub_counter(const Params& p, int layer, int 
          ((row - 2) * kXcds + xcd) * kLineInts;
 }
 
+// The attention edge when the O-projection merges the partials itself: every split-KV instruction arrives once and
+// EVERY O-proj workgroup polls the count.  Pollers and arrivals on one line stand in each other's way, so an arrival
+// goes to eight lines, one per XCD, and a workgroup polls the line of its own XCD alone (32 pollers on a line instead of
+// 256).  The lines: the edge's sub-counters with QMK_FLAG_XCD_COUNTERS; otherwise, if the launcher says so (a bit of
+// Params::flags that no caller can set), the 256 words from word 0 of row 2 on — a tagged launch leaves counter rows
+// 3, 4 and 5 unused.  The kernels that run several rows keep word 0 (their rows' counters lie 32 words apart).
+constexpr uint32_t kFlagAttentionRows2To5 = 1u << 16;
+// (host side) the choice for a batch-1 launch with these flags and this counter tensor.  The eightfold arrivals pay
+// while a layer has few of them (measured: 16 arrivals +1.8 %, 32 +1.0 %, 64 -0.5 %): a model with more than
+// eight KV heads keeps word 0 in a tagged launch.
+inline uint32_t attention_lines_flag(uint32_t flags, int num_layer_barriers, int barrier_slots, int kv_heads) {
+  if ((flags & QMK_FLAG_TAGGED) && !(flags & QMK_FLAG_XCD_COUNTERS) && kv_heads <= 8 && num_layer_barriers >= 6 &&
+      4 * barrier_slots >= kXcds * kLineInts)
+    return kFlagAttentionRows2To5;
+  return 0u;
+}
+
 // Arrival on an all-to-all edge (counter row 2..5, slot 0).
 __device__ __forceinline__ void arrive_all(const Params& p, int layer, int row, int amount) {
   publish(xcd_counters(p) ? sub_counter(p, layer, row, blockIdx.x & (kXcds - 1)) : counter_ptr(p, layer, row, 0), amount);

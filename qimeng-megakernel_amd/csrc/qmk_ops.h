@@ -158,8 +158,11 @@ __device__ __forceinline__ bool wg_wait(const Params& p, Smem<M>& s, const Ctx& 
 // per-XCD sub-counters of the edge when the launch uses them.
 template <class M>
 __device__ __forceinline__ bool wg_wait_all(const Params& p, Smem<M>& s, const Ctx& c, int layer, int row, int slot, int expected) {
-  if (!xcd_counters(p))
+  if (!xcd_counters(p)) {
+    if (row == ROW_REDUCE && (p.flags & kFlagAttentionRows2To5))   // this XCD's line holds the whole count
+      return wg_wait(p, s, c, 1, [&](int) { return counter_ptr(p, layer, ROW_REDUCE, static_cast<int>(blockIdx.x & (kXcds - 1)) * kLineInts); }, expected);
     return wg_wait(p, s, c, 1, [&](int) { return counter_ptr(p, layer, row, slot); }, expected);
+  }
   if (row == ROW_REDUCE) {
     // The attention edge: every split-KV instruction arrives on all eight lines, this XCD's line holds the whole count.
     if (c.tid == 0 && !poll_counter(sub_counter(p, layer, row, blockIdx.x & (kXcds - 1)), expected, p.spin_limit)) {
@@ -896,11 +899,11 @@ __device__ bool op_attn_splitkv(const Params& p, Smem<M>& s, const Ctx& c) {
   __syncthreads();
   QMK_STAMP(3);  // stores acknowledged
   if (merge_mode == 2) {  // one arrival per partial on the attention -> O-proj edge
-    // Per-XCD counters: the arrival goes to EVERY XCD's line, and an O-proj workgroup polls the line of its own XCD
-    // alone — 32 pollers on a line instead of 256 on each of eight that a few dozen arrivals are still updating
-    // (Llama shape: 1 911 -> 1 931 tok/s).
+    // (an arrival on every XCD's line where the launch has such lines: Llama shape 1 911 -> 1 931 tok/s)
     if (xcd_counters(p)) {
       if (c.tid < kXcds) publish(sub_counter(p, layer, ROW_REDUCE, c.tid), 1);
+    } else if (p.flags & kFlagAttentionRows2To5) {
+      if (c.tid < kXcds) publish(counter_ptr(p, layer, ROW_REDUCE, c.tid * kLineInts), 1);
     } else if (c.tid == 0) {
       publish(counter_ptr(p, layer, ROW_REDUCE, 0), 1);
     }
