@@ -482,6 +482,10 @@ __global__ __launch_bounds__(kThreads, 1) void decode_megakernel_moe_rows(const 
     const int total = p.num_layers * p.num_layer_barriers * p.barrier_slots;
     for (int i = threadIdx.x; i < total; i += kThreads)
       __hip_atomic_store(p.barriers + i, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    if (p.flags & kFlagRowAttentionLines)   // the rows' attention counts, which ran through the layers
+      for (int i = threadIdx.x; i < p.batch * kXcds * kLineInts; i += kThreads)
+        __hip_atomic_store(row_attention_line(rows::ws_of(p, i / (kXcds * kLineInts)), p.ws_row_units, 0) + i % (kXcds * kLineInts), 0,
+                           __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     if (threadIdx.x == 0) st_shared32(p.ws + kWsGeneration, (s.b.generation + 1u) & 0x03ffffffu);
   }
 }
@@ -597,6 +601,10 @@ __global__ __launch_bounds__(kThreads, 1) void decode_megakernel_rows(const Para
     const int total = p.num_layers * p.num_layer_barriers * p.barrier_slots;
     for (int i = threadIdx.x; i < total; i += kThreads)
       __hip_atomic_store(p.barriers + i, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    if (p.flags & kFlagRowAttentionLines)   // the rows' attention counts, which ran through the layers
+      for (int i = threadIdx.x; i < p.batch * kXcds * kLineInts; i += kThreads)
+        __hip_atomic_store(row_attention_line(rows::ws_of(p, i / (kXcds * kLineInts)), p.ws_row_units, 0) + i % (kXcds * kLineInts), 0,
+                           __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     if (threadIdx.x == 0) st_shared32(p.ws + kWsGeneration, (s.b.generation + 1u) & 0x03ffffffu);
   }
 }
@@ -1048,7 +1056,7 @@ void fill_moe_params(const QmkMoeArgs* a, DeviceInfo* dev, Params& p) {
 }
 
 // Units from one row's tagged workspace to the next in a launch of several rows: a batch-1 launch's units, in whole lines.
-constexpr int kWsRowUnits = ((kWsMoeUnits + 15) / 16) * 16;
+constexpr int kWsRowUnits = ((kWsMoeUnits + 15) / 16) * 16 + kRowAttentionUnits;   // ... and the row's attention lines
 
 template <class M>
 int decode_step_moe_rows(const QmkMoeRowsArgs* r) {
@@ -1088,6 +1096,7 @@ int decode_step_moe_rows(const QmkMoeRowsArgs* r) {
   Params p{};
   fill_moe_params<M>(a, dev, p);
   p.local_routing = 1;
+  p.flags |= kFlagRowAttentionLines;
   p.ws = static_cast<uint64_t*>(a->workspace);
   p.ws_row_units = kWsRowUnits;
   p.batch = B;
@@ -1114,7 +1123,7 @@ extern "C" int qmk_decode_step_moe(const QmkMoeArgs* a) {
 }
 
 // Units from one row's tagged workspace to the next in a dense launch of several rows.
-constexpr int kWsDenseRowUnits = ((kWsUnits + 15) / 16) * 16;
+constexpr int kWsDenseRowUnits = ((kWsUnits + 15) / 16) * 16 + kRowAttentionUnits;   // ... and the row's attention lines
 
 extern "C" uint64_t qmk_rows_workspace_bytes(int batch_size) {
   if (batch_size < 1 || batch_size > rows::kMaxRows) return 0;
@@ -1188,7 +1197,7 @@ static int decode_step_rows(const QmkRowsArgs* r) {
   p.rms_norm_eps = a->rms_norm_eps;
   p.qkv_blocks_per_head = r->qkv_blocks_per_head > 0 ? r->qkv_blocks_per_head : M::D / 16;
   p.spin_limit = a->spin_limit > 0 ? a->spin_limit : kDefaultSpinLimit;
-  p.flags = QMK_FLAG_TAGGED;
+  p.flags = QMK_FLAG_TAGGED | kFlagRowAttentionLines;
   p.batch = B;
   p.position_ids = a->position_ids;
   p.active_mask = a->active_mask;

@@ -430,6 +430,18 @@ inline uint32_t attention_lines_flag(uint32_t flags, int num_layer_barriers, int
   return 0u;
 }
 
+// The kernels that run several rows: a row's attention output is complete when the last split-KV arrival of each of
+// its KV-head groups has merged the group and counted its heads, and every O-proj workgroup polls that count.  With
+// this bit of Params::flags (the launchers of those kernels set it) the count lives on eight lines at the end of the
+// row's tagged workspace, every arrival goes to all eight and a workgroup polls the line of its own XCD.  The lines
+// are not per layer: a layer's arrivals all precede the next layer's, so layer l waits for (l + 1) x NQ; the
+// workgroup that retires last clears them.
+constexpr uint32_t kFlagRowAttentionLines = 1u << 17;
+constexpr int kRowAttentionUnits = kXcds * kLineInts / 2;   // eight 128-byte lines, in 8-byte units
+__device__ __forceinline__ int32_t* row_attention_line(uint64_t* row_ws, int row_units, int xcd) {
+  return reinterpret_cast<int32_t*>(row_ws + row_units - kRowAttentionUnits) + xcd * kLineInts;
+}
+
 // Arrival on an all-to-all edge (counter row 2..5, slot 0).
 __device__ __forceinline__ void arrive_all(const Params& p, int layer, int row, int amount) {
   publish(xcd_counters(p) ? sub_counter(p, layer, row, blockIdx.x & (kXcds - 1)) : counter_ptr(p, layer, row, 0), amount);

@@ -924,7 +924,11 @@ __device__ bool op_attn_splitkv(const Params& p, Smem<M>& s, const Ctx& c) {
     merge_partials<M>(p, kvh * M::GQA, P, nullptr, true, 0);
     release_stores();
     __syncthreads();
-    if (c.tid == 0) publish(counter_ptr(p, layer, ROW_REDUCE, 0), M::GQA);
+    if (p.flags & kFlagRowAttentionLines) {   // (p is the view of one row of a launch of several)
+      if (c.tid < kXcds) publish(row_attention_line(p.ws, p.ws_row_units, c.tid), M::GQA);
+    } else if (c.tid == 0) {
+      publish(counter_ptr(p, layer, ROW_REDUCE, 0), M::GQA);
+    }
   }
   return true;
 }

@@ -345,9 +345,14 @@ __device__ bool op_qkv(const Params& p, Smem<M>& s, const Ctx& c) {
 }
 
 // Every live row's word on the reduction row has reached `expected` (lane r polls row r's).  False (uniformly) on a timeout.
+// `merged`: the count of the rows' merged head groups, which lives on the lines of the rows' workspaces when the
+// launch has them (this XCD's line; the lines count through the layers).
 template <class M>
-__device__ __forceinline__ bool wait_rows(const Params& p, Smem<M>& s, const Ctx& c, int layer, int expected) {
-  if (c.tid < p.batch && s.live[c.tid] && !poll_counter(counter_ptr(p, layer, ROW_REDUCE, c.tid * M::NQ), expected, p.spin_limit)) {
+__device__ __forceinline__ bool wait_rows(const Params& p, Smem<M>& s, const Ctx& c, int layer, int expected, bool merged = false) {
+  const bool lines = merged && (p.flags & kFlagRowAttentionLines);
+  if (c.tid < p.batch && s.live[c.tid] &&
+      !(lines ? poll_counter(row_attention_line(ws_of(p, c.tid), p.ws_row_units, blockIdx.x & (kXcds - 1)), (layer + 1) * expected, p.spin_limit)
+              : poll_counter(counter_ptr(p, layer, ROW_REDUCE, c.tid * M::NQ), expected, p.spin_limit))) {
     s.b.ctl[0] = 1;
     report_error(p, QMK_DEV_WAIT_TIMEOUT, c.inst_idx, c.opcode, c.tid);
   }
@@ -431,7 +436,7 @@ __device__ bool op_oproj(const Params& p, Smem<M>& s, const Ctx& c, Carried& car
     }
     // The rows' attention outputs are complete in memory: the last split-KV arrival of every (row, KV head) merged its
     // group's partials and counted the group's heads on the row's word of the reduction row.  All rows in one trip.
-    if (!wait_rows(p, s, c, layer, M::NQ)) return false;
+    if (!wait_rows(p, s, c, layer, M::NQ, /*merged=*/true)) return false;
     constexpr int kPieces = (NR * AW + kThreads * 8 - 1) / (kThreads * 8);   // 16-byte pieces per thread
     v4u piece[kPieces];
 #pragma unroll
