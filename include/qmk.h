@@ -333,8 +333,10 @@ int qmk_decode_step_batch(const QmkBatchArgs* args);
  * route (…/multi_batch/decode_kernel/mk.h:9-42) has no counterpart of this stream; a step is the batch-1 route run for
  * every active row, whose results it reproduces bit for bit.  Hand-over is the tagged one (one set of units per row in
  * `workspace`, qmk_rows_workspace_bytes(B) bytes, 128-byte aligned, zeroed once); the split-KV partials of a (row, KV
- * head) are merged by the group's last arrival (merge word 1, O-projection word 5 = 0) or by every O-projection
- * workgroup (merge word 2, word 5 = fan-out).  A row whose active flag is off is left alone; its logits are set to -1e9.
+ * head) are merged by the group's last arrival (merge word 1, O-projection word 5 = 0; the row's count of merged heads
+ * is kept on eight 128-byte lines at the end of the row's workspace, one per XCD, which the launch that retires clears)
+ * or by every O-projection workgroup (merge word 2, word 5 = fan-out).  A row whose active flag is off is left alone;
+ * its logits are set to -1e9.  After a device-side error the caller zeroes `workspace` and `barriers`.
  */
 typedef struct QmkRowsArgs {
   uint32_t struct_size;            /* = sizeof(QmkRowsArgs)                       */

@@ -114,9 +114,11 @@ def test_host_side_argument_errors(lib):
     assert lib.qmk_moe_workspace_bytes(8, 0) == 8 * 2048 * 4 + 128 + lib.qmk_workspace_bytes(0) + moe_units     # no shared expert
     assert lib.qmk_moe_workspace_bytes(9, 4) == 0
     assert lib.qmk_error_string(12345).decode() == "unknown code"
-    # the dense route at 1..4 rows on the row-streaming engine: a set of the dense route's units per row
+    # the dense route at 1..4 rows on the row-streaming engine: per row a set of the dense route's units and the eight
+    # 128-byte lines of the row's attention count
     rows_kernel_mb.get_mk()
-    assert [lib.qmk_rows_workspace_bytes(b) for b in (0, 1, 4, 5)] == [0, lib.qmk_workspace_bytes(0), 4 * lib.qmk_workspace_bytes(0), 0]
+    per_row = lib.qmk_workspace_bytes(0) + 8 * 128
+    assert [lib.qmk_rows_workspace_bytes(b) for b in (0, 1, 4, 5)] == [0, per_row, 4 * per_row, 0]
     assert lib.qmk_decode_step_rows(None) == 1
     d = rows_kernel_mb.QmkRowsArgs()
     d.struct_size = ctypes.sizeof(rows_kernel_mb.QmkRowsArgs)
@@ -128,9 +130,10 @@ def test_host_side_argument_errors(lib):
     assert lib.qmk_decode_step_rows(ctypes.byref(d)) == 3                    # batch_size 0
     d.step.batch_size = 4
     assert lib.qmk_decode_step_rows(ctypes.byref(d)) == 1                    # all tensor pointers are NULL
-    # several requests in one launch: a set of the MoE route's units per row, in whole 128-byte lines
+    # several requests in one launch: per row a set of the MoE route's units, in whole 128-byte lines, and the eight lines
+    # of the row's attention count
     rows_kernel.get_mk()
-    per_row = lib.qmk_moe_workspace_bytes(8, 0) - 8 * 2048 * 4 - 128
+    per_row = lib.qmk_moe_workspace_bytes(8, 0) - 8 * 2048 * 4 - 128 + 8 * 128
     assert per_row % 128 == 0 and [lib.qmk_moe_rows_workspace_bytes(b) for b in (0, 1, 4, 5)] == [0, per_row, 4 * per_row, 0]
     assert lib.qmk_decode_step_moe_rows(None) == 1
     r = rows_kernel.QmkMoeRowsArgs()
