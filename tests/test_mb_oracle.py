@@ -151,6 +151,19 @@ def test_o_proj_blocks_go_beside_the_attention_workers():
     assert ref.oproj_round(0, 4)[: len(ref.oproj(0))] == ref.oproj(0)
 
 
+def test_qkv_blocks_go_behind_the_attention_workers():
+    """MI355X template: the QKV round starts behind the split-KV round's workers where both fit side by side, else behind
+    the norm rows' workers, else (and in the reference's template) at worker 0."""
+    def first(sched):
+        r = sched.qkv_round(0, sched.partials_for_capacity(1024))
+        assert len(r) % sched.workers == 0 and [i for i in r if i.opcode() == 2] == sched.qkvproj(0)
+        return next(k for k, i in enumerate(r) if i.opcode() == 2)
+    assert first(S.mi355x_scheduler(8, MB_FULL)) == 64       # 64 slices + 192 blocks = 256 workers
+    assert first(S.mi355x_scheduler(16, MB_FULL)) == 16      # 128 slices: behind the 16 norm rows
+    assert first(S.mi355x_scheduler(8, MB_FULL, skew_upgate=False)) == 0
+    assert first(S.reference_scheduler(8, MB_FULL)) == 0
+
+
 @pytest.mark.parametrize("make,rows", [(S.reference_scheduler, 3), (S.mi355x_scheduler, 8), (S.mi355x_scheduler, 16)])
 def test_every_output_once_and_final_counters(make, rows):
     shape = MB_SMALL
