@@ -45,7 +45,7 @@ MEASURED_TRAFFIC_OVER_ALGORITHMIC = 1.0080
 # The same kernel template on the Qwen3-1.7B shape, contexts 1020..1039 (profiles/decode_megakernel_qwen3_1p7b_hbm_counters.txt).
 MEASURED_TRAFFIC_OVER_ALGORITHMIC_QWEN3_1P7B = 1.0139
 # The same for the batch route's kernel at batch 8 (profiles/decode_megakernel_batch_llama1b_hbm_counters.txt).
-MEASURED_TRAFFIC_OVER_ALGORITHMIC_BATCH8 = 1.0242
+MEASURED_TRAFFIC_OVER_ALGORITHMIC_BATCH8 = 1.0244
 # ... for the rows engine at 4 rows (profiles/decode_megakernel_rows_llama1b_batch4_hbm_counters.txt)
 MEASURED_TRAFFIC_OVER_ALGORITHMIC_ROWS4 = 1.0175
 # ... and for the MoE route's kernel (profiles/decode_megakernel_moe_qwen1p5_a2p7b_hbm_counters.txt).
