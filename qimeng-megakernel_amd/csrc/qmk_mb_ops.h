@@ -886,48 +886,63 @@ __device__ bool op_upgate(const Params& p, Smem<M>& s, const Ctx& c) {
   return true;
 }
 
-// The down projection of a 16-row block for at most 8 batch rows, K = 8192.  With 8 batch rows half of the tile's
+// The down projection of a 16-row block for at most 8 batch rows.  With 8 batch rows half of the tile's
 // columns are empty, and so is half of every activation register: here a tile is 8 weight rows x 8 batch rows, twice —
 // lanes m < 8 of the A operand hold rows 0..7 of one 32-column chunk, lanes m >= 8 the same rows of the NEXT chunk, and
 // the B operand's columns n < 8 / n >= 8 hold the batch rows' shares of those two chunks: C[m][n] is then the first
 // chunk's product for m, n < 8, the second's for m, n >= 8 (the other two quadrants mix chunks and are dropped), and
-// an output is the sum of the two.  A register set (Seg / v4u[8]) covers 8 rows x 512 columns instead of 16 x 256: a
-// wave's 1024 columns of both 8-row halves are the same four weight sets as before, but ALL of its activations are
-// two sets, which fit beside three of them — one round of activation loads behind the wait instead of two dependent
-// ones.  Weight loads take 128 contiguous bytes of 8 rows per instruction (64 bytes of 16 before).
+// an output is the sum of the two.  A register set covers 8 rows x 512 columns instead of 16 x 256 (F = 8192; 8 x 384
+// for F = 6144): a wave's columns of both 8-row halves are four weight sets as before, but ALL of its activations are
+// two sets, which fit beside three (F = 6144: all four) of them — one round of activation loads behind the wait instead
+// of two dependent ones.  Weight loads take 128 contiguous bytes of 8 rows per instruction (64 bytes of 16 before).
 template <class M>
 __device__ __forceinline__ bool op_down_packed(const Params& p, Smem<M>& s, const Ctx& c, int layer, int B, int n0, int n1) {
-  constexpr int kPair = 2 * kChunk;              // columns of a chunk pair
-  constexpr int kPackedSeg = kSegChunks * kPair; // columns of a packed set: 512
-  static_assert(M::F == kWaves * 2 * kPackedSeg, "a wave owns two packed sets of each half");
+  constexpr int kPair = 2 * kChunk;                      // columns of a chunk pair
+  constexpr int NP = M::F / (kWaves * 2 * kPair);        // chunk pairs of a set: 8 (F = 8192: 512 columns), 6 (F = 6144: 384)
+  constexpr int kSetCols = NP * kPair;
+  static_assert(M::F == kWaves * 2 * kSetCols && NP <= kSegChunks, "a wave owns two sets of each half");
+  // Four weight sets of 8 pairs and the activations do not fit the registers: the fourth waits in LDS; four of 6 do.
+  constexpr bool kPark = NP == kSegChunks;
+  struct Set {
+    v4u a[NP];
+  };
   const int lane = c.tid & 63, wave = c.tid >> 6;
   const u16* w = p.down_w + static_cast<size_t>(layer) * M::H * M::F;
-  const int k0 = wave * 2 * kPackedSeg;
+  const int k0 = wave * 2 * kSetCols;
   const int sub = (lane >> 3) & 1, g = lane >> 4;   // which chunk of the pair, which 8 columns of it
   const size_t lane_off = static_cast<size_t>(lane & 7) * M::F + k0 + sub * kChunk + g * 8;
-  auto load_packed = [&](Seg& sg, const u16* at) {
+  auto load_set = [&](Set& sg, const u16* at) {
 #pragma unroll
-    for (int j = 0; j < kSegChunks; ++j) sg.a[j] = *reinterpret_cast<const v4u*>(at + j * kPair);
+    for (int j = 0; j < NP; ++j) sg.a[j] = *reinterpret_cast<const v4u*>(at + j * kPair);
   };
-  // set q of a block: half q >> 1 (rows 8 * half ..), columns k0 + 512 * (q & 1) ..
-  auto wptr = [&](int block, int q) { return w + (static_cast<size_t>(block) * kTile + 8 * (q >> 1)) * M::F + lane_off + (q & 1) * kPackedSeg; };
-  Seg a0, a1, a2, a3;
+  auto mma_set = [&](const Set& sg, const v4u (&x)[NP], f4 acc) {
+#pragma unroll
+    for (int j = 0; j < NP; ++j)
+      acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, sg.a[j]), __builtin_bit_cast(bf16x8, x[j]), acc, 0, 0, 0);
+    return acc;
+  };
+  // set q of a block: half q >> 1 (rows 8 * half ..), columns k0 + kSetCols * (q & 1) ..
+  auto wptr = [&](int block, int q) { return w + (static_cast<size_t>(block) * kTile + 8 * (q >> 1)) * M::F + lane_off + (q & 1) * kSetCols; };
+  Set a0, a1, a2, a3;
   auto request = [&](int block) {
-    load_packed(a0, wptr(block, 0));
-    load_packed(a1, wptr(block, 1));
-    load_packed(a2, wptr(block, 2));
+    load_set(a0, wptr(block, 0));
+    load_set(a1, wptr(block, 1));
+    load_set(a2, wptr(block, 2));
+    if constexpr (!kPark) load_set(a3, wptr(block, 3));
   };
   if (n0 < n1) {
     request(n0);
-    load_packed(a3, wptr(n0, 3));   // the fourth set waits in LDS: the registers hold three weight sets and the activations
+    if constexpr (kPark) {
+      load_set(a3, wptr(n0, 3));
 #pragma unroll
-    for (int j = 0; j < kSegChunks; ++j) s.seg_park[wave][j][lane] = a3.a[j];
+      for (int j = 0; j < NP; ++j) s.seg_park[wave][j][lane] = a3.a[j];
+    }
   }
   if (!wait_edge(p, s, c, layer, ROW_UPGATE, M::F / kTile)) return false;
   u16* const mine = p.hidden + static_cast<size_t>(c.tid & 15) * M::H + 2 * (c.tid >> 4);
   const bool adds = c.tid < 8 * kTile && (c.tid & 15) < B && s.active[c.tid & 15];
   // this lane's share of silu_out: batch row l % 8, the chunk of the pair its weight lanes hold
-  v4u xa[kSegChunks], xb[kSegChunks];
+  v4u xa[NP], xb[NP];
   {
     u16* base = p.silu_out;
     asm volatile("" : "+s"(base));
@@ -936,24 +951,26 @@ __device__ __forceinline__ bool op_down_packed(const Params& p, Smem<M>& s, cons
     const uint32_t row = (lane & 7) < B ? static_cast<uint32_t>(lane & 7) : 0u;
     const uint32_t at = (row * M::F + k0 + sub * kChunk + g * 8) * 2;
 #pragma unroll
-    for (int j = 0; j < kSegChunks; ++j) {
+    for (int j = 0; j < NP; ++j) {
       xa[j] = __builtin_bit_cast(v4u, __builtin_amdgcn_raw_buffer_load_b128(rsrc, at + j * kPair * 2, 0, 16));
-      xb[j] = __builtin_bit_cast(v4u, __builtin_amdgcn_raw_buffer_load_b128(rsrc, at + (kPackedSeg + j * kPair) * 2, 0, 16));
+      xb[j] = __builtin_bit_cast(v4u, __builtin_amdgcn_raw_buffer_load_b128(rsrc, at + (kSetCols + j * kPair) * 2, 0, 16));
     }
   }
   int parity = 0;
   for (int blk = n0; blk < n1; ++blk) {
     const uint32_t old = adds ? ld_shared32(mine + blk * kTile) : 0u;   // the pair this thread adds to, in time for the epilogue
-    f4 lo = mma_seg(a0, xa, f4{0.f, 0.f, 0.f, 0.f});   // rows 0..7
-    f4 hi = mma_seg(a2, xa, f4{0.f, 0.f, 0.f, 0.f});   // rows 8..15
-    lo = mma_seg(a1, xb, lo);
-    if (blk == n0) {
+    f4 lo = mma_set(a0, xa, f4{0.f, 0.f, 0.f, 0.f});   // rows 0..7
+    f4 hi = mma_set(a2, xa, f4{0.f, 0.f, 0.f, 0.f});   // rows 8..15
+    lo = mma_set(a1, xb, lo);
+    if constexpr (kPark) {
+      if (blk == n0) {
 #pragma unroll
-      for (int j = 0; j < kSegChunks; ++j) a3.a[j] = s.seg_park[wave][j][lane];
-    } else {
-      load_packed(a3, wptr(blk, 3));
+        for (int j = 0; j < NP; ++j) a3.a[j] = s.seg_park[wave][j][lane];
+      } else {
+        load_set(a3, wptr(blk, 3));
+      }
     }
-    hi = mma_seg(a3, xb, hi);
+    hi = mma_set(a3, xb, hi);
     park(s, parity, 0, wave, lane, lo);
     park(s, parity, 1, wave, lane, hi);
     QMK_MB_STAMP(0);
@@ -995,9 +1012,8 @@ __device__ bool op_down(const Params& p, Smem<M>& s, const Ctx& c) {
   const int R = s.inst[7];   // rows per block: 16 (the reference's), or 8 (one block per workgroup on 256 CUs)
   if (s.inst[6] != kMaxBatch || (R != kTile && R != kTile / 2)) return bad_operand(p, s, c, 7);
   if (n0 < 0 || n1 < n0 || n1 > M::H / R) return bad_operand(p, s, c, 4);
-  if constexpr (NS == 4) {   // at most 8 batch rows: half-tiles, all activations in one round (8 rows: +1.4 %)
-    if (B <= kMaxBatch / 2 && R == kTile) return op_down_packed<M>(p, s, c, layer, B, n0, n1);   // uniform
-  }
+  // at most 8 batch rows: half-tiles, all activations in one round (Llama shape, 8 rows: +1.4 %)
+  if (B <= kMaxBatch / 2 && R == kTile) return op_down_packed<M>(p, s, c, layer, B, n0, n1);   // uniform
   const int lane = c.tid & 63, wave = c.tid >> 6;
   const u16* w = p.down_w + static_cast<size_t>(layer) * M::H * M::F;
   const int k0 = wave * NS * kSeg;
