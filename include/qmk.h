@@ -240,10 +240,12 @@ int qmk_decode_step_static(const QmkArgs* args);
  * route: Llama-3.2-1B, and Qwen3-1.7B with the Qwen3 op set (opcode 2 leaves the raw QKV rows, opcode 3
  * applies the per-head RMSNorm and RoPE to its row's q and k and appends the cache row).
  * Flags: QMK_FLAG_KEEP_BARRIERS, and QMK_FLAG_XCD_COUNTERS in this route's form: the blocks of the
- * O-projection, the up/gate and the down projection (counter rows 4, 6, 7) are counted on words 32, 64 .. 256 of
- * their row (the sender's workgroup index modulo 8 chooses: one 128-byte line per XCD) instead of on word 0, and
- * the instructions that wait for them add the eight words up; needs barrier_slots >= 288.  Hundreds of arrivals
- * from eight XCDs on one line are seen 2 us later than on eight.  No counterpart in the reference.
+ * O-projection, the up/gate and the down projection (counter rows 4, 6, 7) are counted on words 0, 32 .. 224 of
+ * their row (the sender's workgroup index modulo 8 chooses: one 128-byte line per XCD) instead of all on word 0, and
+ * the instructions that wait for them add the eight words up; a norm row (counter rows 0, 5, 8) arrives on all eight
+ * of those words of its row and a waiting workgroup polls the one of its own XCD; the head counters of row 1 and the
+ * row counters of row 3 move a line apart (word i -> 32 (i % 8) + i / 8).  Needs barrier_slots >= 256.  Hundreds of
+ * arrivals from eight XCDs on one line are seen 2 us later than on eight.  No counterpart in the reference.
  */
 typedef struct QmkBatchArgs {
   uint32_t struct_size;            /* = sizeof(QmkBatchArgs)                      */

@@ -832,8 +832,8 @@ static int decode_step_batch(const QmkBatchArgs* a) {
       a->vocab_size < 1 || a->rope_rows < 1 || a->kv_block_size < 1 || a->oproj_blocks < 0 || a->down_blocks < 0)
     return QMK_ERR_SHAPE;
   if (a->flags & ~(QMK_FLAG_KEEP_BARRIERS | QMK_FLAG_XCD_COUNTERS)) return QMK_ERR_SHAPE;
-  // eight sub-counters, a 128-byte line each, behind word 0 of the O-projection's, the up/gate's and the down projection's row
-  if ((a->flags & QMK_FLAG_XCD_COUNTERS) && a->barrier_slots < kLineInts * (1 + mb::kSpread)) return QMK_ERR_SHAPE;
+  // eight sub-counters, a 128-byte line each, in the O-projection's, the up/gate's and the down projection's row
+  if ((a->flags & QMK_FLAG_XCD_COUNTERS) && a->barrier_slots < kLineInts * mb::kSpread) return QMK_ERR_SHAPE;
   if (a->position_ids == nullptr && (a->pos_id < 0 || a->pos_id >= a->max_seq_len || a->pos_id >= a->rope_rows)) return QMK_ERR_POSITION;
   // the column window: all columns, or a part of them with counters that outlive the launch
   if (a->first_inst < 0 || a->inst_count < 0 || (a->inst_count == 0 && a->first_inst != 0) ||

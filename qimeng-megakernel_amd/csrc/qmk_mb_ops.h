@@ -130,18 +130,18 @@ __device__ __forceinline__ void publish_after_stores(const Params& p, const Ctx&
 // The O-projection, the up/gate and the down projection each count 128..512 blocks on word 0 of their counter row, and
 // every one of those arrivals is a read-modify-write of the same line from another XCD: the last of them is seen
 // microseconds after it was sent.  With the flag an arrival goes to the sub-counter of the sender's XCD (workgroup % 8:
-// word 32 * (1 + xcd) of the same row, a line of its own; the rows have no other user beyond word 0), and a waiting
-// workgroup's first eight lanes read the eight words and add them up.
+// word 32 * xcd of the same row, a line of its own; the rows have no other user, and word 0 is one of the eight), and a
+// waiting workgroup's first eight lanes read the eight words and add them up.  A row needs 256 words for it.
 constexpr int kSpread = kXcds;
 __device__ __forceinline__ bool spread_counters(const Params& p) { return (p.flags & QMK_FLAG_XCD_COUNTERS) != 0; }
 __device__ __forceinline__ void publish_edge_after_stores(const Params& p, const Ctx& c, int layer, int row, int amount) {
-  publish_after_stores(p, c, layer, row, spread_counters(p) ? kLineInts * (1 + static_cast<int>(blockIdx.x & (kSpread - 1))) : 0, amount);
+  publish_after_stores(p, c, layer, row, spread_counters(p) ? kLineInts * static_cast<int>(blockIdx.x & (kSpread - 1)) : 0, amount);
 }
 template <class S>
 __device__ __forceinline__ bool wait_edge(const Params& p, S& s, const Ctx& c, int layer, int row, int expected) {
   if (!spread_counters(p)) return wait_counter(p, s, c, layer, row, expected);
   if (c.tid < kSpread) {
-    const int32_t* mine = counter_ptr(p, layer, row, kLineInts * (1 + c.tid));
+    const int32_t* mine = counter_ptr(p, layer, row, kLineInts * c.tid);
     uint32_t polls = 0;
     while (true) {
       int v = __hip_atomic_load(mine, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
@@ -168,9 +168,9 @@ __device__ __forceinline__ bool wait_edge(const Params& p, S& s, const Ctx& c, i
 }
 
 // Counters that are neighbours in one line by the reference's layout (the 48 head counters of the QKV projection, the B
-// row counters of the attention outputs) move a line apart with the flag: word i -> line 1 + i % 8, word i / 8 of it
+// row counters of the attention outputs) move a line apart with the flag: word i -> line i % 8, word i / 8 of it
 // (Llama shape, 8 rows: +0.5 %).
-__device__ __forceinline__ int apart(const Params& p, int i) { return spread_counters(p) ? kLineInts * (1 + (i & 7)) + (i >> 3) : i; }
+__device__ __forceinline__ int apart(const Params& p, int i) { return spread_counters(p) ? kLineInts * (i & 7) + (i >> 3) : i; }
 
 // The B rows of an RMSNorm round are few arrivals, but every workgroup of the next GEMM polls them: 128..256 pollers on
 // one line stand in each other's way (and in the arrivals').  With the flag a row arrives on all eight lines, and a
@@ -178,7 +178,7 @@ __device__ __forceinline__ int apart(const Params& p, int i) { return spread_cou
 template <class S>
 __device__ __forceinline__ bool wait_rows_done(const Params& p, S& s, const Ctx& c, int layer, int row, int expected) {
   if (spread_counters(p))
-    return wait_counters(p, s, c, 1, [&](int) { return counter_ptr(p, layer, row, kLineInts * (1 + static_cast<int>(blockIdx.x & (kSpread - 1)))); },
+    return wait_counters(p, s, c, 1, [&](int) { return counter_ptr(p, layer, row, kLineInts * static_cast<int>(blockIdx.x & (kSpread - 1))); },
                          [&](int) { return expected; });
   return wait_counter(p, s, c, layer, row, expected);
 }
@@ -225,7 +225,7 @@ __device__ bool op_rms_row(const Params& p, Smem<M>& s, const Ctx& c) {
   if (spread_counters(p)) {   // one arrival on every XCD's line: each consumer polls the line of its own XCD
     release_stores();
     __syncthreads();
-    if (c.tid < kSpread) publish(counter_ptr(p, layer, my_row, kLineInts * (1 + c.tid)), 1);
+    if (c.tid < kSpread) publish(counter_ptr(p, layer, my_row, kLineInts * c.tid), 1);
     return true;
   }
   publish_after_stores(p, c, layer, my_row, 0, 1);

@@ -108,12 +108,13 @@ class BatchMegaKernel:
     ``reset_barriers``: the kernel clears the counters when it retires (default) or leaves their
     final values in place like the reference kernel, whose host loop zeroes them before every step.
     ``xcd_counters``: the blocks of the O-projection, the up/gate and the down projection are counted on eight
-    sub-counters (words 32, 64, .. 256 of their counter row, one 128-byte line per XCD) instead of on word 0, where
+    sub-counters (words 0, 32, .. 224 of their counter row, one 128-byte line per XCD) instead of all on word 0, where
     hundreds of arrivals from eight XCDs queue on one line.  Taken when the kernel clears the counters itself and
-    a row has the 288 words (batches of 6 and more); a launch that keeps the counters leaves the reference's words.
+    a row has the 256 words (Llama shape: 6 rows and more, Qwen3-1.7B shape: 8 and more); a launch that keeps the counters
+    leaves the reference's words.
     """
 
-    XCD_COUNTER_WORDS = 32 * 9
+    XCD_COUNTER_WORDS = 32 * 8
 
     def __init__(self, lib: ctypes.CDLL, *, reset_barriers: bool = True, spin_limit: int = 0, xcd_counters: bool = True):
         self._lib = lib

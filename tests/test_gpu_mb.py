@@ -238,7 +238,7 @@ def test_step_run_column_by_column_equals_the_step_run_whole(weights):
 
 def test_arrivals_counted_per_xcd_change_no_result(weights):
     """The blocks of the O-projection, the up/gate and the down projection counted on eight sub-counters of their rows
-    (QMK_FLAG_XCD_COUNTERS; taken by default when the kernel clears the counters and a row has 288 words) against the
+    (QMK_FLAG_XCD_COUNTERS; taken by default when the kernel clears the counters and a row has 256 words) against the
     same step counted on word 0: every buffer bit for bit, the counters cleared; a launch that keeps the counters
     stays with the reference's words, and rows too short for the sub-counters are refused."""
     rows = 8
@@ -268,8 +268,8 @@ def test_arrivals_counted_per_xcd_change_no_result(weights):
     assert spread.barriers[:, 6, 0].tolist() == [blocks] * MB_SMALL.num_hidden_layers and int(spread.barriers[:, 6, 1:].abs().sum()) == 0
     args = mk_kernel.QmkBatchArgs()
     ctypes.memmove(ctypes.byref(args), ctypes.byref(mk._args), ctypes.sizeof(args))
-    assert args.flags & 2 and args.barrier_slots >= 288
-    args.barrier_slots = 287
+    assert args.flags & 2 and args.barrier_slots >= 256
+    args.barrier_slots = 255
     assert mk._lib.qmk_decode_step_batch(ctypes.byref(args)) != 0
 
 
