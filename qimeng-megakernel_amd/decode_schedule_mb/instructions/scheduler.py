@@ -153,6 +153,13 @@ class BatchScheduler:
             return plain + [NoOp()] * (-len(plain) % self.workers)
         slices = len(self.attention_split_kv(layer, num_partials))
         start = next((at for at in (slices, self.batch_size) if at + len(plain) <= self.workers), 0)
+        others = self.workers - self.batch_size
+        blocks = _ceil_div(self.shape.qkv_out_dim, TILE_N_GRANULARITY)
+        if start == 0 and 0 < others and blocks <= 2 * others:
+            # A block for every worker (Qwen3-1.7B shape: 256): the norm rows' workers still get none, a few of the others
+            # two — a second block costs 1 us, a block behind a norm row ends the phase 2.7 us late.
+            start = self.batch_size
+            plain = [QKVProj_GEMM_RoPE(layer, self.batch_size, 0, lo, hi) for lo, hi in _spans(blocks, others)]
         return [NoOp()] * start + plain + [NoOp()] * (self.workers - start - len(plain))
 
     def oproj_round(self, layer: int, num_partials: int) -> list[Instruction]:
