@@ -450,6 +450,11 @@ typedef struct QmkMoeArgs {
                                       opcode 9 only reports it — for streams in which nothing runs beside the router and the
                                       top-k (no shared expert), where that hand-over would leave the whole device waiting;
                                       such a stream may place opcode 9 behind its queue's routed up/gate tiles          */
+  int32_t qkv_tile;                /* rows per tile of opcode 1 (its tile_N_granularity word): 16 (0 = 16), or 8, 4 or 2 where
+                                      16 deals the tiles unevenly (5120 rows: 320 tiles of 16 leave a quarter of 256 queues
+                                      with two, 1280 tiles of 4 give each five); fixes the final value of a head's QKV
+                                      counter (D / qkv_tile)                                                          */
+  int32_t reserved0;               /* 0 */
 } QmkMoeArgs;
 
 int qmk_decode_step_moe(const QmkMoeArgs* args);

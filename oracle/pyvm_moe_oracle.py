@@ -71,6 +71,8 @@ class MoeInstructionVM:
     def rms_qkvproj_gemv_rope(self, g: Any, ins: Any) -> None:
         s = self.shape
         layer, d, tile = ins.layer_idx, s.head_dim, ins.tile_N_granularity
+        assert tile % 2 == 0 and d % tile == 0     # a tile holds whole RoPE pairs of one head
+        self._qkv_tile = tile                      # a head's counter ends at d / (the stream's tile): 16 rows in the reference
         if layer > 0:
             assert self._layer_complete(g, layer - 1)
         y = rms_norm(g.hidden_states.reshape(-1), g.attn_norm_weights[layer], s.rms_norm_eps).reshape(-1)
@@ -115,10 +117,11 @@ class MoeInstructionVM:
         ratio, d = s.num_attention_heads // s.num_key_value_heads, s.head_dim
         layer, kvh = ins.layer_idx, ins.kv_head_idx
         done = g.barriers[layer, 0]
+        per_head = d // getattr(self, "_qkv_tile", TILE)
         for i in range(ratio):
-            assert int(done[kvh * ratio + i]) == d // TILE
-        assert int(done[s.num_attention_heads + kvh]) == d // TILE
-        assert int(done[s.num_attention_heads + s.num_key_value_heads + kvh]) == d // TILE
+            assert int(done[kvh * ratio + i]) == per_head
+        assert int(done[s.num_attention_heads + kvh]) == per_head
+        assert int(done[s.num_attention_heads + s.num_key_value_heads + kvh]) == per_head
         seq_len = int(g.position_id or 0) + 1
         total = math.ceil(seq_len / s.attn_kv_block_size)
         per = math.ceil(total / ins.num_partials)

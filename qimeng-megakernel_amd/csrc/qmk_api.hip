@@ -927,6 +927,9 @@ namespace {
 template <class M>
 void fill_moe_params(const QmkMoeArgs* a, DeviceInfo* dev, Params& p);
 
+// Rows per tile of opcode 1 that QmkMoeArgs may name: the powers of two from 2 (one RoPE pair) to 16; 0 stands for 16.
+static bool qkv_tile_ok(int tile) { return tile == 0 || tile == 2 || tile == 4 || tile == 8 || tile == 16; }
+
 template <class M>
 int decode_step_moe(const QmkMoeArgs* a) {
   const void* required[] = {a->instructions, a->hidden_states, a->normed_hidden_states, a->q_post_rope, a->k_cache, a->v_cache,
@@ -959,6 +962,7 @@ int decode_step_moe(const QmkMoeArgs* a) {
   if (a->norm_topk_prob != 0 && a->norm_topk_prob != 1) return QMK_ERR_SHAPE;
   const int oproj_tile = a->oproj_tile == 0 ? moe::kTile : a->oproj_tile;
   if ((oproj_tile != 8 && oproj_tile != 16) || (a->local_routing != 0 && a->local_routing != 1)) return QMK_ERR_SHAPE;
+  if (!qkv_tile_ok(a->qkv_tile) || a->reserved0 != 0) return QMK_ERR_SHAPE;
   if (a->flags & ~(QMK_FLAG_KEEP_BARRIERS | QMK_FLAG_TAGGED)) return QMK_ERR_SHAPE;
   // tagged units carry the launch count, which the retiring launch advances, and six bits of layer
   if ((a->flags & QMK_FLAG_TAGGED) && ((a->flags & QMK_FLAG_KEEP_BARRIERS) || a->num_layers > 63)) return QMK_ERR_SHAPE;
@@ -1024,7 +1028,7 @@ void fill_moe_params(const QmkMoeArgs* a, DeviceInfo* dev, Params& p) {
   p.pos_id = a->pos_id;
   p.attn_scale = a->attn_scale;
   p.rms_norm_eps = a->rms_norm_eps;
-  p.qkv_blocks_per_head = M::D / 16;
+  p.qkv_blocks_per_head = M::D / (a->qkv_tile == 0 ? moe::kTile : a->qkv_tile);
   p.oproj_blocks = M::H / oproj_tile;
   p.down_arrivals = M::H / 16;           // what completes a layer here: the combine step's tiles
   p.spin_limit = a->spin_limit > 0 ? a->spin_limit : kDefaultSpinLimit;
@@ -1085,6 +1089,7 @@ int decode_step_moe_rows(const QmkMoeRowsArgs* r) {
   if (a->norm_topk_prob != 0 && a->norm_topk_prob != 1) return QMK_ERR_SHAPE;
   const int oproj_tile = a->oproj_tile == 0 ? moe::kTile : a->oproj_tile;
   if (oproj_tile != 8 && oproj_tile != 16) return QMK_ERR_SHAPE;
+  if (!qkv_tile_ok(a->qkv_tile) || a->reserved0 != 0) return QMK_ERR_SHAPE;
   if (a->flags != QMK_FLAG_TAGGED) return QMK_ERR_SHAPE;   // tagged hand-over, self-clearing counters: nothing else is built
   if (reinterpret_cast<uintptr_t>(a->workspace) % 128 != 0 || a->workspace_bytes < qmk_moe_rows_workspace_bytes(B)) return QMK_ERR_SHAPE;
 

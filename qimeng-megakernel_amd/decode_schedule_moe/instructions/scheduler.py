@@ -7,6 +7,7 @@ Emission order per layer 1 -> 2 -> 3 -> 4 -> 8 -> 9 -> 10 -> 11 -> 12 -> 13 -> 1
 """
 from __future__ import annotations
 
+import dataclasses
 from dataclasses import dataclass
 from typing import Sequence
 
@@ -69,8 +70,9 @@ class MoeScheduler:
                                        # the top-k instruction runs last in its layer on a queue without a combine instruction (it only reports the routing)
 
     def qkvproj(self, layer: int) -> list[Instruction]:
-        tiles = _ceil_div(self.shape.qkv_out_dim, TILE_N_GRANULARITY)
-        return [RMS_QKVProj_GEMV_RoPE(layer, 0, lo, hi) for lo, hi in _spans(tiles, self.sm_count)]
+        tile = self.shape.qkv_tile
+        tiles = _ceil_div(self.shape.qkv_out_dim, tile)
+        return [RMS_QKVProj_GEMV_RoPE(layer, 0, lo, hi, tile_N_granularity=tile) for lo, hi in _spans(tiles, self.sm_count)]
 
     def attention_split_kv(self, layer: int) -> list[Instruction]:
         if self.merge_in_oproj:
@@ -373,5 +375,7 @@ def deal(instructions: Sequence[Instruction], queues: int) -> list[list[Instruct
 
 
 def reference_scheduler(shape: MoeShape | None = None, sm_count: int = A100_SM_COUNT) -> MoeScheduler:
-    shape = shape or QwenMoeConfig.shape()
+    """The reference's stream for ``shape``: its queue count, its split-KV fan-out and its QKV tiles of 16 rows (a launch
+    of this stream takes ``.shape`` of the result, whose ``qkv_tile`` says so)."""
+    shape = dataclasses.replace(shape or QwenMoeConfig.shape(), qkv_tile=TILE_N_GRANULARITY)
     return MoeScheduler(shape, sm_count, num_partials_for(sm_count, shape))

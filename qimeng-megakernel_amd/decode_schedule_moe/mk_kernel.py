@@ -66,7 +66,8 @@ class QmkMoeArgs(ctypes.Structure):
                                    "shared_k_slices")]
         + [("attn_scale", ctypes.c_float), ("rms_norm_eps", ctypes.c_float), ("timeline", _P), ("stream", _P), ("workspace", _P),
            ("workspace_bytes", ctypes.c_uint64)]
-        + [(name, _P) for name in _QWEN3_EXTRA] + [("norm_topk_prob", _I), ("routed_upgate_tile", _I), ("oproj_tile", _I), ("local_routing", _I)]
+        + [(name, _P) for name in _QWEN3_EXTRA] + [("norm_topk_prob", _I), ("routed_upgate_tile", _I), ("oproj_tile", _I), ("local_routing", _I),
+           ("qkv_tile", _I), ("reserved0", _I)]
     )
 
 
@@ -197,6 +198,7 @@ class MoeMegaKernel:
         a.shared_k_slices = int(s.num_downproj_split_k_shared) if s.has_shared_expert else 0
         a.norm_topk_prob, a.routed_upgate_tile, a.oproj_tile = int(bool(s.norm_topk_prob)), int(s.routed_upgate_tile), int(s.oproj_tile)
         a.local_routing = int(self.local_routing if self.local_routing is not None else not s.has_shared_expert)
+        a.qkv_tile = int(s.qkv_tile)
         nbytes = int(self._lib.qmk_moe_workspace_bytes(k, a.shared_k_slices))
         if nbytes == 0:
             raise ValueError(f"top_k {k} / {a.shared_k_slices} K slices are outside what the kernel supports")

@@ -34,6 +34,7 @@ class MoeShape:
     num_downproj_split_k_shared: int = 4
     routed_upgate_tile: int = 16            # outputs per tile of the routed up/gate instructions (16, or 8)
     oproj_tile: int = 16                    # rows per tile of the O-projection instructions (16, or 8: one tile per queue of 256)
+    qkv_tile: int = 16                      # rows per tile of the QKV instructions (16, 8, 4 or 2: whichever deals them evenly)
 
     @property
     def has_shared_expert(self) -> bool:
@@ -90,15 +91,18 @@ class MoeShape:
         return self.weight_bytes_per_token() + kv * context_len + kv
 
 
-QWEN1_5_MOE_A2_7B = MoeShape()
+#: Qwen1.5-MoE-A2.7B, the reference's shape.  QKV tiles of 8 rows: 768 of them, three per queue of a 256-CU device
+#: (384 tiles of 16 leave half of the queues with two); `reference_scheduler` emits the reference's tiles of 16.
+QWEN1_5_MOE_A2_7B = MoeShape(qkv_tile=8)
 
 #: Qwen3-30B-A3B shape: 48 layers, 32 query / 4 KV heads of 128 (attention output 4096 wide), per-head QK RMSNorm,
 #: no QKV bias, 128 experts of 768 with renormalised top-8 routing, no shared expert, untied LM head; 61 GB in bf16.
-#: Routed up/gate tiles of 8 outputs: 8 x 96 = 768 tiles, three per queue of a 256-CU device.
+#: Routed up/gate tiles of 8 outputs: 8 x 96 = 768 tiles, three per queue of a 256-CU device; QKV tiles of 4 rows:
+#: 1280 tiles, five per queue (320 tiles of 16 leave a quarter of the queues with two).
 QWEN3_30B_A3B = MoeShape(
     num_hidden_layers=48, num_attention_heads=32, num_key_value_heads=4, intermediate_size=0, moe_intermediate_size=768,
     num_experts=128, num_experts_per_tok=8, norm_topk_prob=True, qkv_bias=False, qk_norm=True, attn_reduction_size=8,
-    num_downproj_split_k_shared=0, routed_upgate_tile=8, oproj_tile=8,
+    num_downproj_split_k_shared=0, routed_upgate_tile=8, oproj_tile=8, qkv_tile=4,
 )
 
 MAX_OPCODE = 14

@@ -172,6 +172,7 @@ class MoeRowsMegaKernel:
         a.max_seq_len, a.max_splits, a.vocab_size, a.rope_rows = S, P, V, int(g.rope_cos.shape[0])
         a.num_experts, a.top_k, a.shared_ffn, a.moe_ffn, a.shared_k_slices = E, k, 0, Fm, 0
         a.norm_topk_prob, a.routed_upgate_tile, a.oproj_tile, a.local_routing = int(bool(s.norm_topk_prob)), 0, int(s.oproj_tile), 1
+        a.qkv_tile = int(s.qkv_tile)
         a.flags = _single.QMK_FLAG_TAGGED
         nbytes = int(self._lib.qmk_moe_rows_workspace_bytes(B))
         if nbytes == 0:

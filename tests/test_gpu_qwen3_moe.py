@@ -139,6 +139,39 @@ def test_one_op_against_the_vm(weights, stage, position):
         assert float(gpu.routed_out_f32.abs().max()) == 0.0 == float(cpu.routed_out_f32.abs().max())
 
 
+@pytest.mark.parametrize("tile", [16, 8, 4, 2])
+def test_qkv_tiles_of_every_size_give_the_same_rows(weights, tile):
+    """The rows per QKV tile are the stream's choice (``QmkMoeArgs.qkv_tile`` fixes what a head's counter ends at): the
+    projection's output is the same bits whatever the tile, the counters are the VM's, and the attention that waits on
+    them runs.  A stream whose tile is not the launch's is refused on the device; a tile the ABI does not list by the host."""
+    shape = dataclasses.replace(SMALL, qkv_tile=tile)
+    QwenMoeConfig.set_shape(shape)
+    cpu, gpu = make_pair(weights, shape=shape)
+    sched = mk_kernel.mi355x_scheduler(shape, tagged=False)
+    stream = sched.qkvproj(0) + sched.attention_split_kv(0)
+    assert all(i.tile_N_granularity == tile for i in sched.qkvproj(0))
+    MoeInstructionVM(shape).run(cpu, copy.deepcopy(stream))
+    run_kernel(gpu, stream)
+    assert torch.equal(gpu.barriers.cpu(), cpu.barriers) and int(cpu.barriers[0, 0, 0]) == shape.head_dim // tile
+    bf16_close(gpu.qkv_raw, cpu.qkv_raw, ulps=1.0, floor=2.0 ** -6, name="qkv_raw")
+    if tile != 16:
+        QwenMoeConfig.set_shape(SMALL if SMALL.qkv_tile != tile else dataclasses.replace(SMALL, qkv_tile=16))
+        other = make_pair(weights)[1]
+        QwenMoeConfig.set_shape(shape)
+        run_kernel(other, stream)
+        assert torch.equal(other.qkv_raw, gpu.qkv_raw)                      # the same rows from tiles of another size
+    wrong = dataclasses.replace(shape, qkv_tile=16 if tile != 16 else 8)    # the launch says one tile, the stream another
+    QwenMoeConfig.set_shape(wrong)
+    mk = mk_kernel.get_mk(reset_barriers=False, spin_limit=1 << 18)
+    gpu.barriers.zero_()
+    mk_kernel.run_instructions(gpu, copy.deepcopy(sched.qkvproj(0)), mk=mk)
+    with pytest.raises(RuntimeError, match="operand"):
+        mk.check()
+    QwenMoeConfig.set_shape(dataclasses.replace(shape, qkv_tile=6))
+    with pytest.raises(RuntimeError, match="dimension out of range"):
+        mk_kernel.run_instructions(gpu, copy.deepcopy(sched.qkvproj(0)), mk=mk_kernel.get_mk(reset_barriers=False))
+
+
 @pytest.mark.parametrize("position,partials", [(41, 3), (0, 2), (95, 6), (95, 8)])
 @pytest.mark.parametrize("mode", ["oproj", "last"])
 def test_streams_without_reduction_instructions(weights, position, partials, mode):

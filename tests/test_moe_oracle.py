@@ -98,7 +98,12 @@ def test_every_tile_once(queues):
     for i in layer:
         if i.opcode() in spans:
             spans[i.opcode()] += range(i.tile_N_start_idx, i.tile_N_end_idx)
-    assert spans[1] == list(range(s.qkv_out_dim // 16)) and spans[4] == spans[14] == list(range(s.num_hidden_blocks))
+    assert spans[1] == list(range(s.qkv_out_dim // s.qkv_tile)) and spans[4] == spans[14] == list(range(s.num_hidden_blocks))
+    assert all(i.tile_N_granularity == s.qkv_tile for i in layer if i.opcode() == 1)
+    if queues == 256:    # the tile of the shape deals the QKV rows evenly; the reference's tile of 16 does not
+        assert {i.tile_N_end_idx - i.tile_N_start_idx for i in layer if i.opcode() == 1} == {3} and s.qkv_tile == 8
+        sixteen = S.reference_scheduler(s, 256).qkvproj(3)
+        assert {i.tile_N_end_idx - i.tile_N_start_idx for i in sixteen} == {1, 2} and all(i.tile_N_granularity == 16 for i in sixteen)
     assert spans[10] == list(range(s.intermediate_size // 16))
     assert sum(i.init_shared_out for i in layer if i.opcode() == 10) == 1
     routers = [i for i in layer if i.opcode() == 8]
@@ -162,7 +167,7 @@ def test_vm_agrees_with_fused_and_counters_complete(weights, merge):
     s = SMALL
     for layer in range(s.num_hidden_layers):
         bar = v.barriers[layer]
-        assert bar[0, : s.num_heads].tolist() == [s.head_dim // 16] * s.num_heads
+        assert bar[0, : s.num_heads].tolist() == [s.head_dim // s.qkv_tile] * s.num_heads
         if merge == "last":
             assert bar[1, : s.num_attention_heads].tolist() == [sched.num_partials] * s.num_attention_heads
         else:                                # split-KV instructions count on the reduction row only

@@ -150,7 +150,7 @@ def test_vm_against_fused_and_final_counters(weights, stream):
     s = SMALL
     for layer in range(s.num_hidden_layers):
         bar = v.barriers[layer]
-        assert bar[0, : s.num_heads].tolist() == [s.head_dim // 16] * s.num_heads
+        assert bar[0, : s.num_heads].tolist() == [s.head_dim // sched.shape.qkv_tile] * s.num_heads      # 16 rows in the reference's stream, 4 in this one's
         assert int(bar[3, 0]) == s.num_oproj_blocks and int(bar[13, 0]) == s.num_hidden_blocks
         assert bar[7, :2].tolist() == [s.num_experts, 1] and int(bar[8, 0]) == 1
         assert int(bar[9].abs().sum()) == 0 == int(bar[10].abs().sum())             # no shared expert: its rows stay clear
@@ -180,7 +180,8 @@ def test_committing_down_projection_equals_down_projections_plus_combine(weights
 
 def test_full_size_stream():
     """The stream a request of the full shape runs: 48 layers on 256 queues, 768 routed up/gate tiles of 8 outputs per
-    layer dealt three to a queue, one O-projection tile of 8 rows per queue, every queue in dependency order."""
+    layer dealt three to a queue, one O-projection tile of 8 rows per queue, five QKV tiles of 4 rows per queue, every
+    queue in dependency order."""
     sched = mk_kernel.mi355x_scheduler(QWEN3_30B_A3B, tagged=False)
     queues = sched.queues(2)
     assert len(queues) == 256 and sched.num_partials == 2
@@ -191,6 +192,7 @@ def test_full_size_stream():
         layer0 = [i for i in q if i.padded()[1] == 0]
         assert sum(i.padded()[4] - i.padded()[3] for i in layer0 if i.opcode() == 12) == 3
         assert sum(i.padded()[4] - i.padded()[3] for i in layer0 if i.opcode() == 4) == 1
+        assert [(i.padded()[4] - i.padded()[3], i.padded()[6]) for i in layer0 if i.opcode() == 1] == [(5, 4)]
         assert all(i.padded()[3] == 1 for i in layer0 if i.opcode() == 13)           # a down projection waits for its own slot
     flat = [i for q in queues for i in q]
     assert sum(1 for i in flat if i.opcode() == 9) == 2 and sum(1 for i in flat if i.opcode() == 8) == 2 * 16
