@@ -169,7 +169,8 @@ class MoeScheduler:
     # them, and the down projections wait for the slowest queue.  Placed: the last queues of the device take the
     # router and the top-k and no shared up/gate rows; the O-projection queues take one shared up/gate tile and
     # the queues that only wait during the O-projection two; the routed up/gate tiles go where the shared ones
-    # left room (three tiles of the two phases per queue at most).
+    # left room (three tiles of the two phases per queue at most), filling the queues up to one level of weight
+    # rows streamed between the attention and the down projections (`_room_for_routed_rows`).
 
     def _roles(self) -> tuple[list[int], list[int], int]:
         """(queues of the O-projection and the expert phases, queues of the router and the top-k, O-proj count)."""
@@ -210,13 +211,30 @@ class MoeScheduler:
                 lo += size
         return out
 
+    def _room_for_routed_rows(self, shared: dict[int, int], routed_rows: int) -> list[float]:
+        """Per queue, the weight rows of the routed up/gate phase that bring every queue to the same number of rows
+        streamed between the attention and the down projections (O-projection rows, two per shared up/gate output, two
+        per routed one): the level that ``routed_rows`` fill up.  The queues of the router and the top-k count as the
+        least loaded of the others: their routed rows cannot start before everybody's."""
+        main, _, _ = self._roles()
+        load = {q: 2.0 * TILE_N_GRANULARITY * shared.get(q, 0) for q in main}
+        wide = self.shape.num_attention_heads * self.shape.head_dim / self.shape.hidden_size     # an O-projection row in rows of H
+        for i, ins in enumerate(self.oproj(0)):
+            load[main[i % len(main)]] += (ins.tile_N_end_idx - ins.tile_N_start_idx) * ins.tile_N_granularity * wide
+        least = min(load.values())
+        loads = [load.get(q, least) for q in range(self.sm_count)]
+        lo, hi = least, max(loads) + routed_rows
+        for _ in range(60):                      # the level T with sum(max(0, T - load)) = routed_rows
+            mid = (lo + hi) / 2
+            lo, hi = (mid, hi) if sum(max(0.0, mid - x) for x in loads) < routed_rows else (lo, mid)
+        return [max(0.0, hi - x) for x in loads]
+
     def _placed_routed_upgate(self, layer: int) -> list[tuple[int, Instruction]]:
         shared = self._shared_sizes()
         blocks, slots, tile = self.shape.num_routed_upgate_blocks, self.shape.num_experts_per_tok, self.shape.routed_upgate_tile
         queues = list(range(self.sm_count))
         if self.shape.has_shared_expert:
-            most = max(shared.values()) + 1
-            weights = [most - shared.get(q, most - 2) for q in queues]
+            weights = self._room_for_routed_rows(shared, 2 * tile * blocks * slots)
         else:                                    # nothing else in the phase: the tiles evenly on all queues
             weights = [1] * len(queues)
         sizes = self._weighted_sizes(blocks * slots, weights)

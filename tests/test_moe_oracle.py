@@ -231,6 +231,13 @@ def test_placed_stream_is_the_same_instructions_by_role():
     assert len(side) == 9 and not any(i.opcode() in (4, 10) for q in side for i in q)
     tiles = [sum(i.padded()[4] - i.padded()[3] for i in q if i.opcode() in (10, 12)) for q in layer0]
     assert max(tiles) == 3 and sum(tiles) == 2 * 352
+    # weight rows of H per queue between the attention and the down projections (an up/gate output streams two): the routed
+    # tiles fill the queues up to one level, 96 rows, as far as tiles of 16 outputs can (the queues of the router and the
+    # top-k, which start last, get what the least loaded of the others gets)
+    rows = [sum((i.padded()[4] - i.padded()[3]) * (16 if i.opcode() == 4 else 32) for i in q if i.opcode() in (4, 10, 12)) for q in layer0]
+    main = [r for r, q in zip(rows, layer0) if not any(i.opcode() in (8, 9) for i in q)]
+    assert sum(rows) == 256 * 96 and set(main) == {80, 96, 112} and Counter(main)[96] >= 119
+    assert all(sum((i.padded()[4] - i.padded()[3]) for i in q if i.opcode() == 12) == 2 for q in side)
 
 
 def _crafted(weights, layer=0):
