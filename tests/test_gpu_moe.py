@@ -8,8 +8,10 @@ recorded from the reference.
 """
 import copy
 import dataclasses
+import hashlib
 import json
 
+import numpy as np
 import pytest
 import torch
 
@@ -177,10 +179,15 @@ def test_lm_head_against_the_vm(weights):
 
 @pytest.mark.parametrize("queues", [256, 108])
 def test_whole_step(weights, queues):
-    """One step of both layers and the LM head: the reference's stream on 108 queues unchanged, and on 256."""
+    """One step of both layers and the LM head: the reference's stream on 108 queues unchanged (its QKV tiles of 16 rows:
+    the launch takes the tile from the scheduler's shape), and the same order of instructions on 256 with this build's tiles."""
     cpu, gpu = make_pair(weights)
-    sched = S.MoeScheduler(SMALL, queues, num_partials_for(queues, SMALL))
+    sched = S.reference_scheduler(SMALL) if queues == 108 else S.MoeScheduler(SMALL, queues, num_partials_for(queues, SMALL))
+    assert (sched.sm_count, sched.shape.qkv_tile) == ((108, 16) if queues == 108 else (256, SMALL.qkv_tile))
+    QwenMoeConfig.set_shape(sched.shape)
     mine = sched.instruction_list()
+    if queues == 108:     # word for word the list whose digest was recorded from the reference's scheduler
+        assert hashlib.sha256(np.asarray([i.padded() for i in mine], dtype=np.int32).tobytes()).hexdigest() == FIX["instruction_list_sha256"]
     MoeInstructionVM(SMALL).run(cpu, copy.deepcopy(mine))
     run_kernel(gpu, mine, queues=queues)
     assert torch.equal(gpu.barriers.cpu(), cpu.barriers)
